@@ -1,0 +1,182 @@
+/*
+ * CPU restatement of the YVEX attention hot path.  TEST INFRASTRUCTURE ONLY.
+ *
+ * This library is the parity checker for the gfx950 attention backend.  It is
+ * linked or loaded only by tests, by the smoke check and by the benchmark's
+ * CPU-baseline leg; no product code path may call into it.
+ *
+ * Every function names the reference source (relative to the yailabs/clori
+ * tree) whose arithmetic it restates.  Pin status of each function:
+ *
+ *   yvo_exp, yvo_attention_head      pinned: reference literals
+ *       (tests/unit/backend_ops.c:455-510), position-0 / uniform / dominant-key
+ *       closed forms, libm brute force, and the compiled reference operator
+ *       (oracle/_ref) on seeded inputs
+ *   yvo_gqa_attention                pinned: reference KAT
+ *       (tests/unit/cuda/quant_qtype.c:2117-2136) and the reference tests'
+ *       integer-pattern inputs against an independent float two-pass softmax
+ *   yvo_bf16_*, yvo_f16_*            pinned: reference literals
+ *       (tests/reference/deepseek_attention.c:2696-2698), exhaustive 2^16
+ *       round trips, compiled reference codecs (oracle/_ref)
+ *   yvo_q8_0_*                       pinned: golden block
+ *       (tests/unit/quant_numeric.c:514-526), zero block, refusal cases,
+ *       compiled reference decode via oracle/_ref is not available (the block
+ *       encoder is a static function) -> invariants: decode(encode(x)) error
+ *       <= scale/2, idempotence
+ *   yvo_shared_kv_head               pinned: sink KAT
+ *       (tests/reference/deepseek_attention.c:2722-2725); sink=-inf reduces to
+ *       yvo_attention_head within 1e-6
+ *   yvo_paged_*, yvo_mla_*, yvo_lse_merge
+ *       parity unpinned by the reference (it has no page table, no LSE, no
+ *       split-K, no Q8_0 KV cache).  Pinned here only by construction
+ *       invariants: paged == contiguous on the gathered copy (bit-exact),
+ *       page-placement permutation invariance, LSE closed forms, merge
+ *       associativity.
+ */
+#ifndef YVEX_ATTENTION_ORACLE_H
+#define YVEX_ATTENTION_ORACLE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Status values mirror include/yvex/core.h:13-26 of the reference. */
+enum {
+    YVO_OK = 0,
+    YVO_ERR_FORMAT = -4,
+    YVO_ERR_UNSUPPORTED = -5,
+    YVO_ERR_BOUNDS = -7,
+    YVO_ERR_STATE = -8,
+    YVO_ERR_INVALID_ARG = -10
+};
+
+enum { YVO_Q8_0_ELEMENTS = 32, YVO_Q8_0_BYTES = 34 };
+
+/* src/backend/cpu.c:217-255 */
+double yvo_exp(double x);
+
+/* src/gguf/quant_scalar.c:40-143 */
+float yvo_f16_decode(uint16_t bits);
+uint16_t yvo_f16_encode(float value);
+float yvo_bf16_decode(uint16_t bits);
+uint16_t yvo_bf16_encode(float value);
+void yvo_bf16_decode_n(const uint16_t *src, float *dst, size_t n);
+void yvo_bf16_encode_n(const float *src, uint16_t *dst, size_t n);
+
+/* src/gguf/quant_block.c:160-186 (encode), :819-833 (decode).  encode returns 1 on
+ * success and 0 when the scale is not representable, like the reference. */
+int yvo_q8_0_encode_block(const float *source, unsigned char *encoded);
+int yvo_q8_0_decode_block(const unsigned char *encoded, float *out);
+/* Row helpers: n must be a multiple of 32. Return YVO_OK or YVO_ERR_FORMAT/BOUNDS. */
+int yvo_q8_0_encode_row(const float *source, size_t n, unsigned char *encoded);
+int yvo_q8_0_decode_row(const unsigned char *encoded, size_t n, float *out);
+
+/*
+ * One head, one query (src/backend/cpu.c:307-399).  K and V rows are addressed
+ * as base + i*stride (elements); the reference operator is the stride == head_dim
+ * case.  score/prob may be NULL (then internal scratch is used); lse may be NULL.
+ * LSE is max + ln(sum_exp) formed from the same doubles the reference computes.
+ */
+int yvo_attention_head(const float *q, const float *k, size_t k_stride,
+                       const float *v, size_t v_stride, uint64_t seq_len,
+                       uint64_t position, uint64_t head_dim, float scale,
+                       int causal, float *score, float *prob, float *out,
+                       double *lse);
+
+/*
+ * Multi-token grouped-query attention, token/head/dim layout, strides in
+ * elements per token (0 = packed), visibility source <= query_start + t for the
+ * causal mask (include/yvex/internal/transformer.h:258-275,
+ * src/backend/cuda/exact_attention.c:8-53,
+ * src/backend/cuda/transformer_kernels.cu:146-166).  Each (token, head) unit is
+ * evaluated with yvo_attention_head; scale is 1/sqrt(head_dim) as float.
+ * out is packed [Tq, Hq, d] F32; lse (optional) is [Tq, Hq] doubles.
+ * threads <= 1 runs serially.
+ */
+int yvo_gqa_attention(const float *q, const float *k, const float *v, float *out,
+                      double *lse, uint64_t query_tokens, uint64_t kv_tokens,
+                      uint64_t query_start, uint64_t query_heads,
+                      uint64_t kv_heads, uint64_t head_dim, uint64_t q_stride,
+                      uint64_t k_stride, uint64_t v_stride, int causal,
+                      int threads);
+
+/* bf16 in / bf16 out wrapper used for BASELINE configs 1 and 2: widens exactly to
+ * F32, runs yvo_gqa_attention, returns the F32 result and its RNE bf16 rounding. */
+int yvo_gqa_attention_bf16(const uint16_t *q, const uint16_t *k, const uint16_t *v,
+                           float *out_f32, uint16_t *out_bf16, double *lse,
+                           uint64_t query_tokens, uint64_t kv_tokens,
+                           uint64_t query_start, uint64_t query_heads,
+                           uint64_t kv_heads, uint64_t head_dim, int causal,
+                           int threads);
+
+/*
+ * Paged decode.  Canonical pool layout (token-major rows, the reference's
+ * [token, kv_head, dim] history rows cut into pages):
+ *   bf16:  K and V pools are uint16 [pool_pages][page_tokens][kv_heads][head_dim]
+ *   q8_0:  K and V pools are bytes  [pool_pages][page_tokens][kv_heads][head_dim/32][34]
+ * page_table is int32 [sessions][table_stride]; context[s] tokens are visible
+ * (non-causal over the first context[s] tokens; the single query sits at the
+ * last position).  Refuses (YVO_ERR_BOUNDS) a page id outside [0,pool_pages) or
+ * a context needing more than table_stride pages; context 0 is YVO_ERR_INVALID_ARG.
+ * q is bf16 [sessions][query_heads][head_dim].
+ */
+int yvo_paged_decode_bf16(const uint16_t *q, const uint16_t *k_pool,
+                          const uint16_t *v_pool, const int32_t *page_table,
+                          const int32_t *context, float *out_f32,
+                          uint16_t *out_bf16, double *lse, uint64_t sessions,
+                          uint64_t query_heads, uint64_t kv_heads,
+                          uint64_t head_dim, uint64_t page_tokens,
+                          uint64_t pool_pages, uint64_t table_stride, int threads);
+
+int yvo_paged_decode_q8_0(const uint16_t *q, const unsigned char *k_pool,
+                          const unsigned char *v_pool, const int32_t *page_table,
+                          const int32_t *context, float *out_f32,
+                          uint16_t *out_bf16, double *lse, uint64_t sessions,
+                          uint64_t query_heads, uint64_t kv_heads,
+                          uint64_t head_dim, uint64_t page_tokens,
+                          uint64_t pool_pages, uint64_t table_stride, int threads);
+
+/*
+ * Shared-KV head with optional sink logit (src/graph/core.c:361-388,471-508):
+ * every row is both key (first key_dim lanes) and value (first value_dim lanes);
+ * two passes, double score and denominator, libm exp, float accumulator updated
+ * as dest += (float)(w * row), divide in double.  sink may be NULL (no sink).
+ * rows are addressed as base + i*row_stride.  The reference has key_dim ==
+ * value_dim == head_dimension; the absorbed-MLA form uses key_dim 576, value_dim 512.
+ */
+int yvo_shared_kv_head(const float *q, const float *rows, size_t row_stride,
+                       uint64_t row_count, uint64_t key_dim, uint64_t value_dim,
+                       double scale, const float *sink, float *out, double *lse);
+
+/*
+ * Absorbed-latent MLA decode over a paged latent cache (BASELINE config 5).
+ * q bf16 [batch][heads][key_dim]; pool bf16 [pool_pages][page_tokens][key_dim];
+ * value = first value_dim lanes of each row; scale = 1/sqrt(key_dim) in double
+ * (src/graph/core.c:604).  Output is F32 plus RNE bf16 [batch][heads][value_dim].
+ */
+int yvo_mla_decode_bf16(const uint16_t *q, const uint16_t *pool,
+                        const int32_t *page_table, const int32_t *context,
+                        float *out_f32, uint16_t *out_bf16, double *lse,
+                        uint64_t batch, uint64_t heads, uint64_t key_dim,
+                        uint64_t value_dim, uint64_t page_tokens,
+                        uint64_t pool_pages, uint64_t table_stride, int threads);
+
+/*
+ * Log-sum-exp merge of split partials for one head: part p holds a normalised
+ * output o_p[dim] and lse_p; result = sum_p exp(lse_p - L) o_p with
+ * L = log sum_p exp(lse_p).  Parts with lse = -inf are empty.
+ */
+int yvo_lse_merge(const float *part_out, const double *part_lse, uint64_t parts,
+                  uint64_t dim, float *out, double *lse);
+
+/* Number of worker threads the *_threads arguments are clamped to. */
+int yvo_hardware_threads(void);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* YVEX_ATTENTION_ORACLE_H */

@@ -1,0 +1,225 @@
+"""ctypes access to the CPU oracle (test infrastructure) and, when it has been
+built, to the compiled reference operator in oracle/_ref.
+
+Only tests, the smoke check and the benchmark's CPU leg may import this module.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+ORACLE_DIR = os.path.join(ROOT, "oracle")
+ORACLE_SO = os.path.join(ORACLE_DIR, "libyvex_oracle.so")
+REF_SO = os.path.join(ORACLE_DIR, "_ref", "libyvex_ref.so")
+
+u64 = C.c_uint64
+f32p = C.POINTER(C.c_float)
+f64p = C.POINTER(C.c_double)
+u16p = C.POINTER(C.c_uint16)
+u8p = C.POINTER(C.c_ubyte)
+i32p = C.POINTER(C.c_int32)
+
+
+def _ptr(a, typ):
+    if a is None:
+        return C.cast(None, typ)
+    assert a.flags["C_CONTIGUOUS"]
+    return a.ctypes.data_as(typ)
+
+
+def load_oracle():
+    if not os.path.exists(ORACLE_SO):
+        subprocess.check_call(["make", "-C", ORACLE_DIR, "all"])
+    lib = C.CDLL(ORACLE_SO)
+    lib.yvo_exp.restype = C.c_double
+    lib.yvo_exp.argtypes = [C.c_double]
+    lib.yvo_f16_decode.restype = C.c_float
+    lib.yvo_f16_decode.argtypes = [C.c_uint16]
+    lib.yvo_f16_encode.restype = C.c_uint16
+    lib.yvo_f16_encode.argtypes = [C.c_float]
+    lib.yvo_bf16_decode.restype = C.c_float
+    lib.yvo_bf16_decode.argtypes = [C.c_uint16]
+    lib.yvo_bf16_encode.restype = C.c_uint16
+    lib.yvo_bf16_encode.argtypes = [C.c_float]
+    lib.yvo_bf16_decode_n.argtypes = [u16p, f32p, C.c_size_t]
+    lib.yvo_bf16_encode_n.argtypes = [f32p, u16p, C.c_size_t]
+    lib.yvo_q8_0_encode_block.argtypes = [f32p, u8p]
+    lib.yvo_q8_0_decode_block.argtypes = [u8p, f32p]
+    lib.yvo_q8_0_encode_row.argtypes = [f32p, C.c_size_t, u8p]
+    lib.yvo_q8_0_decode_row.argtypes = [u8p, C.c_size_t, f32p]
+    lib.yvo_attention_head.argtypes = [f32p, f32p, C.c_size_t, f32p, C.c_size_t, u64, u64, u64,
+                                       C.c_float, C.c_int, f32p, f32p, f32p, f64p]
+    lib.yvo_gqa_attention.argtypes = [f32p, f32p, f32p, f32p, f64p] + [u64] * 9 + [C.c_int, C.c_int]
+    lib.yvo_gqa_attention_bf16.argtypes = [u16p, u16p, u16p, f32p, u16p, f64p] + [u64] * 6 + [C.c_int, C.c_int]
+    paged = [i32p, i32p, f32p, u16p, f64p] + [u64] * 7 + [C.c_int]
+    lib.yvo_paged_decode_bf16.argtypes = [u16p, u16p, u16p] + paged
+    lib.yvo_paged_decode_q8_0.argtypes = [u16p, u8p, u8p] + paged
+    lib.yvo_shared_kv_head.argtypes = [f32p, f32p, C.c_size_t, u64, u64, u64, C.c_double, f32p, f32p, f64p]
+    lib.yvo_mla_decode_bf16.argtypes = [u16p, u16p, i32p, i32p, f32p, u16p, f64p] + [u64] * 7 + [C.c_int]
+    lib.yvo_lse_merge.argtypes = [f32p, f64p, u64, u64, f32p, f64p]
+    return lib
+
+
+def load_reference():
+    """The compiled reference operator, or None when oracle/_ref was not built."""
+    if not os.path.exists(REF_SO):
+        return None
+    lib = C.CDLL(REF_SO)
+    lib.yvref_op_attention.argtypes = [f32p, f32p, f32p, C.c_ulonglong, C.c_ulonglong,
+                                       C.c_ulonglong, C.c_float, C.c_int, f32p, f32p, f32p]
+    lib.yvref_f16_decode.restype = C.c_float
+    lib.yvref_f16_decode.argtypes = [C.c_ushort]
+    lib.yvref_f16_encode.restype = C.c_ushort
+    lib.yvref_f16_encode.argtypes = [C.c_float]
+    lib.yvref_bf16_decode.restype = C.c_float
+    lib.yvref_bf16_decode.argtypes = [C.c_ushort]
+    lib.yvref_bf16_encode.restype = C.c_ushort
+    lib.yvref_bf16_encode.argtypes = [C.c_float]
+    lib.yvref_bf16_encode_n.argtypes = [f32p, u16p, C.c_size_t]
+    lib.yvref_f16_encode_n.argtypes = [f32p, u16p, C.c_size_t]
+    lib.yvref_f16_decode_n.argtypes = [u16p, f32p, C.c_size_t]
+    if hasattr(lib, "yvref_q8_0_encode_block"):
+        lib.yvref_q8_0_encode_block.argtypes = [f32p, u8p]
+        lib.yvref_q8_0_decode_block.argtypes = [u8p, f32p]
+    return lib
+
+
+class Oracle:
+    """numpy-facing wrapper over the oracle library."""
+
+    def __init__(self):
+        self.lib = load_oracle()
+        self.threads = int(self.lib.yvo_hardware_threads())
+
+    # -- codecs -----------------------------------------------------------
+    def bf16_encode(self, x):
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        out = np.empty(x.shape, dtype=np.uint16)
+        self.lib.yvo_bf16_encode_n(_ptr(x, f32p), _ptr(out, u16p), x.size)
+        return out
+
+    def bf16_decode(self, b):
+        b = np.ascontiguousarray(b, dtype=np.uint16)
+        out = np.empty(b.shape, dtype=np.float32)
+        self.lib.yvo_bf16_decode_n(_ptr(b, u16p), _ptr(out, f32p), b.size)
+        return out
+
+    def q8_0_encode_rows(self, x):
+        """x float32 [..., n] (n % 32 == 0) -> uint8 [..., n/32*34]."""
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        n = x.shape[-1]
+        rows = x.reshape(-1, n)
+        out = np.empty((rows.shape[0], n // 32 * 34), dtype=np.uint8)
+        rc = self.lib.yvo_q8_0_encode_row(_ptr(rows, f32p), rows.size, _ptr(out, u8p))
+        assert rc == 0, rc
+        return out.reshape(x.shape[:-1] + (n // 32 * 34,))
+
+    def q8_0_decode_rows(self, b, n):
+        b = np.ascontiguousarray(b, dtype=np.uint8)
+        rows = b.reshape(-1, n // 32 * 34)
+        out = np.empty((rows.shape[0], n), dtype=np.float32)
+        rc = self.lib.yvo_q8_0_decode_row(_ptr(rows, u8p), out.size, _ptr(out, f32p))
+        assert rc == 0, rc
+        return out.reshape(b.shape[:-1] + (n,))
+
+    # -- attention ----------------------------------------------------------
+    def attention_head(self, q, k, v, position, scale, causal=True):
+        q = np.ascontiguousarray(q, dtype=np.float32)
+        k = np.ascontiguousarray(k, dtype=np.float32)
+        v = np.ascontiguousarray(v, dtype=np.float32)
+        n, d = k.shape
+        score = np.zeros(n, dtype=np.float32)
+        prob = np.zeros(n, dtype=np.float32)
+        out = np.zeros(d, dtype=np.float32)
+        lse = C.c_double(0.0)
+        rc = self.lib.yvo_attention_head(_ptr(q, f32p), _ptr(k, f32p), d, _ptr(v, f32p), d, n,
+                                         position, d, scale, int(causal), _ptr(score, f32p),
+                                         _ptr(prob, f32p), _ptr(out, f32p), C.byref(lse))
+        return rc, out, score, prob, lse.value
+
+    def gqa(self, q, k, v, query_start=0, causal=True, q_stride=0, k_stride=0, v_stride=0,
+            query_tokens=None, kv_tokens=None, query_heads=None, kv_heads=None, head_dim=None,
+            threads=None):
+        """q/k/v float32; when strides are 0 shapes are [T,H,d]."""
+        q = np.ascontiguousarray(q, dtype=np.float32)
+        k = np.ascontiguousarray(k, dtype=np.float32)
+        v = np.ascontiguousarray(v, dtype=np.float32)
+        if query_tokens is None:
+            query_tokens, query_heads, head_dim = q.shape
+            kv_tokens, kv_heads, _ = k.shape
+        out = np.zeros((query_tokens, query_heads, head_dim), dtype=np.float32)
+        lse = np.zeros((query_tokens, query_heads), dtype=np.float64)
+        rc = self.lib.yvo_gqa_attention(_ptr(q, f32p), _ptr(k, f32p), _ptr(v, f32p),
+                                        _ptr(out, f32p), _ptr(lse, f64p), query_tokens,
+                                        kv_tokens, query_start, query_heads, kv_heads, head_dim,
+                                        q_stride, k_stride, v_stride, int(causal),
+                                        threads or self.threads)
+        return rc, out, lse
+
+    def gqa_bf16(self, q, k, v, query_start=0, causal=True, threads=None):
+        """q uint16 [Tq,Hq,d], k/v uint16 [Tk,Hkv,d] -> (rc, out_f32, out_bf16, lse)."""
+        tq, hq, d = q.shape
+        tk, hkv, _ = k.shape
+        out = np.zeros((tq, hq, d), dtype=np.float32)
+        outb = np.zeros((tq, hq, d), dtype=np.uint16)
+        lse = np.zeros((tq, hq), dtype=np.float64)
+        rc = self.lib.yvo_gqa_attention_bf16(_ptr(q, u16p), _ptr(k, u16p), _ptr(v, u16p),
+                                             _ptr(out, f32p), _ptr(outb, u16p), _ptr(lse, f64p),
+                                             tq, tk, query_start, hq, hkv, d, int(causal),
+                                             threads or self.threads)
+        return rc, out, outb, lse
+
+    def paged_decode(self, q, k_pool, v_pool, page_table, context, kv_heads, page_tokens,
+                     q8=False, threads=None):
+        """q uint16 [S,Hq,d]; canonical pools (see the oracle header)."""
+        s, hq, d = q.shape
+        pool_pages = k_pool.shape[0]
+        page_table = np.ascontiguousarray(page_table, dtype=np.int32)
+        context = np.ascontiguousarray(context, dtype=np.int32)
+        out = np.zeros((s, hq, d), dtype=np.float32)
+        outb = np.zeros((s, hq, d), dtype=np.uint16)
+        lse = np.zeros((s, hq), dtype=np.float64)
+        fn = self.lib.yvo_paged_decode_q8_0 if q8 else self.lib.yvo_paged_decode_bf16
+        pt = u8p if q8 else u16p
+        rc = fn(_ptr(q, u16p), _ptr(k_pool, pt), _ptr(v_pool, pt), _ptr(page_table, i32p),
+                _ptr(context, i32p), _ptr(out, f32p), _ptr(outb, u16p), _ptr(lse, f64p), s, hq,
+                kv_heads, d, page_tokens, pool_pages, page_table.shape[1],
+                threads or self.threads)
+        return rc, out, outb, lse
+
+    def shared_kv_head(self, q, rows, key_dim, value_dim, scale, sink=None):
+        q = np.ascontiguousarray(q, dtype=np.float32)
+        rows = np.ascontiguousarray(rows, dtype=np.float32)
+        out = np.zeros(value_dim, dtype=np.float32)
+        lse = C.c_double(0.0)
+        sink_arr = None if sink is None else np.array([sink], dtype=np.float32)
+        rc = self.lib.yvo_shared_kv_head(_ptr(q, f32p), _ptr(rows, f32p), rows.shape[1],
+                                         rows.shape[0], key_dim, value_dim, scale,
+                                         _ptr(sink_arr, f32p), _ptr(out, f32p), C.byref(lse))
+        return rc, out, lse.value
+
+    def mla_decode(self, q, pool, page_table, context, value_dim, page_tokens, threads=None):
+        b, h, kd = q.shape
+        page_table = np.ascontiguousarray(page_table, dtype=np.int32)
+        context = np.ascontiguousarray(context, dtype=np.int32)
+        out = np.zeros((b, h, value_dim), dtype=np.float32)
+        outb = np.zeros((b, h, value_dim), dtype=np.uint16)
+        lse = np.zeros((b, h), dtype=np.float64)
+        rc = self.lib.yvo_mla_decode_bf16(_ptr(q, u16p), _ptr(pool, u16p), _ptr(page_table, i32p),
+                                          _ptr(context, i32p), _ptr(out, f32p), _ptr(outb, u16p),
+                                          _ptr(lse, f64p), b, h, kd, value_dim, page_tokens,
+                                          pool.shape[0], page_table.shape[1],
+                                          threads or self.threads)
+        return rc, out, outb, lse
+
+    def lse_merge(self, part_out, part_lse):
+        part_out = np.ascontiguousarray(part_out, dtype=np.float32)
+        part_lse = np.ascontiguousarray(part_lse, dtype=np.float64)
+        parts, dim = part_out.shape
+        out = np.zeros(dim, dtype=np.float32)
+        lse = C.c_double(0.0)
+        rc = self.lib.yvo_lse_merge(_ptr(part_out, f32p), _ptr(part_lse, f64p), parts, dim,
+                                    _ptr(out, f32p), C.byref(lse))
+        return rc, out, lse.value

@@ -1,0 +1,474 @@
+"""Pins the CPU oracle: reference-held vectors, the compiled reference operator
+(oracle/_ref, when built), closed forms and brute force.  CPU only."""
+import math
+
+import numpy as np
+import pytest
+
+import reference_vectors as rv
+from oracle_binding import Oracle, load_reference, _ptr, f32p, u16p, u8p
+
+ORACLE = Oracle()
+REF = load_reference()
+needs_ref = pytest.mark.skipif(REF is None, reason="oracle/_ref not built (reference tree absent)")
+
+
+# ---------------------------------------------------------------- exp -------
+
+def test_exp_matches_libm_and_clamps():
+    xs = np.concatenate([np.linspace(-60, 0, 4001), np.linspace(0, 60, 401)])
+    for x in xs:
+        got = ORACLE.lib.yvo_exp(float(x))
+        assert abs(got - math.exp(x)) <= 1e-13 * math.exp(x)   # range reduction by repeated ln2 steps
+    assert ORACLE.lib.yvo_exp(-60.0000001) == 0.0          # below -60 is exactly zero
+    assert ORACLE.lib.yvo_exp(100.0) == ORACLE.lib.yvo_exp(60.0)   # clamp above 60
+    assert ORACLE.lib.yvo_exp(0.0) == 1.0
+
+
+# ------------------------------------------------------------- codecs -------
+
+def test_bf16_reference_literals():
+    for value, bits in rv.BF16_LITERALS:
+        assert ORACLE.lib.yvo_bf16_encode(value) == bits
+
+
+def test_bf16_exhaustive_round_trip_and_ties():
+    bits = np.arange(1 << 16, dtype=np.uint16)
+    vals = ORACLE.bf16_decode(bits)
+    back = ORACLE.bf16_encode(vals)
+    nan = np.isnan(vals)
+    assert np.array_equal(back[~nan], bits[~nan])
+    assert np.all((back[nan] & 0x0040) != 0)        # NaNs come back quiet
+    # ties go to even: 1 + 2^-8 is halfway between 0x3f80 and 0x3f81 -> even (0x3f80);
+    # 1 + 3*2^-8 is halfway between 0x3f81 and 0x3f82 -> even (0x3f82)
+    assert ORACLE.lib.yvo_bf16_encode(1.0 + 2.0 ** -8) == 0x3F80
+    assert ORACLE.lib.yvo_bf16_encode(1.0 + 3 * 2.0 ** -8) == 0x3F82
+    # independent check against numpy integer arithmetic on random floats
+    rng = np.random.default_rng(7)
+    x = rng.standard_normal(200000).astype(np.float32) * np.float32(37.0)
+    u = x.view(np.uint32)
+    expect = ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+    assert np.array_equal(ORACLE.bf16_encode(x), expect)
+
+
+def test_f16_exhaustive_round_trip_against_numpy():
+    bits = np.arange(1 << 16, dtype=np.uint16)
+    expect = bits.view(np.float16).astype(np.float32)
+    got = np.array([ORACLE.lib.yvo_f16_decode(int(b)) for b in bits], dtype=np.float32)
+    nan = np.isnan(expect)
+    assert np.array_equal(got[~nan].view(np.uint32), expect[~nan].view(np.uint32))
+    assert np.all(np.isnan(got[nan]))
+    back = np.array([ORACLE.lib.yvo_f16_encode(float(v)) for v in got[~nan]], dtype=np.uint16)
+    assert np.array_equal(back, bits[~nan])
+    # RNE against numpy for random floats incl. subnormal and overflow ranges
+    rng = np.random.default_rng(11)
+    x = np.concatenate([rng.standard_normal(20000) * s for s in (1e-8, 1e-5, 1e-3, 1.0, 3e4, 1e6)])
+    x = x.astype(np.float32)
+    mine = np.array([ORACLE.lib.yvo_f16_encode(float(v)) for v in x], dtype=np.uint16)
+    with np.errstate(over="ignore"):
+        assert np.array_equal(mine, x.astype(np.float16).view(np.uint16))
+
+
+@needs_ref
+def test_codecs_match_compiled_reference():
+    rng = np.random.default_rng(3)
+    x = np.concatenate([rng.standard_normal(300000) * s for s in (1e-8, 1e-4, 1.0, 1e5)])
+    x = np.concatenate([x, [0.0, -0.0, np.inf, -np.inf, np.nan, 65504.0, 65520.0, 6e-8, 3e-8]])
+    x = x.astype(np.float32)
+    ref_b = np.empty(x.size, dtype=np.uint16)
+    ref_h = np.empty(x.size, dtype=np.uint16)
+    REF.yvref_bf16_encode_n(_ptr(x, f32p), _ptr(ref_b, u16p), x.size)
+    REF.yvref_f16_encode_n(_ptr(x, f32p), _ptr(ref_h, u16p), x.size)
+    assert np.array_equal(ORACLE.bf16_encode(x), ref_b)
+    mine_h = np.array([ORACLE.lib.yvo_f16_encode(float(v)) for v in x], dtype=np.uint16)
+    # python float() of a float32 NaN loses nothing that matters here: compare non-NaN exactly
+    ok = ~np.isnan(x)
+    assert np.array_equal(mine_h[ok], ref_h[ok])
+    bits = np.arange(1 << 16, dtype=np.uint16)
+    ref_d = np.empty(bits.size, dtype=np.float32)
+    REF.yvref_f16_decode_n(_ptr(bits, u16p), _ptr(ref_d, f32p), bits.size)
+    mine_d = np.array([ORACLE.lib.yvo_f16_decode(int(b)) for b in bits], dtype=np.float32)
+    assert np.array_equal(mine_d.view(np.uint32), ref_d.view(np.uint32))
+
+
+def test_q8_0_golden_zero_and_refusals():
+    enc = ORACLE.q8_0_encode_rows(rv.Q8_0_GOLDEN_SOURCE)
+    assert bytes(enc[:6]) == rv.Q8_0_GOLDEN_PREFIX            # halfway codes round away from zero
+    assert not enc[6:].any()
+    zero = ORACLE.q8_0_encode_rows(np.zeros(32, dtype=np.float32))
+    assert not zero.any()                                        # canonical zero block
+    assert np.array_equal(ORACLE.q8_0_decode_rows(zero, 32).view(np.uint32),
+                          np.zeros(32, dtype=np.uint32))
+    out = np.empty(34, dtype=np.uint8)
+    huge = np.full(32, np.finfo(np.float32).max, dtype=np.float32)
+    assert ORACLE.lib.yvo_q8_0_encode_block(_ptr(huge, f32p), _ptr(out, u8p)) == 0
+    bad = np.zeros(34, dtype=np.uint8)
+    bad[1] = 0x7C                                                 # +inf scale
+    dec = np.empty(32, dtype=np.float32)
+    assert ORACLE.lib.yvo_q8_0_decode_block(_ptr(bad, u8p), _ptr(dec, f32p)) == 0
+    bad[1] = 0xBC                                                 # negative scale
+    assert ORACLE.lib.yvo_q8_0_decode_block(_ptr(bad, u8p), _ptr(dec, f32p)) == 0
+
+
+def test_q8_0_invariants():
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((512, 128)).astype(np.float32)
+    enc = ORACLE.q8_0_encode_rows(x)
+    dec = ORACLE.q8_0_decode_rows(enc, 128)
+    scales = enc.reshape(512, 4, 34)[:, :, :2].copy().view(np.float16).astype(np.float32)
+    err = np.abs(dec - x).reshape(512, 4, 32)
+    # half a step, plus the clamp slack when the f16 scale rounded below absmax/127
+    amax = np.abs(x).reshape(512, 4, 32).max(axis=2, keepdims=True)
+    slack = np.maximum(amax - 127.0 * scales, 0.0)
+    assert np.all(err <= scales / 2 + slack + 1e-7)
+    # idempotent on decoded values
+    assert np.array_equal(ORACLE.q8_0_encode_rows(dec), enc)
+    codes = enc.reshape(512, 4, 34)[:, :, 2:].view(np.int8)
+    assert codes.min() >= -127
+
+
+@needs_ref
+def test_q8_0_matches_compiled_reference():
+    rng = np.random.default_rng(9)
+    x = (rng.standard_normal((4000, 32)) * rng.uniform(1e-6, 50.0, (4000, 1))).astype(np.float32)
+    x[0] = 0.0
+    x[1, 3] = 0.5 * 127 / 127   # exact-half code cases
+    mine = ORACLE.q8_0_encode_rows(x)
+    for row in range(x.shape[0]):
+        out = np.zeros(34, dtype=np.uint8)
+        src = np.ascontiguousarray(x[row])
+        assert REF.yvref_q8_0_encode_block(_ptr(src, f32p), _ptr(out, u8p)) == 0
+        assert np.array_equal(out, mine[row]), row
+        dec = np.zeros(32, dtype=np.float32)
+        assert REF.yvref_q8_0_decode_block(_ptr(out, u8p), _ptr(dec, f32p)) == 0
+        assert np.array_equal(dec.view(np.uint32),
+                              ORACLE.q8_0_decode_rows(mine[row], 32).view(np.uint32))
+
+
+# --------------------------------------------------- single-head operator ----
+
+def test_single_head_reference_literals():
+    rc, out, _, _, _ = ORACLE.attention_head(rv.CPU_OP_QUERY, rv.CPU_OP_KEYS, rv.CPU_OP_VALUES,
+                                             0, rv.CPU_OP_SCALE)
+    assert rc == 0 and np.allclose(out, rv.CPU_OP_VALUES[0], atol=1e-6)
+    rc, out, score, prob, lse = ORACLE.attention_head(rv.CPU_OP_QUERY, rv.CPU_OP_KEYS,
+                                                      rv.CPU_OP_VALUES, 2, rv.CPU_OP_SCALE)
+    assert rc == 0 and abs(out[0] - rv.CPU_OP_VALUES[0, 0]) > 1e-4
+    s = (rv.CPU_OP_KEYS.astype(np.float64) @ rv.CPU_OP_QUERY.astype(np.float64)) * 0.5
+    p = np.exp(s - s.max())
+    p /= p.sum()
+    assert np.allclose(out, p @ rv.CPU_OP_VALUES.astype(np.float64), atol=1e-5)
+    assert abs(lse - (s.max() + math.log(np.exp(s - s.max()).sum()))) < 1e-7
+    assert abs(prob.sum() - 1.0) < 1e-6
+    rc, *_ = ORACLE.attention_head(rv.CPU_OP_QUERY, rv.CPU_OP_KEYS, rv.CPU_OP_VALUES, 3,
+                                   rv.CPU_OP_SCALE)
+    assert rc == -7                                               # YVEX_ERR_BOUNDS
+    for bad in (0.0, -1.0, float("nan"), float("inf")):
+        rc, *_ = ORACLE.attention_head(rv.CPU_OP_QUERY, rv.CPU_OP_KEYS, rv.CPU_OP_VALUES, 0, bad)
+        assert rc == -10                                          # YVEX_ERR_INVALID_ARG
+
+
+def test_single_head_closed_forms():
+    rng = np.random.default_rng(1)
+    n, d = 300, 64
+    k = rng.standard_normal((n, d)).astype(np.float32)
+    v = rng.standard_normal((n, d)).astype(np.float32)
+    # Q = 0  =>  uniform mean of the visible values, LSE = ln(visible)
+    rc, out, _, prob, lse = ORACLE.attention_head(np.zeros(d, np.float32), k, v, 99, 0.125)
+    assert rc == 0 and np.allclose(out, v[:100].astype(np.float64).mean(axis=0), atol=1e-6)
+    assert abs(lse - math.log(100)) < 1e-12 and not prob[100:].any()
+    # one dominant key => that value row; masked future rows are never read
+    q = rng.standard_normal(d).astype(np.float32)
+    k2 = k * np.float32(0.01)
+    k2[17] = q * np.float32(40.0)
+    k2[250] = q * np.float32(400.0)          # beyond the causal position: must not matter
+    rc, out, *_ = ORACLE.attention_head(q, k2, v, 200, 1.0)
+    assert rc == 0 and np.allclose(out, v[17], atol=1e-6)
+    # non-causal sees every row
+    rc, out, *_ = ORACLE.attention_head(q, k2, v, 0, 1.0, causal=False)
+    assert rc == 0 and np.allclose(out, v[250], atol=1e-6)
+
+
+def test_single_head_brute_force_libm():
+    rng = np.random.default_rng(2)
+    for n, d, scale in ((1, 8, 1.0), (7, 16, 0.25), (513, 128, 0.088388346)):
+        q = rng.standard_normal(d).astype(np.float32)
+        k = rng.standard_normal((n, d)).astype(np.float32)
+        v = rng.standard_normal((n, d)).astype(np.float32)
+        pos = n - 1
+        rc, out, score, prob, lse = ORACLE.attention_head(q, k, v, pos, scale)
+        s = (k.astype(np.float64) @ q.astype(np.float64)) * np.float64(np.float32(scale))
+        e = np.exp(s - s.max())
+        expect = (e / e.sum()) @ v.astype(np.float64)
+        assert rc == 0 and np.allclose(out, expect, atol=3e-6)
+        assert abs(lse - (s.max() + math.log(e.sum()))) < 1e-6
+
+
+@needs_ref
+def test_single_head_bit_exact_against_compiled_reference():
+    """The restatement must reproduce the reference operator bit for bit, including the
+    float score store and both probability roundings."""
+    rng = np.random.default_rng(4)
+    cases = [(3, 4, 0, 0.5, 1), (64, 128, 63, 0.0883883461356163, 1),
+             (777, 128, 500, 0.0883883461356163, 1), (777, 96, 3, 0.3, 0),
+             (4096, 128, 4095, 0.0883883461356163, 1), (2000, 256, 1999, 0.0625, 1)]
+    for n, d, pos, scale, causal in cases:
+        q = (rng.standard_normal(d) * 1.5).astype(np.float32)
+        k = rng.standard_normal((n, d)).astype(np.float32)
+        v = rng.standard_normal((n, d)).astype(np.float32)
+        rs = np.zeros(n, np.float32)
+        rp = np.zeros(n, np.float32)
+        ro = np.zeros(d, np.float32)
+        rc_ref = REF.yvref_op_attention(_ptr(q, f32p), _ptr(k, f32p), _ptr(v, f32p), n, pos, d,
+                                        scale, causal, _ptr(rs, f32p), _ptr(rp, f32p),
+                                        _ptr(ro, f32p))
+        rc, out, score, prob, _ = ORACLE.attention_head(q, k, v, pos, scale, bool(causal))
+        assert rc == rc_ref == 0
+        assert np.array_equal(score.view(np.uint32), rs.view(np.uint32))
+        assert np.array_equal(prob.view(np.uint32), rp.view(np.uint32))
+        assert np.array_equal(out.view(np.uint32), ro.view(np.uint32))
+    # refusal statuses agree too
+    q = np.ones(4, np.float32)
+    k = np.ones((3, 4), np.float32)
+    for n, pos, scale in ((3, 3, 0.5), (3, 0, 0.0), (3, 0, float("nan")), (0, 0, 0.5)):
+        rc_ref = REF.yvref_op_attention(_ptr(q, f32p), _ptr(k, f32p), _ptr(k, f32p), n, pos, 4,
+                                        scale, 1, None, None, None)
+        rc = ORACLE.lib.yvo_attention_head(_ptr(q, f32p), _ptr(k, f32p), 4, _ptr(k, f32p), 4, n,
+                                           pos, 4, scale, 1, None, None, _ptr(q.copy(), f32p),
+                                           None)
+        assert rc == rc_ref and rc != 0
+
+
+# ------------------------------------------------------- multi-token GQA ----
+
+def test_gqa_reference_known_answer():
+    q, k, v, mixed = rv.gqa_kat()
+    rc, out, _ = ORACLE.gqa(q, k, v, causal=True)
+    assert rc == 0
+    assert np.array_equal(out[0], np.array([[2.0, 4.0], [2.0, 4.0]], dtype=np.float32))
+    assert np.allclose(out[1], mixed, atol=1e-6)
+    rc, out, _ = ORACLE.gqa(q, k, v, causal=False)
+    assert rc == 0 and np.allclose(out, np.broadcast_to(mixed, (2, 2, 2)), atol=1e-6)
+
+
+@pytest.mark.parametrize("maker,start,tol_abs,tol_rel", [
+    (rv.small_5x128, 0, 2e-5, 0.0),
+    (rv.qwen_24_4_256, 0, 2e-4, 2e-4),
+    (rv.tiled_257x128, 0, 0.0, 2e-3),
+])
+def test_gqa_reference_patterns_against_float_checker(maker, start, tol_abs, tol_rel):
+    q, k, v = maker()
+    for causal in (True, False):
+        rc, out, _ = ORACLE.gqa(q, k, v, query_start=start, causal=causal)
+        ref = rv.float_two_pass_gqa(q, k, v, start, causal)
+        assert rc == 0
+        assert np.all(np.abs(out - ref) <= tol_abs + tol_rel * (1.0 + np.abs(ref)) + 1e-7)
+
+
+def test_gqa_cached_decode_and_query_range():
+    q, k, v = rv.cached_decode_qwen()
+    rc, out, _ = ORACLE.gqa(q, k, v, query_start=2, causal=True)
+    ref = rv.float_two_pass_gqa(q, k, v, 2, True)
+    assert rc == 0 and np.all(np.abs(out - ref) <= 2e-4 * (1.0 + np.abs(ref)))
+    rc, *_ = ORACLE.gqa(q, k, v, query_start=3, causal=True)      # query range beyond KV
+    assert rc == -10
+
+
+def test_gqa_strided_views_equal_packed():
+    q, k, v = rv.strided_qwen()
+    tq, hq, d = q.shape
+    tk, hkv, _ = k.shape
+    qi = np.zeros((tq, 2 * hq * d), np.float32)          # [Q | gate]
+    qi[:, :hq * d] = q.reshape(tq, -1)
+    qi[:, hq * d:] = 123.0
+    kv = np.zeros((tk, 2 * hkv * d), np.float32)         # [K | V]
+    kv[:, :hkv * d] = k.reshape(tk, -1)
+    kv[:, hkv * d:] = v.reshape(tk, -1)
+    rc, packed, _ = ORACLE.gqa(q, k, v, query_start=2, causal=True)
+    v_view = kv.reshape(-1)[hkv * d:]
+    rc2, strided, _ = ORACLE.gqa(qi, kv, np.ascontiguousarray(v_view), query_start=2, causal=True,
+                                 q_stride=2 * hq * d, k_stride=2 * hkv * d,
+                                 v_stride=2 * hkv * d, query_tokens=tq, kv_tokens=tk,
+                                 query_heads=hq, kv_heads=hkv, head_dim=d)
+    assert rc == rc2 == 0 and np.array_equal(packed, strided)
+    rc3, *_ = ORACLE.gqa(qi, kv, kv, q_stride=hq * d - 1, query_tokens=tq, kv_tokens=tk,
+                         query_heads=hq, kv_heads=hkv, head_dim=d)
+    assert rc3 == -10                                             # stride below row width
+
+
+def test_gqa_uniform_analytic():
+    q, k, v = rv.uniform_large(65, 2)
+    rc, out, lse = ORACLE.gqa(q, k, v, causal=False)
+    assert rc == 0 and np.array_equal(out, v)
+    assert np.allclose(lse, math.log(65), atol=1e-12)
+
+
+def test_gqa_rows_equal_single_head_operator():
+    rng = np.random.default_rng(6)
+    q = rng.standard_normal((4, 8, 32)).astype(np.float32)
+    k = rng.standard_normal((9, 2, 32)).astype(np.float32)
+    v = rng.standard_normal((9, 2, 32)).astype(np.float32)
+    rc, out, lse = ORACLE.gqa(q, k, v, query_start=5, causal=True)
+    assert rc == 0
+    scale = float(np.float32(1.0) / np.sqrt(np.float32(32)))
+    for t in range(4):
+        for h in range(8):
+            rc1, o1, _, _, l1 = ORACLE.attention_head(q[t, h], k[:, h // 4], v[:, h // 4], 5 + t,
+                                                     scale)
+            assert rc1 == 0 and np.array_equal(o1, out[t, h]) and l1 == lse[t, h]
+
+
+# ------------------------------------------------ paged decode (new surface) --
+
+def _paged_case(rng, sessions, hq, hkv, d, page_tokens, contexts, q8=False, spare=3):
+    need = [(c + page_tokens - 1) // page_tokens for c in contexts]
+    pool_pages = sum(need) + spare
+    perm = rng.permutation(pool_pages)
+    table = np.full((sessions, max(need) + 1), -1, dtype=np.int32)
+    at = 0
+    for s, n in enumerate(need):
+        table[s, :n] = perm[at:at + n]
+        at += n
+    kf = ORACLE.bf16_decode(ORACLE.bf16_encode(
+        rng.standard_normal((pool_pages, page_tokens, hkv, d)).astype(np.float32)))
+    vf = ORACLE.bf16_decode(ORACLE.bf16_encode(
+        rng.standard_normal((pool_pages, page_tokens, hkv, d)).astype(np.float32)))
+    q = ORACLE.bf16_encode(rng.standard_normal((sessions, hq, d)).astype(np.float32))
+    if q8:
+        kp, vp = ORACLE.q8_0_encode_rows(kf), ORACLE.q8_0_encode_rows(vf)
+        kf, vf = ORACLE.q8_0_decode_rows(kp, d), ORACLE.q8_0_decode_rows(vp, d)
+    else:
+        kp, vp = ORACLE.bf16_encode(kf), ORACLE.bf16_encode(vf)
+    return q, kp, vp, kf, vf, table, np.array(contexts, dtype=np.int32)
+
+
+@pytest.mark.parametrize("q8", [False, True])
+def test_paged_equals_contiguous_on_gathered_copy(q8):
+    rng = np.random.default_rng(21)
+    contexts = [1, 15, 16, 17, 100, 333]
+    q, kp, vp, kf, vf, table, ctx = _paged_case(rng, 6, 8, 2, 64, 16, contexts, q8=q8)
+    rc, out, outb, lse = ORACLE.paged_decode(q, kp, vp, table, ctx, 2, 16, q8=q8)
+    assert rc == 0
+    qf = ORACLE.bf16_decode(q)
+    for s, n in enumerate(contexts):
+        pages = table[s, :(n + 15) // 16]
+        kc = kf[pages].reshape(-1, 2, 64)[:n]
+        vc = vf[pages].reshape(-1, 2, 64)[:n]
+        rc2, ref, lse2 = ORACLE.gqa(qf[s:s + 1], kc, vc, query_start=n - 1, causal=True)
+        assert rc2 == 0
+        assert np.array_equal(out[s], ref[0]) and np.array_equal(lse[s], lse2[0])
+        assert np.array_equal(outb[s], ORACLE.bf16_encode(ref[0]))
+
+
+def test_paged_placement_invariance_and_refusals():
+    rng = np.random.default_rng(22)
+    contexts = [40, 70]
+    q, kp, vp, _, _, table, ctx = _paged_case(rng, 2, 4, 1, 32, 16, contexts)
+    rc, out, _, lse = ORACLE.paged_decode(q, kp, vp, table, ctx, 1, 16)
+    # move every page to a new slot and rewrite the table: same answer, bit for bit
+    pool_pages = kp.shape[0]
+    perm = rng.permutation(pool_pages)
+    kp2, vp2 = np.empty_like(kp), np.empty_like(vp)
+    kp2[perm], vp2[perm] = kp, vp
+    table2 = np.where(table >= 0, perm[np.maximum(table, 0)], -1).astype(np.int32)
+    rc2, out2, _, lse2 = ORACLE.paged_decode(q, kp2, vp2, table2, ctx, 1, 16)
+    assert rc == rc2 == 0 and np.array_equal(out, out2) and np.array_equal(lse, lse2)
+    # stale entries beyond the used pages are ignored
+    table3 = table.copy()
+    table3[0, 3:] = 10 ** 6
+    rc3, out3, *_ = ORACLE.paged_decode(q, kp, vp, table3, ctx, 1, 16)
+    assert rc3 == 0 and np.array_equal(out3, out)
+    bad = table.copy()
+    bad[1, 2] = pool_pages                                           # out of range
+    assert ORACLE.paged_decode(q, kp, vp, bad, ctx, 1, 16)[0] == -7
+    bad[1, 2] = -1
+    assert ORACLE.paged_decode(q, kp, vp, bad, ctx, 1, 16)[0] == -7
+    assert ORACLE.paged_decode(q, kp, vp, table, np.array([40, 0], np.int32), 1, 16)[0] == -10
+    too_long = np.array([40, table.shape[1] * 16 + 1], np.int32)
+    assert ORACLE.paged_decode(q, kp, vp, table, too_long, 1, 16)[0] == -7
+
+
+# --------------------------------------------------- shared-KV / MLA / merge --
+
+def test_shared_kv_sink_known_answer():
+    kat = rv.SINK_KAT
+    # logits are produced as q.row*scale with q = [1,0,...]: put the logit in a key-only lane
+    rows = np.array([[kat["values"][0][0], kat["values"][0][1], kat["logits"][0]],
+                     [kat["values"][1][0], kat["values"][1][1], kat["logits"][1]]], np.float32)
+    q = np.array([0.0, 0.0, 1.0], np.float32)
+    rc, out, lse = ORACLE.shared_kv_head(q, rows, 3, 2, 1.0, sink=kat["sink"])
+    assert rc == 0 and np.allclose(out, kat["expected"], atol=1e-7)
+    assert abs(lse - math.log(4.0)) < 1e-7                 # e^0 + e^0 + e^{ln 2}
+    # a very negative sink is the reference's "no sink" (tests/unit/deepseek_attention.c:589-628)
+    rc, out_lo, _ = ORACLE.shared_kv_head(q, rows, 3, 2, 1.0, sink=-100.0)
+    rc2, out_no, _ = ORACLE.shared_kv_head(q, rows, 3, 2, 1.0, sink=None)
+    assert rc == rc2 == 0 and np.allclose(out_lo, out_no, atol=1e-7)
+    assert np.allclose(out_no, [(1 + 2 * 3) / 3, (2 + 2 * 4) / 3], atol=1e-6)
+
+
+def test_shared_kv_without_sink_equals_plain_operator():
+    rng = np.random.default_rng(31)
+    n, kd, vd = 200, 48, 32
+    rows = rng.standard_normal((n, kd)).astype(np.float32)
+    q = rng.standard_normal(kd).astype(np.float32)
+    scale = 1.0 / math.sqrt(kd)
+    rc, out, lse = ORACLE.shared_kv_head(q, rows, kd, vd, scale)
+    # plain operator on K = rows, V = first vd lanes (zero-pad V to kd lanes for the shape rule)
+    rc2, ref, _, _, lse2 = ORACLE.attention_head(q, rows, rows, n - 1, np.float32(scale))
+    assert rc == rc2 == 0
+    assert np.allclose(out, ref[:vd], atol=2e-6) and abs(lse - lse2) < 1e-6
+    # output is a convex combination of the latent rows
+    assert np.all(out <= rows[:, :vd].max(axis=0) + 1e-6)
+    assert np.all(out >= rows[:, :vd].min(axis=0) - 1e-6)
+
+
+def test_mla_paged_equals_per_head_shared_kv():
+    rng = np.random.default_rng(32)
+    batch, heads, kd, vd, pt = 3, 5, 96, 64, 8
+    contexts = [5, 8, 29]
+    need = [(c + pt - 1) // pt for c in contexts]
+    pool_pages = sum(need) + 2
+    perm = rng.permutation(pool_pages)
+    table = np.zeros((batch, max(need)), np.int32)
+    at = 0
+    for b, n in enumerate(need):
+        table[b, :n] = perm[at:at + n]
+        at += n
+    pool = ORACLE.bf16_encode(rng.standard_normal((pool_pages, pt, kd)).astype(np.float32))
+    q = ORACLE.bf16_encode(rng.standard_normal((batch, heads, kd)).astype(np.float32))
+    rc, out, outb, lse = ORACLE.mla_decode(q, pool, table, np.array(contexts, np.int32), vd, pt)
+    assert rc == 0
+    pf, qf = ORACLE.bf16_decode(pool), ORACLE.bf16_decode(q)
+    for b, n in enumerate(contexts):
+        rows = pf[table[b, :need[b]]].reshape(-1, kd)[:n]
+        for h in range(heads):
+            rc1, o1, l1 = ORACLE.shared_kv_head(qf[b, h], rows, kd, vd, 1.0 / math.sqrt(kd))
+            assert rc1 == 0 and np.array_equal(o1, out[b, h]) and l1 == lse[b, h]
+    assert np.array_equal(outb, ORACLE.bf16_encode(out))
+
+
+def test_lse_merge_is_associative_with_single_pass():
+    rng = np.random.default_rng(33)
+    n, d = 1000, 32
+    q = rng.standard_normal(d).astype(np.float32)
+    k = rng.standard_normal((n, d)).astype(np.float32)
+    v = rng.standard_normal((n, d)).astype(np.float32)
+    scale = 0.2
+    rc, full, _, _, full_lse = ORACLE.attention_head(q, k, v, n - 1, scale)
+    for cuts in ([0, 1000], [0, 1, 1000], [0, 137, 512, 999, 1000], list(range(0, 1001, 50))):
+        outs, lses = [], []
+        for a, b in zip(cuts[:-1], cuts[1:]):
+            rc1, o, _, _, l = ORACLE.attention_head(q, k[a:b], v[a:b], b - a - 1, scale)
+            assert rc1 == 0
+            outs.append(o)
+            lses.append(l)
+        rc2, merged, merged_lse = ORACLE.lse_merge(np.array(outs), np.array(lses))
+        assert rc2 == 0 and np.allclose(merged, full, atol=1e-6)
+        assert abs(merged_lse - full_lse) < 1e-6
+    # uniform scores: LSE = s + ln n
+    rc, _, _, _, lse = ORACLE.attention_head(np.zeros(d, np.float32), k, v, n - 1, scale)
+    assert abs(lse - math.log(n)) < 1e-12
+    # an empty part (lse = -inf) does not contribute
+    rc, merged, merged_lse = ORACLE.lse_merge(np.array([full, np.zeros(d, np.float32)]),
+                                              np.array([full_lse, -np.inf]))
+    assert rc == 0 and np.allclose(merged, full, atol=1e-7) and abs(merged_lse - full_lse) < 1e-12
