@@ -1,0 +1,363 @@
+"""Thin object wrapper over the C ABI, shaped like the reference's backend API so a
+test reads like the reference's own (open -> tensor_alloc/write -> operation -> read).
+
+Every numerical operation is executed by libyvex_rocm.so on the GPU; nothing here
+computes attention and nothing here falls back to the host.
+"""
+import ctypes as C
+
+import numpy as np
+
+from . import binding as B
+
+
+class YvexError(RuntimeError):
+    """A refused call: carries the reference status code, the stage and the message."""
+
+    def __init__(self, code, where, message):
+        super().__init__("%s at %s: %s" % (B_status_name(code), where, message))
+        self.code = code
+        self.where = where
+        self.message = message
+
+
+_LIB = None
+
+
+def lib():
+    global _LIB
+    if _LIB is None:
+        _LIB = B.load()
+    return _LIB
+
+
+def B_status_name(code):
+    return lib().yvex_status_name(code).decode()
+
+
+def _check(rc, err):
+    if rc != B.YVEX_OK:
+        raise YvexError(rc, err.where.decode(errors="replace"), err.message.decode(errors="replace"))
+
+
+_NP_DTYPE = {B.DTYPE_F32: np.float32, B.DTYPE_BF16: np.uint16, B.DTYPE_F16: np.float16,
+             B.DTYPE_I32: np.int32, B.DTYPE_I8: np.int8, B.DTYPE_I64: np.int64}
+
+
+class Tensor:
+    """One backend-owned device tensor (struct yvex_device_tensor)."""
+
+    def __init__(self, backend, handle, dtype, shape):
+        self.backend = backend
+        self.handle = handle
+        self.dtype = dtype
+        self.shape = tuple(shape)
+
+    @property
+    def nbytes(self):
+        return int(lib().yvex_device_tensor_bytes(self.handle))
+
+    @property
+    def is_written(self):
+        return bool(lib().yvex_device_tensor_is_written(self.handle))
+
+    def write(self, array):
+        array = np.ascontiguousarray(array)
+        err = B.Error()
+        _check(lib().yvex_backend_tensor_write(self.backend.handle, self.handle,
+                                               array.ctypes.data, array.nbytes, C.byref(err)), err)
+        self._keep = None
+        return self
+
+    def read(self, np_dtype=None, shape=None):
+        np_dtype = np_dtype or _NP_DTYPE[self.dtype]
+        out = np.empty(self.nbytes // np.dtype(np_dtype).itemsize, dtype=np_dtype)
+        err = B.Error()
+        _check(lib().yvex_backend_tensor_read(self.backend.handle, self.handle, out.ctypes.data,
+                                              out.nbytes, C.byref(err)), err)
+        return out.reshape(shape or self.shape)
+
+    def zero(self):
+        err = B.Error()
+        _check(lib().yvex_backend_tensor_zero(self.backend.handle, self.handle, C.byref(err)), err)
+
+    def release(self):
+        if self.handle:
+            err = B.Error()
+            ptr = B.TensorP(self.handle.contents)
+            rc = lib().yvex_backend_tensor_release(self.backend.handle, C.byref(ptr), C.byref(err))
+            _check(rc, err)
+            self.handle = None
+
+    def view(self, byte_offset, dtype, shape):
+        """Sub-view made the way the reference does it: copy the struct, offset `data`
+        (src/backend/core.c:1763-1778).  The view borrows this tensor's storage."""
+        view = B.DeviceTensor()
+        C.memmove(C.byref(view), self.handle, C.sizeof(B.DeviceTensor))
+        count = int(np.prod(shape))
+        view.dtype = dtype
+        view.rank = len(shape)
+        for i in range(4):
+            view.dims[i] = shape[i] if i < len(shape) else 0
+        view.bytes = count * B.DTYPE_BYTES[dtype]
+        view.data = self.handle.contents.data + byte_offset
+        tensor = Tensor(self.backend, C.pointer(view), dtype, shape)
+        tensor._parent = self
+        return tensor
+
+
+class Backend:
+    """struct yvex_backend of kind ROCM."""
+
+    def __init__(self, device=None, memory_limit_bytes=0, kind=B.KIND_ROCM):
+        self.handle = C.c_void_p()
+        options = B.BackendOptions(kind, device.encode() if device else None, memory_limit_bytes)
+        err = B.Error()
+        _check(lib().yvex_backend_open(C.byref(self.handle), C.byref(options), C.byref(err)), err)
+        self.tensors = []
+
+    # -- lifecycle --------------------------------------------------------
+    def close(self):
+        if self.handle:
+            for tensor in self.tensors:
+                if tensor.handle:
+                    lib().yvex_backend_tensor_free(self.handle, tensor.handle)
+                    tensor.handle = None
+            err = B.Error()
+            rc = lib().yvex_backend_close_checked(C.byref(self.handle), C.byref(err))
+            _check(rc, err)
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+    @property
+    def status(self):
+        return int(lib().yvex_backend_status_of(self.handle))
+
+    def sync(self):
+        err = B.Error()
+        _check(lib().yvex_backend_sync(self.handle, C.byref(err)), err)
+
+    def memory_stats(self):
+        out, err = B.MemoryStats(), B.Error()
+        _check(lib().yvex_backend_get_memory_stats(self.handle, C.byref(out), C.byref(err)), err)
+        return out
+
+    def device_info(self):
+        out, err = B.DeviceInfo(), B.Error()
+        _check(lib().yvex_backend_get_device_info(self.handle, C.byref(out), C.byref(err)), err)
+        return out
+
+    def report(self):
+        out, err = B.RocmReport(), B.Error()
+        _check(lib().yvex_backend_rocm_report_get(self.handle, C.byref(out), C.byref(err)), err)
+        return out
+
+    def query_capability(self, variant):
+        out, err = B.CapabilityResult(), B.Error()
+        _check(lib().yvex_backend_query_capability(self.handle, variant, C.byref(out),
+                                                   C.byref(err)), err)
+        return out
+
+    def supports(self, capability):
+        return bool(lib().yvex_backend_supports(self.handle, capability))
+
+    def set_completion_mode(self, mode):
+        err = B.Error()
+        _check(lib().yvex_backend_rocm_completion_mode_set(self.handle, mode, C.byref(err)), err)
+
+    def timing_begin(self):
+        err = B.Error()
+        _check(lib().yvex_backend_rocm_timing_begin(self.handle, C.byref(err)), err)
+
+    def timing_end(self):
+        ms, err = C.c_double(0.0), B.Error()
+        _check(lib().yvex_backend_rocm_timing_end(self.handle, C.byref(ms), C.byref(err)), err)
+        return ms.value
+
+    # -- tensors ----------------------------------------------------------
+    def tensor(self, name, dtype, shape, data=None, nbytes=None):
+        desc = B.TensorDesc()
+        desc.name = name.encode()
+        desc.dtype = dtype
+        desc.rank = len(shape)
+        for i, dim in enumerate(shape):
+            desc.dims[i] = dim
+        desc.bytes = nbytes if nbytes is not None else int(np.prod(shape)) * B.DTYPE_BYTES[dtype]
+        handle, err = B.TensorP(), B.Error()
+        _check(lib().yvex_backend_tensor_alloc(self.handle, C.byref(desc), C.byref(handle),
+                                               C.byref(err)), err)
+        tensor = Tensor(self, handle, dtype, shape)
+        self.tensors.append(tensor)
+        if data is not None:
+            tensor.write(data)
+        return tensor
+
+    def workspace_attach(self, tensor, generation=1):
+        err = B.Error()
+        _check(lib().yvex_backend_workspace_attach(self.handle, tensor.handle, generation,
+                                                   C.byref(err)), err)
+
+    def workspace_detach(self):
+        lib().yvex_backend_workspace_detach(self.handle)
+
+    # -- operations ---------------------------------------------------------
+    def op_attention(self, query, keys, values, seq_len, position, scale, causal, score, prob, out):
+        err = B.Error()
+        _check(lib().yvex_backend_op_attention(self.handle, query.handle, keys.handle,
+                                               values.handle, seq_len, position, scale,
+                                               int(causal), score.handle, prob.handle, out.handle,
+                                               C.byref(err)), err)
+
+    def transformer_operations(self):
+        ops = lib().yvex_backend_transformer_operations_get(self.handle)
+        return ops.contents if ops else None
+
+    def rocm_attention_operations(self):
+        ops = lib().yvex_backend_rocm_attention_operations_get(self.handle)
+        return ops.contents if ops else None
+
+    @staticmethod
+    def attention_requirement(query_tokens, kv_tokens, query_heads, kv_heads, head_dim,
+                              causal=True, query_start=0, dtype=B.DTYPE_F32,
+                              contract=B.NUMERIC_EXACT_F32, q_stride=0, k_stride=0, v_stride=0,
+                              deterministic=1):
+        r = B.AttentionRequirement()
+        r.query_tokens, r.key_value_tokens, r.query_start = query_tokens, kv_tokens, query_start
+        r.query_heads, r.key_value_heads, r.head_dimension = query_heads, kv_heads, head_dim
+        r.query_token_stride, r.key_token_stride, r.value_token_stride = q_stride, k_stride, v_stride
+        r.query_dtype = r.key_dtype = r.value_dtype = r.output_dtype = dtype
+        r.layout = B.LAYOUT_TOKEN_HEAD_DIM
+        r.mask = B.MASK_CAUSAL if causal else B.MASK_FULL
+        r.numeric_contract = contract
+        r.deterministic = deterministic
+        return r
+
+    def attention_workspace_required(self, requirement):
+        ops = self.transformer_operations()
+        if ops is None:
+            raise YvexError(B.YVEX_ERR_UNSUPPORTED, "transformer_operations", "not published")
+        out, err = B.ull(0), B.Error()
+        _check(ops.attention_workspace_required(C.byref(requirement), C.byref(out), C.byref(err)),
+               err)
+        return out.value
+
+    def attention_execute(self, requirement, query, key, value, output, lse=None):
+        ops = self.transformer_operations()
+        if ops is None:
+            raise YvexError(B.YVEX_ERR_UNSUPPORTED, "transformer_operations", "not published")
+        request = B.AttentionRequest(requirement, query.handle, key.handle, value.handle,
+                                     output.handle)
+        facts, err = B.OperationFacts(), B.Error()
+        if lse is None:
+            rc = ops.attention_execute(self.handle, C.byref(request), C.byref(facts), C.byref(err))
+        else:
+            rocm = self.rocm_attention_operations()
+            rc = rocm.attention_execute_lse(self.handle, C.byref(request), lse.handle,
+                                            C.byref(facts), C.byref(err))
+        _check(rc, err)
+        return facts
+
+    @staticmethod
+    def paged_requirement(sessions, query_heads, kv_heads, head_dim, page_tokens, pool_pages,
+                          table_stride, max_context, storage=B.KV_BF16,
+                          contract=B.NUMERIC_BF16_F32_ACCUMULATE, deterministic=1):
+        r = B.PagedDecodeRequirement()
+        r.sessions, r.query_heads, r.key_value_heads = sessions, query_heads, kv_heads
+        r.head_dimension, r.page_tokens, r.pool_pages = head_dim, page_tokens, pool_pages
+        r.page_table_stride, r.max_context_tokens = table_stride, max_context
+        r.kv_storage, r.numeric_contract, r.deterministic = storage, contract, deterministic
+        return r
+
+    def paged_decode_workspace_required(self, requirement):
+        out, err = B.ull(0), B.Error()
+        ops = self.rocm_attention_operations()
+        _check(ops.paged_decode_workspace_required(C.byref(requirement), C.byref(out),
+                                                   C.byref(err)), err)
+        return out.value
+
+    def paged_decode_execute(self, requirement, query, key_pages, value_pages, page_table,
+                             context, output, lse=None):
+        ops = self.rocm_attention_operations()
+        if ops is None:
+            raise YvexError(B.YVEX_ERR_UNSUPPORTED, "rocm_attention_operations", "not published")
+        request = B.PagedDecodeRequest(requirement, query.handle, key_pages.handle,
+                                       value_pages.handle, page_table.handle, context.handle,
+                                       output.handle, lse.handle if lse else None)
+        facts, err = B.OperationFacts(), B.Error()
+        _check(ops.paged_decode_execute(self.handle, C.byref(request), C.byref(facts),
+                                        C.byref(err)), err)
+        return facts
+
+    @staticmethod
+    def mla_requirement(batch, heads, key_dim, value_dim, page_tokens, pool_pages, table_stride,
+                        max_context, contract=B.NUMERIC_BF16_F32_ACCUMULATE, deterministic=1):
+        r = B.MlaDecodeRequirement()
+        r.batch, r.heads, r.key_dimension, r.value_dimension = batch, heads, key_dim, value_dim
+        r.page_tokens, r.pool_pages, r.page_table_stride = page_tokens, pool_pages, table_stride
+        r.max_context_tokens, r.numeric_contract, r.deterministic = max_context, contract, deterministic
+        return r
+
+    def mla_decode_execute(self, requirement, query, latent_pages, page_table, context, output,
+                           lse=None):
+        ops = self.rocm_attention_operations()
+        if ops is None:
+            raise YvexError(B.YVEX_ERR_UNSUPPORTED, "rocm_attention_operations", "not published")
+        request = B.MlaDecodeRequest(requirement, query.handle, latent_pages.handle,
+                                     page_table.handle, context.handle, output.handle,
+                                     lse.handle if lse else None)
+        facts, err = B.OperationFacts(), B.Error()
+        _check(ops.mla_decode_execute(self.handle, C.byref(request), C.byref(facts),
+                                      C.byref(err)), err)
+        return facts
+
+
+# -- host helpers that are part of the product (layout + codecs, no attention math) --
+
+def kv_pack_pages(rows, storage, is_value, kv_heads, head_dim=128, page_tokens=16):
+    """rows: token-major [pool_pages][page_tokens][kv_heads][row] (uint16 for BF16, uint8
+    canonical blocks for Q8_0) -> packed device layout as a flat uint8 array."""
+    rows = np.ascontiguousarray(rows)
+    pool_pages = rows.shape[0]
+    block = int(lib().yvex_rocm_kv_page_block_bytes(storage, head_dim, page_tokens))
+    packed = np.empty(pool_pages * kv_heads * block, dtype=np.uint8)
+    err = B.Error()
+    _check(lib().yvex_rocm_kv_pack_pages(storage, int(is_value), rows.ctypes.data, pool_pages,
+                                         page_tokens, kv_heads, head_dim, packed.ctypes.data,
+                                         C.byref(err)), err)
+    return packed
+
+
+def kv_unpack_pages(packed, storage, is_value, pool_pages, kv_heads, head_dim=128, page_tokens=16):
+    packed = np.ascontiguousarray(packed, dtype=np.uint8)
+    if storage == B.KV_BF16:
+        rows = np.empty((pool_pages, page_tokens, kv_heads, head_dim), dtype=np.uint16)
+    else:
+        rows = np.empty((pool_pages, page_tokens, kv_heads, head_dim // 32 * 34), dtype=np.uint8)
+    err = B.Error()
+    _check(lib().yvex_rocm_kv_unpack_pages(storage, int(is_value), packed.ctypes.data, pool_pages,
+                                           page_tokens, kv_heads, head_dim, rows.ctypes.data,
+                                           C.byref(err)), err)
+    return rows
+
+
+def q8_0_encode_rows(x):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    n = x.shape[-1]
+    out = np.empty(x.shape[:-1] + (n // 32 * 34,), dtype=np.uint8)
+    err = B.Error()
+    _check(lib().yvex_rocm_q8_0_encode_row(x.ctypes.data, x.size, out.ctypes.data, C.byref(err)),
+           err)
+    return out
+
+
+def q8_0_decode_rows(b, n):
+    b = np.ascontiguousarray(b, dtype=np.uint8)
+    out = np.empty(b.shape[:-1] + (n,), dtype=np.float32)
+    err = B.Error()
+    _check(lib().yvex_rocm_q8_0_decode_row(b.ctypes.data, out.size, out.ctypes.data, C.byref(err)),
+           err)
+    return out

@@ -1,0 +1,296 @@
+"""ctypes declarations for libyvex_rocm.so (the C ABI of include/yvex_rocm.h).
+
+The library is the product; this module only declares its types and prototypes.
+There is no fallback: a missing library raises at import.
+"""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIBRARY_PATH = os.path.join(_HERE, "libyvex_rocm.so")
+
+# ---- status --------------------------------------------------------------
+YVEX_OK = 0
+YVEX_ERR = -1
+YVEX_ERR_NOMEM = -2
+YVEX_ERR_IO = -3
+YVEX_ERR_FORMAT = -4
+YVEX_ERR_UNSUPPORTED = -5
+YVEX_ERR_BACKEND = -6
+YVEX_ERR_BOUNDS = -7
+YVEX_ERR_STATE = -8
+YVEX_ERR_CANCELLED = -9
+YVEX_ERR_INVALID_ARG = -10
+YVEX_ERR_TIMEOUT = -11
+
+# ---- enums ---------------------------------------------------------------
+DTYPE_F32, DTYPE_F16, DTYPE_BF16, DTYPE_F64 = 1, 2, 3, 4
+DTYPE_I8, DTYPE_I16, DTYPE_I32, DTYPE_I64 = 5, 6, 7, 8
+DTYPE_Q8_0 = 13
+DTYPE_BYTES = {DTYPE_F32: 4, DTYPE_F16: 2, DTYPE_BF16: 2, DTYPE_F64: 8, DTYPE_I8: 1,
+               DTYPE_I16: 2, DTYPE_I32: 4, DTYPE_I64: 8}
+
+KIND_CPU, KIND_CUDA, KIND_METAL, KIND_ROCM = 0, 1, 2, 3
+STATUS_READY, STATUS_CONTEXT_READY, STATUS_UNSUPPORTED, STATUS_FAILED = 0, 1, 2, 3
+
+CAP_TENSOR_ALLOC, CAP_TENSOR_READ_WRITE = 0, 1
+CAP_OP_ATTENTION = 7
+
+VARIANT_TENSOR_ALLOC, VARIANT_TENSOR_ZERO, VARIANT_TENSOR_WRITE = 0, 1, 2
+VARIANT_TENSOR_READ, VARIANT_TENSOR_COPY = 3, 4
+VARIANT_MATMUL_F32 = 10
+VARIANT_ATTENTION_CAUSAL_F32, VARIANT_ATTENTION_NONCAUSAL_F32 = 13, 14
+VARIANT_ATTENTION_ENCODED = 16
+VARIANT_COUNT = 17
+VARIANT_ROCM_GQA_F32, VARIANT_ROCM_GQA_BF16 = 64, 65
+VARIANT_ROCM_PAGED_BF16, VARIANT_ROCM_PAGED_Q8_0, VARIANT_ROCM_MLA_BF16 = 66, 67, 68
+
+CAPABILITY_UNSUPPORTED, CAPABILITY_SUPPORTED, CAPABILITY_FAILED = 0, 1, 2
+(REASON_NONE, REASON_DRIVER_UNAVAILABLE, REASON_DEVICE_UNAVAILABLE, REASON_CONTEXT_UNAVAILABLE,
+ REASON_KERNEL_BUNDLE_ABSENT, REASON_KERNEL_BUNDLE_REJECTED, REASON_FUNCTION_MISSING,
+ REASON_VARIANT_UNSUPPORTED, REASON_LAUNCH_FAILED, REASON_SYNCHRONIZATION_FAILED,
+ REASON_CLEANUP_FAILED) = range(11)
+
+LAYOUT_TOKEN_HEAD_DIM = 1
+MASK_FULL, MASK_CAUSAL = 1, 2
+NUMERIC_EXACT_F32, NUMERIC_BF16_F32_ACCUMULATE = 1, 2
+KV_BF16, KV_Q8_0 = 1, 2
+COMPLETION_IMMEDIATE, COMPLETION_DEFERRED = 0, 1
+
+ull = C.c_ulonglong
+
+
+class Error(C.Structure):
+    _fields_ = [("code", C.c_int), ("where", C.c_char * 96), ("message", C.c_char * 256)]
+
+
+class BackendOptions(C.Structure):
+    _fields_ = [("kind", C.c_int), ("device", C.c_char_p), ("memory_limit_bytes", ull)]
+
+
+class MemoryStats(C.Structure):
+    _fields_ = [(n, ull) for n in ("allocated_bytes", "allocation_count", "allocation_events",
+                                   "release_events", "h2d_bytes", "d2h_bytes",
+                                   "peak_allocated_bytes", "memory_limit_bytes")]
+
+
+class TensorDesc(C.Structure):
+    _fields_ = [("name", C.c_char_p), ("dtype", C.c_int), ("rank", C.c_uint),
+                ("dims", ull * 4), ("bytes", ull)]
+
+
+class DeviceInfo(C.Structure):
+    _fields_ = [("kind", C.c_int), ("name", C.c_char_p), ("device_index", C.c_int),
+                ("compute_capability_major", C.c_int), ("compute_capability_minor", C.c_int),
+                ("global_memory_bytes", ull), ("free_memory_bytes", ull),
+                ("total_memory_bytes", ull), ("unified_addressing", C.c_int),
+                ("managed_memory", C.c_int)]
+
+
+class CapabilityResult(C.Structure):
+    _fields_ = [("backend_kind", C.c_int), ("variant", C.c_int), ("state", C.c_int),
+                ("reason", C.c_int), ("input_dtype", C.c_int), ("weight_dtype", C.c_int),
+                ("output_dtype", C.c_int), ("context_available", C.c_int),
+                ("kernel_bundle_available", C.c_int), ("function_available", C.c_int)]
+
+
+class OperationFacts(C.Structure):
+    _fields_ = [(n, ull) for n in ("h2d_bytes", "d2h_bytes", "d2d_bytes", "kernel_launches",
+                                   "upload_count", "download_count", "queue_synchronizations",
+                                   "device_synchronizations", "active_weight_bytes",
+                                   "state_bytes", "activation_bytes", "temporary_bytes",
+                                   "accelerated_matrix_launches")] + [
+        ("compulsory_memory_facts_available", C.c_int)]
+
+
+class DeviceTensor(C.Structure):
+    _fields_ = [("owner", C.c_void_p), ("owner_id", ull), ("name", C.c_char_p),
+                ("dtype", C.c_int), ("rank", C.c_uint), ("dims", ull * 4), ("bytes", ull),
+                ("data", C.c_void_p), ("host_data", C.c_void_p),
+                ("backend_allocation", C.c_void_p), ("resident_bytes", ull),
+                ("virtual_reserved", C.c_int), ("is_written", C.c_int),
+                ("host_accessible", C.c_int), ("borrowed_host", C.c_int)]
+
+
+TensorP = C.POINTER(DeviceTensor)
+
+
+class AttentionRequirement(C.Structure):
+    _fields_ = [(n, ull) for n in ("query_tokens", "key_value_tokens", "query_start",
+                                   "query_heads", "key_value_heads", "head_dimension",
+                                   "query_token_stride", "key_token_stride",
+                                   "value_token_stride")] + [
+        ("query_dtype", C.c_int), ("key_dtype", C.c_int), ("value_dtype", C.c_int),
+        ("output_dtype", C.c_int), ("layout", C.c_int), ("mask", C.c_int),
+        ("numeric_contract", C.c_int), ("deterministic", C.c_int)]
+
+
+class AttentionRequest(C.Structure):
+    _fields_ = [("requirement", AttentionRequirement), ("query", TensorP), ("key", TensorP),
+                ("value", TensorP), ("output", TensorP)]
+
+
+class PagedDecodeRequirement(C.Structure):
+    _fields_ = [(n, ull) for n in ("sessions", "query_heads", "key_value_heads",
+                                   "head_dimension", "page_tokens", "pool_pages",
+                                   "page_table_stride", "max_context_tokens")] + [
+        ("kv_storage", C.c_int), ("numeric_contract", C.c_int), ("deterministic", C.c_int)]
+
+
+class PagedDecodeRequest(C.Structure):
+    _fields_ = [("requirement", PagedDecodeRequirement), ("query", TensorP),
+                ("key_pages", TensorP), ("value_pages", TensorP), ("page_table", TensorP),
+                ("context_tokens", TensorP), ("output", TensorP), ("lse", TensorP)]
+
+
+class MlaDecodeRequirement(C.Structure):
+    _fields_ = [(n, ull) for n in ("batch", "heads", "key_dimension", "value_dimension",
+                                   "page_tokens", "pool_pages", "page_table_stride",
+                                   "max_context_tokens")] + [
+        ("numeric_contract", C.c_int), ("deterministic", C.c_int)]
+
+
+class MlaDecodeRequest(C.Structure):
+    _fields_ = [("requirement", MlaDecodeRequirement), ("query", TensorP),
+                ("latent_pages", TensorP), ("page_table", TensorP), ("context_tokens", TensorP),
+                ("output", TensorP), ("lse", TensorP)]
+
+
+ErrorP = C.POINTER(Error)
+FactsP = C.POINTER(OperationFacts)
+ullP = C.POINTER(ull)
+
+WORKSPACE_FN = C.CFUNCTYPE(C.c_int, C.POINTER(AttentionRequirement), ullP, ErrorP)
+EXECUTE_FN = C.CFUNCTYPE(C.c_int, C.c_void_p, C.POINTER(AttentionRequest), FactsP, ErrorP)
+EXECUTE_LSE_FN = C.CFUNCTYPE(C.c_int, C.c_void_p, C.POINTER(AttentionRequest), TensorP, FactsP,
+                             ErrorP)
+PAGED_WORKSPACE_FN = C.CFUNCTYPE(C.c_int, C.POINTER(PagedDecodeRequirement), ullP, ErrorP)
+PAGED_EXECUTE_FN = C.CFUNCTYPE(C.c_int, C.c_void_p, C.POINTER(PagedDecodeRequest), FactsP, ErrorP)
+MLA_WORKSPACE_FN = C.CFUNCTYPE(C.c_int, C.POINTER(MlaDecodeRequirement), ullP, ErrorP)
+MLA_EXECUTE_FN = C.CFUNCTYPE(C.c_int, C.c_void_p, C.POINTER(MlaDecodeRequest), FactsP, ErrorP)
+
+
+class TransformerOperations(C.Structure):
+    _fields_ = [("attention_workspace_required", WORKSPACE_FN),
+                ("attention_execute", EXECUTE_FN)]
+
+
+class RocmAttentionOperations(C.Structure):
+    _fields_ = [("attention_execute_lse", EXECUTE_LSE_FN),
+                ("paged_decode_workspace_required", PAGED_WORKSPACE_FN),
+                ("paged_decode_execute", PAGED_EXECUTE_FN),
+                ("mla_decode_workspace_required", MLA_WORKSPACE_FN),
+                ("mla_decode_execute", MLA_EXECUTE_FN)]
+
+
+class RocmReport(C.Structure):
+    _fields_ = [("driver_loaded", C.c_int), ("device_ready", C.c_int), ("bundle_built", C.c_int),
+                ("bundle_admitted", C.c_int), ("image_count", C.c_uint),
+                ("function_count", C.c_uint), ("architecture", C.c_char * 32),
+                ("device_name", C.c_char * 128), ("driver_library", C.c_char * 256),
+                ("rejection", C.c_char * 256)]
+
+
+#: every symbol include/yvex_rocm.h declares
+EXPORTED_SYMBOLS = [
+    "yvex_status_name", "yvex_error_clear", "yvex_error_set",
+    "yvex_backend_open", "yvex_backend_open_rocm_impl", "yvex_backend_rocm_context_available",
+    "yvex_backend_rocm_available", "yvex_backend_close_checked", "yvex_backend_close",
+    "yvex_backend_kind_of", "yvex_backend_kind_name", "yvex_backend_kind_parse",
+    "yvex_backend_status_of", "yvex_backend_status_name", "yvex_backend_get_memory_stats",
+    "yvex_backend_get_device_info", "yvex_backend_tensor_alloc", "yvex_backend_tensor_free",
+    "yvex_backend_tensor_release", "yvex_device_tensor_name", "yvex_device_tensor_bytes",
+    "yvex_device_tensor_is_written", "yvex_backend_tensor_write", "yvex_backend_tensor_read",
+    "yvex_backend_tensor_zero", "yvex_backend_tensor_copy", "yvex_backend_tensor_owned_by",
+    "yvex_backend_tensor_f32_subview", "yvex_backend_sync", "yvex_backend_supports",
+    "yvex_backend_capability_name", "yvex_backend_query_capability",
+    "yvex_backend_operation_variant_name", "yvex_backend_capability_state_name",
+    "yvex_backend_capability_reason_name", "yvex_backend_workspace_attach",
+    "yvex_backend_workspace_detach", "yvex_backend_workspace_acquire",
+    "yvex_backend_op_attention", "yvex_backend_transformer_operations_get",
+    "yvex_backend_rocm_attention_operations_get", "yvex_backend_rocm_completion_mode_set",
+    "yvex_backend_rocm_timing_begin", "yvex_backend_rocm_timing_end",
+    "yvex_backend_rocm_report_get", "yvex_quant_f16_decode", "yvex_quant_f16_encode",
+    "yvex_quant_bf16_decode", "yvex_quant_bf16_encode", "yvex_rocm_q8_0_encode_row",
+    "yvex_rocm_q8_0_decode_row", "yvex_rocm_kv_page_block_bytes", "yvex_rocm_kv_pack_pages",
+    "yvex_rocm_kv_unpack_pages",
+]
+
+
+def load(path=None):
+    """Loads the library and sets prototypes.  Raises OSError when it is not built."""
+    path = path or LIBRARY_PATH
+    if not os.path.exists(path):
+        raise OSError("libyvex_rocm.so is not built: run `make -C clori_amd/csrc` "
+                      "(or __graft_entry__.build())")
+    lib = C.CDLL(path)
+    vp = C.c_void_p
+    lib.yvex_status_name.restype = C.c_char_p
+    lib.yvex_status_name.argtypes = [C.c_int]
+    lib.yvex_backend_open.argtypes = [C.POINTER(vp), C.POINTER(BackendOptions), ErrorP]
+    lib.yvex_backend_open_rocm_impl.argtypes = [C.POINTER(vp), C.c_char_p, ull, ErrorP]
+    lib.yvex_backend_close_checked.argtypes = [C.POINTER(vp), ErrorP]
+    lib.yvex_backend_close.argtypes = [vp]
+    lib.yvex_backend_close.restype = None
+    lib.yvex_backend_kind_of.argtypes = [vp]
+    lib.yvex_backend_kind_name.restype = C.c_char_p
+    lib.yvex_backend_kind_name.argtypes = [C.c_int]
+    lib.yvex_backend_kind_parse.argtypes = [C.c_char_p, C.POINTER(C.c_int), ErrorP]
+    lib.yvex_backend_status_of.argtypes = [vp]
+    lib.yvex_backend_status_name.restype = C.c_char_p
+    lib.yvex_backend_status_name.argtypes = [C.c_int]
+    lib.yvex_backend_get_memory_stats.argtypes = [vp, C.POINTER(MemoryStats), ErrorP]
+    lib.yvex_backend_get_device_info.argtypes = [vp, C.POINTER(DeviceInfo), ErrorP]
+    lib.yvex_backend_tensor_alloc.argtypes = [vp, C.POINTER(TensorDesc), C.POINTER(TensorP), ErrorP]
+    lib.yvex_backend_tensor_free.argtypes = [vp, TensorP]
+    lib.yvex_backend_tensor_free.restype = None
+    lib.yvex_backend_tensor_release.argtypes = [vp, C.POINTER(TensorP), ErrorP]
+    lib.yvex_device_tensor_name.restype = C.c_char_p
+    lib.yvex_device_tensor_name.argtypes = [TensorP]
+    lib.yvex_device_tensor_bytes.restype = ull
+    lib.yvex_device_tensor_bytes.argtypes = [TensorP]
+    lib.yvex_device_tensor_is_written.argtypes = [TensorP]
+    lib.yvex_backend_tensor_write.argtypes = [vp, TensorP, vp, ull, ErrorP]
+    lib.yvex_backend_tensor_read.argtypes = [vp, TensorP, vp, ull, ErrorP]
+    lib.yvex_backend_tensor_zero.argtypes = [vp, TensorP, ErrorP]
+    lib.yvex_backend_tensor_copy.argtypes = [vp, TensorP, TensorP, ErrorP]
+    lib.yvex_backend_tensor_owned_by.argtypes = [vp, TensorP]
+    lib.yvex_backend_tensor_f32_subview.argtypes = [TensorP, ull, ull, TensorP]
+    lib.yvex_backend_sync.argtypes = [vp, ErrorP]
+    lib.yvex_backend_supports.argtypes = [vp, C.c_int]
+    lib.yvex_backend_capability_name.restype = C.c_char_p
+    lib.yvex_backend_capability_name.argtypes = [C.c_int]
+    lib.yvex_backend_query_capability.argtypes = [vp, C.c_int, C.POINTER(CapabilityResult), ErrorP]
+    for fn in ("yvex_backend_operation_variant_name", "yvex_backend_capability_state_name",
+               "yvex_backend_capability_reason_name"):
+        getattr(lib, fn).restype = C.c_char_p
+        getattr(lib, fn).argtypes = [C.c_int]
+    lib.yvex_backend_workspace_attach.argtypes = [vp, TensorP, ull, ErrorP]
+    lib.yvex_backend_workspace_detach.argtypes = [vp]
+    lib.yvex_backend_workspace_detach.restype = None
+    lib.yvex_backend_workspace_acquire.argtypes = [vp, ull, ull, ullP]
+    lib.yvex_backend_op_attention.argtypes = [vp, TensorP, TensorP, TensorP, ull, ull, C.c_float,
+                                              C.c_int, TensorP, TensorP, TensorP, ErrorP]
+    lib.yvex_backend_transformer_operations_get.restype = C.POINTER(TransformerOperations)
+    lib.yvex_backend_transformer_operations_get.argtypes = [vp]
+    lib.yvex_backend_rocm_attention_operations_get.restype = C.POINTER(RocmAttentionOperations)
+    lib.yvex_backend_rocm_attention_operations_get.argtypes = [vp]
+    lib.yvex_backend_rocm_completion_mode_set.argtypes = [vp, C.c_int, ErrorP]
+    lib.yvex_backend_rocm_timing_begin.argtypes = [vp, ErrorP]
+    lib.yvex_backend_rocm_timing_end.argtypes = [vp, C.POINTER(C.c_double), ErrorP]
+    lib.yvex_backend_rocm_report_get.argtypes = [vp, C.POINTER(RocmReport), ErrorP]
+    lib.yvex_quant_f16_decode.restype = C.c_float
+    lib.yvex_quant_f16_decode.argtypes = [C.c_ushort]
+    lib.yvex_quant_f16_encode.restype = C.c_ushort
+    lib.yvex_quant_f16_encode.argtypes = [C.c_float]
+    lib.yvex_quant_bf16_decode.restype = C.c_float
+    lib.yvex_quant_bf16_decode.argtypes = [C.c_ushort]
+    lib.yvex_quant_bf16_encode.restype = C.c_ushort
+    lib.yvex_quant_bf16_encode.argtypes = [C.c_float]
+    lib.yvex_rocm_q8_0_encode_row.argtypes = [vp, ull, vp, ErrorP]
+    lib.yvex_rocm_q8_0_decode_row.argtypes = [vp, ull, vp, ErrorP]
+    lib.yvex_rocm_kv_page_block_bytes.restype = ull
+    lib.yvex_rocm_kv_page_block_bytes.argtypes = [C.c_int, ull, ull]
+    lib.yvex_rocm_kv_pack_pages.argtypes = [C.c_int, C.c_int, vp, ull, ull, ull, ull, vp, ErrorP]
+    lib.yvex_rocm_kv_unpack_pages.argtypes = [C.c_int, C.c_int, vp, ull, ull, ull, ull, vp, ErrorP]
+    return lib

@@ -1,0 +1,596 @@
+/* Attention operations of the ROCm arm: admission, workspace, launch geometry and
+ * physical facts.  No arithmetic happens on the host.
+ *
+ *   yvex_rocm_op_attention            src/backend/cuda/ops.c:1717-1807 (bounded primitive)
+ *   attention_workspace_required /
+ *   attention_execute                 src/backend/cuda/exact_attention.c:8-107,
+ *                                     src/backend/cuda/transformer.c:725-807
+ *   paged / MLA decode                new surface (the reference has no paged KV)
+ */
+#include "rocm_state.h"
+
+#include <math.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include "../kernel_params.h"
+
+enum {
+    ROCM_EXACT_HEAD_MAX = 256,   /* src/backend/cuda/exact_attention.c:6 */
+    ROCM_MFMA_HEAD_DIM = 128,
+    ROCM_PAGE_TOKENS = 16,
+    ROCM_GROUP_MAX = 16,
+    ROCM_CHUNK_MIN = 64,
+    ROCM_CHUNK_MAX = 1024,
+    ROCM_WORK_ALIGNMENT = 256    /* src/backend/cuda/transformer.c:17 */
+};
+
+static int refuse(yvex_error *err, yvex_status status, const char *where, const char *reason)
+{
+    yvex_error_set(err, status, where, reason);
+    return status;
+}
+
+static unsigned long long align_up(unsigned long long value, unsigned long long alignment)
+{
+    return (value + alignment - 1ull) / alignment * alignment;
+}
+
+/* ------------------------------------------------- bounded primitive ---- */
+
+int yvex_rocm_op_attention(yvex_backend *backend, const yvex_device_tensor *query,
+                           const yvex_device_tensor *keys, const yvex_device_tensor *values,
+                           unsigned long long seq_len, unsigned long long position, float scale,
+                           int causal, yvex_device_tensor *score_scratch,
+                           yvex_device_tensor *probability_scratch, yvex_device_tensor *out,
+                           yvex_error *err)
+{
+    static const char where[] = "yvex_backend_op_attention";
+    yvex_rocm_backend_state *state = yvex_rocm_state(backend);
+    yvex_backend_operation_variant variant = causal
+                                                 ? YVEX_BACKEND_VARIANT_ATTENTION_CAUSAL_F32
+                                                 : YVEX_BACKEND_VARIANT_ATTENTION_NONCAUSAL_F32;
+    yvex_rocm_attention_f32_params params;
+    unsigned long long head_dim = 0ull, kv_elements = 0ull;
+    int rc;
+    if (!isfinite(scale) || scale <= 0.0f)
+        return refuse(err, YVEX_ERR_INVALID_ARG, where, "scale must be finite and positive");
+    rc = yvex_backend_validate_attention(backend, query, keys, values, seq_len, position,
+                                         score_scratch, probability_scratch, out, &head_dim,
+                                         &kv_elements, where, err);
+    if (rc != YVEX_OK) return rc;
+    rc = yvex_rocm_require_capability(backend, variant, where, err);
+    if (rc != YVEX_OK) return rc;
+    memset(&params, 0, sizeof(params));
+    params.q = (const float *)query->data;
+    params.k = (const float *)keys->data;
+    params.v = (const float *)values->data;
+    params.score = (float *)score_scratch->data;
+    params.prob = (float *)probability_scratch->data;
+    params.out = (float *)out->data;
+    params.status = state->device_status;
+    params.seq_len = seq_len;
+    params.position = position;
+    params.head_dim = head_dim;
+    params.scale = scale;
+    params.causal = causal ? 1 : 0;
+    rc = yvex_rocm_launch(backend, YVEX_ROCM_FN_ATTENTION_F32, variant, 1u, 1u, 1u, 256u, 0u,
+                          &params, where, err);
+    if (rc == YVEX_OK) rc = yvex_rocm_complete(backend, variant, where, NULL, err);
+    if (rc != YVEX_OK) return rc;
+    score_scratch->is_written = 1;
+    probability_scratch->is_written = 1;
+    out->is_written = 1;
+    yvex_error_clear(err);
+    return YVEX_OK;
+}
+
+/* ------------------------------------------------ split-K decode core ---- */
+
+/* The chunk is a pure function of the request geometry (never of the device) so the
+ * planner's workspace_required and the execution always agree.  It aims at roughly 32
+ * waves per compute unit of a 256-CU part over the worst-case token count. */
+static unsigned int decode_chunk_tokens(unsigned long long sessions, unsigned long long kv_heads,
+                                        unsigned long long max_context)
+{
+    const char *forced = getenv("YVEX_ROCM_DECODE_CHUNK");
+    unsigned long long chunk;
+    if (forced && atoi(forced) >= ROCM_PAGE_TOKENS)
+        chunk = (unsigned long long)atoi(forced);
+    else
+        chunk = sessions * kv_heads * max_context / (256ull * 32ull);
+    chunk = align_up(chunk ? chunk : 1ull, ROCM_PAGE_TOKENS);
+    if (chunk < ROCM_CHUNK_MIN) chunk = ROCM_CHUNK_MIN;
+    if (chunk > ROCM_CHUNK_MAX) chunk = ROCM_CHUNK_MAX;
+    return (unsigned int)chunk;
+}
+
+static int decode_workspace_bytes(unsigned long long sessions, unsigned long long max_chunks,
+                                  unsigned long long query_heads, unsigned long long head_dim,
+                                  unsigned long long *acc_bytes, unsigned long long *total)
+{
+    unsigned long long slots, acc, ml;
+    if (!yvex_core_u64_mul(sessions, max_chunks, &slots) ||
+        !yvex_core_u64_mul(slots, query_heads, &slots) ||
+        !yvex_core_u64_mul(slots, head_dim * sizeof(float), &acc) ||
+        !yvex_core_u64_mul(slots, 2ull * sizeof(float), &ml))
+        return 0;
+    acc = align_up(acc, ROCM_WORK_ALIGNMENT);
+    ml = align_up(ml, ROCM_WORK_ALIGNMENT);
+    if (!yvex_core_u64_add(acc, ml, total)) return 0;
+    *acc_bytes = acc;
+    return 1;
+}
+
+typedef struct {
+    yvex_rocm_function_id function;
+    yvex_backend_operation_variant variant;
+    const void *q, *k, *v;
+    const int32_t *page_table, *context;
+    void *out, *lse;
+    unsigned long long sessions, query_heads, kv_heads, head_dim;
+    unsigned long long pool_pages, table_stride, max_context, fixed_context;
+    unsigned long long k_token_stride, v_token_stride;
+    float scale;
+} decode_job;
+
+/* Launches the partial kernel and the merge kernel and completes the operation. */
+static int decode_run(yvex_backend *backend, const decode_job *job, const char *where,
+                      yvex_backend_operation_facts *facts, yvex_error *err)
+{
+    yvex_rocm_backend_state *state = yvex_rocm_state(backend);
+    yvex_rocm_decode_params dp;
+    yvex_rocm_decode_merge_params mp;
+    unsigned long long acc_bytes = 0ull, total = 0ull, max_chunks;
+    unsigned int chunk = decode_chunk_tokens(job->sessions, job->kv_heads, job->max_context);
+    void *work = NULL;
+    yvex_error cleanup;
+    int owned = 0, rc, cleanup_rc;
+    max_chunks = (job->max_context + chunk - 1ull) / chunk;
+    if (job->sessions > 65535ull || job->kv_heads > 65535ull || job->query_heads > 65535ull ||
+        max_chunks > 0x7fffffffull ||
+        !decode_workspace_bytes(job->sessions, max_chunks, job->query_heads, job->head_dim,
+                                &acc_bytes, &total))
+        return refuse(err, YVEX_ERR_BOUNDS, where, "decode geometry exceeds admitted integer range");
+    backend_workspace_reset(backend);
+    rc = yvex_rocm_temporary_acquire(backend, total, &work, &owned, where, err);
+    if (rc != YVEX_OK) return rc;
+    memset(&dp, 0, sizeof(dp));
+    dp.q = (const uint16_t *)job->q;
+    dp.k_pool = job->k;
+    dp.v_pool = job->v;
+    dp.page_table = job->page_table;
+    dp.context = job->context;
+    dp.part_acc = (float *)work;
+    dp.part_ml = (float *)((unsigned char *)work + acc_bytes);
+    dp.status = state->device_status;
+    dp.k_token_stride = job->k_token_stride;
+    dp.v_token_stride = job->v_token_stride;
+    dp.sessions = (uint32_t)job->sessions;
+    dp.query_heads = (uint32_t)job->query_heads;
+    dp.kv_heads = (uint32_t)job->kv_heads;
+    dp.head_dim = (uint32_t)job->head_dim;
+    dp.pool_pages = (uint32_t)job->pool_pages;
+    dp.table_stride = (uint32_t)job->table_stride;
+    dp.chunk_tokens = chunk;
+    dp.max_chunks = (uint32_t)max_chunks;
+    dp.fixed_context = (uint32_t)job->fixed_context;
+    dp.scale_log2 = job->scale * 1.4426950408889634f;
+    rc = yvex_rocm_launch(backend, job->function, job->variant, (unsigned int)max_chunks,
+                          (unsigned int)job->kv_heads, (unsigned int)job->sessions, 64u, 0u, &dp,
+                          where, err);
+    if (rc == YVEX_OK) {
+        memset(&mp, 0, sizeof(mp));
+        mp.part_acc = dp.part_acc;
+        mp.part_ml = dp.part_ml;
+        mp.context = job->context;
+        mp.out = (uint16_t *)job->out;
+        mp.lse = (float *)job->lse;
+        mp.status = state->device_status;
+        mp.sessions = dp.sessions;
+        mp.query_heads = dp.query_heads;
+        mp.head_dim = dp.head_dim;
+        mp.chunk_tokens = chunk;
+        mp.max_chunks = dp.max_chunks;
+        mp.fixed_context = dp.fixed_context;
+        rc = yvex_rocm_launch(backend, YVEX_ROCM_FN_DECODE_MERGE,
+                              YVEX_BACKEND_VARIANT_ROCM_ATTENTION_PAGED_BF16,
+                              (unsigned int)job->query_heads, (unsigned int)job->sessions, 1u,
+                              (unsigned int)job->head_dim, 0u, &mp, where, err);
+    }
+    if (rc == YVEX_OK) {
+        facts->kernel_launches = 2ull;
+        facts->accelerated_matrix_launches = 1ull;
+        facts->temporary_bytes = total;
+        facts->compulsory_memory_facts_available = 1;
+        rc = yvex_rocm_complete(backend, job->variant, where, facts, err);
+    }
+    yvex_error_clear(&cleanup);
+    cleanup_rc = yvex_rocm_temporary_release(backend, work, total, owned, &cleanup);
+    backend_workspace_reset(backend);
+    if (rc == YVEX_OK && cleanup_rc != YVEX_OK) {
+        rc = cleanup_rc;
+        if (err) *err = cleanup;
+    }
+    return rc;
+}
+
+/* ------------------------------------------- multi-token GQA contract ---- */
+
+static int attention_validate(const yvex_transformer_attention_requirement *r, const char *stage,
+                              yvex_error *err)
+{
+    unsigned long long query_end, query_width, kv_width;
+    if (!r || !r->query_tokens || !r->key_value_tokens ||
+        !yvex_core_u64_add(r->query_start, r->query_tokens, &query_end) ||
+        query_end > r->key_value_tokens || !r->query_heads || !r->key_value_heads ||
+        r->query_heads % r->key_value_heads || !r->head_dimension ||
+        !yvex_core_u64_mul(r->query_heads, r->head_dimension, &query_width) ||
+        !yvex_core_u64_mul(r->key_value_heads, r->head_dimension, &kv_width) ||
+        (r->query_token_stride && r->query_token_stride < query_width) ||
+        (r->key_token_stride && r->key_token_stride < kv_width) ||
+        (r->value_token_stride && r->value_token_stride < kv_width))
+        return refuse(err, YVEX_ERR_INVALID_ARG, stage,
+                      "complete exact-attention geometry is required");
+    if (r->layout != YVEX_TRANSFORMER_ATTENTION_LAYOUT_TOKEN_HEAD_DIM ||
+        r->mask < YVEX_TRANSFORMER_ATTENTION_MASK_FULL ||
+        r->mask > YVEX_TRANSFORMER_ATTENTION_MASK_CAUSAL || !r->deterministic)
+        return refuse(err, YVEX_ERR_UNSUPPORTED, stage,
+                      "ROCm requires deterministic token/head/dimension attention");
+    if (r->numeric_contract == YVEX_TRANSFORMER_ATTENTION_NUMERIC_EXACT_F32) {
+        if (r->head_dimension > ROCM_EXACT_HEAD_MAX || r->query_dtype != YVEX_DTYPE_F32 ||
+            r->key_dtype != YVEX_DTYPE_F32 || r->value_dtype != YVEX_DTYPE_F32 ||
+            r->output_dtype != YVEX_DTYPE_F32)
+            return refuse(err, YVEX_ERR_UNSUPPORTED, stage,
+                          "ROCm requires deterministic token/head/dimension exact F32 attention");
+    } else if (r->numeric_contract == YVEX_TRANSFORMER_ATTENTION_NUMERIC_BF16_F32_ACCUMULATE) {
+        if (r->head_dimension != ROCM_MFMA_HEAD_DIM || r->query_dtype != YVEX_DTYPE_BF16 ||
+            r->key_dtype != YVEX_DTYPE_BF16 || r->value_dtype != YVEX_DTYPE_BF16 ||
+            r->output_dtype != YVEX_DTYPE_BF16 ||
+            r->query_heads / r->key_value_heads > ROCM_GROUP_MAX ||
+            r->key_value_tokens > 0x7fffffffull || (r->query_token_stride % 8ull) ||
+            (r->key_token_stride % 8ull) || (r->value_token_stride % 8ull))
+            return refuse(err, YVEX_ERR_UNSUPPORTED, stage,
+                          "ROCm bf16 attention requires BF16 tensors, head dimension 128, "
+                          "a query group of at most 16 and 16-byte aligned token strides");
+    } else {
+        return refuse(err, YVEX_ERR_UNSUPPORTED, stage,
+                      "ROCm admits the exact F32 and the bf16/fp32-accumulate contracts only");
+    }
+    yvex_error_clear(err);
+    return YVEX_OK;
+}
+
+static unsigned long long visible_tokens(const yvex_transformer_attention_requirement *r)
+{
+    return r->mask == YVEX_TRANSFORMER_ATTENTION_MASK_CAUSAL ? r->query_start + r->query_tokens
+                                                             : r->key_value_tokens;
+}
+
+static int rocm_attention_workspace_required(const yvex_transformer_attention_requirement *r,
+                                             unsigned long long *bytes, yvex_error *err)
+{
+    static const char where[] = "rocm.transformer.attention.workspace";
+    unsigned long long acc = 0ull, total = 0ull, chunk, max_chunks;
+    int rc;
+    if (bytes) *bytes = 0ull;
+    rc = attention_validate(r, where, err);
+    if (rc != YVEX_OK) return rc;
+    if (!bytes) return refuse(err, YVEX_ERR_INVALID_ARG, where, "workspace byte output is required");
+    if (r->numeric_contract == YVEX_TRANSFORMER_ATTENTION_NUMERIC_BF16_F32_ACCUMULATE &&
+        r->query_tokens == 1ull) {
+        /* split-K decode partials; geometry must match decode_run */
+        chunk = decode_chunk_tokens(1ull, r->key_value_heads, visible_tokens(r));
+        max_chunks = (visible_tokens(r) + chunk - 1ull) / chunk;
+        if (!decode_workspace_bytes(1ull, max_chunks, r->query_heads, r->head_dimension, &acc,
+                                    &total))
+            return refuse(err, YVEX_ERR_BOUNDS, where, "decode workspace geometry overflowed");
+        *bytes = total;
+    }
+    yvex_error_clear(err);
+    return YVEX_OK;
+}
+
+static int view_ok(const yvex_backend *backend, const yvex_device_tensor *tensor, yvex_dtype dtype,
+                   unsigned long long elements, int require_written)
+{
+    unsigned long long bytes;
+    return backend_tensor_owner_is(backend, tensor) && (!require_written || tensor->is_written) &&
+           tensor->dtype == dtype && tensor->data &&
+           yvex_core_u64_mul(elements, yvex_dtype_element_bytes(dtype), &bytes) &&
+           tensor->bytes == bytes;
+}
+
+static int attention_execute_common(yvex_backend *backend,
+                                    const yvex_transformer_attention_request *request,
+                                    yvex_device_tensor *lse, yvex_backend_operation_facts *facts,
+                                    yvex_error *err)
+{
+    static const char where[] = "rocm.transformer.attention";
+    yvex_rocm_backend_state *state = yvex_rocm_state(backend);
+    const yvex_transformer_attention_requirement *r;
+    unsigned long long q_width, kv_width, q_stride, k_stride, v_stride;
+    unsigned long long q_elements, k_elements, v_elements, o_elements, rows;
+    int exact, rc, causal;
+    if (!request || !request->query || !request->key || !request->value || !request->output ||
+        !facts)
+        return refuse(err, YVEX_ERR_INVALID_ARG, where,
+                      "complete exact-attention tensors and result facts are required");
+    rc = backend_dispatch_admit(backend, where, err);
+    if (rc != YVEX_OK) return rc;
+    r = &request->requirement;
+    rc = attention_validate(r, where, err);
+    if (rc != YVEX_OK) return rc;
+    memset(facts, 0, sizeof(*facts));
+    exact = r->numeric_contract == YVEX_TRANSFORMER_ATTENTION_NUMERIC_EXACT_F32;
+    causal = r->mask == YVEX_TRANSFORMER_ATTENTION_MASK_CAUSAL;
+    q_width = r->query_heads * r->head_dimension;
+    kv_width = r->key_value_heads * r->head_dimension;
+    q_stride = r->query_token_stride ? r->query_token_stride : q_width;
+    k_stride = r->key_token_stride ? r->key_token_stride : kv_width;
+    v_stride = r->value_token_stride ? r->value_token_stride : kv_width;
+    /* src/backend/cuda/transformer.c:746-770: every view is exactly as large as its
+     * strides imply, inputs are written, everything belongs to this backend */
+    if (!state || !yvex_core_u64_mul(r->query_tokens, r->query_heads, &rows) ||
+        rows > 0xffffffffull ||
+        !yvex_core_u64_mul(r->query_tokens - 1ull, q_stride, &q_elements) ||
+        !yvex_core_u64_add(q_elements, q_width, &q_elements) ||
+        !yvex_core_u64_mul(r->query_tokens, q_width, &o_elements) ||
+        !yvex_core_u64_mul(r->key_value_tokens - 1ull, k_stride, &k_elements) ||
+        !yvex_core_u64_add(k_elements, kv_width, &k_elements) ||
+        !yvex_core_u64_mul(r->key_value_tokens - 1ull, v_stride, &v_elements) ||
+        !yvex_core_u64_add(v_elements, kv_width, &v_elements) ||
+        !view_ok(backend, request->query, r->query_dtype, q_elements, 1) ||
+        !view_ok(backend, request->key, r->key_dtype, k_elements, 1) ||
+        !view_ok(backend, request->value, r->value_dtype, v_elements, 1) ||
+        !view_ok(backend, request->output, r->output_dtype, o_elements, 0) ||
+        (lse && !view_ok(backend, lse, YVEX_DTYPE_F32, rows, 0)))
+        return refuse(err, YVEX_ERR_FORMAT, "rocm.transformer.gqa",
+                      "bounded Q/K/V views matching the declared token strides are required");
+    if (exact) {
+        yvex_rocm_gqa_f32_params params;
+        memset(&params, 0, sizeof(params));
+        params.q = (const float *)request->query->data;
+        params.k = (const float *)request->key->data;
+        params.v = (const float *)request->value->data;
+        params.out = (float *)request->output->data;
+        params.lse = lse ? (float *)lse->data : NULL;
+        params.status = state->device_status;
+        params.query_tokens = r->query_tokens;
+        params.kv_tokens = r->key_value_tokens;
+        params.query_start = r->query_start;
+        params.query_heads = r->query_heads;
+        params.kv_heads = r->key_value_heads;
+        params.head_dim = r->head_dimension;
+        params.q_stride = q_stride;
+        params.k_stride = k_stride;
+        params.v_stride = v_stride;
+        params.scale = 1.0f / sqrtf((float)r->head_dimension);
+        params.causal = causal;
+        backend_workspace_reset(backend);
+        rc = yvex_rocm_launch(backend, YVEX_ROCM_FN_GQA_F32,
+                              YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_F32, (unsigned int)rows, 1u,
+                              1u, 64u, 0u, &params, "rocm.transformer.gqa", err);
+        if (rc == YVEX_OK) {
+            facts->kernel_launches = 1ull;
+            facts->compulsory_memory_facts_available = 1;
+            rc = yvex_rocm_complete(backend, YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_F32,
+                                    "rocm.transformer.gqa", facts, err);
+        }
+    } else if (r->query_tokens == 1ull) {
+        decode_job job;
+        memset(&job, 0, sizeof(job));
+        job.function = YVEX_ROCM_FN_DECODE_ROWS_BF16;
+        job.variant = YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_BF16;
+        job.q = request->query->data;
+        job.k = request->key->data;
+        job.v = request->value->data;
+        job.out = request->output->data;
+        job.lse = lse ? lse->data : NULL;
+        job.sessions = 1ull;
+        job.query_heads = r->query_heads;
+        job.kv_heads = r->key_value_heads;
+        job.head_dim = r->head_dimension;
+        job.max_context = job.fixed_context = visible_tokens(r);
+        job.k_token_stride = k_stride;
+        job.v_token_stride = v_stride;
+        job.scale = 1.0f / sqrtf((float)r->head_dimension);
+        rc = decode_run(backend, &job, "rocm.transformer.gqa.decode", facts, err);
+    } else {
+        rc = refuse(err, YVEX_ERR_UNSUPPORTED, where,
+                    "bf16 multi-token attention is not admitted by this kernel bundle");
+    }
+    if (rc != YVEX_OK) return rc;
+    request->output->is_written = 1;
+    if (lse) lse->is_written = 1;
+    yvex_error_clear(err);
+    return YVEX_OK;
+}
+
+static int rocm_attention_execute(yvex_backend *backend,
+                                  const yvex_transformer_attention_request *request,
+                                  yvex_backend_operation_facts *facts, yvex_error *err)
+{
+    return attention_execute_common(backend, request, NULL, facts, err);
+}
+
+static int rocm_attention_execute_lse(yvex_backend *backend,
+                                      const yvex_transformer_attention_request *request,
+                                      yvex_device_tensor *lse, yvex_backend_operation_facts *facts,
+                                      yvex_error *err)
+{
+    if (!lse)
+        return refuse(err, YVEX_ERR_INVALID_ARG, "rocm.transformer.attention",
+                      "an LSE output tensor is required");
+    return attention_execute_common(backend, request, lse, facts, err);
+}
+
+/* ------------------------------------------------------- paged decode ---- */
+
+static int paged_validate(const yvex_rocm_paged_decode_requirement *r, const char *where,
+                          yvex_error *err)
+{
+    unsigned long long capacity;
+    if (!r || !r->sessions || !r->query_heads || !r->key_value_heads ||
+        r->query_heads % r->key_value_heads || !r->head_dimension || !r->page_tokens ||
+        !r->pool_pages || !r->page_table_stride || !r->max_context_tokens ||
+        !yvex_core_u64_mul(r->page_table_stride, r->page_tokens, &capacity) ||
+        r->max_context_tokens > capacity)
+        return refuse(err, YVEX_ERR_INVALID_ARG, where, "complete paged-decode geometry is required");
+    if (r->head_dimension != ROCM_MFMA_HEAD_DIM || r->page_tokens != ROCM_PAGE_TOKENS ||
+        r->query_heads / r->key_value_heads > ROCM_GROUP_MAX ||
+        (r->kv_storage != YVEX_ROCM_KV_BF16 && r->kv_storage != YVEX_ROCM_KV_Q8_0) ||
+        r->numeric_contract != YVEX_TRANSFORMER_ATTENTION_NUMERIC_BF16_F32_ACCUMULATE ||
+        !r->deterministic || r->pool_pages > 0x7fffffffull || capacity > 0x7fffffffull)
+        return refuse(err, YVEX_ERR_UNSUPPORTED, where,
+                      "ROCm paged decode requires head dimension 128, 16-token pages, a query "
+                      "group of at most 16 and the deterministic bf16/fp32-accumulate contract");
+    yvex_error_clear(err);
+    return YVEX_OK;
+}
+
+static int rocm_paged_decode_workspace_required(const yvex_rocm_paged_decode_requirement *r,
+                                                unsigned long long *bytes, yvex_error *err)
+{
+    static const char where[] = "rocm.attention.paged.workspace";
+    unsigned long long acc = 0ull, total = 0ull, chunk, max_chunks;
+    int rc;
+    if (bytes) *bytes = 0ull;
+    rc = paged_validate(r, where, err);
+    if (rc != YVEX_OK) return rc;
+    if (!bytes) return refuse(err, YVEX_ERR_INVALID_ARG, where, "workspace byte output is required");
+    chunk = decode_chunk_tokens(r->sessions, r->key_value_heads, r->max_context_tokens);
+    max_chunks = (r->max_context_tokens + chunk - 1ull) / chunk;
+    if (!decode_workspace_bytes(r->sessions, max_chunks, r->query_heads, r->head_dimension, &acc,
+                                &total))
+        return refuse(err, YVEX_ERR_BOUNDS, where, "decode workspace geometry overflowed");
+    *bytes = total;
+    yvex_error_clear(err);
+    return YVEX_OK;
+}
+
+static int rocm_paged_decode_execute(yvex_backend *backend,
+                                     const yvex_rocm_paged_decode_request *request,
+                                     yvex_backend_operation_facts *facts, yvex_error *err)
+{
+    static const char where[] = "rocm.attention.paged";
+    const yvex_rocm_paged_decode_requirement *r;
+    unsigned long long q_elements, pool_bytes, block_bytes, table_elements;
+    yvex_dtype pool_dtype;
+    decode_job job;
+    int rc;
+    if (!request || !request->query || !request->key_pages || !request->value_pages ||
+        !request->page_table || !request->context_tokens || !request->output || !facts)
+        return refuse(err, YVEX_ERR_INVALID_ARG, where,
+                      "complete paged-decode tensors and result facts are required");
+    rc = backend_dispatch_admit(backend, where, err);
+    if (rc != YVEX_OK) return rc;
+    r = &request->requirement;
+    rc = paged_validate(r, where, err);
+    if (rc != YVEX_OK) return rc;
+    memset(facts, 0, sizeof(*facts));
+    pool_dtype = r->kv_storage == YVEX_ROCM_KV_BF16 ? YVEX_DTYPE_BF16 : YVEX_DTYPE_I8;
+    block_bytes = yvex_rocm_kv_page_block_bytes(r->kv_storage, r->head_dimension, r->page_tokens);
+    q_elements = r->sessions * r->query_heads * r->head_dimension;
+    table_elements = r->sessions * r->page_table_stride;
+    if (!yvex_core_u64_mul(r->pool_pages * r->key_value_heads, block_bytes, &pool_bytes) ||
+        !view_ok(backend, request->query, YVEX_DTYPE_BF16, q_elements, 1) ||
+        !view_ok(backend, request->key_pages, pool_dtype,
+                 pool_bytes / yvex_dtype_element_bytes(pool_dtype), 1) ||
+        !view_ok(backend, request->value_pages, pool_dtype,
+                 pool_bytes / yvex_dtype_element_bytes(pool_dtype), 1) ||
+        !view_ok(backend, request->page_table, YVEX_DTYPE_I32, table_elements, 1) ||
+        !view_ok(backend, request->context_tokens, YVEX_DTYPE_I32, r->sessions, 1) ||
+        !view_ok(backend, request->output, YVEX_DTYPE_BF16, q_elements, 0) ||
+        (request->lse &&
+         !view_ok(backend, request->lse, YVEX_DTYPE_F32, r->sessions * r->query_heads, 0)))
+        return refuse(err, YVEX_ERR_FORMAT, where,
+                      "query, page pools, page table, context lengths and outputs must be written "
+                      "tensors of this backend with the declared geometry");
+    memset(&job, 0, sizeof(job));
+    if (r->kv_storage == YVEX_ROCM_KV_BF16) {
+        job.function = YVEX_ROCM_FN_DECODE_PAGED_BF16;
+        job.variant = YVEX_BACKEND_VARIANT_ROCM_ATTENTION_PAGED_BF16;
+    } else {
+        job.function = YVEX_ROCM_FN_DECODE_PAGED_Q8_0;
+        job.variant = YVEX_BACKEND_VARIANT_ROCM_ATTENTION_PAGED_Q8_0;
+    }
+    job.q = request->query->data;
+    job.k = request->key_pages->data;
+    job.v = request->value_pages->data;
+    job.page_table = (const int32_t *)request->page_table->data;
+    job.context = (const int32_t *)request->context_tokens->data;
+    job.out = request->output->data;
+    job.lse = request->lse ? request->lse->data : NULL;
+    job.sessions = r->sessions;
+    job.query_heads = r->query_heads;
+    job.kv_heads = r->key_value_heads;
+    job.head_dim = r->head_dimension;
+    job.pool_pages = r->pool_pages;
+    job.table_stride = r->page_table_stride;
+    job.max_context = r->max_context_tokens;
+    job.scale = 1.0f / sqrtf((float)r->head_dimension);
+    rc = decode_run(backend, &job, where, facts, err);
+    if (rc != YVEX_OK) return rc;
+    request->output->is_written = 1;
+    if (request->lse) request->lse->is_written = 1;
+    yvex_error_clear(err);
+    return YVEX_OK;
+}
+
+/* --------------------------------------------------------- MLA decode ---- */
+
+static int rocm_mla_decode_workspace_required(const yvex_rocm_mla_decode_requirement *r,
+                                              unsigned long long *bytes, yvex_error *err)
+{
+    (void)r;
+    if (bytes) *bytes = 0ull;
+    return refuse(err, YVEX_ERR_UNSUPPORTED, "rocm.attention.mla.workspace",
+                  "absorbed MLA decode is not admitted by this kernel bundle");
+}
+
+static int rocm_mla_decode_execute(yvex_backend *backend,
+                                   const yvex_rocm_mla_decode_request *request,
+                                   yvex_backend_operation_facts *facts, yvex_error *err)
+{
+    (void)backend;
+    (void)request;
+    (void)facts;
+    return refuse(err, YVEX_ERR_UNSUPPORTED, "rocm.attention.mla",
+                  "absorbed MLA decode is not admitted by this kernel bundle");
+}
+
+/* ---------------------------------------------------------- op tables ---- */
+
+static const yvex_backend_transformer_operations rocm_transformer_ops = {
+    .attention_workspace_required = rocm_attention_workspace_required,
+    .attention_execute = rocm_attention_execute,
+};
+
+static const yvex_backend_rocm_attention_operations rocm_attention_ops = {
+    .attention_execute_lse = rocm_attention_execute_lse,
+    .paged_decode_workspace_required = rocm_paged_decode_workspace_required,
+    .paged_decode_execute = rocm_paged_decode_execute,
+    .mla_decode_workspace_required = rocm_mla_decode_workspace_required,
+    .mla_decode_execute = rocm_mla_decode_execute,
+};
+
+/* A table is published only once the kernel bundle is admitted
+ * (tests/unit/backend_cpu.c:44-48 asserts the same rule for a backend without kernels). */
+const yvex_backend_transformer_operations *yvex_rocm_transformer_operations(
+    const yvex_backend *backend)
+{
+    const yvex_rocm_backend_state *state = yvex_rocm_state(backend);
+    return state && state->kernel_bundle_state == YVEX_ROCM_KERNEL_BUNDLE_ADMITTED
+               ? &rocm_transformer_ops
+               : NULL;
+}
+
+const yvex_backend_rocm_attention_operations *yvex_rocm_attention_operations(
+    const yvex_backend *backend)
+{
+    const yvex_rocm_backend_state *state = yvex_rocm_state(backend);
+    return state && state->kernel_bundle_state == YVEX_ROCM_KERNEL_BUNDLE_ADMITTED
+               ? &rocm_attention_ops
+               : NULL;
+}

@@ -1,0 +1,525 @@
+/* ROCm backend arm: runtime binding, device and stream ownership, tensor traffic,
+ * synchronisation, timing and the vtable.  Structure follows the reference's CUDA arm
+ * (src/backend/cuda/backend.c:836-1100,1561-1789): the opener binds the runtime, takes
+ * the device, creates the launch stream, admits the kernel bundle and publishes READY;
+ * without a bundle it publishes CONTEXT_READY and every operation variant refuses. */
+#include "rocm_state.h"
+
+#include <stdlib.h>
+#include <string.h>
+
+static int refuse(yvex_error *err, yvex_status status, const char *where, const char *reason)
+{
+    yvex_error_set(err, status, where, reason);
+    return status;
+}
+
+static char *text_dup(const char *text)
+{
+    size_t n = strlen(text ? text : "") + 1u;
+    char *copy = (char *)malloc(n);
+    if (copy) memcpy(copy, text ? text : "", n);
+    return copy;
+}
+
+/* ------------------------------------------------------------- tensors ---- */
+
+/* src/backend/cuda/backend.c:836-905: capability, limit, allocate, zero, publish. */
+static int rocm_tensor_alloc(yvex_backend *backend, const yvex_backend_tensor_desc *desc,
+                             yvex_device_tensor **out, yvex_error *err)
+{
+    static const char where[] = "rocm.tensor_alloc";
+    yvex_rocm_backend_state *state = yvex_rocm_state(backend);
+    yvex_device_tensor *tensor;
+    void *ptr = NULL;
+    unsigned int i;
+    int rc;
+    if (!backend || !state || !out)
+        return refuse(err, YVEX_ERR_INVALID_ARG, where, "backend and out are required");
+    *out = NULL;
+    rc = yvex_rocm_require_capability(backend, YVEX_BACKEND_VARIANT_TENSOR_ALLOC, where, err);
+    if (rc == YVEX_OK)
+        rc = yvex_rocm_require_capability(backend, YVEX_BACKEND_VARIANT_TENSOR_ZERO, where, err);
+    if (rc != YVEX_OK) return rc;
+    rc = yvex_backend_memory_can_add(backend, desc->bytes, "ROCm", where, err);
+    if (rc != YVEX_OK) return rc;
+    rc = yvex_rocm_status(&state->driver, state->driver.hipMalloc(&ptr, (size_t)desc->bytes),
+                          where, err);
+    if (rc != YVEX_OK) {
+        if (err) err->code = YVEX_ERR_NOMEM;
+        return YVEX_ERR_NOMEM;
+    }
+    rc = yvex_rocm_status(&state->driver,
+                          state->driver.hipMemsetAsync(ptr, 0, (size_t)desc->bytes, state->stream),
+                          where, err);
+    if (rc == YVEX_OK)
+        rc = yvex_rocm_synchronize(backend, YVEX_BACKEND_VARIANT_TENSOR_ZERO,
+                                   "rocm.tensor_alloc.zero_sync", err);
+    tensor = rc == YVEX_OK ? (yvex_device_tensor *)calloc(1, sizeof(*tensor)) : NULL;
+    if (rc == YVEX_OK && !tensor) rc = refuse(err, YVEX_ERR_NOMEM, where, "failed to allocate ROCm tensor object");
+    if (rc == YVEX_OK && !(tensor->name = text_dup(desc->name))) {
+        free(tensor);
+        rc = refuse(err, YVEX_ERR_NOMEM, where, "failed to copy ROCm tensor name");
+    }
+    if (rc != YVEX_OK) {
+        (void)state->driver.hipFree(ptr);
+        return rc;
+    }
+    tensor->owner = backend;
+    tensor->owner_id = backend->tensor_id_next++;
+    tensor->dtype = desc->dtype;
+    tensor->rank = desc->rank;
+    for (i = 0; i < desc->rank; ++i) tensor->dims[i] = desc->dims[i];
+    tensor->bytes = desc->bytes;
+    tensor->data = (unsigned char *)ptr;
+    tensor->backend_allocation = ptr;
+    backend_memory_acquire(backend, desc->bytes);
+    state->live_tensors += 1ull;
+    *out = tensor;
+    yvex_error_clear(err);
+    return YVEX_OK;
+}
+
+static int rocm_tensor_free(yvex_backend *backend, yvex_device_tensor *tensor, yvex_error *err)
+{
+    static const char where[] = "rocm.tensor_free";
+    yvex_rocm_backend_state *state = yvex_rocm_state(backend);
+    int rc;
+    if (!backend || !state || !tensor)
+        return refuse(err, YVEX_ERR_INVALID_ARG, where, "backend and tensor are required");
+    if (!backend_tensor_owner_is(backend, tensor))
+        return refuse(err, YVEX_ERR_STATE, where, "tensor does not belong to this backend");
+    if (backend->workspace_device_tensor == tensor) yvex_backend_workspace_detach(backend);
+    /* nothing may still read the allocation: drain the stream first */
+    rc = yvex_rocm_status(&state->driver, state->driver.hipStreamSynchronize(state->stream), where,
+                          err);
+    if (rc == YVEX_OK && getenv("YVEX_TEST_ROCM_CLEANUP_FAILURE"))
+        rc = refuse(err, YVEX_ERR_BACKEND, where, "injected ROCm tensor cleanup failure");
+    if (rc == YVEX_OK && tensor->backend_allocation)
+        rc = yvex_rocm_status(&state->driver, state->driver.hipFree(tensor->backend_allocation),
+                              where, err);
+    if (rc != YVEX_OK) {
+        state->backend_failure_reason = YVEX_BACKEND_CAPABILITY_REASON_CLEANUP_FAILED;
+        backend->status = YVEX_BACKEND_STATUS_FAILED;
+        return rc;
+    }
+    backend_memory_release(backend, tensor->bytes);
+    if (state->live_tensors) state->live_tensors -= 1ull;
+    tensor->owner = NULL;
+    tensor->owner_id = 0ull;
+    free(tensor->name);
+    free(tensor);
+    yvex_error_clear(err);
+    return YVEX_OK;
+}
+
+static int rocm_copy(yvex_backend *backend, void *dst, const void *src, unsigned long long bytes,
+                     hipMemcpyKind kind, yvex_backend_operation_variant variant, const char *where,
+                     yvex_error *err)
+{
+    yvex_rocm_backend_state *state = yvex_rocm_state(backend);
+    int rc = yvex_rocm_require_capability(backend, variant, where, err);
+    if (rc != YVEX_OK) return rc;
+    rc = yvex_rocm_status(&state->driver,
+                          state->driver.hipMemcpyAsync(dst, src, (size_t)bytes, kind, state->stream),
+                          where, err);
+    if (rc == YVEX_OK) rc = yvex_rocm_synchronize(backend, variant, where, err);
+    return rc;
+}
+
+static int rocm_tensor_write(yvex_backend *backend, yvex_device_tensor *tensor, const void *src,
+                             unsigned long long len, yvex_error *err)
+{
+    static const char where[] = "rocm.tensor_write";
+    int rc = yvex_backend_tensor_rw_validate(where, backend, tensor, len, err);
+    if (rc != YVEX_OK) return rc;
+    rc = rocm_copy(backend, tensor->data, src, len, hipMemcpyHostToDevice,
+                   YVEX_BACKEND_VARIANT_TENSOR_WRITE, where, err);
+    if (rc != YVEX_OK) return rc;
+    backend->stats.h2d_bytes += len;
+    tensor->is_written = 1;
+    yvex_error_clear(err);
+    return YVEX_OK;
+}
+
+static int rocm_tensor_read(yvex_backend *backend, const yvex_device_tensor *tensor, void *dst,
+                            unsigned long long len, yvex_error *err)
+{
+    static const char where[] = "rocm.tensor_read";
+    int rc = yvex_backend_tensor_rw_validate(where, backend, tensor, len, err);
+    if (rc != YVEX_OK) return rc;
+    rc = rocm_copy(backend, dst, tensor->data, len, hipMemcpyDeviceToHost,
+                   YVEX_BACKEND_VARIANT_TENSOR_READ, where, err);
+    if (rc != YVEX_OK) return rc;
+    backend->stats.d2h_bytes += len;
+    yvex_error_clear(err);
+    return YVEX_OK;
+}
+
+static int rocm_tensor_zero(yvex_backend *backend, yvex_device_tensor *tensor, yvex_error *err)
+{
+    static const char where[] = "rocm.tensor_zero";
+    yvex_rocm_backend_state *state = yvex_rocm_state(backend);
+    int rc;
+    if (!backend_tensor_owner_is(backend, tensor))
+        return refuse(err, YVEX_ERR_STATE, where, "tensor does not belong to this backend");
+    rc = yvex_rocm_require_capability(backend, YVEX_BACKEND_VARIANT_TENSOR_ZERO, where, err);
+    if (rc != YVEX_OK) return rc;
+    rc = yvex_rocm_status(&state->driver,
+                          state->driver.hipMemsetAsync(tensor->data, 0, (size_t)tensor->bytes,
+                                                       state->stream),
+                          where, err);
+    if (rc == YVEX_OK) rc = yvex_rocm_synchronize(backend, YVEX_BACKEND_VARIANT_TENSOR_ZERO, where, err);
+    if (rc != YVEX_OK) return rc;
+    tensor->is_written = 1;
+    yvex_error_clear(err);
+    return YVEX_OK;
+}
+
+static int rocm_tensor_copy(yvex_backend *backend, yvex_device_tensor *dst,
+                            const yvex_device_tensor *src, yvex_error *err)
+{
+    static const char where[] = "rocm.tensor_copy";
+    int rc = yvex_backend_tensor_copy_validate(backend, dst, src, where, err);
+    if (rc != YVEX_OK) return rc;
+    rc = rocm_copy(backend, dst->data, src->data, src->bytes, hipMemcpyDeviceToDevice,
+                   YVEX_BACKEND_VARIANT_TENSOR_COPY, where, err);
+    if (rc != YVEX_OK) return rc;
+    dst->is_written = 1;
+    yvex_error_clear(err);
+    return YVEX_OK;
+}
+
+/* Synchronise; in DEFERRED completion mode this is also where the device status word of
+ * the operations enqueued since the last check is read and reported. */
+static int rocm_sync(yvex_backend *backend, yvex_error *err)
+{
+    yvex_rocm_backend_state *state = yvex_rocm_state(backend);
+    if (state && state->status_dirty)
+        return yvex_rocm_status_check(backend, "rocm.sync.status", NULL, err);
+    return yvex_rocm_synchronize(backend, YVEX_BACKEND_VARIANT_TENSOR_READ, "rocm.sync", err);
+}
+
+static int rocm_memory_stats(const yvex_backend *backend, yvex_backend_memory_stats *out,
+                             yvex_error *err)
+{
+    *out = backend->stats;
+    yvex_error_clear(err);
+    return YVEX_OK;
+}
+
+static int rocm_device_info(const yvex_backend *backend, yvex_backend_device_info *out,
+                            yvex_error *err)
+{
+    yvex_rocm_backend_state *state = yvex_rocm_state(backend);
+    size_t free_bytes = 0u, total_bytes = 0u;
+    *out = backend->device_info;
+    if (state && state->stream &&
+        state->driver.hipMemGetInfo(&free_bytes, &total_bytes) == hipSuccess) {
+        out->free_memory_bytes = free_bytes;
+        out->total_memory_bytes = total_bytes;
+    }
+    yvex_error_clear(err);
+    return YVEX_OK;
+}
+
+/* ---------------------------------------------------------- temporaries ---- */
+
+/* Operation temporaries come from the attached workspace when it has room
+ * (src/backend/residency.c:251-283), otherwise from a counted allocation that the
+ * operation releases before it returns. */
+int yvex_rocm_temporary_acquire(yvex_backend *backend, unsigned long long bytes, void **address,
+                                int *owned, const char *where, yvex_error *err)
+{
+    yvex_rocm_backend_state *state = yvex_rocm_state(backend);
+    unsigned long long device_address = 0ull;
+    int hit = yvex_backend_workspace_acquire(backend, bytes, 256ull, &device_address);
+    *address = NULL;
+    *owned = 0;
+    if (hit == YVEX_BACKEND_RESIDENT_HIT) {
+        *address = (void *)(uintptr_t)device_address;
+        return YVEX_OK;
+    }
+    if (hit == YVEX_BACKEND_RESIDENT_INVALID)
+        return refuse(err, YVEX_ERR_BOUNDS, where, "temporary workspace geometry is invalid");
+    if (getenv("YVEX_TEST_ROCM_ATTENTION_FAILURE") &&
+        strcmp(getenv("YVEX_TEST_ROCM_ATTENTION_FAILURE"), "allocation") == 0)
+        return refuse(err, YVEX_ERR_NOMEM, where, "injected ROCm temporary allocation failure");
+    if (yvex_backend_memory_can_add(backend, bytes, "ROCm", where, err) != YVEX_OK)
+        return YVEX_ERR_NOMEM;
+    if (yvex_rocm_status(&state->driver, state->driver.hipMalloc(address, (size_t)bytes), where,
+                         err) != YVEX_OK) {
+        if (err) err->code = YVEX_ERR_NOMEM;
+        return YVEX_ERR_NOMEM;
+    }
+    backend_memory_acquire(backend, bytes);
+    *owned = 1;
+    return YVEX_OK;
+}
+
+int yvex_rocm_temporary_release(yvex_backend *backend, void *address, unsigned long long bytes,
+                                int owned, yvex_error *err)
+{
+    yvex_rocm_backend_state *state = yvex_rocm_state(backend);
+    int rc;
+    if (!owned || !address) return YVEX_OK;
+    rc = yvex_rocm_status(&state->driver, state->driver.hipStreamSynchronize(state->stream),
+                          "rocm.temporary.release", err);
+    if (rc == YVEX_OK)
+        rc = yvex_rocm_status(&state->driver, state->driver.hipFree(address),
+                              "rocm.temporary.release", err);
+    if (rc != YVEX_OK) {
+        state->backend_failure_reason = YVEX_BACKEND_CAPABILITY_REASON_CLEANUP_FAILED;
+        backend->status = YVEX_BACKEND_STATUS_FAILED;
+        return rc;
+    }
+    backend_memory_release(backend, bytes);
+    return YVEX_OK;
+}
+
+/* ------------------------------------------------------- open and close ---- */
+
+static int rocm_close(yvex_backend *backend, yvex_error *err)
+{
+    yvex_rocm_backend_state *state = yvex_rocm_state(backend);
+    int rc;
+    if (!state) {
+        yvex_error_clear(err);
+        return YVEX_OK;
+    }
+    if (state->stream) (void)state->driver.hipStreamSynchronize(state->stream);
+    rc = yvex_rocm_kernel_bundle_close(backend, err);
+    if (rc != YVEX_OK) return rc; /* impl retained: checked close can be retried */
+    if (state->device_status) (void)state->driver.hipFree(state->device_status);
+    if (state->timing_start) (void)state->driver.hipEventDestroy(state->timing_start);
+    if (state->timing_stop) (void)state->driver.hipEventDestroy(state->timing_stop);
+    if (state->stream) (void)state->driver.hipStreamDestroy(state->stream);
+    yvex_rocm_driver_unload(&state->driver);
+    free(state);
+    backend->impl = NULL;
+    yvex_error_clear(err);
+    return YVEX_OK;
+}
+
+static const yvex_backend_vtable rocm_vtable = {
+    .close = rocm_close,
+    .memory_stats = rocm_memory_stats,
+    .device_info = rocm_device_info,
+    .tensor_alloc = rocm_tensor_alloc,
+    .tensor_free = rocm_tensor_free,
+    .tensor_write = rocm_tensor_write,
+    .tensor_read = rocm_tensor_read,
+    .tensor_zero = rocm_tensor_zero,
+    .tensor_copy = rocm_tensor_copy,
+    .sync = rocm_sync,
+    .query_capability = yvex_rocm_query_capability,
+    .op_attention = yvex_rocm_op_attention,
+    .transformer_operations = yvex_rocm_transformer_operations,
+    .rocm_attention_operations = yvex_rocm_attention_operations,
+};
+
+static int parse_device(const char *device, int *index)
+{
+    char *end = NULL;
+    long value;
+    *index = 0;
+    if (!device || !*device) return 1;
+    value = strtol(device, &end, 10);
+    if (!end || *end != '\0' || value < 0 || value > 1023) return 0;
+    *index = (int)value;
+    return 1;
+}
+
+int yvex_backend_open_rocm_impl(yvex_backend **out, const char *device,
+                                unsigned long long memory_limit_bytes, yvex_error *err)
+{
+    static const char where[] = "yvex_backend_open_rocm";
+    yvex_backend *backend;
+    yvex_rocm_backend_state *state;
+    yvex_error admit;
+    int count = 0, value = 0, rc;
+    size_t total = 0u;
+    if (!out) return refuse(err, YVEX_ERR_INVALID_ARG, where, "out is required");
+    *out = NULL;
+    backend = (yvex_backend *)calloc(1, sizeof(*backend));
+    state = (yvex_rocm_backend_state *)calloc(1, sizeof(*state));
+    if (!backend || !state) {
+        free(backend);
+        free(state);
+        return refuse(err, YVEX_ERR_NOMEM, where, "failed to allocate ROCm backend");
+    }
+    backend->kind = YVEX_BACKEND_KIND_ROCM;
+    backend->status = YVEX_BACKEND_STATUS_UNSUPPORTED;
+    backend->vtable = &rocm_vtable;
+    backend->impl = state;
+    backend->tensor_id_next = 1ull;
+    backend->stats.memory_limit_bytes = memory_limit_bytes;
+    state->kernel_bundle_reason = YVEX_BACKEND_CAPABILITY_REASON_KERNEL_BUNDLE_ABSENT;
+    state->kernel_bundle_failure_variant = YVEX_BACKEND_VARIANT_COUNT;
+
+    rc = parse_device(device, &state->device_index)
+             ? YVEX_OK
+             : refuse(err, YVEX_ERR_INVALID_ARG, where, "device must be a non-negative index");
+    if (rc == YVEX_OK) rc = yvex_rocm_driver_load(&state->driver, err);
+    if (rc == YVEX_OK && state->driver.hipInit(0u) != hipSuccess)
+        rc = refuse(err, YVEX_ERR_UNSUPPORTED, where, "HIP runtime initialisation failed");
+    if (rc == YVEX_OK &&
+        (state->driver.hipGetDeviceCount(&count) != hipSuccess || count <= state->device_index))
+        rc = refuse(err, YVEX_ERR_UNSUPPORTED, where, "no usable ROCm device");
+    if (rc == YVEX_OK)
+        rc = yvex_rocm_status(&state->driver, state->driver.hipSetDevice(state->device_index),
+                              where, err);
+    if (rc == YVEX_OK)
+        rc = yvex_rocm_status(&state->driver, state->driver.hipStreamCreate(&state->stream), where,
+                              err);
+    if (rc == YVEX_OK)
+        rc = yvex_rocm_status(&state->driver, state->driver.hipEventCreate(&state->timing_start),
+                              where, err);
+    if (rc == YVEX_OK)
+        rc = yvex_rocm_status(&state->driver, state->driver.hipEventCreate(&state->timing_stop),
+                              where, err);
+    if (rc == YVEX_OK)
+        rc = yvex_rocm_status(&state->driver,
+                              state->driver.hipMalloc((void **)&state->device_status, 256u), where,
+                              err);
+    if (rc == YVEX_OK)
+        rc = yvex_rocm_status(&state->driver,
+                              state->driver.hipMemsetAsync(state->device_status, 0, 256u,
+                                                           state->stream),
+                              where, err);
+    if (rc == YVEX_OK)
+        rc = yvex_rocm_status(&state->driver, state->driver.hipStreamSynchronize(state->stream),
+                              where, err);
+    if (rc != YVEX_OK) {
+        yvex_error keep = err ? *err : (yvex_error){0};
+        yvex_error scratch;
+        if (state->device_status) (void)state->driver.hipFree(state->device_status);
+        if (state->timing_start) (void)state->driver.hipEventDestroy(state->timing_start);
+        if (state->timing_stop) (void)state->driver.hipEventDestroy(state->timing_stop);
+        if (state->stream) (void)state->driver.hipStreamDestroy(state->stream);
+        (void)scratch;
+        free(state);
+        free(backend);
+        if (err) *err = keep;
+        return rc;
+    }
+
+    backend->device_info.kind = YVEX_BACKEND_KIND_ROCM;
+    backend->device_info.device_index = state->device_index;
+    if (state->driver.hipDeviceGetName(backend->device_name_storage,
+                                       (int)sizeof(backend->device_name_storage),
+                                       state->device_index) != hipSuccess)
+        yvex_core_text_copy(backend->device_name_storage, sizeof(backend->device_name_storage),
+                            "rocm");
+    backend->device_info.name = backend->device_name_storage;
+    if (state->driver.hipDeviceGetAttribute(&value, hipDeviceAttributeComputeCapabilityMajor,
+                                            state->device_index) == hipSuccess)
+        backend->device_info.compute_capability_major = value;
+    if (state->driver.hipDeviceGetAttribute(&value, hipDeviceAttributeComputeCapabilityMinor,
+                                            state->device_index) == hipSuccess)
+        backend->device_info.compute_capability_minor = value;
+    if (state->driver.hipDeviceGetAttribute(&value, hipDeviceAttributeMultiprocessorCount,
+                                            state->device_index) == hipSuccess)
+        state->compute_units = value;
+    if (state->driver.hipDeviceTotalMem(&total, state->device_index) == hipSuccess) {
+        backend->device_info.global_memory_bytes = total;
+        backend->device_info.total_memory_bytes = total;
+    }
+    backend->device_info.unified_addressing = 1;
+
+    backend->status = YVEX_BACKEND_STATUS_CONTEXT_READY;
+    yvex_error_clear(&admit);
+    if (yvex_rocm_kernel_bundle_admit(backend, &admit) == YVEX_OK)
+        backend->status = YVEX_BACKEND_STATUS_READY;
+    else if (!state->kernel_bundle_rejection[0])
+        yvex_core_text_copy(state->kernel_bundle_rejection,
+                            sizeof(state->kernel_bundle_rejection), admit.message);
+    *out = backend;
+    yvex_error_clear(err);
+    return YVEX_OK;
+}
+
+/* ------------------------------------------------------ NEW SURFACE bits ---- */
+
+int yvex_backend_rocm_completion_mode_set(yvex_backend *backend, yvex_rocm_completion_mode mode,
+                                          yvex_error *err)
+{
+    yvex_rocm_backend_state *state = yvex_rocm_state(backend);
+    int rc;
+    if (!state || (mode != YVEX_ROCM_COMPLETION_IMMEDIATE && mode != YVEX_ROCM_COMPLETION_DEFERRED))
+        return refuse(err, YVEX_ERR_INVALID_ARG, "rocm.completion_mode",
+                      "ROCm backend and a known completion mode are required");
+    rc = backend_dispatch_admit(backend, "rocm.completion_mode", err);
+    if (rc != YVEX_OK) return rc;
+    if (state->status_dirty) {
+        rc = yvex_rocm_status_check(backend, "rocm.completion_mode", NULL, err);
+        if (rc != YVEX_OK) return rc;
+    }
+    state->completion_mode = mode;
+    yvex_error_clear(err);
+    return YVEX_OK;
+}
+
+int yvex_backend_rocm_timing_begin(yvex_backend *backend, yvex_error *err)
+{
+    yvex_rocm_backend_state *state = yvex_rocm_state(backend);
+    int rc;
+    if (!state) return refuse(err, YVEX_ERR_INVALID_ARG, "rocm.timing", "ROCm backend is required");
+    rc = backend_dispatch_admit(backend, "rocm.timing", err);
+    if (rc != YVEX_OK) return rc;
+    rc = yvex_rocm_status(&state->driver,
+                          state->driver.hipEventRecord(state->timing_start, state->stream),
+                          "rocm.timing.begin", err);
+    if (rc == YVEX_OK) state->timing_active = 1;
+    return rc;
+}
+
+int yvex_backend_rocm_timing_end(yvex_backend *backend, double *milliseconds, yvex_error *err)
+{
+    yvex_rocm_backend_state *state = yvex_rocm_state(backend);
+    float elapsed = 0.0f;
+    int rc;
+    if (!state || !milliseconds || !state->timing_active)
+        return refuse(err, YVEX_ERR_STATE, "rocm.timing.end", "timing was not started");
+    rc = yvex_rocm_status(&state->driver,
+                          state->driver.hipEventRecord(state->timing_stop, state->stream),
+                          "rocm.timing.end", err);
+    if (rc == YVEX_OK)
+        rc = yvex_rocm_status(&state->driver, state->driver.hipEventSynchronize(state->timing_stop),
+                              "rocm.timing.end", err);
+    if (rc == YVEX_OK)
+        rc = yvex_rocm_status(&state->driver,
+                              state->driver.hipEventElapsedTime(&elapsed, state->timing_start,
+                                                                state->timing_stop),
+                              "rocm.timing.end", err);
+    state->timing_active = 0;
+    if (rc != YVEX_OK) return rc;
+    *milliseconds = (double)elapsed;
+    yvex_error_clear(err);
+    return YVEX_OK;
+}
+
+extern const char yvex_rocm_bundle_architecture[];
+
+int yvex_backend_rocm_report_get(const yvex_backend *backend, yvex_backend_rocm_report *out,
+                                 yvex_error *err)
+{
+    yvex_rocm_backend_state *state = yvex_rocm_state(backend);
+    unsigned int f;
+    if (!state || !out)
+        return refuse(err, YVEX_ERR_INVALID_ARG, "rocm.report", "ROCm backend and out are required");
+    memset(out, 0, sizeof(*out));
+    out->driver_loaded = state->driver.library != NULL;
+    out->device_ready = state->stream != NULL;
+    out->bundle_built = yvex_rocm_bundle_image_count() != 0u;
+    out->bundle_admitted = state->kernel_bundle_state == YVEX_ROCM_KERNEL_BUNDLE_ADMITTED;
+    out->image_count = yvex_rocm_bundle_image_count();
+    for (f = 0u; f < YVEX_ROCM_FN_COUNT; ++f) out->function_count += state->functions[f] != NULL;
+    yvex_core_text_copy(out->architecture, sizeof(out->architecture), yvex_rocm_bundle_architecture);
+    yvex_core_text_copy(out->device_name, sizeof(out->device_name), backend->device_name_storage);
+    yvex_core_text_copy(out->driver_library, sizeof(out->driver_library),
+                        state->driver.library_name);
+    yvex_core_text_copy(out->rejection, sizeof(out->rejection), state->kernel_bundle_rejection);
+    yvex_error_clear(err);
+    return YVEX_OK;
+}

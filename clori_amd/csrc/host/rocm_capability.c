@@ -1,0 +1,420 @@
+/* Kernel-bundle admission, capability projection and fail-closed launch/synchronise
+ * for the ROCm arm.  The rules are those of src/backend/cuda/capability.c in the
+ * reference: nothing is published before every image loaded and every required symbol
+ * resolved (all or nothing); an absent bundle leaves the backend CONTEXT_READY with
+ * tensor traffic only; a launch failure fails that variant; a synchronise or cleanup
+ * failure fails the whole backend.  Test-only fault injection uses
+ * YVEX_TEST_ROCM_BUNDLE_FAILURE (module | symbol | <function name>),
+ * YVEX_TEST_ROCM_LAUNCH_FAILURE, YVEX_TEST_ROCM_SYNC_FAILURE (all | <variant name>) and
+ * YVEX_TEST_ROCM_CLEANUP_FAILURE, mirroring the YVEX_TEST_CUDA_* switches. */
+#include "rocm_state.h"
+
+#include <stdlib.h>
+#include <string.h>
+
+typedef struct {
+    const char *name;
+    const unsigned char *begin, *end;
+} yvex_rocm_bundle_image;
+
+/* Generated next to the code objects by the build (bundle_table.c). */
+extern const yvex_rocm_bundle_image yvex_rocm_bundle_images[];
+extern const unsigned int yvex_rocm_bundle_image_total;
+extern const char yvex_rocm_bundle_architecture[];
+
+typedef struct {
+    const char *symbol;
+    yvex_backend_operation_variant variant;
+    yvex_rocm_function_id slot;
+} rocm_kernel_binding;
+
+static const rocm_kernel_binding rocm_kernel_bindings[] = {
+    {"yvex_rocm_attention_f32", YVEX_BACKEND_VARIANT_ATTENTION_CAUSAL_F32,
+     YVEX_ROCM_FN_ATTENTION_F32},
+    {"yvex_rocm_gqa_f32", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_F32, YVEX_ROCM_FN_GQA_F32},
+    {"yvex_rocm_fill_u32", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_F32, YVEX_ROCM_FN_FILL_U32},
+    {"yvex_rocm_decode_paged_bf16", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_PAGED_BF16,
+     YVEX_ROCM_FN_DECODE_PAGED_BF16},
+    {"yvex_rocm_decode_merge", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_PAGED_BF16,
+     YVEX_ROCM_FN_DECODE_MERGE},
+    {"yvex_rocm_decode_rows_bf16", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_BF16,
+     YVEX_ROCM_FN_DECODE_ROWS_BF16},
+};
+#define ROCM_KERNEL_BINDING_COUNT (sizeof(rocm_kernel_bindings) / sizeof(rocm_kernel_bindings[0]))
+
+unsigned int yvex_rocm_bundle_image_count(void) { return yvex_rocm_bundle_image_total; }
+
+static int test_failure_matches(const char *name, yvex_backend_operation_variant variant)
+{
+    const char *value = getenv(name);
+    return value && value[0] != '\0' &&
+           (strcmp(value, "all") == 0 ||
+            strcmp(value, yvex_backend_operation_variant_name(variant)) == 0);
+}
+
+static void capability_fail(yvex_backend *backend, yvex_backend_operation_variant variant,
+                            yvex_backend_capability_reason reason)
+{
+    yvex_rocm_backend_state *state = yvex_rocm_state(backend);
+    if (!state || (int)variant < 0 || variant >= YVEX_BACKEND_VARIANT_ROCM_END) return;
+    state->variant_failures[variant] = reason;
+    if (reason == YVEX_BACKEND_CAPABILITY_REASON_SYNCHRONIZATION_FAILED ||
+        reason == YVEX_BACKEND_CAPABILITY_REASON_CLEANUP_FAILED) {
+        state->backend_failure_reason = reason;
+        backend->status = YVEX_BACKEND_STATUS_FAILED;
+    }
+}
+
+static void bundle_reject(yvex_rocm_backend_state *state, yvex_backend_capability_reason reason,
+                          yvex_backend_operation_variant variant, const yvex_error *err)
+{
+    state->kernel_bundle_state = YVEX_ROCM_KERNEL_BUNDLE_REJECTED;
+    state->kernel_bundle_reason = reason;
+    state->kernel_bundle_failure_variant = variant;
+    yvex_core_text_copy(state->kernel_bundle_rejection, sizeof(state->kernel_bundle_rejection),
+                        err ? err->message : "");
+}
+
+/* src/backend/cuda/capability.c:511-620: handles are committed only after every image
+ * loaded and every symbol resolved; otherwise everything loaded so far is unloaded. */
+int yvex_rocm_kernel_bundle_admit(yvex_backend *backend, yvex_error *err)
+{
+    yvex_rocm_backend_state *state = yvex_rocm_state(backend);
+    hipModule_t modules[YVEX_ROCM_MODULE_MAX] = {0};
+    hipFunction_t functions[YVEX_ROCM_FN_COUNT] = {0};
+    const char *injected = getenv("YVEX_TEST_ROCM_BUNDLE_FAILURE");
+    unsigned int loaded = 0u, index;
+    size_t b;
+    int rc = YVEX_OK;
+    if (!backend || !state || !state->stream) {
+        yvex_error_set(err, YVEX_ERR_STATE, "rocm.kernels.admit",
+                       "ROCm context is required for kernel admission");
+        return YVEX_ERR_STATE;
+    }
+    rc = backend_dispatch_admit(backend, "rocm.kernels.admit", err);
+    if (rc != YVEX_OK) return rc;
+    if (state->module_count) {
+        if (state->kernel_bundle_state == YVEX_ROCM_KERNEL_BUNDLE_ADMITTED) {
+            yvex_error_clear(err);
+            return YVEX_OK;
+        }
+        yvex_error_set(err, YVEX_ERR_STATE, "rocm.kernels.admit",
+                       "retained ROCm module ownership requires checked cleanup");
+        return YVEX_ERR_STATE;
+    }
+    memset(state->functions, 0, sizeof(state->functions));
+    state->kernel_bundle_state = YVEX_ROCM_KERNEL_BUNDLE_ABSENT;
+    state->kernel_bundle_reason = YVEX_BACKEND_CAPABILITY_REASON_KERNEL_BUNDLE_ABSENT;
+    state->kernel_bundle_failure_variant = YVEX_BACKEND_VARIANT_COUNT;
+    state->kernel_bundle_rejection[0] = '\0';
+    if (!yvex_rocm_bundle_image_total) {
+        yvex_error_set(err, YVEX_ERR_UNSUPPORTED, "rocm.kernels.admit",
+                       "gfx950 kernel bundle was not built");
+        return YVEX_ERR_UNSUPPORTED;
+    }
+    if (yvex_rocm_bundle_image_total > YVEX_ROCM_MODULE_MAX) {
+        yvex_error_set(err, YVEX_ERR_BOUNDS, "rocm.kernels.admit",
+                       "kernel bundle holds more images than the module table");
+        bundle_reject(state, YVEX_BACKEND_CAPABILITY_REASON_KERNEL_BUNDLE_REJECTED,
+                      YVEX_BACKEND_VARIANT_COUNT, err);
+        return YVEX_ERR_BOUNDS;
+    }
+    for (loaded = 0u; loaded < yvex_rocm_bundle_image_total; ++loaded) {
+        const yvex_rocm_bundle_image *image = &yvex_rocm_bundle_images[loaded];
+        if (injected && strcmp(injected, "module") == 0) {
+            yvex_error_set(err, YVEX_ERR_BACKEND, "rocm.kernels.load",
+                           "injected ROCm module admission failure");
+            rc = YVEX_ERR_BACKEND;
+        } else if (image->end <= image->begin) {
+            yvex_error_setf(err, YVEX_ERR_FORMAT, "rocm.kernels.load", "empty code object: %s",
+                            image->name);
+            rc = YVEX_ERR_FORMAT;
+        } else {
+            rc = yvex_rocm_status(&state->driver,
+                                  state->driver.hipModuleLoadData(&modules[loaded], image->begin),
+                                  "rocm.kernels.load", err);
+        }
+        if (rc != YVEX_OK) {
+            bundle_reject(state, YVEX_BACKEND_CAPABILITY_REASON_KERNEL_BUNDLE_REJECTED,
+                          YVEX_BACKEND_VARIANT_COUNT, err);
+            goto reject;
+        }
+    }
+    for (b = 0; b < ROCM_KERNEL_BINDING_COUNT; ++b) {
+        const rocm_kernel_binding *binding = &rocm_kernel_bindings[b];
+        hipFunction_t function = NULL;
+        if (!(injected && (strcmp(injected, "symbol") == 0 ||
+                           strcmp(injected, binding->symbol) == 0))) {
+            for (index = 0u; index < loaded && !function; ++index)
+                if (state->driver.hipModuleGetFunction(&function, modules[index],
+                                                       binding->symbol) != hipSuccess)
+                    function = NULL;
+        }
+        if (!function) {
+            yvex_error_setf(err, YVEX_ERR_BACKEND, "rocm.kernels.resolve",
+                            "required ROCm function unavailable: %s", binding->symbol);
+            rc = YVEX_ERR_BACKEND;
+            bundle_reject(state, YVEX_BACKEND_CAPABILITY_REASON_FUNCTION_MISSING,
+                          binding->variant, err);
+            goto reject;
+        }
+        functions[binding->slot] = function;
+    }
+    memcpy(state->modules, modules, loaded * sizeof(modules[0]));
+    state->module_count = loaded;
+    memcpy(state->functions, functions, sizeof(functions));
+    state->kernel_bundle_state = YVEX_ROCM_KERNEL_BUNDLE_ADMITTED;
+    state->kernel_bundle_reason = YVEX_BACKEND_CAPABILITY_REASON_NONE;
+    yvex_error_clear(err);
+    return YVEX_OK;
+reject:
+    for (index = 0u; index < loaded; ++index)
+        if (modules[index]) (void)state->driver.hipModuleUnload(modules[index]);
+    return rc;
+}
+
+/* src/backend/cuda/capability.c:622-657 */
+int yvex_rocm_kernel_bundle_close(yvex_backend *backend, yvex_error *err)
+{
+    yvex_rocm_backend_state *state = yvex_rocm_state(backend);
+    unsigned int index;
+    int rc = YVEX_OK;
+    if (!state) {
+        yvex_error_clear(err);
+        return YVEX_OK;
+    }
+    for (index = 0u; index < state->module_count; ++index) {
+        int unload_rc;
+        if (!state->modules[index]) continue;
+        if (getenv("YVEX_TEST_ROCM_CLEANUP_FAILURE")) {
+            yvex_error_set(err, YVEX_ERR_BACKEND, "rocm.kernels.unload",
+                           "injected ROCm module cleanup failure");
+            unload_rc = YVEX_ERR_BACKEND;
+        } else {
+            unload_rc = yvex_rocm_status(&state->driver,
+                                         state->driver.hipModuleUnload(state->modules[index]),
+                                         "rocm.kernels.unload", err);
+        }
+        if (unload_rc == YVEX_OK)
+            state->modules[index] = NULL;
+        else
+            rc = unload_rc;
+    }
+    if (rc != YVEX_OK) {
+        state->kernel_bundle_reason = YVEX_BACKEND_CAPABILITY_REASON_CLEANUP_FAILED;
+        state->backend_failure_reason = YVEX_BACKEND_CAPABILITY_REASON_CLEANUP_FAILED;
+        backend->status = YVEX_BACKEND_STATUS_FAILED;
+        return rc;
+    }
+    state->module_count = 0u;
+    memset(state->functions, 0, sizeof(state->functions));
+    state->kernel_bundle_state = YVEX_ROCM_KERNEL_BUNDLE_ABSENT;
+    state->kernel_bundle_reason = YVEX_BACKEND_CAPABILITY_REASON_KERNEL_BUNDLE_ABSENT;
+    yvex_error_clear(err);
+    return YVEX_OK;
+}
+
+static int variant_functions_present(const yvex_rocm_backend_state *state,
+                                     yvex_backend_operation_variant variant, int *bound)
+{
+    size_t b;
+    *bound = 0;
+    if (variant == YVEX_BACKEND_VARIANT_ATTENTION_NONCAUSAL_F32)
+        variant = YVEX_BACKEND_VARIANT_ATTENTION_CAUSAL_F32;
+    for (b = 0; b < ROCM_KERNEL_BINDING_COUNT; ++b) {
+        if (rocm_kernel_bindings[b].variant != variant) continue;
+        *bound = 1;
+        if (!state->functions[rocm_kernel_bindings[b].slot]) return 0;
+    }
+    return *bound;
+}
+
+static int publish(yvex_backend_capability_result *out, yvex_backend_capability_state state,
+                   yvex_backend_capability_reason reason, int function_available,
+                   yvex_error *err)
+{
+    out->state = state;
+    out->reason = reason;
+    out->function_available = function_available;
+    yvex_error_clear(err);
+    return YVEX_OK;
+}
+
+/* src/backend/cuda/capability.c:659-722 */
+int yvex_rocm_query_capability(const yvex_backend *backend, yvex_backend_operation_variant variant,
+                               yvex_backend_capability_result *out, yvex_error *err)
+{
+    yvex_rocm_backend_state *state = yvex_rocm_state(backend);
+    int bound, present;
+    if (!backend || !state || !out) {
+        yvex_error_set(err, YVEX_ERR_INVALID_ARG, "rocm.query_capability",
+                       "backend, ROCm state, and out are required");
+        return YVEX_ERR_INVALID_ARG;
+    }
+    out->context_available = state->stream != NULL;
+    out->kernel_bundle_available = state->kernel_bundle_state == YVEX_ROCM_KERNEL_BUNDLE_ADMITTED;
+    if (!state->stream)
+        return publish(out, YVEX_BACKEND_CAPABILITY_UNSUPPORTED,
+                       YVEX_BACKEND_CAPABILITY_REASON_CONTEXT_UNAVAILABLE, 0, err);
+    if (backend->status == YVEX_BACKEND_STATUS_FAILED &&
+        state->backend_failure_reason != YVEX_BACKEND_CAPABILITY_REASON_NONE)
+        return publish(out, YVEX_BACKEND_CAPABILITY_FAILED, state->backend_failure_reason, 0, err);
+    if (state->variant_failures[variant] != YVEX_BACKEND_CAPABILITY_REASON_NONE)
+        return publish(out, YVEX_BACKEND_CAPABILITY_FAILED, state->variant_failures[variant], 0,
+                       err);
+    if (variant >= YVEX_BACKEND_VARIANT_TENSOR_ALLOC && variant <= YVEX_BACKEND_VARIANT_TENSOR_COPY)
+        return publish(out, YVEX_BACKEND_CAPABILITY_SUPPORTED, YVEX_BACKEND_CAPABILITY_REASON_NONE,
+                       1, err);
+    if (state->kernel_bundle_state == YVEX_ROCM_KERNEL_BUNDLE_ABSENT)
+        return publish(out, YVEX_BACKEND_CAPABILITY_UNSUPPORTED,
+                       YVEX_BACKEND_CAPABILITY_REASON_KERNEL_BUNDLE_ABSENT, 0, err);
+    if (state->kernel_bundle_state == YVEX_ROCM_KERNEL_BUNDLE_REJECTED) {
+        yvex_backend_capability_reason reason = state->kernel_bundle_reason;
+        if (reason == YVEX_BACKEND_CAPABILITY_REASON_FUNCTION_MISSING &&
+            state->kernel_bundle_failure_variant != variant)
+            reason = YVEX_BACKEND_CAPABILITY_REASON_KERNEL_BUNDLE_REJECTED;
+        return publish(out, YVEX_BACKEND_CAPABILITY_FAILED, reason, 0, err);
+    }
+    present = variant_functions_present(state, variant, &bound);
+    if (!bound)
+        /* a variant this backend has no kernel for (embed, matmul, MoE, ...) */
+        return publish(out, YVEX_BACKEND_CAPABILITY_UNSUPPORTED,
+                       YVEX_BACKEND_CAPABILITY_REASON_VARIANT_UNSUPPORTED, 0, err);
+    return publish(out,
+                   present ? YVEX_BACKEND_CAPABILITY_SUPPORTED : YVEX_BACKEND_CAPABILITY_FAILED,
+                   present ? YVEX_BACKEND_CAPABILITY_REASON_NONE
+                           : YVEX_BACKEND_CAPABILITY_REASON_FUNCTION_MISSING,
+                   present, err);
+}
+
+/* src/backend/cuda/capability.c:724-748 */
+int yvex_rocm_require_capability(yvex_backend *backend, yvex_backend_operation_variant variant,
+                                 const char *where, yvex_error *err)
+{
+    yvex_backend_capability_result result;
+    int rc = yvex_backend_query_capability(backend, variant, &result, err);
+    if (rc != YVEX_OK) return rc;
+    if (result.state == YVEX_BACKEND_CAPABILITY_SUPPORTED) return YVEX_OK;
+    rc = result.state == YVEX_BACKEND_CAPABILITY_FAILED ? YVEX_ERR_BACKEND : YVEX_ERR_UNSUPPORTED;
+    yvex_error_setf(err, rc, where ? where : "rocm.require_capability", "%s refused: %s",
+                    yvex_backend_operation_variant_name(variant),
+                    yvex_backend_capability_reason_name(result.reason));
+    return rc;
+}
+
+/* src/backend/cuda/capability.c:750-791 */
+int yvex_rocm_launch(yvex_backend *backend, yvex_rocm_function_id function,
+                     yvex_backend_operation_variant variant, unsigned int grid_x,
+                     unsigned int grid_y, unsigned int grid_z, unsigned int block,
+                     unsigned int lds_bytes, void *params, const char *where, yvex_error *err)
+{
+    yvex_rocm_backend_state *state = yvex_rocm_state(backend);
+    void *arguments[1];
+    int rc = yvex_rocm_require_capability(backend, variant, where, err);
+    if (rc != YVEX_OK) return rc;
+    if (!state || function >= YVEX_ROCM_FN_COUNT || !state->functions[function]) {
+        capability_fail(backend, variant, YVEX_BACKEND_CAPABILITY_REASON_FUNCTION_MISSING);
+        yvex_error_set(err, YVEX_ERR_BACKEND, where, "admitted ROCm function handle is missing");
+        return YVEX_ERR_BACKEND;
+    }
+    if (!grid_x || !grid_y || !grid_z || !block || block > 1024u) {
+        yvex_error_set(err, YVEX_ERR_BOUNDS, where, "launch geometry is out of range");
+        return YVEX_ERR_BOUNDS;
+    }
+    if (test_failure_matches("YVEX_TEST_ROCM_LAUNCH_FAILURE", variant)) {
+        capability_fail(backend, variant, YVEX_BACKEND_CAPABILITY_REASON_LAUNCH_FAILED);
+        yvex_error_set(err, YVEX_ERR_BACKEND, where, "injected ROCm launch failure");
+        return YVEX_ERR_BACKEND;
+    }
+    arguments[0] = params;
+    rc = yvex_rocm_status(&state->driver,
+                          state->driver.hipModuleLaunchKernel(state->functions[function], grid_x,
+                                                              grid_y, grid_z, block, 1u, 1u,
+                                                              lds_bytes, state->stream, arguments,
+                                                              NULL),
+                          where, err);
+    if (rc != YVEX_OK) capability_fail(backend, variant, YVEX_BACKEND_CAPABILITY_REASON_LAUNCH_FAILED);
+    return rc;
+}
+
+/* src/backend/cuda/capability.c:793-830 */
+int yvex_rocm_synchronize(yvex_backend *backend, yvex_backend_operation_variant variant,
+                          const char *where, yvex_error *err)
+{
+    yvex_rocm_backend_state *state = yvex_rocm_state(backend);
+    int rc = backend_dispatch_admit(backend, where, err);
+    if (rc != YVEX_OK) return rc;
+    if (!state) {
+        yvex_error_set(err, YVEX_ERR_STATE, where, "ROCm backend state is missing");
+        return YVEX_ERR_STATE;
+    }
+    if (test_failure_matches("YVEX_TEST_ROCM_SYNC_FAILURE", variant)) {
+        capability_fail(backend, variant, YVEX_BACKEND_CAPABILITY_REASON_SYNCHRONIZATION_FAILED);
+        yvex_error_set(err, YVEX_ERR_BACKEND, where, "injected ROCm synchronization failure");
+        return YVEX_ERR_BACKEND;
+    }
+    rc = yvex_rocm_status(&state->driver, state->driver.hipStreamSynchronize(state->stream), where,
+                          err);
+    if (rc != YVEX_OK)
+        capability_fail(backend, variant, YVEX_BACKEND_CAPABILITY_REASON_SYNCHRONIZATION_FAILED);
+    return rc;
+}
+
+/* Reads the device status word (the stream is synchronised by the copy's own wait),
+ * clears it when set, and maps it like src/backend/cuda/transformer.c:648-660. */
+int yvex_rocm_status_check(yvex_backend *backend, const char *where,
+                           yvex_backend_operation_facts *facts, yvex_error *err)
+{
+    yvex_rocm_backend_state *state = yvex_rocm_state(backend);
+    int32_t host_status = 0;
+    int rc;
+    rc = yvex_rocm_status(&state->driver,
+                          state->driver.hipMemcpyAsync(&host_status, state->device_status,
+                                                       sizeof(host_status), hipMemcpyDeviceToHost,
+                                                       state->stream),
+                          where, err);
+    if (rc == YVEX_OK)
+        rc = yvex_rocm_synchronize(backend, YVEX_BACKEND_VARIANT_TENSOR_READ, where, err);
+    if (rc != YVEX_OK) return rc;
+    state->status_dirty = 0;
+    backend->stats.d2h_bytes += sizeof(host_status);
+    if (facts) {
+        facts->download_count += 1ull;
+        facts->d2h_bytes += sizeof(host_status);
+        facts->device_synchronizations += 1ull;
+    }
+    if (!host_status) {
+        yvex_error_clear(err);
+        return YVEX_OK;
+    }
+    rc = yvex_rocm_status(&state->driver,
+                          state->driver.hipMemsetAsync(state->device_status, 0,
+                                                       sizeof(host_status), state->stream),
+                          where, err);
+    if (rc != YVEX_OK) return rc;
+    switch (host_status) {
+    case 2:
+        yvex_error_set(err, YVEX_ERR_BOUNDS, where,
+                       "attention kernel refused a page id or context length out of range");
+        return YVEX_ERR_BOUNDS;
+    case 3:
+        yvex_error_set(err, YVEX_ERR_STATE, where, "attention softmax sum is zero");
+        return YVEX_ERR_STATE;
+    default:
+        yvex_error_set(err, YVEX_ERR_FORMAT, where, "attention produced invalid numerics");
+        return YVEX_ERR_FORMAT;
+    }
+}
+
+int yvex_rocm_complete(yvex_backend *backend, yvex_backend_operation_variant variant,
+                       const char *where, yvex_backend_operation_facts *facts, yvex_error *err)
+{
+    yvex_rocm_backend_state *state = yvex_rocm_state(backend);
+    (void)variant;
+    if (state->completion_mode == YVEX_ROCM_COMPLETION_DEFERRED) {
+        state->status_dirty = 1;
+        yvex_error_clear(err);
+        return YVEX_OK;
+    }
+    return yvex_rocm_status_check(backend, where, facts, err);
+}

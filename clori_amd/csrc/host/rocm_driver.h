@@ -1,0 +1,40 @@
+/* The thin C-ABI layer between the C11 host and HIP: a table of runtime entry points
+ * resolved with dlopen/dlsym, the way the reference binds the CUDA driver
+ * (src/backend/cuda/private.h:102-206, src/backend/cuda/info.c:47-49).  Because the
+ * runtime is a struct of function pointers a test can substitute another library
+ * (YVEX_TEST_ROCM_DRIVER_LIBRARY) and exercise admission, bookkeeping and failure
+ * transitions of the host code on a machine with no GPU. */
+#ifndef YVEX_ROCM_DRIVER_H
+#define YVEX_ROCM_DRIVER_H
+
+#ifndef __HIP_PLATFORM_AMD__
+#define __HIP_PLATFORM_AMD__ 1
+#endif
+#include <hip/hip_runtime_api.h>
+
+#include "yvex_rocm.h"
+
+#define YVEX_ROCM_DRIVER_ENTRIES(X)                                                      \
+    X(hipInit) X(hipGetDeviceCount) X(hipSetDevice) X(hipDeviceGetName)                  \
+    X(hipDeviceGetAttribute) X(hipDeviceTotalMem) X(hipMemGetInfo) X(hipGetErrorString)  \
+    X(hipStreamCreate) X(hipStreamDestroy) X(hipStreamSynchronize) X(hipMalloc) X(hipFree) \
+    X(hipMemcpyAsync) X(hipMemsetAsync) X(hipModuleLoadData) X(hipModuleUnload)          \
+    X(hipModuleGetFunction) X(hipModuleLaunchKernel) X(hipEventCreate) X(hipEventDestroy) \
+    X(hipEventRecord) X(hipEventSynchronize) X(hipEventElapsedTime)
+
+typedef struct yvex_rocm_driver {
+    void *library;
+    char library_name[256];
+#define X(name) __typeof__(&name) name;
+    YVEX_ROCM_DRIVER_ENTRIES(X)
+#undef X
+} yvex_rocm_driver;
+
+/* Loads the runtime library and resolves every entry or none (YVEX_ERR_UNSUPPORTED). */
+int yvex_rocm_driver_load(yvex_rocm_driver *driver, yvex_error *err);
+void yvex_rocm_driver_unload(yvex_rocm_driver *driver);
+/* Maps a hipError_t to YVEX_OK / YVEX_ERR_BACKEND with the runtime's message. */
+int yvex_rocm_status(const yvex_rocm_driver *driver, hipError_t code, const char *where,
+                     yvex_error *err);
+
+#endif /* YVEX_ROCM_DRIVER_H */

@@ -1,0 +1,102 @@
+/* State of one ROCm backend instance, shared by the arm's translation units. */
+#ifndef YVEX_ROCM_STATE_H
+#define YVEX_ROCM_STATE_H
+
+#include "private.h"
+#include "rocm_driver.h"
+
+#define YVEX_ROCM_MODULE_MAX 8u
+
+/* Every device function of the bundle.  The order indexes yvex_rocm_backend_state.functions
+ * and the binding table in rocm_capability.c. */
+typedef enum {
+    YVEX_ROCM_FN_ATTENTION_F32 = 0,
+    YVEX_ROCM_FN_GQA_F32,
+    YVEX_ROCM_FN_FILL_U32,
+    YVEX_ROCM_FN_DECODE_PAGED_BF16,
+    YVEX_ROCM_FN_DECODE_ROWS_BF16,
+    YVEX_ROCM_FN_DECODE_MERGE,
+    YVEX_ROCM_FN_DECODE_PAGED_Q8_0,
+    YVEX_ROCM_FN_PREFILL_BF16,
+    YVEX_ROCM_FN_MLA_DECODE_BF16,
+    YVEX_ROCM_FN_COUNT
+} yvex_rocm_function_id;
+
+typedef enum {
+    YVEX_ROCM_KERNEL_BUNDLE_ABSENT = 0,
+    YVEX_ROCM_KERNEL_BUNDLE_ADMITTED,
+    YVEX_ROCM_KERNEL_BUNDLE_REJECTED
+} yvex_rocm_kernel_bundle_state;
+
+typedef struct yvex_rocm_backend_state {
+    yvex_rocm_driver driver;
+    int device_index;
+    int compute_units;
+    hipStream_t stream;
+    hipEvent_t timing_start, timing_stop;
+    int timing_active;
+    hipModule_t modules[YVEX_ROCM_MODULE_MAX];
+    unsigned int module_count;
+    hipFunction_t functions[YVEX_ROCM_FN_COUNT];
+    yvex_rocm_kernel_bundle_state kernel_bundle_state;
+    yvex_backend_capability_reason kernel_bundle_reason;
+    yvex_backend_operation_variant kernel_bundle_failure_variant;
+    char kernel_bundle_rejection[YVEX_ERROR_MESSAGE_CAP];
+    /* per-variant and whole-backend failure reasons (src/backend/cuda/capability.c:447-461) */
+    yvex_backend_capability_reason variant_failures[YVEX_BACKEND_VARIANT_ROCM_END];
+    yvex_backend_capability_reason backend_failure_reason;
+    int32_t *device_status; /* one status word, zero between operations */
+    int status_dirty;       /* deferred mode: launches since the last check */
+    yvex_rocm_completion_mode completion_mode;
+    unsigned long long live_tensors;
+} yvex_rocm_backend_state;
+
+static inline yvex_rocm_backend_state *yvex_rocm_state(const yvex_backend *backend)
+{
+    return backend && backend->kind == YVEX_BACKEND_KIND_ROCM
+               ? (yvex_rocm_backend_state *)backend->impl
+               : NULL;
+}
+
+/* rocm_capability.c */
+int yvex_rocm_kernel_bundle_admit(yvex_backend *backend, yvex_error *err);
+int yvex_rocm_kernel_bundle_close(yvex_backend *backend, yvex_error *err);
+int yvex_rocm_query_capability(const yvex_backend *backend, yvex_backend_operation_variant variant,
+                               yvex_backend_capability_result *out, yvex_error *err);
+int yvex_rocm_require_capability(yvex_backend *backend, yvex_backend_operation_variant variant,
+                                 const char *where, yvex_error *err);
+unsigned int yvex_rocm_bundle_image_count(void);
+/* One kernel launch on the backend stream; params is the kernel's single argument block. */
+int yvex_rocm_launch(yvex_backend *backend, yvex_rocm_function_id function,
+                     yvex_backend_operation_variant variant, unsigned int grid_x,
+                     unsigned int grid_y, unsigned int grid_z, unsigned int block,
+                     unsigned int lds_bytes, void *params, const char *where, yvex_error *err);
+/* Stream synchronise; a failure moves the whole backend to FAILED. */
+int yvex_rocm_synchronize(yvex_backend *backend, yvex_backend_operation_variant variant,
+                          const char *where, yvex_error *err);
+/* Ends an operation: IMMEDIATE mode synchronises, reads the device status word and
+ * maps it to a status; DEFERRED mode only marks the word as pending. */
+int yvex_rocm_complete(yvex_backend *backend, yvex_backend_operation_variant variant,
+                       const char *where, yvex_backend_operation_facts *facts, yvex_error *err);
+int yvex_rocm_status_check(yvex_backend *backend, const char *where,
+                           yvex_backend_operation_facts *facts, yvex_error *err);
+
+/* rocm_backend.c */
+int yvex_rocm_temporary_acquire(yvex_backend *backend, unsigned long long bytes, void **address,
+                                int *owned, const char *where, yvex_error *err);
+int yvex_rocm_temporary_release(yvex_backend *backend, void *address, unsigned long long bytes,
+                                int owned, yvex_error *err);
+
+/* rocm_attention.c */
+int yvex_rocm_op_attention(yvex_backend *backend, const yvex_device_tensor *query,
+                           const yvex_device_tensor *keys, const yvex_device_tensor *values,
+                           unsigned long long seq_len, unsigned long long position, float scale,
+                           int causal, yvex_device_tensor *score_scratch,
+                           yvex_device_tensor *probability_scratch, yvex_device_tensor *out,
+                           yvex_error *err);
+const yvex_backend_transformer_operations *yvex_rocm_transformer_operations(
+    const yvex_backend *backend);
+const yvex_backend_rocm_attention_operations *yvex_rocm_attention_operations(
+    const yvex_backend *backend);
+
+#endif /* YVEX_ROCM_STATE_H */

@@ -1,0 +1,99 @@
+/* Kernel argument blocks shared by the C11 host and the gfx950 device code.  Each
+ * kernel takes exactly one of these structs by value.  Only fixed-width scalars and
+ * pointers, ordered so that no implicit padding exists on either compiler. */
+#ifndef YVEX_ROCM_KERNEL_PARAMS_H
+#define YVEX_ROCM_KERNEL_PARAMS_H
+
+#include <stdint.h>
+
+/* Device status word values, as in the reference kernels (atomicCAS(status,0,1) for a
+ * numeric failure, atomicCAS(status,0,2) for a contract violation). */
+enum {
+    YVEX_ROCM_DEVICE_OK = 0,
+    YVEX_ROCM_DEVICE_NUMERIC = 1,
+    YVEX_ROCM_DEVICE_CONTRACT = 2,
+    YVEX_ROCM_DEVICE_SOFTMAX_ZERO = 3
+};
+
+typedef struct {
+    const float *q, *k, *v;
+    float *score, *prob, *out;
+    int32_t *status;
+    uint64_t seq_len, position, head_dim;
+    float scale;
+    int32_t causal;
+} yvex_rocm_attention_f32_params;
+
+typedef struct {
+    const float *q, *k, *v;
+    float *out;
+    float *lse; /* optional [Tq][Hq] */
+    int32_t *status;
+    uint64_t query_tokens, kv_tokens, query_start, query_heads, kv_heads, head_dim;
+    uint64_t q_stride, k_stride, v_stride;
+    float scale;
+    int32_t causal;
+} yvex_rocm_gqa_f32_params;
+
+typedef struct {
+    uint32_t *data;
+    uint64_t words;
+    uint32_t value;
+    uint32_t reserved;
+} yvex_rocm_fill_params;
+
+/* Split-K decode.  One wave per (chunk, kv head, session).  part_acc is
+ * [sessions][max_chunks][query_heads][head_dim] F32 (unnormalised), part_ml is
+ * [sessions][max_chunks][query_heads][2] F32 = (running max in log2 units, sum). */
+typedef struct {
+    const uint16_t *q;
+    const void *k_pool, *v_pool;
+    const int32_t *page_table; /* NULL for the token-major layout */
+    const int32_t *context;    /* NULL: every session uses fixed_context */
+    float *part_acc, *part_ml;
+    int32_t *status;
+    uint64_t k_token_stride, v_token_stride; /* token-major layout: elements per token */
+    uint32_t sessions, query_heads, kv_heads, head_dim;
+    uint32_t pool_pages, table_stride, chunk_tokens, max_chunks;
+    uint32_t fixed_context, reserved;
+    float scale_log2; /* softmax scale * log2(e) */
+    float reserved_f;
+} yvex_rocm_decode_params;
+
+typedef struct {
+    const float *part_acc, *part_ml;
+    const int32_t *context;
+    uint16_t *out; /* bf16 [sessions][query_heads][head_dim] */
+    float *lse;    /* optional F32 [sessions][query_heads] */
+    int32_t *status;
+    uint32_t sessions, query_heads, head_dim, chunk_tokens, max_chunks, fixed_context;
+} yvex_rocm_decode_merge_params;
+
+/* Causal / full GQA prefill on bf16 token-major tensors. */
+typedef struct {
+    const uint16_t *q, *k, *v;
+    uint16_t *out;
+    float *lse; /* optional F32 [Tq][Hq] */
+    int32_t *status;
+    const uint32_t *tasks; /* [task_count][4]: q head, q tile, first kv tile, end kv tile */
+    uint64_t q_stride, k_stride, v_stride; /* elements per token */
+    uint32_t query_tokens, kv_tokens, query_start, query_heads, kv_heads, head_dim;
+    uint32_t causal, task_count;
+    float scale_log2;
+    float reserved_f;
+} yvex_rocm_prefill_params;
+
+/* Absorbed-latent MLA decode, split over the context. */
+typedef struct {
+    const uint16_t *q;      /* [batch][heads][key_dim] */
+    const uint16_t *pool;   /* [pool_pages][page_tokens][key_dim] */
+    const int32_t *page_table, *context;
+    float *part_acc, *part_ml; /* [batch][max_chunks][heads][value_dim], [..][heads][2] */
+    int32_t *status;
+    uint32_t batch, heads, key_dim, value_dim;
+    uint32_t page_tokens, pool_pages, table_stride, chunk_tokens, max_chunks, reserved;
+    float scale_log2;
+    float reserved_f;
+} yvex_rocm_mla_params;
+
+#endif /* YVEX_ROCM_KERNEL_PARAMS_H */

@@ -1,0 +1,72 @@
+// Small device helpers shared by the gfx950 attention kernels: MFMA operand types,
+// 16-byte global loads, wave64 lane exchange and bf16 conversion.
+#ifndef YVEX_ROCM_KERNELS_MFMA_H
+#define YVEX_ROCM_KERNELS_MFMA_H
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef short short4v __attribute__((ext_vector_type(4)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+#define YVEX_LOG2E 1.4426950408889634f
+#define YVEX_LN2 0.6931471805599453f
+
+__device__ inline u32x4 load_b128(const void *p) { return *reinterpret_cast<const u32x4 *>(p); }
+__device__ inline u32x2 load_b64(const void *p) { return *reinterpret_cast<const u32x2 *>(p); }
+
+__device__ inline bf16x8 as_bf16x8(u32x4 v) { return __builtin_bit_cast(bf16x8, v); }
+__device__ inline short4v as_short4(u32x2 v) { return __builtin_bit_cast(short4v, v); }
+
+// S(16x16) += A(16x32) * B(32x16): lane l supplies A[l%16][8*(l/16)..+7] and
+// B[8*(l/16)..+7][l%16]; the result lane l holds C[4*(l/16)+i][l%16], i = 0..3.
+__device__ inline floatx4 mfma_16x16x32(bf16x8 a, bf16x8 b, floatx4 c)
+{
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+
+// C(16x16) += A(16x16) * B(16x16): lane l supplies A[l%16][4*(l/16)..+3] and
+// B[4*(l/16)..+3][l%16].
+__device__ inline floatx4 mfma_16x16x16(short4v a, short4v b, floatx4 c)
+{
+    return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, b, c, 0, 0, 0);
+}
+
+// C(32x32) += A(32x16) * B(16x32): lane l supplies A[l%32][8*(l/32)..+7] and
+// B[8*(l/32)..+7][l%32]; the result lane l holds C[8*(i/4) + 4*(l/32) + i%4][l%32].
+__device__ inline floatx16 mfma_32x32x16(bf16x8 a, bf16x8 b, floatx16 c)
+{
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+}
+
+__device__ inline float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ inline float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
+
+__device__ inline float xor_lanes(float v, int mask) { return __shfl_xor(v, mask, 64); }
+
+// Round-to-nearest-even narrowing with the quiet-NaN policy of the reference codec
+// (src/gguf/quant_scalar.c:131-143).
+__device__ inline uint16_t bf16_bits(float v)
+{
+    uint32_t u = __builtin_bit_cast(uint32_t, v);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);
+    return (uint16_t)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
+}
+
+__device__ inline uint32_t pack_bf16x2(float lo, float hi)
+{
+    return (uint32_t)bf16_bits(lo) | ((uint32_t)bf16_bits(hi) << 16);
+}
+
+__device__ inline float bf16_to_f32(uint16_t b)
+{
+    return __builtin_bit_cast(float, (uint32_t)b << 16);
+}
+
+#endif  // YVEX_ROCM_KERNELS_MFMA_H

@@ -1,0 +1,488 @@
+/*
+ * C ABI of the MI355X (gfx950) attention backend for YVEX.
+ *
+ * Every type and function below either mirrors one interface of the reference
+ * tree (cited as path:line, relative to yailabs/clori) with the same name,
+ * argument meaning and error behaviour, or is marked NEW SURFACE where the
+ * reference has no counterpart (paged KV, Q8_0 KV, LSE output, absorbed MLA).
+ * Only plain C types cross this boundary: opaque handles, integers, pointers.
+ *
+ * The library talks to the HIP runtime through a dlopen'ed function table and
+ * loads its gfx950 code objects from an embedded bundle; it never computes
+ * attention on the host and has no CPU fallback: when the device, the bundle or
+ * an exact implementation is unavailable every operation refuses.
+ */
+#ifndef YVEX_ROCM_H
+#define YVEX_ROCM_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- status and error: include/yvex/core.h:13-48 ------------------------ */
+typedef enum {
+    YVEX_OK = 0,
+    YVEX_ERR = -1,
+    YVEX_ERR_NOMEM = -2,
+    YVEX_ERR_IO = -3,
+    YVEX_ERR_FORMAT = -4,
+    YVEX_ERR_UNSUPPORTED = -5,
+    YVEX_ERR_BACKEND = -6,
+    YVEX_ERR_BOUNDS = -7,
+    YVEX_ERR_STATE = -8,
+    YVEX_ERR_CANCELLED = -9,
+    YVEX_ERR_INVALID_ARG = -10,
+    YVEX_ERR_TIMEOUT = -11
+} yvex_status;
+
+#define YVEX_ERROR_WHERE_CAP 96
+#define YVEX_ERROR_MESSAGE_CAP 256
+
+typedef struct {
+    yvex_status code;
+    char where[YVEX_ERROR_WHERE_CAP];
+    char message[YVEX_ERROR_MESSAGE_CAP];
+} yvex_error;
+
+const char *yvex_status_name(yvex_status status);
+void yvex_error_clear(yvex_error *err);
+void yvex_error_set(yvex_error *err, yvex_status code, const char *where, const char *message);
+
+/* ---- dtypes: include/yvex/model.h:19-59 (values are part of the ABI) ----- */
+typedef enum {
+    YVEX_DTYPE_UNKNOWN = 0,
+    YVEX_DTYPE_F32 = 1,
+    YVEX_DTYPE_F16 = 2,
+    YVEX_DTYPE_BF16 = 3,
+    YVEX_DTYPE_F64 = 4,
+    YVEX_DTYPE_I8 = 5,
+    YVEX_DTYPE_I16 = 6,
+    YVEX_DTYPE_I32 = 7,
+    YVEX_DTYPE_I64 = 8,
+    YVEX_DTYPE_Q8_0 = 13
+} yvex_dtype;
+
+#define YVEX_TENSOR_MAX_DIMS 4u
+
+/* ---- backend objects: include/yvex/backend.h:13-140 ---------------------- */
+typedef struct yvex_backend yvex_backend;
+typedef struct yvex_device_tensor yvex_device_tensor;
+
+typedef enum {
+    YVEX_BACKEND_KIND_CPU = 0,
+    YVEX_BACKEND_KIND_CUDA,
+    YVEX_BACKEND_KIND_METAL,
+    YVEX_BACKEND_KIND_ROCM
+} yvex_backend_kind;
+
+typedef enum {
+    YVEX_BACKEND_STATUS_READY = 0,
+    YVEX_BACKEND_STATUS_CONTEXT_READY,
+    YVEX_BACKEND_STATUS_UNSUPPORTED,
+    YVEX_BACKEND_STATUS_FAILED
+} yvex_backend_status;
+
+typedef struct {
+    yvex_backend_kind kind;
+    const char *device;
+    unsigned long long memory_limit_bytes;
+} yvex_backend_options;
+
+typedef struct {
+    unsigned long long allocated_bytes;
+    unsigned long long allocation_count, allocation_events, release_events;
+    unsigned long long h2d_bytes, d2h_bytes;
+    unsigned long long peak_allocated_bytes;
+    unsigned long long memory_limit_bytes;
+} yvex_backend_memory_stats;
+
+typedef struct {
+    const char *name;
+    yvex_dtype dtype;
+    unsigned int rank;
+    unsigned long long dims[YVEX_TENSOR_MAX_DIMS];
+    unsigned long long bytes;
+} yvex_backend_tensor_desc;
+
+typedef struct {
+    yvex_backend_kind kind;
+    const char *name;
+    int device_index;
+    int compute_capability_major;
+    int compute_capability_minor;
+    unsigned long long global_memory_bytes;
+    unsigned long long free_memory_bytes;
+    unsigned long long total_memory_bytes;
+    int unified_addressing;
+    int managed_memory;
+} yvex_backend_device_info;
+
+typedef enum {
+    YVEX_BACKEND_CAP_TENSOR_ALLOC = 0,
+    YVEX_BACKEND_CAP_TENSOR_READ_WRITE,
+    YVEX_BACKEND_CAP_OP_EMBED,
+    YVEX_BACKEND_CAP_OP_MATMUL,
+    YVEX_BACKEND_CAP_OP_MLP,
+    YVEX_BACKEND_CAP_OP_RMS_NORM,
+    YVEX_BACKEND_CAP_OP_ROPE,
+    YVEX_BACKEND_CAP_OP_ATTENTION
+} yvex_backend_capability;
+
+/* Values 0..16 are the reference's (include/yvex/backend.h:72-91).  Values from 64
+ * are NEW SURFACE: one variant per attention kernel family of this backend so that a
+ * capability query names exactly what is admitted. */
+typedef enum {
+    YVEX_BACKEND_VARIANT_TENSOR_ALLOC = 0,
+    YVEX_BACKEND_VARIANT_TENSOR_ZERO,
+    YVEX_BACKEND_VARIANT_TENSOR_WRITE,
+    YVEX_BACKEND_VARIANT_TENSOR_READ,
+    YVEX_BACKEND_VARIANT_TENSOR_COPY,
+    YVEX_BACKEND_VARIANT_EMBED_F32_TO_F32,
+    YVEX_BACKEND_VARIANT_EMBED_F16_TO_F32,
+    YVEX_BACKEND_VARIANT_RMS_NORM_F32_WEIGHT_F32,
+    YVEX_BACKEND_VARIANT_RMS_NORM_F32_WEIGHT_F16,
+    YVEX_BACKEND_VARIANT_ROPE_F32,
+    YVEX_BACKEND_VARIANT_MATMUL_F32,
+    YVEX_BACKEND_VARIANT_MLP_DENSE_F32,
+    YVEX_BACKEND_VARIANT_MLP_ROUTED_F32,
+    YVEX_BACKEND_VARIANT_ATTENTION_CAUSAL_F32,
+    YVEX_BACKEND_VARIANT_ATTENTION_NONCAUSAL_F32,
+    YVEX_BACKEND_VARIANT_QTYPE_ROW_DOT,
+    YVEX_BACKEND_VARIANT_ATTENTION_ENCODED,
+    YVEX_BACKEND_VARIANT_COUNT,
+    YVEX_BACKEND_VARIANT_ROCM_FIRST = 64,
+    YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_F32 = 64,
+    YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_BF16,
+    YVEX_BACKEND_VARIANT_ROCM_ATTENTION_PAGED_BF16,
+    YVEX_BACKEND_VARIANT_ROCM_ATTENTION_PAGED_Q8_0,
+    YVEX_BACKEND_VARIANT_ROCM_ATTENTION_MLA_BF16,
+    YVEX_BACKEND_VARIANT_ROCM_END
+} yvex_backend_operation_variant;
+
+typedef enum {
+    YVEX_BACKEND_CAPABILITY_UNSUPPORTED = 0,
+    YVEX_BACKEND_CAPABILITY_SUPPORTED,
+    YVEX_BACKEND_CAPABILITY_FAILED
+} yvex_backend_capability_state;
+
+typedef enum {
+    YVEX_BACKEND_CAPABILITY_REASON_NONE = 0,
+    YVEX_BACKEND_CAPABILITY_REASON_DRIVER_UNAVAILABLE,
+    YVEX_BACKEND_CAPABILITY_REASON_DEVICE_UNAVAILABLE,
+    YVEX_BACKEND_CAPABILITY_REASON_CONTEXT_UNAVAILABLE,
+    YVEX_BACKEND_CAPABILITY_REASON_KERNEL_BUNDLE_ABSENT,
+    YVEX_BACKEND_CAPABILITY_REASON_KERNEL_BUNDLE_REJECTED,
+    YVEX_BACKEND_CAPABILITY_REASON_FUNCTION_MISSING,
+    YVEX_BACKEND_CAPABILITY_REASON_VARIANT_UNSUPPORTED,
+    YVEX_BACKEND_CAPABILITY_REASON_LAUNCH_FAILED,
+    YVEX_BACKEND_CAPABILITY_REASON_SYNCHRONIZATION_FAILED,
+    YVEX_BACKEND_CAPABILITY_REASON_CLEANUP_FAILED
+} yvex_backend_capability_reason;
+
+typedef struct {
+    yvex_backend_kind backend_kind;
+    yvex_backend_operation_variant variant;
+    yvex_backend_capability_state state;
+    yvex_backend_capability_reason reason;
+    yvex_dtype input_dtype;
+    yvex_dtype weight_dtype;
+    yvex_dtype output_dtype;
+    int context_available;
+    int kernel_bundle_available;
+    int function_available;
+} yvex_backend_capability_result;
+
+/* include/yvex/internal/backend.h:284-290 */
+typedef struct yvex_backend_operation_facts {
+    unsigned long long h2d_bytes, d2h_bytes, d2d_bytes, kernel_launches, upload_count;
+    unsigned long long download_count, queue_synchronizations, device_synchronizations;
+    unsigned long long active_weight_bytes, state_bytes;
+    unsigned long long activation_bytes, temporary_bytes, accelerated_matrix_launches;
+    int compulsory_memory_facts_available;
+} yvex_backend_operation_facts;
+
+/* include/yvex/internal/backend.h:215-228.  Callers may copy a tensor struct and
+ * offset `data` to form a sub-view (src/backend/core.c:1763-1778). */
+struct yvex_device_tensor {
+    yvex_backend *owner;
+    unsigned long long owner_id;
+    char *name;
+    yvex_dtype dtype;
+    unsigned int rank;
+    unsigned long long dims[YVEX_TENSOR_MAX_DIMS];
+    unsigned long long bytes;
+    unsigned char *data, *host_data;
+    void *backend_allocation;
+    unsigned long long resident_bytes;
+    int virtual_reserved;
+    int is_written, host_accessible, borrowed_host;
+};
+
+/* ---- lifecycle: include/yvex/backend.h:143-160, src/backend/core.c:255-416 --- */
+/* Opens kind ROCM only; any other kind is YVEX_ERR_UNSUPPORTED ("backend %s is not
+ * implemented", src/backend/core.c:280-283).  `device` is NULL / "" / "0".."N". */
+int yvex_backend_open(yvex_backend **out, const yvex_backend_options *options, yvex_error *err);
+/* The opener the reference's yvex_backend_open would call from its ROCM arm, next to
+ * yvex_backend_open_cuda_impl (src/backend/core.c:276-279). */
+int yvex_backend_open_rocm_impl(yvex_backend **out, const char *device,
+                                unsigned long long memory_limit_bytes, yvex_error *err);
+int yvex_backend_rocm_context_available(void);
+int yvex_backend_rocm_available(void);
+int yvex_backend_close_checked(yvex_backend **backend, yvex_error *err);
+void yvex_backend_close(yvex_backend *backend);
+
+yvex_backend_kind yvex_backend_kind_of(const yvex_backend *backend);
+const char *yvex_backend_kind_name(yvex_backend_kind kind);
+/* src/backend/core.c:204-216, widened to accept "rocm". */
+int yvex_backend_kind_parse(const char *name, yvex_backend_kind *out, yvex_error *err);
+yvex_backend_status yvex_backend_status_of(const yvex_backend *backend);
+const char *yvex_backend_status_name(yvex_backend_status status);
+int yvex_backend_get_memory_stats(const yvex_backend *backend, yvex_backend_memory_stats *out,
+                                  yvex_error *err);
+int yvex_backend_get_device_info(const yvex_backend *backend, yvex_backend_device_info *out,
+                                 yvex_error *err);
+
+/* ---- tensors: include/yvex/backend.h:169-199, src/backend/core.c:1143-1290 ---- */
+int yvex_backend_tensor_alloc(yvex_backend *backend, const yvex_backend_tensor_desc *desc,
+                              yvex_device_tensor **out, yvex_error *err);
+void yvex_backend_tensor_free(yvex_backend *backend, yvex_device_tensor *tensor);
+int yvex_backend_tensor_release(yvex_backend *backend, yvex_device_tensor **tensor,
+                                yvex_error *err);
+const char *yvex_device_tensor_name(const yvex_device_tensor *tensor);
+unsigned long long yvex_device_tensor_bytes(const yvex_device_tensor *tensor);
+int yvex_device_tensor_is_written(const yvex_device_tensor *tensor);
+int yvex_backend_tensor_write(yvex_backend *backend, yvex_device_tensor *tensor, const void *src,
+                              unsigned long long len, yvex_error *err);
+int yvex_backend_tensor_read(yvex_backend *backend, const yvex_device_tensor *tensor, void *dst,
+                             unsigned long long len, yvex_error *err);
+int yvex_backend_tensor_zero(yvex_backend *backend, yvex_device_tensor *tensor, yvex_error *err);
+int yvex_backend_tensor_copy(yvex_backend *backend, yvex_device_tensor *dst,
+                             const yvex_device_tensor *src, yvex_error *err);
+int yvex_backend_tensor_owned_by(const yvex_backend *backend, const yvex_device_tensor *tensor);
+/* src/backend/core.c:1763-1778: rank-1 F32 view of `count` elements at `offset`. */
+int yvex_backend_tensor_f32_subview(const yvex_device_tensor *source, unsigned long long offset,
+                                    unsigned long long count, yvex_device_tensor *view);
+int yvex_backend_sync(yvex_backend *backend, yvex_error *err);
+
+/* ---- capability: include/yvex/backend.h:201-213, src/backend/cuda/capability.c:622-760 */
+int yvex_backend_supports(const yvex_backend *backend, yvex_backend_capability capability);
+const char *yvex_backend_capability_name(yvex_backend_capability capability);
+int yvex_backend_query_capability(const yvex_backend *backend,
+                                  yvex_backend_operation_variant variant,
+                                  yvex_backend_capability_result *out, yvex_error *err);
+const char *yvex_backend_operation_variant_name(yvex_backend_operation_variant variant);
+const char *yvex_backend_capability_state_name(yvex_backend_capability_state state);
+const char *yvex_backend_capability_reason_name(yvex_backend_capability_reason reason);
+
+/* ---- reusable device workspace: src/backend/residency.c:207-283 ----------- */
+typedef enum {
+    YVEX_BACKEND_RESIDENT_INVALID = -1,
+    YVEX_BACKEND_RESIDENT_MISS = 0,
+    YVEX_BACKEND_RESIDENT_HIT = 1
+} yvex_backend_resident_result;
+int yvex_backend_workspace_attach(yvex_backend *backend, const yvex_device_tensor *device_tensor,
+                                  unsigned long long generation, yvex_error *err);
+void yvex_backend_workspace_detach(yvex_backend *backend);
+int yvex_backend_workspace_acquire(yvex_backend *backend, unsigned long long bytes,
+                                   unsigned long long alignment,
+                                   unsigned long long *device_address);
+
+/* ---- bounded single-head primitive: include/yvex/backend.h:244-255,
+ *      src/backend/core.c:1095-1141,1547-1616, src/backend/cuda/ops.c:1717-1807 ---- */
+int yvex_backend_op_attention(yvex_backend *backend, const yvex_device_tensor *query,
+                              const yvex_device_tensor *keys, const yvex_device_tensor *values,
+                              unsigned long long seq_len, unsigned long long position,
+                              float scale, int causal, yvex_device_tensor *score_scratch,
+                              yvex_device_tensor *probability_scratch, yvex_device_tensor *out,
+                              yvex_error *err);
+
+/* ---- multi-token attention contract: include/yvex/internal/transformer.h:245-275 ---- */
+typedef enum {
+    YVEX_TRANSFORMER_ATTENTION_LAYOUT_UNKNOWN = 0,
+    YVEX_TRANSFORMER_ATTENTION_LAYOUT_TOKEN_HEAD_DIM
+} yvex_transformer_attention_layout;
+typedef enum {
+    YVEX_TRANSFORMER_ATTENTION_MASK_UNKNOWN = 0,
+    YVEX_TRANSFORMER_ATTENTION_MASK_FULL,
+    YVEX_TRANSFORMER_ATTENTION_MASK_CAUSAL
+} yvex_transformer_attention_mask;
+/* EXACT_F32 is the reference's only contract.  BF16_F32_ACCUMULATE is NEW SURFACE:
+ * bf16 Q/K/V/output, fp32 scores, fp32 online softmax, fp32 accumulation, MFMA
+ * products; it is never substituted for EXACT_F32 (a request states its contract and
+ * is refused when that contract is not admitted). */
+typedef enum {
+    YVEX_TRANSFORMER_ATTENTION_NUMERIC_UNKNOWN = 0,
+    YVEX_TRANSFORMER_ATTENTION_NUMERIC_EXACT_F32,
+    YVEX_TRANSFORMER_ATTENTION_NUMERIC_BF16_F32_ACCUMULATE
+} yvex_transformer_attention_numeric_contract;
+
+typedef struct yvex_transformer_attention_requirement {
+    unsigned long long query_tokens, key_value_tokens, query_start;
+    unsigned long long query_heads, key_value_heads, head_dimension;
+    /* 0 = packed; otherwise elements (of the tensor's dtype) per token */
+    unsigned long long query_token_stride, key_token_stride, value_token_stride;
+    yvex_dtype query_dtype, key_dtype, value_dtype, output_dtype;
+    yvex_transformer_attention_layout layout;
+    yvex_transformer_attention_mask mask;
+    yvex_transformer_attention_numeric_contract numeric_contract;
+    int deterministic;
+} yvex_transformer_attention_requirement;
+
+typedef struct yvex_transformer_attention_request {
+    yvex_transformer_attention_requirement requirement;
+    const yvex_device_tensor *query, *key, *value;
+    yvex_device_tensor *output;
+} yvex_transformer_attention_request;
+
+/* The attention members of struct yvex_backend_transformer_operations
+ * (include/yvex/internal/transformer.h:291-294), same signatures. */
+typedef struct yvex_backend_transformer_operations {
+    int (*attention_workspace_required)(const yvex_transformer_attention_requirement *,
+                                        unsigned long long *, yvex_error *);
+    int (*attention_execute)(yvex_backend *, const yvex_transformer_attention_request *,
+                             yvex_backend_operation_facts *, yvex_error *);
+} yvex_backend_transformer_operations;
+/* include/yvex/internal/backend.h:211-212; NULL when the kernel bundle is not admitted. */
+const yvex_backend_transformer_operations *yvex_backend_transformer_operations_get(
+    const yvex_backend *backend);
+
+/* ======================= NEW SURFACE (no reference counterpart) ============ */
+
+/* KV cache storage kinds for paged decode. */
+typedef enum {
+    YVEX_ROCM_KV_BF16 = 1,
+    YVEX_ROCM_KV_Q8_0 = 2
+} yvex_rocm_kv_storage;
+
+/*
+ * Paged GQA decode: one query token per session against a paged KV pool.
+ * Device page layouts (head_dimension 128, page_tokens 16), per (page, kv_head):
+ *   BF16  K block: uint16 [d/8][16 tokens][8]           (4096 B)
+ *         V block: uint16 [d][16 tokens]                (4096 B)
+ *   Q8_0  K block: int8 [4 lane groups][16 tokens][4 blocks][8] + f16 scale [16 tokens][4 blocks]
+ *         V block: int8 [4 token groups][16 dims][8 dim blocks][4 tokens] + f16 scale [16 tokens][4 blocks]
+ *                                                        (2176 B each)
+ * Pool = [pool_pages][key_value_heads][block].  yvex_rocm_kv_pack_* build these from
+ * token-major rows.  page_table is I32 [sessions][page_table_stride]; context_tokens is
+ * I32 [sessions] (both device tensors).  Output is BF16 [sessions][query_heads][d], lse is
+ * F32 [sessions][query_heads] (natural-log log-sum-exp of the scaled scores; optional).
+ */
+typedef struct yvex_rocm_paged_decode_requirement {
+    unsigned long long sessions, query_heads, key_value_heads, head_dimension;
+    unsigned long long page_tokens, pool_pages, page_table_stride;
+    /* upper bound on any session's context, used only to size the launch and workspace */
+    unsigned long long max_context_tokens;
+    yvex_rocm_kv_storage kv_storage;
+    yvex_transformer_attention_numeric_contract numeric_contract;
+    int deterministic;
+} yvex_rocm_paged_decode_requirement;
+
+typedef struct yvex_rocm_paged_decode_request {
+    yvex_rocm_paged_decode_requirement requirement;
+    const yvex_device_tensor *query, *key_pages, *value_pages, *page_table, *context_tokens;
+    yvex_device_tensor *output, *lse;
+} yvex_rocm_paged_decode_request;
+
+/*
+ * Absorbed-latent MLA decode: `heads` query heads share one latent row per token;
+ * score over key_dimension (latent + rope), value = first value_dimension lanes.
+ * Pool: BF16 [pool_pages][page_tokens][key_dimension] (token-major, page_tokens 64).
+ * query BF16 [batch][heads][key_dimension]; output BF16 [batch][heads][value_dimension].
+ */
+typedef struct yvex_rocm_mla_decode_requirement {
+    unsigned long long batch, heads, key_dimension, value_dimension;
+    unsigned long long page_tokens, pool_pages, page_table_stride, max_context_tokens;
+    yvex_transformer_attention_numeric_contract numeric_contract;
+    int deterministic;
+} yvex_rocm_mla_decode_requirement;
+
+typedef struct yvex_rocm_mla_decode_request {
+    yvex_rocm_mla_decode_requirement requirement;
+    const yvex_device_tensor *query, *latent_pages, *page_table, *context_tokens;
+    yvex_device_tensor *output, *lse;
+} yvex_rocm_mla_decode_request;
+
+typedef struct yvex_backend_rocm_attention_operations {
+    /* attention_execute with an additional F32 [query_tokens][query_heads] LSE output */
+    int (*attention_execute_lse)(yvex_backend *, const yvex_transformer_attention_request *,
+                                 yvex_device_tensor *lse, yvex_backend_operation_facts *,
+                                 yvex_error *);
+    int (*paged_decode_workspace_required)(const yvex_rocm_paged_decode_requirement *,
+                                           unsigned long long *, yvex_error *);
+    int (*paged_decode_execute)(yvex_backend *, const yvex_rocm_paged_decode_request *,
+                                yvex_backend_operation_facts *, yvex_error *);
+    int (*mla_decode_workspace_required)(const yvex_rocm_mla_decode_requirement *,
+                                         unsigned long long *, yvex_error *);
+    int (*mla_decode_execute)(yvex_backend *, const yvex_rocm_mla_decode_request *,
+                              yvex_backend_operation_facts *, yvex_error *);
+} yvex_backend_rocm_attention_operations;
+const yvex_backend_rocm_attention_operations *yvex_backend_rocm_attention_operations_get(
+    const yvex_backend *backend);
+
+/*
+ * Completion mode.  IMMEDIATE (default) is the reference's behaviour: every operation
+ * synchronises once and reads the device status word before returning
+ * (src/backend/cuda/transformer.c:655-673).  DEFERRED enqueues only; the status word is
+ * checked by the next yvex_backend_sync, which reports the first recorded failure.
+ */
+typedef enum {
+    YVEX_ROCM_COMPLETION_IMMEDIATE = 0,
+    YVEX_ROCM_COMPLETION_DEFERRED = 1
+} yvex_rocm_completion_mode;
+int yvex_backend_rocm_completion_mode_set(yvex_backend *backend, yvex_rocm_completion_mode mode,
+                                          yvex_error *err);
+
+/* Device-event timing on the backend's stream (cf. yvex_cuda_timing,
+ * src/backend/cuda/private.h:421-428).  end() synchronises and returns milliseconds. */
+int yvex_backend_rocm_timing_begin(yvex_backend *backend, yvex_error *err);
+int yvex_backend_rocm_timing_end(yvex_backend *backend, double *milliseconds, yvex_error *err);
+
+/* Kernel-bundle facts (cf. `inspect backend cuda`, src/backend/core.c:1824-1916). */
+typedef struct {
+    int driver_loaded, device_ready, bundle_built, bundle_admitted;
+    unsigned int image_count, function_count;
+    char architecture[32];
+    char device_name[128];
+    char driver_library[256];
+    char rejection[YVEX_ERROR_MESSAGE_CAP];
+} yvex_backend_rocm_report;
+int yvex_backend_rocm_report_get(const yvex_backend *backend, yvex_backend_rocm_report *out,
+                                 yvex_error *err);
+
+/* ---- scalar and block codecs (host): src/gguf/quant_scalar.c:40-143,
+ *      src/gguf/quant_block.c:160-186,819-833 ------------------------------- */
+float yvex_quant_f16_decode(unsigned short bits);
+unsigned short yvex_quant_f16_encode(float value);
+float yvex_quant_bf16_decode(unsigned short bits);
+unsigned short yvex_quant_bf16_encode(float value);
+#define YVEX_QUANT_Q8_0_ELEMENTS 32u
+#define YVEX_QUANT_Q8_0_BYTES 34u
+/* Row forms (elements % 32 == 0).  encode refuses an unrepresentable scale with
+ * YVEX_ERR_BOUNDS; decode refuses a negative or non-finite scale with YVEX_ERR_FORMAT. */
+int yvex_rocm_q8_0_encode_row(const float *source, unsigned long long elements,
+                              unsigned char *encoded, yvex_error *err);
+int yvex_rocm_q8_0_decode_row(const unsigned char *encoded, unsigned long long elements,
+                              float *out, yvex_error *err);
+
+/* ---- host-side page packers (layout only, bytes are moved, never recomputed) ---- */
+unsigned long long yvex_rocm_kv_page_block_bytes(yvex_rocm_kv_storage storage,
+                                                 unsigned long long head_dimension,
+                                                 unsigned long long page_tokens);
+/* rows: token-major [pool_pages][page_tokens][kv_heads][row] where row is d bf16 values
+ * (BF16) or d/32 canonical 34-byte blocks (Q8_0).  is_value selects the V block layout. */
+int yvex_rocm_kv_pack_pages(yvex_rocm_kv_storage storage, int is_value, const void *rows,
+                            unsigned long long pool_pages, unsigned long long page_tokens,
+                            unsigned long long kv_heads, unsigned long long head_dimension,
+                            void *packed, yvex_error *err);
+int yvex_rocm_kv_unpack_pages(yvex_rocm_kv_storage storage, int is_value, const void *packed,
+                              unsigned long long pool_pages, unsigned long long page_tokens,
+                              unsigned long long kv_heads, unsigned long long head_dimension,
+                              void *rows, yvex_error *err);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* YVEX_ROCM_H */

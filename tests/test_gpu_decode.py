@@ -1,0 +1,201 @@
+"""GPU parity: split-K decode (token-major and paged bf16) against the CPU oracle,
+called through the C ABI."""
+import numpy as np
+import pytest
+
+from clori_amd import binding as B
+from clori_amd.backend import YvexError, kv_pack_pages
+from gpu_common import ORACLE, assert_close_bf16, assert_lse, backend, bf16_normal  # noqa: F401
+
+pytestmark = pytest.mark.gpu
+
+
+def run_rows_decode(backend, q, k, v, query_start, causal=True, k_stride=0, v_stride=0,
+                    kv_storage=None):
+    """q uint16 [1,Hq,d]; k/v uint16 [Tk,Hkv,d] (or interleaved storage with strides)."""
+    _, hq, d = q.shape
+    tk, hkv = k.shape[0], k.shape[1]
+    req = backend.attention_requirement(1, tk, hq, hkv, d, causal=causal, query_start=query_start,
+                                        dtype=B.DTYPE_BF16,
+                                        contract=B.NUMERIC_BF16_F32_ACCUMULATE,
+                                        k_stride=k_stride, v_stride=v_stride)
+    tq = backend.tensor("q", B.DTYPE_BF16, q.shape, q)
+    if kv_storage is None:
+        tk_ = backend.tensor("k", B.DTYPE_BF16, k.shape, k)
+        tv_ = backend.tensor("v", B.DTYPE_BF16, v.shape, v)
+    else:
+        store = backend.tensor("kv", B.DTYPE_BF16, kv_storage.shape, kv_storage)
+        width = hkv * d
+        count = (tk - 1) * k_stride + width
+        tk_ = store.view(0, B.DTYPE_BF16, (count,))
+        tv_ = store.view(width * 2, B.DTYPE_BF16, (count,))
+    out = backend.tensor("o", B.DTYPE_BF16, q.shape)
+    lse = backend.tensor("lse", B.DTYPE_F32, (1, hq))
+    facts = backend.attention_execute(req, tq, tk_, tv_, out, lse=lse)
+    result = out.read(), lse.read(), facts
+    return result
+
+
+def test_config1_contiguous_decode_matches_cpu_operator(backend):
+    """BASELINE config 1: B=1, 32/8 heads, d=128, ctx 4096, contiguous KV, seed 1."""
+    rng = np.random.default_rng(1)
+    q = bf16_normal(rng, (1, 32, 128))
+    k = bf16_normal(rng, (4096, 8, 128))
+    v = bf16_normal(rng, (4096, 8, 128))
+    got, lse, facts = run_rows_decode(backend, q, k, v, query_start=4095)
+    rc, ref, _, ref_lse = ORACLE.gqa_bf16(q, k, v, query_start=4095, causal=True)
+    assert rc == 0
+    assert_close_bf16(got, ref, "config1")
+    assert_lse(lse, ref_lse, "config1")
+    assert facts.kernel_launches == 2 and facts.device_synchronizations == 1
+    assert facts.temporary_bytes > 0
+
+
+@pytest.mark.parametrize("ctx", [1, 2, 15, 16, 17, 63, 64, 65, 1000, 1025])
+def test_rows_decode_ragged_lengths(backend, ctx):
+    rng = np.random.default_rng(100 + ctx)
+    q = bf16_normal(rng, (1, 8, 128))
+    k = bf16_normal(rng, (ctx + 3, 2, 128))
+    v = bf16_normal(rng, (ctx + 3, 2, 128))
+    got, lse, _ = run_rows_decode(backend, q, k, v, query_start=ctx - 1)
+    rc, ref, _, ref_lse = ORACLE.gqa_bf16(q, k, v, query_start=ctx - 1, causal=True)
+    assert rc == 0
+    assert_close_bf16(got, ref, "ctx=%d" % ctx)
+    assert_lse(lse, ref_lse, "ctx=%d" % ctx)
+    # FULL mask sees the rows past the query position too
+    got, lse, _ = run_rows_decode(backend, q, k, v, query_start=ctx - 1, causal=False)
+    rc, ref, _, ref_lse = ORACLE.gqa_bf16(q, k, v, query_start=ctx - 1, causal=False)
+    assert_close_bf16(got, ref, "full ctx=%d" % ctx)
+    assert_lse(lse, ref_lse, "full ctx=%d" % ctx)
+
+
+def test_rows_decode_interleaved_kv_history_rows(backend):
+    """The reference caller passes K at offset 0 and V at offset kv_width of one interleaved
+    [K|V] history row with stride 2*kv_width (src/runtime/stateful_attention.c:326-352)."""
+    rng = np.random.default_rng(7)
+    tk, hq, hkv, d = 300, 16, 4, 128
+    q = bf16_normal(rng, (1, hq, d))
+    k = bf16_normal(rng, (tk, hkv, d))
+    v = bf16_normal(rng, (tk, hkv, d))
+    width = hkv * d
+    store = np.zeros((tk, 2 * width), dtype=np.uint16)
+    store[:, :width] = k.reshape(tk, width)
+    store[:, width:] = v.reshape(tk, width)
+    got, lse, _ = run_rows_decode(backend, q, k, v, query_start=tk - 1, k_stride=2 * width,
+                                  v_stride=2 * width, kv_storage=store)
+    packed, lse2, _ = run_rows_decode(backend, q, k, v, query_start=tk - 1)
+    assert np.array_equal(got, packed) and np.array_equal(lse, lse2)   # strided == packed, bit for bit
+    rc, ref, _, ref_lse = ORACLE.gqa_bf16(q, k, v, query_start=tk - 1, causal=True)
+    assert_close_bf16(got, ref, "interleaved")
+
+
+def make_paged_case(rng, contexts, hq, hkv, d=128, page_tokens=16, spare=5, q8=False):
+    sessions = len(contexts)
+    need = [(c + page_tokens - 1) // page_tokens for c in contexts]
+    pool_pages = sum(need) + spare
+    perm = rng.permutation(pool_pages).astype(np.int32)
+    stride = max(need) + 2
+    table = np.full((sessions, stride), 0, dtype=np.int32)
+    at = 0
+    for s, n in enumerate(need):
+        table[s, :n] = perm[at:at + n]
+        at += n
+    k_rows = bf16_normal(rng, (pool_pages, page_tokens, hkv, d))
+    v_rows = bf16_normal(rng, (pool_pages, page_tokens, hkv, d))
+    q = bf16_normal(rng, (sessions, hq, d))
+    return q, k_rows, v_rows, table, np.array(contexts, dtype=np.int32), pool_pages
+
+
+def run_paged(backend, q, k_rows, v_rows, table, ctx, hkv, pool_pages, storage=B.KV_BF16,
+              max_context=None):
+    sessions, hq, d = q.shape
+    kp = kv_pack_pages(k_rows, storage, False, hkv)
+    vp = kv_pack_pages(v_rows, storage, True, hkv)
+    pool_dtype = B.DTYPE_BF16 if storage == B.KV_BF16 else B.DTYPE_I8
+    elems = kp.size // B.DTYPE_BYTES[pool_dtype]
+    tq = backend.tensor("q", B.DTYPE_BF16, q.shape, q)
+    tkp = backend.tensor("kpool", pool_dtype, (elems,), kp)
+    tvp = backend.tensor("vpool", pool_dtype, (elems,), vp)
+    tt = backend.tensor("table", B.DTYPE_I32, table.shape, table)
+    tc = backend.tensor("ctx", B.DTYPE_I32, ctx.shape, ctx)
+    out = backend.tensor("o", B.DTYPE_BF16, q.shape)
+    lse = backend.tensor("lse", B.DTYPE_F32, (sessions, hq))
+    req = backend.paged_requirement(sessions, hq, hkv, d, 16, pool_pages, table.shape[1],
+                                    max_context or int(table.shape[1] * 16), storage=storage)
+    facts = backend.paged_decode_execute(req, tq, tkp, tvp, tt, tc, out, lse)
+    return out.read(), lse.read(), facts
+
+
+def test_paged_decode_matches_oracle_ragged(backend):
+    rng = np.random.default_rng(3)
+    contexts = [1, 15, 16, 17, 100, 333, 1024, 1025, 2500]
+    q, k_rows, v_rows, table, ctx, pool_pages = make_paged_case(rng, contexts, 32, 8)
+    got, lse, facts = run_paged(backend, q, k_rows, v_rows, table, ctx, 8, pool_pages)
+    rc, ref, _, ref_lse = ORACLE.paged_decode(q, k_rows, v_rows, table, ctx, 8, 16)
+    assert rc == 0
+    assert_close_bf16(got, ref, "paged")
+    assert_lse(lse, ref_lse, "paged")
+    assert facts.kernel_launches == 2 and facts.device_synchronizations == 1
+
+
+def test_paged_decode_page_placement_is_bit_invariant(backend):
+    """Moving every page to another pool slot and rewriting the table must not change a
+    single output bit (index handling is exact)."""
+    rng = np.random.default_rng(4)
+    contexts = [40, 700, 129]
+    q, k_rows, v_rows, table, ctx, pool_pages = make_paged_case(rng, contexts, 8, 2)
+    got, lse, _ = run_paged(backend, q, k_rows, v_rows, table, ctx, 2, pool_pages)
+    perm = rng.permutation(pool_pages)
+    k2, v2 = np.empty_like(k_rows), np.empty_like(v_rows)
+    k2[perm], v2[perm] = k_rows, v_rows
+    table2 = perm[table].astype(np.int32)
+    got2, lse2, _ = run_paged(backend, q, k2, v2, table2, ctx, 2, pool_pages)
+    assert np.array_equal(got, got2) and np.array_equal(lse, lse2)
+    # garbage (NaN bit patterns) in rows past each context must not leak into the result
+    k3, v3 = k_rows.copy(), v_rows.copy()
+    for s, c in enumerate(contexts):
+        last = table[s, (c - 1) // 16]
+        k3[last, c % 16 or 16:] = 0x7FC0
+        v3[last, c % 16 or 16:] = 0x7FC0
+    got3, lse3, _ = run_paged(backend, q, k3, v3, table, ctx, 2, pool_pages)
+    assert np.array_equal(got, got3) and np.array_equal(lse, lse3)
+
+
+def test_paged_decode_refuses_bad_page_ids_and_lengths(backend):
+    rng = np.random.default_rng(5)
+    contexts = [50, 90]
+    q, k_rows, v_rows, table, ctx, pool_pages = make_paged_case(rng, contexts, 8, 2)
+    bad = table.copy()
+    bad[1, 3] = pool_pages
+    with pytest.raises(YvexError) as e:
+        run_paged(backend, q, k_rows, v_rows, bad, ctx, 2, pool_pages)
+    assert e.value.code == B.YVEX_ERR_BOUNDS
+    bad[1, 3] = -1
+    with pytest.raises(YvexError) as e:
+        run_paged(backend, q, k_rows, v_rows, bad, ctx, 2, pool_pages)
+    assert e.value.code == B.YVEX_ERR_BOUNDS
+    with pytest.raises(YvexError) as e:
+        run_paged(backend, q, k_rows, v_rows, table, np.array([50, 0], np.int32), 2, pool_pages)
+    assert e.value.code == B.YVEX_ERR_BOUNDS
+    too_long = np.array([50, table.shape[1] * 16 + 1], np.int32)
+    with pytest.raises(YvexError) as e:
+        run_paged(backend, q, k_rows, v_rows, table, too_long, 2, pool_pages)
+    assert e.value.code == B.YVEX_ERR_BOUNDS
+    # the backend stays usable after a refusal and the next call is clean
+    got, _, _ = run_paged(backend, q, k_rows, v_rows, table, ctx, 2, pool_pages)
+    rc, ref, _, _ = ORACLE.paged_decode(q, k_rows, v_rows, table, ctx, 2, 16)
+    assert_close_bf16(got, ref, "after refusal")
+
+
+def test_config3_shape_sample(backend):
+    """BASELINE config 3 at reduced session count (the oracle finishes in seconds): 32/8
+    heads, d=128, contexts uniform in [512,16384], seeded permutation page tables."""
+    rng = np.random.default_rng(3)
+    contexts = [int(c) for c in rng.integers(512, 16385, size=6)]
+    q, k_rows, v_rows, table, ctx, pool_pages = make_paged_case(rng, contexts, 32, 8)
+    got, lse, _ = run_paged(backend, q, k_rows, v_rows, table, ctx, 8, pool_pages,
+                            max_context=16384 if table.shape[1] * 16 >= 16384 else None)
+    rc, ref, _, ref_lse = ORACLE.paged_decode(q, k_rows, v_rows, table, ctx, 8, 16)
+    assert rc == 0
+    assert_close_bf16(got, ref, "config3")
+    assert_lse(lse, ref_lse, "config3")

@@ -1,0 +1,206 @@
+"""GPU parity for the exact F32 contract: the reference's own test vectors and refusal
+behaviour (tests/unit/backend_ops.c:444-532, tests/unit/cuda/ops.c:567-623,
+tests/unit/cuda/quant_qtype.c:2100-2970), run through the C ABI."""
+import math
+
+import numpy as np
+import pytest
+
+import reference_vectors as rv
+from clori_amd import binding as B
+from clori_amd.backend import YvexError
+from gpu_common import ORACLE, backend  # noqa: F401
+
+pytestmark = pytest.mark.gpu
+
+
+def f32(backend, name, array=None, shape=None):
+    if array is not None:
+        array = np.ascontiguousarray(array, dtype=np.float32)
+        return backend.tensor(name, B.DTYPE_F32, array.shape, array)
+    return backend.tensor(name, B.DTYPE_F32, shape)
+
+
+def test_bounded_primitive_reference_literals(backend):
+    q = f32(backend, "attention_query", rv.CPU_OP_QUERY)
+    k = f32(backend, "attention_keys", rv.CPU_OP_KEYS)
+    v = f32(backend, "attention_values", rv.CPU_OP_VALUES)
+    s = f32(backend, "attention_scores", shape=(3,))
+    p = f32(backend, "attention_probabilities", shape=(3,))
+    o = f32(backend, "attention_out", shape=(4,))
+    assert not o.is_written
+    backend.op_attention(q, k, v, 3, 0, 0.5, True, s, p, o)
+    assert np.allclose(o.read(), rv.CPU_OP_VALUES[0], atol=1e-6) and o.is_written
+    backend.op_attention(q, k, v, 3, 2, 0.5, True, s, p, o)
+    rc, ref, ref_s, ref_p, _ = ORACLE.attention_head(rv.CPU_OP_QUERY, rv.CPU_OP_KEYS,
+                                                     rv.CPU_OP_VALUES, 2, 0.5)
+    assert np.allclose(o.read(), ref, atol=1e-6)
+    assert np.allclose(s.read(), ref_s, atol=1e-7) and np.allclose(p.read(), ref_p, atol=1e-7)
+    backend.op_attention(q, k, v, 3, 0, 0.5, False, s, p, o)      # non-causal sees all rows
+    assert np.allclose(o.read(), ref, atol=1e-6)
+    with pytest.raises(YvexError) as e:
+        backend.op_attention(q, k, v, 3, 3, 0.5, True, s, p, o)
+    assert e.value.code == B.YVEX_ERR_BOUNDS and "position-out-of-range" in e.value.message
+    with pytest.raises(YvexError) as e:
+        backend.op_attention(q, k, v, 0, 0, 0.5, True, s, p, o)
+    assert e.value.code == B.YVEX_ERR_INVALID_ARG
+    for scale in (float("nan"), 0.0, -1.0, float("inf")):
+        with pytest.raises(YvexError) as e:
+            backend.op_attention(q, k, v, 3, 0, scale, True, s, p, o)
+        assert e.value.code == B.YVEX_ERR_INVALID_ARG
+    wrong = f32(backend, "wrong", shape=(5,))
+    with pytest.raises(YvexError) as e:
+        backend.op_attention(q, k, v, 3, 0, 0.5, True, s, p, wrong)
+    assert e.value.code == B.YVEX_ERR_FORMAT
+    half = backend.tensor("half", B.DTYPE_BF16, (4,))
+    with pytest.raises(YvexError) as e:
+        backend.op_attention(q, k, v, 3, 0, 0.5, True, s, p, half)
+    assert e.value.code == B.YVEX_ERR_UNSUPPORTED
+
+
+def test_bounded_primitive_long_row_matches_cpu_operator(backend):
+    rng = np.random.default_rng(12)
+    n, d = 4096, 128
+    qv = rng.standard_normal(d).astype(np.float32)
+    kv = rng.standard_normal((n, d)).astype(np.float32)
+    vv = rng.standard_normal((n, d)).astype(np.float32)
+    q, k, v = f32(backend, "q", qv), f32(backend, "k", kv), f32(backend, "v", vv)
+    s, p, o = f32(backend, "s", shape=(n,)), f32(backend, "p", shape=(n,)), f32(backend, "o", shape=(d,))
+    scale = 1.0 / math.sqrt(d)
+    backend.op_attention(q, k, v, n, n - 1, scale, True, s, p, o)
+    rc, ref, ref_s, ref_p, _ = ORACLE.attention_head(qv, kv, vv, n - 1, scale)
+    assert np.allclose(o.read(), ref, atol=1e-6)
+    assert np.allclose(s.read(), ref_s, atol=1e-6) and abs(p.read().sum() - 1.0) < 1e-5
+
+
+def execute(backend, q, k, v, query_start=0, causal=True, **kw):
+    tq, hq, d = q.shape
+    tk, hkv, _ = k.shape
+    req = backend.attention_requirement(tq, tk, hq, hkv, d, causal=causal, query_start=query_start,
+                                        **kw)
+    out = f32(backend, "out", shape=(tq, hq, d))
+    facts = backend.attention_execute(req, f32(backend, "q", q), f32(backend, "k", k),
+                                      f32(backend, "v", v), out)
+    return out.read(), facts
+
+
+def test_gqa_known_answer(backend):
+    q, k, v, mixed = rv.gqa_kat()
+    out, facts = execute(backend, q, k, v, causal=True)
+    assert facts.kernel_launches == 1 and facts.device_synchronizations == 1
+    assert np.array_equal(out[0], np.array([[2.0, 4.0], [2.0, 4.0]], np.float32))
+    assert np.allclose(out[1], mixed, atol=1e-6)
+    out, _ = execute(backend, q, k, v, causal=False)
+    assert np.allclose(out, np.broadcast_to(mixed, (2, 2, 2)), atol=1e-6)
+    req = backend.attention_requirement(2, 2, 2, 1, 2)
+    assert backend.attention_workspace_required(req) == 0
+
+
+@pytest.mark.parametrize("maker,tol_abs,tol_rel", [
+    (rv.small_5x128, 2e-5, 0.0), (rv.qwen_24_4_256, 2e-4, 2e-4), (rv.tiled_257x128, 0.0, 2e-3)])
+def test_gqa_reference_patterns(backend, maker, tol_abs, tol_rel):
+    q, k, v = maker()
+    for causal in (True, False):
+        out, _ = execute(backend, q, k, v, causal=causal)
+        rc, ref, _ = ORACLE.gqa(q, k, v, causal=causal)
+        assert rc == 0
+        assert np.all(np.abs(out - ref) <= tol_abs + tol_rel * (1.0 + np.abs(ref)) + 1e-7)
+        assert np.abs(out - ref).max() < 2e-6          # and far tighter against the CPU operator
+        again, _ = execute(backend, q, k, v, causal=causal)
+        assert np.array_equal(out, again)               # deterministic: byte-identical repeat
+
+
+def test_gqa_cached_decode_strided_and_refusals(backend):
+    q, k, v = rv.cached_decode_qwen()
+    out, _ = execute(backend, q, k, v, query_start=2)
+    rc, ref, _ = ORACLE.gqa(q, k, v, query_start=2)
+    assert np.abs(out - ref).max() < 2e-6
+    with pytest.raises(YvexError) as e:
+        execute(backend, q, k, v, query_start=3)                    # query range beyond KV
+    assert e.value.code == B.YVEX_ERR_INVALID_ARG
+    # strided [Q|gate] and [K|V] views
+    q, k, v = rv.strided_qwen()
+    tq, hq, d = q.shape
+    tk, hkv, _ = k.shape
+    qi = np.full((tq, 2 * hq * d), 55.0, np.float32)
+    qi[:, :hq * d] = q.reshape(tq, -1)
+    kvi = np.zeros((tk, 2 * hkv * d), np.float32)
+    kvi[:, :hkv * d] = k.reshape(tk, -1)
+    kvi[:, hkv * d:] = v.reshape(tk, -1)
+    qs = f32(backend, "q-storage", qi)
+    kvs = f32(backend, "kv-storage", kvi)
+    q_view = qs.view(0, B.DTYPE_F32, ((tq - 1) * 2 * hq * d + hq * d,))
+    k_view = kvs.view(0, B.DTYPE_F32, ((tk - 1) * 2 * hkv * d + hkv * d,))
+    v_view = kvs.view(hkv * d * 4, B.DTYPE_F32, ((tk - 1) * 2 * hkv * d + hkv * d,))
+    out_t = f32(backend, "out", shape=(tq, hq, d))
+    req = backend.attention_requirement(tq, tk, hq, hkv, d, query_start=2, q_stride=2 * hq * d,
+                                        k_stride=2 * hkv * d, v_stride=2 * hkv * d)
+    backend.attention_execute(req, q_view, k_view, v_view, out_t)
+    packed, _ = execute(backend, q, k, v, query_start=2)
+    assert np.array_equal(out_t.read(), packed)                     # strided == packed, bit for bit
+    req.query_token_stride = hq * d - 1
+    with pytest.raises(YvexError) as e:
+        backend.attention_execute(req, q_view, k_view, v_view, out_t)
+    assert e.value.code == B.YVEX_ERR_INVALID_ARG                   # stride below the row width
+
+
+def test_gqa_admission_is_fail_closed(backend):
+    q, k, v = rv.small_5x128()
+    # head dimension beyond the admitted bound
+    req = backend.attention_requirement(3, 3, 24, 4, 257)
+    with pytest.raises(YvexError) as e:
+        backend.attention_workspace_required(req)
+    assert e.value.code == B.YVEX_ERR_UNSUPPORTED
+    # a bf16 output under the exact contract is a silent precision change: refused
+    req = backend.attention_requirement(5, 5, 1, 1, 128)
+    req.output_dtype = B.DTYPE_BF16
+    with pytest.raises(YvexError) as e:
+        backend.attention_workspace_required(req)
+    assert e.value.code == B.YVEX_ERR_UNSUPPORTED
+    # F32 tensors under the bf16 contract are refused as well
+    req = backend.attention_requirement(5, 5, 1, 1, 128, contract=B.NUMERIC_BF16_F32_ACCUMULATE)
+    with pytest.raises(YvexError) as e:
+        backend.attention_workspace_required(req)
+    assert e.value.code == B.YVEX_ERR_UNSUPPORTED
+    req = backend.attention_requirement(5, 5, 1, 1, 128, deterministic=0)
+    with pytest.raises(YvexError) as e:
+        backend.attention_workspace_required(req)
+    assert e.value.code == B.YVEX_ERR_UNSUPPORTED
+    # NaN input -> YVEX_ERR_FORMAT through the device status word; output stays unwritten
+    qn = q.copy()
+    qn[2, 0, 5] = np.nan
+    req = backend.attention_requirement(5, 5, 1, 1, 128)
+    out = f32(backend, "out", shape=(5, 1, 128))
+    with pytest.raises(YvexError) as e:
+        backend.attention_execute(req, f32(backend, "q", qn), f32(backend, "k", k),
+                                  f32(backend, "v", v), out)
+    assert e.value.code == B.YVEX_ERR_FORMAT and not out.is_written
+    # inputs that were never written are refused
+    with pytest.raises(YvexError) as e:
+        backend.attention_execute(req, f32(backend, "q", shape=(5, 1, 128)), f32(backend, "k", k),
+                                  f32(backend, "v", v), out)
+    assert e.value.code == B.YVEX_ERR_FORMAT
+    good, _ = execute(backend, q, k, v)                            # backend still healthy
+    assert np.all(np.isfinite(good))
+
+
+def test_gqa_uniform_analytic_large(backend):
+    for tokens in (65, 5757):
+        q, k, v = rv.uniform_large(tokens, 2)
+        out, _ = execute(backend, q, k, v, causal=False)
+        assert np.abs(out - v).max() <= 2e-3 and np.abs(out - v).max() < 1e-5
+
+
+def test_lse_output_exact_contract(backend):
+    rng = np.random.default_rng(8)
+    q = rng.standard_normal((3, 4, 64)).astype(np.float32)
+    k = rng.standard_normal((9, 2, 64)).astype(np.float32)
+    v = rng.standard_normal((9, 2, 64)).astype(np.float32)
+    req = backend.attention_requirement(3, 9, 4, 2, 64, query_start=6)
+    out = f32(backend, "out", shape=(3, 4, 64))
+    lse = f32(backend, "lse", shape=(3, 4))
+    backend.attention_execute(req, f32(backend, "q", q), f32(backend, "k", k), f32(backend, "v", v),
+                              out, lse=lse)
+    rc, ref, ref_lse = ORACLE.gqa(q, k, v, query_start=6)
+    assert np.abs(out.read() - ref).max() < 2e-6
+    assert np.abs(lse.read() - ref_lse).max() < 1e-5
