@@ -1,0 +1,262 @@
+#!/usr/bin/env python3
+"""Benchmark of the attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu]
+
+A step is one pass of the attention operator over one batch of synthetic input that is
+already resident in HBM.  Workloads are BASELINE.json's configurations:
+
+    prefill2   causal GQA prefill, T=2048, 40/8 heads, d=128            (MFMA bound)
+    decode1    contiguous decode, 32/8 heads, d=128, context 4096        (HBM bound)
+    paged3     32 sessions, paged bf16 KV, contexts U[512,16384]         (HBM bound)
+    paged4     32 sessions, paged Q8_0 KV, contexts U[4096,32768]        (HBM bound)
+    mla5       absorbed MLA decode, batch 16, 128 heads, context 8192    (HBM bound)
+
+Prints ONE JSON line.  `value` is the headline workload's throughput; every workload
+that ran is listed under "workloads" with its own roofline figures.  Timing uses HIP
+events recorded on the backend's own stream (the stream the kernels are launched on).
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+from clori_amd import binding as B  # noqa: E402
+from clori_amd.backend import Backend  # noqa: E402
+
+HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
+
+
+def bf16_bits(x):
+    """float32 -> bf16 bits (RNE) with integer arithmetic; inputs are finite."""
+    u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32)
+    return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+
+
+def random_bf16(rng, count, unique=1 << 24):
+    """`count` N(0,1) bf16 values.  Beyond `unique` values the block repeats: throughput
+    does not depend on the values and generation stays in seconds."""
+    base = bf16_bits(rng.standard_normal(min(count, unique), dtype=np.float32))
+    if count <= unique:
+        return base
+    reps = (count + unique - 1) // unique
+    return np.tile(base, reps)[:count]
+
+
+def time_steps(backend, run, steps, warmup):
+    """W untimed steps, then K steps bracketed by device events and by a synchronise on
+    both sides.  Returns (device ms per step, wall ms per step)."""
+    backend.set_completion_mode(B.COMPLETION_DEFERRED)
+    for _ in range(warmup):
+        run()
+    backend.sync()
+    t0 = time.perf_counter()
+    backend.timing_begin()
+    for _ in range(steps):
+        run()
+    device_ms = backend.timing_end()
+    backend.sync()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    backend.set_completion_mode(B.COMPLETION_IMMEDIATE)
+    return device_ms / steps, wall_ms / steps
+
+
+# --------------------------------------------------------------------- workloads --
+
+def workload_paged(backend, rng, steps, warmup, q8=False):
+    sessions, hq, hkv, d, page = 32, 32, 8, 128, 16
+    lo, hi = (4096, 32768) if q8 else (512, 16384)
+    contexts = rng.integers(lo, hi + 1, size=sessions).astype(np.int32)
+    need = (contexts + page - 1) // page
+    pool_pages = int(need.sum())
+    stride = int(hi // page)
+    perm = rng.permutation(pool_pages).astype(np.int32)
+    table = np.zeros((sessions, stride), dtype=np.int32)
+    at = 0
+    for s in range(sessions):
+        table[s, :need[s]] = perm[at:at + need[s]]
+        at += int(need[s])
+    storage = B.KV_Q8_0 if q8 else B.KV_BF16
+    block = 2176 if q8 else 4096
+    pool_bytes = pool_pages * hkv * block
+    if q8:
+        # int8 codes in [-127,127] and f16 scales near 1/40: any bytes are valid Q8_0 as long
+        # as scales are finite and non-negative; layout = codes then scales per block
+        pool = np.empty((pool_pages * hkv, block), dtype=np.uint8)
+        codes = rng.integers(-127, 128, size=(1 << 22), dtype=np.int8).view(np.uint8)
+        reps = (pool_pages * hkv * 2048 + codes.size - 1) // codes.size
+        pool[:, :2048] = np.tile(codes, reps)[:pool_pages * hkv * 2048].reshape(-1, 2048)
+        pool[:, 2048:] = np.tile(np.float16(0.025).view(np.uint8) if False else
+                                 np.array([0.025], np.float16).view(np.uint8), 64)[None, :]
+        k_pool = backend.tensor("k-pages", B.DTYPE_I8, (pool_bytes,), pool)
+        v_pool = backend.tensor("v-pages", B.DTYPE_I8, (pool_bytes,), pool[::-1].copy())
+    else:
+        k_pool = backend.tensor("k-pages", B.DTYPE_BF16, (pool_bytes // 2,),
+                                random_bf16(rng, pool_bytes // 2))
+        v_pool = backend.tensor("v-pages", B.DTYPE_BF16, (pool_bytes // 2,),
+                                random_bf16(rng, pool_bytes // 2))
+    q = backend.tensor("q", B.DTYPE_BF16, (sessions, hq, d), random_bf16(rng, sessions * hq * d))
+    tt = backend.tensor("table", B.DTYPE_I32, table.shape, table)
+    tc = backend.tensor("ctx", B.DTYPE_I32, contexts.shape, contexts)
+    out = backend.tensor("out", B.DTYPE_BF16, (sessions, hq, d))
+    lse = backend.tensor("lse", B.DTYPE_F32, (sessions, hq))
+    req = backend.paged_requirement(sessions, hq, hkv, d, page, pool_pages, stride, hi,
+                                    storage=storage)
+    work = backend.tensor("workspace", B.DTYPE_I8,
+                          (backend.paged_decode_workspace_required(req),))
+    backend.workspace_attach(work)
+    run = lambda: backend.paged_decode_execute(req, q, k_pool, v_pool, tt, tc, out, lse)  # noqa: E731
+    facts = run()
+    ms, wall = time_steps(backend, run, steps, warmup)
+    backend.workspace_detach()
+    tokens = int(contexts.sum())
+    per_token = 2 * hkv * (136 if q8 else 256)
+    algo = tokens * per_token + int(need.sum()) * 4 + sessions * 4 + 2 * sessions * hq * d * 2 + \
+        sessions * hq * 4
+    assert np.all(np.isfinite(lse.read()))
+    return dict(name="paged4" if q8 else "paged3",
+                workload="paged %s GQA decode: 32 sessions, 32/8 heads, d=128, contexts U[%d,%d], "
+                         "16-token pages, seeded permutation page tables" %
+                         ("Q8_0" if q8 else "bf16", lo, hi),
+                bound="hbm", algorithmic_bytes=algo, tokens=tokens, ms=ms, wall_ms=wall,
+                launches=int(facts.kernel_launches),
+                dominant_kernel="yvex_rocm_decode_paged_q8_0" if q8 else "yvex_rocm_decode_paged_bf16")
+
+
+def workload_decode1(backend, rng, steps, warmup):
+    hq, hkv, d, ctx = 32, 8, 128, 4096
+    q = backend.tensor("q", B.DTYPE_BF16, (1, hq, d), random_bf16(rng, hq * d))
+    k = backend.tensor("k", B.DTYPE_BF16, (ctx, hkv, d), random_bf16(rng, ctx * hkv * d))
+    v = backend.tensor("v", B.DTYPE_BF16, (ctx, hkv, d), random_bf16(rng, ctx * hkv * d))
+    out = backend.tensor("out", B.DTYPE_BF16, (1, hq, d))
+    lse = backend.tensor("lse", B.DTYPE_F32, (1, hq))
+    req = backend.attention_requirement(1, ctx, hq, hkv, d, causal=True, query_start=ctx - 1,
+                                        dtype=B.DTYPE_BF16,
+                                        contract=B.NUMERIC_BF16_F32_ACCUMULATE)
+    work = backend.tensor("workspace", B.DTYPE_I8, (backend.attention_workspace_required(req),))
+    backend.workspace_attach(work)
+    run = lambda: backend.attention_execute(req, q, k, v, out, lse=lse)  # noqa: E731
+    facts = run()
+    ms, wall = time_steps(backend, run, steps, warmup)
+    backend.workspace_detach()
+    algo = 2 * ctx * hkv * d * 2 + 2 * hq * d * 2 + hq * 4
+    return dict(name="decode1",
+                workload="GQA decode: batch 1, 32/8 heads, d=128, context 4096, contiguous bf16 KV",
+                bound="hbm", algorithmic_bytes=algo, tokens=ctx, ms=ms, wall_ms=wall,
+                launches=int(facts.kernel_launches), dominant_kernel="yvex_rocm_decode_rows_bf16")
+
+
+WORKLOADS = {
+    "decode1": workload_decode1,
+    "paged3": lambda b, r, s, w: workload_paged(b, r, s, w, q8=False),
+    "paged4": lambda b, r, s, w: workload_paged(b, r, s, w, q8=True),
+}
+SEEDS = {"decode1": 1, "prefill2": 2, "paged3": 3, "paged4": 4, "mla5": 5}
+
+
+def roofline(result):
+    seconds = result["ms"] * 1e-3
+    if result["bound"] == "hbm":
+        achieved = result["algorithmic_bytes"] / seconds / 1e9
+        return dict(bound="hbm", achieved=achieved, peak=HBM_PEAK_GBS, unit="GB/s",
+                    frac=achieved / HBM_PEAK_GBS, traffic=None,
+                    kernel=result["dominant_kernel"])
+    achieved = result["flops"] / seconds / 1e12
+    return dict(bound="mfma", achieved=achieved, peak=MFMA_BF16_PEAK_TFLOPS, unit="TFLOP/s",
+                frac=achieved / MFMA_BF16_PEAK_TFLOPS, traffic=None,
+                kernel=result["dominant_kernel"])
+
+
+def cpu_baseline(name):
+    """The oracle (a port of the reference CPU operator) timed on this host's cores on a
+    bounded sample of the same workload."""
+    from oracle_binding import Oracle
+    oracle = Oracle()
+    rng = np.random.default_rng(SEEDS[name])
+    threads = oracle.threads
+    if name in ("paged3", "paged4"):
+        sessions, hq, hkv, d, page = 2, 32, 8, 128, 16
+        contexts = np.array([8192, 8192], dtype=np.int32)
+        pool_pages = int(contexts.sum()) // page
+        table = rng.permutation(pool_pages).astype(np.int32).reshape(sessions, -1)
+        k = bf16_bits(rng.standard_normal((pool_pages, page, hkv, d), dtype=np.float32))
+        v = bf16_bits(rng.standard_normal((pool_pages, page, hkv, d), dtype=np.float32))
+        q = bf16_bits(rng.standard_normal((sessions, hq, d), dtype=np.float32))
+        q8 = name == "paged4"
+        if q8:
+            k = oracle.q8_0_encode_rows(oracle.bf16_decode(k))
+            v = oracle.q8_0_encode_rows(oracle.bf16_decode(v))
+        t0 = time.perf_counter()
+        rc, *_ = oracle.paged_decode(q, k, v, table, contexts, hkv, page, q8=q8)
+        dt = time.perf_counter() - t0
+        assert rc == 0
+        per_token = 2 * hkv * (136 if q8 else 256)
+        value = int(contexts.sum()) * per_token / dt / 1e9
+        return dict(value=value, unit="GB/s", cores=threads, kind="port",
+                    sample="2 sessions x 8192 tokens of the same shape, %.1f s" % dt)
+    if name == "decode1":
+        q = bf16_bits(rng.standard_normal((1, 32, 128), dtype=np.float32))
+        k = bf16_bits(rng.standard_normal((4096, 8, 128), dtype=np.float32))
+        v = bf16_bits(rng.standard_normal((4096, 8, 128), dtype=np.float32))
+        reps, t0 = 20, time.perf_counter()
+        for _ in range(reps):
+            rc, *_ = oracle.gqa_bf16(q, k, v, query_start=4095)
+        dt = (time.perf_counter() - t0) / reps
+        return dict(value=(2 * 4096 * 8 * 128 * 2) / dt / 1e9, unit="GB/s", cores=threads,
+                    kind="port", sample="the full workload, mean of %d runs" % reps)
+    return None
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="paged3",
+                    help="headline workload, or 'all' to run every workload")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU; --gpus %d is not supported "
+                 "(attention shards by session or head without exchange)" % args.gpus)
+    names = list(WORKLOADS) if args.workload == "all" else [args.workload]
+    headline = "paged3" if args.workload == "all" else args.workload
+    results = {}
+    for name in names:
+        backend = Backend()
+        if backend.status != B.STATUS_READY:
+            sys.exit("bench.py: ROCm backend is not ready: %s" % backend.report().rejection.decode())
+        rng = np.random.default_rng(SEEDS[name])
+        results[name] = WORKLOADS[name](backend, rng, args.steps, args.warmup)
+        backend.close()
+    head = results[headline]
+    roof = roofline(head)
+    line = {
+        "metric": "decode attn HBM GB/s" if head["bound"] == "hbm" else "prefill attn TFLOPS",
+        "value": roof["achieved"],
+        "unit": roof["unit"],
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": head["ms"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": head["workload"], "name": head["name"],
+                   "kernel_launches_per_step": head["launches"]},
+        "roofline": roof,
+        "cpu_baseline": None if args.no_cpu else cpu_baseline(headline),
+        "workloads": {n: dict(ms_per_step=r["ms"], wall_ms_per_step=r["wall_ms"],
+                              roofline=roofline(r)) for n, r in results.items()},
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()
