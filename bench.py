@@ -76,6 +76,8 @@ def workload_paged(backend, rng, steps, warmup, q8=False):
     sessions, hq, hkv, d, page = 32, 32, 8, 128, 16
     lo, hi = (4096, 32768) if q8 else (512, 16384)
     contexts = rng.integers(lo, hi + 1, size=sessions).astype(np.int32)
+    if os.environ.get("YVEX_BENCH_UNIFORM_CONTEXT"):   # tuning aid: equal-length sessions
+        contexts[:] = int(os.environ["YVEX_BENCH_UNIFORM_CONTEXT"])
     need = (contexts + page - 1) // page
     pool_pages = int(need.sum())
     stride = int(hi // page)

@@ -92,12 +92,19 @@ __device__ inline void consume(State &st, const Tile &t, const bf16x8 (&q)[4], f
     mloc = fmaxf(mloc, xor_lanes(mloc, 16));
     mloc = fmaxf(mloc, xor_lanes(mloc, 32));
     const float m_new = fmaxf(st.m, mloc);
-    const float alpha = fast_exp2(st.m - m_new);
+    // The running maximum rarely moves after the first tiles: rescale the accumulators
+    // only when some lane of the wave saw a larger score.
+    if (__builtin_amdgcn_ballot_w64(m_new > st.m) != 0ull) {
+        const float alpha = fast_exp2(st.m - m_new);
+        st.l *= alpha;
+#pragma unroll
+        for (int b = 0; b < 8; ++b) st.o[b] *= alpha;
+        st.m = m_new;
+    }
     float p[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) p[i] = fast_exp2(x[i] - m_new);
-    st.l = st.l * alpha + ((p[0] + p[1]) + (p[2] + p[3]));
-    st.m = m_new;
+    for (int i = 0; i < 4; ++i) p[i] = fast_exp2(x[i] - st.m);
+    st.l += (p[0] + p[1]) + (p[2] + p[3]);
     u32x2 pb;
     pb.x = pack_bf16x2(p[0], p[1]);
     pb.y = pack_bf16x2(p[2], p[3]);
@@ -114,15 +121,15 @@ __device__ inline void consume(State &st, const Tile &t, const bf16x8 (&q)[4], f
             u32x2 v = t.v[b];
             v.x &= keep_lo;
             v.y &= keep_hi;
-            st.o[b] = mfma_16x16x16(as_short4(v), pv, st.o[b] * alpha);
+            st.o[b] = mfma_16x16x16(as_short4(v), pv, st.o[b]);
         }
     } else {
 #pragma unroll
-        for (int b = 0; b < 8; ++b) st.o[b] = mfma_16x16x16(as_short4(t.v[b]), pv, st.o[b] * alpha);
+        for (int b = 0; b < 8; ++b) st.o[b] = mfma_16x16x16(as_short4(t.v[b]), pv, st.o[b]);
     }
 }
 
-template <bool PAGED>
+template <bool PAGED, int kDepth>
 __device__ inline void decode_body(const yvex_rocm_decode_params &p)
 {
     const int lane = threadIdx.x, n = lane & 15, g = lane >> 4;
@@ -189,16 +196,31 @@ __device__ inline void decode_body(const yvex_rocm_decode_params &p)
     st.m = -INFINITY;
     st.l = 0.f;
 
-    Tile a, b;
-    fetch(a, 0u);
+    // Ring of kDepth tile buffers: kDepth-1 tiles (8 KB each) stay in flight per wave
+    // while one is consumed.  Every refill in the steady-state loop is unconditional (the
+    // index is clamped to the last tile, a cache hit) so the number of outstanding loads
+    // is the same on every trip and the waits the compiler places are partial
+    // (vmcnt > 0) instead of draining the whole queue.
+    Tile ring[kDepth];
+    const uint32_t last_tile = tiles - 1u;
+#pragma unroll
+    for (int r = 0; r < kDepth; ++r) fetch(ring[r], min((uint32_t)r, last_tile));
     uint32_t i = 0u;
-    for (;;) {
-        if (i + 1u < tiles) fetch(b, i + 1u);
-        consume(st, a, q, p.scale_log2, min((uint32_t)kPageTokens, t1 - (t0 + i * kPageTokens)), lane);
-        if (++i >= tiles) break;
-        if (i + 1u < tiles) fetch(a, i + 1u);
-        consume(st, b, q, p.scale_log2, min((uint32_t)kPageTokens, t1 - (t0 + i * kPageTokens)), lane);
-        if (++i >= tiles) break;
+    for (; i + kDepth <= tiles; i += kDepth) {
+#pragma unroll
+        for (int r = 0; r < kDepth; ++r) {
+            const uint32_t tile = i + (uint32_t)r;
+            consume(st, ring[r], q, p.scale_log2,
+                    min((uint32_t)kPageTokens, t1 - (t0 + tile * kPageTokens)), lane);
+            fetch(ring[r], min(tile + kDepth, last_tile));
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < kDepth - 1; ++r) {
+        const uint32_t tile = i + (uint32_t)r;
+        if (tile < tiles)
+            consume(st, ring[r], q, p.scale_log2,
+                    min((uint32_t)kPageTokens, t1 - (t0 + tile * kPageTokens)), lane);
     }
 
     float l = st.l;
@@ -219,16 +241,16 @@ __device__ inline void decode_body(const yvex_rocm_decode_params &p)
 
 }  // namespace
 
-extern "C" __global__ void __launch_bounds__(64)
+extern "C" __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 yvex_rocm_decode_paged_bf16(const yvex_rocm_decode_params p)
 {
-    decode_body<true>(p);
+    decode_body<true, 3>(p);
 }
 
 extern "C" __global__ void __launch_bounds__(64)
 yvex_rocm_decode_rows_bf16(const yvex_rocm_decode_params p)
 {
-    decode_body<false>(p);
+    decode_body<false, 2>(p);
 }
 
 // Log-sum-exp merge of the chunk partials of one (session, query head); one thread per
@@ -241,10 +263,14 @@ yvex_rocm_decode_merge(const yvex_rocm_decode_merge_params p)
     if (ctx == 0u || d >= p.head_dim) return;
     const uint32_t chunks = min(p.max_chunks, (ctx + p.chunk_tokens - 1u) / p.chunk_tokens);
     const uint64_t base = ((uint64_t)session * p.max_chunks) * p.query_heads + head;
+    // The chunk loops carry no dependent loads: unrolled, eight partial rows are in
+    // flight per thread, which is what keeps this pass in the microsecond range.
     float top = -INFINITY;
+#pragma unroll 8
     for (uint32_t c = 0; c < chunks; ++c)
         top = fmaxf(top, p.part_ml[(base + (uint64_t)c * p.query_heads) * 2]);
     float total = 0.f, acc = 0.f;
+#pragma unroll 8
     for (uint32_t c = 0; c < chunks; ++c) {
         const uint64_t slot = base + (uint64_t)c * p.query_heads;
         const float w = fast_exp2(p.part_ml[slot * 2] - top);
