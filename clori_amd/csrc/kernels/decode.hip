@@ -20,6 +20,16 @@
 // src/runtime/stateful_attention.c:326-352 are addressable): K rows are read in 16-byte
 // pieces, V is gathered transposed.
 //
+// Q8_0 paged layout, per (page, kv head): the canonical GGUF blocks (32 int8 codes and
+// one f16 scale along the head dimension) are kept byte for byte but stored as
+//     K codes  int8 [4 lane groups g][16 tokens][4 blocks j][8]     code(t, 32j+8g+e)
+//     V codes  int8 [4 token groups][16 dims m][8 dim blocks b][4]  code(4tg+i, 16b+m)
+//     scales   f16  [16 tokens][4 blocks]  after each 2048-byte code area
+// so that every lane reads 32 contiguous bytes of codes.  Codes are widened to bf16 in
+// registers (exact: |code| <= 127); a 32-wide MFMA covers exactly one quantisation
+// block, so the K scale is applied to the fp32 partial dot per block, and the V scale
+// is folded into the probabilities per 32-lane block before the second product.
+//
 // Partials (running max in log2 units, sum, unnormalised accumulator) go to the
 // workspace; yvex_rocm_decode_merge combines them with a log-sum-exp merge.
 #include "mfma.h"
@@ -31,69 +41,24 @@ namespace {
 constexpr int kHeadDim = 128;
 constexpr int kPageTokens = 16;
 
-struct Tile {
-    u32x4 k[4];  // K[token = lane%16][32*j + 8*(lane/16) .. +7]
-    u32x2 v[8];  // V[tokens 4*(lane/16)..+3][dim 16*b + lane%16]
-};
 
 __device__ inline void flag(int32_t *status, int code) { atomicCAS(status, 0, code); }
-
-__device__ inline void load_tile_paged(Tile &t, const uint16_t *kblock, const uint16_t *vblock,
-                                       int lane)
-{
-    const int n = lane & 15, g = lane >> 4;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) t.k[j] = load_b128(kblock + (j * 64 + lane) * 8);
-#pragma unroll
-    for (int b = 0; b < 8; ++b) t.v[b] = load_b64(vblock + (b * 16 + n) * 16 + g * 4);
-}
-
-// rows_left: tokens available from `first` on (rows beyond are clamped to the last
-// valid row so no out-of-range address is formed; they are masked later).
-__device__ inline void load_tile_rows(Tile &t, const uint16_t *k, const uint16_t *v,
-                                      uint64_t k_stride, uint64_t v_stride, uint32_t first,
-                                      uint32_t rows_left, int lane)
-{
-    const int n = lane & 15, g = lane >> 4;
-    const uint32_t last = rows_left - 1u;
-    const uint16_t *krow = k + (uint64_t)(first + min((uint32_t)n, last)) * k_stride;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) t.k[j] = load_b128(krow + j * 32 + g * 8);
-    const uint16_t *v0 = v + (uint64_t)(first + min((uint32_t)(g * 4 + 0), last)) * v_stride;
-    const uint16_t *v1 = v + (uint64_t)(first + min((uint32_t)(g * 4 + 1), last)) * v_stride;
-    const uint16_t *v2 = v + (uint64_t)(first + min((uint32_t)(g * 4 + 2), last)) * v_stride;
-    const uint16_t *v3 = v + (uint64_t)(first + min((uint32_t)(g * 4 + 3), last)) * v_stride;
-#pragma unroll
-    for (int b = 0; b < 8; ++b) {
-        const int c = b * 16 + n;
-        t.v[b].x = (uint32_t)v0[c] | ((uint32_t)v1[c] << 16);
-        t.v[b].y = (uint32_t)v2[c] | ((uint32_t)v3[c] << 16);
-    }
-}
 
 struct State {
     floatx4 o[8];  // O^T[dim 16*b + 4*(lane/16) + i][head lane%16]
     float m, l;    // running max (log2 units) and per-lane partial sum
 };
 
-// valid: number of real tokens in this 16-token tile (1..16).
-__device__ inline void consume(State &st, const Tile &t, const bf16x8 (&q)[4], float scale_log2,
-                               uint32_t valid, int lane)
+// Online-softmax step shared by every KV format: takes the scaled scores of the lane's
+// four tokens (masked ones at -inf), updates (m, l), rescales the accumulators only when
+// some lane of the wave saw a larger score (after the first tiles the running maximum
+// rarely moves), and returns the four probabilities.
+__device__ inline void softmax_step(State &st, const float (&x)[4], float (&p)[4])
 {
-    const int g = lane >> 4;
-    floatx4 s = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int j = 0; j < 4; ++j) s = mfma_16x16x32(as_bf16x8(t.k[j]), q[j], s);
-    float x[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-        x[i] = (uint32_t)(g * 4 + i) < valid ? s[i] * scale_log2 : -INFINITY;
     float mloc = fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3]));
     mloc = fmaxf(mloc, xor_lanes(mloc, 16));
     mloc = fmaxf(mloc, xor_lanes(mloc, 32));
     const float m_new = fmaxf(st.m, mloc);
-    // The running maximum rarely moves after the first tiles: rescale the accumulators
-    // only when some lane of the wave saw a larger score.
     if (__builtin_amdgcn_ballot_w64(m_new > st.m) != 0ull) {
         const float alpha = fast_exp2(st.m - m_new);
         st.l *= alpha;
@@ -101,37 +66,198 @@ __device__ inline void consume(State &st, const Tile &t, const bf16x8 (&q)[4], f
         for (int b = 0; b < 8; ++b) st.o[b] *= alpha;
         st.m = m_new;
     }
-    float p[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) p[i] = fast_exp2(x[i] - st.m);
     st.l += (p[0] + p[1]) + (p[2] + p[3]);
-    u32x2 pb;
-    pb.x = pack_bf16x2(p[0], p[1]);
-    pb.y = pack_bf16x2(p[2], p[3]);
-    const short4v pv = as_short4(pb);
-    if (valid < (uint32_t)kPageTokens) {
-        // rows past the context may hold anything (even NaN): a zero weight does not
-        // neutralise them inside the MFMA, so clear them in the V operand
-        uint32_t keep_lo = ((uint32_t)(g * 4 + 0) < valid ? 0x0000ffffu : 0u) |
-                           ((uint32_t)(g * 4 + 1) < valid ? 0xffff0000u : 0u);
-        uint32_t keep_hi = ((uint32_t)(g * 4 + 2) < valid ? 0x0000ffffu : 0u) |
-                           ((uint32_t)(g * 4 + 3) < valid ? 0xffff0000u : 0u);
-#pragma unroll
-        for (int b = 0; b < 8; ++b) {
-            u32x2 v = t.v[b];
-            v.x &= keep_lo;
-            v.y &= keep_hi;
-            st.o[b] = mfma_16x16x16(as_short4(v), pv, st.o[b]);
-        }
-    } else {
-#pragma unroll
-        for (int b = 0; b < 8; ++b) st.o[b] = mfma_16x16x16(as_short4(t.v[b]), pv, st.o[b]);
-    }
 }
 
-template <bool PAGED, int kDepth>
+// ---- bf16 KV --------------------------------------------------------------------
+struct Bf16Tile {
+    u32x4 k[4];  // K[token = lane%16][32*j + 8*(lane/16) .. +7]
+    u32x2 v[8];  // V[tokens 4*(lane/16)..+3][dim 16*b + lane%16]
+};
+
+struct Bf16Kv {
+    typedef Bf16Tile Tile;
+    static constexpr uint32_t kBlockBytes = kPageTokens * kHeadDim * 2;
+
+    __device__ static inline void load_paged(Tile &t, const unsigned char *kblock,
+                                             const unsigned char *vblock, int lane)
+    {
+        const int n = lane & 15, g = lane >> 4;
+        const uint16_t *k = (const uint16_t *)kblock, *v = (const uint16_t *)vblock;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) t.k[j] = load_b128(k + (j * 64 + lane) * 8);
+#pragma unroll
+        for (int b = 0; b < 8; ++b) t.v[b] = load_b64(v + (b * 16 + n) * 16 + g * 4);
+    }
+
+    // rows_left: tokens available from `first` on (rows beyond are clamped to the last
+    // valid row so no out-of-range address is formed; they are masked later).
+    __device__ static inline void load_rows(Tile &t, const unsigned char *kbytes,
+                                            const unsigned char *vbytes,
+                                            const yvex_rocm_decode_params &p, uint32_t first,
+                                            uint32_t rows_left, int lane)
+    {
+        const int n = lane & 15, g = lane >> 4;
+        const uint16_t *k = (const uint16_t *)kbytes, *v = (const uint16_t *)vbytes;
+        const uint32_t last = rows_left - 1u;
+        const uint16_t *krow = k + (uint64_t)(first + min((uint32_t)n, last)) * p.k_token_stride;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) t.k[j] = load_b128(krow + j * 32 + g * 8);
+        const uint16_t *v0 = v + (uint64_t)(first + min((uint32_t)(g * 4 + 0), last)) * p.v_token_stride;
+        const uint16_t *v1 = v + (uint64_t)(first + min((uint32_t)(g * 4 + 1), last)) * p.v_token_stride;
+        const uint16_t *v2 = v + (uint64_t)(first + min((uint32_t)(g * 4 + 2), last)) * p.v_token_stride;
+        const uint16_t *v3 = v + (uint64_t)(first + min((uint32_t)(g * 4 + 3), last)) * p.v_token_stride;
+#pragma unroll
+        for (int b = 0; b < 8; ++b) {
+            const int c = b * 16 + n;
+            t.v[b].x = (uint32_t)v0[c] | ((uint32_t)v1[c] << 16);
+            t.v[b].y = (uint32_t)v2[c] | ((uint32_t)v3[c] << 16);
+        }
+    }
+
+    // valid: number of real tokens in this 16-token tile (1..16).
+    __device__ static inline void consume(State &st, const Tile &t, const bf16x8 (&q)[4],
+                                          float scale_log2, uint32_t valid, int lane)
+    {
+        const int g = lane >> 4;
+        floatx4 s = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) s = mfma_16x16x32(as_bf16x8(t.k[j]), q[j], s);
+        float x[4], p[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            x[i] = (uint32_t)(g * 4 + i) < valid ? s[i] * scale_log2 : -INFINITY;
+        softmax_step(st, x, p);
+        u32x2 pb;
+        pb.x = pack_bf16x2(p[0], p[1]);
+        pb.y = pack_bf16x2(p[2], p[3]);
+        const short4v pv = as_short4(pb);
+        if (valid < (uint32_t)kPageTokens) {
+            // rows past the context may hold anything (even NaN): a zero weight does not
+            // neutralise them inside the MFMA, so clear them in the V operand
+            uint32_t keep_lo = ((uint32_t)(g * 4 + 0) < valid ? 0x0000ffffu : 0u) |
+                               ((uint32_t)(g * 4 + 1) < valid ? 0xffff0000u : 0u);
+            uint32_t keep_hi = ((uint32_t)(g * 4 + 2) < valid ? 0x0000ffffu : 0u) |
+                               ((uint32_t)(g * 4 + 3) < valid ? 0xffff0000u : 0u);
+#pragma unroll
+            for (int b = 0; b < 8; ++b) {
+                u32x2 v = t.v[b];
+                v.x &= keep_lo;
+                v.y &= keep_hi;
+                st.o[b] = mfma_16x16x16(as_short4(v), pv, st.o[b]);
+            }
+        } else {
+#pragma unroll
+            for (int b = 0; b < 8; ++b)
+                st.o[b] = mfma_16x16x16(as_short4(t.v[b]), pv, st.o[b]);
+        }
+    }
+};
+
+// ---- Q8_0 KV ----------------------------------------------------------------------
+struct Q8Tile {
+    u32x4 kc[2];  // 32 K codes: token lane%16, lanes 32j + 8*(lane/16) + e at byte 8j + e
+    u32x4 ks[2];  // 16 f16 K scales: tokens 4*(lane/16)+i, block j at half index 4i + j
+    u32x4 vc[2];  // 32 V codes: dim 16b + lane%16, tokens 4*(lane/16)+i at byte 4b + i
+    u32x4 vs[2];  // 16 f16 V scales, same indexing as ks
+};
+
+// Sign-extends byte `k` of a word and widens it: exact for every int8 code.
+__device__ inline float code_f32(uint32_t word, int k)
+{
+    return (float)((int32_t)(word << (24 - 8 * k)) >> 24);
+}
+
+__device__ inline float half_f32(uint32_t word, int hi)
+{
+    return (float)__builtin_bit_cast(_Float16, (uint16_t)(hi ? word >> 16 : word & 0xffffu));
+}
+
+struct Q8Kv {
+    typedef Q8Tile Tile;
+    static constexpr uint32_t kCodeBytes = kPageTokens * kHeadDim;
+    static constexpr uint32_t kBlockBytes = kCodeBytes + kPageTokens * (kHeadDim / 32) * 2;
+
+    __device__ static inline void load_paged(Tile &t, const unsigned char *kblock,
+                                             const unsigned char *vblock, int lane)
+    {
+        const int g = lane >> 4;
+        t.kc[0] = load_b128(kblock + lane * 32);
+        t.kc[1] = load_b128(kblock + lane * 32 + 16);
+        t.ks[0] = load_b128(kblock + kCodeBytes + g * 32);
+        t.ks[1] = load_b128(kblock + kCodeBytes + g * 32 + 16);
+        t.vc[0] = load_b128(vblock + lane * 32);
+        t.vc[1] = load_b128(vblock + lane * 32 + 16);
+        t.vs[0] = load_b128(vblock + kCodeBytes + g * 32);
+        t.vs[1] = load_b128(vblock + kCodeBytes + g * 32 + 16);
+    }
+
+    __device__ static inline void load_rows(Tile &, const unsigned char *, const unsigned char *,
+                                            const yvex_rocm_decode_params &, uint32_t, uint32_t, int)
+    {
+    }
+
+    __device__ static inline void consume(State &st, const Tile &t, const bf16x8 (&q)[4],
+                                          float scale_log2, uint32_t valid, int lane)
+    {
+        const int g = lane >> 4;
+        float x[4] = {0.f, 0.f, 0.f, 0.f}, p[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            // block j: bytes 8j..8j+7 of the lane's 32 code bytes
+            const uint32_t w0 = t.kc[j >> 1][(j & 1) * 2], w1 = t.kc[j >> 1][(j & 1) * 2 + 1];
+            u32x4 a;
+            a.x = pack_bf16x2_exact(code_f32(w0, 0), code_f32(w0, 1));
+            a.y = pack_bf16x2_exact(code_f32(w0, 2), code_f32(w0, 3));
+            a.z = pack_bf16x2_exact(code_f32(w1, 0), code_f32(w1, 1));
+            a.w = pack_bf16x2_exact(code_f32(w1, 2), code_f32(w1, 3));
+            const floatx4 s = mfma_16x16x32(as_bf16x8(a), q[j], (floatx4){0.f, 0.f, 0.f, 0.f});
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int h = 4 * i + j;  // scale of (token 4g+i, block j)
+                x[i] += half_f32(t.ks[h >> 3][(h >> 1) & 3], h & 1) * s[i];
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            x[i] = (uint32_t)(g * 4 + i) < valid ? x[i] * scale_log2 : -INFINITY;
+        softmax_step(st, x, p);
+        const bool tail = valid < (uint32_t)kPageTokens;  // wave-uniform
+        // fold the V scale of each 32-lane block into the probabilities; masked tokens
+        // get an exact zero whatever their (possibly garbage) scale bits are
+        short4v pv[4];
+#pragma unroll
+        for (int jb = 0; jb < 4; ++jb) {
+            float w[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int h = 4 * i + jb;
+                const float vs = half_f32(t.vs[h >> 3][(h >> 1) & 3], h & 1);
+                w[i] = p[i] * vs;
+                if (tail && (uint32_t)(g * 4 + i) >= valid) w[i] = 0.f;
+            }
+            u32x2 pb;
+            pb.x = pack_bf16x2(w[0], w[1]);
+            pb.y = pack_bf16x2(w[2], w[3]);
+            pv[jb] = as_short4(pb);
+        }
+#pragma unroll
+        for (int b = 0; b < 8; ++b) {
+            const uint32_t w = t.vc[b >> 2][b & 3];
+            u32x2 a;
+            a.x = pack_bf16x2_exact(code_f32(w, 0), code_f32(w, 1));
+            a.y = pack_bf16x2_exact(code_f32(w, 2), code_f32(w, 3));
+            st.o[b] = mfma_16x16x16(as_short4(a), pv[b >> 1], st.o[b]);
+        }
+    }
+};
+
+template <class Kv, bool PAGED, int kDepth>
 __device__ inline void decode_body(const yvex_rocm_decode_params &p)
 {
+    typedef typename Kv::Tile Tile;
     const int lane = threadIdx.x, n = lane & 15, g = lane >> 4;
     const uint32_t chunk = blockIdx.x, kv_head = blockIdx.y, session = blockIdx.z;
     const uint32_t limit = PAGED ? p.table_stride * (uint32_t)kPageTokens : p.fixed_context;
@@ -160,7 +286,8 @@ __device__ inline void decode_body(const yvex_rocm_decode_params &p)
     }
 
     int32_t my_page = 0;
-    const uint16_t *kbase = (const uint16_t *)p.k_pool, *vbase = (const uint16_t *)p.v_pool;
+    const unsigned char *kbase = (const unsigned char *)p.k_pool;
+    const unsigned char *vbase = (const unsigned char *)p.v_pool;
     if (PAGED) {
         // one coalesced read brings the chunk's page ids into the wave (chunk <= 64 pages)
         const int32_t *table =
@@ -173,20 +300,18 @@ __device__ inline void decode_body(const yvex_rocm_decode_params &p)
             }
         }
     } else {
-        kbase += (uint64_t)kv_head * kHeadDim;
-        vbase += (uint64_t)kv_head * kHeadDim;
+        kbase += (uint64_t)kv_head * kHeadDim * 2u;
+        vbase += (uint64_t)kv_head * kHeadDim * 2u;
     }
-    const uint64_t block_elems = (uint64_t)kPageTokens * kHeadDim;
 
     auto fetch = [&](Tile &t, uint32_t i) {
         if (PAGED) {
             const uint32_t page = (uint32_t)__builtin_amdgcn_readlane(my_page, (int)i);
-            const uint64_t off = ((uint64_t)page * p.kv_heads + kv_head) * block_elems;
-            load_tile_paged(t, kbase + off, vbase + off, lane);
+            const uint64_t off = ((uint64_t)page * p.kv_heads + kv_head) * Kv::kBlockBytes;
+            Kv::load_paged(t, kbase + off, vbase + off, lane);
         } else {
             const uint32_t first = t0 + i * kPageTokens;
-            load_tile_rows(t, kbase, vbase, p.k_token_stride, p.v_token_stride, first,
-                           t1 - first, lane);
+            Kv::load_rows(t, kbase, vbase, p, first, t1 - first, lane);
         }
     };
 
@@ -196,11 +321,11 @@ __device__ inline void decode_body(const yvex_rocm_decode_params &p)
     st.m = -INFINITY;
     st.l = 0.f;
 
-    // Ring of kDepth tile buffers: kDepth-1 tiles (8 KB each) stay in flight per wave
-    // while one is consumed.  Every refill in the steady-state loop is unconditional (the
-    // index is clamped to the last tile, a cache hit) so the number of outstanding loads
-    // is the same on every trip and the waits the compiler places are partial
-    // (vmcnt > 0) instead of draining the whole queue.
+    // Ring of kDepth tile buffers: kDepth-1 tiles stay in flight per wave while one is
+    // consumed.  Every refill in the steady-state loop is unconditional (the index is
+    // clamped to the last tile, a cache hit) so the number of outstanding loads is the
+    // same on every trip and the waits the compiler places are partial (vmcnt > 0)
+    // instead of draining the whole queue.
     Tile ring[kDepth];
     const uint32_t last_tile = tiles - 1u;
 #pragma unroll
@@ -210,8 +335,8 @@ __device__ inline void decode_body(const yvex_rocm_decode_params &p)
 #pragma unroll
         for (int r = 0; r < kDepth; ++r) {
             const uint32_t tile = i + (uint32_t)r;
-            consume(st, ring[r], q, p.scale_log2,
-                    min((uint32_t)kPageTokens, t1 - (t0 + tile * kPageTokens)), lane);
+            Kv::consume(st, ring[r], q, p.scale_log2,
+                        min((uint32_t)kPageTokens, t1 - (t0 + tile * kPageTokens)), lane);
             fetch(ring[r], min(tile + kDepth, last_tile));
         }
     }
@@ -219,8 +344,8 @@ __device__ inline void decode_body(const yvex_rocm_decode_params &p)
     for (int r = 0; r < kDepth - 1; ++r) {
         const uint32_t tile = i + (uint32_t)r;
         if (tile < tiles)
-            consume(st, ring[r], q, p.scale_log2,
-                    min((uint32_t)kPageTokens, t1 - (t0 + tile * kPageTokens)), lane);
+            Kv::consume(st, ring[r], q, p.scale_log2,
+                        min((uint32_t)kPageTokens, t1 - (t0 + tile * kPageTokens)), lane);
     }
 
     float l = st.l;
@@ -244,13 +369,19 @@ __device__ inline void decode_body(const yvex_rocm_decode_params &p)
 extern "C" __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 yvex_rocm_decode_paged_bf16(const yvex_rocm_decode_params p)
 {
-    decode_body<true, 3>(p);
+    decode_body<Bf16Kv, true, 3>(p);
+}
+
+extern "C" __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2)))
+yvex_rocm_decode_paged_q8_0(const yvex_rocm_decode_params p)
+{
+    decode_body<Q8Kv, true, 3>(p);
 }
 
 extern "C" __global__ void __launch_bounds__(64)
 yvex_rocm_decode_rows_bf16(const yvex_rocm_decode_params p)
 {
-    decode_body<false, 2>(p);
+    decode_body<Bf16Kv, false, 2>(p);
 }
 
 // Log-sum-exp merge of the chunk partials of one (session, query head); one thread per

@@ -59,9 +59,21 @@ __device__ inline uint16_t bf16_bits(float v)
     return (uint16_t)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
 }
 
+// Two floats -> packed bf16 pair with the hardware's round-to-nearest-even convert
+// (v_cvt_pk_bf16_f32).
 __device__ inline uint32_t pack_bf16x2(float lo, float hi)
 {
-    return (uint32_t)bf16_bits(lo) | ((uint32_t)bf16_bits(hi) << 16);
+    typedef float floatx2 __attribute__((ext_vector_type(2)));
+    const floatx2 f = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2));
+}
+
+// Packs the upper halves of two floats whose lower 16 bits are known to be zero (small
+// integers): exact, one v_perm_b32.
+__device__ inline uint32_t pack_bf16x2_exact(float lo, float hi)
+{
+    return __builtin_amdgcn_perm(__builtin_bit_cast(uint32_t, hi), __builtin_bit_cast(uint32_t, lo),
+                                 0x07060302u);
 }
 
 __device__ inline float bf16_to_f32(uint16_t b)

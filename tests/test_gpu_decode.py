@@ -199,3 +199,63 @@ def test_config3_shape_sample(backend):
     assert rc == 0
     assert_close_bf16(got, ref, "config3")
     assert_lse(lse, ref_lse, "config3")
+
+
+# ------------------------------------------------------------- Q8_0 paged KV ----
+
+def make_q8_case(rng, contexts, hq, hkv, d=128):
+    q, k_rows, v_rows, table, ctx, pool_pages = make_paged_case(rng, contexts, hq, hkv, d)
+    # quantise on the host with the product's own encoder (round-to-nearest absmax/127)
+    from clori_amd.backend import q8_0_encode_rows
+    k_blocks = q8_0_encode_rows(ORACLE.bf16_decode(k_rows))
+    v_blocks = q8_0_encode_rows(ORACLE.bf16_decode(v_rows))
+    return q, k_blocks, v_blocks, table, ctx, pool_pages
+
+
+def test_q8_0_paged_decode_matches_cpu_on_same_bytes(backend):
+    rng = np.random.default_rng(4)
+    contexts = [1, 15, 16, 17, 100, 333, 1024, 1025, 4097]
+    q, k_blocks, v_blocks, table, ctx, pool_pages = make_q8_case(rng, contexts, 32, 8)
+    got, lse, facts = run_paged(backend, q, k_blocks, v_blocks, table, ctx, 8, pool_pages,
+                                storage=B.KV_Q8_0)
+    rc, ref, _, ref_lse = ORACLE.paged_decode(q, k_blocks, v_blocks, table, ctx, 8, 16, q8=True)
+    assert rc == 0
+    assert_close_bf16(got, ref, "q8_0 paged")
+    assert_lse(lse, ref_lse, "q8_0 paged")
+    assert facts.kernel_launches == 2
+
+
+def test_q8_0_paged_placement_invariance_and_garbage_tail(backend):
+    rng = np.random.default_rng(44)
+    contexts = [40, 700, 129]
+    q, k_blocks, v_blocks, table, ctx, pool_pages = make_q8_case(rng, contexts, 8, 2)
+    got, lse, _ = run_paged(backend, q, k_blocks, v_blocks, table, ctx, 2, pool_pages,
+                            storage=B.KV_Q8_0)
+    perm = rng.permutation(pool_pages)
+    k2, v2 = np.empty_like(k_blocks), np.empty_like(v_blocks)
+    k2[perm], v2[perm] = k_blocks, v_blocks
+    got2, lse2, _ = run_paged(backend, q, k2, v2, perm[table].astype(np.int32), ctx, 2,
+                              pool_pages, storage=B.KV_Q8_0)
+    assert np.array_equal(got, got2) and np.array_equal(lse, lse2)
+    # rows past each context filled with 0xFF bytes (NaN scales, -1 codes) must not matter
+    k3, v3 = k_blocks.copy(), v_blocks.copy()
+    for s, c in enumerate(contexts):
+        last = table[s, (c - 1) // 16]
+        k3[last, c % 16 or 16:] = 0xFF
+        v3[last, c % 16 or 16:] = 0xFF
+    got3, lse3, _ = run_paged(backend, q, k3, v3, table, ctx, 2, pool_pages, storage=B.KV_Q8_0)
+    assert np.array_equal(got, got3) and np.array_equal(lse, lse3)
+
+
+def test_config4_shape_sample(backend):
+    """BASELINE config 4 at reduced session count: contexts uniform in [4096,32768], K/V as
+    GGUF Q8_0 blocks quantised on the host from N(0,1) bf16 values, seed 4."""
+    rng = np.random.default_rng(4)
+    contexts = [int(c) for c in rng.integers(4096, 32769, size=3)]
+    q, k_blocks, v_blocks, table, ctx, pool_pages = make_q8_case(rng, contexts, 32, 8)
+    got, lse, _ = run_paged(backend, q, k_blocks, v_blocks, table, ctx, 8, pool_pages,
+                            storage=B.KV_Q8_0)
+    rc, ref, _, ref_lse = ORACLE.paged_decode(q, k_blocks, v_blocks, table, ctx, 8, 16, q8=True)
+    assert rc == 0
+    assert_close_bf16(got, ref, "config4")
+    assert_lse(lse, ref_lse, "config4")
