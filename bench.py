@@ -157,7 +157,32 @@ def workload_decode1(backend, rng, steps, warmup):
                 launches=int(facts.kernel_launches), dominant_kernel="yvex_rocm_decode_rows_bf16")
 
 
+def workload_prefill2(backend, rng, steps, warmup):
+    t, hq, hkv, d = 2048, 40, 8, 128
+    sq = rng.uniform(0.5, 1.5, size=(1, hq, 1)).astype(np.float32)
+    skv = rng.uniform(0.5, 1.5, size=(1, hkv, 1)).astype(np.float32)
+    qv = bf16_bits(rng.standard_normal((t, hq, d), dtype=np.float32) * sq)
+    kv = bf16_bits(rng.standard_normal((t, hkv, d), dtype=np.float32) * skv)
+    vv = bf16_bits(rng.standard_normal((t, hkv, d), dtype=np.float32) * skv)
+    q = backend.tensor("q", B.DTYPE_BF16, (t, hq, d), qv)
+    k = backend.tensor("k", B.DTYPE_BF16, (t, hkv, d), kv)
+    v = backend.tensor("v", B.DTYPE_BF16, (t, hkv, d), vv)
+    out = backend.tensor("out", B.DTYPE_BF16, (t, hq, d))
+    req = backend.attention_requirement(t, t, hq, hkv, d, causal=True, dtype=B.DTYPE_BF16,
+                                        contract=B.NUMERIC_BF16_F32_ACCUMULATE)
+    run = lambda: backend.attention_execute(req, q, k, v, out)  # noqa: E731
+    facts = run()
+    ms, wall = time_steps(backend, run, steps, warmup)
+    flops = 4 * d * hq * t * (t + 1) // 2      # causal-useful multiply-adds * 2, QK^T and PV
+    return dict(name="prefill2",
+                workload="causal GQA prefill: batch 1, seq 2048, 40/8 heads, d=128, bf16",
+                bound="mfma", flops=flops, algorithmic_bytes=(2 * t * hq * d + 2 * t * hkv * d) * 2,
+                ms=ms, wall_ms=wall, launches=int(facts.kernel_launches),
+                dominant_kernel="yvex_rocm_prefill_bf16")
+
+
 WORKLOADS = {
+    "prefill2": workload_prefill2,
     "decode1": workload_decode1,
     "paged3": lambda b, r, s, w: workload_paged(b, r, s, w, q8=False),
     "paged4": lambda b, r, s, w: workload_paged(b, r, s, w, q8=True),

@@ -22,6 +22,7 @@ enum {
     ROCM_GROUP_MAX = 16,
     ROCM_CHUNK_MIN = 64,
     ROCM_CHUNK_MAX = 1024,
+    ROCM_PREFILL_ROWS = 256,     /* query rows per workgroup of the prefill kernel */
     ROCM_WORK_ALIGNMENT = 256    /* src/backend/cuda/transformer.c:17 */
 };
 
@@ -397,8 +398,42 @@ static int attention_execute_common(yvex_backend *backend,
         job.scale = 1.0f / sqrtf((float)r->head_dimension);
         rc = decode_run(backend, &job, "rocm.transformer.gqa.decode", facts, err);
     } else {
-        rc = refuse(err, YVEX_ERR_UNSUPPORTED, where,
-                    "bf16 multi-token attention is not admitted by this kernel bundle");
+        yvex_rocm_prefill_params params;
+        const unsigned long long q_tiles = (r->query_tokens + ROCM_PREFILL_ROWS - 1ull) /
+                                           ROCM_PREFILL_ROWS;
+        memset(&params, 0, sizeof(params));
+        params.q = (const uint16_t *)request->query->data;
+        params.k = (const uint16_t *)request->key->data;
+        params.v = (const uint16_t *)request->value->data;
+        params.out = (uint16_t *)request->output->data;
+        params.lse = lse ? (float *)lse->data : NULL;
+        params.status = state->device_status;
+        params.q_stride = q_stride;
+        params.k_stride = k_stride;
+        params.v_stride = v_stride;
+        params.query_tokens = (uint32_t)r->query_tokens;
+        params.kv_tokens = (uint32_t)r->key_value_tokens;
+        params.query_start = (uint32_t)r->query_start;
+        params.query_heads = (uint32_t)r->query_heads;
+        params.kv_heads = (uint32_t)r->key_value_heads;
+        params.head_dim = (uint32_t)r->head_dimension;
+        params.causal = (uint32_t)causal;
+        params.scale_log2 = (1.0f / sqrtf((float)r->head_dimension)) * 1.4426950408889634f;
+        backend_workspace_reset(backend);
+        if (r->query_heads > 65535ull || q_tiles > 65535ull)
+            return refuse(err, YVEX_ERR_BOUNDS, where,
+                          "prefill geometry exceeds admitted launch range");
+        rc = yvex_rocm_launch(backend, YVEX_ROCM_FN_PREFILL_BF16,
+                              YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_BF16,
+                              (unsigned int)r->query_heads, (unsigned int)q_tiles, 1u, 256u, 0u,
+                              &params, "rocm.transformer.gqa.prefill", err);
+        if (rc == YVEX_OK) {
+            facts->kernel_launches = 1ull;
+            facts->accelerated_matrix_launches = 1ull;
+            facts->compulsory_memory_facts_available = 1;
+            rc = yvex_rocm_complete(backend, YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_BF16,
+                                    "rocm.transformer.gqa.prefill", facts, err);
+        }
     }
     if (rc != YVEX_OK) return rc;
     request->output->is_written = 1;
