@@ -181,11 +181,42 @@ def workload_prefill2(backend, rng, steps, warmup):
                 dominant_kernel="yvex_rocm_prefill_bf16")
 
 
+def workload_mla5(backend, rng, steps, warmup):
+    batch, heads, kd, vd, page, ctx = 16, 128, 576, 512, 64, 8192
+    pages_each = ctx // page
+    pool_pages = batch * pages_each
+    table = rng.permutation(pool_pages).astype(np.int32).reshape(batch, pages_each)
+    contexts = np.full(batch, ctx, dtype=np.int32)
+    pool = backend.tensor("latent-pages", B.DTYPE_BF16, (pool_pages, page, kd),
+                          random_bf16(rng, pool_pages * page * kd))
+    q = backend.tensor("q", B.DTYPE_BF16, (batch, heads, kd), random_bf16(rng, batch * heads * kd))
+    tt = backend.tensor("table", B.DTYPE_I32, table.shape, table)
+    tc = backend.tensor("ctx", B.DTYPE_I32, contexts.shape, contexts)
+    out = backend.tensor("out", B.DTYPE_BF16, (batch, heads, vd))
+    lse = backend.tensor("lse", B.DTYPE_F32, (batch, heads))
+    req = backend.mla_requirement(batch, heads, kd, vd, page, pool_pages, pages_each, ctx)
+    work = backend.tensor("workspace", B.DTYPE_I8, (backend.mla_decode_workspace_required(req),))
+    backend.workspace_attach(work)
+    run = lambda: backend.mla_decode_execute(req, q, pool, tt, tc, out, lse)  # noqa: E731
+    facts = run()
+    ms, wall = time_steps(backend, run, steps, warmup)
+    backend.workspace_detach()
+    algo = batch * ctx * kd * 2 + batch * heads * (kd + vd) * 2 + table.size * 4 + batch * heads * 4
+    assert np.all(np.isfinite(lse.read()))
+    return dict(name="mla5",
+                workload="absorbed MLA decode: batch 16, 128 heads, latent 512 + rope 64, "
+                         "context 8192 in 64-token pages",
+                bound="hbm", algorithmic_bytes=algo, flops=batch * heads * ctx * 2 * (kd + vd),
+                ms=ms, wall_ms=wall, launches=int(facts.kernel_launches),
+                dominant_kernel="yvex_rocm_mla_decode_bf16")
+
+
 WORKLOADS = {
     "prefill2": workload_prefill2,
     "decode1": workload_decode1,
     "paged3": lambda b, r, s, w: workload_paged(b, r, s, w, q8=False),
     "paged4": lambda b, r, s, w: workload_paged(b, r, s, w, q8=True),
+    "mla5": workload_mla5,
 }
 SEEDS = {"decode1": 1, "prefill2": 2, "paged3": 3, "paged4": 4, "mla5": 5}
 

@@ -301,6 +301,13 @@ class Backend:
         r.max_context_tokens, r.numeric_contract, r.deterministic = max_context, contract, deterministic
         return r
 
+    def mla_decode_workspace_required(self, requirement):
+        out, err = B.ull(0), B.Error()
+        ops = self.rocm_attention_operations()
+        _check(ops.mla_decode_workspace_required(C.byref(requirement), C.byref(out),
+                                                 C.byref(err)), err)
+        return out.value
+
     def mla_decode_execute(self, requirement, query, latent_pages, page_table, context, output,
                            lse=None):
         ops = self.rocm_attention_operations()

@@ -575,24 +575,164 @@ static int rocm_paged_decode_execute(yvex_backend *backend,
 
 /* --------------------------------------------------------- MLA decode ---- */
 
+enum { ROCM_MLA_HEADS = 128, ROCM_MLA_KEY_DIM = 576, ROCM_MLA_VALUE_DIM = 512,
+       ROCM_MLA_PAGE_TOKENS = 64 };
+
+static int mla_validate(const yvex_rocm_mla_decode_requirement *r, const char *where,
+                        yvex_error *err)
+{
+    unsigned long long capacity;
+    if (!r || !r->batch || !r->heads || !r->key_dimension || !r->value_dimension ||
+        r->value_dimension > r->key_dimension || !r->page_tokens || !r->pool_pages ||
+        !r->page_table_stride || !r->max_context_tokens ||
+        !yvex_core_u64_mul(r->page_table_stride, r->page_tokens, &capacity) ||
+        r->max_context_tokens > capacity)
+        return refuse(err, YVEX_ERR_INVALID_ARG, where, "complete MLA decode geometry is required");
+    if (r->heads != ROCM_MLA_HEADS || r->key_dimension != ROCM_MLA_KEY_DIM ||
+        r->value_dimension != ROCM_MLA_VALUE_DIM || r->page_tokens != ROCM_MLA_PAGE_TOKENS ||
+        r->numeric_contract != YVEX_TRANSFORMER_ATTENTION_NUMERIC_BF16_F32_ACCUMULATE ||
+        !r->deterministic || r->pool_pages > 0x7fffffffull || capacity > 0x7fffffffull ||
+        r->batch > 65535ull)
+        return refuse(err, YVEX_ERR_UNSUPPORTED, where,
+                      "ROCm MLA decode requires 128 heads, a 512+64 latent row, 64-token pages "
+                      "and the deterministic bf16/fp32-accumulate contract");
+    yvex_error_clear(err);
+    return YVEX_OK;
+}
+
+/* Chunks are a function of the request geometry only: about one workgroup per compute
+ * unit of a 256-CU part, in whole pages. */
+static unsigned int mla_chunk_tokens(const yvex_rocm_mla_decode_requirement *r)
+{
+    const char *forced = getenv("YVEX_ROCM_MLA_CHUNK");
+    unsigned long long per_batch = 256ull / r->batch ? 256ull / r->batch : 1ull;
+    unsigned long long chunk = (r->max_context_tokens + per_batch - 1ull) / per_batch;
+    if (forced && atoi(forced) >= ROCM_MLA_PAGE_TOKENS) chunk = (unsigned long long)atoi(forced);
+    chunk = align_up(chunk, ROCM_MLA_PAGE_TOKENS);
+    return (unsigned int)chunk;
+}
+
 static int rocm_mla_decode_workspace_required(const yvex_rocm_mla_decode_requirement *r,
                                               unsigned long long *bytes, yvex_error *err)
 {
-    (void)r;
+    static const char where[] = "rocm.attention.mla.workspace";
+    unsigned long long acc = 0ull, total = 0ull, chunk, max_chunks;
+    int rc;
     if (bytes) *bytes = 0ull;
-    return refuse(err, YVEX_ERR_UNSUPPORTED, "rocm.attention.mla.workspace",
-                  "absorbed MLA decode is not admitted by this kernel bundle");
+    rc = mla_validate(r, where, err);
+    if (rc != YVEX_OK) return rc;
+    if (!bytes) return refuse(err, YVEX_ERR_INVALID_ARG, where, "workspace byte output is required");
+    chunk = mla_chunk_tokens(r);
+    max_chunks = (r->max_context_tokens + chunk - 1ull) / chunk;
+    if (!decode_workspace_bytes(r->batch, max_chunks, r->heads, r->value_dimension, &acc, &total))
+        return refuse(err, YVEX_ERR_BOUNDS, where, "MLA workspace geometry overflowed");
+    *bytes = total;
+    yvex_error_clear(err);
+    return YVEX_OK;
 }
 
 static int rocm_mla_decode_execute(yvex_backend *backend,
                                    const yvex_rocm_mla_decode_request *request,
                                    yvex_backend_operation_facts *facts, yvex_error *err)
 {
-    (void)backend;
-    (void)request;
-    (void)facts;
-    return refuse(err, YVEX_ERR_UNSUPPORTED, "rocm.attention.mla",
-                  "absorbed MLA decode is not admitted by this kernel bundle");
+    static const char where[] = "rocm.attention.mla";
+    const yvex_backend_operation_variant variant = YVEX_BACKEND_VARIANT_ROCM_ATTENTION_MLA_BF16;
+    yvex_rocm_backend_state *state = yvex_rocm_state(backend);
+    const yvex_rocm_mla_decode_requirement *r;
+    yvex_rocm_mla_params kp;
+    yvex_rocm_decode_merge_params mp;
+    unsigned long long acc_bytes = 0ull, total = 0ull, max_chunks, chunk;
+    void *work = NULL;
+    yvex_error cleanup;
+    int owned = 0, rc, cleanup_rc;
+    if (!request || !request->query || !request->latent_pages || !request->page_table ||
+        !request->context_tokens || !request->output || !facts)
+        return refuse(err, YVEX_ERR_INVALID_ARG, where,
+                      "complete MLA decode tensors and result facts are required");
+    rc = backend_dispatch_admit(backend, where, err);
+    if (rc != YVEX_OK) return rc;
+    r = &request->requirement;
+    rc = mla_validate(r, where, err);
+    if (rc != YVEX_OK) return rc;
+    memset(facts, 0, sizeof(*facts));
+    if (!state ||
+        !view_ok(backend, request->query, YVEX_DTYPE_BF16, r->batch * r->heads * r->key_dimension, 1) ||
+        !view_ok(backend, request->latent_pages, YVEX_DTYPE_BF16,
+                 r->pool_pages * r->page_tokens * r->key_dimension, 1) ||
+        !view_ok(backend, request->page_table, YVEX_DTYPE_I32, r->batch * r->page_table_stride, 1) ||
+        !view_ok(backend, request->context_tokens, YVEX_DTYPE_I32, r->batch, 1) ||
+        !view_ok(backend, request->output, YVEX_DTYPE_BF16,
+                 r->batch * r->heads * r->value_dimension, 0) ||
+        (request->lse && !view_ok(backend, request->lse, YVEX_DTYPE_F32, r->batch * r->heads, 0)))
+        return refuse(err, YVEX_ERR_FORMAT, where,
+                      "query, latent pages, page table, context lengths and outputs must be "
+                      "written tensors of this backend with the declared geometry");
+    chunk = mla_chunk_tokens(r);
+    max_chunks = (r->max_context_tokens + chunk - 1ull) / chunk;
+    if (max_chunks > 0x7fffffffull ||
+        !decode_workspace_bytes(r->batch, max_chunks, r->heads, r->value_dimension, &acc_bytes,
+                                &total))
+        return refuse(err, YVEX_ERR_BOUNDS, where, "MLA decode geometry exceeds admitted range");
+    backend_workspace_reset(backend);
+    rc = yvex_rocm_temporary_acquire(backend, total, &work, &owned, where, err);
+    if (rc != YVEX_OK) return rc;
+    memset(&kp, 0, sizeof(kp));
+    kp.q = (const uint16_t *)request->query->data;
+    kp.pool = (const uint16_t *)request->latent_pages->data;
+    kp.page_table = (const int32_t *)request->page_table->data;
+    kp.context = (const int32_t *)request->context_tokens->data;
+    kp.part_acc = (float *)work;
+    kp.part_ml = (float *)((unsigned char *)work + acc_bytes);
+    kp.status = state->device_status;
+    kp.batch = (uint32_t)r->batch;
+    kp.heads = (uint32_t)r->heads;
+    kp.key_dim = (uint32_t)r->key_dimension;
+    kp.value_dim = (uint32_t)r->value_dimension;
+    kp.page_tokens = (uint32_t)r->page_tokens;
+    kp.pool_pages = (uint32_t)r->pool_pages;
+    kp.table_stride = (uint32_t)r->page_table_stride;
+    kp.chunk_tokens = (uint32_t)chunk;
+    kp.max_chunks = (uint32_t)max_chunks;
+    /* src/graph/core.c:604: scale = 1/sqrt(head_dimension), here over the 576-lane key */
+    kp.scale_log2 = (float)(1.4426950408889634 / sqrt((double)r->key_dimension));
+    rc = yvex_rocm_launch(backend, YVEX_ROCM_FN_MLA_DECODE_BF16, variant, (unsigned int)max_chunks,
+                          (unsigned int)r->batch, 1u, 256u, 0u, &kp, where, err);
+    if (rc == YVEX_OK) {
+        memset(&mp, 0, sizeof(mp));
+        mp.part_acc = kp.part_acc;
+        mp.part_ml = kp.part_ml;
+        mp.context = kp.context;
+        mp.out = (uint16_t *)request->output->data;
+        mp.lse = request->lse ? (float *)request->lse->data : NULL;
+        mp.status = state->device_status;
+        mp.sessions = kp.batch;
+        mp.query_heads = kp.heads;
+        mp.head_dim = kp.value_dim;
+        mp.chunk_tokens = kp.chunk_tokens;
+        mp.max_chunks = kp.max_chunks;
+        rc = yvex_rocm_launch(backend, YVEX_ROCM_FN_DECODE_MERGE, variant, (unsigned int)r->heads,
+                              (unsigned int)r->batch, 1u, (unsigned int)r->value_dimension, 0u, &mp,
+                              where, err);
+    }
+    if (rc == YVEX_OK) {
+        facts->kernel_launches = 2ull;
+        facts->accelerated_matrix_launches = 1ull;
+        facts->temporary_bytes = total;
+        facts->compulsory_memory_facts_available = 1;
+        rc = yvex_rocm_complete(backend, variant, where, facts, err);
+    }
+    yvex_error_clear(&cleanup);
+    cleanup_rc = yvex_rocm_temporary_release(backend, work, total, owned, &cleanup);
+    backend_workspace_reset(backend);
+    if (rc == YVEX_OK && cleanup_rc != YVEX_OK) {
+        rc = cleanup_rc;
+        if (err) *err = cleanup;
+    }
+    if (rc != YVEX_OK) return rc;
+    request->output->is_written = 1;
+    if (request->lse) request->lse->is_written = 1;
+    yvex_error_clear(err);
+    return YVEX_OK;
 }
 
 /* ---------------------------------------------------------- op tables ---- */

@@ -386,7 +386,7 @@ yvex_rocm_decode_rows_bf16(const yvex_rocm_decode_params p)
 
 // Log-sum-exp merge of the chunk partials of one (session, query head); one thread per
 // output lane.  grid = (query_heads, sessions), block = head_dim.
-extern "C" __global__ void __launch_bounds__(256)
+extern "C" __global__ void __launch_bounds__(512)
 yvex_rocm_decode_merge(const yvex_rocm_decode_merge_params p)
 {
     const uint32_t head = blockIdx.x, session = blockIdx.y, d = threadIdx.x;

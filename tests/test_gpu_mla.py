@@ -1,0 +1,88 @@
+"""GPU parity: absorbed-latent MLA decode against the shared-KV CPU restatement
+(src/graph/core.c:361-508 semantics), through the C ABI."""
+import numpy as np
+import pytest
+
+from clori_amd import binding as B
+from clori_amd.backend import YvexError
+from gpu_common import ORACLE, assert_close_bf16, assert_lse, backend, bf16_normal  # noqa: F401
+
+pytestmark = pytest.mark.gpu
+
+HEADS, KEY_DIM, VALUE_DIM, PAGE = 128, 576, 512, 64
+
+
+def make_case(rng, contexts, spare=2):
+    batch = len(contexts)
+    need = [(c + PAGE - 1) // PAGE for c in contexts]
+    pool_pages = sum(need) + spare
+    perm = rng.permutation(pool_pages).astype(np.int32)
+    table = np.zeros((batch, max(need) + 1), dtype=np.int32)
+    at = 0
+    for b, n in enumerate(need):
+        table[b, :n] = perm[at:at + n]
+        at += n
+    pool = bf16_normal(rng, (pool_pages, PAGE, KEY_DIM))
+    q = bf16_normal(rng, (batch, HEADS, KEY_DIM))
+    return q, pool, table, np.array(contexts, dtype=np.int32)
+
+
+def run_mla(backend, q, pool, table, ctx, max_context=None):
+    batch = q.shape[0]
+    req = backend.mla_requirement(batch, HEADS, KEY_DIM, VALUE_DIM, PAGE, pool.shape[0],
+                                  table.shape[1], max_context or int(table.shape[1] * PAGE))
+    out = backend.tensor("o", B.DTYPE_BF16, (batch, HEADS, VALUE_DIM))
+    lse = backend.tensor("lse", B.DTYPE_F32, (batch, HEADS))
+    facts = backend.mla_decode_execute(
+        req, backend.tensor("q", B.DTYPE_BF16, q.shape, q),
+        backend.tensor("pool", B.DTYPE_BF16, pool.shape, pool),
+        backend.tensor("table", B.DTYPE_I32, table.shape, table),
+        backend.tensor("ctx", B.DTYPE_I32, ctx.shape, ctx), out, lse)
+    return out.read(), lse.read(), facts
+
+
+def test_mla_decode_matches_shared_kv_oracle_ragged(backend):
+    rng = np.random.default_rng(5)
+    contexts = [1, 31, 32, 33, 64, 65, 500, 1300]
+    q, pool, table, ctx = make_case(rng, contexts)
+    got, lse, facts = run_mla(backend, q, pool, table, ctx)
+    rc, ref, _, ref_lse = ORACLE.mla_decode(q, pool, table, ctx, VALUE_DIM, PAGE)
+    assert rc == 0
+    assert_close_bf16(got, ref, "mla ragged")
+    assert_lse(lse, ref_lse, "mla ragged")
+    assert facts.kernel_launches == 2 and facts.device_synchronizations == 1
+
+
+def test_config5_shape_sample(backend):
+    """BASELINE config 5 at reduced batch: 128 heads, 512+64 latent, context 8192 in 64-token
+    pages, scale 1/sqrt(576), seed 5."""
+    rng = np.random.default_rng(5)
+    q, pool, table, ctx = make_case(rng, [8192, 8192])
+    got, lse, _ = run_mla(backend, q, pool, table, ctx, max_context=8192)
+    rc, ref, _, ref_lse = ORACLE.mla_decode(q, pool, table, ctx, VALUE_DIM, PAGE)
+    assert rc == 0
+    assert_close_bf16(got, ref, "config5")
+    assert_lse(lse, ref_lse, "config5")
+
+
+def test_mla_page_placement_invariance_and_refusals(backend):
+    rng = np.random.default_rng(55)
+    q, pool, table, ctx = make_case(rng, [200, 77])
+    got, lse, _ = run_mla(backend, q, pool, table, ctx)
+    perm = rng.permutation(pool.shape[0])
+    pool2 = np.empty_like(pool)
+    pool2[perm] = pool
+    got2, lse2, _ = run_mla(backend, q, pool2, perm[table].astype(np.int32), ctx)
+    assert np.array_equal(got, got2) and np.array_equal(lse, lse2)
+    bad = table.copy()
+    bad[0, 1] = pool.shape[0]
+    with pytest.raises(YvexError) as e:
+        run_mla(backend, q, pool, bad, ctx)
+    assert e.value.code == B.YVEX_ERR_BOUNDS
+    with pytest.raises(YvexError) as e:
+        run_mla(backend, q, pool, table, np.array([200, 0], np.int32))
+    assert e.value.code == B.YVEX_ERR_BOUNDS
+    req = backend.mla_requirement(2, 64, KEY_DIM, VALUE_DIM, PAGE, 8, 4, 256)
+    with pytest.raises(YvexError) as e:
+        backend.mla_decode_workspace_required(req)
+    assert e.value.code == B.YVEX_ERR_UNSUPPORTED
