@@ -339,7 +339,7 @@ def kv_pack_pages(rows, storage, is_value, kv_heads, head_dim=128, page_tokens=1
 
 
 def kv_unpack_pages(packed, storage, is_value, pool_pages, kv_heads, head_dim=128, page_tokens=16):
-    packed = np.ascontiguousarray(packed, dtype=np.uint8)
+    packed = np.ascontiguousarray(packed).reshape(-1).view(np.uint8)
     if storage == B.KV_BF16:
         rows = np.empty((pool_pages, page_tokens, kv_heads, head_dim), dtype=np.uint16)
     else:

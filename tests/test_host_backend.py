@@ -1,0 +1,571 @@
+"""Host-side behaviour of the C backend on a machine without a GPU: symbol export,
+fail-closed admission, argument-check order, bookkeeping, failure transitions and
+checked cleanup.  A stand-in HIP runtime (tests/fake_hip) is injected through
+YVEX_TEST_ROCM_DRIVER_LIBRARY; its kernel launches do nothing, so no numerics are
+tested here (those are the GPU tests)."""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+from clori_amd import binding as B
+from clori_amd.backend import (Backend, YvexError, kv_pack_pages, kv_unpack_pages, lib,
+                               q8_0_decode_rows, q8_0_encode_rows)
+from oracle_binding import Oracle
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+FAKE_DIR = os.path.join(ROOT, "tests", "fake_hip")
+FAKE_SO = os.path.join(FAKE_DIR, "libfakehip.so")
+ORACLE = Oracle()
+
+
+@pytest.fixture(scope="module", autouse=True)
+def fake_runtime():
+    subprocess.check_call(["gcc", "-std=c11", "-O1", "-fPIC", "-shared", "-I/opt/rocm/include",
+                           "-o", FAKE_SO, os.path.join(FAKE_DIR, "fake_hip.c")])
+    os.environ["YVEX_TEST_ROCM_DRIVER_LIBRARY"] = FAKE_SO
+    yield C.CDLL(FAKE_SO)
+    for name in list(os.environ):
+        if name.startswith(("YVEX_TEST_ROCM_", "FAKE_HIP_")):
+            del os.environ[name]
+
+
+@pytest.fixture
+def env():
+    """Sets variables for one test and restores them afterwards."""
+    touched = []
+
+    def setter(name, value):
+        touched.append((name, os.environ.get(name)))
+        if value is None:
+            os.environ.pop(name, None)
+        else:
+            os.environ[name] = value
+    yield setter
+    for name, old in reversed(touched):
+        if old is None:
+            os.environ.pop(name, None)
+        else:
+            os.environ[name] = old
+
+
+def f32(backend, name, shape, data=None):
+    return backend.tensor(name, B.DTYPE_F32, shape,
+                          None if data is None else np.asarray(data, dtype=np.float32))
+
+
+def written(backend, name, dtype, shape):
+    t = backend.tensor(name, dtype, shape)
+    t.zero()
+    return t
+
+
+# ------------------------------------------------------------------ exports ----
+
+def test_library_exports_every_declared_symbol():
+    library = lib()
+    for name in B.EXPORTED_SYMBOLS:
+        assert hasattr(library, name), name
+    header = open(os.path.join(ROOT, "include", "yvex_rocm.h")).read()
+    for name in B.EXPORTED_SYMBOLS:
+        assert name + "(" in header, "declared in binding but not in the header: " + name
+
+
+def test_names_match_the_reference_vocabulary():
+    library = lib()
+    assert library.yvex_status_name(B.YVEX_ERR_BOUNDS) == b"YVEX_ERR_BOUNDS"
+    assert library.yvex_backend_kind_name(B.KIND_ROCM) == b"rocm"
+    assert library.yvex_backend_status_name(B.STATUS_CONTEXT_READY) == b"context-ready"
+    assert library.yvex_backend_operation_variant_name(13) == b"attention-causal-f32"
+    assert library.yvex_backend_operation_variant_name(16) == b"encoded-attention"
+    assert library.yvex_backend_capability_reason_name(4) == b"kernel-bundle-absent"
+    assert library.yvex_backend_capability_reason_name(6) == b"required-function-missing"
+    assert library.yvex_backend_capability_name(B.CAP_OP_ATTENTION) == b"op_attention"
+    kind, err = C.c_int(-1), B.Error()
+    assert library.yvex_backend_kind_parse(b"rocm", C.byref(kind), C.byref(err)) == 0
+    assert kind.value == B.KIND_ROCM
+    assert library.yvex_backend_kind_parse(b"vulkan", C.byref(kind), C.byref(err)) == \
+        B.YVEX_ERR_INVALID_ARG and b"unknown backend kind: vulkan" in err.message
+
+
+def test_other_kinds_are_not_implemented_here():
+    for kind in (B.KIND_CPU, B.KIND_CUDA, B.KIND_METAL):
+        with pytest.raises(YvexError) as e:
+            Backend(kind=kind)
+        assert e.value.code == B.YVEX_ERR_UNSUPPORTED and "is not implemented" in e.value.message
+
+
+def test_open_without_a_device_fails_closed(env):
+    env("FAKE_HIP_DEVICES", "0")
+    with pytest.raises(YvexError) as e:
+        Backend()
+    assert e.value.code == B.YVEX_ERR_UNSUPPORTED
+    env("FAKE_HIP_DEVICES", None)
+    env("FAKE_HIP_INIT", "fail")
+    with pytest.raises(YvexError) as e:
+        Backend()
+    assert e.value.code == B.YVEX_ERR_UNSUPPORTED
+    env("FAKE_HIP_INIT", None)
+    env("YVEX_TEST_ROCM_DRIVER_LIBRARY", "/nonexistent/libhip.so")
+    with pytest.raises(YvexError) as e:
+        Backend()
+    assert e.value.code == B.YVEX_ERR_UNSUPPORTED and "unavailable" in e.value.message
+    assert lib().yvex_backend_rocm_available() == 0
+
+
+# ---------------------------------------------------------- admission ----
+
+def test_ready_backend_publishes_attention_only():
+    with Backend() as b:
+        report = b.report()
+        assert b.status == B.STATUS_READY and report.bundle_admitted and report.bundle_built
+        assert report.architecture == b"gfx950" and report.function_count >= 9
+        assert report.device_name == b"fake-gfx950"
+        for variant in (B.VARIANT_TENSOR_ALLOC, B.VARIANT_TENSOR_COPY,
+                        B.VARIANT_ATTENTION_CAUSAL_F32, B.VARIANT_ATTENTION_NONCAUSAL_F32,
+                        B.VARIANT_ROCM_GQA_F32, B.VARIANT_ROCM_GQA_BF16, B.VARIANT_ROCM_PAGED_BF16,
+                        B.VARIANT_ROCM_PAGED_Q8_0, B.VARIANT_ROCM_MLA_BF16):
+            r = b.query_capability(variant)
+            assert r.state == B.CAPABILITY_SUPPORTED and r.reason == B.REASON_NONE, variant
+            assert r.context_available and r.kernel_bundle_available and r.function_available
+        for variant in (B.VARIANT_MATMUL_F32, B.VARIANT_ATTENTION_ENCODED, 5, 9, 15):
+            r = b.query_capability(variant)      # embed, rope, qtype, ... : not this backend's
+            assert r.state == B.CAPABILITY_UNSUPPORTED and r.reason == B.REASON_VARIANT_UNSUPPORTED
+        assert b.supports(B.CAP_TENSOR_ALLOC) and b.supports(B.CAP_TENSOR_READ_WRITE)
+        assert b.supports(B.CAP_OP_ATTENTION) and not b.supports(3)
+        r = b.query_capability(B.VARIANT_ROCM_PAGED_Q8_0)
+        assert (r.input_dtype, r.weight_dtype, r.output_dtype) == (B.DTYPE_BF16, B.DTYPE_Q8_0,
+                                                                   B.DTYPE_BF16)
+        with pytest.raises(YvexError) as e:
+            b.query_capability(40)
+        assert e.value.code == B.YVEX_ERR_INVALID_ARG
+        assert b.transformer_operations() is not None
+        assert b.rocm_attention_operations() is not None
+        info = b.device_info()
+        assert info.kind == B.KIND_ROCM and info.name == b"fake-gfx950"
+
+
+@pytest.mark.parametrize("injected,reason_for_attention", [
+    ("module", B.REASON_KERNEL_BUNDLE_REJECTED),
+    ("symbol", B.REASON_FUNCTION_MISSING),
+    ("yvex_rocm_decode_merge", B.REASON_KERNEL_BUNDLE_REJECTED),
+])
+def test_rejected_bundle_publishes_nothing(env, fake_runtime, injected, reason_for_attention):
+    env("YVEX_TEST_ROCM_BUNDLE_FAILURE", injected)
+    with Backend() as b:
+        assert b.status == B.STATUS_CONTEXT_READY
+        report = b.report()
+        assert not report.bundle_admitted and report.function_count == 0 and report.rejection
+        assert fake_runtime.fake_hip_live_modules() == 0          # everything loaded was unloaded
+        r = b.query_capability(B.VARIANT_ATTENTION_CAUSAL_F32)
+        assert r.state == B.CAPABILITY_FAILED and r.reason == reason_for_attention
+        if injected == "yvex_rocm_decode_merge":
+            r = b.query_capability(B.VARIANT_ROCM_PAGED_BF16)      # the variant that lost a symbol
+            assert r.reason == B.REASON_FUNCTION_MISSING
+        assert b.transformer_operations() is None and b.rocm_attention_operations() is None
+        assert not b.supports(B.CAP_OP_ATTENTION) and b.supports(B.CAP_TENSOR_ALLOC)
+        t = f32(b, "x", (4,), [1, 2, 3, 4])                        # tensor traffic still works
+        assert np.array_equal(t.read(), [1, 2, 3, 4])
+        q, k = f32(b, "q", (4,), np.ones(4)), f32(b, "k", (3, 4), np.ones((3, 4)))
+        s, o = f32(b, "s", (3,)), f32(b, "o", (4,))
+        with pytest.raises(YvexError) as e:
+            b.op_attention(q, k, k, 3, 0, 0.5, True, s, s, o)
+        assert e.value.code == B.YVEX_ERR_BACKEND and "refused" in e.value.message
+        assert not o.is_written
+
+
+def test_missing_function_in_runtime_rejects_the_whole_bundle(env):
+    env("FAKE_HIP_MISSING_FUNCTION", "yvex_rocm_prefill_bf16")
+    with Backend() as b:
+        assert b.status == B.STATUS_CONTEXT_READY
+        assert b.query_capability(B.VARIANT_ROCM_GQA_BF16).reason == B.REASON_FUNCTION_MISSING
+        assert b.query_capability(B.VARIANT_ROCM_MLA_BF16).reason == \
+            B.REASON_KERNEL_BUNDLE_REJECTED
+        assert b"yvex_rocm_prefill_bf16" in b.report().rejection
+
+
+def test_bundle_absent_build_reports_absent_and_refuses(tmp_path):
+    out = tmp_path / "libyvex_rocm_nobundle.so"
+    subprocess.check_call(["make", "-s", "-C", os.path.join(ROOT, "clori_amd", "csrc"), "BUNDLE=0",
+                           "BUILD=%s" % (tmp_path / "build"), "OUT=%s" % out])
+    script = """
+import sys, ctypes as C
+sys.path.insert(0, %r)
+from clori_amd import binding as B
+lib = B.load(%r)
+handle, err = C.c_void_p(), B.Error()
+opts = B.BackendOptions(B.KIND_ROCM, None, 0)
+assert lib.yvex_backend_open(C.byref(handle), C.byref(opts), C.byref(err)) == 0
+assert lib.yvex_backend_status_of(handle) == B.STATUS_CONTEXT_READY
+res = B.CapabilityResult()
+assert lib.yvex_backend_query_capability(handle, B.VARIANT_ATTENTION_CAUSAL_F32, C.byref(res), C.byref(err)) == 0
+assert res.state == B.CAPABILITY_UNSUPPORTED and res.reason == B.REASON_KERNEL_BUNDLE_ABSENT
+assert lib.yvex_backend_query_capability(handle, B.VARIANT_TENSOR_ALLOC, C.byref(res), C.byref(err)) == 0
+assert res.state == B.CAPABILITY_SUPPORTED
+assert not lib.yvex_backend_transformer_operations_get(handle)
+rep = B.RocmReport()
+lib.yvex_backend_rocm_report_get(handle, C.byref(rep), C.byref(err))
+assert not rep.bundle_built and rep.image_count == 0
+assert lib.yvex_backend_close_checked(C.byref(handle), C.byref(err)) == 0
+print("absent-ok")
+""" % (ROOT, str(out))
+    result = subprocess.run(["python3", "-c", script], capture_output=True, text=True,
+                            env=dict(os.environ))
+    assert "absent-ok" in result.stdout, result.stderr
+
+
+# ------------------------------------------------------------- tensors ----
+
+def test_tensor_lifecycle_and_accounting(fake_runtime):
+    with Backend(memory_limit_bytes=1 << 20) as b:
+        base = fake_runtime.fake_hip_live_allocations()
+        t = f32(b, "weights", (16, 4))
+        assert np.all(t.read() == 0) and not t.is_written          # read before write is zero
+        t.write(np.arange(64, dtype=np.float32))
+        assert t.is_written and np.array_equal(t.read().ravel(), np.arange(64))
+        stats = b.memory_stats()
+        assert stats.allocated_bytes == 256 and stats.allocation_count == 1
+        assert stats.h2d_bytes == 256 and stats.d2h_bytes == 512 and stats.memory_limit_bytes == 1 << 20
+        err = B.Error()
+        short = np.zeros(3, np.float32)
+        rc = lib().yvex_backend_tensor_write(b.handle, t.handle, short.ctypes.data, 12, C.byref(err))
+        assert rc == B.YVEX_ERR_BOUNDS and b"does not match tensor bytes" in err.message
+        with pytest.raises(YvexError) as e:
+            b.tensor("too-big", B.DTYPE_I8, (1 << 21,))
+        assert e.value.code == B.YVEX_ERR_NOMEM and "memory limit" in e.value.message
+        with pytest.raises(YvexError) as e:
+            b.tensor("zero-dim", B.DTYPE_F32, (0,), nbytes=4)
+        assert e.value.code == B.YVEX_ERR_INVALID_ARG
+        desc, handle = B.TensorDesc(b"rank5", B.DTYPE_F32, 5), B.TensorP()
+        desc.bytes = 4
+        assert lib().yvex_backend_tensor_alloc(b.handle, C.byref(desc), C.byref(handle),
+                                               C.byref(err)) == B.YVEX_ERR_INVALID_ARG
+        u = f32(b, "copy", (16, 4))
+        rc = lib().yvex_backend_tensor_copy(b.handle, u.handle, t.handle, C.byref(err))
+        assert rc == 0 and np.array_equal(u.read(), t.read())
+        v = f32(b, "other-shape", (64,))
+        assert lib().yvex_backend_tensor_copy(b.handle, v.handle, t.handle, C.byref(err)) == \
+            B.YVEX_ERR_BOUNDS
+        with Backend() as other:                                     # a foreign tensor is refused
+            foreign = f32(other, "foreign", (16, 4))
+            assert lib().yvex_backend_tensor_copy(b.handle, foreign.handle, t.handle,
+                                                  C.byref(err)) == B.YVEX_ERR_STATE
+            assert not lib().yvex_backend_tensor_owned_by(b.handle, foreign.handle)
+        t.release()
+        assert t.handle is None
+        stats = b.memory_stats()
+        assert stats.allocation_count == 2 and stats.release_events == 1
+        assert stats.peak_allocated_bytes >= 768
+        assert fake_runtime.fake_hip_live_allocations() == base + 2
+
+
+def test_f32_subview_matches_reference_rules():
+    with Backend() as b:
+        t = f32(b, "row", (8, 4), np.arange(32))
+        view = B.DeviceTensor()
+        assert lib().yvex_backend_tensor_f32_subview(t.handle, 4, 8, C.byref(view)) == 1
+        assert view.rank == 1 and view.dims[0] == 8 and view.bytes == 32
+        assert view.data == t.handle.contents.data + 16
+        assert lib().yvex_backend_tensor_f32_subview(t.handle, 30, 8, C.byref(view)) == 0
+        assert lib().yvex_backend_tensor_f32_subview(t.handle, 0, 0, C.byref(view)) == 0
+
+
+# ------------------------------------------------- operation admission ----
+
+def test_bounded_primitive_refusal_order_and_facts(fake_runtime):
+    with Backend() as b:
+        q, k, v = f32(b, "q", (4,), np.ones(4)), f32(b, "k", (3, 4), np.ones((3, 4))), \
+            f32(b, "v", (3, 4), np.ones((3, 4)))
+        s, p, o = f32(b, "s", (3,)), f32(b, "p", (3,)), f32(b, "o", (4,))
+        before = fake_runtime.fake_hip_launches()
+        b.op_attention(q, k, v, 3, 2, 0.5, True, s, p, o)
+        assert fake_runtime.fake_hip_launches() == before + 1
+        assert o.is_written and s.is_written and p.is_written
+        cases = [((0, 0, 0.5), B.YVEX_ERR_INVALID_ARG), ((3, 3, 0.5), B.YVEX_ERR_BOUNDS),
+                 ((3, 9, float("nan")), B.YVEX_ERR_BOUNDS),      # position is checked before scale
+                 ((3, 0, float("nan")), B.YVEX_ERR_INVALID_ARG), ((3, 0, 0.0), B.YVEX_ERR_INVALID_ARG),
+                 ((3, 0, -2.0), B.YVEX_ERR_INVALID_ARG)]
+        for (seq, pos, scale), code in cases:
+            with pytest.raises(YvexError) as e:
+                b.op_attention(q, k, v, seq, pos, scale, True, s, p, o)
+            assert e.value.code == code, (seq, pos, scale)
+        with pytest.raises(YvexError) as e:                          # dtype before shape
+            b.op_attention(q, k, v, 3, 0, 0.5, True, s, p, b.tensor("h", B.DTYPE_BF16, (9,)))
+        assert e.value.code == B.YVEX_ERR_UNSUPPORTED
+        with pytest.raises(YvexError) as e:
+            b.op_attention(q, k, v, 3, 0, 0.5, True, s, p, f32(b, "o5", (5,)))
+        assert e.value.code == B.YVEX_ERR_FORMAT and "output must have dims" in e.value.message
+        with pytest.raises(YvexError) as e:
+            b.op_attention(q, f32(b, "k2", (4, 4)), v, 3, 0, 0.5, True, s, p, o)
+        assert e.value.code == B.YVEX_ERR_FORMAT
+        with pytest.raises(YvexError) as e:
+            b.op_attention(f32(b, "q2", (2, 2)), k, v, 3, 0, 0.5, True, s, p, o)
+        assert e.value.code == B.YVEX_ERR_FORMAT
+        with Backend() as other:
+            with pytest.raises(YvexError) as e:
+                b.op_attention(f32(other, "q", (4,)), k, v, 3, 0, 0.5, True, s, p, o)
+            assert e.value.code == B.YVEX_ERR_STATE
+        err = B.Error()
+        rc = lib().yvex_backend_op_attention(b.handle, None, k.handle, v.handle, 3, 0, 0.5, 1,
+                                             s.handle, p.handle, o.handle, C.byref(err))
+        assert rc == B.YVEX_ERR_INVALID_ARG
+
+
+def test_attention_execute_contracts_facts_and_workspace(fake_runtime):
+    with Backend() as b:
+        # exact F32: one launch, one synchronisation, a 4-byte status read-back
+        req = b.attention_requirement(3, 5, 4, 2, 64, query_start=2)
+        q, k = written(b, "q", B.DTYPE_F32, (3, 4, 64)), written(b, "k", B.DTYPE_F32, (5, 2, 64))
+        out = b.tensor("o", B.DTYPE_F32, (3, 4, 64))
+        facts = b.attention_execute(req, q, k, k, out)
+        assert (facts.kernel_launches, facts.device_synchronizations, facts.d2h_bytes,
+                facts.download_count) == (1, 1, 4, 1) and out.is_written
+        assert b.attention_workspace_required(req) == 0
+        # bf16 decode: two launches, workspace == planned bytes, attached workspace is used
+        req = b.attention_requirement(1, 4096, 32, 8, 128, query_start=4095, dtype=B.DTYPE_BF16,
+                                      contract=B.NUMERIC_BF16_F32_ACCUMULATE)
+        planned = b.attention_workspace_required(req)
+        assert planned > 0 and planned % 256 == 0
+        qb = written(b, "q", B.DTYPE_BF16, (1, 32, 128))
+        kb = written(b, "k", B.DTYPE_BF16, (4096, 8, 128))
+        ob = b.tensor("o", B.DTYPE_BF16, (1, 32, 128))
+        live = fake_runtime.fake_hip_live_allocations()
+        facts = b.attention_execute(req, qb, kb, kb, ob)
+        assert facts.kernel_launches == 2 and facts.temporary_bytes == planned
+        assert fake_runtime.fake_hip_live_allocations() == live      # temporary released
+        work = b.tensor("workspace", B.DTYPE_I8, (planned,))
+        b.workspace_attach(work)
+        with pytest.raises(YvexError) as e:
+            b.workspace_attach(work)
+        assert e.value.code == B.YVEX_ERR_STATE
+        live = fake_runtime.fake_hip_live_allocations()
+        stats_before = b.memory_stats().allocation_events
+        facts = b.attention_execute(req, qb, kb, kb, ob)
+        assert facts.temporary_bytes == planned
+        assert b.memory_stats().allocation_events == stats_before    # no counted temporary
+        b.workspace_detach()
+        # bf16 prefill: one launch
+        req = b.attention_requirement(300, 300, 8, 2, 128, dtype=B.DTYPE_BF16,
+                                      contract=B.NUMERIC_BF16_F32_ACCUMULATE)
+        qp, kp = written(b, "q", B.DTYPE_BF16, (300, 8, 128)), written(b, "k", B.DTYPE_BF16, (300, 2, 128))
+        facts = b.attention_execute(req, qp, kp, kp, b.tensor("o", B.DTYPE_BF16, (300, 8, 128)))
+        assert facts.kernel_launches == 1 and facts.accelerated_matrix_launches == 1
+        # refusals
+        unwritten = b.tensor("k-unwritten", B.DTYPE_BF16, (300, 2, 128))
+        with pytest.raises(YvexError) as e:
+            b.attention_execute(req, qp, unwritten, kp, b.tensor("o", B.DTYPE_BF16, (300, 8, 128)))
+        assert e.value.code == B.YVEX_ERR_FORMAT
+        for mutate, code in [(dict(query_heads=9), B.YVEX_ERR_INVALID_ARG),
+                             (dict(query_start=1), B.YVEX_ERR_INVALID_ARG),
+                             (dict(key_token_stride=255), B.YVEX_ERR_INVALID_ARG),
+                             (dict(head_dimension=64), B.YVEX_ERR_UNSUPPORTED),
+                             (dict(deterministic=0), B.YVEX_ERR_UNSUPPORTED),
+                             (dict(output_dtype=B.DTYPE_F32), B.YVEX_ERR_UNSUPPORTED),
+                             (dict(numeric_contract=7), B.YVEX_ERR_UNSUPPORTED),
+                             (dict(layout=0), B.YVEX_ERR_UNSUPPORTED)]:
+            bad = b.attention_requirement(300, 300, 8, 2, 128, dtype=B.DTYPE_BF16,
+                                          contract=B.NUMERIC_BF16_F32_ACCUMULATE)
+            for key, value in mutate.items():
+                setattr(bad, key, value)
+            with pytest.raises(YvexError) as e:
+                b.attention_workspace_required(bad)
+            assert e.value.code == code, mutate
+
+
+def test_paged_and_mla_admission():
+    with Backend() as b:
+        ok = b.paged_requirement(4, 32, 8, 128, 16, 100, 64, 1024)
+        assert b.paged_decode_workspace_required(ok) > 0
+        for mutate, code in [(dict(head_dimension=64), B.YVEX_ERR_UNSUPPORTED),
+                             (dict(page_tokens=32), B.YVEX_ERR_UNSUPPORTED),
+                             (dict(kv_storage=9), B.YVEX_ERR_UNSUPPORTED),
+                             (dict(numeric_contract=B.NUMERIC_EXACT_F32), B.YVEX_ERR_UNSUPPORTED),
+                             (dict(query_heads=33), B.YVEX_ERR_INVALID_ARG),
+                             (dict(max_context_tokens=1025), B.YVEX_ERR_INVALID_ARG),
+                             (dict(pool_pages=0), B.YVEX_ERR_INVALID_ARG)]:
+            bad = b.paged_requirement(4, 32, 8, 128, 16, 100, 64, 1024)
+            for key, value in mutate.items():
+                setattr(bad, key, value)
+            with pytest.raises(YvexError) as e:
+                b.paged_decode_workspace_required(bad)
+            assert e.value.code == code, mutate
+        q = written(b, "q", B.DTYPE_BF16, (4, 32, 128))
+        pool = written(b, "pool", B.DTYPE_BF16, (100 * 8 * 2048,))
+        table, ctx = written(b, "t", B.DTYPE_I32, (4, 64)), written(b, "c", B.DTYPE_I32, (4,))
+        out = b.tensor("o", B.DTYPE_BF16, (4, 32, 128))
+        facts = b.paged_decode_execute(ok, q, pool, pool, table, ctx, out)
+        assert facts.kernel_launches == 2 and out.is_written
+        small = written(b, "small-pool", B.DTYPE_BF16, (99 * 8 * 2048,))
+        with pytest.raises(YvexError) as e:
+            b.paged_decode_execute(ok, q, small, pool, table, ctx, out)
+        assert e.value.code == B.YVEX_ERR_FORMAT
+        mla = b.mla_requirement(16, 128, 576, 512, 64, 2048, 128, 8192)
+        assert b.mla_decode_workspace_required(mla) > 0
+        bad = b.mla_requirement(16, 64, 576, 512, 64, 2048, 128, 8192)
+        with pytest.raises(YvexError) as e:
+            b.mla_decode_workspace_required(bad)
+        assert e.value.code == B.YVEX_ERR_UNSUPPORTED
+
+
+# ------------------------------------------------- failure transitions ----
+
+def test_launch_failure_fails_only_that_variant(env):
+    with Backend() as b:
+        q, k = f32(b, "q", (4,), np.ones(4)), f32(b, "k", (3, 4), np.ones((3, 4)))
+        s, o = f32(b, "s", (3,)), f32(b, "o", (4,))
+        env("YVEX_TEST_ROCM_LAUNCH_FAILURE", "attention-causal-f32")
+        with pytest.raises(YvexError) as e:
+            b.op_attention(q, k, k, 3, 0, 0.5, True, s, s, o)
+        assert e.value.code == B.YVEX_ERR_BACKEND and not o.is_written
+        env("YVEX_TEST_ROCM_LAUNCH_FAILURE", None)
+        r = b.query_capability(B.VARIANT_ATTENTION_CAUSAL_F32)
+        assert r.state == B.CAPABILITY_FAILED and r.reason == B.REASON_LAUNCH_FAILED
+        assert b.status == B.STATUS_READY                             # backend survives
+        assert b.query_capability(B.VARIANT_ROCM_GQA_F32).state == B.CAPABILITY_SUPPORTED
+        with pytest.raises(YvexError) as e:                           # the failed variant stays failed
+            b.op_attention(q, k, k, 3, 0, 0.5, True, s, s, o)
+        assert e.value.code == B.YVEX_ERR_BACKEND
+        b.op_attention(q, k, k, 3, 0, 0.5, False, s, s, o)            # non-causal variant unaffected
+
+
+def test_runtime_launch_error_is_reported(env):
+    with Backend() as b:
+        req = b.attention_requirement(2, 2, 2, 1, 8)
+        q, k = written(b, "q", B.DTYPE_F32, (2, 2, 8)), written(b, "k", B.DTYPE_F32, (2, 1, 8))
+        out = b.tensor("o", B.DTYPE_F32, (2, 2, 8))
+        env("FAKE_HIP_LAUNCH", "fail")
+        with pytest.raises(YvexError) as e:
+            b.attention_execute(req, q, k, k, out)
+        assert e.value.code == B.YVEX_ERR_BACKEND and "HIP error" in e.value.message
+        assert not out.is_written
+        assert b.query_capability(B.VARIANT_ROCM_GQA_F32).reason == B.REASON_LAUNCH_FAILED
+
+
+def test_synchronisation_failure_fails_the_backend(env):
+    b = Backend()
+    q, k = f32(b, "q", (4,), np.ones(4)), f32(b, "k", (3, 4), np.ones((3, 4)))
+    s, o = f32(b, "s", (3,)), f32(b, "o", (4,))
+    env("YVEX_TEST_ROCM_SYNC_FAILURE", "all")
+    with pytest.raises(YvexError) as e:
+        b.op_attention(q, k, k, 3, 0, 0.5, True, s, s, o)
+    assert e.value.code == B.YVEX_ERR_BACKEND
+    env("YVEX_TEST_ROCM_SYNC_FAILURE", None)
+    assert b.status == B.STATUS_FAILED
+    r = b.query_capability(B.VARIANT_ATTENTION_CAUSAL_F32)
+    assert r.state == B.CAPABILITY_FAILED and r.reason == B.REASON_SYNCHRONIZATION_FAILED
+    with pytest.raises(YvexError) as e:
+        b.op_attention(q, k, k, 3, 0, 0.5, True, s, s, o)
+    assert e.value.code == B.YVEX_ERR_STATE and "cleanup only" in e.value.message
+    with pytest.raises(YvexError) as e:
+        b.tensor("late", B.DTYPE_F32, (4,))
+    assert e.value.code == B.YVEX_ERR_STATE
+    b.close()                                                      # checked close still discharges
+
+
+def test_checked_close_retains_the_owner_until_cleanup_succeeds(env, fake_runtime):
+    handle, err = C.c_void_p(), B.Error()
+    options = B.BackendOptions(B.KIND_ROCM, None, 0)
+    assert lib().yvex_backend_open(C.byref(handle), C.byref(options), C.byref(err)) == 0
+    env("YVEX_TEST_ROCM_CLEANUP_FAILURE", "1")
+    rc = lib().yvex_backend_close_checked(C.byref(handle), C.byref(err))
+    assert rc == B.YVEX_ERR_BACKEND and handle.value                # owner retained for a retry
+    result = B.CapabilityResult()
+    lib().yvex_backend_query_capability(handle, B.VARIANT_TENSOR_ALLOC, C.byref(result), C.byref(err))
+    assert result.state == B.CAPABILITY_FAILED and result.reason == B.REASON_CLEANUP_FAILED
+    env("YVEX_TEST_ROCM_CLEANUP_FAILURE", None)
+    assert lib().yvex_backend_close_checked(C.byref(handle), C.byref(err)) == 0
+    assert not handle.value and fake_runtime.fake_hip_live_modules() == 0
+    assert lib().yvex_backend_close_checked(C.byref(handle), C.byref(err)) == 0   # idempotent
+
+
+def test_deferred_completion_checks_status_at_sync():
+    with Backend() as b:
+        req = b.attention_requirement(2, 2, 2, 1, 8)
+        q, k = written(b, "q", B.DTYPE_F32, (2, 2, 8)), written(b, "k", B.DTYPE_F32, (2, 1, 8))
+        out = b.tensor("o", B.DTYPE_F32, (2, 2, 8))
+        b.set_completion_mode(B.COMPLETION_DEFERRED)
+        d2h = b.memory_stats().d2h_bytes
+        facts = b.attention_execute(req, q, k, k, out)
+        assert facts.device_synchronizations == 0 and facts.d2h_bytes == 0
+        assert b.memory_stats().d2h_bytes == d2h
+        b.sync()                                                   # reads the status word once
+        assert b.memory_stats().d2h_bytes == d2h + 4
+        b.set_completion_mode(B.COMPLETION_IMMEDIATE)
+        b.timing_begin()
+        assert b.timing_end() == 1.0
+        with pytest.raises(YvexError) as e:
+            b.timing_end()
+        assert e.value.code == B.YVEX_ERR_STATE
+
+
+# ------------------------------------------------ codecs and page layout ----
+
+def test_host_codecs_match_the_oracle_bit_for_bit():
+    library = lib()
+    bits = np.arange(1 << 16, dtype=np.uint16)
+    for b16 in bits[::7]:
+        f = ORACLE.lib.yvo_f16_decode(int(b16))
+        g = library.yvex_quant_f16_decode(int(b16))
+        assert (np.isnan(f) and np.isnan(g)) or np.float32(f).view(np.uint32) == np.float32(g).view(np.uint32)
+        assert np.float32(ORACLE.lib.yvo_bf16_decode(int(b16))).view(np.uint32) == \
+            np.float32(library.yvex_quant_bf16_decode(int(b16))).view(np.uint32) or np.isnan(g)
+    rng = np.random.default_rng(17)
+    x = np.concatenate([rng.standard_normal(6000) * s for s in (1e-8, 3e-8, 1e-5, 1e-3, 1.0, 7e4)])
+    x = np.concatenate([x, [0.0, -0.0, 65504.0, 65519.9, 65520.0, 2.0 ** -24, 2.0 ** -25, 6.1e-5,
+                            np.inf, -np.inf]]).astype(np.float32)
+    for value in x:
+        assert library.yvex_quant_f16_encode(float(value)) == ORACLE.lib.yvo_f16_encode(float(value)), value
+        assert library.yvex_quant_bf16_encode(float(value)) == ORACLE.lib.yvo_bf16_encode(float(value))
+    rows = (rng.standard_normal((300, 128)) * rng.uniform(1e-4, 30, (300, 1))).astype(np.float32)
+    rows[0] = 0.0
+    enc = q8_0_encode_rows(rows)
+    assert np.array_equal(enc, ORACLE.q8_0_encode_rows(rows))
+    assert np.array_equal(q8_0_decode_rows(enc, 128).view(np.uint32),
+                          ORACLE.q8_0_decode_rows(enc, 128).view(np.uint32))
+    golden = np.zeros(32, np.float32)
+    golden[:4] = [127.0, -127.0, 0.5, -0.5]
+    assert bytes(q8_0_encode_rows(golden)[:6]) == bytes([0x00, 0x3C, 0x7F, 0x81, 0x01, 0xFF])
+    with pytest.raises(YvexError) as e:
+        q8_0_encode_rows(np.full(32, np.finfo(np.float32).max, np.float32))
+    assert e.value.code == B.YVEX_ERR_BOUNDS
+    bad = np.zeros(34, np.uint8)
+    bad[1] = 0x7C
+    with pytest.raises(YvexError) as e:
+        q8_0_decode_rows(bad, 32)
+    assert e.value.code == B.YVEX_ERR_FORMAT
+
+
+def test_page_layouts_follow_the_documented_index_formulas():
+    rng = np.random.default_rng(23)
+    pages, hkv, d = 3, 2, 128
+    rows = rng.integers(0, 1 << 16, size=(pages, 16, hkv, d), dtype=np.uint16)
+    for is_value in (False, True):
+        packed = kv_pack_pages(rows, B.KV_BF16, is_value, hkv).view(np.uint16).reshape(pages, hkv, 2048)
+        t, c = np.meshgrid(np.arange(16), np.arange(d), indexing="ij")
+        index = c * 16 + t if is_value else ((c // 8) * 16 + t) * 8 + c % 8
+        for page in range(pages):
+            for head in range(hkv):
+                assert np.array_equal(packed[page, head][index], rows[page, :, head, :])
+        back = kv_unpack_pages(packed, B.KV_BF16, is_value, pages, hkv)
+        assert np.array_equal(back, rows)
+    blocks = rng.integers(0, 256, size=(pages, 16, hkv, 4 * 34), dtype=np.uint8)
+    for is_value in (False, True):
+        packed = kv_pack_pages(blocks, B.KV_Q8_0, is_value, hkv).reshape(pages, hkv, 2176)
+        canon = blocks.reshape(pages, 16, hkv, 4, 34)
+        t, c = np.meshgrid(np.arange(16), np.arange(d), indexing="ij")
+        if is_value:
+            index = (((t // 4) * 16 + c % 16) * 8 + c // 16) * 4 + t % 4
+        else:
+            index = ((((c % 32) // 8) * 16 + t) * 4 + c // 32) * 8 + c % 8
+        for page in range(pages):
+            for head in range(hkv):
+                codes = canon[page, :, head, :, 2:].reshape(16, d)
+                assert np.array_equal(packed[page, head, :2048][index], codes)
+                scales = canon[page, :, head, :, :2].reshape(16 * 4 * 2)
+                assert np.array_equal(packed[page, head, 2048:], scales)
+        assert np.array_equal(kv_unpack_pages(packed, B.KV_Q8_0, is_value, pages, hkv), blocks)
+    with pytest.raises(YvexError) as e:
+        kv_pack_pages(rows, B.KV_BF16, False, hkv, head_dim=64)
+    assert e.value.code == B.YVEX_ERR_UNSUPPORTED
