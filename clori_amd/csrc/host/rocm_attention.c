@@ -20,8 +20,8 @@ enum {
     ROCM_MFMA_HEAD_DIM = 128,
     ROCM_PAGE_TOKENS = 16,
     ROCM_GROUP_MAX = 16,
-    ROCM_CHUNK_MIN = 64,
-    ROCM_CHUNK_MAX = 1024,
+    ROCM_DECODE_WAVES = 2048,
+    ROCM_DECODE_MIN_TILES = 4,
     ROCM_PREFILL_ROWS = 256,     /* query rows per workgroup of the prefill kernel */
     ROCM_WORK_ALIGNMENT = 256    /* src/backend/cuda/transformer.c:17 */
 };
@@ -88,39 +88,50 @@ int yvex_rocm_op_attention(yvex_backend *backend, const yvex_device_tensor *quer
 
 /* ------------------------------------------------ split-K decode core ---- */
 
-/* The chunk is a pure function of the request geometry (never of the device) so the
- * planner's workspace_required and the execution always agree.  It aims at roughly 32
- * waves per compute unit of a 256-CU part over the worst-case token count. */
-static unsigned int decode_chunk_tokens(unsigned long long sessions, unsigned long long kv_heads,
-                                        unsigned long long max_context)
+/* Wave count and workspace of the balanced split-K decode are pure functions of the
+ * request geometry (never of the device) so the planner's workspace_required and the
+ * execution always agree: 2048 waves = 2 per SIMD of a 256-CU part, fewer when the
+ * worst-case work cannot give each wave ROCM_DECODE_MIN_TILES tiles. */
+static unsigned int decode_wave_count(unsigned long long sessions, unsigned long long kv_heads,
+                                      unsigned long long max_context)
 {
-    const char *forced = getenv("YVEX_ROCM_DECODE_CHUNK");
-    unsigned long long chunk;
-    if (forced && atoi(forced) >= ROCM_PAGE_TOKENS)
-        chunk = (unsigned long long)atoi(forced);
-    else
-        chunk = sessions * kv_heads * max_context / (256ull * 32ull);
-    chunk = align_up(chunk ? chunk : 1ull, ROCM_PAGE_TOKENS);
-    if (chunk < ROCM_CHUNK_MIN) chunk = ROCM_CHUNK_MIN;
-    if (chunk > ROCM_CHUNK_MAX) chunk = ROCM_CHUNK_MAX;
-    return (unsigned int)chunk;
+    const char *forced = getenv("YVEX_ROCM_DECODE_WAVES");
+    unsigned long long tiles = sessions * kv_heads *
+                               ((max_context + ROCM_PAGE_TOKENS - 1ull) / ROCM_PAGE_TOKENS);
+    unsigned long long waves = (tiles + ROCM_DECODE_MIN_TILES - 1ull) / ROCM_DECODE_MIN_TILES;
+    unsigned long long cap = forced && atoi(forced) > 0 ? (unsigned long long)atoi(forced)
+                                                        : ROCM_DECODE_WAVES;
+    if (waves > cap) waves = cap;
+    return (unsigned int)(waves ? waves : 1ull);
 }
 
-static int decode_workspace_bytes(unsigned long long sessions, unsigned long long max_chunks,
-                                  unsigned long long query_heads, unsigned long long head_dim,
-                                  unsigned long long *acc_bytes, unsigned long long *total)
+static int decode_workspace_bytes(unsigned long long slots, unsigned long long heads,
+                                  unsigned long long head_dim, unsigned long long *acc_bytes,
+                                  unsigned long long *total)
 {
-    unsigned long long slots, acc, ml;
-    if (!yvex_core_u64_mul(sessions, max_chunks, &slots) ||
-        !yvex_core_u64_mul(slots, query_heads, &slots) ||
-        !yvex_core_u64_mul(slots, head_dim * sizeof(float), &acc) ||
-        !yvex_core_u64_mul(slots, 2ull * sizeof(float), &ml))
+    unsigned long long rows, acc, ml;
+    if (!yvex_core_u64_mul(slots, heads, &rows) ||
+        !yvex_core_u64_mul(rows, head_dim * sizeof(float), &acc) ||
+        !yvex_core_u64_mul(rows, 2ull * sizeof(float), &ml))
         return 0;
     acc = align_up(acc, ROCM_WORK_ALIGNMENT);
     ml = align_up(ml, ROCM_WORK_ALIGNMENT);
     if (!yvex_core_u64_add(acc, ml, total)) return 0;
     *acc_bytes = acc;
     return 1;
+}
+
+/* Balanced decode: two slots per wave plus the per-session offset table. */
+static int balanced_workspace_bytes(unsigned long long waves, unsigned long long group,
+                                    unsigned long long head_dim, unsigned long long sessions,
+                                    unsigned long long *acc_bytes, unsigned long long *ml_bytes,
+                                    unsigned long long *total)
+{
+    unsigned long long parts = 0ull, offsets;
+    if (!decode_workspace_bytes(2ull * waves, group, head_dim, acc_bytes, &parts)) return 0;
+    offsets = align_up((sessions + 1ull) * sizeof(uint32_t), ROCM_WORK_ALIGNMENT);
+    *ml_bytes = parts - *acc_bytes;
+    return yvex_core_u64_add(parts, offsets, total);
 }
 
 typedef struct {
@@ -135,23 +146,23 @@ typedef struct {
     float scale;
 } decode_job;
 
-/* Launches the partial kernel and the merge kernel and completes the operation. */
+/* Launches the decode kernel and the finish (merge) kernel and completes the operation. */
 static int decode_run(yvex_backend *backend, const decode_job *job, const char *where,
                       yvex_backend_operation_facts *facts, yvex_error *err)
 {
     yvex_rocm_backend_state *state = yvex_rocm_state(backend);
     yvex_rocm_decode_params dp;
-    yvex_rocm_decode_merge_params mp;
-    unsigned long long acc_bytes = 0ull, total = 0ull, max_chunks;
-    unsigned int chunk = decode_chunk_tokens(job->sessions, job->kv_heads, job->max_context);
+    unsigned long long acc_bytes = 0ull, ml_bytes = 0ull, total = 0ull, items;
+    const unsigned long long group = job->query_heads / job->kv_heads;
+    const unsigned int waves = decode_wave_count(job->sessions, job->kv_heads, job->max_context);
     void *work = NULL;
     yvex_error cleanup;
     int owned = 0, rc, cleanup_rc;
-    max_chunks = (job->max_context + chunk - 1ull) / chunk;
-    if (job->sessions > 65535ull || job->kv_heads > 65535ull || job->query_heads > 65535ull ||
-        max_chunks > 0x7fffffffull ||
-        !decode_workspace_bytes(job->sessions, max_chunks, job->query_heads, job->head_dim,
-                                &acc_bytes, &total))
+    if (!yvex_core_u64_mul(job->sessions * job->kv_heads,
+                           (job->max_context + ROCM_PAGE_TOKENS - 1ull) / ROCM_PAGE_TOKENS, &items) ||
+        items > 0x7fffffffull || job->sessions > 65535ull || job->query_heads > 65535ull ||
+        !balanced_workspace_bytes(waves, group, job->head_dim, job->sessions, &acc_bytes,
+                                  &ml_bytes, &total))
         return refuse(err, YVEX_ERR_BOUNDS, where, "decode geometry exceeds admitted integer range");
     backend_workspace_reset(backend);
     rc = yvex_rocm_temporary_acquire(backend, total, &work, &owned, where, err);
@@ -162,8 +173,11 @@ static int decode_run(yvex_backend *backend, const decode_job *job, const char *
     dp.v_pool = job->v;
     dp.page_table = job->page_table;
     dp.context = job->context;
+    dp.out = (uint16_t *)job->out;
+    dp.lse = (float *)job->lse;
     dp.part_acc = (float *)work;
     dp.part_ml = (float *)((unsigned char *)work + acc_bytes);
+    dp.offsets = (uint32_t *)((unsigned char *)work + acc_bytes + ml_bytes);
     dp.status = state->device_status;
     dp.k_token_stride = job->k_token_stride;
     dp.v_token_stride = job->v_token_stride;
@@ -173,32 +187,16 @@ static int decode_run(yvex_backend *backend, const decode_job *job, const char *
     dp.head_dim = (uint32_t)job->head_dim;
     dp.pool_pages = (uint32_t)job->pool_pages;
     dp.table_stride = (uint32_t)job->table_stride;
-    dp.chunk_tokens = chunk;
-    dp.max_chunks = (uint32_t)max_chunks;
+    dp.min_tiles = ROCM_DECODE_MIN_TILES;
     dp.fixed_context = (uint32_t)job->fixed_context;
+    dp.waves = waves;
     dp.scale_log2 = job->scale * 1.4426950408889634f;
-    rc = yvex_rocm_launch(backend, job->function, job->variant, (unsigned int)max_chunks,
-                          (unsigned int)job->kv_heads, (unsigned int)job->sessions, 64u, 0u, &dp,
-                          where, err);
-    if (rc == YVEX_OK) {
-        memset(&mp, 0, sizeof(mp));
-        mp.part_acc = dp.part_acc;
-        mp.part_ml = dp.part_ml;
-        mp.context = job->context;
-        mp.out = (uint16_t *)job->out;
-        mp.lse = (float *)job->lse;
-        mp.status = state->device_status;
-        mp.sessions = dp.sessions;
-        mp.query_heads = dp.query_heads;
-        mp.head_dim = dp.head_dim;
-        mp.chunk_tokens = chunk;
-        mp.max_chunks = dp.max_chunks;
-        mp.fixed_context = dp.fixed_context;
-        rc = yvex_rocm_launch(backend, YVEX_ROCM_FN_DECODE_MERGE,
-                              YVEX_BACKEND_VARIANT_ROCM_ATTENTION_PAGED_BF16,
+    rc = yvex_rocm_launch(backend, job->function, job->variant, waves, 1u, 1u, 64u, 0u, &dp, where,
+                          err);
+    if (rc == YVEX_OK)
+        rc = yvex_rocm_launch(backend, YVEX_ROCM_FN_DECODE_FINISH, job->variant,
                               (unsigned int)job->query_heads, (unsigned int)job->sessions, 1u,
-                              (unsigned int)job->head_dim, 0u, &mp, where, err);
-    }
+                              (unsigned int)job->head_dim, 0u, &dp, where, err);
     if (rc == YVEX_OK) {
         facts->kernel_launches = 2ull;
         facts->accelerated_matrix_launches = 1ull;
@@ -272,7 +270,7 @@ static int rocm_attention_workspace_required(const yvex_transformer_attention_re
                                              unsigned long long *bytes, yvex_error *err)
 {
     static const char where[] = "rocm.transformer.attention.workspace";
-    unsigned long long acc = 0ull, total = 0ull, chunk, max_chunks;
+    unsigned long long acc = 0ull, ml = 0ull, total = 0ull;
     int rc;
     if (bytes) *bytes = 0ull;
     rc = attention_validate(r, where, err);
@@ -281,10 +279,9 @@ static int rocm_attention_workspace_required(const yvex_transformer_attention_re
     if (r->numeric_contract == YVEX_TRANSFORMER_ATTENTION_NUMERIC_BF16_F32_ACCUMULATE &&
         r->query_tokens == 1ull) {
         /* split-K decode partials; geometry must match decode_run */
-        chunk = decode_chunk_tokens(1ull, r->key_value_heads, visible_tokens(r));
-        max_chunks = (visible_tokens(r) + chunk - 1ull) / chunk;
-        if (!decode_workspace_bytes(1ull, max_chunks, r->query_heads, r->head_dimension, &acc,
-                                    &total))
+        const unsigned int waves = decode_wave_count(1ull, r->key_value_heads, visible_tokens(r));
+        if (!balanced_workspace_bytes(waves, r->query_heads / r->key_value_heads,
+                                      r->head_dimension, 1ull, &acc, &ml, &total))
             return refuse(err, YVEX_ERR_BOUNDS, where, "decode workspace geometry overflowed");
         *bytes = total;
     }
@@ -488,16 +485,16 @@ static int rocm_paged_decode_workspace_required(const yvex_rocm_paged_decode_req
                                                 unsigned long long *bytes, yvex_error *err)
 {
     static const char where[] = "rocm.attention.paged.workspace";
-    unsigned long long acc = 0ull, total = 0ull, chunk, max_chunks;
+    unsigned long long acc = 0ull, ml = 0ull, total = 0ull;
+    unsigned int waves;
     int rc;
     if (bytes) *bytes = 0ull;
     rc = paged_validate(r, where, err);
     if (rc != YVEX_OK) return rc;
     if (!bytes) return refuse(err, YVEX_ERR_INVALID_ARG, where, "workspace byte output is required");
-    chunk = decode_chunk_tokens(r->sessions, r->key_value_heads, r->max_context_tokens);
-    max_chunks = (r->max_context_tokens + chunk - 1ull) / chunk;
-    if (!decode_workspace_bytes(r->sessions, max_chunks, r->query_heads, r->head_dimension, &acc,
-                                &total))
+    waves = decode_wave_count(r->sessions, r->key_value_heads, r->max_context_tokens);
+    if (!balanced_workspace_bytes(waves, r->query_heads / r->key_value_heads, r->head_dimension,
+                                  r->sessions, &acc, &ml, &total))
         return refuse(err, YVEX_ERR_BOUNDS, where, "decode workspace geometry overflowed");
     *bytes = total;
     yvex_error_clear(err);
@@ -624,7 +621,7 @@ static int rocm_mla_decode_workspace_required(const yvex_rocm_mla_decode_require
     if (!bytes) return refuse(err, YVEX_ERR_INVALID_ARG, where, "workspace byte output is required");
     chunk = mla_chunk_tokens(r);
     max_chunks = (r->max_context_tokens + chunk - 1ull) / chunk;
-    if (!decode_workspace_bytes(r->batch, max_chunks, r->heads, r->value_dimension, &acc, &total))
+    if (!decode_workspace_bytes(r->batch * max_chunks, r->heads, r->value_dimension, &acc, &total))
         return refuse(err, YVEX_ERR_BOUNDS, where, "MLA workspace geometry overflowed");
     *bytes = total;
     yvex_error_clear(err);
@@ -670,7 +667,7 @@ static int rocm_mla_decode_execute(yvex_backend *backend,
     chunk = mla_chunk_tokens(r);
     max_chunks = (r->max_context_tokens + chunk - 1ull) / chunk;
     if (max_chunks > 0x7fffffffull ||
-        !decode_workspace_bytes(r->batch, max_chunks, r->heads, r->value_dimension, &acc_bytes,
+        !decode_workspace_bytes(r->batch * max_chunks, r->heads, r->value_dimension, &acc_bytes,
                                 &total))
         return refuse(err, YVEX_ERR_BOUNDS, where, "MLA decode geometry exceeds admitted range");
     backend_workspace_reset(backend);

@@ -42,24 +42,33 @@ typedef struct {
     uint32_t reserved;
 } yvex_rocm_fill_params;
 
-/* Split-K decode.  One wave per (chunk, kv head, session).  part_acc is
- * [sessions][max_chunks][query_heads][head_dim] F32 (unnormalised), part_ml is
- * [sessions][max_chunks][query_heads][2] F32 = (running max in log2 units, sum). */
+/* Split-K decode over a balanced partition.  The (session, kv head, 16-token tile) work
+ * of the whole batch is laid out as one sequence and cut into gridDim.x equal ranges,
+ * one wave each.  A wave that covers a whole (session, kv head) segment publishes the
+ * final rows itself; otherwise it leaves a partial in one of its two slots and the
+ * finish kernel merges the parts in wave order.
+ * part_acc is [2*waves][group][head_dim] F32 (unnormalised), part_ml is
+ * [2*waves][group][2] F32 = (running max in log2 units, sum); offsets is
+ * [sessions + 1] U32: exclusive prefix of work items per session, then the total. */
 typedef struct {
     const uint16_t *q;
     const void *k_pool, *v_pool;
     const int32_t *page_table; /* NULL for the token-major layout */
     const int32_t *context;    /* NULL: every session uses fixed_context */
+    uint16_t *out;             /* bf16 [sessions][query_heads][head_dim] */
+    float *lse;                /* optional F32 [sessions][query_heads] */
     float *part_acc, *part_ml;
+    uint32_t *offsets;
     int32_t *status;
     uint64_t k_token_stride, v_token_stride; /* token-major layout: elements per token */
     uint32_t sessions, query_heads, kv_heads, head_dim;
-    uint32_t pool_pages, table_stride, chunk_tokens, max_chunks;
-    uint32_t fixed_context, reserved;
+    uint32_t pool_pages, table_stride, min_tiles, fixed_context;
+    uint32_t waves, reserved;
     float scale_log2; /* softmax scale * log2(e) */
     float reserved_f;
 } yvex_rocm_decode_params;
 
+/* Log-sum-exp merge of per-chunk partials (used by the MLA path). */
 typedef struct {
     const float *part_acc, *part_ml;
     const int32_t *context;

@@ -30,8 +30,15 @@
 // block, so the K scale is applied to the fp32 partial dot per block, and the V scale
 // is folded into the probabilities per 32-lane block before the second product.
 //
-// Partials (running max in log2 units, sum, unnormalised accumulator) go to the
-// workspace; yvex_rocm_decode_merge combines them with a log-sum-exp merge.
+// Work distribution: the (session, kv head, tile) items of the whole batch form one
+// sequence that is cut into gridDim.x equal ranges, so every wave streams the same
+// number of tiles whatever the mix of context lengths.  A wave that covers a whole
+// (session, kv head) segment publishes its rows directly; a split segment leaves
+// partials (running max in log2 units, sum, unnormalised accumulator) in the workspace
+// and yvex_rocm_decode_finish merges them in wave order with a log-sum-exp merge (a
+// second launch instead of in-kernel signalling: a device-scope release fence per wave
+// costs far more on an 8-XCD part than one more launch).
+// yvex_rocm_decode_merge is the stand-alone merge used by the per-chunk MLA path.
 #include "mfma.h"
 
 #include "../kernel_params.h"
@@ -254,134 +261,286 @@ struct Q8Kv {
     }
 };
 
-template <class Kv, bool PAGED, int kDepth>
-__device__ inline void decode_body(const yvex_rocm_decode_params &p)
+__device__ inline uint32_t wave_inclusive_scan(uint32_t v, int lane)
 {
-    typedef typename Kv::Tile Tile;
-    const int lane = threadIdx.x, n = lane & 15, g = lane >> 4;
-    const uint32_t chunk = blockIdx.x, kv_head = blockIdx.y, session = blockIdx.z;
-    const uint32_t limit = PAGED ? p.table_stride * (uint32_t)kPageTokens : p.fixed_context;
-    const uint32_t ctx = p.context ? (uint32_t)p.context[session] : p.fixed_context;
-    if (ctx == 0u || ctx > limit) {
-        if (chunk == 0u && kv_head == 0u && lane == 0) flag(p.status, YVEX_ROCM_DEVICE_CONTRACT);
-        return;
-    }
-    const uint32_t t0 = chunk * p.chunk_tokens;
-    if (t0 >= ctx) return;
-    const uint32_t t1 = min(ctx, t0 + p.chunk_tokens);
-    const uint32_t group = p.query_heads / p.kv_heads;
-    const uint32_t tiles = (t1 - t0 + kPageTokens - 1) / kPageTokens;
-
-    bf16x8 q[4];
-    {
-        const uint16_t *qrow =
-            p.q + ((uint64_t)session * p.query_heads + kv_head * group + min((uint32_t)n, group - 1u)) *
-                      kHeadDim;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            u32x4 raw = load_b128(qrow + j * 32 + g * 8);
-            if ((uint32_t)n >= group) raw = (u32x4){0u, 0u, 0u, 0u};
-            q[j] = as_bf16x8(raw);
-        }
+    for (int off = 1; off < 64; off <<= 1) {
+        const uint32_t up = __shfl_up(v, off, 64);
+        if (lane >= off) v += up;
+    }
+    return v;
+}
+
+template <class Kv, bool PAGED, int kDepth>
+struct Decoder {
+    typedef typename Kv::Tile Tile;
+    const yvex_rocm_decode_params &p;
+    const int lane, n, g;
+    const uint32_t group, limit;
+
+    __device__ Decoder(const yvex_rocm_decode_params &params)
+        : p(params), lane(threadIdx.x), n(threadIdx.x & 15), g(threadIdx.x >> 4),
+          group(params.query_heads / params.kv_heads),
+          limit(PAGED ? params.table_stride * (uint32_t)kPageTokens : params.fixed_context)
+    {
     }
 
-    int32_t my_page = 0;
-    const unsigned char *kbase = (const unsigned char *)p.k_pool;
-    const unsigned char *vbase = (const unsigned char *)p.v_pool;
-    if (PAGED) {
-        // one coalesced read brings the chunk's page ids into the wave (chunk <= 64 pages)
-        const int32_t *table =
-            p.page_table + (uint64_t)session * p.table_stride + t0 / kPageTokens;
-        if ((uint32_t)lane < tiles) {
-            my_page = table[lane];
-            if (my_page < 0 || (uint32_t)my_page >= p.pool_pages) {
-                flag(p.status, YVEX_ROCM_DEVICE_CONTRACT);
-                my_page = 0;
+    // context of a session, 0 when it is out of contract (flagged once, by wave 0)
+    __device__ inline uint32_t context_of(uint32_t session) const
+    {
+        const uint32_t ctx = p.context ? (uint32_t)p.context[session] : p.fixed_context;
+        if (ctx == 0u || ctx > limit) {
+            if (blockIdx.x == 0u) flag(p.status, YVEX_ROCM_DEVICE_CONTRACT);
+            return 0u;
+        }
+        return ctx;
+    }
+
+    // Finds the session whose block of (tiles * kv_heads) work items contains `target`.
+    // Returns false when target is at or past the end; `total` then holds the item count.
+    __device__ inline bool locate(uint32_t target, uint32_t &session, uint32_t &offset,
+                                  uint32_t &tiles, uint32_t &total) const
+    {
+        uint32_t carry = 0u;
+        for (uint32_t base = 0u; base < p.sessions; base += 64u) {
+            const uint32_t s = base + (uint32_t)lane;
+            const uint32_t t = s < p.sessions ? (context_of(s) + kPageTokens - 1u) / kPageTokens : 0u;
+            const uint32_t items = t * p.kv_heads;
+            const uint32_t incl = wave_inclusive_scan(items, lane);
+            const uint32_t excl = carry + incl - items;
+            const uint64_t hit = __builtin_amdgcn_ballot_w64(items != 0u && target >= excl &&
+                                                             target < excl + items);
+            if (hit != 0ull) {
+                const int src = __builtin_ctzll(hit);
+                session = base + (uint32_t)src;
+                offset = (uint32_t)__builtin_amdgcn_readlane((int)excl, src);
+                tiles = (uint32_t)__builtin_amdgcn_readlane((int)t, src);
+                return true;
+            }
+            carry += (uint32_t)__builtin_amdgcn_readlane((int)incl, 63);
+        }
+        total = carry;
+        return false;
+    }
+
+    // Streams `count` (<= 64) tiles of (session, kv_head) starting at tile `first`.
+    __device__ inline void stream(State &st, const bf16x8 (&q)[4], uint32_t session,
+                                  uint32_t kv_head, uint32_t ctx, uint32_t first,
+                                  uint32_t count) const
+    {
+        const uint32_t t0 = first * kPageTokens;
+        const uint32_t t1 = min(ctx, t0 + count * kPageTokens);
+        int32_t my_page = 0;
+        const unsigned char *kbase = (const unsigned char *)p.k_pool;
+        const unsigned char *vbase = (const unsigned char *)p.v_pool;
+        if (PAGED) {
+            // one coalesced read brings the page ids of these tiles into the wave
+            const int32_t *table = p.page_table + (uint64_t)session * p.table_stride + first;
+            if ((uint32_t)lane < count) {
+                my_page = table[lane];
+                if (my_page < 0 || (uint32_t)my_page >= p.pool_pages) {
+                    flag(p.status, YVEX_ROCM_DEVICE_CONTRACT);
+                    my_page = 0;
+                }
+            }
+        } else {
+            kbase += (uint64_t)kv_head * kHeadDim * 2u;
+            vbase += (uint64_t)kv_head * kHeadDim * 2u;
+        }
+        auto fetch = [&](Tile &t, uint32_t i) {
+            if (PAGED) {
+                const uint32_t page = (uint32_t)__builtin_amdgcn_readlane(my_page, (int)i);
+                const uint64_t off = ((uint64_t)page * p.kv_heads + kv_head) * Kv::kBlockBytes;
+                Kv::load_paged(t, kbase + off, vbase + off, lane);
+            } else {
+                const uint32_t row = t0 + i * kPageTokens;
+                Kv::load_rows(t, kbase, vbase, p, row, t1 - row, lane);
+            }
+        };
+        // Ring of kDepth tile buffers: kDepth-1 tiles stay in flight per wave while one is
+        // consumed.  Every refill in the steady-state loop is unconditional (the index is
+        // clamped to the last tile, a cache hit) so the number of outstanding loads is
+        // the same on every trip and the waits the compiler places are partial
+        // (vmcnt > 0) instead of draining the whole queue.
+        Tile ring[kDepth];
+        const uint32_t last_tile = count - 1u;
+#pragma unroll
+        for (int r = 0; r < kDepth; ++r) fetch(ring[r], min((uint32_t)r, last_tile));
+        uint32_t i = 0u;
+        for (; i + kDepth <= count; i += kDepth) {
+#pragma unroll
+            for (int r = 0; r < kDepth; ++r) {
+                const uint32_t tile = i + (uint32_t)r;
+                Kv::consume(st, ring[r], q, p.scale_log2,
+                            min((uint32_t)kPageTokens, t1 - (t0 + tile * kPageTokens)), lane);
+                fetch(ring[r], min(tile + kDepth, last_tile));
             }
         }
-    } else {
-        kbase += (uint64_t)kv_head * kHeadDim * 2u;
-        vbase += (uint64_t)kv_head * kHeadDim * 2u;
-    }
-
-    auto fetch = [&](Tile &t, uint32_t i) {
-        if (PAGED) {
-            const uint32_t page = (uint32_t)__builtin_amdgcn_readlane(my_page, (int)i);
-            const uint64_t off = ((uint64_t)page * p.kv_heads + kv_head) * Kv::kBlockBytes;
-            Kv::load_paged(t, kbase + off, vbase + off, lane);
-        } else {
-            const uint32_t first = t0 + i * kPageTokens;
-            Kv::load_rows(t, kbase, vbase, p, first, t1 - first, lane);
-        }
-    };
-
-    State st;
 #pragma unroll
-    for (int b = 0; b < 8; ++b) st.o[b] = (floatx4){0.f, 0.f, 0.f, 0.f};
-    st.m = -INFINITY;
-    st.l = 0.f;
-
-    // Ring of kDepth tile buffers: kDepth-1 tiles stay in flight per wave while one is
-    // consumed.  Every refill in the steady-state loop is unconditional (the index is
-    // clamped to the last tile, a cache hit) so the number of outstanding loads is the
-    // same on every trip and the waits the compiler places are partial (vmcnt > 0)
-    // instead of draining the whole queue.
-    Tile ring[kDepth];
-    const uint32_t last_tile = tiles - 1u;
-#pragma unroll
-    for (int r = 0; r < kDepth; ++r) fetch(ring[r], min((uint32_t)r, last_tile));
-    uint32_t i = 0u;
-    for (; i + kDepth <= tiles; i += kDepth) {
-#pragma unroll
-        for (int r = 0; r < kDepth; ++r) {
+        for (int r = 0; r < kDepth - 1; ++r) {
             const uint32_t tile = i + (uint32_t)r;
-            Kv::consume(st, ring[r], q, p.scale_log2,
-                        min((uint32_t)kPageTokens, t1 - (t0 + tile * kPageTokens)), lane);
-            fetch(ring[r], min(tile + kDepth, last_tile));
+            if (tile < count)
+                Kv::consume(st, ring[r], q, p.scale_log2,
+                            min((uint32_t)kPageTokens, t1 - (t0 + tile * kPageTokens)), lane);
         }
-    }
-#pragma unroll
-    for (int r = 0; r < kDepth - 1; ++r) {
-        const uint32_t tile = i + (uint32_t)r;
-        if (tile < tiles)
-            Kv::consume(st, ring[r], q, p.scale_log2,
-                        min((uint32_t)kPageTokens, t1 - (t0 + tile * kPageTokens)), lane);
     }
 
-    float l = st.l;
-    l += xor_lanes(l, 16);
-    l += xor_lanes(l, 32);
-    if ((uint32_t)n < group) {
-        const uint64_t slot =
-            ((uint64_t)session * p.max_chunks + chunk) * p.query_heads + kv_head * group + n;
-        float *acc = p.part_acc + slot * kHeadDim + g * 4;
+    // Publishes normalised rows for the lane's head from a final (m, l, O^T) state.
+    __device__ inline void publish(const State &st, float l, uint32_t session,
+                                   uint32_t kv_head) const
+    {
+        if ((uint32_t)n >= group) return;
+        const uint32_t head = kv_head * group + (uint32_t)n;
+        const float inv = 1.0f / l;
+        uint16_t *dst = p.out + ((uint64_t)session * p.query_heads + head) * kHeadDim + g * 4;
+        bool bad = false;
 #pragma unroll
-        for (int bb = 0; bb < 8; ++bb) *reinterpret_cast<floatx4 *>(acc + bb * 16) = st.o[bb];
-        if (g == 0) {
-            p.part_ml[slot * 2 + 0] = st.m;
-            p.part_ml[slot * 2 + 1] = l;
+        for (int b = 0; b < 8; ++b) {
+            const float a0 = st.o[b][0] * inv, a1 = st.o[b][1] * inv;
+            const float a2 = st.o[b][2] * inv, a3 = st.o[b][3] * inv;
+            bad |= !(isfinite(a0) && isfinite(a1) && isfinite(a2) && isfinite(a3));
+            u32x2 w;
+            w.x = pack_bf16x2(a0, a1);
+            w.y = pack_bf16x2(a2, a3);
+            *reinterpret_cast<u32x2 *>(dst + b * 16) = w;
+        }
+        if (bad) flag(p.status, YVEX_ROCM_DEVICE_NUMERIC);
+        if (p.lse && g == 0)
+            p.lse[(uint64_t)session * p.query_heads + head] = (st.m + fast_log2(l)) * YVEX_LN2;
+    }
+
+    __device__ inline void run() const
+    {
+        const uint32_t wave = blockIdx.x, waves = gridDim.x;
+        uint32_t session = 0u, offset = 0u, tiles = 0u, total = 0u;
+        (void)locate(0xffffffffu, session, offset, tiles, total);
+        if (wave == 0u) publish_offsets(total);
+        if (total == 0u) return;
+        const uint32_t per_wave = max((total + waves - 1u) / waves, p.min_tiles);
+        uint32_t cur = wave * per_wave;
+        if (cur >= total) return;
+        const uint32_t end = min(total, cur + per_wave);
+        while (cur < end) {
+            if (!locate(cur, session, offset, tiles, total)) return;
+            const uint32_t rel = cur - offset;
+            const uint32_t kv_head = rel / tiles, first = rel % tiles;
+            const uint32_t seg_begin = offset + kv_head * tiles, seg_end = seg_begin + tiles;
+            const uint32_t stop = min(seg_end, end), count = stop - cur;
+            const uint32_t ctx = context_of(session);
+
+            bf16x8 q[4];
+            {
+                const uint16_t *qrow = p.q + ((uint64_t)session * p.query_heads + kv_head * group +
+                                              min((uint32_t)n, group - 1u)) * kHeadDim;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    u32x4 raw = load_b128(qrow + j * 32 + g * 8);
+                    if ((uint32_t)n >= group) raw = (u32x4){0u, 0u, 0u, 0u};
+                    q[j] = as_bf16x8(raw);
+                }
+            }
+            State st;
+#pragma unroll
+            for (int b = 0; b < 8; ++b) st.o[b] = (floatx4){0.f, 0.f, 0.f, 0.f};
+            st.m = -INFINITY;
+            st.l = 0.f;
+            for (uint32_t done = 0u; done < count; done += 64u)
+                stream(st, q, session, kv_head, ctx, first + done, min(64u, count - done));
+
+            float l = st.l;
+            l += xor_lanes(l, 16);
+            l += xor_lanes(l, 32);
+            if (first == 0u && stop == seg_end) {
+                publish(st, l, session, kv_head);  // the whole segment was ours
+            } else if ((uint32_t)n < group) {
+                // slot 1 when the segment starts inside this wave's range, else slot 0
+                const uint64_t slot = ((uint64_t)wave * 2u + (first == 0u ? 1u : 0u)) * group + n;
+                float *acc = p.part_acc + slot * kHeadDim + g * 4;
+#pragma unroll
+                for (int b = 0; b < 8; ++b) *reinterpret_cast<floatx4 *>(acc + b * 16) = st.o[b];
+                if (g == 0) {
+                    p.part_ml[slot * 2 + 0] = st.m;
+                    p.part_ml[slot * 2 + 1] = l;
+                }
+            }
+            cur = stop;
         }
     }
-}
+
+    // Wave 0 leaves the exclusive prefix of per-session work items (and the total at
+    // index `sessions`) for the merge kernel.
+    __device__ inline void publish_offsets(uint32_t total) const
+    {
+        uint32_t carry = 0u;
+        for (uint32_t base = 0u; base < p.sessions; base += 64u) {
+            const uint32_t s = base + (uint32_t)lane;
+            const uint32_t t = s < p.sessions ? (context_of(s) + kPageTokens - 1u) / kPageTokens : 0u;
+            const uint32_t items = t * p.kv_heads;
+            const uint32_t incl = wave_inclusive_scan(items, lane);
+            if (s < p.sessions) p.offsets[s] = carry + incl - items;
+            carry += (uint32_t)__builtin_amdgcn_readlane((int)incl, 63);
+        }
+        if (lane == 0) p.offsets[p.sessions] = total;
+    }
+};
 
 }  // namespace
 
 extern "C" __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 yvex_rocm_decode_paged_bf16(const yvex_rocm_decode_params p)
 {
-    decode_body<Bf16Kv, true, 3>(p);
+    Decoder<Bf16Kv, true, 3>(p).run();
 }
 
 extern "C" __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 yvex_rocm_decode_paged_q8_0(const yvex_rocm_decode_params p)
 {
-    decode_body<Q8Kv, true, 3>(p);
+    Decoder<Q8Kv, true, 3>(p).run();
 }
 
 extern "C" __global__ void __launch_bounds__(64)
 yvex_rocm_decode_rows_bf16(const yvex_rocm_decode_params p)
 {
-    decode_body<Bf16Kv, false, 2>(p);
+    Decoder<Bf16Kv, false, 2>(p).run();
+}
+
+// Merge of the split segments of the balanced decode.  grid = (query_heads, sessions),
+// block = head_dim threads (one per output lane).  A segment that one wave covered was
+// already published by that wave and is skipped.
+extern "C" __global__ void __launch_bounds__(128)
+yvex_rocm_decode_finish(const yvex_rocm_decode_params p)
+{
+    const uint32_t head = blockIdx.x, session = blockIdx.y, d = threadIdx.x;
+    const uint32_t group = p.query_heads / p.kv_heads;
+    const uint32_t offset = p.offsets[session], next = p.offsets[session + 1u];
+    const uint32_t total = p.offsets[p.sessions];
+    const uint32_t tiles = (next - offset) / p.kv_heads;
+    if (tiles == 0u || d >= p.head_dim) return;
+    const uint32_t per_wave = max((total + p.waves - 1u) / p.waves, p.min_tiles);
+    const uint32_t kv_head = head / group, hh = head % group;
+    const uint32_t seg_begin = offset + kv_head * tiles, seg_end = seg_begin + tiles;
+    const uint32_t w_first = seg_begin / per_wave, w_last = (seg_end - 1u) / per_wave;
+    if (w_first == w_last) return;
+    auto slot_of = [&](uint32_t j) -> uint64_t {
+        return ((uint64_t)j * 2u + (seg_begin >= j * per_wave ? 1u : 0u)) * group + hh;
+    };
+    // independent loads: unrolled, eight partial rows are in flight per thread
+    float top = -INFINITY;
+#pragma unroll 8
+    for (uint32_t j = w_first; j <= w_last; ++j) top = fmaxf(top, p.part_ml[slot_of(j) * 2u]);
+    float sum = 0.f, acc = 0.f;
+#pragma unroll 8
+    for (uint32_t j = w_first; j <= w_last; ++j) {
+        const uint64_t slot = slot_of(j);
+        const float w = fast_exp2(p.part_ml[slot * 2u] - top);
+        sum += w * p.part_ml[slot * 2u + 1u];
+        acc += w * p.part_acc[slot * p.head_dim + d];
+    }
+    const float o = acc / sum;
+    if (!isfinite(o)) flag(p.status, YVEX_ROCM_DEVICE_NUMERIC);
+    p.out[((uint64_t)session * p.query_heads + head) * p.head_dim + d] = bf16_bits(o);
+    if (p.lse && d == 0u)
+        p.lse[(uint64_t)session * p.query_heads + head] = (top + fast_log2(sum)) * YVEX_LN2;
 }
 
 // Log-sum-exp merge of the chunk partials of one (session, query head); one thread per

@@ -323,7 +323,7 @@ def test_attention_execute_contracts_facts_and_workspace(fake_runtime):
         assert (facts.kernel_launches, facts.device_synchronizations, facts.d2h_bytes,
                 facts.download_count) == (1, 1, 4, 1) and out.is_written
         assert b.attention_workspace_required(req) == 0
-        # bf16 decode: two launches, workspace == planned bytes, attached workspace is used
+        # bf16 decode: two launches (stream + finish), workspace == planned bytes, attached workspace is used
         req = b.attention_requirement(1, 4096, 32, 8, 128, query_start=4095, dtype=B.DTYPE_BF16,
                                       contract=B.NUMERIC_BF16_F32_ACCUMULATE)
         planned = b.attention_workspace_required(req)
