@@ -323,25 +323,26 @@ struct Decoder {
         return false;
     }
 
-    // Streams `count` (<= 64) tiles of (session, kv_head) starting at tile `first`.
+    // Streams `count` (<= 128) tiles of (session, kv_head) starting at tile `first`.
     __device__ inline void stream(State &st, const bf16x8 (&q)[4], uint32_t session,
                                   uint32_t kv_head, uint32_t ctx, uint32_t first,
                                   uint32_t count) const
     {
         const uint32_t t0 = first * kPageTokens;
         const uint32_t t1 = min(ctx, t0 + count * kPageTokens);
-        int32_t my_page = 0;
+        int32_t my_page = 0, my_page_hi = 0;
         const unsigned char *kbase = (const unsigned char *)p.k_pool;
         const unsigned char *vbase = (const unsigned char *)p.v_pool;
         if (PAGED) {
-            // one coalesced read brings the page ids of these tiles into the wave
+            // two coalesced reads bring the page ids of these tiles into the wave
             const int32_t *table = p.page_table + (uint64_t)session * p.table_stride + first;
-            if ((uint32_t)lane < count) {
-                my_page = table[lane];
-                if (my_page < 0 || (uint32_t)my_page >= p.pool_pages) {
-                    flag(p.status, YVEX_ROCM_DEVICE_CONTRACT);
-                    my_page = 0;
-                }
+            if ((uint32_t)lane < count) my_page = table[lane];
+            if ((uint32_t)lane + 64u < count) my_page_hi = table[lane + 64];
+            if (my_page < 0 || (uint32_t)my_page >= p.pool_pages || my_page_hi < 0 ||
+                (uint32_t)my_page_hi >= p.pool_pages) {
+                flag(p.status, YVEX_ROCM_DEVICE_CONTRACT);
+                my_page = 0;
+                my_page_hi = 0;
             }
         } else {
             kbase += (uint64_t)kv_head * kHeadDim * 2u;
@@ -349,7 +350,9 @@ struct Decoder {
         }
         auto fetch = [&](Tile &t, uint32_t i) {
             if (PAGED) {
-                const uint32_t page = (uint32_t)__builtin_amdgcn_readlane(my_page, (int)i);
+                const uint32_t page = (uint32_t)(i < 64u
+                                                     ? __builtin_amdgcn_readlane(my_page, (int)i)
+                                                     : __builtin_amdgcn_readlane(my_page_hi, (int)(i - 64u)));
                 const uint64_t off = ((uint64_t)page * p.kv_heads + kv_head) * Kv::kBlockBytes;
                 Kv::load_paged(t, kbase + off, vbase + off, lane);
             } else {
@@ -444,8 +447,8 @@ struct Decoder {
             for (int b = 0; b < 8; ++b) st.o[b] = (floatx4){0.f, 0.f, 0.f, 0.f};
             st.m = -INFINITY;
             st.l = 0.f;
-            for (uint32_t done = 0u; done < count; done += 64u)
-                stream(st, q, session, kv_head, ctx, first + done, min(64u, count - done));
+            for (uint32_t done = 0u; done < count; done += 128u)
+                stream(st, q, session, kv_head, ctx, first + done, min(128u, count - done));
 
             float l = st.l;
             l += xor_lanes(l, 16);
@@ -524,17 +527,35 @@ yvex_rocm_decode_finish(const yvex_rocm_decode_params p)
     auto slot_of = [&](uint32_t j) -> uint64_t {
         return ((uint64_t)j * 2u + (seg_begin >= j * per_wave ? 1u : 0u)) * group + hh;
     };
-    // independent loads: unrolled, eight partial rows are in flight per thread
-    float top = -INFINITY;
-#pragma unroll 8
-    for (uint32_t j = w_first; j <= w_last; ++j) top = fmaxf(top, p.part_ml[slot_of(j) * 2u]);
-    float sum = 0.f, acc = 0.f;
-#pragma unroll 8
-    for (uint32_t j = w_first; j <= w_last; ++j) {
-        const uint64_t slot = slot_of(j);
-        const float w = fast_exp2(p.part_ml[slot * 2u] - top);
-        sum += w * p.part_ml[slot * 2u + 1u];
-        acc += w * p.part_acc[slot * p.head_dim + d];
+    // one pass, eight parts at a time: all 24 loads of a trip are independent and in
+    // flight together (indices past the end alias the last part with weight zero)
+    float top = -INFINITY, sum = 0.f, acc = 0.f;
+    for (uint32_t j0 = w_first; j0 <= w_last; j0 += 8u) {
+        float m[8], l[8], v[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const uint64_t slot = slot_of(min(j0 + (uint32_t)i, w_last));
+            m[i] = p.part_ml[slot * 2u];
+            l[i] = p.part_ml[slot * 2u + 1u];
+            v[i] = p.part_acc[slot * p.head_dim + d];
+        }
+        float trip = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            if (j0 + (uint32_t)i > w_last) m[i] = -INFINITY;
+            trip = fmaxf(trip, m[i]);
+        }
+        const float m_new = fmaxf(top, trip);
+        const float keep = fast_exp2(top - m_new);
+        sum *= keep;
+        acc *= keep;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const float w = fast_exp2(m[i] - m_new);
+            sum += w * l[i];
+            acc += w * v[i];
+        }
+        top = m_new;
     }
     const float o = acc / sum;
     if (!isfinite(o)) flag(p.status, YVEX_ROCM_DEVICE_NUMERIC);
