@@ -22,7 +22,7 @@ enum {
     ROCM_GROUP_MAX = 16,
     ROCM_DECODE_WAVES = 2048,
     ROCM_DECODE_MIN_TILES = 4,
-    ROCM_PREFILL_ROWS = 256,     /* query rows per workgroup of the prefill kernel */
+    ROCM_PREFILL_ROWS = YVEX_ROCM_PREFILL_ROWS, /* query rows per prefill workgroup */
     ROCM_WORK_ALIGNMENT = 256    /* src/backend/cuda/transformer.c:17 */
 };
 
@@ -417,12 +417,13 @@ static int attention_execute_common(yvex_backend *backend,
         params.causal = (uint32_t)causal;
         params.scale_log2 = (1.0f / sqrtf((float)r->head_dimension)) * 1.4426950408889634f;
         backend_workspace_reset(backend);
-        if (r->query_heads > 65535ull || q_tiles > 65535ull)
+        if (r->query_heads > 65535ull || q_tiles > 65535ull ||
+            r->query_heads * q_tiles > 0x7fffffffull)
             return refuse(err, YVEX_ERR_BOUNDS, where,
                           "prefill geometry exceeds admitted launch range");
         rc = yvex_rocm_launch(backend, YVEX_ROCM_FN_PREFILL_BF16,
                               YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_BF16,
-                              (unsigned int)r->query_heads, (unsigned int)q_tiles, 1u, 256u, 0u,
+                              (unsigned int)(r->query_heads * q_tiles), 1u, 1u, 256u, 0u,
                               &params, "rocm.transformer.gqa.prefill", err);
         if (rc == YVEX_OK) {
             facts->kernel_launches = 1ull;

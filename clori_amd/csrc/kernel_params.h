@@ -78,7 +78,9 @@ typedef struct {
     uint32_t sessions, query_heads, head_dim, chunk_tokens, max_chunks, fixed_context;
 } yvex_rocm_decode_merge_params;
 
-/* Causal / full GQA prefill on bf16 token-major tensors. */
+/* Causal / full GQA prefill on bf16 token-major tensors.  The grid is one-dimensional:
+ * query_heads * ceil(query_tokens / YVEX_ROCM_PREFILL_ROWS) workgroups of 256 threads. */
+#define YVEX_ROCM_PREFILL_ROWS 128
 typedef struct {
     const uint16_t *q, *k, *v;
     uint16_t *out;

@@ -2,9 +2,10 @@
 // fp32 scores, online softmax and accumulation.  head_dim 128, token-major tensors
 // ([token][head][dim], per-token strides in elements).
 //
-// A workgroup of 4 waves owns one (query head, 256-row query tile): each wave owns
-// 64 query rows and walks the key/value tokens in tiles of 64 that the workgroup
-// stages in LDS once and all four waves share.  Both products are computed transposed
+// A workgroup of 4 waves owns one (query head, 128-row query tile): each wave owns
+// 32 query rows and walks the key/value tokens in tiles of 64 that the workgroup
+// stages in LDS once and all four waves share.  Two workgroups are resident per CU, so
+// the softmax VALU work of one overlaps the MFMAs of the other.  Both products are computed transposed
 // so the probabilities never leave registers:
 //     S^T[key][query] = K[key][:] . Q[query][:]        v_mfma_f32_32x32x16_bf16, A = K (LDS)
 //     O^T[dim][query] += V^T[dim][key] . P^T[key][query]                A = V^T (LDS)
@@ -18,6 +19,12 @@
 //     V^T tile  [128 dims][64 keys] bf16, row pitch 136 B   2 x ds_read_b64 per A operand
 // Two buffers of each; the global loads of tile t+1 are issued before the products of
 // tile t and land in registers while the MFMAs run, one barrier per tile.
+//
+// The running maximum is only raised when a tile exceeds it by more than kLazyLog2 (in
+// log2 units), so the accumulator rescale is rare; probabilities are then at most
+// 2^kLazyLog2, harmless in fp32 sums and in the bf16 operand of the second product.
+// Workgroups are numbered so that heavier (later) query tiles start first and, when the
+// kv head count is a multiple of the 8 XCDs, all users of one kv head share an L2.
 #include "mfma.h"
 
 #include "../kernel_params.h"
@@ -32,6 +39,7 @@ constexpr int kKBytes = kKeyTile * kKPitch;   // 17408
 constexpr int kVBytes = kHeadDim * kVPitch;   // 17408
 constexpr int kBufBytes = kKBytes + kVBytes;
 constexpr int kThreads = 256;
+constexpr float kLazyLog2 = 8.0f;
 
 __device__ inline void flag(int32_t *status, int code) { atomicCAS(status, 0, code); }
 
@@ -42,11 +50,12 @@ __device__ inline void prefill_body(const yvex_rocm_prefill_params &p, unsigned 
     constexpr int kRowsPerBlock = 4 * kRowsPerWave;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int n = lane & 31, g = lane >> 5;
-    // heavier (later) query tiles are dispatched first
+    // heavier (later) query tiles are dispatched first; id % kv_heads picks the kv head
     const uint32_t q_tiles = (p.query_tokens + kRowsPerBlock - 1) / kRowsPerBlock;
-    const uint32_t q_tile = q_tiles - 1u - blockIdx.y;
-    const uint32_t head = blockIdx.x;
-    const uint32_t kv_head = head / (p.query_heads / p.kv_heads);
+    const uint32_t q_tile = q_tiles - 1u - blockIdx.x / p.query_heads;
+    const uint32_t in_tile = blockIdx.x % p.query_heads;
+    const uint32_t kv_head = in_tile % p.kv_heads;
+    const uint32_t head = kv_head * (p.query_heads / p.kv_heads) + in_tile / p.kv_heads;
     const uint32_t row0 = q_tile * kRowsPerBlock + wave * kRowsPerWave;  // first row of this wave
 
     // keys visible to the last row of the workgroup bound the walk
@@ -157,46 +166,49 @@ __device__ inline void prefill_body(const yvex_rocm_prefill_params &p, unsigned 
             }
         }
 
-        // ---- scale, mask, online softmax (per lane = per query row) ----------
+        // ---- mask, online softmax (per lane = per query row) ----------------------
+        // scores stay raw; the softmax scale is folded into the exponent's multiply-add
         const bool need_mask = (key0 + kKeyTile - 1u > wave_first_vis) ||
                                (key0 + kKeyTile > p.kv_tokens);
         uint32_t pk[2][NB][8];  // bf16 pairs: [mb][nb][u*4 + pair]
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
-            const uint32_t row = row0 + nb * 32 + n;
-            const uint32_t vis = p.causal ? min(p.query_start + row, p.kv_tokens - 1u)
-                                          : p.kv_tokens - 1u;
+            if (need_mask) {
+                const uint32_t row = row0 + nb * 32 + n;
+                const uint32_t vis = p.causal ? min(p.query_start + row, p.kv_tokens - 1u)
+                                              : p.kv_tokens - 1u;
+#pragma unroll
+                for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) {
+                        const uint32_t key = key0 + mb * 32 + (i >> 2) * 8 + g * 4 + (i & 3);
+                        if (key > vis) s[mb][nb][i] = -INFINITY;
+                    }
+            }
             float mloc = -INFINITY;
 #pragma unroll
             for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    float x = s[mb][nb][i] * p.scale_log2;
-                    if (need_mask) {
-                        const uint32_t key = key0 + mb * 32 + (i >> 2) * 8 + g * 4 + (i & 3);
-                        if (key > vis) x = -INFINITY;
-                    }
-                    s[mb][nb][i] = x;
-                    mloc = fmaxf(mloc, x);
-                }
-            mloc = fmaxf(mloc, xor_lanes(mloc, 32));
-            const float m_new = fmaxf(m_run[nb], mloc);
-            // rows past query_tokens or fully masked keep m = -inf: guard the subtraction
-            const float m_use = m_new == -INFINITY ? 0.f : m_new;
-            if (__builtin_amdgcn_ballot_w64(m_new > m_run[nb]) != 0ull) {
-                const float alpha = fast_exp2(m_run[nb] - m_use);
+                for (int i = 0; i < 16; ++i) mloc = fmaxf(mloc, s[mb][nb][i]);
+            mloc = fmaxf(mloc, xor_lanes(mloc, 32)) * p.scale_log2;
+            if (__builtin_amdgcn_ballot_w64(mloc > m_run[nb] + kLazyLog2) != 0ull) {
+                const float m_new = fmaxf(m_run[nb], mloc);
+                // a row that has seen nothing yet keeps m = -inf: guard the subtraction
+                const float alpha = m_new == -INFINITY ? 1.0f : fast_exp2(m_run[nb] - m_new);
                 l_run[nb] *= alpha;
 #pragma unroll
                 for (int db = 0; db < 4; ++db) o[db][nb] *= alpha;
                 m_run[nb] = m_new;
             }
+            const float neg_m = m_run[nb] == -INFINITY ? 0.f : -m_run[nb];
             float lsum = 0.f;
 #pragma unroll
             for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
                 for (int i = 0; i < 16; i += 2) {
-                    const float p0 = fast_exp2(s[mb][nb][i] - m_use);
-                    const float p1 = fast_exp2(s[mb][nb][i + 1] - m_use);
+                    const float p0 = fast_exp2(__builtin_fmaf(s[mb][nb][i], p.scale_log2, neg_m));
+                    const float p1 =
+                        fast_exp2(__builtin_fmaf(s[mb][nb][i + 1], p.scale_log2, neg_m));
                     lsum += p0 + p1;
                     pk[mb][nb][i >> 1] = pack_bf16x2(p0, p1);
                 }
@@ -263,10 +275,11 @@ __device__ inline void prefill_body(const yvex_rocm_prefill_params &p, unsigned 
 
 }  // namespace
 
-// grid = (query heads, query tiles of 256 rows), block 256, LDS 2 x (K + V^T) tiles.
-extern "C" __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
+// grid = query heads x query tiles of YVEX_ROCM_PREFILL_ROWS rows, block 256,
+// LDS 2 x (K + V^T) tiles; two workgroups per CU.
+extern "C" __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
 yvex_rocm_prefill_bf16(const yvex_rocm_prefill_params p)
 {
     __shared__ __attribute__((aligned(16))) unsigned char lds[2 * kBufBytes];
-    prefill_body<2>(p, lds);
+    prefill_body<YVEX_ROCM_PREFILL_ROWS / 128>(p, lds);
 }
