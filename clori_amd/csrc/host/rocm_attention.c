@@ -417,8 +417,11 @@ static int attention_execute_common(yvex_backend *backend,
         params.causal = (uint32_t)causal;
         params.scale_log2 = (1.0f / sqrtf((float)r->head_dimension)) * 1.4426950408889634f;
         backend_workspace_reset(backend);
+        /* the kernel addresses K and V through 32-bit buffer offsets */
         if (r->query_heads > 65535ull || q_tiles > 65535ull ||
-            r->query_heads * q_tiles > 0x7fffffffull)
+            r->query_heads * q_tiles > 0x7fffffffull ||
+            r->key_value_tokens * k_stride * 2ull >= 0xffffffffull ||
+            r->key_value_tokens * v_stride * 2ull >= 0xffffffffull)
             return refuse(err, YVEX_ERR_BOUNDS, where,
                           "prefill geometry exceeds admitted launch range");
         rc = yvex_rocm_launch(backend, YVEX_ROCM_FN_PREFILL_BF16,

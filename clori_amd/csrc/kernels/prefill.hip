@@ -14,11 +14,18 @@
 // registers 8u..8u+7; V^T is fetched from LDS in the matching key order.  Softmax
 // statistics are per lane (= per query row) plus one exchange with lane^32.
 //
-// LDS layout (chosen so every MFMA operand fetch is bank-conflict free on 64 banks):
-//     K tile    [64 keys][128 dims] bf16, row pitch 272 B   ds_read_b128 per A operand
-//     V^T tile  [128 dims][64 keys] bf16, row pitch 136 B   2 x ds_read_b64 per A operand
-// Two buffers of each; the global loads of tile t+1 are issued before the products of
-// tile t and land in registers while the MFMAs run, one barrier per tile.
+// LDS layout: K and V tiles are both [64 keys][128 dims] bf16 in row-major order with
+// 256-byte rows and no padding; the 16-byte chunk c of row r sits at chunk position
+// c ^ x(r), x(r) = ((r & 3) << 2) | ((r >> 2) & 3).  That makes both operand fetches
+// bank-conflict free: the K operand is one ds_read_b128 per lane (16 rows x one chunk
+// column hit 16 distinct chunk positions), the V^T operand is two ds_read_b64_tr_b16
+// (each 16-lane group transposes 4 keys x 16 dims; 4 consecutive rows place one 64-byte
+// column segment in 4 distinct bank groups).
+// The tiles are filled by buffer loads that write LDS directly (no staging registers,
+// no LDS store instructions): lane L of a 1 KB load owns chunk position L % 16 of row
+// L / 16 and fetches the global chunk that belongs there.  Rows past the end of the
+// tensor read as zero through the buffer range check.  Two buffers; the loads of tile
+// t+1 are issued right after the barrier of tile t, one barrier per tile.
 //
 // The running maximum is only raised when a tile exceeds it by more than kLazyLog2 (in
 // log2 units), so the accumulator rescale is rare; probabilities are then at most
@@ -33,13 +40,17 @@ namespace {
 
 constexpr int kHeadDim = 128;
 constexpr int kKeyTile = 64;
-constexpr int kKPitch = 272;   // bytes per K row in LDS
-constexpr int kVPitch = 136;   // bytes per V^T row in LDS
-constexpr int kKBytes = kKeyTile * kKPitch;   // 17408
-constexpr int kVBytes = kHeadDim * kVPitch;   // 17408
-constexpr int kBufBytes = kKBytes + kVBytes;
+constexpr int kRowBytes = kHeadDim * 2;            // 256
+constexpr int kTileBytes = kKeyTile * kRowBytes;   // 16384 per K or V tile
+constexpr int kBufBytes = 2 * kTileBytes;          // K then V
 constexpr int kThreads = 256;
 constexpr float kLazyLog2 = 8.0f;
+
+typedef __attribute__((address_space(3))) void lds_void;
+typedef __attribute__((address_space(3))) short4v lds_short4;
+
+// chunk swizzle of tile row r
+__device__ inline int swizzle(int r) { return ((r & 3) << 2) | ((r >> 2) & 3); }
 
 __device__ inline void flag(int32_t *status, int code) { atomicCAS(status, 0, code); }
 
@@ -74,44 +85,59 @@ __device__ inline void prefill_body(const yvex_rocm_prefill_params &p, unsigned 
         for (int kk = 0; kk < 8; ++kk) q[nb][kk] = as_bf16x8(load_b128(src + kk * 16));
     }
 
-    const uint16_t *kbase = p.k + (uint64_t)kv_head * kHeadDim;
-    const uint16_t *vbase = p.v + (uint64_t)kv_head * kHeadDim;
+    // ---- tile staging: buffer loads that write LDS directly -----------------------
+    // 1 KB load j of wave w fills rows 16w + 4j .. +3 of the tile; lane L owns chunk
+    // position L % 16 of row 16w + 4j + L / 16 and fetches chunk (L % 16) ^ x(row).
+    const uint32_t k_row_bytes = (uint32_t)p.k_stride * 2u, v_row_bytes = (uint32_t)p.v_stride * 2u;
+    const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)(p.k + (uint64_t)kv_head * kHeadDim), 0,
+        p.kv_tokens * k_row_bytes - kv_head * kRowBytes, 0x00027000);
+    const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)(p.v + (uint64_t)kv_head * kHeadDim), 0,
+        p.kv_tokens * v_row_bytes - kv_head * kRowBytes, 0x00027000);
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    uint32_t k_off[4], v_off[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int r = 16 * wave + 4 * j + (lane >> 4);
+        const uint32_t chunk = (uint32_t)((lane & 15) ^ swizzle(r));
+        k_off[j] = (uint32_t)r * k_row_bytes + chunk * 16u;
+        v_off[j] = (uint32_t)r * v_row_bytes + chunk * 16u;
+    }
+    auto stage_tile = [&](uint32_t tile, int buf) {
+        unsigned char *dst = lds + buf * kBufBytes + wave_u * 4096;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(k_rsrc, (lds_void *)(dst + j * 1024), 16,
+                                                     k_off[j], tile * kKeyTile * k_row_bytes, 0, 0);
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(v_rsrc,
+                                                     (lds_void *)(dst + kTileBytes + j * 1024), 16,
+                                                     v_off[j], tile * kKeyTile * v_row_bytes, 0, 0);
+    };
 
-    // global -> registers for one tile.  K: thread covers rows tid/16 + 16r, chunk tid%16.
-    // V: thread covers keys 4*(tid%16) .. +3 and dims 8*(tid/16) .. +7 (transposed on store).
-    u32x4 kreg[4], vreg[4];
-    auto load_tile = [&](uint32_t tile) {
-        const uint32_t first = tile * kKeyTile;
-        const uint32_t last = p.kv_tokens - 1u;
+    // ---- operand addresses inside a tile ------------------------------------------
+    // K operand (mb, kk): row mb*32 + n, chunk (2kk + g) ^ x(n); one address per kk
+    uint32_t k_addr[8];
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const uint32_t key = min(first + (uint32_t)(tid >> 4) + 16u * r, last);
-            kreg[r] = load_b128(kbase + (uint64_t)key * p.k_stride + (tid & 15) * 8);
-        }
+    for (int kk = 0; kk < 8; ++kk)
+        k_addr[kk] = (uint32_t)(n * kRowBytes + (((2 * kk + g) ^ swizzle(n)) << 4));
+    // V^T operand (db, mb, u, h): 16-lane group b = lane / 16 (dims 16 * (b & 1), key half
+    // g = b / 2), lane a = lane % 16 addresses key row mb*32 + 16u + 8h + 4g + a/4 and
+    // dims db*32 + 16*(b&1) + 4*(a%4) .. +3; one address per (db, h)
+    uint32_t v_addr[4][2];
+    {
+        const int a = lane & 15, b1 = (lane >> 4) & 1;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const uint32_t key = min(first + 4u * (tid & 15) + r, last);
-            vreg[r] = load_b128(vbase + (uint64_t)key * p.v_stride + (tid >> 4) * 8);
-        }
-    };
-    auto store_tile = [&](int buf) {
-        unsigned char *kl = lds + buf * kBufBytes;
-        unsigned char *vl = kl + kKBytes;
+        for (int db = 0; db < 4; ++db)
 #pragma unroll
-        for (int r = 0; r < 4; ++r)
-            *reinterpret_cast<u32x4 *>(kl + ((tid >> 4) + 16 * r) * kKPitch + (tid & 15) * 16) =
-                kreg[r];
-        // transpose 4 keys x 8 dims: dim e of the chunk gets the four keys' values
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            const int w = e >> 1;
-            const uint32_t sel = (e & 1) ? 0x07060302u : 0x05040100u;
-            u32x2 out;
-            out.x = __builtin_amdgcn_perm(vreg[1][w], vreg[0][w], sel);
-            out.y = __builtin_amdgcn_perm(vreg[3][w], vreg[2][w], sel);
-            *reinterpret_cast<u32x2 *>(vl + ((tid >> 4) * 8 + e) * kVPitch + (tid & 15) * 8) = out;
-        }
-    };
+            for (int h = 0; h < 2; ++h) {
+                const int r = 8 * h + 4 * g + (a >> 2);
+                const int chunk = (db * 4 + 2 * b1 + ((a >> 1) & 1)) ^ swizzle(r);
+                v_addr[db][h] = (uint32_t)(kTileBytes + r * kRowBytes + (chunk << 4) + 8 * (a & 1));
+            }
+    }
 
     floatx16 o[4][NB];
 #pragma unroll
@@ -131,21 +157,19 @@ __device__ inline void prefill_body(const yvex_rocm_prefill_params &p, unsigned 
     const bool wave_active = row0 < p.query_tokens;
     // last key visible to the wave's first / last row (causal)
     const uint32_t wave_first_vis = p.causal ? p.query_start + row0 : p.kv_tokens - 1u;
+    const uint32_t wave_last_vis =
+        p.causal ? p.query_start + min(row0 + kRowsPerWave, p.query_tokens) - 1u : p.kv_tokens - 1u;
 
-    load_tile(0u);
+    stage_tile(0u, 0);
     for (uint32_t t = 0; t < tiles; ++t) {
         const int buf = (int)(t & 1u);
-        store_tile(buf);
+        __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's part of tile t is in LDS
         __syncthreads();
-        if (t + 1u < tiles) load_tile(t + 1u);
+        if (t + 1u < tiles) stage_tile(t + 1u, buf ^ 1);
         const uint32_t key0 = t * kKeyTile;
         // a wave whose every row sees nothing of this tile skips the products
-        const uint32_t wave_last_vis = p.causal
-                                           ? p.query_start + min(row0 + kRowsPerWave, p.query_tokens) - 1u
-                                           : p.kv_tokens - 1u;
         if (!wave_active || key0 > wave_last_vis) continue;
-        const unsigned char *kl = lds + buf * kBufBytes;
-        const unsigned char *vl = kl + kKBytes;
+        const unsigned char *tile = lds + buf * kBufBytes;
 
         // ---- S^T = K . Q^T -------------------------------------------------
         floatx16 s[2][NB];
@@ -160,7 +184,7 @@ __device__ inline void prefill_body(const yvex_rocm_prefill_params &p, unsigned 
 #pragma unroll
             for (int mb = 0; mb < 2; ++mb) {
                 const bf16x8 a = as_bf16x8(*reinterpret_cast<const u32x4 *>(
-                    kl + (mb * 32 + n) * kKPitch + kk * 32 + g * 16));
+                    tile + k_addr[kk] + mb * 32 * kRowBytes));
 #pragma unroll
                 for (int nb = 0; nb < NB; ++nb) s[mb][nb] = mfma_32x32x16(a, q[nb][kk], s[mb][nb]);
             }
@@ -229,17 +253,16 @@ __device__ inline void prefill_body(const yvex_rocm_prefill_params &p, unsigned 
                 }
 #pragma unroll
                 for (int db = 0; db < 4; ++db) {
-                    const unsigned char *row = vl + (db * 32 + n) * kVPitch + (mb * 32 + u * 16 + g * 4) * 2;
-                    u32x4 a;
-                    const u32x2 lo = *reinterpret_cast<const u32x2 *>(row);
-                    const u32x2 hi = *reinterpret_cast<const u32x2 *>(row + 16);
-                    a.x = lo.x;
-                    a.y = lo.y;
-                    a.z = hi.x;
-                    a.w = hi.y;
+                    const int base = (mb * 32 + u * 16) * kRowBytes;
+                    const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                        (lds_short4 *)(tile + v_addr[db][0] + base));
+                    const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                        (lds_short4 *)(tile + v_addr[db][1] + base));
+                    typedef short short8v __attribute__((ext_vector_type(8)));
+                    const short8v av = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                    const bf16x8 a = __builtin_bit_cast(bf16x8, av);
 #pragma unroll
-                    for (int nb = 0; nb < NB; ++nb)
-                        o[db][nb] = mfma_32x32x16(as_bf16x8(a), pb[nb], o[db][nb]);
+                    for (int nb = 0; nb < NB; ++nb) o[db][nb] = mfma_32x32x16(a, pb[nb], o[db][nb]);
                 }
             }
     }
