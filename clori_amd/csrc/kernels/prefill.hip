@@ -189,6 +189,14 @@ __device__ inline void prefill_body(const yvex_rocm_prefill_params &p, unsigned 
                 for (int nb = 0; nb < NB; ++nb) s[mb][nb] = mfma_32x32x16(a, q[nb][kk], s[mb][nb]);
             }
         }
+        // keep three operand pairs in flight ahead of the MFMAs that consume them
+        __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);
+#pragma unroll
+        for (int i = 0; i < 5; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 2 * NB, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, 6 * NB, 0);
 
         // ---- mask, online softmax (per lane = per query row) ----------------------
         // scores stay raw; the softmax scale is folded into the exponent's multiply-add
