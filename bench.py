@@ -18,7 +18,6 @@ events recorded on the backend's own stream (the stream the kernels are launched
 """
 import argparse
 import json
-import math
 import os
 import sys
 import time
@@ -52,9 +51,11 @@ def random_bf16(rng, count, unique=1 << 24):
     return np.tile(base, reps)[:count]
 
 
-def time_steps(backend, run, steps, warmup):
+def time_steps(backend, run, steps, warmup, kernel):
     """W untimed steps, then K steps bracketed by device events and by a synchronise on
-    both sides.  Returns (device ms per step, wall ms per step)."""
+    both sides; then the same K steps again with an event pair around every launch of the
+    dominant kernel.  Returns (device ms per step, wall ms per step, ms per launch of the
+    dominant kernel)."""
     backend.set_completion_mode(B.COMPLETION_DEFERRED)
     for _ in range(warmup):
         run()
@@ -66,8 +67,13 @@ def time_steps(backend, run, steps, warmup):
     device_ms = backend.timing_end()
     backend.sync()
     wall_ms = (time.perf_counter() - t0) * 1e3
+    backend.kernel_probe_begin(kernel)
+    for _ in range(min(steps, 256)):
+        run()
+    launches, kernel_ms = backend.kernel_probe_end()
+    backend.sync()
     backend.set_completion_mode(B.COMPLETION_IMMEDIATE)
-    return device_ms / steps, wall_ms / steps
+    return device_ms / steps, wall_ms / steps, kernel_ms / max(launches, 1)
 
 
 # --------------------------------------------------------------------- workloads --
@@ -97,8 +103,7 @@ def workload_paged(backend, rng, steps, warmup, q8=False):
         codes = rng.integers(-127, 128, size=(1 << 22), dtype=np.int8).view(np.uint8)
         reps = (pool_pages * hkv * 2048 + codes.size - 1) // codes.size
         pool[:, :2048] = np.tile(codes, reps)[:pool_pages * hkv * 2048].reshape(-1, 2048)
-        pool[:, 2048:] = np.tile(np.float16(0.025).view(np.uint8) if False else
-                                 np.array([0.025], np.float16).view(np.uint8), 64)[None, :]
+        pool[:, 2048:] = np.tile(np.array([0.025], np.float16).view(np.uint8), 64)[None, :]
         k_pool = backend.tensor("k-pages", B.DTYPE_I8, (pool_bytes,), pool)
         v_pool = backend.tensor("v-pages", B.DTYPE_I8, (pool_bytes,), pool[::-1].copy())
     else:
@@ -118,7 +123,8 @@ def workload_paged(backend, rng, steps, warmup, q8=False):
     backend.workspace_attach(work)
     run = lambda: backend.paged_decode_execute(req, q, k_pool, v_pool, tt, tc, out, lse)  # noqa: E731
     facts = run()
-    ms, wall = time_steps(backend, run, steps, warmup)
+    kernel = "yvex_rocm_decode_paged_q8_0" if q8 else "yvex_rocm_decode_paged_bf16"
+    ms, wall, kms = time_steps(backend, run, steps, warmup, kernel)
     backend.workspace_detach()
     tokens = int(contexts.sum())
     per_token = 2 * hkv * (136 if q8 else 256)
@@ -130,8 +136,7 @@ def workload_paged(backend, rng, steps, warmup, q8=False):
                          "16-token pages, seeded permutation page tables" %
                          ("Q8_0" if q8 else "bf16", lo, hi),
                 bound="hbm", algorithmic_bytes=algo, tokens=tokens, ms=ms, wall_ms=wall,
-                launches=int(facts.kernel_launches),
-                dominant_kernel="yvex_rocm_decode_paged_q8_0" if q8 else "yvex_rocm_decode_paged_bf16")
+                kernel_ms=kms, launches=int(facts.kernel_launches), dominant_kernel=kernel)
 
 
 def workload_decode1(backend, rng, steps, warmup):
@@ -148,12 +153,12 @@ def workload_decode1(backend, rng, steps, warmup):
     backend.workspace_attach(work)
     run = lambda: backend.attention_execute(req, q, k, v, out, lse=lse)  # noqa: E731
     facts = run()
-    ms, wall = time_steps(backend, run, steps, warmup)
+    ms, wall, kms = time_steps(backend, run, steps, warmup, "yvex_rocm_decode_rows_bf16")
     backend.workspace_detach()
     algo = 2 * ctx * hkv * d * 2 + 2 * hq * d * 2 + hq * 4
     return dict(name="decode1",
                 workload="GQA decode: batch 1, 32/8 heads, d=128, context 4096, contiguous bf16 KV",
-                bound="hbm", algorithmic_bytes=algo, tokens=ctx, ms=ms, wall_ms=wall,
+                bound="hbm", algorithmic_bytes=algo, tokens=ctx, ms=ms, wall_ms=wall, kernel_ms=kms,
                 launches=int(facts.kernel_launches), dominant_kernel="yvex_rocm_decode_rows_bf16")
 
 
@@ -172,12 +177,12 @@ def workload_prefill2(backend, rng, steps, warmup):
                                         contract=B.NUMERIC_BF16_F32_ACCUMULATE)
     run = lambda: backend.attention_execute(req, q, k, v, out)  # noqa: E731
     facts = run()
-    ms, wall = time_steps(backend, run, steps, warmup)
+    ms, wall, kms = time_steps(backend, run, steps, warmup, "yvex_rocm_prefill_bf16")
     flops = 4 * d * hq * t * (t + 1) // 2      # causal-useful multiply-adds * 2, QK^T and PV
     return dict(name="prefill2",
                 workload="causal GQA prefill: batch 1, seq 2048, 40/8 heads, d=128, bf16",
                 bound="mfma", flops=flops, algorithmic_bytes=(2 * t * hq * d + 2 * t * hkv * d) * 2,
-                ms=ms, wall_ms=wall, launches=int(facts.kernel_launches),
+                ms=ms, wall_ms=wall, kernel_ms=kms, launches=int(facts.kernel_launches),
                 dominant_kernel="yvex_rocm_prefill_bf16")
 
 
@@ -199,7 +204,7 @@ def workload_mla5(backend, rng, steps, warmup):
     backend.workspace_attach(work)
     run = lambda: backend.mla_decode_execute(req, q, pool, tt, tc, out, lse)  # noqa: E731
     facts = run()
-    ms, wall = time_steps(backend, run, steps, warmup)
+    ms, wall, kms = time_steps(backend, run, steps, warmup, "yvex_rocm_mla_decode_bf16")
     backend.workspace_detach()
     algo = batch * ctx * kd * 2 + batch * heads * (kd + vd) * 2 + table.size * 4 + batch * heads * 4
     assert np.all(np.isfinite(lse.read()))
@@ -207,8 +212,24 @@ def workload_mla5(backend, rng, steps, warmup):
                 workload="absorbed MLA decode: batch 16, 128 heads, latent 512 + rope 64, "
                          "context 8192 in 64-token pages",
                 bound="hbm", algorithmic_bytes=algo, flops=batch * heads * ctx * 2 * (kd + vd),
-                ms=ms, wall_ms=wall, launches=int(facts.kernel_launches),
+                ms=ms, wall_ms=wall, kernel_ms=kms, launches=int(facts.kernel_launches),
                 dominant_kernel="yvex_rocm_mla_decode_bf16")
+
+
+def copy_reference(backend, steps):
+    """A device-to-device copy of known size: the scale for the FETCH_SIZE / WRITE_SIZE
+    counters.  Not a workload of the metric; run as --workload copy."""
+    nbytes = 1 << 30
+    src = backend.tensor("copy-src", B.DTYPE_I8, (nbytes,))
+    dst = backend.tensor("copy-dst", B.DTYPE_I8, (nbytes,))
+    src.zero()
+    backend.sync()
+    backend.timing_begin()
+    for _ in range(steps):
+        dst.copy_from(src)
+    ms = backend.timing_end() / steps
+    return dict(bytes_read=nbytes, bytes_written=nbytes, ms_per_copy=ms,
+                gbs=2 * nbytes / (ms * 1e-3) / 1e9)
 
 
 WORKLOADS = {
@@ -222,28 +243,52 @@ SEEDS = {"decode1": 1, "prefill2": 2, "paged3": 3, "paged4": 4, "mla5": 5}
 
 
 def roofline(result):
-    seconds = result["ms"] * 1e-3
+    """Roofline record of the dominant kernel: algorithmic bytes (or flops) of one launch
+    over that kernel's own mean duration.  `step` repeats the figure for the whole step
+    (every launch of the operator), which is what `value` reports."""
+    seconds = result["kernel_ms"] * 1e-3
+    step_seconds = result["ms"] * 1e-3
     if result["bound"] == "hbm":
         achieved = result["algorithmic_bytes"] / seconds / 1e9
         return dict(bound="hbm", achieved=achieved, peak=HBM_PEAK_GBS, unit="GB/s",
-                    frac=achieved / HBM_PEAK_GBS, traffic=None,
-                    kernel=result["dominant_kernel"])
+                    frac=achieved / HBM_PEAK_GBS, traffic=TRAFFIC.get(result["name"]),
+                    kernel=result["dominant_kernel"], kernel_us=result["kernel_ms"] * 1e3,
+                    step=result["algorithmic_bytes"] / step_seconds / 1e9)
     achieved = result["flops"] / seconds / 1e12
     return dict(bound="mfma", achieved=achieved, peak=MFMA_BF16_PEAK_TFLOPS, unit="TFLOP/s",
-                frac=achieved / MFMA_BF16_PEAK_TFLOPS, traffic=None,
-                kernel=result["dominant_kernel"])
+                frac=achieved / MFMA_BF16_PEAK_TFLOPS, traffic=TRAFFIC.get(result["name"]),
+                kernel=result["dominant_kernel"], kernel_us=result["kernel_ms"] * 1e3,
+                step=result["flops"] / step_seconds / 1e12)
 
 
-def cpu_baseline(name):
-    """The oracle (a port of the reference CPU operator) timed on this host's cores on a
-    bounded sample of the same workload."""
+# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# runs (profiles/), scaled by the same counters on a copy kernel of known size; None where
+# no such run is committed.
+TRAFFIC = {}
+
+
+def repeat_for(seconds, call):
+    """Calls `call` until `seconds` of wall time have passed; returns (runs, mean seconds)."""
+    runs, t0 = 0, time.perf_counter()
+    while True:
+        rc = call()
+        assert rc == 0
+        runs += 1
+        dt = time.perf_counter() - t0
+        if dt >= seconds:
+            return runs, dt / runs
+
+
+def cpu_baseline(name, budget=6.0):
+    """The oracle (a port of the reference CPU operator, all host threads) timed on a bounded
+    sample of the same workload: the sample is repeated for about `budget` seconds."""
     from oracle_binding import Oracle
     oracle = Oracle()
     rng = np.random.default_rng(SEEDS[name])
     threads = oracle.threads
     if name in ("paged3", "paged4"):
-        sessions, hq, hkv, d, page = 2, 32, 8, 128, 16
-        contexts = np.array([8192, 8192], dtype=np.int32)
+        sessions, hq, hkv, d, page = 4, 32, 8, 128, 16
+        contexts = np.full(sessions, 8192, dtype=np.int32)
         pool_pages = int(contexts.sum()) // page
         table = rng.permutation(pool_pages).astype(np.int32).reshape(sessions, -1)
         k = bf16_bits(rng.standard_normal((pool_pages, page, hkv, d), dtype=np.float32))
@@ -253,25 +298,45 @@ def cpu_baseline(name):
         if q8:
             k = oracle.q8_0_encode_rows(oracle.bf16_decode(k))
             v = oracle.q8_0_encode_rows(oracle.bf16_decode(v))
-        t0 = time.perf_counter()
-        rc, *_ = oracle.paged_decode(q, k, v, table, contexts, hkv, page, q8=q8)
-        dt = time.perf_counter() - t0
-        assert rc == 0
+        runs, dt = repeat_for(budget, lambda: oracle.paged_decode(q, k, v, table, contexts, hkv,
+                                                                  page, q8=q8)[0])
         per_token = 2 * hkv * (136 if q8 else 256)
-        value = int(contexts.sum()) * per_token / dt / 1e9
-        return dict(value=value, unit="GB/s", cores=threads, kind="port",
-                    sample="2 sessions x 8192 tokens of the same shape, %.1f s" % dt)
+        return dict(value=int(contexts.sum()) * per_token / dt / 1e9, unit="GB/s", cores=threads,
+                    kind="port", sample="4 sessions x 8192 tokens of the same shape, mean of "
+                                        "%d runs (%.1f s)" % (runs, runs * dt))
     if name == "decode1":
         q = bf16_bits(rng.standard_normal((1, 32, 128), dtype=np.float32))
         k = bf16_bits(rng.standard_normal((4096, 8, 128), dtype=np.float32))
         v = bf16_bits(rng.standard_normal((4096, 8, 128), dtype=np.float32))
-        reps, t0 = 20, time.perf_counter()
-        for _ in range(reps):
-            rc, *_ = oracle.gqa_bf16(q, k, v, query_start=4095)
-        dt = (time.perf_counter() - t0) / reps
+        runs, dt = repeat_for(budget / 2, lambda: oracle.gqa_bf16(q, k, v, query_start=4095)[0])
         return dict(value=(2 * 4096 * 8 * 128 * 2) / dt / 1e9, unit="GB/s", cores=threads,
-                    kind="port", sample="the full workload, mean of %d runs" % reps)
+                    kind="port", sample="the full workload, mean of %d runs (%.1f s)" %
+                                        (runs, runs * dt))
+    if name == "prefill2":
+        t, hq, hkv, d = 1024, 40, 8, 128
+        q = bf16_bits(rng.standard_normal((t, hq, d), dtype=np.float32))
+        k = bf16_bits(rng.standard_normal((t, hkv, d), dtype=np.float32))
+        v = bf16_bits(rng.standard_normal((t, hkv, d), dtype=np.float32))
+        runs, dt = repeat_for(budget, lambda: oracle.gqa_bf16(q, k, v, query_start=0)[0])
+        return dict(value=4 * d * hq * t * (t + 1) // 2 / dt / 1e12, unit="TFLOP/s", cores=threads,
+                    kind="port", sample="the first 1024 tokens of the same shape, mean of %d runs "
+                                        "(%.1f s)" % (runs, runs * dt))
+    if name == "mla5":
+        batch, heads, kd, vd, page, ctx = 2, 128, 576, 512, 64, 4096
+        pages = batch * ctx // page
+        table = rng.permutation(pages).astype(np.int32).reshape(batch, -1)
+        pool = bf16_bits(rng.standard_normal((pages, page, kd), dtype=np.float32))
+        q = bf16_bits(rng.standard_normal((batch, heads, kd), dtype=np.float32))
+        contexts = np.full(batch, ctx, np.int32)
+        runs, dt = repeat_for(budget, lambda: oracle.mla_decode(q, pool, table, contexts, vd,
+                                                                page)[0])
+        return dict(value=batch * ctx * kd * 2 / dt / 1e9, unit="GB/s", cores=threads, kind="port",
+                    sample="2 batch elements x 4096 tokens of the same shape, mean of %d runs "
+                           "(%.1f s)" % (runs, runs * dt))
     return None
+
+
+METRIC = "decode attn HBM GB/s (% of peak); prefill attn TFLOPS (% MFMA peak), 1 GPU"
 
 
 def main():
@@ -279,13 +344,19 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="paged3",
-                    help="headline workload, or 'all' to run every workload")
+    ap.add_argument("--workload", default="all",
+                    help="one workload name, or 'all' (default): every configuration, with "
+                         "the paged bf16 decode as the headline value")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; --gpus %d is not supported "
                  "(attention shards by session or head without exchange)" % args.gpus)
+    if args.workload == "copy":
+        backend = Backend()
+        print(json.dumps({"copy_reference": copy_reference(backend, min(args.steps, 10))}))
+        backend.close()
+        return
     names = list(WORKLOADS) if args.workload == "all" else [args.workload]
     headline = "paged3" if args.workload == "all" else args.workload
     results = {}
@@ -298,9 +369,10 @@ def main():
         backend.close()
     head = results[headline]
     roof = roofline(head)
+    cpu = {} if args.no_cpu else {n: cpu_baseline(n) for n in names}
     line = {
-        "metric": "decode attn HBM GB/s" if head["bound"] == "hbm" else "prefill attn TFLOPS",
-        "value": roof["achieved"],
+        "metric": METRIC,
+        "value": roof["step"],
         "unit": roof["unit"],
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": head["ms"],
@@ -309,9 +381,11 @@ def main():
         "config": {"workload": head["workload"], "name": head["name"],
                    "kernel_launches_per_step": head["launches"]},
         "roofline": roof,
-        "cpu_baseline": None if args.no_cpu else cpu_baseline(headline),
-        "workloads": {n: dict(ms_per_step=r["ms"], wall_ms_per_step=r["wall_ms"],
-                              roofline=roofline(r)) for n, r in results.items()},
+        "cpu_baseline": cpu.get(headline),
+        "workloads": {n: dict(workload=r["workload"], ms_per_step=r["ms"],
+                              wall_ms_per_step=r["wall_ms"], value=roofline(r)["step"],
+                              unit=roofline(r)["unit"], roofline=roofline(r),
+                              cpu_baseline=cpu.get(n)) for n, r in results.items()},
     }
     print(json.dumps(line))
 

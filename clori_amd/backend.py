@@ -81,6 +81,12 @@ class Tensor:
         err = B.Error()
         _check(lib().yvex_backend_tensor_zero(self.backend.handle, self.handle, C.byref(err)), err)
 
+    def copy_from(self, source):
+        """Device-to-device copy of a tensor with the same descriptor."""
+        err = B.Error()
+        _check(lib().yvex_backend_tensor_copy(self.backend.handle, self.handle, source.handle,
+                                              C.byref(err)), err)
+
     def release(self):
         if self.handle:
             err = B.Error()
@@ -177,6 +183,19 @@ class Backend:
         ms, err = C.c_double(0.0), B.Error()
         _check(lib().yvex_backend_rocm_timing_end(self.handle, C.byref(ms), C.byref(err)), err)
         return ms.value
+
+    def kernel_probe_begin(self, kernel):
+        """Brackets every launch of the named bundle kernel with its own event pair."""
+        err = B.Error()
+        _check(lib().yvex_backend_rocm_kernel_probe_begin(self.handle, kernel.encode(),
+                                                          C.byref(err)), err)
+
+    def kernel_probe_end(self):
+        """Returns (measured launches, summed device milliseconds)."""
+        count, ms, err = C.c_uint(0), C.c_double(0.0), B.Error()
+        _check(lib().yvex_backend_rocm_kernel_probe_end(self.handle, C.byref(count), C.byref(ms),
+                                                        C.byref(err)), err)
+        return count.value, ms.value
 
     # -- tensors ----------------------------------------------------------
     def tensor(self, name, dtype, shape, data=None, nbytes=None):

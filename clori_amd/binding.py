@@ -210,6 +210,7 @@ EXPORTED_SYMBOLS = [
     "yvex_backend_op_attention", "yvex_backend_transformer_operations_get",
     "yvex_backend_rocm_attention_operations_get", "yvex_backend_rocm_completion_mode_set",
     "yvex_backend_rocm_timing_begin", "yvex_backend_rocm_timing_end",
+    "yvex_backend_rocm_kernel_probe_begin", "yvex_backend_rocm_kernel_probe_end",
     "yvex_backend_rocm_report_get", "yvex_quant_f16_decode", "yvex_quant_f16_encode",
     "yvex_quant_bf16_decode", "yvex_quant_bf16_encode", "yvex_rocm_q8_0_encode_row",
     "yvex_rocm_q8_0_decode_row", "yvex_rocm_kv_page_block_bytes", "yvex_rocm_kv_pack_pages",
@@ -278,6 +279,8 @@ def load(path=None):
     lib.yvex_backend_rocm_completion_mode_set.argtypes = [vp, C.c_int, ErrorP]
     lib.yvex_backend_rocm_timing_begin.argtypes = [vp, ErrorP]
     lib.yvex_backend_rocm_timing_end.argtypes = [vp, C.POINTER(C.c_double), ErrorP]
+    lib.yvex_backend_rocm_kernel_probe_begin.argtypes = [vp, C.c_char_p, ErrorP]
+    lib.yvex_backend_rocm_kernel_probe_end.argtypes = [vp, C.POINTER(C.c_uint), C.POINTER(C.c_double), ErrorP]
     lib.yvex_backend_rocm_report_get.argtypes = [vp, C.POINTER(RocmReport), ErrorP]
     lib.yvex_quant_f16_decode.restype = C.c_float
     lib.yvex_quant_f16_decode.argtypes = [C.c_ushort]

@@ -8,6 +8,8 @@
 #include <stdlib.h>
 #include <string.h>
 
+static void probe_release(yvex_rocm_backend_state *state);
+
 static int refuse(yvex_error *err, yvex_status status, const char *where, const char *reason)
 {
     yvex_error_set(err, status, where, reason);
@@ -291,6 +293,7 @@ static int rocm_close(yvex_backend *backend, yvex_error *err)
     rc = yvex_rocm_kernel_bundle_close(backend, err);
     if (rc != YVEX_OK) return rc; /* impl retained: checked close can be retried */
     if (state->device_status) (void)state->driver.hipFree(state->device_status);
+    probe_release(state);
     if (state->timing_start) (void)state->driver.hipEventDestroy(state->timing_start);
     if (state->timing_stop) (void)state->driver.hipEventDestroy(state->timing_stop);
     if (state->stream) (void)state->driver.hipStreamDestroy(state->stream);
@@ -343,6 +346,7 @@ int yvex_backend_open_rocm_impl(yvex_backend **out, const char *device,
     *out = NULL;
     backend = (yvex_backend *)calloc(1, sizeof(*backend));
     state = (yvex_rocm_backend_state *)calloc(1, sizeof(*state));
+    if (state) state->probe_function = -1;
     if (!backend || !state) {
         free(backend);
         free(state);
@@ -458,6 +462,78 @@ int yvex_backend_rocm_completion_mode_set(yvex_backend *backend, yvex_rocm_compl
     state->completion_mode = mode;
     yvex_error_clear(err);
     return YVEX_OK;
+}
+
+static void probe_release(yvex_rocm_backend_state *state)
+{
+    unsigned int i;
+    for (i = 0; i < 2u * YVEX_ROCM_PROBE_MAX; ++i)
+        if (state->probe_events[i]) {
+            (void)state->driver.hipEventDestroy(state->probe_events[i]);
+            state->probe_events[i] = NULL;
+        }
+    state->probe_count = 0u;
+    state->probe_function = -1;
+}
+
+int yvex_backend_rocm_kernel_probe_begin(yvex_backend *backend, const char *kernel,
+                                         yvex_error *err)
+{
+    yvex_rocm_backend_state *state = yvex_rocm_state(backend);
+    unsigned int i;
+    int function, rc;
+    if (!state || !kernel)
+        return refuse(err, YVEX_ERR_INVALID_ARG, "rocm.probe", "ROCm backend and kernel name are required");
+    rc = backend_dispatch_admit(backend, "rocm.probe", err);
+    if (rc != YVEX_OK) return rc;
+    function = yvex_rocm_function_find(kernel);
+    if (function < 0 || !state->functions[function])
+        return refuse(err, YVEX_ERR_UNSUPPORTED, "rocm.probe", "no such kernel in the admitted bundle");
+    if (state->probe_function >= 0)
+        return refuse(err, YVEX_ERR_STATE, "rocm.probe", "a kernel probe is already open");
+    for (i = 0; i < 2u * YVEX_ROCM_PROBE_MAX; ++i) {
+        if (state->probe_events[i]) continue;
+        rc = yvex_rocm_status(&state->driver, state->driver.hipEventCreate(&state->probe_events[i]),
+                              "rocm.probe.begin", err);
+        if (rc != YVEX_OK) {
+            probe_release(state);
+            return rc;
+        }
+    }
+    state->probe_count = 0u;
+    state->probe_function = function;
+    yvex_error_clear(err);
+    return YVEX_OK;
+}
+
+int yvex_backend_rocm_kernel_probe_end(yvex_backend *backend, unsigned int *launches,
+                                       double *milliseconds, yvex_error *err)
+{
+    yvex_rocm_backend_state *state = yvex_rocm_state(backend);
+    double total = 0.0;
+    unsigned int i;
+    int rc = YVEX_OK;
+    if (!state || !launches || !milliseconds || state->probe_function < 0)
+        return refuse(err, YVEX_ERR_STATE, "rocm.probe.end", "no kernel probe is open");
+    state->probe_function = -1;
+    if (state->probe_count)
+        rc = yvex_rocm_status(&state->driver,
+                              state->driver.hipEventSynchronize(
+                                  state->probe_events[2u * state->probe_count - 1u]),
+                              "rocm.probe.end", err);
+    for (i = 0; rc == YVEX_OK && i < state->probe_count; ++i) {
+        float elapsed = 0.0f;
+        rc = yvex_rocm_status(&state->driver,
+                              state->driver.hipEventElapsedTime(&elapsed, state->probe_events[2u * i],
+                                                                state->probe_events[2u * i + 1u]),
+                              "rocm.probe.end", err);
+        total += (double)elapsed;
+    }
+    *launches = rc == YVEX_OK ? state->probe_count : 0u;
+    *milliseconds = rc == YVEX_OK ? total : 0.0;
+    state->probe_count = 0u;
+    if (rc == YVEX_OK) yvex_error_clear(err);
+    return rc;
 }
 
 int yvex_backend_rocm_timing_begin(yvex_backend *backend, yvex_error *err)

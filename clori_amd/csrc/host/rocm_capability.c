@@ -310,6 +310,17 @@ int yvex_rocm_require_capability(yvex_backend *backend, yvex_backend_operation_v
     return rc;
 }
 
+/* Function id of a bundle symbol, -1 when the bundle has no such kernel. */
+int yvex_rocm_function_find(const char *symbol)
+{
+    size_t i;
+    if (!symbol) return -1;
+    for (i = 0; i < sizeof(rocm_kernel_bindings) / sizeof(rocm_kernel_bindings[0]); ++i)
+        if (strcmp(rocm_kernel_bindings[i].symbol, symbol) == 0)
+            return (int)rocm_kernel_bindings[i].slot;
+    return -1;
+}
+
 /* src/backend/cuda/capability.c:750-791 */
 int yvex_rocm_launch(yvex_backend *backend, yvex_rocm_function_id function,
                      yvex_backend_operation_variant variant, unsigned int grid_x,
@@ -318,6 +329,7 @@ int yvex_rocm_launch(yvex_backend *backend, yvex_rocm_function_id function,
 {
     yvex_rocm_backend_state *state = yvex_rocm_state(backend);
     void *arguments[1];
+    int probe;
     int rc = yvex_rocm_require_capability(backend, variant, where, err);
     if (rc != YVEX_OK) return rc;
     if (!state || function >= YVEX_ROCM_FN_COUNT || !state->functions[function]) {
@@ -335,12 +347,20 @@ int yvex_rocm_launch(yvex_backend *backend, yvex_rocm_function_id function,
         return YVEX_ERR_BACKEND;
     }
     arguments[0] = params;
+    probe = state->probe_function == (int)function && state->probe_count < YVEX_ROCM_PROBE_MAX;
+    if (probe)
+        probe = state->driver.hipEventRecord(state->probe_events[2u * state->probe_count],
+                                             state->stream) == hipSuccess;
     rc = yvex_rocm_status(&state->driver,
                           state->driver.hipModuleLaunchKernel(state->functions[function], grid_x,
                                                               grid_y, grid_z, block, 1u, 1u,
                                                               lds_bytes, state->stream, arguments,
                                                               NULL),
                           where, err);
+    if (probe && rc == YVEX_OK &&
+        state->driver.hipEventRecord(state->probe_events[2u * state->probe_count + 1u],
+                                     state->stream) == hipSuccess)
+        state->probe_count++;
     if (rc != YVEX_OK) capability_fail(backend, variant, YVEX_BACKEND_CAPABILITY_REASON_LAUNCH_FAILED);
     return rc;
 }

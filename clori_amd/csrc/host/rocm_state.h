@@ -23,6 +23,8 @@ typedef enum {
     YVEX_ROCM_FN_COUNT
 } yvex_rocm_function_id;
 
+#define YVEX_ROCM_PROBE_MAX 256u
+
 typedef enum {
     YVEX_ROCM_KERNEL_BUNDLE_ABSENT = 0,
     YVEX_ROCM_KERNEL_BUNDLE_ADMITTED,
@@ -36,6 +38,10 @@ typedef struct yvex_rocm_backend_state {
     hipStream_t stream;
     hipEvent_t timing_start, timing_stop;
     int timing_active;
+    /* per-kernel probe: event pairs around launches of one function */
+    hipEvent_t probe_events[2 * YVEX_ROCM_PROBE_MAX];
+    unsigned int probe_count;
+    int probe_function; /* -1: closed */
     hipModule_t modules[YVEX_ROCM_MODULE_MAX];
     unsigned int module_count;
     hipFunction_t functions[YVEX_ROCM_FN_COUNT];
@@ -68,6 +74,7 @@ int yvex_rocm_require_capability(yvex_backend *backend, yvex_backend_operation_v
                                  const char *where, yvex_error *err);
 unsigned int yvex_rocm_bundle_image_count(void);
 /* One kernel launch on the backend stream; params is the kernel's single argument block. */
+int yvex_rocm_function_find(const char *symbol);
 int yvex_rocm_launch(yvex_backend *backend, yvex_rocm_function_id function,
                      yvex_backend_operation_variant variant, unsigned int grid_x,
                      unsigned int grid_y, unsigned int grid_z, unsigned int block,

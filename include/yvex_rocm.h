@@ -439,6 +439,15 @@ int yvex_backend_rocm_completion_mode_set(yvex_backend *backend, yvex_rocm_compl
 int yvex_backend_rocm_timing_begin(yvex_backend *backend, yvex_error *err);
 int yvex_backend_rocm_timing_end(yvex_backend *backend, double *milliseconds, yvex_error *err);
 
+/* Per-kernel device time: while a probe is open, every launch of the named kernel on the
+ * backend's stream is bracketed by its own event pair (at most 256 launches; later ones
+ * are not measured).  end() synchronises and returns the measured launch count and the
+ * sum of their durations.  The name is the kernel symbol in the bundle. */
+int yvex_backend_rocm_kernel_probe_begin(yvex_backend *backend, const char *kernel,
+                                         yvex_error *err);
+int yvex_backend_rocm_kernel_probe_end(yvex_backend *backend, unsigned int *launches,
+                                       double *milliseconds, yvex_error *err);
+
 /* Kernel-bundle facts (cf. `inspect backend cuda`, src/backend/core.c:1824-1916). */
 typedef struct {
     int driver_loaded, device_ready, bundle_built, bundle_admitted;
