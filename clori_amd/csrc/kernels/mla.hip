@@ -8,9 +8,20 @@
 // dimension of 32x32x16 MFMA tiles.  Per 32-token tile staged in LDS:
 //     S^T[token][head] = C[token][:576] . Q[head][:576]      36 MFMAs, A = rows (LDS)
 //     online softmax per lane (= per head), exp2 with scale*log2e folded in
-//     O^T[dim][head]  += C^T[dim][token] . P^T[token][head]  32 MFMAs, A = transposed copy
-// The latent tile is kept twice in LDS: row-major for the score product and transposed
-// ([dim][token]) for the value product; both pitches are bank-conflict free.
+//     O^T[dim][head]  += C^T[dim][token] . P^T[token][head]  32 MFMAs, A = transposed read
+// The latent tile is kept once in LDS, row-major with 1152-byte rows and no padding; the
+// 16-byte chunk c of row r sits at chunk position c ^ x(r) with
+// x(r) = (((r >> 1) & 1) << 2) | ((r >> 2) & 3), which only permutes chunks inside
+// aligned groups of 8.  Rows are 128 bytes apart modulo the 256-byte bank span, so
+// this makes the row fetch of the first product (ds_read_b128, lane = token) and the
+// transposed fetch of the second (ds_read_b64_tr_b16, 4 tokens x 16 dims per 16 lanes)
+// both bank-conflict free.
+// Tiles are filled by buffer loads that write LDS directly: lane L of 1 KB load j of
+// wave w owns linear chunk (9w + j) * 64 + L of the tile and fetches the global chunk that
+// belongs there.  A tile never straddles a page (pages are multiples of 32 tokens), so
+// the page id is wave-uniform and the buffer descriptor is rebuilt per tile from the page
+// base; rows past the context read as zero through the descriptor's range check.
+// Four LDS buffers form a ring with three tiles in flight.
 // Unnormalised partials (max in log2 units, sum, accumulator) go to the workspace and
 // yvex_rocm_decode_merge performs the log-sum-exp merge.
 #include "mfma.h"
@@ -21,24 +32,33 @@ namespace {
 
 constexpr int kKeyDim = 576;
 constexpr int kValueDim = 512;
-constexpr int kTile = 32;                       // tokens per LDS tile
-constexpr int kRowPitch = kKeyDim * 2 + 16;     // 1168 B: ds_read_b128 rows hit distinct banks
-constexpr int kTPitch = kTile * 2 + 8;          // 72 B: ds_read_b64 rows hit distinct banks
-constexpr int kRowBytes = kTile * kRowPitch;    // 37376
-constexpr int kTBytes = kValueDim * kTPitch;    // 36864
-constexpr int kBufBytes = kRowBytes + kTBytes;  // 74240
+constexpr int kTile = 32;                          // tokens per LDS tile
+constexpr int kRowBytes = kKeyDim * 2;             // 1152
+constexpr int kRowChunks = kRowBytes / 16;         // 72
+constexpr int kTileBytes = kTile * kRowBytes;      // 36864
+constexpr int kBuffers = 4;
+constexpr int kLoadsPerWave = kTileBytes / 1024 / 4;  // 9
 constexpr int kHeadsPerWave = 32;
+constexpr float kLazyLog2 = 8.0f;
+
+typedef __attribute__((address_space(3))) void lds_void;
+typedef __attribute__((address_space(3))) short4v lds_short4;
+typedef short short8v __attribute__((ext_vector_type(8)));
 
 __device__ inline void flag(int32_t *status, int code) { atomicCAS(status, 0, code); }
 
+__device__ inline int swizzle(int r) { return (((r >> 1) & 1) << 2) | ((r >> 2) & 3); }
+
 }  // namespace
 
-// grid = (chunks, batch), block 256 (heads must be 128), LDS 2 * kBufBytes = 145 KB.
+// grid = (chunks, batch), block 256 (heads must be 128, pages a multiple of 32 tokens),
+// LDS 4 x 36 KB.
 extern "C" __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
 yvex_rocm_mla_decode_bf16(const yvex_rocm_mla_params p)
 {
-    __shared__ __attribute__((aligned(16))) unsigned char lds[2 * kBufBytes];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    __shared__ __attribute__((aligned(16))) unsigned char lds[kBuffers * kTileBytes];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n = lane & 31, g = lane >> 5;
     const uint32_t chunk = blockIdx.x, batch = blockIdx.y;
     const uint32_t ctx = (uint32_t)p.context[batch];
@@ -60,53 +80,63 @@ yvex_rocm_mla_decode_bf16(const yvex_rocm_mla_params p)
         for (int kk = 0; kk < 36; ++kk) q[kk] = as_bf16x8(load_b128(src + kk * 16));
     }
 
+    // ---- tile staging --------------------------------------------------------------
     const int32_t *table = p.page_table + (uint64_t)batch * p.table_stride;
-    // staging registers: 8 x 16 B of the latent part (2 groups of 4 tokens x 8 dims, to be
-    // transposed) + 1 x 16 B of the rope part
-    u32x4 lat[2][4], rope;
-    auto row_ptr = [&](uint32_t token) -> const uint16_t * {
-        token = min(token, t1 - 1u);
-        int32_t page = table[token / p.page_tokens];
-        if (page < 0 || (uint32_t)page >= p.pool_pages) {
-            flag(p.status, YVEX_ROCM_DEVICE_CONTRACT);
-            page = 0;
-        }
-        return p.pool + ((uint64_t)page * p.page_tokens + token % p.page_tokens) * kKeyDim;
-    };
-    // item = tid + 256*s covers (token group tg = item % 8, dim chunk dc = item / 8)
-    auto load_tile = [&](uint32_t tile) {
+    uint32_t stage_off[kLoadsPerWave];
+#pragma unroll
+    for (int j = 0; j < kLoadsPerWave; ++j) {
+        const int linear = (wave * kLoadsPerWave + j) * 64 + lane;
+        const int r = linear / kRowChunks, pos = linear % kRowChunks;
+        stage_off[j] = (uint32_t)(r * kRowBytes + ((pos ^ swizzle(r)) << 4));
+    }
+    // always issues kLoadsPerWave loads (with an empty range past the last tile) so that
+    // the outstanding-load count at the top of every iteration is the same
+    auto stage_tile = [&](uint32_t tile) {
         const uint32_t first = t0 + tile * kTile;
-#pragma unroll
-        for (int s = 0; s < 2; ++s) {
-            const int item = tid + 256 * s, tg = item & 7, dc = item >> 3;
-#pragma unroll
-            for (int r = 0; r < 4; ++r)
-                lat[s][r] = load_b128(row_ptr(first + tg * 4 + r) + dc * 8);
-        }
-        rope = load_b128(row_ptr(first + (tid >> 3)) + kValueDim + (tid & 7) * 8);
-    };
-    auto store_tile = [&](int buf) {
-        unsigned char *rows = lds + buf * kBufBytes;
-        unsigned char *tr = rows + kRowBytes;
-#pragma unroll
-        for (int s = 0; s < 2; ++s) {
-            const int item = tid + 256 * s, tg = item & 7, dc = item >> 3;
-#pragma unroll
-            for (int r = 0; r < 4; ++r)
-                *reinterpret_cast<u32x4 *>(rows + (tg * 4 + r) * kRowPitch + dc * 16) = lat[s][r];
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const int w = e >> 1;
-                const uint32_t sel = (e & 1) ? 0x07060302u : 0x05040100u;
-                u32x2 out;
-                out.x = __builtin_amdgcn_perm(lat[s][1][w], lat[s][0][w], sel);
-                out.y = __builtin_amdgcn_perm(lat[s][3][w], lat[s][2][w], sel);
-                *reinterpret_cast<u32x2 *>(tr + (dc * 8 + e) * kTPitch + tg * 8) = out;
+        uint32_t valid = 0u;
+        const uint16_t *base = p.pool;
+        if (tile < tiles) {
+            int32_t page = table[first / p.page_tokens];
+            if (page < 0 || (uint32_t)page >= p.pool_pages) {
+                if (lane == 0) flag(p.status, YVEX_ROCM_DEVICE_CONTRACT);
+                page = 0;
             }
+            valid = min((uint32_t)kTile, t1 - first);
+            base = p.pool + ((uint64_t)(uint32_t)page * p.page_tokens + first % p.page_tokens) * kKeyDim;
         }
-        *reinterpret_cast<u32x4 *>(rows + (tid >> 3) * kRowPitch + kValueDim * 2 + (tid & 7) * 16) =
-            rope;
+        const __amdgpu_buffer_rsrc_t rsrc =
+            __builtin_amdgcn_make_buffer_rsrc((void *)base, 0, valid * kRowBytes, 0x00027000);
+        unsigned char *dst = lds + (tile % kBuffers) * kTileBytes + wave * (kLoadsPerWave * 1024);
+#pragma unroll
+        for (int j = 0; j < kLoadsPerWave; ++j)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_void *)(dst + j * 1024), 16,
+                                                     stage_off[j], 0, 0, 0);
     };
+
+    // ---- operand addresses inside a tile ----------------------------------------------
+    // first product, k-step kk: row n, chunk 2kk + g; one address per kk % 4, the rest is
+    // an immediate (kk / 4) * 128
+    uint32_t k_addr[4];
+#pragma unroll
+    for (int k4 = 0; k4 < 4; ++k4)
+        k_addr[k4] = (uint32_t)(n * kRowBytes + (((2 * k4 + g) ^ swizzle(n)) << 4));
+    // second product, (db, u, h): 16-lane group b = lane / 16 covers dims 16 * (b & 1) of
+    // the 32-dim block and token half g = b / 2; lane a = lane % 16 addresses token row
+    // 16u + 8h + 4g + a / 4 and dims db*32 + 16*(b&1) + 4*(a%4) .. +3.  The swizzle flips
+    // the chunk's bit 2 by (a >> 3) & 1: one address per (db parity, h), the rest is an
+    // immediate (db - parity) * 64 + u * 16 rows.
+    uint32_t v_addr[2][2];
+    {
+        const int a = lane & 15, b1 = (lane >> 4) & 1;
+#pragma unroll
+        for (int par = 0; par < 2; ++par)
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const int r = 8 * h + 4 * g + (a >> 2);
+                const int chunk16 = (par * 4 + 2 * b1 + ((a >> 1) & 1)) ^ swizzle(r);
+                v_addr[par][h] = (uint32_t)(r * kRowBytes + (chunk16 << 4) + 8 * (a & 1));
+            }
+    }
 
     floatx16 o[16];
 #pragma unroll
@@ -115,74 +145,98 @@ yvex_rocm_mla_decode_bf16(const yvex_rocm_mla_params p)
         for (int i = 0; i < 16; ++i) o[db][i] = 0.f;
     float m_run = -INFINITY, l_run = 0.f;
 
-    load_tile(0u);
+    stage_tile(0u);
+    stage_tile(1u);
+    stage_tile(2u);
     for (uint32_t t = 0; t < tiles; ++t) {
-        const int buf = (int)(t & 1u);
-        store_tile(buf);
+        // two younger tiles stay in flight: vmcnt(2 * kLoadsPerWave), then everyone's part
+        __builtin_amdgcn_s_waitcnt(0x4f72);
         __syncthreads();
-        if (t + 1u < tiles) load_tile(t + 1u);
-        const unsigned char *rows = lds + buf * kBufBytes;
-        const unsigned char *tr = rows + kRowBytes;
+        stage_tile(t + 3u);
+        const unsigned char *tile = lds + (t % kBuffers) * kTileBytes;
         const uint32_t key0 = t0 + t * kTile;
 
+        // ---- S^T = C . Q^T ---------------------------------------------------------
         floatx16 s;
 #pragma unroll
         for (int i = 0; i < 16; ++i) s[i] = 0.f;
 #pragma unroll
         for (int kk = 0; kk < 36; ++kk) {
             const bf16x8 a = as_bf16x8(
-                *reinterpret_cast<const u32x4 *>(rows + n * kRowPitch + kk * 32 + g * 16));
+                *reinterpret_cast<const u32x4 *>(tile + k_addr[kk & 3] + (kk >> 2) * 128));
             s = mfma_32x32x16(a, q[kk], s);
         }
-        const bool tail = key0 + kTile > t1;
+        __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);
+#pragma unroll
+        for (int i = 0; i < 30; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, 6, 0);
+
+        // ---- online softmax per lane (= per head) --------------------------------------
+        if (key0 + kTile > t1) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i)
+                if (key0 + (i >> 2) * 8 + g * 4 + (i & 3) >= t1) s[i] = -INFINITY;
+        }
         float mloc = -INFINITY;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            float x = s[i] * p.scale_log2;
-            if (tail && key0 + (i >> 2) * 8 + g * 4 + (i & 3) >= t1) x = -INFINITY;
-            s[i] = x;
-            mloc = fmaxf(mloc, x);
-        }
-        mloc = fmaxf(mloc, xor_lanes(mloc, 32));
-        const float m_new = fmaxf(m_run, mloc);
-        if (__builtin_amdgcn_ballot_w64(m_new > m_run) != 0ull) {
-            const float alpha = fast_exp2(m_run - m_new);
+        for (int i = 0; i < 16; ++i) mloc = fmaxf(mloc, s[i]);
+        mloc *= p.scale_log2;
+        if (__builtin_amdgcn_ballot_w64(mloc > m_run + kLazyLog2) != 0ull) {
+            // both token halves of a head must agree on the reference maximum
+            const float m_new = fmaxf(m_run, fmaxf(mloc, xor_lanes(mloc, 32)));
+            const float alpha = m_new == -INFINITY ? 1.0f : fast_exp2(m_run - m_new);
             l_run *= alpha;
+            // one block at a time through the VALU; the accumulators live in AGPRs
 #pragma unroll
-            for (int db = 0; db < 16; ++db) o[db] *= alpha;
+            for (int db = 0; db < 16; ++db) {
+                asm volatile("" : "+a"(o[db]));
+                o[db] *= alpha;
+                asm volatile("" : "+a"(o[db]));
+            }
             m_run = m_new;
         }
+        const float neg_m = m_run == -INFINITY ? 0.f : -m_run;
         uint32_t pk[8];
         float lsum = 0.f;
 #pragma unroll
         for (int i = 0; i < 16; i += 2) {
-            const float p0 = fast_exp2(s[i] - m_run), p1 = fast_exp2(s[i + 1] - m_run);
+            const float p0 = fast_exp2(__builtin_fmaf(s[i], p.scale_log2, neg_m));
+            const float p1 = fast_exp2(__builtin_fmaf(s[i + 1], p.scale_log2, neg_m));
             lsum += p0 + p1;
             pk[i >> 1] = pack_bf16x2(p0, p1);
         }
         l_run += lsum;
+
+        // ---- O^T += C^T . P^T ----------------------------------------------------------
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
             const u32x4 w = {pk[u * 4 + 0], pk[u * 4 + 1], pk[u * 4 + 2], pk[u * 4 + 3]};
             const bf16x8 pb = as_bf16x8(w);
 #pragma unroll
             for (int db = 0; db < 16; ++db) {
-                const unsigned char *src = tr + (db * 32 + n) * kTPitch + (u * 16 + g * 4) * 2;
-                const u32x2 lo = *reinterpret_cast<const u32x2 *>(src);
-                const u32x2 hi = *reinterpret_cast<const u32x2 *>(src + 16);
-                u32x4 a;
-                a.x = lo.x;
-                a.y = lo.y;
-                a.z = hi.x;
-                a.w = hi.y;
-                if (tail) {
-                    // tokens past the context alias the last valid row (finite unless the
-                    // data itself is not), their weights are exact zeros
-                }
-                o[db] = mfma_32x32x16(as_bf16x8(a), pb, o[db]);
+                const int imm = (db & ~1) * 64 + u * 16 * kRowBytes;
+                const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    (lds_short4 *)(tile + v_addr[db & 1][0] + imm));
+                const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    (lds_short4 *)(tile + v_addr[db & 1][1] + imm));
+                const short8v av = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                o[db] = mfma_32x32x16(__builtin_bit_cast(bf16x8, av), pb, o[db]);
             }
         }
+        // three transposed operand pairs in flight ahead of the MFMAs that consume them
+        __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);
+#pragma unroll
+        for (int i = 0; i < 29; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, 3, 0);
     }
+    // drain the loads that were issued past the last tile before the workgroup ends
+    __builtin_amdgcn_s_waitcnt(0x0f70);
 
     float l = l_run;
     l += xor_lanes(l, 32);
