@@ -610,6 +610,8 @@ static unsigned int mla_chunk_tokens(const yvex_rocm_mla_decode_requirement *r)
     unsigned long long chunk = (r->max_context_tokens + per_batch - 1ull) / per_batch;
     if (forced && atoi(forced) >= ROCM_MLA_PAGE_TOKENS) chunk = (unsigned long long)atoi(forced);
     chunk = align_up(chunk, ROCM_MLA_PAGE_TOKENS);
+    if (chunk > (unsigned long long)YVEX_ROCM_MLA_MAX_CHUNK_PAGES * ROCM_MLA_PAGE_TOKENS)
+        chunk = (unsigned long long)YVEX_ROCM_MLA_MAX_CHUNK_PAGES * ROCM_MLA_PAGE_TOKENS;
     return (unsigned int)chunk;
 }
 

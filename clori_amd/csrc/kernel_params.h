@@ -94,7 +94,9 @@ typedef struct {
     float reserved_f;
 } yvex_rocm_prefill_params;
 
-/* Absorbed-latent MLA decode, split over the context. */
+/* Absorbed-latent MLA decode, split over the context.  A chunk spans at most
+ * YVEX_ROCM_MLA_MAX_CHUNK_PAGES pages (the kernel keeps their ids in LDS). */
+#define YVEX_ROCM_MLA_MAX_CHUNK_PAGES 256
 typedef struct {
     const uint16_t *q;      /* [batch][heads][key_dim] */
     const uint16_t *pool;   /* [pool_pages][page_tokens][key_dim] */

@@ -21,7 +21,8 @@
 // belongs there.  A tile never straddles a page (pages are multiples of 32 tokens), so
 // the page id is wave-uniform and the buffer descriptor is rebuilt per tile from the page
 // base; rows past the context read as zero through the descriptor's range check.
-// Four LDS buffers form a ring with three tiles in flight.
+// Four LDS buffers form a ring with three tiles in flight.  The page ids of the chunk are
+// copied to LDS first, so staging never waits on a dependent global load.
 // Unnormalised partials (max in log2 units, sum, accumulator) go to the workspace and
 // yvex_rocm_decode_merge performs the log-sum-exp merge.
 #include "mfma.h"
@@ -40,6 +41,7 @@ constexpr int kBuffers = 4;
 constexpr int kLoadsPerWave = kTileBytes / 1024 / 4;  // 9
 constexpr int kHeadsPerWave = 32;
 constexpr float kLazyLog2 = 8.0f;
+constexpr int kMaxChunkPages = YVEX_ROCM_MLA_MAX_CHUNK_PAGES;  // page ids of the chunk, kept in LDS
 
 typedef __attribute__((address_space(3))) void lds_void;
 typedef __attribute__((address_space(3))) short4v lds_short4;
@@ -57,6 +59,7 @@ extern "C" __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_pe
 yvex_rocm_mla_decode_bf16(const yvex_rocm_mla_params p)
 {
     __shared__ __attribute__((aligned(16))) unsigned char lds[kBuffers * kTileBytes];
+    __shared__ int32_t chunk_pages[kMaxChunkPages];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n = lane & 31, g = lane >> 5;
@@ -81,7 +84,23 @@ yvex_rocm_mla_decode_bf16(const yvex_rocm_mla_params p)
     }
 
     // ---- tile staging --------------------------------------------------------------
+    // the chunk's page ids are fetched once, so staging a tile never waits on global memory
     const int32_t *table = p.page_table + (uint64_t)batch * p.table_stride;
+    const uint32_t first_page = t0 / p.page_tokens;
+    const uint32_t chunk_page_count = (t1 - 1u) / p.page_tokens - first_page + 1u;
+    if (chunk_page_count > (uint32_t)kMaxChunkPages) {
+        if (tid == 0) flag(p.status, YVEX_ROCM_DEVICE_CONTRACT);
+        return;
+    }
+    for (uint32_t i = tid; i < chunk_page_count; i += 256u) {
+        int32_t page = table[first_page + i];
+        if (page < 0 || (uint32_t)page >= p.pool_pages) {
+            flag(p.status, YVEX_ROCM_DEVICE_CONTRACT);
+            page = 0;
+        }
+        chunk_pages[i] = page;
+    }
+    __syncthreads();
     uint32_t stage_off[kLoadsPerWave];
 #pragma unroll
     for (int j = 0; j < kLoadsPerWave; ++j) {
@@ -96,13 +115,10 @@ yvex_rocm_mla_decode_bf16(const yvex_rocm_mla_params p)
         uint32_t valid = 0u;
         const uint16_t *base = p.pool;
         if (tile < tiles) {
-            int32_t page = table[first / p.page_tokens];
-            if (page < 0 || (uint32_t)page >= p.pool_pages) {
-                if (lane == 0) flag(p.status, YVEX_ROCM_DEVICE_CONTRACT);
-                page = 0;
-            }
+            const uint32_t page = (uint32_t)__builtin_amdgcn_readfirstlane(
+                chunk_pages[first / p.page_tokens - first_page]);
             valid = min((uint32_t)kTile, t1 - first);
-            base = p.pool + ((uint64_t)(uint32_t)page * p.page_tokens + first % p.page_tokens) * kKeyDim;
+            base = p.pool + ((uint64_t)page * p.page_tokens + first % p.page_tokens) * kKeyDim;
         }
         const __amdgpu_buffer_rsrc_t rsrc =
             __builtin_amdgcn_make_buffer_rsrc((void *)base, 0, valid * kRowBytes, 0x00027000);
@@ -148,7 +164,11 @@ yvex_rocm_mla_decode_bf16(const yvex_rocm_mla_params p)
     stage_tile(0u);
     stage_tile(1u);
     stage_tile(2u);
+#ifdef MLA_PROBE_TILES
+    for (uint32_t t = 0; t < MLA_PROBE_TILES; ++t) {
+#else
     for (uint32_t t = 0; t < tiles; ++t) {
+#endif
         // two younger tiles stay in flight: vmcnt(2 * kLoadsPerWave), then everyone's part
         __builtin_amdgcn_s_waitcnt(0x4f72);
         __syncthreads();
@@ -238,6 +258,9 @@ yvex_rocm_mla_decode_bf16(const yvex_rocm_mla_params p)
     // drain the loads that were issued past the last tile before the workgroup ends
     __builtin_amdgcn_s_waitcnt(0x0f70);
 
+#ifdef MLA_PROBE_SKIP_STORE
+    if (l_run != 12345.0f) return;
+#endif
     float l = l_run;
     l += xor_lanes(l, 32);
     const uint64_t slot = ((uint64_t)batch * p.max_chunks + chunk) * p.heads + head;
