@@ -106,12 +106,12 @@ static unsigned int decode_wave_count(unsigned long long sessions, unsigned long
 }
 
 static int decode_workspace_bytes(unsigned long long slots, unsigned long long heads,
-                                  unsigned long long head_dim, unsigned long long *acc_bytes,
-                                  unsigned long long *total)
+                                  unsigned long long head_dim, unsigned long long element_bytes,
+                                  unsigned long long *acc_bytes, unsigned long long *total)
 {
     unsigned long long rows, acc, ml;
     if (!yvex_core_u64_mul(slots, heads, &rows) ||
-        !yvex_core_u64_mul(rows, head_dim * sizeof(float), &acc) ||
+        !yvex_core_u64_mul(rows, head_dim * element_bytes, &acc) ||
         !yvex_core_u64_mul(rows, 2ull * sizeof(float), &ml))
         return 0;
     acc = align_up(acc, ROCM_WORK_ALIGNMENT);
@@ -128,7 +128,7 @@ static int balanced_workspace_bytes(unsigned long long waves, unsigned long long
                                     unsigned long long *total)
 {
     unsigned long long parts = 0ull, offsets;
-    if (!decode_workspace_bytes(2ull * waves, group, head_dim, acc_bytes, &parts)) return 0;
+    if (!decode_workspace_bytes(2ull * waves, group, head_dim, sizeof(float), acc_bytes, &parts)) return 0;
     offsets = align_up((sessions + 1ull) * sizeof(uint32_t), ROCM_WORK_ALIGNMENT);
     *ml_bytes = parts - *acc_bytes;
     return yvex_core_u64_add(parts, offsets, total);
@@ -627,7 +627,8 @@ static int rocm_mla_decode_workspace_required(const yvex_rocm_mla_decode_require
     if (!bytes) return refuse(err, YVEX_ERR_INVALID_ARG, where, "workspace byte output is required");
     chunk = mla_chunk_tokens(r);
     max_chunks = (r->max_context_tokens + chunk - 1ull) / chunk;
-    if (!decode_workspace_bytes(r->batch * max_chunks, r->heads, r->value_dimension, &acc, &total))
+    if (!decode_workspace_bytes(r->batch * max_chunks, r->heads, r->value_dimension,
+                                sizeof(uint16_t), &acc, &total))
         return refuse(err, YVEX_ERR_BOUNDS, where, "MLA workspace geometry overflowed");
     *bytes = total;
     yvex_error_clear(err);
@@ -673,8 +674,8 @@ static int rocm_mla_decode_execute(yvex_backend *backend,
     chunk = mla_chunk_tokens(r);
     max_chunks = (r->max_context_tokens + chunk - 1ull) / chunk;
     if (max_chunks > 0x7fffffffull ||
-        !decode_workspace_bytes(r->batch * max_chunks, r->heads, r->value_dimension, &acc_bytes,
-                                &total))
+        !decode_workspace_bytes(r->batch * max_chunks, r->heads, r->value_dimension,
+                                sizeof(uint16_t), &acc_bytes, &total))
         return refuse(err, YVEX_ERR_BOUNDS, where, "MLA decode geometry exceeds admitted range");
     backend_workspace_reset(backend);
     rc = yvex_rocm_temporary_acquire(backend, total, &work, &owned, where, err);
@@ -684,7 +685,7 @@ static int rocm_mla_decode_execute(yvex_backend *backend,
     kp.pool = (const uint16_t *)request->latent_pages->data;
     kp.page_table = (const int32_t *)request->page_table->data;
     kp.context = (const int32_t *)request->context_tokens->data;
-    kp.part_acc = (float *)work;
+    kp.part_acc = (uint16_t *)work;
     kp.part_ml = (float *)((unsigned char *)work + acc_bytes);
     kp.status = state->device_status;
     kp.batch = (uint32_t)r->batch;

@@ -586,7 +586,7 @@ yvex_rocm_decode_merge(const yvex_rocm_decode_merge_params p)
         const uint64_t slot = base + (uint64_t)c * p.query_heads;
         const float w = fast_exp2(p.part_ml[slot * 2] - top);
         total += w * p.part_ml[slot * 2 + 1];
-        acc += w * p.part_acc[slot * p.head_dim + d];
+        acc += w * bf16_to_f32(p.part_acc[slot * p.head_dim + d]);
     }
     const float o = acc / total;
     if (!isfinite(o)) flag(p.status, YVEX_ROCM_DEVICE_NUMERIC);

@@ -23,7 +23,7 @@
 // base; rows past the context read as zero through the descriptor's range check.
 // Four LDS buffers form a ring with three tiles in flight.  The page ids of the chunk are
 // copied to LDS first, so staging never waits on a dependent global load.
-// Unnormalised partials (max in log2 units, sum, accumulator) go to the workspace and
+// Unnormalised partials (max in log2 units, sum, bf16 accumulator) go to the workspace and
 // yvex_rocm_decode_merge performs the log-sum-exp merge.
 #include "mfma.h"
 
@@ -264,15 +264,32 @@ yvex_rocm_mla_decode_bf16(const yvex_rocm_mla_params p)
     float l = l_run;
     l += xor_lanes(l, 32);
     const uint64_t slot = ((uint64_t)batch * p.max_chunks + chunk) * p.heads + head;
-    float *acc = p.part_acc + slot * kValueDim;
+    // The accumulators are lane = head, registers = dims; through LDS they become one
+    // contiguous 1 KB bf16 row per head, written by one 16-byte store per lane.
+    constexpr int kOutPitch = kValueDim * 2 + 16;  // 1040 B, keeps 16-byte alignment
+    static_assert(4 * kHeadsPerWave * kOutPitch <= kBuffers * kTileBytes, "epilogue fits the tiles");
+    __syncthreads();  // every wave is done with the tile buffers
+    unsigned char *rows = lds + wave * (kHeadsPerWave * kOutPitch);
 #pragma unroll
     for (int db = 0; db < 16; ++db)
 #pragma unroll
         for (int grp = 0; grp < 4; ++grp) {
-            floatx4 v = {o[db][grp * 4 + 0], o[db][grp * 4 + 1], o[db][grp * 4 + 2],
-                         o[db][grp * 4 + 3]};
-            *reinterpret_cast<floatx4 *>(acc + db * 32 + grp * 8 + g * 4) = v;
+            u32x2 v;
+            v.x = pack_bf16x2(o[db][grp * 4 + 0], o[db][grp * 4 + 1]);
+            v.y = pack_bf16x2(o[db][grp * 4 + 2], o[db][grp * 4 + 3]);
+            *reinterpret_cast<u32x2 *>(rows + n * kOutPitch + (db * 32 + grp * 8 + g * 4) * 2) = v;
         }
+    // only this wave reads what it wrote: no workgroup barrier needed
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+    {
+        const uint64_t slot0 = ((uint64_t)batch * p.max_chunks + chunk) * p.heads + wave * kHeadsPerWave;
+        uint16_t *dst = p.part_acc + slot0 * kValueDim + lane * 8;
+#pragma unroll 8
+        for (int hh = 0; hh < kHeadsPerWave; ++hh) {
+            const u32x4 v = *reinterpret_cast<const u32x4 *>(rows + hh * kOutPitch + lane * 16);
+            *reinterpret_cast<u32x4 *>(dst + (uint64_t)hh * kValueDim) = v;
+        }
+    }
     if (g == 0) {
         p.part_ml[slot * 2 + 0] = m_run;
         p.part_ml[slot * 2 + 1] = l;
