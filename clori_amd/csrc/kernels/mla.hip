@@ -41,15 +41,32 @@ constexpr int kBuffers = 4;
 constexpr int kLoadsPerWave = kTileBytes / 1024 / 4;  // 9
 constexpr int kHeadsPerWave = 32;
 constexpr float kLazyLog2 = 8.0f;
+constexpr int kQkDepth = 4;  // operand fetches in flight ahead of the first product
 constexpr int kMaxChunkPages = YVEX_ROCM_MLA_MAX_CHUNK_PAGES;  // page ids of the chunk, kept in LDS
 
 typedef __attribute__((address_space(3))) void lds_void;
 typedef __attribute__((address_space(3))) short4v lds_short4;
 typedef short short8v __attribute__((ext_vector_type(8)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
 
 __device__ inline void flag(int32_t *status, int code) { atomicCAS(status, 0, code); }
 
 __device__ inline int swizzle(int r) { return (((r >> 1) & 1) << 2) | ((r >> 2) & 3); }
+
+#ifdef MLA_PROBE_CLOCK
+// timing probe: phase cycle counts of wave 0 of workgroup (0, 0), summed over its tiles
+__device__ unsigned long long yvex_mla_clock[8];
+#define MLA_STAMP(slot)                                                        \
+    do {                                                                       \
+        __builtin_amdgcn_sched_barrier(0);                                     \
+        const unsigned long long now_ = __builtin_readcyclecounter();          \
+        clock_acc[slot] += now_ - clock_prev;                                  \
+        clock_prev = now_;                                                     \
+        __builtin_amdgcn_sched_barrier(0);                                     \
+    } while (0)
+#else
+#define MLA_STAMP(slot) do { } while (0)
+#endif
 
 }  // namespace
 
@@ -101,6 +118,8 @@ yvex_rocm_mla_decode_bf16(const yvex_rocm_mla_params p)
         chunk_pages[i] = page;
     }
     __syncthreads();
+    static_assert(kLoadsPerWave == 9, "the staging block issues nine loads");
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)lds;
     uint32_t stage_off[kLoadsPerWave];
 #pragma unroll
     for (int j = 0; j < kLoadsPerWave; ++j) {
@@ -120,13 +139,33 @@ yvex_rocm_mla_decode_bf16(const yvex_rocm_mla_params p)
             valid = min((uint32_t)kTile, t1 - first);
             base = p.pool + ((uint64_t)page * p.page_tokens + first % p.page_tokens) * kKeyDim;
         }
-        const __amdgpu_buffer_rsrc_t rsrc =
-            __builtin_amdgcn_make_buffer_rsrc((void *)base, 0, valid * kRowBytes, 0x00027000);
-        unsigned char *dst = lds + (tile % kBuffers) * kTileBytes + wave * (kLoadsPerWave * 1024);
-#pragma unroll
-        for (int j = 0; j < kLoadsPerWave; ++j)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_void *)(dst + j * 1024), 16,
-                                                     stage_off[j], 0, 0, 0);
+        // raw buffer descriptor: base, stride 0, byte range, untyped dword format
+        const uint64_t address = (uint64_t)base;
+        i32x4 rsrc;
+        rsrc.x = __builtin_amdgcn_readfirstlane((int)(uint32_t)address);
+        rsrc.y = __builtin_amdgcn_readfirstlane((int)(uint32_t)(address >> 32) & 0xffff);
+        rsrc.z = __builtin_amdgcn_readfirstlane((int)(valid * kRowBytes));
+        rsrc.w = 0x00027000;
+        const uint32_t dst = __builtin_amdgcn_readfirstlane(
+            lds_base + (tile % kBuffers) * kTileBytes + wave * (kLoadsPerWave * 1024));
+        // Issued as one opaque block: the compiler would otherwise make every later LDS
+        // read wait for these loads (it cannot see that the ring buffers do not alias),
+        // which serialises the ring.  M0 carries the LDS destination of each load.
+        asm volatile(
+            "s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %2, %1, 0 offen lds\n\t"
+            "s_add_u32 m0, m0, 0x400\n\ts_nop 0\n\tbuffer_load_dwordx4 %3, %1, 0 offen lds\n\t"
+            "s_add_u32 m0, m0, 0x400\n\ts_nop 0\n\tbuffer_load_dwordx4 %4, %1, 0 offen lds\n\t"
+            "s_add_u32 m0, m0, 0x400\n\ts_nop 0\n\tbuffer_load_dwordx4 %5, %1, 0 offen lds\n\t"
+            "s_add_u32 m0, m0, 0x400\n\ts_nop 0\n\tbuffer_load_dwordx4 %6, %1, 0 offen lds\n\t"
+            "s_add_u32 m0, m0, 0x400\n\ts_nop 0\n\tbuffer_load_dwordx4 %7, %1, 0 offen lds\n\t"
+            "s_add_u32 m0, m0, 0x400\n\ts_nop 0\n\tbuffer_load_dwordx4 %8, %1, 0 offen lds\n\t"
+            "s_add_u32 m0, m0, 0x400\n\ts_nop 0\n\tbuffer_load_dwordx4 %9, %1, 0 offen lds\n\t"
+            "s_add_u32 m0, m0, 0x400\n\ts_nop 0\n\tbuffer_load_dwordx4 %10, %1, 0 offen lds"
+            :
+            : "s"(dst), "s"(rsrc), "v"(stage_off[0]), "v"(stage_off[1]), "v"(stage_off[2]),
+              "v"(stage_off[3]), "v"(stage_off[4]), "v"(stage_off[5]), "v"(stage_off[6]),
+              "v"(stage_off[7]), "v"(stage_off[8])
+            : "memory", "scc");
     };
 
     // ---- operand addresses inside a tile ----------------------------------------------
@@ -161,9 +200,14 @@ yvex_rocm_mla_decode_bf16(const yvex_rocm_mla_params p)
         for (int i = 0; i < 16; ++i) o[db][i] = 0.f;
     float m_run = -INFINITY, l_run = 0.f;
 
+#ifdef MLA_PROBE_CLOCK
+    unsigned long long clock_acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    unsigned long long clock_prev = __builtin_readcyclecounter();
+#endif
     stage_tile(0u);
     stage_tile(1u);
     stage_tile(2u);
+    MLA_STAMP(0);
 #ifdef MLA_PROBE_TILES
     for (uint32_t t = 0; t < MLA_PROBE_TILES; ++t) {
 #else
@@ -171,29 +215,44 @@ yvex_rocm_mla_decode_bf16(const yvex_rocm_mla_params p)
 #endif
         // two younger tiles stay in flight: vmcnt(2 * kLoadsPerWave), then everyone's part
         __builtin_amdgcn_s_waitcnt(0x4f72);
+        MLA_STAMP(1);
         __syncthreads();
+        MLA_STAMP(2);
+#ifndef MLA_PROBE_SKIP_STAGE
         stage_tile(t + 3u);
+#else
+        stage_tile(tiles + 3u);
+#endif
+        MLA_STAMP(3);
         const unsigned char *tile = lds + (t % kBuffers) * kTileBytes;
         const uint32_t key0 = t0 + t * kTile;
 
         // ---- S^T = C . Q^T ---------------------------------------------------------
+        // operand fetches run kQkDepth k-steps ahead of the MFMAs; the order is pinned
+        // with scheduling barriers because the register budget leaves the scheduler no
+        // room to do it on its own
         floatx16 s;
 #pragma unroll
         for (int i = 0; i < 16; ++i) s[i] = 0.f;
+#ifndef MLA_PROBE_SKIP_QK
+        {
+            u32x4 frag[kQkDepth];
 #pragma unroll
-        for (int kk = 0; kk < 36; ++kk) {
-            const bf16x8 a = as_bf16x8(
-                *reinterpret_cast<const u32x4 *>(tile + k_addr[kk & 3] + (kk >> 2) * 128));
-            s = mfma_32x32x16(a, q[kk], s);
-        }
-        __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);
+            for (int kk = 0; kk < kQkDepth; ++kk)
+                frag[kk] = *reinterpret_cast<const u32x4 *>(tile + k_addr[kk & 3] + (kk >> 2) * 128);
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int i = 0; i < 30; ++i) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            for (int kk = 0; kk < 36; ++kk) {
+                s = mfma_32x32x16(as_bf16x8(frag[kk % kQkDepth]), q[kk], s);
+                if (kk + kQkDepth < 36)
+                    frag[kk % kQkDepth] = *reinterpret_cast<const u32x4 *>(
+                        tile + k_addr[(kk + kQkDepth) & 3] + ((kk + kQkDepth) >> 2) * 128);
+                __builtin_amdgcn_sched_barrier(0);
+            }
         }
-        __builtin_amdgcn_sched_group_barrier(0x008, 6, 0);
+#endif
 
+        MLA_STAMP(4);
         // ---- online softmax per lane (= per head) --------------------------------------
         if (key0 + kTile > t1) {
 #pragma unroll
@@ -230,7 +289,9 @@ yvex_rocm_mla_decode_bf16(const yvex_rocm_mla_params p)
         }
         l_run += lsum;
 
+        MLA_STAMP(5);
         // ---- O^T += C^T . P^T ----------------------------------------------------------
+#ifndef MLA_PROBE_SKIP_PV
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
             const u32x4 w = {pk[u * 4 + 0], pk[u * 4 + 1], pk[u * 4 + 2], pk[u * 4 + 3]};
@@ -254,12 +315,20 @@ yvex_rocm_mla_decode_bf16(const yvex_rocm_mla_params p)
             __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
         }
         __builtin_amdgcn_sched_group_barrier(0x008, 3, 0);
+#else
+        o[0][0] += __builtin_bit_cast(float, pk[0] ^ pk[3] ^ pk[5]);
+#endif
+        MLA_STAMP(6);
     }
     // drain the loads that were issued past the last tile before the workgroup ends
     __builtin_amdgcn_s_waitcnt(0x0f70);
 
 #ifdef MLA_PROBE_SKIP_STORE
     if (l_run != 12345.0f) return;
+#endif
+#ifdef MLA_PROBE_CLOCK
+    if (blockIdx.x == 0 && blockIdx.y == 0 && tid == 0)
+        for (int i = 0; i < 8; ++i) yvex_mla_clock[i] = clock_acc[i];
 #endif
     float l = l_run;
     l += xor_lanes(l, 32);
