@@ -21,11 +21,13 @@
 // belongs there.  A tile never straddles a page (pages are multiples of 32 tokens), so
 // the page id is wave-uniform and the buffer descriptor is rebuilt per tile from the page
 // base; rows past the context read as zero through the descriptor's range check.
-// Four LDS buffers form a ring with three tiles in flight.  The page ids of the chunk are
+// Four LDS buffers form a ring: two tiles being read, two in flight.  The page ids of the chunk are
 // copied to LDS first, so staging never waits on a dependent global load.
 // Unnormalised partials (max in log2 units, sum, bf16 accumulator) go to the workspace and
 // yvex_rocm_decode_merge performs the log-sum-exp merge.
 #include "mfma.h"
+
+#include <type_traits>
 
 #include "../kernel_params.h"
 
@@ -193,67 +195,63 @@ yvex_rocm_mla_decode_bf16(const yvex_rocm_mla_params p)
             }
     }
 
+    // one staging load, for spreading a tile's nine loads over the first product
+    auto stage_one = [&](uint32_t dst, i32x4 rsrc, uint32_t offset) {
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %2, %1, 0 offen lds"
+                     :
+                     : "s"(dst), "s"(rsrc), "v"(offset)
+                     : "memory");
+    };
+    auto stage_target = [&](uint32_t tile, uint32_t &dst, i32x4 &rsrc) {
+        const uint32_t first = t0 + tile * kTile;
+        uint32_t valid = 0u;
+        const uint16_t *base = p.pool;
+        if (tile < tiles) {
+            const uint32_t page = (uint32_t)__builtin_amdgcn_readfirstlane(
+                chunk_pages[first / p.page_tokens - first_page]);
+            valid = min((uint32_t)kTile, t1 - first);
+            base = p.pool + ((uint64_t)page * p.page_tokens + first % p.page_tokens) * kKeyDim;
+        }
+        const uint64_t address = (uint64_t)base;
+        rsrc.x = __builtin_amdgcn_readfirstlane((int)(uint32_t)address);
+        rsrc.y = __builtin_amdgcn_readfirstlane((int)(uint32_t)(address >> 32) & 0xffff);
+        rsrc.z = __builtin_amdgcn_readfirstlane((int)(valid * kRowBytes));
+        rsrc.w = 0x00027000;
+        dst = __builtin_amdgcn_readfirstlane(lds_base + (tile % kBuffers) * kTileBytes +
+                                             wave * (kLoadsPerWave * 1024));
+    };
+
     floatx16 o[16];
 #pragma unroll
     for (int db = 0; db < 16; ++db)
 #pragma unroll
         for (int i = 0; i < 16; ++i) o[db][i] = 0.f;
-    float m_run = -INFINITY, l_run = 0.f;
+    float m_run = -INFINITY, neg_m = 0.f, l_run = 0.f;
 
-#ifdef MLA_PROBE_CLOCK
-    unsigned long long clock_acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-    unsigned long long clock_prev = __builtin_readcyclecounter();
-#endif
-    stage_tile(0u);
-    stage_tile(1u);
-    stage_tile(2u);
-    MLA_STAMP(0);
-#ifdef MLA_PROBE_TILES
-    for (uint32_t t = 0; t < MLA_PROBE_TILES; ++t) {
-#else
-    for (uint32_t t = 0; t < tiles; ++t) {
-#endif
-        // two younger tiles stay in flight: vmcnt(2 * kLoadsPerWave), then everyone's part
-        __builtin_amdgcn_s_waitcnt(0x4f72);
-        MLA_STAMP(1);
-        __syncthreads();
-        MLA_STAMP(2);
-#ifndef MLA_PROBE_SKIP_STAGE
-        stage_tile(t + 3u);
-#else
-        stage_tile(tiles + 3u);
-#endif
-        MLA_STAMP(3);
-        const unsigned char *tile = lds + (t % kBuffers) * kTileBytes;
-        const uint32_t key0 = t0 + t * kTile;
-
-        // ---- S^T = C . Q^T ---------------------------------------------------------
-        // operand fetches run kQkDepth k-steps ahead of the MFMAs; the order is pinned
-        // with scheduling barriers because the register budget leaves the scheduler no
-        // room to do it on its own
-        floatx16 s;
+    // S^T of one tile; `extra(kk)` is work placed behind MFMA kk (operand fetches run
+    // kQkDepth k-steps ahead; the order is pinned with scheduling barriers because the
+    // register budget leaves the scheduler no room to do it on its own)
+    auto score = [&](const unsigned char *tile, floatx16 &s, auto extra) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) s[i] = 0.f;
-#ifndef MLA_PROBE_SKIP_QK
-        {
-            u32x4 frag[kQkDepth];
+        u32x4 frag[kQkDepth];
 #pragma unroll
-            for (int kk = 0; kk < kQkDepth; ++kk)
-                frag[kk] = *reinterpret_cast<const u32x4 *>(tile + k_addr[kk & 3] + (kk >> 2) * 128);
+        for (int kk = 0; kk < kQkDepth; ++kk)
+            frag[kk] = *reinterpret_cast<const u32x4 *>(tile + k_addr[kk & 3] + (kk >> 2) * 128);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int kk = 0; kk < 36; ++kk) {
+            s = mfma_32x32x16(as_bf16x8(frag[kk % kQkDepth]), q[kk], s);
+            if (kk + kQkDepth < 36)
+                frag[kk % kQkDepth] = *reinterpret_cast<const u32x4 *>(
+                    tile + k_addr[(kk + kQkDepth) & 3] + ((kk + kQkDepth) >> 2) * 128);
+            extra(kk);
             __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int kk = 0; kk < 36; ++kk) {
-                s = mfma_32x32x16(as_bf16x8(frag[kk % kQkDepth]), q[kk], s);
-                if (kk + kQkDepth < 36)
-                    frag[kk % kQkDepth] = *reinterpret_cast<const u32x4 *>(
-                        tile + k_addr[(kk + kQkDepth) & 3] + ((kk + kQkDepth) >> 2) * 128);
-                __builtin_amdgcn_sched_barrier(0);
-            }
         }
-#endif
-
-        MLA_STAMP(4);
-        // ---- online softmax per lane (= per head) --------------------------------------
+    };
+    // masks the tail, then raises the running maximum if this tile needs it (both token
+    // halves of a head must agree on the reference maximum)
+    auto settle = [&](uint32_t key0, floatx16 &s, uint32_t (&pending)[8]) {
         if (key0 + kTile > t1) {
 #pragma unroll
             for (int i = 0; i < 16; ++i)
@@ -264,7 +262,6 @@ yvex_rocm_mla_decode_bf16(const yvex_rocm_mla_params p)
         for (int i = 0; i < 16; ++i) mloc = fmaxf(mloc, s[i]);
         mloc *= p.scale_log2;
         if (__builtin_amdgcn_ballot_w64(mloc > m_run + kLazyLog2) != 0ull) {
-            // both token halves of a head must agree on the reference maximum
             const float m_new = fmaxf(m_run, fmaxf(mloc, xor_lanes(mloc, 32)));
             const float alpha = m_new == -INFINITY ? 1.0f : fast_exp2(m_run - m_new);
             l_run *= alpha;
@@ -275,23 +272,32 @@ yvex_rocm_mla_decode_bf16(const yvex_rocm_mla_params p)
                 o[db] *= alpha;
                 asm volatile("" : "+a"(o[db]));
             }
-            m_run = m_new;
-        }
-        const float neg_m = m_run == -INFINITY ? 0.f : -m_run;
-        uint32_t pk[8];
-        float lsum = 0.f;
+            // probabilities computed under the old maximum that are not in O yet
 #pragma unroll
-        for (int i = 0; i < 16; i += 2) {
-            const float p0 = fast_exp2(__builtin_fmaf(s[i], p.scale_log2, neg_m));
-            const float p1 = fast_exp2(__builtin_fmaf(s[i + 1], p.scale_log2, neg_m));
-            lsum += p0 + p1;
-            pk[i >> 1] = pack_bf16x2(p0, p1);
+            for (int j = 0; j < 8; ++j)
+                pending[j] = pack_bf16x2(bf16_to_f32((uint16_t)(pending[j] & 0xffffu)) * alpha,
+                                         bf16_to_f32((uint16_t)(pending[j] >> 16)) * alpha);
+            m_run = m_new;
+            neg_m = m_new == -INFINITY ? 0.f : -m_new;
         }
-        l_run += lsum;
+    };
 
-        MLA_STAMP(5);
-        // ---- O^T += C^T . P^T ----------------------------------------------------------
-#ifndef MLA_PROBE_SKIP_PV
+#ifdef MLA_PROBE_CLOCK
+    unsigned long long clock_acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    unsigned long long clock_prev = __builtin_readcyclecounter();
+#endif
+    // Software pipeline over tiles: step t computes the scores of tile t (with the loads
+    // of tile t+2 spread behind its MFMAs), settles the maximum, then issues the O^T update
+    // with tile t-1 and, behind its MFMAs, the exponentials of tile t.  Tiles t-1 and t
+    // are being read during a step, tiles t+1 and t+2 are in flight.
+    stage_tile(0u);
+    stage_tile(1u);
+    MLA_STAMP(0);
+    uint32_t pk_prev[8], pk_cur[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) pk_prev[j] = 0u;
+    // O^T += C^T . P^T with the tile at `tile`
+    auto accumulate = [&](const unsigned char *tile, const uint32_t (&pk)[8]) {
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
             const u32x4 w = {pk[u * 4 + 0], pk[u * 4 + 1], pk[u * 4 + 2], pk[u * 4 + 3]};
@@ -307,19 +313,81 @@ yvex_rocm_mla_decode_bf16(const yvex_rocm_mla_params p)
                 o[db] = mfma_32x32x16(__builtin_bit_cast(bf16x8, av), pb, o[db]);
             }
         }
-        // three transposed operand pairs in flight ahead of the MFMAs that consume them
-        __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);
+    };
+    auto step = [&](uint32_t t, auto with_update) {
+        // tile t has landed when at most one younger tile is outstanding: vmcnt(9)
+        __builtin_amdgcn_s_waitcnt(0x0f79);
+        MLA_STAMP(1);
+        __syncthreads();
+        MLA_STAMP(2);
+        uint32_t stage_dst;
+        i32x4 stage_rsrc;
+        stage_target(t + 2u, stage_dst, stage_rsrc);
+        MLA_STAMP(3);
+        const unsigned char *tile = lds + (t % kBuffers) * kTileBytes;
+        const unsigned char *prev_tile = lds + ((t + kBuffers - 1u) % kBuffers) * kTileBytes;
+
+        // ---- S^T of tile t, the loads of tile t+2 behind its MFMAs ------------------------
+        floatx16 s;
+        score(tile, s, [&](int kk) {
+            if ((kk & 3) == 1) stage_one(stage_dst + (kk >> 2) * 1024, stage_rsrc, stage_off[kk >> 2]);
+        });
+        MLA_STAMP(4);
+        settle(t0 + t * kTile, s, pk_prev);
+        MLA_STAMP(5);
+
+        // ---- O^T update with tile t-1 (none in the first step) and the exponentials of
+        //      tile t behind its MFMAs -------------------------------------------------------
+        float lsum = 0.f;
 #pragma unroll
-        for (int i = 0; i < 29; ++i) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+        for (int i = 0; i < 16; i += 2) {
+            const float p0 = fast_exp2(__builtin_fmaf(s[i], p.scale_log2, neg_m));
+            const float p1 = fast_exp2(__builtin_fmaf(s[i + 1], p.scale_log2, neg_m));
+            lsum += p0 + p1;
+            pk_cur[i >> 1] = pack_bf16x2(p0, p1);
         }
-        __builtin_amdgcn_sched_group_barrier(0x008, 3, 0);
-#else
-        o[0][0] += __builtin_bit_cast(float, pk[0] ^ pk[3] ^ pk[5]);
-#endif
+        l_run += lsum;
+        if (decltype(with_update)::value) {
+            accumulate(prev_tile, pk_prev);
+            // three transposed operand pairs in flight ahead of the MFMAs that consume them,
+            // one exponential behind every second MFMA
+            __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);
+#pragma unroll
+            for (int i = 0; i < 14; ++i) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x400, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+            }
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x400, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x400, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) pk_prev[j] = pk_cur[j];
         MLA_STAMP(6);
+    };
+    step(0u, std::integral_constant<bool, false>());
+#ifdef MLA_PROBE_TILES
+    for (uint32_t t = 1; t < MLA_PROBE_TILES; ++t)
+#else
+    for (uint32_t t = 1; t < tiles; ++t)
+#endif
+        step(t, std::integral_constant<bool, true>());
+    // the update with the last tile
+    __builtin_amdgcn_sched_barrier(0);
+    accumulate(lds + ((tiles - 1u) % kBuffers) * kTileBytes, pk_prev);
+    __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);
+#pragma unroll
+    for (int i = 0; i < 29; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
     }
+    __builtin_amdgcn_sched_group_barrier(0x008, 3, 0);
     // drain the loads that were issued past the last tile before the workgroup ends
     __builtin_amdgcn_s_waitcnt(0x0f70);
 
