@@ -714,9 +714,9 @@ static int rocm_mla_decode_execute(yvex_backend *backend,
         mp.head_dim = kp.value_dim;
         mp.chunk_tokens = kp.chunk_tokens;
         mp.max_chunks = kp.max_chunks;
-        rc = yvex_rocm_launch(backend, YVEX_ROCM_FN_DECODE_MERGE, variant, (unsigned int)r->heads,
-                              (unsigned int)r->batch, 1u, (unsigned int)r->value_dimension, 0u, &mp,
-                              where, err);
+        rc = yvex_rocm_launch(backend, YVEX_ROCM_FN_DECODE_MERGE, variant,
+                              (unsigned int)((r->heads + 3ull) / 4ull), (unsigned int)r->batch, 1u,
+                              256u, 0u, &mp, where, err);
     }
     if (rc == YVEX_OK) {
         facts->kernel_launches = 2ull;

@@ -564,33 +564,51 @@ yvex_rocm_decode_finish(const yvex_rocm_decode_params p)
         p.lse[(uint64_t)session * p.query_heads + head] = (top + fast_log2(sum)) * YVEX_LN2;
 }
 
-// Log-sum-exp merge of the chunk partials of one (session, query head); one thread per
-// output lane.  grid = (query_heads, sessions), block = head_dim.
-extern "C" __global__ void __launch_bounds__(512)
+// Log-sum-exp merge of the chunk partials of one (session, query head): one wave per head,
+// eight output dims per lane (one 16-byte load of bf16 partials per chunk), four heads per
+// workgroup.  grid = (ceil(query_heads / 4), sessions), block = 256; head_dim = 512.
+extern "C" __global__ void __launch_bounds__(256)
 yvex_rocm_decode_merge(const yvex_rocm_decode_merge_params p)
 {
-    const uint32_t head = blockIdx.x, session = blockIdx.y, d = threadIdx.x;
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t head = blockIdx.x * 4u + (threadIdx.x >> 6), session = blockIdx.y;
     const uint32_t ctx = p.context ? (uint32_t)p.context[session] : p.fixed_context;
-    if (ctx == 0u || d >= p.head_dim) return;
+    if (ctx == 0u || head >= p.query_heads || lane * 8u >= p.head_dim) return;
     const uint32_t chunks = min(p.max_chunks, (ctx + p.chunk_tokens - 1u) / p.chunk_tokens);
     const uint64_t base = ((uint64_t)session * p.max_chunks) * p.query_heads + head;
     // The chunk loops carry no dependent loads: unrolled, eight partial rows are in
-    // flight per thread, which is what keeps this pass in the microsecond range.
+    // flight per lane, which is what keeps this pass in the microsecond range.
     float top = -INFINITY;
 #pragma unroll 8
     for (uint32_t c = 0; c < chunks; ++c)
         top = fmaxf(top, p.part_ml[(base + (uint64_t)c * p.query_heads) * 2]);
-    float total = 0.f, acc = 0.f;
+    float total = 0.f, acc[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] = 0.f;
 #pragma unroll 8
     for (uint32_t c = 0; c < chunks; ++c) {
         const uint64_t slot = base + (uint64_t)c * p.query_heads;
         const float w = fast_exp2(p.part_ml[slot * 2] - top);
         total += w * p.part_ml[slot * 2 + 1];
-        acc += w * bf16_to_f32(p.part_acc[slot * p.head_dim + d]);
+        const u32x4 row = load_b128(p.part_acc + slot * p.head_dim + lane * 8u);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            acc[2 * i + 0] += w * bf16_to_f32((uint16_t)(row[i] & 0xffffu));
+            acc[2 * i + 1] += w * bf16_to_f32((uint16_t)(row[i] >> 16));
+        }
     }
-    const float o = acc / total;
-    if (!isfinite(o)) flag(p.status, YVEX_ROCM_DEVICE_NUMERIC);
-    p.out[((uint64_t)session * p.query_heads + head) * p.head_dim + d] = bf16_bits(o);
-    if (p.lse && d == 0u)
+    const float inv = 1.0f / total;
+    bool bad = false;
+    u32x4 out;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const float a = acc[2 * i] * inv, b = acc[2 * i + 1] * inv;
+        bad |= !(isfinite(a) && isfinite(b));
+        out[i] = (uint32_t)bf16_bits(a) | ((uint32_t)bf16_bits(b) << 16);
+    }
+    if (bad) flag(p.status, YVEX_ROCM_DEVICE_NUMERIC);
+    *reinterpret_cast<u32x4 *>(p.out + ((uint64_t)session * p.query_heads + head) * p.head_dim +
+                               lane * 8u) = out;
+    if (p.lse && lane == 0u)
         p.lse[(uint64_t)session * p.query_heads + head] = (top + fast_log2(total)) * YVEX_LN2;
 }

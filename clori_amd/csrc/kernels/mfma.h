@@ -81,4 +81,39 @@ __device__ inline float bf16_to_f32(uint16_t b)
     return __builtin_bit_cast(float, (uint32_t)b << 16);
 }
 
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+
+// Raw buffer descriptor over [base, base + bytes): stride 0, untyped dword format; loads
+// past the range return zero.  All four words are made wave-uniform.
+__device__ inline i32x4 raw_buffer(const void *base, uint32_t bytes)
+{
+    const uint64_t address = (uint64_t)base;
+    i32x4 rsrc;
+    rsrc.x = __builtin_amdgcn_readfirstlane((int)(uint32_t)address);
+    rsrc.y = __builtin_amdgcn_readfirstlane((int)((uint32_t)(address >> 32) & 0xffffu));
+    rsrc.z = __builtin_amdgcn_readfirstlane((int)bytes);
+    rsrc.w = 0x00027000;
+    return rsrc;
+}
+
+// One buffer load of 16 bytes per lane that writes LDS directly: lane L's data lands at LDS
+// byte address lds_address + 16 * L (M0 carries the wave-uniform destination).  Issued as
+// opaque assembly on purpose: for the builtin form the compiler makes every later LDS read
+// wait for all outstanding loads (it cannot see that ring buffers do not alias), which
+// serialises any ring of tiles.  The caller waits with s_waitcnt vmcnt and a barrier.
+__device__ inline void lds_dma_b128(uint32_t lds_address, i32x4 rsrc, uint32_t lane_offset,
+                                    uint32_t uniform_offset)
+{
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %2, %1, %3 offen lds"
+                 :
+                 : "s"(lds_address), "s"(rsrc), "v"(lane_offset), "s"(uniform_offset)
+                 : "memory");
+}
+
+// LDS byte address of a pointer into a __shared__ array.
+__device__ inline uint32_t lds_address_of(const void *p)
+{
+    return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const unsigned char *)p;
+}
+
 #endif  // YVEX_ROCM_KERNELS_MFMA_H

@@ -16,7 +16,7 @@
 // this makes the row fetch of the first product (ds_read_b128, lane = token) and the
 // transposed fetch of the second (ds_read_b64_tr_b16, 4 tokens x 16 dims per 16 lanes)
 // both bank-conflict free.
-// Tiles are filled by buffer loads that write LDS directly: lane L of 1 KB load j of
+// Tiles are filled by buffer loads that write LDS directly (lds_dma_b128): lane L of 1 KB load j of
 // wave w owns linear chunk (9w + j) * 64 + L of the tile and fetches the global chunk that
 // belongs there.  A tile never straddles a page (pages are multiples of 32 tokens), so
 // the page id is wave-uniform and the buffer descriptor is rebuilt per tile from the page
@@ -46,10 +46,8 @@ constexpr float kLazyLog2 = 8.0f;
 constexpr int kQkDepth = 4;  // operand fetches in flight ahead of the first product
 constexpr int kMaxChunkPages = YVEX_ROCM_MLA_MAX_CHUNK_PAGES;  // page ids of the chunk, kept in LDS
 
-typedef __attribute__((address_space(3))) void lds_void;
 typedef __attribute__((address_space(3))) short4v lds_short4;
 typedef short short8v __attribute__((ext_vector_type(8)));
-typedef int i32x4 __attribute__((ext_vector_type(4)));
 
 __device__ inline void flag(int32_t *status, int code) { atomicCAS(status, 0, code); }
 
@@ -120,8 +118,8 @@ yvex_rocm_mla_decode_bf16(const yvex_rocm_mla_params p)
         chunk_pages[i] = page;
     }
     __syncthreads();
-    static_assert(kLoadsPerWave == 9, "the staging block issues nine loads");
-    const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)lds;
+    static_assert(kLoadsPerWave == 9, "the loads of a tile ride behind k-steps 1, 5, .. 33");
+    const uint32_t lds_base = lds_address_of(lds);
     uint32_t stage_off[kLoadsPerWave];
 #pragma unroll
     for (int j = 0; j < kLoadsPerWave; ++j) {
@@ -129,9 +127,10 @@ yvex_rocm_mla_decode_bf16(const yvex_rocm_mla_params p)
         const int r = linear / kRowChunks, pos = linear % kRowChunks;
         stage_off[j] = (uint32_t)(r * kRowBytes + ((pos ^ swizzle(r)) << 4));
     }
-    // always issues kLoadsPerWave loads (with an empty range past the last tile) so that
-    // the outstanding-load count at the top of every iteration is the same
-    auto stage_tile = [&](uint32_t tile) {
+    // A tile's destination and descriptor.  Loads are always issued (with an empty range
+    // past the last tile) so that the outstanding-load count at the top of every step is
+    // the same.
+    auto stage_target = [&](uint32_t tile, uint32_t &dst, i32x4 &rsrc) {
         const uint32_t first = t0 + tile * kTile;
         uint32_t valid = 0u;
         const uint16_t *base = p.pool;
@@ -141,33 +140,16 @@ yvex_rocm_mla_decode_bf16(const yvex_rocm_mla_params p)
             valid = min((uint32_t)kTile, t1 - first);
             base = p.pool + ((uint64_t)page * p.page_tokens + first % p.page_tokens) * kKeyDim;
         }
-        // raw buffer descriptor: base, stride 0, byte range, untyped dword format
-        const uint64_t address = (uint64_t)base;
+        rsrc = raw_buffer(base, valid * kRowBytes);
+        dst = __builtin_amdgcn_readfirstlane(lds_base + (tile % kBuffers) * kTileBytes +
+                                             wave * (kLoadsPerWave * 1024));
+    };
+    auto stage_tile = [&](uint32_t tile) {
+        uint32_t dst;
         i32x4 rsrc;
-        rsrc.x = __builtin_amdgcn_readfirstlane((int)(uint32_t)address);
-        rsrc.y = __builtin_amdgcn_readfirstlane((int)(uint32_t)(address >> 32) & 0xffff);
-        rsrc.z = __builtin_amdgcn_readfirstlane((int)(valid * kRowBytes));
-        rsrc.w = 0x00027000;
-        const uint32_t dst = __builtin_amdgcn_readfirstlane(
-            lds_base + (tile % kBuffers) * kTileBytes + wave * (kLoadsPerWave * 1024));
-        // Issued as one opaque block: the compiler would otherwise make every later LDS
-        // read wait for these loads (it cannot see that the ring buffers do not alias),
-        // which serialises the ring.  M0 carries the LDS destination of each load.
-        asm volatile(
-            "s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %2, %1, 0 offen lds\n\t"
-            "s_add_u32 m0, m0, 0x400\n\ts_nop 0\n\tbuffer_load_dwordx4 %3, %1, 0 offen lds\n\t"
-            "s_add_u32 m0, m0, 0x400\n\ts_nop 0\n\tbuffer_load_dwordx4 %4, %1, 0 offen lds\n\t"
-            "s_add_u32 m0, m0, 0x400\n\ts_nop 0\n\tbuffer_load_dwordx4 %5, %1, 0 offen lds\n\t"
-            "s_add_u32 m0, m0, 0x400\n\ts_nop 0\n\tbuffer_load_dwordx4 %6, %1, 0 offen lds\n\t"
-            "s_add_u32 m0, m0, 0x400\n\ts_nop 0\n\tbuffer_load_dwordx4 %7, %1, 0 offen lds\n\t"
-            "s_add_u32 m0, m0, 0x400\n\ts_nop 0\n\tbuffer_load_dwordx4 %8, %1, 0 offen lds\n\t"
-            "s_add_u32 m0, m0, 0x400\n\ts_nop 0\n\tbuffer_load_dwordx4 %9, %1, 0 offen lds\n\t"
-            "s_add_u32 m0, m0, 0x400\n\ts_nop 0\n\tbuffer_load_dwordx4 %10, %1, 0 offen lds"
-            :
-            : "s"(dst), "s"(rsrc), "v"(stage_off[0]), "v"(stage_off[1]), "v"(stage_off[2]),
-              "v"(stage_off[3]), "v"(stage_off[4]), "v"(stage_off[5]), "v"(stage_off[6]),
-              "v"(stage_off[7]), "v"(stage_off[8])
-            : "memory", "scc");
+        stage_target(tile, dst, rsrc);
+#pragma unroll
+        for (int j = 0; j < kLoadsPerWave; ++j) lds_dma_b128(dst + j * 1024, rsrc, stage_off[j], 0u);
     };
 
     // ---- operand addresses inside a tile ----------------------------------------------
@@ -194,32 +176,6 @@ yvex_rocm_mla_decode_bf16(const yvex_rocm_mla_params p)
                 v_addr[par][h] = (uint32_t)(r * kRowBytes + (chunk16 << 4) + 8 * (a & 1));
             }
     }
-
-    // one staging load, for spreading a tile's nine loads over the first product
-    auto stage_one = [&](uint32_t dst, i32x4 rsrc, uint32_t offset) {
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %2, %1, 0 offen lds"
-                     :
-                     : "s"(dst), "s"(rsrc), "v"(offset)
-                     : "memory");
-    };
-    auto stage_target = [&](uint32_t tile, uint32_t &dst, i32x4 &rsrc) {
-        const uint32_t first = t0 + tile * kTile;
-        uint32_t valid = 0u;
-        const uint16_t *base = p.pool;
-        if (tile < tiles) {
-            const uint32_t page = (uint32_t)__builtin_amdgcn_readfirstlane(
-                chunk_pages[first / p.page_tokens - first_page]);
-            valid = min((uint32_t)kTile, t1 - first);
-            base = p.pool + ((uint64_t)page * p.page_tokens + first % p.page_tokens) * kKeyDim;
-        }
-        const uint64_t address = (uint64_t)base;
-        rsrc.x = __builtin_amdgcn_readfirstlane((int)(uint32_t)address);
-        rsrc.y = __builtin_amdgcn_readfirstlane((int)(uint32_t)(address >> 32) & 0xffff);
-        rsrc.z = __builtin_amdgcn_readfirstlane((int)(valid * kRowBytes));
-        rsrc.w = 0x00027000;
-        dst = __builtin_amdgcn_readfirstlane(lds_base + (tile % kBuffers) * kTileBytes +
-                                             wave * (kLoadsPerWave * 1024));
-    };
 
     floatx16 o[16];
 #pragma unroll
@@ -330,7 +286,7 @@ yvex_rocm_mla_decode_bf16(const yvex_rocm_mla_params p)
         // ---- S^T of tile t, the loads of tile t+2 behind its MFMAs ------------------------
         floatx16 s;
         score(tile, s, [&](int kk) {
-            if ((kk & 3) == 1) stage_one(stage_dst + (kk >> 2) * 1024, stage_rsrc, stage_off[kk >> 2]);
+            if ((kk & 3) == 1) lds_dma_b128(stage_dst + (kk >> 2) * 1024, stage_rsrc, stage_off[kk >> 2], 0u);
         });
         MLA_STAMP(4);
         settle(t0 + t * kTile, s, pk_prev);
