@@ -264,8 +264,8 @@ def roofline(result):
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # runs (profiles/), scaled by the same counters on a copy kernel of known size; None where
 # no such run is committed.
-TRAFFIC = {"paged3": 1033350210, "paged4": 1512968247, "decode1": 18117049,
-           "prefill2": 50470939}
+TRAFFIC = {"paged3": 1033350292, "paged4": 1512968367, "decode1": 18117050,
+           "prefill2": 50475981, "mla5": 204071018}
 
 
 def repeat_for(seconds, call):
