@@ -25,7 +25,8 @@
 // no LDS store instructions): lane L of a 1 KB load owns chunk position L % 16 of row
 // L / 16 and fetches the global chunk that belongs there.  Rows past the end of the
 // tensor read as zero through the buffer range check.  Two buffers; the loads of tile
-// t+1 are issued right after the barrier of tile t, one barrier per tile.
+// t+1 are issued one by one behind the first MFMAs of tile t (issuing one costs the wave
+// about 50 cycles), one barrier per tile.
 //
 // The running maximum is only raised when a tile exceeds it by more than kLazyLog2 (in
 // log2 units), so the accumulator rescale is rare; probabilities are then at most
@@ -46,13 +47,27 @@ constexpr int kBufBytes = 2 * kTileBytes;          // K then V
 constexpr int kThreads = 256;
 constexpr float kLazyLog2 = 8.0f;
 
-typedef __attribute__((address_space(3))) void lds_void;
 typedef __attribute__((address_space(3))) short4v lds_short4;
 
 // chunk swizzle of tile row r
 __device__ inline int swizzle(int r) { return ((r & 3) << 2) | ((r >> 2) & 3); }
 
 __device__ inline void flag(int32_t *status, int code) { atomicCAS(status, 0, code); }
+
+#ifdef PREFILL_PROBE_CLOCK
+// timing probe: phase cycle counts of wave 0 of workgroup 0, summed over its tiles
+__device__ unsigned long long yvex_prefill_clock[8];
+#define PREFILL_STAMP(slot)                                                    \
+    do {                                                                       \
+        __builtin_amdgcn_sched_barrier(0);                                     \
+        const unsigned long long now_ = __builtin_readcyclecounter();          \
+        clock_acc[slot] += now_ - clock_prev;                                  \
+        clock_prev = now_;                                                     \
+        __builtin_amdgcn_sched_barrier(0);                                     \
+    } while (0)
+#else
+#define PREFILL_STAMP(slot) do { } while (0)
+#endif
 
 template <int NB>
 __device__ inline void prefill_body(const yvex_rocm_prefill_params &p, unsigned char *lds)
@@ -89,12 +104,11 @@ __device__ inline void prefill_body(const yvex_rocm_prefill_params &p, unsigned 
     // 1 KB load j of wave w fills rows 16w + 4j .. +3 of the tile; lane L owns chunk
     // position L % 16 of row 16w + 4j + L / 16 and fetches chunk (L % 16) ^ x(row).
     const uint32_t k_row_bytes = (uint32_t)p.k_stride * 2u, v_row_bytes = (uint32_t)p.v_stride * 2u;
-    const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-        (void *)(p.k + (uint64_t)kv_head * kHeadDim), 0,
-        p.kv_tokens * k_row_bytes - kv_head * kRowBytes, 0x00027000);
-    const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-        (void *)(p.v + (uint64_t)kv_head * kHeadDim), 0,
-        p.kv_tokens * v_row_bytes - kv_head * kRowBytes, 0x00027000);
+    const i32x4 k_rsrc = raw_buffer(p.k + (uint64_t)kv_head * kHeadDim,
+                                    p.kv_tokens * k_row_bytes - kv_head * kRowBytes);
+    const i32x4 v_rsrc = raw_buffer(p.v + (uint64_t)kv_head * kHeadDim,
+                                    p.kv_tokens * v_row_bytes - kv_head * kRowBytes);
+    const uint32_t lds_base = lds_address_of(lds);
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);
     uint32_t k_off[4], v_off[4];
 #pragma unroll
@@ -104,17 +118,18 @@ __device__ inline void prefill_body(const yvex_rocm_prefill_params &p, unsigned 
         k_off[j] = (uint32_t)r * k_row_bytes + chunk * 16u;
         v_off[j] = (uint32_t)r * v_row_bytes + chunk * 16u;
     }
+    // load j (0..7) of a tile: 0..3 fill this wave's K rows, 4..7 its V rows
+    auto stage_one = [&](uint32_t tile, int buf, int j) {
+        const uint32_t dst = lds_base + buf * kBufBytes + wave_u * 4096;
+        if (j < 4)
+            lds_dma_b128(dst + j * 1024, k_rsrc, k_off[j], tile * kKeyTile * k_row_bytes);
+        else
+            lds_dma_b128(dst + kTileBytes + (j - 4) * 1024, v_rsrc, v_off[j - 4],
+                         tile * kKeyTile * v_row_bytes);
+    };
     auto stage_tile = [&](uint32_t tile, int buf) {
-        unsigned char *dst = lds + buf * kBufBytes + wave_u * 4096;
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(k_rsrc, (lds_void *)(dst + j * 1024), 16,
-                                                     k_off[j], tile * kKeyTile * k_row_bytes, 0, 0);
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(v_rsrc,
-                                                     (lds_void *)(dst + kTileBytes + j * 1024), 16,
-                                                     v_off[j], tile * kKeyTile * v_row_bytes, 0, 0);
+        for (int j = 0; j < 8; ++j) stage_one(tile, buf, j);
     };
 
     // ---- operand addresses inside a tile ------------------------------------------
@@ -160,15 +175,25 @@ __device__ inline void prefill_body(const yvex_rocm_prefill_params &p, unsigned 
     const uint32_t wave_last_vis =
         p.causal ? p.query_start + min(row0 + kRowsPerWave, p.query_tokens) - 1u : p.kv_tokens - 1u;
 
+#ifdef PREFILL_PROBE_CLOCK
+    unsigned long long clock_acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    unsigned long long clock_prev = __builtin_readcyclecounter();
+#endif
     stage_tile(0u, 0);
     for (uint32_t t = 0; t < tiles; ++t) {
         const int buf = (int)(t & 1u);
         __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's part of tile t is in LDS
+        PREFILL_STAMP(0);
         __syncthreads();
-        if (t + 1u < tiles) stage_tile(t + 1u, buf ^ 1);
+        PREFILL_STAMP(1);
         const uint32_t key0 = t * kKeyTile;
+        const bool more = t + 1u < tiles;
         // a wave whose every row sees nothing of this tile skips the products
-        if (!wave_active || key0 > wave_last_vis) continue;
+        if (!wave_active || key0 > wave_last_vis) {
+            if (more) stage_tile(t + 1u, buf ^ 1);
+            continue;
+        }
+        PREFILL_STAMP(2);
         const unsigned char *tile = lds + buf * kBufBytes;
 
         // ---- S^T = K . Q^T -------------------------------------------------
@@ -179,25 +204,31 @@ __device__ inline void prefill_body(const yvex_rocm_prefill_params &p, unsigned 
             for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
                 for (int i = 0; i < 16; ++i) s[mb][nb][i] = 0.f;
+        {
+            // operand fetches run kDepth steps ahead of the MFMAs, the eight loads of the
+            // next tile ride behind the first eight steps; the order is pinned
+            constexpr int kDepth = 4;
+            auto fetch = [&](int i) {  // i = kk * 2 + mb
+                return *reinterpret_cast<const u32x4 *>(tile + k_addr[i >> 1] +
+                                                        (i & 1) * 32 * kRowBytes);
+            };
+            u32x4 frag[kDepth];
 #pragma unroll
-        for (int kk = 0; kk < 8; ++kk) {
+            for (int i = 0; i < kDepth; ++i) frag[i] = fetch(i);
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int mb = 0; mb < 2; ++mb) {
-                const bf16x8 a = as_bf16x8(*reinterpret_cast<const u32x4 *>(
-                    tile + k_addr[kk] + mb * 32 * kRowBytes));
+            for (int i = 0; i < 16; ++i) {
+                const bf16x8 a = as_bf16x8(frag[i % kDepth]);
 #pragma unroll
-                for (int nb = 0; nb < NB; ++nb) s[mb][nb] = mfma_32x32x16(a, q[nb][kk], s[mb][nb]);
+                for (int nb = 0; nb < NB; ++nb)
+                    s[i & 1][nb] = mfma_32x32x16(a, q[nb][i >> 1], s[i & 1][nb]);
+                if (i + kDepth < 16) frag[i % kDepth] = fetch(i + kDepth);
+                if (i < 8 && more) stage_one(t + 1u, buf ^ 1, i);
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
-        // keep three operand pairs in flight ahead of the MFMAs that consume them
-        __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);
-#pragma unroll
-        for (int i = 0; i < 5; ++i) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 2 * NB, 0);
-            __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-        }
-        __builtin_amdgcn_sched_group_barrier(0x008, 6 * NB, 0);
 
+        PREFILL_STAMP(3);
         // ---- mask, online softmax (per lane = per query row) ----------------------
         // scores stay raw; the softmax scale is folded into the exponent's multiply-add
         const bool need_mask = (key0 + kKeyTile - 1u > wave_first_vis) ||
@@ -247,6 +278,7 @@ __device__ inline void prefill_body(const yvex_rocm_prefill_params &p, unsigned 
             l_run[nb] += lsum;
         }
 
+        PREFILL_STAMP(4);
         // ---- O^T += V^T . P^T -------------------------------------------------
 #pragma unroll
         for (int mb = 0; mb < 2; ++mb)
@@ -273,8 +305,13 @@ __device__ inline void prefill_body(const yvex_rocm_prefill_params &p, unsigned 
                     for (int nb = 0; nb < NB; ++nb) o[db][nb] = mfma_32x32x16(a, pb[nb], o[db][nb]);
                 }
             }
+        PREFILL_STAMP(5);
     }
 
+#ifdef PREFILL_PROBE_CLOCK
+    if (blockIdx.x == 0 && tid == 0)
+        for (int i = 0; i < 8; ++i) yvex_prefill_clock[i] = clock_acc[i];
+#endif
     // ---- epilogue: normalise, publish bf16 rows and LSE -------------------------
     if (!wave_active) return;
 #pragma unroll
