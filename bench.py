@@ -73,7 +73,9 @@ def time_steps(backend, run, steps, warmup, kernel):
     launches, kernel_ms = backend.kernel_probe_end()
     backend.sync()
     backend.set_completion_mode(B.COMPLETION_IMMEDIATE)
-    return device_ms / steps, wall_ms / steps, kernel_ms / max(launches, 1)
+    # an event pair around one launch adds a few microseconds: a kernel cannot take longer than
+    # the step that contains it
+    return device_ms / steps, wall_ms / steps, min(kernel_ms / max(launches, 1), device_ms / steps)
 
 
 # --------------------------------------------------------------------- workloads --

@@ -576,26 +576,44 @@ yvex_rocm_decode_merge(const yvex_rocm_decode_merge_params p)
     if (ctx == 0u || head >= p.query_heads || lane * 8u >= p.head_dim) return;
     const uint32_t chunks = min(p.max_chunks, (ctx + p.chunk_tokens - 1u) / p.chunk_tokens);
     const uint64_t base = ((uint64_t)session * p.max_chunks) * p.query_heads + head;
-    // The chunk loops carry no dependent loads: unrolled, eight partial rows are in
-    // flight per lane, which is what keeps this pass in the microsecond range.
-    float top = -INFINITY;
-#pragma unroll 8
-    for (uint32_t c = 0; c < chunks; ++c)
-        top = fmaxf(top, p.part_ml[(base + (uint64_t)c * p.query_heads) * 2]);
-    float total = 0.f, acc[8];
+    // Sixteen chunks per trip, every load of a trip independent of the others (indices past
+    // the end alias the last chunk with weight zero): one memory round trip per trip, which
+    // is what keeps this pass in the microsecond range.
+    float top = -INFINITY, total = 0.f, acc[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) acc[i] = 0.f;
-#pragma unroll 8
-    for (uint32_t c = 0; c < chunks; ++c) {
-        const uint64_t slot = base + (uint64_t)c * p.query_heads;
-        const float w = fast_exp2(p.part_ml[slot * 2] - top);
-        total += w * p.part_ml[slot * 2 + 1];
-        const u32x4 row = load_b128(p.part_acc + slot * p.head_dim + lane * 8u);
+    for (uint32_t c0 = 0; c0 < chunks; c0 += 16u) {
+        float m[16], l[16];
+        u32x4 row[16];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            acc[2 * i + 0] += w * bf16_to_f32((uint16_t)(row[i] & 0xffffu));
-            acc[2 * i + 1] += w * bf16_to_f32((uint16_t)(row[i] >> 16));
+        for (int j = 0; j < 16; ++j) {
+            const uint64_t slot = base + (uint64_t)min(c0 + (uint32_t)j, chunks - 1u) * p.query_heads;
+            m[j] = p.part_ml[slot * 2];
+            l[j] = p.part_ml[slot * 2 + 1];
+            row[j] = load_b128(p.part_acc + slot * p.head_dim + lane * 8u);
         }
+        float trip = -INFINITY;
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            if (c0 + (uint32_t)j >= chunks) m[j] = -INFINITY;
+            trip = fmaxf(trip, m[j]);
+        }
+        const float m_new = fmaxf(top, trip);
+        const float keep = fast_exp2(top - m_new);  // 0 on the first trip (top = -inf)
+        total *= keep;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[i] *= keep;
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            const float w = fast_exp2(m[j] - m_new);
+            total += w * l[j];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                acc[2 * i + 0] += w * bf16_to_f32((uint16_t)(row[j][i] & 0xffffu));
+                acc[2 * i + 1] += w * bf16_to_f32((uint16_t)(row[j][i] >> 16));
+            }
+        }
+        top = m_new;
     }
     const float inv = 1.0f / total;
     bool bad = false;
