@@ -1,0 +1,88 @@
+#!/usr/bin/env python3
+"""Writes tests/golden/reference_attention.npz: outputs of the REFERENCE's own CPU attention
+operator and codecs (compiled from its sources into oracle/_ref by `make -C oracle ref`)
+on inputs that the test regenerates from closed-form integer patterns.
+
+Run in a container that has the reference tree:  python tests/golden/make_golden.py
+The fixture holds data only (inputs are formulas, outputs are arrays); it lets the oracle
+be checked bit for bit where the reference cannot be built.
+"""
+import ctypes as C
+import os
+import sys
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.dirname(HERE))
+from oracle_binding import f32p, load_reference, _ptr  # noqa: E402
+
+# (name, seq_len, head_dim, position, causal)
+CASES = [
+    ("one-key", 1, 128, 0, 1),
+    ("five-keys", 5, 128, 4, 1),
+    ("mid-causal", 64, 128, 37, 1),
+    ("odd-257-full", 257, 128, 0, 0),
+    ("narrow-d64", 300, 64, 299, 1),
+    ("decode-4096", 4096, 128, 4095, 1),
+    ("long-16384", 16384, 128, 16383, 1),
+]
+
+
+def pattern(count, mul, add, mod, offset, div):
+    """The integer generators of the reference's own tests
+    (tests/unit/cuda/quant_qtype.c:2293-2296): ((i * mul + add) % mod - offset) / div."""
+    i = np.arange(count, dtype=np.int64)
+    return (((i * mul + add) % mod - offset).astype(np.float32) / np.float32(div)).astype(np.float32)
+
+
+def inputs(seq_len, head_dim):
+    q = pattern(head_dim, 3, 0, 19, 9, 8)
+    k = pattern(seq_len * head_dim, 5, 2, 23, 11, 9).reshape(seq_len, head_dim)
+    v = pattern(seq_len * head_dim, 7, 1, 29, 14, 10).reshape(seq_len, head_dim)
+    return q, k, v
+
+
+def main():
+    ref = load_reference()
+    if ref is None:
+        sys.exit("oracle/_ref/libyvex_ref.so is not built: run `make -C oracle ref`")
+    out = {}
+    for name, n, d, position, causal in CASES:
+        q, k, v = inputs(n, d)
+        score = np.zeros(n, np.float32)
+        prob = np.zeros(n, np.float32)
+        o = np.zeros(d, np.float32)
+        rc = ref.yvref_op_attention(_ptr(q, f32p), _ptr(k, f32p), _ptr(v, f32p), n, position, d,
+                                    np.float32(1.0 / np.sqrt(d)), causal, _ptr(score, f32p),
+                                    _ptr(prob, f32p), _ptr(o, f32p))
+        assert rc == 0, (name, rc)
+        out[name + "/out"] = o
+        # score and prob rows are long: keep both ends and strided samples
+        keep = np.unique(np.concatenate([np.arange(min(n, 16)), np.arange(max(n - 16, 0), n),
+                                         np.arange(0, n, 97)]))
+        out[name + "/index"] = keep.astype(np.int64)
+        out[name + "/score"] = score[keep]
+        out[name + "/prob"] = prob[keep]
+    # codecs: bf16 / f16 encodings of a float sweep, Q8_0 of two blocks
+    sweep = np.concatenate([pattern(4096, 37, 5, 1009, 504, 64),
+                            np.array([0.0, -0.0, 1.00390625, 1.01171875, 65504.0, 7e-8, -3e38],
+                                     np.float32)])
+    sweep = np.ascontiguousarray(sweep, np.float32)
+    bits = np.zeros(sweep.size, np.uint16)
+    ref.yvref_bf16_encode_n(_ptr(sweep, f32p), bits.ctypes.data_as(C.POINTER(C.c_uint16)), sweep.size)
+    out["codec/bf16"] = bits.copy()
+    ref.yvref_f16_encode_n(_ptr(sweep, f32p), bits.ctypes.data_as(C.POINTER(C.c_uint16)), sweep.size)
+    out["codec/f16"] = bits.copy()
+    blocks = pattern(64, 11, 3, 61, 30, 7)
+    enc = np.zeros(68, np.uint8)
+    for b in range(2):
+        ref.yvref_q8_0_encode_block(_ptr(np.ascontiguousarray(blocks[32 * b:32 * b + 32]), f32p),
+                                    enc[34 * b:].ctypes.data_as(C.POINTER(C.c_ubyte)))
+    out["codec/q8_0"] = enc
+    np.savez_compressed(os.path.join(HERE, "reference_attention.npz"), **out)
+    print("wrote", len(out), "arrays")
+
+
+if __name__ == "__main__":
+    main()

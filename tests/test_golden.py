@@ -1,0 +1,45 @@
+"""The oracle against committed outputs of the reference's own CPU operator and codecs
+(tests/golden/reference_attention.npz, written by tests/golden/make_golden.py from the
+reference compiled in place).  Bit-exact: same double accumulation, float score store, own
+exp and two float roundings of the probabilities as src/backend/cpu.c:307-399."""
+import importlib.util
+import os
+
+import numpy as np
+import pytest
+
+from oracle_binding import Oracle
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+spec = importlib.util.spec_from_file_location("make_golden",
+                                              os.path.join(HERE, "golden", "make_golden.py"))
+make_golden = importlib.util.module_from_spec(spec)
+spec.loader.exec_module(make_golden)
+
+GOLDEN = np.load(os.path.join(HERE, "golden", "reference_attention.npz"), allow_pickle=False)
+ORACLE = Oracle()
+
+
+@pytest.mark.parametrize("case", make_golden.CASES, ids=[c[0] for c in make_golden.CASES])
+def test_attention_head_matches_reference_output_bits(case):
+    name, n, d, position, causal = case
+    q, k, v = make_golden.inputs(n, d)
+    rc, out, score, prob, _ = ORACLE.attention_head(q, k, v, position, np.float32(1.0 / np.sqrt(d)),
+                                                    causal=bool(causal))
+    assert rc == 0
+    keep = GOLDEN[name + "/index"]
+    assert np.array_equal(out.view(np.uint32), GOLDEN[name + "/out"].view(np.uint32))
+    assert np.array_equal(score[keep].view(np.uint32), GOLDEN[name + "/score"].view(np.uint32))
+    assert np.array_equal(prob[keep].view(np.uint32), GOLDEN[name + "/prob"].view(np.uint32))
+
+
+def test_codecs_match_reference_bits():
+    sweep = np.concatenate([make_golden.pattern(4096, 37, 5, 1009, 504, 64),
+                            np.array([0.0, -0.0, 1.00390625, 1.01171875, 65504.0, 7e-8, -3e38],
+                                     np.float32)]).astype(np.float32)
+    assert np.array_equal(ORACLE.bf16_encode(sweep), GOLDEN["codec/bf16"])
+    f16 = np.array([ORACLE.lib.yvo_f16_encode(float(x)) for x in sweep], dtype=np.uint16)
+    assert np.array_equal(f16, GOLDEN["codec/f16"])
+    blocks = make_golden.pattern(64, 11, 3, 61, 30, 7)
+    enc = ORACLE.q8_0_encode_rows(blocks.reshape(2, 32)).reshape(-1)
+    assert np.array_equal(enc, GOLDEN["codec/q8_0"])
