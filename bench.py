@@ -218,6 +218,49 @@ def workload_mla5(backend, rng, steps, warmup):
                 dominant_kernel="yvex_rocm_mla_decode_bf16")
 
 
+def workload_append(backend, rng, steps, warmup, q8=False):
+    """The KV page writer on a prefill-sized batch: 16 sessions x 2048 new tokens, 8 kv heads,
+    d=128, rotate-half on the whole key row, unaligned start positions.  Not one of the
+    metric's configurations: run by name."""
+    sessions, hkv, d, page, new = 16, 8, 128, 16, 2048
+    starts = rng.integers(0, 4096, size=sessions).astype(np.int32)
+    counts = np.full(sessions, new, np.int32)
+    stride = int((starts.max() + new + page - 1) // page)
+    pool_pages = sessions * stride
+    table = rng.permutation(pool_pages).astype(np.int32).reshape(sessions, stride)
+    total = sessions * new
+    block = 2176 if q8 else 4096
+    pool_bytes = pool_pages * hkv * block
+    pool_dtype = B.DTYPE_I8 if q8 else B.DTYPE_BF16
+    elems = pool_bytes // B.DTYPE_BYTES[pool_dtype]
+    angles = rng.uniform(-3.0, 3.0, size=(total, d)).astype(np.float32)
+    t = [backend.tensor("k-new", B.DTYPE_BF16, (total, hkv, d), random_bf16(rng, total * hkv * d)),
+         backend.tensor("v-new", B.DTYPE_BF16, (total, hkv, d), random_bf16(rng, total * hkv * d)),
+         backend.tensor("rows", B.DTYPE_I32, (sessions,), (np.arange(sessions) * new).astype(np.int32)),
+         backend.tensor("starts", B.DTYPE_I32, (sessions,), starts),
+         backend.tensor("counts", B.DTYPE_I32, (sessions,), counts),
+         backend.tensor("table", B.DTYPE_I32, table.shape, table),
+         backend.tensor("k-pages", pool_dtype, (elems,)),
+         backend.tensor("v-pages", pool_dtype, (elems,))]
+    t[6].zero()
+    t[7].zero()
+    cosine = backend.tensor("cos", B.DTYPE_F32, angles.shape, np.cos(angles))
+    sine = backend.tensor("sin", B.DTYPE_F32, angles.shape, np.sin(angles))
+    storage = B.KV_Q8_0 if q8 else B.KV_BF16
+    run = lambda: backend.kv_append_execute(*t, hkv, pool_pages, new, storage=storage,  # noqa: E731
+                                            cosine=cosine, sine=sine, rotary_dimension=d)
+    facts = run()
+    kernel = "yvex_rocm_kv_append_q8_0" if q8 else "yvex_rocm_kv_append_bf16"
+    ms, wall, kms = time_steps(backend, run, steps, warmup, kernel)
+    # per token: K and V rows in (bf16), both page rows out, half a cos and half a sin row
+    algo = total * (2 * hkv * d * 2 + 2 * hkv * (136 if q8 else 256) + d * 4) + 3 * sessions * 4
+    return dict(name="append_q8_0" if q8 else "append_bf16",
+                workload="KV page writer, %s pages: 16 sessions x 2048 new tokens, 8 kv heads, "
+                         "d=128, rotary 128, unaligned starts" % ("Q8_0" if q8 else "bf16"),
+                bound="hbm", algorithmic_bytes=algo, tokens=total, ms=ms, wall_ms=wall,
+                kernel_ms=kms, launches=int(facts.kernel_launches), dominant_kernel=kernel)
+
+
 def copy_reference(backend, steps):
     """A device-to-device copy of known size: the scale for the FETCH_SIZE / WRITE_SIZE
     counters.  Not a workload of the metric; run as --workload copy."""
@@ -241,7 +284,13 @@ WORKLOADS = {
     "paged4": lambda b, r, s, w: workload_paged(b, r, s, w, q8=True),
     "mla5": workload_mla5,
 }
-SEEDS = {"decode1": 1, "prefill2": 2, "paged3": 3, "paged4": 4, "mla5": 5}
+# measured by name only (rows next to the metric's path, not configurations of the metric)
+EXTRA_WORKLOADS = {
+    "append_bf16": lambda b, r, s, w: workload_append(b, r, s, w, q8=False),
+    "append_q8_0": lambda b, r, s, w: workload_append(b, r, s, w, q8=True),
+}
+SEEDS = {"decode1": 1, "prefill2": 2, "paged3": 3, "paged4": 4, "mla5": 5, "append_bf16": 6,
+         "append_q8_0": 7}
 
 
 def roofline(result):
@@ -368,11 +417,11 @@ def main():
         if backend.status != B.STATUS_READY:
             sys.exit("bench.py: ROCm backend is not ready: %s" % backend.report().rejection.decode())
         rng = np.random.default_rng(SEEDS[name])
-        results[name] = WORKLOADS[name](backend, rng, args.steps, args.warmup)
+        results[name] = {**WORKLOADS, **EXTRA_WORKLOADS}[name](backend, rng, args.steps, args.warmup)
         backend.close()
     head = results[headline]
     roof = roofline(head)
-    cpu = {} if args.no_cpu else {n: cpu_baseline(n) for n in names}
+    cpu = {} if args.no_cpu else {n: cpu_baseline(n) for n in names if n in WORKLOADS}
     line = {
         "metric": METRIC,
         "value": roof["step"],

@@ -341,6 +341,33 @@ class Backend:
         return facts
 
 
+    # -- KV page writer ---------------------------------------------------
+    def kv_append_execute(self, key, value, row_start, position_start, token_count, page_table,
+                          k_pool, v_pool, kv_heads, pool_pages, max_tokens_per_session,
+                          storage=B.KV_BF16, cosine=None, sine=None, rotary_dimension=0,
+                          head_dimension=128, page_tokens=16):
+        """Writes the new rows into the paged pools; all arguments are device tensors."""
+        ops = self.rocm_attention_operations()
+        if ops is None:
+            raise YvexError(B.YVEX_ERR_UNSUPPORTED, "rocm_attention_operations", "not published")
+        r = B.KvAppendRequirement()
+        r.sessions = row_start.shape[0]
+        r.total_tokens = key.shape[0]
+        r.max_tokens_per_session = max_tokens_per_session
+        r.key_value_heads, r.head_dimension, r.page_tokens = kv_heads, head_dimension, page_tokens
+        r.pool_pages, r.page_table_stride = pool_pages, page_table.shape[1]
+        r.rotary_dimension, r.storage = rotary_dimension, storage
+        request = B.KvAppendRequest(r, key.handle, value.handle,
+                                    cosine.handle if cosine else None,
+                                    sine.handle if sine else None, row_start.handle,
+                                    position_start.handle, token_count.handle, page_table.handle,
+                                    k_pool.handle, v_pool.handle)
+        facts, err = B.OperationFacts(), B.Error()
+        _check(ops.kv_append_execute(self.handle, C.byref(request), C.byref(facts), C.byref(err)),
+               err)
+        return facts
+
+
 # -- host helpers that are part of the product (layout + codecs, no attention math) --
 
 def kv_pack_pages(rows, storage, is_value, kv_heads, head_dim=128, page_tokens=16):

@@ -156,6 +156,20 @@ class MlaDecodeRequest(C.Structure):
                 ("output", TensorP), ("lse", TensorP)]
 
 
+class KvAppendRequirement(C.Structure):
+    _fields_ = [(n, ull) for n in ("sessions", "total_tokens", "max_tokens_per_session",
+                                   "key_value_heads", "head_dimension", "page_tokens",
+                                   "pool_pages", "page_table_stride", "rotary_dimension")] + [
+        ("storage", C.c_int)]
+
+
+class KvAppendRequest(C.Structure):
+    _fields_ = [("requirement", KvAppendRequirement), ("key", TensorP), ("value", TensorP),
+                ("cosine", TensorP), ("sine", TensorP), ("row_start", TensorP),
+                ("position_start", TensorP), ("token_count", TensorP), ("page_table", TensorP),
+                ("k_pool", TensorP), ("v_pool", TensorP)]
+
+
 ErrorP = C.POINTER(Error)
 FactsP = C.POINTER(OperationFacts)
 ullP = C.POINTER(ull)
@@ -175,12 +189,16 @@ class TransformerOperations(C.Structure):
                 ("attention_execute", EXECUTE_FN)]
 
 
+KV_APPEND_FN = C.CFUNCTYPE(C.c_int, C.c_void_p, C.POINTER(KvAppendRequest), FactsP, ErrorP)
+
+
 class RocmAttentionOperations(C.Structure):
     _fields_ = [("attention_execute_lse", EXECUTE_LSE_FN),
                 ("paged_decode_workspace_required", PAGED_WORKSPACE_FN),
                 ("paged_decode_execute", PAGED_EXECUTE_FN),
                 ("mla_decode_workspace_required", MLA_WORKSPACE_FN),
-                ("mla_decode_execute", MLA_EXECUTE_FN)]
+                ("mla_decode_execute", MLA_EXECUTE_FN),
+                ("kv_append_execute", KV_APPEND_FN)]
 
 
 class RocmReport(C.Structure):

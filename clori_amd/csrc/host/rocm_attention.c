@@ -739,6 +739,106 @@ static int rocm_mla_decode_execute(yvex_backend *backend,
     return YVEX_OK;
 }
 
+/* ------------------------------------------------------------ KV append ---- */
+
+/* Writes new key/value rows into the paged pools (rotary on the keys, Q8_0 quantise on
+ * write).  One launch; the pools stay written tensors. */
+static int rocm_kv_append_execute(yvex_backend *backend, const yvex_rocm_kv_append_request *request,
+                                  yvex_backend_operation_facts *facts, yvex_error *err)
+{
+    static const char where[] = "rocm.attention.kv_append";
+    yvex_rocm_backend_state *state = yvex_rocm_state(backend);
+    const yvex_rocm_kv_append_requirement *r;
+    yvex_rocm_kv_append_params kp;
+    yvex_backend_operation_variant variant;
+    yvex_dtype pool_dtype;
+    unsigned long long block_bytes, pool_bytes, row_elements, capacity, page_slots;
+    int rc;
+    if (!request || !request->key || !request->value || !request->row_start ||
+        !request->position_start || !request->token_count || !request->page_table ||
+        !request->k_pool || !request->v_pool || !facts)
+        return refuse(err, YVEX_ERR_INVALID_ARG, where,
+                      "complete KV-append tensors and result facts are required");
+    rc = backend_dispatch_admit(backend, where, err);
+    if (rc != YVEX_OK) return rc;
+    r = &request->requirement;
+    if (!r->sessions || !r->total_tokens || !r->max_tokens_per_session || !r->key_value_heads ||
+        !r->head_dimension || !r->page_tokens || !r->pool_pages || !r->page_table_stride ||
+        r->max_tokens_per_session > r->total_tokens ||
+        !yvex_core_u64_mul(r->page_table_stride, r->page_tokens, &capacity) ||
+        (r->rotary_dimension && (!request->cosine || !request->sine)))
+        return refuse(err, YVEX_ERR_INVALID_ARG, where, "complete KV-append geometry is required");
+    block_bytes = yvex_rocm_kv_page_block_bytes(r->storage, r->head_dimension, r->page_tokens);
+    if (!block_bytes || r->rotary_dimension > r->head_dimension || r->rotary_dimension % 16ull ||
+        r->sessions > 65535ull || r->key_value_heads > 65535ull || r->pool_pages > 0x7fffffffull ||
+        capacity > 0x7fffffffull || r->total_tokens > 0x7fffffffull)
+        return refuse(err, YVEX_ERR_UNSUPPORTED, where,
+                      "ROCm KV append requires head dimension 128, 16-token pages, BF16 or Q8_0 "
+                      "storage and a rotary dimension that is a multiple of 16");
+    memset(facts, 0, sizeof(*facts));
+    pool_dtype = r->storage == YVEX_ROCM_KV_BF16 ? YVEX_DTYPE_BF16 : YVEX_DTYPE_I8;
+    row_elements = r->total_tokens * r->key_value_heads * r->head_dimension;
+    /* the pools may be fresh (all zero) or hold earlier tokens: written state is not required */
+    if (!state || !yvex_core_u64_mul(r->pool_pages * r->key_value_heads, block_bytes, &pool_bytes) ||
+        !view_ok(backend, request->key, YVEX_DTYPE_BF16, row_elements, 1) ||
+        !view_ok(backend, request->value, YVEX_DTYPE_BF16, row_elements, 1) ||
+        (r->rotary_dimension &&
+         (!view_ok(backend, request->cosine, YVEX_DTYPE_F32, r->total_tokens * r->rotary_dimension, 1) ||
+          !view_ok(backend, request->sine, YVEX_DTYPE_F32, r->total_tokens * r->rotary_dimension, 1))) ||
+        !view_ok(backend, request->row_start, YVEX_DTYPE_I32, r->sessions, 1) ||
+        !view_ok(backend, request->position_start, YVEX_DTYPE_I32, r->sessions, 1) ||
+        !view_ok(backend, request->token_count, YVEX_DTYPE_I32, r->sessions, 1) ||
+        !view_ok(backend, request->page_table, YVEX_DTYPE_I32, r->sessions * r->page_table_stride, 1) ||
+        !view_ok(backend, request->k_pool, pool_dtype,
+                 pool_bytes / yvex_dtype_element_bytes(pool_dtype), 0) ||
+        !view_ok(backend, request->v_pool, pool_dtype,
+                 pool_bytes / yvex_dtype_element_bytes(pool_dtype), 0))
+        return refuse(err, YVEX_ERR_FORMAT, where,
+                      "rows, tables, descriptors and pools must be tensors of this backend with "
+                      "the declared geometry");
+    memset(&kp, 0, sizeof(kp));
+    kp.key = (const uint16_t *)request->key->data;
+    kp.value = (const uint16_t *)request->value->data;
+    kp.cosine = r->rotary_dimension ? (const float *)request->cosine->data : NULL;
+    kp.sine = r->rotary_dimension ? (const float *)request->sine->data : NULL;
+    kp.row_start = (const int32_t *)request->row_start->data;
+    kp.position_start = (const int32_t *)request->position_start->data;
+    kp.token_count = (const int32_t *)request->token_count->data;
+    kp.page_table = (const int32_t *)request->page_table->data;
+    kp.k_pool = request->k_pool->data;
+    kp.v_pool = request->v_pool->data;
+    kp.status = state->device_status;
+    kp.total_tokens = r->total_tokens;
+    kp.sessions = (uint32_t)r->sessions;
+    kp.kv_heads = (uint32_t)r->key_value_heads;
+    kp.head_dim = (uint32_t)r->head_dimension;
+    kp.rotary_dim = (uint32_t)r->rotary_dimension;
+    kp.pool_pages = (uint32_t)r->pool_pages;
+    kp.table_stride = (uint32_t)r->page_table_stride;
+    /* a run of n tokens touches at most (n + page - 2) / page + 1 pages */
+    page_slots = (r->max_tokens_per_session + r->page_tokens - 2ull) / r->page_tokens + 1ull;
+    if (page_slots > 0x7fffffffull)
+        return refuse(err, YVEX_ERR_BOUNDS, where, "KV-append geometry exceeds admitted range");
+    variant = r->storage == YVEX_ROCM_KV_BF16 ? YVEX_BACKEND_VARIANT_ROCM_ATTENTION_PAGED_BF16
+                                               : YVEX_BACKEND_VARIANT_ROCM_ATTENTION_PAGED_Q8_0;
+    backend_workspace_reset(backend);
+    rc = yvex_rocm_launch(backend,
+                          r->storage == YVEX_ROCM_KV_BF16 ? YVEX_ROCM_FN_KV_APPEND_BF16
+                                                          : YVEX_ROCM_FN_KV_APPEND_Q8_0,
+                          variant, (unsigned int)page_slots, (unsigned int)r->key_value_heads,
+                          (unsigned int)r->sessions, 64u, 0u, &kp, where, err);
+    if (rc == YVEX_OK) {
+        facts->kernel_launches = 1ull;
+        facts->compulsory_memory_facts_available = 1;
+        rc = yvex_rocm_complete(backend, variant, where, facts, err);
+    }
+    if (rc != YVEX_OK) return rc;
+    request->k_pool->is_written = 1;
+    request->v_pool->is_written = 1;
+    yvex_error_clear(err);
+    return YVEX_OK;
+}
+
 /* ---------------------------------------------------------- op tables ---- */
 
 static const yvex_backend_transformer_operations rocm_transformer_ops = {
@@ -752,6 +852,7 @@ static const yvex_backend_rocm_attention_operations rocm_attention_ops = {
     .paged_decode_execute = rocm_paged_decode_execute,
     .mla_decode_workspace_required = rocm_mla_decode_workspace_required,
     .mla_decode_execute = rocm_mla_decode_execute,
+    .kv_append_execute = rocm_kv_append_execute,
 };
 
 /* A table is published only once the kernel bundle is admitted

@@ -20,6 +20,8 @@ typedef enum {
     YVEX_ROCM_FN_DECODE_PAGED_Q8_0,
     YVEX_ROCM_FN_PREFILL_BF16,
     YVEX_ROCM_FN_MLA_DECODE_BF16,
+    YVEX_ROCM_FN_KV_APPEND_BF16,
+    YVEX_ROCM_FN_KV_APPEND_Q8_0,
     YVEX_ROCM_FN_COUNT
 } yvex_rocm_function_id;
 

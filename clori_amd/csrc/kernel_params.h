@@ -112,4 +112,19 @@ typedef struct {
     float reserved_f;
 } yvex_rocm_mla_params;
 
+/* KV page writer: new key/value rows -> paged pools (bf16 or Q8_0), rotary on the keys. */
+typedef struct {
+    const uint16_t *key, *value;      /* bf16 [total_tokens][kv_heads][head_dim] */
+    const float *cosine, *sine;       /* F32 [total_tokens][rotary_dim]; unused when rotary_dim = 0 */
+    const int32_t *row_start;         /* [sessions] first input row of the session's new tokens */
+    const int32_t *position_start;    /* [sessions] position of its first new token */
+    const int32_t *token_count;       /* [sessions] new tokens (0: nothing to do) */
+    const int32_t *page_table;        /* [sessions][table_stride] */
+    void *k_pool, *v_pool;
+    int32_t *status;
+    uint64_t total_tokens;
+    uint32_t sessions, kv_heads, head_dim, rotary_dim;
+    uint32_t pool_pages, table_stride;
+} yvex_rocm_kv_append_params;
+
 #endif /* YVEX_ROCM_KERNEL_PARAMS_H */

@@ -404,6 +404,29 @@ typedef struct yvex_rocm_mla_decode_request {
     yvex_device_tensor *output, *lse;
 } yvex_rocm_mla_decode_request;
 
+/* KV page writer (no reference counterpart as one operation: it is the rotary step of
+ * src/runtime/decoder.c:1236-1242 fused with the history append of
+ * src/runtime/stateful_attention.c:183-243, writing the paged device layouts).  Session s
+ * contributes token_count[s] consecutive rows of `key` / `value` starting at row_start[s];
+ * they become positions position_start[s] .. of that session.  rotary_dimension = 0 writes
+ * the keys as given; otherwise cosine / sine are F32 [total_tokens][rotary_dimension] tables
+ * indexed by input row (src/backend/cuda/transformer_kernels.cu:79-108). */
+typedef struct yvex_rocm_kv_append_requirement {
+    unsigned long long sessions, total_tokens, max_tokens_per_session;
+    unsigned long long key_value_heads, head_dimension, page_tokens, pool_pages, page_table_stride;
+    unsigned long long rotary_dimension;
+    yvex_rocm_kv_storage storage;
+} yvex_rocm_kv_append_requirement;
+
+typedef struct yvex_rocm_kv_append_request {
+    yvex_rocm_kv_append_requirement requirement;
+    const yvex_device_tensor *key, *value;                /* BF16 [total_tokens][kv_heads][d] */
+    const yvex_device_tensor *cosine, *sine;              /* F32, or NULL without rotary */
+    const yvex_device_tensor *row_start, *position_start, *token_count; /* I32 [sessions] */
+    const yvex_device_tensor *page_table;                 /* I32 [sessions][stride] */
+    yvex_device_tensor *k_pool, *v_pool;
+} yvex_rocm_kv_append_request;
+
 typedef struct yvex_backend_rocm_attention_operations {
     /* attention_execute with an additional F32 [query_tokens][query_heads] LSE output */
     int (*attention_execute_lse)(yvex_backend *, const yvex_transformer_attention_request *,
@@ -417,6 +440,8 @@ typedef struct yvex_backend_rocm_attention_operations {
                                          unsigned long long *, yvex_error *);
     int (*mla_decode_execute)(yvex_backend *, const yvex_rocm_mla_decode_request *,
                               yvex_backend_operation_facts *, yvex_error *);
+    int (*kv_append_execute)(yvex_backend *, const yvex_rocm_kv_append_request *,
+                             yvex_backend_operation_facts *, yvex_error *);
 } yvex_backend_rocm_attention_operations;
 const yvex_backend_rocm_attention_operations *yvex_backend_rocm_attention_operations_get(
     const yvex_backend *backend);

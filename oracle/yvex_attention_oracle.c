@@ -624,3 +624,31 @@ int yvo_lse_merge(const float *part_out, const double *part_lse, uint64_t parts,
     if (lse) *lse = top + log(total);
     return YVO_OK;
 }
+
+/* src/backend/cuda/transformer_kernels.cu:79-108 */
+int yvo_rotary_half_bf16(uint16_t *values, const float *cosines, const float *sines,
+                         uint64_t tokens, uint64_t heads, uint64_t head_dim,
+                         uint64_t rotary_dim)
+{
+    const uint64_t half = rotary_dim / 2u;
+    uint64_t vector, lane;
+    if (!values || !cosines || !sines || !tokens || !heads || !half || rotary_dim > head_dim)
+        return -1;
+    for (vector = 0; vector < tokens * heads; ++vector) {
+        const uint64_t token = vector / heads;
+        uint16_t *base = values + vector * head_dim;
+        for (lane = 0; lane < half; ++lane) {
+            const float cosine = cosines[token * rotary_dim + lane];
+            const float sine = sines[token * rotary_dim + lane];
+            const float first = yvo_bf16_decode(base[lane]);
+            const float second = yvo_bf16_decode(base[half + lane]);
+            float first_product = yvo_bf16_decode(yvo_bf16_encode(first * cosine));
+            float second_product = yvo_bf16_decode(yvo_bf16_encode(second * sine));
+            base[lane] = yvo_bf16_encode(first_product - second_product);
+            first_product = yvo_bf16_decode(yvo_bf16_encode(second * cosine));
+            second_product = yvo_bf16_decode(yvo_bf16_encode(first * sine));
+            base[half + lane] = yvo_bf16_encode(first_product + second_product);
+        }
+    }
+    return 0;
+}

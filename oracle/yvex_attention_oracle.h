@@ -26,6 +26,9 @@
  *   yvo_shared_kv_head               pinned: sink KAT
  *       (tests/reference/deepseek_attention.c:2722-2725); sink=-inf reduces to
  *       yvo_attention_head within 1e-6
+ *   yvo_rotary_half_bf16             pinned: known-answer case
+ *       (tests/unit/cuda/quant_qtype.c:1988-2061), identity, quarter turn,
+ *       float64 rotation within bf16 rounding
  *   yvo_paged_*, yvo_mla_*, yvo_lse_merge
  *       parity unpinned by the reference (it has no page table, no LSE, no
  *       split-K, no Q8_0 KV cache).  Pinned here only by construction
@@ -171,6 +174,21 @@ int yvo_mla_decode_bf16(const uint16_t *q, const uint16_t *pool,
  */
 int yvo_lse_merge(const float *part_out, const double *part_lse, uint64_t parts,
                   uint64_t dim, float *out, double *lse);
+
+/*
+ * Rotate-half position encoding on packed bf16 [tokens][heads][head_dim] vectors in
+ * place, with explicit F32 cos/sin tables [tokens][rotary_dim] (only the first
+ * rotary_dim / 2 entries of a row are used) and every product and sum rounded to bf16:
+ * restates src/backend/cuda/transformer_kernels.cu:79-108 (yvex_rotary_half_f32), whose
+ * F32 values are bf16-representable.  Pinned by the known-answer case the reference's own
+ * GPU test holds (tests/unit/cuda/quant_qtype.c:1988-2061: one 4-wide vector, rotary
+ * dimension 2, untouched suffix), by the identity rotation (cos 1, sin 0), the quarter
+ * turn (cos 0, sin 1: halves swap with one sign flip), norm preservation up to bf16
+ * rounding and a float64 rotation within that rounding.
+ */
+int yvo_rotary_half_bf16(uint16_t *values, const float *cosines, const float *sines,
+                         uint64_t tokens, uint64_t heads, uint64_t head_dim,
+                         uint64_t rotary_dim);
 
 /* Number of worker threads the *_threads arguments are clamped to. */
 int yvo_hardware_threads(void);

@@ -57,6 +57,7 @@ def load_oracle():
     lib.yvo_paged_decode_bf16.argtypes = [u16p, u16p, u16p] + paged
     lib.yvo_paged_decode_q8_0.argtypes = [u16p, u8p, u8p] + paged
     lib.yvo_shared_kv_head.argtypes = [f32p, f32p, C.c_size_t, u64, u64, u64, C.c_double, f32p, f32p, f64p]
+    lib.yvo_rotary_half_bf16.argtypes = [u16p, f32p, f32p] + [u64] * 4
     lib.yvo_mla_decode_bf16.argtypes = [u16p, u16p, i32p, i32p, f32p, u16p, f64p] + [u64] * 7 + [C.c_int]
     lib.yvo_lse_merge.argtypes = [f32p, f64p, u64, u64, f32p, f64p]
     return lib
@@ -199,6 +200,17 @@ class Oracle:
                                          rows.shape[0], key_dim, value_dim, scale,
                                          _ptr(sink_arr, f32p), _ptr(out, f32p), C.byref(lse))
         return rc, out, lse.value
+
+    def rotary_half_bf16(self, values, cosines, sines, rotary_dim):
+        """values uint16 [tokens, heads, d] -> rotated copy (rotate-half, bf16 roundings)."""
+        out = np.ascontiguousarray(values).copy()
+        tokens, heads, d = out.shape
+        cosines = np.ascontiguousarray(cosines, dtype=np.float32)
+        sines = np.ascontiguousarray(sines, dtype=np.float32)
+        rc = self.lib.yvo_rotary_half_bf16(_ptr(out, u16p), _ptr(cosines, f32p), _ptr(sines, f32p),
+                                           tokens, heads, d, rotary_dim)
+        assert rc == 0
+        return out
 
     def mla_decode(self, q, pool, page_table, context, value_dim, page_tokens, threads=None):
         b, h, kd = q.shape

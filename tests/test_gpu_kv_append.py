@@ -1,0 +1,152 @@
+"""GPU parity: the KV page writer (rotary on the keys, bf16 and Q8_0 pages) against the CPU
+restatement, bit for bit, through the C ABI; then decode over the pages it wrote."""
+import numpy as np
+import pytest
+
+from clori_amd import binding as B
+from clori_amd.backend import YvexError, kv_pack_pages, kv_unpack_pages, q8_0_encode_rows
+from gpu_common import ORACLE, assert_close_bf16, assert_lse, backend, bf16_normal  # noqa: F401
+
+pytestmark = pytest.mark.gpu
+
+HKV, D, PAGE = 8, 128, 16
+
+
+def expected_rows(canonical, k_new, v_new, table, starts, counts, row_starts, q8):
+    """Applies the append on the canonical [page][token][head][row] host copy."""
+    k_rows, v_rows = canonical
+    for s in range(len(starts)):
+        for i in range(counts[s]):
+            pos = starts[s] + i
+            page, slot = table[s, pos // PAGE], pos % PAGE
+            for pool, new in ((k_rows, k_new), (v_rows, v_new)):
+                row = new[row_starts[s] + i]
+                pool[page, slot] = q8_0_encode_rows(ORACLE.bf16_decode(row)).reshape(HKV, -1) \
+                    if q8 else row
+    return k_rows, v_rows
+
+
+def run_case(backend, rng, starts, counts, storage, rotary_dim, pool_state="zero"):
+    sessions = len(starts)
+    q8 = storage == B.KV_Q8_0
+    stride = max((s + c + PAGE - 1) // PAGE for s, c in zip(starts, counts)) + 1
+    pool_pages = sessions * stride + 3
+    table = rng.permutation(pool_pages)[:sessions * stride].astype(np.int32).reshape(sessions, stride)
+    total = int(sum(counts))
+    row_starts = np.concatenate([[0], np.cumsum(counts)[:-1]]).astype(np.int32)
+    k_new = bf16_normal(rng, (total, HKV, D))
+    v_new = bf16_normal(rng, (total, HKV, D))
+    angles = rng.uniform(-3.0, 3.0, size=(total, max(rotary_dim, 16))).astype(np.float32)
+    cosine, sine = np.cos(angles).astype(np.float32), np.sin(angles).astype(np.float32)
+    # pools start either zeroed or holding earlier tokens everywhere
+    row_width = (D // 32) * 34 if q8 else D
+    row_dtype = np.uint8 if q8 else np.uint16
+    if pool_state == "zero":
+        k_rows = np.zeros((pool_pages, PAGE, HKV, row_width), row_dtype)
+        v_rows = np.zeros((pool_pages, PAGE, HKV, row_width), row_dtype)
+    else:
+        old_k, old_v = bf16_normal(rng, (pool_pages, PAGE, HKV, D)), bf16_normal(rng, (pool_pages, PAGE, HKV, D))
+        k_rows = q8_0_encode_rows(ORACLE.bf16_decode(old_k)).reshape(pool_pages, PAGE, HKV, -1) if q8 else old_k
+        v_rows = q8_0_encode_rows(ORACLE.bf16_decode(old_v)).reshape(pool_pages, PAGE, HKV, -1) if q8 else old_v
+    pool_dtype = B.DTYPE_I8 if q8 else B.DTYPE_BF16
+    kp, vp = kv_pack_pages(k_rows, storage, False, HKV), kv_pack_pages(v_rows, storage, True, HKV)
+    elems = kp.size // B.DTYPE_BYTES[pool_dtype]
+    t = dict(
+        key=backend.tensor("k-new", B.DTYPE_BF16, k_new.shape, k_new),
+        value=backend.tensor("v-new", B.DTYPE_BF16, v_new.shape, v_new),
+        cosine=backend.tensor("cos", B.DTYPE_F32, cosine.shape, cosine),
+        sine=backend.tensor("sin", B.DTYPE_F32, sine.shape, sine),
+        row_start=backend.tensor("rows", B.DTYPE_I32, (sessions,), row_starts),
+        position_start=backend.tensor("starts", B.DTYPE_I32, (sessions,), np.array(starts, np.int32)),
+        token_count=backend.tensor("counts", B.DTYPE_I32, (sessions,), np.array(counts, np.int32)),
+        page_table=backend.tensor("table", B.DTYPE_I32, table.shape, table),
+        k_pool=backend.tensor("kpool", pool_dtype, (elems,), kp),
+        v_pool=backend.tensor("vpool", pool_dtype, (elems,), vp))
+    use_rotary = rotary_dim > 0
+    facts = backend.kv_append_execute(
+        t["key"], t["value"], t["row_start"], t["position_start"], t["token_count"],
+        t["page_table"], t["k_pool"], t["v_pool"], HKV, pool_pages, max(max(counts), 1),
+        storage=storage, cosine=t["cosine"] if use_rotary else None,
+        sine=t["sine"] if use_rotary else None, rotary_dimension=rotary_dim)
+    assert facts.kernel_launches == 1
+    got_k = kv_unpack_pages(t["k_pool"].read(np.uint8, (-1,)), storage, False, pool_pages, HKV)
+    got_v = kv_unpack_pages(t["v_pool"].read(np.uint8, (-1,)), storage, True, pool_pages, HKV)
+    k_rot = ORACLE.rotary_half_bf16(k_new, cosine[:, :rotary_dim], sine[:, :rotary_dim], rotary_dim) \
+        if use_rotary else k_new
+    want_k, want_v = expected_rows((k_rows.copy(), v_rows.copy()), k_rot, v_new, table, starts,
+                                   counts, row_starts, q8)
+    return t, (got_k, got_v), (want_k, want_v), table, pool_pages
+
+
+@pytest.mark.parametrize("storage", [B.KV_BF16, B.KV_Q8_0], ids=["bf16", "q8_0"])
+@pytest.mark.parametrize("rotary_dim", [0, 64, 128])
+def test_append_writes_exactly_the_host_layout(backend, storage, rotary_dim):
+    """Decode-style (one token) and prefill-style (many tokens, unaligned starts) appends into
+    pools that already hold other tokens: every byte of both pools equals the host-side
+    restatement (rotary, Q8_0 encoder, page packer), untouched tokens included."""
+    rng = np.random.default_rng(11 + rotary_dim)
+    starts, counts = [0, 5, 16, 31, 47, 100], [1, 1, 40, 0, 17, 33]
+    t, got, want, _, _ = run_case(backend, rng, starts, counts, storage, rotary_dim, "filled")
+    assert np.array_equal(got[0].reshape(want[0].shape), want[0])
+    assert np.array_equal(got[1].reshape(want[1].shape), want[1])
+    for x in t.values():
+        x.release()
+
+
+def test_decode_over_appended_pages_matches_cpu_operator(backend):
+    """Prefill-style append of whole contexts, then paged decode on those pages."""
+    rng = np.random.default_rng(21)
+    contexts = [700, 129, 2049]
+    t, got, want, table, pool_pages = run_case(backend, rng, [0, 0, 0], contexts, B.KV_BF16, 128)
+    assert np.array_equal(got[0].reshape(want[0].shape), want[0])
+    q = bf16_normal(rng, (len(contexts), 32, D))
+    ctx = np.array(contexts, np.int32)
+    tq = backend.tensor("q", B.DTYPE_BF16, q.shape, q)
+    tc = backend.tensor("ctx", B.DTYPE_I32, ctx.shape, ctx)
+    out = backend.tensor("o", B.DTYPE_BF16, q.shape)
+    lse = backend.tensor("lse", B.DTYPE_F32, (len(contexts), 32))
+    req = backend.paged_requirement(len(contexts), 32, HKV, D, PAGE, pool_pages, table.shape[1],
+                                    int(table.shape[1] * PAGE), storage=B.KV_BF16)
+    backend.paged_decode_execute(req, tq, t["k_pool"], t["v_pool"], t["page_table"], tc, out, lse)
+    rc, ref, _, ref_lse = ORACLE.paged_decode(q, want[0], want[1], table, ctx, HKV, PAGE)
+    assert rc == 0
+    assert_close_bf16(out.read(), ref, "decode after append")
+    assert_lse(lse.read(), ref_lse, "decode after append")
+
+
+def small_append(backend, k_new, start, count, pool_pages=4):
+    table = np.array([[0, 1]], np.int32)
+    tensors = [
+        backend.tensor("k", B.DTYPE_BF16, k_new.shape, k_new),
+        backend.tensor("v", B.DTYPE_BF16, k_new.shape, k_new),
+        backend.tensor("r", B.DTYPE_I32, (1,), np.array([0], np.int32)),
+        backend.tensor("s", B.DTYPE_I32, (1,), np.array([start], np.int32)),
+        backend.tensor("c", B.DTYPE_I32, (1,), np.array([count], np.int32)),
+        backend.tensor("t", B.DTYPE_I32, table.shape, table),
+        backend.tensor("kp", B.DTYPE_BF16, (pool_pages * HKV * PAGE * D,)),
+        backend.tensor("vp", B.DTYPE_BF16, (pool_pages * HKV * PAGE * D,))]
+    try:
+        return backend.kv_append_execute(*tensors, HKV, pool_pages, count)
+    finally:
+        for x in tensors:
+            x.release()
+
+
+def test_append_refusals(backend):
+    rng = np.random.default_rng(31)
+    # the same call inside the table succeeds
+    small_append(backend, bf16_normal(rng, (4, HKV, D)), 20, 4)
+    # a run that leaves the two-page table: device contract -> BOUNDS
+    with pytest.raises(YvexError) as e:
+        small_append(backend, bf16_normal(rng, (4, HKV, D)), 30, 4)
+    assert e.value.code == B.YVEX_ERR_BOUNDS
+    # a NaN key -> FORMAT
+    k_bad = bf16_normal(rng, (2, HKV, D))
+    k_bad[1, 3, 7] = 0x7FC0
+    with pytest.raises(YvexError) as e:
+        small_append(backend, k_bad, 0, 2)
+    assert e.value.code == B.YVEX_ERR_FORMAT
+    # rotary dimension that is not a multiple of 16 -> UNSUPPORTED (refused on the host)
+    with pytest.raises(YvexError) as e:
+        run_case(backend, rng, [0], [1], B.KV_BF16, 24)
+    assert e.value.code == B.YVEX_ERR_UNSUPPORTED

@@ -409,6 +409,49 @@ def test_paged_and_mla_admission():
         assert e.value.code == B.YVEX_ERR_UNSUPPORTED
 
 
+def test_kv_append_admission():
+    """Refusal order of the page writer: arguments, then geometry the kernels do not cover,
+    then tensor views; one launch, both pools marked written."""
+    with Backend() as b:
+        sessions, total, hkv, pages, stride = 3, 10, 8, 12, 4
+        key = written(b, "k", B.DTYPE_BF16, (total, hkv, 128))
+        value = written(b, "v", B.DTYPE_BF16, (total, hkv, 128))
+        cosine, sine = written(b, "cos", B.DTYPE_F32, (total, 64)), written(b, "sin", B.DTYPE_F32, (total, 64))
+        rows, starts, counts = (written(b, n, B.DTYPE_I32, (sessions,)) for n in ("r", "s", "c"))
+        table = written(b, "t", B.DTYPE_I32, (sessions, stride))
+        k_pool = b.tensor("kp", B.DTYPE_BF16, (pages * hkv * 2048,))
+        v_pool = b.tensor("vp", B.DTYPE_BF16, (pages * hkv * 2048,))
+        args = (key, value, rows, starts, counts, table, k_pool, v_pool, hkv, pages, 8)
+        facts = b.kv_append_execute(*args, cosine=cosine, sine=sine, rotary_dimension=64)
+        assert facts.kernel_launches == 1 and k_pool.is_written and v_pool.is_written
+        q_pool = b.tensor("qp", B.DTYPE_I8, (pages * hkv * 2176,))
+        assert b.kv_append_execute(key, value, rows, starts, counts, table, q_pool, q_pool, hkv,
+                                   pages, 8, storage=B.KV_Q8_0).kernel_launches == 1
+        for kwargs, code in [(dict(head_dimension=64), B.YVEX_ERR_UNSUPPORTED),
+                             (dict(page_tokens=64), B.YVEX_ERR_UNSUPPORTED),
+                             (dict(storage=7), B.YVEX_ERR_UNSUPPORTED),
+                             (dict(rotary_dimension=24, cosine=cosine, sine=sine), B.YVEX_ERR_UNSUPPORTED),
+                             (dict(rotary_dimension=256, cosine=cosine, sine=sine), B.YVEX_ERR_UNSUPPORTED),
+                             (dict(rotary_dimension=64), B.YVEX_ERR_INVALID_ARG),        # no tables
+                             (dict(rotary_dimension=128, cosine=cosine, sine=sine), B.YVEX_ERR_FORMAT)]:
+            with pytest.raises(YvexError) as e:
+                b.kv_append_execute(*args, **kwargs)
+            assert e.value.code == code, kwargs
+        with pytest.raises(YvexError) as e:        # pool one page short
+            b.kv_append_execute(key, value, rows, starts, counts, table, k_pool, v_pool, hkv,
+                                pages + 1, 8)
+        assert e.value.code == B.YVEX_ERR_FORMAT
+        with pytest.raises(YvexError) as e:        # a session cannot hold more rows than exist
+            b.kv_append_execute(key, value, rows, starts, counts, table, k_pool, v_pool, hkv,
+                                pages, total + 1)
+        assert e.value.code == B.YVEX_ERR_INVALID_ARG
+        unwritten = b.tensor("k2", B.DTYPE_BF16, (total, hkv, 128))
+        with pytest.raises(YvexError) as e:
+            b.kv_append_execute(unwritten, value, rows, starts, counts, table, k_pool, v_pool,
+                                hkv, pages, 8)
+        assert e.value.code == B.YVEX_ERR_FORMAT
+
+
 # ------------------------------------------------- failure transitions ----
 
 def test_launch_failure_fails_only_that_variant(env):

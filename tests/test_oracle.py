@@ -472,3 +472,43 @@ def test_lse_merge_is_associative_with_single_pass():
     rc, merged, merged_lse = ORACLE.lse_merge(np.array([full, np.zeros(d, np.float32)]),
                                               np.array([full_lse, -np.inf]))
     assert rc == 0 and np.allclose(merged, full, atol=1e-7) and abs(merged_lse - full_lse) < 1e-12
+
+
+# ------------------------------------------------------------- rotary -------
+
+def test_rotary_reference_known_answer():
+    """tests/unit/cuda/quant_qtype.c:1988-2061: products staged through bf16, the sum
+    rounded again, the non-rotary suffix untouched.  The literals are those products worked
+    by hand: -1.34375*0.63671875 -> -0.85546875, -2.0625*0.546875 -> -1.125, and so on."""
+    values = ORACLE.bf16_encode(np.array([[[-1.34375, -2.0625, 3.0, 4.0]]], np.float32))
+    cosines = np.full((1, 2), 0.63671875, np.float32)
+    sines = np.full((1, 2), 0.546875, np.float32)
+    got = ORACLE.bf16_decode(ORACLE.rotary_half_bf16(values, cosines, sines, 2))
+    assert got.tolist() == [[[0.26953125, -2.046875, 3.0, 4.0]]]
+
+
+def test_rotary_closed_forms():
+    rng = np.random.default_rng(44)
+    tokens, heads, d = 5, 3, 128
+    x = ORACLE.bf16_encode(rng.standard_normal((tokens, heads, d)).astype(np.float32))
+    xf = ORACLE.bf16_decode(x)
+    for rotary in (32, 64, 128):
+        half = rotary // 2
+        one, zero = np.ones((tokens, rotary), np.float32), np.zeros((tokens, rotary), np.float32)
+        assert np.array_equal(ORACLE.rotary_half_bf16(x, one, zero, rotary), x)
+        quarter = ORACLE.bf16_decode(ORACLE.rotary_half_bf16(x, zero, one, rotary))
+        assert np.array_equal(quarter[..., :half], -xf[..., half:rotary])
+        assert np.array_equal(quarter[..., half:rotary], xf[..., :half])
+        assert np.array_equal(quarter[..., rotary:], xf[..., rotary:])
+        # per-token angles: float64 rotation within bf16 rounding, norms kept; the second
+        # half of each table row is never read
+        angles = rng.uniform(-3.0, 3.0, (tokens, rotary))
+        angles[:, half:] = np.nan
+        cosines, sines = np.cos(angles).astype(np.float32), np.sin(angles).astype(np.float32)
+        got = ORACLE.bf16_decode(ORACLE.rotary_half_bf16(x, cosines, sines, rotary)).astype(np.float64)
+        c, s = np.cos(angles[:, None, :half]), np.sin(angles[:, None, :half])
+        a, b = xf[..., :half].astype(np.float64), xf[..., half:rotary].astype(np.float64)
+        want = np.concatenate([a * c - b * s, b * c + a * s, xf[..., rotary:]], axis=-1)
+        assert np.all(np.isfinite(got))
+        assert np.max(np.abs(got - want)) < 3 * 2.0 ** -8 * np.max(np.abs(xf))
+        assert np.allclose(np.linalg.norm(got, axis=-1), np.linalg.norm(xf, axis=-1), rtol=5e-3)
