@@ -825,8 +825,11 @@ static int rocm_kv_append_execute(yvex_backend *backend, const yvex_rocm_kv_appe
     rc = yvex_rocm_launch(backend,
                           r->storage == YVEX_ROCM_KV_BF16 ? YVEX_ROCM_FN_KV_APPEND_BF16
                                                           : YVEX_ROCM_FN_KV_APPEND_Q8_0,
-                          variant, (unsigned int)page_slots, (unsigned int)r->key_value_heads,
-                          (unsigned int)r->sessions, 64u, 0u, &kp, where, err);
+                          variant, (unsigned int)page_slots,
+                          (unsigned int)((r->key_value_heads + YVEX_ROCM_KV_APPEND_HEADS - 1ull) /
+                                         YVEX_ROCM_KV_APPEND_HEADS),
+                          (unsigned int)r->sessions, 64u * YVEX_ROCM_KV_APPEND_HEADS, 0u, &kp, where,
+                          err);
     if (rc == YVEX_OK) {
         facts->kernel_launches = 1ull;
         facts->compulsory_memory_facts_available = 1;

@@ -112,7 +112,9 @@ typedef struct {
     float reserved_f;
 } yvex_rocm_mla_params;
 
-/* KV page writer: new key/value rows -> paged pools (bf16 or Q8_0), rotary on the keys. */
+/* KV page writer: new key/value rows -> paged pools (bf16 or Q8_0), rotary on the keys.
+ * A workgroup is YVEX_ROCM_KV_APPEND_HEADS waves, one kv head each. */
+#define YVEX_ROCM_KV_APPEND_HEADS 4
 typedef struct {
     const uint16_t *key, *value;      /* bf16 [total_tokens][kv_heads][head_dim] */
     const float *cosine, *sine;       /* F32 [total_tokens][rotary_dim]; unused when rotary_dim = 0 */

@@ -5,9 +5,15 @@
 // (src/runtime/decoder.c:1236-1242 rotary, src/runtime/stateful_attention.c:183-243 append).
 //
 // One wave owns one (session, touched page, kv head): it reads up to 16 rows of 256 bytes,
-// and writes one 4096-byte (bf16) or 2176-byte (Q8_0) block per pool.  A page that is only
-// partly covered by the new tokens keeps its other tokens (read-modify-write inside the
-// wave; sessions never share a page).
+// and writes one 4096-byte (bf16) or 2176-byte (Q8_0) block per pool; a workgroup is four
+// such waves (four kv heads of one page).  Every global load of a wave is issued before the
+// first result is used.  A page that is only partly covered by the new tokens keeps its
+// other tokens (read-modify-write inside the wave; sessions never share a page).
+//
+// Keys are handled as 16-byte chunks (token t, dims 8*c8 .. 8*c8+7).  With rotary dimension
+// R the chunks c8 < R/16 are the lower half, R/16 <= c8 < R/8 the upper half, the rest are
+// copied.  The lane of a lower chunk loads its partner chunk and one cos and one sin piece
+// and produces both rotated chunks; the lanes of upper chunks load and compute nothing.
 //
 // Rotary (src/backend/cuda/transformer_kernels.cu:79-108): with half = rotary_dim / 2 and
 // c < half, first = k[c], second = k[c + half], cosine/sine = table[row][c]:
@@ -30,11 +36,31 @@ namespace {
 
 constexpr int kHeadDim = 128;
 constexpr int kPageTokens = 16;
+constexpr int kWaves = YVEX_ROCM_KV_APPEND_HEADS;
+constexpr int kRowPitch = kHeadDim + 8;       // bf16 elements per LDS row (272 bytes)
+constexpr int kCodePitch = kHeadDim + 16;     // bytes per LDS row of value codes
 
 __device__ inline void flag(int32_t *status, int code) { atomicCAS(status, 0, code); }
 
-// bf16 bits of a float with the reference's rounding; inputs here are finite or flagged
-__device__ inline float round_bf16(float v) { return bf16_to_f32(bf16_bits(v)); }
+__device__ inline float bf16_of(const u32x4 &w, int i)
+{
+    const uint32_t word = w[i >> 1];
+    return __builtin_bit_cast(float, (i & 1) ? word & 0xffff0000u : word << 16);
+}
+
+// the two bf16 values of a packed word as floats
+__device__ inline float low_half(uint32_t w) { return __builtin_bit_cast(float, w << 16); }
+__device__ inline float high_half(uint32_t w) { return __builtin_bit_cast(float, w & 0xffff0000u); }
+
+// true when none of the eight bf16 values is an infinity or a NaN
+__device__ inline bool finite_bits(const u32x4 &w)
+{
+    bool ok = true;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+        ok &= (w[j] & 0x7f80u) != 0x7f80u && (w[j] & 0x7f800000u) != 0x7f800000u;
+    return ok;
+}
 
 struct Span {
     uint32_t page_id;   // pool page
@@ -48,6 +74,10 @@ __device__ inline Span locate(const yvex_rocm_kv_append_params &p)
 {
     Span s;
     s.valid = false;
+    s.page_id = 0u;
+    s.lo = 0u;
+    s.hi = 1u;
+    s.row = 0u;
     const uint32_t session = blockIdx.z, slot = blockIdx.x;
     const int32_t count = p.token_count[session], start = p.position_start[session];
     const int32_t row0 = p.row_start[session];
@@ -76,168 +106,282 @@ __device__ inline Span locate(const yvex_rocm_kv_append_params &p)
     return s;
 }
 
-// Eight consecutive dims [c0, c0+8) of input row `row`, kv head `head`, as floats; keys get
-// the rotary applied.  Returns false when a value is not finite.
-__device__ inline bool load_eight(const yvex_rocm_kv_append_params &p, const uint16_t *src,
-                                  uint32_t row, uint32_t head, uint32_t c0, bool rotate,
-                                  float (&out)[8])
+// Input row that lands in token slot t; slots outside [lo, hi) read a neighbouring row of the
+// span (the value is loaded and dropped) so that loads need no branches.
+__device__ inline uint32_t row_of(const Span &s, uint32_t t)
 {
-    const uint16_t *base = src + ((uint64_t)row * p.kv_heads + head) * kHeadDim;
-    const u32x4 own = load_b128(base + c0);
-    bool ok = true;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        out[2 * i + 0] = bf16_to_f32((uint16_t)(own[i] & 0xffffu));
-        out[2 * i + 1] = bf16_to_f32((uint16_t)(own[i] >> 16));
+    return s.row + (min(max(t, s.lo), s.hi - 1u) - s.lo);
+}
+
+enum Role { kLower, kUpper, kPlain };
+
+// One key chunk in flight: raw loads first, arithmetic later.
+struct KeyChunk {
+    u32x4 own, other, cs[2], sn[2];
+    uint32_t t, c8;
+    int role;
+};
+
+__device__ inline void key_issue(const yvex_rocm_kv_append_params &p, const Span &s, uint32_t head,
+                                 uint32_t id, KeyChunk &k)
+{
+    const uint32_t pairs = p.rotary_dim / 16u;   // chunks in each rotary half
+    k.t = id & 15u;
+    k.c8 = id >> 4;
+    k.role = k.c8 < pairs ? kLower : k.c8 < 2u * pairs ? kUpper : kPlain;
+    const uint32_t row = row_of(s, k.t);
+    const uint16_t *base = p.key + ((uint64_t)row * p.kv_heads + head) * kHeadDim + k.c8 * 8u;
+    if (k.role != kUpper) k.own = load_b128(base);
+    if (k.role == kLower) {
+        const uint64_t at = (uint64_t)row * p.rotary_dim + k.c8 * 8u;
+        k.other = load_b128(base + p.rotary_dim / 2u);
+        k.cs[0] = load_b128(p.cosine + at);
+        k.cs[1] = load_b128(p.cosine + at + 4);
+        k.sn[0] = load_b128(p.sine + at);
+        k.sn[1] = load_b128(p.sine + at + 4);
     }
-    if (rotate && c0 < p.rotary_dim) {
-        const uint32_t half = p.rotary_dim / 2u;
-        const bool upper = c0 >= half;
-        const uint32_t partner_c = upper ? c0 - half : c0 + half, table_c = upper ? c0 - half : c0;
-        const u32x4 other = load_b128(base + partner_c);
-        const float *cs = p.cosine + (uint64_t)row * p.rotary_dim + table_c;
-        const float *sn = p.sine + (uint64_t)row * p.rotary_dim + table_c;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const uint32_t word = other[i >> 1];
-            const float partner = bf16_to_f32((uint16_t)((i & 1) ? word >> 16 : word & 0xffffu));
-            const float cosine = cs[i], sine = sn[i];
-            ok &= isfinite(cosine) && isfinite(sine);
-            // lower half: first = own, second = partner; upper half: first = partner, second = own
-            const float a = round_bf16(out[i] * cosine);
-            const float b = round_bf16(partner * sine);
-            out[i] = round_bf16(upper ? a + b : a - b);
-        }
+}
+
+// Rotated (or copied) chunk(s) as packed bf16; `upper` is produced by lower-half lanes only.
+// Returns false when a table entry, an input or a result is not finite.
+__device__ inline bool key_finish(const KeyChunk &k, u32x4 &lower, u32x4 &upper)
+{
+    if (k.role == kUpper) return true;
+    if (k.role == kPlain) {
+        lower = k.own;
+        return finite_bits(k.own);
     }
+    // Two dims at a time; v_cvt_pk_bf16_f32 rounds to nearest even exactly as the reference
+    // codec does for every finite value and for overflow.  A non-finite table entry or input
+    // always leaves a non-finite result (inf * 0 and inf - inf are NaN), so checking the
+    // results covers all of them.
 #pragma unroll
-    for (int i = 0; i < 8; ++i) ok &= isfinite(out[i]);
-    return ok;
+    for (int j = 0; j < 4; ++j) {
+        const float first0 = bf16_of(k.own, 2 * j), first1 = bf16_of(k.own, 2 * j + 1);
+        const float second0 = bf16_of(k.other, 2 * j), second1 = bf16_of(k.other, 2 * j + 1);
+        const uint32_t c0 = k.cs[j >> 1][(2 * j) & 3], c1 = k.cs[j >> 1][(2 * j + 1) & 3];
+        const uint32_t s0 = k.sn[j >> 1][(2 * j) & 3], s1 = k.sn[j >> 1][(2 * j + 1) & 3];
+        const float cosine0 = __builtin_bit_cast(float, c0), cosine1 = __builtin_bit_cast(float, c1);
+        const float sine0 = __builtin_bit_cast(float, s0), sine1 = __builtin_bit_cast(float, s1);
+        const uint32_t fc = pack_bf16x2(first0 * cosine0, first1 * cosine1);
+        const uint32_t ss = pack_bf16x2(second0 * sine0, second1 * sine1);
+        const uint32_t sc = pack_bf16x2(second0 * cosine0, second1 * cosine1);
+        const uint32_t fs = pack_bf16x2(first0 * sine0, first1 * sine1);
+        lower[j] = pack_bf16x2(low_half(fc) - low_half(ss), high_half(fc) - high_half(ss));
+        upper[j] = pack_bf16x2(low_half(sc) + low_half(fs), high_half(sc) + high_half(fs));
+    }
+    return finite_bits(lower) && finite_bits(upper);
 }
 
 }  // namespace
 
-// grid = (pages a session can touch, kv heads, sessions), block 64.
-extern "C" __global__ void __launch_bounds__(64)
+// grid = (pages a session can touch, kv heads / 4, sessions), block 256: wave w writes kv head
+// 4 * blockIdx.y + w.
+extern "C" __global__ void __launch_bounds__(64 * kWaves)
 yvex_rocm_kv_append_bf16(const yvex_rocm_kv_append_params p)
 {
-    __shared__ uint16_t v_rows[kPageTokens][kHeadDim + 8];
+    __shared__ __attribute__((aligned(16))) uint16_t v_rows_all[kWaves][kPageTokens][kRowPitch];
     const Span s = locate(p);
-    if (!s.valid) return;
-    const uint32_t lane = threadIdx.x, head = blockIdx.y;
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const uint32_t head = blockIdx.y * kWaves + wave;
+    const bool active = s.valid && head < p.kv_heads;
+    uint16_t (*v_rows)[kRowPitch] = v_rows_all[wave];
     const uint64_t block = ((uint64_t)s.page_id * p.kv_heads + head) * (kPageTokens * kHeadDim);
     uint16_t *kdst = (uint16_t *)p.k_pool + block, *vdst = (uint16_t *)p.v_pool + block;
+    const bool partial = s.lo != 0u || s.hi != (uint32_t)kPageTokens;
+    const uint32_t pairs = p.rotary_dim / 16u;
     bool ok = true;
-    // keys: 256 chunks of 8 dims, chunk id = c8 * 16 + t is also its place in the block
+    KeyChunk k[4];
+    u32x4 v[4], old[4] = {};
+    if (active) {
+        // every load of the wave, then the arithmetic
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const uint32_t id = lane + 64u * i, t = id & 15u, c8 = id >> 4;
-        if (t < s.lo || t >= s.hi) continue;
-        float k[8];
-        ok &= load_eight(p, p.key, s.row + (t - s.lo), head, c8 * 8u, p.rotary_dim != 0u, k);
-        u32x4 w;
+        for (int i = 0; i < 4; ++i) key_issue(p, s, head, lane + 64u * i, k[i]);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) w[j] = (uint32_t)bf16_bits(k[2 * j]) | ((uint32_t)bf16_bits(k[2 * j + 1]) << 16);
-        *reinterpret_cast<u32x4 *>(kdst + id * 8u) = w;
-    }
-    // values: through LDS, then 8 tokens of one dim per 16-byte piece
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t id = lane + 64u * i, t = id >> 4, c8 = id & 15u;
+            v[i] = load_b128(p.value + ((uint64_t)row_of(s, t) * p.kv_heads + head) * kHeadDim + c8 * 8u);
+        }
+        if (partial) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const uint32_t id = lane + 64u * i, t = id >> 4, c8 = id & 15u;
-        if (t < s.lo || t >= s.hi) continue;
-        float v[8];
-        ok &= load_eight(p, p.value, s.row + (t - s.lo), head, c8 * 8u, false, v);
+            for (int i = 0; i < 4; ++i) old[i] = load_b128(vdst + (lane + 64u * i) * 8u);
+        }
+        // keys: chunk (c8, t) sits at 16-byte slot c8 * 16 + t of the block
 #pragma unroll
-        for (int j = 0; j < 8; ++j) v_rows[t][c8 * 8u + j] = bf16_bits(v[j]);
+        for (int i = 0; i < 4; ++i) {
+            u32x4 lower, upper;
+            ok &= key_finish(k[i], lower, upper);
+            if (k[i].t < s.lo || k[i].t >= s.hi) continue;
+            if (k[i].role != kUpper)
+                *reinterpret_cast<u32x4 *>(kdst + (k[i].c8 * 16u + k[i].t) * 8u) = lower;
+            if (k[i].role == kLower)
+                *reinterpret_cast<u32x4 *>(kdst + ((k[i].c8 + pairs) * 16u + k[i].t) * 8u) = upper;
+        }
+        // values: rows into LDS, then 8 tokens of one dim per 16-byte piece
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t id = lane + 64u * i, t = id >> 4, c8 = id & 15u;
+            if (t >= s.lo && t < s.hi) ok &= finite_bits(v[i]);
+            *reinterpret_cast<u32x4 *>(&v_rows[t][c8 * 8u]) = v[i];
+        }
     }
     __syncthreads();
+    if (active) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const uint32_t id = lane + 64u * i, c = id >> 1, t8 = (id & 1u) * 8u;
-        if (t8 + 8u <= s.lo || t8 >= s.hi) continue;
-        u32x4 w = *reinterpret_cast<const u32x4 *>(vdst + c * 16u + t8);  // tokens that stay
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t id = lane + 64u * i, c = id >> 1, t8 = (id & 1u) * 8u;
+            if (t8 + 8u <= s.lo || t8 >= s.hi) continue;
+            u32x4 w;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            const uint32_t t = t8 + j;
-            if (t < s.lo || t >= s.hi) continue;
-            const uint32_t bits = v_rows[t][c];
-            w[j >> 1] = (j & 1) ? (w[j >> 1] & 0x0000ffffu) | (bits << 16)
-                                : (w[j >> 1] & 0xffff0000u) | bits;
+            for (int j = 0; j < 4; ++j)
+                w[j] = (uint32_t)v_rows[t8 + 2 * j][c] | ((uint32_t)v_rows[t8 + 2 * j + 1][c] << 16);
+            if (partial) {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const uint32_t t = t8 + j, mask = (j & 1) ? 0xffff0000u : 0x0000ffffu;
+                    if (t < s.lo || t >= s.hi) w[j >> 1] = (w[j >> 1] & ~mask) | (old[i][j >> 1] & mask);
+                }
+            }
+            *reinterpret_cast<u32x4 *>(vdst + id * 8u) = w;
         }
-        *reinterpret_cast<u32x4 *>(vdst + c * 16u + t8) = w;
+        if (!ok) flag(p.status, YVEX_ROCM_DEVICE_NUMERIC);
     }
-    if (!ok) flag(p.status, YVEX_ROCM_DEVICE_NUMERIC);
 }
 
-// grid as above.  Lane (t = lane / 4, j = lane % 4) owns the 32 dims of Q8_0 block j of token t.
-extern "C" __global__ void __launch_bounds__(64)
+namespace {
+
+// Q8_0 block of 32 values: f16 scale bits and 32 codes packed four to a word.
+__device__ inline bool quantise(const float (&x)[32], uint16_t &scale_bits, uint32_t (&codes)[8])
+{
+    float maximum = 0.f;
+#pragma unroll
+    for (int e = 0; e < 32; ++e) maximum = fmaxf(maximum, fabsf(x[e]));
+    const _Float16 half = (_Float16)(maximum / 127.0f);
+    const float scale = (float)half;
+    const float inverse = scale != 0.f ? 1.0f / scale : 0.f;
+    scale_bits = __builtin_bit_cast(uint16_t, half);
+#pragma unroll
+    for (int w = 0; w < 8; ++w) {
+        uint32_t word = 0u;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const float scaled = roundf(x[4 * w + e] * inverse);
+            const int code = scaled < -127.f ? -127 : scaled > 127.f ? 127 : (int)scaled;
+            word |= ((uint32_t)code & 0xffu) << (8 * e);
+        }
+        codes[w] = word;
+    }
+    return isfinite(scale) && !(maximum > 0.f && scale == 0.f);
+}
+
+}  // namespace
+
+// grid and waves as above.  After the rotary, lane (t = lane / 4, j = lane % 4) owns the 32
+// dims of Q8_0 block j of token t.
+extern "C" __global__ void __launch_bounds__(64 * kWaves)
 yvex_rocm_kv_append_q8_0(const yvex_rocm_kv_append_params p)
 {
-    __shared__ unsigned char v_codes[kPageTokens][kHeadDim + 16];
+    __shared__ __attribute__((aligned(16))) uint16_t k_rows_all[kWaves][kPageTokens][kRowPitch];
+    __shared__ __attribute__((aligned(16))) unsigned char v_codes_all[kWaves][kPageTokens][kCodePitch];
     const Span s = locate(p);
-    if (!s.valid) return;
-    const uint32_t lane = threadIdx.x, head = blockIdx.y;
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const uint32_t head = blockIdx.y * kWaves + wave;
+    const bool active = s.valid && head < p.kv_heads;
+    uint16_t (*k_rows)[kRowPitch] = k_rows_all[wave];
+    unsigned char (*v_codes)[kCodePitch] = v_codes_all[wave];
     const uint32_t t = lane >> 2, j = lane & 3u;
-    constexpr uint32_t kBlockBytes = kPageTokens * kHeadDim + kPageTokens * 4 * 2;
+    constexpr uint32_t kCodeBytes = kPageTokens * kHeadDim;
+    constexpr uint32_t kBlockBytes = kCodeBytes + kPageTokens * 4 * 2;
     const uint64_t block = ((uint64_t)s.page_id * p.kv_heads + head) * kBlockBytes;
     unsigned char *kdst = (unsigned char *)p.k_pool + block, *vdst = (unsigned char *)p.v_pool + block;
+    const bool partial = s.lo != 0u || s.hi != (uint32_t)kPageTokens;
     const bool mine = t >= s.lo && t < s.hi;
+    const uint32_t pairs = p.rotary_dim / 16u;
     bool ok = true, representable = true;
+    KeyChunk k[4];
+    u32x4 v[4];
+    uint32_t old[8] = {0u, 0u, 0u, 0u, 0u, 0u, 0u, 0u};
+    if (active) {
 #pragma unroll
-    for (int pool = 0; pool < 2; ++pool) {
-        if (!mine) continue;
-        const uint16_t *src = pool == 0 ? p.key : p.value;
-        float x[32];
-        float maximum = 0.f;
+        for (int i = 0; i < 4; ++i) key_issue(p, s, head, lane + 64u * i, k[i]);
+        {
+            const uint16_t *src = p.value + ((uint64_t)row_of(s, t) * p.kv_heads + head) * kHeadDim + 32u * j;
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-            float part[8];
-            ok &= load_eight(p, src, s.row + (t - s.lo), head, 32u * j + 8u * g,
-                             pool == 0 && p.rotary_dim != 0u, part);
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                x[8 * g + e] = part[e];
-                maximum = fmaxf(maximum, fabsf(part[e]));
-            }
+            for (int g = 0; g < 4; ++g) v[g] = load_b128(src + 8 * g);
         }
-        const _Float16 half = (_Float16)(maximum / 127.0f);
-        const float scale = (float)half;
-        representable &= isfinite(scale) && !(maximum > 0.f && scale == 0.f);
-        const float inverse = scale != 0.f ? 1.0f / scale : 0.f;
-        unsigned char *dst = pool == 0 ? kdst : vdst;
-        *reinterpret_cast<uint16_t *>(dst + kPageTokens * kHeadDim + (t * 4u + j) * 2u) =
-            __builtin_bit_cast(uint16_t, half);
+        if (partial) {
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-            uint32_t packed[2] = {0u, 0u};
+            for (int i = 0; i < 8; ++i)
+                old[i] = *reinterpret_cast<const uint32_t *>(vdst + (lane + 64u * i) * 4u);
+        }
+        // rotated key rows into LDS
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const float scaled = roundf(x[8 * g + e] * inverse);
-                const int code = scaled < -127.f ? -127 : scaled > 127.f ? 127 : (int)scaled;
-                packed[e >> 2] |= ((uint32_t)code & 0xffu) << (8 * (e & 3));
-                if (pool == 1) v_codes[t][32u * j + 8u * g + e] = (unsigned char)code;
+        for (int i = 0; i < 4; ++i) {
+            u32x4 lower, upper;
+            ok &= key_finish(k[i], lower, upper) || k[i].t < s.lo || k[i].t >= s.hi;
+            if (k[i].role != kUpper)
+                *reinterpret_cast<u32x4 *>(&k_rows[k[i].t][k[i].c8 * 8u]) = lower;
+            if (k[i].role == kLower)
+                *reinterpret_cast<u32x4 *>(&k_rows[k[i].t][(k[i].c8 + pairs) * 8u]) = upper;
+        }
+        // values: quantise this lane's block, codes into LDS, scale straight to the pool
+        if (mine) {
+            float x[32];
+            uint32_t codes[8];
+            uint16_t scale_bits;
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                ok &= finite_bits(v[g]);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) x[8 * g + e] = bf16_of(v[g], e);
             }
-            if (pool == 0) {
-                u32x2 w = {packed[0], packed[1]};
-                *reinterpret_cast<u32x2 *>(kdst + (((g * 16u + t) * 4u + j) * 8u)) = w;
+            representable &= quantise(x, scale_bits, codes);
+            *reinterpret_cast<uint16_t *>(vdst + kCodeBytes + (t * 4u + j) * 2u) = scale_bits;
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const u32x2 w = {codes[2 * g], codes[2 * g + 1]};
+                *reinterpret_cast<u32x2 *>(&v_codes[t][32u * j + 8u * g]) = w;
             }
         }
     }
     __syncthreads();
-    // value codes: 4-byte groups (4 tokens of one dim) at ((tg*16 + m)*8 + b)*4, c = 16b + m
+    if (active) {
+        if (mine) {
+            float x[32];
+            uint32_t codes[8];
+            uint16_t scale_bits;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        const uint32_t id = lane + 64u * i;  // 512 groups = tg (4) x m (16) x b (8)
-        const uint32_t b = id & 7u, m = (id >> 3) & 15u, tg = id >> 7, c = 16u * b + m;
-        if (4u * tg + 4u <= s.lo || 4u * tg >= s.hi) continue;
-        uint32_t w = *reinterpret_cast<const uint32_t *>(vdst + id * 4u);  // tokens that stay
+            for (int g = 0; g < 4; ++g) {
+                const u32x4 w = *reinterpret_cast<const u32x4 *>(&k_rows[t][32u * j + 8u * g]);
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            const uint32_t tt = 4u * tg + q;
-            if (tt < s.lo || tt >= s.hi) continue;
-            w = (w & ~(0xffu << (8 * q))) | ((uint32_t)v_codes[tt][c] << (8 * q));
+                for (int e = 0; e < 8; ++e) x[8 * g + e] = bf16_of(w, e);
+            }
+            representable &= quantise(x, scale_bits, codes);
+            *reinterpret_cast<uint16_t *>(kdst + kCodeBytes + (t * 4u + j) * 2u) = scale_bits;
+            // key codes: 8-byte groups at ((g * 16 + t) * 4 + j) * 8, dims 32j + 8g + e
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const u32x2 w = {codes[2 * g], codes[2 * g + 1]};
+                *reinterpret_cast<u32x2 *>(kdst + ((g * 16u + t) * 4u + j) * 8u) = w;
+            }
         }
-        *reinterpret_cast<uint32_t *>(vdst + id * 4u) = w;
+        // value codes: 4-byte groups (4 tokens of one dim) at ((tg*16 + m)*8 + b)*4, c = 16b + m
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const uint32_t id = lane + 64u * i;  // 512 groups = tg (4) x m (16) x b (8)
+            const uint32_t b = id & 7u, m = (id >> 3) & 15u, tg = id >> 7, c = 16u * b + m;
+            if (4u * tg + 4u <= s.lo || 4u * tg >= s.hi) continue;
+            uint32_t w = 0u;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const uint32_t tt = 4u * tg + q;
+                const bool fresh = tt >= s.lo && tt < s.hi;
+                const uint32_t byte = fresh ? (uint32_t)v_codes[tt][c] : (old[i] >> (8 * q)) & 0xffu;
+                w |= byte << (8 * q);
+            }
+            *reinterpret_cast<uint32_t *>(vdst + id * 4u) = w;
+        }
+        if (!ok) flag(p.status, YVEX_ROCM_DEVICE_NUMERIC);
+        if (!representable) flag(p.status, YVEX_ROCM_DEVICE_CONTRACT);
     }
-    if (!ok) flag(p.status, YVEX_ROCM_DEVICE_NUMERIC);
-    if (!representable) flag(p.status, YVEX_ROCM_DEVICE_CONTRACT);
 }
