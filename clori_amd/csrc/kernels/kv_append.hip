@@ -253,6 +253,7 @@ namespace {
 // Q8_0 block of 32 values: f16 scale bits and 32 codes packed four to a word.
 __device__ inline bool quantise(const float (&x)[32], uint16_t &scale_bits, uint32_t (&codes)[8])
 {
+#pragma clang fp contract(off)   // the product is rounded before the rounding add, as in the reference
     float maximum = 0.f;
 #pragma unroll
     for (int e = 0; e < 32; ++e) maximum = fmaxf(maximum, fabsf(x[e]));
@@ -260,13 +261,17 @@ __device__ inline bool quantise(const float (&x)[32], uint16_t &scale_bits, uint
     const float scale = (float)half;
     const float inverse = scale != 0.f ? 1.0f / scale : 0.f;
     scale_bits = __builtin_bit_cast(uint16_t, half);
+    // roundf (half away from zero) as a truncating convert of x + copysign(0.5 - 2^-25, x):
+    // exact for |x| < 2^23 (ties land on or above the next integer, the value just below a
+    // tie stays below it), then the clamp on the integer
+    const float nudge = __builtin_bit_cast(float, 0x3effffffu);
 #pragma unroll
     for (int w = 0; w < 8; ++w) {
         uint32_t word = 0u;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-            const float scaled = roundf(x[4 * w + e] * inverse);
-            const int code = scaled < -127.f ? -127 : scaled > 127.f ? 127 : (int)scaled;
+            const float scaled = x[4 * w + e] * inverse;
+            const int code = min(max((int)(scaled + copysignf(nudge, scaled)), -127), 127);
             word |= ((uint32_t)code & 0xffu) << (8 * e);
         }
         codes[w] = word;

@@ -132,6 +132,43 @@ def small_append(backend, k_new, start, count, pool_pages=4):
             x.release()
 
 
+def test_q8_0_ties_round_half_away_from_zero(backend):
+    """Blocks whose scale is exactly 1 and whose values sit on k + 0.5: the reference encoder
+    rounds them away from zero (roundf); also the largest magnitudes and signed zeros."""
+    ladder = np.array([127.0] + [k + 0.5 for k in range(0, 31)], np.float32)
+    rows = np.zeros((3, HKV, D), np.float32)
+    for h in range(HKV):
+        rows[0, h] = np.tile(ladder, 4) * np.where(np.arange(D) % 3 == h % 3, -1.0, 1.0)
+        rows[1, h] = np.tile(np.array([127.0, 126.5, -126.5, 125.5, -0.0, 0.0, 63.5, -64.5] * 4,
+                                      np.float32), 4)
+        rows[2, h] = np.tile(ladder[::-1], 4) * 2.0 ** (h - 4)      # other exact scales
+    new = ORACLE.bf16_encode(rows)
+    assert np.array_equal(ORACLE.bf16_decode(new), rows)            # all bf16-representable
+    table = np.array([[1, 0]], np.int32)
+    pool_bytes = 2 * HKV * 2176
+    tensors = [backend.tensor("k", B.DTYPE_BF16, new.shape, new),
+               backend.tensor("v", B.DTYPE_BF16, new.shape, new[::-1].copy()),
+               backend.tensor("r", B.DTYPE_I32, (1,), np.array([0], np.int32)),
+               backend.tensor("s", B.DTYPE_I32, (1,), np.array([14], np.int32)),
+               backend.tensor("c", B.DTYPE_I32, (1,), np.array([3], np.int32)),
+               backend.tensor("t", B.DTYPE_I32, table.shape, table),
+               backend.tensor("kp", B.DTYPE_I8, (pool_bytes,)),
+               backend.tensor("vp", B.DTYPE_I8, (pool_bytes,))]
+    tensors[6].zero()
+    tensors[7].zero()
+    backend.kv_append_execute(*tensors, HKV, 2, 3, storage=B.KV_Q8_0)
+    want = q8_0_encode_rows(rows).reshape(3, HKV, -1)
+    for pool, rows_in in ((tensors[6], want), (tensors[7], want[::-1])):
+        got = kv_unpack_pages(pool.read(np.uint8, (-1,)), B.KV_Q8_0, False if pool is tensors[6] else True,
+                              2, HKV).reshape(2, PAGE, HKV, -1)
+        # positions 14, 15 -> page id 1 slots 14, 15; position 16 -> page id 0 slot 0
+        assert np.array_equal(got[1, 14], rows_in[0])
+        assert np.array_equal(got[1, 15], rows_in[1])
+        assert np.array_equal(got[0, 0], rows_in[2])
+    for x in tensors:
+        x.release()
+
+
 def test_append_refusals(backend):
     rng = np.random.default_rng(31)
     # the same call inside the table succeeds
