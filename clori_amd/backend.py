@@ -264,14 +264,19 @@ class Backend:
                err)
         return out.value
 
-    def attention_execute(self, requirement, query, key, value, output, lse=None):
+    def attention_execute(self, requirement, query, key, value, output, lse=None, gate=None):
         ops = self.transformer_operations()
         if ops is None:
             raise YvexError(B.YVEX_ERR_UNSUPPORTED, "transformer_operations", "not published")
         request = B.AttentionRequest(requirement, query.handle, key.handle, value.handle,
                                      output.handle)
         facts, err = B.OperationFacts(), B.Error()
-        if lse is None:
+        if gate is not None:
+            epilogue = B.AttentionEpilogue(gate.handle)
+            rc = self.rocm_attention_operations().attention_execute_fused(
+                self.handle, C.byref(request), C.byref(epilogue), lse.handle if lse else None,
+                C.byref(facts), C.byref(err))
+        elif lse is None:
             rc = ops.attention_execute(self.handle, C.byref(request), C.byref(facts), C.byref(err))
         else:
             rocm = self.rocm_attention_operations()
@@ -299,7 +304,7 @@ class Backend:
         return out.value
 
     def paged_decode_execute(self, requirement, query, key_pages, value_pages, page_table,
-                             context, output, lse=None):
+                             context, output, lse=None, gate=None):
         ops = self.rocm_attention_operations()
         if ops is None:
             raise YvexError(B.YVEX_ERR_UNSUPPORTED, "rocm_attention_operations", "not published")
@@ -307,8 +312,14 @@ class Backend:
                                        value_pages.handle, page_table.handle, context.handle,
                                        output.handle, lse.handle if lse else None)
         facts, err = B.OperationFacts(), B.Error()
-        _check(ops.paged_decode_execute(self.handle, C.byref(request), C.byref(facts),
-                                        C.byref(err)), err)
+        if gate is not None:
+            epilogue = B.AttentionEpilogue(gate.handle)
+            rc = ops.paged_decode_execute_fused(self.handle, C.byref(request), C.byref(epilogue),
+                                                C.byref(facts), C.byref(err))
+        else:
+            rc = ops.paged_decode_execute(self.handle, C.byref(request), C.byref(facts),
+                                          C.byref(err))
+        _check(rc, err)
         return facts
 
     @staticmethod

@@ -192,13 +192,25 @@ class TransformerOperations(C.Structure):
 KV_APPEND_FN = C.CFUNCTYPE(C.c_int, C.c_void_p, C.POINTER(KvAppendRequest), FactsP, ErrorP)
 
 
+class AttentionEpilogue(C.Structure):
+    _fields_ = [("output_gate", TensorP)]
+
+
+EXECUTE_FUSED_FN = C.CFUNCTYPE(C.c_int, C.c_void_p, C.POINTER(AttentionRequest),
+                               C.POINTER(AttentionEpilogue), TensorP, FactsP, ErrorP)
+PAGED_EXECUTE_FUSED_FN = C.CFUNCTYPE(C.c_int, C.c_void_p, C.POINTER(PagedDecodeRequest),
+                                     C.POINTER(AttentionEpilogue), FactsP, ErrorP)
+
+
 class RocmAttentionOperations(C.Structure):
     _fields_ = [("attention_execute_lse", EXECUTE_LSE_FN),
                 ("paged_decode_workspace_required", PAGED_WORKSPACE_FN),
                 ("paged_decode_execute", PAGED_EXECUTE_FN),
                 ("mla_decode_workspace_required", MLA_WORKSPACE_FN),
                 ("mla_decode_execute", MLA_EXECUTE_FN),
-                ("kv_append_execute", KV_APPEND_FN)]
+                ("kv_append_execute", KV_APPEND_FN),
+                ("attention_execute_fused", EXECUTE_FUSED_FN),
+                ("paged_decode_execute_fused", PAGED_EXECUTE_FUSED_FN)]
 
 
 class RocmReport(C.Structure):

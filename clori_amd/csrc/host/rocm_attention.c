@@ -140,6 +140,7 @@ typedef struct {
     const void *q, *k, *v;
     const int32_t *page_table, *context;
     void *out, *lse;
+    const void *gate;
     unsigned long long sessions, query_heads, kv_heads, head_dim;
     unsigned long long pool_pages, table_stride, max_context, fixed_context;
     unsigned long long k_token_stride, v_token_stride;
@@ -175,6 +176,7 @@ static int decode_run(yvex_backend *backend, const decode_job *job, const char *
     dp.context = job->context;
     dp.out = (uint16_t *)job->out;
     dp.lse = (float *)job->lse;
+    dp.gate = (const uint16_t *)job->gate;
     dp.part_acc = (float *)work;
     dp.part_ml = (float *)((unsigned char *)work + acc_bytes);
     dp.offsets = (uint32_t *)((unsigned char *)work + acc_bytes + ml_bytes);
@@ -301,8 +303,8 @@ static int view_ok(const yvex_backend *backend, const yvex_device_tensor *tensor
 
 static int attention_execute_common(yvex_backend *backend,
                                     const yvex_transformer_attention_request *request,
-                                    yvex_device_tensor *lse, yvex_backend_operation_facts *facts,
-                                    yvex_error *err)
+                                    yvex_device_tensor *lse, const yvex_device_tensor *gate,
+                                    yvex_backend_operation_facts *facts, yvex_error *err)
 {
     static const char where[] = "rocm.transformer.attention";
     yvex_rocm_backend_state *state = yvex_rocm_state(backend);
@@ -322,6 +324,9 @@ static int attention_execute_common(yvex_backend *backend,
     memset(facts, 0, sizeof(*facts));
     exact = r->numeric_contract == YVEX_TRANSFORMER_ATTENTION_NUMERIC_EXACT_F32;
     causal = r->mask == YVEX_TRANSFORMER_ATTENTION_MASK_CAUSAL;
+    if (gate && exact)
+        return refuse(err, YVEX_ERR_UNSUPPORTED, where,
+                      "the fused output gate requires the BF16 numeric contract");
     q_width = r->query_heads * r->head_dimension;
     kv_width = r->key_value_heads * r->head_dimension;
     q_stride = r->query_token_stride ? r->query_token_stride : q_width;
@@ -342,7 +347,9 @@ static int attention_execute_common(yvex_backend *backend,
         !view_ok(backend, request->key, r->key_dtype, k_elements, 1) ||
         !view_ok(backend, request->value, r->value_dtype, v_elements, 1) ||
         !view_ok(backend, request->output, r->output_dtype, o_elements, 0) ||
-        (lse && !view_ok(backend, lse, YVEX_DTYPE_F32, rows, 0)))
+        (lse && !view_ok(backend, lse, YVEX_DTYPE_F32, rows, 0)) ||
+        (gate && (!view_ok(backend, gate, YVEX_DTYPE_BF16, o_elements, 1) ||
+                  gate->data == request->output->data)))
         return refuse(err, YVEX_ERR_FORMAT, "rocm.transformer.gqa",
                       "bounded Q/K/V views matching the declared token strides are required");
     if (exact) {
@@ -385,6 +392,7 @@ static int attention_execute_common(yvex_backend *backend,
         job.v = request->value->data;
         job.out = request->output->data;
         job.lse = lse ? lse->data : NULL;
+        job.gate = gate ? gate->data : NULL;
         job.sessions = 1ull;
         job.query_heads = r->query_heads;
         job.kv_heads = r->key_value_heads;
@@ -404,6 +412,7 @@ static int attention_execute_common(yvex_backend *backend,
         params.v = (const uint16_t *)request->value->data;
         params.out = (uint16_t *)request->output->data;
         params.lse = lse ? (float *)lse->data : NULL;
+        params.gate = gate ? (const uint16_t *)gate->data : NULL;
         params.status = state->device_status;
         params.q_stride = q_stride;
         params.k_stride = k_stride;
@@ -447,7 +456,7 @@ static int rocm_attention_execute(yvex_backend *backend,
                                   const yvex_transformer_attention_request *request,
                                   yvex_backend_operation_facts *facts, yvex_error *err)
 {
-    return attention_execute_common(backend, request, NULL, facts, err);
+    return attention_execute_common(backend, request, NULL, NULL, facts, err);
 }
 
 static int rocm_attention_execute_lse(yvex_backend *backend,
@@ -458,7 +467,19 @@ static int rocm_attention_execute_lse(yvex_backend *backend,
     if (!lse)
         return refuse(err, YVEX_ERR_INVALID_ARG, "rocm.transformer.attention",
                       "an LSE output tensor is required");
-    return attention_execute_common(backend, request, lse, facts, err);
+    return attention_execute_common(backend, request, lse, NULL, facts, err);
+}
+
+static int rocm_attention_execute_fused(yvex_backend *backend,
+                                        const yvex_transformer_attention_request *request,
+                                        const yvex_rocm_attention_epilogue *epilogue,
+                                        yvex_device_tensor *lse,
+                                        yvex_backend_operation_facts *facts, yvex_error *err)
+{
+    if (!epilogue || !epilogue->output_gate)
+        return refuse(err, YVEX_ERR_INVALID_ARG, "rocm.transformer.attention",
+                      "an epilogue with an output gate tensor is required");
+    return attention_execute_common(backend, request, lse, epilogue->output_gate, facts, err);
 }
 
 /* ------------------------------------------------------- paged decode ---- */
@@ -505,9 +526,10 @@ static int rocm_paged_decode_workspace_required(const yvex_rocm_paged_decode_req
     return YVEX_OK;
 }
 
-static int rocm_paged_decode_execute(yvex_backend *backend,
-                                     const yvex_rocm_paged_decode_request *request,
-                                     yvex_backend_operation_facts *facts, yvex_error *err)
+static int paged_decode_execute_common(yvex_backend *backend,
+                                       const yvex_rocm_paged_decode_request *request,
+                                       const yvex_device_tensor *gate,
+                                       yvex_backend_operation_facts *facts, yvex_error *err)
 {
     static const char where[] = "rocm.attention.paged";
     const yvex_rocm_paged_decode_requirement *r;
@@ -539,7 +561,9 @@ static int rocm_paged_decode_execute(yvex_backend *backend,
         !view_ok(backend, request->context_tokens, YVEX_DTYPE_I32, r->sessions, 1) ||
         !view_ok(backend, request->output, YVEX_DTYPE_BF16, q_elements, 0) ||
         (request->lse &&
-         !view_ok(backend, request->lse, YVEX_DTYPE_F32, r->sessions * r->query_heads, 0)))
+         !view_ok(backend, request->lse, YVEX_DTYPE_F32, r->sessions * r->query_heads, 0)) ||
+        (gate && (!view_ok(backend, gate, YVEX_DTYPE_BF16, q_elements, 1) ||
+                  gate->data == request->output->data)))
         return refuse(err, YVEX_ERR_FORMAT, where,
                       "query, page pools, page table, context lengths and outputs must be written "
                       "tensors of this backend with the declared geometry");
@@ -558,6 +582,7 @@ static int rocm_paged_decode_execute(yvex_backend *backend,
     job.context = (const int32_t *)request->context_tokens->data;
     job.out = request->output->data;
     job.lse = request->lse ? request->lse->data : NULL;
+    job.gate = gate ? gate->data : NULL;
     job.sessions = r->sessions;
     job.query_heads = r->query_heads;
     job.kv_heads = r->key_value_heads;
@@ -572,6 +597,24 @@ static int rocm_paged_decode_execute(yvex_backend *backend,
     if (request->lse) request->lse->is_written = 1;
     yvex_error_clear(err);
     return YVEX_OK;
+}
+
+static int rocm_paged_decode_execute(yvex_backend *backend,
+                                     const yvex_rocm_paged_decode_request *request,
+                                     yvex_backend_operation_facts *facts, yvex_error *err)
+{
+    return paged_decode_execute_common(backend, request, NULL, facts, err);
+}
+
+static int rocm_paged_decode_execute_fused(yvex_backend *backend,
+                                           const yvex_rocm_paged_decode_request *request,
+                                           const yvex_rocm_attention_epilogue *epilogue,
+                                           yvex_backend_operation_facts *facts, yvex_error *err)
+{
+    if (!epilogue || !epilogue->output_gate)
+        return refuse(err, YVEX_ERR_INVALID_ARG, "rocm.attention.paged",
+                      "an epilogue with an output gate tensor is required");
+    return paged_decode_execute_common(backend, request, epilogue->output_gate, facts, err);
 }
 
 /* --------------------------------------------------------- MLA decode ---- */
@@ -856,6 +899,8 @@ static const yvex_backend_rocm_attention_operations rocm_attention_ops = {
     .mla_decode_workspace_required = rocm_mla_decode_workspace_required,
     .mla_decode_execute = rocm_mla_decode_execute,
     .kv_append_execute = rocm_kv_append_execute,
+    .attention_execute_fused = rocm_attention_execute_fused,
+    .paged_decode_execute_fused = rocm_paged_decode_execute_fused,
 };
 
 /* A table is published only once the kernel bundle is admitted

@@ -66,6 +66,7 @@ typedef struct {
     uint32_t waves, reserved;
     float scale_log2; /* softmax scale * log2(e) */
     float reserved_f;
+    const uint16_t *gate; /* optional bf16 [sessions][query_heads][head_dim] sigmoid output gate */
 } yvex_rocm_decode_params;
 
 /* Log-sum-exp merge of per-chunk partials (used by the MLA path).  The accumulators are
@@ -94,6 +95,7 @@ typedef struct {
     uint32_t causal, task_count;
     float scale_log2;
     float reserved_f;
+    const uint16_t *gate; /* optional bf16 [Tq][Hq][head_dim] sigmoid output gate */
 } yvex_rocm_prefill_params;
 
 /* Absorbed-latent MLA decode, split over the context.  A chunk spans at most

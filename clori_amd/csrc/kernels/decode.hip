@@ -523,7 +523,16 @@ yvex_rocm_decode_finish(const yvex_rocm_decode_params p)
     const uint32_t kv_head = head / group, hh = head % group;
     const uint32_t seg_begin = offset + kv_head * tiles, seg_end = seg_begin + tiles;
     const uint32_t w_first = seg_begin / per_wave, w_last = (seg_end - 1u) / per_wave;
-    if (w_first == w_last) return;
+    if (w_first == w_last) {
+        // published by the decode kernel itself; only the output gate is left to apply
+        if (p.gate) {
+            const uint64_t at = ((uint64_t)session * p.query_heads + head) * p.head_dim + d;
+            const float o = bf16_to_f32(p.out[at]) * sigmoid(bf16_to_f32(p.gate[at]));
+            if (!isfinite(o)) flag(p.status, YVEX_ROCM_DEVICE_NUMERIC);
+            p.out[at] = bf16_bits(o);
+        }
+        return;
+    }
     auto slot_of = [&](uint32_t j) -> uint64_t {
         return ((uint64_t)j * 2u + (seg_begin >= j * per_wave ? 1u : 0u)) * group + hh;
     };
@@ -557,9 +566,11 @@ yvex_rocm_decode_finish(const yvex_rocm_decode_params p)
         }
         top = m_new;
     }
-    const float o = acc / sum;
+    float o = acc / sum;
+    const uint64_t at = ((uint64_t)session * p.query_heads + head) * p.head_dim + d;
+    if (p.gate) o = bf16_to_f32(bf16_bits(o)) * sigmoid(bf16_to_f32(p.gate[at]));
     if (!isfinite(o)) flag(p.status, YVEX_ROCM_DEVICE_NUMERIC);
-    p.out[((uint64_t)session * p.query_heads + head) * p.head_dim + d] = bf16_bits(o);
+    p.out[at] = bf16_bits(o);
     if (p.lse && d == 0u)
         p.lse[(uint64_t)session * p.query_heads + head] = (top + fast_log2(sum)) * YVEX_LN2;
 }

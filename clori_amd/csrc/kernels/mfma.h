@@ -81,6 +81,34 @@ __device__ inline float bf16_to_f32(uint16_t b)
     return __builtin_bit_cast(float, (uint32_t)b << 16);
 }
 
+// Sigmoid output gate (src/backend/cuda/transformer_kernels.cu:353-364, applied after
+// attention at src/runtime/decoder.c:1266-1269): the published bf16 value times
+// 1 / (1 + exp(-gate)) in F32, rounded to bf16 again.
+__device__ inline float sigmoid(float x)
+{
+    return __builtin_amdgcn_rcpf(1.0f + fast_exp2(x * -1.4426950408889634f));
+}
+
+// Four published values (two packed words) times the gates of the same four dims.
+__device__ inline u32x2 gate_four(u32x2 w, const uint16_t *gate)
+{
+    const u32x2 g = load_b64(gate);
+    u32x2 r;
+    r.x = pack_bf16x2(__builtin_bit_cast(float, w.x << 16) * sigmoid(__builtin_bit_cast(float, g.x << 16)),
+                      __builtin_bit_cast(float, w.x & 0xffff0000u) *
+                          sigmoid(__builtin_bit_cast(float, g.x & 0xffff0000u)));
+    r.y = pack_bf16x2(__builtin_bit_cast(float, w.y << 16) * sigmoid(__builtin_bit_cast(float, g.y << 16)),
+                      __builtin_bit_cast(float, w.y & 0xffff0000u) *
+                          sigmoid(__builtin_bit_cast(float, g.y & 0xffff0000u)));
+    return r;
+}
+
+// true when a packed pair holds an infinity or a NaN
+__device__ inline bool pair_not_finite(uint32_t w)
+{
+    return (w & 0x7f80u) == 0x7f80u || (w & 0x7f800000u) == 0x7f800000u;
+}
+
 typedef int i32x4 __attribute__((ext_vector_type(4)));
 
 // Raw buffer descriptor over [base, base + bytes): stride 0, untyped dword format; loads

@@ -333,6 +333,10 @@ __device__ inline void prefill_body(const yvex_rocm_prefill_params &p, unsigned 
                 u32x2 w;
                 w.x = pack_bf16x2(a0, a1);
                 w.y = pack_bf16x2(a2, a3);
+                if (p.gate && live) {
+                    w = gate_four(w, p.gate + (dst - p.out) + db * 32 + grp * 8 + g * 4);
+                    bad |= pair_not_finite(w.x) || pair_not_finite(w.y);
+                }
                 if (live) *reinterpret_cast<u32x2 *>(dst + db * 32 + grp * 8 + g * 4) = w;
             }
         if (live && bad) flag(p.status, YVEX_ROCM_DEVICE_NUMERIC);

@@ -427,6 +427,18 @@ typedef struct yvex_rocm_kv_append_request {
     yvex_device_tensor *k_pool, *v_pool;
 } yvex_rocm_kv_append_request;
 
+/*
+ * Epilogue fused into the attention kernels.  The arithmetic is the reference's sigmoid
+ * output gate (yvex_sigmoid_product_bf16_f32, src/backend/cuda/transformer_kernels.cu:353-364),
+ * which the decoder runs as a separate pass right after attention
+ * (src/runtime/decoder.c:1266-1269): output = bf16(bf16(attention) * 1 / (1 + exp(-gate))).
+ * output_gate is a written BF16 tensor with the geometry of the output
+ * ([rows][query_heads][head_dimension], packed).  Only the BF16 contract takes an epilogue.
+ */
+typedef struct yvex_rocm_attention_epilogue {
+    const yvex_device_tensor *output_gate;
+} yvex_rocm_attention_epilogue;
+
 typedef struct yvex_backend_rocm_attention_operations {
     /* attention_execute with an additional F32 [query_tokens][query_heads] LSE output */
     int (*attention_execute_lse)(yvex_backend *, const yvex_transformer_attention_request *,
@@ -442,6 +454,14 @@ typedef struct yvex_backend_rocm_attention_operations {
                               yvex_backend_operation_facts *, yvex_error *);
     int (*kv_append_execute)(yvex_backend *, const yvex_rocm_kv_append_request *,
                              yvex_backend_operation_facts *, yvex_error *);
+    /* attention_execute / paged_decode_execute with the epilogue applied before the rows are
+     * published; lse may be NULL */
+    int (*attention_execute_fused)(yvex_backend *, const yvex_transformer_attention_request *,
+                                   const yvex_rocm_attention_epilogue *, yvex_device_tensor *lse,
+                                   yvex_backend_operation_facts *, yvex_error *);
+    int (*paged_decode_execute_fused)(yvex_backend *, const yvex_rocm_paged_decode_request *,
+                                      const yvex_rocm_attention_epilogue *,
+                                      yvex_backend_operation_facts *, yvex_error *);
 } yvex_backend_rocm_attention_operations;
 const yvex_backend_rocm_attention_operations *yvex_backend_rocm_attention_operations_get(
     const yvex_backend *backend);

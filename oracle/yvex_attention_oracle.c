@@ -652,3 +652,15 @@ int yvo_rotary_half_bf16(uint16_t *values, const float *cosines, const float *si
     }
     return 0;
 }
+
+/* src/backend/cuda/transformer_kernels.cu:353-364 */
+int yvo_sigmoid_gate_bf16(const float *values, const float *gate, uint64_t count, float *out)
+{
+    uint64_t index;
+    if (!values || !gate || !out) return YVO_ERR_INVALID_ARG;
+    for (index = 0; index < count; ++index) {
+        const float scale = 1.0f / (1.0f + expf(-gate[index]));
+        out[index] = yvo_bf16_decode(yvo_bf16_encode(values[index] * scale));
+    }
+    return YVO_OK;
+}

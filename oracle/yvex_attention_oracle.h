@@ -29,6 +29,8 @@
  *   yvo_rotary_half_bf16             pinned: known-answer case
  *       (tests/unit/cuda/quant_qtype.c:1988-2061), identity, quarter turn,
  *       float64 rotation within bf16 rounding
+ *   yvo_sigmoid_gate_bf16            pinned: known-answer case
+ *       (tests/unit/cuda/quant_qtype.c:2979-2981,3019-3033), closed forms
  *   yvo_paged_*, yvo_mla_*, yvo_lse_merge
  *       parity unpinned by the reference (it has no page table, no LSE, no
  *       split-K, no Q8_0 KV cache).  Pinned here only by construction
@@ -189,6 +191,16 @@ int yvo_lse_merge(const float *part_out, const double *part_lse, uint64_t parts,
 int yvo_rotary_half_bf16(uint16_t *values, const float *cosines, const float *sines,
                          uint64_t tokens, uint64_t heads, uint64_t head_dim,
                          uint64_t rotary_dim);
+
+/*
+ * Sigmoid output gate on attention rows: out = bf16(values * (1 / (1 + expf(-gate)))), all
+ * F32 carriers; restates src/backend/cuda/transformer_kernels.cu:353-364
+ * (yvex_sigmoid_product_bf16_f32), which the decoder applies to the published attention
+ * rows (src/runtime/decoder.c:1266-1269).  Pinned by the reference's known-answer case
+ * (tests/unit/cuda/quant_qtype.c:2979-2981,3019-3033: values {1,-2,0.5,4}, gates
+ * {0, ln 3, -ln 3, 1}), gate 0 halves, large gates saturate to identity and zero.
+ */
+int yvo_sigmoid_gate_bf16(const float *values, const float *gate, uint64_t count, float *out);
 
 /* Number of worker threads the *_threads arguments are clamped to. */
 int yvo_hardware_threads(void);

@@ -58,6 +58,7 @@ def load_oracle():
     lib.yvo_paged_decode_q8_0.argtypes = [u16p, u8p, u8p] + paged
     lib.yvo_shared_kv_head.argtypes = [f32p, f32p, C.c_size_t, u64, u64, u64, C.c_double, f32p, f32p, f64p]
     lib.yvo_rotary_half_bf16.argtypes = [u16p, f32p, f32p] + [u64] * 4
+    lib.yvo_sigmoid_gate_bf16.argtypes = [f32p, f32p, u64, f32p]
     lib.yvo_mla_decode_bf16.argtypes = [u16p, u16p, i32p, i32p, f32p, u16p, f64p] + [u64] * 7 + [C.c_int]
     lib.yvo_lse_merge.argtypes = [f32p, f64p, u64, u64, f32p, f64p]
     return lib
@@ -209,6 +210,16 @@ class Oracle:
         sines = np.ascontiguousarray(sines, dtype=np.float32)
         rc = self.lib.yvo_rotary_half_bf16(_ptr(out, u16p), _ptr(cosines, f32p), _ptr(sines, f32p),
                                            tokens, heads, d, rotary_dim)
+        assert rc == 0
+        return out
+
+    def sigmoid_gate_bf16(self, values, gate):
+        """F32 values (bf16-representable) times sigmoid(gate), rounded to bf16; F32 out."""
+        values = np.ascontiguousarray(values, dtype=np.float32)
+        gate = np.ascontiguousarray(gate, dtype=np.float32)
+        out = np.zeros_like(values)
+        rc = self.lib.yvo_sigmoid_gate_bf16(_ptr(values, f32p), _ptr(gate, f32p), values.size,
+                                            _ptr(out, f32p))
         assert rc == 0
         return out
 

@@ -452,6 +452,43 @@ def test_kv_append_admission():
         assert e.value.code == B.YVEX_ERR_FORMAT
 
 
+def test_fused_gate_admission():
+    """The epilogue entry points: an epilogue is required, the gate has the output geometry
+    and is a written tensor other than the output, and only the BF16 contract takes one."""
+    with Backend() as b:
+        ops = b.rocm_attention_operations()
+        req = b.attention_requirement(4, 4, 2, 1, 128, dtype=B.DTYPE_BF16,
+                                      contract=B.NUMERIC_BF16_F32_ACCUMULATE)
+        q = written(b, "q", B.DTYPE_BF16, (4, 2, 128))
+        k, v = written(b, "k", B.DTYPE_BF16, (4, 1, 128)), written(b, "v", B.DTYPE_BF16, (4, 1, 128))
+        out = b.tensor("o", B.DTYPE_BF16, (4, 2, 128))
+        gate = written(b, "g", B.DTYPE_BF16, (4, 2, 128))
+        assert b.attention_execute(req, q, k, v, out, gate=gate).kernel_launches == 1
+        assert out.is_written
+        request = B.AttentionRequest(req, q.handle, k.handle, v.handle, out.handle)
+        facts, err = B.OperationFacts(), B.Error()
+        assert ops.attention_execute_fused(b.handle, C.byref(request), None, None, C.byref(facts),
+                                           C.byref(err)) == B.YVEX_ERR_INVALID_ARG
+        empty = B.AttentionEpilogue(None)
+        assert ops.attention_execute_fused(b.handle, C.byref(request), C.byref(empty), None,
+                                           C.byref(facts), C.byref(err)) == B.YVEX_ERR_INVALID_ARG
+        for bad in (written(b, "g1", B.DTYPE_BF16, (4, 2, 64)), written(b, "g2", B.DTYPE_F32, (4, 2, 128)),
+                    b.tensor("g3", B.DTYPE_BF16, (4, 2, 128)), out):
+            with pytest.raises(YvexError) as e:
+                b.attention_execute(req, q, k, v, out, gate=bad)
+            assert e.value.code == B.YVEX_ERR_FORMAT
+        paged = b.paged_requirement(4, 32, 8, 128, 16, 100, 64, 1024)
+        pq = written(b, "pq", B.DTYPE_BF16, (4, 32, 128))
+        pool = written(b, "pool", B.DTYPE_BF16, (100 * 8 * 2048,))
+        table, ctx = written(b, "t", B.DTYPE_I32, (4, 64)), written(b, "c", B.DTYPE_I32, (4,))
+        pout = b.tensor("po", B.DTYPE_BF16, (4, 32, 128))
+        pgate = written(b, "pg", B.DTYPE_BF16, (4, 32, 128))
+        assert b.paged_decode_execute(paged, pq, pool, pool, table, ctx, pout, gate=pgate).kernel_launches == 2
+        with pytest.raises(YvexError) as e:
+            b.paged_decode_execute(paged, pq, pool, pool, table, ctx, pout, gate=gate)
+        assert e.value.code == B.YVEX_ERR_FORMAT
+
+
 # ------------------------------------------------- failure transitions ----
 
 def test_launch_failure_fails_only_that_variant(env):

@@ -512,3 +512,29 @@ def test_rotary_closed_forms():
         assert np.all(np.isfinite(got))
         assert np.max(np.abs(got - want)) < 3 * 2.0 ** -8 * np.max(np.abs(xf))
         assert np.allclose(np.linalg.norm(got, axis=-1), np.linalg.norm(xf, axis=-1), rtol=5e-3)
+
+
+# -------------------------------------------------------- output gate -------
+
+def test_sigmoid_gate_reference_known_answer():
+    """tests/unit/cuda/quant_qtype.c:2979-2981,3019-3033.  sigmoid(0) = 1/2, sigmoid(+-ln 3)
+    = 3/4 and 1/4, sigmoid(1) = 0.7310586: 4 * 0.7310586 = 2.9242 rounds to 2.921875 in bf16."""
+    values = np.array([1.0, -2.0, 0.5, 4.0], np.float32)
+    gates = np.array([0.0, 1.0986122886681098, -1.0986122886681098, 1.0], np.float32)
+    assert ORACLE.sigmoid_gate_bf16(values, gates).tolist() == [0.5, -1.5, 0.125, 2.921875]
+
+
+def test_sigmoid_gate_closed_forms():
+    rng = np.random.default_rng(55)
+    values = ORACLE.bf16_decode(ORACLE.bf16_encode(rng.standard_normal(4096).astype(np.float32)))
+    assert np.array_equal(ORACLE.sigmoid_gate_bf16(values, np.full(4096, 40.0)), values)
+    assert np.all(ORACLE.sigmoid_gate_bf16(values, np.full(4096, -200.0)) == 0.0)
+    half = ORACLE.sigmoid_gate_bf16(values, np.zeros(4096))
+    assert np.array_equal(half, values * 0.5)              # exact: a power-of-two scale
+    gates = rng.uniform(-8.0, 8.0, 4096).astype(np.float32)
+    want = values.astype(np.float64) / (1.0 + np.exp(-gates.astype(np.float64)))
+    got = ORACLE.sigmoid_gate_bf16(values, gates)
+    assert np.max(np.abs(got - want) / np.maximum(np.abs(want), 1e-30)) <= 2.0 ** -8
+    # symmetry sigmoid(g) + sigmoid(-g) = 1 on a value whose products are exact in bf16
+    plus, minus = ORACLE.sigmoid_gate_bf16(np.ones(4096), gates), ORACLE.sigmoid_gate_bf16(np.ones(4096), -gates)
+    assert np.max(np.abs(plus + minus - 1.0)) <= 2.0 ** -8
