@@ -620,7 +620,7 @@ static int rocm_paged_decode_execute_fused(yvex_backend *backend,
 /* --------------------------------------------------------- MLA decode ---- */
 
 enum { ROCM_MLA_HEADS = 128, ROCM_MLA_KEY_DIM = 576, ROCM_MLA_VALUE_DIM = 512,
-       ROCM_MLA_PAGE_TOKENS = 64 };
+       ROCM_MLA_PAGE_TOKENS = 64, ROCM_MLA_TILE_TOKENS = 32 };
 
 static int mla_validate(const yvex_rocm_mla_decode_requirement *r, const char *where,
                         yvex_error *err)
@@ -636,7 +636,7 @@ static int mla_validate(const yvex_rocm_mla_decode_requirement *r, const char *w
         r->value_dimension != ROCM_MLA_VALUE_DIM || r->page_tokens != ROCM_MLA_PAGE_TOKENS ||
         r->numeric_contract != YVEX_TRANSFORMER_ATTENTION_NUMERIC_BF16_F32_ACCUMULATE ||
         !r->deterministic || r->pool_pages > 0x7fffffffull || capacity > 0x7fffffffull ||
-        r->batch > 65535ull)
+        r->batch > 65535ull || r->sliding_window > 0x7fffffffull)
         return refuse(err, YVEX_ERR_UNSUPPORTED, where,
                       "ROCm MLA decode requires 128 heads, a 512+64 latent row, 64-token pages "
                       "and the deterministic bf16/fp32-accumulate contract");
@@ -646,15 +646,27 @@ static int mla_validate(const yvex_rocm_mla_decode_requirement *r, const char *w
 
 /* Chunks are a function of the request geometry only: about one workgroup per compute
  * unit of a 256-CU part, in whole pages. */
+/* Tokens a session can have live: the context, or with a sliding window the window plus the
+ * part of a 32-token tile in front of it. */
+static unsigned long long mla_live_tokens(const yvex_rocm_mla_decode_requirement *r)
+{
+    if (r->sliding_window && r->sliding_window + ROCM_MLA_TILE_TOKENS - 1ull < r->max_context_tokens)
+        return r->sliding_window + ROCM_MLA_TILE_TOKENS - 1ull;
+    return r->max_context_tokens;
+}
+
 static unsigned int mla_chunk_tokens(const yvex_rocm_mla_decode_requirement *r)
 {
     const char *forced = getenv("YVEX_ROCM_MLA_CHUNK");
     unsigned long long per_batch = 256ull / r->batch ? 256ull / r->batch : 1ull;
-    unsigned long long chunk = (r->max_context_tokens + per_batch - 1ull) / per_batch;
+    unsigned long long chunk = (mla_live_tokens(r) + per_batch - 1ull) / per_batch;
     if (forced && atoi(forced) >= ROCM_MLA_PAGE_TOKENS) chunk = (unsigned long long)atoi(forced);
     chunk = align_up(chunk, ROCM_MLA_PAGE_TOKENS);
-    if (chunk > (unsigned long long)YVEX_ROCM_MLA_MAX_CHUNK_PAGES * ROCM_MLA_PAGE_TOKENS)
-        chunk = (unsigned long long)YVEX_ROCM_MLA_MAX_CHUNK_PAGES * ROCM_MLA_PAGE_TOKENS;
+    /* a windowed chunk may start in the middle of a page and so touch one page more */
+    if (chunk > (unsigned long long)(YVEX_ROCM_MLA_MAX_CHUNK_PAGES - (r->sliding_window ? 1 : 0)) *
+                    ROCM_MLA_PAGE_TOKENS)
+        chunk = (unsigned long long)(YVEX_ROCM_MLA_MAX_CHUNK_PAGES - (r->sliding_window ? 1 : 0)) *
+                ROCM_MLA_PAGE_TOKENS;
     return (unsigned int)chunk;
 }
 
@@ -669,7 +681,7 @@ static int rocm_mla_decode_workspace_required(const yvex_rocm_mla_decode_require
     if (rc != YVEX_OK) return rc;
     if (!bytes) return refuse(err, YVEX_ERR_INVALID_ARG, where, "workspace byte output is required");
     chunk = mla_chunk_tokens(r);
-    max_chunks = (r->max_context_tokens + chunk - 1ull) / chunk;
+    max_chunks = (mla_live_tokens(r) + chunk - 1ull) / chunk;
     if (!decode_workspace_bytes(r->batch * max_chunks, r->heads, r->value_dimension,
                                 sizeof(uint16_t), &acc, &total))
         return refuse(err, YVEX_ERR_BOUNDS, where, "MLA workspace geometry overflowed");
@@ -710,12 +722,13 @@ static int rocm_mla_decode_execute(yvex_backend *backend,
         !view_ok(backend, request->context_tokens, YVEX_DTYPE_I32, r->batch, 1) ||
         !view_ok(backend, request->output, YVEX_DTYPE_BF16,
                  r->batch * r->heads * r->value_dimension, 0) ||
-        (request->lse && !view_ok(backend, request->lse, YVEX_DTYPE_F32, r->batch * r->heads, 0)))
+        (request->lse && !view_ok(backend, request->lse, YVEX_DTYPE_F32, r->batch * r->heads, 0)) ||
+        (request->sinks && !view_ok(backend, request->sinks, YVEX_DTYPE_F32, r->heads, 1)))
         return refuse(err, YVEX_ERR_FORMAT, where,
                       "query, latent pages, page table, context lengths and outputs must be "
                       "written tensors of this backend with the declared geometry");
     chunk = mla_chunk_tokens(r);
-    max_chunks = (r->max_context_tokens + chunk - 1ull) / chunk;
+    max_chunks = (mla_live_tokens(r) + chunk - 1ull) / chunk;
     if (max_chunks > 0x7fffffffull ||
         !decode_workspace_bytes(r->batch * max_chunks, r->heads, r->value_dimension,
                                 sizeof(uint16_t), &acc_bytes, &total))
@@ -740,6 +753,7 @@ static int rocm_mla_decode_execute(yvex_backend *backend,
     kp.table_stride = (uint32_t)r->page_table_stride;
     kp.chunk_tokens = (uint32_t)chunk;
     kp.max_chunks = (uint32_t)max_chunks;
+    kp.window = (uint32_t)r->sliding_window;
     /* src/graph/core.c:604: scale = 1/sqrt(head_dimension), here over the 576-lane key */
     kp.scale_log2 = (float)(1.4426950408889634 / sqrt((double)r->key_dimension));
     rc = yvex_rocm_launch(backend, YVEX_ROCM_FN_MLA_DECODE_BF16, variant, (unsigned int)max_chunks,
@@ -757,6 +771,9 @@ static int rocm_mla_decode_execute(yvex_backend *backend,
         mp.head_dim = kp.value_dim;
         mp.chunk_tokens = kp.chunk_tokens;
         mp.max_chunks = kp.max_chunks;
+        mp.sinks = request->sinks ? (const float *)request->sinks->data : NULL;
+        mp.window = kp.window;
+        mp.window_align = ROCM_MLA_TILE_TOKENS;
         rc = yvex_rocm_launch(backend, YVEX_ROCM_FN_DECODE_MERGE, variant,
                               (unsigned int)((r->heads + 3ull) / 4ull), (unsigned int)r->batch, 1u,
                               256u, 0u, &mp, where, err);

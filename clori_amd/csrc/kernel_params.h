@@ -69,7 +69,8 @@ typedef struct {
     const uint16_t *gate; /* optional bf16 [sessions][query_heads][head_dim] sigmoid output gate */
 } yvex_rocm_decode_params;
 
-/* Log-sum-exp merge of per-chunk partials (used by the MLA path).  The accumulators are
+/* Log-sum-exp merge of per-chunk partials (used by the MLA path).  With a sliding window the
+ * chunks start at the first visible token rounded down to window_align, as in the producer.  The accumulators are
  * unnormalised and stored as bf16: they are 44 % of that path's HBM traffic in fp32. */
 typedef struct {
     const uint16_t *part_acc;
@@ -79,6 +80,9 @@ typedef struct {
     float *lse;    /* optional F32 [sessions][query_heads] */
     int32_t *status;
     uint32_t sessions, query_heads, head_dim, chunk_tokens, max_chunks, fixed_context;
+    const float *sinks; /* optional F32 [query_heads]: one extra logit per head with value 0 */
+    uint32_t window;    /* sliding window of the producing kernel (sets its first chunk) */
+    uint32_t window_align; /* the producer starts its chunks at first_visible rounded down to this */
 } yvex_rocm_decode_merge_params;
 
 /* Causal / full GQA prefill on bf16 token-major tensors.  The grid is one-dimensional:
@@ -109,7 +113,8 @@ typedef struct {
     float *part_ml;     /* [batch][max_chunks][heads][2] */
     int32_t *status;
     uint32_t batch, heads, key_dim, value_dim;
-    uint32_t page_tokens, pool_pages, table_stride, chunk_tokens, max_chunks, reserved;
+    uint32_t page_tokens, pool_pages, table_stride, chunk_tokens, max_chunks;
+    uint32_t window; /* sliding window in tokens, 0: the whole context */
     float scale_log2;
     float reserved_f;
 } yvex_rocm_mla_params;

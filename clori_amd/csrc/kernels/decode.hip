@@ -585,7 +585,9 @@ yvex_rocm_decode_merge(const yvex_rocm_decode_merge_params p)
     const uint32_t head = blockIdx.x * 4u + (threadIdx.x >> 6), session = blockIdx.y;
     const uint32_t ctx = p.context ? (uint32_t)p.context[session] : p.fixed_context;
     if (ctx == 0u || head >= p.query_heads || lane * 8u >= p.head_dim) return;
-    const uint32_t chunks = min(p.max_chunks, (ctx + p.chunk_tokens - 1u) / p.chunk_tokens);
+    const uint32_t first_visible = p.window != 0u && ctx > p.window ? ctx - p.window : 0u;
+    const uint32_t live = ctx - (first_visible & ~(p.window_align - 1u));
+    const uint32_t chunks = min(p.max_chunks, (live + p.chunk_tokens - 1u) / p.chunk_tokens);
     const uint64_t base = ((uint64_t)session * p.max_chunks) * p.query_heads + head;
     // Sixteen chunks per trip, every load of a trip independent of the others (indices past
     // the end alias the last chunk with weight zero): one memory round trip per trip, which
@@ -626,8 +628,20 @@ yvex_rocm_decode_merge(const yvex_rocm_decode_merge_params p)
         }
         top = m_new;
     }
-    const float inv = 1.0f / total;
     bool bad = false;
+    if (p.sinks) {
+        // the head's sink logit joins the softmax with a zero value row
+        // (src/graph/core.c:471-508): it only enlarges the denominator
+        const float sink = p.sinks[head] * 1.4426950408889634f;  // log2 units, as the maxima
+        bad |= !isfinite(sink);
+        const float m_new = fmaxf(top, sink);
+        const float keep = fast_exp2(top - m_new);
+        total = total * keep + fast_exp2(sink - m_new);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[i] *= keep;
+        top = m_new;
+    }
+    const float inv = 1.0f / total;
     u32x4 out;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {

@@ -86,7 +86,10 @@ yvex_rocm_mla_decode_bf16(const yvex_rocm_mla_params p)
         if (chunk == 0u && tid == 0) flag(p.status, YVEX_ROCM_DEVICE_CONTRACT);
         return;
     }
-    const uint32_t t0 = chunk * p.chunk_tokens;
+    // sliding window (src/backend/cuda/attention_kernels.cu:79-84): positions below
+    // ctx - window are not visible; chunks start at the tile that holds the first visible one
+    const uint32_t w0 = p.window != 0u && ctx > p.window ? ctx - p.window : 0u;
+    const uint32_t t0 = (w0 & ~(uint32_t)(kTile - 1)) + chunk * p.chunk_tokens;
     if (t0 >= ctx) return;
     const uint32_t t1 = min(ctx, t0 + p.chunk_tokens);
     const uint32_t tiles = (t1 - t0 + kTile - 1) / kTile;
@@ -205,13 +208,14 @@ yvex_rocm_mla_decode_bf16(const yvex_rocm_mla_params p)
             __builtin_amdgcn_sched_barrier(0);
         }
     };
-    // masks the tail, then raises the running maximum if this tile needs it (both token
+    // masks the tail (and the keys in front of a sliding window), then raises the running maximum if this tile needs it (both token
     // halves of a head must agree on the reference maximum)
     auto settle = [&](uint32_t key0, floatx16 &s, uint32_t (&pending)[8]) {
-        if (key0 + kTile > t1) {
+        if (key0 + kTile > t1 || key0 < w0) {
+            // visible keys are w0 <= key < t1: one unsigned compare
 #pragma unroll
             for (int i = 0; i < 16; ++i)
-                if (key0 + (i >> 2) * 8 + g * 4 + (i & 3) >= t1) s[i] = -INFINITY;
+                if (key0 + (i >> 2) * 8 + g * 4 + (i & 3) - w0 >= t1 - w0) s[i] = -INFINITY;
         }
         float mloc = -INFINITY;
 #pragma unroll

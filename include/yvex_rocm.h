@@ -396,12 +396,20 @@ typedef struct yvex_rocm_mla_decode_requirement {
     unsigned long long page_tokens, pool_pages, page_table_stride, max_context_tokens;
     yvex_transformer_attention_numeric_contract numeric_contract;
     int deterministic;
+    /* Sliding-window position filter of the shared-KV reduce
+     * (src/backend/cuda/attention_kernels.cu:79-84): the query at position context - 1 sees
+     * positions >= context - sliding_window.  0: the whole context. */
+    unsigned long long sliding_window;
 } yvex_rocm_mla_decode_requirement;
 
 typedef struct yvex_rocm_mla_decode_request {
     yvex_rocm_mla_decode_requirement requirement;
     const yvex_device_tensor *query, *latent_pages, *page_table, *context_tokens;
     yvex_device_tensor *output, *lse;
+    /* Optional F32 [heads] sink logits (src/graph/core.c:471-508, attention_kernels.cu:164-166):
+     * each seeds the head's maximum and adds exp(sink - max) to its denominator with a zero
+     * value row; the LSE output includes it.  NULL: no sink. */
+    const yvex_device_tensor *sinks;
 } yvex_rocm_mla_decode_request;
 
 /* KV page writer (no reference counterpart as one operation: it is the rotary step of

@@ -545,7 +545,8 @@ int yvo_mla_decode_bf16(const uint16_t *q, const uint16_t *pool,
                         float *out_f32, uint16_t *out_bf16, double *lse,
                         uint64_t batch, uint64_t heads, uint64_t key_dim,
                         uint64_t value_dim, uint64_t page_tokens,
-                        uint64_t pool_pages, uint64_t table_stride, int threads)
+                        uint64_t pool_pages, uint64_t table_stride,
+                        const float *sinks, uint64_t sliding_window, int threads)
 {
     uint64_t b;
     double scale;
@@ -569,14 +570,19 @@ int yvo_mla_decode_bf16(const uint16_t *q, const uint16_t *pool,
     threads = clamp_threads(threads);
 #pragma omp parallel for schedule(dynamic, 1) num_threads(threads)
     for (unit = 0; unit < (long long)batch; ++unit) {
-        uint64_t n = (uint64_t)context[unit], t, h;
+        /* src/backend/cuda/attention_kernels.cu:79-84: the token at position context - 1
+         * sees positions first .. context - 1, first = context - window (or 0) */
+        const uint64_t total = (uint64_t)context[unit];
+        const uint64_t first = sliding_window && total > sliding_window ? total - sliding_window : 0u;
+        uint64_t n = total - first, t, h;
         float *rows = (float *)malloc((size_t)(n * key_dim) * sizeof(float));
         float *qf = (float *)malloc((size_t)key_dim * sizeof(float));
         float *of = (float *)malloc((size_t)value_dim * sizeof(float));
         int rc = rows && qf && of ? YVO_OK : YVO_ERR_STATE;
         for (t = 0; rc == YVO_OK && t < n; ++t) {
-            uint64_t page = (uint64_t)page_table[(uint64_t)unit * table_stride + t / page_tokens];
-            yvo_bf16_decode_n(pool + (page * page_tokens + t % page_tokens) * key_dim,
+            const uint64_t at = first + t;
+            uint64_t page = (uint64_t)page_table[(uint64_t)unit * table_stride + at / page_tokens];
+            yvo_bf16_decode_n(pool + (page * page_tokens + at % page_tokens) * key_dim,
                               rows + t * key_dim, (size_t)key_dim);
         }
         for (h = 0; rc == YVO_OK && h < heads; ++h) {
@@ -585,7 +591,7 @@ int yvo_mla_decode_bf16(const uint16_t *q, const uint16_t *pool,
             double unit_lse = 0.0;
             yvo_bf16_decode_n(q + qo, qf, (size_t)key_dim);
             rc = yvo_shared_kv_head(qf, rows, (size_t)key_dim, n, key_dim, value_dim,
-                                    scale, NULL, of, &unit_lse);
+                                    scale, sinks ? sinks + h : NULL, of, &unit_lse);
             if (rc != YVO_OK) break;
             if (out_f32) memcpy(out_f32 + oo, of, (size_t)value_dim * sizeof(float));
             if (out_bf16) yvo_bf16_encode_n(of, out_bf16 + oo, (size_t)value_dim);

@@ -161,13 +161,18 @@ int yvo_shared_kv_head(const float *q, const float *rows, size_t row_stride,
  * q bf16 [batch][heads][key_dim]; pool bf16 [pool_pages][page_tokens][key_dim];
  * value = first value_dim lanes of each row; scale = 1/sqrt(key_dim) in double
  * (src/graph/core.c:604).  Output is F32 plus RNE bf16 [batch][heads][value_dim].
+ * sinks: optional F32 [heads] sink logits handed to yvo_shared_kv_head; sliding_window:
+ * 0 for the whole context, else only positions >= context - sliding_window are rows
+ * (the position filter of src/backend/cuda/attention_kernels.cu:79-84 for the token at
+ * position context - 1).
  */
 int yvo_mla_decode_bf16(const uint16_t *q, const uint16_t *pool,
                         const int32_t *page_table, const int32_t *context,
                         float *out_f32, uint16_t *out_bf16, double *lse,
                         uint64_t batch, uint64_t heads, uint64_t key_dim,
                         uint64_t value_dim, uint64_t page_tokens,
-                        uint64_t pool_pages, uint64_t table_stride, int threads);
+                        uint64_t pool_pages, uint64_t table_stride,
+                        const float *sinks, uint64_t sliding_window, int threads);
 
 /*
  * Log-sum-exp merge of split partials for one head: part p holds a normalised

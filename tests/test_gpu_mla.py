@@ -27,18 +27,23 @@ def make_case(rng, contexts, spare=2):
     return q, pool, table, np.array(contexts, dtype=np.int32)
 
 
-def run_mla(backend, q, pool, table, ctx, max_context=None):
+def run_mla(backend, q, pool, table, ctx, max_context=None, sinks=None, window=0):
     batch = q.shape[0]
     req = backend.mla_requirement(batch, HEADS, KEY_DIM, VALUE_DIM, PAGE, pool.shape[0],
-                                  table.shape[1], max_context or int(table.shape[1] * PAGE))
+                                  table.shape[1], max_context or int(table.shape[1] * PAGE),
+                                  sliding_window=window)
     out = backend.tensor("o", B.DTYPE_BF16, (batch, HEADS, VALUE_DIM))
     lse = backend.tensor("lse", B.DTYPE_F32, (batch, HEADS))
-    facts = backend.mla_decode_execute(
-        req, backend.tensor("q", B.DTYPE_BF16, q.shape, q),
-        backend.tensor("pool", B.DTYPE_BF16, pool.shape, pool),
-        backend.tensor("table", B.DTYPE_I32, table.shape, table),
-        backend.tensor("ctx", B.DTYPE_I32, ctx.shape, ctx), out, lse)
-    return out.read(), lse.read(), facts
+    tensors = [backend.tensor("q", B.DTYPE_BF16, q.shape, q),
+               backend.tensor("pool", B.DTYPE_BF16, pool.shape, pool),
+               backend.tensor("table", B.DTYPE_I32, table.shape, table),
+               backend.tensor("ctx", B.DTYPE_I32, ctx.shape, ctx)]
+    ts = backend.tensor("sinks", B.DTYPE_F32, (HEADS,), sinks) if sinks is not None else None
+    facts = backend.mla_decode_execute(req, *tensors, out, lse, sinks=ts)
+    result = out.read(), lse.read(), facts
+    for t in tensors + [out, lse] + ([ts] if ts else []):
+        t.release()
+    return result
 
 
 def test_mla_decode_matches_shared_kv_oracle_ragged(backend):
@@ -86,3 +91,54 @@ def test_mla_page_placement_invariance_and_refusals(backend):
     with pytest.raises(YvexError) as e:
         backend.mla_decode_workspace_required(req)
     assert e.value.code == B.YVEX_ERR_UNSUPPORTED
+
+
+@pytest.mark.parametrize("window", [0, 1, 31, 32, 33, 100, 1024, 100000])
+def test_mla_sink_logits_and_sliding_window(backend, window):
+    """Per-head sink logits in the softmax denominator and the sliding-window position filter
+    (src/backend/cuda/attention_kernels.cu:79-84,164-166), ragged contexts around the 32-token
+    tile and 64-token page edges."""
+    rng = np.random.default_rng(500 + window)
+    contexts = [1, 31, 32, 33, 63, 64, 65, 100, 129, 500, 1300, 4097]
+    q, pool, table, ctx = make_case(rng, contexts)
+    sinks = (rng.standard_normal(HEADS) * 3.0).astype(np.float32)
+    got, lse, facts = run_mla(backend, q, pool, table, ctx, sinks=sinks, window=window)
+    rc, ref, _, ref_lse = ORACLE.mla_decode(q, pool, table, ctx, VALUE_DIM, PAGE, sinks=sinks,
+                                            sliding_window=window)
+    assert rc == 0
+    assert_close_bf16(got, ref, "mla sink window=%d" % window)
+    assert_lse(lse, ref_lse, "mla sink window=%d" % window)
+    assert facts.kernel_launches == 2
+    # without sinks the window alone
+    got, lse, _ = run_mla(backend, q, pool, table, ctx, window=window)
+    rc, ref, _, ref_lse = ORACLE.mla_decode(q, pool, table, ctx, VALUE_DIM, PAGE,
+                                            sliding_window=window)
+    assert rc == 0
+    assert_close_bf16(got, ref, "mla window=%d" % window)
+    assert_lse(lse, ref_lse, "mla window=%d" % window)
+
+
+def test_mla_window_at_config5_context(backend):
+    """Context 8192 with a 4096-token window: only the last 4096 positions count, and the
+    workspace shrinks with the window."""
+    rng = np.random.default_rng(58)
+    q, pool, table, ctx = make_case(rng, [8192, 8000, 4096, 5000])
+    full = backend.mla_requirement(4, HEADS, KEY_DIM, VALUE_DIM, PAGE, pool.shape[0], table.shape[1], 8192)
+    windowed = backend.mla_requirement(4, HEADS, KEY_DIM, VALUE_DIM, PAGE, pool.shape[0], table.shape[1],
+                                       8192, sliding_window=4096)
+    assert backend.mla_decode_workspace_required(windowed) < backend.mla_decode_workspace_required(full)
+    got, lse, _ = run_mla(backend, q, pool, table, ctx, max_context=8192, window=4096)
+    rc, ref, _, ref_lse = ORACLE.mla_decode(q, pool, table, ctx, VALUE_DIM, PAGE, sliding_window=4096)
+    assert rc == 0
+    assert_close_bf16(got, ref, "mla window 4096")
+    assert_lse(lse, ref_lse, "mla window 4096")
+
+
+def test_mla_non_finite_sink_is_a_numeric_failure(backend):
+    rng = np.random.default_rng(59)
+    q, pool, table, ctx = make_case(rng, [70])
+    sinks = np.zeros(HEADS, np.float32)
+    sinks[17] = np.inf
+    with pytest.raises(YvexError) as e:
+        run_mla(backend, q, pool, table, ctx, sinks=sinks)
+    assert e.value.code == B.YVEX_ERR_FORMAT

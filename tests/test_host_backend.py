@@ -403,6 +403,19 @@ def test_paged_and_mla_admission():
         assert e.value.code == B.YVEX_ERR_FORMAT
         mla = b.mla_requirement(16, 128, 576, 512, 64, 2048, 128, 8192)
         assert b.mla_decode_workspace_required(mla) > 0
+        windowed = b.mla_requirement(16, 128, 576, 512, 64, 2048, 128, 8192, sliding_window=1024)
+        assert 0 < b.mla_decode_workspace_required(windowed) < b.mla_decode_workspace_required(mla)
+        mq = written(b, "mq", B.DTYPE_BF16, (16, 128, 576))
+        latent = written(b, "latent", B.DTYPE_BF16, (2048, 64, 576))
+        mtable, mctx = written(b, "mt", B.DTYPE_I32, (16, 128)), written(b, "mc", B.DTYPE_I32, (16,))
+        mout = b.tensor("mo", B.DTYPE_BF16, (16, 128, 512))
+        sinks = written(b, "sinks", B.DTYPE_F32, (128,))
+        assert b.mla_decode_execute(windowed, mq, latent, mtable, mctx, mout, sinks=sinks).kernel_launches == 2
+        for wrong in (written(b, "s1", B.DTYPE_F32, (64,)), written(b, "s2", B.DTYPE_BF16, (128,)),
+                      b.tensor("s3", B.DTYPE_F32, (128,))):
+            with pytest.raises(YvexError) as e:
+                b.mla_decode_execute(mla, mq, latent, mtable, mctx, mout, sinks=wrong)
+            assert e.value.code == B.YVEX_ERR_FORMAT
         bad = b.mla_requirement(16, 64, 576, 512, 64, 2048, 128, 8192)
         with pytest.raises(YvexError) as e:
             b.mla_decode_workspace_required(bad)

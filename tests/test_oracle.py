@@ -538,3 +538,57 @@ def test_sigmoid_gate_closed_forms():
     # symmetry sigmoid(g) + sigmoid(-g) = 1 on a value whose products are exact in bf16
     plus, minus = ORACLE.sigmoid_gate_bf16(np.ones(4096), gates), ORACLE.sigmoid_gate_bf16(np.ones(4096), -gates)
     assert np.max(np.abs(plus + minus - 1.0)) <= 2.0 ** -8
+
+
+# ------------------------------------------- MLA sink and sliding window ----
+
+def _mla_case(rng, contexts, heads=4, kd=64, vd=48, pt=16):
+    need = [(c + pt - 1) // pt for c in contexts]
+    pool_pages = sum(need) + 1
+    perm = rng.permutation(pool_pages).astype(np.int32)
+    table = np.zeros((len(contexts), max(need)), np.int32)
+    at = 0
+    for b, n in enumerate(need):
+        table[b, :n] = perm[at:at + n]
+        at += n
+    pool = ORACLE.bf16_encode(rng.standard_normal((pool_pages, pt, kd)).astype(np.float32))
+    q = ORACLE.bf16_encode(rng.standard_normal((len(contexts), heads, kd)).astype(np.float32))
+    return q, pool, table, np.array(contexts, np.int32), vd, pt
+
+
+def test_mla_sink_is_one_more_logit_with_a_zero_row():
+    """With a sink s: out = out0 * e^lse0 / (e^lse0 + e^s) and lse = log(e^lse0 + e^s), where
+    (out0, lse0) is the result without it (softmax over one more logit whose value is 0)."""
+    rng = np.random.default_rng(66)
+    q, pool, table, ctx, vd, pt = _mla_case(rng, [1, 5, 40, 333])
+    sinks = np.array([-3.0, 0.0, 1.5, 9.0], np.float32)
+    rc0, out0, _, lse0 = ORACLE.mla_decode(q, pool, table, ctx, vd, pt)
+    rc1, out1, _, lse1 = ORACLE.mla_decode(q, pool, table, ctx, vd, pt, sinks=sinks)
+    assert rc0 == 0 and rc1 == 0
+    keep = 1.0 / (1.0 + np.exp(sinks[None, :].astype(np.float64) - lse0))
+    assert np.allclose(out1, out0 * keep[..., None], rtol=1e-5, atol=1e-7)
+    assert np.allclose(lse1, np.logaddexp(lse0, sinks[None, :]), atol=1e-9)
+    rc, _, _, _ = ORACLE.mla_decode(q, pool, table, ctx, vd, pt,
+                                    sinks=np.array([0, np.inf, 0, 0], np.float32))
+    assert rc != 0                                         # a non-finite sink is refused
+
+
+@pytest.mark.parametrize("window", [1, 7, 16, 100, 10 ** 6])
+def test_mla_sliding_window_equals_decode_on_the_trimmed_context(window):
+    rng = np.random.default_rng(67)
+    contexts = [1, 16, 17, 90, 257]
+    q, pool, table, ctx, vd, pt = _mla_case(rng, contexts)
+    rc, out, outb, lse = ORACLE.mla_decode(q, pool, table, ctx, vd, pt, sliding_window=window)
+    assert rc == 0
+    for b, n in enumerate(contexts):
+        first = max(0, n - window)
+        rows = pool[table[b, :(n + pt - 1) // pt]].reshape(-1, pool.shape[-1])[first:n]
+        live = n - first
+        pages = (live + pt - 1) // pt
+        trimmed = np.zeros((pages, pt, pool.shape[-1]), np.uint16)
+        trimmed.reshape(-1, pool.shape[-1])[:live] = rows
+        rc1, out1, outb1, lse1 = ORACLE.mla_decode(
+            q[b:b + 1], trimmed, np.arange(pages, dtype=np.int32)[None, :],
+            np.array([live], np.int32), vd, pt)
+        assert rc1 == 0
+        assert np.array_equal(out1[0], out[b]) and np.array_equal(lse1[0], lse[b])
