@@ -325,12 +325,16 @@ class Backend:
     @staticmethod
     def mla_requirement(batch, heads, key_dim, value_dim, page_tokens, pool_pages, table_stride,
                         max_context, contract=B.NUMERIC_BF16_F32_ACCUMULATE, deterministic=1,
-                        sliding_window=0):
+                        sliding_window=0, compressed_pool_pages=0, compressed_table_stride=0,
+                        max_compressed_tokens=0):
         r = B.MlaDecodeRequirement()
         r.batch, r.heads, r.key_dimension, r.value_dimension = batch, heads, key_dim, value_dim
         r.page_tokens, r.pool_pages, r.page_table_stride = page_tokens, pool_pages, table_stride
         r.max_context_tokens, r.numeric_contract, r.deterministic = max_context, contract, deterministic
         r.sliding_window = sliding_window
+        r.compressed_pool_pages = compressed_pool_pages
+        r.compressed_page_table_stride = compressed_table_stride
+        r.max_compressed_tokens = max_compressed_tokens
         return r
 
     def mla_decode_workspace_required(self, requirement):
@@ -341,14 +345,17 @@ class Backend:
         return out.value
 
     def mla_decode_execute(self, requirement, query, latent_pages, page_table, context, output,
-                           lse=None, sinks=None):
+                           lse=None, sinks=None, compressed=None):
+        """compressed: optional (pages, page table, visible row counts) device tensors."""
         ops = self.rocm_attention_operations()
         if ops is None:
             raise YvexError(B.YVEX_ERR_UNSUPPORTED, "rocm_attention_operations", "not published")
         request = B.MlaDecodeRequest(requirement, query.handle, latent_pages.handle,
                                      page_table.handle, context.handle, output.handle,
                                      lse.handle if lse else None,
-                                     sinks.handle if sinks else None)
+                                     sinks.handle if sinks else None,
+                                     *(x.handle for x in (compressed or (None, None, None))
+                                       if x is not None))
         facts, err = B.OperationFacts(), B.Error()
         _check(ops.mla_decode_execute(self.handle, C.byref(request), C.byref(facts),
                                       C.byref(err)), err)

@@ -147,13 +147,17 @@ class MlaDecodeRequirement(C.Structure):
     _fields_ = [(n, ull) for n in ("batch", "heads", "key_dimension", "value_dimension",
                                    "page_tokens", "pool_pages", "page_table_stride",
                                    "max_context_tokens")] + [
-        ("numeric_contract", C.c_int), ("deterministic", C.c_int), ("sliding_window", ull)]
+        ("numeric_contract", C.c_int), ("deterministic", C.c_int), ("sliding_window", ull),
+        ("compressed_pool_pages", ull), ("compressed_page_table_stride", ull),
+        ("max_compressed_tokens", ull)]
 
 
 class MlaDecodeRequest(C.Structure):
     _fields_ = [("requirement", MlaDecodeRequirement), ("query", TensorP),
                 ("latent_pages", TensorP), ("page_table", TensorP), ("context_tokens", TensorP),
-                ("output", TensorP), ("lse", TensorP), ("sinks", TensorP)]
+                ("output", TensorP), ("lse", TensorP), ("sinks", TensorP),
+                ("compressed_pages", TensorP), ("compressed_page_table", TensorP),
+                ("compressed_tokens", TensorP)]
 
 
 class KvAppendRequirement(C.Structure):

@@ -630,13 +630,19 @@ static int mla_validate(const yvex_rocm_mla_decode_requirement *r, const char *w
         r->value_dimension > r->key_dimension || !r->page_tokens || !r->pool_pages ||
         !r->page_table_stride || !r->max_context_tokens ||
         !yvex_core_u64_mul(r->page_table_stride, r->page_tokens, &capacity) ||
-        r->max_context_tokens > capacity)
+        r->max_context_tokens > capacity ||
+        (r->max_compressed_tokens &&
+         (!r->compressed_pool_pages || !r->compressed_page_table_stride ||
+          r->compressed_page_table_stride > 0xffffffffull ||
+          r->max_compressed_tokens > r->compressed_page_table_stride * r->page_tokens)))
         return refuse(err, YVEX_ERR_INVALID_ARG, where, "complete MLA decode geometry is required");
     if (r->heads != ROCM_MLA_HEADS || r->key_dimension != ROCM_MLA_KEY_DIM ||
         r->value_dimension != ROCM_MLA_VALUE_DIM || r->page_tokens != ROCM_MLA_PAGE_TOKENS ||
         r->numeric_contract != YVEX_TRANSFORMER_ATTENTION_NUMERIC_BF16_F32_ACCUMULATE ||
         !r->deterministic || r->pool_pages > 0x7fffffffull || capacity > 0x7fffffffull ||
-        r->batch > 65535ull || r->sliding_window > 0x7fffffffull)
+        r->batch > 65535ull || r->sliding_window > 0x7fffffffull ||
+        r->compressed_pool_pages > 0x7fffffffull ||
+        r->compressed_page_table_stride * r->page_tokens > 0x7fffffffull)
         return refuse(err, YVEX_ERR_UNSUPPORTED, where,
                       "ROCm MLA decode requires 128 heads, a 512+64 latent row, 64-token pages "
                       "and the deterministic bf16/fp32-accumulate contract");
@@ -655,34 +661,56 @@ static unsigned long long mla_live_tokens(const yvex_rocm_mla_decode_requirement
     return r->max_context_tokens;
 }
 
+static unsigned int mla_chunk_for(const yvex_rocm_mla_decode_requirement *r,
+                                  unsigned long long tokens, int windowed);
+
 static unsigned int mla_chunk_tokens(const yvex_rocm_mla_decode_requirement *r)
+{
+    return mla_chunk_for(r, mla_live_tokens(r), r->sliding_window != 0ull);
+}
+
+static unsigned int mla_chunk_for(const yvex_rocm_mla_decode_requirement *r,
+                                  unsigned long long tokens, int windowed)
 {
     const char *forced = getenv("YVEX_ROCM_MLA_CHUNK");
     unsigned long long per_batch = 256ull / r->batch ? 256ull / r->batch : 1ull;
-    unsigned long long chunk = (mla_live_tokens(r) + per_batch - 1ull) / per_batch;
+    unsigned long long chunk = (tokens + per_batch - 1ull) / per_batch;
     if (forced && atoi(forced) >= ROCM_MLA_PAGE_TOKENS) chunk = (unsigned long long)atoi(forced);
     chunk = align_up(chunk, ROCM_MLA_PAGE_TOKENS);
     /* a windowed chunk may start in the middle of a page and so touch one page more */
-    if (chunk > (unsigned long long)(YVEX_ROCM_MLA_MAX_CHUNK_PAGES - (r->sliding_window ? 1 : 0)) *
+    if (chunk > (unsigned long long)(YVEX_ROCM_MLA_MAX_CHUNK_PAGES - (windowed ? 1 : 0)) *
                     ROCM_MLA_PAGE_TOKENS)
-        chunk = (unsigned long long)(YVEX_ROCM_MLA_MAX_CHUNK_PAGES - (r->sliding_window ? 1 : 0)) *
+        chunk = (unsigned long long)(YVEX_ROCM_MLA_MAX_CHUNK_PAGES - (windowed ? 1 : 0)) *
                 ROCM_MLA_PAGE_TOKENS;
     return (unsigned int)chunk;
+}
+
+/* Chunk sizes and partial slots per batch element: the local set, then the compressed one. */
+static void mla_partition(const yvex_rocm_mla_decode_requirement *r, unsigned long long *chunk,
+                          unsigned long long *max_chunks, unsigned long long *extra_chunk,
+                          unsigned long long *extra_max_chunks)
+{
+    *chunk = mla_chunk_tokens(r);
+    *max_chunks = (mla_live_tokens(r) + *chunk - 1ull) / *chunk;
+    *extra_chunk = *extra_max_chunks = 0ull;
+    if (r->max_compressed_tokens) {
+        *extra_chunk = mla_chunk_for(r, r->max_compressed_tokens, 0);
+        *extra_max_chunks = (r->max_compressed_tokens + *extra_chunk - 1ull) / *extra_chunk;
+    }
 }
 
 static int rocm_mla_decode_workspace_required(const yvex_rocm_mla_decode_requirement *r,
                                               unsigned long long *bytes, yvex_error *err)
 {
     static const char where[] = "rocm.attention.mla.workspace";
-    unsigned long long acc = 0ull, total = 0ull, chunk, max_chunks;
+    unsigned long long acc = 0ull, total = 0ull, chunk, max_chunks, extra_chunk, extra_max_chunks;
     int rc;
     if (bytes) *bytes = 0ull;
     rc = mla_validate(r, where, err);
     if (rc != YVEX_OK) return rc;
     if (!bytes) return refuse(err, YVEX_ERR_INVALID_ARG, where, "workspace byte output is required");
-    chunk = mla_chunk_tokens(r);
-    max_chunks = (mla_live_tokens(r) + chunk - 1ull) / chunk;
-    if (!decode_workspace_bytes(r->batch * max_chunks, r->heads, r->value_dimension,
+    mla_partition(r, &chunk, &max_chunks, &extra_chunk, &extra_max_chunks);
+    if (!decode_workspace_bytes(r->batch * (max_chunks + extra_max_chunks), r->heads, r->value_dimension,
                                 sizeof(uint16_t), &acc, &total))
         return refuse(err, YVEX_ERR_BOUNDS, where, "MLA workspace geometry overflowed");
     *bytes = total;
@@ -700,7 +728,7 @@ static int rocm_mla_decode_execute(yvex_backend *backend,
     const yvex_rocm_mla_decode_requirement *r;
     yvex_rocm_mla_params kp;
     yvex_rocm_decode_merge_params mp;
-    unsigned long long acc_bytes = 0ull, total = 0ull, max_chunks, chunk;
+    unsigned long long acc_bytes = 0ull, total = 0ull, max_chunks, chunk, extra_chunk, extra_max_chunks;
     void *work = NULL;
     yvex_error cleanup;
     int owned = 0, rc, cleanup_rc;
@@ -723,14 +751,21 @@ static int rocm_mla_decode_execute(yvex_backend *backend,
         !view_ok(backend, request->output, YVEX_DTYPE_BF16,
                  r->batch * r->heads * r->value_dimension, 0) ||
         (request->lse && !view_ok(backend, request->lse, YVEX_DTYPE_F32, r->batch * r->heads, 0)) ||
-        (request->sinks && !view_ok(backend, request->sinks, YVEX_DTYPE_F32, r->heads, 1)))
+        (request->sinks && !view_ok(backend, request->sinks, YVEX_DTYPE_F32, r->heads, 1)) ||
+        (r->max_compressed_tokens &&
+         (!request->compressed_pages || !request->compressed_page_table ||
+          !request->compressed_tokens ||
+          !view_ok(backend, request->compressed_pages, YVEX_DTYPE_BF16,
+                   r->compressed_pool_pages * r->page_tokens * r->key_dimension, 1) ||
+          !view_ok(backend, request->compressed_page_table, YVEX_DTYPE_I32,
+                   r->batch * r->compressed_page_table_stride, 1) ||
+          !view_ok(backend, request->compressed_tokens, YVEX_DTYPE_I32, r->batch, 1))))
         return refuse(err, YVEX_ERR_FORMAT, where,
                       "query, latent pages, page table, context lengths and outputs must be "
                       "written tensors of this backend with the declared geometry");
-    chunk = mla_chunk_tokens(r);
-    max_chunks = (mla_live_tokens(r) + chunk - 1ull) / chunk;
-    if (max_chunks > 0x7fffffffull ||
-        !decode_workspace_bytes(r->batch * max_chunks, r->heads, r->value_dimension,
+    mla_partition(r, &chunk, &max_chunks, &extra_chunk, &extra_max_chunks);
+    if (max_chunks + extra_max_chunks > 0x7fffffffull ||
+        !decode_workspace_bytes(r->batch * (max_chunks + extra_max_chunks), r->heads, r->value_dimension,
                                 sizeof(uint16_t), &acc_bytes, &total))
         return refuse(err, YVEX_ERR_BOUNDS, where, "MLA decode geometry exceeds admitted range");
     backend_workspace_reset(backend);
@@ -754,10 +789,28 @@ static int rocm_mla_decode_execute(yvex_backend *backend,
     kp.chunk_tokens = (uint32_t)chunk;
     kp.max_chunks = (uint32_t)max_chunks;
     kp.window = (uint32_t)r->sliding_window;
+    kp.slot_stride = (uint32_t)(max_chunks + extra_max_chunks);
     /* src/graph/core.c:604: scale = 1/sqrt(head_dimension), here over the 576-lane key */
     kp.scale_log2 = (float)(1.4426950408889634 / sqrt((double)r->key_dimension));
     rc = yvex_rocm_launch(backend, YVEX_ROCM_FN_MLA_DECODE_BF16, variant, (unsigned int)max_chunks,
                           (unsigned int)r->batch, 1u, 256u, 0u, &kp, where, err);
+    if (rc == YVEX_OK && extra_max_chunks) {
+        /* the compressed rows: same kernel over the second pool, partials after the local ones */
+        yvex_rocm_mla_params cp = kp;
+        cp.pool = (const uint16_t *)request->compressed_pages->data;
+        cp.page_table = (const int32_t *)request->compressed_page_table->data;
+        cp.context = (const int32_t *)request->compressed_tokens->data;
+        cp.pool_pages = (uint32_t)r->compressed_pool_pages;
+        cp.table_stride = (uint32_t)r->compressed_page_table_stride;
+        cp.chunk_tokens = (uint32_t)extra_chunk;
+        cp.max_chunks = (uint32_t)extra_max_chunks;
+        cp.window = 0u;
+        cp.first_slot = (uint32_t)max_chunks;
+        cp.empty_ok = 1u;
+        rc = yvex_rocm_launch(backend, YVEX_ROCM_FN_MLA_DECODE_BF16, variant,
+                              (unsigned int)extra_max_chunks, (unsigned int)r->batch, 1u, 256u, 0u,
+                              &cp, where, err);
+    }
     if (rc == YVEX_OK) {
         memset(&mp, 0, sizeof(mp));
         mp.part_acc = kp.part_acc;
@@ -774,13 +827,18 @@ static int rocm_mla_decode_execute(yvex_backend *backend,
         mp.sinks = request->sinks ? (const float *)request->sinks->data : NULL;
         mp.window = kp.window;
         mp.window_align = ROCM_MLA_TILE_TOKENS;
+        if (extra_max_chunks) {
+            mp.extra_context = (const int32_t *)request->compressed_tokens->data;
+            mp.extra_chunk_tokens = (uint32_t)extra_chunk;
+            mp.extra_max_chunks = (uint32_t)extra_max_chunks;
+        }
         rc = yvex_rocm_launch(backend, YVEX_ROCM_FN_DECODE_MERGE, variant,
                               (unsigned int)((r->heads + 3ull) / 4ull), (unsigned int)r->batch, 1u,
                               256u, 0u, &mp, where, err);
     }
     if (rc == YVEX_OK) {
-        facts->kernel_launches = 2ull;
-        facts->accelerated_matrix_launches = 1ull;
+        facts->kernel_launches = extra_max_chunks ? 3ull : 2ull;
+        facts->accelerated_matrix_launches = extra_max_chunks ? 2ull : 1ull;
         facts->temporary_bytes = total;
         facts->compulsory_memory_facts_available = 1;
         rc = yvex_rocm_complete(backend, variant, where, facts, err);

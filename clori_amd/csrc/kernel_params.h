@@ -83,6 +83,10 @@ typedef struct {
     const float *sinks; /* optional F32 [query_heads]: one extra logit per head with value 0 */
     uint32_t window;    /* sliding window of the producing kernel (sets its first chunk) */
     uint32_t window_align; /* the producer starts its chunks at first_visible rounded down to this */
+    /* second candidate set: its chunks sit in slots max_chunks .. max_chunks + extra_max_chunks - 1
+     * of each batch element; extra_context NULL: none */
+    const int32_t *extra_context;
+    uint32_t extra_chunk_tokens, extra_max_chunks;
 } yvex_rocm_decode_merge_params;
 
 /* Causal / full GQA prefill on bf16 token-major tensors.  The grid is one-dimensional:
@@ -117,6 +121,10 @@ typedef struct {
     uint32_t window; /* sliding window in tokens, 0: the whole context */
     float scale_log2;
     float reserved_f;
+    uint32_t first_slot;  /* partial slot of chunk 0 (a second candidate set writes after the first) */
+    uint32_t slot_stride; /* partial slots per batch element, all sets together */
+    uint32_t empty_ok;    /* a context of 0 rows is an empty set, not a contract violation */
+    uint32_t reserved;
 } yvex_rocm_mla_params;
 
 /* KV page writer: new key/value rows -> paged pools (bf16 or Q8_0), rotary on the keys.

@@ -587,8 +587,14 @@ yvex_rocm_decode_merge(const yvex_rocm_decode_merge_params p)
     if (ctx == 0u || head >= p.query_heads || lane * 8u >= p.head_dim) return;
     const uint32_t first_visible = p.window != 0u && ctx > p.window ? ctx - p.window : 0u;
     const uint32_t live = ctx - (first_visible & ~(p.window_align - 1u));
-    const uint32_t chunks = min(p.max_chunks, (live + p.chunk_tokens - 1u) / p.chunk_tokens);
-    const uint64_t base = ((uint64_t)session * p.max_chunks) * p.query_heads + head;
+    const uint32_t own = min(p.max_chunks, (live + p.chunk_tokens - 1u) / p.chunk_tokens);
+    // the chunks of a second candidate set follow the max_chunks slots of the first
+    const uint32_t extra_ctx = p.extra_context ? (uint32_t)p.extra_context[session] : 0u;
+    const uint32_t extra = p.extra_context
+        ? min(p.extra_max_chunks, (extra_ctx + p.extra_chunk_tokens - 1u) / p.extra_chunk_tokens) : 0u;
+    const uint32_t chunks = own + extra, skip = p.max_chunks - own;
+    const uint64_t base =
+        ((uint64_t)session * (p.max_chunks + (p.extra_context ? p.extra_max_chunks : 0u))) * p.query_heads + head;
     // Sixteen chunks per trip, every load of a trip independent of the others (indices past
     // the end alias the last chunk with weight zero): one memory round trip per trip, which
     // is what keeps this pass in the microsecond range.
@@ -600,7 +606,8 @@ yvex_rocm_decode_merge(const yvex_rocm_decode_merge_params p)
         u32x4 row[16];
 #pragma unroll
         for (int j = 0; j < 16; ++j) {
-            const uint64_t slot = base + (uint64_t)min(c0 + (uint32_t)j, chunks - 1u) * p.query_heads;
+            const uint32_t c = min(c0 + (uint32_t)j, chunks - 1u);
+            const uint64_t slot = base + (uint64_t)(c < own ? c : c + skip) * p.query_heads;
             m[j] = p.part_ml[slot * 2];
             l[j] = p.part_ml[slot * 2 + 1];
             row[j] = load_b128(p.part_acc + slot * p.head_dim + lane * 8u);

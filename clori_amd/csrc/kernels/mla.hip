@@ -82,6 +82,7 @@ yvex_rocm_mla_decode_bf16(const yvex_rocm_mla_params p)
     const int n = lane & 31, g = lane >> 5;
     const uint32_t chunk = blockIdx.x, batch = blockIdx.y;
     const uint32_t ctx = (uint32_t)p.context[batch];
+    if (ctx == 0u && p.empty_ok != 0u) return;
     if (ctx == 0u || ctx > p.table_stride * p.page_tokens) {
         if (chunk == 0u && tid == 0) flag(p.status, YVEX_ROCM_DEVICE_CONTRACT);
         return;
@@ -360,7 +361,7 @@ yvex_rocm_mla_decode_bf16(const yvex_rocm_mla_params p)
 #endif
     float l = l_run;
     l += xor_lanes(l, 32);
-    const uint64_t slot = ((uint64_t)batch * p.max_chunks + chunk) * p.heads + head;
+    const uint64_t slot = ((uint64_t)batch * p.slot_stride + p.first_slot + chunk) * p.heads + head;
     // The accumulators are lane = head, registers = dims; through LDS they become one
     // contiguous 1 KB bf16 row per head, written by one 16-byte store per lane.
     constexpr int kOutPitch = kValueDim * 2 + 16;  // 1040 B, keeps 16-byte alignment
@@ -379,7 +380,7 @@ yvex_rocm_mla_decode_bf16(const yvex_rocm_mla_params p)
     // only this wave reads what it wrote: no workgroup barrier needed
     __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
     {
-        const uint64_t slot0 = ((uint64_t)batch * p.max_chunks + chunk) * p.heads + wave * kHeadsPerWave;
+        const uint64_t slot0 = ((uint64_t)batch * p.slot_stride + p.first_slot + chunk) * p.heads + wave * kHeadsPerWave;
         uint16_t *dst = p.part_acc + slot0 * kValueDim + lane * 8;
 #pragma unroll 8
         for (int hh = 0; hh < kHeadsPerWave; ++hh) {

@@ -400,6 +400,11 @@ typedef struct yvex_rocm_mla_decode_requirement {
      * (src/backend/cuda/attention_kernels.cu:79-84): the query at position context - 1 sees
      * positions >= context - sliding_window.  0: the whole context. */
     unsigned long long sliding_window;
+    /* Second candidate set of the shared-KV reduce: compressed rows visited after the local
+     * ones inside the same softmax (src/graph/core.c:437-468, the dense class whose visible
+     * rows are a prefix; attention_kernels.cu:85-97).  Same row format and page size as the
+     * latent pool.  max_compressed_tokens = 0: no such set. */
+    unsigned long long compressed_pool_pages, compressed_page_table_stride, max_compressed_tokens;
 } yvex_rocm_mla_decode_requirement;
 
 typedef struct yvex_rocm_mla_decode_request {
@@ -410,6 +415,11 @@ typedef struct yvex_rocm_mla_decode_request {
      * each seeds the head's maximum and adds exp(sink - max) to its denominator with a zero
      * value row; the LSE output includes it.  NULL: no sink. */
     const yvex_device_tensor *sinks;
+    /* With max_compressed_tokens > 0: BF16 [compressed_pool_pages][page_tokens][key_dimension],
+     * I32 [batch][compressed_page_table_stride], and I32 [batch] visible compressed rows per
+     * session (0 allowed: position + ratio - 1 <= token position holds for a prefix of
+     * floor(context / ratio) rows, which the caller passes). */
+    const yvex_device_tensor *compressed_pages, *compressed_page_table, *compressed_tokens;
 } yvex_rocm_mla_decode_request;
 
 /* KV page writer (no reference counterpart as one operation: it is the rotary step of

@@ -546,7 +546,10 @@ int yvo_mla_decode_bf16(const uint16_t *q, const uint16_t *pool,
                         uint64_t batch, uint64_t heads, uint64_t key_dim,
                         uint64_t value_dim, uint64_t page_tokens,
                         uint64_t pool_pages, uint64_t table_stride,
-                        const float *sinks, uint64_t sliding_window, int threads)
+                        const float *sinks, uint64_t sliding_window,
+                        const uint16_t *compressed_pool, const int32_t *compressed_table,
+                        const int32_t *compressed_count, uint64_t compressed_pool_pages,
+                        uint64_t compressed_table_stride, int threads)
 {
     uint64_t b;
     double scale;
@@ -564,6 +567,16 @@ int yvo_mla_decode_bf16(const uint16_t *q, const uint16_t *pool,
             int32_t id = page_table[b * table_stride + p];
             if (id < 0 || (uint64_t)id >= pool_pages) return YVO_ERR_BOUNDS;
         }
+        if (compressed_pool) {
+            if (!compressed_table || !compressed_count || compressed_count[b] < 0)
+                return YVO_ERR_INVALID_ARG;
+            pages = ((uint64_t)compressed_count[b] + page_tokens - 1u) / page_tokens;
+            if (pages > compressed_table_stride) return YVO_ERR_BOUNDS;
+            for (p = 0; p < pages; ++p) {
+                int32_t id = compressed_table[b * compressed_table_stride + p];
+                if (id < 0 || (uint64_t)id >= compressed_pool_pages) return YVO_ERR_BOUNDS;
+            }
+        }
     }
     /* src/graph/core.c:604 */
     scale = 1.0 / sqrt((double)key_dim);
@@ -574,12 +587,22 @@ int yvo_mla_decode_bf16(const uint16_t *q, const uint16_t *pool,
          * sees positions first .. context - 1, first = context - window (or 0) */
         const uint64_t total = (uint64_t)context[unit];
         const uint64_t first = sliding_window && total > sliding_window ? total - sliding_window : 0u;
-        uint64_t n = total - first, t, h;
+        /* src/graph/core.c:437-468: the compressed rows follow the local ones in the same
+         * two passes (one maximum, one denominator) */
+        const uint64_t extra = compressed_pool ? (uint64_t)compressed_count[unit] : 0u;
+        const uint64_t local = total - first;
+        uint64_t n = local + extra, t, h;
         float *rows = (float *)malloc((size_t)(n * key_dim) * sizeof(float));
         float *qf = (float *)malloc((size_t)key_dim * sizeof(float));
         float *of = (float *)malloc((size_t)value_dim * sizeof(float));
         int rc = rows && qf && of ? YVO_OK : YVO_ERR_STATE;
-        for (t = 0; rc == YVO_OK && t < n; ++t) {
+        for (t = 0; rc == YVO_OK && t < extra; ++t) {
+            uint64_t page = (uint64_t)compressed_table[(uint64_t)unit * compressed_table_stride +
+                                                       t / page_tokens];
+            yvo_bf16_decode_n(compressed_pool + (page * page_tokens + t % page_tokens) * key_dim,
+                              rows + (local + t) * key_dim, (size_t)key_dim);
+        }
+        for (t = 0; rc == YVO_OK && t < local; ++t) {
             const uint64_t at = first + t;
             uint64_t page = (uint64_t)page_table[(uint64_t)unit * table_stride + at / page_tokens];
             yvo_bf16_decode_n(pool + (page * page_tokens + at % page_tokens) * key_dim,

@@ -164,7 +164,9 @@ int yvo_shared_kv_head(const float *q, const float *rows, size_t row_stride,
  * sinks: optional F32 [heads] sink logits handed to yvo_shared_kv_head; sliding_window:
  * 0 for the whole context, else only positions >= context - sliding_window are rows
  * (the position filter of src/backend/cuda/attention_kernels.cu:79-84 for the token at
- * position context - 1).
+ * position context - 1).  compressed_pool (optional): a second paged row set of the same
+ * format; its first compressed_count[b] rows join the same softmax after the local rows
+ * (src/graph/core.c:437-468, the class whose visible compressed rows are a prefix).
  */
 int yvo_mla_decode_bf16(const uint16_t *q, const uint16_t *pool,
                         const int32_t *page_table, const int32_t *context,
@@ -172,7 +174,10 @@ int yvo_mla_decode_bf16(const uint16_t *q, const uint16_t *pool,
                         uint64_t batch, uint64_t heads, uint64_t key_dim,
                         uint64_t value_dim, uint64_t page_tokens,
                         uint64_t pool_pages, uint64_t table_stride,
-                        const float *sinks, uint64_t sliding_window, int threads);
+                        const float *sinks, uint64_t sliding_window,
+                        const uint16_t *compressed_pool, const int32_t *compressed_table,
+                        const int32_t *compressed_count, uint64_t compressed_pool_pages,
+                        uint64_t compressed_table_stride, int threads);
 
 /*
  * Log-sum-exp merge of split partials for one head: part p holds a normalised

@@ -27,11 +27,16 @@ def make_case(rng, contexts, spare=2):
     return q, pool, table, np.array(contexts, dtype=np.int32)
 
 
-def run_mla(backend, q, pool, table, ctx, max_context=None, sinks=None, window=0):
+def run_mla(backend, q, pool, table, ctx, max_context=None, sinks=None, window=0, compressed=None):
     batch = q.shape[0]
+    extra = {}
+    if compressed is not None:
+        extra = dict(compressed_pool_pages=compressed[0].shape[0],
+                     compressed_table_stride=compressed[1].shape[1],
+                     max_compressed_tokens=int(compressed[1].shape[1] * PAGE))
     req = backend.mla_requirement(batch, HEADS, KEY_DIM, VALUE_DIM, PAGE, pool.shape[0],
                                   table.shape[1], max_context or int(table.shape[1] * PAGE),
-                                  sliding_window=window)
+                                  sliding_window=window, **extra)
     out = backend.tensor("o", B.DTYPE_BF16, (batch, HEADS, VALUE_DIM))
     lse = backend.tensor("lse", B.DTYPE_F32, (batch, HEADS))
     tensors = [backend.tensor("q", B.DTYPE_BF16, q.shape, q),
@@ -39,9 +44,14 @@ def run_mla(backend, q, pool, table, ctx, max_context=None, sinks=None, window=0
                backend.tensor("table", B.DTYPE_I32, table.shape, table),
                backend.tensor("ctx", B.DTYPE_I32, ctx.shape, ctx)]
     ts = backend.tensor("sinks", B.DTYPE_F32, (HEADS,), sinks) if sinks is not None else None
-    facts = backend.mla_decode_execute(req, *tensors, out, lse, sinks=ts)
+    tc = None
+    if compressed is not None:
+        tc = [backend.tensor("cpool", B.DTYPE_BF16, compressed[0].shape, compressed[0]),
+              backend.tensor("ctable", B.DTYPE_I32, compressed[1].shape, compressed[1]),
+              backend.tensor("ccount", B.DTYPE_I32, compressed[2].shape, compressed[2])]
+    facts = backend.mla_decode_execute(req, *tensors, out, lse, sinks=ts, compressed=tc)
     result = out.read(), lse.read(), facts
-    for t in tensors + [out, lse] + ([ts] if ts else []):
+    for t in tensors + [out, lse] + ([ts] if ts else []) + (tc or []):
         t.release()
     return result
 
@@ -142,3 +152,24 @@ def test_mla_non_finite_sink_is_a_numeric_failure(backend):
     with pytest.raises(YvexError) as e:
         run_mla(backend, q, pool, table, ctx, sinks=sinks)
     assert e.value.code == B.YVEX_ERR_FORMAT
+
+
+@pytest.mark.parametrize("window", [0, 128])
+def test_mla_compressed_candidate_rows(backend, window):
+    """A second paged row set (compressed rows, src/graph/core.c:437-468) in the same softmax:
+    counts of 0, below one tile, across pages and chunks; with sinks and a local window."""
+    rng = np.random.default_rng(600 + window)
+    contexts = [1, 70, 128, 129, 1000, 4097, 8192, 300]
+    counts = [0, 1, 31, 64, 65, 32, 64, 700]
+    q, pool, table, ctx = make_case(rng, contexts)
+    _, cpool, ctable, _ = make_case(rng, [max(c, 1) for c in counts])
+    ccount = np.array(counts, np.int32)
+    sinks = (rng.standard_normal(HEADS) * 2.0).astype(np.float32)
+    got, lse, facts = run_mla(backend, q, pool, table, ctx, sinks=sinks, window=window,
+                              compressed=(cpool, ctable, ccount))
+    rc, ref, _, ref_lse = ORACLE.mla_decode(q, pool, table, ctx, VALUE_DIM, PAGE, sinks=sinks,
+                                            sliding_window=window, compressed=(cpool, ctable, ccount))
+    assert rc == 0
+    assert_close_bf16(got, ref, "mla compressed window=%d" % window)
+    assert_lse(lse, ref_lse, "mla compressed window=%d" % window)
+    assert facts.kernel_launches == 3 and facts.accelerated_matrix_launches == 2

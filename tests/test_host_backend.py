@@ -411,6 +411,21 @@ def test_paged_and_mla_admission():
         mout = b.tensor("mo", B.DTYPE_BF16, (16, 128, 512))
         sinks = written(b, "sinks", B.DTYPE_F32, (128,))
         assert b.mla_decode_execute(windowed, mq, latent, mtable, mctx, mout, sinks=sinks).kernel_launches == 2
+        both = b.mla_requirement(16, 128, 576, 512, 64, 2048, 128, 8192, compressed_pool_pages=40,
+                                 compressed_table_stride=2, max_compressed_tokens=128)
+        assert b.mla_decode_workspace_required(both) > b.mla_decode_workspace_required(mla)
+        cpool = written(b, "cp", B.DTYPE_BF16, (40, 64, 576))
+        ctable, ccount = written(b, "ct", B.DTYPE_I32, (16, 2)), written(b, "cc", B.DTYPE_I32, (16,))
+        facts = b.mla_decode_execute(both, mq, latent, mtable, mctx, mout, compressed=[cpool, ctable, ccount])
+        assert facts.kernel_launches == 3
+        with pytest.raises(YvexError) as e:                 # declared but not passed
+            b.mla_decode_execute(both, mq, latent, mtable, mctx, mout)
+        assert e.value.code == B.YVEX_ERR_FORMAT
+        with pytest.raises(YvexError) as e:                 # more rows than the table can address
+            b.mla_decode_workspace_required(b.mla_requirement(
+                16, 128, 576, 512, 64, 2048, 128, 8192, compressed_pool_pages=40,
+                compressed_table_stride=2, max_compressed_tokens=129))
+        assert e.value.code == B.YVEX_ERR_INVALID_ARG
         for wrong in (written(b, "s1", B.DTYPE_F32, (64,)), written(b, "s2", B.DTYPE_BF16, (128,)),
                       b.tensor("s3", B.DTYPE_F32, (128,))):
             with pytest.raises(YvexError) as e:

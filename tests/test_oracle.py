@@ -592,3 +592,33 @@ def test_mla_sliding_window_equals_decode_on_the_trimmed_context(window):
             np.array([live], np.int32), vd, pt)
         assert rc1 == 0
         assert np.array_equal(out1[0], out[b]) and np.array_equal(lse1[0], lse[b])
+
+
+def test_mla_compressed_rows_join_the_same_softmax_after_the_local_rows():
+    """Local window rows then the visible compressed prefix == one context holding those rows in
+    that order, bit for bit; an empty compressed set changes nothing."""
+    rng = np.random.default_rng(68)
+    contexts, counts, window = [3, 40, 130], [0, 5, 33], 32
+    q, pool, table, ctx, vd, pt = _mla_case(rng, contexts)
+    _, cpool, ctable, ccount, _, _ = _mla_case(rng, [max(c, 1) for c in counts])
+    ccount = np.array(counts, np.int32)
+    sinks = np.array([0.5, -1.0, 2.0, 0.0], np.float32)
+    rc, out, _, lse = ORACLE.mla_decode(q, pool, table, ctx, vd, pt, sinks=sinks,
+                                        sliding_window=window, compressed=(cpool, ctable, ccount))
+    assert rc == 0
+    kd = pool.shape[-1]
+    for b, n in enumerate(contexts):
+        first = max(0, n - window)
+        rows = np.concatenate([
+            pool[table[b, :(n + pt - 1) // pt]].reshape(-1, kd)[first:n],
+            cpool[ctable[b, :(counts[b] + pt - 1) // pt]].reshape(-1, kd)[:counts[b]]])
+        pages = (len(rows) + pt - 1) // pt
+        joined = np.zeros((pages, pt, kd), np.uint16)
+        joined.reshape(-1, kd)[:len(rows)] = rows
+        rc1, out1, _, lse1 = ORACLE.mla_decode(q[b:b + 1], joined, np.arange(pages, dtype=np.int32)[None, :],
+                                               np.array([len(rows)], np.int32), vd, pt, sinks=sinks)
+        assert rc1 == 0 and np.array_equal(out1[0], out[b]) and np.array_equal(lse1[0], lse[b])
+    rc2, out2, _, lse2 = ORACLE.mla_decode(q, pool, table, ctx, vd, pt, sinks=sinks, sliding_window=window,
+                                           compressed=(cpool, ctable, np.zeros(3, np.int32)))
+    rc3, out3, _, lse3 = ORACLE.mla_decode(q, pool, table, ctx, vd, pt, sinks=sinks, sliding_window=window)
+    assert rc2 == 0 and rc3 == 0 and np.array_equal(out2, out3) and np.array_equal(lse2, lse3)
