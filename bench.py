@@ -51,22 +51,34 @@ def random_bf16(rng, count, unique=1 << 24):
     return np.tile(base, reps)[:count]
 
 
+RECORDED_STEPS = bool(int(os.environ.get("YVEX_BENCH_RECORDED", "0")))
+
+
 def time_steps(backend, run, steps, warmup, kernel):
     """W untimed steps, then K steps bracketed by device events and by a synchronise on
     both sides; then the same K steps again with an event pair around every launch of the
     dominant kernel.  Returns (device ms per step, wall ms per step, ms per launch of the
     dominant kernel)."""
     backend.set_completion_mode(B.COMPLETION_DEFERRED)
-    for _ in range(warmup):
+    step, graph = run, None
+    if RECORDED_STEPS:
+        # the step's launches recorded once and replayed with one call per step
+        backend.graph_begin()
         run()
+        graph = backend.graph_end()
+        step = lambda: backend.graph_launch(graph)  # noqa: E731
+    for _ in range(warmup):
+        step()
     backend.sync()
     t0 = time.perf_counter()
     backend.timing_begin()
     for _ in range(steps):
-        run()
+        step()
     device_ms = backend.timing_end()
     backend.sync()
     wall_ms = (time.perf_counter() - t0) * 1e3
+    if graph is not None:
+        backend.graph_release(graph)
     backend.kernel_probe_begin(kernel)
     for _ in range(min(steps, 256)):
         run()

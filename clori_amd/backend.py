@@ -184,6 +184,27 @@ class Backend:
         _check(lib().yvex_backend_rocm_timing_end(self.handle, C.byref(ms), C.byref(err)), err)
         return ms.value
 
+    # -- recorded launch sequences -------------------------------------
+    def graph_begin(self):
+        err = B.Error()
+        _check(lib().yvex_backend_rocm_graph_begin(self.handle, C.byref(err)), err)
+
+    def graph_end(self):
+        """Ends the recording and returns the handle of the recorded sequence."""
+        graph, err = C.c_void_p(), B.Error()
+        _check(lib().yvex_backend_rocm_graph_end(self.handle, C.byref(graph), C.byref(err)), err)
+        return graph
+
+    def graph_launch(self, graph):
+        facts, err = B.OperationFacts(), B.Error()
+        _check(lib().yvex_backend_rocm_graph_launch(self.handle, graph, C.byref(facts),
+                                                    C.byref(err)), err)
+        return facts
+
+    def graph_release(self, graph):
+        err = B.Error()
+        _check(lib().yvex_backend_rocm_graph_release(self.handle, C.byref(graph), C.byref(err)), err)
+
     def kernel_probe_begin(self, kernel):
         """Brackets every launch of the named bundle kernel with its own event pair."""
         err = B.Error()

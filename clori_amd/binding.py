@@ -245,6 +245,8 @@ EXPORTED_SYMBOLS = [
     "yvex_backend_rocm_attention_operations_get", "yvex_backend_rocm_completion_mode_set",
     "yvex_backend_rocm_timing_begin", "yvex_backend_rocm_timing_end",
     "yvex_backend_rocm_kernel_probe_begin", "yvex_backend_rocm_kernel_probe_end",
+    "yvex_backend_rocm_graph_begin", "yvex_backend_rocm_graph_end",
+    "yvex_backend_rocm_graph_launch", "yvex_backend_rocm_graph_release",
     "yvex_backend_rocm_report_get", "yvex_quant_f16_decode", "yvex_quant_f16_encode",
     "yvex_quant_bf16_decode", "yvex_quant_bf16_encode", "yvex_rocm_q8_0_encode_row",
     "yvex_rocm_q8_0_decode_row", "yvex_rocm_kv_page_block_bytes", "yvex_rocm_kv_pack_pages",
@@ -315,6 +317,10 @@ def load(path=None):
     lib.yvex_backend_rocm_timing_end.argtypes = [vp, C.POINTER(C.c_double), ErrorP]
     lib.yvex_backend_rocm_kernel_probe_begin.argtypes = [vp, C.c_char_p, ErrorP]
     lib.yvex_backend_rocm_kernel_probe_end.argtypes = [vp, C.POINTER(C.c_uint), C.POINTER(C.c_double), ErrorP]
+    lib.yvex_backend_rocm_graph_begin.argtypes = [vp, ErrorP]
+    lib.yvex_backend_rocm_graph_end.argtypes = [vp, C.POINTER(C.c_void_p), ErrorP]
+    lib.yvex_backend_rocm_graph_launch.argtypes = [vp, C.c_void_p, FactsP, ErrorP]
+    lib.yvex_backend_rocm_graph_release.argtypes = [vp, C.POINTER(C.c_void_p), ErrorP]
     lib.yvex_backend_rocm_report_get.argtypes = [vp, C.POINTER(RocmReport), ErrorP]
     lib.yvex_quant_f16_decode.restype = C.c_float
     lib.yvex_quant_f16_decode.argtypes = [C.c_ushort]

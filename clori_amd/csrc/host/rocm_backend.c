@@ -91,6 +91,9 @@ static int rocm_tensor_free(yvex_backend *backend, yvex_device_tensor *tensor, y
         return refuse(err, YVEX_ERR_INVALID_ARG, where, "backend and tensor are required");
     if (!backend_tensor_owner_is(backend, tensor))
         return refuse(err, YVEX_ERR_STATE, where, "tensor does not belong to this backend");
+    if (state->recording)
+        return refuse(err, YVEX_ERR_STATE, where,
+                      "not available while a launch sequence is being recorded");
     if (backend->workspace_device_tensor == tensor) yvex_backend_workspace_detach(backend);
     /* nothing may still read the allocation: drain the stream first */
     rc = yvex_rocm_status(&state->driver, state->driver.hipStreamSynchronize(state->stream), where,
@@ -197,6 +200,9 @@ static int rocm_tensor_copy(yvex_backend *backend, yvex_device_tensor *dst,
 static int rocm_sync(yvex_backend *backend, yvex_error *err)
 {
     yvex_rocm_backend_state *state = yvex_rocm_state(backend);
+    if (state && state->recording)
+        return refuse(err, YVEX_ERR_STATE, "rocm.sync",
+                      "cannot wait for the stream while a launch sequence is being recorded");
     if (state && state->status_dirty)
         return yvex_rocm_status_check(backend, "rocm.sync.status", NULL, err);
     return yvex_rocm_synchronize(backend, YVEX_BACKEND_VARIANT_TENSOR_READ, "rocm.sync", err);
@@ -244,6 +250,9 @@ int yvex_rocm_temporary_acquire(yvex_backend *backend, unsigned long long bytes,
     }
     if (hit == YVEX_BACKEND_RESIDENT_INVALID)
         return refuse(err, YVEX_ERR_BOUNDS, where, "temporary workspace geometry is invalid");
+    if (state->recording)
+        return refuse(err, YVEX_ERR_STATE, where,
+                      "a recorded operation needs an attached workspace that holds its temporaries");
     if (getenv("YVEX_TEST_ROCM_ATTENTION_FAILURE") &&
         strcmp(getenv("YVEX_TEST_ROCM_ATTENTION_FAILURE"), "allocation") == 0)
         return refuse(err, YVEX_ERR_NOMEM, where, "injected ROCm temporary allocation failure");
@@ -288,6 +297,12 @@ static int rocm_close(yvex_backend *backend, yvex_error *err)
     if (!state) {
         yvex_error_clear(err);
         return YVEX_OK;
+    }
+    if (state->recording) { /* an abandoned recording: end it and drop what it held */
+        hipGraph_t dropped = NULL;
+        (void)state->driver.hipStreamEndCapture(state->stream, &dropped);
+        if (dropped) (void)state->driver.hipGraphDestroy(dropped);
+        state->recording = 0;
     }
     if (state->stream) (void)state->driver.hipStreamSynchronize(state->stream);
     rc = yvex_rocm_kernel_bundle_close(backend, err);
@@ -455,6 +470,9 @@ int yvex_backend_rocm_completion_mode_set(yvex_backend *backend, yvex_rocm_compl
                       "ROCm backend and a known completion mode are required");
     rc = backend_dispatch_admit(backend, "rocm.completion_mode", err);
     if (rc != YVEX_OK) return rc;
+    if (state->recording)
+        return refuse(err, YVEX_ERR_STATE, "rocm.completion_mode",
+                      "not available while a launch sequence is being recorded");
     if (state->status_dirty) {
         rc = yvex_rocm_status_check(backend, "rocm.completion_mode", NULL, err);
         if (rc != YVEX_OK) return rc;
@@ -543,6 +561,9 @@ int yvex_backend_rocm_timing_begin(yvex_backend *backend, yvex_error *err)
     if (!state) return refuse(err, YVEX_ERR_INVALID_ARG, "rocm.timing", "ROCm backend is required");
     rc = backend_dispatch_admit(backend, "rocm.timing", err);
     if (rc != YVEX_OK) return rc;
+    if (state->recording)
+        return refuse(err, YVEX_ERR_STATE, "rocm.timing",
+                      "not available while a launch sequence is being recorded");
     rc = yvex_rocm_status(&state->driver,
                           state->driver.hipEventRecord(state->timing_start, state->stream),
                           "rocm.timing.begin", err);
@@ -555,8 +576,9 @@ int yvex_backend_rocm_timing_end(yvex_backend *backend, double *milliseconds, yv
     yvex_rocm_backend_state *state = yvex_rocm_state(backend);
     float elapsed = 0.0f;
     int rc;
-    if (!state || !milliseconds || !state->timing_active)
-        return refuse(err, YVEX_ERR_STATE, "rocm.timing.end", "timing was not started");
+    if (!state || !milliseconds || !state->timing_active || state->recording)
+        return refuse(err, YVEX_ERR_STATE, "rocm.timing.end",
+                      "timing was not started, or a launch sequence is being recorded");
     rc = yvex_rocm_status(&state->driver,
                           state->driver.hipEventRecord(state->timing_stop, state->stream),
                           "rocm.timing.end", err);
@@ -571,6 +593,127 @@ int yvex_backend_rocm_timing_end(yvex_backend *backend, double *milliseconds, yv
     state->timing_active = 0;
     if (rc != YVEX_OK) return rc;
     *milliseconds = (double)elapsed;
+    yvex_error_clear(err);
+    return YVEX_OK;
+}
+
+/* ---------------------------------------------- recorded launch sequences ---- */
+
+int yvex_backend_rocm_graph_begin(yvex_backend *backend, yvex_error *err)
+{
+    static const char where[] = "rocm.graph.begin";
+    yvex_rocm_backend_state *state = yvex_rocm_state(backend);
+    int rc;
+    if (!state) return refuse(err, YVEX_ERR_INVALID_ARG, where, "ROCm backend is required");
+    rc = backend_dispatch_admit(backend, where, err);
+    if (rc != YVEX_OK) return rc;
+    if (state->recording)
+        return refuse(err, YVEX_ERR_STATE, where, "a launch sequence is already being recorded");
+    if (state->kernel_bundle_state != YVEX_ROCM_KERNEL_BUNDLE_ADMITTED)
+        return refuse(err, YVEX_ERR_UNSUPPORTED, where, "no kernel bundle is admitted");
+    if (state->timing_active || state->probe_function >= 0)
+        return refuse(err, YVEX_ERR_STATE, where, "close the timing or probe section first");
+    /* earlier deferred work is checked before the stream stops executing */
+    if (state->status_dirty) {
+        rc = yvex_rocm_status_check(backend, where, NULL, err);
+        if (rc != YVEX_OK) return rc;
+    }
+    rc = yvex_rocm_status(&state->driver,
+                          state->driver.hipStreamBeginCapture(state->stream,
+                                                              hipStreamCaptureModeThreadLocal),
+                          where, err);
+    if (rc != YVEX_OK) return rc;
+    state->recording = 1;
+    state->recorded_launches = 0ull;
+    yvex_error_clear(err);
+    return YVEX_OK;
+}
+
+int yvex_backend_rocm_graph_end(yvex_backend *backend, yvex_rocm_graph **out, yvex_error *err)
+{
+    static const char where[] = "rocm.graph.end";
+    yvex_rocm_backend_state *state = yvex_rocm_state(backend);
+    yvex_rocm_graph *graph;
+    hipGraph_t captured = NULL;
+    int rc;
+    if (out) *out = NULL;
+    if (!state || !out) return refuse(err, YVEX_ERR_INVALID_ARG, where, "backend and out are required");
+    if (!state->recording) return refuse(err, YVEX_ERR_STATE, where, "no launch sequence is being recorded");
+    rc = yvex_rocm_status(&state->driver, state->driver.hipStreamEndCapture(state->stream, &captured),
+                          where, err);
+    state->recording = 0;
+    if (rc != YVEX_OK) {
+        if (captured) (void)state->driver.hipGraphDestroy(captured);
+        return rc;
+    }
+    graph = (yvex_rocm_graph *)calloc(1u, sizeof(*graph));
+    if (!graph) {
+        (void)state->driver.hipGraphDestroy(captured);
+        return refuse(err, YVEX_ERR_NOMEM, where, "out of host memory");
+    }
+    graph->graph = captured;
+    graph->kernel_launches = state->recorded_launches;
+    rc = yvex_rocm_status(&state->driver,
+                          state->driver.hipGraphInstantiate(&graph->executable, captured, NULL, NULL, 0u),
+                          where, err);
+    if (rc != YVEX_OK) {
+        (void)state->driver.hipGraphDestroy(captured);
+        free(graph);
+        return rc;
+    }
+    state->live_graphs++;
+    *out = graph;
+    yvex_error_clear(err);
+    return YVEX_OK;
+}
+
+int yvex_backend_rocm_graph_launch(yvex_backend *backend, yvex_rocm_graph *graph,
+                                   yvex_backend_operation_facts *facts, yvex_error *err)
+{
+    static const char where[] = "rocm.graph.launch";
+    yvex_rocm_backend_state *state = yvex_rocm_state(backend);
+    int rc;
+    if (!state || !graph || !graph->executable)
+        return refuse(err, YVEX_ERR_INVALID_ARG, where, "backend and a recorded sequence are required");
+    rc = backend_dispatch_admit(backend, where, err);
+    if (rc != YVEX_OK) return rc;
+    if (state->recording)
+        return refuse(err, YVEX_ERR_STATE, where, "a launch sequence is being recorded");
+    if (facts) memset(facts, 0, sizeof(*facts));
+    rc = yvex_rocm_status(&state->driver, state->driver.hipGraphLaunch(graph->executable, state->stream),
+                          where, err);
+    if (rc != YVEX_OK) {
+        state->backend_failure_reason = YVEX_BACKEND_CAPABILITY_REASON_LAUNCH_FAILED;
+        backend->status = YVEX_BACKEND_STATUS_FAILED;
+        return rc;
+    }
+    if (facts) {
+        facts->kernel_launches = graph->kernel_launches;
+        facts->compulsory_memory_facts_available = 1;
+    }
+    return yvex_rocm_complete(backend, YVEX_BACKEND_VARIANT_TENSOR_READ, where, facts, err);
+}
+
+int yvex_backend_rocm_graph_release(yvex_backend *backend, yvex_rocm_graph **graph, yvex_error *err)
+{
+    static const char where[] = "rocm.graph.release";
+    yvex_rocm_backend_state *state = yvex_rocm_state(backend);
+    int rc;
+    if (!state || !graph) return refuse(err, YVEX_ERR_INVALID_ARG, where, "backend and graph are required");
+    if (!*graph) {
+        yvex_error_clear(err);
+        return YVEX_OK;
+    }
+    if (state->recording)
+        return refuse(err, YVEX_ERR_STATE, where, "a launch sequence is being recorded");
+    /* a replay may still be running */
+    rc = yvex_rocm_status(&state->driver, state->driver.hipStreamSynchronize(state->stream), where, err);
+    if (rc != YVEX_OK) return rc;
+    if ((*graph)->executable) (void)state->driver.hipGraphExecDestroy((*graph)->executable);
+    if ((*graph)->graph) (void)state->driver.hipGraphDestroy((*graph)->graph);
+    free(*graph);
+    *graph = NULL;
+    if (state->live_graphs) state->live_graphs--;
     yvex_error_clear(err);
     return YVEX_OK;
 }

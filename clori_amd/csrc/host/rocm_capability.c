@@ -304,8 +304,15 @@ int yvex_rocm_require_capability(yvex_backend *backend, yvex_backend_operation_v
                                  const char *where, yvex_error *err)
 {
     yvex_backend_capability_result result;
+    const yvex_rocm_backend_state *state = yvex_rocm_state(backend);
     int rc = yvex_backend_query_capability(backend, variant, &result, err);
     if (rc != YVEX_OK) return rc;
+    /* tensor traffic allocates, copies, clears or waits: none of it can be recorded */
+    if (state && state->recording && variant <= YVEX_BACKEND_VARIANT_TENSOR_COPY) {
+        yvex_error_set(err, YVEX_ERR_STATE, where ? where : "rocm.require_capability",
+                       "not available while a launch sequence is being recorded");
+        return YVEX_ERR_STATE;
+    }
     if (result.state == YVEX_BACKEND_CAPABILITY_SUPPORTED) return YVEX_OK;
     rc = result.state == YVEX_BACKEND_CAPABILITY_FAILED ? YVEX_ERR_BACKEND : YVEX_ERR_UNSUPPORTED;
     yvex_error_setf(err, rc, where ? where : "rocm.require_capability", "%s refused: %s",
@@ -351,7 +358,8 @@ int yvex_rocm_launch(yvex_backend *backend, yvex_rocm_function_id function,
         return YVEX_ERR_BACKEND;
     }
     arguments[0] = params;
-    probe = state->probe_function == (int)function && state->probe_count < YVEX_ROCM_PROBE_MAX;
+    probe = !state->recording && state->probe_function == (int)function &&
+            state->probe_count < YVEX_ROCM_PROBE_MAX;
     if (probe)
         probe = state->driver.hipEventRecord(state->probe_events[2u * state->probe_count],
                                              state->stream) == hipSuccess;
@@ -366,6 +374,7 @@ int yvex_rocm_launch(yvex_backend *backend, yvex_rocm_function_id function,
                                      state->stream) == hipSuccess)
         state->probe_count++;
     if (rc != YVEX_OK) capability_fail(backend, variant, YVEX_BACKEND_CAPABILITY_REASON_LAUNCH_FAILED);
+    else if (state->recording) state->recorded_launches++;
     return rc;
 }
 
@@ -378,6 +387,11 @@ int yvex_rocm_synchronize(yvex_backend *backend, yvex_backend_operation_variant 
     if (rc != YVEX_OK) return rc;
     if (!state) {
         yvex_error_set(err, YVEX_ERR_STATE, where, "ROCm backend state is missing");
+        return YVEX_ERR_STATE;
+    }
+    if (state->recording) {
+        yvex_error_set(err, YVEX_ERR_STATE, where,
+                       "cannot wait for the stream while a launch sequence is being recorded");
         return YVEX_ERR_STATE;
     }
     if (test_failure_matches("YVEX_TEST_ROCM_SYNC_FAILURE", variant)) {
@@ -400,6 +414,11 @@ int yvex_rocm_status_check(yvex_backend *backend, const char *where,
     yvex_rocm_backend_state *state = yvex_rocm_state(backend);
     int32_t host_status = 0;
     int rc;
+    if (state->recording) {
+        yvex_error_set(err, YVEX_ERR_STATE, where,
+                       "cannot read the device status while a launch sequence is being recorded");
+        return YVEX_ERR_STATE;
+    }
     rc = yvex_rocm_status(&state->driver,
                           state->driver.hipMemcpyAsync(&host_status, state->device_status,
                                                        sizeof(host_status), hipMemcpyDeviceToHost,
@@ -443,6 +462,10 @@ int yvex_rocm_complete(yvex_backend *backend, yvex_backend_operation_variant var
 {
     yvex_rocm_backend_state *state = yvex_rocm_state(backend);
     (void)variant;
+    if (state->recording) { /* nothing ran: the replay completes the operation */
+        yvex_error_clear(err);
+        return YVEX_OK;
+    }
     if (state->completion_mode == YVEX_ROCM_COMPLETION_DEFERRED) {
         state->status_dirty = 1;
         yvex_error_clear(err);

@@ -58,7 +58,17 @@ typedef struct yvex_rocm_backend_state {
     int status_dirty;       /* deferred mode: launches since the last check */
     yvex_rocm_completion_mode completion_mode;
     unsigned long long live_tensors;
+    int recording;                  /* a launch sequence is being recorded on the stream */
+    unsigned long long live_graphs; /* recorded sequences not yet released */
+    unsigned long long recorded_launches; /* kernel launches of the sequence being recorded */
 } yvex_rocm_backend_state;
+
+/* A recorded launch sequence (rocm_backend.c). */
+struct yvex_rocm_graph {
+    hipGraph_t graph;
+    hipGraphExec_t executable;
+    unsigned long long kernel_launches;
+};
 
 static inline yvex_rocm_backend_state *yvex_rocm_state(const yvex_backend *backend)
 {

@@ -497,6 +497,27 @@ typedef enum {
 int yvex_backend_rocm_completion_mode_set(yvex_backend *backend, yvex_rocm_completion_mode mode,
                                           yvex_error *err);
 
+/*
+ * Recorded launch sequences (no reference counterpart; for launch-bound steps such as a
+ * single-session decode, where two kernel launches cost more host time than device time).
+ * Between begin and end the attention operations of this backend are recorded on its stream
+ * instead of being run: they validate and launch as usual but nothing executes, no status is
+ * read, and results are undefined until the sequence is replayed.  Everything that would
+ * allocate, free, copy, clear or wait is refused with YVEX_ERR_STATE while recording: attach
+ * a workspace large enough for the recorded operations first.  launch() enqueues the whole
+ * sequence with one call and then completes like any operation (status check in the
+ * immediate mode, at the next sync in the deferred mode).  The tensors the recorded
+ * operations named must stay allocated, at the same geometry, until the sequence is
+ * released; their contents may change between replays.
+ */
+typedef struct yvex_rocm_graph yvex_rocm_graph;
+int yvex_backend_rocm_graph_begin(yvex_backend *backend, yvex_error *err);
+int yvex_backend_rocm_graph_end(yvex_backend *backend, yvex_rocm_graph **out, yvex_error *err);
+int yvex_backend_rocm_graph_launch(yvex_backend *backend, yvex_rocm_graph *graph,
+                                   yvex_backend_operation_facts *facts, yvex_error *err);
+int yvex_backend_rocm_graph_release(yvex_backend *backend, yvex_rocm_graph **graph,
+                                    yvex_error *err);
+
 /* Device-event timing on the backend's stream (cf. yvex_cuda_timing,
  * src/backend/cuda/private.h:421-428).  end() synchronises and returns milliseconds. */
 int yvex_backend_rocm_timing_begin(yvex_backend *backend, yvex_error *err);

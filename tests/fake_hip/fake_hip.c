@@ -14,6 +14,8 @@
 #include <string.h>
 
 static unsigned long long launches, allocations, frees, loads, unloads;
+static int capturing;                       /* a stream capture is open */
+static unsigned long long captured_launches;
 
 unsigned long long fake_hip_launches(void) { return launches; }
 unsigned long long fake_hip_live_allocations(void) { return allocations - frees; }
@@ -151,7 +153,8 @@ hipError_t hipModuleLaunchKernel(hipFunction_t f, unsigned int gx, unsigned int 
     (void)f; (void)gx; (void)gy; (void)gz; (void)bx; (void)by; (void)bz;
     (void)shared; (void)stream; (void)params; (void)extra;
     if (env_is("FAKE_HIP_LAUNCH", "fail")) return hipErrorLaunchFailure;
-    ++launches;
+    if (capturing) ++captured_launches;
+    else ++launches;
     return hipSuccess;
 }
 
@@ -172,3 +175,48 @@ hipError_t hipEventElapsedTime(float *ms, hipEvent_t start, hipEvent_t stop)
     *ms = 1.0f;
     return hipSuccess;
 }
+
+/* Stream capture: while a capture is open launches are counted into the graph instead of
+ * the launch counter; a replay adds them. */
+struct fake_graph { unsigned long long launches; };
+
+hipError_t hipStreamBeginCapture(hipStream_t stream, hipStreamCaptureMode mode)
+{
+    (void)stream; (void)mode;
+    if (capturing) return hipErrorIllegalState;
+    capturing = 1;
+    captured_launches = 0;
+    return hipSuccess;
+}
+
+hipError_t hipStreamEndCapture(hipStream_t stream, hipGraph_t *graph)
+{
+    struct fake_graph *g;
+    (void)stream;
+    if (!capturing) return hipErrorIllegalState;
+    capturing = 0;
+    g = (struct fake_graph *)calloc(1, sizeof(*g));
+    g->launches = captured_launches;
+    *graph = (hipGraph_t)g;
+    return hipSuccess;
+}
+
+hipError_t hipGraphInstantiate(hipGraphExec_t *exec, hipGraph_t graph, hipGraphNode_t *error_node,
+                               char *log, size_t log_size)
+{
+    struct fake_graph *g = (struct fake_graph *)calloc(1, sizeof(*g));
+    (void)error_node; (void)log; (void)log_size;
+    g->launches = ((struct fake_graph *)graph)->launches;
+    *exec = (hipGraphExec_t)g;
+    return hipSuccess;
+}
+
+hipError_t hipGraphLaunch(hipGraphExec_t exec, hipStream_t stream)
+{
+    (void)stream;
+    launches += ((struct fake_graph *)exec)->launches;
+    return hipSuccess;
+}
+
+hipError_t hipGraphExecDestroy(hipGraphExec_t exec) { free(exec); return hipSuccess; }
+hipError_t hipGraphDestroy(hipGraph_t graph) { free(graph); return hipSuccess; }

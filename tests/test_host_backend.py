@@ -517,6 +517,51 @@ def test_fused_gate_admission():
         assert e.value.code == B.YVEX_ERR_FORMAT
 
 
+def test_recorded_sequence_rules(fake_runtime):
+    """Recording: operations launch into the sequence, everything that allocates, copies,
+    clears or waits is refused, a replay counts the recorded launches."""
+    with Backend() as b:
+        req = b.attention_requirement(1, 300, 8, 2, 128, query_start=299, dtype=B.DTYPE_BF16,
+                                      contract=B.NUMERIC_BF16_F32_ACCUMULATE)
+        q = written(b, "q", B.DTYPE_BF16, (1, 8, 128))
+        k, v = written(b, "k", B.DTYPE_BF16, (300, 2, 128)), written(b, "v", B.DTYPE_BF16, (300, 2, 128))
+        out = b.tensor("o", B.DTYPE_BF16, (1, 8, 128))
+        with pytest.raises(YvexError) as e:
+            b.graph_end()
+        assert e.value.code == B.YVEX_ERR_STATE
+        b.graph_begin()
+        with pytest.raises(YvexError) as e:                   # no workspace: would allocate
+            b.attention_execute(req, q, k, v, out)
+        assert e.value.code == B.YVEX_ERR_STATE
+        for call in (lambda: b.tensor("x", B.DTYPE_F32, (4,)), lambda: q.zero(), lambda: q.read(),
+                     lambda: q.release(), b.sync, b.graph_begin, b.timing_begin,
+                     lambda: b.set_completion_mode(B.COMPLETION_DEFERRED)):
+            with pytest.raises(YvexError) as e:
+                call()
+            assert e.value.code == B.YVEX_ERR_STATE
+        empty = b.graph_end()                                  # an empty sequence is legal
+        assert b.graph_launch(empty).kernel_launches == 0
+        b.graph_release(empty)
+        work = b.tensor("work", B.DTYPE_I8, (b.attention_workspace_required(req) + (1 << 20),))
+        b.workspace_attach(work)
+        before = fake_runtime.fake_hip_launches()
+        b.graph_begin()
+        facts = b.attention_execute(req, q, k, v, out)
+        assert facts.kernel_launches == 2 and facts.device_synchronizations == 0
+        assert fake_runtime.fake_hip_launches() == before      # recorded, not run
+        graph = b.graph_end()
+        for n in (1, 2, 3):
+            facts = b.graph_launch(graph)
+            assert facts.kernel_launches == 2 and facts.device_synchronizations == 1
+            assert fake_runtime.fake_hip_launches() == before + 2 * n
+        b.set_completion_mode(B.COMPLETION_DEFERRED)
+        assert b.graph_launch(graph).device_synchronizations == 0
+        b.sync()
+        b.set_completion_mode(B.COMPLETION_IMMEDIATE)
+        b.graph_release(graph)
+        b.workspace_detach()
+
+
 # ------------------------------------------------- failure transitions ----
 
 def test_launch_failure_fails_only_that_variant(env):
