@@ -431,6 +431,14 @@ def main():
         rng = np.random.default_rng(SEEDS[name])
         results[name] = {**WORKLOADS, **EXTRA_WORKLOADS}[name](backend, rng, args.steps, args.warmup)
         backend.close()
+    # what the part sustains on a plain streaming read and on a copy (the library's own probe):
+    # context for the roofline fractions, which are quoted against the published 8 TB/s
+    backend = Backend()
+    evidence = backend.bandwidth_probe()
+    backend.close()
+    device_probe = {"hbm_stream_read_gbs": evidence.sustainable_read_bytes_per_second / 1e9,
+                    "device_copy_gbs": evidence.sustainable_copy_bytes_per_second / 1e9,
+                    "working_set_bytes": int(evidence.working_set_bytes)}
     head = results[headline]
     roof = roofline(head)
     cpu = {} if args.no_cpu else {n: cpu_baseline(n) for n in names if n in WORKLOADS}
@@ -446,6 +454,7 @@ def main():
                    "kernel_launches_per_step": head["launches"]},
         "roofline": roof,
         "cpu_baseline": cpu.get(headline),
+        "device_probe": device_probe,
         "workloads": {n: dict(workload=r["workload"], ms_per_step=r["ms"],
                               wall_ms_per_step=r["wall_ms"], value=roofline(r)["step"],
                               unit=roofline(r)["unit"], roofline=roofline(r),

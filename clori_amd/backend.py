@@ -184,6 +184,12 @@ class Backend:
         _check(lib().yvex_backend_rocm_timing_end(self.handle, C.byref(ms), C.byref(err)), err)
         return ms.value
 
+    def bandwidth_probe(self):
+        """Measured streaming-read and copy rates of the device (kept after the first call)."""
+        evidence, err = B.BandwidthEvidence(), B.Error()
+        _check(lib().yvex_backend_bandwidth_probe(self.handle, C.byref(evidence), C.byref(err)), err)
+        return evidence
+
     # -- recorded launch sequences -------------------------------------
     def graph_begin(self):
         err = B.Error()

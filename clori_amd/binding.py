@@ -196,6 +196,16 @@ class TransformerOperations(C.Structure):
 KV_APPEND_FN = C.CFUNCTYPE(C.c_int, C.c_void_p, C.POINTER(KvAppendRequest), FactsP, ErrorP)
 
 
+class BandwidthEvidence(C.Structure):
+    _fields_ = [("schema_version", C.c_uint), ("working_set_bytes", ull), ("iterations", ull),
+                ("sample_count", ull), ("stream_elapsed_ns", ull * 5), ("copy_elapsed_ns", ull * 5),
+                ("coherent_host_elapsed_ns", ull * 5),
+                ("sustainable_read_bytes_per_second", ull),
+                ("sustainable_copy_bytes_per_second", ull),
+                ("sustainable_coherent_host_bytes_per_second", ull),
+                ("kernel_bundle_identity", C.c_char * 65), ("identity", C.c_char * 65)]
+
+
 class AttentionEpilogue(C.Structure):
     _fields_ = [("output_gate", TensorP)]
 
@@ -245,7 +255,7 @@ EXPORTED_SYMBOLS = [
     "yvex_backend_rocm_attention_operations_get", "yvex_backend_rocm_completion_mode_set",
     "yvex_backend_rocm_timing_begin", "yvex_backend_rocm_timing_end",
     "yvex_backend_rocm_kernel_probe_begin", "yvex_backend_rocm_kernel_probe_end",
-    "yvex_backend_rocm_graph_begin", "yvex_backend_rocm_graph_end",
+    "yvex_backend_bandwidth_probe", "yvex_backend_rocm_graph_begin", "yvex_backend_rocm_graph_end",
     "yvex_backend_rocm_graph_launch", "yvex_backend_rocm_graph_release",
     "yvex_backend_rocm_report_get", "yvex_quant_f16_decode", "yvex_quant_f16_encode",
     "yvex_quant_bf16_decode", "yvex_quant_bf16_encode", "yvex_rocm_q8_0_encode_row",
@@ -317,6 +327,7 @@ def load(path=None):
     lib.yvex_backend_rocm_timing_end.argtypes = [vp, C.POINTER(C.c_double), ErrorP]
     lib.yvex_backend_rocm_kernel_probe_begin.argtypes = [vp, C.c_char_p, ErrorP]
     lib.yvex_backend_rocm_kernel_probe_end.argtypes = [vp, C.POINTER(C.c_uint), C.POINTER(C.c_double), ErrorP]
+    lib.yvex_backend_bandwidth_probe.argtypes = [vp, C.POINTER(BandwidthEvidence), ErrorP]
     lib.yvex_backend_rocm_graph_begin.argtypes = [vp, ErrorP]
     lib.yvex_backend_rocm_graph_end.argtypes = [vp, C.POINTER(C.c_void_p), ErrorP]
     lib.yvex_backend_rocm_graph_launch.argtypes = [vp, C.c_void_p, FactsP, ErrorP]

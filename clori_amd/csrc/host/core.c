@@ -210,6 +210,23 @@ int yvex_backend_get_device_info(const yvex_backend *backend, yvex_backend_devic
     return backend->vtable->device_info(backend, out, err);
 }
 
+/* src/backend/core.c:483-502 */
+int yvex_backend_bandwidth_probe(yvex_backend *backend, yvex_backend_bandwidth_evidence *out,
+                                 yvex_error *err)
+{
+    int rc;
+    if (out) memset(out, 0, sizeof(*out));
+    if (!backend || !out)
+        return refuse(err, YVEX_ERR_INVALID_ARG, "backend.bandwidth",
+                      "backend and bandwidth output are required");
+    rc = backend_dispatch_admit(backend, "backend.bandwidth", err);
+    if (rc != YVEX_OK) return rc;
+    if (!backend->vtable || !backend->vtable->bandwidth_probe)
+        return refuse(err, YVEX_ERR_UNSUPPORTED, "backend.bandwidth",
+                      "backend does not provide measured bandwidth evidence");
+    return backend->vtable->bandwidth_probe(backend, out, err);
+}
+
 /* ------------------------------------------------------------- tensors ---- */
 
 /* src/backend/core.c:1143-1171 */

@@ -29,6 +29,7 @@ typedef struct yvex_backend_vtable {
     int (*tensor_copy)(yvex_backend *, yvex_device_tensor *, const yvex_device_tensor *,
                        yvex_error *);
     int (*sync)(yvex_backend *, yvex_error *);
+    int (*bandwidth_probe)(yvex_backend *, yvex_backend_bandwidth_evidence *, yvex_error *);
     int (*query_capability)(const yvex_backend *, yvex_backend_operation_variant,
                             yvex_backend_capability_result *, yvex_error *);
     int (*op_attention)(yvex_backend *, const yvex_device_tensor *, const yvex_device_tensor *,

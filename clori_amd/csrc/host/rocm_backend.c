@@ -8,6 +8,8 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include "../kernel_params.h"
+
 static void probe_release(yvex_rocm_backend_state *state);
 
 static int refuse(yvex_error *err, yvex_status status, const char *where, const char *reason)
@@ -208,6 +210,131 @@ static int rocm_sync(yvex_backend *backend, yvex_error *err)
     return yvex_rocm_synchronize(backend, YVEX_BACKEND_VARIANT_TENSOR_READ, "rocm.sync", err);
 }
 
+/* ---------------------------------------------------------- bandwidth ---- */
+
+static unsigned long long median_of(const unsigned long long *samples, unsigned int count)
+{
+    unsigned long long sorted[YVEX_BACKEND_BANDWIDTH_SAMPLE_COUNT];
+    unsigned int i, j;
+    for (i = 0; i < count; ++i) {
+        unsigned long long value = samples[i];
+        for (j = i; j > 0 && sorted[j - 1] > value; --j) sorted[j] = sorted[j - 1];
+        sorted[j] = value;
+    }
+    return sorted[count / 2u];
+}
+
+/* One timed sample: `iterations` passes of the streaming read, or of the copy. */
+static int bandwidth_sample(yvex_backend *backend, yvex_device_tensor *source,
+                            yvex_device_tensor *copy, yvex_device_tensor *sink, int copying,
+                            unsigned long long iterations, unsigned long long *elapsed_ns,
+                            yvex_error *err)
+{
+    static const char where[] = "rocm.bandwidth";
+    yvex_rocm_backend_state *state = yvex_rocm_state(backend);
+    yvex_rocm_stream_params params;
+    unsigned long long i;
+    double milliseconds = 0.0;
+    int rc;
+    memset(&params, 0, sizeof(params));
+    params.data = source->data;
+    params.sink = (uint32_t *)sink->data;
+    params.words = source->bytes / 16ull;
+    params.never = 0x5ca1ab1eu; /* the working set is all zero */
+    rc = yvex_backend_rocm_timing_begin(backend, err);
+    for (i = 0; rc == YVEX_OK && i < iterations; ++i) {
+        if (copying)
+            rc = yvex_rocm_status(&state->driver,
+                                  state->driver.hipMemcpyAsync(copy->data, source->data,
+                                                               (size_t)source->bytes,
+                                                               hipMemcpyDeviceToDevice,
+                                                               state->stream),
+                                  where, err);
+        else
+            rc = yvex_rocm_launch(backend, YVEX_ROCM_FN_STREAM_READ,
+                                  YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_F32,
+                                  (unsigned int)(state->compute_units > 0 ? state->compute_units * 8 : 2048),
+                                  1u, 1u, 256u, 0u, &params, where, err);
+    }
+    if (rc == YVEX_OK) rc = yvex_backend_rocm_timing_end(backend, &milliseconds, err);
+    else state->timing_active = 0;
+    if (rc != YVEX_OK) return rc;
+    *elapsed_ns = (unsigned long long)(milliseconds * 1.0e6);
+    if (!*elapsed_ns) *elapsed_ns = 1ull;
+    return YVEX_OK;
+}
+
+/* src/backend/cuda/backend.c:1428-1530: allocate the working set, warm up, take the samples,
+ * publish medians; the evidence of the first successful run is kept. */
+static int rocm_bandwidth_probe(yvex_backend *backend, yvex_backend_bandwidth_evidence *out,
+                                yvex_error *err)
+{
+    static const char where[] = "rocm.bandwidth";
+    yvex_rocm_backend_state *state = yvex_rocm_state(backend);
+    yvex_backend_bandwidth_evidence evidence;
+    yvex_backend_tensor_desc descriptor;
+    yvex_device_tensor *source = NULL, *copy = NULL, *sink = NULL;
+    const char *forced = getenv("YVEX_ROCM_BANDWIDTH_BYTES");
+    unsigned long long scratch;
+    yvex_error cleanup;
+    unsigned int sample;
+    int rc;
+    if (!state || !out) return refuse(err, YVEX_ERR_INVALID_ARG, where, "backend and out are required");
+    if (state->bandwidth_ready) {
+        *out = state->bandwidth_evidence;
+        yvex_error_clear(err);
+        return YVEX_OK;
+    }
+    if (state->kernel_bundle_state != YVEX_ROCM_KERNEL_BUNDLE_ADMITTED)
+        return refuse(err, YVEX_ERR_UNSUPPORTED, where, "no kernel bundle is admitted");
+    if (state->recording || state->timing_active)
+        return refuse(err, YVEX_ERR_STATE, where, "close the recording or timing section first");
+    memset(&evidence, 0, sizeof(evidence));
+    evidence.schema_version = YVEX_BACKEND_BANDWIDTH_SCHEMA_V1;
+    /* well beyond the 256 MB last-level cache of the part */
+    evidence.working_set_bytes = forced && atoll(forced) >= 8192 ? (unsigned long long)atoll(forced) & ~8191ull
+                                                                 : 1ull << 30;
+    evidence.iterations = 8ull;
+    evidence.sample_count = YVEX_BACKEND_BANDWIDTH_SAMPLE_COUNT;
+    memset(&descriptor, 0, sizeof(descriptor));
+    descriptor.dtype = YVEX_DTYPE_I8;
+    descriptor.rank = 1u;
+    descriptor.dims[0] = descriptor.bytes = evidence.working_set_bytes;
+    descriptor.name = "bandwidth-source";
+    rc = yvex_backend_tensor_alloc(backend, &descriptor, &source, err);
+    descriptor.name = "bandwidth-copy";
+    if (rc == YVEX_OK) rc = yvex_backend_tensor_alloc(backend, &descriptor, &copy, err);
+    descriptor.name = "bandwidth-sink";
+    descriptor.dims[0] = descriptor.bytes = 256ull;
+    if (rc == YVEX_OK) rc = yvex_backend_tensor_alloc(backend, &descriptor, &sink, err);
+    /* warm-up pass of each kind, not timed */
+    if (rc == YVEX_OK) rc = bandwidth_sample(backend, source, copy, sink, 0, 1ull, &scratch, err);
+    if (rc == YVEX_OK) rc = bandwidth_sample(backend, source, copy, sink, 1, 1ull, &scratch, err);
+    for (sample = 0u; rc == YVEX_OK && sample < evidence.sample_count; ++sample)
+        rc = bandwidth_sample(backend, source, copy, sink, 0, evidence.iterations,
+                              &evidence.stream_elapsed_ns[sample], err);
+    for (sample = 0u; rc == YVEX_OK && sample < evidence.sample_count; ++sample)
+        rc = bandwidth_sample(backend, source, copy, sink, 1, evidence.iterations,
+                              &evidence.copy_elapsed_ns[sample], err);
+    if (rc == YVEX_OK) {
+        const double read_ns = (double)median_of(evidence.stream_elapsed_ns, evidence.sample_count);
+        const double copy_ns = (double)median_of(evidence.copy_elapsed_ns, evidence.sample_count);
+        const double bytes = (double)evidence.working_set_bytes * (double)evidence.iterations;
+        evidence.sustainable_read_bytes_per_second = (unsigned long long)(bytes / read_ns * 1.0e9);
+        evidence.sustainable_copy_bytes_per_second = (unsigned long long)(2.0 * bytes / copy_ns * 1.0e9);
+    }
+    yvex_error_clear(&cleanup);
+    if (sink) (void)yvex_backend_tensor_release(backend, &sink, &cleanup);
+    if (copy) (void)yvex_backend_tensor_release(backend, &copy, &cleanup);
+    if (source) (void)yvex_backend_tensor_release(backend, &source, &cleanup);
+    if (rc != YVEX_OK) return rc;
+    state->bandwidth_evidence = evidence;
+    state->bandwidth_ready = 1;
+    *out = evidence;
+    yvex_error_clear(err);
+    return YVEX_OK;
+}
+
 static int rocm_memory_stats(const yvex_backend *backend, yvex_backend_memory_stats *out,
                              yvex_error *err)
 {
@@ -330,6 +457,7 @@ static const yvex_backend_vtable rocm_vtable = {
     .tensor_zero = rocm_tensor_zero,
     .tensor_copy = rocm_tensor_copy,
     .sync = rocm_sync,
+    .bandwidth_probe = rocm_bandwidth_probe,
     .query_capability = yvex_rocm_query_capability,
     .op_attention = yvex_rocm_op_attention,
     .transformer_operations = yvex_rocm_transformer_operations,

@@ -33,6 +33,7 @@ static const rocm_kernel_binding rocm_kernel_bindings[] = {
      YVEX_ROCM_FN_ATTENTION_F32},
     {"yvex_rocm_gqa_f32", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_F32, YVEX_ROCM_FN_GQA_F32},
     {"yvex_rocm_fill_u32", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_F32, YVEX_ROCM_FN_FILL_U32},
+    {"yvex_rocm_stream_read", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_F32, YVEX_ROCM_FN_STREAM_READ},
     {"yvex_rocm_decode_paged_bf16", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_PAGED_BF16,
      YVEX_ROCM_FN_DECODE_PAGED_BF16},
     {"yvex_rocm_decode_merge", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_PAGED_BF16,

@@ -22,6 +22,7 @@ typedef enum {
     YVEX_ROCM_FN_MLA_DECODE_BF16,
     YVEX_ROCM_FN_KV_APPEND_BF16,
     YVEX_ROCM_FN_KV_APPEND_Q8_0,
+    YVEX_ROCM_FN_STREAM_READ,
     YVEX_ROCM_FN_COUNT
 } yvex_rocm_function_id;
 
@@ -61,6 +62,8 @@ typedef struct yvex_rocm_backend_state {
     int recording;                  /* a launch sequence is being recorded on the stream */
     unsigned long long live_graphs; /* recorded sequences not yet released */
     unsigned long long recorded_launches; /* kernel launches of the sequence being recorded */
+    int bandwidth_ready; /* the probe ran: later calls return the kept evidence */
+    yvex_backend_bandwidth_evidence bandwidth_evidence;
 } yvex_rocm_backend_state;
 
 /* A recorded launch sequence (rocm_backend.c). */

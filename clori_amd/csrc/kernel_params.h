@@ -42,6 +42,16 @@ typedef struct {
     uint32_t reserved;
 } yvex_rocm_fill_params;
 
+/* Streaming read of `words` 16-byte words; the sink is written only if the XOR of
+ * everything read equals `never` (it does not: the loads cannot be dropped). */
+typedef struct {
+    const void *data;
+    uint32_t *sink;
+    uint64_t words;
+    uint32_t never;
+    uint32_t reserved;
+} yvex_rocm_stream_params;
+
 /* Split-K decode over a balanced partition.  The (session, kv head, 16-token tile) work
  * of the whole batch is laid out as one sequence and cut into gridDim.x equal ranges,
  * one wave each.  A wave that covers a whole (session, kv head) segment publishes the

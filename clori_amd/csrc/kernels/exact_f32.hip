@@ -176,3 +176,27 @@ yvex_rocm_fill_u32(const yvex_rocm_fill_params p)
     const uint64_t stride = (uint64_t)gridDim.x * 256u;
     for (; i < p.words; i += stride) p.data[i] = p.value;
 }
+
+// Streaming read for the bandwidth probe (the counterpart of the in-place pass the reference
+// times in src/backend/cuda/backend.c:1356-1399): each wave takes whole 8 KB blocks, eight
+// independent 1 KB wave-loads in flight, blocks dealt round-robin to the waves; nothing is
+// written.  The working set is a whole number of blocks.
+extern "C" __global__ void __launch_bounds__(256)
+yvex_rocm_stream_read(const yvex_rocm_stream_params p)
+{
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    const u32x4 *words = reinterpret_cast<const u32x4 *>(p.data);
+    const uint64_t lane = threadIdx.x & 63u;
+    const uint64_t wave = ((uint64_t)blockIdx.x * 256u + threadIdx.x) >> 6;
+    const uint64_t waves = (uint64_t)gridDim.x * 4u, blocks = p.words / 512u;
+    u32x4 acc = {0u, 0u, 0u, 0u};
+    for (uint64_t b = wave; b < blocks; b += waves) {
+        const u32x4 *base = words + b * 512u + lane;
+        u32x4 v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = base[j * 64];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc ^= v[j];
+    }
+    if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == p.never) p.sink[0] = 1u;
+}

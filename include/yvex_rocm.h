@@ -498,6 +498,31 @@ int yvex_backend_rocm_completion_mode_set(yvex_backend *backend, yvex_rocm_compl
                                           yvex_error *err);
 
 /*
+ * Measured device bandwidth (include/yvex/internal/backend.h:180-192,261;
+ * src/backend/core.c:483-502 dispatch, src/backend/cuda/backend.c:1356-1500 the CUDA probe).
+ * Same record, same rule: five samples of `iterations` passes over a working set, the
+ * sustainable rate is bytes over the median sample.  stream_* times a pure streaming read of
+ * the working set (HBM read rate), copy_* a device-to-device copy (counted as read plus
+ * write).  The coherent-host fields are for unified-memory parts and stay zero here; the
+ * identity strings are left empty.  The first successful probe is kept and returned again.
+ */
+#define YVEX_BACKEND_BANDWIDTH_SCHEMA_V1 1u
+#define YVEX_BACKEND_BANDWIDTH_SAMPLE_COUNT 5u
+#define YVEX_SHA256_HEX_BYTES 65u
+typedef struct {
+    unsigned int schema_version;
+    unsigned long long working_set_bytes, iterations, sample_count;
+    unsigned long long stream_elapsed_ns[YVEX_BACKEND_BANDWIDTH_SAMPLE_COUNT];
+    unsigned long long copy_elapsed_ns[YVEX_BACKEND_BANDWIDTH_SAMPLE_COUNT];
+    unsigned long long coherent_host_elapsed_ns[YVEX_BACKEND_BANDWIDTH_SAMPLE_COUNT];
+    unsigned long long sustainable_read_bytes_per_second, sustainable_copy_bytes_per_second;
+    unsigned long long sustainable_coherent_host_bytes_per_second;
+    char kernel_bundle_identity[YVEX_SHA256_HEX_BYTES], identity[YVEX_SHA256_HEX_BYTES];
+} yvex_backend_bandwidth_evidence;
+int yvex_backend_bandwidth_probe(yvex_backend *backend, yvex_backend_bandwidth_evidence *out,
+                                 yvex_error *err);
+
+/*
  * Recorded launch sequences (no reference counterpart; for launch-bound steps such as a
  * single-session decode, where two kernel launches cost more host time than device time).
  * Between begin and end the attention operations of this backend are recorded on its stream

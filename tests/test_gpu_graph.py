@@ -128,3 +128,13 @@ def test_recorded_decode_step_appends_then_attends(backend):
         assert np.array_equal(rec_v.read(np.uint8, (-1,)), eag_v.read(np.uint8, (-1,))), "step %d" % step
     backend.graph_release(graph)
     backend.workspace_detach()
+
+
+def test_bandwidth_probe_on_the_device(backend):
+    """The probe's record on a real part: a streaming read of 1 GiB sustains terabytes per
+    second, below the published peak; the copy moves read plus write."""
+    e = backend.bandwidth_probe()
+    assert e.working_set_bytes == 1 << 30 and e.sample_count == 5
+    assert 1.0e12 < e.sustainable_read_bytes_per_second < 8.5e12
+    assert 1.0e12 < e.sustainable_copy_bytes_per_second < 8.5e12
+    assert max(e.stream_elapsed_ns) < 2 * min(e.stream_elapsed_ns)

@@ -562,6 +562,27 @@ def test_recorded_sequence_rules(fake_runtime):
         b.workspace_detach()
 
 
+def test_bandwidth_probe_record(env, fake_runtime):
+    """Five samples of eight passes each for the read and for the copy, medians published,
+    the working set released, the first evidence kept."""
+    env("YVEX_ROCM_BANDWIDTH_BYTES", str(1 << 20))
+    with Backend() as b:
+        live, launches = fake_runtime.fake_hip_live_allocations(), fake_runtime.fake_hip_launches()
+        e = b.bandwidth_probe()
+        assert e.schema_version == 1 and e.working_set_bytes == 1 << 20
+        assert e.iterations == 8 and e.sample_count == 5
+        assert fake_runtime.fake_hip_launches() == launches + 1 + 5 * 8
+        assert fake_runtime.fake_hip_live_allocations() == live
+        assert all(x > 0 for x in e.stream_elapsed_ns) and all(x > 0 for x in e.copy_elapsed_ns)
+        assert e.sustainable_read_bytes_per_second > 0 and e.sustainable_copy_bytes_per_second > 0
+        assert list(e.coherent_host_elapsed_ns) == [0] * 5
+        again = b.bandwidth_probe()
+        assert fake_runtime.fake_hip_launches() == launches + 1 + 5 * 8       # not measured twice
+        assert again.sustainable_read_bytes_per_second == e.sustainable_read_bytes_per_second
+        b.graph_begin()
+        b.graph_release(b.graph_end())
+
+
 # ------------------------------------------------- failure transitions ----
 
 def test_launch_failure_fails_only_that_variant(env):
