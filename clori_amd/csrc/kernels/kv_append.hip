@@ -89,6 +89,12 @@ __device__ inline Span locate(const yvex_rocm_kv_append_params &p)
     }
     const uint32_t first_page = (uint32_t)start / kPageTokens;
     const uint32_t last_page = ((uint32_t)start + (uint32_t)count - 1u) / kPageTokens;
+    if (last_page - first_page >= gridDim.x) {
+        // more tokens than the launch was sized for (max_tokens_per_session): refuse rather
+        // than drop the pages no workgroup covers
+        if (slot == 0u && blockIdx.y == 0u && threadIdx.x == 0) flag(p.status, YVEX_ROCM_DEVICE_CONTRACT);
+        return s;
+    }
     const uint32_t page = first_page + slot;
     if (page > last_page) return s;
     const int32_t id = p.page_table[(uint64_t)session * p.table_stride + page];

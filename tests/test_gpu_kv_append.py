@@ -177,6 +177,19 @@ def test_append_refusals(backend):
     with pytest.raises(YvexError) as e:
         small_append(backend, bf16_normal(rng, (4, HKV, D)), 30, 4)
     assert e.value.code == B.YVEX_ERR_BOUNDS
+    # more tokens in a session than the request declared -> BOUNDS, nothing dropped silently
+    with pytest.raises(YvexError) as e:
+        k_new = bf16_normal(rng, (32, HKV, D))
+        tensors = [backend.tensor("k", B.DTYPE_BF16, k_new.shape, k_new),
+                   backend.tensor("v", B.DTYPE_BF16, k_new.shape, k_new),
+                   backend.tensor("r", B.DTYPE_I32, (1,), np.array([0], np.int32)),
+                   backend.tensor("s", B.DTYPE_I32, (1,), np.array([0], np.int32)),
+                   backend.tensor("c", B.DTYPE_I32, (1,), np.array([32], np.int32)),
+                   backend.tensor("t", B.DTYPE_I32, (1, 2), np.array([[0, 1]], np.int32)),
+                   backend.tensor("kp", B.DTYPE_BF16, (4 * HKV * PAGE * D,)),
+                   backend.tensor("vp", B.DTYPE_BF16, (4 * HKV * PAGE * D,))]
+        backend.kv_append_execute(*tensors, HKV, 4, 1)        # declared: one token per session
+    assert e.value.code == B.YVEX_ERR_BOUNDS
     # a NaN key -> FORMAT
     k_bad = bf16_normal(rng, (2, HKV, D))
     k_bad[1, 3, 7] = 0x7FC0
