@@ -327,8 +327,9 @@ def roofline(result):
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # runs (profiles/), scaled by the same counters on a copy kernel of known size; None where
 # no such run is committed.
-TRAFFIC = {"paged3": 1033350292, "paged4": 1512968367, "decode1": 18117050,
-           "prefill2": 50475981, "mla5": 204071018}
+TRAFFIC = {"paged3": 1033345728, "paged4": 1512954963, "decode1": 18117066,
+           "prefill2": 50569339, "mla5": 204066874, "append_bf16": 303924258,
+           "append_q8_0": 239926575}
 
 
 def repeat_for(seconds, call):
