@@ -107,10 +107,9 @@ typedef struct {
     uint16_t *out;
     float *lse; /* optional F32 [Tq][Hq] */
     int32_t *status;
-    const uint32_t *tasks; /* [task_count][4]: q head, q tile, first kv tile, end kv tile */
     uint64_t q_stride, k_stride, v_stride; /* elements per token */
     uint32_t query_tokens, kv_tokens, query_start, query_heads, kv_heads, head_dim;
-    uint32_t causal, task_count;
+    uint32_t causal, reserved;
     float scale_log2;
     float reserved_f;
     const uint16_t *gate; /* optional bf16 [Tq][Hq][head_dim] sigmoid output gate */
