@@ -555,7 +555,8 @@ int yvex_backend_open_rocm_impl(yvex_backend **out, const char *device,
     backend->device_info.device_index = state->device_index;
     if (state->driver.hipDeviceGetName(backend->device_name_storage,
                                        (int)sizeof(backend->device_name_storage),
-                                       state->device_index) != hipSuccess)
+                                       state->device_index) != hipSuccess ||
+        backend->device_name_storage[0] == '\0') /* some drivers publish an empty marketing name */
         yvex_core_text_copy(backend->device_name_storage, sizeof(backend->device_name_storage),
                             "rocm");
     backend->device_info.name = backend->device_name_storage;
