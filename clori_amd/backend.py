@@ -353,7 +353,7 @@ class Backend:
     def mla_requirement(batch, heads, key_dim, value_dim, page_tokens, pool_pages, table_stride,
                         max_context, contract=B.NUMERIC_BF16_F32_ACCUMULATE, deterministic=1,
                         sliding_window=0, compressed_pool_pages=0, compressed_table_stride=0,
-                        max_compressed_tokens=0):
+                        max_compressed_tokens=0, compressed_selected_stride=0):
         r = B.MlaDecodeRequirement()
         r.batch, r.heads, r.key_dimension, r.value_dimension = batch, heads, key_dim, value_dim
         r.page_tokens, r.pool_pages, r.page_table_stride = page_tokens, pool_pages, table_stride
@@ -362,6 +362,7 @@ class Backend:
         r.compressed_pool_pages = compressed_pool_pages
         r.compressed_page_table_stride = compressed_table_stride
         r.max_compressed_tokens = max_compressed_tokens
+        r.compressed_selected_stride = compressed_selected_stride
         return r
 
     def mla_decode_workspace_required(self, requirement):
@@ -373,7 +374,8 @@ class Backend:
 
     def mla_decode_execute(self, requirement, query, latent_pages, page_table, context, output,
                            lse=None, sinks=None, compressed=None):
-        """compressed: optional (pages, page table, visible row counts) device tensors."""
+        """compressed: optional (pages, page table, row counts[, selected row lists]) device
+        tensors."""
         ops = self.rocm_attention_operations()
         if ops is None:
             raise YvexError(B.YVEX_ERR_UNSUPPORTED, "rocm_attention_operations", "not published")

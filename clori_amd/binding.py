@@ -149,7 +149,7 @@ class MlaDecodeRequirement(C.Structure):
                                    "max_context_tokens")] + [
         ("numeric_contract", C.c_int), ("deterministic", C.c_int), ("sliding_window", ull),
         ("compressed_pool_pages", ull), ("compressed_page_table_stride", ull),
-        ("max_compressed_tokens", ull)]
+        ("max_compressed_tokens", ull), ("compressed_selected_stride", ull)]
 
 
 class MlaDecodeRequest(C.Structure):
@@ -157,7 +157,7 @@ class MlaDecodeRequest(C.Structure):
                 ("latent_pages", TensorP), ("page_table", TensorP), ("context_tokens", TensorP),
                 ("output", TensorP), ("lse", TensorP), ("sinks", TensorP),
                 ("compressed_pages", TensorP), ("compressed_page_table", TensorP),
-                ("compressed_tokens", TensorP)]
+                ("compressed_tokens", TensorP), ("compressed_selected", TensorP)]
 
 
 class KvAppendRequirement(C.Structure):

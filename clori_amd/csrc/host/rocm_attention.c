@@ -634,14 +634,15 @@ static int mla_validate(const yvex_rocm_mla_decode_requirement *r, const char *w
         (r->max_compressed_tokens &&
          (!r->compressed_pool_pages || !r->compressed_page_table_stride ||
           r->compressed_page_table_stride > 0xffffffffull ||
-          r->max_compressed_tokens > r->compressed_page_table_stride * r->page_tokens)))
+          r->max_compressed_tokens > r->compressed_page_table_stride * r->page_tokens)) ||
+        (r->compressed_selected_stride && !r->max_compressed_tokens))
         return refuse(err, YVEX_ERR_INVALID_ARG, where, "complete MLA decode geometry is required");
     if (r->heads != ROCM_MLA_HEADS || r->key_dimension != ROCM_MLA_KEY_DIM ||
         r->value_dimension != ROCM_MLA_VALUE_DIM || r->page_tokens != ROCM_MLA_PAGE_TOKENS ||
         r->numeric_contract != YVEX_TRANSFORMER_ATTENTION_NUMERIC_BF16_F32_ACCUMULATE ||
         !r->deterministic || r->pool_pages > 0x7fffffffull || capacity > 0x7fffffffull ||
         r->batch > 65535ull || r->sliding_window > 0x7fffffffull ||
-        r->compressed_pool_pages > 0x7fffffffull ||
+        r->compressed_pool_pages > 0x7fffffffull || r->compressed_selected_stride > 0x7fffffull ||
         r->compressed_page_table_stride * r->page_tokens > 0x7fffffffull)
         return refuse(err, YVEX_ERR_UNSUPPORTED, where,
                       "ROCm MLA decode requires 128 heads, a 512+64 latent row, 64-token pages "
@@ -694,9 +695,28 @@ static void mla_partition(const yvex_rocm_mla_decode_requirement *r, unsigned lo
     *max_chunks = (mla_live_tokens(r) + *chunk - 1ull) / *chunk;
     *extra_chunk = *extra_max_chunks = 0ull;
     if (r->max_compressed_tokens) {
-        *extra_chunk = mla_chunk_for(r, r->max_compressed_tokens, 0);
-        *extra_max_chunks = (r->max_compressed_tokens + *extra_chunk - 1ull) / *extra_chunk;
+        const unsigned long long rows = r->compressed_selected_stride ? r->compressed_selected_stride
+                                                                      : r->max_compressed_tokens;
+        *extra_chunk = mla_chunk_for(r, rows, 0);
+        *extra_max_chunks = (rows + *extra_chunk - 1ull) / *extra_chunk;
     }
+}
+
+/* Bytes behind the partials for the gathered rows of the selected class and their identity
+ * page table; 0 without a selection. */
+static int mla_gather_bytes(const yvex_rocm_mla_decode_requirement *r, unsigned long long *pages_each,
+                            unsigned long long *rows_bytes, unsigned long long *table_bytes)
+{
+    *pages_each = *rows_bytes = *table_bytes = 0ull;
+    if (!r->compressed_selected_stride) return 1;
+    *pages_each = (r->compressed_selected_stride + r->page_tokens - 1ull) / r->page_tokens;
+    if (!yvex_core_u64_mul(r->batch * *pages_each, r->page_tokens * r->key_dimension * sizeof(uint16_t),
+                           rows_bytes) ||
+        r->batch * *pages_each > 0x7fffffffull)
+        return 0;
+    *rows_bytes = align_up(*rows_bytes, ROCM_WORK_ALIGNMENT);
+    *table_bytes = align_up(r->batch * *pages_each * sizeof(int32_t), ROCM_WORK_ALIGNMENT);
+    return 1;
 }
 
 static int rocm_mla_decode_workspace_required(const yvex_rocm_mla_decode_requirement *r,
@@ -704,6 +724,7 @@ static int rocm_mla_decode_workspace_required(const yvex_rocm_mla_decode_require
 {
     static const char where[] = "rocm.attention.mla.workspace";
     unsigned long long acc = 0ull, total = 0ull, chunk, max_chunks, extra_chunk, extra_max_chunks;
+    unsigned long long gather_pages, gather_rows, gather_table;
     int rc;
     if (bytes) *bytes = 0ull;
     rc = mla_validate(r, where, err);
@@ -711,7 +732,9 @@ static int rocm_mla_decode_workspace_required(const yvex_rocm_mla_decode_require
     if (!bytes) return refuse(err, YVEX_ERR_INVALID_ARG, where, "workspace byte output is required");
     mla_partition(r, &chunk, &max_chunks, &extra_chunk, &extra_max_chunks);
     if (!decode_workspace_bytes(r->batch * (max_chunks + extra_max_chunks), r->heads, r->value_dimension,
-                                sizeof(uint16_t), &acc, &total))
+                                sizeof(uint16_t), &acc, &total) ||
+        !mla_gather_bytes(r, &gather_pages, &gather_rows, &gather_table) ||
+        !yvex_core_u64_add(total, gather_rows + gather_table, &total))
         return refuse(err, YVEX_ERR_BOUNDS, where, "MLA workspace geometry overflowed");
     *bytes = total;
     yvex_error_clear(err);
@@ -729,9 +752,10 @@ static int rocm_mla_decode_execute(yvex_backend *backend,
     yvex_rocm_mla_params kp;
     yvex_rocm_decode_merge_params mp;
     unsigned long long acc_bytes = 0ull, total = 0ull, max_chunks, chunk, extra_chunk, extra_max_chunks;
+    unsigned long long gather_pages, gather_rows, gather_table, partial_bytes;
     void *work = NULL;
     yvex_error cleanup;
-    int owned = 0, rc, cleanup_rc;
+    int owned = 0, rc, cleanup_rc, gathered = 0;
     if (!request || !request->query || !request->latent_pages || !request->page_table ||
         !request->context_tokens || !request->output || !facts)
         return refuse(err, YVEX_ERR_INVALID_ARG, where,
@@ -759,15 +783,26 @@ static int rocm_mla_decode_execute(yvex_backend *backend,
                    r->compressed_pool_pages * r->page_tokens * r->key_dimension, 1) ||
           !view_ok(backend, request->compressed_page_table, YVEX_DTYPE_I32,
                    r->batch * r->compressed_page_table_stride, 1) ||
-          !view_ok(backend, request->compressed_tokens, YVEX_DTYPE_I32, r->batch, 1))))
+          !view_ok(backend, request->compressed_tokens, YVEX_DTYPE_I32, r->batch, 1) ||
+          (r->compressed_selected_stride &&
+           (!request->compressed_selected ||
+            !view_ok(backend, request->compressed_selected, YVEX_DTYPE_I32,
+                     r->batch * r->compressed_selected_stride, 1))))))
         return refuse(err, YVEX_ERR_FORMAT, where,
                       "query, latent pages, page table, context lengths and outputs must be "
                       "written tensors of this backend with the declared geometry");
     mla_partition(r, &chunk, &max_chunks, &extra_chunk, &extra_max_chunks);
     if (max_chunks + extra_max_chunks > 0x7fffffffull ||
         !decode_workspace_bytes(r->batch * (max_chunks + extra_max_chunks), r->heads, r->value_dimension,
-                                sizeof(uint16_t), &acc_bytes, &total))
+                                sizeof(uint16_t), &acc_bytes, &total) ||
+        !mla_gather_bytes(r, &gather_pages, &gather_rows, &gather_table) ||
+        !yvex_core_u64_add(total, gather_rows + gather_table, &partial_bytes))
         return refuse(err, YVEX_ERR_BOUNDS, where, "MLA decode geometry exceeds admitted range");
+    { /* partials first, then the gathered rows and their page table */
+        const unsigned long long partials = total;
+        total = partial_bytes;
+        partial_bytes = partials;
+    }
     backend_workspace_reset(backend);
     rc = yvex_rocm_temporary_acquire(backend, total, &work, &owned, where, err);
     if (rc != YVEX_OK) return rc;
@@ -807,7 +842,36 @@ static int rocm_mla_decode_execute(yvex_backend *backend,
         cp.window = 0u;
         cp.first_slot = (uint32_t)max_chunks;
         cp.empty_ok = 1u;
-        rc = yvex_rocm_launch(backend, YVEX_ROCM_FN_MLA_DECODE_BF16, variant,
+        if (r->compressed_selected_stride) {
+            /* the selected class: copy the listed rows next to each other, then walk them */
+            yvex_rocm_gather_rows_params gp;
+            memset(&gp, 0, sizeof(gp));
+            gp.pool = cp.pool;
+            gp.page_table = cp.page_table;
+            gp.selected = (const int32_t *)request->compressed_selected->data;
+            gp.count = cp.context;
+            gp.rows = (uint16_t *)((unsigned char *)work + partial_bytes);
+            gp.table = (int32_t *)((unsigned char *)work + partial_bytes + gather_rows);
+            gp.status = state->device_status;
+            gp.batch = kp.batch;
+            gp.page_tokens = kp.page_tokens;
+            gp.pool_pages = cp.pool_pages;
+            gp.table_stride = cp.table_stride;
+            gp.selected_stride = (uint32_t)r->compressed_selected_stride;
+            gp.pages_each = (uint32_t)gather_pages;
+            gp.row_elements = kp.key_dim;
+            gp.max_rows = (uint32_t)r->max_compressed_tokens;
+            rc = yvex_rocm_launch(backend, YVEX_ROCM_FN_GATHER_ROWS, variant,
+                                  (unsigned int)r->compressed_selected_stride, (unsigned int)r->batch,
+                                  1u, 128u, 0u, &gp, where, err);
+            cp.pool = gp.rows;
+            cp.page_table = gp.table;
+            cp.pool_pages = (uint32_t)(r->batch * gather_pages);
+            cp.table_stride = (uint32_t)gather_pages;
+            if (rc == YVEX_OK) gathered = 1;
+        }
+        if (rc == YVEX_OK)
+            rc = yvex_rocm_launch(backend, YVEX_ROCM_FN_MLA_DECODE_BF16, variant,
                               (unsigned int)extra_max_chunks, (unsigned int)r->batch, 1u, 256u, 0u,
                               &cp, where, err);
     }
@@ -837,7 +901,7 @@ static int rocm_mla_decode_execute(yvex_backend *backend,
                               256u, 0u, &mp, where, err);
     }
     if (rc == YVEX_OK) {
-        facts->kernel_launches = extra_max_chunks ? 3ull : 2ull;
+        facts->kernel_launches = (extra_max_chunks ? 3ull : 2ull) + (gathered ? 1ull : 0ull);
         facts->accelerated_matrix_launches = extra_max_chunks ? 2ull : 1ull;
         facts->temporary_bytes = total;
         facts->compulsory_memory_facts_available = 1;

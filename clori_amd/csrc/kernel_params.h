@@ -136,6 +136,21 @@ typedef struct {
     uint32_t reserved;
 } yvex_rocm_mla_params;
 
+/* Gathers the selected compressed rows of every batch element into a contiguous paged pool
+ * (batch * pages_each pages of page_tokens rows) and writes the identity page table for it.
+ * grid = (selected_stride, batch), block = 128. */
+typedef struct {
+    const uint16_t *pool;         /* [pool_pages][page_tokens][row_elements] */
+    const int32_t *page_table;    /* [batch][table_stride] */
+    const int32_t *selected;      /* [batch][selected_stride] logical row indices */
+    const int32_t *count;         /* [batch] list entries */
+    uint16_t *rows;               /* [batch * pages_each][page_tokens][row_elements] */
+    int32_t *table;               /* [batch][pages_each] */
+    int32_t *status;
+    uint32_t batch, page_tokens, pool_pages, table_stride;
+    uint32_t selected_stride, pages_each, row_elements, max_rows;
+} yvex_rocm_gather_rows_params;
+
 /* KV page writer: new key/value rows -> paged pools (bf16 or Q8_0), rotary on the keys.
  * A workgroup is YVEX_ROCM_KV_APPEND_HEADS waves, one kv head each. */
 #define YVEX_ROCM_KV_APPEND_HEADS 4

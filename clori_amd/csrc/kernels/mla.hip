@@ -393,3 +393,36 @@ yvex_rocm_mla_decode_bf16(const yvex_rocm_mla_params p)
         p.part_ml[slot * 2 + 1] = l;
     }
 }
+
+// Row gather for the selected class of compressed candidates (src/graph/core.c:443-452): list
+// entry i of batch element b names a compressed row; it is copied to row i of that element's
+// slice of a contiguous pool, so that the decode kernel above walks the list as an ordinary
+// paged context.  One workgroup per list entry, 16 bytes per lane.
+extern "C" __global__ void __launch_bounds__(128)
+yvex_rocm_gather_rows(const yvex_rocm_gather_rows_params p)
+{
+    const uint32_t entry = blockIdx.x, batch = blockIdx.y, lane = threadIdx.x;
+    const int32_t count = p.count[batch];
+    if (count < 0 || (uint32_t)count > p.selected_stride) {
+        if (entry == 0u && lane == 0u) atomicCAS(p.status, 0, YVEX_ROCM_DEVICE_CONTRACT);
+        return;
+    }
+    if (entry % p.page_tokens == 0u && lane == 0u)
+        p.table[(uint64_t)batch * p.pages_each + entry / p.page_tokens] =
+            (int32_t)(batch * p.pages_each + entry / p.page_tokens);
+    if (entry >= (uint32_t)count) return;
+    const int32_t index = p.selected[(uint64_t)batch * p.selected_stride + entry];
+    if (index < 0 || (uint32_t)index >= p.max_rows) {
+        if (lane == 0u) atomicCAS(p.status, 0, YVEX_ROCM_DEVICE_CONTRACT);
+        return;
+    }
+    const int32_t page = p.page_table[(uint64_t)batch * p.table_stride + (uint32_t)index / p.page_tokens];
+    if (page < 0 || (uint32_t)page >= p.pool_pages) {
+        if (lane == 0u) atomicCAS(p.status, 0, YVEX_ROCM_DEVICE_CONTRACT);
+        return;
+    }
+    const uint16_t *src = p.pool + ((uint64_t)page * p.page_tokens + (uint32_t)index % p.page_tokens) * p.row_elements;
+    uint16_t *dst = p.rows + ((uint64_t)batch * p.pages_each * p.page_tokens + entry) * p.row_elements;
+    if (lane * 8u < p.row_elements)
+        *reinterpret_cast<u32x4 *>(dst + lane * 8u) = load_b128(src + lane * 8u);
+}

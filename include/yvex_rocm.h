@@ -405,6 +405,10 @@ typedef struct yvex_rocm_mla_decode_requirement {
      * rows are a prefix; attention_kernels.cu:85-97).  Same row format and page size as the
      * latent pool.  max_compressed_tokens = 0: no such set. */
     unsigned long long compressed_pool_pages, compressed_page_table_stride, max_compressed_tokens;
+    /* The selected class (src/graph/core.c:443-452, attention_kernels.cu:88-90): the visible
+     * compressed rows are the entries of a per-session index list, in list order, instead of
+     * a prefix.  compressed_selected_stride is the list capacity; 0: the prefix class. */
+    unsigned long long compressed_selected_stride;
 } yvex_rocm_mla_decode_requirement;
 
 typedef struct yvex_rocm_mla_decode_request {
@@ -420,6 +424,10 @@ typedef struct yvex_rocm_mla_decode_request {
      * session (0 allowed: position + ratio - 1 <= token position holds for a prefix of
      * floor(context / ratio) rows, which the caller passes). */
     const yvex_device_tensor *compressed_pages, *compressed_page_table, *compressed_tokens;
+    /* With compressed_selected_stride > 0: I32 [batch][compressed_selected_stride] indices of
+     * compressed rows (positions in the session's compressed sequence, below
+     * max_compressed_tokens); compressed_tokens then holds the number of list entries. */
+    const yvex_device_tensor *compressed_selected;
 } yvex_rocm_mla_decode_request;
 
 /* KV page writer (no reference counterpart as one operation: it is the rotary step of

@@ -549,7 +549,8 @@ int yvo_mla_decode_bf16(const uint16_t *q, const uint16_t *pool,
                         const float *sinks, uint64_t sliding_window,
                         const uint16_t *compressed_pool, const int32_t *compressed_table,
                         const int32_t *compressed_count, uint64_t compressed_pool_pages,
-                        uint64_t compressed_table_stride, int threads)
+                        uint64_t compressed_table_stride, const int32_t *selected,
+                        uint64_t selected_stride, int threads)
 {
     uint64_t b;
     double scale;
@@ -570,6 +571,18 @@ int yvo_mla_decode_bf16(const uint16_t *q, const uint16_t *pool,
         if (compressed_pool) {
             if (!compressed_table || !compressed_count || compressed_count[b] < 0)
                 return YVO_ERR_INVALID_ARG;
+            if (selected) {
+                /* src/graph/core.c:443-452: the list names the rows, in list order */
+                if ((uint64_t)compressed_count[b] > selected_stride) return YVO_ERR_BOUNDS;
+                for (p = 0; p < (uint64_t)compressed_count[b]; ++p) {
+                    int32_t index = selected[b * selected_stride + p], id;
+                    if (index < 0 || (uint64_t)index / page_tokens >= compressed_table_stride)
+                        return YVO_ERR_BOUNDS;
+                    id = compressed_table[b * compressed_table_stride + (uint64_t)index / page_tokens];
+                    if (id < 0 || (uint64_t)id >= compressed_pool_pages) return YVO_ERR_BOUNDS;
+                }
+                continue;
+            }
             pages = ((uint64_t)compressed_count[b] + page_tokens - 1u) / page_tokens;
             if (pages > compressed_table_stride) return YVO_ERR_BOUNDS;
             for (p = 0; p < pages; ++p) {
@@ -597,9 +610,10 @@ int yvo_mla_decode_bf16(const uint16_t *q, const uint16_t *pool,
         float *of = (float *)malloc((size_t)value_dim * sizeof(float));
         int rc = rows && qf && of ? YVO_OK : YVO_ERR_STATE;
         for (t = 0; rc == YVO_OK && t < extra; ++t) {
+            const uint64_t at = selected ? (uint64_t)selected[(uint64_t)unit * selected_stride + t] : t;
             uint64_t page = (uint64_t)compressed_table[(uint64_t)unit * compressed_table_stride +
-                                                       t / page_tokens];
-            yvo_bf16_decode_n(compressed_pool + (page * page_tokens + t % page_tokens) * key_dim,
+                                                       at / page_tokens];
+            yvo_bf16_decode_n(compressed_pool + (page * page_tokens + at % page_tokens) * key_dim,
                               rows + (local + t) * key_dim, (size_t)key_dim);
         }
         for (t = 0; rc == YVO_OK && t < local; ++t) {

@@ -167,6 +167,9 @@ int yvo_shared_kv_head(const float *q, const float *rows, size_t row_stride,
  * position context - 1).  compressed_pool (optional): a second paged row set of the same
  * format; its first compressed_count[b] rows join the same softmax after the local rows
  * (src/graph/core.c:437-468, the class whose visible compressed rows are a prefix).
+ * selected (optional, int32 [batch][selected_stride]): the compressed rows are instead the
+ * listed positions of the session's compressed sequence, in list order, compressed_count[b]
+ * of them (the selected class, src/graph/core.c:443-452).
  */
 int yvo_mla_decode_bf16(const uint16_t *q, const uint16_t *pool,
                         const int32_t *page_table, const int32_t *context,
@@ -177,7 +180,8 @@ int yvo_mla_decode_bf16(const uint16_t *q, const uint16_t *pool,
                         const float *sinks, uint64_t sliding_window,
                         const uint16_t *compressed_pool, const int32_t *compressed_table,
                         const int32_t *compressed_count, uint64_t compressed_pool_pages,
-                        uint64_t compressed_table_stride, int threads);
+                        uint64_t compressed_table_stride, const int32_t *selected,
+                        uint64_t selected_stride, int threads);
 
 /*
  * Log-sum-exp merge of split partials for one head: part p holds a normalised

@@ -59,7 +59,7 @@ def load_oracle():
     lib.yvo_shared_kv_head.argtypes = [f32p, f32p, C.c_size_t, u64, u64, u64, C.c_double, f32p, f32p, f64p]
     lib.yvo_rotary_half_bf16.argtypes = [u16p, f32p, f32p] + [u64] * 4
     lib.yvo_sigmoid_gate_bf16.argtypes = [f32p, f32p, u64, f32p]
-    lib.yvo_mla_decode_bf16.argtypes = [u16p, u16p, i32p, i32p, f32p, u16p, f64p] + [u64] * 7 + [f32p, u64, u16p, i32p, i32p, u64, u64, C.c_int]
+    lib.yvo_mla_decode_bf16.argtypes = [u16p, u16p, i32p, i32p, f32p, u16p, f64p] + [u64] * 7 + [f32p, u64, u16p, i32p, i32p, u64, u64, i32p, u64, C.c_int]
     lib.yvo_lse_merge.argtypes = [f32p, f64p, u64, u64, f32p, f64p]
     return lib
 
@@ -224,9 +224,9 @@ class Oracle:
         return out
 
     def mla_decode(self, q, pool, page_table, context, value_dim, page_tokens, threads=None,
-                   sinks=None, sliding_window=0, compressed=None):
+                   sinks=None, sliding_window=0, compressed=None, selected=None):
         """compressed: optional (pool uint16 [pages][page_tokens][kd], table int32 [b][stride],
-        counts int32 [b]) second row set."""
+        counts int32 [b]) second row set; selected: optional int32 [b][capacity] row lists."""
         b, h, kd = q.shape
         page_table = np.ascontiguousarray(page_table, dtype=np.int32)
         context = np.ascontiguousarray(context, dtype=np.int32)
@@ -235,13 +235,15 @@ class Oracle:
         lse = np.zeros((b, h), dtype=np.float64)
         if sinks is not None:
             sinks = np.ascontiguousarray(sinks, dtype=np.float32)
-        extra = (None, None, None, 0, 0)
+        extra = (None, None, None, 0, 0, None, 0)
         if compressed is not None:
             cpool = np.ascontiguousarray(compressed[0], dtype=np.uint16)
             ctable = np.ascontiguousarray(compressed[1], dtype=np.int32)
             ccount = np.ascontiguousarray(compressed[2], dtype=np.int32)
+            chosen = np.ascontiguousarray(selected, dtype=np.int32) if selected is not None else None
             extra = (_ptr(cpool, u16p), _ptr(ctable, i32p), _ptr(ccount, i32p), cpool.shape[0],
-                     ctable.shape[1])
+                     ctable.shape[1], _ptr(chosen, i32p) if chosen is not None else None,
+                     chosen.shape[1] if chosen is not None else 0)
         rc = self.lib.yvo_mla_decode_bf16(_ptr(q, u16p), _ptr(pool, u16p), _ptr(page_table, i32p),
                                           _ptr(context, i32p), _ptr(out, f32p), _ptr(outb, u16p),
                                           _ptr(lse, f64p), b, h, kd, value_dim, page_tokens,

@@ -27,13 +27,15 @@ def make_case(rng, contexts, spare=2):
     return q, pool, table, np.array(contexts, dtype=np.int32)
 
 
-def run_mla(backend, q, pool, table, ctx, max_context=None, sinks=None, window=0, compressed=None):
+def run_mla(backend, q, pool, table, ctx, max_context=None, sinks=None, window=0, compressed=None,
+            selected=None):
     batch = q.shape[0]
     extra = {}
     if compressed is not None:
         extra = dict(compressed_pool_pages=compressed[0].shape[0],
                      compressed_table_stride=compressed[1].shape[1],
-                     max_compressed_tokens=int(compressed[1].shape[1] * PAGE))
+                     max_compressed_tokens=int(compressed[1].shape[1] * PAGE),
+                     compressed_selected_stride=selected.shape[1] if selected is not None else 0)
     req = backend.mla_requirement(batch, HEADS, KEY_DIM, VALUE_DIM, PAGE, pool.shape[0],
                                   table.shape[1], max_context or int(table.shape[1] * PAGE),
                                   sliding_window=window, **extra)
@@ -49,6 +51,8 @@ def run_mla(backend, q, pool, table, ctx, max_context=None, sinks=None, window=0
         tc = [backend.tensor("cpool", B.DTYPE_BF16, compressed[0].shape, compressed[0]),
               backend.tensor("ctable", B.DTYPE_I32, compressed[1].shape, compressed[1]),
               backend.tensor("ccount", B.DTYPE_I32, compressed[2].shape, compressed[2])]
+        if selected is not None:
+            tc.append(backend.tensor("selected", B.DTYPE_I32, selected.shape, selected))
     facts = backend.mla_decode_execute(req, *tensors, out, lse, sinks=ts, compressed=tc)
     result = out.read(), lse.read(), facts
     for t in tensors + [out, lse] + ([ts] if ts else []) + (tc or []):
@@ -173,3 +177,31 @@ def test_mla_compressed_candidate_rows(backend, window):
     assert_close_bf16(got, ref, "mla compressed window=%d" % window)
     assert_lse(lse, ref_lse, "mla compressed window=%d" % window)
     assert facts.kernel_launches == 3 and facts.accelerated_matrix_launches == 2
+
+
+def test_mla_selected_compressed_rows(backend):
+    """The selected class (src/graph/core.c:443-452): per-session index lists into the compressed
+    sequence, gathered in list order (repeats allowed), list lengths from 0 to the capacity."""
+    rng = np.random.default_rng(700)
+    contexts = [1, 70, 129, 1000, 4097, 300]
+    stored = [64, 10, 200, 700, 2048, 65]
+    capacity = 512
+    counts = np.array([0, 1, 31, 512, 300, 65], np.int32)
+    q, pool, table, ctx = make_case(rng, contexts)
+    _, cpool, ctable, _ = make_case(rng, stored)
+    lists = np.stack([rng.integers(0, stored[i], capacity) for i in range(len(stored))]).astype(np.int32)
+    sinks = (rng.standard_normal(HEADS) * 2.0).astype(np.float32)
+    got, lse, facts = run_mla(backend, q, pool, table, ctx, sinks=sinks, window=128,
+                              compressed=(cpool, ctable, counts), selected=lists)
+    rc, ref, _, ref_lse = ORACLE.mla_decode(q, pool, table, ctx, VALUE_DIM, PAGE, sinks=sinks,
+                                            sliding_window=128, compressed=(cpool, ctable, counts),
+                                            selected=lists)
+    assert rc == 0
+    assert_close_bf16(got, ref, "mla selected")
+    assert_lse(lse, ref_lse, "mla selected")
+    assert facts.kernel_launches == 4
+    bad = lists.copy()
+    bad[3, 100] = int(ctable.shape[1] * PAGE)          # one past what the table can address
+    with pytest.raises(YvexError) as e:
+        run_mla(backend, q, pool, table, ctx, compressed=(cpool, ctable, counts), selected=bad)
+    assert e.value.code == B.YVEX_ERR_BOUNDS

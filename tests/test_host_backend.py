@@ -421,6 +421,21 @@ def test_paged_and_mla_admission():
         with pytest.raises(YvexError) as e:                 # declared but not passed
             b.mla_decode_execute(both, mq, latent, mtable, mctx, mout)
         assert e.value.code == B.YVEX_ERR_FORMAT
+        chosen = b.mla_requirement(16, 128, 576, 512, 64, 2048, 128, 8192, compressed_pool_pages=40,
+                                   compressed_table_stride=2, max_compressed_tokens=128,
+                                   compressed_selected_stride=96)
+        assert b.mla_decode_workspace_required(chosen) > b.mla_decode_workspace_required(both)
+        lists = written(b, "sel", B.DTYPE_I32, (16, 96))
+        facts = b.mla_decode_execute(chosen, mq, latent, mtable, mctx, mout,
+                                     compressed=[cpool, ctable, ccount, lists])
+        assert facts.kernel_launches == 4 and facts.accelerated_matrix_launches == 2
+        with pytest.raises(YvexError) as e:                 # a list without the class declared on it
+            b.mla_decode_execute(chosen, mq, latent, mtable, mctx, mout, compressed=[cpool, ctable, ccount])
+        assert e.value.code == B.YVEX_ERR_FORMAT
+        with pytest.raises(YvexError) as e:                 # a list needs a compressed set
+            b.mla_decode_workspace_required(b.mla_requirement(
+                16, 128, 576, 512, 64, 2048, 128, 8192, compressed_selected_stride=96))
+        assert e.value.code == B.YVEX_ERR_INVALID_ARG
         with pytest.raises(YvexError) as e:                 # more rows than the table can address
             b.mla_decode_workspace_required(b.mla_requirement(
                 16, 128, 576, 512, 64, 2048, 128, 8192, compressed_pool_pages=40,

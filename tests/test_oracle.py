@@ -622,3 +622,36 @@ def test_mla_compressed_rows_join_the_same_softmax_after_the_local_rows():
                                            compressed=(cpool, ctable, np.zeros(3, np.int32)))
     rc3, out3, _, lse3 = ORACLE.mla_decode(q, pool, table, ctx, vd, pt, sinks=sinks, sliding_window=window)
     assert rc2 == 0 and rc3 == 0 and np.array_equal(out2, out3) and np.array_equal(lse2, lse3)
+
+
+def test_mla_selected_rows_are_the_listed_rows_in_list_order():
+    """The identity list equals the prefix class bit for bit; an arbitrary list (repeats
+    allowed) equals one context holding the local rows then the listed rows."""
+    rng = np.random.default_rng(69)
+    contexts, stored = [20, 130], [40, 90]
+    q, pool, table, ctx, vd, pt = _mla_case(rng, contexts)
+    _, cpool, ctable, _, _, _ = _mla_case(rng, stored)
+    kd = pool.shape[-1]
+    counts = np.array([7, 33], np.int32)
+    identity = np.tile(np.arange(40, dtype=np.int32), (2, 1))
+    a = ORACLE.mla_decode(q, pool, table, ctx, vd, pt, compressed=(cpool, ctable, counts))
+    b = ORACLE.mla_decode(q, pool, table, ctx, vd, pt, compressed=(cpool, ctable, counts), selected=identity)
+    assert a[0] == 0 and b[0] == 0 and np.array_equal(a[1], b[1]) and np.array_equal(a[3], b[3])
+    lists = np.stack([rng.integers(0, stored[i], 40) for i in range(2)]).astype(np.int32)
+    rc, out, _, lse = ORACLE.mla_decode(q, pool, table, ctx, vd, pt, compressed=(cpool, ctable, counts),
+                                        selected=lists)
+    assert rc == 0
+    for i, n in enumerate(contexts):
+        local = pool[table[i, :(n + pt - 1) // pt]].reshape(-1, kd)[:n]
+        stored_rows = cpool[ctable[i, :(stored[i] + pt - 1) // pt]].reshape(-1, kd)
+        rows = np.concatenate([local, stored_rows[lists[i, :counts[i]]]])
+        pages = (len(rows) + pt - 1) // pt
+        joined = np.zeros((pages, pt, kd), np.uint16)
+        joined.reshape(-1, kd)[:len(rows)] = rows
+        rc1, out1, _, lse1 = ORACLE.mla_decode(q[i:i + 1], joined, np.arange(pages, dtype=np.int32)[None, :],
+                                               np.array([len(rows)], np.int32), vd, pt)
+        assert rc1 == 0 and np.array_equal(out1[0], out[i]) and np.array_equal(lse1[0], lse[i])
+    bad = lists.copy()
+    bad[1, 3] = 10 ** 6
+    assert ORACLE.mla_decode(q, pool, table, ctx, vd, pt, compressed=(cpool, ctable, counts),
+                             selected=bad)[0] != 0
