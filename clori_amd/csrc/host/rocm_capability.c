@@ -362,19 +362,32 @@ int yvex_rocm_launch(yvex_backend *backend, yvex_rocm_function_id function,
     arguments[0] = params;
     probe = !state->recording && state->probe_function == (int)function &&
             state->probe_count < YVEX_ROCM_PROBE_MAX;
-    if (probe)
-        probe = state->driver.hipEventRecord(state->probe_events[2u * state->probe_count],
-                                             state->stream) == hipSuccess;
-    rc = yvex_rocm_status(&state->driver,
-                          state->driver.hipModuleLaunchKernel(state->functions[function], grid_x,
-                                                              grid_y, grid_z, block, 1u, 1u,
-                                                              lds_bytes, state->stream, arguments,
-                                                              NULL),
-                          where, err);
-    if (probe && rc == YVEX_OK &&
-        state->driver.hipEventRecord(state->probe_events[2u * state->probe_count + 1u],
-                                     state->stream) == hipSuccess)
-        state->probe_count++;
+    if (probe && state->driver.timed_launch && (unsigned long long)grid_x * block <= 0xffffffffull) {
+        /* the two events take the kernel's own begin and end timestamps */
+        rc = yvex_rocm_status(&state->driver,
+                              state->driver.timed_launch(state->functions[function], grid_x * block,
+                                                         grid_y, grid_z, block, 1u, 1u, lds_bytes,
+                                                         state->stream, arguments, NULL,
+                                                         state->probe_events[2u * state->probe_count],
+                                                         state->probe_events[2u * state->probe_count + 1u],
+                                                         0u),
+                              where, err);
+        if (rc == YVEX_OK) state->probe_count++;
+    } else {
+        if (probe)
+            probe = state->driver.hipEventRecord(state->probe_events[2u * state->probe_count],
+                                                 state->stream) == hipSuccess;
+        rc = yvex_rocm_status(&state->driver,
+                              state->driver.hipModuleLaunchKernel(state->functions[function], grid_x,
+                                                                  grid_y, grid_z, block, 1u, 1u,
+                                                                  lds_bytes, state->stream, arguments,
+                                                                  NULL),
+                              where, err);
+        if (probe && rc == YVEX_OK &&
+            state->driver.hipEventRecord(state->probe_events[2u * state->probe_count + 1u],
+                                         state->stream) == hipSuccess)
+            state->probe_count++;
+    }
     if (rc != YVEX_OK) capability_fail(backend, variant, YVEX_BACKEND_CAPABILITY_REASON_LAUNCH_FAILED);
     else if (state->recording) state->recorded_launches++;
     return rc;

@@ -43,6 +43,8 @@ int yvex_rocm_driver_load(yvex_rocm_driver *driver, yvex_error *err)
     }
     YVEX_ROCM_DRIVER_ENTRIES(X)
 #undef X
+    driver->timed_launch =
+        (yvex_rocm_timed_launch_fn)dlsym(driver->library, "hipExtModuleLaunchKernel");
     yvex_error_clear(err);
     return YVEX_OK;
 }

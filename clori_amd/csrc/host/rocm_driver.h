@@ -24,12 +24,19 @@
     X(hipStreamBeginCapture) X(hipStreamEndCapture) X(hipGraphInstantiate) X(hipGraphLaunch) \
     X(hipGraphExecDestroy) X(hipGraphDestroy)
 
+/* hipExtModuleLaunchKernel (hip/hip_ext.h, a C++ header): a launch whose two events take the
+ * kernel's own begin and end timestamps.  Work sizes are in threads, not workgroups. */
+typedef hipError_t (*yvex_rocm_timed_launch_fn)(hipFunction_t, uint32_t, uint32_t, uint32_t, uint32_t,
+                                                uint32_t, uint32_t, size_t, hipStream_t, void **,
+                                                void **, hipEvent_t, hipEvent_t, uint32_t);
+
 typedef struct yvex_rocm_driver {
     void *library;
     char library_name[256];
 #define X(name) __typeof__(&name) name;
     YVEX_ROCM_DRIVER_ENTRIES(X)
 #undef X
+    yvex_rocm_timed_launch_fn timed_launch; /* optional: NULL when the runtime lacks it */
 } yvex_rocm_driver;
 
 /* Loads the runtime library and resolves every entry or none (YVEX_ERR_UNSUPPORTED). */
