@@ -23,20 +23,27 @@
  *       compiled reference decode via oracle/_ref is not available (the block
  *       encoder is a static function) -> invariants: decode(encode(x)) error
  *       <= scale/2, idempotence
- *   yvo_shared_kv_head               pinned: sink KAT
- *       (tests/reference/deepseek_attention.c:2722-2725); sink=-inf reduces to
- *       yvo_attention_head within 1e-6
+ *   yvo_shared_kv_head, and through it yvo_mla_decode_bf16 with sink logits, the
+ *   sliding window and the dense compressed rows
+ *       pinned: sink KAT (tests/reference/deepseek_attention.c:2722-2725); the
+ *       reference's own reduce (yvex_attention_reduce_chunk, src/graph/core.c)
+ *       compiled into oracle/_ref/libyvex_ref_reduce.so, bit for bit on every
+ *       lane it does not rotate and on the other two after the same rotation;
+ *       committed outputs of that reduce (tests/golden); the sink-free path
+ *       equals a sink that underflows, bit for bit
  *   yvo_rotary_half_bf16             pinned: known-answer case
  *       (tests/unit/cuda/quant_qtype.c:1988-2061), identity, quarter turn,
  *       float64 rotation within bf16 rounding
  *   yvo_sigmoid_gate_bf16            pinned: known-answer case
  *       (tests/unit/cuda/quant_qtype.c:2979-2981,3019-3033), closed forms
- *   yvo_paged_*, yvo_mla_*, yvo_lse_merge
+ *   yvo_paged_*, the page tables and LSE output of yvo_mla_*, the selected
+ *   compressed class, yvo_lse_merge
  *       parity unpinned by the reference (it has no page table, no LSE, no
- *       split-K, no Q8_0 KV cache).  Pinned here only by construction
- *       invariants: paged == contiguous on the gathered copy (bit-exact),
- *       page-placement permutation invariance, LSE closed forms, merge
- *       associativity.
+ *       split-K, no Q8_0 KV cache; its selected class needs the indexer that
+ *       is outside this path).  Pinned here only by construction invariants:
+ *       paged == contiguous on the gathered copy (bit-exact), page-placement
+ *       permutation invariance, LSE closed forms, merge associativity,
+ *       selected list == the listed rows concatenated (bit-exact).
  */
 #ifndef YVEX_ATTENTION_ORACLE_H
 #define YVEX_ATTENTION_ORACLE_H

@@ -15,7 +15,8 @@ import numpy as np
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, os.path.dirname(HERE))
-from oracle_binding import f32p, load_reference, _ptr  # noqa: E402
+from oracle_binding import (f32p, load_reference, load_reference_reduce, reference_reduce,  # noqa: E402
+                            _ptr)
 
 # (name, seq_len, head_dim, position, causal)
 CASES = [
@@ -27,6 +28,29 @@ CASES = [
     ("decode-4096", 4096, 128, 4095, 1),
     ("long-16384", 16384, 128, 16383, 1),
 ]
+
+
+# Shared-KV reduce of one query token (yvex_attention_reduce_chunk):
+# (name, attention class, sliding window, context, stored compressed rows, heads, dim)
+REDUCE_CASES = [
+    ("reduce-one-row", 0, 128, 1, 0, 2, 64),
+    ("reduce-window-16", 0, 16, 90, 0, 4, 64),
+    ("reduce-window-wide", 0, 1 << 20, 300, 0, 4, 64),
+    ("reduce-compressed-127", 2, 64, 127, 3, 4, 64),
+    ("reduce-compressed-128", 2, 64, 128, 3, 4, 64),
+    ("reduce-compressed-700", 2, 128, 700, 7, 4, 128),
+]
+REDUCE_RATIO = 128
+
+
+def reduce_inputs(heads, dim, context, stored):
+    """bf16-representable patterns: query, local rows (positions 0 .. context-1), compressed
+    rows (positions 0, 128, 256, ...), sink logits."""
+    q = pattern(heads * dim, 3, 0, 19, 9, 8).reshape(heads, dim)
+    local = pattern(context * dim, 5, 2, 23, 11, 16).reshape(context, dim)
+    compressed = pattern(max(stored, 1) * dim, 7, 1, 29, 14, 16).reshape(-1, dim)[:stored]
+    sinks = pattern(heads, 1, 0, 5, 2, 2)
+    return q, local, compressed, sinks
 
 
 def pattern(count, mul, add, mod, offset, div):
@@ -80,6 +104,17 @@ def main():
         ref.yvref_q8_0_encode_block(_ptr(np.ascontiguousarray(blocks[32 * b:32 * b + 32]), f32p),
                                     enc[34 * b:].ctypes.data_as(C.POINTER(C.c_ubyte)))
     out["codec/q8_0"] = enc
+    reduce = load_reference_reduce()
+    if reduce is None:
+        sys.exit("oracle/_ref/libyvex_ref_reduce.so is not built: run `make -C oracle ref`")
+    for name, attention_class, window, context, stored, heads, dim in REDUCE_CASES:
+        q, local, compressed, sinks = reduce_inputs(heads, dim, context, stored)
+        rc, o = reference_reduce(reduce, q, local, np.arange(context), compressed,
+                                 np.arange(stored) * REDUCE_RATIO, sinks, window,
+                                 REDUCE_RATIO if attention_class == 2 else 0, attention_class,
+                                 context - 1)
+        assert rc == 0, (name, rc)
+        out[name + "/out"] = o
     np.savez_compressed(os.path.join(HERE, "reference_attention.npz"), **out)
     print("wrote", len(out), "arrays")
 

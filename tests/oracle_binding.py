@@ -64,6 +64,41 @@ def load_oracle():
     return lib
 
 
+REF_REDUCE_SO = os.path.join(os.path.dirname(REF_SO), "libyvex_ref_reduce.so")
+
+
+def load_reference_reduce():
+    """The compiled reference shared-KV reduce, or None when oracle/_ref was not built."""
+    if not os.path.exists(REF_REDUCE_SO):
+        return None
+    lib = C.CDLL(REF_REDUCE_SO)
+    u64p = C.POINTER(C.c_ulonglong)
+    lib.yvref_attention_reduce.argtypes = [f32p, f32p, u64p, u64, f32p, u64p, u64, f32p, u64, u64,
+                                           u64, u64, C.c_uint, u64, u64, u64, f32p]
+    return lib
+
+
+def reference_reduce(lib, query, local, local_positions, compressed, compressed_positions, sinks,
+                     sliding_window, compression_ratio, attention_class, position,
+                     rope_dims=2, theta=10000):
+    """One query token through the reference reduce; returns (status, out [heads][dim])."""
+    query = np.ascontiguousarray(query, dtype=np.float32)
+    local = np.ascontiguousarray(local, dtype=np.float32)
+    local_positions = np.ascontiguousarray(local_positions, dtype=np.uint64)
+    compressed = np.ascontiguousarray(compressed, dtype=np.float32).reshape(-1, query.shape[1])
+    compressed_positions = np.ascontiguousarray(compressed_positions, dtype=np.uint64)
+    sinks = np.ascontiguousarray(sinks, dtype=np.float32)
+    out = np.zeros_like(query)
+    u64p = C.POINTER(C.c_ulonglong)
+    rc = lib.yvref_attention_reduce(
+        _ptr(query, f32p), _ptr(local, f32p), _ptr(local_positions, u64p), local.shape[0],
+        _ptr(compressed, f32p) if len(compressed) else None,
+        _ptr(compressed_positions, u64p) if len(compressed) else None, compressed.shape[0],
+        _ptr(sinks, f32p), query.shape[0], query.shape[1], sliding_window, compression_ratio,
+        attention_class, position, rope_dims, theta, _ptr(out, f32p))
+    return rc, out
+
+
 def load_reference():
     """The compiled reference operator, or None when oracle/_ref was not built."""
     if not os.path.exists(REF_SO):

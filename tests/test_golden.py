@@ -43,3 +43,39 @@ def test_codecs_match_reference_bits():
     blocks = make_golden.pattern(64, 11, 3, 61, 30, 7)
     enc = ORACLE.q8_0_encode_rows(blocks.reshape(2, 32)).reshape(-1)
     assert np.array_equal(enc, GOLDEN["codec/q8_0"])
+
+
+@pytest.mark.parametrize("case", make_golden.REDUCE_CASES, ids=[c[0] for c in make_golden.REDUCE_CASES])
+def test_shared_kv_reduce_matches_reference_output_bits(case):
+    """yvo_mla_decode_bf16 (sink logits, sliding window, dense compressed rows; key_dim ==
+    value_dim as in the reference) against committed outputs of yvex_attention_reduce_chunk.
+    The reference rounds the row to bf16, rotates its last two lanes back by the position
+    and rounds again (src/graph/core.c:499-507): the other lanes compare as they are, the last
+    two after the same rotation."""
+    import math
+    name, attention_class, window, context, stored, heads, dim = case
+    q, local, compressed, sinks = make_golden.reduce_inputs(heads, dim, context, stored)
+    page = 16
+
+    def paged(rows):
+        pages = max((len(rows) + page - 1) // page, 1)
+        pool = np.zeros((pages, page, dim), np.uint16)
+        pool.reshape(-1, dim)[:len(rows)] = ORACLE.bf16_encode(rows)
+        return pool, np.arange(pages, dtype=np.int32)[None, :]
+
+    pool, table = paged(local)
+    cpool, ctable = paged(compressed)
+    visible = np.array([context // make_golden.REDUCE_RATIO if attention_class == 2 else 0], np.int32)
+    rc, out, _, _ = ORACLE.mla_decode(ORACLE.bf16_encode(q)[None], pool, table,
+                                      np.array([context], np.int32), dim, page, sinks=sinks,
+                                      sliding_window=window,
+                                      compressed=(cpool, ctable, visible) if attention_class == 2 else None)
+    assert rc == 0
+    mine = ORACLE.bf16_decode(ORACLE.bf16_encode(out[0]))
+    want = GOLDEN[name + "/out"]
+    assert np.array_equal(mine[:, :-2].view(np.uint32), want[:, :-2].view(np.uint32))
+    c, s = math.cos(float(context - 1)), -math.sin(float(context - 1))
+    for h in range(heads):
+        x, y = float(mine[h, -2]), float(mine[h, -1])
+        tail = ORACLE.bf16_decode(ORACLE.bf16_encode(np.array([x * c - y * s, x * s + y * c], np.float32)))
+        assert np.array_equal(tail, want[h, -2:])

@@ -6,11 +6,15 @@ import numpy as np
 import pytest
 
 import reference_vectors as rv
-from oracle_binding import Oracle, load_reference, _ptr, f32p, u16p, u8p
+from oracle_binding import (Oracle, load_reference, load_reference_reduce, reference_reduce, _ptr,
+                            f32p, u16p, u8p)
 
 ORACLE = Oracle()
 REF = load_reference()
 needs_ref = pytest.mark.skipif(REF is None, reason="oracle/_ref not built (reference tree absent)")
+REF_REDUCE = load_reference_reduce()
+needs_ref_reduce = pytest.mark.skipif(REF_REDUCE is None,
+                                      reason="oracle/_ref not built (reference tree absent)")
 
 
 # ---------------------------------------------------------------- exp -------
@@ -655,3 +659,62 @@ def test_mla_selected_rows_are_the_listed_rows_in_list_order():
     bad[1, 3] = 10 ** 6
     assert ORACLE.mla_decode(q, pool, table, ctx, vd, pt, compressed=(cpool, ctable, counts),
                              selected=bad)[0] != 0
+
+
+# ------------------------- the shared-KV oracle against the compiled reference reduce ----
+
+def _reference_tail(row_bf16, position, theta=10000):
+    """What the reference does to a published row after the softmax (src/graph/core.c:499-507):
+    the last two lanes rotated back by the token position, then rounded to bf16 again."""
+    row = row_bf16.astype(np.float64).copy()
+    c, s = math.cos(float(position)), -math.sin(float(position))      # pair 0: frequency 1
+    x, y = row[-2], row[-1]
+    row[-2], row[-1] = np.float32(x * c - y * s), np.float32(x * s + y * c)
+    return ORACLE.bf16_decode(ORACLE.bf16_encode(row.astype(np.float32)))
+
+
+@needs_ref_reduce
+@pytest.mark.parametrize("attention_class,window,contexts", [
+    (0, 10 ** 6, [1, 2, 17, 300]), (0, 16, [1, 16, 17, 90]), (0, 1, [5]),
+    (2, 64, [1, 127, 128, 129, 700]), (2, 10 ** 6, [255, 256, 1000]),
+])
+def test_mla_oracle_matches_compiled_reference_reduce(attention_class, window, contexts):
+    """Sink logits, the sliding-window filter and the dense compressed class of
+    yvo_mla_decode_bf16 (paged rows, key_dim == value_dim as in the reference) against
+    yvex_attention_reduce_chunk compiled from the reference sources: every lane the reference
+    does not rotate is bit-identical, and so are the two it rotates once the same rotation
+    is applied."""
+    rng = np.random.default_rng(71 + attention_class + window % 97)
+    heads, d, pt, ratio = 4, 64, 16, 128
+    q, pool, table, ctx, _, _ = _mla_case(rng, contexts, heads=heads, kd=d, vd=d, pt=pt)
+    stored = [n // ratio + 2 for n in contexts]                      # two not yet visible
+    _, cpool, ctable, _, _, _ = _mla_case(rng, stored, heads=heads, kd=d, vd=d, pt=pt)
+    visible = np.array([n // ratio for n in contexts], np.int32) if attention_class == 2 \
+        else np.zeros(len(contexts), np.int32)
+    sinks = (rng.standard_normal(heads) * 2.0).astype(np.float32)
+    rc, out, _, _ = ORACLE.mla_decode(q, pool, table, ctx, d, pt, sinks=sinks, sliding_window=window,
+                                      compressed=(cpool, ctable, visible) if attention_class == 2 else None)
+    assert rc == 0
+    for b, n in enumerate(contexts):
+        local = ORACLE.bf16_decode(pool[table[b, :(n + pt - 1) // pt]].reshape(-1, d)[:n])
+        comp = ORACLE.bf16_decode(cpool[ctable[b, :(stored[b] + pt - 1) // pt]].reshape(-1, d)[:stored[b]])
+        rc1, ref = reference_reduce(
+            REF_REDUCE, ORACLE.bf16_decode(q[b]), local, np.arange(n), comp if attention_class == 2 else
+            np.zeros((0, d), np.float32), np.arange(stored[b]) * ratio if attention_class == 2 else [],
+            sinks, window, ratio if attention_class == 2 else 0, attention_class, n - 1)
+        assert rc1 == 0
+        mine = ORACLE.bf16_decode(ORACLE.bf16_encode(out[b]))
+        assert np.array_equal(mine[:, :-2], ref[:, :-2]), (attention_class, window, n)
+        for h in range(heads):
+            assert np.array_equal(_reference_tail(mine[h], n - 1)[-2:], ref[h, -2:])
+
+
+@needs_ref_reduce
+def test_no_sink_equals_a_sink_that_underflows():
+    """The reference always has a sink; the oracle's sink-free path equals a sink so negative
+    that exp() of it is zero, which is how the sink-free configurations are tied to it."""
+    rng = np.random.default_rng(72)
+    q, pool, table, ctx, vd, pt = _mla_case(rng, [1, 40, 333])
+    a = ORACLE.mla_decode(q, pool, table, ctx, vd, pt)
+    b = ORACLE.mla_decode(q, pool, table, ctx, vd, pt, sinks=np.full(4, -1e30, np.float32))
+    assert a[0] == 0 and b[0] == 0 and np.array_equal(a[1], b[1]) and np.array_equal(a[3], b[3])
