@@ -456,6 +456,14 @@ def main():
         "roofline": roof,
         "cpu_baseline": cpu.get(headline),
         "device_probe": device_probe,
+        # the metric has two halves; `value` carries the first (decode, HBM GB/s), this the
+        # second (causal prefill, TFLOP/s), when that workload ran
+        "prefill": ({"metric": "prefill attn TFLOPS (% MFMA peak)",
+                     "value": roofline(results["prefill2"])["step"], "unit": "TFLOP/s",
+                     "ms_per_step": results["prefill2"]["ms"],
+                     "config": {"workload": results["prefill2"]["workload"]},
+                     "roofline": roofline(results["prefill2"]),
+                     "cpu_baseline": cpu.get("prefill2")} if "prefill2" in results else None),
         "workloads": {n: dict(workload=r["workload"], ms_per_step=r["ms"],
                               wall_ms_per_step=r["wall_ms"], value=roofline(r)["step"],
                               unit=roofline(r)["unit"], roofline=roofline(r),

@@ -19,10 +19,10 @@
  *       (tests/reference/deepseek_attention.c:2696-2698), exhaustive 2^16
  *       round trips, compiled reference codecs (oracle/_ref)
  *   yvo_q8_0_*                       pinned: golden block
- *       (tests/unit/quant_numeric.c:514-526), zero block, refusal cases,
- *       compiled reference decode via oracle/_ref is not available (the block
- *       encoder is a static function) -> invariants: decode(encode(x)) error
- *       <= scale/2, idempotence
+ *       (tests/unit/quant_numeric.c:514-526), zero block, refusal cases, the
+ *       compiled reference block encoder and decoder (oracle/_ref, through
+ *       yvex_quant_encode_block / yvex_quant_decode_block) on seeded blocks,
+ *       and the invariants decode(encode(x)) error <= scale/2, idempotence
  *   yvo_shared_kv_head, and through it yvo_mla_decode_bf16 with sink logits, the
  *   sliding window and the dense compressed rows
  *       pinned: sink KAT (tests/reference/deepseek_attention.c:2722-2725); the
