@@ -392,7 +392,8 @@ yvex_rocm_kv_append_q8_0(const yvex_rocm_kv_append_params p)
             }
             *reinterpret_cast<uint32_t *>(vdst + id * 4u) = w;
         }
-        if (!ok) flag(p.status, YVEX_ROCM_DEVICE_NUMERIC);
-        if (!representable) flag(p.status, YVEX_ROCM_DEVICE_CONTRACT);
+        // a block whose scale f16 cannot hold is refused like a non-finite value, as the
+        // reference encoder refuses it (src/gguf/quant_block.c:172-174)
+        if (!ok || !representable) flag(p.status, YVEX_ROCM_DEVICE_NUMERIC);
     }
 }

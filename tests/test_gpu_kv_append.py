@@ -196,6 +196,20 @@ def test_append_refusals(backend):
     with pytest.raises(YvexError) as e:
         small_append(backend, k_bad, 0, 2)
     assert e.value.code == B.YVEX_ERR_FORMAT
+    # a Q8_0 block whose scale overflows f16 (max / 127 > 65504) -> FORMAT, as the encoder refuses it
+    huge = bf16_normal(rng, (1, HKV, D))
+    huge[0, 2, 40] = ORACLE.bf16_encode(np.array([1.0e7], np.float32))[0]
+    tensors = [backend.tensor("k", B.DTYPE_BF16, huge.shape, huge),
+               backend.tensor("v", B.DTYPE_BF16, huge.shape, huge),
+               backend.tensor("r", B.DTYPE_I32, (1,), np.array([0], np.int32)),
+               backend.tensor("s", B.DTYPE_I32, (1,), np.array([0], np.int32)),
+               backend.tensor("c", B.DTYPE_I32, (1,), np.array([1], np.int32)),
+               backend.tensor("t", B.DTYPE_I32, (1, 2), np.array([[0, 1]], np.int32)),
+               backend.tensor("kp", B.DTYPE_I8, (4 * HKV * 2176,)),
+               backend.tensor("vp", B.DTYPE_I8, (4 * HKV * 2176,))]
+    with pytest.raises(YvexError) as e:
+        backend.kv_append_execute(*tensors, HKV, 4, 1, storage=B.KV_Q8_0)
+    assert e.value.code == B.YVEX_ERR_FORMAT
     # rotary dimension that is not a multiple of 16 -> UNSUPPORTED (refused on the host)
     with pytest.raises(YvexError) as e:
         run_case(backend, rng, [0], [1], B.KV_BF16, 24)
