@@ -4,7 +4,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu]
 
 A step is one pass of the attention operator over one batch of synthetic input that is
-already resident in HBM.  Workloads are BASELINE.json's configurations:
+already resident in HBM.  Workloads are the five configurations the metric is quoted on:
 
     prefill2   causal GQA prefill, T=2048, 40/8 heads, d=128            (MFMA bound)
     decode1    contiguous decode, 32/8 heads, d=128, context 4096        (HBM bound)

@@ -115,7 +115,7 @@ int yvo_gqa_attention(const float *q, const float *k, const float *v, float *out
                       uint64_t k_stride, uint64_t v_stride, int causal,
                       int threads);
 
-/* bf16 in / bf16 out wrapper used for BASELINE configs 1 and 2: widens exactly to
+/* bf16 in / bf16 out wrapper used for benchmark configurations 1 and 2: widens exactly to
  * F32, runs yvo_gqa_attention, returns the F32 result and its RNE bf16 rounding. */
 int yvo_gqa_attention_bf16(const uint16_t *q, const uint16_t *k, const uint16_t *v,
                            float *out_f32, uint16_t *out_bf16, double *lse,
@@ -164,7 +164,7 @@ int yvo_shared_kv_head(const float *q, const float *rows, size_t row_stride,
                        double scale, const float *sink, float *out, double *lse);
 
 /*
- * Absorbed-latent MLA decode over a paged latent cache (BASELINE config 5).
+ * Absorbed-latent MLA decode over a paged latent cache (benchmark configuration 5).
  * q bf16 [batch][heads][key_dim]; pool bf16 [pool_pages][page_tokens][key_dim];
  * value = first value_dim lanes of each row; scale = 1/sqrt(key_dim) in double
  * (src/graph/core.c:604).  Output is F32 plus RNE bf16 [batch][heads][value_dim].

@@ -37,7 +37,7 @@ def run_rows_decode(backend, q, k, v, query_start, causal=True, k_stride=0, v_st
 
 
 def test_config1_contiguous_decode_matches_cpu_operator(backend):
-    """BASELINE config 1: B=1, 32/8 heads, d=128, ctx 4096, contiguous KV, seed 1."""
+    """Benchmark configuration 1: B=1, 32/8 heads, d=128, ctx 4096, contiguous KV, seed 1."""
     rng = np.random.default_rng(1)
     q = bf16_normal(rng, (1, 32, 128))
     k = bf16_normal(rng, (4096, 8, 128))
@@ -188,7 +188,7 @@ def test_paged_decode_refuses_bad_page_ids_and_lengths(backend):
 
 
 def test_config3_shape_sample(backend):
-    """BASELINE config 3 at reduced session count (the oracle finishes in seconds): 32/8
+    """Benchmark configuration 3 at reduced session count (the oracle finishes in seconds): 32/8
     heads, d=128, contexts uniform in [512,16384], seeded permutation page tables."""
     rng = np.random.default_rng(3)
     contexts = [int(c) for c in rng.integers(512, 16385, size=6)]
@@ -248,7 +248,7 @@ def test_q8_0_paged_placement_invariance_and_garbage_tail(backend):
 
 
 def test_config4_shape_sample(backend):
-    """BASELINE config 4 at reduced session count: contexts uniform in [4096,32768], K/V as
+    """Benchmark configuration 4 at reduced session count: contexts uniform in [4096,32768], K/V as
     GGUF Q8_0 blocks quantised on the host from N(0,1) bf16 values, seed 4."""
     rng = np.random.default_rng(4)
     contexts = [int(c) for c in rng.integers(4096, 32769, size=3)]

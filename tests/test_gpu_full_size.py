@@ -1,4 +1,4 @@
-"""GPU parity at BASELINE.json's full sizes (configs 3, 4 and 5), against the CPU oracle on
+"""GPU parity at the benchmark's full sizes (configs 3, 4 and 5), against the CPU oracle on
 the same bytes, through the C ABI.
 
 The oracle is multi-threaded C and finishes these sizes in seconds.  To keep input

@@ -25,7 +25,7 @@ def unrelated_eager_work(backend, rng):
 
 
 def test_recorded_row_decode_replays_equal_eager(backend):
-    """BASELINE config 1 (B=1, 32/8 heads, ctx 4096) as a recorded two-launch sequence."""
+    """Benchmark configuration 1 (B=1, 32/8 heads, ctx 4096) as a recorded two-launch sequence."""
     rng = np.random.default_rng(801)
     ctx = 4096
     k, v = bf16_normal(rng, (ctx, 8, 128)), bf16_normal(rng, (ctx, 8, 128))

@@ -73,7 +73,7 @@ def test_mla_decode_matches_shared_kv_oracle_ragged(backend):
 
 
 def test_config5_shape_sample(backend):
-    """BASELINE config 5 at reduced batch: 128 heads, 512+64 latent, context 8192 in 64-token
+    """Benchmark configuration 5 at reduced batch: 128 heads, 512+64 latent, context 8192 in 64-token
     pages, scale 1/sqrt(576), seed 5."""
     rng = np.random.default_rng(5)
     q, pool, table, ctx = make_case(rng, [8192, 8192])

@@ -49,7 +49,7 @@ def test_prefill_matches_cpu_operator(backend, tq, tk, start, hq, hkv, causal):
 
 
 def test_config2_prefill_qwen_shape(backend):
-    """BASELINE config 2: T=2048, 40/8 heads, d=128, causal, N(0,1) values with a per-head
+    """Benchmark configuration 2: T=2048, 40/8 heads, d=128, causal, N(0,1) values with a per-head
     scale drawn U[0.5,1.5], seed 2."""
     rng = np.random.default_rng(2)
     t, hq, hkv, d = 2048, 40, 8, 128
