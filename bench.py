@@ -51,6 +51,7 @@ def random_bf16(rng, count, unique=1 << 24):
     return np.tile(base, reps)[:count]
 
 
+SPIN_UP_SECONDS = float(os.environ.get("YVEX_BENCH_SPIN_UP", "0.2"))
 RECORDED_STEPS = bool(int(os.environ.get("YVEX_BENCH_RECORDED", "0")))
 
 
@@ -67,6 +68,13 @@ def time_steps(backend, run, steps, warmup, kernel):
         run()
         graph = backend.graph_end()
         step = lambda: backend.graph_launch(graph)  # noqa: E731
+    # the part raises its clocks only under sustained load: keep it busy for SPIN_UP_SECONDS
+    # before the W warm-up steps, all untimed
+    spin_until = time.perf_counter() + SPIN_UP_SECONDS
+    while time.perf_counter() < spin_until:
+        for _ in range(16):
+            step()
+        backend.sync()
     for _ in range(warmup):
         step()
     backend.sync()
