@@ -335,9 +335,9 @@ def roofline(result):
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # runs (profiles/), scaled by the same counters on a copy kernel of known size; None where
 # no such run is committed.
-TRAFFIC = {"paged3": 1033345728, "paged4": 1512954963, "decode1": 18117066,
-           "prefill2": 50569339, "mla5": 204066874, "append_bf16": 303924258,
-           "append_q8_0": 239926575}
+TRAFFIC = {"paged3": 1033354309, "paged4": 1512935981, "decode1": 18116273,
+           "prefill2": 50570411, "mla5": 204069253, "append_bf16": 303974816,
+           "append_q8_0": 239922751}
 
 
 def repeat_for(seconds, call):
