@@ -795,14 +795,12 @@ static int rocm_mla_decode_execute(yvex_backend *backend,
     if (max_chunks + extra_max_chunks > 0x7fffffffull ||
         !decode_workspace_bytes(r->batch * (max_chunks + extra_max_chunks), r->heads, r->value_dimension,
                                 sizeof(uint16_t), &acc_bytes, &total) ||
-        !mla_gather_bytes(r, &gather_pages, &gather_rows, &gather_table) ||
-        !yvex_core_u64_add(total, gather_rows + gather_table, &partial_bytes))
+        !mla_gather_bytes(r, &gather_pages, &gather_rows, &gather_table))
         return refuse(err, YVEX_ERR_BOUNDS, where, "MLA decode geometry exceeds admitted range");
-    { /* partials first, then the gathered rows and their page table */
-        const unsigned long long partials = total;
-        total = partial_bytes;
-        partial_bytes = partials;
-    }
+    /* partials first, then the gathered rows and their page table */
+    partial_bytes = total;
+    if (!yvex_core_u64_add(partial_bytes, gather_rows + gather_table, &total))
+        return refuse(err, YVEX_ERR_BOUNDS, where, "MLA decode geometry exceeds admitted range");
     backend_workspace_reset(backend);
     rc = yvex_rocm_temporary_acquire(backend, total, &work, &owned, where, err);
     if (rc != YVEX_OK) return rc;
