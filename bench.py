@@ -335,9 +335,9 @@ def roofline(result):
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # runs (profiles/), scaled by the same counters on a copy kernel of known size; None where
 # no such run is committed.
-TRAFFIC = {"paged3": 1033354309, "paged4": 1512935981, "decode1": 18116273,
-           "prefill2": 50570411, "mla5": 204069253, "append_bf16": 303974816,
-           "append_q8_0": 239922751}
+TRAFFIC = {"paged3": 1033352906, "paged4": 1512941054, "decode1": 18116274,
+           "prefill2": 50570700, "mla5": 204069246, "append_bf16": 303927100,
+           "append_q8_0": 239929618}
 
 
 def repeat_for(seconds, call):
