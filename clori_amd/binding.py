@@ -188,9 +188,20 @@ MLA_WORKSPACE_FN = C.CFUNCTYPE(C.c_int, C.POINTER(MlaDecodeRequirement), ullP, E
 MLA_EXECUTE_FN = C.CFUNCTYPE(C.c_int, C.c_void_p, C.POINTER(MlaDecodeRequest), FactsP, ErrorP)
 
 
+#: members of struct yvex_backend_transformer_operations in the reference's order
+#: (include/yvex/internal/transformer.h:276-339); only the two attention slots are published
+TRANSFORMER_OPERATION_SLOTS = (
+    "initial", "feature_mean", "final", "attention_workspace_required", "attention_execute",
+    "gated_delta_workspace_required", "gated_delta_execute", "linear_workspace_required",
+    "linear_compile", "linear_execute", "linear_summary", "linear_release", "rotary_half_f32",
+    "split_interleaved_two_f32", "silu_product_bf16", "sigmoid_product_bf16", "add_bf16",
+    "bf16_round", "dense_decoder_execute")
+
+
 class TransformerOperations(C.Structure):
-    _fields_ = [("attention_workspace_required", WORKSPACE_FN),
-                ("attention_execute", EXECUTE_FN)]
+    _fields_ = [(name, {"attention_workspace_required": WORKSPACE_FN,
+                        "attention_execute": EXECUTE_FN}.get(name, C.c_void_p))
+                for name in TRANSFORMER_OPERATION_SLOTS]
 
 
 KV_APPEND_FN = C.CFUNCTYPE(C.c_int, C.c_void_p, C.POINTER(KvAppendRequest), FactsP, ErrorP)
@@ -252,6 +263,7 @@ EXPORTED_SYMBOLS = [
     "yvex_backend_capability_reason_name", "yvex_backend_workspace_attach",
     "yvex_backend_workspace_detach", "yvex_backend_workspace_acquire",
     "yvex_backend_op_attention", "yvex_backend_transformer_operations_get",
+    "yvex_backend_attention_execute", "yvex_backend_attention_complete",
     "yvex_backend_rocm_attention_operations_get", "yvex_backend_rocm_completion_mode_set",
     "yvex_backend_rocm_timing_begin", "yvex_backend_rocm_timing_end",
     "yvex_backend_rocm_kernel_probe_begin", "yvex_backend_rocm_kernel_probe_end",

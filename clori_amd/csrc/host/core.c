@@ -535,6 +535,53 @@ const yvex_backend_rocm_attention_operations *yvex_backend_rocm_attention_operat
                : NULL;
 }
 
+/* The encoded-attention transaction (include/yvex/internal/backend.h:193-198).  The
+ * reference's only implementation is the CUDA one (src/backend/cuda/attention.c:1924);
+ * this backend owns none of the job's projection, compressor or indexer stages, so the
+ * symbol answers the way an unadmitted capability does: argument errors first, then the
+ * lifecycle gate, then a CAPABILITY failure with YVEX_ERR_UNSUPPORTED.  The job is not read
+ * and the output record is not written. */
+int yvex_backend_attention_execute(yvex_backend *backend, const yvex_backend_attention_job *job,
+                                   yvex_backend_attention_output *output,
+                                   yvex_backend_attention_failure *failure, yvex_error *err)
+{
+    static const char where[] = "rocm.attention.encoded";
+    int rc;
+    if (failure) memset(failure, 0, sizeof(*failure));
+    yvex_error_clear(err);
+    if (!backend || !job || !output) {
+        if (failure) {
+            failure->code = YVEX_BACKEND_ATTENTION_FAILURE_INVALID_ARGUMENT;
+            failure->stage = where;
+            failure->expected = 1ull;
+        }
+        return refuse(err, YVEX_ERR_INVALID_ARG, where,
+                      "backend, attention job and output record are required");
+    }
+    rc = backend_dispatch_admit(backend, where, err);
+    if (rc != YVEX_OK) return rc;
+    if (failure) {
+        failure->code = YVEX_BACKEND_ATTENTION_FAILURE_CAPABILITY;
+        failure->stage = where;
+        failure->expected = 1ull;
+    }
+    return refuse(err, YVEX_ERR_UNSUPPORTED, where,
+                  "the encoded attention transaction is not admitted by the ROCm backend");
+}
+
+/* src/backend/cuda/attention_completion.c:110-120: a completion this backend never made
+ * pending has no valid owner. */
+int yvex_backend_attention_complete(yvex_backend *backend,
+                                    yvex_backend_attention_completion *completion,
+                                    int barrier_observed, yvex_error *err)
+{
+    (void)backend;
+    (void)completion;
+    (void)barrier_observed;
+    return refuse(err, YVEX_ERR_INVALID_ARG, "rocm.attention.complete",
+                  "ROCm attention completion owner is invalid");
+}
+
 /* ----------------------------------------------------------- workspace ---- */
 
 /* src/backend/residency.c:207-231 (the kind check admits ROCM here). */

@@ -336,17 +336,118 @@ typedef struct yvex_transformer_attention_request {
     yvex_device_tensor *output;
 } yvex_transformer_attention_request;
 
-/* The attention members of struct yvex_backend_transformer_operations
- * (include/yvex/internal/transformer.h:291-294), same signatures. */
+/* struct yvex_backend_transformer_operations, include/yvex/internal/transformer.h:276-339:
+ * every member of the reference table, in the reference's order and with the reference's
+ * signatures, so that a caller compiled against the reference header finds
+ * attention_workspace_required and attention_execute at the same offsets in the table
+ * this backend returns.  The request/plan types of the slots this backend does not
+ * publish are opaque here (only pointers to them cross the boundary); those slots are
+ * NULL in the ROCm table, which the reference's callers treat as "not published" and
+ * refuse with YVEX_ERR_UNSUPPORTED (src/runtime/stateful_attention.c:294-298). */
+typedef struct yvex_gated_delta_plan yvex_gated_delta_plan;
+typedef struct yvex_gated_delta_device_request yvex_gated_delta_device_request;
+typedef struct yvex_gated_delta_device_result yvex_gated_delta_device_result;
+typedef struct yvex_transformer_linear_compile_request yvex_transformer_linear_compile_request;
+typedef struct yvex_transformer_linear_executable yvex_transformer_linear_executable;
+typedef struct yvex_transformer_linear_executable_summary yvex_transformer_linear_executable_summary;
+typedef struct yvex_transformer_linear_execution_request yvex_transformer_linear_execution_request;
+typedef struct yvex_transformer_dense_decoder_request yvex_transformer_dense_decoder_request;
+typedef struct yvex_transformer_dense_decoder_result yvex_transformer_dense_decoder_result;
 typedef struct yvex_backend_transformer_operations {
+    int (*initial)(yvex_backend *, const yvex_device_tensor *, unsigned int, unsigned long long,
+                   unsigned long long, unsigned long long, yvex_device_tensor *,
+                   yvex_device_tensor *, yvex_backend_operation_facts *, yvex_error *);
+    int (*feature_mean)(yvex_backend *, const yvex_device_tensor *, unsigned long long,
+                        unsigned long long, unsigned long long, yvex_device_tensor *,
+                        yvex_device_tensor *, unsigned long long, unsigned long long,
+                        unsigned long long, float *, yvex_backend_operation_facts *, yvex_error *);
+    int (*final)(yvex_backend *, const yvex_device_tensor *, const yvex_device_tensor *,
+                 const yvex_device_tensor *, const yvex_device_tensor *, const yvex_device_tensor *,
+                 unsigned long long, unsigned long long, unsigned long long, double, double,
+                 yvex_device_tensor *, yvex_device_tensor *, yvex_backend_operation_facts *,
+                 yvex_error *);
     int (*attention_workspace_required)(const yvex_transformer_attention_requirement *,
                                         unsigned long long *, yvex_error *);
     int (*attention_execute)(yvex_backend *, const yvex_transformer_attention_request *,
                              yvex_backend_operation_facts *, yvex_error *);
+    int (*gated_delta_workspace_required)(const yvex_gated_delta_plan *, unsigned long long,
+                                          unsigned long long *, yvex_error *);
+    int (*gated_delta_execute)(yvex_backend *, const yvex_gated_delta_plan *,
+                               const yvex_gated_delta_device_request *,
+                               yvex_gated_delta_device_result *, yvex_backend_operation_facts *,
+                               yvex_error *);
+    int (*linear_workspace_required)(const yvex_transformer_linear_compile_request *,
+                                     unsigned long long *, yvex_error *);
+    int (*linear_compile)(yvex_backend *, const yvex_transformer_linear_compile_request *,
+                          yvex_transformer_linear_executable **,
+                          yvex_transformer_linear_executable_summary *, yvex_error *);
+    int (*linear_execute)(yvex_backend *, const yvex_transformer_linear_execution_request *,
+                          yvex_backend_operation_facts *, yvex_error *);
+    int (*linear_summary)(const yvex_transformer_linear_executable *,
+                          yvex_transformer_linear_executable_summary *, yvex_error *);
+    int (*linear_release)(yvex_backend *, yvex_transformer_linear_executable **, yvex_error *);
+    int (*rotary_half_f32)(yvex_backend *, yvex_device_tensor *, const yvex_device_tensor *,
+                           const yvex_device_tensor *, unsigned long long, unsigned long long,
+                           unsigned long long, unsigned long long, yvex_backend_operation_facts *,
+                           yvex_error *);
+    int (*split_interleaved_two_f32)(yvex_backend *, const yvex_device_tensor *,
+                                     yvex_device_tensor *, yvex_device_tensor *, unsigned long long,
+                                     unsigned long long, unsigned long long,
+                                     yvex_backend_operation_facts *, yvex_error *);
+    int (*silu_product_bf16)(yvex_backend *, const yvex_device_tensor *, const yvex_device_tensor *,
+                             yvex_device_tensor *, unsigned long long,
+                             yvex_backend_operation_facts *, yvex_error *);
+    int (*sigmoid_product_bf16)(yvex_backend *, const yvex_device_tensor *,
+                                const yvex_device_tensor *, yvex_device_tensor *, unsigned long long,
+                                yvex_backend_operation_facts *, yvex_error *);
+    int (*add_bf16)(yvex_backend *, const yvex_device_tensor *, const yvex_device_tensor *,
+                    yvex_device_tensor *, unsigned long long, unsigned long long,
+                    yvex_backend_operation_facts *, yvex_error *);
+    int (*bf16_round)(yvex_backend *, yvex_device_tensor *, unsigned long long,
+                      yvex_backend_operation_facts *, yvex_error *);
+    int (*dense_decoder_execute)(yvex_backend *, const yvex_transformer_dense_decoder_request *,
+                                 yvex_transformer_dense_decoder_result *, yvex_error *);
 } yvex_backend_transformer_operations;
 /* include/yvex/internal/backend.h:211-212; NULL when the kernel bundle is not admitted. */
 const yvex_backend_transformer_operations *yvex_backend_transformer_operations_get(
     const yvex_backend *backend);
+
+/* ---- encoded attention transaction: include/yvex/internal/backend.h:143-198,
+ *      src/backend/cuda/attention.c:1915-1990, attention_completion.c:110-160 ----
+ * The reference's whole-layer DeepSeek attention job (projections, compressor, indexer,
+ * reduce, output) behind one symbol.  This backend owns only the reduce stage
+ * (mla_decode_execute below), so the symbol is exported and fails closed: the failure
+ * record says CAPABILITY at stage "rocm.attention.encoded" and the status is
+ * YVEX_ERR_UNSUPPORTED, the same answer query_capability gives for
+ * YVEX_BACKEND_VARIANT_ATTENTION_ENCODED.  Nothing of the job is read and `output` is left
+ * untouched, so the job and output records stay opaque here. */
+typedef struct yvex_backend_attention_job yvex_backend_attention_job;
+typedef struct yvex_backend_attention_output yvex_backend_attention_output;
+typedef struct yvex_backend_attention_completion yvex_backend_attention_completion;
+typedef enum {
+    YVEX_BACKEND_ATTENTION_FAILURE_NONE = 0,
+    YVEX_BACKEND_ATTENTION_FAILURE_INVALID_ARGUMENT,
+    YVEX_BACKEND_ATTENTION_FAILURE_CAPABILITY,
+    YVEX_BACKEND_ATTENTION_FAILURE_BUDGET,
+    YVEX_BACKEND_ATTENTION_FAILURE_ALLOCATION,
+    YVEX_BACKEND_ATTENTION_FAILURE_COPY,
+    YVEX_BACKEND_ATTENTION_FAILURE_LAUNCH,
+    YVEX_BACKEND_ATTENTION_FAILURE_SYNCHRONIZE,
+    YVEX_BACKEND_ATTENTION_FAILURE_NUMERIC,
+    YVEX_BACKEND_ATTENTION_FAILURE_CANCELLED,
+    YVEX_BACKEND_ATTENTION_FAILURE_CLEANUP
+} yvex_backend_attention_failure_code;
+typedef struct {
+    yvex_backend_attention_failure_code code;
+    const char *stage;
+    unsigned long long expected, actual;
+} yvex_backend_attention_failure;
+int yvex_backend_attention_execute(yvex_backend *backend, const yvex_backend_attention_job *job,
+                                   yvex_backend_attention_output *output,
+                                   yvex_backend_attention_failure *failure, yvex_error *err);
+int yvex_backend_attention_complete(yvex_backend *backend,
+                                    yvex_backend_attention_completion *completion,
+                                    int barrier_observed, yvex_error *err);
 
 /* ======================= NEW SURFACE (no reference counterpart) ============ */
 

@@ -147,6 +147,38 @@ def test_ready_backend_publishes_attention_only():
         assert info.kind == B.KIND_ROCM and info.name == b"fake-gfx950"
 
 
+def test_encoded_attention_transaction_fails_closed():
+    """include/yvex/internal/backend.h:193-198: the symbol exists and refuses; the table the
+    backend returns has the reference's slot order with only the attention slots published."""
+    library = lib()
+
+    class Failure(C.Structure):
+        _fields_ = [("code", C.c_int), ("stage", C.c_char_p), ("expected", C.c_ulonglong),
+                    ("actual", C.c_ulonglong)]
+    library.yvex_backend_attention_execute.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p,
+                                                       C.POINTER(Failure), C.POINTER(B.Error)]
+    library.yvex_backend_attention_complete.argtypes = [C.c_void_p, C.c_void_p, C.c_int,
+                                                        C.POINTER(B.Error)]
+    job, output = C.create_string_buffer(4096), C.create_string_buffer(b"\x5a" * 1024, 1024)
+    with Backend() as b:
+        failure, err = Failure(), B.Error()
+        rc = library.yvex_backend_attention_execute(b.handle, job, output, C.byref(failure),
+                                                    C.byref(err))
+        assert rc == B.YVEX_ERR_UNSUPPORTED and err.code == B.YVEX_ERR_UNSUPPORTED
+        assert failure.code == 2 and failure.stage == b"rocm.attention.encoded"   # CAPABILITY
+        assert output.raw == b"\x5a" * 1024                       # the output record is untouched
+        assert b.query_capability(B.VARIANT_ATTENTION_ENCODED).state == B.CAPABILITY_UNSUPPORTED
+        rc = library.yvex_backend_attention_execute(b.handle, None, output, C.byref(failure),
+                                                    C.byref(err))
+        assert rc == B.YVEX_ERR_INVALID_ARG and failure.code == 1
+        rc = library.yvex_backend_attention_complete(b.handle, job, 0, C.byref(err))
+        assert rc == B.YVEX_ERR_INVALID_ARG
+        ops = b.transformer_operations()
+        for name in B.TRANSFORMER_OPERATION_SLOTS:
+            published = bool(getattr(ops, name))
+            assert published == (name in ("attention_workspace_required", "attention_execute")), name
+
+
 @pytest.mark.parametrize("injected,reason_for_attention", [
     ("module", B.REASON_KERNEL_BUNDLE_REJECTED),
     ("symbol", B.REASON_FUNCTION_MISSING),
