@@ -349,6 +349,17 @@ class Backend:
         _check(rc, err)
         return facts
 
+    def paged_decode_execute_static(self, requirement, query, key_pages, value_pages, page_table,
+                                    context, output, lse=None):
+        """paged_decode_execute through the exported entry point that allocates nothing."""
+        request = B.PagedDecodeRequest(requirement, query.handle, key_pages.handle,
+                                       value_pages.handle, page_table.handle, context.handle,
+                                       output.handle, lse.handle if lse else None)
+        facts, err = B.OperationFacts(), B.Error()
+        _check(lib().yvex_backend_rocm_paged_decode_execute_static(
+            self.handle, C.byref(request), C.byref(facts), C.byref(err)), err)
+        return facts
+
     @staticmethod
     def mla_requirement(batch, heads, key_dim, value_dim, page_tokens, pool_pages, table_stride,
                         max_context, contract=B.NUMERIC_BF16_F32_ACCUMULATE, deterministic=1,

@@ -264,7 +264,8 @@ EXPORTED_SYMBOLS = [
     "yvex_backend_workspace_detach", "yvex_backend_workspace_acquire",
     "yvex_backend_op_attention", "yvex_backend_transformer_operations_get",
     "yvex_backend_attention_execute", "yvex_backend_attention_complete",
-    "yvex_backend_rocm_attention_operations_get", "yvex_backend_rocm_completion_mode_set",
+    "yvex_backend_rocm_attention_operations_get", "yvex_backend_rocm_paged_decode_execute_static",
+    "yvex_backend_rocm_completion_mode_set",
     "yvex_backend_rocm_timing_begin", "yvex_backend_rocm_timing_end",
     "yvex_backend_rocm_kernel_probe_begin", "yvex_backend_rocm_kernel_probe_end",
     "yvex_backend_bandwidth_probe", "yvex_backend_rocm_graph_begin", "yvex_backend_rocm_graph_end",
@@ -334,6 +335,8 @@ def load(path=None):
     lib.yvex_backend_transformer_operations_get.argtypes = [vp]
     lib.yvex_backend_rocm_attention_operations_get.restype = C.POINTER(RocmAttentionOperations)
     lib.yvex_backend_rocm_attention_operations_get.argtypes = [vp]
+    lib.yvex_backend_rocm_paged_decode_execute_static.argtypes = [
+        vp, C.POINTER(PagedDecodeRequest), FactsP, ErrorP]
     lib.yvex_backend_rocm_completion_mode_set.argtypes = [vp, C.c_int, ErrorP]
     lib.yvex_backend_rocm_timing_begin.argtypes = [vp, ErrorP]
     lib.yvex_backend_rocm_timing_end.argtypes = [vp, C.POINTER(C.c_double), ErrorP]

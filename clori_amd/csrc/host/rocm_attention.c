@@ -14,6 +14,10 @@
 #include <string.h>
 
 #include "../kernel_params.h"
+#include "rocm_scratch.h"
+
+_Static_assert(YVEX_ROCM_STATIC_SCRATCH_BYTES == YVEX_ROCM_STATIC_WORKSPACE_BYTES,
+               "the public limit and the device array must have the same size");
 
 enum {
     ROCM_EXACT_HEAD_MAX = 256,   /* src/backend/cuda/exact_attention.c:6 */
@@ -145,6 +149,9 @@ typedef struct {
     unsigned long long pool_pages, table_stride, max_context, fixed_context;
     unsigned long long k_token_stride, v_token_stride;
     float scale;
+    /* when set, the partials live here (nothing is acquired or released) */
+    void *fixed_work;
+    unsigned long long fixed_work_bytes;
 } decode_job;
 
 /* Launches the decode kernel and the finish (merge) kernel and completes the operation. */
@@ -166,8 +173,16 @@ static int decode_run(yvex_backend *backend, const decode_job *job, const char *
                                   &ml_bytes, &total))
         return refuse(err, YVEX_ERR_BOUNDS, where, "decode geometry exceeds admitted integer range");
     backend_workspace_reset(backend);
-    rc = yvex_rocm_temporary_acquire(backend, total, &work, &owned, where, err);
-    if (rc != YVEX_OK) return rc;
+    if (job->fixed_work) {
+        if (total > job->fixed_work_bytes)
+            return refuse(err, YVEX_ERR_BOUNDS, where,
+                          "decode partials exceed the fixed device scratch "
+                          "(YVEX_ROCM_STATIC_WORKSPACE_BYTES)");
+        work = job->fixed_work;
+    } else {
+        rc = yvex_rocm_temporary_acquire(backend, total, &work, &owned, where, err);
+        if (rc != YVEX_OK) return rc;
+    }
     memset(&dp, 0, sizeof(dp));
     dp.q = (const uint16_t *)job->q;
     dp.k_pool = job->k;
@@ -528,7 +543,8 @@ static int rocm_paged_decode_workspace_required(const yvex_rocm_paged_decode_req
 
 static int paged_decode_execute_common(yvex_backend *backend,
                                        const yvex_rocm_paged_decode_request *request,
-                                       const yvex_device_tensor *gate,
+                                       const yvex_device_tensor *gate, void *fixed_work,
+                                       unsigned long long fixed_work_bytes,
                                        yvex_backend_operation_facts *facts, yvex_error *err)
 {
     static const char where[] = "rocm.attention.paged";
@@ -591,6 +607,8 @@ static int paged_decode_execute_common(yvex_backend *backend,
     job.table_stride = r->page_table_stride;
     job.max_context = r->max_context_tokens;
     job.scale = 1.0f / sqrtf((float)r->head_dimension);
+    job.fixed_work = fixed_work;
+    job.fixed_work_bytes = fixed_work_bytes;
     rc = decode_run(backend, &job, where, facts, err);
     if (rc != YVEX_OK) return rc;
     request->output->is_written = 1;
@@ -603,7 +621,32 @@ static int rocm_paged_decode_execute(yvex_backend *backend,
                                      const yvex_rocm_paged_decode_request *request,
                                      yvex_backend_operation_facts *facts, yvex_error *err)
 {
-    return paged_decode_execute_common(backend, request, NULL, facts, err);
+    return paged_decode_execute_common(backend, request, NULL, NULL, 0ull, facts, err);
+}
+
+/* paged_decode_execute for callers that cannot allocate: the split-K partials go to the
+ * fixed device array of rocm_scratch.hip, whose address was taken when the backend was
+ * opened.  No allocation or release call is made on this path, whether or not a workspace
+ * is attached. */
+int yvex_backend_rocm_paged_decode_execute_static(yvex_backend *backend,
+                                                  const yvex_rocm_paged_decode_request *request,
+                                                  yvex_backend_operation_facts *facts,
+                                                  yvex_error *err)
+{
+    static const char where[] = "rocm.attention.paged.static";
+    yvex_rocm_backend_state *state = yvex_rocm_state(backend);
+    if (!state)
+        return refuse(err, YVEX_ERR_INVALID_ARG, where, "a ROCm backend is required");
+    if (state->kernel_bundle_state != YVEX_ROCM_KERNEL_BUNDLE_ADMITTED)
+        return refuse(err, YVEX_ERR_UNSUPPORTED, where, "no kernel bundle is admitted");
+    if (!state->static_scratch) {
+        yvex_error_setf(err, YVEX_ERR_UNSUPPORTED, where,
+                        "the fixed device scratch is unavailable on this device (HIP error %d)",
+                        state->static_scratch_error);
+        return YVEX_ERR_UNSUPPORTED;
+    }
+    return paged_decode_execute_common(backend, request, NULL, state->static_scratch,
+                                       YVEX_ROCM_STATIC_SCRATCH_BYTES, facts, err);
 }
 
 static int rocm_paged_decode_execute_fused(yvex_backend *backend,
@@ -614,7 +657,8 @@ static int rocm_paged_decode_execute_fused(yvex_backend *backend,
     if (!epilogue || !epilogue->output_gate)
         return refuse(err, YVEX_ERR_INVALID_ARG, "rocm.attention.paged",
                       "an epilogue with an output gate tensor is required");
-    return paged_decode_execute_common(backend, request, epilogue->output_gate, facts, err);
+    return paged_decode_execute_common(backend, request, epilogue->output_gate, NULL, 0ull, facts,
+                                       err);
 }
 
 /* --------------------------------------------------------- MLA decode ---- */

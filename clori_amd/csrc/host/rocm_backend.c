@@ -9,6 +9,7 @@
 #include <string.h>
 
 #include "../kernel_params.h"
+#include "rocm_scratch.h"
 
 static void probe_release(yvex_rocm_backend_state *state);
 
@@ -550,6 +551,11 @@ int yvex_backend_open_rocm_impl(yvex_backend **out, const char *device,
         if (err) *err = keep;
         return rc;
     }
+
+    /* the fixed scratch of the entry point that allocates nothing: resolved here, once per
+     * device, with the device current; its absence only disables that entry point */
+    (void)yvex_rocm_static_scratch_resolve(state->device_index, &state->static_scratch,
+                                           &state->static_scratch_error);
 
     backend->device_info.kind = YVEX_BACKEND_KIND_ROCM;
     backend->device_info.device_index = state->device_index;

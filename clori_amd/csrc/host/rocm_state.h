@@ -63,6 +63,8 @@ typedef struct yvex_rocm_backend_state {
     int recording;                  /* a launch sequence is being recorded on the stream */
     unsigned long long live_graphs; /* recorded sequences not yet released */
     unsigned long long recorded_launches; /* kernel launches of the sequence being recorded */
+    void *static_scratch;     /* device address of the fixed scratch array on this device, or NULL */
+    int static_scratch_error; /* the runtime's code when it could not be resolved */
     int bandwidth_ready; /* the probe ran: later calls return the kept evidence */
     yvex_backend_bandwidth_evidence bandwidth_evidence;
 } yvex_rocm_backend_state;

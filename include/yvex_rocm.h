@@ -594,6 +594,24 @@ const yvex_backend_rocm_attention_operations *yvex_backend_rocm_attention_operat
     const yvex_backend *backend);
 
 /*
+ * paged_decode_execute for callers that cannot allocate.  It has no counterpart in the
+ * reference; it is for code that runs where hipMalloc is not allowed: under stream capture,
+ * in tight serving loops, in harnesses that forbid allocation.  Same request, same kernels
+ * and bit-identical results as paged_decode_execute, but the split-K partials go to a fixed
+ * device array of YVEX_ROCM_STATIC_WORKSPACE_BYTES that each GPU holds from the moment the
+ * library is loaded until the process ends; an attached workspace is ignored and no
+ * allocation or release call is made.  A request whose partials need more
+ * (paged_decode_workspace_required tells) is refused with YVEX_ERR_BOUNDS.  Every call on a
+ * GPU shares that GPU's array: calls that overlap on one GPU race (one backend stream
+ * serialises its own calls; two backends on one device must not use it at the same time).
+ */
+#define YVEX_ROCM_STATIC_WORKSPACE_BYTES (16ull << 20)
+int yvex_backend_rocm_paged_decode_execute_static(yvex_backend *backend,
+                                                  const yvex_rocm_paged_decode_request *request,
+                                                  yvex_backend_operation_facts *facts,
+                                                  yvex_error *err);
+
+/*
  * Completion mode.  IMMEDIATE (default) is the reference's behaviour: every operation
  * synchronises once and reads the device status word before returning
  * (src/backend/cuda/transformer.c:655-673).  DEFERRED enqueues only; the status word is
