@@ -99,13 +99,10 @@ int yvex_rocm_op_attention(yvex_backend *backend, const yvex_device_tensor *quer
 static unsigned int decode_wave_count(unsigned long long sessions, unsigned long long kv_heads,
                                       unsigned long long max_context)
 {
-    const char *forced = getenv("YVEX_ROCM_DECODE_WAVES");
     unsigned long long tiles = sessions * kv_heads *
                                ((max_context + ROCM_PAGE_TOKENS - 1ull) / ROCM_PAGE_TOKENS);
     unsigned long long waves = (tiles + ROCM_DECODE_MIN_TILES - 1ull) / ROCM_DECODE_MIN_TILES;
-    unsigned long long cap = forced && atoi(forced) > 0 ? (unsigned long long)atoi(forced)
-                                                        : ROCM_DECODE_WAVES;
-    if (waves > cap) waves = cap;
+    if (waves > ROCM_DECODE_WAVES) waves = ROCM_DECODE_WAVES;
     return (unsigned int)(waves ? waves : 1ull);
 }
 
@@ -717,10 +714,8 @@ static unsigned int mla_chunk_tokens(const yvex_rocm_mla_decode_requirement *r)
 static unsigned int mla_chunk_for(const yvex_rocm_mla_decode_requirement *r,
                                   unsigned long long tokens, int windowed)
 {
-    const char *forced = getenv("YVEX_ROCM_MLA_CHUNK");
     unsigned long long per_batch = 256ull / r->batch ? 256ull / r->batch : 1ull;
     unsigned long long chunk = (tokens + per_batch - 1ull) / per_batch;
-    if (forced && atoi(forced) >= ROCM_MLA_PAGE_TOKENS) chunk = (unsigned long long)atoi(forced);
     chunk = align_up(chunk, ROCM_MLA_PAGE_TOKENS);
     /* a windowed chunk may start in the middle of a page and so touch one page more */
     if (chunk > (unsigned long long)(YVEX_ROCM_MLA_MAX_CHUNK_PAGES - (windowed ? 1 : 0)) *

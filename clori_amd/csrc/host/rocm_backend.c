@@ -275,7 +275,7 @@ static int rocm_bandwidth_probe(yvex_backend *backend, yvex_backend_bandwidth_ev
     yvex_backend_bandwidth_evidence evidence;
     yvex_backend_tensor_desc descriptor;
     yvex_device_tensor *source = NULL, *copy = NULL, *sink = NULL;
-    const char *forced = getenv("YVEX_ROCM_BANDWIDTH_BYTES");
+    const char *forced = getenv("YVEX_TEST_ROCM_BANDWIDTH_BYTES");
     unsigned long long scratch;
     yvex_error cleanup;
     unsigned int sample;

@@ -58,6 +58,10 @@ static const rocm_kernel_binding rocm_kernel_bindings[] = {
 
 unsigned int yvex_rocm_bundle_image_count(void) { return yvex_rocm_bundle_image_total; }
 
+/* Failure injection for the host tests, named and read the way the reference's CUDA arm does
+ * it (getenv("YVEX_TEST_CUDA_ATTENTION_FAILURE"), src/backend/cuda/ops.c:88-200;
+ * YVEX_TEST_CUDA_*_FAILURE, src/backend/cuda/residency.c:57-240): only variables with the
+ * YVEX_TEST_ROCM_ prefix are ever read, and none of them changes launch geometry. */
 static int test_failure_matches(const char *name, yvex_backend_operation_variant variant)
 {
     const char *value = getenv(name);

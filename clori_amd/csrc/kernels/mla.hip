@@ -53,21 +53,6 @@ __device__ inline void flag(int32_t *status, int code) { atomicCAS(status, 0, co
 
 __device__ inline int swizzle(int r) { return (((r >> 1) & 1) << 2) | ((r >> 2) & 3); }
 
-#ifdef MLA_PROBE_CLOCK
-// timing probe: phase cycle counts of wave 0 of workgroup (0, 0), summed over its tiles
-__device__ unsigned long long yvex_mla_clock[8];
-#define MLA_STAMP(slot)                                                        \
-    do {                                                                       \
-        __builtin_amdgcn_sched_barrier(0);                                     \
-        const unsigned long long now_ = __builtin_readcyclecounter();          \
-        clock_acc[slot] += now_ - clock_prev;                                  \
-        clock_prev = now_;                                                     \
-        __builtin_amdgcn_sched_barrier(0);                                     \
-    } while (0)
-#else
-#define MLA_STAMP(slot) do { } while (0)
-#endif
-
 }  // namespace
 
 // grid = (chunks, batch), block 256 (heads must be 128, pages a multiple of 32 tokens),
@@ -243,17 +228,12 @@ yvex_rocm_mla_decode_bf16(const yvex_rocm_mla_params p)
         }
     };
 
-#ifdef MLA_PROBE_CLOCK
-    unsigned long long clock_acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-    unsigned long long clock_prev = __builtin_readcyclecounter();
-#endif
     // Software pipeline over tiles: step t computes the scores of tile t (with the loads
     // of tile t+2 spread behind its MFMAs), settles the maximum, then issues the O^T update
     // with tile t-1 and, behind its MFMAs, the exponentials of tile t.  Tiles t-1 and t
     // are being read during a step, tiles t+1 and t+2 are in flight.
     stage_tile(0u);
     stage_tile(1u);
-    MLA_STAMP(0);
     uint32_t pk_prev[8], pk_cur[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) pk_prev[j] = 0u;
@@ -278,13 +258,10 @@ yvex_rocm_mla_decode_bf16(const yvex_rocm_mla_params p)
     auto step = [&](uint32_t t, auto with_update) {
         // tile t has landed when at most one younger tile is outstanding: vmcnt(9)
         __builtin_amdgcn_s_waitcnt(0x0f79);
-        MLA_STAMP(1);
         __syncthreads();
-        MLA_STAMP(2);
         uint32_t stage_dst;
         i32x4 stage_rsrc;
         stage_target(t + 2u, stage_dst, stage_rsrc);
-        MLA_STAMP(3);
         const unsigned char *tile = lds + (t % kBuffers) * kTileBytes;
         const unsigned char *prev_tile = lds + ((t + kBuffers - 1u) % kBuffers) * kTileBytes;
 
@@ -293,9 +270,7 @@ yvex_rocm_mla_decode_bf16(const yvex_rocm_mla_params p)
         score(tile, s, [&](int kk) {
             if ((kk & 3) == 1) lds_dma_b128(stage_dst + (kk >> 2) * 1024, stage_rsrc, stage_off[kk >> 2], 0u);
         });
-        MLA_STAMP(4);
         settle(t0 + t * kTile, s, pk_prev);
-        MLA_STAMP(5);
 
         // ---- O^T update with tile t-1 (none in the first step) and the exponentials of
         //      tile t behind its MFMAs -------------------------------------------------------
@@ -330,14 +305,9 @@ yvex_rocm_mla_decode_bf16(const yvex_rocm_mla_params p)
         }
 #pragma unroll
         for (int j = 0; j < 8; ++j) pk_prev[j] = pk_cur[j];
-        MLA_STAMP(6);
     };
     step(0u, std::integral_constant<bool, false>());
-#ifdef MLA_PROBE_TILES
-    for (uint32_t t = 1; t < MLA_PROBE_TILES; ++t)
-#else
     for (uint32_t t = 1; t < tiles; ++t)
-#endif
         step(t, std::integral_constant<bool, true>());
     // the update with the last tile
     __builtin_amdgcn_sched_barrier(0);
@@ -352,13 +322,6 @@ yvex_rocm_mla_decode_bf16(const yvex_rocm_mla_params p)
     // drain the loads that were issued past the last tile before the workgroup ends
     __builtin_amdgcn_s_waitcnt(0x0f70);
 
-#ifdef MLA_PROBE_SKIP_STORE
-    if (l_run != 12345.0f) return;
-#endif
-#ifdef MLA_PROBE_CLOCK
-    if (blockIdx.x == 0 && blockIdx.y == 0 && tid == 0)
-        for (int i = 0; i < 8; ++i) yvex_mla_clock[i] = clock_acc[i];
-#endif
     float l = l_run;
     l += xor_lanes(l, 32);
     const uint64_t slot = ((uint64_t)batch * p.slot_stride + p.first_slot + chunk) * p.heads + head;

@@ -54,21 +54,6 @@ __device__ inline int swizzle(int r) { return ((r & 3) << 2) | ((r >> 2) & 3); }
 
 __device__ inline void flag(int32_t *status, int code) { atomicCAS(status, 0, code); }
 
-#ifdef PREFILL_PROBE_CLOCK
-// timing probe: phase cycle counts of wave 0 of workgroup 0, summed over its tiles
-__device__ unsigned long long yvex_prefill_clock[8];
-#define PREFILL_STAMP(slot)                                                    \
-    do {                                                                       \
-        __builtin_amdgcn_sched_barrier(0);                                     \
-        const unsigned long long now_ = __builtin_readcyclecounter();          \
-        clock_acc[slot] += now_ - clock_prev;                                  \
-        clock_prev = now_;                                                     \
-        __builtin_amdgcn_sched_barrier(0);                                     \
-    } while (0)
-#else
-#define PREFILL_STAMP(slot) do { } while (0)
-#endif
-
 template <int NB>
 __device__ inline void prefill_body(const yvex_rocm_prefill_params &p, unsigned char *lds)
 {
@@ -175,17 +160,11 @@ __device__ inline void prefill_body(const yvex_rocm_prefill_params &p, unsigned 
     const uint32_t wave_last_vis =
         p.causal ? p.query_start + min(row0 + kRowsPerWave, p.query_tokens) - 1u : p.kv_tokens - 1u;
 
-#ifdef PREFILL_PROBE_CLOCK
-    unsigned long long clock_acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-    unsigned long long clock_prev = __builtin_readcyclecounter();
-#endif
     stage_tile(0u, 0);
     for (uint32_t t = 0; t < tiles; ++t) {
         const int buf = (int)(t & 1u);
         __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's part of tile t is in LDS
-        PREFILL_STAMP(0);
         __syncthreads();
-        PREFILL_STAMP(1);
         const uint32_t key0 = t * kKeyTile;
         const bool more = t + 1u < tiles;
         // a wave whose every row sees nothing of this tile skips the products
@@ -193,7 +172,6 @@ __device__ inline void prefill_body(const yvex_rocm_prefill_params &p, unsigned 
             if (more) stage_tile(t + 1u, buf ^ 1);
             continue;
         }
-        PREFILL_STAMP(2);
         const unsigned char *tile = lds + buf * kBufBytes;
 
         // ---- S^T = K . Q^T -------------------------------------------------
@@ -228,7 +206,6 @@ __device__ inline void prefill_body(const yvex_rocm_prefill_params &p, unsigned 
             }
         }
 
-        PREFILL_STAMP(3);
         // ---- mask, online softmax (per lane = per query row) ----------------------
         // scores stay raw; the softmax scale is folded into the exponent's multiply-add
         const bool need_mask = (key0 + kKeyTile - 1u > wave_first_vis) ||
@@ -278,7 +255,6 @@ __device__ inline void prefill_body(const yvex_rocm_prefill_params &p, unsigned 
             l_run[nb] += lsum;
         }
 
-        PREFILL_STAMP(4);
         // ---- O^T += V^T . P^T -------------------------------------------------
 #pragma unroll
         for (int mb = 0; mb < 2; ++mb)
@@ -305,13 +281,8 @@ __device__ inline void prefill_body(const yvex_rocm_prefill_params &p, unsigned 
                     for (int nb = 0; nb < NB; ++nb) o[db][nb] = mfma_32x32x16(a, pb[nb], o[db][nb]);
                 }
             }
-        PREFILL_STAMP(5);
     }
 
-#ifdef PREFILL_PROBE_CLOCK
-    if (blockIdx.x == 0 && tid == 0)
-        for (int i = 0; i < 8; ++i) yvex_prefill_clock[i] = clock_acc[i];
-#endif
     // ---- epilogue: normalise, publish bf16 rows and LSE -------------------------
     if (!wave_active) return;
 #pragma unroll

@@ -612,7 +612,7 @@ def test_recorded_sequence_rules(fake_runtime):
 def test_bandwidth_probe_record(env, fake_runtime):
     """Five samples of eight passes each for the read and for the copy, medians published,
     the working set released, the first evidence kept."""
-    env("YVEX_ROCM_BANDWIDTH_BYTES", str(1 << 20))
+    env("YVEX_TEST_ROCM_BANDWIDTH_BYTES", str(1 << 20))
     with Backend() as b:
         live, launches = fake_runtime.fake_hip_live_allocations(), fake_runtime.fake_hip_launches()
         e = b.bandwidth_probe()
