@@ -25,7 +25,7 @@ enum {
     ROCM_PAGE_TOKENS = 16,
     ROCM_GROUP_MAX = 16,
     ROCM_DECODE_WAVES = 2048,
-    ROCM_DECODE_MIN_TILES = 4,
+    ROCM_DECODE_MIN_TILES = 8, /* 8 and 16 measure alike on a 4096-token context; 4 and 32 are a third slower */
     ROCM_PREFILL_ROWS = YVEX_ROCM_PREFILL_ROWS, /* query rows per prefill workgroup */
     ROCM_WORK_ALIGNMENT = 256    /* src/backend/cuda/transformer.c:17 */
 };
@@ -122,7 +122,12 @@ static int decode_workspace_bytes(unsigned long long slots, unsigned long long h
     return 1;
 }
 
-/* Balanced decode: two slots per wave plus the per-session offset table. */
+/* A launch that fills the device merges its split segments with a second kernel; a smaller
+ * one is bound by launch latency and merges inside the decode kernel (arrival counters). */
+static int decode_merges_in_kernel(unsigned int waves) { return waves < ROCM_DECODE_WAVES; }
+
+/* Balanced decode: two partial slots per wave, then (two-kernel form) the per-session offset
+ * table. */
 static int balanced_workspace_bytes(unsigned long long waves, unsigned long long group,
                                     unsigned long long head_dim, unsigned long long sessions,
                                     unsigned long long *acc_bytes, unsigned long long *ml_bytes,
@@ -130,13 +135,14 @@ static int balanced_workspace_bytes(unsigned long long waves, unsigned long long
 {
     unsigned long long parts = 0ull, offsets;
     if (!decode_workspace_bytes(2ull * waves, group, head_dim, sizeof(float), acc_bytes, &parts)) return 0;
-    offsets = align_up((sessions + 1ull) * sizeof(uint32_t), ROCM_WORK_ALIGNMENT);
+    offsets = decode_merges_in_kernel((unsigned int)waves)
+                  ? 0ull : align_up((sessions + 1ull) * sizeof(uint32_t), ROCM_WORK_ALIGNMENT);
     *ml_bytes = parts - *acc_bytes;
     return yvex_core_u64_add(parts, offsets, total);
 }
 
 typedef struct {
-    yvex_rocm_function_id function;
+    yvex_rocm_function_id function, merged_function; /* two-launch form, one-launch form */
     yvex_backend_operation_variant variant;
     const void *q, *k, *v;
     const int32_t *page_table, *context;
@@ -151,7 +157,8 @@ typedef struct {
     unsigned long long fixed_work_bytes;
 } decode_job;
 
-/* Launches the decode kernel and the finish (merge) kernel and completes the operation. */
+/* Launches the decode kernel, the finish (merge) kernel when the launch fills the device, and
+ * completes the operation. */
 static int decode_run(yvex_backend *backend, const decode_job *job, const char *where,
                       yvex_backend_operation_facts *facts, yvex_error *err)
 {
@@ -160,12 +167,14 @@ static int decode_run(yvex_backend *backend, const decode_job *job, const char *
     unsigned long long acc_bytes = 0ull, ml_bytes = 0ull, total = 0ull, items;
     const unsigned long long group = job->query_heads / job->kv_heads;
     const unsigned int waves = decode_wave_count(job->sessions, job->kv_heads, job->max_context);
+    const int in_kernel = decode_merges_in_kernel(waves);
     void *work = NULL;
     yvex_error cleanup;
     int owned = 0, rc, cleanup_rc;
     if (!yvex_core_u64_mul(job->sessions * job->kv_heads,
                            (job->max_context + ROCM_PAGE_TOKENS - 1ull) / ROCM_PAGE_TOKENS, &items) ||
         items > 0x7fffffffull || job->sessions > 65535ull || job->query_heads > 65535ull ||
+        (in_kernel && job->sessions * job->kv_heads > YVEX_ROCM_DECODE_SEGMENTS_MAX) ||
         !balanced_workspace_bytes(waves, group, job->head_dim, job->sessions, &acc_bytes,
                                   &ml_bytes, &total))
         return refuse(err, YVEX_ERR_BOUNDS, where, "decode geometry exceeds admitted integer range");
@@ -191,7 +200,8 @@ static int decode_run(yvex_backend *backend, const decode_job *job, const char *
     dp.gate = (const uint16_t *)job->gate;
     dp.part_acc = (float *)work;
     dp.part_ml = (float *)((unsigned char *)work + acc_bytes);
-    dp.offsets = (uint32_t *)((unsigned char *)work + acc_bytes + ml_bytes);
+    dp.arrivals = in_kernel ? state->decode_arrivals : NULL;
+    dp.offsets = in_kernel ? NULL : (uint32_t *)((unsigned char *)work + acc_bytes + ml_bytes);
     dp.status = state->device_status;
     dp.k_token_stride = job->k_token_stride;
     dp.v_token_stride = job->v_token_stride;
@@ -205,19 +215,25 @@ static int decode_run(yvex_backend *backend, const decode_job *job, const char *
     dp.fixed_context = (uint32_t)job->fixed_context;
     dp.waves = waves;
     dp.scale_log2 = job->scale * 1.4426950408889634f;
-    rc = yvex_rocm_launch(backend, job->function, job->variant, waves, 1u, 1u, 64u, 0u, &dp, where,
-                          err);
-    if (rc == YVEX_OK)
+    rc = yvex_rocm_launch(backend, in_kernel ? job->merged_function : job->function, job->variant,
+                          waves, 1u, 1u, 64u, 0u, &dp, where, err);
+    if (rc == YVEX_OK && !in_kernel)
         rc = yvex_rocm_launch(backend, YVEX_ROCM_FN_DECODE_FINISH, job->variant,
                               (unsigned int)job->query_heads, (unsigned int)job->sessions, 1u,
                               (unsigned int)job->head_dim, 0u, &dp, where, err);
     if (rc == YVEX_OK) {
-        facts->kernel_launches = 2ull;
+        facts->kernel_launches = in_kernel ? 1ull : 2ull;
         facts->accelerated_matrix_launches = 1ull;
         facts->temporary_bytes = total;
         facts->compulsory_memory_facts_available = 1;
         rc = yvex_rocm_complete(backend, job->variant, where, facts, err);
     }
+    /* a launch that did not run to a clean end may leave arrival counts behind */
+    if (rc != YVEX_OK && in_kernel && !state->recording &&
+        backend->status != YVEX_BACKEND_STATUS_FAILED)
+        (void)state->driver.hipMemsetAsync(state->decode_arrivals, 0,
+                                           YVEX_ROCM_DECODE_SEGMENTS_MAX * sizeof(uint32_t),
+                                           state->stream);
     yvex_error_clear(&cleanup);
     cleanup_rc = yvex_rocm_temporary_release(backend, work, total, owned, &cleanup);
     backend_workspace_reset(backend);
@@ -398,6 +414,7 @@ static int attention_execute_common(yvex_backend *backend,
         decode_job job;
         memset(&job, 0, sizeof(job));
         job.function = YVEX_ROCM_FN_DECODE_ROWS_BF16;
+        job.merged_function = YVEX_ROCM_FN_DECODE_ROWS_BF16_MERGED;
         job.variant = YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_BF16;
         job.q = request->query->data;
         job.k = request->key->data;
@@ -583,9 +600,11 @@ static int paged_decode_execute_common(yvex_backend *backend,
     memset(&job, 0, sizeof(job));
     if (r->kv_storage == YVEX_ROCM_KV_BF16) {
         job.function = YVEX_ROCM_FN_DECODE_PAGED_BF16;
+        job.merged_function = YVEX_ROCM_FN_DECODE_PAGED_BF16_MERGED;
         job.variant = YVEX_BACKEND_VARIANT_ROCM_ATTENTION_PAGED_BF16;
     } else {
         job.function = YVEX_ROCM_FN_DECODE_PAGED_Q8_0;
+        job.merged_function = YVEX_ROCM_FN_DECODE_PAGED_Q8_0_MERGED;
         job.variant = YVEX_BACKEND_VARIANT_ROCM_ATTENTION_PAGED_Q8_0;
     }
     job.q = request->query->data;

@@ -436,6 +436,7 @@ static int rocm_close(yvex_backend *backend, yvex_error *err)
     rc = yvex_rocm_kernel_bundle_close(backend, err);
     if (rc != YVEX_OK) return rc; /* impl retained: checked close can be retried */
     if (state->device_status) (void)state->driver.hipFree(state->device_status);
+    if (state->decode_arrivals) (void)state->driver.hipFree(state->decode_arrivals);
     probe_release(state);
     if (state->timing_start) (void)state->driver.hipEventDestroy(state->timing_start);
     if (state->timing_stop) (void)state->driver.hipEventDestroy(state->timing_stop);
@@ -536,12 +537,24 @@ int yvex_backend_open_rocm_impl(yvex_backend **out, const char *device,
                                                            state->stream),
                               where, err);
     if (rc == YVEX_OK)
+        rc = yvex_rocm_status(&state->driver,
+                              state->driver.hipMalloc((void **)&state->decode_arrivals,
+                                                      YVEX_ROCM_DECODE_SEGMENTS_MAX * sizeof(uint32_t)),
+                              where, err);
+    if (rc == YVEX_OK)
+        rc = yvex_rocm_status(&state->driver,
+                              state->driver.hipMemsetAsync(state->decode_arrivals, 0,
+                                                           YVEX_ROCM_DECODE_SEGMENTS_MAX * sizeof(uint32_t),
+                                                           state->stream),
+                              where, err);
+    if (rc == YVEX_OK)
         rc = yvex_rocm_status(&state->driver, state->driver.hipStreamSynchronize(state->stream),
                               where, err);
     if (rc != YVEX_OK) {
         yvex_error keep = err ? *err : (yvex_error){0};
         yvex_error scratch;
         if (state->device_status) (void)state->driver.hipFree(state->device_status);
+        if (state->decode_arrivals) (void)state->driver.hipFree(state->decode_arrivals);
         if (state->timing_start) (void)state->driver.hipEventDestroy(state->timing_start);
         if (state->timing_stop) (void)state->driver.hipEventDestroy(state->timing_stop);
         if (state->stream) (void)state->driver.hipStreamDestroy(state->stream);

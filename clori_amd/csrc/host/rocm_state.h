@@ -18,6 +18,9 @@ typedef enum {
     YVEX_ROCM_FN_DECODE_MERGE,
     YVEX_ROCM_FN_DECODE_FINISH,
     YVEX_ROCM_FN_DECODE_PAGED_Q8_0,
+    YVEX_ROCM_FN_DECODE_PAGED_BF16_MERGED,
+    YVEX_ROCM_FN_DECODE_PAGED_Q8_0_MERGED,
+    YVEX_ROCM_FN_DECODE_ROWS_BF16_MERGED,
     YVEX_ROCM_FN_PREFILL_BF16,
     YVEX_ROCM_FN_MLA_DECODE_BF16,
     YVEX_ROCM_FN_KV_APPEND_BF16,
@@ -28,6 +31,8 @@ typedef enum {
 } yvex_rocm_function_id;
 
 #define YVEX_ROCM_PROBE_MAX 256u
+/* (session, kv head) segments one split-K decode launch may have: one arrival counter each */
+#define YVEX_ROCM_DECODE_SEGMENTS_MAX (1u << 18)
 
 typedef enum {
     YVEX_ROCM_KERNEL_BUNDLE_ABSENT = 0,
@@ -57,6 +62,7 @@ typedef struct yvex_rocm_backend_state {
     yvex_backend_capability_reason variant_failures[YVEX_BACKEND_VARIANT_ROCM_END];
     yvex_backend_capability_reason backend_failure_reason;
     int32_t *device_status; /* one status word, zero between operations */
+    uint32_t *decode_arrivals; /* YVEX_ROCM_DECODE_SEGMENTS_MAX counters, zero between operations */
     int status_dirty;       /* deferred mode: launches since the last check */
     yvex_rocm_completion_mode completion_mode;
     unsigned long long live_tensors;

@@ -55,11 +55,14 @@ typedef struct {
 /* Split-K decode over a balanced partition.  The (session, kv head, 16-token tile) work
  * of the whole batch is laid out as one sequence and cut into gridDim.x equal ranges,
  * one wave each.  A wave that covers a whole (session, kv head) segment publishes the
- * final rows itself; otherwise it leaves a partial in one of its two slots and the
- * finish kernel merges the parts in wave order.
+ * final rows itself; otherwise it leaves a partial in one of its two slots, adds one to the
+ * segment's arrival counter, and the wave that completes the count merges the parts in
+ * wave order and publishes.
  * part_acc is [2*waves][group][head_dim] F32 (unnormalised), part_ml is
- * [2*waves][group][2] F32 = (running max in log2 units, sum); offsets is
- * [sessions + 1] U32: exclusive prefix of work items per session, then the total. */
+ * [2*waves][group][2] F32 = (running max in log2 units, sum); arrivals is
+ * [sessions][kv_heads] U32, zero before the launch and zero again after it, or NULL: then
+ * wave 0 writes offsets ([sessions + 1] U32: exclusive prefix of work items per session, then
+ * the total) and yvex_rocm_decode_finish merges in a second launch. */
 typedef struct {
     const uint16_t *q;
     const void *k_pool, *v_pool;
@@ -68,6 +71,7 @@ typedef struct {
     uint16_t *out;             /* bf16 [sessions][query_heads][head_dim] */
     float *lse;                /* optional F32 [sessions][query_heads] */
     float *part_acc, *part_ml;
+    uint32_t *arrivals;
     uint32_t *offsets;
     int32_t *status;
     uint64_t k_token_stride, v_token_stride; /* token-major layout: elements per token */

@@ -17,8 +17,9 @@
 //     V block  uint16 [128 lanes][16 tokens]                   elem(t,c) = c*16 + t
 // Token-major layout (the reference's [token][kv head][dim] history rows, with a
 // per-token stride so the interleaved [K|V] rows of
-// src/runtime/stateful_attention.c:326-352 are addressable): K rows are read in 16-byte
-// pieces, V is gathered transposed.
+// src/runtime/stateful_attention.c:326-352 are addressable): K and V rows are both read in
+// 16-byte pieces; the V tile (16 tokens x 128 dims) is turned into the V^T operand through
+// 4 KB of LDS private to the wave (ds_write_b128 of swizzled rows, ds_read_b64_tr_b16 back).
 //
 // Q8_0 paged layout, per (page, kv head): the canonical GGUF blocks (32 int8 codes and
 // one f16 scale along the head dimension) are kept byte for byte but stored as
@@ -33,11 +34,23 @@
 // Work distribution: the (session, kv head, tile) items of the whole batch form one
 // sequence that is cut into gridDim.x equal ranges, so every wave streams the same
 // number of tiles whatever the mix of context lengths.  A wave that covers a whole
-// (session, kv head) segment publishes its rows directly; a split segment leaves
-// partials (running max in log2 units, sum, unnormalised accumulator) in the workspace
-// and yvex_rocm_decode_finish merges them in wave order with a log-sum-exp merge (a
-// second launch instead of in-kernel signalling: a device-scope release fence per wave
-// costs far more on an 8-XCD part than one more launch).
+// (session, kv head) segment publishes its rows directly.  The waves of a split segment
+// leave partials (running max in log2 units, sum, unnormalised accumulator) in the
+// workspace.  Two ways to merge them, chosen by the host from the launch size:
+//   * launches that do not fill the device are bound by launch latency, so the merge
+//     happens in this kernel: each wave counts itself in on a per-segment arrival counter
+//     and the wave that arrives last merges all partials of the segment in wave order (the
+//     result does not depend on who was last) and publishes.  One launch.
+//   * full-size launches use yvex_rocm_decode_finish as a second launch: with every SIMD
+//     streaming, the device-scope stores, the counter and the merge's load trips at the end
+//     of each wave cost more (measured +6..11 us on 190..275 us) than one more launch.
+//   Visibility across the eight XCDs without a cache write-back per wave: the partials are
+// written with device-scope write-through stores (sc1), the wave waits for them to complete
+// (s_waitcnt vmcnt(0)) and only then adds to the counter with a device-scope atomic; the
+// merging wave, after seeing the full count, reads them with device-scope loads (sc1), not
+// through an L2 invalidate, which stalls the waves of the XCD that are still streaming.  The
+// counters live in backend-owned memory that is zero between launches: the last arriver
+// puts its counter back to zero.
 // yvex_rocm_decode_merge is the stand-alone merge used by the per-chunk MLA path.
 #include "mfma.h"
 
@@ -50,6 +63,26 @@ constexpr int kPageTokens = 16;
 
 
 __device__ inline void flag(int32_t *status, int code) { atomicCAS(status, 0, code); }
+
+// 16 / 8 bytes to global memory, visible device-wide once the store has completed: the
+// write-through form (sc1) the memory model uses for device-scope atomic stores on this
+// multi-XCD part.  Plain stores would sit in the XCD's L2 until a write-back.
+__device__ inline void store_b128_device(void *p, floatx4 v)
+{
+    asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(p), "v"(v) : "memory");
+}
+__device__ inline void store_b64_device(void *p, float a, float b)
+{
+    typedef float floatx2 __attribute__((ext_vector_type(2)));
+    const floatx2 v = {a, b};
+    asm volatile("global_store_dwordx2 %0, %1, off sc1" : : "v"(p), "v"(v) : "memory");
+}
+
+typedef __attribute__((address_space(3))) short4v lds_short4;
+// LDS staging of a token-major V tile: row r (256 bytes) keeps its 16-byte chunk c at
+// position c ^ (r & 14), which spreads the 16 rows a transposed read touches over all banks
+// (each 32-byte column segment is hit by exactly two rows).
+__device__ inline uint32_t vt_offset(int row, int chunk) { return (uint32_t)(row * 256 + ((chunk ^ (row & 14)) << 4)); }
 
 struct State {
     floatx4 o[8];  // O^T[dim 16*b + 4*(lane/16) + i][head lane%16]
@@ -81,7 +114,8 @@ __device__ inline void softmax_step(State &st, const float (&x)[4], float (&p)[4
 // ---- bf16 KV --------------------------------------------------------------------
 struct Bf16Tile {
     u32x4 k[4];  // K[token = lane%16][32*j + 8*(lane/16) .. +7]
-    u32x2 v[8];  // V[tokens 4*(lane/16)..+3][dim 16*b + lane%16]
+    u32x2 v[8];  // paged: V[tokens 4*(lane/16)..+3][dim 16*b + lane%16]
+                 // token-major: raw row chunks, (v[2j], v[2j+1]) = V[token 4j + lane/16][8*(lane%16)..+7]
 };
 
 struct Bf16Kv {
@@ -112,15 +146,32 @@ struct Bf16Kv {
         const uint16_t *krow = k + (uint64_t)(first + min((uint32_t)n, last)) * p.k_token_stride;
 #pragma unroll
         for (int j = 0; j < 4; ++j) t.k[j] = load_b128(krow + j * 32 + g * 8);
-        const uint16_t *v0 = v + (uint64_t)(first + min((uint32_t)(g * 4 + 0), last)) * p.v_token_stride;
-        const uint16_t *v1 = v + (uint64_t)(first + min((uint32_t)(g * 4 + 1), last)) * p.v_token_stride;
-        const uint16_t *v2 = v + (uint64_t)(first + min((uint32_t)(g * 4 + 2), last)) * p.v_token_stride;
-        const uint16_t *v3 = v + (uint64_t)(first + min((uint32_t)(g * 4 + 3), last)) * p.v_token_stride;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint16_t *vrow = v + (uint64_t)(first + min((uint32_t)(4 * j + g), last)) * p.v_token_stride;
+            const u32x4 chunk = load_b128(vrow + n * 8);
+            t.v[2 * j] = (u32x2){chunk.x, chunk.y};
+            t.v[2 * j + 1] = (u32x2){chunk.z, chunk.w};
+        }
+    }
+
+    // Token-major tiles: the raw V rows go through the wave's LDS area and come back as the
+    // V^T operand (lane (a, g) gets V[tokens 4g..4g+3][dim 16b + a]).  LDS operations of one
+    // wave execute in order, so the area can be reused tile after tile without a barrier.
+    __device__ static inline void transpose_rows(Tile &t, unsigned char *vt, int lane)
+    {
+        const int a = lane & 15, g = lane >> 4;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const u32x4 chunk = {t.v[2 * j].x, t.v[2 * j].y, t.v[2 * j + 1].x, t.v[2 * j + 1].y};
+            *reinterpret_cast<u32x4 *>(vt + vt_offset(4 * j + g, a)) = chunk;
+        }
+        const int row = 4 * g + (a >> 2);
 #pragma unroll
         for (int b = 0; b < 8; ++b) {
-            const int c = b * 16 + n;
-            t.v[b].x = (uint32_t)v0[c] | ((uint32_t)v1[c] << 16);
-            t.v[b].y = (uint32_t)v2[c] | ((uint32_t)v3[c] << 16);
+            const short4v w = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                (lds_short4 *)(vt + vt_offset(row, 2 * b + ((a >> 1) & 1)) + 8 * (a & 1)));
+            t.v[b] = __builtin_bit_cast(u32x2, w);
         }
     }
 
@@ -205,6 +256,7 @@ struct Q8Kv {
                                             const yvex_rocm_decode_params &, uint32_t, uint32_t, int)
     {
     }
+    __device__ static inline void transpose_rows(Tile &, unsigned char *, int) {}
 
     __device__ static inline void consume(State &st, const Tile &t, const bf16x8 (&q)[4],
                                           float scale_log2, uint32_t valid, int lane)
@@ -271,15 +323,20 @@ __device__ inline uint32_t wave_inclusive_scan(uint32_t v, int lane)
     return v;
 }
 
-template <class Kv, bool PAGED, int kDepth>
+// MERGE: split segments are merged in this kernel (arrival counters) instead of by
+// yvex_rocm_decode_finish; a compile-time choice so that the full-size kernels carry none of
+// the merge or gate code: with either present the compiler moves the tile bookkeeping of the
+// streaming loop from scalar to vector registers and the paged bf16 kernel loses 4 %.
+template <class Kv, bool PAGED, int kDepth, bool MERGE>
 struct Decoder {
     typedef typename Kv::Tile Tile;
     const yvex_rocm_decode_params &p;
+    unsigned char *const vt;  // token-major layout: 4 KB of LDS for the V transposition
     const int lane, n, g;
     const uint32_t group, limit;
 
-    __device__ Decoder(const yvex_rocm_decode_params &params)
-        : p(params), lane(threadIdx.x), n(threadIdx.x & 15), g(threadIdx.x >> 4),
+    __device__ Decoder(const yvex_rocm_decode_params &params, unsigned char *transpose_area)
+        : p(params), vt(transpose_area), lane(threadIdx.x), n(threadIdx.x & 15), g(threadIdx.x >> 4),
           group(params.query_heads / params.kv_heads),
           limit(PAGED ? params.table_stride * (uint32_t)kPageTokens : params.fixed_context)
     {
@@ -374,6 +431,7 @@ struct Decoder {
 #pragma unroll
             for (int r = 0; r < kDepth; ++r) {
                 const uint32_t tile = i + (uint32_t)r;
+                if (!PAGED) Kv::transpose_rows(ring[r], vt, lane);
                 Kv::consume(st, ring[r], q, p.scale_log2,
                             min((uint32_t)kPageTokens, t1 - (t0 + tile * kPageTokens)), lane);
                 fetch(ring[r], min(tile + kDepth, last_tile));
@@ -382,9 +440,11 @@ struct Decoder {
 #pragma unroll
         for (int r = 0; r < kDepth - 1; ++r) {
             const uint32_t tile = i + (uint32_t)r;
-            if (tile < count)
+            if (tile < count) {
+                if (!PAGED) Kv::transpose_rows(ring[r], vt, lane);
                 Kv::consume(st, ring[r], q, p.scale_log2,
                             min((uint32_t)kPageTokens, t1 - (t0 + tile * kPageTokens)), lane);
+            }
         }
     }
 
@@ -405,6 +465,10 @@ struct Decoder {
             u32x2 w;
             w.x = pack_bf16x2(a0, a1);
             w.y = pack_bf16x2(a2, a3);
+            if (MERGE && p.gate) {  // two-launch form: the finish kernel applies the gate
+                w = gate_four(w, p.gate + (dst - p.out) + b * 16);
+                bad |= pair_not_finite(w.x) || pair_not_finite(w.y);
+            }
             *reinterpret_cast<u32x2 *>(dst + b * 16) = w;
         }
         if (bad) flag(p.status, YVEX_ROCM_DEVICE_NUMERIC);
@@ -412,12 +476,140 @@ struct Decoder {
             p.lse[(uint64_t)session * p.query_heads + head] = (st.m + fast_log2(l)) * YVEX_LN2;
     }
 
+    // Leaves the wave's part of a split segment in its workspace slot.  With arrival counters
+    // the stores are written through to device scope and the wave waits until they have
+    // completed; without, the finish kernel reads them after this kernel has ended.
+    __device__ inline void leave_partial(const State &st, float l, uint32_t wave, bool starts_here) const
+    {
+        if ((uint32_t)n < group) {
+            // slot 1 when the segment starts inside this wave's range, else slot 0
+            const uint64_t slot = ((uint64_t)wave * 2u + (starts_here ? 1u : 0u)) * group + n;
+            float *acc = p.part_acc + slot * kHeadDim + g * 4;
+            if (MERGE) {
+#pragma unroll
+                for (int b = 0; b < 8; ++b) store_b128_device(acc + b * 16, st.o[b]);
+                if (g == 0) store_b64_device(p.part_ml + slot * 2, st.m, l);
+            } else {
+#pragma unroll
+                for (int b = 0; b < 8; ++b) *reinterpret_cast<floatx4 *>(acc + b * 16) = st.o[b];
+                if (g == 0) {
+                    p.part_ml[slot * 2 + 0] = st.m;
+                    p.part_ml[slot * 2 + 1] = l;
+                }
+            }
+        }
+        if (MERGE) __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+    }
+
+    // Log-sum-exp merge of the partials that waves w_first..w_last left for one segment, in
+    // wave order, and publication of the rows.  Lane = (head hl of a block of four, dims
+    // 8c..8c+7); kMergeWidth partials are in flight per trip (indices past the end alias the
+    // last one with weight zero).
+    __device__ inline void merge_segment(uint32_t session, uint32_t kv_head, uint32_t seg_begin,
+                                         uint32_t per_wave, uint32_t w_first, uint32_t w_last) const
+    {
+        constexpr int kMergeWidth = 8;
+        const uint32_t hl = (uint32_t)lane >> 4, c = (uint32_t)lane & 15u;
+        for (uint32_t h0 = 0u; h0 < group; h0 += 4u) {
+            const bool live = h0 + hl < group;
+            const uint32_t hh = min(h0 + hl, group - 1u);
+            float top = -INFINITY, sum = 0.f, acc[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc[i] = 0.f;
+            for (uint32_t j0 = w_first; j0 <= w_last; j0 += (uint32_t)kMergeWidth) {
+                // device-scope loads (sc1): they see the write-through stores of the other
+                // XCDs without an L2 invalidate, which would stall the waves still streaming
+                uint64_t ml[kMergeWidth], part[kMergeWidth][4];
+#pragma unroll
+                for (int i = 0; i < kMergeWidth; ++i) {
+                    const uint32_t j = min(j0 + (uint32_t)i, w_last);
+                    const uint64_t slot = ((uint64_t)j * 2u + (seg_begin >= j * per_wave ? 1u : 0u)) * group + hh;
+                    const uint64_t *row = reinterpret_cast<const uint64_t *>(p.part_acc + slot * kHeadDim + c * 8u);
+                    ml[i] = __hip_atomic_load(reinterpret_cast<const uint64_t *>(p.part_ml + slot * 2u),
+                                              __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        part[i][e] = __hip_atomic_load(row + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+                typedef float floatx2 __attribute__((ext_vector_type(2)));
+                float m[kMergeWidth], l[kMergeWidth];
+                float trip = -INFINITY;
+#pragma unroll
+                for (int i = 0; i < kMergeWidth; ++i) {
+                    const floatx2 pair = __builtin_bit_cast(floatx2, ml[i]);  // (max, sum)
+                    m[i] = j0 + (uint32_t)i > w_last ? -INFINITY : pair.x;  // past the end: weight zero
+                    l[i] = pair.y;
+                    trip = fmaxf(trip, m[i]);
+                }
+                const float m_new = fmaxf(top, trip);
+                const float keep = fast_exp2(top - m_new);  // 0 on the first trip
+                sum *= keep;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) acc[i] *= keep;
+#pragma unroll
+                for (int i = 0; i < kMergeWidth; ++i) {
+                    const float w = fast_exp2(m[i] - m_new);
+                    sum += w * l[i];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const floatx2 two = __builtin_bit_cast(floatx2, part[i][e]);
+                        acc[2 * e] += w * two.x;
+                        acc[2 * e + 1] += w * two.y;
+                    }
+                }
+                top = m_new;
+            }
+            if (!live) continue;
+            const uint32_t head = kv_head * group + hh;
+            const uint64_t at = ((uint64_t)session * p.query_heads + head) * kHeadDim + c * 8u;
+            const float inv = 1.0f / sum;
+            bool bad = false;
+            u32x2 w0, w1;
+            {
+                const float a0 = acc[0] * inv, a1 = acc[1] * inv, a2 = acc[2] * inv, a3 = acc[3] * inv;
+                const float a4 = acc[4] * inv, a5 = acc[5] * inv, a6 = acc[6] * inv, a7 = acc[7] * inv;
+                bad |= !(isfinite(a0) && isfinite(a1) && isfinite(a2) && isfinite(a3) &&
+                         isfinite(a4) && isfinite(a5) && isfinite(a6) && isfinite(a7));
+                w0.x = pack_bf16x2(a0, a1);
+                w0.y = pack_bf16x2(a2, a3);
+                w1.x = pack_bf16x2(a4, a5);
+                w1.y = pack_bf16x2(a6, a7);
+            }
+            if (p.gate) {
+                w0 = gate_four(w0, p.gate + at);
+                w1 = gate_four(w1, p.gate + at + 4);
+                bad |= pair_not_finite(w0.x) || pair_not_finite(w0.y) || pair_not_finite(w1.x) ||
+                       pair_not_finite(w1.y);
+            }
+            *reinterpret_cast<u32x4 *>(p.out + at) = (u32x4){w0.x, w0.y, w1.x, w1.y};
+            if (bad) flag(p.status, YVEX_ROCM_DEVICE_NUMERIC);
+            if (p.lse && c == 0u)
+                p.lse[(uint64_t)session * p.query_heads + head] = (top + fast_log2(sum)) * YVEX_LN2;
+        }
+    }
+
+    // Wave 0 leaves the exclusive prefix of per-session work items (and the total at index
+    // `sessions`) for the finish kernel.
+    __device__ inline void publish_offsets(uint32_t total) const
+    {
+        uint32_t carry = 0u;
+        for (uint32_t base = 0u; base < p.sessions; base += 64u) {
+            const uint32_t s = base + (uint32_t)lane;
+            const uint32_t t = s < p.sessions ? (context_of(s) + kPageTokens - 1u) / kPageTokens : 0u;
+            const uint32_t items = t * p.kv_heads;
+            const uint32_t incl = wave_inclusive_scan(items, lane);
+            if (s < p.sessions) p.offsets[s] = carry + incl - items;
+            carry += (uint32_t)__builtin_amdgcn_readlane((int)incl, 63);
+        }
+        if (lane == 0) p.offsets[p.sessions] = total;
+    }
+
     __device__ inline void run() const
     {
         const uint32_t wave = blockIdx.x, waves = gridDim.x;
         uint32_t session = 0u, offset = 0u, tiles = 0u, total = 0u;
         (void)locate(0xffffffffu, session, offset, tiles, total);
-        if (wave == 0u) publish_offsets(total);
+        if (wave == 0u && !MERGE) publish_offsets(total);
         if (total == 0u) return;
         const uint32_t per_wave = max((total + waves - 1u) / waves, p.min_tiles);
         uint32_t cur = wave * per_wave;
@@ -455,61 +647,56 @@ struct Decoder {
             l += xor_lanes(l, 32);
             if (first == 0u && stop == seg_end) {
                 publish(st, l, session, kv_head);  // the whole segment was ours
-            } else if ((uint32_t)n < group) {
-                // slot 1 when the segment starts inside this wave's range, else slot 0
-                const uint64_t slot = ((uint64_t)wave * 2u + (first == 0u ? 1u : 0u)) * group + n;
-                float *acc = p.part_acc + slot * kHeadDim + g * 4;
-#pragma unroll
-                for (int b = 0; b < 8; ++b) *reinterpret_cast<floatx4 *>(acc + b * 16) = st.o[b];
-                if (g == 0) {
-                    p.part_ml[slot * 2 + 0] = st.m;
-                    p.part_ml[slot * 2 + 1] = l;
+            } else {
+                leave_partial(st, l, wave, first == 0u);
+                if (!MERGE) {
+                    cur = stop;
+                    continue;  // the finish kernel merges
+                }
+                // count this wave in; whoever completes the count merges the segment
+                const uint32_t w_first = seg_begin / per_wave, w_last = (seg_end - 1u) / per_wave;
+                uint32_t *arrivals = p.arrivals + (uint64_t)session * p.kv_heads + kv_head;
+                uint32_t before = 0u;
+                if (lane == 0)
+                    before = __hip_atomic_fetch_add(arrivals, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                before = (uint32_t)__builtin_amdgcn_readfirstlane((int)before);
+                if (before == w_last - w_first) {
+                    if (lane == 0)
+                        __hip_atomic_store(arrivals, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    // no cache invalidate: the merge reads with device-scope loads; this only
+                    // keeps the compiler from moving them above the count
+                    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+                    merge_segment(session, kv_head, seg_begin, per_wave, w_first, w_last);
                 }
             }
             cur = stop;
         }
     }
-
-    // Wave 0 leaves the exclusive prefix of per-session work items (and the total at
-    // index `sessions`) for the merge kernel.
-    __device__ inline void publish_offsets(uint32_t total) const
-    {
-        uint32_t carry = 0u;
-        for (uint32_t base = 0u; base < p.sessions; base += 64u) {
-            const uint32_t s = base + (uint32_t)lane;
-            const uint32_t t = s < p.sessions ? (context_of(s) + kPageTokens - 1u) / kPageTokens : 0u;
-            const uint32_t items = t * p.kv_heads;
-            const uint32_t incl = wave_inclusive_scan(items, lane);
-            if (s < p.sessions) p.offsets[s] = carry + incl - items;
-            carry += (uint32_t)__builtin_amdgcn_readlane((int)incl, 63);
-        }
-        if (lane == 0) p.offsets[p.sessions] = total;
-    }
 };
 
 }  // namespace
 
-extern "C" __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2)))
-yvex_rocm_decode_paged_bf16(const yvex_rocm_decode_params p)
-{
-    Decoder<Bf16Kv, true, 3>(p).run();
-}
+#define YVEX_DECODE_KERNEL(name, Kv, PAGED, DEPTH, MERGE)                                           \
+    extern "C" __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2)))  \
+    name(const yvex_rocm_decode_params p)                                                      \
+    {                                                                                          \
+        __shared__ __attribute__((aligned(16))) unsigned char vt[PAGED ? 16 : kPageTokens * kHeadDim * 2]; \
+        Decoder<Kv, PAGED, DEPTH, MERGE>(p, vt).run();                                         \
+    }
 
-extern "C" __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2)))
-yvex_rocm_decode_paged_q8_0(const yvex_rocm_decode_params p)
-{
-    Decoder<Q8Kv, true, 3>(p).run();
-}
+// full-size launches: partials for yvex_rocm_decode_finish
+YVEX_DECODE_KERNEL(yvex_rocm_decode_paged_bf16, Bf16Kv, true, 3, false)
+YVEX_DECODE_KERNEL(yvex_rocm_decode_paged_q8_0, Q8Kv, true, 3, false)
+YVEX_DECODE_KERNEL(yvex_rocm_decode_rows_bf16, Bf16Kv, false, 2, false)
+// launches that do not fill the device: merge in the kernel, one launch
+YVEX_DECODE_KERNEL(yvex_rocm_decode_paged_bf16_merged, Bf16Kv, true, 3, true)
+YVEX_DECODE_KERNEL(yvex_rocm_decode_paged_q8_0_merged, Q8Kv, true, 3, true)
+YVEX_DECODE_KERNEL(yvex_rocm_decode_rows_bf16_merged, Bf16Kv, false, 2, true)
 
-extern "C" __global__ void __launch_bounds__(64)
-yvex_rocm_decode_rows_bf16(const yvex_rocm_decode_params p)
-{
-    Decoder<Bf16Kv, false, 2>(p).run();
-}
-
-// Merge of the split segments of the balanced decode.  grid = (query_heads, sessions),
-// block = head_dim threads (one per output lane).  A segment that one wave covered was
-// already published by that wave and is skipped.
+// Merge of the split segments of the balanced decode when the decode kernel was launched
+// without arrival counters (large launches).  grid = (query_heads, sessions), block =
+// head_dim threads (one per output lane).  A segment that one wave covered was already
+// published by that wave and is skipped.
 extern "C" __global__ void __launch_bounds__(128)
 yvex_rocm_decode_finish(const yvex_rocm_decode_params p)
 {

@@ -47,7 +47,7 @@ def test_config1_contiguous_decode_matches_cpu_operator(backend):
     assert rc == 0
     assert_close_bf16(got, ref, "config1")
     assert_lse(lse, ref_lse, "config1")
-    assert facts.kernel_launches == 2 and facts.device_synchronizations == 1
+    assert facts.kernel_launches == 1 and facts.device_synchronizations == 1
     assert facts.temporary_bytes > 0
 
 
@@ -135,7 +135,7 @@ def test_paged_decode_matches_oracle_ragged(backend):
     assert rc == 0
     assert_close_bf16(got, ref, "paged")
     assert_lse(lse, ref_lse, "paged")
-    assert facts.kernel_launches == 2 and facts.device_synchronizations == 1
+    assert facts.kernel_launches in (1, 2) and facts.device_synchronizations == 1
 
 
 def test_paged_decode_page_placement_is_bit_invariant(backend):
@@ -222,7 +222,7 @@ def test_q8_0_paged_decode_matches_cpu_on_same_bytes(backend):
     assert rc == 0
     assert_close_bf16(got, ref, "q8_0 paged")
     assert_lse(lse, ref_lse, "q8_0 paged")
-    assert facts.kernel_launches == 2
+    assert facts.kernel_launches in (1, 2)
 
 
 def test_q8_0_paged_placement_invariance_and_garbage_tail(backend):

@@ -70,7 +70,7 @@ def test_row_decode_with_fused_gate(backend, ctx):
     plain, fused = backend.tensor("o", B.DTYPE_BF16, q.shape), backend.tensor("og", B.DTYPE_BF16, q.shape)
     backend.attention_execute(req, *t, plain)
     facts = backend.attention_execute(req, *t, fused, gate=tg)
-    assert facts.kernel_launches == 2
+    assert facts.kernel_launches == 1
     rc, ref, _, _ = ORACLE.gqa_bf16(q, k, v, query_start=ctx - 1, causal=True)
     assert rc == 0
     assert_close_bf16(fused.read(), gated_reference(ref, gate), "row decode gate ctx=%d" % ctx)
@@ -82,7 +82,7 @@ def test_row_decode_with_fused_gate(backend, ctx):
 @pytest.mark.parametrize("q8", [False, True], ids=["bf16", "q8_0"])
 def test_paged_decode_with_fused_gate(backend, q8):
     """Short contexts (rows published by the decode kernel itself) and long ones (merged by
-    the finish kernel) in one batch: the gate reaches both."""
+    the merging wave) in one batch: the gate reaches both."""
     rng = np.random.default_rng(7200 + q8)
     sessions, hq, hkv, d, page = 6, 32, 8, 128, 16
     contexts = np.array([1, 16, 33, 900, 5000, 12000], np.int32)
@@ -113,7 +113,7 @@ def test_paged_decode_with_fused_gate(backend, q8):
                                     int(stride * page), storage=storage)
     backend.paged_decode_execute(req, *t, plain)
     facts = backend.paged_decode_execute(req, *t, fused, gate=tg)
-    assert facts.kernel_launches == 2
+    assert facts.kernel_launches in (1, 2)
     rc, ref, _, _ = ORACLE.paged_decode(q, k_rows, v_rows, table, contexts, hkv, page, q8=q8)
     assert rc == 0
     assert_close_bf16(fused.read(), gated_reference(ref, gate), "paged gate")

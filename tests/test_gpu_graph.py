@@ -44,7 +44,7 @@ def test_recorded_row_decode_replays_equal_eager(backend):
         tq.write(q)
         out.zero()
         facts = backend.graph_launch(graph)
-        assert facts.kernel_launches == 2
+        assert facts.kernel_launches == 1
         got = out.read()
         unrelated_eager_work(backend, rng)
         backend.attention_execute(req, tq, tk, tv, eager)
@@ -119,7 +119,7 @@ def test_recorded_decode_step_appends_then_attends(backend):
         tensors["q"].write(bf16_normal(rng, (sessions, hq, d)))
         tensors["gate"].write(bf16_normal(rng, (sessions, hq, d)))
         facts = backend.graph_launch(graph)
-        assert facts.kernel_launches == 3
+        assert facts.kernel_launches == 2
         got = rec_out.read()
         unrelated_eager_work(backend, rng)
         step_operations(eag_k, eag_v, eag_out)

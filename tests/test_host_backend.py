@@ -355,7 +355,7 @@ def test_attention_execute_contracts_facts_and_workspace(fake_runtime):
         assert (facts.kernel_launches, facts.device_synchronizations, facts.d2h_bytes,
                 facts.download_count) == (1, 1, 4, 1) and out.is_written
         assert b.attention_workspace_required(req) == 0
-        # bf16 decode: two launches (stream + finish), workspace == planned bytes, attached workspace is used
+        # bf16 decode: one launch (split segments are merged in the kernel), workspace == planned bytes, attached workspace is used
         req = b.attention_requirement(1, 4096, 32, 8, 128, query_start=4095, dtype=B.DTYPE_BF16,
                                       contract=B.NUMERIC_BF16_F32_ACCUMULATE)
         planned = b.attention_workspace_required(req)
@@ -365,7 +365,7 @@ def test_attention_execute_contracts_facts_and_workspace(fake_runtime):
         ob = b.tensor("o", B.DTYPE_BF16, (1, 32, 128))
         live = fake_runtime.fake_hip_live_allocations()
         facts = b.attention_execute(req, qb, kb, kb, ob)
-        assert facts.kernel_launches == 2 and facts.temporary_bytes == planned
+        assert facts.kernel_launches == 1 and facts.temporary_bytes == planned
         assert fake_runtime.fake_hip_live_allocations() == live      # temporary released
         work = b.tensor("workspace", B.DTYPE_I8, (planned,))
         b.workspace_attach(work)
@@ -428,7 +428,7 @@ def test_paged_and_mla_admission():
         table, ctx = written(b, "t", B.DTYPE_I32, (4, 64)), written(b, "c", B.DTYPE_I32, (4,))
         out = b.tensor("o", B.DTYPE_BF16, (4, 32, 128))
         facts = b.paged_decode_execute(ok, q, pool, pool, table, ctx, out)
-        assert facts.kernel_launches == 2 and out.is_written
+        assert facts.kernel_launches == 1 and out.is_written
         small = written(b, "small-pool", B.DTYPE_BF16, (99 * 8 * 2048,))
         with pytest.raises(YvexError) as e:
             b.paged_decode_execute(ok, q, small, pool, table, ctx, out)
@@ -558,7 +558,7 @@ def test_fused_gate_admission():
         table, ctx = written(b, "t", B.DTYPE_I32, (4, 64)), written(b, "c", B.DTYPE_I32, (4,))
         pout = b.tensor("po", B.DTYPE_BF16, (4, 32, 128))
         pgate = written(b, "pg", B.DTYPE_BF16, (4, 32, 128))
-        assert b.paged_decode_execute(paged, pq, pool, pool, table, ctx, pout, gate=pgate).kernel_launches == 2
+        assert b.paged_decode_execute(paged, pq, pool, pool, table, ctx, pout, gate=pgate).kernel_launches == 1
         with pytest.raises(YvexError) as e:
             b.paged_decode_execute(paged, pq, pool, pool, table, ctx, pout, gate=gate)
         assert e.value.code == B.YVEX_ERR_FORMAT
@@ -594,13 +594,13 @@ def test_recorded_sequence_rules(fake_runtime):
         before = fake_runtime.fake_hip_launches()
         b.graph_begin()
         facts = b.attention_execute(req, q, k, v, out)
-        assert facts.kernel_launches == 2 and facts.device_synchronizations == 0
+        assert facts.kernel_launches == 1 and facts.device_synchronizations == 0
         assert fake_runtime.fake_hip_launches() == before      # recorded, not run
         graph = b.graph_end()
         for n in (1, 2, 3):
             facts = b.graph_launch(graph)
-            assert facts.kernel_launches == 2 and facts.device_synchronizations == 1
-            assert fake_runtime.fake_hip_launches() == before + 2 * n
+            assert facts.kernel_launches == 1 and facts.device_synchronizations == 1
+            assert fake_runtime.fake_hip_launches() == before + n
         b.set_completion_mode(B.COMPLETION_DEFERRED)
         assert b.graph_launch(graph).device_synchronizations == 0
         b.sync()

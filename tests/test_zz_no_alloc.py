@@ -43,7 +43,7 @@ def run_both(backend, contexts, hq, hkv, storage, seed):
             assert backend.memory_stats().allocation_events == before   # nothing was acquired
         else:
             facts = backend.paged_decode_execute(req, tq, tkp, tvp, tt, tc, out, lse)
-        assert facts.kernel_launches == 2
+        assert facts.kernel_launches in (1, 2)
         results.append((out.read(), lse.read()))
     (ref_out, ref_lse), (got_out, got_lse) = results
     assert np.array_equal(got_out, ref_out), "output bits differ from paged_decode_execute"
