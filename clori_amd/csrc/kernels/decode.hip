@@ -67,15 +67,17 @@ __device__ inline void flag(int32_t *status, int code) { atomicCAS(status, 0, co
 // 16 / 8 bytes to global memory, visible device-wide once the store has completed: the
 // write-through form (sc1) the memory model uses for device-scope atomic stores on this
 // multi-XCD part.  Plain stores would sit in the XCD's L2 until a write-back.
-__device__ inline void store_b128_device(void *p, floatx4 v)
-{
-    asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(p), "v"(v) : "memory");
-}
 __device__ inline void store_b64_device(void *p, float a, float b)
 {
     typedef float floatx2 __attribute__((ext_vector_type(2)));
     const floatx2 v = {a, b};
-    asm volatile("global_store_dwordx2 %0, %1, off sc1" : : "v"(p), "v"(v) : "memory");
+    __hip_atomic_store(reinterpret_cast<uint64_t *>(p), __builtin_bit_cast(uint64_t, v),
+                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ inline void store_b128_device(void *p, floatx4 v)
+{
+    store_b64_device(p, v[0], v[1]);
+    store_b64_device(reinterpret_cast<float *>(p) + 2, v[2], v[3]);
 }
 
 typedef __attribute__((address_space(3))) short4v lds_short4;
