@@ -475,3 +475,16 @@ def q8_0_decode_rows(b, n):
     _check(lib().yvex_rocm_q8_0_decode_row(b.ctypes.data, out.size, out.ctypes.data, C.byref(err)),
            err)
     return out
+
+
+def benchmark_summarize(seconds, prefix=""):
+    """Distribution fields of a benchmark record from per-iteration samples in seconds
+    (src/runtime/benchmark.c:421-447): {"minimum_ns": ..., "p50_ns": ..., ...}, each name
+    prefixed with `prefix` ("device_" for device timing).  Raises YvexError on samples that are
+    not finite and positive."""
+    samples = np.ascontiguousarray(seconds, dtype=np.float64).copy()
+    out, err = B.TimingDistribution(), B.Error()
+    _check(lib().yvex_runtime_benchmark_samples_summarize(
+        samples.ctypes.data_as(C.POINTER(C.c_double)), samples.size, C.byref(out), C.byref(err)), err)
+    return {prefix + lib().yvex_runtime_benchmark_statistic_name(i).decode(): int(out.values[i])
+            for i in range(B.BENCHMARK_STATISTIC_COUNT)}

@@ -246,6 +246,14 @@ class RocmReport(C.Structure):
                 ("rejection", C.c_char * 256)]
 
 
+#: include/yvex/internal/benchmark.h:82-97
+BENCHMARK_STATISTIC_COUNT = 8
+
+
+class TimingDistribution(C.Structure):
+    _fields_ = [("available", C.c_int), ("values", ull * BENCHMARK_STATISTIC_COUNT)]
+
+
 #: every symbol include/yvex_rocm.h declares
 EXPORTED_SYMBOLS = [
     "yvex_status_name", "yvex_error_clear", "yvex_error_set",
@@ -270,7 +278,10 @@ EXPORTED_SYMBOLS = [
     "yvex_backend_rocm_kernel_probe_begin", "yvex_backend_rocm_kernel_probe_end",
     "yvex_backend_bandwidth_probe", "yvex_backend_rocm_graph_begin", "yvex_backend_rocm_graph_end",
     "yvex_backend_rocm_graph_launch", "yvex_backend_rocm_graph_release",
-    "yvex_backend_rocm_report_get", "yvex_quant_f16_decode", "yvex_quant_f16_encode",
+    "yvex_backend_rocm_report_get", "yvex_backend_report_build",
+    "yvex_backend_bundle_admission_name", "yvex_backend_render", "yvex_backend_command",
+    "yvex_rocm_info_command", "yvex_runtime_benchmark_samples_summarize",
+    "yvex_runtime_benchmark_statistic_name", "yvex_quant_f16_decode", "yvex_quant_f16_encode",
     "yvex_quant_bf16_decode", "yvex_quant_bf16_encode", "yvex_rocm_q8_0_encode_row",
     "yvex_rocm_q8_0_decode_row", "yvex_rocm_kv_page_block_bytes", "yvex_rocm_kv_pack_pages",
     "yvex_rocm_kv_unpack_pages",
@@ -348,6 +359,16 @@ def load(path=None):
     lib.yvex_backend_rocm_graph_launch.argtypes = [vp, C.c_void_p, FactsP, ErrorP]
     lib.yvex_backend_rocm_graph_release.argtypes = [vp, C.POINTER(C.c_void_p), ErrorP]
     lib.yvex_backend_rocm_report_get.argtypes = [vp, C.POINTER(RocmReport), ErrorP]
+    lib.yvex_backend_report_build.argtypes = [vp, vp, ErrorP]
+    lib.yvex_backend_bundle_admission_name.restype = C.c_char_p
+    lib.yvex_backend_bundle_admission_name.argtypes = [C.c_int]
+    lib.yvex_backend_render.argtypes = [vp, vp]
+    lib.yvex_backend_command.argtypes = [C.c_int, C.POINTER(C.c_char_p)]
+    lib.yvex_rocm_info_command.argtypes = [C.c_int, C.POINTER(C.c_char_p)]
+    lib.yvex_runtime_benchmark_samples_summarize.argtypes = [
+        C.POINTER(C.c_double), ull, C.POINTER(TimingDistribution), ErrorP]
+    lib.yvex_runtime_benchmark_statistic_name.restype = C.c_char_p
+    lib.yvex_runtime_benchmark_statistic_name.argtypes = [C.c_int]
     lib.yvex_quant_f16_decode.restype = C.c_float
     lib.yvex_quant_f16_decode.argtypes = [C.c_ushort]
     lib.yvex_quant_f16_encode.restype = C.c_ushort

@@ -696,6 +696,92 @@ typedef struct {
 int yvex_backend_rocm_report_get(const yvex_backend *backend, yvex_backend_rocm_report *out,
                                  yvex_error *err);
 
+/*
+ * Immutable backend reports and the inspection commands over them
+ * (include/yvex/internal/backend.h:501-533, src/backend/core.c:1824-1916,
+ * src/cli/render/backend.c:51-160, src/cli/commands/backend.c:11-52).  The first three report
+ * kinds keep the reference's values; the ROCM kinds are the `inspect rocm [bandwidth]`
+ * counterparts of the CUDA ones.  A backend that cannot be opened here is reported, not
+ * failed: available = 0, the reason text, exit_code 5.  `variants` holds the reference's
+ * variants in order, then this backend's attention variants.
+ */
+typedef enum {
+    YVEX_BACKEND_REPORT_CAPABILITIES = 0,
+    YVEX_BACKEND_REPORT_CUDA_INFO,
+    YVEX_BACKEND_REPORT_CUDA_BANDWIDTH,
+    YVEX_BACKEND_REPORT_ROCM_INFO,
+    YVEX_BACKEND_REPORT_ROCM_BANDWIDTH
+} yvex_backend_report_kind;
+typedef enum {
+    YVEX_BACKEND_BUNDLE_NOT_APPLICABLE = 0,
+    YVEX_BACKEND_BUNDLE_ABSENT,
+    YVEX_BACKEND_BUNDLE_ADMITTED,
+    YVEX_BACKEND_BUNDLE_REJECTED
+} yvex_backend_bundle_admission;
+typedef struct {
+    yvex_backend_report_kind kind;
+    yvex_backend_kind backend_kind;
+} yvex_backend_report_request;
+#define YVEX_BACKEND_REPORT_VARIANT_CAP \
+    (YVEX_BACKEND_VARIANT_COUNT + (YVEX_BACKEND_VARIANT_ROCM_END - YVEX_BACKEND_VARIANT_ROCM_FIRST))
+typedef struct {
+    yvex_backend_report_kind kind;
+    yvex_backend_kind backend_kind;
+    yvex_backend_status backend_status;
+    int exit_code, available, has_device_info, kernel_bundle_native;
+    yvex_backend_device_info device_info;
+    char device_name[128], reason[256], kernel_bundle_architecture[16];
+    char kernel_bundle_identity[YVEX_SHA256_HEX_BYTES];
+    yvex_backend_memory_stats memory;
+    int capabilities[YVEX_BACKEND_CAP_OP_ATTENTION + 1];
+    yvex_backend_capability_result variants[YVEX_BACKEND_REPORT_VARIANT_CAP];
+    unsigned int variant_count, context_available;
+    yvex_backend_bundle_admission bundle_admission;
+    yvex_backend_capability_reason bundle_reason;
+    yvex_backend_bandwidth_evidence bandwidth;
+    unsigned int kernel_image_count, kernel_function_count;
+    char driver_library[256];
+} yvex_backend_report;
+int yvex_backend_report_build(const yvex_backend_report_request *request,
+                              yvex_backend_report *report, yvex_error *err);
+const char *yvex_backend_bundle_admission_name(yvex_backend_bundle_admission admission);
+/* `fp` is a FILE *; declared void * so that this header needs no <stdio.h>. */
+int yvex_backend_render(void *fp, const yvex_backend_report *report);
+/* Command entry points with the adapter's argv: {program, "backend", "rocm"} and
+ * {program, "rocm-info"[, "bandwidth"]}.  They print to stdout (errors to stderr) and return
+ * the process exit code: 0, 5 when the backend is unsupported here, 2 for a grammar error
+ * (src/cli/io/out.c:1277-1292). */
+int yvex_backend_command(int argc, char **argv);
+int yvex_rocm_info_command(int argc, char **argv);
+
+/*
+ * Sample summary of a component benchmark (include/yvex/internal/benchmark.h:82-97,
+ * src/runtime/benchmark.c:388-447,559-573): sorts `seconds` in place, takes nearest-rank
+ * percentiles sample[(count * p + 99) / 100 - 1], the mean and the population standard
+ * deviation, and stores them as whole nanoseconds.  Samples must be finite and positive.
+ */
+typedef enum {
+    YVEX_RUNTIME_BENCHMARK_MINIMUM = 0,
+    YVEX_RUNTIME_BENCHMARK_P50,
+    YVEX_RUNTIME_BENCHMARK_P90,
+    YVEX_RUNTIME_BENCHMARK_P95,
+    YVEX_RUNTIME_BENCHMARK_P99,
+    YVEX_RUNTIME_BENCHMARK_MAXIMUM,
+    YVEX_RUNTIME_BENCHMARK_MEAN,
+    YVEX_RUNTIME_BENCHMARK_STANDARD_DEVIATION,
+    YVEX_RUNTIME_BENCHMARK_STATISTIC_COUNT
+} yvex_runtime_benchmark_statistic;
+typedef struct {
+    int available;
+    unsigned long long values[YVEX_RUNTIME_BENCHMARK_STATISTIC_COUNT];
+} yvex_runtime_benchmark_timing_distribution;
+int yvex_runtime_benchmark_samples_summarize(double *seconds, unsigned long long count,
+                                             yvex_runtime_benchmark_timing_distribution *out,
+                                             yvex_error *err);
+/* Field name of a statistic in a benchmark record ("minimum_ns", "p50_ns", ...;
+ * src/runtime/benchmark.c:127-140); device timing prefixes it with "device_". */
+const char *yvex_runtime_benchmark_statistic_name(yvex_runtime_benchmark_statistic statistic);
+
 /* ---- scalar and block codecs (host): src/gguf/quant_scalar.c:40-143,
  *      src/gguf/quant_block.c:160-186,819-833 ------------------------------- */
 float yvex_quant_f16_decode(unsigned short bits);

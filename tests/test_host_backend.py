@@ -246,6 +246,19 @@ print("absent-ok")
     result = subprocess.run(["python3", "-c", script], capture_output=True, text=True,
                             env=dict(os.environ))
     assert "absent-ok" in result.stdout, result.stderr
+    # the inspection command of the same build, with the lines the reference's bundle-less
+    # build prints (tests/test_cuda_failclosed.sh:59-80)
+    shown = subprocess.run([str(tmp_path / "yvex-rocm"), "inspect", "backend", "rocm"],
+                           capture_output=True, text=True, env=dict(os.environ))
+    assert shown.returncode == 0, shown.stderr
+    for line in ("status: context-ready", "  tensor_alloc: yes", "  tensor_read_write: yes",
+                 "  op_attention: no", "context_available: yes", "kernel_bundle: absent",
+                 "kernel_bundle_reason: kernel-bundle-absent", "kernel_bundle_native: no",
+                 "  attention-noncausal-f32: unsupported (kernel-bundle-absent)",
+                 "  encoded-attention: unsupported (kernel-bundle-absent)",
+                 "  rocm-attention-paged-bf16: unsupported (kernel-bundle-absent)",
+                 "status: backend-capabilities"):
+        assert line + "\n" in shown.stdout, line
 
 
 # ------------------------------------------------------------- tensors ----
