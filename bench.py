@@ -55,11 +55,17 @@ SPIN_UP_SECONDS = float(os.environ.get("YVEX_BENCH_SPIN_UP", "0.2"))
 RECORDED_STEPS = bool(int(os.environ.get("YVEX_BENCH_RECORDED", "0")))
 
 
-def time_steps(backend, run, steps, warmup, kernel):
-    """W untimed steps, then K steps bracketed by device events and by a synchronise on
-    both sides; then the same K steps again with an event pair around every launch of the
-    dominant kernel.  Returns (device ms per step, wall ms per step, ms per launch of the
-    dominant kernel)."""
+RECORD_ITERATIONS = 100       # per-dispatch samples of the benchmark record
+
+
+def time_steps(backend, run, steps, warmup, kernels):
+    """W untimed steps, then K steps bracketed by device events and by a synchronise on both
+    sides: that is the step time `value` is computed from.  Afterwards, outside the timed
+    region: for each kernel of the step, the same steps again with an event pair around
+    every launch of that kernel (mean duration per launch, the first kernel named is the
+    dominant one), and RECORD_ITERATIONS single dispatches each timed on the host and on the
+    device, from which the benchmark record's distributions are taken."""
+    from clori_amd.backend import benchmark_summarize
     backend.set_completion_mode(B.COMPLETION_DEFERRED)
     step, graph = run, None
     if RECORDED_STEPS:
@@ -87,18 +93,52 @@ def time_steps(backend, run, steps, warmup, kernel):
     wall_ms = (time.perf_counter() - t0) * 1e3
     if graph is not None:
         backend.graph_release(graph)
-    backend.kernel_probe_begin(kernel)
-    for _ in range(min(steps, 256)):
-        run()
-    launches, kernel_ms = backend.kernel_probe_end()
-    backend.sync()
+    kernel_ms = {}
+    for kernel in kernels:
+        backend.kernel_probe_begin(kernel)
+        for _ in range(min(steps, 128)):
+            run()
+        launches, total_ms = backend.kernel_probe_end()
+        backend.sync()
+        if launches:
+            kernel_ms[kernel] = total_ms / launches
+    # per-dispatch samples: each dispatch completes (status read back) before the next starts
     backend.set_completion_mode(B.COMPLETION_IMMEDIATE)
-    # an event pair around one launch adds a few microseconds: a kernel cannot take longer than
-    # the step that contains it
-    return device_ms / steps, wall_ms / steps, min(kernel_ms / max(launches, 1), device_ms / steps)
+    before = backend.memory_stats()
+    host_s, device_s, facts = [], [], None
+    for _ in range(RECORD_ITERATIONS):
+        h0 = time.perf_counter()
+        backend.timing_begin()
+        facts = run()
+        device_s.append(backend.timing_end() * 1e-3)
+        host_s.append(time.perf_counter() - h0)
+    after = backend.memory_stats()
+    record = {"benchmark_scope": "attention_component", "warmup_count": warmup,
+              "iteration_count": RECORD_ITERATIONS, "first_execution_ns": int(host_s[0] * 1e9 + 0.5)}
+    record.update(benchmark_summarize(host_s))
+    record["device_timing_available"] = True
+    record.update(benchmark_summarize(device_s, prefix="device_"))
+    record.update({
+        "h2d_bytes": int(after.h2d_bytes - before.h2d_bytes),
+        "d2h_bytes": int(after.d2h_bytes - before.d2h_bytes),
+        "warm_device_allocations": int(after.allocation_events - before.allocation_events),
+        "warm_device_frees": int(after.release_events - before.release_events),
+        "last_dispatch_kernel_launches": int(facts.kernel_launches),
+        "last_dispatch_peak_device_bytes": int(after.peak_allocated_bytes),
+        "resident_bytes": int(after.allocated_bytes)})
+    return dict(ms=device_ms / steps, wall_ms=wall_ms / steps, kernel_ms=kernel_ms, record=record)
 
 
 # --------------------------------------------------------------------- workloads --
+
+def decode_kernels(kernel, facts):
+    """Kernels of one decode step.  A launch that does not fill the device merges its split
+    segments in the kernel itself (one launch, the `_merged` build of the kernel); a full-size
+    launch leaves the merge to a second, small kernel."""
+    if facts.kernel_launches == 1:
+        return [kernel + "_merged"]
+    return [kernel, "yvex_rocm_decode_finish"]
+
 
 def workload_paged(backend, rng, steps, warmup, q8=False):
     sessions, hq, hkv, d, page = 32, 32, 8, 128, 16
@@ -146,7 +186,8 @@ def workload_paged(backend, rng, steps, warmup, q8=False):
     run = lambda: backend.paged_decode_execute(req, q, k_pool, v_pool, tt, tc, out, lse)  # noqa: E731
     facts = run()
     kernel = "yvex_rocm_decode_paged_q8_0" if q8 else "yvex_rocm_decode_paged_bf16"
-    ms, wall, kms = time_steps(backend, run, steps, warmup, kernel)
+    kernels = decode_kernels(kernel, facts)
+    timed = time_steps(backend, run, steps, warmup, kernels)
     backend.workspace_detach()
     tokens = int(contexts.sum())
     per_token = 2 * hkv * (136 if q8 else 256)
@@ -157,8 +198,8 @@ def workload_paged(backend, rng, steps, warmup, q8=False):
                 workload="paged %s GQA decode: 32 sessions, 32/8 heads, d=128, contexts U[%d,%d], "
                          "16-token pages, seeded permutation page tables" %
                          ("Q8_0" if q8 else "bf16", lo, hi),
-                bound="hbm", algorithmic_bytes=algo, tokens=tokens, ms=ms, wall_ms=wall,
-                kernel_ms=kms, launches=int(facts.kernel_launches), dominant_kernel=kernel)
+                bound="hbm", algorithmic_bytes=algo, tokens=tokens,
+                launches=int(facts.kernel_launches), kernels=kernels, **timed)
 
 
 def workload_decode1(backend, rng, steps, warmup):
@@ -175,15 +216,14 @@ def workload_decode1(backend, rng, steps, warmup):
     backend.workspace_attach(work)
     run = lambda: backend.attention_execute(req, q, k, v, out, lse=lse)  # noqa: E731
     facts = run()
-    # a launch that does not fill the device merges its split segments in the kernel itself
-    kernel = "yvex_rocm_decode_rows_bf16" + ("_merged" if facts.kernel_launches == 1 else "")
-    ms, wall, kms = time_steps(backend, run, steps, warmup, kernel)
+    kernels = decode_kernels("yvex_rocm_decode_rows_bf16", facts)
+    timed = time_steps(backend, run, steps, warmup, kernels)
     backend.workspace_detach()
     algo = 2 * ctx * hkv * d * 2 + 2 * hq * d * 2 + hq * 4
     return dict(name="decode1",
                 workload="GQA decode: batch 1, 32/8 heads, d=128, context 4096, contiguous bf16 KV",
-                bound="hbm", algorithmic_bytes=algo, tokens=ctx, ms=ms, wall_ms=wall, kernel_ms=kms,
-                launches=int(facts.kernel_launches), dominant_kernel=kernel)
+                bound="hbm", algorithmic_bytes=algo, tokens=ctx,
+                launches=int(facts.kernel_launches), kernels=kernels, **timed)
 
 
 def workload_prefill2(backend, rng, steps, warmup):
@@ -201,13 +241,13 @@ def workload_prefill2(backend, rng, steps, warmup):
                                         contract=B.NUMERIC_BF16_F32_ACCUMULATE)
     run = lambda: backend.attention_execute(req, q, k, v, out)  # noqa: E731
     facts = run()
-    ms, wall, kms = time_steps(backend, run, steps, warmup, "yvex_rocm_prefill_bf16")
+    kernels = ["yvex_rocm_prefill_bf16"]
+    timed = time_steps(backend, run, steps, warmup, kernels)
     flops = 4 * d * hq * t * (t + 1) // 2      # causal-useful multiply-adds * 2, QK^T and PV
     return dict(name="prefill2",
                 workload="causal GQA prefill: batch 1, seq 2048, 40/8 heads, d=128, bf16",
                 bound="mfma", flops=flops, algorithmic_bytes=(2 * t * hq * d + 2 * t * hkv * d) * 2,
-                ms=ms, wall_ms=wall, kernel_ms=kms, launches=int(facts.kernel_launches),
-                dominant_kernel="yvex_rocm_prefill_bf16")
+                launches=int(facts.kernel_launches), kernels=kernels, **timed)
 
 
 def workload_mla5(backend, rng, steps, warmup):
@@ -228,7 +268,8 @@ def workload_mla5(backend, rng, steps, warmup):
     backend.workspace_attach(work)
     run = lambda: backend.mla_decode_execute(req, q, pool, tt, tc, out, lse)  # noqa: E731
     facts = run()
-    ms, wall, kms = time_steps(backend, run, steps, warmup, "yvex_rocm_mla_decode_bf16")
+    kernels = ["yvex_rocm_mla_decode_bf16", "yvex_rocm_decode_merge"]
+    timed = time_steps(backend, run, steps, warmup, kernels)
     backend.workspace_detach()
     algo = batch * ctx * kd * 2 + batch * heads * (kd + vd) * 2 + table.size * 4 + batch * heads * 4
     assert np.all(np.isfinite(lse.read()))
@@ -236,8 +277,7 @@ def workload_mla5(backend, rng, steps, warmup):
                 workload="absorbed MLA decode: batch 16, 128 heads, latent 512 + rope 64, "
                          "context 8192 in 64-token pages",
                 bound="hbm", algorithmic_bytes=algo, flops=batch * heads * ctx * 2 * (kd + vd),
-                ms=ms, wall_ms=wall, kernel_ms=kms, launches=int(facts.kernel_launches),
-                dominant_kernel="yvex_rocm_mla_decode_bf16")
+                launches=int(facts.kernel_launches), kernels=kernels, **timed)
 
 
 def workload_append(backend, rng, steps, warmup, q8=False):
@@ -273,14 +313,15 @@ def workload_append(backend, rng, steps, warmup, q8=False):
                                             cosine=cosine, sine=sine, rotary_dimension=d)
     facts = run()
     kernel = "yvex_rocm_kv_append_q8_0" if q8 else "yvex_rocm_kv_append_bf16"
-    ms, wall, kms = time_steps(backend, run, steps, warmup, kernel)
+    kernels = [kernel]
+    timed = time_steps(backend, run, steps, warmup, kernels)
     # per token: K and V rows in (bf16), both page rows out, half a cos and half a sin row
     algo = total * (2 * hkv * d * 2 + 2 * hkv * (136 if q8 else 256) + d * 4) + 3 * sessions * 4
     return dict(name="append_q8_0" if q8 else "append_bf16",
                 workload="KV page writer, %s pages: 16 sessions x 2048 new tokens, 8 kv heads, "
                          "d=128, rotary 128, unaligned starts" % ("Q8_0" if q8 else "bf16"),
-                bound="hbm", algorithmic_bytes=algo, tokens=total, ms=ms, wall_ms=wall,
-                kernel_ms=kms, launches=int(facts.kernel_launches), dominant_kernel=kernel)
+                bound="hbm", algorithmic_bytes=algo, tokens=total,
+                launches=int(facts.kernel_launches), kernels=kernels, **timed)
 
 
 def copy_reference(backend, steps):
@@ -315,48 +356,66 @@ SEEDS = {"decode1": 1, "prefill2": 2, "paged3": 3, "paged4": 4, "mla5": 5, "appe
          "append_q8_0": 7}
 
 
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+
+
+def measured_traffic(name, kernel):
+    """HBM bytes per launch of `kernel` in workload `name`, from the committed counter summary
+    (rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs, each scaled by what the same counter
+    reads for a device copy of known size).  Not measured in this process: None when the file
+    has no entry for this kernel."""
+    try:
+        with open(TRAFFIC_FILE, encoding="utf-8") as stream:
+            table = json.load(stream)
+    except (OSError, ValueError):
+        return None
+    entry = table.get("workloads", {}).get(name, {}).get(kernel)
+    return None if entry is None else int(entry["hbm_bytes"])
+
+
 def roofline(result):
-    """Roofline record of the dominant kernel: algorithmic bytes (or flops) of one launch
-    over that kernel's own mean duration.  `step` repeats the figure for the whole step
-    (every launch of the operator), which is what `value` reports."""
-    seconds = result["kernel_ms"] * 1e-3
+    """Roofline record of the dominant kernel.  `achieved` is the algorithmic bytes (or flops)
+    of one launch over that kernel's own mean duration and `frac` (= `kernel_frac`) its share
+    of the published peak.  `step_achieved` / `step_frac` are the same quantity over the whole
+    step, every launch and the gaps between them included: that is what `value` reports.  Both
+    are as measured; the event pair around a single launch costs a few microseconds, so for a
+    step of one short kernel the per-launch figure can come out longer than the step."""
+    kernel = result["kernels"][0]
+    if kernel not in result["kernel_ms"]:
+        sys.exit("bench.py: kernel %s was not launched by workload %s" % (kernel, result["name"]))
+    seconds = result["kernel_ms"][kernel] * 1e-3
     step_seconds = result["ms"] * 1e-3
     if result["bound"] == "hbm":
-        achieved = result["algorithmic_bytes"] / seconds / 1e9
-        return dict(bound="hbm", achieved=achieved, peak=HBM_PEAK_GBS, unit="GB/s",
-                    frac=achieved / HBM_PEAK_GBS, traffic=TRAFFIC.get(result["name"]),
-                    kernel=result["dominant_kernel"], kernel_us=result["kernel_ms"] * 1e3,
-                    step=result["algorithmic_bytes"] / step_seconds / 1e9)
-    achieved = result["flops"] / seconds / 1e12
-    return dict(bound="mfma", achieved=achieved, peak=MFMA_BF16_PEAK_TFLOPS, unit="TFLOP/s",
-                frac=achieved / MFMA_BF16_PEAK_TFLOPS, traffic=TRAFFIC.get(result["name"]),
-                kernel=result["dominant_kernel"], kernel_us=result["kernel_ms"] * 1e3,
-                step=result["flops"] / step_seconds / 1e12)
+        work, scale, peak, unit = result["algorithmic_bytes"], 1e9, HBM_PEAK_GBS, "GB/s"
+    else:
+        work, scale, peak, unit = result["flops"], 1e12, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s"
+    achieved, step_achieved = work / seconds / scale, work / step_seconds / scale
+    return dict(bound=result["bound"], achieved=achieved, peak=peak, unit=unit, frac=achieved / peak,
+                traffic=measured_traffic(result["name"], kernel),
+                traffic_source="profiles/hbm_traffic.json (rocprofv3 --pmc, not this run)",
+                kernel=kernel, kernel_us=seconds * 1e6, kernel_frac=achieved / peak,
+                step_us=step_seconds * 1e6, step_achieved=step_achieved,
+                step_frac=step_achieved / peak,
+                kernels_us={k: v * 1e3 for k, v in result["kernel_ms"].items()})
 
 
-# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# runs (profiles/), scaled by the same counters on a copy kernel of known size; None where
-# no such run is committed.
-TRAFFIC = {"paged3": 1033352906, "paged4": 1512941054, "decode1": 18116274,
-           "prefill2": 50570700, "mla5": 204069246, "append_bf16": 303927100,
-           "append_q8_0": 239929618}
-
-
-def repeat_for(seconds, call):
-    """Calls `call` until `seconds` of wall time have passed; returns (runs, mean seconds)."""
-    runs, t0 = 0, time.perf_counter()
+def repeat_for(seconds, call, least=3):
+    """Calls `call` at least `least` times and until `seconds` of wall time have passed;
+    returns (runs, median seconds of one run, total seconds)."""
+    durations, t0 = [], time.perf_counter()
     while True:
+        c0 = time.perf_counter()
         rc = call()
+        durations.append(time.perf_counter() - c0)
         assert rc == 0
-        runs += 1
-        dt = time.perf_counter() - t0
-        if dt >= seconds:
-            return runs, dt / runs
+        if len(durations) >= least and time.perf_counter() - t0 >= seconds:
+            return len(durations), float(np.median(durations)), time.perf_counter() - t0
 
 
 def cpu_baseline(name, budget=6.0):
     """The oracle (a port of the reference CPU operator, all host threads) timed on a bounded
-    sample of the same workload: the sample is repeated for about `budget` seconds."""
+    sample of the same workload: the sample is repeated at least three times and for about `budget` seconds, and the median run
+    is reported."""
     from oracle_binding import Oracle
     oracle = Oracle()
     rng = np.random.default_rng(SEEDS[name])
@@ -373,29 +432,29 @@ def cpu_baseline(name, budget=6.0):
         if q8:
             k = oracle.q8_0_encode_rows(oracle.bf16_decode(k))
             v = oracle.q8_0_encode_rows(oracle.bf16_decode(v))
-        runs, dt = repeat_for(budget, lambda: oracle.paged_decode(q, k, v, table, contexts, hkv,
+        runs, dt, spent = repeat_for(budget, lambda: oracle.paged_decode(q, k, v, table, contexts, hkv,
                                                                   page, q8=q8)[0])
         per_token = 2 * hkv * (136 if q8 else 256)
         return dict(value=int(contexts.sum()) * per_token / dt / 1e9, unit="GB/s", cores=threads,
-                    kind="port", sample="4 sessions x 8192 tokens of the same shape, mean of "
-                                        "%d runs (%.1f s)" % (runs, runs * dt))
+                    kind="port", sample="4 sessions x 8192 tokens of the same shape, median of "
+                                        "%d runs (%.1f s)" % (runs, spent))
     if name == "decode1":
         q = bf16_bits(rng.standard_normal((1, 32, 128), dtype=np.float32))
         k = bf16_bits(rng.standard_normal((4096, 8, 128), dtype=np.float32))
         v = bf16_bits(rng.standard_normal((4096, 8, 128), dtype=np.float32))
-        runs, dt = repeat_for(budget / 2, lambda: oracle.gqa_bf16(q, k, v, query_start=4095)[0])
+        runs, dt, spent = repeat_for(budget / 2, lambda: oracle.gqa_bf16(q, k, v, query_start=4095)[0])
         return dict(value=(2 * 4096 * 8 * 128 * 2) / dt / 1e9, unit="GB/s", cores=threads,
-                    kind="port", sample="the full workload, mean of %d runs (%.1f s)" %
-                                        (runs, runs * dt))
+                    kind="port", sample="the full workload, median of %d runs (%.1f s)" %
+                                        (runs, spent))
     if name == "prefill2":
         t, hq, hkv, d = 1024, 40, 8, 128
         q = bf16_bits(rng.standard_normal((t, hq, d), dtype=np.float32))
         k = bf16_bits(rng.standard_normal((t, hkv, d), dtype=np.float32))
         v = bf16_bits(rng.standard_normal((t, hkv, d), dtype=np.float32))
-        runs, dt = repeat_for(budget, lambda: oracle.gqa_bf16(q, k, v, query_start=0)[0])
+        runs, dt, spent = repeat_for(budget, lambda: oracle.gqa_bf16(q, k, v, query_start=0)[0])
         return dict(value=4 * d * hq * t * (t + 1) // 2 / dt / 1e12, unit="TFLOP/s", cores=threads,
-                    kind="port", sample="the first 1024 tokens of the same shape, mean of %d runs "
-                                        "(%.1f s)" % (runs, runs * dt))
+                    kind="port", sample="the first 1024 tokens of the same shape, median of %d runs "
+                                        "(%.1f s)" % (runs, spent))
     if name == "mla5":
         batch, heads, kd, vd, page, ctx = 2, 128, 576, 512, 64, 4096
         pages = batch * ctx // page
@@ -403,11 +462,11 @@ def cpu_baseline(name, budget=6.0):
         pool = bf16_bits(rng.standard_normal((pages, page, kd), dtype=np.float32))
         q = bf16_bits(rng.standard_normal((batch, heads, kd), dtype=np.float32))
         contexts = np.full(batch, ctx, np.int32)
-        runs, dt = repeat_for(budget, lambda: oracle.mla_decode(q, pool, table, contexts, vd,
+        runs, dt, spent = repeat_for(budget, lambda: oracle.mla_decode(q, pool, table, contexts, vd,
                                                                 page)[0])
         return dict(value=batch * ctx * kd * 2 / dt / 1e9, unit="GB/s", cores=threads, kind="port",
-                    sample="2 batch elements x 4096 tokens of the same shape, mean of %d runs "
-                           "(%.1f s)" % (runs, runs * dt))
+                    sample="2 batch elements x 4096 tokens of the same shape, median of %d runs "
+                           "(%.1f s)" % (runs, spent))
     return None
 
 
@@ -455,7 +514,7 @@ def main():
     cpu = {} if args.no_cpu else {n: cpu_baseline(n) for n in names if n in WORKLOADS}
     line = {
         "metric": METRIC,
-        "value": roof["step"],
+        "value": roof["step_achieved"],
         "unit": roof["unit"],
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": head["ms"],
@@ -464,19 +523,21 @@ def main():
         "config": {"workload": head["workload"], "name": head["name"],
                    "kernel_launches_per_step": head["launches"]},
         "roofline": roof,
+        "benchmark_record": head["record"],
         "cpu_baseline": cpu.get(headline),
         "device_probe": device_probe,
         # the metric has two halves; `value` carries the first (decode, HBM GB/s), this the
         # second (causal prefill, TFLOP/s), when that workload ran
         "prefill": ({"metric": "prefill attn TFLOPS (% MFMA peak)",
-                     "value": roofline(results["prefill2"])["step"], "unit": "TFLOP/s",
+                     "value": roofline(results["prefill2"])["step_achieved"], "unit": "TFLOP/s",
                      "ms_per_step": results["prefill2"]["ms"],
                      "config": {"workload": results["prefill2"]["workload"]},
                      "roofline": roofline(results["prefill2"]),
                      "cpu_baseline": cpu.get("prefill2")} if "prefill2" in results else None),
         "workloads": {n: dict(workload=r["workload"], ms_per_step=r["ms"],
-                              wall_ms_per_step=r["wall_ms"], value=roofline(r)["step"],
-                              unit=roofline(r)["unit"], roofline=roofline(r),
+                              wall_ms_per_step=r["wall_ms"],
+                              value=roofline(r)["step_achieved"], unit=roofline(r)["unit"],
+                              roofline=roofline(r), benchmark_record=r["record"],
                               cpu_baseline=cpu.get(n)) for n, r in results.items()},
     }
     print(json.dumps(line))
