@@ -364,7 +364,11 @@ class Backend:
     def mla_requirement(batch, heads, key_dim, value_dim, page_tokens, pool_pages, table_stride,
                         max_context, contract=B.NUMERIC_BF16_F32_ACCUMULATE, deterministic=1,
                         sliding_window=0, compressed_pool_pages=0, compressed_table_stride=0,
-                        max_compressed_tokens=0, compressed_selected_stride=0):
+                        max_compressed_tokens=0, compressed_selected_stride=0,
+                        output_inverse_rope=None, scale=0.0):
+        """output_inverse_rope: optional dict(rope_dimensions, theta[, scaling_factor,
+        original_context, beta_fast, beta_slow]) rotating the published rows back by the query
+        token's position; scale: softmax scale, 0 = 1 / sqrt(key_dim)."""
         r = B.MlaDecodeRequirement()
         r.batch, r.heads, r.key_dimension, r.value_dimension = batch, heads, key_dim, value_dim
         r.page_tokens, r.pool_pages, r.page_table_stride = page_tokens, pool_pages, table_stride
@@ -374,6 +378,9 @@ class Backend:
         r.compressed_page_table_stride = compressed_table_stride
         r.max_compressed_tokens = max_compressed_tokens
         r.compressed_selected_stride = compressed_selected_stride
+        for name, value in (output_inverse_rope or {}).items():
+            setattr(r.output_inverse_rope, name, value)
+        r.scale = scale
         return r
 
     def mla_decode_workspace_required(self, requirement):
@@ -384,9 +391,10 @@ class Backend:
         return out.value
 
     def mla_decode_execute(self, requirement, query, latent_pages, page_table, context, output,
-                           lse=None, sinks=None, compressed=None):
+                           lse=None, sinks=None, compressed=None, output_positions=None):
         """compressed: optional (pages, page table, row counts[, selected row lists]) device
-        tensors."""
+        tensors; output_positions: optional I64 [batch] query token positions for the output
+        rotation."""
         ops = self.rocm_attention_operations()
         if ops is None:
             raise YvexError(B.YVEX_ERR_UNSUPPORTED, "rocm_attention_operations", "not published")
@@ -396,6 +404,8 @@ class Backend:
                                      sinks.handle if sinks else None,
                                      *(x.handle for x in (compressed or (None, None, None))
                                        if x is not None))
+        if output_positions is not None:
+            request.output_positions = output_positions.handle
         facts, err = B.OperationFacts(), B.Error()
         _check(ops.mla_decode_execute(self.handle, C.byref(request), C.byref(facts),
                                       C.byref(err)), err)

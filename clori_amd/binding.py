@@ -143,13 +143,20 @@ class PagedDecodeRequest(C.Structure):
                 ("context_tokens", TensorP), ("output", TensorP), ("lse", TensorP)]
 
 
+class AttentionPosition(C.Structure):
+    """yvex_backend_attention_position (include/yvex/internal/backend.h:51-54)."""
+    _fields_ = [(n, ull) for n in ("theta", "scaling_factor", "original_context", "beta_fast",
+                                   "beta_slow", "rope_dimensions")]
+
+
 class MlaDecodeRequirement(C.Structure):
     _fields_ = [(n, ull) for n in ("batch", "heads", "key_dimension", "value_dimension",
                                    "page_tokens", "pool_pages", "page_table_stride",
                                    "max_context_tokens")] + [
         ("numeric_contract", C.c_int), ("deterministic", C.c_int), ("sliding_window", ull),
         ("compressed_pool_pages", ull), ("compressed_page_table_stride", ull),
-        ("max_compressed_tokens", ull), ("compressed_selected_stride", ull)]
+        ("max_compressed_tokens", ull), ("compressed_selected_stride", ull),
+        ("output_inverse_rope", AttentionPosition), ("scale", C.c_float)]
 
 
 class MlaDecodeRequest(C.Structure):
@@ -157,7 +164,8 @@ class MlaDecodeRequest(C.Structure):
                 ("latent_pages", TensorP), ("page_table", TensorP), ("context_tokens", TensorP),
                 ("output", TensorP), ("lse", TensorP), ("sinks", TensorP),
                 ("compressed_pages", TensorP), ("compressed_page_table", TensorP),
-                ("compressed_tokens", TensorP), ("compressed_selected", TensorP)]
+                ("compressed_tokens", TensorP), ("compressed_selected", TensorP),
+                ("output_positions", TensorP)]
 
 
 class KvAppendRequirement(C.Structure):

@@ -707,8 +707,51 @@ static int mla_validate(const yvex_rocm_mla_decode_requirement *r, const char *w
         return refuse(err, YVEX_ERR_UNSUPPORTED, where,
                       "ROCm MLA decode requires 128 heads, a 512+64 latent row, 64-token pages "
                       "and the deterministic bf16/fp32-accumulate contract");
+    if (r->output_inverse_rope.rope_dimensions) {
+        const yvex_backend_attention_position *position = &r->output_inverse_rope;
+        /* src/backend/cuda/kernels.cu:1006-1012: the same refusals as the reference's rotation */
+        if (position->theta <= 1ull ||
+            (position->original_context &&
+             (!position->scaling_factor || !position->beta_slow ||
+              position->beta_fast <= position->beta_slow)))
+            return refuse(err, YVEX_ERR_INVALID_ARG, where, "output rotation policy is invalid");
+        if ((position->rope_dimensions & 7ull) || position->rope_dimensions > r->value_dimension ||
+            position->rope_dimensions > 2ull * YVEX_ROCM_ROPE_PAIRS_MAX)
+            return refuse(err, YVEX_ERR_UNSUPPORTED, where,
+                          "ROCm MLA decode rotates at most 128 output lanes, in multiples of 8");
+    }
+    if (!(r->scale >= 0.0f) || !isfinite(r->scale))
+        return refuse(err, YVEX_ERR_INVALID_ARG, where, "softmax scale must be finite and not negative");
     yvex_error_clear(err);
     return YVEX_OK;
+}
+
+/* Frequency of rotary pair `pair` (src/graph/numeric.c:877-917): theta^(-2 pair / dims), and
+ * with a YaRN policy the blend between that and the same divided by the scaling factor, by a
+ * linear ramp between the two corner pairs that beta_fast and beta_slow set. */
+static double mla_rope_frequency(const yvex_backend_attention_position *position,
+                                 unsigned long long pair)
+{
+    static const double pi = 3.14159265358979323846264338327950288;
+    const double dims = (double)position->rope_dimensions;
+    double frequency = 1.0 / pow((double)position->theta, (double)(pair * 2ull) / dims);
+    if (position->original_context && position->scaling_factor) {
+        const double denominator = 2.0 * log((double)position->theta);
+        double low = floor(dims * log((double)position->original_context /
+                                      ((double)position->beta_fast * 2.0 * pi)) / denominator);
+        double high = ceil(dims * log((double)position->original_context /
+                                      ((double)position->beta_slow * 2.0 * pi)) / denominator);
+        double ramp, smooth;
+        if (low < 0.0) low = 0.0;
+        if (high > dims - 1.0) high = dims - 1.0;
+        if (low == high) high += 0.001;
+        ramp = ((double)pair - low) / (high - low);
+        if (ramp < 0.0) ramp = 0.0;
+        if (ramp > 1.0) ramp = 1.0;
+        smooth = 1.0 - ramp;
+        frequency = frequency / (double)position->scaling_factor * (1.0 - smooth) + frequency * smooth;
+    }
+    return frequency;
 }
 
 /* Chunks are a function of the request geometry only: about one workgroup per compute
@@ -834,6 +877,9 @@ static int rocm_mla_decode_execute(yvex_backend *backend,
                  r->batch * r->heads * r->value_dimension, 0) ||
         (request->lse && !view_ok(backend, request->lse, YVEX_DTYPE_F32, r->batch * r->heads, 0)) ||
         (request->sinks && !view_ok(backend, request->sinks, YVEX_DTYPE_F32, r->heads, 1)) ||
+        (request->output_positions &&
+         (!r->output_inverse_rope.rope_dimensions ||
+          !view_ok(backend, request->output_positions, YVEX_DTYPE_I64, r->batch, 1))) ||
         (r->max_compressed_tokens &&
          (!request->compressed_pages || !request->compressed_page_table ||
           !request->compressed_tokens ||
@@ -882,7 +928,8 @@ static int rocm_mla_decode_execute(yvex_backend *backend,
     kp.window = (uint32_t)r->sliding_window;
     kp.slot_stride = (uint32_t)(max_chunks + extra_max_chunks);
     /* src/graph/core.c:604: scale = 1/sqrt(head_dimension), here over the 576-lane key */
-    kp.scale_log2 = (float)(1.4426950408889634 / sqrt((double)r->key_dimension));
+    kp.scale_log2 = (float)(1.4426950408889634 *
+                            (r->scale > 0.0f ? (double)r->scale : 1.0 / sqrt((double)r->key_dimension)));
     rc = yvex_rocm_launch(backend, YVEX_ROCM_FN_MLA_DECODE_BF16, variant, (unsigned int)max_chunks,
                           (unsigned int)r->batch, 1u, 256u, 0u, &kp, where, err);
     if (rc == YVEX_OK && extra_max_chunks) {
@@ -947,12 +994,22 @@ static int rocm_mla_decode_execute(yvex_backend *backend,
         mp.sinks = request->sinks ? (const float *)request->sinks->data : NULL;
         mp.window = kp.window;
         mp.window_align = ROCM_MLA_TILE_TOKENS;
+        if (r->output_inverse_rope.rope_dimensions) {
+            unsigned long long pair;
+            mp.rope_dims = (uint32_t)r->output_inverse_rope.rope_dimensions;
+            mp.positions = request->output_positions
+                               ? (const int64_t *)request->output_positions->data : NULL;
+            for (pair = 0ull; pair < r->output_inverse_rope.rope_dimensions / 2ull; ++pair)
+                mp.rope_frequency[pair] = mla_rope_frequency(&r->output_inverse_rope, pair);
+        }
         if (extra_max_chunks) {
             mp.extra_context = (const int32_t *)request->compressed_tokens->data;
             mp.extra_chunk_tokens = (uint32_t)extra_chunk;
             mp.extra_max_chunks = (uint32_t)extra_max_chunks;
         }
-        rc = yvex_rocm_launch(backend, YVEX_ROCM_FN_DECODE_MERGE, variant,
+        rc = yvex_rocm_launch(backend,
+                              mp.rope_dims ? YVEX_ROCM_FN_DECODE_MERGE_ROPE : YVEX_ROCM_FN_DECODE_MERGE,
+                              variant,
                               (unsigned int)((r->heads + 3ull) / 4ull), (unsigned int)r->batch, 1u,
                               256u, 0u, &mp, where, err);
     }

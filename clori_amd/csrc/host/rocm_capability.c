@@ -38,6 +38,8 @@ static const rocm_kernel_binding rocm_kernel_bindings[] = {
      YVEX_ROCM_FN_DECODE_PAGED_BF16},
     {"yvex_rocm_decode_merge", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_PAGED_BF16,
      YVEX_ROCM_FN_DECODE_MERGE},
+    {"yvex_rocm_decode_merge_rope", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_MLA_BF16,
+     YVEX_ROCM_FN_DECODE_MERGE_ROPE},
     {"yvex_rocm_decode_finish", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_PAGED_BF16,
      YVEX_ROCM_FN_DECODE_FINISH},
     {"yvex_rocm_decode_rows_bf16", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_BF16,

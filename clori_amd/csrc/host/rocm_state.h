@@ -16,6 +16,7 @@ typedef enum {
     YVEX_ROCM_FN_DECODE_PAGED_BF16,
     YVEX_ROCM_FN_DECODE_ROWS_BF16,
     YVEX_ROCM_FN_DECODE_MERGE,
+    YVEX_ROCM_FN_DECODE_MERGE_ROPE,
     YVEX_ROCM_FN_DECODE_FINISH,
     YVEX_ROCM_FN_DECODE_PAGED_Q8_0,
     YVEX_ROCM_FN_DECODE_PAGED_BF16_MERGED,

@@ -83,6 +83,8 @@ typedef struct {
     const uint16_t *gate; /* optional bf16 [sessions][query_heads][head_dim] sigmoid output gate */
 } yvex_rocm_decode_params;
 
+#define YVEX_ROCM_ROPE_PAIRS_MAX 64
+
 /* Log-sum-exp merge of per-chunk partials (used by the MLA path).  With a sliding window the
  * chunks start at the first visible token rounded down to window_align, as in the producer.  The accumulators are
  * unnormalised and stored as bf16: they are 44 % of that path's HBM traffic in fp32. */
@@ -101,6 +103,11 @@ typedef struct {
      * of each batch element; extra_context NULL: none */
     const int32_t *extra_context;
     uint32_t extra_chunk_tokens, extra_max_chunks;
+    /* inverse rotation of the last rope_dims lanes of each published row (0: none): angle of
+     * pair i = position * rope_frequency[i]; positions NULL: context - 1 */
+    const int64_t *positions;
+    uint32_t rope_dims, reserved;
+    double rope_frequency[YVEX_ROCM_ROPE_PAIRS_MAX];
 } yvex_rocm_decode_merge_params;
 
 /* Causal / full GQA prefill on bf16 token-major tensors.  The grid is one-dimensional:

@@ -767,8 +767,11 @@ yvex_rocm_decode_finish(const yvex_rocm_decode_params p)
 // Log-sum-exp merge of the chunk partials of one (session, query head): one wave per head,
 // eight output dims per lane (one 16-byte load of bf16 partials per chunk), four heads per
 // workgroup.  grid = (ceil(query_heads / 4), sessions), block = 256; head_dim = 512.
-extern "C" __global__ void __launch_bounds__(256)
-yvex_rocm_decode_merge(const yvex_rocm_decode_merge_params p)
+// kRope: the build that also turns the rope lanes of the published row back (its double
+// precision sine and cosine double the register use, so rows without a rotation keep their
+// own build).
+template <bool kRope>
+__device__ __forceinline__ void decode_merge_rows(const yvex_rocm_decode_merge_params &p)
 {
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t head = blockIdx.x * 4u + (threadIdx.x >> 6), session = blockIdx.y;
@@ -838,11 +841,27 @@ yvex_rocm_decode_merge(const yvex_rocm_decode_merge_params p)
         top = m_new;
     }
     const float inv = 1.0f / total;
+    // Inverse rotation of the rope lanes (src/graph/core.c:499-507): the row is rounded to
+    // bf16, its last rope_dims lanes are turned back by the token position in adjacent pairs,
+    // in double as the reference does it (src/graph/numeric.c:935-947), and rounded again.  A
+    // lane's eight dims hold four whole pairs; rope_dims and head_dim are multiples of 8.
+    const uint32_t rope_start = p.head_dim - p.rope_dims;
+    const bool turn = kRope && p.rope_dims != 0u && lane * 8u >= rope_start;
+    const double position =
+        turn ? (p.positions ? (double)(uint64_t)p.positions[session] : (double)(ctx - 1u)) : 0.0;
     u32x4 out;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        const float a = acc[2 * i] * inv, b = acc[2 * i + 1] * inv;
+        float a = acc[2 * i] * inv, b = acc[2 * i + 1] * inv;
         bad |= !(isfinite(a) && isfinite(b));
+        if (kRope && turn) {
+            const double angle = position * p.rope_frequency[(lane * 8u - rope_start) / 2u + (uint32_t)i];
+            const double c = cos(angle), s = -sin(angle);
+            const double x = (double)bf16_to_f32(bf16_bits(a)), y = (double)bf16_to_f32(bf16_bits(b));
+            a = (float)(x * c - y * s);
+            b = (float)(x * s + y * c);
+            bad |= !(isfinite(a) && isfinite(b));
+        }
         out[i] = (uint32_t)bf16_bits(a) | ((uint32_t)bf16_bits(b) << 16);
     }
     if (bad) flag(p.status, YVEX_ROCM_DEVICE_NUMERIC);
@@ -850,4 +869,16 @@ yvex_rocm_decode_merge(const yvex_rocm_decode_merge_params p)
                                lane * 8u) = out;
     if (p.lse && lane == 0u)
         p.lse[(uint64_t)session * p.query_heads + head] = (top + fast_log2(total)) * YVEX_LN2;
+}
+
+extern "C" __global__ void __launch_bounds__(256)
+yvex_rocm_decode_merge(const yvex_rocm_decode_merge_params p)
+{
+    decode_merge_rows<false>(p);
+}
+
+extern "C" __global__ void __launch_bounds__(256)
+yvex_rocm_decode_merge_rope(const yvex_rocm_decode_merge_params p)
+{
+    decode_merge_rows<true>(p);
 }

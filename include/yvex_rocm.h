@@ -492,6 +492,13 @@ typedef struct yvex_rocm_paged_decode_request {
  * Pool: BF16 [pool_pages][page_tokens][key_dimension] (token-major, page_tokens 64).
  * query BF16 [batch][heads][key_dimension]; output BF16 [batch][heads][value_dimension].
  */
+/* Rotary position policy of an attention layer: the fields the rotation reads
+ * (include/yvex/internal/backend.h:51-54, same names and order). */
+typedef struct {
+    unsigned long long theta, scaling_factor, original_context;
+    unsigned long long beta_fast, beta_slow, rope_dimensions;
+} yvex_backend_attention_position;
+
 typedef struct yvex_rocm_mla_decode_requirement {
     unsigned long long batch, heads, key_dimension, value_dimension;
     unsigned long long page_tokens, pool_pages, page_table_stride, max_context_tokens;
@@ -510,6 +517,17 @@ typedef struct yvex_rocm_mla_decode_requirement {
      * compressed rows are the entries of a per-session index list, in list order, instead of
      * a prefix.  compressed_selected_stride is the list capacity; 0: the prefix class. */
     unsigned long long compressed_selected_stride;
+    /* Inverse rotation of the published rows (src/graph/core.c:499-507,
+     * src/backend/cuda/attention.c:1424-1429): each head's row is rounded to bf16, its LAST
+     * rope_dimensions lanes are rotated back by the query token's position, adjacent pairs
+     * (2i, 2i+1), angle = position * frequency(i) with the YaRN ramp of
+     * src/graph/numeric.c:877-917 when original_context and scaling_factor are set, and the
+     * row is rounded again.  rope_dimensions = 0: rows are published as they are.  Admitted:
+     * rope_dimensions a multiple of 8, at most 128 and at most value_dimension; theta > 1;
+     * with original_context set, scaling_factor >= 1 and beta_fast > beta_slow >= 1. */
+    yvex_backend_attention_position output_inverse_rope;
+    /* Softmax scale; 0 selects 1 / sqrt(key_dimension) (src/graph/core.c:604). */
+    float scale;
 } yvex_rocm_mla_decode_requirement;
 
 typedef struct yvex_rocm_mla_decode_request {
@@ -529,6 +547,10 @@ typedef struct yvex_rocm_mla_decode_request {
      * compressed rows (positions in the session's compressed sequence, below
      * max_compressed_tokens); compressed_tokens then holds the number of list entries. */
     const yvex_device_tensor *compressed_selected;
+    /* With output_inverse_rope: optional I64 [batch] absolute position of each query token
+     * (token_position + token of src/graph/core.c:475); NULL: context_tokens[b] - 1, the
+     * position of the newest row of a history that starts at 0. */
+    const yvex_device_tensor *output_positions;
 } yvex_rocm_mla_decode_request;
 
 /* KV page writer (no reference counterpart as one operation: it is the rotary step of

@@ -11,8 +11,9 @@
  *
  * What the reference does after the softmax belongs to its model family and is kept as it
  * is: the rows are rounded to bf16, the last rope_dims lanes are rotated back by the
- * token's position, and the row is rounded again (src/graph/core.c:499-507).  The caller
- * asks for rope_dims = 2, so every lane but the last two is bf16(softmax row).
+ * token's position, and the row is rounded again (src/graph/core.c:499-507).  A caller
+ * that asks for rope_dims = 2 gets bf16(softmax row) on every lane but the last two; the
+ * rotation's own policy fields (theta and the YaRN scaling) are passed through.
  */
 #include <string.h>
 
@@ -40,6 +41,9 @@ YVREF_EXPORT int yvref_attention_reduce(const float *query, const float *local,
                                         unsigned long long compression_ratio,
                                         unsigned int attention_class, unsigned long long position,
                                         unsigned long long rope_dims, unsigned long long theta,
+                                        unsigned long long scaling_factor,
+                                        unsigned long long original_context,
+                                        unsigned long long beta_fast, unsigned long long beta_slow,
                                         float *out)
 {
     yvex_attention_layer_plan layer;
@@ -61,6 +65,10 @@ YVREF_EXPORT int yvref_attention_reduce(const float *query, const float *local,
     layer.rope_head_dimension = rope_dims;
     layer.position.rope_dimension = rope_dims;
     layer.position.theta = theta;
+    layer.position.scaling_factor = scaling_factor;
+    layer.position.original_context = original_context;
+    layer.position.beta_fast = beta_fast;
+    layer.position.beta_slow = beta_slow;
     history.token_count = local_count - 1ull;
     history.local_tail_count = local_count - 1ull;
     history.local_kv = local;

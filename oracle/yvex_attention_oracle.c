@@ -495,6 +495,76 @@ int yvo_paged_decode_q8_0(const uint16_t *q, const unsigned char *k_pool,
                         page_tokens, pool_pages, table_stride, threads);
 }
 
+/* ------------------------------------------------ rotary positions ---- */
+
+/* src/graph/numeric.c:877-917 */
+double yvo_yarn_frequency(const yvo_position_policy *policy, uint64_t pair, uint64_t rope_dims)
+{
+    static const double pi = 3.14159265358979323846264338327950288;
+    double frequency;
+    if (!policy || rope_dims < 2u || policy->theta <= 1u) return 0.0;
+    frequency = 1.0 / pow((double)policy->theta, (double)(pair * 2u) / (double)rope_dims);
+    if (policy->original_context && policy->scaling_factor) {
+        const double denominator = 2.0 * log((double)policy->theta);
+        double low = floor((double)rope_dims *
+                           log((double)policy->original_context /
+                               ((double)policy->beta_fast * 2.0 * pi)) / denominator);
+        double high = ceil((double)rope_dims *
+                           log((double)policy->original_context /
+                               ((double)policy->beta_slow * 2.0 * pi)) / denominator);
+        double ramp, smooth;
+        if (low < 0.0) low = 0.0;
+        if (high > (double)rope_dims - 1.0) high = (double)rope_dims - 1.0;
+        if (low == high) high += 0.001;
+        ramp = ((double)pair - low) / (high - low);
+        if (ramp < 0.0) ramp = 0.0;
+        if (ramp > 1.0) ramp = 1.0;
+        smooth = 1.0 - ramp;
+        frequency = frequency / (double)policy->scaling_factor * (1.0 - smooth) + frequency * smooth;
+    }
+    return frequency;
+}
+
+/* src/graph/numeric.c:919-949 */
+int yvo_rope_apply(float *values, uint64_t count, uint64_t rope_dims, uint64_t position,
+                   const yvo_position_policy *policy, int inverse)
+{
+    uint64_t start, i;
+    if (!values || !count || rope_dims < 2u || rope_dims > count || !policy || policy->theta <= 1u)
+        return YVO_ERR_INVALID_ARG;
+    if (rope_dims & 1u) rope_dims--;
+    start = count - rope_dims;
+    for (i = 0; i < rope_dims; i += 2u) {
+        const double angle = (double)position * yvo_yarn_frequency(policy, i / 2u, rope_dims);
+        const double c = cos(angle), s = inverse ? -sin(angle) : sin(angle);
+        const double x = values[start + i], y = values[start + i + 1u];
+        if (!isfinite(x) || !isfinite(y) || !isfinite(c) || !isfinite(s)) return YVO_ERR_FORMAT;
+        values[start + i] = (float)(x * c - y * s);
+        values[start + i + 1u] = (float)(x * s + y * c);
+    }
+    return YVO_OK;
+}
+
+/* src/graph/core.c:499-507 */
+int yvo_reduce_output_finish(float *rows, uint64_t heads, uint64_t dim, uint64_t position,
+                             const yvo_position_policy *policy)
+{
+    uint64_t head, lane;
+    if (!rows || !heads || !dim || !policy) return YVO_ERR_INVALID_ARG;
+    for (head = 0; head < heads; ++head) {
+        float *row = rows + head * dim;
+        int rc;
+        for (lane = 0; lane < dim; ++lane) row[lane] = yvo_bf16_decode(yvo_bf16_encode(row[lane]));
+        rc = yvo_rope_apply(row, dim, policy->rope_dimensions, position, policy, 1);
+        if (rc != YVO_OK) return rc;
+        for (lane = 0; lane < dim; ++lane) {
+            if (!isfinite(row[lane])) return YVO_ERR_FORMAT;
+            row[lane] = yvo_bf16_decode(yvo_bf16_encode(row[lane]));
+        }
+    }
+    return YVO_OK;
+}
+
 /* ------------------------------------------------ shared-KV (MLA) head ---- */
 
 /* src/graph/core.c:361-388 (row visit) and :471-508 (head): the sink logit seeds

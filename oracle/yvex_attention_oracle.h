@@ -31,7 +31,13 @@
  *       lane it does not rotate and on the other two after the same rotation;
  *       committed outputs of that reduce (tests/golden); the sink-free path
  *       equals a sink that underflows, bit for bit
- *   yvo_rotary_half_bf16             pinned: known-answer case
+ *   yvo_yarn_frequency, yvo_rope_apply, yvo_reduce_output_finish
+       pinned: the reference's own reduce (oracle/_ref/libyvex_ref_reduce.so) run with
+       64 rope lanes, with and without the YaRN ramp, bit for bit on every lane of the
+       published row; committed outputs of that reduce (tests/golden); forward then
+       inverse rotation returns the row within float rounding; position 0 is the
+       identity; pair 0 has frequency 1
+   yvo_rotary_half_bf16             pinned: known-answer case
  *       (tests/unit/cuda/quant_qtype.c:1988-2061), identity, quarter turn,
  *       float64 rotation within bf16 rounding
  *   yvo_sigmoid_gate_bf16            pinned: known-answer case
@@ -197,6 +203,25 @@ int yvo_mla_decode_bf16(const uint16_t *q, const uint16_t *pool,
  */
 int yvo_lse_merge(const float *part_out, const double *part_lse, uint64_t parts,
                   uint64_t dim, float *out, double *lse);
+
+/*
+ * Rotary position policy (include/yvex/internal/backend.h:51-54, the fields the rotation
+ * reads) and the rotation itself (src/graph/numeric.c:877-949): the LAST rope_dims lanes of
+ * a row of `count` lanes, adjacent pairs (2i, 2i+1), angle = position * frequency(i) with
+ * the YaRN ramp when original_context and scaling_factor are set; all in double, each
+ * result rounded to float.  inverse rotates by the negative angle.
+ */
+typedef struct {
+    uint64_t theta, scaling_factor, original_context, beta_fast, beta_slow, rope_dimensions;
+} yvo_position_policy;
+double yvo_yarn_frequency(const yvo_position_policy *policy, uint64_t pair, uint64_t rope_dims);
+int yvo_rope_apply(float *values, uint64_t count, uint64_t rope_dims, uint64_t position,
+                   const yvo_position_policy *policy, int inverse);
+/* What the shared-KV reduce does to each head's row after the softmax
+ * (src/graph/core.c:499-507): round to bf16, rotate the rope lanes back by the token's
+ * position, round again.  rows is [heads][dim] float, in place. */
+int yvo_reduce_output_finish(float *rows, uint64_t heads, uint64_t dim, uint64_t position,
+                             const yvo_position_policy *policy);
 
 /*
  * Rotate-half position encoding on packed bf16 [tokens][heads][head_dim] vectors in

@@ -41,6 +41,19 @@ REDUCE_CASES = [
     ("reduce-compressed-700", 2, 128, 700, 7, 4, 128),
 ]
 REDUCE_RATIO = 128
+# the same reduce with a real rope tail: (name, attention_class, window, context, stored, heads,
+# dim, position policy).  Policy = rope lanes, theta and the YaRN fields of the reference's
+# position policy; the second one is the DeepSeek-style long-context scaling
+# (factor 40 over an original context of 4096, beta 32 / 1).
+ROPE_PLAIN = dict(rope_dims=64, theta=10000)
+ROPE_YARN = dict(rope_dims=64, theta=10000, scaling_factor=40, original_context=4096, beta_fast=32,
+                 beta_slow=1)
+REDUCE_ROPE_CASES = [
+    ("reduce-rope-plain", 0, 1 << 20, 300, 0, 4, 128, ROPE_PLAIN),
+    ("reduce-rope-yarn", 0, 1 << 20, 300, 0, 4, 128, ROPE_YARN),
+    ("reduce-rope-yarn-compressed", 2, 64, 700, 7, 4, 128, ROPE_YARN),
+    ("reduce-rope-all-lanes", 0, 16, 90, 0, 2, 64, dict(rope_dims=64, theta=500000)),
+]
 
 
 def reduce_inputs(heads, dim, context, stored):
@@ -113,6 +126,14 @@ def main():
                                  np.arange(stored) * REDUCE_RATIO, sinks, window,
                                  REDUCE_RATIO if attention_class == 2 else 0, attention_class,
                                  context - 1)
+        assert rc == 0, (name, rc)
+        out[name + "/out"] = o
+    for name, attention_class, window, context, stored, heads, dim, policy in REDUCE_ROPE_CASES:
+        q, local, compressed, sinks = reduce_inputs(heads, dim, context, stored)
+        rc, o = reference_reduce(reduce, q, local, np.arange(context), compressed,
+                                 np.arange(stored) * REDUCE_RATIO, sinks, window,
+                                 REDUCE_RATIO if attention_class == 2 else 0, attention_class,
+                                 context - 1, **policy)
         assert rc == 0, (name, rc)
         out[name + "/out"] = o
     np.savez_compressed(os.path.join(HERE, "reference_attention.npz"), **out)

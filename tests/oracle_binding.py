@@ -22,6 +22,12 @@ u8p = C.POINTER(C.c_ubyte)
 i32p = C.POINTER(C.c_int32)
 
 
+class PositionPolicy(C.Structure):
+    """yvo_position_policy (the fields of include/yvex/internal/backend.h:51-54)."""
+    _fields_ = [("theta", u64), ("scaling_factor", u64), ("original_context", u64),
+                ("beta_fast", u64), ("beta_slow", u64), ("rope_dimensions", u64)]
+
+
 def _ptr(a, typ):
     if a is None:
         return C.cast(None, typ)
@@ -60,6 +66,10 @@ def load_oracle():
     lib.yvo_rotary_half_bf16.argtypes = [u16p, f32p, f32p] + [u64] * 4
     lib.yvo_sigmoid_gate_bf16.argtypes = [f32p, f32p, u64, f32p]
     lib.yvo_mla_decode_bf16.argtypes = [u16p, u16p, i32p, i32p, f32p, u16p, f64p] + [u64] * 7 + [f32p, u64, u16p, i32p, i32p, u64, u64, i32p, u64, C.c_int]
+    lib.yvo_yarn_frequency.restype = C.c_double
+    lib.yvo_yarn_frequency.argtypes = [C.POINTER(PositionPolicy), u64, u64]
+    lib.yvo_rope_apply.argtypes = [f32p, u64, u64, u64, C.POINTER(PositionPolicy), C.c_int]
+    lib.yvo_reduce_output_finish.argtypes = [f32p, u64, u64, u64, C.POINTER(PositionPolicy)]
     lib.yvo_lse_merge.argtypes = [f32p, f64p, u64, u64, f32p, f64p]
     return lib
 
@@ -74,13 +84,14 @@ def load_reference_reduce():
     lib = C.CDLL(REF_REDUCE_SO)
     u64p = C.POINTER(C.c_ulonglong)
     lib.yvref_attention_reduce.argtypes = [f32p, f32p, u64p, u64, f32p, u64p, u64, f32p, u64, u64,
-                                           u64, u64, C.c_uint, u64, u64, u64, f32p]
+                                           u64, u64, C.c_uint, u64, u64, u64, u64, u64, u64, u64, f32p]
     return lib
 
 
 def reference_reduce(lib, query, local, local_positions, compressed, compressed_positions, sinks,
                      sliding_window, compression_ratio, attention_class, position,
-                     rope_dims=2, theta=10000):
+                     rope_dims=2, theta=10000, scaling_factor=0, original_context=0, beta_fast=0,
+                     beta_slow=0):
     """One query token through the reference reduce; returns (status, out [heads][dim])."""
     query = np.ascontiguousarray(query, dtype=np.float32)
     local = np.ascontiguousarray(local, dtype=np.float32)
@@ -95,7 +106,8 @@ def reference_reduce(lib, query, local, local_positions, compressed, compressed_
         _ptr(compressed, f32p) if len(compressed) else None,
         _ptr(compressed_positions, u64p) if len(compressed) else None, compressed.shape[0],
         _ptr(sinks, f32p), query.shape[0], query.shape[1], sliding_window, compression_ratio,
-        attention_class, position, rope_dims, theta, _ptr(out, f32p))
+        attention_class, position, rope_dims, theta, scaling_factor, original_context, beta_fast,
+        beta_slow, _ptr(out, f32p))
     return rc, out
 
 
@@ -286,6 +298,24 @@ class Oracle:
                                           _ptr(sinks, f32p) if sinks is not None else None,
                                           sliding_window, *extra, threads or self.threads)
         return rc, out, outb, lse
+
+    @staticmethod
+    def position_policy(rope_dims, theta=10000, scaling_factor=0, original_context=0, beta_fast=0,
+                        beta_slow=0):
+        return PositionPolicy(theta, scaling_factor, original_context, beta_fast, beta_slow, rope_dims)
+
+    def rope_apply(self, row, position, policy, inverse=False):
+        out = np.ascontiguousarray(row, dtype=np.float32).copy()
+        rc = self.lib.yvo_rope_apply(_ptr(out, f32p), out.size, policy.rope_dimensions, position,
+                                     C.byref(policy), int(inverse))
+        return rc, out
+
+    def reduce_output_finish(self, rows, position, policy):
+        """rows float [heads][dim] -> bf16 round, inverse rotation of the rope lanes, bf16 round."""
+        out = np.ascontiguousarray(rows, dtype=np.float32).copy()
+        rc = self.lib.yvo_reduce_output_finish(_ptr(out, f32p), out.shape[0], out.shape[1], position,
+                                               C.byref(policy))
+        return rc, out
 
     def lse_merge(self, part_out, part_lse):
         part_out = np.ascontiguousarray(part_out, dtype=np.float32)

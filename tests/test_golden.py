@@ -79,3 +79,38 @@ def test_shared_kv_reduce_matches_reference_output_bits(case):
         x, y = float(mine[h, -2]), float(mine[h, -1])
         tail = ORACLE.bf16_decode(ORACLE.bf16_encode(np.array([x * c - y * s, x * s + y * c], np.float32)))
         assert np.array_equal(tail, want[h, -2:])
+
+
+@pytest.mark.parametrize("case", make_golden.REDUCE_ROPE_CASES,
+                         ids=[c[0] for c in make_golden.REDUCE_ROPE_CASES])
+def test_reduce_output_rotation_matches_reference_output_bits(case):
+    """The whole published row of yvex_attention_reduce_chunk with a real rope tail (64 rope
+    lanes, plain and YaRN-scaled frequencies, src/graph/core.c:499-507 and
+    src/graph/numeric.c:877-949): yvo_mla_decode_bf16 followed by yvo_reduce_output_finish
+    equals the committed reference output on every lane, bit for bit."""
+    name, attention_class, window, context, stored, heads, dim, policy = case
+    q, local, compressed, sinks = make_golden.reduce_inputs(heads, dim, context, stored)
+    page = 16
+
+    def paged(rows):
+        pages = max((len(rows) + page - 1) // page, 1)
+        pool = np.zeros((pages, page, dim), np.uint16)
+        pool.reshape(-1, dim)[:len(rows)] = ORACLE.bf16_encode(rows)
+        return pool, np.arange(pages, dtype=np.int32)[None, :]
+
+    pool, table = paged(local)
+    cpool, ctable = paged(compressed)
+    visible = np.array([context // make_golden.REDUCE_RATIO if attention_class == 2 else 0], np.int32)
+    rc, out, _, _ = ORACLE.mla_decode(ORACLE.bf16_encode(q)[None], pool, table,
+                                      np.array([context], np.int32), dim, page, sinks=sinks,
+                                      sliding_window=window,
+                                      compressed=(cpool, ctable, visible) if attention_class == 2 else None)
+    assert rc == 0
+    rc, mine = ORACLE.reduce_output_finish(out[0], context - 1, ORACLE.position_policy(**policy))
+    assert rc == 0
+    want = GOLDEN[name + "/out"]
+    assert np.array_equal(mine.view(np.uint32), want.view(np.uint32))
+    # the rotation did something: the rope lanes differ from the unrotated row
+    plain = ORACLE.bf16_decode(ORACLE.bf16_encode(out[0]))
+    assert not np.array_equal(plain[:, -policy["rope_dims"]:], want[:, -policy["rope_dims"]:])
+    assert np.array_equal(plain[:, :dim - policy["rope_dims"]], want[:, :dim - policy["rope_dims"]])

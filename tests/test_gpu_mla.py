@@ -28,7 +28,7 @@ def make_case(rng, contexts, spare=2):
 
 
 def run_mla(backend, q, pool, table, ctx, max_context=None, sinks=None, window=0, compressed=None,
-            selected=None):
+            selected=None, rope=None, positions=None, scale=0.0):
     batch = q.shape[0]
     extra = {}
     if compressed is not None:
@@ -38,7 +38,8 @@ def run_mla(backend, q, pool, table, ctx, max_context=None, sinks=None, window=0
                      compressed_selected_stride=selected.shape[1] if selected is not None else 0)
     req = backend.mla_requirement(batch, HEADS, KEY_DIM, VALUE_DIM, PAGE, pool.shape[0],
                                   table.shape[1], max_context or int(table.shape[1] * PAGE),
-                                  sliding_window=window, **extra)
+                                  sliding_window=window, output_inverse_rope=rope, scale=scale,
+                                  **extra)
     out = backend.tensor("o", B.DTYPE_BF16, (batch, HEADS, VALUE_DIM))
     lse = backend.tensor("lse", B.DTYPE_F32, (batch, HEADS))
     tensors = [backend.tensor("q", B.DTYPE_BF16, q.shape, q),
@@ -53,9 +54,12 @@ def run_mla(backend, q, pool, table, ctx, max_context=None, sinks=None, window=0
               backend.tensor("ccount", B.DTYPE_I32, compressed[2].shape, compressed[2])]
         if selected is not None:
             tc.append(backend.tensor("selected", B.DTYPE_I32, selected.shape, selected))
-    facts = backend.mla_decode_execute(req, *tensors, out, lse, sinks=ts, compressed=tc)
+    tp = backend.tensor("positions", B.DTYPE_I64, (batch,), np.asarray(positions, np.int64)) \
+        if positions is not None else None
+    facts = backend.mla_decode_execute(req, *tensors, out, lse, sinks=ts, compressed=tc,
+                                       output_positions=tp)
     result = out.read(), lse.read(), facts
-    for t in tensors + [out, lse] + ([ts] if ts else []) + (tc or []):
+    for t in tensors + [out, lse] + ([ts] if ts else []) + (tc or []) + ([tp] if tp else []):
         t.release()
     return result
 
@@ -205,3 +209,81 @@ def test_mla_selected_compressed_rows(backend):
     with pytest.raises(YvexError) as e:
         run_mla(backend, q, pool, table, ctx, compressed=(cpool, ctable, counts), selected=bad)
     assert e.value.code == B.YVEX_ERR_BOUNDS
+
+
+ROPE_POLICIES = [
+    dict(rope_dimensions=64, theta=10000),
+    dict(rope_dimensions=64, theta=10000, scaling_factor=40, original_context=4096, beta_fast=32,
+         beta_slow=1),
+    dict(rope_dimensions=128, theta=500000, scaling_factor=8, original_context=8192, beta_fast=32,
+         beta_slow=1),
+    dict(rope_dimensions=8, theta=10000),
+]
+
+
+def oracle_policy(rope):
+    return ORACLE.position_policy(rope["rope_dimensions"], **{k: v for k, v in rope.items()
+                                                             if k != "rope_dimensions"})
+
+
+@pytest.mark.parametrize("rope", ROPE_POLICIES, ids=["plain64", "yarn64", "yarn128", "plain8"])
+def test_mla_output_inverse_rotation(backend, rope):
+    """The rotation the shared-KV reduce applies to its published rows (src/graph/core.c:499-507:
+    bf16 round, the last rope lanes turned back by the token position with the frequencies of
+    src/graph/numeric.c:877-917, bf16 round).  Checked twice: against the oracle end to end
+    within the bf16 tolerance of the attention itself, and bit for bit against the oracle's
+    rotation applied to the rows the same kernels publish without it."""
+    rng = np.random.default_rng(600 + rope["rope_dimensions"])
+    contexts = [1, 33, 64, 500, 1300, 4097]
+    q, pool, table, ctx = make_case(rng, contexts)
+    sinks = (rng.standard_normal(HEADS) * 3.0).astype(np.float32)
+    plain, lse0, _ = run_mla(backend, q, pool, table, ctx, sinks=sinks)
+    got, lse, facts = run_mla(backend, q, pool, table, ctx, sinks=sinks, rope=rope)
+    assert facts.kernel_launches == 2 and np.array_equal(lse, lse0)
+    rc, ref, _, _ = ORACLE.mla_decode(q, pool, table, ctx, VALUE_DIM, PAGE, sinks=sinks)
+    assert rc == 0
+    policy = oracle_policy(rope)
+    keep = VALUE_DIM - rope["rope_dimensions"]
+    for b, n in enumerate(contexts):
+        rc, want = ORACLE.reduce_output_finish(ref[b], n - 1, policy)
+        assert rc == 0
+        assert_close_bf16(got[b:b + 1], want[None], "mla rotation b=%d" % b)
+        rc, exact = ORACLE.reduce_output_finish(ORACLE.bf16_decode(plain[b]), n - 1, policy)
+        assert rc == 0
+        assert np.array_equal(got[b], ORACLE.bf16_encode(exact)), (rope, n)
+        assert np.array_equal(got[b][:, :keep], plain[b][:, :keep])
+        if n > 1:
+            assert not np.array_equal(got[b][:, keep:], plain[b][:, keep:])
+    # explicit positions: long-context angles on the same rows
+    where = [20000 + 7 * b for b in range(len(contexts))]
+    got, _, _ = run_mla(backend, q, pool, table, ctx, sinks=sinks, rope=rope, positions=where)
+    for b in range(len(contexts)):
+        rc, exact = ORACLE.reduce_output_finish(ORACLE.bf16_decode(plain[b]), where[b], policy)
+        assert rc == 0
+        assert np.array_equal(got[b], ORACLE.bf16_encode(exact)), (rope, where[b])
+
+
+def test_mla_rotation_and_scale_refusals_and_explicit_scale(backend):
+    rng = np.random.default_rng(601)
+    q, pool, table, ctx = make_case(rng, [200, 77])
+    for bad, code in ((dict(rope_dimensions=64, theta=1), B.YVEX_ERR_INVALID_ARG),
+                      (dict(rope_dimensions=64, theta=10000, original_context=4096, scaling_factor=40,
+                            beta_fast=1, beta_slow=1), B.YVEX_ERR_INVALID_ARG),
+                      (dict(rope_dimensions=64, theta=10000, original_context=4096), B.YVEX_ERR_INVALID_ARG),
+                      (dict(rope_dimensions=12, theta=10000), B.YVEX_ERR_UNSUPPORTED),
+                      (dict(rope_dimensions=256, theta=10000), B.YVEX_ERR_UNSUPPORTED)):
+        with pytest.raises(YvexError) as e:
+            run_mla(backend, q, pool, table, ctx, rope=bad)
+        assert e.value.code == code, bad
+    with pytest.raises(YvexError) as e:                 # positions without a rotation to use them
+        run_mla(backend, q, pool, table, ctx, positions=[1, 2])
+    assert e.value.code == B.YVEX_ERR_FORMAT
+    with pytest.raises(YvexError) as e:
+        run_mla(backend, q, pool, table, ctx, scale=float("nan"))
+    assert e.value.code == B.YVEX_ERR_INVALID_ARG
+    # an explicit scale: twice the default on a query halved (exact in bf16) gives the same scores
+    base, lse0, _ = run_mla(backend, q, pool, table, ctx)
+    half = ORACLE.bf16_encode(ORACLE.bf16_decode(q) * 0.5)
+    got, lse, _ = run_mla(backend, half, pool, table, ctx, scale=2.0 / np.sqrt(KEY_DIM))
+    assert np.array_equal(got, base)
+    assert np.allclose(lse, lse0, rtol=0, atol=2e-6)

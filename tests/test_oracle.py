@@ -1,5 +1,6 @@
 """Pins the CPU oracle: reference-held vectors, the compiled reference operator
 (oracle/_ref, when built), closed forms and brute force.  CPU only."""
+import ctypes as C
 import math
 
 import numpy as np
@@ -664,13 +665,13 @@ def test_mla_selected_rows_are_the_listed_rows_in_list_order():
 # ------------------------- the shared-KV oracle against the compiled reference reduce ----
 
 def _reference_tail(row_bf16, position, theta=10000):
-    """What the reference does to a published row after the softmax (src/graph/core.c:499-507):
-    the last two lanes rotated back by the token position, then rounded to bf16 again."""
-    row = row_bf16.astype(np.float64).copy()
-    c, s = math.cos(float(position)), -math.sin(float(position))      # pair 0: frequency 1
-    x, y = row[-2], row[-1]
-    row[-2], row[-1] = np.float32(x * c - y * s), np.float32(x * s + y * c)
-    return ORACLE.bf16_decode(ORACLE.bf16_encode(row.astype(np.float32)))
+    """What the reference does to a published row after the softmax (src/graph/core.c:499-507)
+    when it is run with two rope lanes: the last two lanes rotated back by the token position,
+    then rounded to bf16 again."""
+    rc, out = ORACLE.reduce_output_finish(row_bf16[None, :], position,
+                                          ORACLE.position_policy(2, theta=theta))
+    assert rc == 0
+    return out[0]
 
 
 @needs_ref_reduce
@@ -718,3 +719,90 @@ def test_no_sink_equals_a_sink_that_underflows():
     a = ORACLE.mla_decode(q, pool, table, ctx, vd, pt)
     b = ORACLE.mla_decode(q, pool, table, ctx, vd, pt, sinks=np.full(4, -1e30, np.float32))
     assert a[0] == 0 and b[0] == 0 and np.array_equal(a[1], b[1]) and np.array_equal(a[3], b[3])
+
+
+# ------------------------------------------ the output rotation of the shared-KV reduce ----
+
+ROPE_POLICIES = [
+    dict(rope_dims=64, theta=10000),
+    dict(rope_dims=64, theta=10000, scaling_factor=40, original_context=4096, beta_fast=32, beta_slow=1),
+    dict(rope_dims=32, theta=500000, scaling_factor=8, original_context=8192, beta_fast=32, beta_slow=1),
+    dict(rope_dims=2, theta=10000),
+]
+
+
+@needs_ref_reduce
+@pytest.mark.parametrize("policy", ROPE_POLICIES, ids=["plain64", "yarn64", "yarn32", "plain2"])
+@pytest.mark.parametrize("dim", [64, 128])
+def test_reduce_output_finish_matches_compiled_reference_reduce(policy, dim):
+    """yvo_reduce_output_finish (bf16 round, inverse rotation of the rope lanes with the
+    reference's frequency rule, bf16 round) after yvo_mla_decode_bf16 against the published
+    rows of yvex_attention_reduce_chunk compiled from the reference sources, every lane, bit
+    for bit; positions up to 20000 so that the angle reduction matters."""
+    rng = np.random.default_rng(91 + dim + policy["rope_dims"])
+    heads, pt = 4, 16
+    contexts = [1, 2, 77, 300, 1500]
+    q, pool, table, ctx, _, _ = _mla_case(rng, contexts, heads=heads, kd=dim, vd=dim, pt=pt)
+    sinks = (rng.standard_normal(heads) * 2.0).astype(np.float32)
+    rc, out, _, _ = ORACLE.mla_decode(q, pool, table, ctx, dim, pt, sinks=sinks)
+    assert rc == 0
+    for b, n in enumerate(contexts):
+        local = ORACLE.bf16_decode(pool[table[b, :(n + pt - 1) // pt]].reshape(-1, dim)[:n])
+        # the reference takes the token position separately from the rows' positions: a large
+        # offset exercises the rotation at long-context angles with a short history
+        offset = [0, 20000][b % 2]
+        rc1, ref = reference_reduce(REF_REDUCE, ORACLE.bf16_decode(q[b]), local,
+                                    np.arange(n) + offset, np.zeros((0, dim), np.float32), [],
+                                    sinks, 10 ** 6, 0, 0, n - 1 + offset, **policy)
+        assert rc1 == 0
+        rc2, mine = ORACLE.reduce_output_finish(out[b], n - 1 + offset,
+                                                ORACLE.position_policy(**policy))
+        assert rc2 == 0
+        assert np.array_equal(mine.view(np.uint32), ref.view(np.uint32)), (policy, dim, n)
+
+
+def test_yarn_frequency_closed_forms():
+    """Without scaling the frequency of pair i is theta^(-2i/dims) (pair 0: exactly 1).  With
+    the YaRN ramp the pairs below the low corner keep that frequency and the pairs above the
+    high corner have it divided by the factor (src/graph/numeric.c:888-915)."""
+    plain = ORACLE.position_policy(64, theta=10000)
+    f = [ORACLE.lib.yvo_yarn_frequency(C.byref(plain), i, 64) for i in range(32)]
+    assert f[0] == 1.0
+    assert np.allclose(f, 10000.0 ** (-np.arange(32) * 2 / 64), rtol=1e-15)
+    yarn = ORACLE.position_policy(64, theta=10000, scaling_factor=40, original_context=4096,
+                                  beta_fast=32, beta_slow=1)
+    g = [ORACLE.lib.yvo_yarn_frequency(C.byref(yarn), i, 64) for i in range(32)]
+    low = math.floor(64 * math.log(4096 / (32 * 2 * math.pi)) / (2 * math.log(10000)))
+    high = math.ceil(64 * math.log(4096 / (1 * 2 * math.pi)) / (2 * math.log(10000)))
+    assert 0 < low < high < 31
+    for i in range(32):
+        if i <= low:
+            assert g[i] == f[i]
+        elif i >= high:
+            assert math.isclose(g[i], f[i] / 40, rel_tol=1e-15)
+        else:
+            assert f[i] / 40 < g[i] < f[i]
+    assert all(a > b for a, b in zip(g, g[1:]))          # still strictly decreasing
+
+
+def test_rope_apply_properties():
+    rng = np.random.default_rng(92)
+    policy = ORACLE.position_policy(64, theta=10000, scaling_factor=40, original_context=4096,
+                                    beta_fast=32, beta_slow=1)
+    row = rng.standard_normal(128).astype(np.float32)
+    rc, same = ORACLE.rope_apply(row, 0, policy)                      # position 0: identity
+    assert rc == 0 and np.array_equal(same, row)
+    rc, turned = ORACLE.rope_apply(row, 4321, policy)
+    assert rc == 0 and np.array_equal(turned[:64], row[:64])          # only the last 64 lanes move
+    assert not np.array_equal(turned[64:], row[64:])
+    pairs = turned[64:].reshape(-1, 2).astype(np.float64)
+    assert np.allclose((pairs ** 2).sum(1), (row[64:].reshape(-1, 2).astype(np.float64) ** 2).sum(1),
+                       rtol=1e-6)                                      # a rotation keeps pair norms
+    rc, back = ORACLE.rope_apply(turned, 4321, policy, inverse=True)
+    assert rc == 0 and np.allclose(back, row, atol=1e-6)
+    # pair 0 turns by exactly `position` radians (frequency 1)
+    rc, unit = ORACLE.rope_apply(np.array([1.0, 0.0], np.float32), 3, ORACLE.position_policy(2))
+    assert rc == 0 and np.allclose(unit, [math.cos(3.0), math.sin(3.0)], atol=1e-7)
+    # refusals of the reference (numeric.c:930-932): theta <= 1, more rope lanes than lanes
+    assert ORACLE.rope_apply(row, 1, ORACLE.position_policy(64, theta=1))[0] != 0
+    assert ORACLE.rope_apply(row[:32], 1, ORACLE.position_policy(64))[0] != 0
