@@ -97,6 +97,11 @@ static int rocm_tensor_free(yvex_backend *backend, yvex_device_tensor *tensor, y
     if (state->recording)
         return refuse(err, YVEX_ERR_STATE, where,
                       "not available while a launch sequence is being recorded");
+    /* a recorded sequence holds the device addresses of the tensors its operations named and
+     * of the workspace: none of them may go away before the sequence does */
+    if (state->live_graphs && !backend_cleanup_only(backend))
+        return refuse(err, YVEX_ERR_STATE, where,
+                      "recorded launch sequences still name device tensors: release them first");
     if (backend->workspace_device_tensor == tensor) yvex_backend_workspace_detach(backend);
     /* nothing may still read the allocation: drain the stream first */
     rc = yvex_rocm_status(&state->driver, state->driver.hipStreamSynchronize(state->stream), where,
@@ -801,6 +806,8 @@ int yvex_backend_rocm_graph_end(yvex_backend *backend, yvex_rocm_graph **out, yv
     }
     graph->graph = captured;
     graph->kernel_launches = state->recorded_launches;
+    graph->workspace_address = backend->workspace_device_address;
+    graph->workspace_bytes = backend->workspace_bytes;
     rc = yvex_rocm_status(&state->driver,
                           state->driver.hipGraphInstantiate(&graph->executable, captured, NULL, NULL, 0u),
                           where, err);
@@ -827,6 +834,12 @@ int yvex_backend_rocm_graph_launch(yvex_backend *backend, yvex_rocm_graph *graph
     if (rc != YVEX_OK) return rc;
     if (state->recording)
         return refuse(err, YVEX_ERR_STATE, where, "a launch sequence is being recorded");
+    /* the recorded launches write to the workspace that was attached then: a replay after it
+     * was detached or replaced would write to memory the caller has taken back */
+    if (graph->kernel_launches && (graph->workspace_address != backend->workspace_device_address ||
+                                   graph->workspace_bytes != backend->workspace_bytes))
+        return refuse(err, YVEX_ERR_STATE, where,
+                      "the workspace attached when the sequence was recorded is no longer attached");
     if (facts) memset(facts, 0, sizeof(*facts));
     rc = yvex_rocm_status(&state->driver, state->driver.hipGraphLaunch(graph->executable, state->stream),
                           where, err);

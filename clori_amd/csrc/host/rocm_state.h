@@ -81,6 +81,8 @@ struct yvex_rocm_graph {
     hipGraph_t graph;
     hipGraphExec_t executable;
     unsigned long long kernel_launches;
+    /* the workspace the recorded launches write their temporaries to */
+    unsigned long long workspace_address, workspace_bytes;
 };
 
 static inline yvex_rocm_backend_state *yvex_rocm_state(const yvex_backend *backend)

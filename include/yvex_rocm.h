@@ -559,7 +559,13 @@ typedef struct yvex_rocm_mla_decode_request {
  * contributes token_count[s] consecutive rows of `key` / `value` starting at row_start[s];
  * they become positions position_start[s] .. of that session.  rotary_dimension = 0 writes
  * the keys as given; otherwise cosine / sine are F32 [total_tokens][rotary_dimension] tables
- * indexed by input row (src/backend/cuda/transformer_kernels.cu:79-108). */
+ * indexed by input row (src/backend/cuda/transformer_kernels.cu:79-108).
+ * Caller contract: within one call no page id appears in the rows of two sessions, and the
+ * token ranges of one session do not overlap.  A V page block is filled by a read-modify-
+ * write of whole 16-byte groups, one workgroup per (session, page): two sessions writing the
+ * same page in one launch race on it and the result is undefined (nothing is flagged).  Pages
+ * shared between sessions (a common prefix) are fine as long as no session of the call
+ * writes to them. */
 typedef struct yvex_rocm_kv_append_requirement {
     unsigned long long sessions, total_tokens, max_tokens_per_session;
     unsigned long long key_value_heads, head_dimension, page_tokens, pool_pages, page_table_stride;
@@ -682,7 +688,10 @@ int yvex_backend_bandwidth_probe(yvex_backend *backend, yvex_backend_bandwidth_e
  * sequence with one call and then completes like any operation (status check in the
  * immediate mode, at the next sync in the deferred mode).  The tensors the recorded
  * operations named must stay allocated, at the same geometry, until the sequence is
- * released; their contents may change between replays.
+ * released; their contents may change between replays.  The library holds the caller to it
+ * where it can: while any sequence is unreleased, freeing a tensor of the backend is refused
+ * with YVEX_ERR_STATE, and a replay is refused with YVEX_ERR_STATE unless the workspace that
+ * was attached during the recording is still the attached one.
  */
 typedef struct yvex_rocm_graph yvex_rocm_graph;
 int yvex_backend_rocm_graph_begin(yvex_backend *backend, yvex_error *err);

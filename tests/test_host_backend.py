@@ -618,8 +618,26 @@ def test_recorded_sequence_rules(fake_runtime):
         assert b.graph_launch(graph).device_synchronizations == 0
         b.sync()
         b.set_completion_mode(B.COMPLETION_IMMEDIATE)
+        # the sequence holds device addresses: nothing it may name can be freed while it lives,
+        # and it is not replayed without the workspace it was recorded with
+        live = fake_runtime.fake_hip_live_allocations()
+        for tensor in (q, out, work):
+            with pytest.raises(YvexError) as e:
+                tensor.release()
+            assert e.value.code == B.YVEX_ERR_STATE and "recorded launch sequences" in e.value.message
+        assert fake_runtime.fake_hip_live_allocations() == live
+        b.workspace_detach()
+        launched = fake_runtime.fake_hip_launches()
+        with pytest.raises(YvexError) as e:
+            b.graph_launch(graph)
+        assert e.value.code == B.YVEX_ERR_STATE and "workspace" in e.value.message
+        assert fake_runtime.fake_hip_launches() == launched
+        b.workspace_attach(work)
+        assert b.graph_launch(graph).kernel_launches == 1
         b.graph_release(graph)
         b.workspace_detach()
+        work.release()
+        assert fake_runtime.fake_hip_live_allocations() == live - 1
 
 
 def test_bandwidth_probe_record(env, fake_runtime):
