@@ -12,6 +12,9 @@ already resident in HBM.  Workloads are the five configurations the metric is qu
     paged4     32 sessions, paged Q8_0 KV, contexts U[4096,32768]        (HBM bound)
     mla5       absorbed MLA decode, batch 16, 128 heads, context 8192    (HBM bound)
 
+By name only (not configurations of the metric): exact2 (configuration 2 under the EXACT_F32
+contract, against the fp32 matrix peak), append_bf16 / append_q8_0 (the KV page writer), copy.
+
 Prints ONE JSON line.  `value` is the headline workload's throughput; every workload
 that ran is listed under "workloads" with its own roofline figures.  Timing uses HIP
 events recorded on the backend's own stream (the stream the kernels are launched on).
@@ -33,6 +36,7 @@ from clori_amd.backend import Backend  # noqa: E402
 
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
+MFMA_F32_PEAK_TFLOPS = 157.3    # MI355X dense fp32 matrix, published
 
 
 def bf16_bits(x):
@@ -250,6 +254,27 @@ def workload_prefill2(backend, rng, steps, warmup):
                 launches=int(facts.kernel_launches), kernels=kernels, **timed)
 
 
+def workload_exact2(backend, rng, steps, warmup):
+    """Configuration 2 under the EXACT_F32 contract (F32 tensors, F32 products): the request
+    the reference's engine makes.  Not one of the metric's configurations: run by name."""
+    t, hq, hkv, d = 2048, 40, 8, 128
+    q = backend.tensor("q", B.DTYPE_F32, (t, hq, d), rng.standard_normal((t, hq, d), dtype=np.float32))
+    k = backend.tensor("k", B.DTYPE_F32, (t, hkv, d), rng.standard_normal((t, hkv, d), dtype=np.float32))
+    v = backend.tensor("v", B.DTYPE_F32, (t, hkv, d), rng.standard_normal((t, hkv, d), dtype=np.float32))
+    out = backend.tensor("out", B.DTYPE_F32, (t, hq, d))
+    req = backend.attention_requirement(t, t, hq, hkv, d, causal=True)
+    run = lambda: backend.attention_execute(req, q, k, v, out)  # noqa: E731
+    facts = run()
+    kernels = ["yvex_rocm_gqa_f32_tile_128"]
+    timed = time_steps(backend, run, steps, warmup, kernels)
+    return dict(name="exact2",
+                workload="causal GQA prefill, EXACT_F32 contract: batch 1, seq 2048, 40/8 heads, "
+                         "d=128, f32 in and out",
+                bound="mfma", flops=4 * d * hq * t * (t + 1) // 2, peak_tflops=MFMA_F32_PEAK_TFLOPS,
+                algorithmic_bytes=(2 * t * hq * d + 2 * t * hkv * d) * 4, dtype="f32",
+                launches=int(facts.kernel_launches), kernels=kernels, **timed)
+
+
 def workload_mla5(backend, rng, steps, warmup):
     batch, heads, kd, vd, page, ctx = 16, 128, 576, 512, 64, 8192
     pages_each = ctx // page
@@ -351,9 +376,10 @@ WORKLOADS = {
 EXTRA_WORKLOADS = {
     "append_bf16": lambda b, r, s, w: workload_append(b, r, s, w, q8=False),
     "append_q8_0": lambda b, r, s, w: workload_append(b, r, s, w, q8=True),
+    "exact2": workload_exact2,
 }
 SEEDS = {"decode1": 1, "prefill2": 2, "paged3": 3, "paged4": 4, "mla5": 5, "append_bf16": 6,
-         "append_q8_0": 7}
+         "append_q8_0": 7, "exact2": 8}
 
 
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
@@ -388,7 +414,8 @@ def roofline(result):
     if result["bound"] == "hbm":
         work, scale, peak, unit = result["algorithmic_bytes"], 1e9, HBM_PEAK_GBS, "GB/s"
     else:
-        work, scale, peak, unit = result["flops"], 1e12, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s"
+        work, scale, unit = result["flops"], 1e12, "TFLOP/s"
+        peak = result.get("peak_tflops", MFMA_BF16_PEAK_TFLOPS)
     achieved, step_achieved = work / seconds / scale, work / step_seconds / scale
     return dict(bound=result["bound"], achieved=achieved, peak=peak, unit=unit, frac=achieved / peak,
                 traffic=measured_traffic(result["name"], kernel),
@@ -455,6 +482,15 @@ def cpu_baseline(name, budget=6.0):
         return dict(value=4 * d * hq * t * (t + 1) // 2 / dt / 1e12, unit="TFLOP/s", cores=threads,
                     kind="port", sample="the first 1024 tokens of the same shape, median of %d runs "
                                         "(%.1f s)" % (runs, spent))
+    if name == "exact2":
+        t, hq, hkv, d = 512, 40, 8, 128
+        q = rng.standard_normal((t, hq, d), dtype=np.float32)
+        k = rng.standard_normal((t, hkv, d), dtype=np.float32)
+        v = rng.standard_normal((t, hkv, d), dtype=np.float32)
+        runs, dt, spent = repeat_for(budget, lambda: oracle.gqa(q, k, v)[0])
+        return dict(value=4 * d * hq * t * (t + 1) // 2 / dt / 1e12, unit="TFLOP/s", cores=threads,
+                    kind="port", sample="the first 512 tokens of the same shape, median of %d runs "
+                                        "(%.1f s)" % (runs, spent))
     if name == "mla5":
         batch, heads, kd, vd, page, ctx = 2, 128, 576, 512, 64, 4096
         pages = batch * ctx // page
@@ -511,7 +547,7 @@ def main():
                     "working_set_bytes": int(evidence.working_set_bytes)}
     head = results[headline]
     roof = roofline(head)
-    cpu = {} if args.no_cpu else {n: cpu_baseline(n) for n in names if n in WORKLOADS}
+    cpu = {} if args.no_cpu else {n: cpu_baseline(n) for n in names}
     line = {
         "metric": METRIC,
         "value": roof["step_achieved"],
@@ -519,7 +555,7 @@ def main():
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": head["ms"],
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16", "data": "synthetic",
+        "dtype": head.get("dtype", "bf16"), "data": "synthetic",
         "config": {"workload": head["workload"], "name": head["name"],
                    "kernel_launches_per_step": head["launches"]},
         "roofline": roof,

@@ -329,6 +329,30 @@ static int view_ok(const yvex_backend *backend, const yvex_device_tensor *tensor
            tensor->bytes == bytes;
 }
 
+/* The EXACT_F32 request has two kernels.  Prefill-shaped requests (at least 32 query tokens,
+ * head dimension 64 or 128, 16-byte aligned rows) run in 32 x 32 tiles on the fp32 matrix
+ * cores with float statistics, the arithmetic of the reference's own device kernel
+ * (src/backend/cuda/transformer_kernels.cu:136-208).  Everything else (single-token decode,
+ * other head dimensions up to 256, unaligned views) runs one wave per (token, head) with
+ * double-precision statistics.  The choice is a function of the request geometry only. */
+enum { ROCM_EXACT_TILE_QUERIES = 128, ROCM_EXACT_TILE_MIN_TOKENS = 32 };
+
+static int exact_tile_function(const yvex_transformer_attention_requirement *r,
+                               unsigned long long q_stride, unsigned long long k_stride,
+                               unsigned long long v_stride,
+                               const yvex_transformer_attention_request *request,
+                               yvex_rocm_function_id *function)
+{
+    if (r->query_tokens < ROCM_EXACT_TILE_MIN_TOKENS ||
+        (r->head_dimension != 64ull && r->head_dimension != 128ull) ||
+        ((q_stride | k_stride | v_stride) & 3ull) ||
+        (((uintptr_t)request->query->data | (uintptr_t)request->key->data |
+          (uintptr_t)request->value->data | (uintptr_t)request->output->data) & 15u))
+        return 0;
+    *function = r->head_dimension == 64ull ? YVEX_ROCM_FN_GQA_F32_TILE_64 : YVEX_ROCM_FN_GQA_F32_TILE_128;
+    return 1;
+}
+
 static int attention_execute_common(yvex_backend *backend,
                                     const yvex_transformer_attention_request *request,
                                     yvex_device_tensor *lse, const yvex_device_tensor *gate,
@@ -382,6 +406,8 @@ static int attention_execute_common(yvex_backend *backend,
                       "bounded Q/K/V views matching the declared token strides are required");
     if (exact) {
         yvex_rocm_gqa_f32_params params;
+        yvex_rocm_function_id tile_function = YVEX_ROCM_FN_GQA_F32;
+        int tiled = 0;
         memset(&params, 0, sizeof(params));
         params.q = (const float *)request->query->data;
         params.k = (const float *)request->key->data;
@@ -401,11 +427,25 @@ static int attention_execute_common(yvex_backend *backend,
         params.scale = 1.0f / sqrtf((float)r->head_dimension);
         params.causal = causal;
         backend_workspace_reset(backend);
-        rc = yvex_rocm_launch(backend, YVEX_ROCM_FN_GQA_F32,
-                              YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_F32, (unsigned int)rows, 1u,
-                              1u, 64u, 0u, &params, "rocm.transformer.gqa", err);
+        if (exact_tile_function(r, q_stride, k_stride, v_stride, request, &tile_function)) {
+            /* 128 query tokens of one head per workgroup, on the fp32 matrix cores */
+            const unsigned long long groups =
+                r->query_heads * ((r->query_tokens + ROCM_EXACT_TILE_QUERIES - 1ull) / ROCM_EXACT_TILE_QUERIES);
+            if (groups > 0x7fffffffull)
+                return refuse(err, YVEX_ERR_BOUNDS, "rocm.transformer.gqa",
+                              "attention geometry exceeds the launch range");
+            rc = yvex_rocm_launch(backend, tile_function, YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_F32,
+                                  (unsigned int)groups, 1u, 1u, 256u, 0u, &params,
+                                  "rocm.transformer.gqa", err);
+            tiled = 1;
+        } else {
+            rc = yvex_rocm_launch(backend, YVEX_ROCM_FN_GQA_F32,
+                                  YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_F32, (unsigned int)rows, 1u,
+                                  1u, 64u, 0u, &params, "rocm.transformer.gqa", err);
+        }
         if (rc == YVEX_OK) {
             facts->kernel_launches = 1ull;
+            facts->accelerated_matrix_launches = tiled ? 1ull : 0ull;
             facts->compulsory_memory_facts_available = 1;
             rc = yvex_rocm_complete(backend, YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_F32,
                                     "rocm.transformer.gqa", facts, err);

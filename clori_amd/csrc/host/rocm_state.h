@@ -12,6 +12,8 @@
 typedef enum {
     YVEX_ROCM_FN_ATTENTION_F32 = 0,
     YVEX_ROCM_FN_GQA_F32,
+    YVEX_ROCM_FN_GQA_F32_TILE_64,
+    YVEX_ROCM_FN_GQA_F32_TILE_128,
     YVEX_ROCM_FN_FILL_U32,
     YVEX_ROCM_FN_DECODE_PAGED_BF16,
     YVEX_ROCM_FN_DECODE_ROWS_BF16,

@@ -1,0 +1,230 @@
+// EXACT_F32 grouped-query attention on the fp32 matrix cores of gfx950 (wave64).
+//
+// F32 tensors in, F32 out, every product an F32 product: the numeric contract of the
+// reference's only attention request (src/backend/cuda/exact_attention.c:35-49) and the
+// arithmetic of its own device kernel (float dot products, float online softmax,
+// src/backend/cuda/transformer_kernels.cu:136-208), here in 32x32 tiles on
+// v_mfma_f32_32x32x2_f32 instead of one row at a time.
+//
+// One workgroup = 128 consecutive query tokens of one query head, four waves of 32 queries.
+// Key and value rows of the head's KV group go through LDS in tiles of 32 tokens, shared by
+// the four waves, double buffered: the rows of tile t+1 are fetched into registers before
+// the matrix work of tile t and written to the other buffer after it.
+//
+// Per tile a wave computes S^T = K Q^T (keys x queries), so that a lane owns one query
+// column and 16 of the 32 key rows: the softmax statistics are in-lane but for one exchange
+// with the lane 32 apart, and the exponentials are already in the operand layout of
+// O^T += V^T P^T (head dims x queries), whose 32x32 blocks stay in registers for the whole
+// row of tiles.  The contraction index of an MFMA is split between the two lane halves
+// (lane / 32); both products are sums over it, so each half takes the part that is
+// contiguous for it: half the head dimension for S^T, its own 16 key rows for O^T.
+//
+// grid = query_heads * ceil(query_tokens / 128), the longest (last) query tiles first;
+// block = 256.
+#include <hip/hip_runtime.h>
+
+#include "../kernel_params.h"
+#include "mfma.h"
+
+namespace {
+
+__device__ inline void flag_status(int32_t *status, int code)
+{
+    atomicCAS(status, 0, code);
+}
+
+__device__ inline floatx16 mfma_32x32x2(float a, float b, floatx16 c)
+{
+    return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
+}
+
+// kBlocks: head_dim / 32.
+template <int kBlocks>
+struct GqaTile {
+    static constexpr int kDim = 32 * kBlocks, kHalf = kDim / 2;
+    static constexpr int kKeys = 32, kQueries = 128;
+    // row strides in floats: the K operand is read 16 bytes per lane with the key in the lane
+    // index (stride = 4 mod 64 banks), the V operand 4 bytes per lane with rows 4 apart in the
+    // two lane halves (4 * stride = 32 mod 64 banks)
+    static constexpr int kKStride = kDim + 4, kVStride = kDim + 8;
+    static constexpr int kStageFloats = kKeys * (kKStride + kVStride);
+    static constexpr int kChunks = kDim / 32;  // 16-byte pieces of a K (or V) tile per thread
+
+    const yvex_rocm_gqa_f32_params &p;
+    float *lds;
+    const int tid, lane, wave, column, half;
+
+    __device__ GqaTile(const yvex_rocm_gqa_f32_params &params, float *shared)
+        : p(params), lds(shared), tid(threadIdx.x), lane(threadIdx.x & 63), wave(threadIdx.x >> 6),
+          column(threadIdx.x & 31), half((threadIdx.x >> 5) & 1)
+    {
+    }
+
+    struct Staged {
+        floatx4 k[kChunks], v[kChunks];
+    };
+
+    // rows of key tile `tile` for this thread; rows past the end read as zero
+    __device__ void fetch(uint64_t tile, uint64_t kv_head, Staged &s) const
+    {
+#pragma unroll
+        for (int j = 0; j < kChunks; ++j) {
+            const int c = tid + 256 * j, row = c / (kDim / 4), piece = c % (kDim / 4);
+            const uint64_t key = tile * kKeys + (uint64_t)row;
+            const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
+            s.k[j] = zero;
+            s.v[j] = zero;
+            if (key < p.kv_tokens) {
+                s.k[j] = *reinterpret_cast<const floatx4 *>(p.k + key * p.k_stride + kv_head * kDim + 4 * piece);
+                s.v[j] = *reinterpret_cast<const floatx4 *>(p.v + key * p.v_stride + kv_head * kDim + 4 * piece);
+            }
+        }
+    }
+
+    __device__ void stage(int buffer, const Staged &s) const
+    {
+        float *kt = lds + buffer * kStageFloats, *vt = kt + kKeys * kKStride;
+#pragma unroll
+        for (int j = 0; j < kChunks; ++j) {
+            const int c = tid + 256 * j, row = c / (kDim / 4), piece = c % (kDim / 4);
+            *reinterpret_cast<floatx4 *>(kt + row * kKStride + 4 * piece) = s.k[j];
+            *reinterpret_cast<floatx4 *>(vt + row * kVStride + 4 * piece) = s.v[j];
+        }
+    }
+
+    __device__ void run() const
+    {
+        const uint64_t tiles_q = (p.query_tokens + kQueries - 1) / kQueries;
+        const uint64_t head = blockIdx.x % p.query_heads;
+        const uint64_t q_tile = tiles_q - 1 - blockIdx.x / p.query_heads;
+        const uint64_t kv_head = head / (p.query_heads / p.kv_heads);
+        const uint64_t q0 = q_tile * kQueries + (uint64_t)wave * 32u;
+        // rows past the last query repeat it: they compute, they are not stored
+        const uint64_t token = min(q0 + (uint64_t)column, p.query_tokens - 1);
+        const uint64_t own = p.query_start + token;  // absolute position of this lane's query
+        // last key any query of the workgroup, and of this wave, may see
+        const uint64_t group_last = p.causal
+            ? min(p.kv_tokens, p.query_start + min((q_tile + 1) * kQueries, p.query_tokens))
+            : p.kv_tokens;
+        const uint64_t wave_last = p.causal
+            ? min(p.kv_tokens, p.query_start + min(q0 + 32u, p.query_tokens))
+            : p.kv_tokens;
+        const uint64_t tiles = (group_last + kKeys - 1) / kKeys;
+        const uint64_t wave_tiles = q0 < p.query_tokens ? (wave_last + kKeys - 1) / kKeys : 0;
+
+        // this lane's half of its query row: Q[token][half * kHalf + s], s = 0 .. kHalf-1
+        float q[kHalf];
+        {
+            const float *row = p.q + token * p.q_stride + head * kDim + half * kHalf;
+#pragma unroll
+            for (int s = 0; s < kHalf; s += 4) {
+                const floatx4 piece = *reinterpret_cast<const floatx4 *>(row + s);
+                q[s] = piece[0];
+                q[s + 1] = piece[1];
+                q[s + 2] = piece[2];
+                q[s + 3] = piece[3];
+            }
+        }
+
+        floatx16 out[kBlocks];
+#pragma unroll
+        for (int b = 0; b < kBlocks; ++b)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) out[b][i] = 0.f;
+        float top = -INFINITY, sum = 0.f;  // running maximum (natural units), this half's share of the denominator
+
+        Staged next;
+        fetch(0, kv_head, next);
+        stage(0, next);
+        __syncthreads();
+        for (uint64_t t = 0; t < tiles; ++t) {
+            const bool more = t + 1 < tiles;
+            if (more) fetch(t + 1, kv_head, next);
+            if (t < wave_tiles) {
+                const float *kt = lds + (int)(t & 1) * kStageFloats, *vt = kt + kKeys * kKStride;
+                // S^T (32 keys x 32 queries): the key row is the lane's column index
+                floatx16 s;
+#pragma unroll
+                for (int i = 0; i < 16; ++i) s[i] = 0.f;
+                const float *krow = kt + column * kKStride + half * kHalf;
+#pragma unroll
+                for (int step = 0; step < kHalf; step += 4) {
+                    const floatx4 piece = *reinterpret_cast<const floatx4 *>(krow + step);
+                    s = mfma_32x32x2(piece[0], q[step], s);
+                    s = mfma_32x32x2(piece[1], q[step + 1], s);
+                    s = mfma_32x32x2(piece[2], q[step + 2], s);
+                    s = mfma_32x32x2(piece[3], q[step + 3], s);
+                }
+                // lane holds keys 8 * (i / 4) + 4 * half + i % 4 of the tile for its query
+                float peak = -INFINITY;
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const uint64_t key = t * kKeys + (uint64_t)(8 * (i / 4) + 4 * half + i % 4);
+                    const bool visible = key < p.kv_tokens && (!p.causal || key <= own);
+                    s[i] = visible ? s[i] * p.scale : -INFINITY;
+                    peak = fmaxf(peak, s[i]);
+                }
+                peak = fmaxf(peak, xor_lanes(peak, 32));
+                const float top_new = fmaxf(top, peak);
+                // key 0 is visible to every query, so top_new is finite from the first tile on
+                const float keep = fast_exp2((top - top_new) * YVEX_LOG2E);
+                sum *= keep;
+#pragma unroll
+                for (int b = 0; b < kBlocks; ++b)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) out[b][i] *= keep;
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    s[i] = fast_exp2((s[i] - top_new) * YVEX_LOG2E);
+                    sum += s[i];
+                }
+                top = top_new;
+                // O^T (head dims x queries) += V^T P^T over this lane half's 16 keys
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const float *vrow = vt + (8 * (i / 4) + 4 * half + i % 4) * kVStride + column;
+#pragma unroll
+                    for (int b = 0; b < kBlocks; ++b) out[b] = mfma_32x32x2(vrow[32 * b], s[i], out[b]);
+                }
+            }
+            if (more) stage((int)((t + 1) & 1), next);
+            __syncthreads();
+        }
+
+        if (q0 + (uint64_t)column >= p.query_tokens) return;
+        sum += xor_lanes(sum, 32);
+        if (!(sum > 0.f) || !isfinite(sum) || !isfinite(top)) {
+            flag_status(p.status, YVEX_ROCM_DEVICE_NUMERIC);
+            return;
+        }
+        float *row = p.out + (token * p.query_heads + head) * kDim;
+        bool bad = false;
+#pragma unroll
+        for (int b = 0; b < kBlocks; ++b)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                floatx4 piece;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    piece[r] = out[b][4 * g + r] / sum;
+                    bad |= !isfinite(piece[r]);
+                }
+                *reinterpret_cast<floatx4 *>(row + 32 * b + 8 * g + 4 * half) = piece;
+            }
+        if (bad) flag_status(p.status, YVEX_ROCM_DEVICE_NUMERIC);
+        if (p.lse && half == 0) p.lse[token * p.query_heads + head] = top + logf(sum);
+    }
+};
+
+}  // namespace
+
+#define YVEX_GQA_F32_TILE_KERNEL(name, blocks)                                                  \
+    extern "C" __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))  \
+    name(const yvex_rocm_gqa_f32_params p)                                                        \
+    {                                                                                             \
+        __shared__ __attribute__((aligned(16))) float lds[2 * GqaTile<blocks>::kStageFloats];     \
+        GqaTile<blocks>(p, lds).run();                                                            \
+    }
+
+YVEX_GQA_F32_TILE_KERNEL(yvex_rocm_gqa_f32_tile_64, 2)
+YVEX_GQA_F32_TILE_KERNEL(yvex_rocm_gqa_f32_tile_128, 4)
