@@ -81,14 +81,6 @@ yvex_rocm_mla_decode_bf16(const yvex_rocm_mla_params p)
     const uint32_t tiles = (t1 - t0 + kTile - 1) / kTile;
     const uint32_t head = wave * kHeadsPerWave + n;
 
-    // Q fragments: B operand, lane (n, g) holds Q[head n][16*kk + 8g .. +7], kk = 0..35
-    bf16x8 q[36];
-    {
-        const uint16_t *src = p.q + ((uint64_t)batch * p.heads + head) * kKeyDim + g * 8;
-#pragma unroll
-        for (int kk = 0; kk < 36; ++kk) q[kk] = as_bf16x8(load_b128(src + kk * 16));
-    }
-
     // ---- tile staging --------------------------------------------------------------
     // the chunk's page ids are fetched once, so staging a tile never waits on global memory
     const int32_t *table = p.page_table + (uint64_t)batch * p.table_stride;
@@ -98,15 +90,6 @@ yvex_rocm_mla_decode_bf16(const yvex_rocm_mla_params p)
         if (tid == 0) flag(p.status, YVEX_ROCM_DEVICE_CONTRACT);
         return;
     }
-    for (uint32_t i = tid; i < chunk_page_count; i += 256u) {
-        int32_t page = table[first_page + i];
-        if (page < 0 || (uint32_t)page >= p.pool_pages) {
-            flag(p.status, YVEX_ROCM_DEVICE_CONTRACT);
-            page = 0;
-        }
-        chunk_pages[i] = page;
-    }
-    __syncthreads();
     static_assert(kLoadsPerWave == 9, "the loads of a tile ride behind k-steps 1, 5, .. 33");
     const uint32_t lds_base = lds_address_of(lds);
     uint32_t stage_off[kLoadsPerWave];
@@ -116,6 +99,31 @@ yvex_rocm_mla_decode_bf16(const yvex_rocm_mla_params p)
         const int r = linear / kRowChunks, pos = linear % kRowChunks;
         stage_off[j] = (uint32_t)(r * kRowBytes + ((pos ^ swizzle(r)) << 4));
     }
+    // The queries of the batch element first: 128 rows of 1152 bytes are exactly the four tile
+    // buffers, so they are staged like four tiles (coalesced 1 KB loads, same swizzle) and each
+    // wave then takes its 32 heads out of "tile" `wave` with the row fetch of the first product.
+    // A lane's fragments sit 1152 bytes apart in global memory; fetched directly they cost 36
+    // loads of 32 separate lines each and five microseconds before the first tile could start.
+    static_assert(4 * kHeadsPerWave * kRowBytes == kBuffers * kTileBytes, "Q fills the tile ring exactly");
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const i32x4 rsrc = raw_buffer(p.q + ((uint64_t)batch * p.heads + j * kHeadsPerWave) * kKeyDim,
+                                      kHeadsPerWave * kRowBytes);
+        const uint32_t dst = __builtin_amdgcn_readfirstlane(lds_base + j * kTileBytes +
+                                                            wave * (kLoadsPerWave * 1024));
+#pragma unroll
+        for (int i = 0; i < kLoadsPerWave; ++i) lds_dma_b128(dst + i * 1024, rsrc, stage_off[i], 0u);
+    }
+    for (uint32_t i = tid; i < chunk_page_count; i += 256u) {
+        int32_t page = table[first_page + i];
+        if (page < 0 || (uint32_t)page >= p.pool_pages) {
+            flag(p.status, YVEX_ROCM_DEVICE_CONTRACT);
+            page = 0;
+        }
+        chunk_pages[i] = page;
+    }
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's share of Q has landed
+    __syncthreads();                     // ... and everybody's, and the page ids
     // A tile's destination and descriptor.  Loads are always issued (with an empty range
     // past the last tile) so that the outstanding-load count at the top of every step is
     // the same.
@@ -165,6 +173,16 @@ yvex_rocm_mla_decode_bf16(const yvex_rocm_mla_params p)
                 v_addr[par][h] = (uint32_t)(r * kRowBytes + (chunk16 << 4) + 8 * (a & 1));
             }
     }
+
+    // Q fragments: B operand, lane (n, g) holds Q[head n][16*kk + 8g .. +7], kk = 0..35
+    bf16x8 q[36];
+    {
+        const unsigned char *rows = lds + wave * kTileBytes;
+#pragma unroll
+        for (int kk = 0; kk < 36; ++kk)
+            q[kk] = as_bf16x8(*reinterpret_cast<const u32x4 *>(rows + k_addr[kk & 3] + (kk >> 2) * 128));
+    }
+    __syncthreads();  // the buffers are free for tiles once every wave holds its fragments
 
     floatx16 o[16];
 #pragma unroll
