@@ -99,9 +99,14 @@ static int rocm_tensor_free(yvex_backend *backend, yvex_device_tensor *tensor, y
                       "not available while a launch sequence is being recorded");
     /* a recorded sequence holds the device addresses of the tensors its operations named and
      * of the workspace: none of them may go away before the sequence does */
-    if (state->live_graphs && !backend_cleanup_only(backend))
-        return refuse(err, YVEX_ERR_STATE, where,
-                      "recorded launch sequences still name device tensors: release them first");
+    if (!backend_cleanup_only(backend)) {
+        const yvex_rocm_graph *graph;
+        for (graph = state->graphs; graph; graph = graph->next)
+            if (tensor->owner_id < graph->tensor_id_mark)
+                return refuse(err, YVEX_ERR_STATE, where,
+                              "a recorded launch sequence may still name this tensor: release the "
+                              "sequence first");
+    }
     if (backend->workspace_device_tensor == tensor) yvex_backend_workspace_detach(backend);
     /* nothing may still read the allocation: drain the stream first */
     rc = yvex_rocm_status(&state->driver, state->driver.hipStreamSynchronize(state->stream), where,
@@ -808,6 +813,7 @@ int yvex_backend_rocm_graph_end(yvex_backend *backend, yvex_rocm_graph **out, yv
     graph->kernel_launches = state->recorded_launches;
     graph->workspace_address = backend->workspace_device_address;
     graph->workspace_bytes = backend->workspace_bytes;
+    graph->tensor_id_mark = backend->tensor_id_next;
     rc = yvex_rocm_status(&state->driver,
                           state->driver.hipGraphInstantiate(&graph->executable, captured, NULL, NULL, 0u),
                           where, err);
@@ -817,6 +823,8 @@ int yvex_backend_rocm_graph_end(yvex_backend *backend, yvex_rocm_graph **out, yv
         return rc;
     }
     state->live_graphs++;
+    graph->next = state->graphs;
+    state->graphs = graph;
     *out = graph;
     yvex_error_clear(err);
     return YVEX_OK;
@@ -870,6 +878,11 @@ int yvex_backend_rocm_graph_release(yvex_backend *backend, yvex_rocm_graph **gra
     /* a replay may still be running */
     rc = yvex_rocm_status(&state->driver, state->driver.hipStreamSynchronize(state->stream), where, err);
     if (rc != YVEX_OK) return rc;
+    {
+        yvex_rocm_graph **link = &state->graphs;
+        while (*link && *link != *graph) link = &(*link)->next;
+        if (*link) *link = (*graph)->next;
+    }
     if ((*graph)->executable) (void)state->driver.hipGraphExecDestroy((*graph)->executable);
     if ((*graph)->graph) (void)state->driver.hipGraphDestroy((*graph)->graph);
     free(*graph);

@@ -71,6 +71,7 @@ typedef struct yvex_rocm_backend_state {
     unsigned long long live_tensors;
     int recording;                  /* a launch sequence is being recorded on the stream */
     unsigned long long live_graphs; /* recorded sequences not yet released */
+    struct yvex_rocm_graph *graphs; /* ... and the list of them */
     unsigned long long recorded_launches; /* kernel launches of the sequence being recorded */
     void *static_scratch;     /* device address of the fixed scratch array on this device, or NULL */
     int static_scratch_error; /* the runtime's code when it could not be resolved */
@@ -85,6 +86,10 @@ struct yvex_rocm_graph {
     unsigned long long kernel_launches;
     /* the workspace the recorded launches write their temporaries to */
     unsigned long long workspace_address, workspace_bytes;
+    /* tensors with an id below this one existed when the recording ended: the sequence may
+     * name any of them */
+    unsigned long long tensor_id_mark;
+    struct yvex_rocm_graph *next; /* the backend's list of unreleased sequences */
 };
 
 static inline yvex_rocm_backend_state *yvex_rocm_state(const yvex_backend *backend)

@@ -689,9 +689,10 @@ int yvex_backend_bandwidth_probe(yvex_backend *backend, yvex_backend_bandwidth_e
  * immediate mode, at the next sync in the deferred mode).  The tensors the recorded
  * operations named must stay allocated, at the same geometry, until the sequence is
  * released; their contents may change between replays.  The library holds the caller to it
- * where it can: while any sequence is unreleased, freeing a tensor of the backend is refused
- * with YVEX_ERR_STATE, and a replay is refused with YVEX_ERR_STATE unless the workspace that
- * was attached during the recording is still the attached one.
+ * where it can: freeing a tensor that existed when an unreleased sequence was recorded is
+ * refused with YVEX_ERR_STATE (tensors allocated afterwards are free to go), and a replay is
+ * refused with YVEX_ERR_STATE unless the workspace that was attached during the recording is
+ * still the attached one.
  */
 typedef struct yvex_rocm_graph yvex_rocm_graph;
 int yvex_backend_rocm_graph_begin(yvex_backend *backend, yvex_error *err);

@@ -624,7 +624,10 @@ def test_recorded_sequence_rules(fake_runtime):
         for tensor in (q, out, work):
             with pytest.raises(YvexError) as e:
                 tensor.release()
-            assert e.value.code == B.YVEX_ERR_STATE and "recorded launch sequences" in e.value.message
+            assert e.value.code == B.YVEX_ERR_STATE and "recorded launch sequence" in e.value.message
+        assert fake_runtime.fake_hip_live_allocations() == live
+        later = b.tensor("later", B.DTYPE_F32, (16,))         # allocated after the recording:
+        later.release()                                        # the sequence cannot name it
         assert fake_runtime.fake_hip_live_allocations() == live
         b.workspace_detach()
         launched = fake_runtime.fake_hip_launches()
