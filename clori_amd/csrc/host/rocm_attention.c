@@ -719,7 +719,7 @@ static int rocm_paged_decode_execute_fused(yvex_backend *backend,
 
 /* --------------------------------------------------------- MLA decode ---- */
 
-enum { ROCM_MLA_HEADS = 128, ROCM_MLA_KEY_DIM = 576, ROCM_MLA_VALUE_DIM = 512,
+enum { ROCM_MLA_HEADS = 128, ROCM_MLA_REDUCE_HEADS = 64, ROCM_MLA_KEY_DIM = 576, ROCM_MLA_VALUE_DIM = 512,
        ROCM_MLA_PAGE_TOKENS = 64, ROCM_MLA_TILE_TOKENS = 32 };
 
 static int mla_validate(const yvex_rocm_mla_decode_requirement *r, const char *where,
@@ -737,7 +737,11 @@ static int mla_validate(const yvex_rocm_mla_decode_requirement *r, const char *w
           r->max_compressed_tokens > r->compressed_page_table_stride * r->page_tokens)) ||
         (r->compressed_selected_stride && !r->max_compressed_tokens))
         return refuse(err, YVEX_ERR_INVALID_ARG, where, "complete MLA decode geometry is required");
-    if (r->heads != ROCM_MLA_HEADS || r->key_dimension != ROCM_MLA_KEY_DIM ||
+    /* two geometries: the absorbed form (128 heads, 512 latent + 64 rope lanes scored, 512
+     * lanes returned) and the reference's own reduce (64 heads, key and value the same 512-lane
+     * row with the rope lanes inside, tests/unit/deepseek_arch_ir.c:110-125) */
+    if (!((r->heads == ROCM_MLA_HEADS && r->key_dimension == ROCM_MLA_KEY_DIM) ||
+          (r->heads == ROCM_MLA_REDUCE_HEADS && r->key_dimension == ROCM_MLA_VALUE_DIM)) ||
         r->value_dimension != ROCM_MLA_VALUE_DIM || r->page_tokens != ROCM_MLA_PAGE_TOKENS ||
         r->numeric_contract != YVEX_TRANSFORMER_ATTENTION_NUMERIC_BF16_F32_ACCUMULATE ||
         !r->deterministic || r->pool_pages > 0x7fffffffull || capacity > 0x7fffffffull ||
@@ -745,8 +749,9 @@ static int mla_validate(const yvex_rocm_mla_decode_requirement *r, const char *w
         r->compressed_pool_pages > 0x7fffffffull || r->compressed_selected_stride > 0x7fffffull ||
         r->compressed_page_table_stride * r->page_tokens > 0x7fffffffull)
         return refuse(err, YVEX_ERR_UNSUPPORTED, where,
-                      "ROCm MLA decode requires 128 heads, a 512+64 latent row, 64-token pages "
-                      "and the deterministic bf16/fp32-accumulate contract");
+                      "ROCm MLA decode requires 128 heads with a 512+64 latent row or 64 heads with a "
+                      "512-lane row, 64-token pages and the deterministic bf16/fp32-accumulate "
+                      "contract");
     if (r->output_inverse_rope.rope_dimensions) {
         const yvex_backend_attention_position *position = &r->output_inverse_rope;
         /* src/backend/cuda/kernels.cu:1006-1012: the same refusals as the reference's rotation */
@@ -892,6 +897,7 @@ static int rocm_mla_decode_execute(yvex_backend *backend,
     const yvex_rocm_mla_decode_requirement *r;
     yvex_rocm_mla_params kp;
     yvex_rocm_decode_merge_params mp;
+    yvex_rocm_function_id decode_function;
     unsigned long long acc_bytes = 0ull, total = 0ull, max_chunks, chunk, extra_chunk, extra_max_chunks;
     unsigned long long gather_pages, gather_rows, gather_table, partial_bytes;
     void *work = NULL;
@@ -970,7 +976,9 @@ static int rocm_mla_decode_execute(yvex_backend *backend,
     /* src/graph/core.c:604: scale = 1/sqrt(head_dimension), here over the 576-lane key */
     kp.scale_log2 = (float)(1.4426950408889634 *
                             (r->scale > 0.0f ? (double)r->scale : 1.0 / sqrt((double)r->key_dimension)));
-    rc = yvex_rocm_launch(backend, YVEX_ROCM_FN_MLA_DECODE_BF16, variant, (unsigned int)max_chunks,
+    decode_function = r->key_dimension == ROCM_MLA_KEY_DIM ? YVEX_ROCM_FN_MLA_DECODE_BF16
+                                                           : YVEX_ROCM_FN_MLA_DECODE_512_BF16;
+    rc = yvex_rocm_launch(backend, decode_function, variant, (unsigned int)max_chunks,
                           (unsigned int)r->batch, 1u, 256u, 0u, &kp, where, err);
     if (rc == YVEX_OK && extra_max_chunks) {
         /* the compressed rows: same kernel over the second pool, partials after the local ones */
@@ -1014,7 +1022,7 @@ static int rocm_mla_decode_execute(yvex_backend *backend,
             if (rc == YVEX_OK) gathered = 1;
         }
         if (rc == YVEX_OK)
-            rc = yvex_rocm_launch(backend, YVEX_ROCM_FN_MLA_DECODE_BF16, variant,
+            rc = yvex_rocm_launch(backend, decode_function, variant,
                               (unsigned int)extra_max_chunks, (unsigned int)r->batch, 1u, 256u, 0u,
                               &cp, where, err);
     }

@@ -52,6 +52,8 @@ static const rocm_kernel_binding rocm_kernel_bindings[] = {
      YVEX_ROCM_FN_PREFILL_BF16},
     {"yvex_rocm_mla_decode_bf16", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_MLA_BF16,
      YVEX_ROCM_FN_MLA_DECODE_BF16},
+    {"yvex_rocm_mla_decode_512_bf16", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_MLA_BF16,
+     YVEX_ROCM_FN_MLA_DECODE_512_BF16},
     {"yvex_rocm_decode_paged_q8_0", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_PAGED_Q8_0,
      YVEX_ROCM_FN_DECODE_PAGED_Q8_0},
     {"yvex_rocm_decode_paged_bf16_merged", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_PAGED_BF16,

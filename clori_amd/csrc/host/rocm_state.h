@@ -26,6 +26,7 @@ typedef enum {
     YVEX_ROCM_FN_DECODE_ROWS_BF16_MERGED,
     YVEX_ROCM_FN_PREFILL_BF16,
     YVEX_ROCM_FN_MLA_DECODE_BF16,
+    YVEX_ROCM_FN_MLA_DECODE_512_BF16,
     YVEX_ROCM_FN_KV_APPEND_BF16,
     YVEX_ROCM_FN_KV_APPEND_Q8_0,
     YVEX_ROCM_FN_STREAM_READ,

@@ -510,7 +510,9 @@ struct Decoder {
     __device__ inline void merge_segment(uint32_t session, uint32_t kv_head, uint32_t seg_begin,
                                          uint32_t per_wave, uint32_t w_first, uint32_t w_last) const
     {
-        constexpr int kMergeWidth = 8;
+        // the token-major kernel keeps a two-deep ring and has the registers for twice as many
+        // partials in flight: a 4096-token context (32 partials per head) merges in two trips
+        constexpr int kMergeWidth = PAGED ? 8 : 16;
         const uint32_t hl = (uint32_t)lane >> 4, c = (uint32_t)lane & 15u;
         for (uint32_t h0 = 0u; h0 < group; h0 += 4u) {
             const bool live = h0 + hl < group;

@@ -33,14 +33,12 @@
 
 namespace {
 
-constexpr int kKeyDim = 576;
 constexpr int kValueDim = 512;
 constexpr int kTile = 32;                          // tokens per LDS tile
-constexpr int kRowBytes = kKeyDim * 2;             // 1152
+constexpr int kRowBytes = 1152;                    // LDS row pitch, for both geometries
 constexpr int kRowChunks = kRowBytes / 16;         // 72
 constexpr int kTileBytes = kTile * kRowBytes;      // 36864
 constexpr int kBuffers = 4;
-constexpr int kLoadsPerWave = kTileBytes / 1024 / 4;  // 9
 constexpr int kHeadsPerWave = 32;
 constexpr float kLazyLog2 = 8.0f;
 constexpr int kQkDepth = 4;  // operand fetches in flight ahead of the first product
@@ -53,15 +51,28 @@ __device__ inline void flag(int32_t *status, int code) { atomicCAS(status, 0, co
 
 __device__ inline int swizzle(int r) { return (((r >> 1) & 1) << 2) | ((r >> 2) & 3); }
 
-}  // namespace
-
-// grid = (chunks, batch), block 256 (heads must be 128, pages a multiple of 32 tokens),
-// LDS 4 x 36 KB.
-extern "C" __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
-yvex_rocm_mla_decode_bf16(const yvex_rocm_mla_params p)
+// Two geometries share the code.  <576, 128>: the absorbed form, rows of 512 latent + 64 rope
+// lanes, 128 heads on four waves; a tile is 36 KB of contiguous rows and every wave stages
+// nine linear 1 KB pieces of it.  <512, 64>: the reference's own reduce geometry
+// (tests/unit/deepseek_arch_ir.c:110-125: 64 heads, one 512-lane row per token with the rope
+// lanes inside, key and value the same row); rows are 1024 bytes in memory and keep the
+// 1152-byte pitch in LDS (so the bank analysis above holds unchanged), every wave stages
+// eight whole rows, one per load, and waves 2 and 3 only stage: they own no heads.
+template <int kKeyDim, int kHeads>
+__device__ __forceinline__ void mla_decode(const yvex_rocm_mla_params &p, unsigned char *lds,
+                                           int32_t *chunk_pages)
 {
-    __shared__ __attribute__((aligned(16))) unsigned char lds[kBuffers * kTileBytes];
-    __shared__ int32_t chunk_pages[kMaxChunkPages];
+    constexpr int kSteps = kKeyDim / 16;                     // k-steps of the first product
+    constexpr int kSourceRowBytes = kKeyDim * 2;             // row size in global memory
+    constexpr bool kRowPerLoad = kSourceRowBytes == 1024;    // one 1 KB load is one row
+    constexpr int kLoadsPerWave = kRowPerLoad ? kTile / 4 : kTileBytes / 1024 / 4;  // 8 or 9
+    constexpr int kLoadPitch = kRowPerLoad ? kRowBytes : 1024;  // LDS distance between a wave's loads
+    constexpr int kActiveWaves = kHeads / kHeadsPerWave;
+    static_assert(kSteps % 4 == 0 && kSteps / 4 == kLoadsPerWave,
+                  "the loads of a tile ride behind k-steps 1, 5, 9, ...");
+    static_assert(kRowPerLoad || kSourceRowBytes == kRowBytes, "rows are 1024 or 1152 bytes");
+    // at most one younger tile outstanding: vmcnt(kLoadsPerWave), lgkmcnt and expcnt untouched
+    constexpr int kWaitTile = 0x0f70 | kLoadsPerWave;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n = lane & 31, g = lane >> 5;
@@ -90,29 +101,35 @@ yvex_rocm_mla_decode_bf16(const yvex_rocm_mla_params p)
         if (tid == 0) flag(p.status, YVEX_ROCM_DEVICE_CONTRACT);
         return;
     }
-    static_assert(kLoadsPerWave == 9, "the loads of a tile ride behind k-steps 1, 5, .. 33");
     const uint32_t lds_base = lds_address_of(lds);
+    // source offset of this lane's 16 bytes in load j: the chunk that belongs at the lane's
+    // (linear) LDS position
     uint32_t stage_off[kLoadsPerWave];
 #pragma unroll
     for (int j = 0; j < kLoadsPerWave; ++j) {
-        const int linear = (wave * kLoadsPerWave + j) * 64 + lane;
-        const int r = linear / kRowChunks, pos = linear % kRowChunks;
-        stage_off[j] = (uint32_t)(r * kRowBytes + ((pos ^ swizzle(r)) << 4));
+        if (kRowPerLoad) {
+            const int r = wave * kLoadsPerWave + j;
+            stage_off[j] = (uint32_t)(r * kSourceRowBytes + ((lane ^ swizzle(r)) << 4));
+        } else {
+            const int linear = (wave * kLoadsPerWave + j) * 64 + lane;
+            const int r = linear / kRowChunks, pos = linear % kRowChunks;
+            stage_off[j] = (uint32_t)(r * kRowBytes + ((pos ^ swizzle(r)) << 4));
+        }
     }
     // The queries of the batch element first: 128 rows of 1152 bytes are exactly the four tile
     // buffers, so they are staged like four tiles (coalesced 1 KB loads, same swizzle) and each
     // wave then takes its 32 heads out of "tile" `wave` with the row fetch of the first product.
     // A lane's fragments sit 1152 bytes apart in global memory; fetched directly they cost 36
     // loads of 32 separate lines each and five microseconds before the first tile could start.
-    static_assert(4 * kHeadsPerWave * kRowBytes == kBuffers * kTileBytes, "Q fills the tile ring exactly");
+    static_assert(kActiveWaves * kHeadsPerWave * kRowBytes <= kBuffers * kTileBytes, "Q fits the tile ring");
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < kActiveWaves; ++j) {
         const i32x4 rsrc = raw_buffer(p.q + ((uint64_t)batch * p.heads + j * kHeadsPerWave) * kKeyDim,
-                                      kHeadsPerWave * kRowBytes);
+                                      kHeadsPerWave * kSourceRowBytes);
         const uint32_t dst = __builtin_amdgcn_readfirstlane(lds_base + j * kTileBytes +
-                                                            wave * (kLoadsPerWave * 1024));
+                                                            wave * (kLoadsPerWave * kLoadPitch));
 #pragma unroll
-        for (int i = 0; i < kLoadsPerWave; ++i) lds_dma_b128(dst + i * 1024, rsrc, stage_off[i], 0u);
+        for (int i = 0; i < kLoadsPerWave; ++i) lds_dma_b128(dst + i * kLoadPitch, rsrc, stage_off[i], 0u);
     }
     for (uint32_t i = tid; i < chunk_page_count; i += 256u) {
         int32_t page = table[first_page + i];
@@ -137,16 +154,16 @@ yvex_rocm_mla_decode_bf16(const yvex_rocm_mla_params p)
             valid = min((uint32_t)kTile, t1 - first);
             base = p.pool + ((uint64_t)page * p.page_tokens + first % p.page_tokens) * kKeyDim;
         }
-        rsrc = raw_buffer(base, valid * kRowBytes);
+        rsrc = raw_buffer(base, valid * kSourceRowBytes);
         dst = __builtin_amdgcn_readfirstlane(lds_base + (tile % kBuffers) * kTileBytes +
-                                             wave * (kLoadsPerWave * 1024));
+                                             wave * (kLoadsPerWave * kLoadPitch));
     };
     auto stage_tile = [&](uint32_t tile) {
         uint32_t dst;
         i32x4 rsrc;
         stage_target(tile, dst, rsrc);
 #pragma unroll
-        for (int j = 0; j < kLoadsPerWave; ++j) lds_dma_b128(dst + j * 1024, rsrc, stage_off[j], 0u);
+        for (int j = 0; j < kLoadsPerWave; ++j) lds_dma_b128(dst + j * kLoadPitch, rsrc, stage_off[j], 0u);
     };
 
     // ---- operand addresses inside a tile ----------------------------------------------
@@ -175,14 +192,28 @@ yvex_rocm_mla_decode_bf16(const yvex_rocm_mla_params p)
     }
 
     // Q fragments: B operand, lane (n, g) holds Q[head n][16*kk + 8g .. +7], kk = 0..35
-    bf16x8 q[36];
+    bf16x8 q[kSteps];
     {
         const unsigned char *rows = lds + wave * kTileBytes;
 #pragma unroll
-        for (int kk = 0; kk < 36; ++kk)
+        for (int kk = 0; kk < kSteps; ++kk)
             q[kk] = as_bf16x8(*reinterpret_cast<const u32x4 *>(rows + k_addr[kk & 3] + (kk >> 2) * 128));
     }
     __syncthreads();  // the buffers are free for tiles once every wave holds its fragments
+    if (kActiveWaves < 4 && wave >= kActiveWaves) {
+        // a wave without heads: it stages its quarter of every tile and keeps the barriers of
+        // the computing waves (one per tile, one before their epilogue)
+        stage_tile(0u);
+        stage_tile(1u);
+        for (uint32_t t = 0; t < tiles; ++t) {
+            __builtin_amdgcn_s_waitcnt(kWaitTile);
+            __syncthreads();
+            stage_tile(t + 2u);
+        }
+        __builtin_amdgcn_s_waitcnt(0x0f70);
+        __syncthreads();
+        return;
+    }
 
     floatx16 o[16];
 #pragma unroll
@@ -203,9 +234,9 @@ yvex_rocm_mla_decode_bf16(const yvex_rocm_mla_params p)
             frag[kk] = *reinterpret_cast<const u32x4 *>(tile + k_addr[kk & 3] + (kk >> 2) * 128);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int kk = 0; kk < 36; ++kk) {
+        for (int kk = 0; kk < kSteps; ++kk) {
             s = mfma_32x32x16(as_bf16x8(frag[kk % kQkDepth]), q[kk], s);
-            if (kk + kQkDepth < 36)
+            if (kk + kQkDepth < kSteps)
                 frag[kk % kQkDepth] = *reinterpret_cast<const u32x4 *>(
                     tile + k_addr[(kk + kQkDepth) & 3] + ((kk + kQkDepth) >> 2) * 128);
             extra(kk);
@@ -275,7 +306,7 @@ yvex_rocm_mla_decode_bf16(const yvex_rocm_mla_params p)
     };
     auto step = [&](uint32_t t, auto with_update) {
         // tile t has landed when at most one younger tile is outstanding: vmcnt(9)
-        __builtin_amdgcn_s_waitcnt(0x0f79);
+        __builtin_amdgcn_s_waitcnt(kWaitTile);
         __syncthreads();
         uint32_t stage_dst;
         i32x4 stage_rsrc;
@@ -286,7 +317,7 @@ yvex_rocm_mla_decode_bf16(const yvex_rocm_mla_params p)
         // ---- S^T of tile t, the loads of tile t+2 behind its MFMAs ------------------------
         floatx16 s;
         score(tile, s, [&](int kk) {
-            if ((kk & 3) == 1) lds_dma_b128(stage_dst + (kk >> 2) * 1024, stage_rsrc, stage_off[kk >> 2], 0u);
+            if ((kk & 3) == 1) lds_dma_b128(stage_dst + (kk >> 2) * kLoadPitch, stage_rsrc, stage_off[kk >> 2], 0u);
         });
         settle(t0 + t * kTile, s, pk_prev);
 
@@ -374,6 +405,21 @@ yvex_rocm_mla_decode_bf16(const yvex_rocm_mla_params p)
         p.part_ml[slot * 2 + 1] = l;
     }
 }
+
+}  // namespace
+
+// grid = (chunks, batch), block 256 (pages a multiple of 32 tokens), LDS 4 x 36 KB.
+#define YVEX_MLA_KERNEL(name, key_dim, heads)                                                       \
+    extern "C" __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))     \
+    name(const yvex_rocm_mla_params p)                                                               \
+    {                                                                                                \
+        __shared__ __attribute__((aligned(16))) unsigned char lds[kBuffers * kTileBytes];            \
+        __shared__ int32_t chunk_pages[kMaxChunkPages];                                              \
+        mla_decode<key_dim, heads>(p, lds, chunk_pages);                                             \
+    }
+
+YVEX_MLA_KERNEL(yvex_rocm_mla_decode_bf16, 576, 128)
+YVEX_MLA_KERNEL(yvex_rocm_mla_decode_512_bf16, 512, 64)
 
 // Row gather for the selected class of compressed candidates (src/graph/core.c:443-452): list
 // entry i of batch element b names a compressed row; it is copied to row i of that element's

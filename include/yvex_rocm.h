@@ -487,10 +487,14 @@ typedef struct yvex_rocm_paged_decode_request {
 } yvex_rocm_paged_decode_request;
 
 /*
- * Absorbed-latent MLA decode: `heads` query heads share one latent row per token;
- * score over key_dimension (latent + rope), value = first value_dimension lanes.
+ * Shared-KV (MLA) decode: `heads` query heads share one row per token; score over
+ * key_dimension lanes, value = the first value_dimension lanes of the same row.
  * Pool: BF16 [pool_pages][page_tokens][key_dimension] (token-major, page_tokens 64).
  * query BF16 [batch][heads][key_dimension]; output BF16 [batch][heads][value_dimension].
+ * Admitted geometries: the absorbed form, 128 heads, key_dimension 576 (512 latent + 64 rope),
+ * value_dimension 512; and the reference's own reduce (src/graph/core.c:361-508,
+ * tests/unit/deepseek_arch_ir.c:110-125), 64 heads, key_dimension == value_dimension == 512
+ * with the rope lanes inside the row.
  */
 /* Rotary position policy of an attention layer: the fields the rotation reads
  * (include/yvex/internal/backend.h:51-54, same names and order). */

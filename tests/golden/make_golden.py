@@ -56,6 +56,11 @@ REDUCE_ROPE_CASES = [
 ]
 
 
+# the reduce at the reference model's own geometry (tests/unit/deepseek_arch_ir.c:110-125:
+# 64 heads, 512 lanes, 64 rope lanes inside, window 128, ratio 128), dense compressed class
+MODEL_GEOMETRY_CASE = ("reduce-model-geometry", 2, 128, 700, 7, 64, 512, ROPE_YARN)
+
+
 def reduce_inputs(heads, dim, context, stored):
     """bf16-representable patterns: query, local rows (positions 0 .. context-1), compressed
     rows (positions 0, 128, 256, ...), sink logits."""
@@ -128,7 +133,7 @@ def main():
                                  context - 1)
         assert rc == 0, (name, rc)
         out[name + "/out"] = o
-    for name, attention_class, window, context, stored, heads, dim, policy in REDUCE_ROPE_CASES:
+    for name, attention_class, window, context, stored, heads, dim, policy in REDUCE_ROPE_CASES + [MODEL_GEOMETRY_CASE]:
         q, local, compressed, sinks = reduce_inputs(heads, dim, context, stored)
         rc, o = reference_reduce(reduce, q, local, np.arange(context), compressed,
                                  np.arange(stored) * REDUCE_RATIO, sinks, window,

@@ -81,8 +81,8 @@ def test_shared_kv_reduce_matches_reference_output_bits(case):
         assert np.array_equal(tail, want[h, -2:])
 
 
-@pytest.mark.parametrize("case", make_golden.REDUCE_ROPE_CASES,
-                         ids=[c[0] for c in make_golden.REDUCE_ROPE_CASES])
+@pytest.mark.parametrize("case", make_golden.REDUCE_ROPE_CASES + [make_golden.MODEL_GEOMETRY_CASE],
+                         ids=[c[0] for c in make_golden.REDUCE_ROPE_CASES + [make_golden.MODEL_GEOMETRY_CASE]])
 def test_reduce_output_rotation_matches_reference_output_bits(case):
     """The whole published row of yvex_attention_reduce_chunk with a real rope tail (64 rope
     lanes, plain and YaRN-scaled frequencies, src/graph/core.c:499-507 and

@@ -12,7 +12,7 @@ pytestmark = pytest.mark.gpu
 HEADS, KEY_DIM, VALUE_DIM, PAGE = 128, 576, 512, 64
 
 
-def make_case(rng, contexts, spare=2):
+def make_case(rng, contexts, spare=2, heads=HEADS, key_dim=KEY_DIM):
     batch = len(contexts)
     need = [(c + PAGE - 1) // PAGE for c in contexts]
     pool_pages = sum(need) + spare
@@ -22,31 +22,31 @@ def make_case(rng, contexts, spare=2):
     for b, n in enumerate(need):
         table[b, :n] = perm[at:at + n]
         at += n
-    pool = bf16_normal(rng, (pool_pages, PAGE, KEY_DIM))
-    q = bf16_normal(rng, (batch, HEADS, KEY_DIM))
+    pool = bf16_normal(rng, (pool_pages, PAGE, key_dim))
+    q = bf16_normal(rng, (batch, heads, key_dim))
     return q, pool, table, np.array(contexts, dtype=np.int32)
 
 
 def run_mla(backend, q, pool, table, ctx, max_context=None, sinks=None, window=0, compressed=None,
             selected=None, rope=None, positions=None, scale=0.0):
-    batch = q.shape[0]
+    batch, heads, key_dim = q.shape
     extra = {}
     if compressed is not None:
         extra = dict(compressed_pool_pages=compressed[0].shape[0],
                      compressed_table_stride=compressed[1].shape[1],
                      max_compressed_tokens=int(compressed[1].shape[1] * PAGE),
                      compressed_selected_stride=selected.shape[1] if selected is not None else 0)
-    req = backend.mla_requirement(batch, HEADS, KEY_DIM, VALUE_DIM, PAGE, pool.shape[0],
+    req = backend.mla_requirement(batch, heads, key_dim, VALUE_DIM, PAGE, pool.shape[0],
                                   table.shape[1], max_context or int(table.shape[1] * PAGE),
                                   sliding_window=window, output_inverse_rope=rope, scale=scale,
                                   **extra)
-    out = backend.tensor("o", B.DTYPE_BF16, (batch, HEADS, VALUE_DIM))
-    lse = backend.tensor("lse", B.DTYPE_F32, (batch, HEADS))
+    out = backend.tensor("o", B.DTYPE_BF16, (batch, heads, VALUE_DIM))
+    lse = backend.tensor("lse", B.DTYPE_F32, (batch, heads))
     tensors = [backend.tensor("q", B.DTYPE_BF16, q.shape, q),
                backend.tensor("pool", B.DTYPE_BF16, pool.shape, pool),
                backend.tensor("table", B.DTYPE_I32, table.shape, table),
                backend.tensor("ctx", B.DTYPE_I32, ctx.shape, ctx)]
-    ts = backend.tensor("sinks", B.DTYPE_F32, (HEADS,), sinks) if sinks is not None else None
+    ts = backend.tensor("sinks", B.DTYPE_F32, (heads,), sinks) if sinks is not None else None
     tc = None
     if compressed is not None:
         tc = [backend.tensor("cpool", B.DTYPE_BF16, compressed[0].shape, compressed[0]),
@@ -287,3 +287,79 @@ def test_mla_rotation_and_scale_refusals_and_explicit_scale(backend):
     got, lse, _ = run_mla(backend, half, pool, table, ctx, scale=2.0 / np.sqrt(KEY_DIM))
     assert np.array_equal(got, base)
     assert np.allclose(lse, lse0, rtol=0, atol=2e-6)
+
+
+# ------------------------------------- the reference's own reduce geometry (64 heads, 512) ----
+
+R_HEADS, R_DIM = 64, 512
+YARN = dict(rope_dimensions=64, theta=10000, scaling_factor=40, original_context=4096, beta_fast=32,
+            beta_slow=1)
+
+
+@pytest.mark.parametrize("window", [0, 128])
+def test_reduce_geometry_matches_shared_kv_oracle(backend, window):
+    """64 heads over one 512-lane row per token, key and value the same row with the rope lanes
+    inside (tests/unit/deepseek_arch_ir.c:110-125), sink logits, the model's 128-token window,
+    dense compressed rows and the output rotation: the whole reduce of src/graph/core.c:471-508."""
+    rng = np.random.default_rng(700 + window)
+    contexts = [1, 31, 33, 64, 65, 129, 500, 1300, 4097]
+    q, pool, table, ctx = make_case(rng, contexts, heads=R_HEADS, key_dim=R_DIM)
+    ratio = 128
+    stored = [n // ratio + 1 for n in contexts]
+    _, cpool, ctable, _ = make_case(rng, stored, heads=R_HEADS, key_dim=R_DIM)
+    visible = np.array([n // ratio for n in contexts], np.int32)
+    sinks = (rng.standard_normal(R_HEADS) * 3.0).astype(np.float32)
+    got, lse, facts = run_mla(backend, q, pool, table, ctx, sinks=sinks, window=window,
+                              compressed=(cpool, ctable, visible), rope=YARN)
+    assert facts.kernel_launches == 3
+    rc, ref, _, ref_lse = ORACLE.mla_decode(q, pool, table, ctx, R_DIM, PAGE, sinks=sinks,
+                                            sliding_window=window, compressed=(cpool, ctable, visible))
+    assert rc == 0
+    policy = oracle_policy(YARN)
+    for b, n in enumerate(contexts):
+        rc, want = ORACLE.reduce_output_finish(ref[b], n - 1, policy)
+        assert rc == 0
+        assert_close_bf16(got[b:b + 1], want[None], "reduce geometry b=%d window=%d" % (b, window))
+    assert_lse(lse, ref_lse, "reduce geometry window=%d" % window)
+    # the plain decode of the same geometry, and placement invariance
+    plain, lse0, facts = run_mla(backend, q, pool, table, ctx)
+    assert facts.kernel_launches == 2
+    rc, ref, _, ref_lse = ORACLE.mla_decode(q, pool, table, ctx, R_DIM, PAGE)
+    assert_close_bf16(plain, ref, "reduce geometry plain")
+    assert_lse(lse0, ref_lse, "reduce geometry plain")
+    perm = rng.permutation(pool.shape[0])
+    pool2 = np.empty_like(pool)
+    pool2[perm] = pool
+    again, lse2, _ = run_mla(backend, q, pool2, perm[table].astype(np.int32), ctx)
+    assert np.array_equal(plain, again) and np.array_equal(lse0, lse2)
+
+
+def test_reduce_geometry_against_the_reference_reduce(backend):
+    """The device result at the reference's geometry against the reference's own
+    yvex_attention_reduce_chunk: the compiled one where it was built, and its committed output
+    (tests/golden, case reduce-model-geometry) everywhere."""
+    import importlib.util
+    import os
+    here = os.path.dirname(os.path.abspath(__file__))
+    spec = importlib.util.spec_from_file_location("make_golden", os.path.join(here, "golden", "make_golden.py"))
+    golden_inputs = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(golden_inputs)
+    golden = np.load(os.path.join(here, "golden", "reference_attention.npz"), allow_pickle=False)
+    name, attention_class, window, context, stored, heads, dim, policy = golden_inputs.MODEL_GEOMETRY_CASE
+    assert (heads, dim) == (R_HEADS, R_DIM)
+    qf, local, compressed, sinks = golden_inputs.reduce_inputs(heads, dim, context, stored)
+
+    def paged(rows):
+        pages = max((len(rows) + PAGE - 1) // PAGE, 1)
+        pool = np.zeros((pages, PAGE, dim), np.uint16)
+        pool.reshape(-1, dim)[:len(rows)] = ORACLE.bf16_encode(rows)
+        return pool, np.arange(pages, dtype=np.int32)[None, :]
+
+    pool, table = paged(local)
+    cpool, ctable = paged(compressed)
+    visible = np.array([context // golden_inputs.REDUCE_RATIO], np.int32)
+    rope = dict(rope_dimensions=policy["rope_dims"], **{k: v for k, v in policy.items() if k != "rope_dims"})
+    got, _, _ = run_mla(backend, ORACLE.bf16_encode(qf)[None], pool, table, np.array([context], np.int32),
+                        sinks=sinks, window=window, compressed=(cpool, ctable, visible), rope=rope)
+    want = golden[name + "/out"]
+    assert_close_bf16(got, want[None], "reference reduce, committed output")
