@@ -330,7 +330,7 @@ static int view_ok(const yvex_backend *backend, const yvex_device_tensor *tensor
 }
 
 /* The EXACT_F32 request has two kernels.  Prefill-shaped requests (at least 32 query tokens,
- * head dimension 64 or 128, 16-byte aligned rows) run in 32 x 32 tiles on the fp32 matrix
+ * head dimension 64, 128 or 256, 16-byte aligned rows) run in 32 x 32 tiles on the fp32 matrix
  * cores with float statistics, the arithmetic of the reference's own device kernel
  * (src/backend/cuda/transformer_kernels.cu:136-208).  Everything else (single-token decode,
  * other head dimensions up to 256, unaligned views) runs one wave per (token, head) with
@@ -344,12 +344,14 @@ static int exact_tile_function(const yvex_transformer_attention_requirement *r,
                                yvex_rocm_function_id *function)
 {
     if (r->query_tokens < ROCM_EXACT_TILE_MIN_TOKENS ||
-        (r->head_dimension != 64ull && r->head_dimension != 128ull) ||
+        (r->head_dimension != 64ull && r->head_dimension != 128ull && r->head_dimension != 256ull) ||
         ((q_stride | k_stride | v_stride) & 3ull) ||
         (((uintptr_t)request->query->data | (uintptr_t)request->key->data |
           (uintptr_t)request->value->data | (uintptr_t)request->output->data) & 15u))
         return 0;
-    *function = r->head_dimension == 64ull ? YVEX_ROCM_FN_GQA_F32_TILE_64 : YVEX_ROCM_FN_GQA_F32_TILE_128;
+    *function = r->head_dimension == 64ull    ? YVEX_ROCM_FN_GQA_F32_TILE_64
+                : r->head_dimension == 128ull ? YVEX_ROCM_FN_GQA_F32_TILE_128
+                                              : YVEX_ROCM_FN_GQA_F32_TILE_256;
     return 1;
 }
 

@@ -36,6 +36,8 @@ static const rocm_kernel_binding rocm_kernel_bindings[] = {
      YVEX_ROCM_FN_GQA_F32_TILE_64},
     {"yvex_rocm_gqa_f32_tile_128", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_F32,
      YVEX_ROCM_FN_GQA_F32_TILE_128},
+    {"yvex_rocm_gqa_f32_tile_256", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_F32,
+     YVEX_ROCM_FN_GQA_F32_TILE_256},
     {"yvex_rocm_fill_u32", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_F32, YVEX_ROCM_FN_FILL_U32},
     {"yvex_rocm_stream_read", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_F32, YVEX_ROCM_FN_STREAM_READ},
     {"yvex_rocm_decode_paged_bf16", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_PAGED_BF16,

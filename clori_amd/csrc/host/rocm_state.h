@@ -14,6 +14,7 @@ typedef enum {
     YVEX_ROCM_FN_GQA_F32,
     YVEX_ROCM_FN_GQA_F32_TILE_64,
     YVEX_ROCM_FN_GQA_F32_TILE_128,
+    YVEX_ROCM_FN_GQA_F32_TILE_256,
     YVEX_ROCM_FN_FILL_U32,
     YVEX_ROCM_FN_DECODE_PAGED_BF16,
     YVEX_ROCM_FN_DECODE_ROWS_BF16,

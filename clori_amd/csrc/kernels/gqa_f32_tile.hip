@@ -60,35 +60,32 @@ struct GqaTile {
     {
     }
 
+    // This thread's 16-byte pieces of one K or V tile on their way from global memory to LDS.
     struct Staged {
-        floatx4 k[kChunks], v[kChunks];
+        floatx4 piece[kChunks];
     };
 
-    // rows of key tile `tile` for this thread; rows past the end read as zero
-    __device__ void fetch(uint64_t tile, uint64_t kv_head, Staged &s) const
+    // rows of tile `tile` of `rows` (K or V, `stride` elements per token); rows past the end
+    // read as zero
+    __device__ void fetch(const float *rows, uint64_t stride, uint64_t tile, uint64_t kv_head, Staged &s) const
     {
 #pragma unroll
         for (int j = 0; j < kChunks; ++j) {
             const int c = tid + 256 * j, row = c / (kDim / 4), piece = c % (kDim / 4);
             const uint64_t key = tile * kKeys + (uint64_t)row;
             const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
-            s.k[j] = zero;
-            s.v[j] = zero;
-            if (key < p.kv_tokens) {
-                s.k[j] = *reinterpret_cast<const floatx4 *>(p.k + key * p.k_stride + kv_head * kDim + 4 * piece);
-                s.v[j] = *reinterpret_cast<const floatx4 *>(p.v + key * p.v_stride + kv_head * kDim + 4 * piece);
-            }
+            s.piece[j] = zero;
+            if (key < p.kv_tokens)
+                s.piece[j] = *reinterpret_cast<const floatx4 *>(rows + key * stride + kv_head * kDim + 4 * piece);
         }
     }
 
-    __device__ void stage(int buffer, const Staged &s) const
+    __device__ void stage(float *tile, int row_stride, const Staged &s) const
     {
-        float *kt = lds + buffer * kStageFloats, *vt = kt + kKeys * kKStride;
 #pragma unroll
         for (int j = 0; j < kChunks; ++j) {
             const int c = tid + 256 * j, row = c / (kDim / 4), piece = c % (kDim / 4);
-            *reinterpret_cast<floatx4 *>(kt + row * kKStride + 4 * piece) = s.k[j];
-            *reinterpret_cast<floatx4 *>(vt + row * kVStride + 4 * piece) = s.v[j];
+            *reinterpret_cast<floatx4 *>(tile + row * row_stride + 4 * piece) = s.piece[j];
         }
     }
 
@@ -133,17 +130,25 @@ struct GqaTile {
             for (int i = 0; i < 16; ++i) out[b][i] = 0.f;
         float top = -INFINITY, sum = 0.f;  // running maximum (natural units), this half's share of the denominator
 
+        // The rows of tile t+1 travel in two halves so that only one tile's worth of registers
+        // is tied up: K is fetched before the first product of tile t and written to the other
+        // buffer after it, V likewise around the second product.  Every wave left both halves
+        // of that buffer at the barrier that ended tile t-1.
         Staged next;
-        fetch(0, kv_head, next);
-        stage(0, next);
+        fetch(p.k, p.k_stride, 0, kv_head, next);
+        stage(lds, kKStride, next);
+        fetch(p.v, p.v_stride, 0, kv_head, next);
+        stage(lds + kKeys * kKStride, kVStride, next);
         __syncthreads();
         for (uint64_t t = 0; t < tiles; ++t) {
             const bool more = t + 1 < tiles;
-            if (more) fetch(t + 1, kv_head, next);
-            if (t < wave_tiles) {
-                const float *kt = lds + (int)(t & 1) * kStageFloats, *vt = kt + kKeys * kKStride;
+            float *other = lds + (int)((t + 1) & 1) * kStageFloats;
+            if (more) fetch(p.k, p.k_stride, t + 1, kv_head, next);
+            const bool active = t < wave_tiles;
+            floatx16 s;
+            if (active) {
+                const float *kt = lds + (int)(t & 1) * kStageFloats;
                 // S^T (32 keys x 32 queries): the key row is the lane's column index
-                floatx16 s;
 #pragma unroll
                 for (int i = 0; i < 16; ++i) s[i] = 0.f;
                 const float *krow = kt + column * kKStride + half * kHalf;
@@ -155,6 +160,13 @@ struct GqaTile {
                     s = mfma_32x32x2(piece[2], q[step + 2], s);
                     s = mfma_32x32x2(piece[3], q[step + 3], s);
                 }
+            }
+            if (more) {
+                stage(other, kKStride, next);
+                fetch(p.v, p.v_stride, t + 1, kv_head, next);
+            }
+            if (active) {
+                const float *vt = lds + (int)(t & 1) * kStageFloats + kKeys * kKStride;
                 // lane holds keys 8 * (i / 4) + 4 * half + i % 4 of the tile for its query
                 float peak = -INFINITY;
 #pragma unroll
@@ -187,7 +199,7 @@ struct GqaTile {
                     for (int b = 0; b < kBlocks; ++b) out[b] = mfma_32x32x2(vrow[32 * b], s[i], out[b]);
                 }
             }
-            if (more) stage((int)((t + 1) & 1), next);
+            if (more) stage(other + kKeys * kKStride, kVStride, next);
             __syncthreads();
         }
 
@@ -218,13 +230,16 @@ struct GqaTile {
 
 }  // namespace
 
-#define YVEX_GQA_F32_TILE_KERNEL(name, blocks)                                                  \
-    extern "C" __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))  \
-    name(const yvex_rocm_gqa_f32_params p)                                                        \
-    {                                                                                             \
-        __shared__ __attribute__((aligned(16))) float lds[2 * GqaTile<blocks>::kStageFloats];     \
-        GqaTile<blocks>(p, lds).run();                                                            \
+// `waves`: waves per SIMD the register budget is sized for.  Head dimension 256 keeps 128
+// query and 128 accumulator registers per lane and runs one workgroup per CU.
+#define YVEX_GQA_F32_TILE_KERNEL(name, blocks, waves)                                                   \
+    extern "C" __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(waves, waves))) \
+    name(const yvex_rocm_gqa_f32_params p)                                                                \
+    {                                                                                                     \
+        __shared__ __attribute__((aligned(16))) float lds[2 * GqaTile<blocks>::kStageFloats];             \
+        GqaTile<blocks>(p, lds).run();                                                                    \
     }
 
-YVEX_GQA_F32_TILE_KERNEL(yvex_rocm_gqa_f32_tile_64, 2)
-YVEX_GQA_F32_TILE_KERNEL(yvex_rocm_gqa_f32_tile_128, 4)
+YVEX_GQA_F32_TILE_KERNEL(yvex_rocm_gqa_f32_tile_64, 2, 2)
+YVEX_GQA_F32_TILE_KERNEL(yvex_rocm_gqa_f32_tile_128, 4, 2)
+YVEX_GQA_F32_TILE_KERNEL(yvex_rocm_gqa_f32_tile_256, 8, 1)

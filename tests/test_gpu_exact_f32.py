@@ -227,6 +227,8 @@ def run_exact(backend, q, k, v, **kw):
     (32, 32, 4, 2, 64, 0, True), (33, 33, 4, 1, 128, 0, True), (128, 128, 2, 2, 128, 0, True),
     (129, 129, 5, 1, 64, 0, True), (257, 257, 8, 2, 128, 0, True), (257, 257, 8, 2, 128, 0, False),
     (100, 371, 4, 4, 64, 271, True), (40, 1000, 10, 2, 128, 960, True), (64, 95, 3, 3, 128, 0, False),
+    (32, 32, 6, 1, 256, 0, True), (161, 161, 6, 2, 256, 0, True), (70, 333, 24, 4, 256, 263, True),
+    (96, 200, 4, 4, 256, 0, False),
 ])
 def test_gqa_matrix_core_kernel_matches_cpu_operator(backend, tq, tk, hq, hkv, d, start, causal):
     """Prefill-shaped EXACT_F32 requests run in tiles on the fp32 matrix cores.  Tolerance is
