@@ -12,8 +12,9 @@ already resident in HBM.  Workloads are the five configurations the metric is qu
     paged4     32 sessions, paged Q8_0 KV, contexts U[4096,32768]        (HBM bound)
     mla5       absorbed MLA decode, batch 16, 128 heads, context 8192    (HBM bound)
 
-By name only (not configurations of the metric): exact2 (configuration 2 under the EXACT_F32
-contract, against the fp32 matrix peak), append_bf16 / append_q8_0 (the KV page writer), copy.
+By name only (not configurations of the metric): exact2 and exact1 (configurations 2 and 1
+under the EXACT_F32 contract: fp32 matrix cores, and double-precision split decode),
+append_bf16 / append_q8_0 (the KV page writer), copy.
 
 Prints ONE JSON line.  `value` is the headline workload's throughput; every workload
 that ran is listed under "workloads" with its own roofline figures.  Timing uses HIP
@@ -275,6 +276,29 @@ def workload_exact2(backend, rng, steps, warmup):
                 launches=int(facts.kernel_launches), kernels=kernels, **timed)
 
 
+def workload_exact1(backend, rng, steps, warmup):
+    """Configuration 1 under the EXACT_F32 contract: the decode step the reference's session
+    layer makes (one query token over the cached F32 history).  Run by name."""
+    hq, hkv, d, ctx = 32, 8, 128, 4096
+    q = backend.tensor("q", B.DTYPE_F32, (1, hq, d), rng.standard_normal((1, hq, d), dtype=np.float32))
+    k = backend.tensor("k", B.DTYPE_F32, (ctx, hkv, d), rng.standard_normal((ctx, hkv, d), dtype=np.float32))
+    v = backend.tensor("v", B.DTYPE_F32, (ctx, hkv, d), rng.standard_normal((ctx, hkv, d), dtype=np.float32))
+    out = backend.tensor("out", B.DTYPE_F32, (1, hq, d))
+    req = backend.attention_requirement(1, ctx, hq, hkv, d, causal=True, query_start=ctx - 1)
+    work = backend.tensor("workspace", B.DTYPE_I8, (backend.attention_workspace_required(req),))
+    backend.workspace_attach(work)
+    run = lambda: backend.attention_execute(req, q, k, v, out)  # noqa: E731
+    facts = run()
+    kernels = ["yvex_rocm_gqa_f32_split", "yvex_rocm_gqa_f32_split_merge"]
+    timed = time_steps(backend, run, steps, warmup, kernels)
+    backend.workspace_detach()
+    return dict(name="exact1",
+                workload="GQA decode, EXACT_F32 contract: batch 1, 32/8 heads, d=128, context 4096, "
+                         "contiguous f32 KV",
+                bound="hbm", algorithmic_bytes=2 * ctx * hkv * d * 4 + 2 * hq * d * 4, tokens=ctx,
+                dtype="f64", launches=int(facts.kernel_launches), kernels=kernels, **timed)
+
+
 def workload_mla5(backend, rng, steps, warmup):
     batch, heads, kd, vd, page, ctx = 16, 128, 576, 512, 64, 8192
     pages_each = ctx // page
@@ -377,9 +401,10 @@ EXTRA_WORKLOADS = {
     "append_bf16": lambda b, r, s, w: workload_append(b, r, s, w, q8=False),
     "append_q8_0": lambda b, r, s, w: workload_append(b, r, s, w, q8=True),
     "exact2": workload_exact2,
+    "exact1": workload_exact1,
 }
 SEEDS = {"decode1": 1, "prefill2": 2, "paged3": 3, "paged4": 4, "mla5": 5, "append_bf16": 6,
-         "append_q8_0": 7, "exact2": 8}
+         "append_q8_0": 7, "exact2": 8, "exact1": 9}
 
 
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
@@ -491,6 +516,13 @@ def cpu_baseline(name, budget=6.0):
         return dict(value=4 * d * hq * t * (t + 1) // 2 / dt / 1e12, unit="TFLOP/s", cores=threads,
                     kind="port", sample="the first 512 tokens of the same shape, median of %d runs "
                                         "(%.1f s)" % (runs, spent))
+    if name == "exact1":
+        q = rng.standard_normal((1, 32, 128), dtype=np.float32)
+        k = rng.standard_normal((4096, 8, 128), dtype=np.float32)
+        v = rng.standard_normal((4096, 8, 128), dtype=np.float32)
+        runs, dt, spent = repeat_for(budget / 2, lambda: oracle.gqa(q, k, v, query_start=4095)[0])
+        return dict(value=(2 * 4096 * 8 * 128 * 4) / dt / 1e9, unit="GB/s", cores=threads, kind="port",
+                    sample="the full workload, median of %d runs (%.1f s)" % (runs, spent))
     if name == "mla5":
         batch, heads, kd, vd, page, ctx = 2, 128, 576, 512, 64, 4096
         pages = batch * ctx // page

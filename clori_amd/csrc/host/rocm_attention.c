@@ -296,6 +296,73 @@ static unsigned long long visible_tokens(const yvex_transformer_attention_requir
                                                              : r->key_value_tokens;
 }
 
+/* The EXACT_F32 request has three kernels; the choice is a function of the request geometry
+ * (and of the 16-byte alignment of the views) only.
+ *   - Prefill-shaped requests (at least 32 query tokens, head dimension 64, 128 or 256) run in
+ *     32 x 32 tiles on the fp32 matrix cores with float statistics, the arithmetic of the
+ *     reference's own device kernel (src/backend/cuda/transformer_kernels.cu:136-208).
+ *   - Other requests over 512 or more keys (the decode step of the session layer,
+ *     src/runtime/stateful_attention.c:326-352) are cut into runs of keys, one wave per
+ *     (token, head, run) with double-precision statistics, and merged by a second launch.
+ *   - Everything else runs one wave per (token, head), double-precision statistics. */
+enum { ROCM_EXACT_TILE_QUERIES = 128, ROCM_EXACT_TILE_MIN_TOKENS = 32, ROCM_EXACT_SPLIT_MIN_KEYS = 512,
+       ROCM_EXACT_SPLIT_WAVES = 2048, ROCM_EXACT_SPLIT_RUN_MIN = 64 };
+
+static int exact_strides_aligned(const yvex_transformer_attention_requirement *r)
+{
+    const unsigned long long q_stride = r->query_token_stride ? r->query_token_stride
+                                                              : r->query_heads * r->head_dimension;
+    const unsigned long long kv_width = r->key_value_heads * r->head_dimension;
+    const unsigned long long k_stride = r->key_token_stride ? r->key_token_stride : kv_width;
+    const unsigned long long v_stride = r->value_token_stride ? r->value_token_stride : kv_width;
+    return ((q_stride | k_stride | v_stride) & 3ull) == 0ull;
+}
+
+static int exact_tile_geometry(const yvex_transformer_attention_requirement *r)
+{
+    return r->query_tokens >= ROCM_EXACT_TILE_MIN_TOKENS &&
+           (r->head_dimension == 64ull || r->head_dimension == 128ull || r->head_dimension == 256ull) &&
+           exact_strides_aligned(r);
+}
+
+/* Runs of the split form: 0 when the request does not take it.  keys_per_run is a multiple of
+ * 64 (the kernel's step); there are about ROCM_EXACT_SPLIT_WAVES waves in all and no run is
+ * shorter than ROCM_EXACT_SPLIT_RUN_MIN keys. */
+static unsigned long long exact_split_runs(const yvex_transformer_attention_requirement *r,
+                                           unsigned long long *keys_per_run)
+{
+    unsigned long long units, runs, per_run;
+    *keys_per_run = 0ull;
+    if (exact_tile_geometry(r) || r->key_value_tokens < ROCM_EXACT_SPLIT_MIN_KEYS ||
+        (r->head_dimension & 7ull) || r->head_dimension > 256ull || !exact_strides_aligned(r) ||
+        !yvex_core_u64_mul(r->query_tokens, r->query_heads, &units) || units > 0x7fffffffull)
+        return 0ull;
+    runs = ROCM_EXACT_SPLIT_WAVES / units ? ROCM_EXACT_SPLIT_WAVES / units : 1ull;
+    if (runs > r->key_value_tokens / ROCM_EXACT_SPLIT_RUN_MIN)
+        runs = r->key_value_tokens / ROCM_EXACT_SPLIT_RUN_MIN;
+    if (runs < 2ull) return 0ull;
+    per_run = align_up((r->key_value_tokens + runs - 1ull) / runs, 64ull);
+    runs = (r->key_value_tokens + per_run - 1ull) / per_run;
+    if (runs < 2ull || runs > 65535ull) return 0ull;
+    *keys_per_run = per_run;
+    return runs;
+}
+
+static int exact_split_workspace(const yvex_transformer_attention_requirement *r,
+                                 unsigned long long runs, unsigned long long *acc_bytes,
+                                 unsigned long long *total)
+{
+    unsigned long long slots, acc, ml;
+    if (!yvex_core_u64_mul(r->query_tokens * r->query_heads, runs, &slots) ||
+        !yvex_core_u64_mul(slots, r->head_dimension * sizeof(double), &acc) ||
+        !yvex_core_u64_mul(slots, 2ull * sizeof(double), &ml))
+        return 0;
+    acc = align_up(acc, ROCM_WORK_ALIGNMENT);
+    ml = align_up(ml, ROCM_WORK_ALIGNMENT);
+    *acc_bytes = acc;
+    return yvex_core_u64_add(acc, ml, total);
+}
+
 static int rocm_attention_workspace_required(const yvex_transformer_attention_requirement *r,
                                              unsigned long long *bytes, yvex_error *err)
 {
@@ -314,6 +381,14 @@ static int rocm_attention_workspace_required(const yvex_transformer_attention_re
                                       r->head_dimension, 1ull, &acc, &ml, &total))
             return refuse(err, YVEX_ERR_BOUNDS, where, "decode workspace geometry overflowed");
         *bytes = total;
+    } else if (r->numeric_contract == YVEX_TRANSFORMER_ATTENTION_NUMERIC_EXACT_F32) {
+        unsigned long long per_run;
+        const unsigned long long runs = exact_split_runs(r, &per_run);
+        if (runs) {
+            if (!exact_split_workspace(r, runs, &acc, &total))
+                return refuse(err, YVEX_ERR_BOUNDS, where, "attention workspace geometry overflowed");
+            *bytes = total;
+        }
     }
     yvex_error_clear(err);
     return YVEX_OK;
@@ -329,23 +404,13 @@ static int view_ok(const yvex_backend *backend, const yvex_device_tensor *tensor
            tensor->bytes == bytes;
 }
 
-/* The EXACT_F32 request has two kernels.  Prefill-shaped requests (at least 32 query tokens,
- * head dimension 64, 128 or 256, 16-byte aligned rows) run in 32 x 32 tiles on the fp32 matrix
- * cores with float statistics, the arithmetic of the reference's own device kernel
- * (src/backend/cuda/transformer_kernels.cu:136-208).  Everything else (single-token decode,
- * other head dimensions up to 256, unaligned views) runs one wave per (token, head) with
- * double-precision statistics.  The choice is a function of the request geometry only. */
-enum { ROCM_EXACT_TILE_QUERIES = 128, ROCM_EXACT_TILE_MIN_TOKENS = 32 };
-
 static int exact_tile_function(const yvex_transformer_attention_requirement *r,
                                unsigned long long q_stride, unsigned long long k_stride,
                                unsigned long long v_stride,
                                const yvex_transformer_attention_request *request,
                                yvex_rocm_function_id *function)
 {
-    if (r->query_tokens < ROCM_EXACT_TILE_MIN_TOKENS ||
-        (r->head_dimension != 64ull && r->head_dimension != 128ull && r->head_dimension != 256ull) ||
-        ((q_stride | k_stride | v_stride) & 3ull) ||
+    if (!exact_tile_geometry(r) || ((q_stride | k_stride | v_stride) & 3ull) ||
         (((uintptr_t)request->query->data | (uintptr_t)request->key->data |
           (uintptr_t)request->value->data | (uintptr_t)request->output->data) & 15u))
         return 0;
@@ -409,7 +474,9 @@ static int attention_execute_common(yvex_backend *backend,
     if (exact) {
         yvex_rocm_gqa_f32_params params;
         yvex_rocm_function_id tile_function = YVEX_ROCM_FN_GQA_F32;
-        int tiled = 0;
+        unsigned long long split_runs = 0ull, split_keys = 0ull, split_bytes = 0ull;
+        void *split_work = NULL;
+        int tiled = 0, split_owned = 0;
         memset(&params, 0, sizeof(params));
         params.q = (const float *)request->query->data;
         params.k = (const float *)request->key->data;
@@ -440,17 +507,55 @@ static int attention_execute_common(yvex_backend *backend,
                                   (unsigned int)groups, 1u, 1u, 256u, 0u, &params,
                                   "rocm.transformer.gqa", err);
             tiled = 1;
+        } else if ((split_runs = exact_split_runs(r, &split_keys)) != 0ull &&
+                   !(((uintptr_t)request->query->data | (uintptr_t)request->key->data |
+                      (uintptr_t)request->value->data) & 15u)) {
+            /* runs of keys, one wave per (token, head, run), then the merge */
+            unsigned long long acc_bytes = 0ull;
+            if (!exact_split_workspace(r, split_runs, &acc_bytes, &split_bytes))
+                return refuse(err, YVEX_ERR_BOUNDS, "rocm.transformer.gqa",
+                              "attention workspace geometry overflowed");
+            rc = yvex_rocm_temporary_acquire(backend, split_bytes, &split_work, &split_owned,
+                                             "rocm.transformer.gqa", err);
+            if (rc != YVEX_OK) return rc;
+            params.part_acc = (double *)split_work;
+            params.part_ml = (double *)((unsigned char *)split_work + acc_bytes);
+            params.splits = (uint32_t)split_runs;
+            params.keys_per_split = (uint32_t)split_keys;
+            rc = yvex_rocm_launch(backend,
+                                  r->head_dimension > 128ull ? YVEX_ROCM_FN_GQA_F32_SPLIT_WIDE
+                                                             : YVEX_ROCM_FN_GQA_F32_SPLIT,
+                                  YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_F32, (unsigned int)rows,
+                                  (unsigned int)split_runs, 1u, 64u, 0u, &params,
+                                  "rocm.transformer.gqa", err);
+            if (rc == YVEX_OK)
+                rc = yvex_rocm_launch(backend, YVEX_ROCM_FN_GQA_F32_SPLIT_MERGE,
+                                      YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_F32, (unsigned int)rows,
+                                      1u, 1u, 256u, 0u, &params, "rocm.transformer.gqa", err);
         } else {
+            split_runs = 0ull;
             rc = yvex_rocm_launch(backend, YVEX_ROCM_FN_GQA_F32,
                                   YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_F32, (unsigned int)rows, 1u,
                                   1u, 64u, 0u, &params, "rocm.transformer.gqa", err);
         }
         if (rc == YVEX_OK) {
-            facts->kernel_launches = 1ull;
+            facts->kernel_launches = split_work ? 2ull : 1ull;
             facts->accelerated_matrix_launches = tiled ? 1ull : 0ull;
+            facts->temporary_bytes = split_bytes;
             facts->compulsory_memory_facts_available = 1;
             rc = yvex_rocm_complete(backend, YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_F32,
                                     "rocm.transformer.gqa", facts, err);
+        }
+        if (split_work) {
+            yvex_error cleanup;
+            int cleanup_rc;
+            yvex_error_clear(&cleanup);
+            cleanup_rc = yvex_rocm_temporary_release(backend, split_work, split_bytes, split_owned, &cleanup);
+            backend_workspace_reset(backend);
+            if (rc == YVEX_OK && cleanup_rc != YVEX_OK) {
+                rc = cleanup_rc;
+                if (err) *err = cleanup;
+            }
         }
     } else if (r->query_tokens == 1ull) {
         decode_job job;

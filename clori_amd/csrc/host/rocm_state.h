@@ -12,6 +12,9 @@
 typedef enum {
     YVEX_ROCM_FN_ATTENTION_F32 = 0,
     YVEX_ROCM_FN_GQA_F32,
+    YVEX_ROCM_FN_GQA_F32_SPLIT,
+    YVEX_ROCM_FN_GQA_F32_SPLIT_WIDE,
+    YVEX_ROCM_FN_GQA_F32_SPLIT_MERGE,
     YVEX_ROCM_FN_GQA_F32_TILE_64,
     YVEX_ROCM_FN_GQA_F32_TILE_128,
     YVEX_ROCM_FN_GQA_F32_TILE_256,

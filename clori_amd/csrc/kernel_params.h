@@ -33,6 +33,11 @@ typedef struct {
     uint64_t q_stride, k_stride, v_stride;
     float scale;
     int32_t causal;
+    /* split form (yvex_rocm_gqa_f32_split + _merge): the keys a query sees are cut into
+     * `splits` runs of keys_per_split; part_acc is F64 [Tq*Hq][splits][head_dim], part_ml
+     * F64 [Tq*Hq][splits][2] = (running maximum, denominator) */
+    double *part_acc, *part_ml;
+    uint32_t splits, keys_per_split;
 } yvex_rocm_gqa_f32_params;
 
 typedef struct {

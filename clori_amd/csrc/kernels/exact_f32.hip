@@ -168,6 +168,272 @@ yvex_rocm_gqa_f32(const yvex_rocm_gqa_f32_params p)
     if (p.lse && lane == 0) p.lse[token * p.query_heads + head] = (float)(m + log(l));
 }
 
+__device__ inline float wave_max_f32(float v)
+{
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
+    return v;
+}
+
+// Sum of a double over the 16 lanes of a DPP row, left in all 16: lane exchanges on the vector
+// ALU (quad permutes, then the half-row and row mirrors), no trip through the LDS permute
+// network.  The order of the additions differs from lane to lane only by commutation, so all
+// 16 lanes hold the same bits.
+template <int kControl>
+__device__ inline double dpp_exchange(double v)
+{
+    const uint64_t bits = __builtin_bit_cast(uint64_t, v);
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(uint32_t)bits, kControl, 0xf, 0xf, true);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(uint32_t)(bits >> 32), kControl, 0xf, 0xf, true);
+    return __builtin_bit_cast(double, (uint64_t)lo | ((uint64_t)hi << 32));
+}
+
+__device__ inline double row_sum(double v)
+{
+    v += dpp_exchange<0xB1>(v);   // quad_perm [1,0,3,2]
+    v += dpp_exchange<0x4E>(v);   // quad_perm [2,3,0,1]
+    v += dpp_exchange<0x141>(v);  // row_half_mirror: the other quad of the half row
+    v += dpp_exchange<0x140>(v);  // row_mirror: the other half of the row
+    return v;
+}
+
+// Decode-shaped EXACT_F32 requests over long contexts: the same arithmetic as
+// yvex_rocm_gqa_f32 (double dot products, the score rounded to float, double exponentials,
+// denominator and accumulators), but the keys a query sees are cut into `splits` runs, one wave
+// per (query token, query head, run), and the runs are merged by yvex_rocm_gqa_f32_split_merge.
+// Inside a run a wave takes 64 keys at a time, four keys per step: the 16 lanes of a group
+// hold 8 head dims each (kPieces = 2 such pieces above 128 dims), so a key or value row is one
+// contiguous read of the group.  The dot product is reduced over the group, lane `piece` of
+// the group keeps the score of the group's key of step `piece` (all 64 keys of the tile, one
+// per lane, for the statistics), and the value sum runs over the same steps with the weight
+// fetched from that lane; the four groups' sums are added once at the end.
+// The rows of several steps are fetched before the first is used, with no branch in between:
+// a key past the run reads the run's last key (its score is masked, its weight is zero), a
+// lane past the head dimension reads the row's last 8 dims against a zero query and its
+// sums are never stored.
+// grid = (query_tokens * query_heads, splits), block 64; head_dim % 8 == 0, <= 128 * kPieces.
+template <int kPieces>
+__device__ __forceinline__ void gqa_f32_split(const yvex_rocm_gqa_f32_params &p)
+{
+    typedef float floatx4 __attribute__((ext_vector_type(4)));
+    constexpr int kBatch = 8 / kPieces;  // steps whose rows are in flight together
+    const int lane = threadIdx.x;
+    const int group = lane >> 4, piece = lane & 15;
+    const uint64_t unit = blockIdx.x, split = blockIdx.y;
+    const uint64_t token = unit / p.query_heads, head = unit % p.query_heads;
+    const uint64_t kv_head = head / (p.query_heads / p.kv_heads);
+    const uint64_t visible = p.causal ? min(p.kv_tokens, p.query_start + token + 1) : p.kv_tokens;
+    const uint64_t d = p.head_dim;
+    const uint64_t k0 = split * p.keys_per_split, k1 = min(visible, k0 + (uint64_t)p.keys_per_split);
+    const uint64_t slot = unit * p.splits + split;
+    uint64_t dim[kPieces];   // first of this lane's 8 dims in piece j, clamped into the row
+    bool live[kPieces];
+#pragma unroll
+    for (int j = 0; j < kPieces; ++j) {
+        const uint64_t want = (uint64_t)piece * 8u + 128u * (uint64_t)j;
+        live[j] = want < d;
+        dim[j] = live[j] ? want : d - 8u;
+    }
+
+    double q[kPieces][8];
+    {
+        const float *row = p.q + token * p.q_stride + head * d;
+#pragma unroll
+        for (int j = 0; j < kPieces; ++j) {
+            const floatx4 a = *reinterpret_cast<const floatx4 *>(row + dim[j]);
+            const floatx4 b = *reinterpret_cast<const floatx4 *>(row + dim[j] + 4u);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                q[j][e] = live[j] ? (double)a[e] : 0.0;
+                q[j][4 + e] = live[j] ? (double)b[e] : 0.0;
+            }
+        }
+    }
+    double acc[kPieces][8];
+#pragma unroll
+    for (int j = 0; j < kPieces; ++j)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[j][e] = 0.0;
+    double m = -INFINITY, l = 0.0;
+    if (k0 < k1) {
+        const float *kbase = p.k + kv_head * d, *vbase = p.v + kv_head * d;
+        for (uint64_t tile = k0; tile < k1; tile += 64u) {
+            // scores: step `it` handles keys tile + 4 * it + group
+            float mine = -INFINITY;
+#pragma unroll
+            for (int it0 = 0; it0 < 16; it0 += kBatch) {
+                floatx4 ra[kBatch][kPieces], rb[kBatch][kPieces];
+#pragma unroll
+                for (int u = 0; u < kBatch; ++u) {
+                    const uint64_t key = min(tile + (uint64_t)(4 * (it0 + u) + group), k1 - 1u);
+#pragma unroll
+                    for (int j = 0; j < kPieces; ++j) {
+                        const float *at = kbase + key * p.k_stride + dim[j];
+                        ra[u][j] = *reinterpret_cast<const floatx4 *>(at);
+                        rb[u][j] = *reinterpret_cast<const floatx4 *>(at + 4u);
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < kBatch; ++u) {
+                    double part = 0.0;
+#pragma unroll
+                    for (int j = 0; j < kPieces; ++j)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            part += q[j][e] * (double)ra[u][j][e];
+                            part += q[j][4 + e] * (double)rb[u][j][e];
+                        }
+                    part = row_sum(part);
+                    const bool seen = tile + (uint64_t)(4 * (it0 + u) + group) < k1;
+                    const float s = seen ? (float)(part * (double)p.scale) : -INFINITY;
+                    if (piece == it0 + u) mine = s;
+                }
+            }
+            // lane (group, piece) now holds the score of key tile + 4 * piece + group
+            const double m_new = fmax(m, (double)wave_max_f32(mine));
+            const double alpha = exp(m - m_new);
+            const double w = mine == -INFINITY ? 0.0 : exp((double)mine - m_new);
+            l = l * alpha + wave_sum(w);
+#pragma unroll
+            for (int j = 0; j < kPieces; ++j)
+#pragma unroll
+                for (int e = 0; e < 8; ++e) acc[j][e] *= alpha;
+            m = m_new;
+#pragma unroll
+            for (int it0 = 0; it0 < 16; it0 += kBatch) {
+                floatx4 ra[kBatch][kPieces], rb[kBatch][kPieces];
+#pragma unroll
+                for (int u = 0; u < kBatch; ++u) {
+                    const uint64_t key = min(tile + (uint64_t)(4 * (it0 + u) + group), k1 - 1u);
+#pragma unroll
+                    for (int j = 0; j < kPieces; ++j) {
+                        const float *at = vbase + key * p.v_stride + dim[j];
+                        ra[u][j] = *reinterpret_cast<const floatx4 *>(at);
+                        rb[u][j] = *reinterpret_cast<const floatx4 *>(at + 4u);
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < kBatch; ++u) {
+                    const double wi = __shfl(w, (lane & 48) + it0 + u, kWave);  // 0 past the run
+#pragma unroll
+                    for (int j = 0; j < kPieces; ++j)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            acc[j][e] += wi * (double)ra[u][j][e];
+                            acc[j][4 + e] += wi * (double)rb[u][j][e];
+                        }
+                }
+            }
+        }
+    }
+    // the four key groups hold partial sums of the same dims
+#pragma unroll
+    for (int j = 0; j < kPieces; ++j)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            acc[j][e] += __shfl_xor(acc[j][e], 16, kWave);
+            acc[j][e] += __shfl_xor(acc[j][e], 32, kWave);
+        }
+    if (group == 0) {
+#pragma unroll
+        for (int j = 0; j < kPieces; ++j)
+            if (live[j])
+#pragma unroll
+                for (int e = 0; e < 8; ++e) p.part_acc[slot * d + dim[j] + (uint64_t)e] = acc[j][e];
+    }
+    if (lane == 0) {
+        p.part_ml[slot * 2u] = m;  // -inf for a run without visible keys
+        p.part_ml[slot * 2u + 1u] = l;
+    }
+}
+
+extern "C" __global__ void __launch_bounds__(64)
+yvex_rocm_gqa_f32_split(const yvex_rocm_gqa_f32_params p)
+{
+    gqa_f32_split<1>(p);
+}
+
+extern "C" __global__ void __launch_bounds__(64)
+yvex_rocm_gqa_f32_split_wide(const yvex_rocm_gqa_f32_params p)
+{
+    gqa_f32_split<2>(p);
+}
+
+// Merge of the runs of one (query token, query head).  Every wave reads the statistics of
+// all runs (64 at a time, one run per lane) and finds the common maximum; wave w then sums the
+// rows of the runs w, w + 4, ... with lane = head dims lane, lane + 64, ..., eight runs in
+// flight, and wave 0 adds the four partial sums through LDS in wave order.
+// grid = query_tokens * query_heads, block 256.
+extern "C" __global__ void __launch_bounds__(256)
+yvex_rocm_gqa_f32_split_merge(const yvex_rocm_gqa_f32_params p)
+{
+    __shared__ double partial[4][5][64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint64_t unit = blockIdx.x, d = p.head_dim;
+    const double *ml = p.part_ml + unit * p.splits * 2u;
+    const double *rows = p.part_acc + unit * p.splits * d;
+    double top = -INFINITY;
+    for (uint32_t base = 0; base < p.splits; base += 64u) {
+        const uint32_t s = base + (uint32_t)lane;
+        top = fmax(top, wave_max(s < p.splits ? ml[s * 2u] : -INFINITY));
+    }
+    double total = 0.0, acc[4] = {0.0, 0.0, 0.0, 0.0};
+    for (uint32_t base = 0; base < p.splits; base += 64u) {
+        const uint32_t s = base + (uint32_t)lane;
+        const double m = s < p.splits ? ml[s * 2u] : -INFINITY;
+        // a run past the visible keys left (-inf, 0): weight zero
+        const double w = m == -INFINITY ? 0.0 : exp(m - top);
+        // this wave's runs only: s % 4 == wave
+        total += wave_sum(s < p.splits && (s & 3u) == (uint32_t)wave ? w * ml[s * 2u + 1u] : 0.0);
+        const uint32_t count = min(64u, p.splits - base);
+        for (uint32_t i0 = (uint32_t)wave; i0 < count; i0 += 32u) {
+            double wi[8], part[8][4];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const uint32_t want = i0 + 4u * (uint32_t)u;
+                const uint32_t i = min(want, count - 1u);
+                wi[u] = want < count ? __shfl(w, (int)i, kWave) : 0.0;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const uint64_t c = (uint64_t)lane + 64u * (uint64_t)j;
+                    part[u][j] = c < d ? rows[(uint64_t)(base + i) * d + c] : 0.0;
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[j] += wi[u] * part[u][j];
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) partial[wave][j][lane] = acc[j];
+    partial[wave][4][lane] = total;
+    __syncthreads();
+    if (wave != 0) return;
+    total = ((partial[0][4][lane] + partial[1][4][lane]) + partial[2][4][lane]) + partial[3][4][lane];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+        acc[j] = ((partial[0][j][lane] + partial[1][j][lane]) + partial[2][j][lane]) + partial[3][j][lane];
+    if (!(total > 0.0) || !isfinite(total) || !isfinite(top)) {
+        if (lane == 0) flag(p.status, YVEX_ROCM_DEVICE_NUMERIC);
+        return;
+    }
+    const uint64_t token = unit / p.query_heads, head = unit % p.query_heads;
+    float *out = p.out + (token * p.query_heads + head) * d;
+    bool bad = false;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const uint64_t c = (uint64_t)lane + 64u * (uint64_t)j;
+        if (c < d) {
+            const float o = (float)(acc[j] / total);
+            bad |= !isfinite(o);
+            out[c] = o;
+        }
+    }
+    if (bad) flag(p.status, YVEX_ROCM_DEVICE_NUMERIC);
+    if (p.lse && lane == 0) p.lse[token * p.query_heads + head] = (float)(top + log(total));
+}
+
 // Word fill, used instead of a memset node so the clear can be recorded in a graph.
 extern "C" __global__ void __launch_bounds__(256)
 yvex_rocm_fill_u32(const yvex_rocm_fill_params p)

@@ -321,3 +321,72 @@ def test_gqa_matrix_core_kernel_config2_shape(backend):
     want = np.repeat(mean, hq // hkv, axis=1)
     assert np.abs(out - want).max() < 1e-5
     assert np.abs(lse - np.log(np.arange(1, t + 1))[:, None]).max() < 1e-5
+
+
+# ------------------------------------------------ decode-shaped requests over long contexts ----
+
+@pytest.mark.parametrize("tq,tk,hq,hkv,d,causal", [
+    (1, 4096, 32, 8, 128, True), (1, 600, 4, 4, 64, True), (4, 5000, 6, 2, 96, True),
+    (2, 1024, 3, 1, 256, True), (1, 513, 2, 2, 8, True), (3, 2000, 4, 2, 128, False),
+    (31, 700, 2, 1, 40, True), (1, 16384, 8, 8, 128, True),
+])
+def test_gqa_split_runs_match_cpu_operator(backend, tq, tk, hq, hkv, d, causal):
+    """The decode step of the session layer under the exact contract (one or a few query tokens
+    over the whole cached history, src/runtime/stateful_attention.c:326-352): the keys are cut
+    into runs, one wave per (token, head, run), double statistics, merged by a second launch.
+    Same tight bound against the CPU operator as the row kernel."""
+    rng = np.random.default_rng(tq * 7 + tk + d)
+    q = rng.standard_normal((tq, hq, d)).astype(np.float32)
+    k = rng.standard_normal((tk, hkv, d)).astype(np.float32)
+    v = rng.standard_normal((tk, hkv, d)).astype(np.float32)
+    start = tk - tq if causal else 0
+    out, lse, facts = run_exact(backend, q, k, v, query_start=start, causal=causal)
+    assert facts.kernel_launches == 2 and facts.accelerated_matrix_launches == 0
+    assert facts.temporary_bytes > 0
+    rc, ref, ref_lse = ORACLE.gqa(q, k, v, query_start=start, causal=causal)
+    assert rc == 0
+    assert np.abs(out - ref).max() < 2e-6, np.abs(out - ref).max()
+    assert np.abs(lse - ref_lse).max() < 1e-5
+    again, _, _ = run_exact(backend, q, k, v, query_start=start, causal=causal)
+    assert np.array_equal(out, again)
+    # with an attached workspace of the advertised size: no temporary, same bits
+    req = backend.attention_requirement(tq, tk, hq, hkv, d, query_start=start, causal=causal)
+    need = backend.attention_workspace_required(req)
+    assert need == facts.temporary_bytes
+    work = backend.tensor("work", B.DTYPE_I8, (need,))
+    backend.workspace_attach(work)
+    before = backend.memory_stats().allocation_events
+    attached, _, facts2 = run_exact(backend, q, k, v, query_start=start, causal=causal)
+    assert backend.memory_stats().allocation_events == before + 5      # the five tensors of run_exact
+    backend.workspace_detach()
+    work.release()
+    assert np.array_equal(out, attached) and facts2.kernel_launches == 2
+
+
+def test_gqa_split_threshold_and_failures(backend):
+    rng = np.random.default_rng(80)
+    q = rng.standard_normal((1, 4, 64)).astype(np.float32)
+    k = rng.standard_normal((511, 2, 64)).astype(np.float32)
+    v = rng.standard_normal((511, 2, 64)).astype(np.float32)
+    out, _, facts = run_exact(backend, q, k, v, query_start=510)
+    assert facts.kernel_launches == 1 and facts.temporary_bytes == 0     # short history: the row kernel
+    rc, ref, _ = ORACLE.gqa(q, k, v, query_start=510)
+    assert np.abs(out - ref).max() < 2e-6
+    k = rng.standard_normal((2048, 2, 64)).astype(np.float32)
+    v = rng.standard_normal((2048, 2, 64)).astype(np.float32)
+    bad = k.copy()
+    bad[1500, 1, 7] = np.inf
+    with pytest.raises(YvexError) as e:
+        run_exact(backend, q, bad, v, query_start=2047)
+    assert e.value.code == B.YVEX_ERR_FORMAT
+    bad = v.copy()
+    bad[3, 0, 63] = np.nan
+    with pytest.raises(YvexError) as e:
+        run_exact(backend, q, k, bad, query_start=2047)
+    assert e.value.code == B.YVEX_ERR_FORMAT
+    good, _, facts = run_exact(backend, q, k, v, query_start=2047)
+    assert facts.kernel_launches == 2 and np.all(np.isfinite(good))
+    # a query in the middle of the history: runs past its visible keys contribute nothing
+    mid, _, _ = run_exact(backend, q, k, v, query_start=700)
+    rc, ref, _ = ORACLE.gqa(q, k[:701], v[:701], query_start=700)
+    assert np.abs(mid - ref).max() < 2e-6
