@@ -212,6 +212,19 @@ __device__ inline double row_sum(double v)
 // lane past the head dimension reads the row's last 8 dims against a zero query and its
 // sums are never stored.
 // grid = (query_tokens * query_heads, splits), block 64; head_dim % 8 == 0, <= 128 * kPieces.
+// Which (token, head) workgroup `unit` of a launch row works on.  Consecutive workgroup ids go
+// to consecutive XCDs, each with its own L2; when the head count is a multiple of eight the
+// heads are dealt so that an XCD gets a contiguous eighth of them, i.e. the query heads that
+// share a KV head read its rows through one L2 (dealt in order, the four heads of a group sat
+// on four XCDs and the history was fetched from memory four times).
+__device__ __forceinline__ void split_unit(const yvex_rocm_gqa_f32_params &p, uint64_t unit, uint64_t &token,
+                                           uint64_t &head)
+{
+    token = unit / p.query_heads;
+    head = unit % p.query_heads;
+    if ((p.query_heads & 7u) == 0u) head = (head & 7u) * (p.query_heads >> 3) + (head >> 3);
+}
+
 template <int kPieces>
 __device__ __forceinline__ void gqa_f32_split(const yvex_rocm_gqa_f32_params &p)
 {
@@ -220,7 +233,8 @@ __device__ __forceinline__ void gqa_f32_split(const yvex_rocm_gqa_f32_params &p)
     const int lane = threadIdx.x;
     const int group = lane >> 4, piece = lane & 15;
     const uint64_t unit = blockIdx.x, split = blockIdx.y;
-    const uint64_t token = unit / p.query_heads, head = unit % p.query_heads;
+    uint64_t token, head;
+    split_unit(p, unit, token, head);
     const uint64_t kv_head = head / (p.query_heads / p.kv_heads);
     const uint64_t visible = p.causal ? min(p.kv_tokens, p.query_start + token + 1) : p.kv_tokens;
     const uint64_t d = p.head_dim;
@@ -418,7 +432,8 @@ yvex_rocm_gqa_f32_split_merge(const yvex_rocm_gqa_f32_params p)
         if (lane == 0) flag(p.status, YVEX_ROCM_DEVICE_NUMERIC);
         return;
     }
-    const uint64_t token = unit / p.query_heads, head = unit % p.query_heads;
+    uint64_t token, head;
+    split_unit(p, unit, token, head);
     float *out = p.out + (token * p.query_heads + head) * d;
     bool bad = false;
 #pragma unroll
