@@ -221,7 +221,9 @@ def workload_decode1(backend, rng, steps, warmup):
     backend.workspace_attach(work)
     run = lambda: backend.attention_execute(req, q, k, v, out, lse=lse)  # noqa: E731
     facts = run()
-    kernels = decode_kernels("yvex_rocm_decode_rows_bf16", facts)
+    # one launch: teams of eight waves per stretch of the history, merged through LDS and then
+    # between the teams by the one that arrives last
+    kernels = ["yvex_rocm_decode_rows_bf16_team"]
     timed = time_steps(backend, run, steps, warmup, kernels)
     backend.workspace_detach()
     algo = 2 * ctx * hkv * d * 2 + 2 * hq * d * 2 + hq * 4

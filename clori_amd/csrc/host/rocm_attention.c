@@ -26,6 +26,10 @@ enum {
     ROCM_GROUP_MAX = 16,
     ROCM_DECODE_WAVES = 2048,
     ROCM_DECODE_MIN_TILES = 8, /* 8 and 16 measure alike on a 4096-token context; 4 and 32 are a third slower */
+    ROCM_TEAM_WAVES = 8,       /* waves of a decode team (one workgroup) */
+    ROCM_TEAM_TILES = 2,       /* tiles a wave of a team is given when the history is short enough (context 4096: 10.3 us; 1: 11.6, 4: 11.9, 8: 15.9) */
+    ROCM_TEAMS_MAX = 32,       /* teams per (session, kv head): two load trips of the last team's merge */
+    ROCM_TEAM_GROUP_MAX = 8,   /* query heads per kv head a team's LDS holds */
     ROCM_PREFILL_ROWS = YVEX_ROCM_PREFILL_ROWS, /* query rows per prefill workgroup */
     ROCM_WORK_ALIGNMENT = 256    /* src/backend/cuda/transformer.c:17 */
 };
@@ -126,6 +130,19 @@ static int decode_workspace_bytes(unsigned long long slots, unsigned long long h
  * one is bound by launch latency and merges inside the decode kernel (arrival counters). */
 static int decode_merges_in_kernel(unsigned int waves) { return waves < ROCM_DECODE_WAVES; }
 
+/* Teams per (session, kv head) of the token-major decode, 0 when that form does not apply
+ * (paged pools, wide groups).  A pure function of the request geometry. */
+static unsigned int decode_team_count(int paged, unsigned long long group, unsigned long long head_dim,
+                                      unsigned long long max_context)
+{
+    const unsigned long long tiles = (max_context + ROCM_PAGE_TOKENS - 1ull) / ROCM_PAGE_TOKENS;
+    unsigned long long teams = (tiles + ROCM_TEAM_WAVES * ROCM_TEAM_TILES - 1ull) /
+                               (ROCM_TEAM_WAVES * ROCM_TEAM_TILES);
+    if (paged || group > ROCM_TEAM_GROUP_MAX || head_dim != ROCM_MFMA_HEAD_DIM) return 0u;
+    if (teams > ROCM_TEAMS_MAX) teams = ROCM_TEAMS_MAX;
+    return (unsigned int)(teams ? teams : 1ull);
+}
+
 /* Balanced decode: two partial slots per wave, then (two-kernel form) the per-session offset
  * table. */
 static int balanced_workspace_bytes(unsigned long long waves, unsigned long long group,
@@ -167,7 +184,9 @@ static int decode_run(yvex_backend *backend, const decode_job *job, const char *
     unsigned long long acc_bytes = 0ull, ml_bytes = 0ull, total = 0ull, items;
     const unsigned long long group = job->query_heads / job->kv_heads;
     const unsigned int waves = decode_wave_count(job->sessions, job->kv_heads, job->max_context);
-    const int in_kernel = decode_merges_in_kernel(waves);
+    const unsigned int teams = decode_team_count(job->page_table != NULL, group, job->head_dim,
+                                                 job->max_context);
+    const int in_kernel = teams || decode_merges_in_kernel(waves);
     void *work = NULL;
     yvex_error cleanup;
     int owned = 0, rc, cleanup_rc;
@@ -175,8 +194,10 @@ static int decode_run(yvex_backend *backend, const decode_job *job, const char *
                            (job->max_context + ROCM_PAGE_TOKENS - 1ull) / ROCM_PAGE_TOKENS, &items) ||
         items > 0x7fffffffull || job->sessions > 65535ull || job->query_heads > 65535ull ||
         (in_kernel && job->sessions * job->kv_heads > YVEX_ROCM_DECODE_SEGMENTS_MAX) ||
-        !balanced_workspace_bytes(waves, group, job->head_dim, job->sessions, &acc_bytes,
-                                  &ml_bytes, &total))
+        !(teams ? decode_workspace_bytes(job->sessions * job->kv_heads * teams, group, job->head_dim,
+                                         sizeof(float), &acc_bytes, &total)
+                : balanced_workspace_bytes(waves, group, job->head_dim, job->sessions, &acc_bytes,
+                                           &ml_bytes, &total)))
         return refuse(err, YVEX_ERR_BOUNDS, where, "decode geometry exceeds admitted integer range");
     backend_workspace_reset(backend);
     if (job->fixed_work) {
@@ -215,8 +236,13 @@ static int decode_run(yvex_backend *backend, const decode_job *job, const char *
     dp.fixed_context = (uint32_t)job->fixed_context;
     dp.waves = waves;
     dp.scale_log2 = job->scale * 1.4426950408889634f;
-    rc = yvex_rocm_launch(backend, in_kernel ? job->merged_function : job->function, job->variant,
-                          waves, 1u, 1u, 64u, 0u, &dp, where, err);
+    if (teams) /* teams of eight waves, merged through LDS and then between the teams */
+        rc = yvex_rocm_launch(backend, YVEX_ROCM_FN_DECODE_ROWS_BF16_TEAM, job->variant, teams,
+                              (unsigned int)job->kv_heads, (unsigned int)job->sessions,
+                              64u * ROCM_TEAM_WAVES, 0u, &dp, where, err);
+    else
+        rc = yvex_rocm_launch(backend, in_kernel ? job->merged_function : job->function, job->variant,
+                              waves, 1u, 1u, 64u, 0u, &dp, where, err);
     if (rc == YVEX_OK && !in_kernel)
         rc = yvex_rocm_launch(backend, YVEX_ROCM_FN_DECODE_FINISH, job->variant,
                               (unsigned int)job->query_heads, (unsigned int)job->sessions, 1u,
@@ -377,8 +403,11 @@ static int rocm_attention_workspace_required(const yvex_transformer_attention_re
         r->query_tokens == 1ull) {
         /* split-K decode partials; geometry must match decode_run */
         const unsigned int waves = decode_wave_count(1ull, r->key_value_heads, visible_tokens(r));
-        if (!balanced_workspace_bytes(waves, r->query_heads / r->key_value_heads,
-                                      r->head_dimension, 1ull, &acc, &ml, &total))
+        const unsigned long long group = r->query_heads / r->key_value_heads;
+        const unsigned int teams = decode_team_count(0, group, r->head_dimension, visible_tokens(r));
+        if (!(teams ? decode_workspace_bytes(r->key_value_heads * teams, group, r->head_dimension,
+                                             sizeof(float), &acc, &total)
+                    : balanced_workspace_bytes(waves, group, r->head_dimension, 1ull, &acc, &ml, &total)))
             return refuse(err, YVEX_ERR_BOUNDS, where, "decode workspace geometry overflowed");
         *bytes = total;
     } else if (r->numeric_contract == YVEX_TRANSFORMER_ATTENTION_NUMERIC_EXACT_F32) {

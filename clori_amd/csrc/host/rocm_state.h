@@ -28,6 +28,7 @@ typedef enum {
     YVEX_ROCM_FN_DECODE_PAGED_BF16_MERGED,
     YVEX_ROCM_FN_DECODE_PAGED_Q8_0_MERGED,
     YVEX_ROCM_FN_DECODE_ROWS_BF16_MERGED,
+    YVEX_ROCM_FN_DECODE_ROWS_BF16_TEAM,
     YVEX_ROCM_FN_PREFILL_BF16,
     YVEX_ROCM_FN_MLA_DECODE_BF16,
     YVEX_ROCM_FN_MLA_DECODE_512_BF16,

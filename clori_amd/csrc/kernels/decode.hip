@@ -74,6 +74,17 @@ __device__ inline void store_b64_device(void *p, float a, float b)
     __hip_atomic_store(reinterpret_cast<uint64_t *>(p), __builtin_bit_cast(uint64_t, v),
                        __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
+// The matching load: sees the write-through stores of the other XCDs without an L2
+// invalidate.
+__device__ inline void load_b64_device(const void *p, float &a, float &b)
+{
+    typedef float floatx2 __attribute__((ext_vector_type(2)));
+    const floatx2 v = __builtin_bit_cast(
+        floatx2, __hip_atomic_load(reinterpret_cast<const uint64_t *>(p), __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT));
+    a = v.x;
+    b = v.y;
+}
 __device__ inline void store_b128_device(void *p, floatx4 v)
 {
     store_b64_device(p, v[0], v[1]);
@@ -338,7 +349,7 @@ struct Decoder {
     const uint32_t group, limit;
 
     __device__ Decoder(const yvex_rocm_decode_params &params, unsigned char *transpose_area)
-        : p(params), vt(transpose_area), lane(threadIdx.x), n(threadIdx.x & 15), g(threadIdx.x >> 4),
+        : p(params), vt(transpose_area), lane(threadIdx.x & 63), n(threadIdx.x & 15), g((threadIdx.x & 63) >> 4),
           group(params.query_heads / params.kv_heads),
           limit(PAGED ? params.table_stride * (uint32_t)kPageTokens : params.fixed_context)
     {
@@ -676,6 +687,162 @@ struct Decoder {
             cur = stop;
         }
     }
+
+    // ---- teams --------------------------------------------------------------------------
+    // The form for a launch that is all latency (one query token per session over a
+    // token-major history): a workgroup is a team of kTeam waves that share one stretch of
+    // one (session, kv head) segment, kTeam times shorter chains of dependent loads per wave
+    // than one wave per stretch would have, and merge their partials through LDS before the
+    // team leaves ONE partial for the segment; the teams of a segment then merge as above
+    // (arrival counter, last team merges in team order).  The exchange between workgroups --
+    // write-through stores, the counter's round trip, the merge's load trip -- costs about
+    // as much as the streaming itself, so it pays to have few, short parts on both levels.
+    // grid = (teams per segment, kv_heads, sessions), block = 64 * kTeam; group <= 8.
+    // team_lds: kTeam areas of 4 KB, a wave's V transposition first and its accumulators
+    // ([group][128] F32) once it has streamed its tiles, then [kTeam][8][2] (max, sum).
+    static constexpr int kTeam = 8;
+    static constexpr uint32_t kTeamArea = kPageTokens * kHeadDim * 2u / sizeof(float);  // floats
+    static constexpr uint32_t kTeamLdsBytes = kTeam * (kPageTokens * kHeadDim * 2u + 8u * 2u * sizeof(float));
+
+    __device__ inline void run_team(float *parts) const
+    {
+        const uint32_t wave = threadIdx.x >> 6;
+        const uint32_t team = blockIdx.x, teams = gridDim.x, kv_head = blockIdx.y, session = blockIdx.z;
+        const uint32_t ctx = context_of(session);
+        if (ctx == 0u) return;  // out of contract (flagged), for the whole workgroup alike
+        const uint32_t tiles = (ctx + kPageTokens - 1u) / kPageTokens;
+        const uint32_t per_wave = (tiles + teams * kTeam - 1u) / (teams * kTeam);
+        const uint32_t first = min(tiles, (team * kTeam + wave) * per_wave);
+        const uint32_t count = min(per_wave, tiles - first);
+
+        bf16x8 q[4];
+        {
+            const uint16_t *qrow = p.q + ((uint64_t)session * p.query_heads + kv_head * group +
+                                          min((uint32_t)n, group - 1u)) * kHeadDim;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                u32x4 raw = load_b128(qrow + j * 32 + g * 8);
+                if ((uint32_t)n >= group) raw = (u32x4){0u, 0u, 0u, 0u};
+                q[j] = as_bf16x8(raw);
+            }
+        }
+        State st;
+#pragma unroll
+        for (int b = 0; b < 8; ++b) st.o[b] = (floatx4){0.f, 0.f, 0.f, 0.f};
+        st.m = -INFINITY;
+        st.l = 0.f;
+        for (uint32_t done = 0u; done < count; done += 128u)
+            stream(st, q, session, kv_head, ctx, first + done, min(128u, count - done));
+        float l = st.l;
+        l += xor_lanes(l, 16);
+        l += xor_lanes(l, 32);
+
+        // the wave's part into LDS (a wave without tiles leaves max -inf, sum 0, zeros)
+        float *acc = parts, *ml = parts + kTeam * kTeamArea;
+        if ((uint32_t)n < group) {
+            float *row = acc + wave * kTeamArea + (uint32_t)n * kHeadDim + g * 4;
+#pragma unroll
+            for (int b = 0; b < 8; ++b) *reinterpret_cast<floatx4 *>(row + b * 16) = st.o[b];
+            if (g == 0) {
+                ml[(wave * 8u + (uint32_t)n) * 2u] = st.m;
+                ml[(wave * 8u + (uint32_t)n) * 2u + 1u] = l;
+            }
+        }
+        __syncthreads();
+
+        // the team's part: thread t merges (head, dim) pairs t, t + 512, ... over the waves,
+        // in wave order
+        const uint32_t values = group * kHeadDim;
+        const uint64_t segment = (uint64_t)session * p.kv_heads + kv_head;
+        const uint64_t slot0 = (segment * teams + team) * group;
+        const bool whole = teams == 1u;
+        for (uint32_t at = threadIdx.x; at < values; at += 64u * kTeam) {
+            const uint32_t hh = at / kHeadDim, d = at % kHeadDim;
+            float top = -INFINITY;
+#pragma unroll
+            for (int w = 0; w < kTeam; ++w) top = fmaxf(top, ml[(w * 8u + hh) * 2u]);
+            float sum = 0.f, o = 0.f;
+#pragma unroll
+            for (int w = 0; w < kTeam; ++w) {
+                const float m = ml[(w * 8u + hh) * 2u];
+                const float weight = m == -INFINITY ? 0.f : fast_exp2(m - top);
+                sum += weight * ml[(w * 8u + hh) * 2u + 1u];
+                o += weight * acc[w * kTeamArea + hh * kHeadDim + d];
+            }
+            if (whole) {
+                publish_value(session, kv_head * group + hh, d, o, sum, top);
+            } else {
+                __hip_atomic_store(p.part_acc + (slot0 + hh) * kHeadDim + d, o, __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+                if (d == 0u) store_b64_device(p.part_ml + (slot0 + hh) * 2u, top, sum);
+            }
+        }
+        if (whole) return;
+        // every thread's stores have completed before the team is counted in
+        __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+        __syncthreads();
+        uint32_t *last = reinterpret_cast<uint32_t *>(parts);  // the LDS parts are done with
+        if (threadIdx.x == 0u) {
+            uint32_t *arrivals = p.arrivals + segment;
+            const uint32_t before =
+                __hip_atomic_fetch_add(arrivals, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (before == teams - 1u)
+                __hip_atomic_store(arrivals, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            *last = before == teams - 1u ? 1u : 0u;
+        }
+        __syncthreads();
+        if (*last == 0u) return;
+        // the last team merges the segment's parts in team order; every load of a thread is
+        // independent of the others (teams past the end alias the last one with weight
+        // zero): one memory round trip per kTeamsPerTrip teams
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+        constexpr uint32_t kTeamsPerTrip = 16u;
+        for (uint32_t at = threadIdx.x; at < values; at += 64u * kTeam) {
+            const uint32_t hh = at / kHeadDim, d = at % kHeadDim;
+            float top = -INFINITY, sum = 0.f, o = 0.f;
+            for (uint32_t t0 = 0u; t0 < teams; t0 += kTeamsPerTrip) {
+                float m[kTeamsPerTrip], part_l[kTeamsPerTrip], v[kTeamsPerTrip];
+#pragma unroll
+                for (uint32_t i = 0u; i < kTeamsPerTrip; ++i) {
+                    const uint64_t slot = (segment * teams + min(t0 + i, teams - 1u)) * group + hh;
+                    load_b64_device(p.part_ml + slot * 2u, m[i], part_l[i]);
+                    v[i] = __hip_atomic_load(p.part_acc + slot * kHeadDim + d, __ATOMIC_RELAXED,
+                                             __HIP_MEMORY_SCOPE_AGENT);
+                }
+                float trip = -INFINITY;
+#pragma unroll
+                for (uint32_t i = 0u; i < kTeamsPerTrip; ++i) {
+                    if (t0 + i >= teams) m[i] = -INFINITY;
+                    trip = fmaxf(trip, m[i]);
+                }
+                const float m_new = fmaxf(top, trip);
+                const float keep = top == -INFINITY ? 0.f : fast_exp2(top - m_new);
+                sum *= keep;
+                o *= keep;
+#pragma unroll
+                for (uint32_t i = 0u; i < kTeamsPerTrip; ++i) {
+                    const float weight = m[i] == -INFINITY ? 0.f : fast_exp2(m[i] - m_new);
+                    sum += weight * part_l[i];
+                    o += weight * v[i];
+                }
+                top = m_new;
+            }
+            publish_value(session, kv_head * group + hh, d, o, sum, top);
+        }
+    }
+
+    // One normalised output value (and, from the thread of dim 0, the row's LSE).
+    __device__ inline void publish_value(uint32_t session, uint32_t head, uint32_t d, float o, float sum,
+                                         float top) const
+    {
+        const uint64_t at = ((uint64_t)session * p.query_heads + head) * kHeadDim + d;
+        float value = o / sum;
+        if (p.gate) value = bf16_to_f32(bf16_bits(value)) * sigmoid(bf16_to_f32(p.gate[at]));
+        if (!isfinite(value)) flag(p.status, YVEX_ROCM_DEVICE_NUMERIC);
+        p.out[at] = bf16_bits(value);
+        if (p.lse && d == 0u)
+            p.lse[(uint64_t)session * p.query_heads + head] = (top + fast_log2(sum)) * YVEX_LN2;
+    }
 };
 
 }  // namespace
@@ -696,6 +863,16 @@ YVEX_DECODE_KERNEL(yvex_rocm_decode_rows_bf16, Bf16Kv, false, 2, false)
 YVEX_DECODE_KERNEL(yvex_rocm_decode_paged_bf16_merged, Bf16Kv, true, 3, true)
 YVEX_DECODE_KERNEL(yvex_rocm_decode_paged_q8_0_merged, Q8Kv, true, 3, true)
 YVEX_DECODE_KERNEL(yvex_rocm_decode_rows_bf16_merged, Bf16Kv, false, 2, true)
+
+// teams of eight waves over a token-major history (see Decoder::run_team)
+extern "C" __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
+yvex_rocm_decode_rows_bf16_team(const yvex_rocm_decode_params p)
+{
+    typedef Decoder<Bf16Kv, false, 2, true> Team;
+    __shared__ __attribute__((aligned(16))) unsigned char team_lds[Team::kTeamLdsBytes];
+    const uint32_t wave = threadIdx.x >> 6;
+    Team(p, team_lds + wave * (kPageTokens * kHeadDim * 2)).run_team(reinterpret_cast<float *>(team_lds));
+}
 
 // Merge of the split segments of the balanced decode when the decode kernel was launched
 // without arrival counters (large launches).  grid = (query_heads, sessions), block =

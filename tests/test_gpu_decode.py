@@ -69,6 +69,27 @@ def test_rows_decode_ragged_lengths(backend, ctx):
     assert_lse(lse, ref_lse, "full ctx=%d" % ctx)
 
 
+@pytest.mark.parametrize("hq,hkv,ctx", [(1, 1, 700), (4, 2, 5000), (10, 2, 300), (64, 8, 9000),
+                                        (8, 1, 20000), (32, 2, 2100), (16, 1, 33)])
+def test_rows_decode_group_sizes_and_team_counts(backend, hq, hkv, ctx):
+    """One query token over a token-major history: groups of 1 to 8 query heads per kv head go
+    through teams of eight waves (1, few, 16 and the maximum of 32 teams per kv head: one and
+    two load trips of the last team's merge), wider groups through one wave per stretch."""
+    rng = np.random.default_rng(hq * 100000 + ctx)
+    q = bf16_normal(rng, (1, hq, 128))
+    k = bf16_normal(rng, (ctx, hkv, 128))
+    v = bf16_normal(rng, (ctx, hkv, 128))
+    got, lse, facts = run_rows_decode(backend, q, k, v, query_start=ctx - 1)
+    rc, ref, _, ref_lse = ORACLE.gqa_bf16(q, k, v, query_start=ctx - 1, causal=True)
+    assert rc == 0
+    label = "hq=%d hkv=%d ctx=%d" % (hq, hkv, ctx)
+    assert_close_bf16(got, ref, label)
+    assert_lse(lse, ref_lse, label)
+    assert facts.kernel_launches == 1
+    again, lse_again, _ = run_rows_decode(backend, q, k, v, query_start=ctx - 1)
+    assert np.array_equal(got, again) and np.array_equal(lse, lse_again)
+
+
 def test_rows_decode_interleaved_kv_history_rows(backend):
     """The reference caller passes K at offset 0 and V at offset kv_width of one interleaved
     [K|V] history row with stride 2*kv_width (src/runtime/stateful_attention.c:326-352)."""
