@@ -291,7 +291,7 @@ def workload_exact1(backend, rng, steps, warmup):
     backend.workspace_attach(work)
     run = lambda: backend.attention_execute(req, q, k, v, out)  # noqa: E731
     facts = run()
-    kernels = ["yvex_rocm_gqa_f32_split", "yvex_rocm_gqa_f32_split_merge"]
+    kernels = ["yvex_rocm_gqa_f32_split"]
     timed = time_steps(backend, run, steps, warmup, kernels)
     backend.workspace_detach()
     return dict(name="exact1",

@@ -329,10 +329,11 @@ static unsigned long long visible_tokens(const yvex_transformer_attention_requir
  *     reference's own device kernel (src/backend/cuda/transformer_kernels.cu:136-208).
  *   - Other requests over 512 or more keys (the decode step of the session layer,
  *     src/runtime/stateful_attention.c:326-352) are cut into runs of keys, one wave per
- *     (token, head, run) with double-precision statistics, and merged by a second launch.
+ *     (token, head, run) with double-precision statistics, eight runs per workgroup; the
+ *     workgroups of a (token, head) merge in the kernel (arrival counters), one launch.
  *   - Everything else runs one wave per (token, head), double-precision statistics. */
 enum { ROCM_EXACT_TILE_QUERIES = 128, ROCM_EXACT_TILE_MIN_TOKENS = 32, ROCM_EXACT_SPLIT_MIN_KEYS = 512,
-       ROCM_EXACT_SPLIT_WAVES = 2048, ROCM_EXACT_SPLIT_RUN_MIN = 64 };
+       ROCM_EXACT_SPLIT_WAVES = 2048, ROCM_EXACT_SPLIT_RUN_MIN = 64, ROCM_EXACT_SPLIT_TEAM = 8 };
 
 static int exact_strides_aligned(const yvex_transformer_attention_requirement *r)
 {
@@ -361,7 +362,8 @@ static unsigned long long exact_split_runs(const yvex_transformer_attention_requ
     *keys_per_run = 0ull;
     if (exact_tile_geometry(r) || r->key_value_tokens < ROCM_EXACT_SPLIT_MIN_KEYS ||
         (r->head_dimension & 7ull) || r->head_dimension > 256ull || !exact_strides_aligned(r) ||
-        !yvex_core_u64_mul(r->query_tokens, r->query_heads, &units) || units > 0x7fffffffull)
+        !yvex_core_u64_mul(r->query_tokens, r->query_heads, &units) ||
+        units > YVEX_ROCM_DECODE_SEGMENTS_MAX /* one arrival counter per (token, head) */)
         return 0ull;
     runs = ROCM_EXACT_SPLIT_WAVES / units ? ROCM_EXACT_SPLIT_WAVES / units : 1ull;
     if (runs > r->key_value_tokens / ROCM_EXACT_SPLIT_RUN_MIN)
@@ -379,7 +381,9 @@ static int exact_split_workspace(const yvex_transformer_attention_requirement *r
                                  unsigned long long *total)
 {
     unsigned long long slots, acc, ml;
-    if (!yvex_core_u64_mul(r->query_tokens * r->query_heads, runs, &slots) ||
+    /* one partial per team of ROCM_EXACT_SPLIT_TEAM runs */
+    if (!yvex_core_u64_mul(r->query_tokens * r->query_heads,
+                           (runs + ROCM_EXACT_SPLIT_TEAM - 1ull) / ROCM_EXACT_SPLIT_TEAM, &slots) ||
         !yvex_core_u64_mul(slots, r->head_dimension * sizeof(double), &acc) ||
         !yvex_core_u64_mul(slots, 2ull * sizeof(double), &ml))
         return 0;
@@ -539,7 +543,7 @@ static int attention_execute_common(yvex_backend *backend,
         } else if ((split_runs = exact_split_runs(r, &split_keys)) != 0ull &&
                    !(((uintptr_t)request->query->data | (uintptr_t)request->key->data |
                       (uintptr_t)request->value->data) & 15u)) {
-            /* runs of keys, one wave per (token, head, run), then the merge */
+            /* runs of keys, one wave per (token, head, run), eight runs per workgroup */
             unsigned long long acc_bytes = 0ull;
             if (!exact_split_workspace(r, split_runs, &acc_bytes, &split_bytes))
                 return refuse(err, YVEX_ERR_BOUNDS, "rocm.transformer.gqa",
@@ -551,16 +555,19 @@ static int attention_execute_common(yvex_backend *backend,
             params.part_ml = (double *)((unsigned char *)split_work + acc_bytes);
             params.splits = (uint32_t)split_runs;
             params.keys_per_split = (uint32_t)split_keys;
+            params.arrivals = state->decode_arrivals;
             rc = yvex_rocm_launch(backend,
                                   r->head_dimension > 128ull ? YVEX_ROCM_FN_GQA_F32_SPLIT_WIDE
                                                              : YVEX_ROCM_FN_GQA_F32_SPLIT,
                                   YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_F32, (unsigned int)rows,
-                                  (unsigned int)split_runs, 1u, 64u, 0u, &params,
-                                  "rocm.transformer.gqa", err);
-            if (rc == YVEX_OK)
-                rc = yvex_rocm_launch(backend, YVEX_ROCM_FN_GQA_F32_SPLIT_MERGE,
-                                      YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_F32, (unsigned int)rows,
-                                      1u, 1u, 256u, 0u, &params, "rocm.transformer.gqa", err);
+                                  (unsigned int)((split_runs + ROCM_EXACT_SPLIT_TEAM - 1ull) /
+                                                 ROCM_EXACT_SPLIT_TEAM),
+                                  1u, 64u * ROCM_EXACT_SPLIT_TEAM, 0u, &params, "rocm.transformer.gqa", err);
+            /* a launch that did not run to a clean end may leave arrival counts behind */
+            if (rc != YVEX_OK && !state->recording && backend->status != YVEX_BACKEND_STATUS_FAILED)
+                (void)state->driver.hipMemsetAsync(state->decode_arrivals, 0,
+                                                   YVEX_ROCM_DECODE_SEGMENTS_MAX * sizeof(uint32_t),
+                                                   state->stream);
         } else {
             split_runs = 0ull;
             rc = yvex_rocm_launch(backend, YVEX_ROCM_FN_GQA_F32,
@@ -568,7 +575,7 @@ static int attention_execute_common(yvex_backend *backend,
                                   1u, 64u, 0u, &params, "rocm.transformer.gqa", err);
         }
         if (rc == YVEX_OK) {
-            facts->kernel_launches = split_work ? 2ull : 1ull;
+            facts->kernel_launches = 1ull;
             facts->accelerated_matrix_launches = tiled ? 1ull : 0ull;
             facts->temporary_bytes = split_bytes;
             facts->compulsory_memory_facts_available = 1;

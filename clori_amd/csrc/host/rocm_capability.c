@@ -36,8 +36,6 @@ static const rocm_kernel_binding rocm_kernel_bindings[] = {
      YVEX_ROCM_FN_GQA_F32_SPLIT},
     {"yvex_rocm_gqa_f32_split_wide", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_F32,
      YVEX_ROCM_FN_GQA_F32_SPLIT_WIDE},
-    {"yvex_rocm_gqa_f32_split_merge", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_F32,
-     YVEX_ROCM_FN_GQA_F32_SPLIT_MERGE},
     {"yvex_rocm_gqa_f32_tile_64", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_F32,
      YVEX_ROCM_FN_GQA_F32_TILE_64},
     {"yvex_rocm_gqa_f32_tile_128", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_F32,

@@ -14,7 +14,6 @@ typedef enum {
     YVEX_ROCM_FN_GQA_F32,
     YVEX_ROCM_FN_GQA_F32_SPLIT,
     YVEX_ROCM_FN_GQA_F32_SPLIT_WIDE,
-    YVEX_ROCM_FN_GQA_F32_SPLIT_MERGE,
     YVEX_ROCM_FN_GQA_F32_TILE_64,
     YVEX_ROCM_FN_GQA_F32_TILE_128,
     YVEX_ROCM_FN_GQA_F32_TILE_256,

@@ -33,11 +33,14 @@ typedef struct {
     uint64_t q_stride, k_stride, v_stride;
     float scale;
     int32_t causal;
-    /* split form (yvex_rocm_gqa_f32_split + _merge): the keys a query sees are cut into
-     * `splits` runs of keys_per_split; part_acc is F64 [Tq*Hq][splits][head_dim], part_ml
-     * F64 [Tq*Hq][splits][2] = (running maximum, denominator) */
+    /* split form (yvex_rocm_gqa_f32_split[_wide]): the keys a query sees are cut into `splits`
+     * runs of keys_per_split, eight consecutive runs per workgroup (a team); part_acc is F64
+     * [Tq*Hq][teams][head_dim], part_ml F64 [Tq*Hq][teams][2] = (running maximum,
+     * denominator), teams = ceil(splits / 8); arrivals holds one counter per (token, head),
+     * zero before the launch and after it */
     double *part_acc, *part_ml;
     uint32_t splits, keys_per_split;
+    uint32_t *arrivals;
 } yvex_rocm_gqa_f32_params;
 
 typedef struct {

@@ -200,7 +200,11 @@ __device__ inline double row_sum(double v)
 // Decode-shaped EXACT_F32 requests over long contexts: the same arithmetic as
 // yvex_rocm_gqa_f32 (double dot products, the score rounded to float, double exponentials,
 // denominator and accumulators), but the keys a query sees are cut into `splits` runs, one wave
-// per (query token, query head, run), and the runs are merged by yvex_rocm_gqa_f32_split_merge.
+// per (query token, query head, run).  A workgroup is a team of kSplitTeam waves on consecutive
+// runs: they merge through LDS in wave order, the team leaves one partial (write-through
+// stores), counts itself in on the arrival counter of its (token, head), and the team that
+// completes the count merges the teams' partials in team order and publishes.  One launch;
+// the result does not depend on who was last.
 // Inside a run a wave takes 64 keys at a time, four keys per step: the 16 lanes of a group
 // hold 8 head dims each (kPieces = 2 such pieces above 128 dims), so a key or value row is one
 // contiguous read of the group.  The dot product is reduced over the group, lane `piece` of
@@ -211,7 +215,23 @@ __device__ inline double row_sum(double v)
 // a key past the run reads the run's last key (its score is masked, its weight is zero), a
 // lane past the head dimension reads the row's last 8 dims against a zero query and its
 // sums are never stored.
-// grid = (query_tokens * query_heads, splits), block 64; head_dim % 8 == 0, <= 128 * kPieces.
+// grid = (query_tokens * query_heads, ceil(splits / kSplitTeam)), block 64 * kSplitTeam;
+// head_dim % 8 == 0, <= 128 * kPieces; LDS: kSplitTeam rows of 256 doubles, then (max, sum) pairs.
+constexpr int kSplitTeam = 8;
+
+// 8 bytes to and from global memory at device scope: write-through stores that are visible to
+// the other XCDs once they have completed, loads that see them without an L2 invalidate.
+__device__ inline void store_f64_device(double *p, double v)
+{
+    __hip_atomic_store(reinterpret_cast<uint64_t *>(p), __builtin_bit_cast(uint64_t, v), __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ inline double load_f64_device(const double *p)
+{
+    return __builtin_bit_cast(double, __hip_atomic_load(reinterpret_cast<const uint64_t *>(p), __ATOMIC_RELAXED,
+                                                        __HIP_MEMORY_SCOPE_AGENT));
+}
+
 // Which (token, head) workgroup `unit` of a launch row works on.  Consecutive workgroup ids go
 // to consecutive XCDs, each with its own L2; when the head count is a multiple of eight the
 // heads are dealt so that an XCD gets a contiguous eighth of them, i.e. the query heads that
@@ -226,20 +246,20 @@ __device__ __forceinline__ void split_unit(const yvex_rocm_gqa_f32_params &p, ui
 }
 
 template <int kPieces>
-__device__ __forceinline__ void gqa_f32_split(const yvex_rocm_gqa_f32_params &p)
+__device__ __forceinline__ void gqa_f32_split(const yvex_rocm_gqa_f32_params &p, double *team_lds)
 {
     typedef float floatx4 __attribute__((ext_vector_type(4)));
     constexpr int kBatch = 8 / kPieces;  // steps whose rows are in flight together
-    const int lane = threadIdx.x;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int group = lane >> 4, piece = lane & 15;
-    const uint64_t unit = blockIdx.x, split = blockIdx.y;
+    // a run past `splits` (the last team's padding) starts past the visible keys: it has none
+    const uint64_t unit = blockIdx.x, split = (uint64_t)blockIdx.y * kSplitTeam + (uint64_t)wave;
     uint64_t token, head;
     split_unit(p, unit, token, head);
     const uint64_t kv_head = head / (p.query_heads / p.kv_heads);
     const uint64_t visible = p.causal ? min(p.kv_tokens, p.query_start + token + 1) : p.kv_tokens;
     const uint64_t d = p.head_dim;
     const uint64_t k0 = split * p.keys_per_split, k1 = min(visible, k0 + (uint64_t)p.keys_per_split);
-    const uint64_t slot = unit * p.splits + split;
     uint64_t dim[kPieces];   // first of this lane's 8 dims in piece j, clamped into the row
     bool live[kPieces];
 #pragma unroll
@@ -348,105 +368,109 @@ __device__ __forceinline__ void gqa_f32_split(const yvex_rocm_gqa_f32_params &p)
             acc[j][e] += __shfl_xor(acc[j][e], 16, kWave);
             acc[j][e] += __shfl_xor(acc[j][e], 32, kWave);
         }
+    // ---- the team: the waves' parts through LDS, merged in wave order ---------------------
+    double *rows = team_lds, *stats = team_lds + kSplitTeam * 256;
     if (group == 0) {
 #pragma unroll
         for (int j = 0; j < kPieces; ++j)
             if (live[j])
 #pragma unroll
-                for (int e = 0; e < 8; ++e) p.part_acc[slot * d + dim[j] + (uint64_t)e] = acc[j][e];
+                for (int e = 0; e < 8; ++e) rows[wave * 256 + (int)dim[j] + e] = acc[j][e];
     }
     if (lane == 0) {
-        p.part_ml[slot * 2u] = m;  // -inf for a run without visible keys
-        p.part_ml[slot * 2u + 1u] = l;
+        stats[wave * 2] = m;  // -inf for a run without visible keys
+        stats[wave * 2 + 1] = l;
     }
-}
-
-extern "C" __global__ void __launch_bounds__(64)
-yvex_rocm_gqa_f32_split(const yvex_rocm_gqa_f32_params p)
-{
-    gqa_f32_split<1>(p);
-}
-
-extern "C" __global__ void __launch_bounds__(64)
-yvex_rocm_gqa_f32_split_wide(const yvex_rocm_gqa_f32_params p)
-{
-    gqa_f32_split<2>(p);
-}
-
-// Merge of the runs of one (query token, query head).  Every wave reads the statistics of
-// all runs (64 at a time, one run per lane) and finds the common maximum; wave w then sums the
-// rows of the runs w, w + 4, ... with lane = head dims lane, lane + 64, ..., eight runs in
-// flight, and wave 0 adds the four partial sums through LDS in wave order.
-// grid = query_tokens * query_heads, block 256.
-extern "C" __global__ void __launch_bounds__(256)
-yvex_rocm_gqa_f32_split_merge(const yvex_rocm_gqa_f32_params p)
-{
-    __shared__ double partial[4][5][64];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const uint64_t unit = blockIdx.x, d = p.head_dim;
-    const double *ml = p.part_ml + unit * p.splits * 2u;
-    const double *rows = p.part_acc + unit * p.splits * d;
-    double top = -INFINITY;
-    for (uint32_t base = 0; base < p.splits; base += 64u) {
-        const uint32_t s = base + (uint32_t)lane;
-        top = fmax(top, wave_max(s < p.splits ? ml[s * 2u] : -INFINITY));
+    __syncthreads();
+    const uint32_t t = threadIdx.x, teams = gridDim.y, team = blockIdx.y;
+    double top = -INFINITY, total = 0.0, o = 0.0;
+#pragma unroll
+    for (int w = 0; w < kSplitTeam; ++w) top = fmax(top, stats[w * 2]);
+#pragma unroll
+    for (int w = 0; w < kSplitTeam; ++w) {
+        const double mw = stats[w * 2];
+        const double weight = mw == -INFINITY ? 0.0 : exp(mw - top);
+        total += weight * stats[w * 2 + 1];
+        if (t < d) o += weight * rows[w * 256 + (int)t];
     }
-    double total = 0.0, acc[4] = {0.0, 0.0, 0.0, 0.0};
-    for (uint32_t base = 0; base < p.splits; base += 64u) {
-        const uint32_t s = base + (uint32_t)lane;
-        const double m = s < p.splits ? ml[s * 2u] : -INFINITY;
-        // a run past the visible keys left (-inf, 0): weight zero
-        const double w = m == -INFINITY ? 0.0 : exp(m - top);
-        // this wave's runs only: s % 4 == wave
-        total += wave_sum(s < p.splits && (s & 3u) == (uint32_t)wave ? w * ml[s * 2u + 1u] : 0.0);
-        const uint32_t count = min(64u, p.splits - base);
-        for (uint32_t i0 = (uint32_t)wave; i0 < count; i0 += 32u) {
-            double wi[8], part[8][4];
+    if (teams > 1u) {
+        // ---- the teams: one partial each, merged in team order by the last to arrive --------
+        const uint64_t slot = unit * teams + team;
+        if (t < d) store_f64_device(p.part_acc + slot * d + t, o);
+        if (t == 0u) {
+            store_f64_device(p.part_ml + slot * 2u, top);
+            store_f64_device(p.part_ml + slot * 2u + 1u, total);
+        }
+        __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this thread's stores have completed
+        __syncthreads();
+        uint32_t *last = reinterpret_cast<uint32_t *>(team_lds);  // the LDS parts are done with
+        if (t == 0u) {
+            const uint32_t before =
+                __hip_atomic_fetch_add(p.arrivals + unit, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (before == teams - 1u)
+                __hip_atomic_store(p.arrivals + unit, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            *last = before == teams - 1u ? 1u : 0u;
+        }
+        __syncthreads();
+        if (*last == 0u) return;
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+        top = -INFINITY;
+        total = 0.0;
+        o = 0.0;
+        // eight teams per trip of independent loads (teams past the end alias the last one
+        // with weight zero)
+        for (uint32_t t0 = 0u; t0 < teams; t0 += 8u) {
+            double mt[8], lt[8], vt[8];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) {
-                const uint32_t want = i0 + 4u * (uint32_t)u;
-                const uint32_t i = min(want, count - 1u);
-                wi[u] = want < count ? __shfl(w, (int)i, kWave) : 0.0;
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const uint64_t c = (uint64_t)lane + 64u * (uint64_t)j;
-                    part[u][j] = c < d ? rows[(uint64_t)(base + i) * d + c] : 0.0;
-                }
+            for (uint32_t i = 0u; i < 8u; ++i) {
+                const uint64_t from = unit * teams + min(t0 + i, teams - 1u);
+                mt[i] = load_f64_device(p.part_ml + from * 2u);
+                lt[i] = load_f64_device(p.part_ml + from * 2u + 1u);
+                vt[i] = t < d ? load_f64_device(p.part_acc + from * d + t) : 0.0;
             }
+            double trip = -INFINITY;
 #pragma unroll
-            for (int u = 0; u < 8; ++u)
+            for (uint32_t i = 0u; i < 8u; ++i) {
+                if (t0 + i >= teams) mt[i] = -INFINITY;
+                trip = fmax(trip, mt[i]);
+            }
+            const double top_new = fmax(top, trip);
+            const double keep = top == -INFINITY ? 0.0 : exp(top - top_new);
+            total *= keep;
+            o *= keep;
 #pragma unroll
-                for (int j = 0; j < 4; ++j) acc[j] += wi[u] * part[u][j];
+            for (uint32_t i = 0u; i < 8u; ++i) {
+                const double weight = mt[i] == -INFINITY ? 0.0 : exp(mt[i] - top_new);
+                total += weight * lt[i];
+                o += weight * vt[i];
+            }
+            top = top_new;
         }
     }
-#pragma unroll
-    for (int j = 0; j < 4; ++j) partial[wave][j][lane] = acc[j];
-    partial[wave][4][lane] = total;
-    __syncthreads();
-    if (wave != 0) return;
-    total = ((partial[0][4][lane] + partial[1][4][lane]) + partial[2][4][lane]) + partial[3][4][lane];
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-        acc[j] = ((partial[0][j][lane] + partial[1][j][lane]) + partial[2][j][lane]) + partial[3][j][lane];
     if (!(total > 0.0) || !isfinite(total) || !isfinite(top)) {
-        if (lane == 0) flag(p.status, YVEX_ROCM_DEVICE_NUMERIC);
+        if (t == 0u) flag(p.status, YVEX_ROCM_DEVICE_NUMERIC);
         return;
     }
-    uint64_t token, head;
-    split_unit(p, unit, token, head);
-    float *out = p.out + (token * p.query_heads + head) * d;
-    bool bad = false;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const uint64_t c = (uint64_t)lane + 64u * (uint64_t)j;
-        if (c < d) {
-            const float o = (float)(acc[j] / total);
-            bad |= !isfinite(o);
-            out[c] = o;
-        }
+    if (t < d) {
+        const float value = (float)(o / total);
+        if (!isfinite(value)) flag(p.status, YVEX_ROCM_DEVICE_NUMERIC);
+        p.out[(token * p.query_heads + head) * d + t] = value;
     }
-    if (bad) flag(p.status, YVEX_ROCM_DEVICE_NUMERIC);
-    if (p.lse && lane == 0) p.lse[token * p.query_heads + head] = (float)(top + log(total));
+    if (p.lse && t == 0u) p.lse[token * p.query_heads + head] = (float)(top + log(total));
+}
+
+extern "C" __global__ void __launch_bounds__(64 * kSplitTeam)
+yvex_rocm_gqa_f32_split(const yvex_rocm_gqa_f32_params p)
+{
+    __shared__ double team_lds[kSplitTeam * 256 + kSplitTeam * 2];
+    gqa_f32_split<1>(p, team_lds);
+}
+
+extern "C" __global__ void __launch_bounds__(64 * kSplitTeam)
+yvex_rocm_gqa_f32_split_wide(const yvex_rocm_gqa_f32_params p)
+{
+    __shared__ double team_lds[kSplitTeam * 256 + kSplitTeam * 2];
+    gqa_f32_split<2>(p, team_lds);
 }
 
 // Word fill, used instead of a memset node so the clear can be recorded in a graph.
