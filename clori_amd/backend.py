@@ -87,6 +87,26 @@ class Tensor:
         _check(lib().yvex_backend_tensor_copy(self.backend.handle, self.handle, source.handle,
                                               C.byref(err)), err)
 
+    # -- tensors over a reserved address range -----------------------------
+    @property
+    def resident_bytes(self):
+        return int(self.handle.contents.resident_bytes)
+
+    def commit(self, byte_offset, nbytes):
+        """Backs the granules under [byte_offset, byte_offset + nbytes) that are not backed
+        yet (zero-filled) and returns how many bytes that added."""
+        delta, err = C.c_ulonglong(0), B.Error()
+        _check(lib().yvex_backend_tensor_commit_range(self.backend.handle, self.handle, byte_offset,
+                                                      nbytes, C.byref(delta), C.byref(err)), err)
+        return delta.value
+
+    def decommit(self):
+        """Returns every committed page, keeps the address range; returns the bytes released."""
+        released, err = C.c_ulonglong(0), B.Error()
+        _check(lib().yvex_backend_tensor_decommit(self.backend.handle, self.handle,
+                                                  C.byref(released), C.byref(err)), err)
+        return released.value
+
     def release(self):
         if self.handle:
             err = B.Error()
@@ -240,6 +260,24 @@ class Backend:
         self.tensors.append(tensor)
         if data is not None:
             tensor.write(data)
+        return tensor
+
+    def reserve(self, name, dtype, shape, nbytes=None):
+        """A tensor that owns a device address range and no memory yet (Tensor.commit backs
+        parts of it).  The granule size is kept as `tensor.granularity`."""
+        desc = B.TensorDesc()
+        desc.name = name.encode()
+        desc.dtype = dtype
+        desc.rank = len(shape)
+        for i, dim in enumerate(shape):
+            desc.dims[i] = dim
+        desc.bytes = nbytes if nbytes is not None else int(np.prod(shape)) * B.DTYPE_BYTES[dtype]
+        handle, granularity, err = B.TensorP(), C.c_ulonglong(0), B.Error()
+        _check(lib().yvex_backend_tensor_reserve(self.handle, C.byref(desc), C.byref(handle),
+                                                 C.byref(granularity), C.byref(err)), err)
+        tensor = Tensor(self, handle, dtype, shape)
+        tensor.granularity = granularity.value
+        self.tensors.append(tensor)
         return tensor
 
     def workspace_attach(self, tensor, generation=1):

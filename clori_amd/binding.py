@@ -270,7 +270,9 @@ EXPORTED_SYMBOLS = [
     "yvex_backend_kind_of", "yvex_backend_kind_name", "yvex_backend_kind_parse",
     "yvex_backend_status_of", "yvex_backend_status_name", "yvex_backend_get_memory_stats",
     "yvex_backend_get_device_info", "yvex_backend_tensor_alloc", "yvex_backend_tensor_free",
-    "yvex_backend_tensor_release", "yvex_device_tensor_name", "yvex_device_tensor_bytes",
+    "yvex_backend_tensor_release", "yvex_backend_virtual_tensor_supported",
+    "yvex_backend_tensor_reserve",
+    "yvex_backend_tensor_commit_range", "yvex_backend_tensor_decommit", "yvex_device_tensor_name", "yvex_device_tensor_bytes",
     "yvex_device_tensor_is_written", "yvex_backend_tensor_write", "yvex_backend_tensor_read",
     "yvex_backend_tensor_zero", "yvex_backend_tensor_copy", "yvex_backend_tensor_owned_by",
     "yvex_backend_tensor_f32_subview", "yvex_backend_sync", "yvex_backend_supports",
@@ -324,6 +326,11 @@ def load(path=None):
     lib.yvex_backend_tensor_free.argtypes = [vp, TensorP]
     lib.yvex_backend_tensor_free.restype = None
     lib.yvex_backend_tensor_release.argtypes = [vp, C.POINTER(TensorP), ErrorP]
+    lib.yvex_backend_virtual_tensor_supported.argtypes = [vp]
+    lib.yvex_backend_tensor_reserve.argtypes = [vp, C.POINTER(TensorDesc), C.POINTER(TensorP),
+                                                C.POINTER(ull), ErrorP]
+    lib.yvex_backend_tensor_commit_range.argtypes = [vp, TensorP, ull, ull, C.POINTER(ull), ErrorP]
+    lib.yvex_backend_tensor_decommit.argtypes = [vp, TensorP, C.POINTER(ull), ErrorP]
     lib.yvex_device_tensor_name.restype = C.c_char_p
     lib.yvex_device_tensor_name.argtypes = [TensorP]
     lib.yvex_device_tensor_bytes.restype = ull

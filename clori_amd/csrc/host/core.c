@@ -318,6 +318,71 @@ int yvex_backend_tensor_alloc(yvex_backend *backend, const yvex_backend_tensor_d
     return backend->vtable->tensor_alloc(backend, desc, out, err);
 }
 
+/* src/backend/residency.c:12-17 */
+int yvex_backend_virtual_tensor_supported(const yvex_backend *backend)
+{
+    return backend && !backend_cleanup_only(backend) &&
+           backend->status != YVEX_BACKEND_STATUS_FAILED && backend->virtual_tensor_ready;
+}
+
+/* src/backend/core.c:613-634 */
+int yvex_backend_tensor_reserve(yvex_backend *backend, const yvex_backend_tensor_desc *desc,
+                                yvex_device_tensor **out, unsigned long long *granularity,
+                                yvex_error *err)
+{
+    static const char where[] = "backend.tensor.reserve";
+    int rc;
+    if (out) *out = NULL;
+    if (granularity) *granularity = 0ull;
+    if (!backend || !out || !granularity)
+        return refuse(err, YVEX_ERR_INVALID_ARG, where,
+                      "backend, tensor output, and granularity output are required");
+    rc = backend_dispatch_admit(backend, where, err);
+    if (rc == YVEX_OK) rc = desc_valid(desc, err);
+    if (rc != YVEX_OK) return rc;
+    if (!backend->vtable || !backend->vtable->tensor_reserve)
+        return refuse(err, YVEX_ERR_UNSUPPORTED, where,
+                      "backend does not support virtual tensor reservation");
+    return backend->vtable->tensor_reserve(backend, desc, out, granularity, err);
+}
+
+/* src/backend/core.c:636-659 */
+int yvex_backend_tensor_commit_range(yvex_backend *backend, yvex_device_tensor *tensor,
+                                     unsigned long long offset, unsigned long long bytes,
+                                     unsigned long long *resident_delta, yvex_error *err)
+{
+    static const char where[] = "backend.tensor.commit";
+    int rc;
+    if (resident_delta) *resident_delta = 0ull;
+    if (!backend || !tensor || !resident_delta || !bytes || offset > tensor->bytes ||
+        bytes > tensor->bytes - offset)
+        return refuse(err, YVEX_ERR_INVALID_ARG, where, "one owned virtual tensor range is required");
+    rc = backend_dispatch_admit(backend, where, err);
+    if (rc != YVEX_OK) return rc;
+    if (!backend->vtable || !backend->vtable->tensor_commit)
+        return refuse(err, YVEX_ERR_UNSUPPORTED, where,
+                      "backend does not support physical page commitment");
+    return backend->vtable->tensor_commit(backend, tensor, offset, bytes, resident_delta, err);
+}
+
+/* src/backend/core.c:661-680 */
+int yvex_backend_tensor_decommit(yvex_backend *backend, yvex_device_tensor *tensor,
+                                 unsigned long long *released_bytes, yvex_error *err)
+{
+    static const char where[] = "backend.tensor.decommit";
+    int rc;
+    if (released_bytes) *released_bytes = 0ull;
+    if (!backend || !tensor || !released_bytes)
+        return refuse(err, YVEX_ERR_INVALID_ARG, where,
+                      "backend, virtual tensor, and release output are required");
+    rc = backend_dispatch_admit(backend, where, err);
+    if (rc != YVEX_OK) return rc;
+    if (!backend->vtable || !backend->vtable->tensor_decommit)
+        return refuse(err, YVEX_ERR_UNSUPPORTED, where,
+                      "backend does not support physical page decommitment");
+    return backend->vtable->tensor_decommit(backend, tensor, released_bytes, err);
+}
+
 /* src/backend/core.c:689-715: release is allowed on a cleanup-only backend. */
 int yvex_backend_tensor_release(yvex_backend *backend, yvex_device_tensor **tensor,
                                 yvex_error *err)
@@ -591,7 +656,7 @@ int yvex_backend_workspace_attach(yvex_backend *backend, const yvex_device_tenso
     if (!backend || backend_cleanup_only(backend) || backend->kind != YVEX_BACKEND_KIND_ROCM ||
         backend->status == YVEX_BACKEND_STATUS_FAILED || !device_tensor ||
         !backend_tensor_owner_is(backend, device_tensor) || !device_tensor->data ||
-        !device_tensor->bytes || !generation)
+        !device_tensor->bytes || device_tensor->virtual_reserved || !generation)
         return refuse(err, YVEX_ERR_INVALID_ARG, "backend.workspace.attach",
                       "same-owner ROCm workspace tensor and generation are required");
     if (backend->workspace_device_tensor)

@@ -20,6 +20,12 @@ typedef struct yvex_backend_vtable {
     int (*device_info)(const yvex_backend *, yvex_backend_device_info *, yvex_error *);
     int (*tensor_alloc)(yvex_backend *, const yvex_backend_tensor_desc *, yvex_device_tensor **,
                         yvex_error *);
+    int (*tensor_reserve)(yvex_backend *, const yvex_backend_tensor_desc *, yvex_device_tensor **,
+                          unsigned long long *, yvex_error *);
+    int (*tensor_commit)(yvex_backend *, yvex_device_tensor *, unsigned long long,
+                         unsigned long long, unsigned long long *, yvex_error *);
+    int (*tensor_decommit)(yvex_backend *, yvex_device_tensor *, unsigned long long *,
+                           yvex_error *);
     int (*tensor_free)(yvex_backend *, yvex_device_tensor *, yvex_error *);
     int (*tensor_write)(yvex_backend *, yvex_device_tensor *, const void *, unsigned long long,
                         yvex_error *);
@@ -54,6 +60,7 @@ struct yvex_backend {
     const yvex_device_tensor *workspace_device_tensor;
     unsigned long long workspace_device_address, workspace_bytes, workspace_cursor;
     unsigned long long workspace_peak, workspace_generation;
+    int virtual_tensor_ready; /* src/backend/private.h:109 */
 };
 
 #define YVEX_BACKEND_LIFECYCLE_CLOSING (1ull << 63)

@@ -68,6 +68,11 @@ int yvex_rocm_op_attention(yvex_backend *backend, const yvex_device_tensor *quer
                                          score_scratch, probability_scratch, out, &head_dim,
                                          &kv_elements, where, err);
     if (rc != YVEX_OK) return rc;
+    if (!yvex_rocm_tensor_backed(query) || !yvex_rocm_tensor_backed(keys) ||
+        !yvex_rocm_tensor_backed(values) || !yvex_rocm_tensor_backed(score_scratch) ||
+        !yvex_rocm_tensor_backed(probability_scratch) || !yvex_rocm_tensor_backed(out))
+        return refuse(err, YVEX_ERR_STATE, where,
+                      "a tensor over a reserved address range reaches pages that are not committed");
     rc = yvex_rocm_require_capability(backend, variant, where, err);
     if (rc != YVEX_OK) return rc;
     memset(&params, 0, sizeof(params));
@@ -431,10 +436,31 @@ static int view_ok(const yvex_backend *backend, const yvex_device_tensor *tensor
                    unsigned long long elements, int require_written)
 {
     unsigned long long bytes;
-    return backend_tensor_owner_is(backend, tensor) && (!require_written || tensor->is_written) &&
-           tensor->dtype == dtype && tensor->data &&
-           yvex_core_u64_mul(elements, yvex_dtype_element_bytes(dtype), &bytes) &&
-           tensor->bytes == bytes;
+    if (!backend_tensor_owner_is(backend, tensor) || (require_written && !tensor->is_written) ||
+        tensor->dtype != dtype || !tensor->data ||
+        !yvex_core_u64_mul(elements, yvex_dtype_element_bytes(dtype), &bytes) ||
+        tensor->bytes != bytes)
+        return 0;
+    if (!yvex_rocm_tensor_backed(tensor)) {
+        yvex_rocm_state(backend)->unbacked_view = 1;
+        return 0;
+    }
+    return 1;
+}
+
+/* The refusal after a view_ok that said no: a view over a reserved address range that
+ * reaches pages nobody committed is a state error of the caller, anything else a
+ * malformed request. */
+static int view_refusal(const yvex_backend *backend, yvex_error *err, const char *where,
+                        const char *reason)
+{
+    yvex_rocm_backend_state *state = yvex_rocm_state(backend);
+    if (state && state->unbacked_view) {
+        state->unbacked_view = 0;
+        return refuse(err, YVEX_ERR_STATE, where,
+                      "a tensor over a reserved address range reaches pages that are not committed");
+    }
+    return refuse(err, YVEX_ERR_FORMAT, where, reason);
 }
 
 static int exact_tile_function(const yvex_transformer_attention_requirement *r,
@@ -502,7 +528,7 @@ static int attention_execute_common(yvex_backend *backend,
         (lse && !view_ok(backend, lse, YVEX_DTYPE_F32, rows, 0)) ||
         (gate && (!view_ok(backend, gate, YVEX_DTYPE_BF16, o_elements, 1) ||
                   gate->data == request->output->data)))
-        return refuse(err, YVEX_ERR_FORMAT, "rocm.transformer.gqa",
+        return view_refusal(backend, err, "rocm.transformer.gqa",
                       "bounded Q/K/V views matching the declared token strides are required");
     if (exact) {
         yvex_rocm_gqa_f32_params params;
@@ -777,7 +803,7 @@ static int paged_decode_execute_common(yvex_backend *backend,
          !view_ok(backend, request->lse, YVEX_DTYPE_F32, r->sessions * r->query_heads, 0)) ||
         (gate && (!view_ok(backend, gate, YVEX_DTYPE_BF16, q_elements, 1) ||
                   gate->data == request->output->data)))
-        return refuse(err, YVEX_ERR_FORMAT, where,
+        return view_refusal(backend, err, where,
                       "query, page pools, page table, context lengths and outputs must be written "
                       "tensors of this backend with the declared geometry");
     memset(&job, 0, sizeof(job));
@@ -1081,7 +1107,7 @@ static int rocm_mla_decode_execute(yvex_backend *backend,
            (!request->compressed_selected ||
             !view_ok(backend, request->compressed_selected, YVEX_DTYPE_I32,
                      r->batch * r->compressed_selected_stride, 1))))))
-        return refuse(err, YVEX_ERR_FORMAT, where,
+        return view_refusal(backend, err, where,
                       "query, latent pages, page table, context lengths and outputs must be "
                       "written tensors of this backend with the declared geometry");
     mla_partition(r, &chunk, &max_chunks, &extra_chunk, &extra_max_chunks);
@@ -1279,7 +1305,7 @@ static int rocm_kv_append_execute(yvex_backend *backend, const yvex_rocm_kv_appe
                  pool_bytes / yvex_dtype_element_bytes(pool_dtype), 0) ||
         !view_ok(backend, request->v_pool, pool_dtype,
                  pool_bytes / yvex_dtype_element_bytes(pool_dtype), 0))
-        return refuse(err, YVEX_ERR_FORMAT, where,
+        return view_refusal(backend, err, where,
                       "rows, tables, descriptors and pools must be tensors of this backend with "
                       "the declared geometry");
     memset(&kp, 0, sizeof(kp));

@@ -29,6 +29,9 @@ static char *text_dup(const char *text)
 
 /* ------------------------------------------------------------- tensors ---- */
 
+static const char kUnbacked[] =
+    "a tensor over a reserved address range reaches pages that are not committed";
+
 /* src/backend/cuda/backend.c:836-905: capability, limit, allocate, zero, publish. */
 static int rocm_tensor_alloc(yvex_backend *backend, const yvex_backend_tensor_desc *desc,
                              yvex_device_tensor **out, yvex_error *err)
@@ -113,7 +116,9 @@ static int rocm_tensor_free(yvex_backend *backend, yvex_device_tensor *tensor, y
                           err);
     if (rc == YVEX_OK && getenv("YVEX_TEST_ROCM_CLEANUP_FAILURE"))
         rc = refuse(err, YVEX_ERR_BACKEND, where, "injected ROCm tensor cleanup failure");
-    if (rc == YVEX_OK && tensor->backend_allocation)
+    if (rc == YVEX_OK && tensor->virtual_reserved)
+        rc = yvex_rocm_virtual_release(backend, tensor, err);
+    else if (rc == YVEX_OK && tensor->backend_allocation)
         rc = yvex_rocm_status(&state->driver, state->driver.hipFree(tensor->backend_allocation),
                               where, err);
     if (rc != YVEX_OK) {
@@ -121,7 +126,8 @@ static int rocm_tensor_free(yvex_backend *backend, yvex_device_tensor *tensor, y
         backend->status = YVEX_BACKEND_STATUS_FAILED;
         return rc;
     }
-    backend_memory_release(backend, tensor->bytes);
+    /* the pages of a virtual range were counted, and given back, extent by extent */
+    if (!tensor->virtual_reserved) backend_memory_release(backend, tensor->bytes);
     if (state->live_tensors) state->live_tensors -= 1ull;
     tensor->owner = NULL;
     tensor->owner_id = 0ull;
@@ -151,6 +157,7 @@ static int rocm_tensor_write(yvex_backend *backend, yvex_device_tensor *tensor, 
     static const char where[] = "rocm.tensor_write";
     int rc = yvex_backend_tensor_rw_validate(where, backend, tensor, len, err);
     if (rc != YVEX_OK) return rc;
+    if (!yvex_rocm_tensor_backed(tensor)) return refuse(err, YVEX_ERR_STATE, where, kUnbacked);
     rc = rocm_copy(backend, tensor->data, src, len, hipMemcpyHostToDevice,
                    YVEX_BACKEND_VARIANT_TENSOR_WRITE, where, err);
     if (rc != YVEX_OK) return rc;
@@ -166,6 +173,7 @@ static int rocm_tensor_read(yvex_backend *backend, const yvex_device_tensor *ten
     static const char where[] = "rocm.tensor_read";
     int rc = yvex_backend_tensor_rw_validate(where, backend, tensor, len, err);
     if (rc != YVEX_OK) return rc;
+    if (!yvex_rocm_tensor_backed(tensor)) return refuse(err, YVEX_ERR_STATE, where, kUnbacked);
     rc = rocm_copy(backend, dst, tensor->data, len, hipMemcpyDeviceToHost,
                    YVEX_BACKEND_VARIANT_TENSOR_READ, where, err);
     if (rc != YVEX_OK) return rc;
@@ -181,6 +189,7 @@ static int rocm_tensor_zero(yvex_backend *backend, yvex_device_tensor *tensor, y
     int rc;
     if (!backend_tensor_owner_is(backend, tensor))
         return refuse(err, YVEX_ERR_STATE, where, "tensor does not belong to this backend");
+    if (!yvex_rocm_tensor_backed(tensor)) return refuse(err, YVEX_ERR_STATE, where, kUnbacked);
     rc = yvex_rocm_require_capability(backend, YVEX_BACKEND_VARIANT_TENSOR_ZERO, where, err);
     if (rc != YVEX_OK) return rc;
     rc = yvex_rocm_status(&state->driver,
@@ -200,6 +209,8 @@ static int rocm_tensor_copy(yvex_backend *backend, yvex_device_tensor *dst,
     static const char where[] = "rocm.tensor_copy";
     int rc = yvex_backend_tensor_copy_validate(backend, dst, src, where, err);
     if (rc != YVEX_OK) return rc;
+    if (!yvex_rocm_tensor_backed(dst) || !yvex_rocm_tensor_backed(src))
+        return refuse(err, YVEX_ERR_STATE, where, kUnbacked);
     rc = rocm_copy(backend, dst->data, src->data, src->bytes, hipMemcpyDeviceToDevice,
                    YVEX_BACKEND_VARIANT_TENSOR_COPY, where, err);
     if (rc != YVEX_OK) return rc;
@@ -463,6 +474,9 @@ static const yvex_backend_vtable rocm_vtable = {
     .memory_stats = rocm_memory_stats,
     .device_info = rocm_device_info,
     .tensor_alloc = rocm_tensor_alloc,
+    .tensor_reserve = yvex_rocm_tensor_reserve,
+    .tensor_commit = yvex_rocm_tensor_commit,
+    .tensor_decommit = yvex_rocm_tensor_decommit,
     .tensor_free = rocm_tensor_free,
     .tensor_write = rocm_tensor_write,
     .tensor_read = rocm_tensor_read,
@@ -598,6 +612,13 @@ int yvex_backend_open_rocm_impl(yvex_backend **out, const char *device,
     if (state->driver.hipDeviceGetAttribute(&value, hipDeviceAttributeMultiprocessorCount,
                                             state->device_index) == hipSuccess)
         state->compute_units = value;
+    state->virtual_memory =
+        state->driver.virtual_memory &&
+        state->driver.hipDeviceGetAttribute(&value,
+                                            hipDeviceAttributeVirtualMemoryManagementSupported,
+                                            state->device_index) == hipSuccess &&
+        value != 0;
+    backend->virtual_tensor_ready = state->virtual_memory;
     if (state->driver.hipDeviceTotalMem(&total, state->device_index) == hipSuccess) {
         backend->device_info.global_memory_bytes = total;
         backend->device_info.total_memory_bytes = total;

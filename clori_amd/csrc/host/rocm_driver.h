@@ -24,6 +24,13 @@
     X(hipStreamBeginCapture) X(hipStreamEndCapture) X(hipGraphInstantiate) X(hipGraphLaunch) \
     X(hipGraphExecDestroy) X(hipGraphDestroy)
 
+/* Virtual memory management: an address range reserved once and backed by physical memory
+ * piece by piece.  Bound all or none; a runtime without them still opens and only the
+ * virtual-range tensor calls refuse. */
+#define YVEX_ROCM_DRIVER_VIRTUAL_ENTRIES(X)                                              \
+    X(hipMemGetAllocationGranularity) X(hipMemAddressReserve) X(hipMemAddressFree)       \
+    X(hipMemCreate) X(hipMemRelease) X(hipMemMap) X(hipMemUnmap) X(hipMemSetAccess)
+
 /* hipExtModuleLaunchKernel (hip/hip_ext.h, a C++ header): a launch whose two events take the
  * kernel's own begin and end timestamps.  Work sizes are in threads, not workgroups. */
 typedef hipError_t (*yvex_rocm_timed_launch_fn)(hipFunction_t, uint32_t, uint32_t, uint32_t, uint32_t,
@@ -35,7 +42,9 @@ typedef struct yvex_rocm_driver {
     char library_name[256];
 #define X(name) __typeof__(&name) name;
     YVEX_ROCM_DRIVER_ENTRIES(X)
+    YVEX_ROCM_DRIVER_VIRTUAL_ENTRIES(X) /* optional: all NULL when any is missing */
 #undef X
+    int virtual_memory;                 /* the virtual memory entries are bound */
     yvex_rocm_timed_launch_fn timed_launch; /* optional: NULL when the runtime lacks it */
 } yvex_rocm_driver;
 

@@ -74,6 +74,8 @@ typedef struct yvex_rocm_backend_state {
     int status_dirty;       /* deferred mode: launches since the last check */
     yvex_rocm_completion_mode completion_mode;
     unsigned long long live_tensors;
+    int unbacked_view;  /* the last view check failed on uncommitted pages, not on geometry */
+    int virtual_memory; /* the runtime and the device can reserve, map and unmap address ranges */
     int recording;                  /* a launch sequence is being recorded on the stream */
     unsigned long long live_graphs; /* recorded sequences not yet released */
     struct yvex_rocm_graph *graphs; /* ... and the list of them */
@@ -133,6 +135,21 @@ int yvex_rocm_temporary_acquire(yvex_backend *backend, unsigned long long bytes,
                                 int *owned, const char *where, yvex_error *err);
 int yvex_rocm_temporary_release(yvex_backend *backend, void *address, unsigned long long bytes,
                                 int owned, yvex_error *err);
+
+/* rocm_virtual.c: tensors over a reserved address range, backed where committed */
+int yvex_rocm_tensor_reserve(yvex_backend *backend, const yvex_backend_tensor_desc *desc,
+                             yvex_device_tensor **out, unsigned long long *granularity,
+                             yvex_error *err);
+int yvex_rocm_tensor_commit(yvex_backend *backend, yvex_device_tensor *tensor,
+                            unsigned long long offset, unsigned long long bytes,
+                            unsigned long long *resident_delta, yvex_error *err);
+int yvex_rocm_tensor_decommit(yvex_backend *backend, yvex_device_tensor *tensor,
+                              unsigned long long *released_bytes, yvex_error *err);
+int yvex_rocm_virtual_release(yvex_backend *backend, yvex_device_tensor *tensor, yvex_error *err);
+/* 1 for an ordinary tensor; for a tensor or view over a reserved range, 1 only when every
+ * byte of it lies on committed pages.  Anything handed to the device is checked with it: a
+ * read or write of an address without memory behind it is a device fault, not an error code. */
+int yvex_rocm_tensor_backed(const yvex_device_tensor *tensor);
 
 /* rocm_attention.c */
 int yvex_rocm_op_attention(yvex_backend *backend, const yvex_device_tensor *query,

@@ -250,6 +250,29 @@ int yvex_backend_tensor_alloc(yvex_backend *backend, const yvex_backend_tensor_d
 void yvex_backend_tensor_free(yvex_backend *backend, yvex_device_tensor *tensor);
 int yvex_backend_tensor_release(yvex_backend *backend, yvex_device_tensor **tensor,
                                 yvex_error *err);
+/* Virtual-range tensors (include/yvex/internal/backend.h:479-483, dispatch
+ * src/backend/core.c:613-680, device side src/backend/cuda/backend.c:500-834): the tensor
+ * owns a stable device address range of desc->bytes and no memory; commit_range backs the
+ * granules (of *granularity bytes) that intersect [offset, offset+bytes) and are not backed
+ * yet, zero-filled, and reports their bytes; it is idempotent and all-or-nothing, and only
+ * committed bytes count against the memory limit.  decommit returns every page and keeps
+ * the range; release returns both.  This is how the reference holds a layer's attention
+ * history that grows with the sequence (src/runtime/state_residency.c:258-287,441-446).
+ * A tensor or view handed to any operation of this backend must lie on committed pages,
+ * else YVEX_ERR_STATE.  Refusals: INVALID_ARG (missing argument, empty or out-of-range
+ * span, foreign or non-virtual tensor), STATE (backend failed / closing / recording),
+ * UNSUPPORTED (runtime or device without virtual memory management), NOMEM (limit). */
+/* include/yvex/internal/backend.h:257, src/backend/residency.c:12-17: what the caller asks
+ * before it plans a paged history (src/runtime/state_residency.c:593). */
+int yvex_backend_virtual_tensor_supported(const yvex_backend *backend);
+int yvex_backend_tensor_reserve(yvex_backend *backend, const yvex_backend_tensor_desc *desc,
+                                yvex_device_tensor **out, unsigned long long *granularity,
+                                yvex_error *err);
+int yvex_backend_tensor_commit_range(yvex_backend *backend, yvex_device_tensor *tensor,
+                                     unsigned long long offset, unsigned long long bytes,
+                                     unsigned long long *resident_delta, yvex_error *err);
+int yvex_backend_tensor_decommit(yvex_backend *backend, yvex_device_tensor *tensor,
+                                 unsigned long long *released_bytes, yvex_error *err);
 const char *yvex_device_tensor_name(const yvex_device_tensor *tensor);
 unsigned long long yvex_device_tensor_bytes(const yvex_device_tensor *tensor);
 int yvex_device_tensor_is_written(const yvex_device_tensor *tensor);

@@ -7,11 +7,13 @@
  * bookkeeping, failure transitions and cleanup of the C host can run on the CPU, the
  * way the reference swaps entries of its driver table in tests/unit/cuda/graph.c:265-289.
  */
+#define _GNU_SOURCE
 #define __HIP_PLATFORM_AMD__ 1
 #include <hip/hip_runtime_api.h>
 
 #include <stdlib.h>
 #include <string.h>
+#include <sys/mman.h>
 
 static unsigned long long launches, allocations, frees, loads, unloads;
 static int capturing;                       /* a stream capture is open */
@@ -53,7 +55,10 @@ hipError_t hipDeviceGetName(char *name, int len, hipDevice_t device)
 hipError_t hipDeviceGetAttribute(int *value, hipDeviceAttribute_t attribute, int device)
 {
     (void)device;
-    *value = attribute == hipDeviceAttributeMultiprocessorCount ? 256 : 9;
+    if (attribute == hipDeviceAttributeVirtualMemoryManagementSupported)
+        *value = env_is("FAKE_HIP_VIRTUAL_MEMORY", "absent") ? 0 : 1;
+    else
+        *value = attribute == hipDeviceAttributeMultiprocessorCount ? 256 : 9;
     return hipSuccess;
 }
 
@@ -220,3 +225,98 @@ hipError_t hipGraphLaunch(hipGraphExec_t exec, hipStream_t stream)
 
 hipError_t hipGraphExecDestroy(hipGraphExec_t exec) { free(exec); return hipSuccess; }
 hipError_t hipGraphDestroy(hipGraph_t graph) { free(graph); return hipSuccess; }
+
+/* Virtual memory management on host pages: a reservation is an inaccessible mapping, mapping
+ * a physical handle makes its pages readable and writable, unmapping takes that away and
+ * drops their contents.  Touching a reserved but unmapped address is a segmentation fault,
+ * as it is a fault on the device. */
+#define FAKE_GRANULARITY ((size_t)1u << 16)
+struct fake_physical { size_t size; };
+static unsigned long long physical_created, physical_released, ranges_reserved, ranges_freed;
+static unsigned long long mapped_bytes;
+
+unsigned long long fake_hip_live_physical(void) { return physical_created - physical_released; }
+unsigned long long fake_hip_live_ranges(void) { return ranges_reserved - ranges_freed; }
+unsigned long long fake_hip_mapped_bytes(void) { return mapped_bytes; }
+
+hipError_t hipMemGetAllocationGranularity(size_t *granularity, const hipMemAllocationProp *prop,
+                                          hipMemAllocationGranularity_flags option)
+{
+    (void)prop; (void)option;
+    *granularity = FAKE_GRANULARITY;
+    return hipSuccess;
+}
+
+hipError_t hipMemAddressReserve(void **ptr, size_t size, size_t alignment, void *addr,
+                                unsigned long long flags)
+{
+    void *base;
+    (void)alignment; (void)addr; (void)flags;
+    if (env_is("FAKE_HIP_RESERVE", "fail") || size % FAKE_GRANULARITY) return hipErrorOutOfMemory;
+    base = mmap(NULL, size, PROT_NONE, MAP_PRIVATE | MAP_ANONYMOUS | MAP_NORESERVE, -1, 0);
+    if (base == MAP_FAILED) return hipErrorOutOfMemory;
+    *ptr = base;
+    ++ranges_reserved;
+    return hipSuccess;
+}
+
+hipError_t hipMemAddressFree(void *ptr, size_t size)
+{
+    if (env_is("FAKE_HIP_ADDRESS_FREE", "fail")) return hipErrorUnknown;
+    if (munmap(ptr, size) != 0) return hipErrorInvalidValue;
+    ++ranges_freed;
+    return hipSuccess;
+}
+
+hipError_t hipMemCreate(hipMemGenericAllocationHandle_t *handle, size_t size,
+                        const hipMemAllocationProp *prop, unsigned long long flags)
+{
+    const char *limit = getenv("FAKE_HIP_PHYSICAL_LIMIT"); /* handles that may be live at once */
+    struct fake_physical *physical;
+    (void)prop; (void)flags;
+    if (size == 0u || size % FAKE_GRANULARITY) return hipErrorInvalidValue;
+    if (limit && fake_hip_live_physical() >= strtoull(limit, NULL, 10)) return hipErrorOutOfMemory;
+    physical = (struct fake_physical *)calloc(1, sizeof(*physical));
+    if (!physical) return hipErrorOutOfMemory;
+    physical->size = size;
+    *handle = (hipMemGenericAllocationHandle_t)physical;
+    ++physical_created;
+    return hipSuccess;
+}
+
+hipError_t hipMemRelease(hipMemGenericAllocationHandle_t handle)
+{
+    if (env_is("FAKE_HIP_RELEASE", "fail")) return hipErrorUnknown;
+    free((struct fake_physical *)handle);
+    ++physical_released;
+    return hipSuccess;
+}
+
+hipError_t hipMemMap(void *ptr, size_t size, size_t offset, hipMemGenericAllocationHandle_t handle,
+                     unsigned long long flags)
+{
+    (void)flags;
+    if (env_is("FAKE_HIP_MAP", "fail")) return hipErrorOutOfMemory;
+    if (offset != 0u || size != ((struct fake_physical *)handle)->size) return hipErrorInvalidValue;
+    if (mprotect(ptr, size, PROT_READ | PROT_WRITE) != 0) return hipErrorInvalidValue;
+    memset(ptr, 0xa5, size); /* fresh device memory is not zero */
+    mapped_bytes += size;
+    return hipSuccess;
+}
+
+hipError_t hipMemUnmap(void *ptr, size_t size)
+{
+    if (env_is("FAKE_HIP_UNMAP", "fail")) return hipErrorUnknown;
+    if (madvise(ptr, size, MADV_DONTNEED) != 0 || mprotect(ptr, size, PROT_NONE) != 0)
+        return hipErrorInvalidValue;
+    mapped_bytes -= size;
+    return hipSuccess;
+}
+
+hipError_t hipMemSetAccess(void *ptr, size_t size, const hipMemAccessDesc *desc, size_t count)
+{
+    (void)ptr; (void)size;
+    if (env_is("FAKE_HIP_ACCESS", "fail")) return hipErrorInvalidValue;
+    return desc && count == 1u && desc->flags == hipMemAccessFlagsProtReadWrite ? hipSuccess
+                                                                               : hipErrorInvalidValue;
+}

@@ -317,6 +317,167 @@ def test_f32_subview_matches_reference_rules():
         assert lib().yvex_backend_tensor_f32_subview(t.handle, 0, 0, C.byref(view)) == 0
 
 
+# ------------------------------------------------ virtual-range tensors ----
+
+def test_virtual_tensor_sequence_of_the_reference_unit_test(fake_runtime):
+    """The steps of tests/unit/cuda/tensor.c:30-89, assertion for assertion."""
+    with Backend() as b:
+        before = b.memory_stats().allocated_bytes
+        t = b.reserve("rocm_virtual_pages", B.DTYPE_I8, (16 << 20,))
+        g = t.granularity
+        assert g and t.handle.contents.virtual_reserved and t.resident_bytes == 0
+        assert b.memory_stats().allocated_bytes == before      # an address range costs no memory
+        assert fake_runtime.fake_hip_live_physical() == 0
+        assert t.commit(g + 1, 1) == g and t.resident_bytes == g     # exactly one granule
+        assert t.commit(g + 2, 1) == 0 and t.resident_bytes == g     # idempotent
+        assert t.commit(3 * g, 1) == g and t.resident_bytes == 2 * g  # a disjoint granule
+        view = t.view(g + 1, B.DTYPE_I8, (1,))
+        view.write(np.array([0x5a], np.int8))
+        assert view.read()[0] == 0x5a
+        assert b.memory_stats().allocated_bytes == before + 2 * g
+        assert t.decommit() == 2 * g and t.resident_bytes == 0 and not t.is_written
+        assert b.memory_stats().allocated_bytes == before
+        assert fake_runtime.fake_hip_live_physical() == 0 and fake_runtime.fake_hip_mapped_bytes() == 0
+        assert fake_runtime.fake_hip_live_ranges() == 1        # the address range is kept
+        t.release()
+        assert t.handle is None and fake_runtime.fake_hip_live_ranges() == 0
+
+
+def test_virtual_tensor_commit_is_zero_filled_granule_by_granule_and_checked(fake_runtime):
+    with Backend(memory_limit_bytes=32 << 20) as b:
+        t = b.reserve("history", B.DTYPE_I8, (64 << 21,))     # 64 granules
+        g = t.granularity
+        assert g == 2 << 20              # the stand-in runtime reports 64 KiB: 2 MiB is the floor
+        # a span that touches five granules backs five, one equal-sized mapping each
+        assert t.commit(2 * g + 5, 4 * g) == 5 * g and fake_runtime.fake_hip_live_physical() == 5
+        assert np.all(t.view(2 * g, B.DTYPE_I8, (5 * g,)).read() == 0)   # fresh pages read as zero
+        # a span around it adds only the missing granules on each side
+        assert t.commit(g, 8 * g) == 3 * g and fake_runtime.fake_hip_live_physical() == 8
+        assert b.memory_stats().allocated_bytes == 8 * g and t.resident_bytes == 8 * g
+        assert fake_runtime.fake_hip_mapped_bytes() == 8 * g
+        # the memory limit counts committed bytes: 32 MiB = 16 granules
+        with pytest.raises(YvexError) as e:
+            t.commit(20 * g, 9 * g)
+        assert e.value.code == B.YVEX_ERR_NOMEM and "memory limit" in e.value.message
+        assert t.resident_bytes == 8 * g and fake_runtime.fake_hip_live_physical() == 8
+        assert t.commit(20 * g, 8 * g) == 8 * g
+        # anything handed to the device must lie on committed pages
+        for bad in (t.view(0, B.DTYPE_I8, (g + 1,)), t.view(9 * g - 1, B.DTYPE_I8, (2,)), t):
+            with pytest.raises(YvexError) as e:
+                bad.read()
+            assert e.value.code == B.YVEX_ERR_STATE and "not committed" in e.value.message
+            with pytest.raises(YvexError) as e:
+                bad.zero()
+            assert e.value.code == B.YVEX_ERR_STATE
+        inside = t.view(g, B.DTYPE_I8, (8 * g,))
+        inside.write(np.full(8 * g, 7, np.int8))
+        assert np.all(inside.read() == 7)
+        # a committed page that is given back and committed again reads as zero again
+        assert t.decommit() == 16 * g
+        assert t.commit(g, 1) == g and np.all(t.view(g, B.DTYPE_I8, (g,)).read() == 0)
+        plain = b.tensor("plain", B.DTYPE_I8, (g + 1,))
+        err = B.Error()
+        assert lib().yvex_backend_tensor_copy(b.handle, plain.handle,
+                                              t.view(0, B.DTYPE_I8, (g + 1,)).handle,
+                                              C.byref(err)) == B.YVEX_ERR_STATE
+        with pytest.raises(YvexError) as e:                     # not a workspace
+            b.workspace_attach(t)
+        assert e.value.code == B.YVEX_ERR_INVALID_ARG
+
+
+def test_virtual_tensor_refusals(env, fake_runtime):
+    with Backend() as b:
+        err, out, gran, delta = B.Error(), B.TensorP(), C.c_ulonglong(5), C.c_ulonglong(5)
+        desc = B.TensorDesc(b"range", B.DTYPE_I8, 1)
+        desc.dims[0] = desc.bytes = 1 << 22
+        L = lib()
+        assert L.yvex_backend_tensor_reserve(b.handle, C.byref(desc), None, C.byref(gran),
+                                             C.byref(err)) == B.YVEX_ERR_INVALID_ARG and gran.value == 0
+        assert L.yvex_backend_tensor_reserve(b.handle, C.byref(desc), C.byref(out), None,
+                                             C.byref(err)) == B.YVEX_ERR_INVALID_ARG
+        desc.bytes = 0
+        assert L.yvex_backend_tensor_reserve(b.handle, C.byref(desc), C.byref(out), C.byref(gran),
+                                             C.byref(err)) == B.YVEX_ERR_INVALID_ARG
+        desc.bytes = 1 << 22
+        t = b.reserve("range", B.DTYPE_I8, (1 << 22,))
+        plain = b.tensor("plain", B.DTYPE_I8, (1 << 22,))
+        for tensor, offset, count in ((t, 0, 0), (t, (1 << 22) + 1, 1), (t, 1 << 22, 1),
+                                      (t, 5, 1 << 22), (plain, 0, 16)):
+            delta.value = 5
+            rc = L.yvex_backend_tensor_commit_range(b.handle, tensor.handle, offset, count,
+                                                    C.byref(delta), C.byref(err))
+            assert rc == B.YVEX_ERR_INVALID_ARG and delta.value == 0, (offset, count)
+        assert L.yvex_backend_tensor_commit_range(b.handle, t.handle, 0, 1, None,
+                                                  C.byref(err)) == B.YVEX_ERR_INVALID_ARG
+        assert L.yvex_backend_tensor_decommit(b.handle, plain.handle, C.byref(delta),
+                                              C.byref(err)) == B.YVEX_ERR_INVALID_ARG
+        assert L.yvex_backend_tensor_decommit(b.handle, t.handle, None,
+                                              C.byref(err)) == B.YVEX_ERR_INVALID_ARG
+        t.commit(0, 1)
+        assert L.yvex_backend_tensor_decommit(b.handle, t.view(16, B.DTYPE_I8, (16,)).handle,
+                                              C.byref(delta), C.byref(err)) == B.YVEX_ERR_INVALID_ARG
+        with Backend() as other:                                # a foreign backend's range
+            assert L.yvex_backend_tensor_commit_range(other.handle, t.handle, 0, 1, C.byref(delta),
+                                                      C.byref(err)) == B.YVEX_ERR_INVALID_ARG
+            assert L.yvex_backend_tensor_decommit(other.handle, t.handle, C.byref(delta),
+                                                  C.byref(err)) == B.YVEX_ERR_INVALID_ARG
+        b.graph_begin()                                         # not while recording
+        for call in (lambda: b.reserve("late", B.DTYPE_I8, (1 << 20,)), lambda: t.commit(1 << 21, 1),
+                     t.decommit):
+            with pytest.raises(YvexError) as e:
+                call()
+            assert e.value.code == B.YVEX_ERR_STATE
+        b.graph_release(b.graph_end())
+        assert lib().yvex_backend_virtual_tensor_supported(b.handle) == 1
+    assert lib().yvex_backend_virtual_tensor_supported(None) == 0
+    env("FAKE_HIP_VIRTUAL_MEMORY", "absent")                    # a device without the feature
+    with Backend() as b:
+        assert lib().yvex_backend_virtual_tensor_supported(b.handle) == 0
+        with pytest.raises(YvexError) as e:
+            b.reserve("range", B.DTYPE_I8, (1 << 20,))
+        assert e.value.code == B.YVEX_ERR_UNSUPPORTED and "unavailable" in e.value.message
+        assert f32(b, "still-works", (4,)).read().sum() == 0
+
+
+@pytest.mark.parametrize("injected", ["FAKE_HIP_MAP", "FAKE_HIP_ACCESS", "FAKE_HIP_PHYSICAL_LIMIT"])
+def test_virtual_tensor_failed_commit_leaves_nothing_behind(env, fake_runtime, injected):
+    with Backend() as b:
+        t = b.reserve("history", B.DTYPE_I8, (32 << 21,))
+        g = t.granularity
+        assert t.commit(4 * g, g) == g
+        stats = b.memory_stats().allocated_bytes
+        # two runs are missing around the committed granule; the limit lets the first through
+        env(injected, "2" if injected == "FAKE_HIP_PHYSICAL_LIMIT" else "fail")
+        with pytest.raises(YvexError) as e:
+            t.commit(2 * g, 6 * g)
+        assert e.value.code == B.YVEX_ERR_BACKEND
+        assert b.status == B.STATUS_READY                       # rolled back cleanly: still usable
+        assert t.resident_bytes == g and b.memory_stats().allocated_bytes == stats
+        assert fake_runtime.fake_hip_live_physical() == 1 and fake_runtime.fake_hip_mapped_bytes() == g
+        env(injected, None)
+        assert t.commit(2 * g, 6 * g) == 5 * g                  # and the same commit then succeeds
+        assert np.all(t.view(2 * g, B.DTYPE_I8, (6 * g,)).read() == 0)
+
+
+def test_virtual_tensor_failed_release_keeps_the_owner(env, fake_runtime):
+    b = Backend()
+    t = b.reserve("history", B.DTYPE_I8, (8 << 21,))
+    t.commit(0, 3 << 21)
+    env("FAKE_HIP_UNMAP", "fail")
+    with pytest.raises(YvexError) as e:
+        t.decommit()
+    assert e.value.code == B.YVEX_ERR_BACKEND and t.resident_bytes == 3 << 21
+    with pytest.raises(YvexError):
+        t.release()                                             # a failed release fails the backend
+    assert t.handle is not None and b.status == B.STATUS_FAILED
+    assert lib().yvex_backend_virtual_tensor_supported(b.handle) == 0   # a failed backend says no
+    env("FAKE_HIP_UNMAP", None)
+    t.release()                                                 # cleanup-only release still works
+    assert fake_runtime.fake_hip_live_physical() == 0 and fake_runtime.fake_hip_live_ranges() == 0
+    b.tensors.clear()
+    b.close()
+
+
 # ------------------------------------------------- operation admission ----
 
 def test_bounded_primitive_refusal_order_and_facts(fake_runtime):
