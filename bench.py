@@ -14,7 +14,7 @@ already resident in HBM.  Workloads are the five configurations the metric is qu
 
 By name only (not configurations of the metric): exact2 and exact1 (configurations 2 and 1
 under the EXACT_F32 contract: fp32 matrix cores, and double-precision split decode),
-append_bf16 / append_q8_0 (the KV page writer), copy.
+append_bf16 / append_q8_0 (the KV page writer), history_append (the token-major writer), copy.
 
 Prints ONE JSON line.  `value` is the headline workload's throughput; every workload
 that ran is listed under "workloads" with its own roofline figures.  Timing uses HIP
@@ -375,6 +375,39 @@ def workload_append(backend, rng, steps, warmup, q8=False):
                 launches=int(facts.kernel_launches), kernels=kernels, **timed)
 
 
+def workload_history_append(backend, rng, steps, warmup):
+    """The token-major history writer on a prompt: 8192 new tokens, 8 kv heads, d=128,
+    rotate-half on the whole key row, into an interleaved [K | V] history that lives in a
+    reserved address range committed for these rows.  Not one of the metric's
+    configurations: run by name."""
+    hkv, d, new, first = 8, 128, 8192, 1000
+    width = hkv * d
+    used = first + new
+    history = backend.reserve("history", B.DTYPE_BF16, (32768, 2 * width))
+    history.commit(0, used * 2 * width * 2)
+    count = (used - 1) * 2 * width + width
+    kh = history.view(0, B.DTYPE_BF16, (count,))
+    vh = history.view(2 * width, B.DTYPE_BF16, (count,))
+    angles = rng.uniform(-3.0, 3.0, size=(new, d)).astype(np.float32)
+    key = backend.tensor("k-new", B.DTYPE_BF16, (new, hkv, d), random_bf16(rng, new * hkv * d))
+    value = backend.tensor("v-new", B.DTYPE_BF16, (new, hkv, d), random_bf16(rng, new * hkv * d))
+    cosine = backend.tensor("cos", B.DTYPE_F32, angles.shape, np.cos(angles))
+    sine = backend.tensor("sin", B.DTYPE_F32, angles.shape, np.sin(angles))
+    run = lambda: backend.history_append_execute(  # noqa: E731
+        key, value, kh, vh, first, hkv, cosine=cosine, sine=sine, rotary_dimension=d,
+        key_token_stride=2 * width, value_token_stride=2 * width)
+    facts = run()
+    kernels = ["yvex_rocm_history_append_bf16"]
+    timed = time_steps(backend, run, steps, warmup, kernels)
+    # per token: K and V rows in, both out, half a cos and half a sin row
+    algo = new * (4 * width * 2 + d * 4)
+    return dict(name="history_append",
+                workload="token-major history writer: 8192 new tokens behind 1000, 8 kv heads, "
+                         "d=128, rotary 128, interleaved [K|V] rows in a reserved address range",
+                bound="hbm", algorithmic_bytes=algo, tokens=new,
+                launches=int(facts.kernel_launches), kernels=kernels, **timed)
+
+
 def copy_reference(backend, steps):
     """A device-to-device copy of known size: the scale for the FETCH_SIZE / WRITE_SIZE
     counters.  Not a workload of the metric; run as --workload copy."""
@@ -402,11 +435,12 @@ WORKLOADS = {
 EXTRA_WORKLOADS = {
     "append_bf16": lambda b, r, s, w: workload_append(b, r, s, w, q8=False),
     "append_q8_0": lambda b, r, s, w: workload_append(b, r, s, w, q8=True),
+    "history_append": workload_history_append,
     "exact2": workload_exact2,
     "exact1": workload_exact1,
 }
 SEEDS = {"decode1": 1, "prefill2": 2, "paged3": 3, "paged4": 4, "mla5": 5, "append_bf16": 6,
-         "append_q8_0": 7, "exact2": 8, "exact1": 9}
+         "append_q8_0": 7, "exact2": 8, "exact1": 9, "history_append": 10}
 
 
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")

@@ -477,6 +477,29 @@ class Backend:
         return facts
 
 
+    def history_append_execute(self, key, value, key_history, value_history, first_row, kv_heads,
+                               head_dimension=128, cosine=None, sine=None, rotary_dimension=0,
+                               key_token_stride=0, value_token_stride=0):
+        """Writes the new rows (keys rotated) into rows first_row.. of the token-major K and V
+        history views; all tensor arguments are device tensors."""
+        ops = self.rocm_attention_operations()
+        if ops is None:
+            raise YvexError(B.YVEX_ERR_UNSUPPORTED, "rocm_attention_operations", "not published")
+        r = B.HistoryAppendRequirement()
+        r.tokens, r.first_row = key.shape[0], first_row
+        r.key_value_heads, r.head_dimension = kv_heads, head_dimension
+        r.rotary_dimension = rotary_dimension
+        r.key_token_stride, r.value_token_stride = key_token_stride, value_token_stride
+        request = B.HistoryAppendRequest(r, key.handle, value.handle,
+                                         cosine.handle if cosine else None,
+                                         sine.handle if sine else None, key_history.handle,
+                                         value_history.handle)
+        facts, err = B.OperationFacts(), B.Error()
+        _check(ops.history_append_execute(self.handle, C.byref(request), C.byref(facts),
+                                          C.byref(err)), err)
+        return facts
+
+
 # -- host helpers that are part of the product (layout + codecs, no attention math) --
 
 def kv_pack_pages(rows, storage, is_value, kv_heads, head_dim=128, page_tokens=16):

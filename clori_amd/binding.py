@@ -235,6 +235,20 @@ PAGED_EXECUTE_FUSED_FN = C.CFUNCTYPE(C.c_int, C.c_void_p, C.POINTER(PagedDecodeR
                                      C.POINTER(AttentionEpilogue), FactsP, ErrorP)
 
 
+class HistoryAppendRequirement(C.Structure):
+    _fields_ = [(n, ull) for n in ("tokens", "first_row", "key_value_heads", "head_dimension",
+                                   "rotary_dimension", "key_token_stride", "value_token_stride")]
+
+
+class HistoryAppendRequest(C.Structure):
+    _fields_ = [("requirement", HistoryAppendRequirement), ("key", TensorP), ("value", TensorP),
+                ("cosine", TensorP), ("sine", TensorP), ("key_history", TensorP),
+                ("value_history", TensorP)]
+
+
+HISTORY_APPEND_FN = C.CFUNCTYPE(C.c_int, C.c_void_p, C.POINTER(HistoryAppendRequest), FactsP, ErrorP)
+
+
 class RocmAttentionOperations(C.Structure):
     _fields_ = [("attention_execute_lse", EXECUTE_LSE_FN),
                 ("paged_decode_workspace_required", PAGED_WORKSPACE_FN),
@@ -243,7 +257,8 @@ class RocmAttentionOperations(C.Structure):
                 ("mla_decode_execute", MLA_EXECUTE_FN),
                 ("kv_append_execute", KV_APPEND_FN),
                 ("attention_execute_fused", EXECUTE_FUSED_FN),
-                ("paged_decode_execute_fused", PAGED_EXECUTE_FUSED_FN)]
+                ("paged_decode_execute_fused", PAGED_EXECUTE_FUSED_FN),
+                ("history_append_execute", HISTORY_APPEND_FN)]
 
 
 class RocmReport(C.Structure):

@@ -1354,6 +1354,98 @@ static int rocm_kv_append_execute(yvex_backend *backend, const yvex_rocm_kv_appe
     return YVEX_OK;
 }
 
+/* ------------------------------------------- token-major history writer ---- */
+
+static int rocm_history_append_execute(yvex_backend *backend,
+                                       const yvex_rocm_history_append_request *request,
+                                       yvex_backend_operation_facts *facts, yvex_error *err)
+{
+    static const char where[] = "rocm.history_append";
+    const yvex_backend_operation_variant variant = YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_BF16;
+    yvex_rocm_backend_state *state = yvex_rocm_state(backend);
+    const yvex_rocm_history_append_requirement *r;
+    yvex_rocm_history_append_params hp;
+    unsigned long long width, k_stride, v_stride, rows, new_elements, k_elements, v_elements, pieces;
+    int rc;
+    if (!request || !request->key || !request->value || !request->key_history ||
+        !request->value_history || !facts)
+        return refuse(err, YVEX_ERR_INVALID_ARG, where,
+                      "complete history-append tensors and result facts are required");
+    rc = backend_dispatch_admit(backend, where, err);
+    if (rc != YVEX_OK) return rc;
+    r = &request->requirement;
+    if (!r->tokens || !r->key_value_heads || !r->head_dimension ||
+        !yvex_core_u64_mul(r->key_value_heads, r->head_dimension, &width) ||
+        !yvex_core_u64_add(r->first_row, r->tokens, &rows) ||
+        (r->rotary_dimension && (!request->cosine || !request->sine)))
+        return refuse(err, YVEX_ERR_INVALID_ARG, where, "complete history-append geometry is required");
+    k_stride = r->key_token_stride ? r->key_token_stride : width;
+    v_stride = r->value_token_stride ? r->value_token_stride : width;
+    if (k_stride < width || v_stride < width)
+        return refuse(err, YVEX_ERR_INVALID_ARG, where,
+                      "a history token stride is narrower than one row of key/value heads");
+    if (r->head_dimension % 8ull || r->head_dimension > 256ull || (k_stride | v_stride) % 8ull ||
+        r->rotary_dimension > r->head_dimension || r->rotary_dimension % 16ull ||
+        r->tokens > 0x7fffffffull || r->key_value_heads > 65535ull)
+        return refuse(err, YVEX_ERR_UNSUPPORTED, where,
+                      "ROCm history append requires a head dimension and token strides that are "
+                      "multiples of 8 (at most 256 lanes per head) and a rotary dimension that is a "
+                      "multiple of 16");
+    memset(facts, 0, sizeof(*facts));
+    if (!state || !yvex_core_u64_mul(r->tokens, width, &new_elements) ||
+        !yvex_core_u64_mul(rows - 1ull, k_stride, &k_elements) ||
+        !yvex_core_u64_add(k_elements, width, &k_elements) ||
+        !yvex_core_u64_mul(rows - 1ull, v_stride, &v_elements) ||
+        !yvex_core_u64_add(v_elements, width, &v_elements) ||
+        !yvex_core_u64_mul(r->tokens * r->key_value_heads, r->head_dimension / 8ull, &pieces) ||
+        (pieces + 255ull) / 256ull > 0x7fffffffull)
+        return refuse(err, YVEX_ERR_BOUNDS, where, "history-append geometry exceeds admitted range");
+    /* a history may be fresh or hold earlier tokens: written state is not required of it */
+    if (!view_ok(backend, request->key, YVEX_DTYPE_BF16, new_elements, 1) ||
+        !view_ok(backend, request->value, YVEX_DTYPE_BF16, new_elements, 1) ||
+        (r->rotary_dimension &&
+         (!view_ok(backend, request->cosine, YVEX_DTYPE_F32, r->tokens * r->rotary_dimension, 1) ||
+          !view_ok(backend, request->sine, YVEX_DTYPE_F32, r->tokens * r->rotary_dimension, 1))) ||
+        !view_ok(backend, request->key_history, YVEX_DTYPE_BF16, k_elements, 0) ||
+        !view_ok(backend, request->value_history, YVEX_DTYPE_BF16, v_elements, 0))
+        return view_refusal(backend, err, where,
+                            "new rows, tables and history views must be tensors of this backend "
+                            "with the declared geometry");
+    if (((uintptr_t)request->key->data | (uintptr_t)request->value->data |
+         (uintptr_t)request->key_history->data | (uintptr_t)request->value_history->data) & 15u)
+        return refuse(err, YVEX_ERR_UNSUPPORTED, where,
+                      "ROCm history append requires 16-byte aligned rows");
+    memset(&hp, 0, sizeof(hp));
+    hp.key = (const uint16_t *)request->key->data;
+    hp.value = (const uint16_t *)request->value->data;
+    hp.cosine = r->rotary_dimension ? (const float *)request->cosine->data : NULL;
+    hp.sine = r->rotary_dimension ? (const float *)request->sine->data : NULL;
+    hp.key_history = (uint16_t *)request->key_history->data;
+    hp.value_history = (uint16_t *)request->value_history->data;
+    hp.status = state->device_status;
+    hp.first_row = r->first_row;
+    hp.key_token_stride = k_stride;
+    hp.value_token_stride = v_stride;
+    hp.tokens = (uint32_t)r->tokens;
+    hp.kv_heads = (uint32_t)r->key_value_heads;
+    hp.head_dim = (uint32_t)r->head_dimension;
+    hp.rotary_dim = (uint32_t)r->rotary_dimension;
+    backend_workspace_reset(backend);
+    rc = yvex_rocm_launch(backend, YVEX_ROCM_FN_HISTORY_APPEND_BF16, variant,
+                          (unsigned int)((pieces + 255ull) / 256ull), 1u, 1u, 256u, 0u, &hp, where,
+                          err);
+    if (rc == YVEX_OK) {
+        facts->kernel_launches = 1ull;
+        facts->compulsory_memory_facts_available = 1;
+        rc = yvex_rocm_complete(backend, variant, where, facts, err);
+    }
+    if (rc != YVEX_OK) return rc;
+    request->key_history->is_written = 1;
+    request->value_history->is_written = 1;
+    yvex_error_clear(err);
+    return YVEX_OK;
+}
+
 /* ---------------------------------------------------------- op tables ---- */
 
 static const yvex_backend_transformer_operations rocm_transformer_ops = {
@@ -1370,6 +1462,7 @@ static const yvex_backend_rocm_attention_operations rocm_attention_ops = {
     .kv_append_execute = rocm_kv_append_execute,
     .attention_execute_fused = rocm_attention_execute_fused,
     .paged_decode_execute_fused = rocm_paged_decode_execute_fused,
+    .history_append_execute = rocm_history_append_execute,
 };
 
 /* A table is published only once the kernel bundle is admitted

@@ -75,6 +75,8 @@ static const rocm_kernel_binding rocm_kernel_bindings[] = {
      YVEX_ROCM_FN_KV_APPEND_BF16},
     {"yvex_rocm_kv_append_q8_0", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_PAGED_Q8_0,
      YVEX_ROCM_FN_KV_APPEND_Q8_0},
+    {"yvex_rocm_history_append_bf16", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_BF16,
+     YVEX_ROCM_FN_HISTORY_APPEND_BF16},
 };
 #define ROCM_KERNEL_BINDING_COUNT (sizeof(rocm_kernel_bindings) / sizeof(rocm_kernel_bindings[0]))
 

@@ -397,3 +397,44 @@ yvex_rocm_kv_append_q8_0(const yvex_rocm_kv_append_params p)
         if (!ok || !representable) flag(p.status, YVEX_ROCM_DEVICE_NUMERIC);
     }
 }
+
+// Token-major history writer: the reference appends the new tokens to a layer's history with
+// two device copies per token, key then value, into rows of [K | V]
+// (src/runtime/stateful_attention.c:183-222) after a separate rotary pass over the keys
+// (src/runtime/decoder.c:1236-1242).  Here one launch does both: thread i owns the 16-byte
+// piece (token, kv head, dims 8 * c8 .. 8 * c8 + 7) of the value row and of the key row, with
+// the rotary roles of the page writer (a lower-half piece produces its upper-half partner).
+extern "C" __global__ void __launch_bounds__(256)
+yvex_rocm_history_append_bf16(const yvex_rocm_history_append_params p)
+{
+    const uint32_t pieces = p.head_dim / 8u, pairs = p.rotary_dim / 16u;
+    const uint64_t id = (uint64_t)blockIdx.x * 256u + threadIdx.x;
+    const uint64_t total = (uint64_t)p.tokens * p.kv_heads * pieces;
+    if (id >= total) return;
+    const uint32_t c8 = (uint32_t)(id % pieces), head = (uint32_t)(id / pieces % p.kv_heads);
+    const uint32_t token = (uint32_t)(id / pieces / p.kv_heads);
+    const uint64_t in = ((uint64_t)token * p.kv_heads + head) * p.head_dim + c8 * 8u;
+    const uint64_t row = p.first_row + token;
+    uint16_t *kdst = p.key_history + row * p.key_token_stride + (uint64_t)head * p.head_dim + c8 * 8u;
+    uint16_t *vdst = p.value_history + row * p.value_token_stride + (uint64_t)head * p.head_dim + c8 * 8u;
+    KeyChunk k;
+    k.t = 0u;
+    k.c8 = c8;
+    k.role = c8 < pairs ? kLower : c8 < 2u * pairs ? kUpper : kPlain;
+    const u32x4 v = load_b128(p.value + in);
+    if (k.role != kUpper) k.own = load_b128(p.key + in);
+    if (k.role == kLower) {
+        const uint64_t at = (uint64_t)token * p.rotary_dim + c8 * 8u;
+        k.other = load_b128(p.key + in + p.rotary_dim / 2u);
+        k.cs[0] = load_b128(p.cosine + at);
+        k.cs[1] = load_b128(p.cosine + at + 4);
+        k.sn[0] = load_b128(p.sine + at);
+        k.sn[1] = load_b128(p.sine + at + 4);
+    }
+    u32x4 lower, upper;
+    bool ok = key_finish(k, lower, upper) && finite_bits(v);
+    *reinterpret_cast<u32x4 *>(vdst) = v;
+    if (k.role != kUpper) *reinterpret_cast<u32x4 *>(kdst) = lower;
+    if (k.role == kLower) *reinterpret_cast<u32x4 *>(kdst + p.rotary_dim / 2u) = upper;
+    if (!ok) flag(p.status, YVEX_ROCM_DEVICE_NUMERIC);
+}

@@ -610,6 +610,37 @@ typedef struct yvex_rocm_kv_append_request {
 } yvex_rocm_kv_append_request;
 
 /*
+ * Token-major history writer: the step in front of attention for the reference's own
+ * history layout.  The reference rotates the new keys in a pass of their own
+ * (src/runtime/decoder.c:1236-1242) and then appends every token with two device copies,
+ * key then value, into row history_tokens + t of the layer's [K | V] history
+ * (src/runtime/stateful_attention.c:183-222).  This does both in one launch: rows
+ * first_row .. first_row + tokens - 1 of key_history and value_history receive the new rows
+ * (keys rotated: rotate-half over the first rotary_dimension lanes of every head,
+ * src/backend/cuda/transformer_kernels.cu:79-108, every product and sum rounded to BF16),
+ * nothing else is touched.  key_history / value_history are the views attention_execute is
+ * handed afterwards for key_value_tokens = first_row + tokens: BF16,
+ * (first_row + tokens - 1) * stride + key_value_heads * head_dimension elements, strides in
+ * elements (0 = packed); for the reference's interleaved rows both views lie in one tensor,
+ * the value view key_value_heads * head_dimension elements behind the key view, stride twice
+ * that.  Over a reserved address range the rows must be committed first.  head_dimension
+ * and both strides must be multiples of 8, rotary_dimension a multiple of 16; non-finite
+ * inputs, table entries or results are YVEX_ERR_FORMAT.
+ */
+typedef struct yvex_rocm_history_append_requirement {
+    unsigned long long tokens, first_row;
+    unsigned long long key_value_heads, head_dimension, rotary_dimension;
+    unsigned long long key_token_stride, value_token_stride;
+} yvex_rocm_history_append_requirement;
+
+typedef struct yvex_rocm_history_append_request {
+    yvex_rocm_history_append_requirement requirement;
+    const yvex_device_tensor *key, *value;   /* BF16 [tokens][kv_heads][d] */
+    const yvex_device_tensor *cosine, *sine; /* F32 [tokens][rotary_dimension], or NULL without rotary */
+    yvex_device_tensor *key_history, *value_history;
+} yvex_rocm_history_append_request;
+
+/*
  * Epilogue fused into the attention kernels.  The arithmetic is the reference's sigmoid
  * output gate (yvex_sigmoid_product_bf16_f32, src/backend/cuda/transformer_kernels.cu:353-364),
  * which the decoder runs as a separate pass right after attention
@@ -644,6 +675,8 @@ typedef struct yvex_backend_rocm_attention_operations {
     int (*paged_decode_execute_fused)(yvex_backend *, const yvex_rocm_paged_decode_request *,
                                       const yvex_rocm_attention_epilogue *,
                                       yvex_backend_operation_facts *, yvex_error *);
+    int (*history_append_execute)(yvex_backend *, const yvex_rocm_history_append_request *,
+                                  yvex_backend_operation_facts *, yvex_error *);
 } yvex_backend_rocm_attention_operations;
 const yvex_backend_rocm_attention_operations *yvex_backend_rocm_attention_operations_get(
     const yvex_backend *backend);

@@ -1,0 +1,150 @@
+"""GPU parity: the token-major history writer (new K/V rows into the reference's [K | V]
+history layout, rotary on the keys) against the CPU restatement, bit for bit, through the C
+ABI; then a history in a reserved address range that is committed, appended to and decoded
+over step by step, the way the reference's caller grows it
+(src/runtime/stateful_attention.c:183-222, src/runtime/state_residency.c:258-287)."""
+import numpy as np
+import pytest
+
+from clori_amd import binding as B
+from clori_amd.backend import YvexError
+from gpu_common import ORACLE, assert_close_bf16, assert_lse, backend, bf16_normal  # noqa: F401
+
+pytestmark = pytest.mark.gpu
+
+
+def tables(rng, tokens, rotary_dim):
+    angles = rng.uniform(-3.0, 3.0, size=(tokens, max(rotary_dim, 16))).astype(np.float32)
+    return np.cos(angles).astype(np.float32), np.sin(angles).astype(np.float32)
+
+
+@pytest.mark.parametrize("tokens,first,hkv,d,rotary,interleaved", [
+    (1, 0, 8, 128, 128, True),        # the first token of a sequence
+    (1, 4095, 8, 128, 64, True),      # one decode step behind a long history
+    (37, 100, 8, 128, 64, True),      # a prompt chunk, partial rotary
+    (300, 7, 2, 128, 0, True),        # no rotary: plain rows
+    (19, 5, 4, 64, 32, True),         # other head widths
+    (6, 9, 2, 256, 256, False),       # separate packed K and V histories
+    (23, 0, 1, 128, 16, False),
+])
+def test_history_append_matches_oracle_bit_for_bit(backend, tokens, first, hkv, d, rotary, interleaved):
+    rng = np.random.default_rng(tokens * 1000 + first + d)
+    width = hkv * d
+    rows = first + tokens + 3                                   # three rows behind stay untouched
+    k_new, v_new = bf16_normal(rng, (tokens, hkv, d)), bf16_normal(rng, (tokens, hkv, d))
+    cosine, sine = tables(rng, tokens, rotary)
+    tk = backend.tensor("k-new", B.DTYPE_BF16, k_new.shape, k_new)
+    tv = backend.tensor("v-new", B.DTYPE_BF16, v_new.shape, v_new)
+    tc = backend.tensor("cos", B.DTYPE_F32, (tokens, max(rotary, 1)), cosine[:, :max(rotary, 1)])
+    ts = backend.tensor("sin", B.DTYPE_F32, (tokens, max(rotary, 1)), sine[:, :max(rotary, 1)])
+    want_k = ORACLE.rotary_half_bf16(k_new, cosine[:, :rotary], sine[:, :rotary], rotary) \
+        if rotary else k_new
+    used = first + tokens
+    if interleaved:
+        before = bf16_normal(rng, (rows, 2 * width))
+        store = backend.tensor("history", B.DTYPE_BF16, before.shape, before)
+        count = (used - 1) * 2 * width + width
+        kh, vh = store.view(0, B.DTYPE_BF16, (count,)), store.view(2 * width, B.DTYPE_BF16, (count,))
+        facts = backend.history_append_execute(
+            tk, tv, kh, vh, first, hkv, head_dimension=d, cosine=tc if rotary else None,
+            sine=ts if rotary else None, rotary_dimension=rotary, key_token_stride=2 * width,
+            value_token_stride=2 * width)
+        want = before.copy()
+        want[first:used, :width] = want_k.reshape(tokens, width)
+        want[first:used, width:] = v_new.reshape(tokens, width)
+        assert np.array_equal(store.read(), want)
+        stores = [store]
+    else:
+        before_k, before_v = bf16_normal(rng, (rows, width)), bf16_normal(rng, (rows, width))
+        sk = backend.tensor("k-history", B.DTYPE_BF16, before_k.shape, before_k)
+        sv = backend.tensor("v-history", B.DTYPE_BF16, before_v.shape, before_v)
+        kh, vh = sk.view(0, B.DTYPE_BF16, (used * width,)), sv.view(0, B.DTYPE_BF16, (used * width,))
+        facts = backend.history_append_execute(
+            tk, tv, kh, vh, first, hkv, head_dimension=d, cosine=tc if rotary else None,
+            sine=ts if rotary else None, rotary_dimension=rotary)
+        want_kh, want_vh = before_k.copy(), before_v.copy()
+        want_kh[first:used] = want_k.reshape(tokens, width)
+        want_vh[first:used] = v_new.reshape(tokens, width)
+        assert np.array_equal(sk.read(), want_kh) and np.array_equal(sv.read(), want_vh)
+        stores = [sk, sv]
+    assert facts.kernel_launches == 1 and facts.device_synchronizations == 1
+    for tensor in stores + [tk, tv, tc, ts]:
+        tensor.release()
+
+
+def test_history_append_refuses_values_that_are_not_finite(backend):
+    rng = np.random.default_rng(5)
+    hkv, d, tokens = 2, 128, 4
+    width = hkv * d
+    k_new, v_new = bf16_normal(rng, (tokens, hkv, d)), bf16_normal(rng, (tokens, hkv, d))
+    store = backend.tensor("history", B.DTYPE_BF16, (tokens, 2 * width))
+    count = (tokens - 1) * 2 * width + width
+    kh, vh = store.view(0, B.DTYPE_BF16, (count,)), store.view(2 * width, B.DTYPE_BF16, (count,))
+    for which in ("key", "value"):
+        bad_k, bad_v = k_new.copy(), v_new.copy()
+        (bad_k if which == "key" else bad_v)[2, 1, 77] = 0x7FC0
+        tk = backend.tensor("k", B.DTYPE_BF16, bad_k.shape, bad_k)
+        tv = backend.tensor("v", B.DTYPE_BF16, bad_v.shape, bad_v)
+        with pytest.raises(YvexError) as e:
+            backend.history_append_execute(tk, tv, kh, vh, 0, hkv, key_token_stride=2 * width,
+                                           value_token_stride=2 * width)
+        assert e.value.code == B.YVEX_ERR_FORMAT, which
+        tk.release()
+        tv.release()
+    store.release()
+
+
+def test_history_grows_in_a_reserved_range_append_then_decode(backend):
+    """Prompt, then single tokens: each step commits the rows it adds (usually nothing new:
+    a 2 MiB granule holds 512 rows here), appends them with the keys rotated, and decodes
+    the step's last token over everything so far.  Every decode must equal the oracle on the
+    rows the oracle rotated itself."""
+    hq, hkv, d, rotary, capacity = 32, 8, 128, 64, 16384
+    width = hkv * d
+    row_bytes = 2 * width * 2
+    rng = np.random.default_rng(99)
+    history = backend.reserve("history", B.DTYPE_BF16, (capacity, 2 * width))
+    k_all = np.empty((0, hkv, d), np.uint16)
+    v_all = np.empty((0, hkv, d), np.uint16)
+    have = 0
+    for step_tokens in (700, 1, 1, 330, 1, 2100, 1):
+        k_new, v_new = bf16_normal(rng, (step_tokens, hkv, d)), bf16_normal(rng, (step_tokens, hkv, d))
+        cosine, sine = tables(rng, step_tokens, rotary)
+        used = have + step_tokens
+        delta = history.commit(have * row_bytes, step_tokens * row_bytes)
+        assert delta % history.granularity == 0
+        assert history.resident_bytes == -(-used * row_bytes // history.granularity) * history.granularity
+        count = (used - 1) * 2 * width + width
+        kh = history.view(0, B.DTYPE_BF16, (count,))
+        vh = history.view(2 * width, B.DTYPE_BF16, (count,))
+        tk = backend.tensor("k-new", B.DTYPE_BF16, k_new.shape, k_new)
+        tv = backend.tensor("v-new", B.DTYPE_BF16, v_new.shape, v_new)
+        tc = backend.tensor("cos", B.DTYPE_F32, cosine[:, :rotary].shape, cosine[:, :rotary])
+        ts = backend.tensor("sin", B.DTYPE_F32, sine[:, :rotary].shape, sine[:, :rotary])
+        backend.history_append_execute(tk, tv, kh, vh, have, hkv, cosine=tc, sine=ts,
+                                       rotary_dimension=rotary, key_token_stride=2 * width,
+                                       value_token_stride=2 * width)
+        assert kh.is_written and vh.is_written                    # the views it wrote are usable as they are
+        k_all = np.concatenate([k_all, ORACLE.rotary_half_bf16(k_new, cosine[:, :rotary],
+                                                               sine[:, :rotary], rotary)])
+        v_all = np.concatenate([v_all, v_new])
+        have = used
+        q = bf16_normal(rng, (1, hq, d))
+        req = backend.attention_requirement(1, have, hq, hkv, d, causal=True, query_start=have - 1,
+                                            dtype=B.DTYPE_BF16,
+                                            contract=B.NUMERIC_BF16_F32_ACCUMULATE,
+                                            k_stride=2 * width, v_stride=2 * width)
+        tq = backend.tensor("q", B.DTYPE_BF16, q.shape, q)
+        out = backend.tensor("o", B.DTYPE_BF16, q.shape)
+        lse = backend.tensor("lse", B.DTYPE_F32, (1, hq))
+        backend.attention_execute(req, tq, kh, vh, out, lse=lse)
+        rc, ref, _, ref_lse = ORACLE.gqa_bf16(q, k_all, v_all, query_start=have - 1, causal=True)
+        assert rc == 0
+        assert_close_bf16(out.read(), ref, "history of %d rows" % have)
+        assert_lse(lse.read(), ref_lse, "history of %d rows" % have)
+        for tensor in (tk, tv, tc, ts, tq, out, lse):
+            tensor.release()
+    got = history.view(0, B.DTYPE_BF16, (have, 2 * width)).read()
+    assert np.array_equal(got[:, :width], k_all.reshape(have, width))
+    assert np.array_equal(got[:, width:], v_all.reshape(have, width))
+    history.release()

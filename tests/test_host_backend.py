@@ -701,6 +701,55 @@ def test_kv_append_admission():
         assert e.value.code == B.YVEX_ERR_FORMAT
 
 
+def test_history_append_admission():
+    """Refusal order of the token-major history writer: arguments, geometry, what the kernel
+    does not cover, then tensor views (uncommitted rows of a reserved range included)."""
+    with Backend() as b:
+        tokens, first, hkv, d = 5, 11, 4, 128
+        width = hkv * d
+        key = written(b, "k", B.DTYPE_BF16, (tokens, hkv, d))
+        value = written(b, "v", B.DTYPE_BF16, (tokens, hkv, d))
+        cosine, sine = written(b, "cos", B.DTYPE_F32, (tokens, 64)), written(b, "sin", B.DTYPE_F32, (tokens, 64))
+        store = b.tensor("history", B.DTYPE_BF16, (first + tokens, 2 * width))
+        count = (first + tokens - 1) * 2 * width + width
+        kh, vh = store.view(0, B.DTYPE_BF16, (count,)), store.view(2 * width, B.DTYPE_BF16, (count,))
+        args = (key, value, kh, vh, first, hkv)
+        strides = dict(key_token_stride=2 * width, value_token_stride=2 * width)
+        facts = b.history_append_execute(*args, cosine=cosine, sine=sine, rotary_dimension=64, **strides)
+        assert facts.kernel_launches == 1 and facts.device_synchronizations == 1
+        assert kh.is_written and vh.is_written
+        for kwargs, code in [(dict(head_dimension=0), B.YVEX_ERR_INVALID_ARG),
+                             (dict(rotary_dimension=64), B.YVEX_ERR_INVALID_ARG),         # no tables
+                             (dict(key_token_stride=width - 8), B.YVEX_ERR_INVALID_ARG),
+                             (dict(key_token_stride=2 * width + 4), B.YVEX_ERR_UNSUPPORTED),
+                             (dict(rotary_dimension=24, cosine=cosine, sine=sine), B.YVEX_ERR_UNSUPPORTED),
+                             (dict(rotary_dimension=256, cosine=cosine, sine=sine), B.YVEX_ERR_UNSUPPORTED),
+                             (dict(rotary_dimension=128, cosine=cosine, sine=sine), B.YVEX_ERR_FORMAT),
+                             (dict(key_token_stride=width), B.YVEX_ERR_FORMAT)]:           # view too long
+            merged = dict(strides)
+            merged.update(kwargs)
+            with pytest.raises(YvexError) as e:
+                b.history_append_execute(*args, **merged)
+            assert e.value.code == code, kwargs
+        with pytest.raises(YvexError) as e:                         # one row beyond the views
+            b.history_append_execute(key, value, kh, vh, first + 1, hkv, **strides)
+        assert e.value.code == B.YVEX_ERR_FORMAT
+        unwritten = b.tensor("k2", B.DTYPE_BF16, (tokens, hkv, d))
+        with pytest.raises(YvexError) as e:
+            b.history_append_execute(unwritten, value, kh, vh, first, hkv, **strides)
+        assert e.value.code == B.YVEX_ERR_FORMAT
+        # a history in a reserved range: the rows must be committed first
+        row_bytes = 2 * width * 2
+        reserved = b.reserve("reserved-history", B.DTYPE_BF16, (8192, 2 * width))
+        rk = reserved.view(0, B.DTYPE_BF16, (count,))
+        rv = reserved.view(2 * width, B.DTYPE_BF16, (count,))
+        with pytest.raises(YvexError) as e:
+            b.history_append_execute(key, value, rk, rv, first, hkv, **strides)
+        assert e.value.code == B.YVEX_ERR_STATE and "not committed" in e.value.message
+        reserved.commit(0, (first + tokens) * row_bytes)
+        assert b.history_append_execute(key, value, rk, rv, first, hkv, **strides).kernel_launches == 1
+
+
 def test_fused_gate_admission():
     """The epilogue entry points: an epilogue is required, the gate has the output geometry
     and is a written tensor other than the output, and only the BF16 contract takes one."""
