@@ -148,3 +148,71 @@ def test_history_grows_in_a_reserved_range_append_then_decode(backend):
     assert np.array_equal(got[:, :width], k_all.reshape(have, width))
     assert np.array_equal(got[:, width:], v_all.reshape(have, width))
     history.release()
+
+
+@pytest.mark.parametrize("seed", [21, 22])
+def test_history_append_random_sweep(backend, seed):
+    """Random geometry: head widths 64 to 256, partial and full rotary, packed, interleaved and
+    padded strides, ordinary tensors and reserved ranges committed for exactly the rows in
+    use.  Byte-exact, and nothing outside the new rows changes."""
+    rng = np.random.default_rng(seed)
+    for _ in range(40):
+        d = int(rng.choice([64, 128, 256]))
+        hkv = int(rng.choice([1, 2, 3, 8]))
+        rotary = int(rng.choice([0, 16, 32, d // 2, d]))
+        tokens = int(rng.choice([1, 1, rng.integers(2, 50), rng.integers(50, 700)]))
+        first = int(rng.choice([0, rng.integers(1, 40), rng.integers(40, 3000)]))
+        width = hkv * d
+        pad = int(rng.choice([0, 8, 64]))
+        interleaved = bool(rng.integers(0, 2))
+        stride = (2 * width if interleaved else width) + pad
+        used = first + tokens
+        rows = used + int(rng.integers(0, 3))
+        reserved = bool(rng.integers(0, 2))
+        k_new, v_new = bf16_normal(rng, (tokens, hkv, d)), bf16_normal(rng, (tokens, hkv, d))
+        cosine, sine = tables(rng, tokens, rotary)
+        want_k = ORACLE.rotary_half_bf16(k_new, cosine[:, :rotary], sine[:, :rotary], rotary) \
+            if rotary else k_new
+        held = []
+
+        def device(*args):
+            held.append(backend.tensor(*args))
+            return held[-1]
+
+        def history(name, before):
+            if not reserved:
+                return device(name, B.DTYPE_BF16, before.shape, before)
+            t = backend.reserve(name, B.DTYPE_BF16, (rows + 5000, stride))
+            held.append(t)
+            t.commit(0, before.nbytes)
+            t.view(0, B.DTYPE_BF16, before.shape).write(before)
+            return t
+        count = (used - 1) * stride + width
+        if interleaved:
+            before = bf16_normal(rng, (rows, stride))
+            store = history("history", before)
+            kh, vh = store.view(0, B.DTYPE_BF16, (count,)), store.view(2 * width, B.DTYPE_BF16, (count,))
+            want = before.copy()
+            want[first:used, :width] = want_k.reshape(tokens, width)
+            want[first:used, width:2 * width] = v_new.reshape(tokens, width)
+            checks = [(store, want)]
+        else:
+            before_k, before_v = bf16_normal(rng, (rows, stride)), bf16_normal(rng, (rows, stride))
+            sk, sv = history("k-history", before_k), history("v-history", before_v)
+            kh, vh = sk.view(0, B.DTYPE_BF16, (count,)), sv.view(0, B.DTYPE_BF16, (count,))
+            want_kh, want_vh = before_k.copy(), before_v.copy()
+            want_kh[first:used, :width] = want_k.reshape(tokens, width)
+            want_vh[first:used, :width] = v_new.reshape(tokens, width)
+            checks = [(sk, want_kh), (sv, want_vh)]
+        label = (seed, d, hkv, rotary, tokens, first, pad, interleaved, reserved)
+        backend.history_append_execute(
+            device("k-new", B.DTYPE_BF16, k_new.shape, k_new), device("v-new", B.DTYPE_BF16, v_new.shape, v_new),
+            kh, vh, first, hkv, head_dimension=d,
+            cosine=device("cos", B.DTYPE_F32, (tokens, rotary), cosine[:, :rotary]) if rotary else None,
+            sine=device("sin", B.DTYPE_F32, (tokens, rotary), sine[:, :rotary]) if rotary else None,
+            rotary_dimension=rotary, key_token_stride=stride, value_token_stride=stride)
+        for store, want in checks:
+            got = store.view(0, B.DTYPE_BF16, want.shape).read()
+            assert np.array_equal(got, want), label
+        for t in held:
+            t.release()
