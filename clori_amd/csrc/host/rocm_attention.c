@@ -1361,11 +1361,13 @@ static int rocm_history_append_execute(yvex_backend *backend,
                                        yvex_backend_operation_facts *facts, yvex_error *err)
 {
     static const char where[] = "rocm.history_append";
-    const yvex_backend_operation_variant variant = YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_BF16;
     yvex_rocm_backend_state *state = yvex_rocm_state(backend);
     const yvex_rocm_history_append_requirement *r;
+    yvex_backend_operation_variant variant;
     yvex_rocm_history_append_params hp;
+    yvex_dtype dtype;
     unsigned long long width, k_stride, v_stride, rows, new_elements, k_elements, v_elements, pieces;
+    unsigned long long piece; /* elements in 16 bytes */
     int rc;
     if (!request || !request->key || !request->value || !request->key_history ||
         !request->value_history || !facts)
@@ -1384,44 +1386,48 @@ static int rocm_history_append_execute(yvex_backend *backend,
     if (k_stride < width || v_stride < width)
         return refuse(err, YVEX_ERR_INVALID_ARG, where,
                       "a history token stride is narrower than one row of key/value heads");
-    if (r->head_dimension % 8ull || r->head_dimension > 256ull || (k_stride | v_stride) % 8ull ||
-        r->rotary_dimension > r->head_dimension || r->rotary_dimension % 16ull ||
+    dtype = request->key->dtype;
+    if (dtype != YVEX_DTYPE_BF16 && dtype != YVEX_DTYPE_F32)
+        return refuse(err, YVEX_ERR_UNSUPPORTED, where,
+                      "ROCm history append takes BF16 or F32 rows and histories of the same type");
+    piece = 16ull / yvex_dtype_element_bytes(dtype);
+    if (r->head_dimension % piece || r->head_dimension > 256ull || (k_stride | v_stride) % piece ||
+        r->rotary_dimension > r->head_dimension || r->rotary_dimension % (2ull * piece) ||
         r->tokens > 0x7fffffffull || r->key_value_heads > 65535ull)
         return refuse(err, YVEX_ERR_UNSUPPORTED, where,
-                      "ROCm history append requires a head dimension and token strides that are "
-                      "multiples of 8 (at most 256 lanes per head) and a rotary dimension that is a "
-                      "multiple of 16");
+                      "ROCm history append requires a head dimension (at most 256) and token strides "
+                      "that are multiples of 16 bytes and rotary halves that are too");
     memset(facts, 0, sizeof(*facts));
     if (!state || !yvex_core_u64_mul(r->tokens, width, &new_elements) ||
         !yvex_core_u64_mul(rows - 1ull, k_stride, &k_elements) ||
         !yvex_core_u64_add(k_elements, width, &k_elements) ||
         !yvex_core_u64_mul(rows - 1ull, v_stride, &v_elements) ||
         !yvex_core_u64_add(v_elements, width, &v_elements) ||
-        !yvex_core_u64_mul(r->tokens * r->key_value_heads, r->head_dimension / 8ull, &pieces) ||
+        !yvex_core_u64_mul(r->tokens * r->key_value_heads, r->head_dimension / piece, &pieces) ||
         (pieces + 255ull) / 256ull > 0x7fffffffull)
         return refuse(err, YVEX_ERR_BOUNDS, where, "history-append geometry exceeds admitted range");
     /* a history may be fresh or hold earlier tokens: written state is not required of it */
-    if (!view_ok(backend, request->key, YVEX_DTYPE_BF16, new_elements, 1) ||
-        !view_ok(backend, request->value, YVEX_DTYPE_BF16, new_elements, 1) ||
+    if (!view_ok(backend, request->key, dtype, new_elements, 1) ||
+        !view_ok(backend, request->value, dtype, new_elements, 1) ||
         (r->rotary_dimension &&
          (!view_ok(backend, request->cosine, YVEX_DTYPE_F32, r->tokens * r->rotary_dimension, 1) ||
           !view_ok(backend, request->sine, YVEX_DTYPE_F32, r->tokens * r->rotary_dimension, 1))) ||
-        !view_ok(backend, request->key_history, YVEX_DTYPE_BF16, k_elements, 0) ||
-        !view_ok(backend, request->value_history, YVEX_DTYPE_BF16, v_elements, 0))
+        !view_ok(backend, request->key_history, dtype, k_elements, 0) ||
+        !view_ok(backend, request->value_history, dtype, v_elements, 0))
         return view_refusal(backend, err, where,
                             "new rows, tables and history views must be tensors of this backend "
-                            "with the declared geometry");
+                            "with the declared geometry and one element type");
     if (((uintptr_t)request->key->data | (uintptr_t)request->value->data |
          (uintptr_t)request->key_history->data | (uintptr_t)request->value_history->data) & 15u)
         return refuse(err, YVEX_ERR_UNSUPPORTED, where,
                       "ROCm history append requires 16-byte aligned rows");
     memset(&hp, 0, sizeof(hp));
-    hp.key = (const uint16_t *)request->key->data;
-    hp.value = (const uint16_t *)request->value->data;
+    hp.key = request->key->data;
+    hp.value = request->value->data;
     hp.cosine = r->rotary_dimension ? (const float *)request->cosine->data : NULL;
     hp.sine = r->rotary_dimension ? (const float *)request->sine->data : NULL;
-    hp.key_history = (uint16_t *)request->key_history->data;
-    hp.value_history = (uint16_t *)request->value_history->data;
+    hp.key_history = request->key_history->data;
+    hp.value_history = request->value_history->data;
     hp.status = state->device_status;
     hp.first_row = r->first_row;
     hp.key_token_stride = k_stride;
@@ -1430,10 +1436,14 @@ static int rocm_history_append_execute(yvex_backend *backend,
     hp.kv_heads = (uint32_t)r->key_value_heads;
     hp.head_dim = (uint32_t)r->head_dimension;
     hp.rotary_dim = (uint32_t)r->rotary_dimension;
+    variant = dtype == YVEX_DTYPE_BF16 ? YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_BF16
+                                       : YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_F32;
     backend_workspace_reset(backend);
-    rc = yvex_rocm_launch(backend, YVEX_ROCM_FN_HISTORY_APPEND_BF16, variant,
-                          (unsigned int)((pieces + 255ull) / 256ull), 1u, 1u, 256u, 0u, &hp, where,
-                          err);
+    rc = yvex_rocm_launch(backend,
+                          dtype == YVEX_DTYPE_BF16 ? YVEX_ROCM_FN_HISTORY_APPEND_BF16
+                                                   : YVEX_ROCM_FN_HISTORY_APPEND_F32,
+                          variant, (unsigned int)((pieces + 255ull) / 256ull), 1u, 1u, 256u, 0u, &hp,
+                          where, err);
     if (rc == YVEX_OK) {
         facts->kernel_launches = 1ull;
         facts->compulsory_memory_facts_available = 1;

@@ -77,6 +77,8 @@ static const rocm_kernel_binding rocm_kernel_bindings[] = {
      YVEX_ROCM_FN_KV_APPEND_Q8_0},
     {"yvex_rocm_history_append_bf16", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_BF16,
      YVEX_ROCM_FN_HISTORY_APPEND_BF16},
+    {"yvex_rocm_history_append_f32", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_F32,
+     YVEX_ROCM_FN_HISTORY_APPEND_F32},
 };
 #define ROCM_KERNEL_BINDING_COUNT (sizeof(rocm_kernel_bindings) / sizeof(rocm_kernel_bindings[0]))
 

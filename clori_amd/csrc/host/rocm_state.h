@@ -34,6 +34,7 @@ typedef enum {
     YVEX_ROCM_FN_KV_APPEND_BF16,
     YVEX_ROCM_FN_KV_APPEND_Q8_0,
     YVEX_ROCM_FN_HISTORY_APPEND_BF16,
+    YVEX_ROCM_FN_HISTORY_APPEND_F32,
     YVEX_ROCM_FN_STREAM_READ,
     YVEX_ROCM_FN_GATHER_ROWS,
     YVEX_ROCM_FN_COUNT

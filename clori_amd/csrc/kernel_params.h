@@ -189,11 +189,12 @@ typedef struct {
 
 /* Token-major history writer: new key/value rows -> rows [first_row, first_row + tokens) of
  * the strided K and V histories the GQA kernels read, rotary on the keys.  One thread per
- * 16-byte piece of a row; grid = ceil(tokens * kv_heads * head_dim / 8 / 256), block = 256. */
+ * 16-byte piece of a row (8 bf16 or 4 F32 lanes); grid = ceil(pieces / 256), block = 256.
+ * The bf16 and the F32 kernel take the same block; pointers are to the element type. */
 typedef struct {
-    const uint16_t *key, *value;      /* bf16 [tokens][kv_heads][head_dim] */
+    const void *key, *value;          /* [tokens][kv_heads][head_dim] */
     const float *cosine, *sine;       /* F32 [tokens][rotary_dim]; unused when rotary_dim = 0 */
-    uint16_t *key_history, *value_history; /* row r of a history at r * its token stride */
+    void *key_history, *value_history; /* row r of a history at r * its token stride */
     int32_t *status;
     uint64_t first_row, key_token_stride, value_token_stride; /* strides in elements */
     uint32_t tokens, kv_heads, head_dim, rotary_dim;

@@ -415,17 +415,18 @@ yvex_rocm_history_append_bf16(const yvex_rocm_history_append_params p)
     const uint32_t token = (uint32_t)(id / pieces / p.kv_heads);
     const uint64_t in = ((uint64_t)token * p.kv_heads + head) * p.head_dim + c8 * 8u;
     const uint64_t row = p.first_row + token;
-    uint16_t *kdst = p.key_history + row * p.key_token_stride + (uint64_t)head * p.head_dim + c8 * 8u;
-    uint16_t *vdst = p.value_history + row * p.value_token_stride + (uint64_t)head * p.head_dim + c8 * 8u;
+    const uint16_t *key = (const uint16_t *)p.key, *value = (const uint16_t *)p.value;
+    uint16_t *kdst = (uint16_t *)p.key_history + row * p.key_token_stride + (uint64_t)head * p.head_dim + c8 * 8u;
+    uint16_t *vdst = (uint16_t *)p.value_history + row * p.value_token_stride + (uint64_t)head * p.head_dim + c8 * 8u;
     KeyChunk k;
     k.t = 0u;
     k.c8 = c8;
     k.role = c8 < pairs ? kLower : c8 < 2u * pairs ? kUpper : kPlain;
-    const u32x4 v = load_b128(p.value + in);
-    if (k.role != kUpper) k.own = load_b128(p.key + in);
+    const u32x4 v = load_b128(value + in);
+    if (k.role != kUpper) k.own = load_b128(key + in);
     if (k.role == kLower) {
         const uint64_t at = (uint64_t)token * p.rotary_dim + c8 * 8u;
-        k.other = load_b128(p.key + in + p.rotary_dim / 2u);
+        k.other = load_b128(key + in + p.rotary_dim / 2u);
         k.cs[0] = load_b128(p.cosine + at);
         k.cs[1] = load_b128(p.cosine + at + 4);
         k.sn[0] = load_b128(p.sine + at);
@@ -436,5 +437,83 @@ yvex_rocm_history_append_bf16(const yvex_rocm_history_append_params p)
     *reinterpret_cast<u32x4 *>(vdst) = v;
     if (k.role != kUpper) *reinterpret_cast<u32x4 *>(kdst) = lower;
     if (k.role == kLower) *reinterpret_cast<u32x4 *>(kdst + p.rotary_dim / 2u) = upper;
+    if (!ok) flag(p.status, YVEX_ROCM_DEVICE_NUMERIC);
+}
+
+namespace {
+
+// a * b and c * d rounded to bf16, as floats
+__device__ inline void rounded_products(float a, float b, float c, float d, float &ab, float &cd)
+{
+    const uint32_t w = pack_bf16x2(a * b, c * d);
+    ab = low_half(w);
+    cd = high_half(w);
+}
+
+__device__ inline bool finite_floats(const u32x4 &w)
+{
+    bool ok = true;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) ok &= (w[j] & 0x7f800000u) != 0x7f800000u;
+    return ok;
+}
+
+}  // namespace
+
+// The F32 form of the history writer, for the histories the reference itself keeps (F32 rows,
+// src/runtime/stateful_attention.c:183-222) and the EXACT_F32 kernels read.  Thread i owns the
+// 16-byte piece (token, kv head, lanes 4 * c4 .. 4 * c4 + 3).  The rotary arithmetic is
+// yvex_rotary_half_f32 (src/backend/cuda/transformer_kernels.cu:79-108): the F32 inputs enter
+// the products as they are, every product and sum is rounded to bf16 and stored as F32.
+extern "C" __global__ void __launch_bounds__(256)
+yvex_rocm_history_append_f32(const yvex_rocm_history_append_params p)
+{
+    const uint32_t pieces = p.head_dim / 4u, pairs = p.rotary_dim / 8u;
+    const uint64_t id = (uint64_t)blockIdx.x * 256u + threadIdx.x;
+    const uint64_t total = (uint64_t)p.tokens * p.kv_heads * pieces;
+    if (id >= total) return;
+    const uint32_t c4 = (uint32_t)(id % pieces), head = (uint32_t)(id / pieces % p.kv_heads);
+    const uint32_t token = (uint32_t)(id / pieces / p.kv_heads);
+    const uint64_t in = ((uint64_t)token * p.kv_heads + head) * p.head_dim + c4 * 4u;
+    const uint64_t row = p.first_row + token;
+    const float *key = (const float *)p.key, *value = (const float *)p.value;
+    float *kdst = (float *)p.key_history + row * p.key_token_stride + (uint64_t)head * p.head_dim + c4 * 4u;
+    float *vdst = (float *)p.value_history + row * p.value_token_stride + (uint64_t)head * p.head_dim + c4 * 4u;
+    const int role = c4 < pairs ? kLower : c4 < 2u * pairs ? kUpper : kPlain;
+    const u32x4 v = load_b128(value + in);
+    u32x4 own = {0u, 0u, 0u, 0u}, other = own, cs = own, sn = own;
+    if (role != kUpper) own = load_b128(key + in);
+    if (role == kLower) {
+        const uint64_t at = (uint64_t)token * p.rotary_dim + c4 * 4u;
+        other = load_b128(key + in + p.rotary_dim / 2u);
+        cs = load_b128(p.cosine + at);
+        sn = load_b128(p.sine + at);
+    }
+    bool ok = finite_floats(v);
+    *reinterpret_cast<u32x4 *>(vdst) = v;
+    if (role == kPlain) {
+        ok &= finite_floats(own);
+        *reinterpret_cast<u32x4 *>(kdst) = own;
+    } else if (role == kLower) {
+        u32x4 lower, upper;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            // the elements go through scalars first: a bit cast applied directly to a vector
+            // element reads element 0 whatever the index with this compiler
+            const uint32_t own_j = own[j], other_j = other[j], cs_j = cs[j], sn_j = sn[j];
+            const float first = __builtin_bit_cast(float, own_j), second = __builtin_bit_cast(float, other_j);
+            const float cosine = __builtin_bit_cast(float, cs_j), sine = __builtin_bit_cast(float, sn_j);
+            float fc, ss, sc, fs, lo, hi;
+            rounded_products(first, cosine, second, sine, fc, ss);
+            rounded_products(second, cosine, first, sine, sc, fs);
+            rounded_products(fc - ss, 1.0f, sc + fs, 1.0f, lo, hi);
+            lower[j] = __builtin_bit_cast(uint32_t, lo);
+            upper[j] = __builtin_bit_cast(uint32_t, hi);
+        }
+        // a non-finite input or table entry always leaves a non-finite result
+        ok &= finite_floats(lower) && finite_floats(upper);
+        *reinterpret_cast<u32x4 *>(kdst) = lower;
+        *reinterpret_cast<u32x4 *>(kdst + p.rotary_dim / 2u) = upper;
+    }
     if (!ok) flag(p.status, YVEX_ROCM_DEVICE_NUMERIC);
 }

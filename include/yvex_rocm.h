@@ -619,13 +619,16 @@ typedef struct yvex_rocm_kv_append_request {
  * (keys rotated: rotate-half over the first rotary_dimension lanes of every head,
  * src/backend/cuda/transformer_kernels.cu:79-108, every product and sum rounded to BF16),
  * nothing else is touched.  key_history / value_history are the views attention_execute is
- * handed afterwards for key_value_tokens = first_row + tokens: BF16,
+ * handed afterwards for key_value_tokens = first_row + tokens:
  * (first_row + tokens - 1) * stride + key_value_heads * head_dimension elements, strides in
  * elements (0 = packed); for the reference's interleaved rows both views lie in one tensor,
  * the value view key_value_heads * head_dimension elements behind the key view, stride twice
- * that.  Over a reserved address range the rows must be committed first.  head_dimension
- * and both strides must be multiples of 8, rotary_dimension a multiple of 16; non-finite
- * inputs, table entries or results are YVEX_ERR_FORMAT.
+ * that.  New rows and histories are all BF16 (the bf16 kernels' histories) or all F32 (the
+ * reference's own histories and the EXACT_F32 kernels'; the F32 inputs enter the rotary
+ * products as they are, as in yvex_rotary_half_f32, and the results are bf16 values stored
+ * as F32).  Over a reserved address range the rows must be committed first.  Rows, strides
+ * and rotary halves must be multiples of 16 bytes; non-finite inputs, table entries or
+ * results are YVEX_ERR_FORMAT.
  */
 typedef struct yvex_rocm_history_append_requirement {
     unsigned long long tokens, first_row;
@@ -635,9 +638,9 @@ typedef struct yvex_rocm_history_append_requirement {
 
 typedef struct yvex_rocm_history_append_request {
     yvex_rocm_history_append_requirement requirement;
-    const yvex_device_tensor *key, *value;   /* BF16 [tokens][kv_heads][d] */
+    const yvex_device_tensor *key, *value;   /* BF16 or F32 [tokens][kv_heads][d] */
     const yvex_device_tensor *cosine, *sine; /* F32 [tokens][rotary_dimension], or NULL without rotary */
-    yvex_device_tensor *key_history, *value_history;
+    yvex_device_tensor *key_history, *value_history; /* the element type of key and value */
 } yvex_rocm_history_append_request;
 
 /*

@@ -766,6 +766,34 @@ int yvo_rotary_half_bf16(uint16_t *values, const float *cosines, const float *si
     return 0;
 }
 
+/* src/backend/cuda/transformer_kernels.cu:79-108 on the F32 values the kernel itself takes:
+ * the inputs enter the products unrounded, every product and sum is rounded to bf16. */
+int yvo_rotary_half_f32(float *values, const float *cosines, const float *sines,
+                        uint64_t tokens, uint64_t heads, uint64_t head_dim,
+                        uint64_t rotary_dim)
+{
+    const uint64_t half = rotary_dim / 2u;
+    uint64_t vector, lane;
+    if (!values || !cosines || !sines || !tokens || !heads || !half || rotary_dim > head_dim)
+        return -1;
+    for (vector = 0; vector < tokens * heads; ++vector) {
+        const uint64_t token = vector / heads;
+        float *base = values + vector * head_dim;
+        for (lane = 0; lane < half; ++lane) {
+            const float cosine = cosines[token * rotary_dim + lane];
+            const float sine = sines[token * rotary_dim + lane];
+            const float first = base[lane], second = base[half + lane];
+            float first_product = yvo_bf16_decode(yvo_bf16_encode(first * cosine));
+            float second_product = yvo_bf16_decode(yvo_bf16_encode(second * sine));
+            base[lane] = yvo_bf16_decode(yvo_bf16_encode(first_product - second_product));
+            first_product = yvo_bf16_decode(yvo_bf16_encode(second * cosine));
+            second_product = yvo_bf16_decode(yvo_bf16_encode(first * sine));
+            base[half + lane] = yvo_bf16_decode(yvo_bf16_encode(first_product + second_product));
+        }
+    }
+    return 0;
+}
+
 /* src/backend/cuda/transformer_kernels.cu:353-364 */
 int yvo_sigmoid_gate_bf16(const float *values, const float *gate, uint64_t count, float *out)
 {

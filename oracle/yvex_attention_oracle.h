@@ -40,6 +40,9 @@
    yvo_rotary_half_bf16             pinned: known-answer case
  *       (tests/unit/cuda/quant_qtype.c:1988-2061), identity, quarter turn,
  *       float64 rotation within bf16 rounding
+ *   yvo_rotary_half_f32              pinned: the same known-answer case on its F32
+ *       literals, bit equality with yvo_rotary_half_bf16 on representable inputs,
+ *       identity and quarter turn on inputs that are not
  *   yvo_sigmoid_gate_bf16            pinned: known-answer case
  *       (tests/unit/cuda/quant_qtype.c:2979-2981,3019-3033), closed forms
  *   yvo_paged_*, the page tables and LSE output of yvo_mla_*, the selected
@@ -237,6 +240,15 @@ int yvo_reduce_output_finish(float *rows, uint64_t heads, uint64_t dim, uint64_t
 int yvo_rotary_half_bf16(uint16_t *values, const float *cosines, const float *sines,
                          uint64_t tokens, uint64_t heads, uint64_t head_dim,
                          uint64_t rotary_dim);
+/* The same kernel on the F32 values it takes in the reference (in place): the inputs enter
+ * the products as they are, products and sums are rounded to bf16 and stored as F32.
+ * Pinned by the reference's known-answer case on its own F32 literals
+ * (tests/unit/cuda/quant_qtype.c:1988-2061), by bit equality with yvo_rotary_half_bf16 on
+ * bf16-representable inputs, and on other inputs by the identity rotation (the result is
+ * the input rounded to bf16) and the quarter turn. */
+int yvo_rotary_half_f32(float *values, const float *cosines, const float *sines,
+                        uint64_t tokens, uint64_t heads, uint64_t head_dim,
+                        uint64_t rotary_dim);
 
 /*
  * Sigmoid output gate on attention rows: out = bf16(values * (1 / (1 + expf(-gate)))), all

@@ -216,3 +216,111 @@ def test_history_append_random_sweep(backend, seed):
             assert np.array_equal(got, want), label
         for t in held:
             t.release()
+
+
+@pytest.mark.parametrize("tokens,first,hkv,d,rotary,interleaved", [
+    (1, 0, 8, 128, 128, True), (1, 1000, 2, 128, 64, True), (45, 3, 4, 64, 32, True),
+    (200, 17, 2, 128, 0, True), (9, 2, 1, 256, 8, False), (33, 0, 3, 96, 48, False),
+])
+def test_history_append_f32_matches_oracle_bit_for_bit(backend, tokens, first, hkv, d, rotary, interleaved):
+    """The F32 form (the reference's own history element type).  The inputs are arbitrary
+    floats, not bf16-representable ones: they enter the products unrounded."""
+    rng = np.random.default_rng(tokens * 77 + first + d)
+    width = hkv * d
+    rows = first + tokens + 2
+    k_new = rng.standard_normal((tokens, hkv, d)).astype(np.float32)
+    v_new = rng.standard_normal((tokens, hkv, d)).astype(np.float32)
+    cosine, sine = tables(rng, tokens, rotary)
+    want_k = ORACLE.rotary_half_f32(k_new, cosine[:, :rotary], sine[:, :rotary], rotary) if rotary else k_new
+    held = [backend.tensor("k-new", B.DTYPE_F32, k_new.shape, k_new),
+            backend.tensor("v-new", B.DTYPE_F32, v_new.shape, v_new)]
+    tc = ts = None
+    if rotary:
+        tc = backend.tensor("cos", B.DTYPE_F32, (tokens, rotary), cosine[:, :rotary])
+        ts = backend.tensor("sin", B.DTYPE_F32, (tokens, rotary), sine[:, :rotary])
+        held += [tc, ts]
+    used = first + tokens
+    if interleaved:
+        before = rng.standard_normal((rows, 2 * width)).astype(np.float32)
+        store = backend.tensor("history", B.DTYPE_F32, before.shape, before)
+        count = (used - 1) * 2 * width + width
+        kh, vh = store.view(0, B.DTYPE_F32, (count,)), store.view(4 * width, B.DTYPE_F32, (count,))
+        strides = dict(key_token_stride=2 * width, value_token_stride=2 * width)
+        want = before.copy()
+        want[first:used, :width] = want_k.reshape(tokens, width)
+        want[first:used, width:] = v_new.reshape(tokens, width)
+        checks = [(store, want)]
+    else:
+        before_k = rng.standard_normal((rows, width)).astype(np.float32)
+        before_v = rng.standard_normal((rows, width)).astype(np.float32)
+        sk = backend.tensor("k-history", B.DTYPE_F32, before_k.shape, before_k)
+        sv = backend.tensor("v-history", B.DTYPE_F32, before_v.shape, before_v)
+        kh, vh = sk.view(0, B.DTYPE_F32, (used * width,)), sv.view(0, B.DTYPE_F32, (used * width,))
+        strides = {}
+        want_kh, want_vh = before_k.copy(), before_v.copy()
+        want_kh[first:used] = want_k.reshape(tokens, width)
+        want_vh[first:used] = v_new.reshape(tokens, width)
+        checks = [(sk, want_kh), (sv, want_vh)]
+    facts = backend.history_append_execute(held[0], held[1], kh, vh, first, hkv, head_dimension=d,
+                                           cosine=tc, sine=ts, rotary_dimension=rotary, **strides)
+    assert facts.kernel_launches == 1
+    for store, want in checks:
+        assert np.array_equal(store.read().view(np.uint32), want.view(np.uint32))
+        store.release()
+    for t in held:
+        t.release()
+    # a bf16 history does not take F32 rows
+    mixed = backend.tensor("bf16-history", B.DTYPE_BF16, (used, width))
+    k2 = backend.tensor("k-new", B.DTYPE_F32, k_new.shape, k_new)
+    with pytest.raises(YvexError) as e:
+        backend.history_append_execute(k2, k2, mixed.view(0, B.DTYPE_BF16, (used * width,)),
+                                       mixed.view(0, B.DTYPE_BF16, (used * width,)), first, hkv,
+                                       head_dimension=d)
+    assert e.value.code == B.YVEX_ERR_FORMAT
+    mixed.release()
+    k2.release()
+
+
+def test_f32_history_in_a_reserved_range_append_then_exact_decode(backend):
+    """The reference's own chain under its own contract: F32 [K | V] rows, rotary products
+    rounded to bf16, EXACT_F32 attention over the strided views."""
+    hq, hkv, d, rotary = 8, 2, 128, 128
+    width = hkv * d
+    row_bytes = 2 * width * 4
+    rng = np.random.default_rng(123)
+    history = backend.reserve("history", B.DTYPE_F32, (8192, 2 * width))
+    k_all = np.empty((0, hkv, d), np.float32)
+    v_all = np.empty((0, hkv, d), np.float32)
+    have = 0
+    for step_tokens in (300, 1, 1500, 1):
+        k_new = ORACLE.bf16_decode(bf16_normal(rng, (step_tokens, hkv, d)))
+        v_new = ORACLE.bf16_decode(bf16_normal(rng, (step_tokens, hkv, d)))
+        cosine, sine = tables(rng, step_tokens, rotary)
+        used = have + step_tokens
+        history.commit(have * row_bytes, step_tokens * row_bytes)
+        count = (used - 1) * 2 * width + width
+        kh = history.view(0, B.DTYPE_F32, (count,))
+        vh = history.view(4 * width, B.DTYPE_F32, (count,))
+        held = [backend.tensor("k-new", B.DTYPE_F32, k_new.shape, k_new),
+                backend.tensor("v-new", B.DTYPE_F32, v_new.shape, v_new),
+                backend.tensor("cos", B.DTYPE_F32, cosine.shape, cosine),
+                backend.tensor("sin", B.DTYPE_F32, sine.shape, sine)]
+        backend.history_append_execute(held[0], held[1], kh, vh, have, hkv, cosine=held[2], sine=held[3],
+                                       rotary_dimension=rotary, key_token_stride=2 * width,
+                                       value_token_stride=2 * width)
+        k_all = np.concatenate([k_all, ORACLE.rotary_half_f32(k_new, cosine, sine, rotary)])
+        v_all = np.concatenate([v_all, v_new])
+        have = used
+        q = ORACLE.bf16_decode(bf16_normal(rng, (1, hq, d)))
+        req = backend.attention_requirement(1, have, hq, hkv, d, causal=True, query_start=have - 1,
+                                            k_stride=2 * width, v_stride=2 * width)
+        tq = backend.tensor("q", B.DTYPE_F32, q.shape, q)
+        out = backend.tensor("o", B.DTYPE_F32, q.shape)
+        backend.attention_execute(req, tq, kh, vh, out)
+        rc, ref = ORACLE.gqa(q, k_all, v_all, query_start=have - 1)[:2]
+        assert rc == 0
+        err = np.abs(out.read() - ref).max()
+        assert err < 2e-6, (have, err)
+        for t in held + [tq, out]:
+            t.release()
+    history.release()

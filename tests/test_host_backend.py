@@ -738,6 +738,25 @@ def test_history_append_admission():
         with pytest.raises(YvexError) as e:
             b.history_append_execute(unwritten, value, kh, vh, first, hkv, **strides)
         assert e.value.code == B.YVEX_ERR_FORMAT
+        # F32 rows go into F32 histories (the reference's own element type), not into BF16 ones
+        key32 = written(b, "k32", B.DTYPE_F32, (tokens, hkv, d))
+        store32 = b.tensor("history32", B.DTYPE_F32, (first + tokens, 2 * width))
+        kh32 = store32.view(0, B.DTYPE_F32, (count,))
+        vh32 = store32.view(4 * width, B.DTYPE_F32, (count,))
+        assert b.history_append_execute(key32, key32, kh32, vh32, first, hkv, cosine=cosine, sine=sine,
+                                        rotary_dimension=64, **strides).kernel_launches == 1
+        for bad in ((key32, value, kh32, vh32), (key32, key32, kh, vh), (key, value, kh32, vh32)):
+            with pytest.raises(YvexError) as e:
+                b.history_append_execute(*bad, first, hkv, **strides)
+            assert e.value.code == B.YVEX_ERR_FORMAT
+        with pytest.raises(YvexError) as e:                         # rotary halves of 4 F32 lanes
+            b.history_append_execute(key32, key32, kh32, vh32, first, hkv, cosine=cosine, sine=sine,
+                                     rotary_dimension=12, **strides)
+        assert e.value.code == B.YVEX_ERR_UNSUPPORTED
+        ints = written(b, "ints", B.DTYPE_I32, (tokens, hkv, d))
+        with pytest.raises(YvexError) as e:
+            b.history_append_execute(ints, ints, kh32, vh32, first, hkv, **strides)
+        assert e.value.code == B.YVEX_ERR_UNSUPPORTED
         # a history in a reserved range: the rows must be committed first
         row_bytes = 2 * width * 2
         reserved = b.reserve("reserved-history", B.DTYPE_BF16, (8192, 2 * width))

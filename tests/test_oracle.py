@@ -519,6 +519,33 @@ def test_rotary_closed_forms():
         assert np.allclose(np.linalg.norm(got, axis=-1), np.linalg.norm(xf, axis=-1), rtol=5e-3)
 
 
+def test_rotary_f32_pins():
+    """The F32 form: the reference's known-answer case on its own literals
+    (tests/unit/cuda/quant_qtype.c:1988-2061), bit equality with the bf16 form where the
+    inputs are representable, and closed forms where they are not."""
+    values = np.array([[[-1.34375, -2.0625, 3.0, 4.0]]], np.float32)
+    cosines, sines = np.full((1, 2), 0.63671875, np.float32), np.full((1, 2), 0.546875, np.float32)
+    assert ORACLE.rotary_half_f32(values, cosines, sines, 2).tolist() == [[[0.26953125, -2.046875, 3.0, 4.0]]]
+    rng = np.random.default_rng(45)
+    tokens, heads, d = 4, 3, 64
+    x = rng.standard_normal((tokens, heads, d)).astype(np.float32)
+    xb = ORACLE.bf16_encode(x)
+    for rotary in (16, 32, 64):
+        half = rotary // 2
+        angles = rng.uniform(-3.0, 3.0, (tokens, rotary))
+        cosines, sines = np.cos(angles).astype(np.float32), np.sin(angles).astype(np.float32)
+        representable = ORACLE.bf16_decode(xb)
+        assert np.array_equal(ORACLE.rotary_half_f32(representable, cosines, sines, rotary),
+                              ORACLE.bf16_decode(ORACLE.rotary_half_bf16(xb, cosines, sines, rotary)))
+        one, zero = np.ones((tokens, rotary), np.float32), np.zeros((tokens, rotary), np.float32)
+        same = ORACLE.rotary_half_f32(x, one, zero, rotary)
+        assert np.array_equal(same[..., :rotary], representable[..., :rotary])   # rounded once
+        assert np.array_equal(same[..., rotary:], x[..., rotary:])               # suffix untouched
+        quarter = ORACLE.rotary_half_f32(x, zero, one, rotary)
+        assert np.array_equal(quarter[..., :half], -representable[..., half:rotary])
+        assert np.array_equal(quarter[..., half:rotary], representable[..., :half])
+
+
 # -------------------------------------------------------- output gate -------
 
 def test_sigmoid_gate_reference_known_answer():
