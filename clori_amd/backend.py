@@ -454,7 +454,7 @@ class Backend:
     def kv_append_execute(self, key, value, row_start, position_start, token_count, page_table,
                           k_pool, v_pool, kv_heads, pool_pages, max_tokens_per_session,
                           storage=B.KV_BF16, cosine=None, sine=None, rotary_dimension=0,
-                          head_dimension=128, page_tokens=16):
+                          head_dimension=128, page_tokens=16, rotary_mode=B.ROTARY_BF16_STAGED):
         """Writes the new rows into the paged pools; all arguments are device tensors."""
         ops = self.rocm_attention_operations()
         if ops is None:
@@ -465,7 +465,7 @@ class Backend:
         r.max_tokens_per_session = max_tokens_per_session
         r.key_value_heads, r.head_dimension, r.page_tokens = kv_heads, head_dimension, page_tokens
         r.pool_pages, r.page_table_stride = pool_pages, page_table.shape[1]
-        r.rotary_dimension, r.storage = rotary_dimension, storage
+        r.rotary_dimension, r.storage, r.rotary_mode = rotary_dimension, storage, rotary_mode
         request = B.KvAppendRequest(r, key.handle, value.handle,
                                     cosine.handle if cosine else None,
                                     sine.handle if sine else None, row_start.handle,
@@ -479,7 +479,8 @@ class Backend:
 
     def history_append_execute(self, key, value, key_history, value_history, first_row, kv_heads,
                                head_dimension=128, cosine=None, sine=None, rotary_dimension=0,
-                               key_token_stride=0, value_token_stride=0):
+                               key_token_stride=0, value_token_stride=0,
+                               rotary_mode=B.ROTARY_BF16_STAGED):
         """Writes the new rows (keys rotated) into rows first_row.. of the token-major K and V
         history views; all tensor arguments are device tensors."""
         ops = self.rocm_attention_operations()
@@ -490,6 +491,7 @@ class Backend:
         r.key_value_heads, r.head_dimension = kv_heads, head_dimension
         r.rotary_dimension = rotary_dimension
         r.key_token_stride, r.value_token_stride = key_token_stride, value_token_stride
+        r.rotary_mode = rotary_mode
         request = B.HistoryAppendRequest(r, key.handle, value.handle,
                                          cosine.handle if cosine else None,
                                          sine.handle if sine else None, key_history.handle,

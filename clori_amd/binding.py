@@ -55,6 +55,7 @@ LAYOUT_TOKEN_HEAD_DIM = 1
 MASK_FULL, MASK_CAUSAL = 1, 2
 NUMERIC_EXACT_F32, NUMERIC_BF16_F32_ACCUMULATE = 1, 2
 KV_BF16, KV_Q8_0 = 1, 2
+ROTARY_BF16_STAGED, ROTARY_F32_ROUNDED = 0, 1
 COMPLETION_IMMEDIATE, COMPLETION_DEFERRED = 0, 1
 
 ull = C.c_ulonglong
@@ -172,7 +173,7 @@ class KvAppendRequirement(C.Structure):
     _fields_ = [(n, ull) for n in ("sessions", "total_tokens", "max_tokens_per_session",
                                    "key_value_heads", "head_dimension", "page_tokens",
                                    "pool_pages", "page_table_stride", "rotary_dimension")] + [
-        ("storage", C.c_int)]
+        ("storage", C.c_int), ("rotary_mode", C.c_int)]
 
 
 class KvAppendRequest(C.Structure):
@@ -237,7 +238,8 @@ PAGED_EXECUTE_FUSED_FN = C.CFUNCTYPE(C.c_int, C.c_void_p, C.POINTER(PagedDecodeR
 
 class HistoryAppendRequirement(C.Structure):
     _fields_ = [(n, ull) for n in ("tokens", "first_row", "key_value_heads", "head_dimension",
-                                   "rotary_dimension", "key_token_stride", "value_token_stride")]
+                                   "rotary_dimension", "key_token_stride", "value_token_stride")] + [
+        ("rotary_mode", C.c_int)]
 
 
 class HistoryAppendRequest(C.Structure):

@@ -1282,6 +1282,7 @@ static int rocm_kv_append_execute(yvex_backend *backend, const yvex_rocm_kv_appe
         return refuse(err, YVEX_ERR_INVALID_ARG, where, "complete KV-append geometry is required");
     block_bytes = yvex_rocm_kv_page_block_bytes(r->storage, r->head_dimension, r->page_tokens);
     if (!block_bytes || r->rotary_dimension > r->head_dimension || r->rotary_dimension % 16ull ||
+        (r->rotary_mode != YVEX_ROCM_ROTARY_BF16_STAGED && r->rotary_mode != YVEX_ROCM_ROTARY_F32_ROUNDED) ||
         r->sessions > 65535ull || r->key_value_heads > 65535ull || r->pool_pages > 0x7fffffffull ||
         capacity > 0x7fffffffull || r->total_tokens > 0x7fffffffull)
         return refuse(err, YVEX_ERR_UNSUPPORTED, where,
@@ -1325,6 +1326,7 @@ static int rocm_kv_append_execute(yvex_backend *backend, const yvex_rocm_kv_appe
     kp.kv_heads = (uint32_t)r->key_value_heads;
     kp.head_dim = (uint32_t)r->head_dimension;
     kp.rotary_dim = (uint32_t)r->rotary_dimension;
+    kp.rotary_mode = (uint32_t)r->rotary_mode;
     kp.pool_pages = (uint32_t)r->pool_pages;
     kp.table_stride = (uint32_t)r->page_table_stride;
     /* a run of n tokens touches at most (n + page - 2) / page + 1 pages */
@@ -1392,6 +1394,7 @@ static int rocm_history_append_execute(yvex_backend *backend,
                       "ROCm history append takes BF16 or F32 rows and histories of the same type");
     piece = 16ull / yvex_dtype_element_bytes(dtype);
     if (r->head_dimension % piece || r->head_dimension > 256ull || (k_stride | v_stride) % piece ||
+        (r->rotary_mode != YVEX_ROCM_ROTARY_BF16_STAGED && r->rotary_mode != YVEX_ROCM_ROTARY_F32_ROUNDED) ||
         r->rotary_dimension > r->head_dimension || r->rotary_dimension % (2ull * piece) ||
         r->tokens > 0x7fffffffull || r->key_value_heads > 65535ull)
         return refuse(err, YVEX_ERR_UNSUPPORTED, where,
@@ -1436,6 +1439,7 @@ static int rocm_history_append_execute(yvex_backend *backend,
     hp.kv_heads = (uint32_t)r->key_value_heads;
     hp.head_dim = (uint32_t)r->head_dimension;
     hp.rotary_dim = (uint32_t)r->rotary_dimension;
+    hp.rotary_mode = (uint32_t)r->rotary_mode;
     variant = dtype == YVEX_DTYPE_BF16 ? YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_BF16
                                        : YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_F32;
     backend_workspace_reset(backend);

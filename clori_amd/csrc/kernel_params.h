@@ -185,6 +185,7 @@ typedef struct {
     uint64_t total_tokens;
     uint32_t sessions, kv_heads, head_dim, rotary_dim;
     uint32_t pool_pages, table_stride;
+    uint32_t rotary_mode;             /* 0: products staged through bf16; 1: F32 rotation, one rounding */
 } yvex_rocm_kv_append_params;
 
 /* Token-major history writer: new key/value rows -> rows [first_row, first_row + tokens) of
@@ -198,6 +199,7 @@ typedef struct {
     int32_t *status;
     uint64_t first_row, key_token_stride, value_token_stride; /* strides in elements */
     uint32_t tokens, kv_heads, head_dim, rotary_dim;
+    uint32_t rotary_mode;             /* as in yvex_rocm_kv_append_params */
 } yvex_rocm_history_append_params;
 
 #endif /* YVEX_ROCM_KERNEL_PARAMS_H */

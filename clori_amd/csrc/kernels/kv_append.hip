@@ -15,11 +15,17 @@
 // copied.  The lane of a lower chunk loads its partner chunk and one cos and one sin piece
 // and produces both rotated chunks; the lanes of upper chunks load and compute nothing.
 //
-// Rotary (src/backend/cuda/transformer_kernels.cu:79-108): with half = rotary_dim / 2 and
-// c < half, first = k[c], second = k[c + half], cosine/sine = table[row][c]:
+// Rotary, mode 0 (src/backend/cuda/transformer_kernels.cu:79-108): with half = rotary_dim / 2
+// and c < half, first = k[c], second = k[c + half], cosine/sine = table[row][c]:
 //     k[c]        = bf16(bf16(first * cosine)  - bf16(second * sine))
 //     k[c + half] = bf16(bf16(second * cosine) + bf16(first * sine))
 // every product and sum rounded to bf16 (round to nearest even), dims >= rotary_dim unchanged.
+// Mode 1 is the order of the reference's decoder (src/runtime/decoder.c:1112-1131): the plain
+// F32 rotation (transformer_kernels.cu:110-134) and then one bf16 rounding,
+//     k[c]        = bf16(fma(first, cosine, -(second * sine)))
+//     k[c + half] = bf16(fma(second, cosine, first * sine))
+// with the first product of each sum fused, as the compilers of both GPU targets contract
+// these expressions at their default flags.
 //
 // Q8_0 (src/gguf/quant_block.c:160-186): per 32 values scale = f16(max|x| / 127), codes =
 // clamp(roundf(x * (1 / f32(scale))), -127, 127), roundf half away from zero.
@@ -150,7 +156,7 @@ __device__ inline void key_issue(const yvex_rocm_kv_append_params &p, const Span
 
 // Rotated (or copied) chunk(s) as packed bf16; `upper` is produced by lower-half lanes only.
 // Returns false when a table entry, an input or a result is not finite.
-__device__ inline bool key_finish(const KeyChunk &k, u32x4 &lower, u32x4 &upper)
+__device__ inline bool key_finish(const KeyChunk &k, u32x4 &lower, u32x4 &upper, bool plain)
 {
     if (k.role == kUpper) return true;
     if (k.role == kPlain) {
@@ -169,6 +175,13 @@ __device__ inline bool key_finish(const KeyChunk &k, u32x4 &lower, u32x4 &upper)
         const uint32_t s0 = k.sn[j >> 1][(2 * j) & 3], s1 = k.sn[j >> 1][(2 * j + 1) & 3];
         const float cosine0 = __builtin_bit_cast(float, c0), cosine1 = __builtin_bit_cast(float, c1);
         const float sine0 = __builtin_bit_cast(float, s0), sine1 = __builtin_bit_cast(float, s1);
+        if (plain) {
+            lower[j] = pack_bf16x2(__builtin_fmaf(first0, cosine0, -(second0 * sine0)),
+                                   __builtin_fmaf(first1, cosine1, -(second1 * sine1)));
+            upper[j] = pack_bf16x2(__builtin_fmaf(second0, cosine0, first0 * sine0),
+                                   __builtin_fmaf(second1, cosine1, first1 * sine1));
+            continue;
+        }
         const uint32_t fc = pack_bf16x2(first0 * cosine0, first1 * cosine1);
         const uint32_t ss = pack_bf16x2(second0 * sine0, second1 * sine1);
         const uint32_t sc = pack_bf16x2(second0 * cosine0, second1 * cosine1);
@@ -216,7 +229,7 @@ yvex_rocm_kv_append_bf16(const yvex_rocm_kv_append_params p)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             u32x4 lower, upper;
-            ok &= key_finish(k[i], lower, upper);
+            ok &= key_finish(k[i], lower, upper, p.rotary_mode != 0u);
             if (k[i].t < s.lo || k[i].t >= s.hi) continue;
             if (k[i].role != kUpper)
                 *reinterpret_cast<u32x4 *>(kdst + (k[i].c8 * 16u + k[i].t) * 8u) = lower;
@@ -329,7 +342,7 @@ yvex_rocm_kv_append_q8_0(const yvex_rocm_kv_append_params p)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             u32x4 lower, upper;
-            ok &= key_finish(k[i], lower, upper) || k[i].t < s.lo || k[i].t >= s.hi;
+            ok &= key_finish(k[i], lower, upper, p.rotary_mode != 0u) || k[i].t < s.lo || k[i].t >= s.hi;
             if (k[i].role != kUpper)
                 *reinterpret_cast<u32x4 *>(&k_rows[k[i].t][k[i].c8 * 8u]) = lower;
             if (k[i].role == kLower)
@@ -403,7 +416,8 @@ yvex_rocm_kv_append_q8_0(const yvex_rocm_kv_append_params p)
 // (src/runtime/stateful_attention.c:183-222) after a separate rotary pass over the keys
 // (src/runtime/decoder.c:1236-1242).  Here one launch does both: thread i owns the 16-byte
 // piece (token, kv head, dims 8 * c8 .. 8 * c8 + 7) of the value row and of the key row, with
-// the rotary roles of the page writer (a lower-half piece produces its upper-half partner).
+// the rotary roles and modes of the page writer (a lower-half piece produces its upper-half
+// partner).
 extern "C" __global__ void __launch_bounds__(256)
 yvex_rocm_history_append_bf16(const yvex_rocm_history_append_params p)
 {
@@ -433,7 +447,7 @@ yvex_rocm_history_append_bf16(const yvex_rocm_history_append_params p)
         k.sn[1] = load_b128(p.sine + at + 4);
     }
     u32x4 lower, upper;
-    bool ok = key_finish(k, lower, upper) && finite_bits(v);
+    bool ok = key_finish(k, lower, upper, p.rotary_mode != 0u) && finite_bits(v);
     *reinterpret_cast<u32x4 *>(vdst) = v;
     if (k.role != kUpper) *reinterpret_cast<u32x4 *>(kdst) = lower;
     if (k.role == kLower) *reinterpret_cast<u32x4 *>(kdst + p.rotary_dim / 2u) = upper;
@@ -464,7 +478,9 @@ __device__ inline bool finite_floats(const u32x4 &w)
 // src/runtime/stateful_attention.c:183-222) and the EXACT_F32 kernels read.  Thread i owns the
 // 16-byte piece (token, kv head, lanes 4 * c4 .. 4 * c4 + 3).  The rotary arithmetic is
 // yvex_rotary_half_f32 (src/backend/cuda/transformer_kernels.cu:79-108): the F32 inputs enter
-// the products as they are, every product and sum is rounded to bf16 and stored as F32.
+// the products as they are, every product and sum is rounded to bf16 and stored as F32.  In
+// mode 1 (the decoder's order) the rotation is plain F32 and every key lane, the ones behind
+// the rotary lanes included, is rounded to bf16 once; values are copied in both modes.
 extern "C" __global__ void __launch_bounds__(256)
 yvex_rocm_history_append_f32(const yvex_rocm_history_append_params p)
 {
@@ -493,6 +509,16 @@ yvex_rocm_history_append_f32(const yvex_rocm_history_append_params p)
     *reinterpret_cast<u32x4 *>(vdst) = v;
     if (role == kPlain) {
         ok &= finite_floats(own);
+        if (p.rotary_mode != 0u) {
+            // the rounding pass of the decoder's order covers the lanes behind the rotary ones too
+#pragma unroll
+            for (int j = 0; j < 4; j += 2) {
+                const uint32_t a = own[j], b = own[j + 1];
+                const uint32_t w = pack_bf16x2(__builtin_bit_cast(float, a), __builtin_bit_cast(float, b));
+                own[j] = w << 16;
+                own[j + 1] = w & 0xffff0000u;
+            }
+        }
         *reinterpret_cast<u32x4 *>(kdst) = own;
     } else if (role == kLower) {
         u32x4 lower, upper;
@@ -504,9 +530,14 @@ yvex_rocm_history_append_f32(const yvex_rocm_history_append_params p)
             const float first = __builtin_bit_cast(float, own_j), second = __builtin_bit_cast(float, other_j);
             const float cosine = __builtin_bit_cast(float, cs_j), sine = __builtin_bit_cast(float, sn_j);
             float fc, ss, sc, fs, lo, hi;
-            rounded_products(first, cosine, second, sine, fc, ss);
-            rounded_products(second, cosine, first, sine, sc, fs);
-            rounded_products(fc - ss, 1.0f, sc + fs, 1.0f, lo, hi);
+            if (p.rotary_mode != 0u) {
+                rounded_products(__builtin_fmaf(first, cosine, -(second * sine)), 1.0f,
+                                 __builtin_fmaf(second, cosine, first * sine), 1.0f, lo, hi);
+            } else {
+                rounded_products(first, cosine, second, sine, fc, ss);
+                rounded_products(second, cosine, first, sine, sc, fs);
+                rounded_products(fc - ss, 1.0f, sc + fs, 1.0f, lo, hi);
+            }
             lower[j] = __builtin_bit_cast(uint32_t, lo);
             upper[j] = __builtin_bit_cast(uint32_t, hi);
         }

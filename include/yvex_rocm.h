@@ -593,11 +593,25 @@ typedef struct yvex_rocm_mla_decode_request {
  * same page in one launch race on it and the result is undefined (nothing is flagged).  Pages
  * shared between sessions (a common prefix) are fine as long as no session of the call
  * writes to them. */
+/* How the keys are rotated on their way into a pool or a history.  The reference has both
+ * orders: BF16_STAGED is its bf16 rotary kernel, every product and sum rounded to bf16
+ * (yvex_rotary_half_f32, src/backend/cuda/transformer_kernels.cu:79-108; the joint transformer
+ * and the text encoder, src/backend/cuda/joint_transformer.c:606-618, text_encoder.c:600-609);
+ * F32_ROUNDED is what its decoder runs in front of attention (decoder_rotary,
+ * src/runtime/decoder.c:1112-1131,1236-1242): the plain F32 rotation
+ * (yvex_rotary_half_plain_f32, transformer_kernels.cu:110-134) and then one bf16 rounding of
+ * every lane of the tensor (decoder_round, src/backend/cuda/kernels.cu:40-58). */
+typedef enum {
+    YVEX_ROCM_ROTARY_BF16_STAGED = 0,
+    YVEX_ROCM_ROTARY_F32_ROUNDED = 1
+} yvex_rocm_rotary_mode;
+
 typedef struct yvex_rocm_kv_append_requirement {
     unsigned long long sessions, total_tokens, max_tokens_per_session;
     unsigned long long key_value_heads, head_dimension, page_tokens, pool_pages, page_table_stride;
     unsigned long long rotary_dimension;
     yvex_rocm_kv_storage storage;
+    yvex_rocm_rotary_mode rotary_mode;
 } yvex_rocm_kv_append_requirement;
 
 typedef struct yvex_rocm_kv_append_request {
@@ -634,6 +648,7 @@ typedef struct yvex_rocm_history_append_requirement {
     unsigned long long tokens, first_row;
     unsigned long long key_value_heads, head_dimension, rotary_dimension;
     unsigned long long key_token_stride, value_token_stride;
+    yvex_rocm_rotary_mode rotary_mode; /* F32_ROUNDED also rounds the key lanes behind the rotary ones */
 } yvex_rocm_history_append_requirement;
 
 typedef struct yvex_rocm_history_append_request {

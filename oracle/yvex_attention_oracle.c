@@ -794,6 +794,38 @@ int yvo_rotary_half_f32(float *values, const float *cosines, const float *sines,
     return 0;
 }
 
+/* The decoder's own order (src/runtime/decoder.c:1112-1131): the plain F32 rotation
+ * (yvex_rotary_half_plain_f32, src/backend/cuda/transformer_kernels.cu:110-134) followed by
+ * the bf16 rounding of the whole tensor (decoder_round -> yvex_attention_bf16_round,
+ * src/backend/cuda/kernels.cu:40-58), suffix lanes included.  The two float expressions
+ * first * cosine - second * sine and second * cosine + first * sine are evaluated with the
+ * contraction LLVM's combiner applies on both GPU targets at default flags: the first
+ * product fused into the sum, the second rounded to float on its own. */
+int yvo_rotary_half_f32_rounded(float *values, const float *cosines, const float *sines,
+                                uint64_t tokens, uint64_t heads, uint64_t head_dim,
+                                uint64_t rotary_dim)
+{
+    const uint64_t half = rotary_dim / 2u;
+    uint64_t vector, lane;
+    if (!values || !cosines || !sines || !tokens || !heads || !half || rotary_dim > head_dim)
+        return -1;
+    for (vector = 0; vector < tokens * heads; ++vector) {
+        const uint64_t token = vector / heads;
+        float *base = values + vector * head_dim;
+        for (lane = 0; lane < half; ++lane) {
+            const float cosine = cosines[token * rotary_dim + lane];
+            const float sine = sines[token * rotary_dim + lane];
+            const float first = base[lane], second = base[half + lane];
+            const float second_sine = second * sine, first_sine = first * sine;
+            base[lane] = fmaf(first, cosine, -second_sine);
+            base[half + lane] = fmaf(second, cosine, first_sine);
+        }
+        for (lane = 0; lane < head_dim; ++lane)
+            base[lane] = yvo_bf16_decode(yvo_bf16_encode(base[lane]));
+    }
+    return 0;
+}
+
 /* src/backend/cuda/transformer_kernels.cu:353-364 */
 int yvo_sigmoid_gate_bf16(const float *values, const float *gate, uint64_t count, float *out)
 {

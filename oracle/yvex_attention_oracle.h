@@ -43,6 +43,10 @@
  *   yvo_rotary_half_f32              pinned: the same known-answer case on its F32
  *       literals, bit equality with yvo_rotary_half_bf16 on representable inputs,
  *       identity and quarter turn on inputs that are not
+ *   yvo_rotary_half_f32_rounded      pinned: known-answer case of the plain rotation
+ *       (tests/unit/cuda/quant_qtype.c:3050-3105), identity, quarter turn, float64
+ *       rotation within one bf16 rounding; the choice of fused product is
+ *       parity unpinned (results within a float rounding of a bf16 tie)
  *   yvo_sigmoid_gate_bf16            pinned: known-answer case
  *       (tests/unit/cuda/quant_qtype.c:2979-2981,3019-3033), closed forms
  *   yvo_paged_*, the page tables and LSE output of yvo_mla_*, the selected
@@ -249,6 +253,18 @@ int yvo_rotary_half_bf16(uint16_t *values, const float *cosines, const float *si
 int yvo_rotary_half_f32(float *values, const float *cosines, const float *sines,
                         uint64_t tokens, uint64_t heads, uint64_t head_dim,
                         uint64_t rotary_dim);
+/* The order the reference's decoder runs in front of attention
+ * (src/runtime/decoder.c:1112-1131, 1236-1242): the plain F32 rotation
+ * (src/backend/cuda/transformer_kernels.cu:110-134) and then one bf16 rounding of every lane
+ * of the tensor (src/backend/cuda/kernels.cu:40-58).  Pinned by the reference's
+ * known-answer case for the plain rotation (tests/unit/cuda/quant_qtype.c:3050-3105, exact
+ * in float), the identity and the quarter turn, a float64 rotation within one bf16
+ * rounding, and agreement with the staged form within one bf16 step.  Which of the two
+ * products of each sum the reference's compiler fuses is not visible in its sources: the
+ * last bit of a result that lies within a float rounding of a bf16 tie is parity unpinned. */
+int yvo_rotary_half_f32_rounded(float *values, const float *cosines, const float *sines,
+                                uint64_t tokens, uint64_t heads, uint64_t head_dim,
+                                uint64_t rotary_dim);
 
 /*
  * Sigmoid output gate on attention rows: out = bf16(values * (1 / (1 + expf(-gate)))), all

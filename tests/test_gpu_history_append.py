@@ -324,3 +324,50 @@ def test_f32_history_in_a_reserved_range_append_then_exact_decode(backend):
         for t in held + [tq, out]:
             t.release()
     history.release()
+
+
+
+@pytest.mark.parametrize("f32", [False, True], ids=["bf16", "f32"])
+@pytest.mark.parametrize("d,rotary", [(128, 64), (64, 64), (256, 32)])
+def test_history_append_in_the_decoder_order_of_rotary(backend, f32, d, rotary):
+    """Mode F32_ROUNDED: plain F32 rotation then one bf16 rounding (the decoder's order,
+    src/runtime/decoder.c:1112-1131).  In F32 the key lanes behind the rotary ones are rounded
+    too, as decoder_round rounds the whole tensor; values are copied as they are."""
+    rng = np.random.default_rng(d + rotary + int(f32))
+    tokens, first, hkv = 29, 6, 3
+    width = hkv * d
+    used = first + tokens
+    cosine, sine = tables(rng, tokens, rotary)
+    if f32:
+        k_new = rng.standard_normal((tokens, hkv, d)).astype(np.float32)
+        v_new = rng.standard_normal((tokens, hkv, d)).astype(np.float32)
+        want_k = ORACLE.rotary_half_f32_rounded(k_new, cosine[:, :rotary], sine[:, :rotary], rotary)
+        dtype, before = B.DTYPE_F32, rng.standard_normal((used, 2 * width)).astype(np.float32)
+        offset = 4 * width
+    else:
+        k_new, v_new = bf16_normal(rng, (tokens, hkv, d)), bf16_normal(rng, (tokens, hkv, d))
+        want_k = ORACLE.bf16_encode(ORACLE.rotary_half_f32_rounded(
+            ORACLE.bf16_decode(k_new), cosine[:, :rotary], sine[:, :rotary], rotary))
+        dtype, before = B.DTYPE_BF16, bf16_normal(rng, (used, 2 * width))
+        offset = 2 * width
+    held = [backend.tensor("k-new", dtype, k_new.shape, k_new), backend.tensor("v-new", dtype, v_new.shape, v_new),
+            backend.tensor("cos", B.DTYPE_F32, (tokens, rotary), cosine[:, :rotary]),
+            backend.tensor("sin", B.DTYPE_F32, (tokens, rotary), sine[:, :rotary]),
+            backend.tensor("history", dtype, before.shape, before)]
+    count = (used - 1) * 2 * width + width
+    kh, vh = held[4].view(0, dtype, (count,)), held[4].view(offset, dtype, (count,))
+    backend.history_append_execute(held[0], held[1], kh, vh, first, hkv, head_dimension=d, cosine=held[2],
+                                   sine=held[3], rotary_dimension=rotary, key_token_stride=2 * width,
+                                   value_token_stride=2 * width, rotary_mode=B.ROTARY_F32_ROUNDED)
+    want = before.copy()
+    want[first:, :width] = want_k.reshape(tokens, width)
+    want[first:, width:] = v_new.reshape(tokens, width)
+    got = held[4].read()
+    assert np.array_equal(got.view(np.uint32 if f32 else np.uint16), want.view(np.uint32 if f32 else np.uint16))
+    with pytest.raises(YvexError) as e:
+        backend.history_append_execute(held[0], held[1], kh, vh, first, hkv, head_dimension=d,
+                                       key_token_stride=2 * width, value_token_stride=2 * width,
+                                       rotary_mode=7)
+    assert e.value.code == B.YVEX_ERR_UNSUPPORTED
+    for t in held:
+        t.release()

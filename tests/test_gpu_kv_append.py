@@ -26,7 +26,8 @@ def expected_rows(canonical, k_new, v_new, table, starts, counts, row_starts, q8
     return k_rows, v_rows
 
 
-def run_case(backend, rng, starts, counts, storage, rotary_dim, pool_state="zero"):
+def run_case(backend, rng, starts, counts, storage, rotary_dim, pool_state="zero",
+             rotary_mode=B.ROTARY_BF16_STAGED):
     sessions = len(starts)
     q8 = storage == B.KV_Q8_0
     stride = max((s + c + PAGE - 1) // PAGE for s, c in zip(starts, counts)) + 1
@@ -67,12 +68,18 @@ def run_case(backend, rng, starts, counts, storage, rotary_dim, pool_state="zero
         t["key"], t["value"], t["row_start"], t["position_start"], t["token_count"],
         t["page_table"], t["k_pool"], t["v_pool"], HKV, pool_pages, max(max(counts), 1),
         storage=storage, cosine=t["cosine"] if use_rotary else None,
-        sine=t["sine"] if use_rotary else None, rotary_dimension=rotary_dim)
+        sine=t["sine"] if use_rotary else None, rotary_dimension=rotary_dim,
+        rotary_mode=rotary_mode)
     assert facts.kernel_launches == 1
     got_k = kv_unpack_pages(t["k_pool"].read(np.uint8, (-1,)), storage, False, pool_pages, HKV)
     got_v = kv_unpack_pages(t["v_pool"].read(np.uint8, (-1,)), storage, True, pool_pages, HKV)
-    k_rot = ORACLE.rotary_half_bf16(k_new, cosine[:, :rotary_dim], sine[:, :rotary_dim], rotary_dim) \
-        if use_rotary else k_new
+    if use_rotary and rotary_mode == B.ROTARY_F32_ROUNDED:
+        k_rot = ORACLE.bf16_encode(ORACLE.rotary_half_f32_rounded(
+            ORACLE.bf16_decode(k_new), cosine[:, :rotary_dim], sine[:, :rotary_dim], rotary_dim))
+    elif use_rotary:
+        k_rot = ORACLE.rotary_half_bf16(k_new, cosine[:, :rotary_dim], sine[:, :rotary_dim], rotary_dim)
+    else:
+        k_rot = k_new
     want_k, want_v = expected_rows((k_rows.copy(), v_rows.copy()), k_rot, v_new, table, starts,
                                    counts, row_starts, q8)
     return t, (got_k, got_v), (want_k, want_v), table, pool_pages
@@ -91,6 +98,36 @@ def test_append_writes_exactly_the_host_layout(backend, storage, rotary_dim):
     assert np.array_equal(got[1].reshape(want[1].shape), want[1])
     for x in t.values():
         x.release()
+
+
+@pytest.mark.parametrize("storage", [B.KV_BF16, B.KV_Q8_0], ids=["bf16", "q8_0"])
+@pytest.mark.parametrize("rotary_dim", [32, 128])
+def test_append_in_the_decoder_order_of_rotary(backend, storage, rotary_dim):
+    """The same appends with the rotation the reference's decoder runs in front of attention
+    (src/runtime/decoder.c:1112-1131): plain F32 rotation, one bf16 rounding.  Byte-exact
+    against that restatement, and different from the staged order somewhere."""
+    rng = np.random.default_rng(31 + rotary_dim)
+    starts, counts = [3, 0, 50, 16], [44, 1, 0, 130]
+    t, got, want, _, _ = run_case(backend, rng, starts, counts, storage, rotary_dim, "filled",
+                                  rotary_mode=B.ROTARY_F32_ROUNDED)
+    assert np.array_equal(got[0].reshape(want[0].shape), want[0])
+    assert np.array_equal(got[1].reshape(want[1].shape), want[1])
+    for x in t.values():
+        x.release()
+    if storage == B.KV_BF16:
+        rng = np.random.default_rng(31 + rotary_dim)
+        t2, staged, _, _, _ = run_case(backend, rng, starts, counts, storage, rotary_dim, "filled")
+        differing = np.count_nonzero(staged[0].reshape(want[0].shape) != want[0])
+        # the orders differ by roundings only, but in a good part of the rotated values
+        assert 0 < differing < want[0].size // 2
+        apart = np.abs(ORACLE.bf16_decode(staged[0].reshape(want[0].shape)).astype(np.float64) -
+                       ORACLE.bf16_decode(want[0]).astype(np.float64))
+        assert apart.max() <= 2.0 ** -5
+        for x in t2.values():
+            x.release()
+    with pytest.raises(YvexError) as e:
+        run_case(backend, np.random.default_rng(1), [0], [1], storage, rotary_dim, rotary_mode=2)
+    assert e.value.code == B.YVEX_ERR_UNSUPPORTED
 
 
 def test_decode_over_appended_pages_matches_cpu_operator(backend):

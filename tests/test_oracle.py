@@ -546,6 +546,42 @@ def test_rotary_f32_pins():
         assert np.array_equal(quarter[..., half:rotary], representable[..., :half])
 
 
+def test_rotary_rounded_pins():
+    """The decoder's order: plain F32 rotation, then one bf16 rounding of every lane.  The
+    reference's known-answer case (tests/unit/cuda/quant_qtype.c:3050-3105: two heads of
+    width 2, cos 0.75, sin 0.5) is exact in float and in bf16."""
+    values = np.array([[[1.0, 2.0], [7.0, 8.0]]], np.float32)
+    cosines, sines = np.full((1, 2), 0.75, np.float32), np.full((1, 2), 0.5, np.float32)
+    assert ORACLE.rotary_half_f32_rounded(values, cosines, sines, 2).tolist() == \
+        [[[-0.25, 2.0], [1.25, 9.5]]]
+    rng = np.random.default_rng(46)
+    tokens, heads, d = 6, 2, 64
+    x = rng.standard_normal((tokens, heads, d)).astype(np.float32)
+    rounded = ORACLE.bf16_decode(ORACLE.bf16_encode(x))
+    for rotary in (16, 32, 64):
+        half = rotary // 2
+        one, zero = np.ones((tokens, rotary), np.float32), np.zeros((tokens, rotary), np.float32)
+        assert np.array_equal(ORACLE.rotary_half_f32_rounded(x, one, zero, rotary), rounded)
+        quarter = ORACLE.rotary_half_f32_rounded(x, zero, one, rotary)
+        assert np.array_equal(quarter[..., :half], -rounded[..., half:rotary])
+        assert np.array_equal(quarter[..., half:rotary], rounded[..., :half])
+        assert np.array_equal(quarter[..., rotary:], rounded[..., rotary:])       # suffix rounded too
+        angles = rng.uniform(-3.0, 3.0, (tokens, rotary))
+        cosines, sines = np.cos(angles).astype(np.float32), np.sin(angles).astype(np.float32)
+        got = ORACLE.rotary_half_f32_rounded(x, cosines, sines, rotary)
+        c = cosines[:, None, :half].astype(np.float64)
+        s = sines[:, None, :half].astype(np.float64)
+        a, b = x[..., :half].astype(np.float64), x[..., half:rotary].astype(np.float64)
+        exact = np.concatenate([a * c - b * s, b * c + a * s, x[..., rotary:]], axis=-1)
+        # one rounding to bf16 of a value that carries at most a float rounding or two
+        step = 2.0 ** (np.floor(np.log2(np.maximum(np.abs(exact), 1e-30))) - 7)
+        assert np.all(np.abs(got - exact) <= 0.5 * step * (1 + 2.0 ** -14) + 1e-12)
+        assert np.array_equal(ORACLE.bf16_decode(ORACLE.bf16_encode(got)), got)
+        # the staged form rounds three times: the two agree within a few bf16 steps of the inputs
+        staged = ORACLE.rotary_half_f32(x, cosines, sines, rotary)
+        assert np.max(np.abs(staged - got)[..., :rotary]) <= 3 * 2.0 ** -8 * np.max(np.abs(x))
+
+
 # -------------------------------------------------------- output gate -------
 
 def test_sigmoid_gate_reference_known_answer():
