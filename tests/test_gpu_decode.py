@@ -280,3 +280,39 @@ def test_config4_shape_sample(backend):
     assert rc == 0
     assert_close_bf16(got, ref, "config4")
     assert_lse(lse, ref_lse, "config4")
+
+
+# ------------------------------------------------------------ long contexts ----
+
+@pytest.mark.parametrize("contexts,q8", [([150000], False), ([90000, 3, 40000], False),
+                                          ([120000], True)])
+def test_paged_decode_long_contexts(backend, contexts, q8):
+    """Contexts far beyond the benchmark's: one (session, kv head) segment is split over
+    hundreds of waves, so the second kernel merges its partials over many load trips, and a
+    three-token session sits between two long ones."""
+    rng = np.random.default_rng(len(contexts) * 1000 + int(q8))
+    make = make_q8_case if q8 else make_paged_case
+    q, k_rows, v_rows, table, ctx, pool_pages = make(rng, contexts, 32, 8)
+    storage = B.KV_Q8_0 if q8 else B.KV_BF16
+    got, lse, facts = run_paged(backend, q, k_rows, v_rows, table, ctx, 8, pool_pages, storage=storage)
+    rc, ref, _, ref_lse = ORACLE.paged_decode(q, k_rows, v_rows, table, ctx, 8, 16, q8=q8)
+    assert rc == 0
+    assert_close_bf16(got, ref, "long paged %s" % contexts)
+    assert_lse(lse, ref_lse, "long paged %s" % contexts)
+    assert facts.kernel_launches == 2
+    again, lse_again, _ = run_paged(backend, q, k_rows, v_rows, table, ctx, 8, pool_pages, storage=storage)
+    assert np.array_equal(got, again) and np.array_equal(lse, lse_again)
+
+
+def test_rows_decode_long_context(backend):
+    rng = np.random.default_rng(150)
+    ctx = 150000
+    q = bf16_normal(rng, (1, 32, 128))
+    k = bf16_normal(rng, (ctx, 8, 128))
+    v = bf16_normal(rng, (ctx, 8, 128))
+    got, lse, facts = run_rows_decode(backend, q, k, v, query_start=ctx - 1)
+    rc, ref, _, ref_lse = ORACLE.gqa_bf16(q, k, v, query_start=ctx - 1, causal=True)
+    assert rc == 0
+    assert_close_bf16(got, ref, "long rows")
+    assert_lse(lse, ref_lse, "long rows")
+    assert facts.kernel_launches == 1

@@ -363,3 +363,15 @@ def test_reduce_geometry_against_the_reference_reduce(backend):
                         sinks=sinks, window=window, compressed=(cpool, ctable, visible), rope=rope)
     want = golden[name + "/out"]
     assert_close_bf16(got, want[None], "reference reduce, committed output")
+
+
+def test_mla_decode_long_context(backend):
+    """A context twelve times the benchmark's next to a seven-token one: hundreds of chunks
+    for one batch element in the merge, one for the other."""
+    rng = np.random.default_rng(55)
+    q, pool, table, ctx = make_case(rng, [100000, 7])
+    got, lse, _ = run_mla(backend, q, pool, table, ctx)
+    rc, ref, _, ref_lse = ORACLE.mla_decode(q, pool, table, ctx, VALUE_DIM, PAGE)
+    assert rc == 0
+    assert_close_bf16(got, ref, "mla long")
+    assert_lse(lse, ref_lse, "mla long")

@@ -117,3 +117,17 @@ def test_prefill_refusals(backend):
                                   backend.tensor("k", B.DTYPE_BF16, k.shape, k),
                                   backend.tensor("v", B.DTYPE_BF16, k.shape, k), out)
     assert e.value.code == B.YVEX_ERR_FORMAT and not out.is_written
+
+
+@pytest.mark.parametrize("tq,tk,start,hq,hkv", [(4100, 4100, 0, 4, 1), (700, 9000, 8300, 4, 2)])
+def test_prefill_long_sequences(backend, tq, tk, start, hq, hkv):
+    """Twice the benchmark's sequence length, and a prompt chunk behind a long history."""
+    rng = np.random.default_rng(tq + tk)
+    q = bf16_normal(rng, (tq, hq, 128))
+    k = bf16_normal(rng, (tk, hkv, 128))
+    v = bf16_normal(rng, (tk, hkv, 128))
+    got, lse, _ = run_prefill(backend, q, k, v, query_start=start, causal=True)
+    rc, ref, _, ref_lse = ORACLE.gqa_bf16(q, k, v, query_start=start, causal=True)
+    assert rc == 0
+    assert_close_bf16(got, ref, "long prefill %d/%d" % (tq, tk))
+    assert_lse(lse, ref_lse, "long prefill %d/%d" % (tq, tk))
