@@ -316,3 +316,19 @@ def test_rows_decode_long_context(backend):
     assert_close_bf16(got, ref, "long rows")
     assert_lse(lse, ref_lse, "long rows")
     assert facts.kernel_launches == 1
+
+
+@pytest.mark.parametrize("q8", [False, True], ids=["bf16", "q8_0"])
+def test_paged_decode_many_short_sessions(backend, q8):
+    """Three thousand sessions of 1 to 100 tokens: more (session, kv head) segments than waves,
+    several whole segments per wave."""
+    rng = np.random.default_rng(3000 + int(q8))
+    contexts = [int(c) for c in rng.integers(1, 101, size=3000)]
+    make = make_q8_case if q8 else make_paged_case
+    q, k_rows, v_rows, table, ctx, pool_pages = make(rng, contexts, 8, 2)
+    got, lse, _ = run_paged(backend, q, k_rows, v_rows, table, ctx, 2, pool_pages,
+                            storage=B.KV_Q8_0 if q8 else B.KV_BF16)
+    rc, ref, _, ref_lse = ORACLE.paged_decode(q, k_rows, v_rows, table, ctx, 2, 16, q8=q8)
+    assert rc == 0
+    assert_close_bf16(got, ref, "many sessions")
+    assert_lse(lse, ref_lse, "many sessions")

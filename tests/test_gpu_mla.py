@@ -375,3 +375,14 @@ def test_mla_decode_long_context(backend):
     assert rc == 0
     assert_close_bf16(got, ref, "mla long")
     assert_lse(lse, ref_lse, "mla long")
+
+
+def test_mla_decode_many_short_contexts(backend):
+    rng = np.random.default_rng(56)
+    contexts = [int(c) for c in rng.integers(1, 200, size=150)]
+    q, pool, table, ctx = make_case(rng, contexts)
+    got, lse, _ = run_mla(backend, q, pool, table, ctx)
+    rc, ref, _, ref_lse = ORACLE.mla_decode(q, pool, table, ctx, VALUE_DIM, PAGE)
+    assert rc == 0
+    assert_close_bf16(got, ref, "mla many")
+    assert_lse(lse, ref_lse, "mla many")
