@@ -14,7 +14,8 @@ already resident in HBM.  Workloads are the five configurations the metric is qu
 
 By name only (not configurations of the metric): exact2 and exact1 (configurations 2 and 1
 under the EXACT_F32 contract: fp32 matrix cores, and double-precision split decode),
-append_bf16 / append_q8_0 (the KV page writer), history_append (the token-major writer), copy.
+append_bf16 / append_q8_0 (the KV page writer), history_append (the token-major writer), paged3_p64 / paged4_p64
+(configurations 3 and 4 with pages of 64 tokens), copy.
 
 Prints ONE JSON line.  `value` is the headline workload's throughput; every workload
 that ran is listed under "workloads" with its own roofline figures.  Timing uses HIP
@@ -145,8 +146,8 @@ def decode_kernels(kernel, facts):
     return [kernel, "yvex_rocm_decode_finish"]
 
 
-def workload_paged(backend, rng, steps, warmup, q8=False):
-    sessions, hq, hkv, d, page = 32, 32, 8, 128, 16
+def workload_paged(backend, rng, steps, warmup, q8=False, page=16):
+    sessions, hq, hkv, d = 32, 32, 8, 128
     lo, hi = (4096, 32768) if q8 else (512, 16384)
     contexts = rng.integers(lo, hi + 1, size=sessions).astype(np.int32)
     if os.environ.get("YVEX_BENCH_UNIFORM_CONTEXT"):   # tuning aid: equal-length sessions
@@ -161,15 +162,16 @@ def workload_paged(backend, rng, steps, warmup, q8=False):
         table[s, :need[s]] = perm[at:at + need[s]]
         at += int(need[s])
     storage = B.KV_Q8_0 if q8 else B.KV_BF16
-    block = 2176 if q8 else 4096
-    pool_bytes = pool_pages * hkv * block
+    block = 2176 if q8 else 4096             # one 16-token block; a page is page // 16 of them
+    blocks = pool_pages * hkv * (page // 16)
+    pool_bytes = blocks * block
     if q8:
         # int8 codes in [-127,127] and f16 scales near 1/40: any bytes are valid Q8_0 as long
         # as scales are finite and non-negative; layout = codes then scales per block
-        pool = np.empty((pool_pages * hkv, block), dtype=np.uint8)
+        pool = np.empty((blocks, block), dtype=np.uint8)
         codes = rng.integers(-127, 128, size=(1 << 22), dtype=np.int8).view(np.uint8)
-        reps = (pool_pages * hkv * 2048 + codes.size - 1) // codes.size
-        pool[:, :2048] = np.tile(codes, reps)[:pool_pages * hkv * 2048].reshape(-1, 2048)
+        reps = (blocks * 2048 + codes.size - 1) // codes.size
+        pool[:, :2048] = np.tile(codes, reps)[:blocks * 2048].reshape(-1, 2048)
         pool[:, 2048:] = np.tile(np.array([0.025], np.float16).view(np.uint8), 64)[None, :]
         k_pool = backend.tensor("k-pages", B.DTYPE_I8, (pool_bytes,), pool)
         v_pool = backend.tensor("v-pages", B.DTYPE_I8, (pool_bytes,), pool[::-1].copy())
@@ -199,10 +201,10 @@ def workload_paged(backend, rng, steps, warmup, q8=False):
     algo = tokens * per_token + int(need.sum()) * 4 + sessions * 4 + 2 * sessions * hq * d * 2 + \
         sessions * hq * 4
     assert np.all(np.isfinite(lse.read()))
-    return dict(name="paged4" if q8 else "paged3",
+    return dict(name=("paged4" if q8 else "paged3") + ("" if page == 16 else "_p%d" % page),
                 workload="paged %s GQA decode: 32 sessions, 32/8 heads, d=128, contexts U[%d,%d], "
-                         "16-token pages, seeded permutation page tables" %
-                         ("Q8_0" if q8 else "bf16", lo, hi),
+                         "%d-token pages, seeded permutation page tables" %
+                         ("Q8_0" if q8 else "bf16", lo, hi, page),
                 bound="hbm", algorithmic_bytes=algo, tokens=tokens,
                 launches=int(facts.kernel_launches), kernels=kernels, **timed)
 
@@ -436,11 +438,13 @@ EXTRA_WORKLOADS = {
     "append_bf16": lambda b, r, s, w: workload_append(b, r, s, w, q8=False),
     "append_q8_0": lambda b, r, s, w: workload_append(b, r, s, w, q8=True),
     "history_append": workload_history_append,
+    "paged3_p64": lambda b, r, s, w: workload_paged(b, r, s, w, q8=False, page=64),
+    "paged4_p64": lambda b, r, s, w: workload_paged(b, r, s, w, q8=True, page=64),
     "exact2": workload_exact2,
     "exact1": workload_exact1,
 }
 SEEDS = {"decode1": 1, "prefill2": 2, "paged3": 3, "paged4": 4, "mla5": 5, "append_bf16": 6,
-         "append_q8_0": 7, "exact2": 8, "exact1": 9, "history_append": 10}
+         "append_q8_0": 7, "exact2": 8, "exact1": 9, "history_append": 10, "paged3_p64": 3, "paged4_p64": 4}
 
 
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")

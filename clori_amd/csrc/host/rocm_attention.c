@@ -172,6 +172,7 @@ typedef struct {
     const void *gate;
     unsigned long long sessions, query_heads, kv_heads, head_dim;
     unsigned long long pool_pages, table_stride, max_context, fixed_context;
+    unsigned int page_shift; /* paged pools: a page is 16 << page_shift tokens */
     unsigned long long k_token_stride, v_token_stride;
     float scale;
     /* when set, the partials live here (nothing is acquired or released) */
@@ -236,6 +237,7 @@ static int decode_run(yvex_backend *backend, const decode_job *job, const char *
     dp.kv_heads = (uint32_t)job->kv_heads;
     dp.head_dim = (uint32_t)job->head_dim;
     dp.pool_pages = (uint32_t)job->pool_pages;
+    dp.page_shift = job->page_shift;
     dp.table_stride = (uint32_t)job->table_stride;
     dp.min_tiles = ROCM_DECODE_MIN_TILES;
     dp.fixed_context = (uint32_t)job->fixed_context;
@@ -732,13 +734,14 @@ static int paged_validate(const yvex_rocm_paged_decode_requirement *r, const cha
         !yvex_core_u64_mul(r->page_table_stride, r->page_tokens, &capacity) ||
         r->max_context_tokens > capacity)
         return refuse(err, YVEX_ERR_INVALID_ARG, where, "complete paged-decode geometry is required");
-    if (r->head_dimension != ROCM_MFMA_HEAD_DIM || r->page_tokens != ROCM_PAGE_TOKENS ||
+    if (r->head_dimension != ROCM_MFMA_HEAD_DIM ||
+        (r->page_tokens != ROCM_PAGE_TOKENS && r->page_tokens != 4ull * ROCM_PAGE_TOKENS) ||
         r->query_heads / r->key_value_heads > ROCM_GROUP_MAX ||
         (r->kv_storage != YVEX_ROCM_KV_BF16 && r->kv_storage != YVEX_ROCM_KV_Q8_0) ||
         r->numeric_contract != YVEX_TRANSFORMER_ATTENTION_NUMERIC_BF16_F32_ACCUMULATE ||
         !r->deterministic || r->pool_pages > 0x7fffffffull || capacity > 0x7fffffffull)
         return refuse(err, YVEX_ERR_UNSUPPORTED, where,
-                      "ROCm paged decode requires head dimension 128, 16-token pages, a query "
+                      "ROCm paged decode requires head dimension 128, pages of 16 or 64 tokens, a query "
                       "group of at most 16 and the deterministic bf16/fp32-accumulate contract");
     yvex_error_clear(err);
     return YVEX_OK;
@@ -829,6 +832,7 @@ static int paged_decode_execute_common(yvex_backend *backend,
     job.kv_heads = r->key_value_heads;
     job.head_dim = r->head_dimension;
     job.pool_pages = r->pool_pages;
+    job.page_shift = r->page_tokens == ROCM_PAGE_TOKENS ? 0u : 2u;
     job.table_stride = r->page_table_stride;
     job.max_context = r->max_context_tokens;
     job.scale = 1.0f / sqrtf((float)r->head_dimension);
@@ -1286,7 +1290,7 @@ static int rocm_kv_append_execute(yvex_backend *backend, const yvex_rocm_kv_appe
         r->sessions > 65535ull || r->key_value_heads > 65535ull || r->pool_pages > 0x7fffffffull ||
         capacity > 0x7fffffffull || r->total_tokens > 0x7fffffffull)
         return refuse(err, YVEX_ERR_UNSUPPORTED, where,
-                      "ROCm KV append requires head dimension 128, 16-token pages, BF16 or Q8_0 "
+                      "ROCm KV append requires head dimension 128, pages of 16 or 64 tokens, BF16 or Q8_0 "
                       "storage and a rotary dimension that is a multiple of 16");
     memset(facts, 0, sizeof(*facts));
     pool_dtype = r->storage == YVEX_ROCM_KV_BF16 ? YVEX_DTYPE_BF16 : YVEX_DTYPE_I8;
@@ -1327,10 +1331,12 @@ static int rocm_kv_append_execute(yvex_backend *backend, const yvex_rocm_kv_appe
     kp.head_dim = (uint32_t)r->head_dimension;
     kp.rotary_dim = (uint32_t)r->rotary_dimension;
     kp.rotary_mode = (uint32_t)r->rotary_mode;
+    kp.page_shift = r->page_tokens == ROCM_PAGE_TOKENS ? 0u : 2u;
     kp.pool_pages = (uint32_t)r->pool_pages;
     kp.table_stride = (uint32_t)r->page_table_stride;
-    /* a run of n tokens touches at most (n + page - 2) / page + 1 pages */
-    page_slots = (r->max_tokens_per_session + r->page_tokens - 2ull) / r->page_tokens + 1ull;
+    /* one workgroup row per 16-token block: a run of n tokens touches at most
+     * (n + 16 - 2) / 16 + 1 of them, whatever the page size */
+    page_slots = (r->max_tokens_per_session + ROCM_PAGE_TOKENS - 2ull) / ROCM_PAGE_TOKENS + 1ull;
     if (page_slots > 0x7fffffffull)
         return refuse(err, YVEX_ERR_BOUNDS, where, "KV-append geometry exceeds admitted range");
     variant = r->storage == YVEX_ROCM_KV_BF16 ? YVEX_BACKEND_VARIANT_ROCM_ATTENTION_PAGED_BF16

@@ -85,7 +85,8 @@ typedef struct {
     uint64_t k_token_stride, v_token_stride; /* token-major layout: elements per token */
     uint32_t sessions, query_heads, kv_heads, head_dim;
     uint32_t pool_pages, table_stride, min_tiles, fixed_context;
-    uint32_t waves, reserved;
+    uint32_t waves;
+    uint32_t page_shift; /* a page is 16 << page_shift tokens: that many consecutive 16-token blocks */
     float scale_log2; /* softmax scale * log2(e) */
     float reserved_f;
     const uint16_t *gate; /* optional bf16 [sessions][query_heads][head_dim] sigmoid output gate */
@@ -186,6 +187,7 @@ typedef struct {
     uint32_t sessions, kv_heads, head_dim, rotary_dim;
     uint32_t pool_pages, table_stride;
     uint32_t rotary_mode;             /* 0: products staged through bf16; 1: F32 rotation, one rounding */
+    uint32_t page_shift;              /* a page is 16 << page_shift tokens: consecutive 16-token blocks */
 } yvex_rocm_kv_append_params;
 
 /* Token-major history writer: new key/value rows -> rows [first_row, first_row + tokens) of

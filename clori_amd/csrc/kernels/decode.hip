@@ -351,7 +351,8 @@ struct Decoder {
     __device__ Decoder(const yvex_rocm_decode_params &params, unsigned char *transpose_area)
         : p(params), vt(transpose_area), lane(threadIdx.x & 63), n(threadIdx.x & 15), g((threadIdx.x & 63) >> 4),
           group(params.query_heads / params.kv_heads),
-          limit(PAGED ? params.table_stride * (uint32_t)kPageTokens : params.fixed_context)
+          limit(PAGED ? params.table_stride * ((uint32_t)kPageTokens << params.page_shift)
+                      : params.fixed_context)
     {
     }
 
@@ -403,11 +404,15 @@ struct Decoder {
         int32_t my_page = 0, my_page_hi = 0;
         const unsigned char *kbase = (const unsigned char *)p.k_pool;
         const unsigned char *vbase = (const unsigned char *)p.v_pool;
+        // a page holds 1 << shift tiles; tile i of this call is block (sub0 + i) of the pages
+        // from the one that holds tile `first` on
+        const uint32_t shift = PAGED ? p.page_shift : 0u, sub0 = first & ((1u << shift) - 1u);
         if (PAGED) {
             // two coalesced reads bring the page ids of these tiles into the wave
-            const int32_t *table = p.page_table + (uint64_t)session * p.table_stride + first;
-            if ((uint32_t)lane < count) my_page = table[lane];
-            if ((uint32_t)lane + 64u < count) my_page_hi = table[lane + 64];
+            const uint32_t pages = (sub0 + count + (1u << shift) - 1u) >> shift;
+            const int32_t *table = p.page_table + (uint64_t)session * p.table_stride + (first >> shift);
+            if ((uint32_t)lane < pages) my_page = table[lane];
+            if ((uint32_t)lane + 64u < pages) my_page_hi = table[lane + 64];
             if (my_page < 0 || (uint32_t)my_page >= p.pool_pages || my_page_hi < 0 ||
                 (uint32_t)my_page_hi >= p.pool_pages) {
                 flag(p.status, YVEX_ROCM_DEVICE_CONTRACT);
@@ -420,10 +425,12 @@ struct Decoder {
         }
         auto fetch = [&](Tile &t, uint32_t i) {
             if (PAGED) {
-                const uint32_t page = (uint32_t)(i < 64u
-                                                     ? __builtin_amdgcn_readlane(my_page, (int)i)
-                                                     : __builtin_amdgcn_readlane(my_page_hi, (int)(i - 64u)));
-                const uint64_t off = ((uint64_t)page * p.kv_heads + kv_head) * Kv::kBlockBytes;
+                const uint32_t at = sub0 + i, slot = at >> shift;
+                const uint32_t page = (uint32_t)(slot < 64u
+                                                     ? __builtin_amdgcn_readlane(my_page, (int)slot)
+                                                     : __builtin_amdgcn_readlane(my_page_hi, (int)(slot - 64u)));
+                const uint64_t off = ((((uint64_t)page * p.kv_heads + kv_head) << shift) +
+                                      (at & ((1u << shift) - 1u))) * Kv::kBlockBytes;
                 Kv::load_paged(t, kbase + off, vbase + off, lane);
             } else {
                 const uint32_t row = t0 + i * kPageTokens;

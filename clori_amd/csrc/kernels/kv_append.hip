@@ -70,6 +70,7 @@ __device__ inline bool finite_bits(const u32x4 &w)
 
 struct Span {
     uint32_t page_id;   // pool page
+    uint32_t sub;       // 16-token block of the page
     uint32_t lo, hi;    // token slots [lo, hi) of the page that are new
     uint32_t row;       // input row of slot lo
     bool valid;
@@ -81,6 +82,7 @@ __device__ inline Span locate(const yvex_rocm_kv_append_params &p)
     Span s;
     s.valid = false;
     s.page_id = 0u;
+    s.sub = 0u;
     s.lo = 0u;
     s.hi = 1u;
     s.row = 0u;
@@ -89,7 +91,7 @@ __device__ inline Span locate(const yvex_rocm_kv_append_params &p)
     const int32_t row0 = p.row_start[session];
     if (count <= 0) return s;
     if (start < 0 || row0 < 0 || (uint64_t)row0 + (uint32_t)count > p.total_tokens ||
-        (uint64_t)start + (uint32_t)count > (uint64_t)p.table_stride * kPageTokens) {
+        (uint64_t)start + (uint32_t)count > ((uint64_t)p.table_stride * kPageTokens) << p.page_shift) {
         if (slot == 0u && blockIdx.y == 0u && threadIdx.x == 0) flag(p.status, YVEX_ROCM_DEVICE_CONTRACT);
         return s;
     }
@@ -103,7 +105,8 @@ __device__ inline Span locate(const yvex_rocm_kv_append_params &p)
     }
     const uint32_t page = first_page + slot;
     if (page > last_page) return s;
-    const int32_t id = p.page_table[(uint64_t)session * p.table_stride + page];
+    // `page` counts 16-token blocks; a pool page holds 1 << page_shift of them
+    const int32_t id = p.page_table[(uint64_t)session * p.table_stride + (page >> p.page_shift)];
     if (id < 0 || (uint32_t)id >= p.pool_pages) {
         if (threadIdx.x == 0) flag(p.status, YVEX_ROCM_DEVICE_CONTRACT);
         return s;
@@ -111,6 +114,7 @@ __device__ inline Span locate(const yvex_rocm_kv_append_params &p)
     const uint32_t begin = max((uint32_t)start, page * kPageTokens);
     const uint32_t end = min((uint32_t)start + (uint32_t)count, (page + 1u) * kPageTokens);
     s.page_id = (uint32_t)id;
+    s.sub = page & ((1u << p.page_shift) - 1u);
     s.lo = begin - page * kPageTokens;
     s.hi = end - page * kPageTokens;
     s.row = (uint32_t)row0 + (begin - (uint32_t)start);
@@ -205,7 +209,8 @@ yvex_rocm_kv_append_bf16(const yvex_rocm_kv_append_params p)
     const uint32_t head = blockIdx.y * kWaves + wave;
     const bool active = s.valid && head < p.kv_heads;
     uint16_t (*v_rows)[kRowPitch] = v_rows_all[wave];
-    const uint64_t block = ((uint64_t)s.page_id * p.kv_heads + head) * (kPageTokens * kHeadDim);
+    const uint64_t block = ((((uint64_t)s.page_id * p.kv_heads + head) << p.page_shift) + s.sub) *
+                           (kPageTokens * kHeadDim);
     uint16_t *kdst = (uint16_t *)p.k_pool + block, *vdst = (uint16_t *)p.v_pool + block;
     const bool partial = s.lo != 0u || s.hi != (uint32_t)kPageTokens;
     const uint32_t pairs = p.rotary_dim / 16u;
@@ -316,7 +321,8 @@ yvex_rocm_kv_append_q8_0(const yvex_rocm_kv_append_params p)
     const uint32_t t = lane >> 2, j = lane & 3u;
     constexpr uint32_t kCodeBytes = kPageTokens * kHeadDim;
     constexpr uint32_t kBlockBytes = kCodeBytes + kPageTokens * 4 * 2;
-    const uint64_t block = ((uint64_t)s.page_id * p.kv_heads + head) * kBlockBytes;
+    const uint64_t block = ((((uint64_t)s.page_id * p.kv_heads + head) << p.page_shift) + s.sub) *
+                           kBlockBytes;
     unsigned char *kdst = (unsigned char *)p.k_pool + block, *vdst = (unsigned char *)p.v_pool + block;
     const bool partial = s.lo != 0u || s.hi != (uint32_t)kPageTokens;
     const bool mine = t >= s.lo && t < s.hi;

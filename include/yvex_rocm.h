@@ -482,13 +482,15 @@ typedef enum {
 
 /*
  * Paged GQA decode: one query token per session against a paged KV pool.
- * Device page layouts (head_dimension 128, page_tokens 16), per (page, kv_head):
+ * Device page layouts (head_dimension 128), per (page, kv_head) and block of 16 tokens; a
+ * page of 16 tokens (page_tokens 16) is one block, a page of 64 tokens (page_tokens 64) four
+ * blocks one behind the other, tokens 16 s .. 16 s + 15 of the page in block s:
  *   BF16  K block: uint16 [d/8][16 tokens][8]           (4096 B)
  *         V block: uint16 [d][16 tokens]                (4096 B)
  *   Q8_0  K block: int8 [4 lane groups][16 tokens][4 blocks][8] + f16 scale [16 tokens][4 blocks]
  *         V block: int8 [4 token groups][16 dims][8 dim blocks][4 tokens] + f16 scale [16 tokens][4 blocks]
  *                                                        (2176 B each)
- * Pool = [pool_pages][key_value_heads][block].  yvex_rocm_kv_pack_* build these from
+ * Pool = [pool_pages][key_value_heads][page_tokens / 16][block].  yvex_rocm_kv_pack_* build these from
  * token-major rows.  page_table is I32 [sessions][page_table_stride]; context_tokens is
  * I32 [sessions] (both device tensors).  Output is BF16 [sessions][query_heads][d], lse is
  * F32 [sessions][query_heads] (natural-log log-sum-exp of the scaled scores; optional).
@@ -586,7 +588,8 @@ typedef struct yvex_rocm_mla_decode_request {
  * contributes token_count[s] consecutive rows of `key` / `value` starting at row_start[s];
  * they become positions position_start[s] .. of that session.  rotary_dimension = 0 writes
  * the keys as given; otherwise cosine / sine are F32 [total_tokens][rotary_dimension] tables
- * indexed by input row (src/backend/cuda/transformer_kernels.cu:79-108).
+ * indexed by input row and the keys are rotated in the order rotary_mode names (below).
+ * page_tokens is 16 or 64 (the layouts of the paged decode).
  * Caller contract: within one call no page id appears in the rows of two sessions, and the
  * token ranges of one session do not overlap.  A V page block is filled by a read-modify-
  * write of whole 16-byte groups, one workgroup per (session, page): two sessions writing the

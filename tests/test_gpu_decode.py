@@ -128,10 +128,10 @@ def make_paged_case(rng, contexts, hq, hkv, d=128, page_tokens=16, spare=5, q8=F
 
 
 def run_paged(backend, q, k_rows, v_rows, table, ctx, hkv, pool_pages, storage=B.KV_BF16,
-              max_context=None):
+              max_context=None, page_tokens=16):
     sessions, hq, d = q.shape
-    kp = kv_pack_pages(k_rows, storage, False, hkv)
-    vp = kv_pack_pages(v_rows, storage, True, hkv)
+    kp = kv_pack_pages(k_rows, storage, False, hkv, page_tokens=page_tokens)
+    vp = kv_pack_pages(v_rows, storage, True, hkv, page_tokens=page_tokens)
     pool_dtype = B.DTYPE_BF16 if storage == B.KV_BF16 else B.DTYPE_I8
     elems = kp.size // B.DTYPE_BYTES[pool_dtype]
     tq = backend.tensor("q", B.DTYPE_BF16, q.shape, q)
@@ -141,8 +141,8 @@ def run_paged(backend, q, k_rows, v_rows, table, ctx, hkv, pool_pages, storage=B
     tc = backend.tensor("ctx", B.DTYPE_I32, ctx.shape, ctx)
     out = backend.tensor("o", B.DTYPE_BF16, q.shape)
     lse = backend.tensor("lse", B.DTYPE_F32, (sessions, hq))
-    req = backend.paged_requirement(sessions, hq, hkv, d, 16, pool_pages, table.shape[1],
-                                    max_context or int(table.shape[1] * 16), storage=storage)
+    req = backend.paged_requirement(sessions, hq, hkv, d, page_tokens, pool_pages, table.shape[1],
+                                    max_context or int(table.shape[1] * page_tokens), storage=storage)
     facts = backend.paged_decode_execute(req, tq, tkp, tvp, tt, tc, out, lse)
     return out.read(), lse.read(), facts
 
@@ -224,8 +224,8 @@ def test_config3_shape_sample(backend):
 
 # ------------------------------------------------------------- Q8_0 paged KV ----
 
-def make_q8_case(rng, contexts, hq, hkv, d=128):
-    q, k_rows, v_rows, table, ctx, pool_pages = make_paged_case(rng, contexts, hq, hkv, d)
+def make_q8_case(rng, contexts, hq, hkv, d=128, page_tokens=16):
+    q, k_rows, v_rows, table, ctx, pool_pages = make_paged_case(rng, contexts, hq, hkv, d, page_tokens)
     # quantise on the host with the product's own encoder (round-to-nearest absmax/127)
     from clori_amd.backend import q8_0_encode_rows
     k_blocks = q8_0_encode_rows(ORACLE.bf16_decode(k_rows))
@@ -332,3 +332,36 @@ def test_paged_decode_many_short_sessions(backend, q8):
     assert rc == 0
     assert_close_bf16(got, ref, "many sessions")
     assert_lse(lse, ref_lse, "many sessions")
+
+
+# ------------------------------------------------------- pages of 64 tokens ----
+
+@pytest.mark.parametrize("q8", [False, True], ids=["bf16", "q8_0"])
+def test_paged_decode_with_pages_of_64_tokens(backend, q8):
+    """Pages of 64 tokens (four 16-token blocks each): ragged contexts around block and page
+    edges against the oracle on 64-token pages, and bit for bit against the same rows cut
+    into 16-token pages."""
+    rng = np.random.default_rng(64 + int(q8))
+    contexts = [1, 15, 16, 17, 63, 64, 65, 127, 129, 1000, 4097, 20000]
+    make = make_q8_case if q8 else make_paged_case
+    storage = B.KV_Q8_0 if q8 else B.KV_BF16
+    q, k_rows, v_rows, table, ctx, pool_pages = make(rng, contexts, 32, 8, page_tokens=64)
+    got, lse, facts = run_paged(backend, q, k_rows, v_rows, table, ctx, 8, pool_pages,
+                                storage=storage, page_tokens=64)
+    rc, ref, _, ref_lse = ORACLE.paged_decode(q, k_rows, v_rows, table, ctx, 8, 64, q8=q8)
+    assert rc == 0
+    assert_close_bf16(got, ref, "64-token pages")
+    assert_lse(lse, ref_lse, "64-token pages")
+    # the same rows as pages of 16: page p of 64 becomes pages 4p .. 4p+3
+    narrow_rows = [rows.reshape((pool_pages * 4, 16) + rows.shape[2:]) for rows in (k_rows, v_rows)]
+    narrow_table = (table[:, :, None] * 4 + np.arange(4, dtype=np.int32)).reshape(len(contexts), -1)
+    got16, lse16, _ = run_paged(backend, q, narrow_rows[0], narrow_rows[1],
+                                np.ascontiguousarray(narrow_table, np.int32), ctx, 8, pool_pages * 4,
+                                storage=storage)
+    assert np.array_equal(got, got16) and np.array_equal(lse, lse16)
+    # a page id out of range is still caught
+    bad = table.copy()
+    bad[11, 5] = pool_pages
+    with pytest.raises(YvexError) as e:
+        run_paged(backend, q, k_rows, v_rows, bad, ctx, 8, pool_pages, storage=storage, page_tokens=64)
+    assert e.value.code == B.YVEX_ERR_BOUNDS

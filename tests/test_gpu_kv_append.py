@@ -251,3 +251,69 @@ def test_append_refusals(backend):
     with pytest.raises(YvexError) as e:
         run_case(backend, rng, [0], [1], B.KV_BF16, 24)
     assert e.value.code == B.YVEX_ERR_UNSUPPORTED
+
+
+@pytest.mark.parametrize("storage", [B.KV_BF16, B.KV_Q8_0], ids=["bf16", "q8_0"])
+def test_append_into_pages_of_64_tokens(backend, storage):
+    """The page writer with pages of 64 tokens (four 16-token blocks per page and kv head):
+    every byte of both pools against the host-side restatement, then decode over them."""
+    rng = np.random.default_rng(640 + storage)
+    q8 = storage == B.KV_Q8_0
+    page, rotary_dim = 64, 64
+    starts, counts = [0, 61, 130, 64, 200], [1, 10, 300, 0, 77]
+    sessions = len(starts)
+    stride = max((s + c + page - 1) // page for s, c in zip(starts, counts)) + 1
+    pool_pages = sessions * stride + 2
+    table = rng.permutation(pool_pages)[:sessions * stride].astype(np.int32).reshape(sessions, stride)
+    total = int(sum(counts))
+    row_starts = np.concatenate([[0], np.cumsum(counts)[:-1]]).astype(np.int32)
+    k_new, v_new = bf16_normal(rng, (total, HKV, D)), bf16_normal(rng, (total, HKV, D))
+    angles = rng.uniform(-3.0, 3.0, size=(total, rotary_dim)).astype(np.float32)
+    cosine, sine = np.cos(angles).astype(np.float32), np.sin(angles).astype(np.float32)
+    old_k, old_v = bf16_normal(rng, (pool_pages, page, HKV, D)), bf16_normal(rng, (pool_pages, page, HKV, D))
+
+    def stored(rows):
+        return q8_0_encode_rows(ORACLE.bf16_decode(rows)).reshape(rows.shape[:-1] + (-1,)) if q8 else rows
+    k_rows, v_rows = stored(old_k), stored(old_v)
+    pool_dtype = B.DTYPE_I8 if q8 else B.DTYPE_BF16
+    kp = kv_pack_pages(k_rows, storage, False, HKV, page_tokens=page)
+    vp = kv_pack_pages(v_rows, storage, True, HKV, page_tokens=page)
+    elems = kp.size // B.DTYPE_BYTES[pool_dtype]
+    t = [backend.tensor("k-new", B.DTYPE_BF16, k_new.shape, k_new),
+         backend.tensor("v-new", B.DTYPE_BF16, v_new.shape, v_new),
+         backend.tensor("rows", B.DTYPE_I32, (sessions,), row_starts),
+         backend.tensor("starts", B.DTYPE_I32, (sessions,), np.array(starts, np.int32)),
+         backend.tensor("counts", B.DTYPE_I32, (sessions,), np.array(counts, np.int32)),
+         backend.tensor("table", B.DTYPE_I32, table.shape, table),
+         backend.tensor("kpool", pool_dtype, (elems,), kp),
+         backend.tensor("vpool", pool_dtype, (elems,), vp)]
+    tc = backend.tensor("cos", B.DTYPE_F32, cosine.shape, cosine)
+    ts = backend.tensor("sin", B.DTYPE_F32, sine.shape, sine)
+    facts = backend.kv_append_execute(*t, HKV, pool_pages, max(counts), storage=storage, cosine=tc, sine=ts,
+                                      rotary_dimension=rotary_dim, page_tokens=page)
+    assert facts.kernel_launches == 1
+    k_rot = ORACLE.rotary_half_bf16(k_new, cosine, sine, rotary_dim)
+    want_k, want_v = k_rows.copy(), v_rows.copy()
+    for s in range(sessions):
+        for i in range(counts[s]):
+            position = starts[s] + i
+            want_k[table[s, position // page], position % page] = stored(k_rot[row_starts[s] + i][None])[0]
+            want_v[table[s, position // page], position % page] = stored(v_new[row_starts[s] + i][None])[0]
+    got_k = kv_unpack_pages(t[6].read(np.uint8, (-1,)), storage, False, pool_pages, HKV, page_tokens=page)
+    got_v = kv_unpack_pages(t[7].read(np.uint8, (-1,)), storage, True, pool_pages, HKV, page_tokens=page)
+    assert np.array_equal(got_k.reshape(want_k.shape), want_k)
+    assert np.array_equal(got_v.reshape(want_v.shape), want_v)
+    # decode over what was written
+    ctx = np.array([s + c for s, c in zip(starts, counts)], np.int32)
+    q = bf16_normal(rng, (sessions, 32, D))
+    tq = backend.tensor("q", B.DTYPE_BF16, q.shape, q)
+    tctx = backend.tensor("ctx", B.DTYPE_I32, ctx.shape, ctx)
+    out = backend.tensor("o", B.DTYPE_BF16, q.shape)
+    req = backend.paged_requirement(sessions, 32, HKV, D, page, pool_pages, stride, stride * page,
+                                    storage=storage)
+    backend.paged_decode_execute(req, tq, t[6], t[7], t[5], tctx, out)
+    rc, ref, _, _ = ORACLE.paged_decode(q, want_k, want_v, table, ctx, HKV, page, q8=q8)
+    assert rc == 0
+    assert_close_bf16(out.read(), ref, "decode over 64-token pages")
+    for x in t + [tc, ts, tq, tctx, out]:
+        x.release()

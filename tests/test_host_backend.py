@@ -603,6 +603,11 @@ def test_paged_and_mla_admission():
         out = b.tensor("o", B.DTYPE_BF16, (4, 32, 128))
         facts = b.paged_decode_execute(ok, q, pool, pool, table, ctx, out)
         assert facts.kernel_launches == 1 and out.is_written
+        # the same pool read as 25 pages of 64 tokens (four 16-token blocks each)
+        wide = b.paged_requirement(4, 32, 8, 128, 64, 25, 16, 1024)
+        assert b.paged_decode_workspace_required(wide) == b.paged_decode_workspace_required(ok)
+        wide_table = written(b, "t64", B.DTYPE_I32, (4, 16))
+        assert b.paged_decode_execute(wide, q, pool, pool, wide_table, ctx, out).kernel_launches == 1
         small = written(b, "small-pool", B.DTYPE_BF16, (99 * 8 * 2048,))
         with pytest.raises(YvexError) as e:
             b.paged_decode_execute(ok, q, small, pool, table, ctx, out)
@@ -673,11 +678,15 @@ def test_kv_append_admission():
         args = (key, value, rows, starts, counts, table, k_pool, v_pool, hkv, pages, 8)
         facts = b.kv_append_execute(*args, cosine=cosine, sine=sine, rotary_dimension=64)
         assert facts.kernel_launches == 1 and k_pool.is_written and v_pool.is_written
+        # pages of 64 tokens: four 16-token blocks each, so a quarter of the pages hold the same rows
+        wide_table = written(b, "t64", B.DTYPE_I32, (sessions, 1))
+        assert b.kv_append_execute(key, value, rows, starts, counts, wide_table, k_pool, v_pool, hkv,
+                                   pages // 4, 8, page_tokens=64).kernel_launches == 1
         q_pool = b.tensor("qp", B.DTYPE_I8, (pages * hkv * 2176,))
         assert b.kv_append_execute(key, value, rows, starts, counts, table, q_pool, q_pool, hkv,
                                    pages, 8, storage=B.KV_Q8_0).kernel_launches == 1
         for kwargs, code in [(dict(head_dimension=64), B.YVEX_ERR_UNSUPPORTED),
-                             (dict(page_tokens=64), B.YVEX_ERR_UNSUPPORTED),
+                             (dict(page_tokens=32), B.YVEX_ERR_UNSUPPORTED),
                              (dict(storage=7), B.YVEX_ERR_UNSUPPORTED),
                              (dict(rotary_dimension=24, cosine=cosine, sine=sine), B.YVEX_ERR_UNSUPPORTED),
                              (dict(rotary_dimension=256, cosine=cosine, sine=sine), B.YVEX_ERR_UNSUPPORTED),
@@ -1050,6 +1059,19 @@ def test_page_layouts_follow_the_documented_index_formulas():
                 scales = canon[page, :, head, :, :2].reshape(16 * 4 * 2)
                 assert np.array_equal(packed[page, head, 2048:], scales)
         assert np.array_equal(kv_unpack_pages(packed, B.KV_Q8_0, is_value, pages, hkv), blocks)
+    # a page of 64 tokens is four 16-token blocks, one behind the other, per (page, kv head)
+    for storage, wide, width in ((B.KV_BF16, rng.integers(0, 1 << 16, size=(pages, 64, hkv, d), dtype=np.uint16), 4096),
+                                 (B.KV_Q8_0, rng.integers(0, 256, size=(pages, 64, hkv, 4 * 34), dtype=np.uint8), 2176)):
+        for is_value in (False, True):
+            packed = kv_pack_pages(wide, storage, is_value, hkv, page_tokens=64).reshape(pages, hkv, 4, width)
+            as_blocks = wide.reshape((pages * 4, 16) + wide.shape[2:])
+            narrow = kv_pack_pages(as_blocks, storage, is_value, hkv).reshape(pages, 4, hkv, width)
+            assert np.array_equal(packed, narrow.transpose(0, 2, 1, 3))
+            back = kv_unpack_pages(packed, storage, is_value, pages, hkv, page_tokens=64)
+            assert np.array_equal(back.reshape(wide.shape), wide)
+    assert lib().yvex_rocm_kv_page_block_bytes(B.KV_BF16, 128, 64) == 4 * 4096
+    assert lib().yvex_rocm_kv_page_block_bytes(B.KV_Q8_0, 128, 64) == 4 * 2176
+    assert lib().yvex_rocm_kv_page_block_bytes(B.KV_BF16, 128, 32) == 0
     with pytest.raises(YvexError) as e:
         kv_pack_pages(rows, B.KV_BF16, False, hkv, head_dim=64)
     assert e.value.code == B.YVEX_ERR_UNSUPPORTED
