@@ -156,6 +156,8 @@ def workload_paged(backend, rng, steps, warmup, q8=False, page=16):
     pool_pages = int(need.sum())
     stride = int(hi // page)
     perm = rng.permutation(pool_pages).astype(np.int32)
+    if os.environ.get("YVEX_BENCH_ORDERED_PAGES"):     # tuning aid: pages in pool order
+        perm = np.arange(pool_pages, dtype=np.int32)
     table = np.zeros((sessions, stride), dtype=np.int32)
     at = 0
     for s in range(sessions):
