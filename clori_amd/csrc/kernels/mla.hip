@@ -42,10 +42,14 @@ constexpr int kBuffers = 4;
 constexpr int kHeadsPerWave = 32;
 constexpr float kLazyLog2 = 8.0f;
 constexpr int kQkDepth = 4;  // operand fetches in flight ahead of the first product
-constexpr int kMaxChunkPages = YVEX_ROCM_MLA_MAX_CHUNK_PAGES;  // page ids of the chunk, kept in LDS
+constexpr uint32_t kPageShift = 6;  // pages of 64 tokens (the host admits no other size)
 
 typedef __attribute__((address_space(3))) short4v lds_short4;
 typedef short short8v __attribute__((ext_vector_type(8)));
+// The page table is read through the constant address space: the address is wave-uniform and
+// nothing writes the table while the kernel runs, so every read is a scalar load that counts
+// on lgkmcnt and leaves the hand-counted vmcnt of the tile ring alone.
+typedef __attribute__((address_space(4))) const int32_t constant_i32;
 
 __device__ inline void flag(int32_t *status, int code) { atomicCAS(status, 0, code); }
 
@@ -59,8 +63,7 @@ __device__ inline int swizzle(int r) { return (((r >> 1) & 1) << 2) | ((r >> 2) 
 // 1152-byte pitch in LDS (so the bank analysis above holds unchanged), every wave stages
 // eight whole rows, one per load, and waves 2 and 3 only stage: they own no heads.
 template <int kKeyDim, int kHeads>
-__device__ __forceinline__ void mla_decode(const yvex_rocm_mla_params &p, unsigned char *lds,
-                                           int32_t *chunk_pages)
+__device__ __forceinline__ void mla_decode(const yvex_rocm_mla_params &p, unsigned char *lds)
 {
     constexpr int kSteps = kKeyDim / 16;                     // k-steps of the first product
     constexpr int kSourceRowBytes = kKeyDim * 2;             // row size in global memory
@@ -68,38 +71,30 @@ __device__ __forceinline__ void mla_decode(const yvex_rocm_mla_params &p, unsign
     constexpr int kLoadsPerWave = kRowPerLoad ? kTile / 4 : kTileBytes / 1024 / 4;  // 8 or 9
     constexpr int kLoadPitch = kRowPerLoad ? kRowBytes : 1024;  // LDS distance between a wave's loads
     constexpr int kActiveWaves = kHeads / kHeadsPerWave;
+    constexpr int kQueryRounds = kActiveWaves / 2;           // two head groups per round
     static_assert(kSteps % 4 == 0 && kSteps / 4 == kLoadsPerWave,
                   "the loads of a tile ride behind k-steps 1, 5, 9, ...");
     static_assert(kRowPerLoad || kSourceRowBytes == kRowBytes, "rows are 1024 or 1152 bytes");
+    static_assert(kActiveWaves == 2 || kActiveWaves == 4, "head groups come in pairs");
     // at most one younger tile outstanding: vmcnt(kLoadsPerWave), lgkmcnt and expcnt untouched
     constexpr int kWaitTile = 0x0f70 | kLoadsPerWave;
+    // at most two younger tiles outstanding
+    constexpr int kWaitTwoTiles = 0x0f70 | ((2 * kLoadsPerWave) & 15) | (((2 * kLoadsPerWave) >> 4) << 14);
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n = lane & 31, g = lane >> 5;
-    const uint32_t chunk = blockIdx.x, batch = blockIdx.y;
-    const uint32_t ctx = (uint32_t)p.context[batch];
-    if (ctx == 0u && p.empty_ok != 0u) return;
-    if (ctx == 0u || ctx > p.table_stride * p.page_tokens) {
-        if (chunk == 0u && tid == 0) flag(p.status, YVEX_ROCM_DEVICE_CONTRACT);
-        return;
-    }
-    // sliding window (src/backend/cuda/attention_kernels.cu:79-84): positions below
-    // ctx - window are not visible; chunks start at the tile that holds the first visible one
-    const uint32_t w0 = p.window != 0u && ctx > p.window ? ctx - p.window : 0u;
-    const uint32_t t0 = (w0 & ~(uint32_t)(kTile - 1)) + chunk * p.chunk_tokens;
-    if (t0 >= ctx) return;
-    const uint32_t t1 = min(ctx, t0 + p.chunk_tokens);
-    const uint32_t tiles = (t1 - t0 + kTile - 1) / kTile;
-    const uint32_t head = wave * kHeadsPerWave + n;
-
-    // ---- tile staging --------------------------------------------------------------
-    // the chunk's page ids are fetched once, so staging a tile never waits on global memory
-    const int32_t *table = p.page_table + (uint64_t)batch * p.table_stride;
-    const uint32_t first_page = t0 / p.page_tokens;
-    const uint32_t chunk_page_count = (t1 - 1u) / p.page_tokens - first_page + 1u;
-    if (chunk_page_count > (uint32_t)kMaxChunkPages) {
-        if (tid == 0) flag(p.status, YVEX_ROCM_DEVICE_CONTRACT);
-        return;
+    // Workgroups go to the eight XCDs round robin by their linear id.  They are renumbered so
+    // that the chunks of a batch element sit on one XCD: its queries (read by every chunk) and
+    // its page table then come from HBM once instead of once per XCD.
+    uint32_t chunk = blockIdx.x, batch = blockIdx.y;
+    {
+        const uint32_t total = gridDim.x * gridDim.y;
+        if ((total & 7u) == 0u) {
+            const uint32_t linear = blockIdx.x + gridDim.x * blockIdx.y;
+            const uint32_t renumbered = (linear & 7u) * (total >> 3) + (linear >> 3);
+            batch = renumbered / gridDim.x;
+            chunk = renumbered % gridDim.x;
+        }
     }
     const uint32_t lds_base = lds_address_of(lds);
     // source offset of this lane's 16 bytes in load j: the chunk that belongs at the lane's
@@ -116,55 +111,89 @@ __device__ __forceinline__ void mla_decode(const yvex_rocm_mla_params &p, unsign
             stage_off[j] = (uint32_t)(r * kRowBytes + ((pos ^ swizzle(r)) << 4));
         }
     }
-    // The queries of the batch element first: 128 rows of 1152 bytes are exactly the four tile
-    // buffers, so they are staged like four tiles (coalesced 1 KB loads, same swizzle) and each
-    // wave then takes its 32 heads out of "tile" `wave` with the row fetch of the first product.
-    // A lane's fragments sit 1152 bytes apart in global memory; fetched directly they cost 36
-    // loads of 32 separate lines each and five microseconds before the first tile could start.
-    static_assert(kActiveWaves * kHeadsPerWave * kRowBytes <= kBuffers * kTileBytes, "Q fits the tile ring");
+    // The queries of the batch element go through the tile buffers too (coalesced 1 KB loads,
+    // same swizzle, 32 heads = one "tile"), two head groups per round into buffers 2 and 3,
+    // while tiles 0 and 1 are already on their way into buffers 0 and 1: the first tiles'
+    // trip to memory runs under the query rounds instead of after them.  A lane's fragments
+    // sit 1152 bytes apart in global memory; fetched directly they cost 36 loads of 32
+    // separate lines each.
+    auto stage_queries = [&](int round) {
 #pragma unroll
-    for (int j = 0; j < kActiveWaves; ++j) {
-        const i32x4 rsrc = raw_buffer(p.q + ((uint64_t)batch * p.heads + j * kHeadsPerWave) * kKeyDim,
-                                      kHeadsPerWave * kSourceRowBytes);
-        const uint32_t dst = __builtin_amdgcn_readfirstlane(lds_base + j * kTileBytes +
-                                                            wave * (kLoadsPerWave * kLoadPitch));
+        for (int j = 0; j < 2; ++j) {
+            const i32x4 rsrc = raw_buffer(
+                p.q + ((uint64_t)batch * p.heads + (2 * round + j) * kHeadsPerWave) * kKeyDim,
+                kHeadsPerWave * kSourceRowBytes);
+            const uint32_t dst = __builtin_amdgcn_readfirstlane(lds_base + (2 + j) * kTileBytes +
+                                                                wave * (kLoadsPerWave * kLoadPitch));
 #pragma unroll
-        for (int i = 0; i < kLoadsPerWave; ++i) lds_dma_b128(dst + i * kLoadPitch, rsrc, stage_off[i], 0u);
-    }
-    for (uint32_t i = tid; i < chunk_page_count; i += 256u) {
-        int32_t page = table[first_page + i];
-        if (page < 0 || (uint32_t)page >= p.pool_pages) {
-            flag(p.status, YVEX_ROCM_DEVICE_CONTRACT);
-            page = 0;
+            for (int i = 0; i < kLoadsPerWave; ++i) lds_dma_b128(dst + i * kLoadPitch, rsrc, stage_off[i], 0u);
         }
-        chunk_pages[i] = page;
+    };
+    // The first query round is on its way before the context length is known: its address
+    // needs only the batch element.  A workgroup that turns out to have nothing to do waits for
+    // these loads before it ends (they write its LDS).
+    stage_queries(0);
+    const uint32_t ctx = (uint32_t)p.context[batch];
+    if (ctx == 0u && p.empty_ok != 0u) {
+        __builtin_amdgcn_s_waitcnt(0x0f70);
+        return;
     }
-    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's share of Q has landed
-    __syncthreads();                     // ... and everybody's, and the page ids
+    if (ctx == 0u || ctx > p.table_stride * p.page_tokens || p.page_tokens != (1u << kPageShift)) {
+        if (chunk == 0u && tid == 0) flag(p.status, YVEX_ROCM_DEVICE_CONTRACT);
+        __builtin_amdgcn_s_waitcnt(0x0f70);
+        return;
+    }
+    // sliding window (src/backend/cuda/attention_kernels.cu:79-84): positions below
+    // ctx - window are not visible; chunks start at the tile that holds the first visible one
+    const uint32_t w0 = p.window != 0u && ctx > p.window ? ctx - p.window : 0u;
+    const uint32_t t0 = (w0 & ~(uint32_t)(kTile - 1)) + chunk * p.chunk_tokens;
+    if (t0 >= ctx) {
+        __builtin_amdgcn_s_waitcnt(0x0f70);
+        return;
+    }
+    const uint32_t t1 = min(ctx, t0 + p.chunk_tokens);
+    const uint32_t tiles = (t1 - t0 + kTile - 1) / kTile;
+    const uint32_t head = wave * kHeadsPerWave + n;
+
+    // ---- tile staging --------------------------------------------------------------
+    // Page ids come by scalar loads, one tile ahead of the staging that needs them; an id
+    // outside the pool is a contract violation (page 0 is read instead, the status says so).
+    constant_i32 *table = (constant_i32 *)(p.page_table + (uint64_t)batch * p.table_stride);
+    const uint32_t last_page_index = (t1 - 1u) >> kPageShift;
+    auto page_fetch = [&](uint32_t tile) -> int32_t {
+        return table[min((t0 + tile * kTile) >> kPageShift, last_page_index)];
+    };
+    auto page_checked = [&](int32_t id) -> uint32_t {
+        const bool outside = id < 0 || (uint32_t)id >= p.pool_pages;
+        if (outside && lane == 0) flag(p.status, YVEX_ROCM_DEVICE_CONTRACT);
+        return (uint32_t)__builtin_amdgcn_readfirstlane(outside ? 0 : id);
+    };
     // A tile's destination and descriptor.  Loads are always issued (with an empty range
     // past the last tile) so that the outstanding-load count at the top of every step is
     // the same.
-    auto stage_target = [&](uint32_t tile, uint32_t &dst, i32x4 &rsrc) {
+    auto stage_target = [&](uint32_t tile, uint32_t page, uint32_t &dst, i32x4 &rsrc) {
         const uint32_t first = t0 + tile * kTile;
         uint32_t valid = 0u;
         const uint16_t *base = p.pool;
         if (tile < tiles) {
-            const uint32_t page = (uint32_t)__builtin_amdgcn_readfirstlane(
-                chunk_pages[first / p.page_tokens - first_page]);
             valid = min((uint32_t)kTile, t1 - first);
-            base = p.pool + ((uint64_t)page * p.page_tokens + first % p.page_tokens) * kKeyDim;
+            base = p.pool + (((uint64_t)page << kPageShift) + (first & ((1u << kPageShift) - 1u))) * kKeyDim;
         }
         rsrc = raw_buffer(base, valid * kSourceRowBytes);
         dst = __builtin_amdgcn_readfirstlane(lds_base + (tile % kBuffers) * kTileBytes +
                                              wave * (kLoadsPerWave * kLoadPitch));
     };
-    auto stage_tile = [&](uint32_t tile) {
+    auto stage_tile = [&](uint32_t tile, uint32_t page) {
         uint32_t dst;
         i32x4 rsrc;
-        stage_target(tile, dst, rsrc);
+        stage_target(tile, page, dst, rsrc);
 #pragma unroll
         for (int j = 0; j < kLoadsPerWave; ++j) lds_dma_b128(dst + j * kLoadPitch, rsrc, stage_off[j], 0u);
     };
+    const int32_t id0 = page_fetch(0u), id1 = page_fetch(1u);
+    int32_t id_ahead = page_fetch(2u);  // fetched a step before the staging that uses it
+    stage_tile(0u, page_checked(id0));
+    stage_tile(1u, page_checked(id1));
 
     // ---- operand addresses inside a tile ----------------------------------------------
     // first product, k-step kk: row n, chunk 2kk + g; one address per kk % 4, the rest is
@@ -191,24 +220,35 @@ __device__ __forceinline__ void mla_decode(const yvex_rocm_mla_params &p, unsign
             }
     }
 
-    // Q fragments: B operand, lane (n, g) holds Q[head n][16*kk + 8g .. +7], kk = 0..35
+    // Q fragments: B operand, lane (n, g) holds Q[head n][16*kk + 8g .. +7], kk = 0..35.  The
+    // head group of wave w arrives in round w / 2, in buffer 2 + w % 2.
     bf16x8 q[kSteps];
-    {
-        const unsigned char *rows = lds + wave * kTileBytes;
+    auto take_queries = [&]() {
+        const unsigned char *rows = lds + (2 + (wave & 1)) * kTileBytes;
 #pragma unroll
         for (int kk = 0; kk < kSteps; ++kk)
             q[kk] = as_bf16x8(*reinterpret_cast<const u32x4 *>(rows + k_addr[kk & 3] + (kk >> 2) * 128));
+    };
+    // round 0 has landed when only the two tiles behind it are outstanding
+    __builtin_amdgcn_s_waitcnt(kWaitTwoTiles);
+    __syncthreads();
+    if (wave < 2) take_queries();
+    if (kQueryRounds == 2) {
+        __syncthreads();  // buffers 2 and 3 are free again
+        stage_queries(1);
+        __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): round 1, and tiles 0 and 1 with it
+        __syncthreads();
+        if (wave >= 2) take_queries();
     }
-    __syncthreads();  // the buffers are free for tiles once every wave holds its fragments
+    __syncthreads();  // buffers 2 and 3 are free for tiles once every wave holds its fragments
     if (kActiveWaves < 4 && wave >= kActiveWaves) {
         // a wave without heads: it stages its quarter of every tile and keeps the barriers of
         // the computing waves (one per tile, one before their epilogue)
-        stage_tile(0u);
-        stage_tile(1u);
         for (uint32_t t = 0; t < tiles; ++t) {
             __builtin_amdgcn_s_waitcnt(kWaitTile);
             __syncthreads();
-            stage_tile(t + 2u);
+            stage_tile(t + 2u, page_checked(id_ahead));
+            id_ahead = page_fetch(t + 3u);
         }
         __builtin_amdgcn_s_waitcnt(0x0f70);
         __syncthreads();
@@ -225,9 +265,13 @@ __device__ __forceinline__ void mla_decode(const yvex_rocm_mla_params &p, unsign
     // S^T of one tile; `extra(kk)` is work placed behind MFMA kk (operand fetches run
     // kQkDepth k-steps ahead; the order is pinned with scheduling barriers because the
     // register budget leaves the scheduler no room to do it on its own)
+    // The score accumulator lives in vector registers (all 256 accumulation registers hold
+    // O^T), which the compiler's own MFMA selection does not offer in a kernel that uses
+    // accumulation registers at all: these 36 MFMAs are written as assembly.  The compiler
+    // still sees their operands (it waits for the LDS fetches), but not their latency: the
+    // wait states a vector instruction needs before it reads an 8-pass MFMA's result are
+    // spent by hand after the last one.
     auto score = [&](const unsigned char *tile, floatx16 &s, auto extra) {
-#pragma unroll
-        for (int i = 0; i < 16; ++i) s[i] = 0.f;
         u32x4 frag[kQkDepth];
 #pragma unroll
         for (int kk = 0; kk < kQkDepth; ++kk)
@@ -235,7 +279,11 @@ __device__ __forceinline__ void mla_decode(const yvex_rocm_mla_params &p, unsign
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int kk = 0; kk < kSteps; ++kk) {
-            s = mfma_32x32x16(as_bf16x8(frag[kk % kQkDepth]), q[kk], s);
+            if (kk == 0)
+                asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(s) : "v"(frag[0]), "v"(q[0]));
+            else
+                asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0"
+                             : "+v"(s) : "v"(frag[kk % kQkDepth]), "v"(q[kk]));
             if (kk + kQkDepth < kSteps)
                 frag[kk % kQkDepth] = *reinterpret_cast<const u32x4 *>(
                     tile + k_addr[(kk + kQkDepth) & 3] + ((kk + kQkDepth) >> 2) * 128);
@@ -245,7 +293,9 @@ __device__ __forceinline__ void mla_decode(const yvex_rocm_mla_params &p, unsign
     };
     // masks the tail (and the keys in front of a sliding window), then raises the running maximum if this tile needs it (both token
     // halves of a head must agree on the reference maximum)
-    auto settle = [&](uint32_t key0, floatx16 &s, uint32_t (&pending)[8]) {
+    // `first`: the chunk's first tile, nothing accumulated yet: the maximum is taken as it is
+    // and there is nothing to rescale (the general path would multiply 256 zeros)
+    auto settle = [&](uint32_t key0, floatx16 &s, uint32_t (&pending)[8], auto first) {
         if (key0 + kTile > t1 || key0 < w0) {
             // visible keys are w0 <= key < t1: one unsigned compare
 #pragma unroll
@@ -256,7 +306,10 @@ __device__ __forceinline__ void mla_decode(const yvex_rocm_mla_params &p, unsign
 #pragma unroll
         for (int i = 0; i < 16; ++i) mloc = fmaxf(mloc, s[i]);
         mloc *= p.scale_log2;
-        if (__builtin_amdgcn_ballot_w64(mloc > m_run + kLazyLog2) != 0ull) {
+        if (decltype(first)::value) {
+            m_run = fmaxf(mloc, xor_lanes(mloc, 32));
+            neg_m = m_run == -INFINITY ? 0.f : -m_run;
+        } else if (__builtin_amdgcn_ballot_w64(mloc > m_run + kLazyLog2) != 0ull) {
             const float m_new = fmaxf(m_run, fmaxf(mloc, xor_lanes(mloc, 32)));
             const float alpha = m_new == -INFINITY ? 1.0f : fast_exp2(m_run - m_new);
             l_run *= alpha;
@@ -281,48 +334,67 @@ __device__ __forceinline__ void mla_decode(const yvex_rocm_mla_params &p, unsign
     // of tile t+2 spread behind its MFMAs), settles the maximum, then issues the O^T update
     // with tile t-1 and, behind its MFMAs, the exponentials of tile t.  Tiles t-1 and t
     // are being read during a step, tiles t+1 and t+2 are in flight.
-    stage_tile(0u);
-    stage_tile(1u);
     uint32_t pk_prev[8], pk_cur[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) pk_prev[j] = 0u;
-    // O^T += C^T . P^T with the tile at `tile`
-    auto accumulate = [&](const unsigned char *tile, const uint32_t (&pk)[8]) {
+    // O^T += C^T . P^T with the tile at `tile`, MFMAs [first, last) of the 32 (token half u =
+    // index / 16, dim block db = index % 16)
+    auto value_operand = [&](const unsigned char *tile, int index) -> bf16x8 {
+        const int u = index >> 4, db = index & 15;
+        const int imm = (db & ~1) * 64 + u * 16 * kRowBytes;
+        const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (lds_short4 *)(tile + v_addr[db & 1][0] + imm));
+        const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (lds_short4 *)(tile + v_addr[db & 1][1] + imm));
+        const short8v av = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        return __builtin_bit_cast(bf16x8, av);
+    };
+    auto accumulate = [&](const unsigned char *tile, const uint32_t (&pk)[8], int first, int last) {
 #pragma unroll
-        for (int u = 0; u < 2; ++u) {
+        for (int index = first; index < last; ++index) {
+            const int u = index >> 4, db = index & 15;
             const u32x4 w = {pk[u * 4 + 0], pk[u * 4 + 1], pk[u * 4 + 2], pk[u * 4 + 3]};
-            const bf16x8 pb = as_bf16x8(w);
-#pragma unroll
-            for (int db = 0; db < 16; ++db) {
-                const int imm = (db & ~1) * 64 + u * 16 * kRowBytes;
-                const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                    (lds_short4 *)(tile + v_addr[db & 1][0] + imm));
-                const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                    (lds_short4 *)(tile + v_addr[db & 1][1] + imm));
-                const short8v av = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-                o[db] = mfma_32x32x16(__builtin_bit_cast(bf16x8, av), pb, o[db]);
-            }
+            o[db] = mfma_32x32x16(value_operand(tile, index), as_bf16x8(w), o[db]);
         }
     };
+    constexpr int kEarly = 4;  // update MFMAs issued under the settling of the next tile's maximum
     auto step = [&](uint32_t t, auto with_update) {
         // tile t has landed when at most one younger tile is outstanding: vmcnt(9)
         __builtin_amdgcn_s_waitcnt(kWaitTile);
         __syncthreads();
         uint32_t stage_dst;
         i32x4 stage_rsrc;
-        stage_target(t + 2u, stage_dst, stage_rsrc);
+        stage_target(t + 2u, page_checked(id_ahead), stage_dst, stage_rsrc);
+        id_ahead = page_fetch(t + 3u);
         const unsigned char *tile = lds + (t % kBuffers) * kTileBytes;
         const unsigned char *prev_tile = lds + ((t + kBuffers - 1u) % kBuffers) * kTileBytes;
 
         // ---- S^T of tile t, the loads of tile t+2 behind its MFMAs ------------------------
         floatx16 s;
+        bf16x8 early[kEarly];
         score(tile, s, [&](int kk) {
             if ((kk & 3) == 1) lds_dma_b128(stage_dst + (kk >> 2) * kLoadPitch, stage_rsrc, stage_off[kk >> 2], 0u);
+            // the last k-steps fetch no further score operand: the first operands of the update
+            // take their place
+            if (decltype(with_update)::value && kk >= kSteps - kEarly)
+                early[kk - (kSteps - kEarly)] = value_operand(prev_tile, kk - (kSteps - kEarly));
         });
-        settle(t0 + t * kTile, s, pk_prev);
+        // The first MFMAs of the update with tile t-1 go out at once: they need nothing of tile t,
+        // and the wait for the last score MFMA, the row maximum and the decision about a new
+        // reference maximum run under them.  Should the maximum move, O (with what these MFMAs
+        // added) and the probabilities still waiting are rescaled together.
+        if (decltype(with_update)::value) {
+            const u32x4 w = {pk_prev[0], pk_prev[1], pk_prev[2], pk_prev[3]};
+#pragma unroll
+            for (int index = 0; index < kEarly; ++index)
+                o[index] = mfma_32x32x16(early[index], as_bf16x8(w), o[index]);
+        }
+        // wait states between the last score MFMA (8 passes) and the first vector read of its result
+        asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 7" : "+v"(s));
+        settle(t0 + t * kTile, s, pk_prev, std::integral_constant<bool, !decltype(with_update)::value>());
 
-        // ---- O^T update with tile t-1 (none in the first step) and the exponentials of
-        //      tile t behind its MFMAs -------------------------------------------------------
+        // ---- the rest of the O^T update with tile t-1 (none in the first step) and the
+        //      exponentials of tile t behind its MFMAs ---------------------------------------
         float lsum = 0.f;
 #pragma unroll
         for (int i = 0; i < 16; i += 2) {
@@ -333,12 +405,12 @@ __device__ __forceinline__ void mla_decode(const yvex_rocm_mla_params &p, unsign
         }
         l_run += lsum;
         if (decltype(with_update)::value) {
-            accumulate(prev_tile, pk_prev);
+            accumulate(prev_tile, pk_prev, kEarly, 32);
             // three transposed operand pairs in flight ahead of the MFMAs that consume them,
             // one exponential behind every second MFMA
             __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);
 #pragma unroll
-            for (int i = 0; i < 14; ++i) {
+            for (int i = 0; i < (32 - kEarly - 4) / 2; ++i) {
                 __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
                 __builtin_amdgcn_sched_group_barrier(0x400, 1, 0);
                 __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
@@ -360,7 +432,7 @@ __device__ __forceinline__ void mla_decode(const yvex_rocm_mla_params &p, unsign
         step(t, std::integral_constant<bool, true>());
     // the update with the last tile
     __builtin_amdgcn_sched_barrier(0);
-    accumulate(lds + ((tiles - 1u) % kBuffers) * kTileBytes, pk_prev);
+    accumulate(lds + ((tiles - 1u) % kBuffers) * kTileBytes, pk_prev, 0, 32);
     __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);
 #pragma unroll
     for (int i = 0; i < 29; ++i) {
@@ -414,8 +486,7 @@ __device__ __forceinline__ void mla_decode(const yvex_rocm_mla_params &p, unsign
     name(const yvex_rocm_mla_params p)                                                               \
     {                                                                                                \
         __shared__ __attribute__((aligned(16))) unsigned char lds[kBuffers * kTileBytes];            \
-        __shared__ int32_t chunk_pages[kMaxChunkPages];                                              \
-        mla_decode<key_dim, heads>(p, lds, chunk_pages);                                             \
+        mla_decode<key_dim, heads>(p, lds);                                                          \
     }
 
 YVEX_MLA_KERNEL(yvex_rocm_mla_decode_bf16, 576, 128)
