@@ -649,61 +649,77 @@ int yvex_backend_attention_complete(yvex_backend *backend,
 
 /* ----------------------------------------------------------- workspace ---- */
 
-/* src/backend/residency.c:207-231 (the kind check admits ROCM here). */
+/* The attached workspace is one tensor of the backend used as a bump arena: operations carve
+ * aligned pieces off its front for the length of one dispatch and the dispatch rewinds it.  The
+ * arena never grows and never allocates.  Behaviour follows the contract of
+ * src/backend/residency.c:207-283 (and tests/test_host_backend.py holds it to that):
+ *   attach   INVALID_ARG unless a live backend of this kind, a written-to-able tensor it owns
+ *            (not a reserved address range) and a non-zero generation; STATE when one is attached
+ *   detach   forgets the arena and its statistics; harmless without one
+ *   acquire  MISS without a usable arena or without room, INVALID for a zero size or an
+ *            alignment that is not a power of two, HIT with the address otherwise */
+static int workspace_backend_live(const yvex_backend *backend)
+{
+    return backend && !backend_cleanup_only(backend) && backend->status != YVEX_BACKEND_STATUS_FAILED;
+}
+
+static int workspace_tensor_usable(const yvex_backend *backend, const yvex_device_tensor *tensor)
+{
+    return tensor && tensor->data && tensor->bytes != 0ull && !tensor->virtual_reserved &&
+           backend_tensor_owner_is(backend, tensor);
+}
+
+static void workspace_bind(yvex_backend *backend, const yvex_device_tensor *tensor,
+                           unsigned long long generation)
+{
+    backend->workspace_device_tensor = tensor;
+    backend->workspace_device_address = tensor ? (unsigned long long)(uintptr_t)tensor->data : 0ull;
+    backend->workspace_bytes = tensor ? tensor->bytes : 0ull;
+    backend->workspace_generation = generation;
+    backend->workspace_cursor = 0ull;
+    backend->workspace_peak = 0ull;
+}
+
 int yvex_backend_workspace_attach(yvex_backend *backend, const yvex_device_tensor *device_tensor,
                                   unsigned long long generation, yvex_error *err)
 {
-    if (!backend || backend_cleanup_only(backend) || backend->kind != YVEX_BACKEND_KIND_ROCM ||
-        backend->status == YVEX_BACKEND_STATUS_FAILED || !device_tensor ||
-        !backend_tensor_owner_is(backend, device_tensor) || !device_tensor->data ||
-        !device_tensor->bytes || device_tensor->virtual_reserved || !generation)
-        return refuse(err, YVEX_ERR_INVALID_ARG, "backend.workspace.attach",
+    static const char where[] = "backend.workspace.attach";
+    if (!workspace_backend_live(backend) || backend->kind != YVEX_BACKEND_KIND_ROCM ||
+        generation == 0ull || !workspace_tensor_usable(backend, device_tensor))
+        return refuse(err, YVEX_ERR_INVALID_ARG, where,
                       "same-owner ROCm workspace tensor and generation are required");
-    if (backend->workspace_device_tensor)
-        return refuse(err, YVEX_ERR_STATE, "backend.workspace.attach",
-                      "backend workspace is already attached");
-    backend->workspace_device_tensor = device_tensor;
-    backend->workspace_device_address = (unsigned long long)(uintptr_t)device_tensor->data;
-    backend->workspace_bytes = device_tensor->bytes;
-    backend->workspace_generation = generation;
+    if (backend->workspace_device_tensor != NULL)
+        return refuse(err, YVEX_ERR_STATE, where, "backend workspace is already attached");
+    workspace_bind(backend, device_tensor, generation);
     yvex_error_clear(err);
     return YVEX_OK;
 }
 
 void yvex_backend_workspace_detach(yvex_backend *backend)
 {
-    if (!backend) return;
-    backend->workspace_device_tensor = NULL;
-    backend->workspace_device_address = 0ull;
-    backend->workspace_bytes = 0ull;
-    backend->workspace_cursor = 0ull;
-    backend->workspace_peak = 0ull;
-    backend->workspace_generation = 0ull;
+    if (backend) workspace_bind(backend, NULL, 0ull);
 }
 
-/* src/backend/residency.c:251-283: bump allocation, never grows, HIT/MISS/INVALID. */
 int yvex_backend_workspace_acquire(yvex_backend *backend, unsigned long long bytes,
                                    unsigned long long alignment,
                                    unsigned long long *device_address)
 {
-    unsigned long long aligned, mask;
+    unsigned long long begin, end, address;
     if (device_address) *device_address = 0ull;
-    if (!backend || backend_cleanup_only(backend) ||
-        backend->status == YVEX_BACKEND_STATUS_FAILED || !device_address ||
-        !backend->workspace_device_tensor)
+    if (!device_address || !workspace_backend_live(backend) || !backend->workspace_device_tensor)
         return YVEX_BACKEND_RESIDENT_MISS;
-    if (!bytes || !alignment || (alignment & (alignment - 1ull)) != 0ull)
+    if (bytes == 0ull || alignment == 0ull || (alignment & (alignment - 1ull)) != 0ull)
         return YVEX_BACKEND_RESIDENT_INVALID;
-    mask = alignment - 1ull;
-    if (backend->workspace_cursor > ULLONG_MAX - mask) return YVEX_BACKEND_RESIDENT_INVALID;
-    aligned = (backend->workspace_cursor + mask) & ~mask;
-    if (aligned > backend->workspace_bytes || bytes > backend->workspace_bytes - aligned ||
-        backend->workspace_device_address > ULLONG_MAX - aligned)
+    /* first multiple of the alignment at or behind the cursor */
+    if (!yvex_core_u64_add(backend->workspace_cursor, alignment - 1ull, &begin))
+        return YVEX_BACKEND_RESIDENT_INVALID;
+    begin -= begin % alignment;
+    if (!yvex_core_u64_add(begin, bytes, &end) || end > backend->workspace_bytes ||
+        !yvex_core_u64_add(backend->workspace_device_address, begin, &address))
         return YVEX_BACKEND_RESIDENT_MISS;
-    *device_address = backend->workspace_device_address + aligned;
-    backend->workspace_cursor = aligned + bytes;
-    if (backend->workspace_cursor > backend->workspace_peak)
-        backend->workspace_peak = backend->workspace_cursor;
+    backend->workspace_cursor = end;
+    if (end > backend->workspace_peak) backend->workspace_peak = end;
+    *device_address = address;
     return YVEX_BACKEND_RESIDENT_HIT;
 }
 

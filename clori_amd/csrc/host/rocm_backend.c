@@ -3,8 +3,10 @@
  * (src/backend/cuda/backend.c:836-1100,1561-1789): the opener binds the runtime, takes
  * the device, creates the launch stream, admits the kernel bundle and publishes READY;
  * without a bundle it publishes CONTEXT_READY and every operation variant refuses. */
+#define _GNU_SOURCE /* dladdr */
 #include "rocm_state.h"
 
+#include <dlfcn.h>
 #include <stdlib.h>
 #include <string.h>
 
@@ -502,6 +504,40 @@ static int parse_device(const char *device, int *index)
     return 1;
 }
 
+/* The fixed device array of the entry point that allocates nothing lives in a companion
+ * object that is linked against the HIP runtime; this library is not, so that it loads (and
+ * answers "unsupported") on a machine without the runtime.  The companion is looked up beside
+ * this library and only when the runtime in use is the real one: under a substituted runtime
+ * (YVEX_TEST_ROCM_DRIVER_LIBRARY) no second runtime is brought into the process.  Its absence
+ * only disables that entry point. */
+static void scratch_companion_resolve(yvex_rocm_backend_state *state)
+{
+    static void *companion;
+    const char *override = getenv("YVEX_TEST_ROCM_DRIVER_LIBRARY");
+    yvex_rocm_static_scratch_resolve_fn resolve;
+    Dl_info self;
+    char path[4096];
+    const char *slash;
+    size_t directory;
+    state->static_scratch = NULL;
+    state->static_scratch_error = 0;
+    if (override && *override) return;
+    if (!companion) {
+        if (!dladdr((void *)&scratch_companion_resolve, &self) || !self.dli_fname) return;
+        slash = strrchr(self.dli_fname, '/');
+        directory = slash ? (size_t)(slash - self.dli_fname) + 1u : 0u;
+        if (directory + sizeof(YVEX_ROCM_SCRATCH_LIBRARY) > sizeof(path)) return;
+        memcpy(path, self.dli_fname, directory);
+        memcpy(path + directory, YVEX_ROCM_SCRATCH_LIBRARY, sizeof(YVEX_ROCM_SCRATCH_LIBRARY));
+        /* stays mapped for the life of the process, like the runtime itself */
+        companion = dlopen(path, RTLD_NOW | RTLD_LOCAL);
+        if (!companion) return;
+    }
+    resolve = (yvex_rocm_static_scratch_resolve_fn)dlsym(companion, YVEX_ROCM_SCRATCH_RESOLVE_SYMBOL);
+    if (resolve)
+        (void)resolve(state->device_index, &state->static_scratch, &state->static_scratch_error);
+}
+
 int yvex_backend_open_rocm_impl(yvex_backend **out, const char *device,
                                 unsigned long long memory_limit_bytes, yvex_error *err)
 {
@@ -591,8 +627,7 @@ int yvex_backend_open_rocm_impl(yvex_backend **out, const char *device,
 
     /* the fixed scratch of the entry point that allocates nothing: resolved here, once per
      * device, with the device current; its absence only disables that entry point */
-    (void)yvex_rocm_static_scratch_resolve(state->device_index, &state->static_scratch,
-                                           &state->static_scratch_error);
+    scratch_companion_resolve(state);
 
     backend->device_info.kind = YVEX_BACKEND_KIND_ROCM;
     backend->device_info.device_index = state->device_index;

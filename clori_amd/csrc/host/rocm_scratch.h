@@ -13,11 +13,17 @@ enum {
     YVEX_ROCM_SCRATCH_UNAVAILABLE = 2
 };
 
+#define YVEX_ROCM_SCRATCH_LIBRARY "libyvex_rocm_scratch.so"
+#define YVEX_ROCM_SCRATCH_RESOLVE_SYMBOL "yvex_rocm_static_scratch_resolve"
+
 #ifdef __cplusplus
 extern "C" {
 #endif
-/* Device address of the scratch array on `device` (resolved on the first call for that
- * device, cached afterwards).  hip_error receives the runtime's code when unavailable. */
+/* Exported by the companion object (rocm_scratch.hip), the only object of this library that is
+ * linked against the HIP runtime: device address of the scratch array on `device` (resolved on
+ * the first call for that device, cached afterwards).  hip_error receives the runtime's code
+ * when unavailable. */
+typedef int (*yvex_rocm_static_scratch_resolve_fn)(int device, void **address, int *hip_error);
 int yvex_rocm_static_scratch_resolve(int device, void **address, int *hip_error);
 #ifdef __cplusplus
 }

@@ -136,7 +136,8 @@ typedef struct {
 } yvex_rocm_prefill_params;
 
 /* Absorbed-latent MLA decode, split over the context.  A chunk spans at most
- * YVEX_ROCM_MLA_MAX_CHUNK_PAGES pages (the kernel keeps their ids in LDS). */
+ * YVEX_ROCM_MLA_MAX_CHUNK_PAGES pages (a bound of the host's partition; the kernel reads the
+ * page ids as it goes). */
 #define YVEX_ROCM_MLA_MAX_CHUNK_PAGES 256
 typedef struct {
     const uint16_t *q;      /* [batch][heads][key_dim] */

@@ -53,6 +53,8 @@
 // puts its counter back to zero.
 // yvex_rocm_decode_merge is the stand-alone merge used by the per-chunk MLA path.
 #include "mfma.h"
+#include "device_scope.h"
+#include "merge_rows.h"
 
 #include "../kernel_params.h"
 
@@ -63,33 +65,6 @@ constexpr int kPageTokens = 16;
 
 
 __device__ inline void flag(int32_t *status, int code) { atomicCAS(status, 0, code); }
-
-// 16 / 8 bytes to global memory, visible device-wide once the store has completed: the
-// write-through form (sc1) the memory model uses for device-scope atomic stores on this
-// multi-XCD part.  Plain stores would sit in the XCD's L2 until a write-back.
-__device__ inline void store_b64_device(void *p, float a, float b)
-{
-    typedef float floatx2 __attribute__((ext_vector_type(2)));
-    const floatx2 v = {a, b};
-    __hip_atomic_store(reinterpret_cast<uint64_t *>(p), __builtin_bit_cast(uint64_t, v),
-                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-// The matching load: sees the write-through stores of the other XCDs without an L2
-// invalidate.
-__device__ inline void load_b64_device(const void *p, float &a, float &b)
-{
-    typedef float floatx2 __attribute__((ext_vector_type(2)));
-    const floatx2 v = __builtin_bit_cast(
-        floatx2, __hip_atomic_load(reinterpret_cast<const uint64_t *>(p), __ATOMIC_RELAXED,
-                                   __HIP_MEMORY_SCOPE_AGENT));
-    a = v.x;
-    b = v.y;
-}
-__device__ inline void store_b128_device(void *p, floatx4 v)
-{
-    store_b64_device(p, v[0], v[1]);
-    store_b64_device(reinterpret_cast<float *>(p) + 2, v[2], v[3]);
-}
 
 typedef __attribute__((address_space(3))) short4v lds_short4;
 // LDS staging of a token-major V tile: row r (256 bytes) keeps its 16-byte chunk c at
@@ -518,7 +493,7 @@ struct Decoder {
                 }
             }
         }
-        if (MERGE) __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+        if (MERGE) stores_completed();
     }
 
     // Log-sum-exp merge of the partials that waves w_first..w_last left for one segment, in
@@ -687,7 +662,7 @@ struct Decoder {
                         __hip_atomic_store(arrivals, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     // no cache invalidate: the merge reads with device-scope loads; this only
                     // keeps the compiler from moving them above the count
-                    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+                    loads_ordered();
                     merge_segment(session, kv_head, seg_begin, per_wave, w_first, w_last);
                 }
             }
@@ -786,7 +761,7 @@ struct Decoder {
         }
         if (whole) return;
         // every thread's stores have completed before the team is counted in
-        __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+        stores_completed();
         __syncthreads();
         uint32_t *last = reinterpret_cast<uint32_t *>(parts);  // the LDS parts are done with
         if (threadIdx.x == 0u) {
@@ -802,7 +777,7 @@ struct Decoder {
         // the last team merges the segment's parts in team order; every load of a thread is
         // independent of the others (teams past the end alias the last one with weight
         // zero): one memory round trip per kTeamsPerTrip teams
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+        loads_ordered();
         constexpr uint32_t kTeamsPerTrip = 16u;
         for (uint32_t at = threadIdx.x; at < values; at += 64u * kTeam) {
             const uint32_t hh = at / kHeadDim, d = at % kHeadDim;
@@ -977,59 +952,21 @@ __device__ __forceinline__ void decode_merge_rows(const yvex_rocm_decode_merge_p
     const uint32_t chunks = own + extra, skip = p.max_chunks - own;
     const uint64_t base =
         ((uint64_t)session * (p.max_chunks + (p.extra_context ? p.extra_max_chunks : 0u))) * p.query_heads + head;
-    // Sixteen chunks per trip, every load of a trip independent of the others (indices past
-    // the end alias the last chunk with weight zero): one memory round trip per trip, which
-    // is what keeps this pass in the microsecond range.
-    float top = -INFINITY, total = 0.f, acc[8];
-#pragma unroll
-    for (int i = 0; i < 8; ++i) acc[i] = 0.f;
-    for (uint32_t c0 = 0; c0 < chunks; c0 += 16u) {
-        float m[16], l[16];
-        u32x4 row[16];
-#pragma unroll
-        for (int j = 0; j < 16; ++j) {
-            const uint32_t c = min(c0 + (uint32_t)j, chunks - 1u);
+    float top, total, acc[8];
+    merge_chunk_rows(
+        chunks,
+        [&](uint32_t c, float &m, float &l) {
             const uint64_t slot = base + (uint64_t)(c < own ? c : c + skip) * p.query_heads;
-            m[j] = p.part_ml[slot * 2];
-            l[j] = p.part_ml[slot * 2 + 1];
-            row[j] = load_b128(p.part_acc + slot * p.head_dim + lane * 8u);
-        }
-        float trip = -INFINITY;
-#pragma unroll
-        for (int j = 0; j < 16; ++j) {
-            if (c0 + (uint32_t)j >= chunks) m[j] = -INFINITY;
-            trip = fmaxf(trip, m[j]);
-        }
-        const float m_new = fmaxf(top, trip);
-        const float keep = fast_exp2(top - m_new);  // 0 on the first trip (top = -inf)
-        total *= keep;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) acc[i] *= keep;
-#pragma unroll
-        for (int j = 0; j < 16; ++j) {
-            const float w = fast_exp2(m[j] - m_new);
-            total += w * l[j];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                acc[2 * i + 0] += w * bf16_to_f32((uint16_t)(row[j][i] & 0xffffu));
-                acc[2 * i + 1] += w * bf16_to_f32((uint16_t)(row[j][i] >> 16));
-            }
-        }
-        top = m_new;
-    }
+            m = p.part_ml[slot * 2];
+            l = p.part_ml[slot * 2 + 1];
+        },
+        [&](uint32_t c) {
+            const uint64_t slot = base + (uint64_t)(c < own ? c : c + skip) * p.query_heads;
+            return load_b128(p.part_acc + slot * p.head_dim + lane * 8u);
+        },
+        top, total, acc);
     bool bad = false;
-    if (p.sinks) {
-        // the head's sink logit joins the softmax with a zero value row
-        // (src/graph/core.c:471-508): it only enlarges the denominator
-        const float sink = p.sinks[head] * 1.4426950408889634f;  // log2 units, as the maxima
-        bad |= !isfinite(sink);
-        const float m_new = fmaxf(top, sink);
-        const float keep = fast_exp2(top - m_new);
-        total = total * keep + fast_exp2(sink - m_new);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) acc[i] *= keep;
-        top = m_new;
-    }
+    if (p.sinks) bad |= !merge_sink(p.sinks[head], top, total, acc);
     const float inv = 1.0f / total;
     // Inverse rotation of the rope lanes (src/graph/core.c:499-507): the row is rounded to
     // bf16, its last rope_dims lanes are turned back by the token position in adjacent pairs,

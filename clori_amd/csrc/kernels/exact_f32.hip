@@ -8,6 +8,8 @@
 // kernels are the throughput path and are never substituted for these.
 #include <hip/hip_runtime.h>
 
+#include "device_scope.h"
+
 #include "../kernel_params.h"
 
 namespace {
@@ -401,7 +403,7 @@ __device__ __forceinline__ void gqa_f32_split(const yvex_rocm_gqa_f32_params &p,
             store_f64_device(p.part_ml + slot * 2u, top);
             store_f64_device(p.part_ml + slot * 2u + 1u, total);
         }
-        __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this thread's stores have completed
+        stores_completed();  // this thread's stores have completed, and nothing moves across
         __syncthreads();
         uint32_t *last = reinterpret_cast<uint32_t *>(team_lds);  // the LDS parts are done with
         if (t == 0u) {
@@ -413,7 +415,7 @@ __device__ __forceinline__ void gqa_f32_split(const yvex_rocm_gqa_f32_params &p,
         }
         __syncthreads();
         if (*last == 0u) return;
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+        loads_ordered();
         top = -INFINITY;
         total = 0.0;
         o = 0.0;

@@ -129,3 +129,34 @@ def test_benchmark_summary_refuses_bad_samples():
         with pytest.raises(K.YvexError) as e:
             K.benchmark_summarize(bad)
         assert e.value.code == B.YVEX_ERR_BOUNDS and e.value.where == "runtime.benchmark"
+
+
+def test_library_loads_and_refuses_without_any_hip_runtime():
+    """The library reaches the HIP runtime through dlopen only (no DT_NEEDED entry for it), so on
+    a machine without the runtime the program still starts, the backend answers "unsupported"
+    and the commands exit with 5 (tests/test_cuda_failclosed.sh:46-79 of the reference asks the
+    same of the CUDA arm).  Here: no library search path at all and a runtime name that does
+    not exist."""
+    library = os.path.join(ROOT, "clori_amd", "libyvex_rocm.so")
+    needed = subprocess.run(["readelf", "-d", library], capture_output=True, text=True, check=True).stdout
+    needed = [line for line in needed.splitlines() if "(NEEDED)" in line]
+    assert needed and not any("hip" in line.lower() or "hsa" in line.lower() for line in needed), needed
+    bare = {"LD_LIBRARY_PATH": "", "PATH": os.environ.get("PATH", "")}
+    for arguments in (("inspect", "backend", "rocm"), ("inspect", "rocm")):
+        env = dict(bare, YVEX_TEST_ROCM_DRIVER_LIBRARY="/nonexistent/libamdhip64.so")
+        done = subprocess.run([PROGRAM, *arguments], env=env, capture_output=True, text=True, timeout=60)
+        assert done.returncode == 5, (arguments, done.stdout, done.stderr)
+        assert "unsupported" in done.stdout or "unavailable" in done.stdout
+
+
+def test_scratch_companion_is_the_only_object_linked_against_the_runtime():
+    """The fixed device array of the entry point that allocates nothing sits in its own shared
+    object beside the library; that object, and nothing else, names the HIP runtime."""
+    companion = os.path.join(ROOT, "clori_amd", "libyvex_rocm_scratch.so")
+    if not os.path.exists(companion):
+        pytest.skip("the companion object is not built")
+    needed = subprocess.run(["readelf", "-d", companion], capture_output=True, text=True, check=True).stdout
+    assert "libamdhip64" in needed
+    symbols = subprocess.run(["nm", "-D", "--defined-only", companion], capture_output=True, text=True,
+                             check=True).stdout
+    assert "yvex_rocm_static_scratch_resolve" in symbols
