@@ -81,6 +81,20 @@ class Tensor:
         err = B.Error()
         _check(lib().yvex_backend_tensor_zero(self.backend.handle, self.handle, C.byref(err)), err)
 
+    def copy_from_async(self, source):
+        """The same copy put on the backend's stream and not waited for
+        (yvex_backend_tensor_copy_async)."""
+        err = B.Error()
+        _check(lib().yvex_backend_tensor_copy_async(self.backend.handle, self.handle, source.handle,
+                                                    C.byref(err)), err)
+
+    def copy_from_shared_async(self, source):
+        """Copy from a tensor of another backend with the same physical owner, ordered by
+        events between the two streams (yvex_backend_tensor_copy_shared_async)."""
+        err = B.Error()
+        _check(lib().yvex_backend_tensor_copy_shared_async(self.backend.handle, self.handle,
+                                                           source.handle, C.byref(err)), err)
+
     def copy_from(self, source):
         """Device-to-device copy of a tensor with the same descriptor."""
         err = B.Error()
@@ -135,11 +149,17 @@ class Tensor:
 class Backend:
     """struct yvex_backend of kind ROCM."""
 
-    def __init__(self, device=None, memory_limit_bytes=0, kind=B.KIND_ROCM):
+    def __init__(self, device=None, memory_limit_bytes=0, kind=B.KIND_ROCM, shared_with=None):
+        """shared_with: a primary Backend; the new one is a session backend on its device
+        (yvex_backend_open_shared_rocm)."""
         self.handle = C.c_void_p()
-        options = B.BackendOptions(kind, device.encode() if device else None, memory_limit_bytes)
         err = B.Error()
-        _check(lib().yvex_backend_open(C.byref(self.handle), C.byref(options), C.byref(err)), err)
+        if shared_with is not None:
+            _check(lib().yvex_backend_open_shared_rocm(C.byref(self.handle), shared_with.handle,
+                                                       memory_limit_bytes, C.byref(err)), err)
+        else:
+            options = B.BackendOptions(kind, device.encode() if device else None, memory_limit_bytes)
+            _check(lib().yvex_backend_open(C.byref(self.handle), C.byref(options), C.byref(err)), err)
         self.tensors = []
 
     # -- lifecycle --------------------------------------------------------

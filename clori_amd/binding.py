@@ -291,7 +291,9 @@ EXPORTED_SYMBOLS = [
     "yvex_backend_tensor_reserve",
     "yvex_backend_tensor_commit_range", "yvex_backend_tensor_decommit", "yvex_device_tensor_name", "yvex_device_tensor_bytes",
     "yvex_device_tensor_is_written", "yvex_backend_tensor_write", "yvex_backend_tensor_read",
-    "yvex_backend_tensor_zero", "yvex_backend_tensor_copy", "yvex_backend_tensor_owned_by",
+    "yvex_backend_tensor_zero", "yvex_backend_tensor_copy", "yvex_backend_tensor_copy_async",
+    "yvex_backend_tensor_copy_shared_async", "yvex_backend_open_shared_rocm",
+    "yvex_backend_tensor_owned_by",
     "yvex_backend_tensor_f32_subview", "yvex_backend_sync", "yvex_backend_supports",
     "yvex_backend_capability_name", "yvex_backend_query_capability",
     "yvex_backend_operation_variant_name", "yvex_backend_capability_state_name",
@@ -357,6 +359,9 @@ def load(path=None):
     lib.yvex_backend_tensor_read.argtypes = [vp, TensorP, vp, ull, ErrorP]
     lib.yvex_backend_tensor_zero.argtypes = [vp, TensorP, ErrorP]
     lib.yvex_backend_tensor_copy.argtypes = [vp, TensorP, TensorP, ErrorP]
+    lib.yvex_backend_tensor_copy_async.argtypes = [vp, TensorP, TensorP, ErrorP]
+    lib.yvex_backend_tensor_copy_shared_async.argtypes = [vp, TensorP, TensorP, ErrorP]
+    lib.yvex_backend_open_shared_rocm.argtypes = [C.POINTER(vp), vp, C.c_ulonglong, ErrorP]
     lib.yvex_backend_tensor_owned_by.argtypes = [vp, TensorP]
     lib.yvex_backend_tensor_f32_subview.argtypes = [TensorP, ull, ull, TensorP]
     lib.yvex_backend_sync.argtypes = [vp, ErrorP]

@@ -125,27 +125,73 @@ int yvex_backend_rocm_context_available(void)
 
 int yvex_backend_rocm_available(void) { return yvex_backend_rocm_context_available(); }
 
-/* src/backend/core.c:331-356: mark CLOSING (sticky) and FAILED so nothing dispatches. */
+/* A primary backend counts the session backends opened on it in the low bits of its lifecycle
+ * word (src/backend/core.c:305-356, src/backend/cuda/backend.c:1598-1623). */
+int yvex_backend_shared_owner_acquire(yvex_backend *owner, yvex_error *err)
+{
+    static const char where[] = "backend.shared.acquire";
+    unsigned long long seen;
+    if (!owner || owner->resource_owner != owner || owner->status == YVEX_BACKEND_STATUS_FAILED)
+        return refuse(err, YVEX_ERR_STATE, where, "one live primary backend resource owner is required");
+    seen = atomic_load_explicit(&owner->lifecycle, memory_order_acquire);
+    do {
+        if ((seen & YVEX_BACKEND_LIFECYCLE_CLOSING) != 0ull ||
+            (seen & YVEX_BACKEND_LIFECYCLE_CHILD_MASK) == YVEX_BACKEND_LIFECYCLE_CHILD_MASK)
+            return refuse(err, YVEX_ERR_STATE, where, "backend resource owner is closing or saturated");
+    } while (!atomic_compare_exchange_weak_explicit(&owner->lifecycle, &seen, seen + 1ull,
+                                                    memory_order_acq_rel, memory_order_acquire));
+    yvex_error_clear(err);
+    return YVEX_OK;
+}
+
+static int shared_owner_release(yvex_backend *owner, yvex_error *err)
+{
+    static const char where[] = "backend.shared.release";
+    unsigned long long seen;
+    if (!owner) return refuse(err, YVEX_ERR_STATE, where, "backend resource owner is required");
+    seen = atomic_load_explicit(&owner->lifecycle, memory_order_acquire);
+    do {
+        if ((seen & YVEX_BACKEND_LIFECYCLE_CHILD_MASK) == 0ull)
+            return refuse(err, YVEX_ERR_STATE, where, "backend shared-resource lease is not registered");
+    } while (!atomic_compare_exchange_weak_explicit(&owner->lifecycle, &seen, seen - 1ull,
+                                                    memory_order_acq_rel, memory_order_acquire));
+    yvex_error_clear(err);
+    return YVEX_OK;
+}
+
+/* src/backend/core.c:330-356: CLOSING is sticky and the backend FAILED from here on, so nothing
+ * dispatches; a primary backend with open session backends is not discharged yet. */
 static int close_admit(yvex_backend *backend, yvex_error *err)
 {
-    atomic_fetch_or_explicit(&backend->lifecycle, YVEX_BACKEND_LIFECYCLE_CLOSING,
-                             memory_order_acq_rel);
+    const unsigned long long before = atomic_fetch_or_explicit(
+        &backend->lifecycle, YVEX_BACKEND_LIFECYCLE_CLOSING, memory_order_acq_rel);
     backend->status = YVEX_BACKEND_STATUS_FAILED;
+    if ((before & YVEX_BACKEND_LIFECYCLE_CHILD_MASK) != 0ull)
+        return refuse(err, YVEX_ERR_STATE, "backend.close.admit",
+                      "backend context still has live shared children");
     yvex_error_clear(err);
     return YVEX_OK;
 }
 
 /* src/backend/core.c:362-416: the owner pointer is nulled only after the arm
- * discharged its resources; a failed discharge keeps the handle for a retry. */
+ * discharged its resources; a failed discharge keeps the handle for a retry.  A session
+ * backend gives its lease back last. */
 int yvex_backend_close_checked(yvex_backend **backend_ptr, yvex_error *err)
 {
-    yvex_backend *backend;
+    yvex_backend *backend, *owner;
     int rc;
     if (!backend_ptr || !*backend_ptr) {
         yvex_error_clear(err);
         return YVEX_OK;
     }
     backend = *backend_ptr;
+    owner = backend->resource_owner;
+    if (backend->shared_owner_registered &&
+        (!owner || owner == backend ||
+         (atomic_load_explicit(&owner->lifecycle, memory_order_acquire) &
+          YVEX_BACKEND_LIFECYCLE_CHILD_MASK) == 0ull))
+        return refuse(err, YVEX_ERR_STATE, "backend.close",
+                      "shared backend owner registration is inconsistent");
     rc = close_admit(backend, err);
     if (rc != YVEX_OK) return rc;
     if (backend->vtable && backend->vtable->close) {
@@ -156,6 +202,18 @@ int yvex_backend_close_checked(yvex_backend **backend_ptr, yvex_error *err)
             if (err) *err = cleanup;
             if (backend->impl) return rc;
         }
+    }
+    if (backend->shared_owner_registered) {
+        yvex_error cleanup;
+        int lease_rc;
+        yvex_error_clear(&cleanup);
+        lease_rc = shared_owner_release(owner, &cleanup);
+        if (lease_rc != YVEX_OK) {
+            if (err) *err = cleanup;
+            return lease_rc;
+        }
+        backend->shared_owner_registered = 0;
+        backend->resource_owner = NULL;
     }
     free(backend);
     *backend_ptr = NULL;
@@ -458,6 +516,48 @@ int yvex_backend_tensor_copy(yvex_backend *backend, yvex_device_tensor *dst,
 {
     TENSOR_DISPATCH("yvex_backend_tensor_copy", backend && dst && src, tensor_copy,
                     backend->vtable->tensor_copy(backend, dst, src, err));
+}
+
+/* src/backend/core.c:822-840: lifecycle, then ownership and descriptors, then the slot. */
+int yvex_backend_tensor_copy_async(yvex_backend *backend, yvex_device_tensor *destination,
+                                   const yvex_device_tensor *source, yvex_error *err)
+{
+    static const char where[] = "backend.tensor.copy-async";
+    int rc = backend_dispatch_admit(backend, where, err);
+    if (rc == YVEX_OK) rc = yvex_backend_tensor_copy_validate(backend, destination, source, where, err);
+    if (rc != YVEX_OK) return rc;
+    if (!backend->vtable || !backend->vtable->tensor_copy_async)
+        return refuse(err, YVEX_ERR_UNSUPPORTED, where,
+                      "backend does not support asynchronous tensor copy");
+    return backend->vtable->tensor_copy_async(backend, destination, source, err);
+}
+
+static yvex_backend *physical_owner(yvex_backend *backend)
+{
+    return backend->resource_owner ? backend->resource_owner : backend;
+}
+
+/* src/backend/core.c:842-874: the executor owns the destination, the source belongs to a
+ * backend with the same physical owner, same descriptors, source written. */
+int yvex_backend_tensor_copy_shared_async(yvex_backend *executor, yvex_device_tensor *destination,
+                                          const yvex_device_tensor *source, yvex_error *err)
+{
+    static const char where[] = "backend.tensor.copy-shared";
+    int rc;
+    if (!executor || !destination || !source || !destination->owner || !source->owner)
+        return refuse(err, YVEX_ERR_INVALID_ARG, where, "executor and two owned tensors are required");
+    rc = backend_dispatch_admit(executor, where, err);
+    if (rc == YVEX_OK) rc = backend_dispatch_admit(source->owner, where, err);
+    if (rc != YVEX_OK) return rc;
+    if (destination->owner != executor ||
+        physical_owner(source->owner) != physical_owner(executor) ||
+        !same_shape(destination, source) || !source->is_written)
+        return refuse(err, YVEX_ERR_INVALID_ARG, where,
+                      "same-physical-owner initialized tensor shapes are required");
+    if (!executor->vtable || !executor->vtable->tensor_copy_shared_async)
+        return refuse(err, YVEX_ERR_UNSUPPORTED, where,
+                      "backend does not support cross-stream tensor copy");
+    return executor->vtable->tensor_copy_shared_async(executor, destination, source, err);
 }
 
 int yvex_backend_sync(yvex_backend *backend, yvex_error *err)

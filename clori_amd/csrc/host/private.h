@@ -34,6 +34,10 @@ typedef struct yvex_backend_vtable {
     int (*tensor_zero)(yvex_backend *, yvex_device_tensor *, yvex_error *);
     int (*tensor_copy)(yvex_backend *, yvex_device_tensor *, const yvex_device_tensor *,
                        yvex_error *);
+    int (*tensor_copy_async)(yvex_backend *, yvex_device_tensor *, const yvex_device_tensor *,
+                             yvex_error *);
+    int (*tensor_copy_shared_async)(yvex_backend *, yvex_device_tensor *,
+                                    const yvex_device_tensor *, yvex_error *);
     int (*sync)(yvex_backend *, yvex_error *);
     int (*bandwidth_probe)(yvex_backend *, yvex_backend_bandwidth_evidence *, yvex_error *);
     int (*query_capability)(const yvex_backend *, yvex_backend_operation_variant,
@@ -55,15 +59,18 @@ struct yvex_backend {
     yvex_backend_device_info device_info;
     char device_name_storage[128];
     void *impl;
-    _Atomic unsigned long long lifecycle;
+    struct yvex_backend *resource_owner; /* itself for a primary backend, the primary for a session backend */
+    _Atomic unsigned long long lifecycle; /* CLOSING bit, below it the count of open session backends */
     unsigned long long tensor_id_next;
     const yvex_device_tensor *workspace_device_tensor;
     unsigned long long workspace_device_address, workspace_bytes, workspace_cursor;
     unsigned long long workspace_peak, workspace_generation;
+    int shared_owner_registered; /* this session backend holds a lease on resource_owner */
     int virtual_tensor_ready; /* src/backend/private.h:109 */
 };
 
 #define YVEX_BACKEND_LIFECYCLE_CLOSING (1ull << 63)
+#define YVEX_BACKEND_LIFECYCLE_CHILD_MASK (YVEX_BACKEND_LIFECYCLE_CLOSING - 1ull)
 
 static inline int backend_cleanup_only(const yvex_backend *backend)
 {
@@ -121,6 +128,9 @@ int yvex_core_u64_mul(unsigned long long left, unsigned long long right,
 void yvex_core_text_copy(char *destination, size_t capacity, const char *source);
 void yvex_error_setf(yvex_error *err, yvex_status code, const char *where, const char *fmt, ...);
 unsigned long long yvex_dtype_element_bytes(yvex_dtype dtype);
+
+/* core.c: lease of a session backend on its primary (src/backend/cuda/backend.c:1598-1623) */
+int yvex_backend_shared_owner_acquire(yvex_backend *owner, yvex_error *err);
 
 /* core.c: shared validators (src/backend/core.c:1143-1171,1224-1290,1547-1616) */
 int yvex_backend_memory_can_add(const yvex_backend *backend, unsigned long long bytes,

@@ -221,6 +221,88 @@ static int rocm_tensor_copy(yvex_backend *backend, yvex_device_tensor *dst,
     return YVEX_OK;
 }
 
+/* src/backend/cuda/backend.c:1159-1191: the copy goes on the launch stream and is not waited
+ * for; whatever is enqueued behind it sees the bytes. */
+static int rocm_tensor_copy_async(yvex_backend *backend, yvex_device_tensor *dst,
+                                  const yvex_device_tensor *src, yvex_error *err)
+{
+    static const char where[] = "runtime.state.residency.copy";
+    yvex_rocm_backend_state *state = yvex_rocm_state(backend);
+    int rc = yvex_backend_tensor_copy_validate(backend, dst, src, where, err);
+    if (rc != YVEX_OK) return rc;
+    if (!state || backend->kind != YVEX_BACKEND_KIND_ROCM)
+        return refuse(err, YVEX_ERR_INVALID_ARG, where, "ROCm state residency requires a ROCm backend");
+    if (!yvex_rocm_tensor_backed(dst) || !yvex_rocm_tensor_backed(src))
+        return refuse(err, YVEX_ERR_STATE, where, kUnbacked);
+    rc = yvex_rocm_require_capability(backend, YVEX_BACKEND_VARIANT_TENSOR_COPY, where, err);
+    if (rc != YVEX_OK) return rc;
+    rc = yvex_rocm_status(&state->driver,
+                          state->driver.hipMemcpyAsync(dst->data, src->data, (size_t)src->bytes,
+                                                       hipMemcpyDeviceToDevice, state->stream),
+                          where, err);
+    if (rc != YVEX_OK) return rc;
+    dst->is_written = src->is_written;
+    yvex_error_clear(err);
+    return YVEX_OK;
+}
+
+/* src/backend/cuda/backend.c:1194-1265: the source belongs to another backend of the same
+ * device.  An event recorded on the source's stream makes the copy wait for whatever produces
+ * the source; an event recorded behind the copy makes the source's stream wait before it
+ * overwrites it.  Both events are released at once: the runtime keeps what a recorded event
+ * needs until the waits that name it have passed. */
+static int rocm_tensor_copy_shared_async(yvex_backend *backend, yvex_device_tensor *dst,
+                                         const yvex_device_tensor *src, yvex_error *err)
+{
+    static const char where[] = "backend.tensor.copy-shared";
+    yvex_rocm_backend_state *state = yvex_rocm_state(backend);
+    yvex_rocm_backend_state *source_state = src && src->owner ? yvex_rocm_state(src->owner) : NULL;
+    hipEvent_t ready = NULL, consumed = NULL;
+    int rc = YVEX_OK, cleanup;
+    if (!state || !source_state || !dst || !state->stream || !source_state->stream)
+        return refuse(err, YVEX_ERR_UNSUPPORTED, where, "ROCm cross-stream event ordering is unavailable");
+    if (!yvex_rocm_tensor_backed(dst) || !yvex_rocm_tensor_backed(src))
+        return refuse(err, YVEX_ERR_STATE, where, kUnbacked);
+    if (source_state->stream != state->stream) {
+        rc = yvex_rocm_status(&state->driver, state->driver.hipEventCreate(&ready), where, err);
+        if (rc == YVEX_OK)
+            rc = yvex_rocm_status(&state->driver, state->driver.hipEventCreate(&consumed), where, err);
+        if (rc == YVEX_OK)
+            rc = yvex_rocm_status(&state->driver,
+                                  state->driver.hipEventRecord(ready, source_state->stream), where, err);
+        if (rc == YVEX_OK)
+            rc = yvex_rocm_status(&state->driver,
+                                  state->driver.hipStreamWaitEvent(state->stream, ready, 0u), where, err);
+    }
+    if (rc == YVEX_OK)
+        rc = yvex_rocm_status(&state->driver,
+                              state->driver.hipMemcpyAsync(dst->data, src->data, (size_t)src->bytes,
+                                                           hipMemcpyDeviceToDevice, state->stream),
+                              where, err);
+    if (rc == YVEX_OK && consumed) {
+        rc = yvex_rocm_status(&state->driver, state->driver.hipEventRecord(consumed, state->stream),
+                              where, err);
+        if (rc == YVEX_OK)
+            rc = yvex_rocm_status(&state->driver,
+                                  state->driver.hipStreamWaitEvent(source_state->stream, consumed, 0u),
+                                  where, err);
+    }
+    if (consumed) {
+        cleanup = yvex_rocm_status(&state->driver, state->driver.hipEventDestroy(consumed), where,
+                                   rc == YVEX_OK ? err : NULL);
+        if (rc == YVEX_OK) rc = cleanup;
+    }
+    if (ready) {
+        cleanup = yvex_rocm_status(&state->driver, state->driver.hipEventDestroy(ready), where,
+                                   rc == YVEX_OK ? err : NULL);
+        if (rc == YVEX_OK) rc = cleanup;
+    }
+    if (rc != YVEX_OK) return rc;
+    dst->is_written = src->is_written;
+    yvex_error_clear(err);
+    return YVEX_OK;
+}
+
 /* Synchronise; in DEFERRED completion mode this is also where the device status word of
  * the operations enqueued since the last check is read and reported. */
 static int rocm_sync(yvex_backend *backend, yvex_error *err)
@@ -484,6 +566,8 @@ static const yvex_backend_vtable rocm_vtable = {
     .tensor_read = rocm_tensor_read,
     .tensor_zero = rocm_tensor_zero,
     .tensor_copy = rocm_tensor_copy,
+    .tensor_copy_async = rocm_tensor_copy_async,
+    .tensor_copy_shared_async = rocm_tensor_copy_shared_async,
     .sync = rocm_sync,
     .bandwidth_probe = rocm_bandwidth_probe,
     .query_capability = yvex_rocm_query_capability,
@@ -538,8 +622,10 @@ static void scratch_companion_resolve(yvex_rocm_backend_state *state)
         (void)resolve(state->device_index, &state->static_scratch, &state->static_scratch_error);
 }
 
-int yvex_backend_open_rocm_impl(yvex_backend **out, const char *device,
-                                unsigned long long memory_limit_bytes, yvex_error *err)
+/* `owner` NULL: a primary backend on the device named by `device`.  Otherwise a session
+ * backend on the owner's device; the caller holds the lease on the owner. */
+static int rocm_open(yvex_backend **out, const char *device, unsigned long long memory_limit_bytes,
+                     yvex_backend *owner, yvex_error *err)
 {
     static const char where[] = "yvex_backend_open_rocm";
     yvex_backend *backend;
@@ -566,9 +652,15 @@ int yvex_backend_open_rocm_impl(yvex_backend **out, const char *device,
     state->kernel_bundle_reason = YVEX_BACKEND_CAPABILITY_REASON_KERNEL_BUNDLE_ABSENT;
     state->kernel_bundle_failure_variant = YVEX_BACKEND_VARIANT_COUNT;
 
-    rc = parse_device(device, &state->device_index)
-             ? YVEX_OK
-             : refuse(err, YVEX_ERR_INVALID_ARG, where, "device must be a non-negative index");
+    backend->resource_owner = owner ? owner : backend;
+    if (owner) {
+        state->device_index = yvex_rocm_state(owner)->device_index;
+        rc = YVEX_OK;
+    } else {
+        rc = parse_device(device, &state->device_index)
+                 ? YVEX_OK
+                 : refuse(err, YVEX_ERR_INVALID_ARG, where, "device must be a non-negative index");
+    }
     if (rc == YVEX_OK) rc = yvex_rocm_driver_load(&state->driver, err);
     if (rc == YVEX_OK && state->driver.hipInit(0u) != hipSuccess)
         rc = refuse(err, YVEX_ERR_UNSUPPORTED, where, "HIP runtime initialisation failed");
@@ -669,6 +761,35 @@ int yvex_backend_open_rocm_impl(yvex_backend **out, const char *device,
                             sizeof(state->kernel_bundle_rejection), admit.message);
     *out = backend;
     yvex_error_clear(err);
+    return YVEX_OK;
+}
+
+int yvex_backend_open_rocm_impl(yvex_backend **out, const char *device,
+                                unsigned long long memory_limit_bytes, yvex_error *err)
+{
+    return rocm_open(out, device, memory_limit_bytes, NULL, err);
+}
+
+/* src/backend/cuda/backend.c:1795-1879.  HIP has no context object to lend: what a session
+ * backend takes from its primary is the device, and the lease that keeps the primary open. */
+int yvex_backend_open_shared_rocm(yvex_backend **out, yvex_backend *context_owner,
+                                  unsigned long long memory_limit_bytes, yvex_error *err)
+{
+    static const char where[] = "rocm.shared.open";
+    int rc;
+    if (out) *out = NULL;
+    if (!out || !context_owner || context_owner->kind != YVEX_BACKEND_KIND_ROCM ||
+        context_owner->resource_owner != context_owner || !yvex_rocm_state(context_owner))
+        return refuse(err, YVEX_ERR_INVALID_ARG, where, "one owning ROCm backend is required");
+    rc = yvex_backend_shared_owner_acquire(context_owner, err);
+    if (rc != YVEX_OK) return rc;
+    rc = rocm_open(out, NULL, memory_limit_bytes, context_owner, err);
+    if (rc != YVEX_OK) {
+        /* nothing was published: give the lease back */
+        atomic_fetch_sub_explicit(&context_owner->lifecycle, 1ull, memory_order_acq_rel);
+        return rc;
+    }
+    (*out)->shared_owner_registered = 1;
     return YVEX_OK;
 }
 

@@ -20,7 +20,7 @@
     X(hipStreamCreate) X(hipStreamDestroy) X(hipStreamSynchronize) X(hipMalloc) X(hipFree) \
     X(hipMemcpyAsync) X(hipMemsetAsync) X(hipModuleLoadData) X(hipModuleUnload)          \
     X(hipModuleGetFunction) X(hipModuleLaunchKernel) X(hipEventCreate) X(hipEventDestroy) \
-    X(hipEventRecord) X(hipEventSynchronize) X(hipEventElapsedTime)                     \
+    X(hipEventRecord) X(hipEventSynchronize) X(hipEventElapsedTime) X(hipStreamWaitEvent) \
     X(hipStreamBeginCapture) X(hipStreamEndCapture) X(hipGraphInstantiate) X(hipGraphLaunch) \
     X(hipGraphExecDestroy) X(hipGraphDestroy)
 

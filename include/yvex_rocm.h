@@ -283,6 +283,30 @@ int yvex_backend_tensor_read(yvex_backend *backend, const yvex_device_tensor *te
 int yvex_backend_tensor_zero(yvex_backend *backend, yvex_device_tensor *tensor, yvex_error *err);
 int yvex_backend_tensor_copy(yvex_backend *backend, yvex_device_tensor *dst,
                              const yvex_device_tensor *src, yvex_error *err);
+/* include/yvex/internal/backend.h (dispatch src/backend/core.c:822-840, vtable slot
+ * src/backend/private.h:45-46, CUDA arm src/backend/cuda/backend.c:1159-1191): the copy is
+ * put on the backend's launch stream and not waited for, so the kernels enqueued after it see
+ * the rows without a synchronisation in between.  This is the call the session layer makes
+ * twice per token when it appends a step's keys and values to the history
+ * (src/runtime/stateful_attention.c:206,215).  Refusals in the reference's order: lifecycle
+ * (YVEX_ERR_STATE), ownership (YVEX_ERR_STATE), descriptors that differ (YVEX_ERR_BOUNDS). */
+int yvex_backend_tensor_copy_async(yvex_backend *backend, yvex_device_tensor *destination,
+                                   const yvex_device_tensor *source, yvex_error *err);
+/* src/backend/core.c:842-874, src/backend/private.h:47-48, CUDA arm
+ * src/backend/cuda/backend.c:1194-1265: copy between two backends that share one physical
+ * owner (a primary backend and the session backends opened on it), ordered by events: the
+ * executor's stream waits for the source's stream before the copy, the source's stream waits
+ * for the copy before it goes on. */
+int yvex_backend_tensor_copy_shared_async(yvex_backend *executor, yvex_device_tensor *destination,
+                                          const yvex_device_tensor *source, yvex_error *err);
+/* include/yvex/internal/backend.h:205-206 (src/backend/cuda/backend.c:1795-1879): a session
+ * backend on the device of a primary one: its own launch stream, timing events, workspace,
+ * kernel functions, arrival counters and status word, memory accounted against its own limit.
+ * The primary holds a lease per session backend and cannot be closed while one is open
+ * (YVEX_ERR_STATE from the close, the handle is retained).  The only thing backends of one
+ * device share is the fixed scratch of yvex_backend_rocm_paged_decode_execute_static. */
+int yvex_backend_open_shared_rocm(yvex_backend **out, yvex_backend *context_owner,
+                                  unsigned long long memory_limit_bytes, yvex_error *err);
 int yvex_backend_tensor_owned_by(const yvex_backend *backend, const yvex_device_tensor *tensor);
 /* src/backend/core.c:1763-1778: rank-1 F32 view of `count` elements at `offset`. */
 int yvex_backend_tensor_f32_subview(const yvex_device_tensor *source, unsigned long long offset,

@@ -172,6 +172,11 @@ hipError_t hipEventCreate(hipEvent_t *event)
 hipError_t hipEventDestroy(hipEvent_t event) { free(event); return hipSuccess; }
 hipError_t hipEventRecord(hipEvent_t event, hipStream_t stream) { (void)event; (void)stream; return hipSuccess; }
 hipError_t hipEventSynchronize(hipEvent_t event) { (void)event; return hipSuccess; }
+hipError_t hipStreamWaitEvent(hipStream_t stream, hipEvent_t event, unsigned int flags)
+{
+    (void)stream; (void)event; (void)flags; /* every stream of the stand-in runs its work at once */
+    return hipSuccess;
+}
 
 hipError_t hipEventElapsedTime(float *ms, hipEvent_t start, hipEvent_t stop)
 {

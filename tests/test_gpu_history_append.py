@@ -371,3 +371,98 @@ def test_history_append_in_the_decoder_order_of_rotary(backend, f32, d, rotary):
     assert e.value.code == B.YVEX_ERR_UNSUPPORTED
     for t in held:
         t.release()
+
+
+def test_session_layer_copy_loop_equals_the_history_writer(backend):
+    """The unchanged caller (src/runtime/stateful_attention.c:183-222): per token, one
+    asynchronous copy of the key row and one of the value row into the [K | V] history row,
+    F32 as the session layer keeps it, nothing waited for; then attention over the views.  The
+    history must equal, byte for byte, what the one-launch writer leaves (no rotary: the
+    session layer's rows arrive rotated), and the attention enqueued right behind the copies,
+    with no synchronisation in between, must equal the attention over the writer's history."""
+    rng = np.random.default_rng(314)
+    hq, hkv, d, have, tokens = 8, 2, 64, 37, 5
+    width = hkv * d
+    rows = have + tokens
+    before = rng.standard_normal((rows, 2 * width)).astype(np.float32)
+    k_new = rng.standard_normal((tokens, hkv, d)).astype(np.float32)
+    v_new = rng.standard_normal((tokens, hkv, d)).astype(np.float32)
+    q = rng.standard_normal((tokens, hq, d)).astype(np.float32)
+    tk = backend.tensor("k-new", B.DTYPE_F32, k_new.shape, k_new)
+    tv = backend.tensor("v-new", B.DTYPE_F32, v_new.shape, v_new)
+    tq = backend.tensor("q", B.DTYPE_F32, q.shape, q)
+    looped = backend.tensor("history-loop", B.DTYPE_F32, before.shape, before)
+    written = backend.tensor("history-writer", B.DTYPE_F32, before.shape, before)
+    out_loop = backend.tensor("out-loop", B.DTYPE_F32, q.shape)
+    out_writer = backend.tensor("out-writer", B.DTYPE_F32, q.shape)
+    count = (rows - 1) * 2 * width + width
+    req = backend.attention_requirement(tokens, rows, hq, hkv, d, causal=True, query_start=have,
+                                        k_stride=2 * width, v_stride=2 * width)
+
+    def views(store):
+        return (store.view(0, B.DTYPE_F32, (count,)), store.view(width * 4, B.DTYPE_F32, (count,)))
+
+    backend.set_completion_mode(B.COMPLETION_DEFERRED)
+    try:
+        row_bytes = 2 * width * 4
+        for token in range(tokens):
+            target = (have + token) * row_bytes
+            looped.view(target, B.DTYPE_F32, (width,)).copy_from_async(
+                tk.view(token * width * 4, B.DTYPE_F32, (width,)))
+            looped.view(target + width * 4, B.DTYPE_F32, (width,)).copy_from_async(
+                tv.view(token * width * 4, B.DTYPE_F32, (width,)))
+        kh, vh = views(looped)
+        backend.attention_execute(req, tq, kh, vh, out_loop)      # no wait since the copies
+        backend.sync()
+    finally:
+        backend.set_completion_mode(B.COMPLETION_IMMEDIATE)
+    kh2, vh2 = views(written)
+    backend.history_append_execute(tk, tv, kh2, vh2, have, hkv, head_dimension=d,
+                                   key_token_stride=2 * width, value_token_stride=2 * width)
+    backend.attention_execute(req, tq, kh2, vh2, out_writer)
+    want = before.copy()
+    want[have:, :width] = k_new.reshape(tokens, width)
+    want[have:, width:] = v_new.reshape(tokens, width)
+    assert np.array_equal(looped.read(), want)
+    assert np.array_equal(written.read(), want)
+    assert np.array_equal(out_loop.read(), out_writer.read())
+    rc, ref = ORACLE.gqa(q, want[:, :width].reshape(rows, hkv, d).copy(),
+                         want[:, width:].reshape(rows, hkv, d).copy(), query_start=have)[:2]
+    assert rc == 0
+    assert np.allclose(out_loop.read(), ref, rtol=2e-5, atol=2e-6)
+    for tensor in (tk, tv, tq, looped, written, out_loop, out_writer):
+        tensor.release()
+
+
+def test_session_backend_on_the_device_copies_between_streams(backend):
+    """A session backend opened on the device of the primary one
+    (yvex_backend_open_shared_rocm) runs its own kernels on its own stream; a tensor written by
+    a kernel of one is copied into the other with yvex_backend_tensor_copy_shared_async, ordered
+    by events, with no host wait between the producing kernel and the copy."""
+    from clori_amd.backend import Backend
+    rng = np.random.default_rng(271)
+    hq, hkv, d, ctx = 8, 2, 128, 900
+    q = bf16_normal(rng, (1, hq, d))
+    k, v = bf16_normal(rng, (ctx, hkv, d)), bf16_normal(rng, (ctx, hkv, d))
+    session = Backend(shared_with=backend)
+    try:
+        assert session.status == B.STATUS_READY
+        tq = session.tensor("q", B.DTYPE_BF16, q.shape, q)
+        tk = session.tensor("k", B.DTYPE_BF16, k.shape, k)
+        tv = session.tensor("v", B.DTYPE_BF16, v.shape, v)
+        produced = session.tensor("out", B.DTYPE_BF16, q.shape)
+        received = backend.tensor("received", B.DTYPE_BF16, q.shape)
+        req = session.attention_requirement(1, ctx, hq, hkv, d, causal=True, query_start=ctx - 1,
+                                            dtype=B.DTYPE_BF16, contract=B.NUMERIC_BF16_F32_ACCUMULATE)
+        session.set_completion_mode(B.COMPLETION_DEFERRED)
+        session.attention_execute(req, tq, tk, tv, produced)       # enqueued on the session's stream
+        received.copy_from_shared_async(produced)                  # primary's stream waits for it
+        got = received.read()
+        session.sync()
+        assert np.array_equal(got, produced.read())
+        rc, ref = ORACLE.gqa_bf16(q, k, v, query_start=ctx - 1)[:2]
+        assert rc == 0
+        assert_close_bf16(got, ref, "session backend")
+        received.release()
+    finally:
+        session.close()

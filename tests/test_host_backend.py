@@ -306,6 +306,110 @@ def test_tensor_lifecycle_and_accounting(fake_runtime):
         assert fake_runtime.fake_hip_live_allocations() == base + 2
 
 
+def test_async_copy_refusal_order_and_effect(fake_runtime):
+    """yvex_backend_tensor_copy_async (src/backend/core.c:822-840): lifecycle first, then
+    ownership (STATE), then descriptors (BOUNDS); the copy itself is not waited for and the
+    destination inherits the source's written flag (src/backend/cuda/backend.c:1159-1191)."""
+    err = B.Error()
+    copy_async = lib().yvex_backend_tensor_copy_async
+    with Backend() as b, Backend() as other:
+        source, target = f32(b, "source", (8, 4)), f32(b, "target", (8, 4))
+        source.write(np.arange(32, dtype=np.float32))
+        assert not target.is_written
+        assert copy_async(b.handle, target.handle, source.handle, C.byref(err)) == 0
+        assert target.is_written and np.array_equal(target.read(), source.read())
+        fresh, into = f32(b, "never-written", (8, 4)), f32(b, "into", (8, 4))
+        into.write(np.ones(32, np.float32))
+        assert copy_async(b.handle, into.handle, fresh.handle, C.byref(err)) == 0
+        assert not into.is_written                                   # flag follows the source
+        reshaped = f32(b, "reshaped", (32,))
+        assert copy_async(b.handle, reshaped.handle, source.handle, C.byref(err)) == B.YVEX_ERR_BOUNDS
+        assert b"descriptors differ" in err.message
+        foreign = f32(other, "foreign", (8, 4))
+        assert copy_async(b.handle, foreign.handle, source.handle, C.byref(err)) == B.YVEX_ERR_STATE
+        assert copy_async(b.handle, target.handle, foreign.handle, C.byref(err)) == B.YVEX_ERR_STATE
+        assert err.where == b"backend.tensor.copy-async"
+        # the session layer's use (src/runtime/stateful_attention.c:183-222): row views of the
+        # projections copied into [K | V] rows of the history
+        history = f32(b, "history", (4, 2, 16))
+        history.zero()
+        keys, values = f32(b, "keys", (2, 16)), f32(b, "values", (2, 16))
+        keys.write(np.arange(32, dtype=np.float32))
+        values.write(-np.arange(32, dtype=np.float32))
+        for token in range(2):
+            history.view((1 + token) * 128, B.DTYPE_F32, (16,)).copy_from_async(
+                keys.view(token * 64, B.DTYPE_F32, (16,)))
+            history.view((1 + token) * 128 + 64, B.DTYPE_F32, (16,)).copy_from_async(
+                values.view(token * 64, B.DTYPE_F32, (16,)))
+        rows = history.read().reshape(4, 32)
+        assert np.all(rows[0] == 0) and np.all(rows[3] == 0)
+        assert np.array_equal(rows[1], np.concatenate([np.arange(16), -np.arange(16)]))
+        assert np.array_equal(rows[2], np.concatenate([np.arange(16, 32), -np.arange(16, 32)]))
+    closed = C.c_void_p()
+    options = B.BackendOptions(B.KIND_ROCM, None, 0)
+    assert lib().yvex_backend_open(C.byref(closed), C.byref(options), C.byref(err)) == 0
+    assert copy_async(None, None, None, C.byref(err)) == B.YVEX_ERR_STATE    # lifecycle gate first
+    assert lib().yvex_backend_close_checked(C.byref(closed), C.byref(err)) == 0
+
+
+def test_session_backends_lease_their_primary_and_copy_between_streams(fake_runtime):
+    """yvex_backend_open_shared_rocm (src/backend/cuda/backend.c:1795-1879) and
+    yvex_backend_tensor_copy_shared_async (src/backend/core.c:842-874): a session backend has
+    its own stream and accounting on the primary's device; the primary cannot be discharged
+    while a session backend is open; a copy across the two is admitted only for one physical
+    owner, equal descriptors and a written source."""
+    err = B.Error()
+    shared_copy = lib().yvex_backend_tensor_copy_shared_async
+    primary = Backend(memory_limit_bytes=1 << 20)
+    session = Backend(shared_with=primary, memory_limit_bytes=1 << 16)
+    second = Backend(shared_with=primary)
+    stranger = Backend()
+    assert session.status == B.STATUS_READY
+    assert session.memory_stats().memory_limit_bytes == 1 << 16
+    source = f32(primary, "weights", (4, 4))
+    source.write(np.arange(16, dtype=np.float32))
+    target = f32(session, "copy", (4, 4))
+    target.copy_from_shared_async(source)                           # primary -> session
+    assert target.is_written and np.array_equal(target.read(), source.read())
+    sibling = f32(second, "sibling", (4, 4))
+    sibling.copy_from_shared_async(target)                          # session -> session
+    assert np.array_equal(sibling.read(), source.read())
+    back = f32(primary, "back", (4, 4))
+    back.copy_from_shared_async(sibling)                            # session -> primary
+    assert np.array_equal(back.read(), source.read())
+    assert primary.memory_stats().allocated_bytes == 128 and session.memory_stats().allocated_bytes == 64
+    # refusals: destination not the executor's, another physical owner, descriptors, unwritten
+    assert shared_copy(primary.handle, target.handle, source.handle, C.byref(err)) == B.YVEX_ERR_INVALID_ARG
+    outsider = f32(stranger, "outsider", (4, 4))
+    outsider.write(np.zeros(16, np.float32))
+    assert shared_copy(session.handle, target.handle, outsider.handle, C.byref(err)) == B.YVEX_ERR_INVALID_ARG
+    assert shared_copy(session.handle, f32(session, "flat", (16,)).handle, source.handle,
+                       C.byref(err)) == B.YVEX_ERR_INVALID_ARG
+    assert shared_copy(session.handle, target.handle, f32(primary, "blank", (4, 4)).handle,
+                       C.byref(err)) == B.YVEX_ERR_INVALID_ARG
+    assert shared_copy(None, target.handle, source.handle, C.byref(err)) == B.YVEX_ERR_INVALID_ARG
+    # a session backend cannot be the owner of another one
+    nested = C.c_void_p()
+    assert lib().yvex_backend_open_shared_rocm(C.byref(nested), session.handle, 0, C.byref(err)) == \
+        B.YVEX_ERR_INVALID_ARG and not nested.value
+    # the primary is not discharged while session backends are open: the close marks it
+    # cleanup-only and keeps the handle; after the sessions are closed it goes
+    stranger.close()
+    for backend in (primary, session, second):
+        for tensor in backend.tensors:
+            tensor.release()
+    handle = C.c_void_p(primary.handle.value)
+    assert lib().yvex_backend_close_checked(C.byref(handle), C.byref(err)) == B.YVEX_ERR_STATE
+    assert handle.value and b"live shared children" in err.message
+    late = C.c_void_p()
+    assert lib().yvex_backend_open_shared_rocm(C.byref(late), handle, 0, C.byref(err)) == B.YVEX_ERR_STATE
+    session.close()
+    assert lib().yvex_backend_close_checked(C.byref(handle), C.byref(err)) == B.YVEX_ERR_STATE
+    second.close()
+    assert lib().yvex_backend_close_checked(C.byref(handle), C.byref(err)) == 0 and not handle.value
+    primary.handle = None
+
+
 def test_f32_subview_matches_reference_rules():
     with Backend() as b:
         t = f32(b, "row", (8, 4), np.arange(32))
