@@ -34,7 +34,7 @@ sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 from clori_amd import binding as B  # noqa: E402
-from clori_amd.backend import Backend  # noqa: E402
+from clori_amd.backend import Backend, kv_pack_pages, q8_0_encode_rows  # noqa: E402
 
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
@@ -47,6 +47,10 @@ def bf16_bits(x):
     return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
 
 
+def bf16_decode(bits):
+    return (np.ascontiguousarray(bits, dtype=np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
 def random_bf16(rng, count, unique=1 << 24):
     """`count` N(0,1) bf16 values.  Beyond `unique` values the block repeats: throughput
     does not depend on the values and generation stays in seconds."""
@@ -57,8 +61,7 @@ def random_bf16(rng, count, unique=1 << 24):
     return np.tile(base, reps)[:count]
 
 
-SPIN_UP_SECONDS = float(os.environ.get("YVEX_BENCH_SPIN_UP", "0.2"))
-RECORDED_STEPS = bool(int(os.environ.get("YVEX_BENCH_RECORDED", "0")))
+SPIN_UP_SECONDS = 0.2        # untimed work before the warm-up steps (--spin-up)
 
 
 RECORD_ITERATIONS = 100       # per-dispatch samples of the benchmark record
@@ -73,13 +76,7 @@ def time_steps(backend, run, steps, warmup, kernels):
     device, from which the benchmark record's distributions are taken."""
     from clori_amd.backend import benchmark_summarize
     backend.set_completion_mode(B.COMPLETION_DEFERRED)
-    step, graph = run, None
-    if RECORDED_STEPS:
-        # the step's launches recorded once and replayed with one call per step
-        backend.graph_begin()
-        run()
-        graph = backend.graph_end()
-        step = lambda: backend.graph_launch(graph)  # noqa: E731
+    step = run
     # the part raises its clocks only under sustained load: keep it busy for SPIN_UP_SECONDS
     # before the W warm-up steps, all untimed
     spin_until = time.perf_counter() + SPIN_UP_SECONDS
@@ -97,8 +94,6 @@ def time_steps(backend, run, steps, warmup, kernels):
     device_ms = backend.timing_end()
     backend.sync()
     wall_ms = (time.perf_counter() - t0) * 1e3
-    if graph is not None:
-        backend.graph_release(graph)
     kernel_ms = {}
     for kernel in kernels:
         backend.kernel_probe_begin(kernel)
@@ -150,14 +145,10 @@ def workload_paged(backend, rng, steps, warmup, q8=False, page=16):
     sessions, hq, hkv, d = 32, 32, 8, 128
     lo, hi = (4096, 32768) if q8 else (512, 16384)
     contexts = rng.integers(lo, hi + 1, size=sessions).astype(np.int32)
-    if os.environ.get("YVEX_BENCH_UNIFORM_CONTEXT"):   # tuning aid: equal-length sessions
-        contexts[:] = int(os.environ["YVEX_BENCH_UNIFORM_CONTEXT"])
     need = (contexts + page - 1) // page
     pool_pages = int(need.sum())
     stride = int(hi // page)
     perm = rng.permutation(pool_pages).astype(np.int32)
-    if os.environ.get("YVEX_BENCH_ORDERED_PAGES"):     # tuning aid: pages in pool order
-        perm = np.arange(pool_pages, dtype=np.int32)
     table = np.zeros((sessions, stride), dtype=np.int32)
     at = 0
     for s in range(sessions):
@@ -168,15 +159,20 @@ def workload_paged(backend, rng, steps, warmup, q8=False, page=16):
     blocks = pool_pages * hkv * (page // 16)
     pool_bytes = blocks * block
     if q8:
-        # int8 codes in [-127,127] and f16 scales near 1/40: any bytes are valid Q8_0 as long
-        # as scales are finite and non-negative; layout = codes then scales per block
-        pool = np.empty((blocks, block), dtype=np.uint8)
-        codes = rng.integers(-127, 128, size=(1 << 22), dtype=np.int8).view(np.uint8)
-        reps = (blocks * 2048 + codes.size - 1) // codes.size
-        pool[:, :2048] = np.tile(codes, reps)[:blocks * 2048].reshape(-1, 2048)
-        pool[:, 2048:] = np.tile(np.array([0.025], np.float16).view(np.uint8), 64)[None, :]
-        k_pool = backend.tensor("k-pages", B.DTYPE_I8, (pool_bytes,), pool)
-        v_pool = backend.tensor("v-pages", B.DTYPE_I8, (pool_bytes,), pool[::-1].copy())
+        # N(0,1) values rounded to bf16 and quantised on the host with the library's Q8_0 encoder
+        # (round-to-nearest absmax/127), packed into the device page layout.  A sample of
+        # SAMPLE_PAGES pages is generated and repeated through the pool: throughput does not
+        # depend on the values and generation stays in seconds.
+        sample_pages = min(pool_pages, 2048)
+
+        def quantised_pool(is_value):
+            values = bf16_decode(random_bf16(rng, sample_pages * page * hkv * d))
+            blocks = q8_0_encode_rows(values.reshape(sample_pages, page, hkv, d))
+            packed = kv_pack_pages(blocks, B.KV_Q8_0, is_value, hkv, d, page)
+            reps = (pool_bytes + packed.size - 1) // packed.size
+            return np.tile(packed, reps)[:pool_bytes]
+        k_pool = backend.tensor("k-pages", B.DTYPE_I8, (pool_bytes,), quantised_pool(False))
+        v_pool = backend.tensor("v-pages", B.DTYPE_I8, (pool_bytes,), quantised_pool(True))
     else:
         k_pool = backend.tensor("k-pages", B.DTYPE_BF16, (pool_bytes // 2,),
                                 random_bf16(rng, pool_bytes // 2))
@@ -205,8 +201,10 @@ def workload_paged(backend, rng, steps, warmup, q8=False, page=16):
     assert np.all(np.isfinite(lse.read()))
     return dict(name=("paged4" if q8 else "paged3") + ("" if page == 16 else "_p%d" % page),
                 workload="paged %s GQA decode: 32 sessions, 32/8 heads, d=128, contexts U[%d,%d], "
-                         "%d-token pages, seeded permutation page tables" %
-                         ("Q8_0" if q8 else "bf16", lo, hi, page),
+                         "%d-token pages, seeded permutation page tables%s" %
+                         ("Q8_0" if q8 else "bf16", lo, hi, page,
+                          ", N(0,1) bf16 values quantised on the host (absmax/127, round to nearest), "
+                          "a 2048-page sample repeated through the pool" if q8 else ""),
                 bound="hbm", algorithmic_bytes=algo, tokens=tokens,
                 launches=int(facts.kernel_launches), kernels=kernels, **timed)
 
@@ -506,6 +504,36 @@ def repeat_for(seconds, call, least=3):
             return len(durations), float(np.median(durations)), time.perf_counter() - t0
 
 
+def reference_operator_leg(rng, keys, heads, d, budget=2.0):
+    """The reference's own CPU operator (yvex_backend_op_attention, compiled from the reference's
+    sources into oracle/_ref, single thread, one query head per call over F32 rows): seconds
+    per head over `keys` keys, median of the runs that fit `budget`.  None where oracle/_ref was
+    not built."""
+    import ctypes
+    from oracle_binding import load_reference
+    ref = load_reference()
+    if ref is None:
+        return None
+    f32p = ctypes.POINTER(ctypes.c_float)
+    q = rng.standard_normal(d, dtype=np.float32)
+    k = rng.standard_normal((keys, d), dtype=np.float32)
+    v = rng.standard_normal((keys, d), dtype=np.float32)
+    out = np.zeros(d, np.float32)
+    score, prob = np.zeros(keys, np.float32), np.zeros(keys, np.float32)
+    ptr = lambda a: a.ctypes.data_as(f32p)  # noqa: E731
+
+    def one_head():
+        rc = ref.yvref_op_attention(ptr(q), ptr(k), ptr(v), keys, keys - 1, d,
+                                    np.float32(1.0 / np.sqrt(d)), 1, ptr(score), ptr(prob), ptr(out))
+        assert rc == 0
+        return rc
+    runs, dt, spent = repeat_for(budget, one_head)
+    return dict(seconds_per_head=dt, keys=keys, head_dim=d, cores=1, kind="reference",
+                sample="yvex_backend_op_attention of the compiled reference, one query head over %d "
+                       "F32 keys, single thread, median of %d runs (%.1f s)" % (keys, runs, spent),
+                heads_of_the_workload=heads)
+
+
 def cpu_baseline(name, budget=6.0):
     """The oracle (a port of the reference CPU operator, all host threads) timed on a bounded
     sample of the same workload: the sample is repeated at least three times and for about `budget` seconds, and the median run
@@ -529,17 +557,23 @@ def cpu_baseline(name, budget=6.0):
         runs, dt, spent = repeat_for(budget, lambda: oracle.paged_decode(q, k, v, table, contexts, hkv,
                                                                   page, q8=q8)[0])
         per_token = 2 * hkv * (136 if q8 else 256)
+        leg = reference_operator_leg(rng, 8192, hq, d)
+        if leg:   # the same bytes per token if one thread ran every query head of a session
+            leg.update(value=8192 * per_token / (leg["seconds_per_head"] * hq) / 1e9, unit="GB/s")
         return dict(value=int(contexts.sum()) * per_token / dt / 1e9, unit="GB/s", cores=threads,
                     kind="port", sample="4 sessions x 8192 tokens of the same shape, median of "
-                                        "%d runs (%.1f s)" % (runs, spent))
+                                        "%d runs (%.1f s)" % (runs, spent), reference_operator=leg)
     if name == "decode1":
         q = bf16_bits(rng.standard_normal((1, 32, 128), dtype=np.float32))
         k = bf16_bits(rng.standard_normal((4096, 8, 128), dtype=np.float32))
         v = bf16_bits(rng.standard_normal((4096, 8, 128), dtype=np.float32))
         runs, dt, spent = repeat_for(budget / 2, lambda: oracle.gqa_bf16(q, k, v, query_start=4095)[0])
+        leg = reference_operator_leg(rng, 4096, 32, 128)
+        if leg:
+            leg.update(value=(2 * 4096 * 8 * 128 * 2) / (leg["seconds_per_head"] * 32) / 1e9, unit="GB/s")
         return dict(value=(2 * 4096 * 8 * 128 * 2) / dt / 1e9, unit="GB/s", cores=threads,
                     kind="port", sample="the full workload, median of %d runs (%.1f s)" %
-                                        (runs, spent))
+                                        (runs, spent), reference_operator=leg)
     if name == "prefill2":
         t, hq, hkv, d = 1024, 40, 8, 128
         q = bf16_bits(rng.standard_normal((t, hq, d), dtype=np.float32))
@@ -584,6 +618,7 @@ METRIC = "decode attn HBM GB/s (% of peak); prefill attn TFLOPS (% MFMA peak), 1
 
 
 def main():
+    global SPIN_UP_SECONDS
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
@@ -592,7 +627,12 @@ def main():
                     help="one workload name, or 'all' (default): every configuration, with "
                          "the paged bf16 decode as the headline value")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--spin-up", type=float, default=SPIN_UP_SECONDS,
+                    help="seconds of untimed steps before the warm-up steps of each workload "
+                         "(the part raises its clocks only under sustained load); printed as "
+                         "spin_up_s")
     args = ap.parse_args()
+    SPIN_UP_SECONDS = args.spin_up
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; --gpus %d is not supported "
                  "(attention shards by session or head without exchange)" % args.gpus)
@@ -626,7 +666,7 @@ def main():
         "metric": METRIC,
         "value": roof["step_achieved"],
         "unit": roof["unit"],
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "spin_up_s": SPIN_UP_SECONDS,
         "ms_per_step": head["ms"],
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": head.get("dtype", "bf16"), "data": "synthetic",
