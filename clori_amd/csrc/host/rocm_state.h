@@ -76,6 +76,7 @@ typedef struct yvex_rocm_backend_state {
     int status_dirty;       /* deferred mode: launches since the last check */
     yvex_rocm_completion_mode completion_mode;
     unsigned long long live_tensors;
+    struct yvex_rocm_virtual_range *virtual_ranges; /* every reserved range that is alive */
     int unbacked_view;  /* the last view check failed on uncommitted pages, not on geometry */
     int virtual_memory; /* the runtime and the device can reserve, map and unmap address ranges */
     int recording;                  /* a launch sequence is being recorded on the stream */

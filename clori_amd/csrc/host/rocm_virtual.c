@@ -32,6 +32,11 @@ typedef struct yvex_rocm_virtual_range {
     size_t logical_bytes, reserved_bytes, granularity, granule_count;
     hipMemGenericAllocationHandle_t *handles; /* per granule */
     unsigned char *state;                     /* per granule: GRANULE_* bits */
+    /* the backend keeps every live range in a list: a view is a struct copy that carries the
+     * range pointer and the owner's id, and may outlive the tensor it was taken from */
+    struct yvex_rocm_virtual_range *next;
+    yvex_device_tensor *owner_tensor; /* the tensor that owns the range: residency is counted there */
+    unsigned long long owner_id;
 } yvex_rocm_virtual_range;
 
 enum { GRANULE_CREATED = 1, GRANULE_MAPPED = 2 };
@@ -56,10 +61,20 @@ static void range_properties(const yvex_rocm_backend_state *state, hipMemAllocat
     }
 }
 
+/* The live range a tensor or a view of it lies in.  The pointer a view carries is only
+ * compared, never followed, until it is found among the backend's live ranges with the id the
+ * view was copied with: a view kept past the release of its tensor finds nothing (and an
+ * address that a later range happens to reuse has another id). */
 static yvex_rocm_virtual_range *range_of(const yvex_device_tensor *tensor)
 {
-    return tensor && tensor->virtual_reserved ? (yvex_rocm_virtual_range *)tensor->backend_allocation
-                                              : NULL;
+    const yvex_rocm_backend_state *state;
+    yvex_rocm_virtual_range *range;
+    if (!tensor || !tensor->virtual_reserved || !tensor->owner || !tensor->owner_id) return NULL;
+    state = yvex_rocm_state(tensor->owner);
+    for (range = state ? state->virtual_ranges : NULL; range; range = range->next)
+        if ((void *)range == tensor->backend_allocation && range->owner_id == tensor->owner_id)
+            return range;
+    return NULL;
 }
 
 /* The granules under [tensor->data + offset, + bytes), or 0 when that is not inside the range. */
@@ -175,6 +190,10 @@ int yvex_rocm_tensor_reserve(yvex_backend *backend, const yvex_backend_tensor_de
     tensor->data = range->address;
     tensor->backend_allocation = range;
     tensor->virtual_reserved = 1;
+    range->owner_tensor = tensor;
+    range->owner_id = tensor->owner_id;
+    range->next = state->virtual_ranges;
+    state->virtual_ranges = range;
     state->live_tensors += 1ull;
     *out = tensor;
     *granularity_out = (unsigned long long)granularity;
@@ -227,6 +246,21 @@ int yvex_rocm_tensor_commit(yvex_backend *backend, yvex_device_tensor *tensor,
     if (state->recording)
         return refuse(err, YVEX_ERR_STATE, where,
                       "not available while a launch sequence is being recorded");
+    /* A granule that an earlier release left half done (unmapped, its memory not given back
+     * yet) is neither backed nor missing: finish that release first, or say why it cannot be
+     * finished; it then counts as missing like any other. */
+    for (granule = first; granule <= last; ++granule)
+        if (range->state[granule] && range->state[granule] != (GRANULE_CREATED | GRANULE_MAPPED)) {
+            rc = granule_release(backend, range, granule, err);
+            if (rc != YVEX_OK) {
+                state->backend_failure_reason = YVEX_BACKEND_CAPABILITY_REASON_CLEANUP_FAILED;
+                backend->status = YVEX_BACKEND_STATUS_FAILED;
+                return rc;
+            }
+            range->owner_tensor->resident_bytes =
+                range->owner_tensor->resident_bytes >= range->granularity
+                    ? range->owner_tensor->resident_bytes - range->granularity : 0ull;
+        }
     for (granule = first; granule <= last; ++granule)
         if (!range->state[granule]) ++missing;
     if (!missing) {
@@ -235,7 +269,7 @@ int yvex_rocm_tensor_commit(yvex_backend *backend, yvex_device_tensor *tensor,
         return YVEX_OK;
     }
     if (!yvex_core_u64_mul(missing, range->granularity, &required) ||
-        tensor->resident_bytes > ULLONG_MAX - required)
+        range->owner_tensor->resident_bytes > ULLONG_MAX - required)
         return refuse(err, YVEX_ERR_BOUNDS, where, "physical page commitment extent overflowed");
     rc = yvex_backend_memory_can_add(backend, required, "ROCm state pages", where, err);
     if (rc != YVEX_OK) return rc;
@@ -246,7 +280,7 @@ int yvex_rocm_tensor_commit(yvex_backend *backend, yvex_device_tensor *tensor,
     range_properties(state, &properties, &access);
     for (granule = first; rc == YVEX_OK && granule <= last; ++granule) {
         unsigned char *address = range->address + granule * range->granularity;
-        if (range->state[granule]) continue; /* half-released granules are decommit's to finish */
+        if (range->state[granule]) continue; /* backed already */
         rc = yvex_rocm_status(&state->driver,
                               state->driver.hipMemCreate(&range->handles[granule], range->granularity,
                                                          &properties, 0ull),
@@ -297,7 +331,9 @@ int yvex_rocm_tensor_commit(yvex_backend *backend, yvex_device_tensor *tensor,
         return rc;
     }
     free(fresh);
-    tensor->resident_bytes += required;
+    /* residency is a property of the range: counted on the tensor that owns it, also when the
+     * commit came through a view */
+    range->owner_tensor->resident_bytes += required;
     *resident_delta = required;
     yvex_error_clear(err);
     return YVEX_OK;
@@ -335,7 +371,13 @@ int yvex_rocm_tensor_decommit(yvex_backend *backend, yvex_device_tensor *tensor,
         }
     tensor->resident_bytes =
         tensor->resident_bytes >= released ? tensor->resident_bytes - released : 0ull;
-    if (rc != YVEX_OK) return rc;
+    if (rc != YVEX_OK) {
+        /* pages that could not be given back: as for a tensor that cannot be freed, the
+         * backend is retained for cleanup only and a later release tries again */
+        state->backend_failure_reason = YVEX_BACKEND_CAPABILITY_REASON_CLEANUP_FAILED;
+        backend->status = YVEX_BACKEND_STATUS_FAILED;
+        return rc;
+    }
     *released_bytes = released;
     tensor->is_written = 0;
     yvex_error_clear(err);
@@ -358,6 +400,11 @@ int yvex_rocm_virtual_release(yvex_backend *backend, yvex_device_tensor *tensor,
                               state->driver.hipMemAddressFree(range->address, range->reserved_bytes),
                               "rocm.tensor.free.address", err);
     if (rc != YVEX_OK) return rc;
+    {
+        yvex_rocm_virtual_range **link = &state->virtual_ranges;
+        while (*link && *link != range) link = &(*link)->next;
+        if (*link) *link = range->next;
+    }
     free(range->handles);
     free(range->state);
     free(range);

@@ -982,6 +982,9 @@ __device__ __forceinline__ void decode_merge_rows(const yvex_rocm_decode_merge_p
         float a = acc[2 * i] * inv, b = acc[2 * i + 1] * inv;
         bad |= !(isfinite(a) && isfinite(b));
         if (kRope && turn) {
+            // products and sums rounded one by one, as the C reference computes them
+            // (src/graph/numeric.c:935-947 is built without contraction)
+#pragma clang fp contract(off)
             const double angle = position * p.rope_frequency[(lane * 8u - rope_start) / 2u + (uint32_t)i];
             const double c = cos(angle), s = -sin(angle);
             const double x = (double)bf16_to_f32(bf16_bits(a)), y = (double)bf16_to_f32(bf16_bits(b));

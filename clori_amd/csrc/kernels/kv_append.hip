@@ -180,6 +180,12 @@ __device__ inline bool key_finish(const KeyChunk &k, u32x4 &lower, u32x4 &upper,
         const float cosine0 = __builtin_bit_cast(float, c0), cosine1 = __builtin_bit_cast(float, c1);
         const float sine0 = __builtin_bit_cast(float, s0), sine1 = __builtin_bit_cast(float, s1);
         if (plain) {
+            // first * cosine - second * sine and second * cosine + first * sine with the second
+            // product rounded and the first fused into the sum: one of the legal contractions of
+            // the reference's plain F32 kernel (src/backend/cuda/transformer_kernels.cu:110-134),
+            // the one LLVM picks for these expressions.  Which one the reference's compiler picks
+            // is not visible in its sources: the last bit of a result next to a bf16 tie is not
+            // pinned by the reference (the unfused evaluation differs there, by one bf16 step).
             lower[j] = pack_bf16x2(__builtin_fmaf(first0, cosine0, -(second0 * sine0)),
                                    __builtin_fmaf(first1, cosine1, -(second1 * sine1)));
             upper[j] = pack_bf16x2(__builtin_fmaf(second0, cosine0, first0 * sine0),

@@ -582,6 +582,49 @@ def test_virtual_tensor_failed_release_keeps_the_owner(env, fake_runtime):
     b.close()
 
 
+def test_virtual_tensor_views_outlive_nothing_and_count_on_the_owner(env, fake_runtime):
+    """A view is a struct copy that carries the range pointer and the owner's id.  Commits
+    through a view are counted on the tensor that owns the range; a view kept past the release
+    of that tensor is refused everywhere instead of reading freed host state; a granule that a
+    failed release left half done is finished by the next commit, not skipped."""
+    b = Backend()
+    owner = b.reserve("history", B.DTYPE_I8, (8 << 21,))
+    view = owner.view(2 << 21, B.DTYPE_I8, (2 << 21,))
+    assert view.commit(0, 2 << 21) == 2 << 21                   # granules 2 and 3
+    assert owner.resident_bytes == 2 << 21
+    assert b.memory_stats().allocated_bytes == 2 << 21
+    view.zero()                                                 # backed: accepted
+    # half-released granule: the unmap goes through, giving the memory back fails
+    env("FAKE_HIP_RELEASE", "fail")
+    with pytest.raises(YvexError) as e:
+        owner.decommit()
+    assert e.value.code == B.YVEX_ERR_BACKEND and b.status == B.STATUS_FAILED
+    env("FAKE_HIP_RELEASE", None)
+    owner.release()                                             # cleanup-only release finishes it
+    assert fake_runtime.fake_hip_live_physical() == 0 and fake_runtime.fake_hip_live_ranges() == 0
+    b.tensors.clear()
+    b.close()
+    # a stale view on a live backend
+    b = Backend()
+    owner = b.reserve("history", B.DTYPE_I8, (4 << 21,))
+    owner.commit(0, 4 << 21)
+    stale = owner.view(0, B.DTYPE_I8, (1 << 21,))
+    target = b.tensor("target", B.DTYPE_I8, (1 << 21,))
+    owner.release()
+    again = b.reserve("again", B.DTYPE_I8, (4 << 21,))          # may reuse the freed host block
+    again.commit(0, 4 << 21)
+    err = B.Error()
+    for call in (lambda: lib().yvex_backend_tensor_zero(b.handle, stale.handle, C.byref(err)),
+                 lambda: lib().yvex_backend_tensor_copy(b.handle, target.handle, stale.handle, C.byref(err)),
+                 lambda: lib().yvex_backend_tensor_copy_async(b.handle, target.handle, stale.handle,
+                                                               C.byref(err))):
+        assert call() == B.YVEX_ERR_STATE, err.message
+    delta = C.c_ulonglong(0)
+    assert lib().yvex_backend_tensor_commit_range(b.handle, stale.handle, 0, 1 << 21, C.byref(delta),
+                                                  C.byref(err)) == B.YVEX_ERR_INVALID_ARG
+    b.close()
+
+
 # ------------------------------------------------- operation admission ----
 
 def test_bounded_primitive_refusal_order_and_facts(fake_runtime):
