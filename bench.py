@@ -15,7 +15,8 @@ already resident in HBM.  Workloads are the five configurations the metric is qu
 By name only (not configurations of the metric): exact2 and exact1 (configurations 2 and 1
 under the EXACT_F32 contract: fp32 matrix cores, and double-precision split decode),
 append_bf16 / append_q8_0 (the KV page writer), history_append (the token-major writer), paged3_p64 / paged4_p64
-(configurations 3 and 4 with pages of 64 tokens), copy.
+(configurations 3 and 4 with pages of 64 tokens), prefill_d256 / prefill_d64 (causal prefill at head
+dimension 256, 24/4 heads, and 64, 16/4 heads), copy.
 
 Prints ONE JSON line.  `value` is the headline workload's throughput; every workload
 that ran is listed under "workloads" with its own roofline figures.  Timing uses HIP
@@ -235,8 +236,8 @@ def workload_decode1(backend, rng, steps, warmup):
                 launches=int(facts.kernel_launches), kernels=kernels, **timed)
 
 
-def workload_prefill2(backend, rng, steps, warmup):
-    t, hq, hkv, d = 2048, 40, 8, 128
+def workload_prefill2(backend, rng, steps, warmup, hq=40, hkv=8, d=128, name="prefill2"):
+    t = 2048
     sq = rng.uniform(0.5, 1.5, size=(1, hq, 1)).astype(np.float32)
     skv = rng.uniform(0.5, 1.5, size=(1, hkv, 1)).astype(np.float32)
     qv = bf16_bits(rng.standard_normal((t, hq, d), dtype=np.float32) * sq)
@@ -250,11 +251,11 @@ def workload_prefill2(backend, rng, steps, warmup):
                                         contract=B.NUMERIC_BF16_F32_ACCUMULATE)
     run = lambda: backend.attention_execute(req, q, k, v, out)  # noqa: E731
     facts = run()
-    kernels = ["yvex_rocm_prefill_bf16"]
+    kernels = ["yvex_rocm_prefill_bf16" + ("" if d == 128 else "_%d" % d)]
     timed = time_steps(backend, run, steps, warmup, kernels)
     flops = 4 * d * hq * t * (t + 1) // 2      # causal-useful multiply-adds * 2, QK^T and PV
-    return dict(name="prefill2",
-                workload="causal GQA prefill: batch 1, seq 2048, 40/8 heads, d=128, bf16",
+    return dict(name=name,
+                workload="causal GQA prefill: batch 1, seq 2048, %d/%d heads, d=%d, bf16" % (hq, hkv, d),
                 bound="mfma", flops=flops, algorithmic_bytes=(2 * t * hq * d + 2 * t * hkv * d) * 2,
                 launches=int(facts.kernel_launches), kernels=kernels, **timed)
 
@@ -442,9 +443,13 @@ EXTRA_WORKLOADS = {
     "paged4_p64": lambda b, r, s, w: workload_paged(b, r, s, w, q8=True, page=64),
     "exact2": workload_exact2,
     "exact1": workload_exact1,
+    # the reference's own Qwen attention geometry (24/4 heads, head dimension 256) and a narrow one
+    "prefill_d256": lambda b, r, s, w: workload_prefill2(b, r, s, w, hq=24, hkv=4, d=256, name="prefill_d256"),
+    "prefill_d64": lambda b, r, s, w: workload_prefill2(b, r, s, w, hq=16, hkv=4, d=64, name="prefill_d64"),
 }
 SEEDS = {"decode1": 1, "prefill2": 2, "paged3": 3, "paged4": 4, "mla5": 5, "append_bf16": 6,
-         "append_q8_0": 7, "exact2": 8, "exact1": 9, "history_append": 10, "paged3_p64": 3, "paged4_p64": 4}
+         "append_q8_0": 7, "exact2": 8, "exact1": 9, "history_append": 10, "paged3_p64": 3, "paged4_p64": 4,
+         "prefill_d256": 11, "prefill_d64": 12}
 
 
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")

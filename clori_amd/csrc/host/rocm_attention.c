@@ -306,14 +306,16 @@ static int attention_validate(const yvex_transformer_attention_requirement *r, c
             return refuse(err, YVEX_ERR_UNSUPPORTED, stage,
                           "ROCm requires deterministic token/head/dimension exact F32 attention");
     } else if (r->numeric_contract == YVEX_TRANSFORMER_ATTENTION_NUMERIC_BF16_F32_ACCUMULATE) {
-        if (r->head_dimension != ROCM_MFMA_HEAD_DIM || r->query_dtype != YVEX_DTYPE_BF16 ||
+        if ((r->head_dimension != 64ull && r->head_dimension != ROCM_MFMA_HEAD_DIM &&
+             r->head_dimension != 256ull) ||
+            r->query_dtype != YVEX_DTYPE_BF16 ||
             r->key_dtype != YVEX_DTYPE_BF16 || r->value_dtype != YVEX_DTYPE_BF16 ||
             r->output_dtype != YVEX_DTYPE_BF16 ||
             r->query_heads / r->key_value_heads > ROCM_GROUP_MAX ||
             r->key_value_tokens > 0x7fffffffull || (r->query_token_stride % 8ull) ||
             (r->key_token_stride % 8ull) || (r->value_token_stride % 8ull))
             return refuse(err, YVEX_ERR_UNSUPPORTED, stage,
-                          "ROCm bf16 attention requires BF16 tensors, head dimension 128, "
+                          "ROCm bf16 attention requires BF16 tensors, head dimension 64, 128 or 256, "
                           "a query group of at most 16 and 16-byte aligned token strides");
     } else {
         return refuse(err, YVEX_ERR_UNSUPPORTED, stage,
@@ -411,7 +413,7 @@ static int rocm_attention_workspace_required(const yvex_transformer_attention_re
     if (rc != YVEX_OK) return rc;
     if (!bytes) return refuse(err, YVEX_ERR_INVALID_ARG, where, "workspace byte output is required");
     if (r->numeric_contract == YVEX_TRANSFORMER_ATTENTION_NUMERIC_BF16_F32_ACCUMULATE &&
-        r->query_tokens == 1ull) {
+        r->query_tokens == 1ull && r->head_dimension == ROCM_MFMA_HEAD_DIM) {
         /* split-K decode partials; geometry must match decode_run */
         const unsigned int waves = decode_wave_count(1ull, r->key_value_heads, visible_tokens(r));
         const unsigned long long group = r->query_heads / r->key_value_heads;
@@ -621,7 +623,9 @@ static int attention_execute_common(yvex_backend *backend,
                 if (err) *err = cleanup;
             }
         }
-    } else if (r->query_tokens == 1ull) {
+    } else if (r->query_tokens == 1ull && r->head_dimension == ROCM_MFMA_HEAD_DIM) {
+        /* the split decode kernels are built for head dimension 128; a single query token of
+         * another width runs as a one-row tile of the prefill kernel below */
         decode_job job;
         memset(&job, 0, sizeof(job));
         job.function = YVEX_ROCM_FN_DECODE_ROWS_BF16;
@@ -673,7 +677,10 @@ static int attention_execute_common(yvex_backend *backend,
             r->key_value_tokens * v_stride * 2ull >= 0xffffffffull)
             return refuse(err, YVEX_ERR_BOUNDS, where,
                           "prefill geometry exceeds admitted launch range");
-        rc = yvex_rocm_launch(backend, YVEX_ROCM_FN_PREFILL_BF16,
+        rc = yvex_rocm_launch(backend,
+                              r->head_dimension == 64ull    ? YVEX_ROCM_FN_PREFILL_BF16_64
+                              : r->head_dimension == 256ull ? YVEX_ROCM_FN_PREFILL_BF16_256
+                                                            : YVEX_ROCM_FN_PREFILL_BF16,
                               YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_BF16,
                               (unsigned int)(r->query_heads * q_tiles), 1u, 1u, 256u, 0u,
                               &params, "rocm.transformer.gqa.prefill", err);

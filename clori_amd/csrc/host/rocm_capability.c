@@ -56,6 +56,10 @@ static const rocm_kernel_binding rocm_kernel_bindings[] = {
      YVEX_ROCM_FN_DECODE_ROWS_BF16},
     {"yvex_rocm_prefill_bf16", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_BF16,
      YVEX_ROCM_FN_PREFILL_BF16},
+    {"yvex_rocm_prefill_bf16_64", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_BF16,
+     YVEX_ROCM_FN_PREFILL_BF16_64},
+    {"yvex_rocm_prefill_bf16_256", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_BF16,
+     YVEX_ROCM_FN_PREFILL_BF16_256},
     {"yvex_rocm_mla_decode_bf16", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_MLA_BF16,
      YVEX_ROCM_FN_MLA_DECODE_BF16},
     {"yvex_rocm_mla_decode_512_bf16", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_MLA_BF16,

@@ -29,6 +29,8 @@ typedef enum {
     YVEX_ROCM_FN_DECODE_ROWS_BF16_MERGED,
     YVEX_ROCM_FN_DECODE_ROWS_BF16_TEAM,
     YVEX_ROCM_FN_PREFILL_BF16,
+    YVEX_ROCM_FN_PREFILL_BF16_64,
+    YVEX_ROCM_FN_PREFILL_BF16_256,
     YVEX_ROCM_FN_MLA_DECODE_BF16,
     YVEX_ROCM_FN_MLA_DECODE_512_BF16,
     YVEX_ROCM_FN_KV_APPEND_BF16,

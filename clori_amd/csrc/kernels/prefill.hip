@@ -1,6 +1,7 @@
 // Causal / full grouped-query attention prefill for gfx950 (wave64), bf16 in and out,
-// fp32 scores, online softmax and accumulation.  head_dim 128, token-major tensors
-// ([token][head][dim], per-token strides in elements).
+// fp32 scores, online softmax and accumulation.  Token-major tensors ([token][head][dim],
+// per-token strides in elements); head_dim 128 is the tuned build, 64 and 256 are the same
+// code with other counts (the numbers in this comment are those of 128).
 //
 // A workgroup of 4 waves owns one (query head, 128-row query tile): each wave owns
 // 32 query rows and walks the key/value tokens in tiles of 64 that the workgroup
@@ -54,11 +55,7 @@
 
 namespace {
 
-constexpr int kHeadDim = 128;
 constexpr int kKeyTile = 64;
-constexpr int kRowBytes = kHeadDim * 2;            // 256
-constexpr int kTileBytes = kKeyTile * kRowBytes;   // 16384 per K or V tile
-constexpr int kBufBytes = 2 * kTileBytes;          // K then V
 constexpr float kLazyLog2 = 8.0f;
 constexpr int kRowsPerWave = 32;
 constexpr int kRowsPerBlock = 4 * kRowsPerWave;
@@ -66,8 +63,21 @@ constexpr int kDepth = 4;  // operand fetches in flight ahead of the MFMA that c
 
 typedef __attribute__((address_space(3))) short4v lds_short4;
 
-// chunk swizzle of tile row r
-__device__ inline int swizzle(int r) { return ((r & 3) << 2) | ((r >> 2) & 3); }
+// Chunk swizzle of tile row r: the 16-byte chunk c of the row sits at chunk position c ^ x(r).
+// Rows of 256 and of 512 bytes all start in the same bank, x(r) permutes the 16 chunk
+// positions of a 256-byte bank span by the row's low four bits (rows r..r+3 go four chunks
+// apart, which is what the transposed read needs; 16 consecutive rows take 16 different
+// positions, which is what the row read needs).  Rows of 128 bytes (head_dim 64) alternate
+// between the two halves of a bank span, so the row's bit 0 already separates them and x(r)
+// permutes the eight chunk positions of a half by bits 1..3: bit 1 moves a row by four
+// chunks (two 32-byte column segments, so that the segments the two dim halves of a
+// transposed read touch stay apart), bits 2 and 3 by two and one.
+template <int D>
+__device__ inline int swizzle(int r)
+{
+    return D == 64 ? ((((r >> 1) & 1) << 2) | (((r >> 2) & 1) << 1) | ((r >> 3) & 1))
+                   : (((r & 3) << 2) | ((r >> 2) & 3));
+}
 
 __device__ inline void flag(int32_t *status, int code) { atomicCAS(status, 0, code); }
 
@@ -81,18 +91,33 @@ __device__ inline float other_half(float v)
     return __builtin_bit_cast(float, (threadIdx.x & 32u) ? r.x : r.y);
 }
 
+template <int kHeadDim>
 struct Prefill {
+    static constexpr int kRowBytes = kHeadDim * 2;            // 256
+    static constexpr int kRowChunks = kRowBytes / 16;         // 16-byte chunks of a row
+    static constexpr int kTileBytes = kKeyTile * kRowBytes;   // 16384 per K or V tile
+    static constexpr int kBufBytes = 2 * kTileBytes;          // K then V
+    static constexpr int kSteps = kHeadDim / 16;              // k-steps of S^T per 32-key half
+    static constexpr int kDimBlocks = kHeadDim / 32;          // 32-dim blocks of O^T
+    static constexpr int kHalfSlots = 2 * kSteps;             // MFMAs of S^T (= of the O^T update) per trip
+    static constexpr int kSlots = 2 * kHalfSlots;
+    static constexpr int kLoads = kTileBytes / 1024 / 4;      // 1 KB loads per wave and K or V tile
+    static constexpr int kLoadRows = 64 / kRowChunks;         // tile rows one 1 KB load covers
+    static constexpr int kSoftmaxSlots = 3 * kSlots / 4;      // the exponentials ride behind these slots
+    static constexpr int kMaxPerSlot = 32 / (kSlots - kSoftmaxSlots);
+    static_assert(kHeadDim == 64 || kHeadDim == 128 || kHeadDim == 256, "head_dim 64, 128 or 256");
+
     const yvex_rocm_prefill_params &p;
     unsigned char *const lds;
     const int lane, wave, n, g;
     uint32_t head, kv_head, row0;
     // staging
     i32x4 k_rsrc, v_rsrc;
-    uint32_t k_row_bytes, v_row_bytes, lds_base, k_off[4], v_off[4];
+    uint32_t k_row_bytes, v_row_bytes, lds_base, k_off[kLoads], v_off[kLoads];
     // operand addresses inside a buffer
-    uint32_t k_addr[8], v_addr[4][2];
-    bf16x8 q[8];
-    floatx16 o[4];
+    uint32_t k_addr[kSteps], v_addr[kDimBlocks][2];
+    bf16x8 q[kSteps];
+    floatx16 o[kDimBlocks];
     float m_run, neg_m, l_run;
 
     __device__ Prefill(const yvex_rocm_prefill_params &params, unsigned char *shared)
@@ -102,19 +127,19 @@ struct Prefill {
     {
     }
 
-    // 1 KB load j (0..3) of this wave for the K or V tile `tile` into buffer `buf`.  A tile
+    // 1 KB load j (0..kLoads-1) of this wave for the K or V tile `tile` into buffer `buf`.  A tile
     // that is not wanted is still "loaded", from an offset past the range of the descriptor:
     // the range check returns zeros without touching memory, and the trip stays branch-free
     // with the same number of loads in flight.
     __device__ inline void stage_k(uint32_t tile, bool wanted, int buf, int j) const
     {
-        lds_dma_b128(lds_base + buf * kBufBytes + wave * 4096 + j * 1024, k_rsrc, k_off[j],
+        lds_dma_b128(lds_base + buf * kBufBytes + wave * (16 * kRowBytes) + j * 1024, k_rsrc, k_off[j],
                      (uint32_t)__builtin_amdgcn_readfirstlane(
                          (int)(wanted ? tile * kKeyTile * k_row_bytes : 0xfffffff0u)));
     }
     __device__ inline void stage_v(uint32_t tile, bool wanted, int buf, int j) const
     {
-        lds_dma_b128(lds_base + buf * kBufBytes + kTileBytes + wave * 4096 + j * 1024, v_rsrc,
+        lds_dma_b128(lds_base + buf * kBufBytes + kTileBytes + wave * (16 * kRowBytes) + j * 1024, v_rsrc,
                      v_off[j],
                      (uint32_t)__builtin_amdgcn_readfirstlane(
                          (int)(wanted ? tile * kKeyTile * v_row_bytes : 0xfffffff0u)));
@@ -125,10 +150,11 @@ struct Prefill {
     {
         return *reinterpret_cast<const u32x4 *>(buf + k_addr[i >> 1] + (i & 1) * 32 * kRowBytes);
     }
-    // V^T operand of O^T MFMA i (i = (mb * 2 + u) * 4 + db): dims db*32 .., keys mb*32 + 16u ..
+    // V^T operand of O^T MFMA i (i = (mb * 2 + u) * kDimBlocks + db): dims db*32 .., keys mb*32 + 16u ..
     __device__ inline u32x4 fetch_v(const unsigned char *buf, int i) const
     {
-        const int db = i & 3, base = ((i >> 3) * 32 + ((i >> 2) & 1) * 16) * kRowBytes;
+        const int db = i % kDimBlocks, grp = i / kDimBlocks;
+        const int base = ((grp >> 1) * 32 + (grp & 1) * 16) * kRowBytes;
         const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
             (lds_short4 *)(buf + v_addr[db][0] + base));
         const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
@@ -162,7 +188,7 @@ struct Prefill {
             const float alpha = m_new == -INFINITY ? 1.0f : fast_exp2(m_run - m_new);
             l_run *= alpha;
 #pragma unroll
-            for (int db = 0; db < 4; ++db) o[db] *= alpha;
+            for (int db = 0; db < kDimBlocks; ++db) o[db] *= alpha;
             m_run = m_new;
             neg_m = m_new == -INFINITY ? 0.f : -m_new;
         }
@@ -200,12 +226,13 @@ struct Prefill {
             const uint32_t row = min(row0 + n, p.query_tokens - 1u);
             const uint16_t *src = p.q + (uint64_t)row * p.q_stride + (uint64_t)head * kHeadDim + g * 8;
 #pragma unroll
-            for (int kk = 0; kk < 8; ++kk) q[kk] = as_bf16x8(load_b128(src + kk * 16));
+            for (int kk = 0; kk < kSteps; ++kk) q[kk] = as_bf16x8(load_b128(src + kk * 16));
         }
 
         // ---- tile staging: buffer loads that write LDS directly -----------------------
         // 1 KB load j of wave w fills rows 16w + 4j .. +3 of the tile; lane L owns chunk
-        // position L % 16 of row 16w + 4j + L / 16 and fetches chunk (L % 16) ^ x(row).
+        // position L % 16 of row 16w + 4j + L / 16 and fetches chunk (L % 16) ^ x(row)
+        // (rows of 128 bytes: eight rows per load, of 512 bytes: two).
         k_row_bytes = (uint32_t)p.k_stride * 2u;
         v_row_bytes = (uint32_t)p.v_stride * 2u;
         k_rsrc = raw_buffer(p.k + (uint64_t)kv_head * kHeadDim,
@@ -214,9 +241,9 @@ struct Prefill {
                             p.kv_tokens * v_row_bytes - kv_head * kRowBytes);
         lds_base = (uint32_t)__builtin_amdgcn_readfirstlane((int)lds_address_of(lds));
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int r = 16 * wave + 4 * j + (lane >> 4);
-            const uint32_t chunk = (uint32_t)((lane & 15) ^ swizzle(r));
+        for (int j = 0; j < kLoads; ++j) {
+            const int r = 16 * wave + kLoadRows * j + lane / kRowChunks;
+            const uint32_t chunk = (uint32_t)((lane % kRowChunks) ^ swizzle<kHeadDim>(r));
             k_off[j] = (uint32_t)r * k_row_bytes + chunk * 16u;
             v_off[j] = (uint32_t)r * v_row_bytes + chunk * 16u;
         }
@@ -224,25 +251,25 @@ struct Prefill {
         // ---- operand addresses inside a buffer ----------------------------------------
         // K operand (mb, kk): row mb*32 + n, chunk (2kk + g) ^ x(n); one address per kk
 #pragma unroll
-        for (int kk = 0; kk < 8; ++kk)
-            k_addr[kk] = (uint32_t)(n * kRowBytes + (((2 * kk + g) ^ swizzle(n)) << 4));
+        for (int kk = 0; kk < kSteps; ++kk)
+            k_addr[kk] = (uint32_t)(n * kRowBytes + (((2 * kk + g) ^ swizzle<kHeadDim>(n)) << 4));
         // V^T operand (db, mb, u, h): 16-lane group b = lane / 16 (dims 16 * (b & 1), key half
         // g = b / 2), lane a = lane % 16 addresses key row mb*32 + 16u + 8h + 4g + a/4 and
         // dims db*32 + 16*(b&1) + 4*(a%4) .. +3; one address per (db, h)
         {
             const int a = lane & 15, b1 = (lane >> 4) & 1;
 #pragma unroll
-            for (int db = 0; db < 4; ++db)
+            for (int db = 0; db < kDimBlocks; ++db)
 #pragma unroll
                 for (int h = 0; h < 2; ++h) {
                     const int r = 8 * h + 4 * g + (a >> 2);
-                    const int chunk = (db * 4 + 2 * b1 + ((a >> 1) & 1)) ^ swizzle(r);
+                    const int chunk = (db * 4 + 2 * b1 + ((a >> 1) & 1)) ^ swizzle<kHeadDim>(r);
                     v_addr[db][h] = (uint32_t)(kTileBytes + r * kRowBytes + (chunk << 4) + 8 * (a & 1));
                 }
         }
 
 #pragma unroll
-        for (int db = 0; db < 4; ++db)
+        for (int db = 0; db < kDimBlocks; ++db)
 #pragma unroll
             for (int i = 0; i < 16; ++i) o[db][i] = 0.f;
         m_run = -INFINITY;
@@ -263,13 +290,13 @@ struct Prefill {
 
         // ---- prologue: K(0) and V(0) land, K(1) starts, S^T of tile 0 --------------------
 #pragma unroll
-        for (int j = 0; j < 4; ++j) stage_k(0u, tiles > 0u, 0, j);
+        for (int j = 0; j < kLoads; ++j) stage_k(0u, tiles > 0u, 0, j);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) stage_v(0u, tiles > 0u, 0, j);
+        for (int j = 0; j < kLoads; ++j) stage_v(0u, tiles > 0u, 0, j);
         __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
         __syncthreads();
 #pragma unroll
-        for (int j = 0; j < 4; ++j) stage_k(1u, tiles > 1u, 1, j);
+        for (int j = 0; j < kLoads; ++j) stage_k(1u, tiles > 1u, 1, j);
         floatx16 s_cur[2];
         if (my_tiles != 0u) {
             const unsigned char *buf = lds;
@@ -277,10 +304,10 @@ struct Prefill {
 #pragma unroll
             for (int i = 0; i < kDepth; ++i) frag[i] = fetch_k(buf, i);
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
+            for (int i = 0; i < kHalfSlots; ++i) {
                 const floatx16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
                 s_cur[i & 1] = mfma_32x32x16(as_bf16x8(frag[i % kDepth]), q[i >> 1], i < 2 ? zero : s_cur[i & 1]);
-                if (i + kDepth < 16) frag[i % kDepth] = fetch_k(buf, i + kDepth);
+                if (i + kDepth < kHalfSlots) frag[i % kDepth] = fetch_k(buf, i + kDepth);
                 __builtin_amdgcn_sched_barrier(0);
             }
             if (needs_mask(0u)) mask_tile(s_cur, 0u);
@@ -300,9 +327,9 @@ struct Prefill {
             if (t >= my_tiles) {
                 // nothing of this tile is visible to the wave: it only keeps staging
 #pragma unroll
-                for (int j = 0; j < 4; ++j) stage_k(t + 2u, stage_next_k, cur, j);
+                for (int j = 0; j < kLoads; ++j) stage_k(t + 2u, stage_next_k, cur, j);
 #pragma unroll
-                for (int j = 0; j < 4; ++j) stage_v(t + 1u, stage_next_v, nxt, j);
+                for (int j = 0; j < kLoads; ++j) stage_v(t + 1u, stage_next_v, nxt, j);
                 return;
             }
             // S^T of tile t+1 is computed in every trip; on the wave's last tile the product
@@ -313,33 +340,35 @@ struct Prefill {
             uint32_t pk[16];  // bf16 pairs of tile t: [mb * 8 + u * 4 + pair]
             float lsum = 0.f, mloc = -INFINITY;
             u32x4 frag[kDepth];
-            // operand of slot i: K fragments for slots 0..15, V^T fragments for 16..31
+            // operand of slot i: K fragments for the first half of the slots, V^T fragments for the second
             auto fetch = [&](int i) -> u32x4 {
-                return i < 16 ? fetch_k(kbuf, i) : fetch_v(vbuf, i - 16);
+                return i < kHalfSlots ? fetch_k(kbuf, i) : fetch_v(vbuf, i - kHalfSlots);
             };
 #pragma unroll
             for (int i = 0; i < kDepth; ++i) frag[i] = fetch(i);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int i = 0; i < 32; ++i) {
+            for (int i = 0; i < kSlots; ++i) {
                 // ---- the MFMA of this slot ----
-                if (i < 16) {
+                if (i < kHalfSlots) {
                     const floatx16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
                     s_next[i & 1] = mfma_32x32x16(as_bf16x8(frag[i % kDepth]), q[i >> 1],
                                                   i < 2 ? zero : s_next[i & 1]);
                 } else {
-                    const int j = i - 16, grp = j >> 2;  // grp = mb * 2 + u
+                    const int j = i - kHalfSlots, grp = j / kDimBlocks;  // grp = mb * 2 + u
                     const u32x4 w = {pk[grp * 4 + 0], pk[grp * 4 + 1], pk[grp * 4 + 2], pk[grp * 4 + 3]};
-                    o[j & 3] = mfma_32x32x16(as_bf16x8(frag[i % kDepth]), as_bf16x8(w), o[j & 3]);
+                    o[j % kDimBlocks] = mfma_32x32x16(as_bf16x8(frag[i % kDepth]), as_bf16x8(w), o[j % kDimBlocks]);
                 }
-                if (i + kDepth < 32) frag[i % kDepth] = fetch(i + kDepth);
+                if (i + kDepth < kSlots) frag[i % kDepth] = fetch(i + kDepth);
                 // ---- one LDS-DMA load of a later tile ----
-                if (i < 4) stage_k(t + 2u, stage_next_k, cur, i);
-                else if (i < 8) stage_v(t + 1u, stage_next_v, nxt, i - 4);
-                // ---- a slice of the softmax of tile t: elements e with 3e/4 == i ----
+                if (i < kLoads) stage_k(t + 2u, stage_next_k, cur, i);
+                else if (i < 2 * kLoads) stage_v(t + 1u, stage_next_v, nxt, i - kLoads);
+                // ---- a slice of the softmax of tile t: the 32 elements spread evenly over
+                //      the first three quarters of the slots (3e/4 == i), each before the
+                //      O^T MFMA that takes its probability ----
 #pragma unroll
-                for (int e = 0; e < 32; ++e) {
-                    if ((3 * e) / 4 != i) continue;
+                for (int e = (i * 32 + kSoftmaxSlots - 1) / kSoftmaxSlots;
+                     e < ((i + 1) * 32 + kSoftmaxSlots - 1) / kSoftmaxSlots && e < 32; ++e) {
                     const int mb = e >> 4, r = e & 15;
                     const float pe = fast_exp2(__builtin_fmaf(s_cur[mb][r], p.scale_log2, neg_m));
                     s_cur[mb][r] = pe;
@@ -347,11 +376,17 @@ struct Prefill {
                     if (r & 1) pk[mb * 8 + (r >> 1)] = pack_bf16x2(s_cur[mb][r - 1], pe);
                 }
                 // ---- the per-lane maximum of tile t+1, once its scores are complete ----
-                if (i >= 24) {
-                    const int k4 = (i - 24) * 4;  // four of the 32 scores per slot
-                    const int mb = k4 >> 4, r = k4 & 15;
-                    mloc = fmaxf(fmaxf(mloc, s_next[mb][r]),
-                                 fmaxf(fmaxf(s_next[mb][r + 1], s_next[mb][r + 2]), s_next[mb][r + 3]));
+                if (i >= kSoftmaxSlots) {
+                    const int first = (i - kSoftmaxSlots) * kMaxPerSlot;  // four of the 32 scores per slot
+#pragma unroll
+                    for (int k4 = first; k4 < first + kMaxPerSlot; k4 += 4) {
+                        const int mb = k4 >> 4, r = k4 & 15;
+                        if (kMaxPerSlot >= 4)
+                            mloc = fmaxf(fmaxf(mloc, s_next[mb][r]),
+                                         fmaxf(fmaxf(s_next[mb][r + 1], s_next[mb][r + 2]), s_next[mb][r + 3]));
+                        else
+                            mloc = fmaxf(mloc, fmaxf(s_next[mb][r], s_next[mb][r + 1]));
+                    }
                     asm volatile("" : "+v"(mloc));  // keeps this slice in its slot
                 }
                 __builtin_amdgcn_sched_barrier(0);
@@ -385,7 +420,7 @@ struct Prefill {
         bool bad = false;
         uint16_t *dst = p.out + ((uint64_t)row * p.query_heads + head) * kHeadDim;
 #pragma unroll
-        for (int db = 0; db < 4; ++db)
+        for (int db = 0; db < kDimBlocks; ++db)
 #pragma unroll
             for (int grp = 0; grp < 4; ++grp) {
                 const float a0 = o[db][grp * 4 + 0] * inv, a1 = o[db][grp * 4 + 1] * inv;
@@ -409,11 +444,18 @@ struct Prefill {
 }  // namespace
 
 // grid = query heads x query tiles of YVEX_ROCM_PREFILL_ROWS rows, block 256,
-// LDS 2 x (K + V) tiles; two workgroups per CU.
-extern "C" __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
-yvex_rocm_prefill_bf16(const yvex_rocm_prefill_params p)
-{
-    static_assert(YVEX_ROCM_PREFILL_ROWS == kRowsPerBlock, "host and kernel agree on the query tile");
-    __shared__ __attribute__((aligned(16))) unsigned char lds[2 * kBufBytes];
-    Prefill(p, lds).run();
-}
+// LDS 2 x (K + V) tiles.  `waves`: waves per SIMD the register budget is sized for: two
+// workgroups per CU for head_dim 64 and 128; head_dim 256 keeps 128 accumulator, 64 query and
+// 64 score registers per lane and its tiles fill 128 KB of LDS: one workgroup per CU.
+#define YVEX_PREFILL_KERNEL(name, head_dim, waves)                                                        \
+    extern "C" __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(waves, waves)))  \
+    name(const yvex_rocm_prefill_params p)                                                                \
+    {                                                                                                     \
+        static_assert(YVEX_ROCM_PREFILL_ROWS == kRowsPerBlock, "host and kernel agree on the query tile"); \
+        __shared__ __attribute__((aligned(16))) unsigned char lds[2 * Prefill<head_dim>::kBufBytes];      \
+        Prefill<head_dim>(p, lds).run();                                                                  \
+    }
+
+YVEX_PREFILL_KERNEL(yvex_rocm_prefill_bf16, 128, 2)
+YVEX_PREFILL_KERNEL(yvex_rocm_prefill_bf16_64, 64, 2)
+YVEX_PREFILL_KERNEL(yvex_rocm_prefill_bf16_256, 256, 1)

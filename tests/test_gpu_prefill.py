@@ -102,7 +102,7 @@ def test_prefill_refusals(backend):
     with pytest.raises(YvexError) as e:                      # query range beyond KV history
         run_prefill(backend, q, k, k, query_start=1)
     assert e.value.code == B.YVEX_ERR_INVALID_ARG
-    req = backend.attention_requirement(4, 4, 2, 1, 64, dtype=B.DTYPE_BF16,
+    req = backend.attention_requirement(4, 4, 2, 1, 96, dtype=B.DTYPE_BF16,
                                         contract=B.NUMERIC_BF16_F32_ACCUMULATE)
     with pytest.raises(YvexError) as e:                      # head dimension the MFMA path lacks
         backend.attention_workspace_required(req)
@@ -131,3 +131,48 @@ def test_prefill_long_sequences(backend, tq, tk, start, hq, hkv):
     assert rc == 0
     assert_close_bf16(got, ref, "long prefill %d/%d" % (tq, tk))
     assert_lse(lse, ref_lse, "long prefill %d/%d" % (tq, tk))
+
+
+@pytest.mark.parametrize("d", [64, 256])
+@pytest.mark.parametrize("tq,tk,start,hq,hkv,causal", [
+    (2, 2, 0, 2, 1, True), (65, 65, 0, 5, 1, True), (257, 257, 0, 4, 2, True),
+    (300, 300, 0, 6, 2, False), (3, 131, 128, 8, 2, True), (200, 1000, 800, 4, 1, True),
+    (1, 700, 699, 8, 2, True),          # one query token: a one-row tile of the same kernel
+])
+def test_prefill_other_head_dimensions(backend, d, tq, tk, start, hq, hkv, causal):
+    """Head dimensions 64 and 256 are the same kernel with other counts (k-steps, dim blocks,
+    loads per tile, LDS swizzle for 128-byte rows)."""
+    rng = np.random.default_rng(d * 100000 + tq * 1000 + tk)
+    q = bf16_normal(rng, (tq, hq, d))
+    k = bf16_normal(rng, (tk, hkv, d))
+    v = bf16_normal(rng, (tk, hkv, d))
+    got, lse, facts = run_prefill(backend, q, k, v, query_start=start, causal=causal)
+    rc, ref, _, ref_lse = ORACLE.gqa_bf16(q, k, v, query_start=start, causal=causal)
+    assert rc == 0
+    label = "d=%d tq=%d tk=%d start=%d %s" % (d, tq, tk, start, "causal" if causal else "full")
+    assert_close_bf16(got, ref, label)
+    assert_lse(lse, ref_lse, label)
+    assert facts.kernel_launches == 1 and facts.accelerated_matrix_launches == 1
+    if causal and start == 0:
+        for h in range(hq):
+            assert np.array_equal(got[0, h], v[0, h // (hq // hkv)])
+
+
+@pytest.mark.parametrize("t,hq,hkv,d", [(1024, 24, 4, 256), (1024, 16, 4, 64)])
+def test_prefill_reference_qwen_patterns(backend, t, hq, hkv, d):
+    """The geometry of the reference's own Qwen attention test (24 query heads, 4 KV heads,
+    head dimension 256: tests/unit/cuda/quant_qtype.c:2413-2454) and its narrow sibling, as
+    causal prefill under the bf16 contract, with per-head scales as in configuration 2."""
+    rng = np.random.default_rng(t + d)
+    sq = rng.uniform(0.5, 1.5, size=(1, hq, 1)).astype(np.float32)
+    skv = rng.uniform(0.5, 1.5, size=(1, hkv, 1)).astype(np.float32)
+    q = ORACLE.bf16_encode(rng.standard_normal((t, hq, d)).astype(np.float32) * sq)
+    k = ORACLE.bf16_encode(rng.standard_normal((t, hkv, d)).astype(np.float32) * skv)
+    v = ORACLE.bf16_encode(rng.standard_normal((t, hkv, d)).astype(np.float32) * skv)
+    got, lse, _ = run_prefill(backend, q, k, v)
+    rc, ref, _, ref_lse = ORACLE.gqa_bf16(q, k, v, query_start=0, causal=True)
+    assert rc == 0
+    assert_close_bf16(got, ref, "qwen pattern d=%d" % d)
+    assert_lse(lse, ref_lse, "qwen pattern d=%d" % d)
+    again, lse2, _ = run_prefill(backend, q, k, v)
+    assert np.array_equal(got, again) and np.array_equal(lse, lse2)

@@ -713,7 +713,7 @@ def test_attention_execute_contracts_facts_and_workspace(fake_runtime):
         for mutate, code in [(dict(query_heads=9), B.YVEX_ERR_INVALID_ARG),
                              (dict(query_start=1), B.YVEX_ERR_INVALID_ARG),
                              (dict(key_token_stride=255), B.YVEX_ERR_INVALID_ARG),
-                             (dict(head_dimension=64), B.YVEX_ERR_UNSUPPORTED),
+                             (dict(head_dimension=96), B.YVEX_ERR_UNSUPPORTED),
                              (dict(deterministic=0), B.YVEX_ERR_UNSUPPORTED),
                              (dict(output_dtype=B.DTYPE_F32), B.YVEX_ERR_UNSUPPORTED),
                              (dict(numeric_contract=7), B.YVEX_ERR_UNSUPPORTED),
@@ -731,7 +731,7 @@ def test_paged_and_mla_admission():
     with Backend() as b:
         ok = b.paged_requirement(4, 32, 8, 128, 16, 100, 64, 1024)
         assert b.paged_decode_workspace_required(ok) > 0
-        for mutate, code in [(dict(head_dimension=64), B.YVEX_ERR_UNSUPPORTED),
+        for mutate, code in [(dict(head_dimension=96), B.YVEX_ERR_UNSUPPORTED),
                              (dict(page_tokens=32), B.YVEX_ERR_UNSUPPORTED),
                              (dict(kv_storage=9), B.YVEX_ERR_UNSUPPORTED),
                              (dict(numeric_contract=B.NUMERIC_EXACT_F32), B.YVEX_ERR_UNSUPPORTED),
@@ -832,7 +832,7 @@ def test_kv_append_admission():
         q_pool = b.tensor("qp", B.DTYPE_I8, (pages * hkv * 2176,))
         assert b.kv_append_execute(key, value, rows, starts, counts, table, q_pool, q_pool, hkv,
                                    pages, 8, storage=B.KV_Q8_0).kernel_launches == 1
-        for kwargs, code in [(dict(head_dimension=64), B.YVEX_ERR_UNSUPPORTED),
+        for kwargs, code in [(dict(head_dimension=96), B.YVEX_ERR_UNSUPPORTED),
                              (dict(page_tokens=32), B.YVEX_ERR_UNSUPPORTED),
                              (dict(storage=7), B.YVEX_ERR_UNSUPPORTED),
                              (dict(rotary_dimension=24, cosine=cosine, sine=sine), B.YVEX_ERR_UNSUPPORTED),
