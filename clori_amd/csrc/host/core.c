@@ -692,13 +692,6 @@ const yvex_backend_transformer_operations *yvex_backend_transformer_operations_g
                : NULL;
 }
 
-const yvex_backend_rocm_attention_operations *yvex_backend_rocm_attention_operations_get(
-    const yvex_backend *backend)
-{
-    return backend && backend->vtable && backend->vtable->rocm_attention_operations
-               ? backend->vtable->rocm_attention_operations(backend)
-               : NULL;
-}
 
 /* The encoded-attention transaction (include/yvex/internal/backend.h:193-198).  The
  * reference's only implementation is the CUDA one (src/backend/cuda/attention.c:1924);

@@ -12,8 +12,12 @@
 #include "yvex_rocm.h"
 
 /* The slots of the reference vtable (src/backend/private.h:16-81) that lie on the
- * attention path.  Everything else (embed, matmul, MoE, sampling, ...) is not
- * published by this backend: its dispatchers answer YVEX_ERR_UNSUPPORTED. */
+ * attention path, under the reference's names.  Everything else (embed, matmul, MoE,
+ * sampling, ...) is not published by this backend: its dispatchers answer
+ * YVEX_ERR_UNSUPPORTED.  There is no slot the reference's table lacks: the operations that
+ * have no reference counterpart are reached through
+ * yvex_backend_rocm_attention_operations_get, which belongs to the ROCm arm and tests the
+ * backend's kind itself. */
 typedef struct yvex_backend_vtable {
     int (*close)(yvex_backend *, yvex_error *);
     int (*memory_stats)(const yvex_backend *, yvex_backend_memory_stats *, yvex_error *);
@@ -47,8 +51,6 @@ typedef struct yvex_backend_vtable {
                         int, yvex_device_tensor *, yvex_device_tensor *, yvex_device_tensor *,
                         yvex_error *);
     const yvex_backend_transformer_operations *(*transformer_operations)(const yvex_backend *);
-    const yvex_backend_rocm_attention_operations *(*rocm_attention_operations)(
-        const yvex_backend *);
 } yvex_backend_vtable;
 
 struct yvex_backend {

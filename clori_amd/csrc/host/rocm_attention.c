@@ -1503,10 +1503,15 @@ const yvex_backend_transformer_operations *yvex_rocm_transformer_operations(
                : NULL;
 }
 
-const yvex_backend_rocm_attention_operations *yvex_rocm_attention_operations(
+/* The operations without a reference counterpart.  Not a vtable slot (the reference's table
+ * has none for them): a function of the ROCm arm that answers for ROCm backends with an
+ * admitted bundle and NULL ("not published") for everything else. */
+const yvex_backend_rocm_attention_operations *yvex_backend_rocm_attention_operations_get(
     const yvex_backend *backend)
 {
-    const yvex_rocm_backend_state *state = yvex_rocm_state(backend);
+    const yvex_rocm_backend_state *state;
+    if (!backend || backend->kind != YVEX_BACKEND_KIND_ROCM) return NULL;
+    state = yvex_rocm_state(backend);
     return state && state->kernel_bundle_state == YVEX_ROCM_KERNEL_BUNDLE_ADMITTED
                ? &rocm_attention_ops
                : NULL;

@@ -573,7 +573,6 @@ static const yvex_backend_vtable rocm_vtable = {
     .query_capability = yvex_rocm_query_capability,
     .op_attention = yvex_rocm_op_attention,
     .transformer_operations = yvex_rocm_transformer_operations,
-    .rocm_attention_operations = yvex_rocm_attention_operations,
 };
 
 static int parse_device(const char *device, int *index)

@@ -165,7 +165,4 @@ int yvex_rocm_op_attention(yvex_backend *backend, const yvex_device_tensor *quer
                            yvex_error *err);
 const yvex_backend_transformer_operations *yvex_rocm_transformer_operations(
     const yvex_backend *backend);
-const yvex_backend_rocm_attention_operations *yvex_rocm_attention_operations(
-    const yvex_backend *backend);
-
 #endif /* YVEX_ROCM_STATE_H */
