@@ -466,8 +466,13 @@ __device__ __forceinline__ void mla_decode(const yvex_rocm_mla_params &p, unsign
     {
         const uint64_t slot0 = ((uint64_t)batch * p.slot_stride + p.first_slot + chunk) * p.heads + wave * kHeadsPerWave;
         uint16_t *dst = p.part_acc + slot0 * kValueDim + lane * 8;
+        // every workgroup starts its 32 rows at another one: the rows of all workgroups are
+        // 1 KB apart at the same offsets of 128 KB regions, and written in step they would all
+        // be in the same memory channels at the same time
+        const int skew = (int)((chunk * 5u + batch * 3u) & 31u);
 #pragma unroll 8
-        for (int hh = 0; hh < kHeadsPerWave; ++hh) {
+        for (int i = 0; i < kHeadsPerWave; ++i) {
+            const int hh = (i + skew) & (kHeadsPerWave - 1);
             const u32x4 v = *reinterpret_cast<const u32x4 *>(rows + hh * kOutPitch + lane * 16);
             *reinterpret_cast<u32x4 *>(dst + (uint64_t)hh * kValueDim) = v;
         }
