@@ -9,6 +9,17 @@
 #include <stdatomic.h>
 #include <stdint.h>
 
+#ifdef YVEX_ROCM_IN_TREE
+/* Inside the reference tree (the root of the tree on the include path, as for the CUDA arm)
+ * the backend object, the vtable and the helpers below are the tree's own; what remains is
+ * the one function of the dispatch layer the arm calls that the tree keeps private to its
+ * CUDA arm (src/backend/cuda/backend.c:1598-1623). */
+#include "src/backend/private.h"
+#include <yvex/internal/core.h>
+#include "yvex_rocm.h"
+int yvex_backend_shared_owner_acquire(yvex_backend *owner, yvex_error *err);
+#else
+
 #include "yvex_rocm.h"
 
 /* The slots of the reference vtable (src/backend/private.h:16-81) that lie on the
@@ -129,7 +140,6 @@ int yvex_core_u64_mul(unsigned long long left, unsigned long long right,
                       unsigned long long *out);
 void yvex_core_text_copy(char *destination, size_t capacity, const char *source);
 void yvex_error_setf(yvex_error *err, yvex_status code, const char *where, const char *fmt, ...);
-unsigned long long yvex_dtype_element_bytes(yvex_dtype dtype);
 
 /* core.c: lease of a session backend on its primary (src/backend/cuda/backend.c:1598-1623) */
 int yvex_backend_shared_owner_acquire(yvex_backend *owner, yvex_error *err);
@@ -152,5 +162,7 @@ int yvex_backend_validate_attention(const yvex_backend *backend, const yvex_devi
                                     yvex_device_tensor *out, unsigned long long *head_dim_out,
                                     unsigned long long *kv_elements_out, const char *where,
                                     yvex_error *err);
+
+#endif /* !YVEX_ROCM_IN_TREE */
 
 #endif /* YVEX_ROCM_HOST_PRIVATE_H */

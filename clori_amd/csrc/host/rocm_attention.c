@@ -442,7 +442,7 @@ static int view_ok(const yvex_backend *backend, const yvex_device_tensor *tensor
     unsigned long long bytes;
     if (!backend_tensor_owner_is(backend, tensor) || (require_written && !tensor->is_written) ||
         tensor->dtype != dtype || !tensor->data ||
-        !yvex_core_u64_mul(elements, yvex_dtype_element_bytes(dtype), &bytes) ||
+        !yvex_core_u64_mul(elements, yvex_rocm_dtype_bytes(dtype), &bytes) ||
         tensor->bytes != bytes)
         return 0;
     if (!yvex_rocm_tensor_backed(tensor)) {
@@ -803,9 +803,9 @@ static int paged_decode_execute_common(yvex_backend *backend,
     if (!yvex_core_u64_mul(r->pool_pages * r->key_value_heads, block_bytes, &pool_bytes) ||
         !view_ok(backend, request->query, YVEX_DTYPE_BF16, q_elements, 1) ||
         !view_ok(backend, request->key_pages, pool_dtype,
-                 pool_bytes / yvex_dtype_element_bytes(pool_dtype), 1) ||
+                 pool_bytes / yvex_rocm_dtype_bytes(pool_dtype), 1) ||
         !view_ok(backend, request->value_pages, pool_dtype,
-                 pool_bytes / yvex_dtype_element_bytes(pool_dtype), 1) ||
+                 pool_bytes / yvex_rocm_dtype_bytes(pool_dtype), 1) ||
         !view_ok(backend, request->page_table, YVEX_DTYPE_I32, table_elements, 1) ||
         !view_ok(backend, request->context_tokens, YVEX_DTYPE_I32, r->sessions, 1) ||
         !view_ok(backend, request->output, YVEX_DTYPE_BF16, q_elements, 0) ||
@@ -1314,9 +1314,9 @@ static int rocm_kv_append_execute(yvex_backend *backend, const yvex_rocm_kv_appe
         !view_ok(backend, request->token_count, YVEX_DTYPE_I32, r->sessions, 1) ||
         !view_ok(backend, request->page_table, YVEX_DTYPE_I32, r->sessions * r->page_table_stride, 1) ||
         !view_ok(backend, request->k_pool, pool_dtype,
-                 pool_bytes / yvex_dtype_element_bytes(pool_dtype), 0) ||
+                 pool_bytes / yvex_rocm_dtype_bytes(pool_dtype), 0) ||
         !view_ok(backend, request->v_pool, pool_dtype,
-                 pool_bytes / yvex_dtype_element_bytes(pool_dtype), 0))
+                 pool_bytes / yvex_rocm_dtype_bytes(pool_dtype), 0))
         return view_refusal(backend, err, where,
                       "rows, tables, descriptors and pools must be tensors of this backend with "
                       "the declared geometry");
@@ -1405,7 +1405,7 @@ static int rocm_history_append_execute(yvex_backend *backend,
     if (dtype != YVEX_DTYPE_BF16 && dtype != YVEX_DTYPE_F32)
         return refuse(err, YVEX_ERR_UNSUPPORTED, where,
                       "ROCm history append takes BF16 or F32 rows and histories of the same type");
-    piece = 16ull / yvex_dtype_element_bytes(dtype);
+    piece = 16ull / yvex_rocm_dtype_bytes(dtype);
     if (r->head_dimension % piece || r->head_dimension > 256ull || (k_stride | v_stride) % piece ||
         (r->rotary_mode != YVEX_ROCM_ROTARY_BF16_STAGED && r->rotary_mode != YVEX_ROCM_ROTARY_F32_ROUNDED) ||
         r->rotary_dimension > r->head_dimension || r->rotary_dimension % (2ull * piece) ||

@@ -104,6 +104,18 @@ struct yvex_rocm_graph {
     struct yvex_rocm_graph *next; /* the backend's list of unreleased sequences */
 };
 
+/* Bytes of one element of the dtypes a device tensor of this backend can have; 0 for any other. */
+static inline unsigned long long yvex_rocm_dtype_bytes(yvex_dtype dtype)
+{
+    switch (dtype) {
+    case YVEX_DTYPE_F32: case YVEX_DTYPE_I32: return 4ull;
+    case YVEX_DTYPE_F16: case YVEX_DTYPE_BF16: case YVEX_DTYPE_I16: return 2ull;
+    case YVEX_DTYPE_F64: case YVEX_DTYPE_I64: return 8ull;
+    case YVEX_DTYPE_I8: return 1ull;
+    default: return 0ull;
+    }
+}
+
 static inline yvex_rocm_backend_state *yvex_rocm_state(const yvex_backend *backend)
 {
     return backend && backend->kind == YVEX_BACKEND_KIND_ROCM

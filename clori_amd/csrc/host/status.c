@@ -75,14 +75,3 @@ int yvex_core_u64_mul(unsigned long long left, unsigned long long right, unsigne
     *out = left * right;
     return 1;
 }
-
-unsigned long long yvex_dtype_element_bytes(yvex_dtype dtype)
-{
-    switch (dtype) {
-    case YVEX_DTYPE_F32: case YVEX_DTYPE_I32: return 4ull;
-    case YVEX_DTYPE_F16: case YVEX_DTYPE_BF16: case YVEX_DTYPE_I16: return 2ull;
-    case YVEX_DTYPE_F64: case YVEX_DTYPE_I64: return 8ull;
-    case YVEX_DTYPE_I8: return 1ull;
-    default: return 0ull;
-    }
-}

@@ -21,6 +21,42 @@
 extern "C" {
 #endif
 
+/*
+ * Two ways to compile against this header.  By default it is self-contained: the reference's
+ * own types are re-declared below with the reference's names, members and values.  With
+ * YVEX_ROCM_IN_TREE defined (the ROCm arm built inside the reference tree) those
+ * declarations come from the reference's headers instead and this header adds only what the
+ * reference lacks; the values the integration adds to the reference's enumerations (the
+ * ROCm operation variants, the bf16 numeric contract, the two ROCm report kinds) are given
+ * as constants of the enumeration's type until the enumerations themselves carry them.
+ * Function declarations are not hidden in either mode: where the reference declares the
+ * same function, the compiler holds the two declarations against each other.
+ */
+#ifdef YVEX_ROCM_IN_TREE
+#include <yvex/backend.h>
+#include <yvex/internal/backend.h>
+#include <yvex/internal/core.h>
+#include <yvex/internal/transformer.h>
+#ifndef YVEX_BACKEND_VARIANT_ROCM_FIRST
+#define YVEX_BACKEND_VARIANT_ROCM_FIRST ((yvex_backend_operation_variant)64)
+#define YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_F32 ((yvex_backend_operation_variant)64)
+#define YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_BF16 ((yvex_backend_operation_variant)65)
+#define YVEX_BACKEND_VARIANT_ROCM_ATTENTION_PAGED_BF16 ((yvex_backend_operation_variant)66)
+#define YVEX_BACKEND_VARIANT_ROCM_ATTENTION_PAGED_Q8_0 ((yvex_backend_operation_variant)67)
+#define YVEX_BACKEND_VARIANT_ROCM_ATTENTION_MLA_BF16 ((yvex_backend_operation_variant)68)
+#define YVEX_BACKEND_VARIANT_ROCM_END ((yvex_backend_operation_variant)69)
+#endif
+#ifndef YVEX_TRANSFORMER_ATTENTION_NUMERIC_BF16_F32_ACCUMULATE
+#define YVEX_TRANSFORMER_ATTENTION_NUMERIC_BF16_F32_ACCUMULATE \
+    ((yvex_transformer_attention_numeric_contract)2)
+#endif
+#ifndef YVEX_BACKEND_REPORT_ROCM_INFO
+#define YVEX_BACKEND_REPORT_ROCM_INFO ((yvex_backend_report_kind)3)
+#define YVEX_BACKEND_REPORT_ROCM_BANDWIDTH ((yvex_backend_report_kind)4)
+#endif
+#endif /* YVEX_ROCM_IN_TREE */
+
+#ifndef YVEX_ROCM_IN_TREE
 /* ---- status and error: include/yvex/core.h:13-48 ------------------------ */
 typedef enum {
     YVEX_OK = 0,
@@ -220,6 +256,8 @@ struct yvex_device_tensor {
     int is_written, host_accessible, borrowed_host;
 };
 
+#endif /* !YVEX_ROCM_IN_TREE */
+
 /* ---- lifecycle: include/yvex/backend.h:143-160, src/backend/core.c:255-416 --- */
 /* Opens kind ROCM only; any other kind is YVEX_ERR_UNSUPPORTED ("backend %s is not
  * implemented", src/backend/core.c:280-283).  `device` is NULL / "" / "0".."N". */
@@ -324,11 +362,13 @@ const char *yvex_backend_capability_state_name(yvex_backend_capability_state sta
 const char *yvex_backend_capability_reason_name(yvex_backend_capability_reason reason);
 
 /* ---- reusable device workspace: src/backend/residency.c:207-283 ----------- */
+#ifndef YVEX_ROCM_IN_TREE
 typedef enum {
     YVEX_BACKEND_RESIDENT_INVALID = -1,
     YVEX_BACKEND_RESIDENT_MISS = 0,
     YVEX_BACKEND_RESIDENT_HIT = 1
 } yvex_backend_resident_result;
+#endif /* !YVEX_ROCM_IN_TREE */
 int yvex_backend_workspace_attach(yvex_backend *backend, const yvex_device_tensor *device_tensor,
                                   unsigned long long generation, yvex_error *err);
 void yvex_backend_workspace_detach(yvex_backend *backend);
@@ -346,6 +386,7 @@ int yvex_backend_op_attention(yvex_backend *backend, const yvex_device_tensor *q
                               yvex_error *err);
 
 /* ---- multi-token attention contract: include/yvex/internal/transformer.h:245-275 ---- */
+#ifndef YVEX_ROCM_IN_TREE
 typedef enum {
     YVEX_TRANSFORMER_ATTENTION_LAYOUT_UNKNOWN = 0,
     YVEX_TRANSFORMER_ATTENTION_LAYOUT_TOKEN_HEAD_DIM
@@ -455,6 +496,7 @@ typedef struct yvex_backend_transformer_operations {
     int (*dense_decoder_execute)(yvex_backend *, const yvex_transformer_dense_decoder_request *,
                                  yvex_transformer_dense_decoder_result *, yvex_error *);
 } yvex_backend_transformer_operations;
+#endif /* !YVEX_ROCM_IN_TREE */
 /* include/yvex/internal/backend.h:211-212; NULL when the kernel bundle is not admitted. */
 const yvex_backend_transformer_operations *yvex_backend_transformer_operations_get(
     const yvex_backend *backend);
@@ -468,6 +510,7 @@ const yvex_backend_transformer_operations *yvex_backend_transformer_operations_g
  * YVEX_ERR_UNSUPPORTED, the same answer query_capability gives for
  * YVEX_BACKEND_VARIANT_ATTENTION_ENCODED.  Nothing of the job is read and `output` is left
  * untouched, so the job and output records stay opaque here. */
+#ifndef YVEX_ROCM_IN_TREE
 typedef struct yvex_backend_attention_job yvex_backend_attention_job;
 typedef struct yvex_backend_attention_output yvex_backend_attention_output;
 typedef struct yvex_backend_attention_completion yvex_backend_attention_completion;
@@ -489,6 +532,7 @@ typedef struct {
     const char *stage;
     unsigned long long expected, actual;
 } yvex_backend_attention_failure;
+#endif /* !YVEX_ROCM_IN_TREE */
 int yvex_backend_attention_execute(yvex_backend *backend, const yvex_backend_attention_job *job,
                                    yvex_backend_attention_output *output,
                                    yvex_backend_attention_failure *failure, yvex_error *err);
@@ -547,10 +591,12 @@ typedef struct yvex_rocm_paged_decode_request {
  */
 /* Rotary position policy of an attention layer: the fields the rotation reads
  * (include/yvex/internal/backend.h:51-54, same names and order). */
+#ifndef YVEX_ROCM_IN_TREE
 typedef struct {
     unsigned long long theta, scaling_factor, original_context;
     unsigned long long beta_fast, beta_slow, rope_dimensions;
 } yvex_backend_attention_position;
+#endif /* !YVEX_ROCM_IN_TREE */
 
 typedef struct yvex_rocm_mla_decode_requirement {
     unsigned long long batch, heads, key_dimension, value_dimension;
@@ -766,6 +812,7 @@ int yvex_backend_rocm_completion_mode_set(yvex_backend *backend, yvex_rocm_compl
  * write).  The coherent-host fields are for unified-memory parts and stay zero here; the
  * identity strings are left empty.  The first successful probe is kept and returned again.
  */
+#ifndef YVEX_ROCM_IN_TREE
 #define YVEX_BACKEND_BANDWIDTH_SCHEMA_V1 1u
 #define YVEX_BACKEND_BANDWIDTH_SAMPLE_COUNT 5u
 #define YVEX_SHA256_HEX_BYTES 65u
@@ -779,6 +826,7 @@ typedef struct {
     unsigned long long sustainable_coherent_host_bytes_per_second;
     char kernel_bundle_identity[YVEX_SHA256_HEX_BYTES], identity[YVEX_SHA256_HEX_BYTES];
 } yvex_backend_bandwidth_evidence;
+#endif /* !YVEX_ROCM_IN_TREE */
 int yvex_backend_bandwidth_probe(yvex_backend *backend, yvex_backend_bandwidth_evidence *out,
                                  yvex_error *err);
 
@@ -842,6 +890,7 @@ int yvex_backend_rocm_report_get(const yvex_backend *backend, yvex_backend_rocm_
  * failed: available = 0, the reason text, exit_code 5.  `variants` holds the reference's
  * variants in order, then this backend's attention variants.
  */
+#ifndef YVEX_ROCM_IN_TREE
 typedef enum {
     YVEX_BACKEND_REPORT_CAPABILITIES = 0,
     YVEX_BACKEND_REPORT_CUDA_INFO,
@@ -879,6 +928,7 @@ typedef struct {
     unsigned int kernel_image_count, kernel_function_count;
     char driver_library[256];
 } yvex_backend_report;
+#endif /* !YVEX_ROCM_IN_TREE */
 int yvex_backend_report_build(const yvex_backend_report_request *request,
                               yvex_backend_report *report, yvex_error *err);
 const char *yvex_backend_bundle_admission_name(yvex_backend_bundle_admission admission);
@@ -897,6 +947,7 @@ int yvex_rocm_info_command(int argc, char **argv);
  * percentiles sample[(count * p + 99) / 100 - 1], the mean and the population standard
  * deviation, and stores them as whole nanoseconds.  Samples must be finite and positive.
  */
+#ifndef YVEX_ROCM_IN_TREE /* in the tree: include/yvex/internal/benchmark.h */
 typedef enum {
     YVEX_RUNTIME_BENCHMARK_MINIMUM = 0,
     YVEX_RUNTIME_BENCHMARK_P50,
@@ -918,6 +969,7 @@ int yvex_runtime_benchmark_samples_summarize(double *seconds, unsigned long long
 /* Field name of a statistic in a benchmark record ("minimum_ns", "p50_ns", ...;
  * src/runtime/benchmark.c:127-140); device timing prefixes it with "device_". */
 const char *yvex_runtime_benchmark_statistic_name(yvex_runtime_benchmark_statistic statistic);
+#endif
 
 /* ---- scalar and block codecs (host): src/gguf/quant_scalar.c:40-143,
  *      src/gguf/quant_block.c:160-186,819-833 ------------------------------- */
@@ -925,8 +977,10 @@ float yvex_quant_f16_decode(unsigned short bits);
 unsigned short yvex_quant_f16_encode(float value);
 float yvex_quant_bf16_decode(unsigned short bits);
 unsigned short yvex_quant_bf16_encode(float value);
+#ifndef YVEX_QUANT_Q8_0_ELEMENTS
 #define YVEX_QUANT_Q8_0_ELEMENTS 32u
 #define YVEX_QUANT_Q8_0_BYTES 34u
+#endif
 /* Row forms (elements % 32 == 0).  encode refuses an unrepresentable scale with
  * YVEX_ERR_BOUNDS; decode refuses a negative or non-finite scale with YVEX_ERR_FORMAT. */
 int yvex_rocm_q8_0_encode_row(const float *source, unsigned long long elements,

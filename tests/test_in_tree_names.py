@@ -88,3 +88,35 @@ def test_every_vtable_slot_the_arm_fills_exists_in_the_reference_table():
         assert normalise(declaration) == normalise(theirs[name]), name
     # operations without a reference counterpart are not a slot: the arm's own getter
     assert "rocm_attention_operations" not in ours
+
+
+IN_TREE_SOURCES = ("rocm_attention.c", "rocm_backend.c", "rocm_capability.c", "rocm_driver.c",
+                   "rocm_virtual.c")
+
+
+@pytest.mark.parametrize("source", IN_TREE_SOURCES)
+def test_the_arm_compiles_against_the_reference_headers(source):
+    """Every file of the ROCm arm goes through the compiler's front end as it would inside the
+    reference tree: YVEX_ROCM_IN_TREE makes clori_amd/csrc/host/private.h include the tree's
+    src/backend/private.h (the tree's struct yvex_backend, its vtable and its helpers) in place
+    of the local mirror, and makes include/yvex_rocm.h take every mirrored type from the tree's
+    public and internal headers.  Types, members, vtable slots and the prototypes of every
+    function both sides declare are held against each other by the compiler, warnings are
+    errors; nothing is linked and the reference's build system is not run."""
+    import shutil
+    import subprocess
+    if not os.path.isdir("/opt/rocm/include/hip"):
+        pytest.skip("the HIP headers the driver table is declared from are not installed")
+    if shutil.which("gcc") is None:
+        pytest.skip("no C compiler")
+    command = ["gcc", "-std=c11", "-fsyntax-only", "-Wall", "-Wextra", "-Wno-unused-parameter",
+               "-Werror", "-DYVEX_ROCM_IN_TREE", "-D__HIP_PLATFORM_AMD__",
+               "-I", os.path.join(ROOT, "include"), "-I", "/root/reference",
+               "-I", "/root/reference/include", "-I", "/opt/rocm/include", "-I", HOST,
+               "-I", os.path.dirname(HOST), os.path.join(HOST, source)]
+    done = subprocess.run(command, capture_output=True, text=True)
+    assert done.returncode == 0, done.stderr[-3000:]
+    # and it is the tree's backend object that was compiled against, not the mirror
+    seen = subprocess.run(["-E" if part == "-fsyntax-only" else part for part in command],
+                          capture_output=True, text=True)
+    assert seen.returncode == 0 and "resident_map_readonly" in seen.stdout
