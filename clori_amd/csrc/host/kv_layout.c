@@ -11,7 +11,8 @@
  * 16 s .. 16 s + 15 in block s: what a wave reads at once is a 16-token block either way, a
  * larger page only makes four of them contiguous.
  *
- * Device layouts, per (page, kv head) and block of 16 tokens, d = 128:
+ * Device layouts, per (page, kv head) and block of 16 tokens; d = 128, and for BF16 pages
+ * also 64 and 256 (the same formulas with fewer or more chunks):
  *   BF16  K  uint16 [d/8][16][8]        elem(t,c) at ((c/8)*16 + t)*8 + c%8
  *         V  uint16 [d][16]             elem(t,c) at c*16 + t
  *   Q8_0  K  codes int8 [4 g][16 t][4 j][8]   code(t, c=32j+8g+e) at ((g*16+t)*4+j)*8+e
@@ -25,11 +26,13 @@
 
 enum { PAGE_TOKENS = 16, HEAD_DIM = 128, Q8_BLOCKS = HEAD_DIM / 32 };
 
-/* bytes of one 16-token block */
-static unsigned long long block16_bytes(yvex_rocm_kv_storage storage)
+/* bytes of one 16-token block; 0 for a storage and head dimension that have no layout */
+static unsigned long long block16_bytes(yvex_rocm_kv_storage storage, unsigned long long head_dimension)
 {
-    if (storage == YVEX_ROCM_KV_BF16) return (unsigned long long)PAGE_TOKENS * HEAD_DIM * 2ull;
-    if (storage == YVEX_ROCM_KV_Q8_0)
+    if (storage == YVEX_ROCM_KV_BF16 &&
+        (head_dimension == 64ull || head_dimension == HEAD_DIM || head_dimension == 256ull))
+        return (unsigned long long)PAGE_TOKENS * head_dimension * 2ull;
+    if (storage == YVEX_ROCM_KV_Q8_0 && head_dimension == HEAD_DIM)
         return (unsigned long long)PAGE_TOKENS * HEAD_DIM + PAGE_TOKENS * Q8_BLOCKS * 2ull;
     return 0ull;
 }
@@ -38,8 +41,8 @@ unsigned long long yvex_rocm_kv_page_block_bytes(yvex_rocm_kv_storage storage,
                                                  unsigned long long head_dimension,
                                                  unsigned long long page_tokens)
 {
-    if (head_dimension != HEAD_DIM || (page_tokens != 16ull && page_tokens != 64ull)) return 0ull;
-    return block16_bytes(storage) * (page_tokens / PAGE_TOKENS);
+    if (page_tokens != 16ull && page_tokens != 64ull) return 0ull;
+    return block16_bytes(storage, head_dimension) * (page_tokens / PAGE_TOKENS);
 }
 
 static size_t bf16_index(int is_value, unsigned int t, unsigned int c)
@@ -67,14 +70,16 @@ static int layout_move(yvex_rocm_kv_storage storage, int is_value, int pack,
 {
     const unsigned long long block = yvex_rocm_kv_page_block_bytes(storage, head_dimension,
                                                                    page_tokens);
-    const size_t row_bytes = storage == YVEX_ROCM_KV_BF16 ? HEAD_DIM * 2u : Q8_BLOCKS * 34u;
-    const unsigned long long sub_blocks = page_tokens / PAGE_TOKENS, sub_bytes = block16_bytes(storage);
+    const size_t row_bytes = storage == YVEX_ROCM_KV_BF16 ? (size_t)head_dimension * 2u : Q8_BLOCKS * 34u;
+    const unsigned long long sub_blocks = page_tokens / PAGE_TOKENS;
+    const unsigned long long sub_bytes = block16_bytes(storage, head_dimension);
     unsigned long long page, head, sub;
     unsigned int t, c;
     if (!rows || !packed || !pool_pages || !kv_heads || !block) {
         yvex_error_set(err, block ? YVEX_ERR_INVALID_ARG : YVEX_ERR_UNSUPPORTED, "rocm.kv.layout",
                        block ? "rows, packed buffer and a non-empty pool are required"
-                             : "page layout requires head dimension 128 and pages of 16 or 64 tokens");
+                             : "page layout requires head dimension 128 (bf16 pages: 64, 128 or 256) "
+                               "and pages of 16 or 64 tokens");
         return block ? YVEX_ERR_INVALID_ARG : YVEX_ERR_UNSUPPORTED;
     }
     for (page = 0ull; page < pool_pages; ++page)
@@ -85,7 +90,7 @@ static int layout_move(yvex_rocm_kv_storage storage, int is_value, int pack,
                 unsigned char *row =
                     rows + ((page * page_tokens + sub * PAGE_TOKENS + t) * kv_heads + head) * row_bytes;
                 if (storage == YVEX_ROCM_KV_BF16) {
-                    for (c = 0u; c < HEAD_DIM; ++c) {
+                    for (c = 0u; c < (unsigned int)head_dimension; ++c) {
                         unsigned char *p = dst + bf16_index(is_value, t, c) * 2u;
                         unsigned char *r = row + (size_t)c * 2u;
                         if (pack) memcpy(p, r, 2u); else memcpy(r, p, 2u);

@@ -178,6 +178,7 @@ typedef struct {
     /* when set, the partials live here (nothing is acquired or released) */
     void *fixed_work;
     unsigned long long fixed_work_bytes;
+    int two_launches; /* the function has no build that merges in the kernel */
 } decode_job;
 
 /* Launches the decode kernel, the finish (merge) kernel when the launch fills the device, and
@@ -192,7 +193,7 @@ static int decode_run(yvex_backend *backend, const decode_job *job, const char *
     const unsigned int waves = decode_wave_count(job->sessions, job->kv_heads, job->max_context);
     const unsigned int teams = decode_team_count(job->page_table != NULL, group, job->head_dim,
                                                  job->max_context);
-    const int in_kernel = teams || decode_merges_in_kernel(waves);
+    const int in_kernel = !job->two_launches && (teams || decode_merges_in_kernel(waves));
     void *work = NULL;
     yvex_error cleanup;
     int owned = 0, rc, cleanup_rc;
@@ -251,8 +252,10 @@ static int decode_run(yvex_backend *backend, const decode_job *job, const char *
         rc = yvex_rocm_launch(backend, in_kernel ? job->merged_function : job->function, job->variant,
                               waves, 1u, 1u, 64u, 0u, &dp, where, err);
     if (rc == YVEX_OK && !in_kernel)
-        rc = yvex_rocm_launch(backend, YVEX_ROCM_FN_DECODE_FINISH, job->variant,
-                              (unsigned int)job->query_heads, (unsigned int)job->sessions, 1u,
+        rc = yvex_rocm_launch(backend,
+                              job->head_dim > 128ull ? YVEX_ROCM_FN_DECODE_FINISH_256
+                                                     : YVEX_ROCM_FN_DECODE_FINISH,
+                              job->variant, (unsigned int)job->query_heads, (unsigned int)job->sessions, 1u,
                               (unsigned int)job->head_dim, 0u, &dp, where, err);
     if (rc == YVEX_OK) {
         facts->kernel_launches = in_kernel ? 1ull : 2ull;
@@ -741,15 +744,19 @@ static int paged_validate(const yvex_rocm_paged_decode_requirement *r, const cha
         !yvex_core_u64_mul(r->page_table_stride, r->page_tokens, &capacity) ||
         r->max_context_tokens > capacity)
         return refuse(err, YVEX_ERR_INVALID_ARG, where, "complete paged-decode geometry is required");
-    if (r->head_dimension != ROCM_MFMA_HEAD_DIM ||
+    /* bf16 pages at head dimension 64, 128 or 256; Q8_0 pages at 128 */
+    if ((r->head_dimension != ROCM_MFMA_HEAD_DIM &&
+         !(r->kv_storage == YVEX_ROCM_KV_BF16 &&
+           (r->head_dimension == 64ull || r->head_dimension == 256ull))) ||
         (r->page_tokens != ROCM_PAGE_TOKENS && r->page_tokens != 4ull * ROCM_PAGE_TOKENS) ||
         r->query_heads / r->key_value_heads > ROCM_GROUP_MAX ||
         (r->kv_storage != YVEX_ROCM_KV_BF16 && r->kv_storage != YVEX_ROCM_KV_Q8_0) ||
         r->numeric_contract != YVEX_TRANSFORMER_ATTENTION_NUMERIC_BF16_F32_ACCUMULATE ||
         !r->deterministic || r->pool_pages > 0x7fffffffull || capacity > 0x7fffffffull)
         return refuse(err, YVEX_ERR_UNSUPPORTED, where,
-                      "ROCm paged decode requires head dimension 128, pages of 16 or 64 tokens, a query "
-                      "group of at most 16 and the deterministic bf16/fp32-accumulate contract");
+                      "ROCm paged decode requires head dimension 128 (bf16 pages: 64, 128 or 256), pages "
+                      "of 16 or 64 tokens, a query group of at most 16 and the deterministic "
+                      "bf16/fp32-accumulate contract");
     yvex_error_clear(err);
     return YVEX_OK;
 }
@@ -817,7 +824,13 @@ static int paged_decode_execute_common(yvex_backend *backend,
                       "query, page pools, page table, context lengths and outputs must be written "
                       "tensors of this backend with the declared geometry");
     memset(&job, 0, sizeof(job));
-    if (r->kv_storage == YVEX_ROCM_KV_BF16) {
+    if (r->kv_storage == YVEX_ROCM_KV_BF16 && r->head_dimension != ROCM_MFMA_HEAD_DIM) {
+        /* the other head dimensions have the two-launch form only */
+        job.function = r->head_dimension == 64ull ? YVEX_ROCM_FN_DECODE_PAGED_BF16_64
+                                                  : YVEX_ROCM_FN_DECODE_PAGED_BF16_256;
+        job.two_launches = 1;
+        job.variant = YVEX_BACKEND_VARIANT_ROCM_ATTENTION_PAGED_BF16;
+    } else if (r->kv_storage == YVEX_ROCM_KV_BF16) {
         job.function = YVEX_ROCM_FN_DECODE_PAGED_BF16;
         job.merged_function = YVEX_ROCM_FN_DECODE_PAGED_BF16_MERGED;
         job.variant = YVEX_BACKEND_VARIANT_ROCM_ATTENTION_PAGED_BF16;

@@ -46,6 +46,12 @@ static const rocm_kernel_binding rocm_kernel_bindings[] = {
     {"yvex_rocm_stream_read", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_F32, YVEX_ROCM_FN_STREAM_READ},
     {"yvex_rocm_decode_paged_bf16", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_PAGED_BF16,
      YVEX_ROCM_FN_DECODE_PAGED_BF16},
+    {"yvex_rocm_decode_paged_bf16_64", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_PAGED_BF16,
+     YVEX_ROCM_FN_DECODE_PAGED_BF16_64},
+    {"yvex_rocm_decode_paged_bf16_256", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_PAGED_BF16,
+     YVEX_ROCM_FN_DECODE_PAGED_BF16_256},
+    {"yvex_rocm_decode_finish_256", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_PAGED_BF16,
+     YVEX_ROCM_FN_DECODE_FINISH_256},
     {"yvex_rocm_decode_merge", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_PAGED_BF16,
      YVEX_ROCM_FN_DECODE_MERGE},
     {"yvex_rocm_decode_merge_rope", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_MLA_BF16,

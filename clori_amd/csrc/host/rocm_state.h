@@ -19,10 +19,13 @@ typedef enum {
     YVEX_ROCM_FN_GQA_F32_TILE_256,
     YVEX_ROCM_FN_FILL_U32,
     YVEX_ROCM_FN_DECODE_PAGED_BF16,
+    YVEX_ROCM_FN_DECODE_PAGED_BF16_64,
+    YVEX_ROCM_FN_DECODE_PAGED_BF16_256,
     YVEX_ROCM_FN_DECODE_ROWS_BF16,
     YVEX_ROCM_FN_DECODE_MERGE,
     YVEX_ROCM_FN_DECODE_MERGE_ROPE,
     YVEX_ROCM_FN_DECODE_FINISH,
+    YVEX_ROCM_FN_DECODE_FINISH_256,
     YVEX_ROCM_FN_DECODE_PAGED_Q8_0,
     YVEX_ROCM_FN_DECODE_PAGED_BF16_MERGED,
     YVEX_ROCM_FN_DECODE_PAGED_Q8_0_MERGED,

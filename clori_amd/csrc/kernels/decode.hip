@@ -72,16 +72,18 @@ typedef __attribute__((address_space(3))) short4v lds_short4;
 // (each 32-byte column segment is hit by exactly two rows).
 __device__ inline uint32_t vt_offset(int row, int chunk) { return (uint32_t)(row * 256 + ((chunk ^ (row & 14)) << 4)); }
 
+template <int kDim>
 struct State {
-    floatx4 o[8];  // O^T[dim 16*b + 4*(lane/16) + i][head lane%16]
-    float m, l;    // running max (log2 units) and per-lane partial sum
+    floatx4 o[kDim / 16];  // O^T[dim 16*b + 4*(lane/16) + i][head lane%16]
+    float m, l;            // running max (log2 units) and per-lane partial sum
 };
 
 // Online-softmax step shared by every KV format: takes the scaled scores of the lane's
 // four tokens (masked ones at -inf), updates (m, l), rescales the accumulators only when
 // some lane of the wave saw a larger score (after the first tiles the running maximum
 // rarely moves), and returns the four probabilities.
-__device__ inline void softmax_step(State &st, const float (&x)[4], float (&p)[4])
+template <int kDim>
+__device__ inline void softmax_step(State<kDim> &st, const float (&x)[4], float (&p)[4])
 {
     float mloc = fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3]));
     mloc = fmaxf(mloc, xor_lanes(mloc, 16));
@@ -91,7 +93,7 @@ __device__ inline void softmax_step(State &st, const float (&x)[4], float (&p)[4
         const float alpha = fast_exp2(st.m - m_new);
         st.l *= alpha;
 #pragma unroll
-        for (int b = 0; b < 8; ++b) st.o[b] *= alpha;
+        for (int b = 0; b < kDim / 16; ++b) st.o[b] *= alpha;
         st.m = m_new;
     }
 #pragma unroll
@@ -100,15 +102,20 @@ __device__ inline void softmax_step(State &st, const float (&x)[4], float (&p)[4
 }
 
 // ---- bf16 KV --------------------------------------------------------------------
+template <int kDim>
 struct Bf16Tile {
-    u32x4 k[4];  // K[token = lane%16][32*j + 8*(lane/16) .. +7]
-    u32x2 v[8];  // paged: V[tokens 4*(lane/16)..+3][dim 16*b + lane%16]
+    u32x4 k[kDim / 32];  // K[token = lane%16][32*j + 8*(lane/16) .. +7]
+    u32x2 v[kDim / 16];  // paged: V[tokens 4*(lane/16)..+3][dim 16*b + lane%16]
                  // token-major: raw row chunks, (v[2j], v[2j+1]) = V[token 4j + lane/16][8*(lane%16)..+7]
 };
 
+// kHeadDimension: 128 is the tuned build (paged and token-major); 64 and 256 are the same
+// paged code with other counts.
+template <int kHeadDimension>
 struct Bf16Kv {
-    typedef Bf16Tile Tile;
-    static constexpr uint32_t kBlockBytes = kPageTokens * kHeadDim * 2;
+    static constexpr int kDim = kHeadDimension;
+    typedef Bf16Tile<kDim> Tile;
+    static constexpr uint32_t kBlockBytes = kPageTokens * kDim * 2;
 
     __device__ static inline void load_paged(Tile &t, const unsigned char *kblock,
                                              const unsigned char *vblock, int lane)
@@ -116,9 +123,9 @@ struct Bf16Kv {
         const int n = lane & 15, g = lane >> 4;
         const uint16_t *k = (const uint16_t *)kblock, *v = (const uint16_t *)vblock;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) t.k[j] = load_b128(k + (j * 64 + lane) * 8);
+        for (int j = 0; j < kDim / 32; ++j) t.k[j] = load_b128(k + (j * 64 + lane) * 8);
 #pragma unroll
-        for (int b = 0; b < 8; ++b) t.v[b] = load_b64(v + (b * 16 + n) * 16 + g * 4);
+        for (int b = 0; b < kDim / 16; ++b) t.v[b] = load_b64(v + (b * 16 + n) * 16 + g * 4);
     }
 
     // rows_left: tokens available from `first` on (rows beyond are clamped to the last
@@ -128,6 +135,7 @@ struct Bf16Kv {
                                             const yvex_rocm_decode_params &p, uint32_t first,
                                             uint32_t rows_left, int lane)
     {
+        static_assert(kDim == 128, "token-major rows: 16 lanes x 8 dims cover the row");
         const int n = lane & 15, g = lane >> 4;
         const uint16_t *k = (const uint16_t *)kbytes, *v = (const uint16_t *)vbytes;
         const uint32_t last = rows_left - 1u;
@@ -164,13 +172,13 @@ struct Bf16Kv {
     }
 
     // valid: number of real tokens in this 16-token tile (1..16).
-    __device__ static inline void consume(State &st, const Tile &t, const bf16x8 (&q)[4],
+    __device__ static inline void consume(State<kDim> &st, const Tile &t, const bf16x8 (&q)[kDim / 32],
                                           float scale_log2, uint32_t valid, int lane)
     {
         const int g = lane >> 4;
         floatx4 s = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int j = 0; j < 4; ++j) s = mfma_16x16x32(as_bf16x8(t.k[j]), q[j], s);
+        for (int j = 0; j < kDim / 32; ++j) s = mfma_16x16x32(as_bf16x8(t.k[j]), q[j], s);
         float x[4], p[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i)
@@ -188,7 +196,7 @@ struct Bf16Kv {
             uint32_t keep_hi = ((uint32_t)(g * 4 + 2) < valid ? 0x0000ffffu : 0u) |
                                ((uint32_t)(g * 4 + 3) < valid ? 0xffff0000u : 0u);
 #pragma unroll
-            for (int b = 0; b < 8; ++b) {
+            for (int b = 0; b < kDim / 16; ++b) {
                 u32x2 v = t.v[b];
                 v.x &= keep_lo;
                 v.y &= keep_hi;
@@ -196,7 +204,7 @@ struct Bf16Kv {
             }
         } else {
 #pragma unroll
-            for (int b = 0; b < 8; ++b)
+            for (int b = 0; b < kDim / 16; ++b)
                 st.o[b] = mfma_16x16x16(as_short4(t.v[b]), pv, st.o[b]);
         }
     }
@@ -222,6 +230,7 @@ __device__ inline float half_f32(uint32_t word, int hi)
 }
 
 struct Q8Kv {
+    static constexpr int kDim = kHeadDim;
     typedef Q8Tile Tile;
     static constexpr uint32_t kCodeBytes = kPageTokens * kHeadDim;
     static constexpr uint32_t kBlockBytes = kCodeBytes + kPageTokens * (kHeadDim / 32) * 2;
@@ -246,7 +255,7 @@ struct Q8Kv {
     }
     __device__ static inline void transpose_rows(Tile &, unsigned char *, int) {}
 
-    __device__ static inline void consume(State &st, const Tile &t, const bf16x8 (&q)[4],
+    __device__ static inline void consume(State<kDim> &st, const Tile &t, const bf16x8 (&q)[4],
                                           float scale_log2, uint32_t valid, int lane)
     {
         const int g = lane >> 4;
@@ -317,7 +326,10 @@ __device__ inline uint32_t wave_inclusive_scan(uint32_t v, int lane)
 // streaming loop from scalar to vector registers and the paged bf16 kernel loses 4 %.
 template <class Kv, bool PAGED, int kDepth, bool MERGE>
 struct Decoder {
+    static constexpr int kDim = Kv::kDim;
+    static_assert(kDim == 128 || (PAGED && !MERGE), "other head dimensions: the two-launch paged form");
     typedef typename Kv::Tile Tile;
+    typedef ::State<kDim> State;
     const yvex_rocm_decode_params &p;
     unsigned char *const vt;  // token-major layout: 4 KB of LDS for the V transposition
     const int lane, n, g;
@@ -370,7 +382,7 @@ struct Decoder {
     }
 
     // Streams `count` (<= 128) tiles of (session, kv_head) starting at tile `first`.
-    __device__ inline void stream(State &st, const bf16x8 (&q)[4], uint32_t session,
+    __device__ inline void stream(State &st, const bf16x8 (&q)[kDim / 32], uint32_t session,
                                   uint32_t kv_head, uint32_t ctx, uint32_t first,
                                   uint32_t count) const
     {
@@ -395,11 +407,11 @@ struct Decoder {
                 my_page_hi = 0;
             }
         } else {
-            kbase += (uint64_t)kv_head * kHeadDim * 2u;
-            vbase += (uint64_t)kv_head * kHeadDim * 2u;
+            kbase += (uint64_t)kv_head * kDim * 2u;
+            vbase += (uint64_t)kv_head * kDim * 2u;
         }
         auto fetch = [&](Tile &t, uint32_t i) {
-            if (PAGED) {
+            if constexpr (PAGED) {
                 const uint32_t at = sub0 + i, slot = at >> shift;
                 const uint32_t page = (uint32_t)(slot < 64u
                                                      ? __builtin_amdgcn_readlane(my_page, (int)slot)
@@ -426,7 +438,7 @@ struct Decoder {
 #pragma unroll
             for (int r = 0; r < kDepth; ++r) {
                 const uint32_t tile = i + (uint32_t)r;
-                if (!PAGED) Kv::transpose_rows(ring[r], vt, lane);
+                if constexpr (!PAGED) Kv::transpose_rows(ring[r], vt, lane);
                 Kv::consume(st, ring[r], q, p.scale_log2,
                             min((uint32_t)kPageTokens, t1 - (t0 + tile * kPageTokens)), lane);
                 fetch(ring[r], min(tile + kDepth, last_tile));
@@ -436,7 +448,7 @@ struct Decoder {
         for (int r = 0; r < kDepth - 1; ++r) {
             const uint32_t tile = i + (uint32_t)r;
             if (tile < count) {
-                if (!PAGED) Kv::transpose_rows(ring[r], vt, lane);
+                if constexpr (!PAGED) Kv::transpose_rows(ring[r], vt, lane);
                 Kv::consume(st, ring[r], q, p.scale_log2,
                             min((uint32_t)kPageTokens, t1 - (t0 + tile * kPageTokens)), lane);
             }
@@ -450,10 +462,10 @@ struct Decoder {
         if ((uint32_t)n >= group) return;
         const uint32_t head = kv_head * group + (uint32_t)n;
         const float inv = 1.0f / l;
-        uint16_t *dst = p.out + ((uint64_t)session * p.query_heads + head) * kHeadDim + g * 4;
+        uint16_t *dst = p.out + ((uint64_t)session * p.query_heads + head) * kDim + g * 4;
         bool bad = false;
 #pragma unroll
-        for (int b = 0; b < 8; ++b) {
+        for (int b = 0; b < kDim / 16; ++b) {
             const float a0 = st.o[b][0] * inv, a1 = st.o[b][1] * inv;
             const float a2 = st.o[b][2] * inv, a3 = st.o[b][3] * inv;
             bad |= !(isfinite(a0) && isfinite(a1) && isfinite(a2) && isfinite(a3));
@@ -479,14 +491,14 @@ struct Decoder {
         if ((uint32_t)n < group) {
             // slot 1 when the segment starts inside this wave's range, else slot 0
             const uint64_t slot = ((uint64_t)wave * 2u + (starts_here ? 1u : 0u)) * group + n;
-            float *acc = p.part_acc + slot * kHeadDim + g * 4;
+            float *acc = p.part_acc + slot * kDim + g * 4;
             if (MERGE) {
 #pragma unroll
-                for (int b = 0; b < 8; ++b) store_b128_device(acc + b * 16, st.o[b]);
+                for (int b = 0; b < kDim / 16; ++b) store_b128_device(acc + b * 16, st.o[b]);
                 if (g == 0) store_b64_device(p.part_ml + slot * 2, st.m, l);
             } else {
 #pragma unroll
-                for (int b = 0; b < 8; ++b) *reinterpret_cast<floatx4 *>(acc + b * 16) = st.o[b];
+                for (int b = 0; b < kDim / 16; ++b) *reinterpret_cast<floatx4 *>(acc + b * 16) = st.o[b];
                 if (g == 0) {
                     p.part_ml[slot * 2 + 0] = st.m;
                     p.part_ml[slot * 2 + 1] = l;
@@ -620,12 +632,12 @@ struct Decoder {
             const uint32_t stop = min(seg_end, end), count = stop - cur;
             const uint32_t ctx = context_of(session);
 
-            bf16x8 q[4];
+            bf16x8 q[kDim / 32];
             {
                 const uint16_t *qrow = p.q + ((uint64_t)session * p.query_heads + kv_head * group +
-                                              min((uint32_t)n, group - 1u)) * kHeadDim;
+                                              min((uint32_t)n, group - 1u)) * kDim;
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
+                for (int j = 0; j < kDim / 32; ++j) {
                     u32x4 raw = load_b128(qrow + j * 32 + g * 8);
                     if ((uint32_t)n >= group) raw = (u32x4){0u, 0u, 0u, 0u};
                     q[j] = as_bf16x8(raw);
@@ -633,7 +645,7 @@ struct Decoder {
             }
             State st;
 #pragma unroll
-            for (int b = 0; b < 8; ++b) st.o[b] = (floatx4){0.f, 0.f, 0.f, 0.f};
+            for (int b = 0; b < kDim / 16; ++b) st.o[b] = (floatx4){0.f, 0.f, 0.f, 0.f};
             st.m = -INFINITY;
             st.l = 0.f;
             for (uint32_t done = 0u; done < count; done += 128u)
@@ -646,10 +658,10 @@ struct Decoder {
                 publish(st, l, session, kv_head);  // the whole segment was ours
             } else {
                 leave_partial(st, l, wave, first == 0u);
-                if (!MERGE) {
+                if constexpr (!MERGE) {
                     cur = stop;
                     continue;  // the finish kernel merges
-                }
+                } else {
                 // count this wave in; whoever completes the count merges the segment
                 const uint32_t w_first = seg_begin / per_wave, w_last = (seg_end - 1u) / per_wave;
                 uint32_t *arrivals = p.arrivals + (uint64_t)session * p.kv_heads + kv_head;
@@ -664,6 +676,7 @@ struct Decoder {
                     // keeps the compiler from moving them above the count
                     loads_ordered();
                     merge_segment(session, kv_head, seg_begin, per_wave, w_first, w_last);
+                }
                 }
             }
             cur = stop;
@@ -829,8 +842,9 @@ struct Decoder {
 
 }  // namespace
 
-#define YVEX_DECODE_KERNEL(name, Kv, PAGED, DEPTH, MERGE)                                           \
-    extern "C" __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2)))  \
+#define YVEX_DECODE_KERNEL(name, Kv, PAGED, DEPTH, MERGE) YVEX_DECODE_KERNEL_WAVES(name, Kv, PAGED, DEPTH, MERGE, 2)
+#define YVEX_DECODE_KERNEL_WAVES(name, Kv, PAGED, DEPTH, MERGE, WAVES)                              \
+    extern "C" __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(WAVES, WAVES))) \
     name(const yvex_rocm_decode_params p)                                                      \
     {                                                                                          \
         __shared__ __attribute__((aligned(16))) unsigned char vt[PAGED ? 16 : kPageTokens * kHeadDim * 2]; \
@@ -838,19 +852,23 @@ struct Decoder {
     }
 
 // full-size launches: partials for yvex_rocm_decode_finish
-YVEX_DECODE_KERNEL(yvex_rocm_decode_paged_bf16, Bf16Kv, true, 3, false)
+YVEX_DECODE_KERNEL(yvex_rocm_decode_paged_bf16, Bf16Kv<128>, true, 3, false)
 YVEX_DECODE_KERNEL(yvex_rocm_decode_paged_q8_0, Q8Kv, true, 3, false)
-YVEX_DECODE_KERNEL(yvex_rocm_decode_rows_bf16, Bf16Kv, false, 2, false)
+YVEX_DECODE_KERNEL(yvex_rocm_decode_rows_bf16, Bf16Kv<128>, false, 2, false)
+// head dimensions 64 and 256: paged bf16 pages only, always with the second launch (one wave
+// per SIMD at 256, whose tiles and accumulators take twice the registers)
+YVEX_DECODE_KERNEL(yvex_rocm_decode_paged_bf16_64, Bf16Kv<64>, true, 3, false)
+YVEX_DECODE_KERNEL_WAVES(yvex_rocm_decode_paged_bf16_256, Bf16Kv<256>, true, 2, false, 1)
 // launches that do not fill the device: merge in the kernel, one launch
-YVEX_DECODE_KERNEL(yvex_rocm_decode_paged_bf16_merged, Bf16Kv, true, 3, true)
+YVEX_DECODE_KERNEL(yvex_rocm_decode_paged_bf16_merged, Bf16Kv<128>, true, 3, true)
 YVEX_DECODE_KERNEL(yvex_rocm_decode_paged_q8_0_merged, Q8Kv, true, 3, true)
-YVEX_DECODE_KERNEL(yvex_rocm_decode_rows_bf16_merged, Bf16Kv, false, 2, true)
+YVEX_DECODE_KERNEL(yvex_rocm_decode_rows_bf16_merged, Bf16Kv<128>, false, 2, true)
 
 // teams of eight waves over a token-major history (see Decoder::run_team)
 extern "C" __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
 yvex_rocm_decode_rows_bf16_team(const yvex_rocm_decode_params p)
 {
-    typedef Decoder<Bf16Kv, false, 2, true> Team;
+    typedef Decoder<Bf16Kv<128>, false, 2, true> Team;
     __shared__ __attribute__((aligned(16))) unsigned char team_lds[Team::kTeamLdsBytes];
     const uint32_t wave = threadIdx.x >> 6;
     Team(p, team_lds + wave * (kPageTokens * kHeadDim * 2)).run_team(reinterpret_cast<float *>(team_lds));
@@ -860,8 +878,7 @@ yvex_rocm_decode_rows_bf16_team(const yvex_rocm_decode_params p)
 // without arrival counters (large launches).  grid = (query_heads, sessions), block =
 // head_dim threads (one per output lane).  A segment that one wave covered was already
 // published by that wave and is skipped.
-extern "C" __global__ void __launch_bounds__(128)
-yvex_rocm_decode_finish(const yvex_rocm_decode_params p)
+__device__ __forceinline__ void decode_finish(const yvex_rocm_decode_params &p)
 {
     const uint32_t head = blockIdx.x, session = blockIdx.y, d = threadIdx.x;
     const uint32_t group = p.query_heads / p.kv_heads;
@@ -927,6 +944,19 @@ yvex_rocm_decode_finish(const yvex_rocm_decode_params p)
     p.out[at] = bf16_bits(o);
     if (p.lse && d == 0u)
         p.lse[(uint64_t)session * p.query_heads + head] = (top + fast_log2(sum)) * YVEX_LN2;
+}
+
+extern "C" __global__ void __launch_bounds__(128)
+yvex_rocm_decode_finish(const yvex_rocm_decode_params p)
+{
+    decode_finish(p);
+}
+
+// head dimension 256: a block of 256 threads
+extern "C" __global__ void __launch_bounds__(256)
+yvex_rocm_decode_finish_256(const yvex_rocm_decode_params p)
+{
+    decode_finish(p);
 }
 
 // Log-sum-exp merge of the chunk partials of one (session, query head): one wave per head,

@@ -130,8 +130,8 @@ def make_paged_case(rng, contexts, hq, hkv, d=128, page_tokens=16, spare=5, q8=F
 def run_paged(backend, q, k_rows, v_rows, table, ctx, hkv, pool_pages, storage=B.KV_BF16,
               max_context=None, page_tokens=16):
     sessions, hq, d = q.shape
-    kp = kv_pack_pages(k_rows, storage, False, hkv, page_tokens=page_tokens)
-    vp = kv_pack_pages(v_rows, storage, True, hkv, page_tokens=page_tokens)
+    kp = kv_pack_pages(k_rows, storage, False, hkv, head_dim=d, page_tokens=page_tokens)
+    vp = kv_pack_pages(v_rows, storage, True, hkv, head_dim=d, page_tokens=page_tokens)
     pool_dtype = B.DTYPE_BF16 if storage == B.KV_BF16 else B.DTYPE_I8
     elems = kp.size // B.DTYPE_BYTES[pool_dtype]
     tq = backend.tensor("q", B.DTYPE_BF16, q.shape, q)
@@ -365,3 +365,42 @@ def test_paged_decode_with_pages_of_64_tokens(backend, q8):
     with pytest.raises(YvexError) as e:
         run_paged(backend, q, k_rows, v_rows, bad, ctx, 8, pool_pages, storage=storage, page_tokens=64)
     assert e.value.code == B.YVEX_ERR_BOUNDS
+
+
+@pytest.mark.parametrize("d,hq,hkv", [(64, 16, 4), (256, 24, 4), (256, 8, 8)])
+@pytest.mark.parametrize("page_tokens", [16, 64])
+def test_paged_decode_other_head_dimensions(backend, d, hq, hkv, page_tokens):
+    """bf16 pages at head dimension 64 and 256 (the reference admits up to 256 and its own
+    Qwen pattern is 24/4/256, tests/unit/cuda/quant_qtype.c:2413-2418): ragged contexts around
+    block and page edges against the oracle, placement invariance bit for bit, garbage past the
+    context; these head dimensions always take the second launch."""
+    rng = np.random.default_rng(1000 + d + page_tokens)
+    contexts = [1, 15, 16, 17, 63, 64, 65, 333, 1024, 1025, 2500, 9000]
+    q, k_rows, v_rows, table, ctx, pool_pages = make_paged_case(rng, contexts, hq, hkv, d=d,
+                                                                 page_tokens=page_tokens)
+    got, lse, facts = run_paged(backend, q, k_rows, v_rows, table, ctx, hkv, pool_pages,
+                                page_tokens=page_tokens)
+    rc, ref, _, ref_lse = ORACLE.paged_decode(q, k_rows, v_rows, table, ctx, hkv, page_tokens)
+    assert rc == 0
+    assert_close_bf16(got, ref, "paged d=%d" % d)
+    assert_lse(lse, ref_lse, "paged d=%d" % d)
+    assert facts.kernel_launches == 2
+    perm = rng.permutation(pool_pages)
+    k2, v2 = np.empty_like(k_rows), np.empty_like(v_rows)
+    k2[perm], v2[perm] = k_rows, v_rows
+    for s, c in enumerate(contexts):  # rows past each context: NaN bit patterns
+        last = perm[table[s, (c - 1) // page_tokens]]
+        k2[last, c % page_tokens or page_tokens:] = 0x7FC0
+        v2[last, c % page_tokens or page_tokens:] = 0x7FC0
+    got2, lse2, _ = run_paged(backend, q, k2, v2, perm[table].astype(np.int32), ctx, hkv, pool_pages,
+                              page_tokens=page_tokens)
+    assert np.array_equal(got, got2) and np.array_equal(lse, lse2)
+
+
+def test_paged_decode_other_head_dimensions_refusals(backend):
+    """Q8_0 pages exist at head dimension 128 only; 96 has no kernel at all."""
+    for d, storage in ((64, B.KV_Q8_0), (256, B.KV_Q8_0), (96, B.KV_BF16)):
+        req = backend.paged_requirement(1, 8, 2, d, 16, 4, 4, 64, storage=storage)
+        with pytest.raises(YvexError) as e:
+            backend.paged_decode_workspace_required(req)
+        assert e.value.code == B.YVEX_ERR_UNSUPPORTED

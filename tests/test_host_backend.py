@@ -1220,5 +1220,23 @@ def test_page_layouts_follow_the_documented_index_formulas():
     assert lib().yvex_rocm_kv_page_block_bytes(B.KV_Q8_0, 128, 64) == 4 * 2176
     assert lib().yvex_rocm_kv_page_block_bytes(B.KV_BF16, 128, 32) == 0
     with pytest.raises(YvexError) as e:
-        kv_pack_pages(rows, B.KV_BF16, False, hkv, head_dim=64)
+        kv_pack_pages(rows, B.KV_BF16, False, hkv, head_dim=96)
     assert e.value.code == B.YVEX_ERR_UNSUPPORTED
+    with pytest.raises(YvexError) as e:
+        kv_pack_pages(rng.integers(0, 256, size=(pages, 16, hkv, 2 * 34), dtype=np.uint8), B.KV_Q8_0, False,
+                      hkv, head_dim=64)
+    assert e.value.code == B.YVEX_ERR_UNSUPPORTED
+    # bf16 pages at head dimension 64 and 256: the same index formulas with other chunk counts
+    for width in (64, 256):
+        wide_rows = rng.integers(0, 1 << 16, size=(pages, 16, hkv, width), dtype=np.uint16)
+        assert lib().yvex_rocm_kv_page_block_bytes(B.KV_BF16, width, 16) == 16 * width * 2
+        for is_value in (False, True):
+            packed = kv_pack_pages(wide_rows, B.KV_BF16, is_value, hkv, head_dim=width).view(np.uint16)
+            packed = packed.reshape(pages, hkv, 16 * width)
+            t, c = np.meshgrid(np.arange(16), np.arange(width), indexing="ij")
+            index = c * 16 + t if is_value else ((c // 8) * 16 + t) * 8 + c % 8
+            for page in range(pages):
+                for head in range(hkv):
+                    assert np.array_equal(packed[page, head][index], wide_rows[page, :, head, :])
+            back = kv_unpack_pages(packed, B.KV_BF16, is_value, pages, hkv, head_dim=width)
+            assert np.array_equal(back, wide_rows)
