@@ -133,17 +133,17 @@ def time_steps(backend, run, steps, warmup, kernels):
 
 # --------------------------------------------------------------------- workloads --
 
-def decode_kernels(kernel, facts):
+def decode_kernels(kernel, facts, finish="yvex_rocm_decode_finish"):
     """Kernels of one decode step.  A launch that does not fill the device merges its split
     segments in the kernel itself (one launch, the `_merged` build of the kernel); a full-size
     launch leaves the merge to a second, small kernel."""
     if facts.kernel_launches == 1:
         return [kernel + "_merged"]
-    return [kernel, "yvex_rocm_decode_finish"]
+    return [kernel, finish]
 
 
-def workload_paged(backend, rng, steps, warmup, q8=False, page=16):
-    sessions, hq, hkv, d = 32, 32, 8, 128
+def workload_paged(backend, rng, steps, warmup, q8=False, page=16, hq=32, hkv=8, d=128, name=None):
+    sessions = 32
     lo, hi = (4096, 32768) if q8 else (512, 16384)
     contexts = rng.integers(lo, hi + 1, size=sessions).astype(np.int32)
     need = (contexts + page - 1) // page
@@ -156,7 +156,7 @@ def workload_paged(backend, rng, steps, warmup, q8=False, page=16):
         table[s, :need[s]] = perm[at:at + need[s]]
         at += int(need[s])
     storage = B.KV_Q8_0 if q8 else B.KV_BF16
-    block = 2176 if q8 else 4096             # one 16-token block; a page is page // 16 of them
+    block = 2176 if q8 else 32 * d           # one 16-token block; a page is page // 16 of them
     blocks = pool_pages * hkv * (page // 16)
     pool_bytes = blocks * block
     if q8:
@@ -191,19 +191,20 @@ def workload_paged(backend, rng, steps, warmup, q8=False, page=16):
     backend.workspace_attach(work)
     run = lambda: backend.paged_decode_execute(req, q, k_pool, v_pool, tt, tc, out, lse)  # noqa: E731
     facts = run()
-    kernel = "yvex_rocm_decode_paged_q8_0" if q8 else "yvex_rocm_decode_paged_bf16"
-    kernels = decode_kernels(kernel, facts)
+    kernel = "yvex_rocm_decode_paged_q8_0" if q8 else \
+        "yvex_rocm_decode_paged_bf16" + ("" if d == 128 else "_%d" % d)
+    kernels = decode_kernels(kernel, facts, "yvex_rocm_decode_finish" + ("_256" if d == 256 else ""))
     timed = time_steps(backend, run, steps, warmup, kernels)
     backend.workspace_detach()
     tokens = int(contexts.sum())
-    per_token = 2 * hkv * (136 if q8 else 256)
+    per_token = 2 * hkv * (136 if q8 else 2 * d)
     algo = tokens * per_token + int(need.sum()) * 4 + sessions * 4 + 2 * sessions * hq * d * 2 + \
         sessions * hq * 4
     assert np.all(np.isfinite(lse.read()))
-    return dict(name=("paged4" if q8 else "paged3") + ("" if page == 16 else "_p%d" % page),
-                workload="paged %s GQA decode: 32 sessions, 32/8 heads, d=128, contexts U[%d,%d], "
+    return dict(name=name or ("paged4" if q8 else "paged3") + ("" if page == 16 else "_p%d" % page),
+                workload="paged %s GQA decode: 32 sessions, %d/%d heads, d=%d, contexts U[%d,%d], "
                          "%d-token pages, seeded permutation page tables%s" %
-                         ("Q8_0" if q8 else "bf16", lo, hi, page,
+                         ("Q8_0" if q8 else "bf16", hq, hkv, d, lo, hi, page,
                           ", N(0,1) bf16 values quantised on the host (absmax/127, round to nearest), "
                           "a 2048-page sample repeated through the pool" if q8 else ""),
                 bound="hbm", algorithmic_bytes=algo, tokens=tokens,
@@ -446,10 +447,12 @@ EXTRA_WORKLOADS = {
     # the reference's own Qwen attention geometry (24/4 heads, head dimension 256) and a narrow one
     "prefill_d256": lambda b, r, s, w: workload_prefill2(b, r, s, w, hq=24, hkv=4, d=256, name="prefill_d256"),
     "prefill_d64": lambda b, r, s, w: workload_prefill2(b, r, s, w, hq=16, hkv=4, d=64, name="prefill_d64"),
+    "paged_d256": lambda b, r, s, w: workload_paged(b, r, s, w, hq=24, hkv=4, d=256, name="paged_d256"),
+    "paged_d64": lambda b, r, s, w: workload_paged(b, r, s, w, hq=16, hkv=4, d=64, name="paged_d64"),
 }
 SEEDS = {"decode1": 1, "prefill2": 2, "paged3": 3, "paged4": 4, "mla5": 5, "append_bf16": 6,
          "append_q8_0": 7, "exact2": 8, "exact1": 9, "history_append": 10, "paged3_p64": 3, "paged4_p64": 4,
-         "prefill_d256": 11, "prefill_d64": 12}
+         "prefill_d256": 11, "prefill_d64": 12, "paged_d256": 13, "paged_d64": 14}
 
 
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")

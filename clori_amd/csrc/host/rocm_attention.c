@@ -1310,8 +1310,8 @@ static int rocm_kv_append_execute(yvex_backend *backend, const yvex_rocm_kv_appe
         r->sessions > 65535ull || r->key_value_heads > 65535ull || r->pool_pages > 0x7fffffffull ||
         capacity > 0x7fffffffull || r->total_tokens > 0x7fffffffull)
         return refuse(err, YVEX_ERR_UNSUPPORTED, where,
-                      "ROCm KV append requires head dimension 128, pages of 16 or 64 tokens, BF16 or Q8_0 "
-                      "storage and a rotary dimension that is a multiple of 16");
+                      "ROCm KV append requires head dimension 128 (bf16 pages: 64, 128 or 256), pages of 16 "
+                      "or 64 tokens, BF16 or Q8_0 storage and a rotary dimension that is a multiple of 16");
     memset(facts, 0, sizeof(*facts));
     pool_dtype = r->storage == YVEX_ROCM_KV_BF16 ? YVEX_DTYPE_BF16 : YVEX_DTYPE_I8;
     row_elements = r->total_tokens * r->key_value_heads * r->head_dimension;
@@ -1363,8 +1363,10 @@ static int rocm_kv_append_execute(yvex_backend *backend, const yvex_rocm_kv_appe
                                                : YVEX_BACKEND_VARIANT_ROCM_ATTENTION_PAGED_Q8_0;
     backend_workspace_reset(backend);
     rc = yvex_rocm_launch(backend,
-                          r->storage == YVEX_ROCM_KV_BF16 ? YVEX_ROCM_FN_KV_APPEND_BF16
-                                                          : YVEX_ROCM_FN_KV_APPEND_Q8_0,
+                          r->storage != YVEX_ROCM_KV_BF16   ? YVEX_ROCM_FN_KV_APPEND_Q8_0
+                          : r->head_dimension == 64ull  ? YVEX_ROCM_FN_KV_APPEND_BF16_64
+                          : r->head_dimension == 256ull ? YVEX_ROCM_FN_KV_APPEND_BF16_256
+                                                        : YVEX_ROCM_FN_KV_APPEND_BF16,
                           variant, (unsigned int)page_slots,
                           (unsigned int)((r->key_value_heads + YVEX_ROCM_KV_APPEND_HEADS - 1ull) /
                                          YVEX_ROCM_KV_APPEND_HEADS),

@@ -83,6 +83,10 @@ static const rocm_kernel_binding rocm_kernel_bindings[] = {
     {"yvex_rocm_gather_rows", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_MLA_BF16, YVEX_ROCM_FN_GATHER_ROWS},
     {"yvex_rocm_kv_append_bf16", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_PAGED_BF16,
      YVEX_ROCM_FN_KV_APPEND_BF16},
+    {"yvex_rocm_kv_append_bf16_64", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_PAGED_BF16,
+     YVEX_ROCM_FN_KV_APPEND_BF16_64},
+    {"yvex_rocm_kv_append_bf16_256", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_PAGED_BF16,
+     YVEX_ROCM_FN_KV_APPEND_BF16_256},
     {"yvex_rocm_kv_append_q8_0", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_PAGED_Q8_0,
      YVEX_ROCM_FN_KV_APPEND_Q8_0},
     {"yvex_rocm_history_append_bf16", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_BF16,

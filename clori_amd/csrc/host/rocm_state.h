@@ -37,6 +37,8 @@ typedef enum {
     YVEX_ROCM_FN_MLA_DECODE_BF16,
     YVEX_ROCM_FN_MLA_DECODE_512_BF16,
     YVEX_ROCM_FN_KV_APPEND_BF16,
+    YVEX_ROCM_FN_KV_APPEND_BF16_64,
+    YVEX_ROCM_FN_KV_APPEND_BF16_256,
     YVEX_ROCM_FN_KV_APPEND_Q8_0,
     YVEX_ROCM_FN_HISTORY_APPEND_BF16,
     YVEX_ROCM_FN_HISTORY_APPEND_F32,

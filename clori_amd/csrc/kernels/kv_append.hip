@@ -138,6 +138,7 @@ struct KeyChunk {
     int role;
 };
 
+template <int kDim = kHeadDim>
 __device__ inline void key_issue(const yvex_rocm_kv_append_params &p, const Span &s, uint32_t head,
                                  uint32_t id, KeyChunk &k)
 {
@@ -146,7 +147,7 @@ __device__ inline void key_issue(const yvex_rocm_kv_append_params &p, const Span
     k.c8 = id >> 4;
     k.role = k.c8 < pairs ? kLower : k.c8 < 2u * pairs ? kUpper : kPlain;
     const uint32_t row = row_of(s, k.t);
-    const uint16_t *base = p.key + ((uint64_t)row * p.kv_heads + head) * kHeadDim + k.c8 * 8u;
+    const uint16_t *base = p.key + ((uint64_t)row * p.kv_heads + head) * kDim + k.c8 * 8u;
     if (k.role != kUpper) k.own = load_b128(base);
     if (k.role == kLower) {
         const uint64_t at = (uint64_t)row * p.rotary_dim + k.c8 * 8u;
@@ -204,41 +205,47 @@ __device__ inline bool key_finish(const KeyChunk &k, u32x4 &lower, u32x4 &upper,
 
 }  // namespace
 
-// grid = (pages a session can touch, kv heads / 4, sessions), block 256: wave w writes kv head
-// 4 * blockIdx.y + w.
-extern "C" __global__ void __launch_bounds__(64 * kWaves)
-yvex_rocm_kv_append_bf16(const yvex_rocm_kv_append_params p)
+namespace {
+
+// The bf16 writer for one head dimension: a wave moves the 16 x kDim / 8 key chunks and as many
+// value chunks of its block, kDim / 32 of each per lane (128 is the tuned build; 64 and 256 are
+// the same code with other counts).
+template <int kDim>
+__device__ __forceinline__ void kv_append_bf16(const yvex_rocm_kv_append_params &p,
+                                               uint16_t (*v_rows_all)[kPageTokens][kDim + 8])
 {
-    __shared__ __attribute__((aligned(16))) uint16_t v_rows_all[kWaves][kPageTokens][kRowPitch];
+    constexpr int kPerLane = kDim / 32;          // 16-byte chunks of K (and of V) per lane
+    constexpr uint32_t kRowChunks = kDim / 8;    // 16-byte chunks of a row
+    constexpr int kRowPitch = kDim + 8;
     const Span s = locate(p);
     const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     const uint32_t head = blockIdx.y * kWaves + wave;
     const bool active = s.valid && head < p.kv_heads;
     uint16_t (*v_rows)[kRowPitch] = v_rows_all[wave];
     const uint64_t block = ((((uint64_t)s.page_id * p.kv_heads + head) << p.page_shift) + s.sub) *
-                           (kPageTokens * kHeadDim);
+                           (kPageTokens * kDim);
     uint16_t *kdst = (uint16_t *)p.k_pool + block, *vdst = (uint16_t *)p.v_pool + block;
     const bool partial = s.lo != 0u || s.hi != (uint32_t)kPageTokens;
     const uint32_t pairs = p.rotary_dim / 16u;
     bool ok = true;
-    KeyChunk k[4];
-    u32x4 v[4], old[4] = {};
+    KeyChunk k[kPerLane];
+    u32x4 v[kPerLane], old[kPerLane] = {};
     if (active) {
         // every load of the wave, then the arithmetic
 #pragma unroll
-        for (int i = 0; i < 4; ++i) key_issue(p, s, head, lane + 64u * i, k[i]);
+        for (int i = 0; i < kPerLane; ++i) key_issue<kDim>(p, s, head, lane + 64u * i, k[i]);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const uint32_t id = lane + 64u * i, t = id >> 4, c8 = id & 15u;
-            v[i] = load_b128(p.value + ((uint64_t)row_of(s, t) * p.kv_heads + head) * kHeadDim + c8 * 8u);
+        for (int i = 0; i < kPerLane; ++i) {
+            const uint32_t id = lane + 64u * i, t = id / kRowChunks, c8 = id % kRowChunks;
+            v[i] = load_b128(p.value + ((uint64_t)row_of(s, t) * p.kv_heads + head) * kDim + c8 * 8u);
         }
         if (partial) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) old[i] = load_b128(vdst + (lane + 64u * i) * 8u);
+            for (int i = 0; i < kPerLane; ++i) old[i] = load_b128(vdst + (lane + 64u * i) * 8u);
         }
         // keys: chunk (c8, t) sits at 16-byte slot c8 * 16 + t of the block
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < kPerLane; ++i) {
             u32x4 lower, upper;
             ok &= key_finish(k[i], lower, upper, p.rotary_mode != 0u);
             if (k[i].t < s.lo || k[i].t >= s.hi) continue;
@@ -249,8 +256,8 @@ yvex_rocm_kv_append_bf16(const yvex_rocm_kv_append_params p)
         }
         // values: rows into LDS, then 8 tokens of one dim per 16-byte piece
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const uint32_t id = lane + 64u * i, t = id >> 4, c8 = id & 15u;
+        for (int i = 0; i < kPerLane; ++i) {
+            const uint32_t id = lane + 64u * i, t = id / kRowChunks, c8 = id % kRowChunks;
             if (t >= s.lo && t < s.hi) ok &= finite_bits(v[i]);
             *reinterpret_cast<u32x4 *>(&v_rows[t][c8 * 8u]) = v[i];
         }
@@ -258,7 +265,7 @@ yvex_rocm_kv_append_bf16(const yvex_rocm_kv_append_params p)
     __syncthreads();
     if (active) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < kPerLane; ++i) {
             const uint32_t id = lane + 64u * i, c = id >> 1, t8 = (id & 1u) * 8u;
             if (t8 + 8u <= s.lo || t8 >= s.hi) continue;
             u32x4 w;
@@ -277,6 +284,21 @@ yvex_rocm_kv_append_bf16(const yvex_rocm_kv_append_params p)
         if (!ok) flag(p.status, YVEX_ROCM_DEVICE_NUMERIC);
     }
 }
+
+}  // namespace
+
+// grid = (pages a session can touch, kv heads / 4, sessions), block 256: wave w writes kv head
+// 4 * blockIdx.y + w.
+#define YVEX_KV_APPEND_BF16_KERNEL(name, head_dim)                                                   \
+    extern "C" __global__ void __launch_bounds__(64 * kWaves) name(const yvex_rocm_kv_append_params p) \
+    {                                                                                                \
+        __shared__ __attribute__((aligned(16))) uint16_t v_rows_all[kWaves][kPageTokens][head_dim + 8]; \
+        kv_append_bf16<head_dim>(p, v_rows_all);                                                      \
+    }
+
+YVEX_KV_APPEND_BF16_KERNEL(yvex_rocm_kv_append_bf16, 128)
+YVEX_KV_APPEND_BF16_KERNEL(yvex_rocm_kv_append_bf16_64, 64)
+YVEX_KV_APPEND_BF16_KERNEL(yvex_rocm_kv_append_bf16_256, 256)
 
 namespace {
 

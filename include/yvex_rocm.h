@@ -550,7 +550,8 @@ typedef enum {
 
 /*
  * Paged GQA decode: one query token per session against a paged KV pool.
- * Device page layouts (head_dimension 128), per (page, kv_head) and block of 16 tokens; a
+ * Device page layouts (head_dimension 128; bf16 pages also 64 and 256, with d/8 chunks of K
+ * and d rows of V in the same order), per (page, kv_head) and block of 16 tokens; a
  * page of 16 tokens (page_tokens 16) is one block, a page of 64 tokens (page_tokens 64) four
  * blocks one behind the other, tokens 16 s .. 16 s + 15 of the page in block s:
  *   BF16  K block: uint16 [d/8][16 tokens][8]           (4096 B)

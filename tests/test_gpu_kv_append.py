@@ -27,7 +27,7 @@ def expected_rows(canonical, k_new, v_new, table, starts, counts, row_starts, q8
 
 
 def run_case(backend, rng, starts, counts, storage, rotary_dim, pool_state="zero",
-             rotary_mode=B.ROTARY_BF16_STAGED):
+             rotary_mode=B.ROTARY_BF16_STAGED, d=D):
     sessions = len(starts)
     q8 = storage == B.KV_Q8_0
     stride = max((s + c + PAGE - 1) // PAGE for s, c in zip(starts, counts)) + 1
@@ -35,22 +35,23 @@ def run_case(backend, rng, starts, counts, storage, rotary_dim, pool_state="zero
     table = rng.permutation(pool_pages)[:sessions * stride].astype(np.int32).reshape(sessions, stride)
     total = int(sum(counts))
     row_starts = np.concatenate([[0], np.cumsum(counts)[:-1]]).astype(np.int32)
-    k_new = bf16_normal(rng, (total, HKV, D))
-    v_new = bf16_normal(rng, (total, HKV, D))
+    k_new = bf16_normal(rng, (total, HKV, d))
+    v_new = bf16_normal(rng, (total, HKV, d))
     angles = rng.uniform(-3.0, 3.0, size=(total, max(rotary_dim, 16))).astype(np.float32)
     cosine, sine = np.cos(angles).astype(np.float32), np.sin(angles).astype(np.float32)
     # pools start either zeroed or holding earlier tokens everywhere
-    row_width = (D // 32) * 34 if q8 else D
+    row_width = (d // 32) * 34 if q8 else d
     row_dtype = np.uint8 if q8 else np.uint16
     if pool_state == "zero":
         k_rows = np.zeros((pool_pages, PAGE, HKV, row_width), row_dtype)
         v_rows = np.zeros((pool_pages, PAGE, HKV, row_width), row_dtype)
     else:
-        old_k, old_v = bf16_normal(rng, (pool_pages, PAGE, HKV, D)), bf16_normal(rng, (pool_pages, PAGE, HKV, D))
+        old_k, old_v = bf16_normal(rng, (pool_pages, PAGE, HKV, d)), bf16_normal(rng, (pool_pages, PAGE, HKV, d))
         k_rows = q8_0_encode_rows(ORACLE.bf16_decode(old_k)).reshape(pool_pages, PAGE, HKV, -1) if q8 else old_k
         v_rows = q8_0_encode_rows(ORACLE.bf16_decode(old_v)).reshape(pool_pages, PAGE, HKV, -1) if q8 else old_v
     pool_dtype = B.DTYPE_I8 if q8 else B.DTYPE_BF16
-    kp, vp = kv_pack_pages(k_rows, storage, False, HKV), kv_pack_pages(v_rows, storage, True, HKV)
+    kp = kv_pack_pages(k_rows, storage, False, HKV, head_dim=d)
+    vp = kv_pack_pages(v_rows, storage, True, HKV, head_dim=d)
     elems = kp.size // B.DTYPE_BYTES[pool_dtype]
     t = dict(
         key=backend.tensor("k-new", B.DTYPE_BF16, k_new.shape, k_new),
@@ -69,10 +70,10 @@ def run_case(backend, rng, starts, counts, storage, rotary_dim, pool_state="zero
         t["page_table"], t["k_pool"], t["v_pool"], HKV, pool_pages, max(max(counts), 1),
         storage=storage, cosine=t["cosine"] if use_rotary else None,
         sine=t["sine"] if use_rotary else None, rotary_dimension=rotary_dim,
-        rotary_mode=rotary_mode)
+        rotary_mode=rotary_mode, head_dimension=d)
     assert facts.kernel_launches == 1
-    got_k = kv_unpack_pages(t["k_pool"].read(np.uint8, (-1,)), storage, False, pool_pages, HKV)
-    got_v = kv_unpack_pages(t["v_pool"].read(np.uint8, (-1,)), storage, True, pool_pages, HKV)
+    got_k = kv_unpack_pages(t["k_pool"].read(np.uint8, (-1,)), storage, False, pool_pages, HKV, head_dim=d)
+    got_v = kv_unpack_pages(t["v_pool"].read(np.uint8, (-1,)), storage, True, pool_pages, HKV, head_dim=d)
     if use_rotary and rotary_mode == B.ROTARY_F32_ROUNDED:
         k_rot = ORACLE.bf16_encode(ORACLE.rotary_half_f32_rounded(
             ORACLE.bf16_decode(k_new), cosine[:, :rotary_dim], sine[:, :rotary_dim], rotary_dim))
@@ -316,4 +317,34 @@ def test_append_into_pages_of_64_tokens(backend, storage):
     assert rc == 0
     assert_close_bf16(out.read(), ref, "decode over 64-token pages")
     for x in t + [tc, ts, tq, tctx, out]:
+        x.release()
+
+
+@pytest.mark.parametrize("d,rotary_dim", [(64, 0), (64, 32), (64, 64), (256, 0), (256, 64), (256, 256)])
+@pytest.mark.parametrize("rotary_mode", [B.ROTARY_BF16_STAGED, B.ROTARY_F32_ROUNDED], ids=["staged", "decoder"])
+def test_append_bf16_pages_at_other_head_dimensions(backend, d, rotary_dim, rotary_mode):
+    """bf16 pages at head dimension 64 and 256: every byte of both pools against the host-side
+    restatement, pools that already hold other tokens, both rotary orders, then a decode over
+    the written pages against the oracle."""
+    rng = np.random.default_rng(500 + d + rotary_dim)
+    starts, counts = [0, 5, 16, 31, 47, 100], [1, 1, 40, 0, 17, 33]
+    t, got, want, table, pool_pages = run_case(backend, rng, starts, counts, B.KV_BF16, rotary_dim,
+                                               "filled", rotary_mode=rotary_mode, d=d)
+    assert np.array_equal(got[0].reshape(want[0].shape), want[0])
+    assert np.array_equal(got[1].reshape(want[1].shape), want[1])
+    hq = 2 * HKV
+    contexts = np.array([s + c for s, c in zip(starts, counts)], np.int32)
+    q = bf16_normal(rng, (len(starts), hq, d))
+    tq = backend.tensor("q", B.DTYPE_BF16, q.shape, q)
+    tc = backend.tensor("ctx", B.DTYPE_I32, contexts.shape, contexts)
+    out = backend.tensor("o", B.DTYPE_BF16, q.shape)
+    lse = backend.tensor("lse", B.DTYPE_F32, (len(starts), hq))
+    req = backend.paged_requirement(len(starts), hq, HKV, d, PAGE, pool_pages, table.shape[1],
+                                    int(table.shape[1] * PAGE))
+    backend.paged_decode_execute(req, tq, t["k_pool"], t["v_pool"], t["page_table"], tc, out, lse)
+    rc, ref, _, ref_lse = ORACLE.paged_decode(q, want[0], want[1], table, contexts, HKV, PAGE)
+    assert rc == 0
+    assert_close_bf16(out.read(), ref, "decode over appended pages d=%d" % d)
+    assert_lse(lse.read(), ref_lse, "decode over appended pages d=%d" % d)
+    for x in list(t.values()) + [tq, tc, out, lse]:
         x.release()
