@@ -1,7 +1,5 @@
 // Log-sum-exp merge of the chunk partials of one (batch element, head) by one wave: eight
-// output dims per lane, one 16-byte piece of each chunk's bf16 accumulator row.  Shared by the
-// stand-alone merge kernel and by the decode kernel that merges in its own launch, so that both
-// publish the same bits.
+// output dims per lane, one 16-byte piece of each chunk's bf16 accumulator row.
 #ifndef YVEX_ROCM_KERNELS_MERGE_ROWS_H
 #define YVEX_ROCM_KERNELS_MERGE_ROWS_H
 
