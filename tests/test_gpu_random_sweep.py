@@ -57,9 +57,10 @@ def prefill_case(c):
     tk = start + tq if causal else tq + int(rng.integers(0, 400))
     if not causal:
         start = 0
-    q, k, v = c.bf16((tq, hq, 128)), c.bf16((tk, hkv, 128)), c.bf16((tk, hkv, 128))
-    gate = c.bf16((tq, hq, 128), 2.0) if rng.integers(0, 2) else None
-    req = b.attention_requirement(tq, tk, hq, hkv, 128, causal=causal, query_start=start,
+    d = int(rng.choice([128, 128, 64, 256]))
+    q, k, v = c.bf16((tq, hq, d)), c.bf16((tk, hkv, d)), c.bf16((tk, hkv, d))
+    gate = c.bf16((tq, hq, d), 2.0) if rng.integers(0, 2) else None
+    req = b.attention_requirement(tq, tk, hq, hkv, d, causal=causal, query_start=start,
                                   dtype=B.DTYPE_BF16, contract=CONTRACT)
     out, lse = c.tensor("o", B.DTYPE_BF16, q.shape), c.tensor("l", B.DTYPE_F32, (tq, hq))
     b.attention_execute(req, c.tensor("q", B.DTYPE_BF16, q.shape, q),
@@ -68,7 +69,7 @@ def prefill_case(c):
                         gate=c.tensor("g", B.DTYPE_BF16, gate.shape, gate) if gate is not None else None)
     rc, ref, _, ref_lse = ORACLE.gqa_bf16(q, k, v, query_start=start, causal=causal)
     assert rc == 0
-    label = ("prefill", tq, tk, start, hq, hkv, causal, gate is not None)
+    label = ("prefill", tq, tk, start, hq, hkv, d, causal, gate is not None)
     close(out.read(), gated(ref, gate) if gate is not None else ref, label)
     assert np.abs(lse.read() - ref_lse).max() <= LSE_ABS, label
 
@@ -89,16 +90,18 @@ def paged_case(c):
     for s in range(sessions):
         table[s, :need[s]] = perm[at:at + need[s]]
         at += int(need[s])
-    kr, vr = c.bf16((pool_pages, 16, hkv, 128)), c.bf16((pool_pages, 16, hkv, 128))
+    d = 128 if q8 else int(rng.choice([128, 128, 64, 256]))   # Q8_0 pages exist at 128 only
+    kr, vr = c.bf16((pool_pages, 16, hkv, d)), c.bf16((pool_pages, 16, hkv, d))
     storage, dtype = (B.KV_Q8_0, B.DTYPE_I8) if q8 else (B.KV_BF16, B.DTYPE_BF16)
     if q8:
         kr = q8_0_encode_rows(ORACLE.bf16_decode(kr))
         vr = q8_0_encode_rows(ORACLE.bf16_decode(vr))
-    kp, vp = kv_pack_pages(kr, storage, False, hkv), kv_pack_pages(vr, storage, True, hkv)
-    q = c.bf16((sessions, hq, 128))
+    kp = kv_pack_pages(kr, storage, False, hkv, head_dim=d)
+    vp = kv_pack_pages(vr, storage, True, hkv, head_dim=d)
+    q = c.bf16((sessions, hq, d))
     gate = c.bf16(q.shape, 2.0) if rng.integers(0, 2) else None
     out, lse = c.tensor("o", B.DTYPE_BF16, q.shape), c.tensor("l", B.DTYPE_F32, (sessions, hq))
-    req = b.paged_requirement(sessions, hq, hkv, 128, 16, pool_pages, stride, stride * 16,
+    req = b.paged_requirement(sessions, hq, hkv, d, 16, pool_pages, stride, stride * 16,
                               storage=storage)
     elements = kp.size // B.DTYPE_BYTES[dtype]
     b.paged_decode_execute(req, c.tensor("q", B.DTYPE_BF16, q.shape, q),
@@ -108,7 +111,7 @@ def paged_case(c):
                            gate=c.tensor("g", B.DTYPE_BF16, gate.shape, gate) if gate is not None else None)
     rc, ref, _, ref_lse = ORACLE.paged_decode(q, kr, vr, table, ctx, hkv, 16, q8=q8)
     assert rc == 0
-    label = ("paged", sessions, hq, hkv, q8, ctx.tolist(), gate is not None)
+    label = ("paged", sessions, hq, hkv, d, q8, ctx.tolist(), gate is not None)
     close(out.read(), gated(ref, gate) if gate is not None else ref, label)
     assert np.abs(lse.read() - ref_lse).max() <= LSE_ABS, label
 

@@ -14,15 +14,15 @@ from test_gpu_decode import make_paged_case
 pytestmark = pytest.mark.gpu
 
 
-def run_both(backend, contexts, hq, hkv, storage, seed):
+def run_both(backend, contexts, hq, hkv, storage, seed, d=128):
     rng = np.random.default_rng(seed)
-    q, k_rows, v_rows, table, ctx, pool_pages = make_paged_case(rng, contexts, hq, hkv)
+    q, k_rows, v_rows, table, ctx, pool_pages = make_paged_case(rng, contexts, hq, hkv, d=d)
     if storage == B.KV_Q8_0:
         from clori_amd.backend import q8_0_encode_rows
         k_rows = q8_0_encode_rows(ORACLE.bf16_decode(k_rows))
         v_rows = q8_0_encode_rows(ORACLE.bf16_decode(v_rows))
-    kp = kv_pack_pages(k_rows, storage, False, hkv)
-    vp = kv_pack_pages(v_rows, storage, True, hkv)
+    kp = kv_pack_pages(k_rows, storage, False, hkv, head_dim=d)
+    vp = kv_pack_pages(v_rows, storage, True, hkv, head_dim=d)
     pool_dtype = B.DTYPE_BF16 if storage == B.KV_BF16 else B.DTYPE_I8
     elems = kp.size // B.DTYPE_BYTES[pool_dtype]
     sessions = len(contexts)
@@ -31,7 +31,7 @@ def run_both(backend, contexts, hq, hkv, storage, seed):
     tvp = backend.tensor("vpool", pool_dtype, (elems,), vp)
     tt = backend.tensor("table", B.DTYPE_I32, table.shape, table)
     tc = backend.tensor("ctx", B.DTYPE_I32, ctx.shape, ctx)
-    req = backend.paged_requirement(sessions, hq, hkv, 128, 16, pool_pages, table.shape[1],
+    req = backend.paged_requirement(sessions, hq, hkv, d, 16, pool_pages, table.shape[1],
                                     int(table.shape[1] * 16), storage=storage)
     results = []
     for static in (False, True):
@@ -60,6 +60,12 @@ def test_static_entry_matches_paged_decode_twice_in_a_row(backend, storage):
     # large first (every wave slot of the scratch is written), then a smaller request
     run_both(backend, [3000, 17, 1024, 2049, 555, 4096, 1, 800], 32, 8, storage, seed=11)
     run_both(backend, [40, 700, 129], 8, 2, storage, seed=12)
+
+
+@pytest.mark.parametrize("d,hq,hkv", [(64, 16, 4), (256, 24, 4)])
+def test_static_entry_at_other_head_dimensions(backend, d, hq, hkv):
+    run_both(backend, [3000, 17, 1024, 2049, 555, 4096, 1, 800], hq, hkv, B.KV_BF16, seed=14, d=d)
+    run_both(backend, [40, 700, 129], hq, hkv, B.KV_BF16, seed=15, d=d)
 
 
 def test_static_entry_refuses_what_does_not_fit(backend):
