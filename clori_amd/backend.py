@@ -370,6 +370,30 @@ class Backend:
         _check(rc, err)
         return facts
 
+    def _elementwise(self, slot, *arguments):
+        ops = self.transformer_operations()
+        if ops is None or not getattr(ops, slot):
+            raise YvexError(B.YVEX_ERR_UNSUPPORTED, "transformer_operations", "not published")
+        facts, err = B.OperationFacts(), B.Error()
+        _check(getattr(ops, slot)(self.handle, *arguments, C.byref(facts), C.byref(err)), err)
+        return facts
+
+    def rotary_half_f32(self, values, cosines, sines, tokens, heads, head_dim, rotary_dim):
+        """The reference's rotary_half_f32 slot: plain F32 rotate-half of `values` in place."""
+        return self._elementwise("rotary_half_f32", values.handle, cosines.handle, sines.handle,
+                                 tokens, heads, head_dim, rotary_dim)
+
+    def split_interleaved_two_f32(self, source, first, second, rows, heads, head_dim):
+        return self._elementwise("split_interleaved_two_f32", source.handle, first.handle,
+                                 second.handle, rows, heads, head_dim)
+
+    def sigmoid_product_bf16(self, values, gate, output, count):
+        return self._elementwise("sigmoid_product_bf16", values.handle, gate.handle, output.handle,
+                                 count)
+
+    def bf16_round(self, values, count):
+        return self._elementwise("bf16_round", values.handle, count)
+
     @staticmethod
     def paged_requirement(sessions, query_heads, kv_heads, head_dim, page_tokens, pool_pages,
                           table_stride, max_context, storage=B.KV_BF16,

@@ -207,9 +207,20 @@ TRANSFORMER_OPERATION_SLOTS = (
     "bf16_round", "dense_decoder_execute")
 
 
+ROTARY_HALF_FN = C.CFUNCTYPE(C.c_int, C.c_void_p, TensorP, TensorP, TensorP, ull, ull, ull, ull, FactsP,
+                             ErrorP)
+SPLIT_TWO_FN = C.CFUNCTYPE(C.c_int, C.c_void_p, TensorP, TensorP, TensorP, ull, ull, ull, FactsP, ErrorP)
+BINARY_FN = C.CFUNCTYPE(C.c_int, C.c_void_p, TensorP, TensorP, TensorP, ull, FactsP, ErrorP)
+ROUND_FN = C.CFUNCTYPE(C.c_int, C.c_void_p, TensorP, ull, FactsP, ErrorP)
+
+
 class TransformerOperations(C.Structure):
     _fields_ = [(name, {"attention_workspace_required": WORKSPACE_FN,
-                        "attention_execute": EXECUTE_FN}.get(name, C.c_void_p))
+                        "attention_execute": EXECUTE_FN,
+                        "rotary_half_f32": ROTARY_HALF_FN,
+                        "split_interleaved_two_f32": SPLIT_TWO_FN,
+                        "sigmoid_product_bf16": BINARY_FN,
+                        "bf16_round": ROUND_FN}.get(name, C.c_void_p))
                 for name in TRANSFORMER_OPERATION_SLOTS]
 
 

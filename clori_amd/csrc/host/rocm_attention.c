@@ -1490,9 +1490,15 @@ static int rocm_history_append_execute(yvex_backend *backend,
 
 /* ---------------------------------------------------------- op tables ---- */
 
+/* The attention slots and the four element-wise slots the reference's decoder calls around
+ * them; every other slot stays NULL ("not published"). */
 static const yvex_backend_transformer_operations rocm_transformer_ops = {
     .attention_workspace_required = rocm_attention_workspace_required,
     .attention_execute = rocm_attention_execute,
+    .rotary_half_f32 = yvex_rocm_rotary_half_f32,
+    .split_interleaved_two_f32 = yvex_rocm_split_interleaved_two_f32,
+    .sigmoid_product_bf16 = yvex_rocm_sigmoid_product_bf16,
+    .bf16_round = yvex_rocm_bf16_round,
 };
 
 static const yvex_backend_rocm_attention_operations rocm_attention_ops = {

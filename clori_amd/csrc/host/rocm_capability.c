@@ -44,6 +44,13 @@ static const rocm_kernel_binding rocm_kernel_bindings[] = {
      YVEX_ROCM_FN_GQA_F32_TILE_256},
     {"yvex_rocm_fill_u32", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_F32, YVEX_ROCM_FN_FILL_U32},
     {"yvex_rocm_stream_read", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_F32, YVEX_ROCM_FN_STREAM_READ},
+    {"yvex_rocm_rotary_half_plain_f32", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_F32,
+     YVEX_ROCM_FN_ROTARY_HALF_PLAIN_F32},
+    {"yvex_rocm_bf16_round_f32", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_F32, YVEX_ROCM_FN_BF16_ROUND_F32},
+    {"yvex_rocm_sigmoid_product_bf16_f32", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_F32,
+     YVEX_ROCM_FN_SIGMOID_PRODUCT_BF16_F32},
+    {"yvex_rocm_split_interleaved_two_f32", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_F32,
+     YVEX_ROCM_FN_SPLIT_INTERLEAVED_TWO_F32},
     {"yvex_rocm_decode_paged_bf16", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_PAGED_BF16,
      YVEX_ROCM_FN_DECODE_PAGED_BF16},
     {"yvex_rocm_decode_paged_bf16_64", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_PAGED_BF16,

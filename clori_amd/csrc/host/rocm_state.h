@@ -43,6 +43,10 @@ typedef enum {
     YVEX_ROCM_FN_HISTORY_APPEND_BF16,
     YVEX_ROCM_FN_HISTORY_APPEND_F32,
     YVEX_ROCM_FN_STREAM_READ,
+    YVEX_ROCM_FN_ROTARY_HALF_PLAIN_F32,
+    YVEX_ROCM_FN_BF16_ROUND_F32,
+    YVEX_ROCM_FN_SIGMOID_PRODUCT_BF16_F32,
+    YVEX_ROCM_FN_SPLIT_INTERLEAVED_TWO_F32,
     YVEX_ROCM_FN_GATHER_ROWS,
     YVEX_ROCM_FN_COUNT
 } yvex_rocm_function_id;
@@ -180,6 +184,24 @@ int yvex_rocm_op_attention(yvex_backend *backend, const yvex_device_tensor *quer
                            int causal, yvex_device_tensor *score_scratch,
                            yvex_device_tensor *probability_scratch, yvex_device_tensor *out,
                            yvex_error *err);
+/* rocm_elementwise.c: the element-wise slots of the transformer operations table */
+int yvex_rocm_rotary_half_f32(yvex_backend *backend, yvex_device_tensor *values,
+                              const yvex_device_tensor *cosines, const yvex_device_tensor *sines,
+                              unsigned long long tokens, unsigned long long heads,
+                              unsigned long long head_dim, unsigned long long rotary_dim,
+                              yvex_backend_operation_facts *facts, yvex_error *err);
+int yvex_rocm_bf16_round(yvex_backend *backend, yvex_device_tensor *values, unsigned long long count,
+                         yvex_backend_operation_facts *facts, yvex_error *err);
+int yvex_rocm_sigmoid_product_bf16(yvex_backend *backend, const yvex_device_tensor *values,
+                                   const yvex_device_tensor *gate, yvex_device_tensor *output,
+                                   unsigned long long count, yvex_backend_operation_facts *facts,
+                                   yvex_error *err);
+int yvex_rocm_split_interleaved_two_f32(yvex_backend *backend, const yvex_device_tensor *input,
+                                        yvex_device_tensor *first, yvex_device_tensor *second,
+                                        unsigned long long rows, unsigned long long heads,
+                                        unsigned long long head_dimension,
+                                        yvex_backend_operation_facts *facts, yvex_error *err);
+
 const yvex_backend_transformer_operations *yvex_rocm_transformer_operations(
     const yvex_backend *backend);
 #endif /* YVEX_ROCM_STATE_H */

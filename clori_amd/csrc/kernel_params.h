@@ -119,6 +119,21 @@ typedef struct {
     double rope_frequency[YVEX_ROCM_ROPE_PAIRS_MAX];
 } yvex_rocm_decode_merge_params;
 
+/* The element-wise operators the reference's decoder runs around attention on F32 activations
+ * (src/runtime/decoder.c:989-997,1030-1046,1112-1131,1266-1269): one thread per element (per
+ * rotated pair for the rotation), blocks of YVEX_ROCM_ELEMENTWISE_BLOCK threads.
+ *   rotary:  values in place, left = cosines, right = sines [tokens][rotary_dim]; count pairs
+ *   round:   values in place; a value that is not finite sets the status word
+ *   sigmoid: values = output, left = values, right = gate
+ *   split:   left = input [rows][heads][2][head_dim], values = first, second = second */
+#define YVEX_ROCM_ELEMENTWISE_BLOCK 256
+typedef struct {
+    float *values, *second;
+    const float *left, *right;
+    int32_t *status;
+    uint64_t count, heads, head_dim, rotary_dim;
+} yvex_rocm_elementwise_params;
+
 /* Causal / full GQA prefill on bf16 token-major tensors.  The grid is one-dimensional:
  * query_heads * ceil(query_tokens / YVEX_ROCM_PREFILL_ROWS) workgroups of 256 threads. */
 #define YVEX_ROCM_PREFILL_ROWS 128

@@ -428,10 +428,18 @@ typedef struct yvex_transformer_attention_request {
  * every member of the reference table, in the reference's order and with the reference's
  * signatures, so that a caller compiled against the reference header finds
  * attention_workspace_required and attention_execute at the same offsets in the table
- * this backend returns.  The request/plan types of the slots this backend does not
- * publish are opaque here (only pointers to them cross the boundary); those slots are
- * NULL in the ROCm table, which the reference's callers treat as "not published" and
- * refuse with YVEX_ERR_UNSUPPORTED (src/runtime/stateful_attention.c:294-298). */
+ * this backend returns.  Published by this backend: the two attention slots and the four
+ * element-wise slots the reference's decoder calls around them on F32 activations
+ * (src/runtime/decoder.c:989-997,1112-1131,1225-1270): rotary_half_f32 (the plain F32
+ * rotate-half, src/backend/cuda/transformer.c:460-470), split_interleaved_two_f32
+ * (src/backend/cuda/decoder.c:11-73), sigmoid_product_bf16 (src/backend/cuda/decoder.c:75-130)
+ * and bf16_round (src/backend/cuda/transformer.c:1356-1392), each with the reference's
+ * validation (YVEX_ERR_FORMAT for anything but packed, written F32 tensors of this backend
+ * with the declared counts; bf16_round also for a value that is not finite).  The request/plan
+ * types of the slots this backend does not publish are opaque here (only pointers to them
+ * cross the boundary); those slots are NULL in the ROCm table, which the reference's callers
+ * treat as "not published" and refuse with YVEX_ERR_UNSUPPORTED
+ * (src/runtime/stateful_attention.c:294-298). */
 typedef struct yvex_gated_delta_plan yvex_gated_delta_plan;
 typedef struct yvex_gated_delta_device_request yvex_gated_delta_device_request;
 typedef struct yvex_gated_delta_device_result yvex_gated_delta_device_result;

@@ -805,6 +805,21 @@ int yvo_rotary_half_f32_rounded(float *values, const float *cosines, const float
                                 uint64_t tokens, uint64_t heads, uint64_t head_dim,
                                 uint64_t rotary_dim)
 {
+    uint64_t index;
+    const int rc = yvo_rotary_half_plain_f32(values, cosines, sines, tokens, heads, head_dim, rotary_dim);
+    if (rc != 0) return rc;
+    for (index = 0; index < tokens * heads * head_dim; ++index)
+        values[index] = yvo_bf16_decode(yvo_bf16_encode(values[index]));
+    return 0;
+}
+
+/* The rotation alone (the kernel behind the rotary_half_f32 operator slot,
+ * src/backend/cuda/capability.c:35, src/backend/cuda/transformer_kernels.cu:110-134), nothing
+ * rounded to bf16, with the contraction described above. */
+int yvo_rotary_half_plain_f32(float *values, const float *cosines, const float *sines,
+                              uint64_t tokens, uint64_t heads, uint64_t head_dim,
+                              uint64_t rotary_dim)
+{
     const uint64_t half = rotary_dim / 2u;
     uint64_t vector, lane;
     if (!values || !cosines || !sines || !tokens || !heads || !half || rotary_dim > head_dim)
@@ -820,8 +835,6 @@ int yvo_rotary_half_f32_rounded(float *values, const float *cosines, const float
             base[lane] = fmaf(first, cosine, -second_sine);
             base[half + lane] = fmaf(second, cosine, first_sine);
         }
-        for (lane = 0; lane < head_dim; ++lane)
-            base[lane] = yvo_bf16_decode(yvo_bf16_encode(base[lane]));
     }
     return 0;
 }

@@ -47,6 +47,9 @@
  *       (tests/unit/cuda/quant_qtype.c:3050-3105), identity, quarter turn, float64
  *       rotation within one bf16 rounding; the choice of fused product is
  *       parity unpinned (results within a float rounding of a bf16 tie)
+ *   yvo_rotary_half_plain_f32        pinned: the same known-answer case (exact in float),
+ *       identity, quarter turn, float64 rotation within two float roundings; the
+ *       choice of fused product is parity unpinned (the last bit of a result)
  *   yvo_sigmoid_gate_bf16            pinned: known-answer case
  *       (tests/unit/cuda/quant_qtype.c:2979-2981,3019-3033), closed forms
  *   yvo_paged_*, the page tables and LSE output of yvo_mla_*, the selected
@@ -265,6 +268,13 @@ int yvo_rotary_half_f32(float *values, const float *cosines, const float *sines,
 int yvo_rotary_half_f32_rounded(float *values, const float *cosines, const float *sines,
                                 uint64_t tokens, uint64_t heads, uint64_t head_dim,
                                 uint64_t rotary_dim);
+/* The rotation alone, nothing rounded to bf16: what the rotary_half_f32 operator slot runs
+ * (src/backend/cuda/capability.c:35 binds it to yvex_rotary_half_plain_f32).  Same pins; with
+ * no bf16 rounding behind it the unpinned choice of fused product is the last bit of every
+ * result that is not exact. */
+int yvo_rotary_half_plain_f32(float *values, const float *cosines, const float *sines,
+                              uint64_t tokens, uint64_t heads, uint64_t head_dim,
+                              uint64_t rotary_dim);
 
 /*
  * Sigmoid output gate on attention rows: out = bf16(values * (1 / (1 + expf(-gate)))), all

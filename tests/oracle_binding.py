@@ -66,6 +66,7 @@ def load_oracle():
     lib.yvo_rotary_half_bf16.argtypes = [u16p, f32p, f32p] + [u64] * 4
     lib.yvo_rotary_half_f32.argtypes = [f32p, f32p, f32p] + [u64] * 4
     lib.yvo_rotary_half_f32_rounded.argtypes = [f32p, f32p, f32p] + [u64] * 4
+    lib.yvo_rotary_half_plain_f32.argtypes = [f32p, f32p, f32p] + [u64] * 4
     lib.yvo_sigmoid_gate_bf16.argtypes = [f32p, f32p, u64, f32p]
     lib.yvo_mla_decode_bf16.argtypes = [u16p, u16p, i32p, i32p, f32p, u16p, f64p] + [u64] * 7 + [f32p, u64, u16p, i32p, i32p, u64, u64, i32p, u64, C.c_int]
     lib.yvo_yarn_frequency.restype = C.c_double
@@ -282,6 +283,17 @@ class Oracle:
         sines = np.ascontiguousarray(sines, dtype=np.float32)
         rc = self.lib.yvo_rotary_half_f32_rounded(_ptr(out, f32p), _ptr(cosines, f32p),
                                                   _ptr(sines, f32p), tokens, heads, d, rotary_dim)
+        assert rc == 0
+        return out
+
+    def rotary_half_plain_f32(self, values, cosines, sines, rotary_dim):
+        """values float32 [tokens, heads, d] -> plain F32 rotation, nothing rounded to bf16."""
+        out = np.ascontiguousarray(values, dtype=np.float32).copy()
+        tokens, heads, d = out.shape
+        cosines = np.ascontiguousarray(cosines, dtype=np.float32)
+        sines = np.ascontiguousarray(sines, dtype=np.float32)
+        rc = self.lib.yvo_rotary_half_plain_f32(_ptr(out, f32p), _ptr(cosines, f32p),
+                                                _ptr(sines, f32p), tokens, heads, d, rotary_dim)
         assert rc == 0
         return out
 

@@ -149,7 +149,8 @@ def test_ready_backend_publishes_attention_only():
 
 def test_encoded_attention_transaction_fails_closed():
     """include/yvex/internal/backend.h:193-198: the symbol exists and refuses; the table the
-    backend returns has the reference's slot order with only the attention slots published."""
+    backend returns has the reference's slot order with the attention slots and the element-wise slots
+    the decoder calls around them published, the rest NULL."""
     library = lib()
 
     class Failure(C.Structure):
@@ -176,7 +177,9 @@ def test_encoded_attention_transaction_fails_closed():
         ops = b.transformer_operations()
         for name in B.TRANSFORMER_OPERATION_SLOTS:
             published = bool(getattr(ops, name))
-            assert published == (name in ("attention_workspace_required", "attention_execute")), name
+            assert published == (name in ("attention_workspace_required", "attention_execute",
+                                              "rotary_half_f32", "split_interleaved_two_f32",
+                                              "sigmoid_product_bf16", "bf16_round")), name
 
 
 @pytest.mark.parametrize("injected,reason_for_attention", [
@@ -1240,3 +1243,40 @@ def test_page_layouts_follow_the_documented_index_formulas():
                     assert np.array_equal(packed[page, head][index], wide_rows[page, :, head, :])
             back = kv_unpack_pages(packed, B.KV_BF16, is_value, pages, hkv, head_dim=width)
             assert np.array_equal(back, wide_rows)
+
+
+def test_elementwise_slots_validate_like_the_reference():
+    """The element-wise slots of the transformer operations table on the stand-in runtime: one
+    launch and one synchronisation each, outputs marked written, and YVEX_ERR_FORMAT for anything
+    but packed, written F32 tensors of this backend with the declared counts
+    (src/backend/cuda/transformer.c:409-441,1356-1372, src/backend/cuda/decoder.c:11-47,75-103);
+    a backend that is closing refuses first (YVEX_ERR_STATE)."""
+    with Backend() as b, Backend() as other:
+        x = written(b, "x", B.DTYPE_F32, (2, 4, 16))
+        table = written(b, "t", B.DTYPE_F32, (2, 8))
+        out, gate = b.tensor("o", B.DTYPE_F32, (2, 4, 16)), written(b, "g", B.DTYPE_F32, (2, 4, 16))
+        first, second = b.tensor("a", B.DTYPE_F32, (64,)), b.tensor("b", B.DTYPE_F32, (64,))
+        for facts in (b.rotary_half_f32(x, table, table, 2, 4, 16, 8), b.bf16_round(x, 128),
+                      b.sigmoid_product_bf16(x, gate, out, 128),
+                      b.split_interleaved_two_f32(x, first, second, 2, 2, 16)):
+            assert facts.kernel_launches == 1 and facts.device_synchronizations == 1
+        assert out.is_written and first.is_written and second.is_written
+        foreign = written(other, "f", B.DTYPE_F32, (2, 4, 16))
+        half = written(b, "h", B.DTYPE_BF16, (128,))
+        fresh = b.tensor("n", B.DTYPE_F32, (128,))
+        for call in (lambda: b.rotary_half_f32(x, table, table, 2, 4, 16, 7),
+                     lambda: b.rotary_half_f32(x, table, table, 2, 4, 16, 0),
+                     lambda: b.rotary_half_f32(x, table, table, 2, 4, 16, 32),
+                     lambda: b.rotary_half_f32(x, table, table, 2, 4, 16, 16),   # tables too short
+                     lambda: b.rotary_half_f32(foreign, table, table, 2, 4, 16, 8),
+                     lambda: b.rotary_half_f32(fresh, table, table, 2, 4, 16, 8),
+                     lambda: b.bf16_round(x, 127), lambda: b.bf16_round(half, 128),
+                     lambda: b.bf16_round(fresh, 128),
+                     lambda: b.sigmoid_product_bf16(x, fresh, out, 128),
+                     lambda: b.sigmoid_product_bf16(x, gate, half, 128),
+                     lambda: b.sigmoid_product_bf16(x, gate, out, 0),
+                     lambda: b.split_interleaved_two_f32(x, first, first, 2, 2, 16),
+                     lambda: b.split_interleaved_two_f32(x, first, second, 2, 4, 16)):
+            with pytest.raises(YvexError) as e:
+                call()
+            assert e.value.code == B.YVEX_ERR_FORMAT

@@ -597,6 +597,45 @@ def test_rotary_rounded_pins():
         assert np.max(np.abs(staged - got)[..., :rotary]) <= 3 * 2.0 ** -8 * np.max(np.abs(x))
 
 
+def test_rotary_plain_pins():
+    """The rotation alone (what the rotary_half_f32 operator slot runs): the reference's
+    known-answer case (tests/unit/cuda/quant_qtype.c:3050-3105), identity, quarter turn, a
+    float64 rotation within two float roundings, the unfused expression within one float
+    rounding, and the rounded form as this one followed by the bf16 rounding."""
+    values = np.array([[[1.0, 2.0], [7.0, 8.0]]], np.float32)
+    cosines, sines = np.full((1, 2), 0.75, np.float32), np.full((1, 2), 0.5, np.float32)
+    assert ORACLE.rotary_half_plain_f32(values, cosines, sines, 2).tolist() == \
+        [[[-0.25, 2.0], [1.25, 9.5]]]
+    rng = np.random.default_rng(47)
+    tokens, heads, d = 5, 3, 64
+    x = rng.standard_normal((tokens, heads, d)).astype(np.float32)
+    for rotary in (2, 16, 64):
+        half = rotary // 2
+        one, zero = np.ones((tokens, rotary), np.float32), np.zeros((tokens, rotary), np.float32)
+        assert np.array_equal(ORACLE.rotary_half_plain_f32(x, one, zero, rotary), x)
+        quarter = ORACLE.rotary_half_plain_f32(x, zero, one, rotary)
+        assert np.array_equal(quarter[..., :half], -x[..., half:rotary])
+        assert np.array_equal(quarter[..., half:rotary], x[..., :half])
+        assert np.array_equal(quarter[..., rotary:], x[..., rotary:])
+        angles = rng.uniform(-3.0, 3.0, (tokens, rotary))
+        cosines, sines = np.cos(angles).astype(np.float32), np.sin(angles).astype(np.float32)
+        got = ORACLE.rotary_half_plain_f32(x, cosines, sines, rotary)
+        c, s = cosines[:, None, :half].astype(np.float64), sines[:, None, :half].astype(np.float64)
+        a, b = x[..., :half].astype(np.float64), x[..., half:rotary].astype(np.float64)
+        exact = np.concatenate([a * c - b * s, b * c + a * s, x[..., rotary:]], axis=-1)
+        scale = np.concatenate([np.abs(a * c) + np.abs(b * s), np.abs(b * c) + np.abs(a * s),
+                                np.zeros_like(x[..., rotary:], np.float64)], axis=-1)
+        assert np.all(np.abs(got - exact) <= 2.0 ** -23 * scale)
+        cf, sf = cosines[:, None, :half], sines[:, None, :half]
+        af, bf = x[..., :half], x[..., half:rotary]
+        unfused = np.concatenate([(af * cf).astype(np.float32) - (bf * sf).astype(np.float32),
+                                  (bf * cf).astype(np.float32) + (af * sf).astype(np.float32),
+                                  x[..., rotary:]], axis=-1).astype(np.float32)
+        assert np.all(np.abs(unfused.astype(np.float64) - got) <= 2.0 ** -23 * scale)
+        assert np.array_equal(ORACLE.bf16_decode(ORACLE.bf16_encode(got)),
+                              ORACLE.rotary_half_f32_rounded(x, cosines, sines, rotary))
+
+
 # -------------------------------------------------------- output gate -------
 
 def test_sigmoid_gate_reference_known_answer():
