@@ -569,6 +569,10 @@ static int attention_execute_common(yvex_backend *backend,
             if (groups > 0x7fffffffull)
                 return refuse(err, YVEX_ERR_BOUNDS, "rocm.transformer.gqa",
                               "attention geometry exceeds the launch range");
+            /* two workgroups per unit at head dimension 64 and 128 (registers and LDS), one at 256 */
+            if (causal && r->head_dimension != 256ull && state->compute_units > 0 &&
+                groups >= 2ull * (unsigned long long)state->compute_units)
+                params.pair_units = (uint32_t)state->compute_units;
             rc = yvex_rocm_launch(backend, tile_function, YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_F32,
                                   (unsigned int)groups, 1u, 1u, 256u, 0u, &params,
                                   "rocm.transformer.gqa", err);

@@ -41,6 +41,9 @@ typedef struct {
     double *part_acc, *part_ml;
     uint32_t splits, keys_per_split;
     uint32_t *arrivals;
+    /* tile form (yvex_rocm_gqa_f32_tile_*): compute units when workgroups b and b + units share
+     * a unit and are to carry equal work (causal launches of at least two tiers of items), else 0 */
+    uint32_t pair_units, reserved_tile;
 } yvex_rocm_gqa_f32_params;
 
 typedef struct {
