@@ -570,12 +570,31 @@ static int attention_execute_common(yvex_backend *backend,
                 return refuse(err, YVEX_ERR_BOUNDS, "rocm.transformer.gqa",
                               "attention geometry exceeds the launch range");
             /* two workgroups per unit at head dimension 64 and 128 (registers and LDS), one at 256 */
-            if (causal && r->head_dimension != 256ull && state->compute_units > 0 &&
-                groups >= 2ull * (unsigned long long)state->compute_units)
-                params.pair_units = (uint32_t)state->compute_units;
+            const unsigned int per_unit = r->head_dimension == 256ull ? 1u : 2u;
+            unsigned int workgroups = 0u;
+            if (causal) {
+                /* a geometry that repeats gets item lists with equal work per unit; until then,
+                 * and when no lists can be made, the pairs of workgroups of a unit at least sum
+                 * to the same */
+                yvex_rocm_schedule_key key;
+                memset(&key, 0, sizeof(key));
+                key.query_tokens = r->query_tokens;
+                key.kv_tokens = r->key_value_tokens;
+                key.query_start = r->query_start;
+                key.query_heads = (uint32_t)r->query_heads;
+                key.item_rows = (uint32_t)ROCM_EXACT_TILE_QUERIES;
+                key.step_keys = 32u;
+                key.per_unit = per_unit;
+                key.kind = (uint32_t)tile_function;
+                if (r->query_heads <= 0xffffull)
+                    workgroups = yvex_rocm_schedule_lists(backend, &key, &params.lists);
+                if (!workgroups && per_unit == 2u && state->compute_units > 0 &&
+                    groups >= 2ull * (unsigned long long)state->compute_units)
+                    params.pair_units = (uint32_t)state->compute_units;
+            }
             rc = yvex_rocm_launch(backend, tile_function, YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_F32,
-                                  (unsigned int)groups, 1u, 1u, 256u, 0u, &params,
-                                  "rocm.transformer.gqa", err);
+                                  workgroups ? workgroups : (unsigned int)groups, 1u, 1u, 256u, 0u,
+                                  &params, "rocm.transformer.gqa", err);
             tiled = 1;
         } else if ((split_runs = exact_split_runs(r, &split_keys)) != 0ull &&
                    !(((uintptr_t)request->query->data | (uintptr_t)request->key->data |

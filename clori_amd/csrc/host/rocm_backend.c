@@ -542,6 +542,7 @@ static int rocm_close(yvex_backend *backend, yvex_error *err)
     if (rc != YVEX_OK) return rc; /* impl retained: checked close can be retried */
     if (state->device_status) (void)state->driver.hipFree(state->device_status);
     if (state->decode_arrivals) (void)state->driver.hipFree(state->decode_arrivals);
+    if (state->schedule_device) (void)state->driver.hipFree(state->schedule_device);
     probe_release(state);
     if (state->timing_start) (void)state->driver.hipEventDestroy(state->timing_start);
     if (state->timing_stop) (void)state->driver.hipEventDestroy(state->timing_stop);
@@ -699,6 +700,11 @@ static int rocm_open(yvex_backend **out, const char *device, unsigned long long 
                                                            state->stream),
                               where, err);
     if (rc == YVEX_OK)
+        rc = yvex_rocm_status(&state->driver,
+                              state->driver.hipMalloc((void **)&state->schedule_device,
+                                                      sizeof(state->schedule.rows)),
+                              where, err);
+    if (rc == YVEX_OK)
         rc = yvex_rocm_status(&state->driver, state->driver.hipStreamSynchronize(state->stream),
                               where, err);
     if (rc != YVEX_OK) {
@@ -706,6 +712,7 @@ static int rocm_open(yvex_backend **out, const char *device, unsigned long long 
         yvex_error scratch;
         if (state->device_status) (void)state->driver.hipFree(state->device_status);
         if (state->decode_arrivals) (void)state->driver.hipFree(state->decode_arrivals);
+        if (state->schedule_device) (void)state->driver.hipFree(state->schedule_device);
         if (state->timing_start) (void)state->driver.hipEventDestroy(state->timing_start);
         if (state->timing_stop) (void)state->driver.hipEventDestroy(state->timing_stop);
         if (state->stream) (void)state->driver.hipStreamDestroy(state->stream);

@@ -61,6 +61,20 @@ typedef enum {
     YVEX_ROCM_KERNEL_BUNDLE_REJECTED
 } yvex_rocm_kernel_bundle_state;
 
+/* What decides the item lists of a causal launch (rocm_schedule.c); zero the padding, the key
+ * is compared as bytes. */
+#define YVEX_ROCM_LISTS_MAX 512u
+#define YVEX_ROCM_LIST_STRIDE 8u
+#define YVEX_ROCM_LIST_ITEMS_MAX 2048u
+typedef struct {
+    unsigned long long query_tokens, kv_tokens, query_start;
+    uint32_t query_heads;
+    uint32_t item_rows;  /* query rows of an item */
+    uint32_t step_keys;  /* keys of one step of an item's walk */
+    uint32_t per_unit;   /* workgroups of the kernel that fit a compute unit */
+    uint32_t kind, reserved; /* kernel family the lists are for */
+} yvex_rocm_schedule_key;
+
 typedef struct yvex_rocm_backend_state {
     yvex_rocm_driver driver;
     int device_index;
@@ -96,6 +110,14 @@ typedef struct yvex_rocm_backend_state {
     unsigned long long recorded_launches; /* kernel launches of the sequence being recorded */
     void *static_scratch;     /* device address of the fixed scratch array on this device, or NULL */
     int static_scratch_error; /* the runtime's code when it could not be resolved */
+    /* the item lists of the last scheduled causal launch (rocm_schedule.c): the geometry, how
+     * often it came in a row, the rows on the host and on the device */
+    struct {
+        yvex_rocm_schedule_key key;
+        uint32_t lists, seen;
+        uint16_t rows[YVEX_ROCM_LISTS_MAX * YVEX_ROCM_LIST_STRIDE];
+    } schedule;
+    uint16_t *schedule_device;
     int bandwidth_ready; /* the probe ran: later calls return the kept evidence */
     yvex_backend_bandwidth_evidence bandwidth_evidence;
 } yvex_rocm_backend_state;
@@ -201,6 +223,10 @@ int yvex_rocm_split_interleaved_two_f32(yvex_backend *backend, const yvex_device
                                         unsigned long long rows, unsigned long long heads,
                                         unsigned long long head_dimension,
                                         yvex_backend_operation_facts *facts, yvex_error *err);
+
+/* rocm_schedule.c */
+unsigned int yvex_rocm_schedule_lists(yvex_backend *backend, const yvex_rocm_schedule_key *key,
+                                      const uint16_t **device_rows);
 
 const yvex_backend_transformer_operations *yvex_rocm_transformer_operations(
     const yvex_backend *backend);

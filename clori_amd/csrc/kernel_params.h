@@ -44,6 +44,10 @@ typedef struct {
     /* tile form (yvex_rocm_gqa_f32_tile_*): compute units when workgroups b and b + units share
      * a unit and are to carry equal work (causal launches of at least two tiers of items), else 0 */
     uint32_t pair_units, reserved_tile;
+    /* tile form, scheduled launches: workgroup b runs the items of row b of `lists`, one after
+     * the other; a row is 8 uint16, the count of items, then the items.  NULL: one item per
+     * workgroup */
+    const uint16_t *lists;
 } yvex_rocm_gqa_f32_params;
 
 typedef struct {

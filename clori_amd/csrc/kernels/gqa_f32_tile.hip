@@ -89,18 +89,41 @@ struct GqaTile {
         }
     }
 
+    // Items (one head, one tile of queries) are numbered heaviest first.  A scheduled launch
+    // hands every workgroup a row of items (the count, then the items, 16 bytes: one scalar
+    // load); otherwise the workgroup runs the one item its number stands for.
     __device__ void run() const
     {
+        uint32_t count = 1u;
+        u32x4 row = {0u, 0u, 0u, 0u};
+        if (p.lists != nullptr) {
+            typedef __attribute__((address_space(4))) const u32x4 constant_u32x4;
+            row = *(constant_u32x4 *)(uintptr_t)(p.lists + (uint64_t)blockIdx.x * 8u);
+            count = min(row.x & 0xffffu, 7u);
+        }
+        for (uint32_t j = 1u; j <= count; ++j) {
+            const uint32_t word = j >> 1 == 0u ? row.x : j >> 1 == 1u ? row.y : j >> 1 == 2u ? row.z : row.w;
+            item(p.lists != nullptr ? (word >> ((j & 1u) * 16u)) & 0xffffu : paired_item());
+            // every wave is done with the tiles in LDS before the next item stages its own
+            if (j < count) __syncthreads();
+        }
+    }
+
+    __device__ uint32_t paired_item() const
+    {
+        // Without lists: the hardware gives workgroup b of the first 2 * pair_units to compute
+        // unit b % pair_units, and the kernel is bound by the matrix cores, so a unit's time
+        // follows the key tiles it walks: the second workgroup of a unit takes the second tier of
+        // items in reverse, and the unit that got the heaviest item gets the lightest of them
+        // (equal sums for causal walks; 433 against 459 us for 40 heads x 16 tiles of 2048 tokens).
+        return blockIdx.x >= p.pair_units && blockIdx.x < 2u * p.pair_units
+                   ? 3u * p.pair_units - 1u - blockIdx.x
+                   : blockIdx.x;
+    }
+
+    __device__ void item(const uint64_t id) const
+    {
         const uint64_t tiles_q = (p.query_tokens + kQueries - 1) / kQueries;
-        // Items (one head, one tile of queries) are numbered heaviest first.  The hardware gives
-        // workgroup b of the first 2 * pair_units to compute unit b % pair_units, and the kernel
-        // is bound by the matrix cores, so a unit's time follows the key tiles it walks: the
-        // second workgroup of a unit takes the second tier of items in reverse, and the unit
-        // that got the heaviest item gets the lightest of them (equal sums for causal walks;
-        // 433 against 459 us for 40 heads x 16 tiles of 2048 tokens).
-        const uint64_t id = blockIdx.x >= p.pair_units && blockIdx.x < 2u * p.pair_units
-                                ? 3u * p.pair_units - 1u - blockIdx.x
-                                : blockIdx.x;
         const uint64_t head = id % p.query_heads;
         const uint64_t q_tile = tiles_q - 1 - id / p.query_heads;
         const uint64_t kv_head = head / (p.query_heads / p.kv_heads);
@@ -212,6 +235,7 @@ struct GqaTile {
             __syncthreads();
         }
 
+        // (no early exit above this point: every wave of the workgroup keeps the barriers)
         if (q0 + (uint64_t)column >= p.query_tokens) return;
         sum += xor_lanes(sum, 32);
         if (!(sum > 0.f) || !isfinite(sum) || !isfinite(top)) {

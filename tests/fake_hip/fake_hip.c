@@ -19,7 +19,12 @@ static unsigned long long launches, allocations, frees, loads, unloads;
 static int capturing;                       /* a stream capture is open */
 static unsigned long long captured_launches;
 
+static unsigned int last_grid_x;
+static unsigned char last_params[512];
 unsigned long long fake_hip_launches(void) { return launches; }
+unsigned int fake_hip_last_grid_x(void) { return last_grid_x; }
+/* the bytes kept of the last launch's parameter struct */
+const unsigned char *fake_hip_last_params(void) { return last_params; }
 unsigned long long fake_hip_live_allocations(void) { return allocations - frees; }
 unsigned long long fake_hip_live_modules(void) { return loads - unloads; }
 
@@ -155,9 +160,20 @@ hipError_t hipModuleLaunchKernel(hipFunction_t f, unsigned int gx, unsigned int 
                                  unsigned int shared, hipStream_t stream, void **params,
                                  void **extra)
 {
-    (void)f; (void)gx; (void)gy; (void)gz; (void)bx; (void)by; (void)bz;
-    (void)shared; (void)stream; (void)params; (void)extra;
+    (void)f; (void)gy; (void)gz; (void)bx; (void)by; (void)bz;
+    (void)shared; (void)stream; (void)extra;
     if (env_is("FAKE_HIP_LAUNCH", "fail")) return hipErrorLaunchFailure;
+    /* the last launch's grid width and the head of its one by-value parameter, for tests that
+     * look at what the host handed to a kernel */
+    last_grid_x = gx;
+    {
+        /* FAKE_HIP_PARAM_BYTES: how many bytes of the parameter struct the test wants kept (it
+         * knows the struct it expects; nothing is read unless it asks) */
+        const char *want = getenv("FAKE_HIP_PARAM_BYTES");
+        size_t bytes = want ? (size_t)strtoul(want, NULL, 10) : 0u;
+        if (bytes > sizeof(last_params)) bytes = sizeof(last_params);
+        if (bytes && params && params[0]) memcpy(last_params, params[0], bytes);
+    }
     if (capturing) ++captured_launches;
     else ++launches;
     return hipSuccess;

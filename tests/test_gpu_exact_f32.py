@@ -323,6 +323,42 @@ def test_gqa_matrix_core_kernel_config2_shape(backend):
     assert np.abs(lse - np.log(np.arange(1, t + 1))[:, None]).max() < 1e-5
 
 
+@pytest.mark.parametrize("tq,start,hq,hkv,d", [(1000, 0, 40, 8, 128), (777, 300, 48, 8, 64),
+                                               (2048, 0, 24, 4, 256)])
+def test_gqa_matrix_core_kernel_scheduled_launch_equals_the_first(backend, tq, start, hq, hkv, d):
+    """A causal geometry that repeats is launched from item lists (equal work per compute unit)
+    from its second call on: the same items, so every output bit and every LSE bit equals the
+    first call's, ragged last tiles and a query offset included; sampled heads against the CPU
+    operator."""
+    rng = np.random.default_rng(tq + d)
+    tk = start + tq
+    q = rng.standard_normal((tq, hq, d)).astype(np.float32)
+    k = rng.standard_normal((tk, hkv, d)).astype(np.float32)
+    v = rng.standard_normal((tk, hkv, d)).astype(np.float32)
+    req = backend.attention_requirement(tq, tk, hq, hkv, d, query_start=start)
+    tensors = [f32(backend, "q", q), f32(backend, "k", k), f32(backend, "v", v)]
+    results = []
+    for _ in range(3):
+        out, lse = f32(backend, "out", shape=(tq, hq, d)), f32(backend, "lse", shape=(tq, hq))
+        facts = backend.attention_execute(req, *tensors, out, lse=lse)
+        assert facts.accelerated_matrix_launches == 1
+        results.append((out.read(), lse.read()))
+        out.release()
+        lse.release()
+    for out, lse in results[1:]:
+        assert np.array_equal(out.view(np.uint32), results[0][0].view(np.uint32))
+        assert np.array_equal(lse.view(np.uint32), results[0][1].view(np.uint32))
+    for head in (0, hq // 2 + 1, hq - 1):
+        group = head // (hq // hkv)
+        rc, ref, ref_lse = ORACLE.gqa(q[:, head:head + 1], k[:, group:group + 1], v[:, group:group + 1],
+                                      query_start=start)
+        assert rc == 0
+        assert np.abs(results[2][0][:, head] - ref[:, 0]).max() < 2e-5
+        assert np.abs(results[2][1][:, head] - ref_lse[:, 0]).max() < 2e-5
+    for t in tensors:
+        t.release()
+
+
 # ------------------------------------------------ decode-shaped requests over long contexts ----
 
 @pytest.mark.parametrize("tq,tk,hq,hkv,d,causal", [

@@ -1280,3 +1280,63 @@ def test_elementwise_slots_validate_like_the_reference():
             with pytest.raises(YvexError) as e:
                 call()
             assert e.value.code == B.YVEX_ERR_FORMAT
+
+
+def test_causal_exact_prefill_gets_item_lists_with_equal_work_per_unit(fake_runtime, env):
+    """A causal EXACT_F32 prefill geometry that comes twice in a row is launched as 2 x 256 lists
+    of items (the stand-in runtime reports 256 compute units): every item exactly once, no list
+    longer than a row holds, and every unit (lists u and u + 256) within one item step of the
+    mean number of key tiles; the first launch of a geometry, and launches too small to fill
+    the units twice, keep one item per workgroup."""
+    fake_runtime.fake_hip_last_grid_x.restype = C.c_uint
+    fake_runtime.fake_hip_last_params.restype = C.POINTER(C.c_ubyte)
+    env("FAKE_HIP_PARAM_BYTES", "176")
+    tokens, hq, hkv, d = 2048, 40, 8, 128
+    items = hq * (tokens // 128)
+    with Backend() as b:
+        q = written(b, "q", B.DTYPE_F32, (tokens, hq, d))
+        k, v = written(b, "k", B.DTYPE_F32, (tokens, hkv, d)), written(b, "v", B.DTYPE_F32, (tokens, hkv, d))
+        out = b.tensor("o", B.DTYPE_F32, (tokens, hq, d))
+        req = b.attention_requirement(tokens, tokens, hq, hkv, d, causal=True)
+
+        def launch():
+            b.attention_execute(req, q, k, v, out)
+            raw = bytes(fake_runtime.fake_hip_last_params()[:176])
+            pair_units = int.from_bytes(raw[160:164], "little")
+            lists = int.from_bytes(raw[168:176], "little")
+            return fake_runtime.fake_hip_last_grid_x(), pair_units, lists
+
+        grid, pair_units, lists = launch()
+        assert grid == items and pair_units == 256 and lists == 0     # first time: pairs only
+        grid, pair_units, lists = launch()
+        assert grid == 512 and pair_units == 0 and lists != 0
+        rows = np.ctypeslib.as_array(C.cast(lists, C.POINTER(C.c_uint16)), shape=(512, 8)).copy()
+        counts = rows[:, 0].astype(int)
+        assert counts.max() <= 7
+        seen = np.concatenate([rows[i, 1:1 + counts[i]] for i in range(512)])
+        assert sorted(seen.tolist()) == list(range(items))
+        steps = lambda item: 4 * (16 - item // hq)                     # key tiles of 32 an item walks
+        per_unit = [sum(steps(i) for i in rows[u, 1:1 + counts[u]]) + sum(steps(i) for i in rows[u + 256, 1:1 + counts[u + 256]])
+                    for u in range(256)]
+        mean = sum(per_unit) / 256.0
+        assert max(per_unit) - min(per_unit) <= 8 and max(per_unit) <= mean + 6, (min(per_unit), max(per_unit), mean)
+        for u in range(512):                                            # heaviest first within a list
+            assert list(rows[u, 1:1 + counts[u]]) == sorted(rows[u, 1:1 + counts[u]])
+        assert launch() == (512, 0, lists)                              # kept while the geometry repeats
+        # too few items to fill the units twice are never scheduled (and leave the lists alone)
+        small = b.attention_requirement(1024, 1024, 8, 8, d, causal=True)
+        q2 = written(b, "q2", B.DTYPE_F32, (1024, 8, d))
+        k2, v2 = written(b, "k2", B.DTYPE_F32, (1024, 8, d)), written(b, "v2", B.DTYPE_F32, (1024, 8, d))
+        out2 = b.tensor("o2", B.DTYPE_F32, (1024, 8, d))
+        for _ in range(3):
+            b.attention_execute(small, q2, k2, v2, out2)
+            assert fake_runtime.fake_hip_last_grid_x() == 64
+        assert launch()[0] == 512
+        # another geometry that can be scheduled takes the place of the first, which starts over
+        other = b.attention_requirement(1024, tokens, hq, hkv, d, causal=True, query_start=1024)
+        q3, out3 = written(b, "q3", B.DTYPE_F32, (1024, hq, d)), b.tensor("o3", B.DTYPE_F32, (1024, hq, d))
+        b.attention_execute(other, q3, k, v, out3)
+        assert fake_runtime.fake_hip_last_grid_x() == 8 * hq
+        b.attention_execute(other, q3, k, v, out3)
+        assert fake_runtime.fake_hip_last_grid_x() == 512
+        assert launch()[0] == items

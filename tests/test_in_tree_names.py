@@ -91,7 +91,7 @@ def test_every_vtable_slot_the_arm_fills_exists_in_the_reference_table():
 
 
 IN_TREE_SOURCES = ("rocm_attention.c", "rocm_backend.c", "rocm_capability.c", "rocm_driver.c",
-                   "rocm_elementwise.c", "rocm_virtual.c")
+                   "rocm_elementwise.c", "rocm_schedule.c", "rocm_virtual.c")
 
 
 @pytest.mark.parametrize("source", IN_TREE_SOURCES)
