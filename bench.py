@@ -305,6 +305,61 @@ def workload_exact1(backend, rng, steps, warmup):
                 dtype="f64", launches=int(facts.kernel_launches), kernels=kernels, **timed)
 
 
+def workload_decoder_block(backend, rng, steps, warmup):
+    """One decode step of the reference's decoder attention block, call for call through the
+    reference's own operator slots (src/runtime/decoder.c:1225-1270,
+    src/runtime/stateful_attention.c:183-222): split the query/gate projection, rotate and round
+    Q and K, two asynchronous copies into the [K | V] history, attention under EXACT_F32 over
+    the strided views, round, sigmoid gate.  Ten launches and copies per step on F32
+    activations; what an unchanged caller pays on this backend.  Run by name."""
+    hq, hkv, d, ctx, rotary = 32, 8, 128, 4096, 64
+    width = hkv * d
+    f32 = lambda name, shape, scale=1.0: backend.tensor(  # noqa: E731
+        name, B.DTYPE_F32, shape, (rng.standard_normal(shape, dtype=np.float32) * scale))
+    qg, k_new, v_new = f32("qg", (1, hq, 2, d)), f32("k-new", (1, hkv, d)), f32("v-new", (1, hkv, d))
+    angles = rng.uniform(-3.0, 3.0, (1, rotary))
+    cosine = backend.tensor("cos", B.DTYPE_F32, (1, rotary), np.cos(angles).astype(np.float32))
+    sine = backend.tensor("sin", B.DTYPE_F32, (1, rotary), np.sin(angles).astype(np.float32))
+    history = f32("history", (ctx, 2 * width))
+    q, gate = backend.tensor("q", B.DTYPE_F32, (1, hq * d)), backend.tensor("gate", B.DTYPE_F32, (1, hq * d))
+    mixer, gated = backend.tensor("mixer", B.DTYPE_F32, (1, hq * d)), backend.tensor("gated", B.DTYPE_F32, (1, hq * d))
+    row = (ctx - 1) * 2 * width * 4
+    k_slot = history.view(row, B.DTYPE_F32, (width,))
+    v_slot = history.view(row + width * 4, B.DTYPE_F32, (width,))
+    k_row, v_row = k_new.view(0, B.DTYPE_F32, (width,)), v_new.view(0, B.DTYPE_F32, (width,))
+    span = (ctx - 1) * 2 * width + width
+    k_view, v_view = history.view(0, B.DTYPE_F32, (span,)), history.view(width * 4, B.DTYPE_F32, (span,))
+    req = backend.attention_requirement(1, ctx, hq, hkv, d, causal=True, query_start=ctx - 1,
+                                        k_stride=2 * width, v_stride=2 * width)
+    work = backend.tensor("workspace", B.DTYPE_I8, (backend.attention_workspace_required(req),))
+    backend.workspace_attach(work)
+
+    def run():
+        backend.split_interleaved_two_f32(qg, q, gate, 1, hq, d)
+        backend.rotary_half_f32(q, cosine, sine, 1, hq, d, rotary)
+        backend.bf16_round(q, hq * d)
+        backend.rotary_half_f32(k_new, cosine, sine, 1, hkv, d, rotary)
+        backend.bf16_round(k_new, width)
+        k_slot.copy_from_async(k_row)
+        v_slot.copy_from_async(v_row)
+        facts = backend.attention_execute(req, q, k_view, v_view, mixer)
+        backend.bf16_round(mixer, hq * d)
+        backend.sigmoid_product_bf16(mixer, gate, gated, hq * d)
+        return facts
+    run()
+    kernels = ["yvex_rocm_gqa_f32_split", "yvex_rocm_rotary_half_plain_f32", "yvex_rocm_bf16_round_f32",
+               "yvex_rocm_sigmoid_product_bf16_f32", "yvex_rocm_split_interleaved_two_f32"]
+    timed = time_steps(backend, run, steps, warmup, kernels)
+    backend.workspace_detach()
+    return dict(name="decoder_block",
+                workload="one decode step of the reference's decoder attention block, call for call "
+                         "(split, rotary and rounding of Q and K, two copies into the [K|V] history, "
+                         "EXACT_F32 attention over 4096 cached tokens, rounding, sigmoid gate): 32/8 "
+                         "heads, d=128, f32 activations",
+                bound="hbm", algorithmic_bytes=2 * ctx * hkv * d * 4 + 2 * hq * d * 4, tokens=ctx,
+                dtype="f64", launches=10, kernels=kernels, **timed)
+
+
 def workload_mla5(backend, rng, steps, warmup):
     batch, heads, kd, vd, page, ctx = 16, 128, 576, 512, 64, 8192
     pages_each = ctx // page
@@ -449,10 +504,11 @@ EXTRA_WORKLOADS = {
     "prefill_d64": lambda b, r, s, w: workload_prefill2(b, r, s, w, hq=16, hkv=4, d=64, name="prefill_d64"),
     "paged_d256": lambda b, r, s, w: workload_paged(b, r, s, w, hq=24, hkv=4, d=256, name="paged_d256"),
     "paged_d64": lambda b, r, s, w: workload_paged(b, r, s, w, hq=16, hkv=4, d=64, name="paged_d64"),
+    "decoder_block": workload_decoder_block,
 }
 SEEDS = {"decode1": 1, "prefill2": 2, "paged3": 3, "paged4": 4, "mla5": 5, "append_bf16": 6,
          "append_q8_0": 7, "exact2": 8, "exact1": 9, "history_append": 10, "paged3_p64": 3, "paged4_p64": 4,
-         "prefill_d256": 11, "prefill_d64": 12, "paged_d256": 13, "paged_d64": 14}
+         "prefill_d256": 11, "prefill_d64": 12, "paged_d256": 13, "paged_d64": 14, "decoder_block": 15}
 
 
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
