@@ -16,7 +16,9 @@ By name only (not configurations of the metric): exact2 and exact1 (configuratio
 under the EXACT_F32 contract: fp32 matrix cores, and double-precision split decode),
 append_bf16 / append_q8_0 (the KV page writer), history_append (the token-major writer), paged3_p64 / paged4_p64
 (configurations 3 and 4 with pages of 64 tokens), prefill_d256 / prefill_d64 (causal prefill at head
-dimension 256, 24/4 heads, and 64, 16/4 heads), copy.
+dimension 256, 24/4 heads, and 64, 16/4 heads), paged_d256 / paged_d64 (configuration 3 at those head
+dimensions), decoder_block / decoder_block_fused (one decode step of the reference's decoder attention
+block: call for call through the reference's slots, and through the two fused entry points), copy.
 
 Prints ONE JSON line.  `value` is the headline workload's throughput; every workload
 that ran is listed under "workloads" with its own roofline figures.  Timing uses HIP
@@ -360,6 +362,49 @@ def workload_decoder_block(backend, rng, steps, warmup):
                 dtype="f64", launches=10, kernels=kernels, **timed)
 
 
+def workload_decoder_block_fused(backend, rng, steps, warmup):
+    """The decode step of workload decoder_block for a caller that keeps bf16 activations and
+    uses the two fused entry points: one launch rotates Q where it lies and writes the rotated
+    key row and the value row into the [K | V] history, one launch is attention over the
+    strided views with the sigmoid gate in its epilogue.  Two launches per step.  Run by name."""
+    hq, hkv, d, ctx, rotary = 32, 8, 128, 4096, 64
+    width = hkv * d
+    bf16 = lambda name, shape: backend.tensor(  # noqa: E731
+        name, B.DTYPE_BF16, shape, random_bf16(rng, int(np.prod(shape))))
+    q, gate = bf16("q", (1, hq, d)), bf16("gate", (1, hq, d))
+    k_new, v_new = bf16("k-new", (1, hkv, d)), bf16("v-new", (1, hkv, d))
+    angles = rng.uniform(-3.0, 3.0, (1, rotary))
+    cosine = backend.tensor("cos", B.DTYPE_F32, (1, rotary), np.cos(angles).astype(np.float32))
+    sine = backend.tensor("sin", B.DTYPE_F32, (1, rotary), np.sin(angles).astype(np.float32))
+    history = bf16("history", (ctx, 2 * width))
+    gated = backend.tensor("gated", B.DTYPE_BF16, (1, hq, d))
+    span = (ctx - 1) * 2 * width + width
+    k_view, v_view = history.view(0, B.DTYPE_BF16, (span,)), history.view(width * 2, B.DTYPE_BF16, (span,))
+    req = backend.attention_requirement(1, ctx, hq, hkv, d, causal=True, query_start=ctx - 1,
+                                        dtype=B.DTYPE_BF16, contract=B.NUMERIC_BF16_F32_ACCUMULATE,
+                                        k_stride=2 * width, v_stride=2 * width)
+    work = backend.tensor("workspace", B.DTYPE_I8, (backend.attention_workspace_required(req),))
+    backend.workspace_attach(work)
+
+    def run():
+        backend.history_append_execute(k_new, v_new, k_view, v_view, ctx - 1, hkv, head_dimension=d,
+                                       cosine=cosine, sine=sine, rotary_dimension=rotary,
+                                       key_token_stride=2 * width, value_token_stride=2 * width,
+                                       query=q, query_heads=hq)
+        return backend.attention_execute(req, q, k_view, v_view, gated, gate=gate)
+    facts = run()
+    kernels = ["yvex_rocm_decode_rows_bf16_team", "yvex_rocm_history_append_bf16"]
+    timed = time_steps(backend, run, steps, warmup, kernels)
+    backend.workspace_detach()
+    return dict(name="decoder_block_fused",
+                workload="one decode step of the decoder attention block through the fused entry "
+                         "points (rotary of Q and K and both history rows in one launch, attention "
+                         "over 4096 cached tokens with the sigmoid gate in its epilogue): 32/8 heads, "
+                         "d=128, bf16 activations",
+                bound="hbm", algorithmic_bytes=2 * ctx * hkv * d * 2 + 3 * hq * d * 2, tokens=ctx,
+                launches=1 + int(facts.kernel_launches), kernels=kernels, **timed)
+
+
 def workload_mla5(backend, rng, steps, warmup):
     batch, heads, kd, vd, page, ctx = 16, 128, 576, 512, 64, 8192
     pages_each = ctx // page
@@ -505,10 +550,12 @@ EXTRA_WORKLOADS = {
     "paged_d256": lambda b, r, s, w: workload_paged(b, r, s, w, hq=24, hkv=4, d=256, name="paged_d256"),
     "paged_d64": lambda b, r, s, w: workload_paged(b, r, s, w, hq=16, hkv=4, d=64, name="paged_d64"),
     "decoder_block": workload_decoder_block,
+    "decoder_block_fused": workload_decoder_block_fused,
 }
 SEEDS = {"decode1": 1, "prefill2": 2, "paged3": 3, "paged4": 4, "mla5": 5, "append_bf16": 6,
          "append_q8_0": 7, "exact2": 8, "exact1": 9, "history_append": 10, "paged3_p64": 3, "paged4_p64": 4,
-         "prefill_d256": 11, "prefill_d64": 12, "paged_d256": 13, "paged_d64": 14, "decoder_block": 15}
+         "prefill_d256": 11, "prefill_d64": 12, "paged_d256": 13, "paged_d64": 14, "decoder_block": 15,
+         "decoder_block_fused": 15}
 
 
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")

@@ -524,9 +524,10 @@ class Backend:
     def history_append_execute(self, key, value, key_history, value_history, first_row, kv_heads,
                                head_dimension=128, cosine=None, sine=None, rotary_dimension=0,
                                key_token_stride=0, value_token_stride=0,
-                               rotary_mode=B.ROTARY_BF16_STAGED):
+                               rotary_mode=B.ROTARY_BF16_STAGED, query=None, query_heads=0):
         """Writes the new rows (keys rotated) into rows first_row.. of the token-major K and V
-        history views; all tensor arguments are device tensors."""
+        history views; all tensor arguments are device tensors.  With query and query_heads
+        the same launch rotates the [tokens][query_heads][d] query tensor where it lies."""
         ops = self.rocm_attention_operations()
         if ops is None:
             raise YvexError(B.YVEX_ERR_UNSUPPORTED, "rocm_attention_operations", "not published")
@@ -536,10 +537,11 @@ class Backend:
         r.rotary_dimension = rotary_dimension
         r.key_token_stride, r.value_token_stride = key_token_stride, value_token_stride
         r.rotary_mode = rotary_mode
+        r.query_heads = query_heads
         request = B.HistoryAppendRequest(r, key.handle, value.handle,
                                          cosine.handle if cosine else None,
                                          sine.handle if sine else None, key_history.handle,
-                                         value_history.handle)
+                                         value_history.handle, query.handle if query else None)
         facts, err = B.OperationFacts(), B.Error()
         _check(ops.history_append_execute(self.handle, C.byref(request), C.byref(facts),
                                           C.byref(err)), err)

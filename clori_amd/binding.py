@@ -250,13 +250,13 @@ PAGED_EXECUTE_FUSED_FN = C.CFUNCTYPE(C.c_int, C.c_void_p, C.POINTER(PagedDecodeR
 class HistoryAppendRequirement(C.Structure):
     _fields_ = [(n, ull) for n in ("tokens", "first_row", "key_value_heads", "head_dimension",
                                    "rotary_dimension", "key_token_stride", "value_token_stride")] + [
-        ("rotary_mode", C.c_int)]
+        ("rotary_mode", C.c_int), ("query_heads", ull)]
 
 
 class HistoryAppendRequest(C.Structure):
     _fields_ = [("requirement", HistoryAppendRequirement), ("key", TensorP), ("value", TensorP),
                 ("cosine", TensorP), ("sine", TensorP), ("key_history", TensorP),
-                ("value_history", TensorP)]
+                ("value_history", TensorP), ("query", TensorP)]
 
 
 HISTORY_APPEND_FN = C.CFUNCTYPE(C.c_int, C.c_void_p, C.POINTER(HistoryAppendRequest), FactsP, ErrorP)

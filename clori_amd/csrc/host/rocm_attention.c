@@ -1420,12 +1420,16 @@ static int rocm_history_append_execute(yvex_backend *backend,
     yvex_rocm_history_append_params hp;
     yvex_dtype dtype;
     unsigned long long width, k_stride, v_stride, rows, new_elements, k_elements, v_elements, pieces;
+    unsigned long long query_elements = 0ull;
     unsigned long long piece; /* elements in 16 bytes */
     int rc;
     if (!request || !request->key || !request->value || !request->key_history ||
         !request->value_history || !facts)
         return refuse(err, YVEX_ERR_INVALID_ARG, where,
                       "complete history-append tensors and result facts are required");
+    if ((request->requirement.query_heads != 0ull) != (request->query != NULL))
+        return refuse(err, YVEX_ERR_INVALID_ARG, where,
+                      "a query tensor and its head count are given together or not at all");
     rc = backend_dispatch_admit(backend, where, err);
     if (rc != YVEX_OK) return rc;
     r = &request->requirement;
@@ -1447,7 +1451,7 @@ static int rocm_history_append_execute(yvex_backend *backend,
     if (r->head_dimension % piece || r->head_dimension > 256ull || (k_stride | v_stride) % piece ||
         (r->rotary_mode != YVEX_ROCM_ROTARY_BF16_STAGED && r->rotary_mode != YVEX_ROCM_ROTARY_F32_ROUNDED) ||
         r->rotary_dimension > r->head_dimension || r->rotary_dimension % (2ull * piece) ||
-        r->tokens > 0x7fffffffull || r->key_value_heads > 65535ull)
+        r->tokens > 0x7fffffffull || r->key_value_heads > 65535ull || r->query_heads > 65535ull)
         return refuse(err, YVEX_ERR_UNSUPPORTED, where,
                       "ROCm history append requires a head dimension (at most 256) and token strides "
                       "that are multiples of 16 bytes and rotary halves that are too");
@@ -1457,12 +1461,15 @@ static int rocm_history_append_execute(yvex_backend *backend,
         !yvex_core_u64_add(k_elements, width, &k_elements) ||
         !yvex_core_u64_mul(rows - 1ull, v_stride, &v_elements) ||
         !yvex_core_u64_add(v_elements, width, &v_elements) ||
-        !yvex_core_u64_mul(r->tokens * r->key_value_heads, r->head_dimension / piece, &pieces) ||
+        !yvex_core_u64_mul(r->tokens * r->query_heads, r->head_dimension, &query_elements) ||
+        !yvex_core_u64_mul(r->tokens * (r->key_value_heads + r->query_heads),
+                           r->head_dimension / piece, &pieces) ||
         (pieces + 255ull) / 256ull > 0x7fffffffull)
         return refuse(err, YVEX_ERR_BOUNDS, where, "history-append geometry exceeds admitted range");
     /* a history may be fresh or hold earlier tokens: written state is not required of it */
     if (!view_ok(backend, request->key, dtype, new_elements, 1) ||
         !view_ok(backend, request->value, dtype, new_elements, 1) ||
+        (request->query && !view_ok(backend, request->query, dtype, query_elements, 1)) ||
         (r->rotary_dimension &&
          (!view_ok(backend, request->cosine, YVEX_DTYPE_F32, r->tokens * r->rotary_dimension, 1) ||
           !view_ok(backend, request->sine, YVEX_DTYPE_F32, r->tokens * r->rotary_dimension, 1))) ||
@@ -1472,9 +1479,23 @@ static int rocm_history_append_execute(yvex_backend *backend,
                             "new rows, tables and history views must be tensors of this backend "
                             "with the declared geometry and one element type");
     if (((uintptr_t)request->key->data | (uintptr_t)request->value->data |
-         (uintptr_t)request->key_history->data | (uintptr_t)request->value_history->data) & 15u)
+         (uintptr_t)request->key_history->data | (uintptr_t)request->value_history->data |
+         (uintptr_t)(request->query ? request->query->data : NULL)) & 15u)
         return refuse(err, YVEX_ERR_UNSUPPORTED, where,
                       "ROCm history append requires 16-byte aligned rows");
+    if (request->query) {
+        /* rotated where it lies by threads of the launch that reads and writes the others */
+        const yvex_device_tensor *others[4] = {request->key, request->value, request->key_history,
+                                               request->value_history};
+        uintptr_t lo = (uintptr_t)request->query->data, hi = lo + request->query->bytes;
+        size_t i;
+        for (i = 0u; i < 4u; ++i) {
+            uintptr_t at = (uintptr_t)others[i]->data;
+            if (at < hi && lo < at + others[i]->bytes)
+                return refuse(err, YVEX_ERR_INVALID_ARG, where,
+                              "the query tensor overlaps another tensor of the request");
+        }
+    }
     memset(&hp, 0, sizeof(hp));
     hp.key = request->key->data;
     hp.value = request->value->data;
@@ -1491,6 +1512,8 @@ static int rocm_history_append_execute(yvex_backend *backend,
     hp.head_dim = (uint32_t)r->head_dimension;
     hp.rotary_dim = (uint32_t)r->rotary_dimension;
     hp.rotary_mode = (uint32_t)r->rotary_mode;
+    hp.query_heads = (uint32_t)r->query_heads;
+    hp.query = request->query ? request->query->data : NULL;
     variant = dtype == YVEX_DTYPE_BF16 ? YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_BF16
                                        : YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_F32;
     backend_workspace_reset(backend);

@@ -215,7 +215,8 @@ typedef struct {
 
 /* Token-major history writer: new key/value rows -> rows [first_row, first_row + tokens) of
  * the strided K and V histories the GQA kernels read, rotary on the keys.  One thread per
- * 16-byte piece of a row (8 bf16 or 4 F32 lanes); grid = ceil(pieces / 256), block = 256.
+ * 16-byte piece of a row (8 bf16 or 4 F32 lanes), the pieces of the optional query tensor
+ * behind those of the keys and values; grid = ceil(pieces / 256), block = 256.
  * The bf16 and the F32 kernel take the same block; pointers are to the element type. */
 typedef struct {
     const void *key, *value;          /* [tokens][kv_heads][head_dim] */
@@ -225,6 +226,8 @@ typedef struct {
     uint64_t first_row, key_token_stride, value_token_stride; /* strides in elements */
     uint32_t tokens, kv_heads, head_dim, rotary_dim;
     uint32_t rotary_mode;             /* as in yvex_rocm_kv_append_params */
+    uint32_t query_heads;             /* 0 without a query tensor */
+    void *query;                      /* [tokens][query_heads][head_dim], rotated where it lies */
 } yvex_rocm_history_append_params;
 
 #endif /* YVEX_ROCM_KERNEL_PARAMS_H */

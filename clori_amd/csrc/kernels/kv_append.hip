@@ -451,26 +451,34 @@ yvex_rocm_kv_append_q8_0(const yvex_rocm_kv_append_params p)
 // (src/runtime/decoder.c:1236-1242).  Here one launch does both: thread i owns the 16-byte
 // piece (token, kv head, dims 8 * c8 .. 8 * c8 + 7) of the value row and of the key row, with
 // the rotary roles and modes of the page writer (a lower-half piece produces its upper-half
-// partner).
+// partner).  With a query tensor, threads behind the key/value pieces own the 16-byte pieces
+// (token, query head) of it and rotate them where they lie, as the decoder rotates the
+// queries in a pass of their own before attention (src/runtime/decoder.c:1235-1238): every
+// location of the tensor is read and written by one thread only.
 extern "C" __global__ void __launch_bounds__(256)
 yvex_rocm_history_append_bf16(const yvex_rocm_history_append_params p)
 {
     const uint32_t pieces = p.head_dim / 8u, pairs = p.rotary_dim / 16u;
     const uint64_t id = (uint64_t)blockIdx.x * 256u + threadIdx.x;
     const uint64_t total = (uint64_t)p.tokens * p.kv_heads * pieces;
-    if (id >= total) return;
-    const uint32_t c8 = (uint32_t)(id % pieces), head = (uint32_t)(id / pieces % p.kv_heads);
-    const uint32_t token = (uint32_t)(id / pieces / p.kv_heads);
-    const uint64_t in = ((uint64_t)token * p.kv_heads + head) * p.head_dim + c8 * 8u;
+    if (id >= total + (uint64_t)p.tokens * p.query_heads * pieces) return;
+    const bool is_query = id >= total;
+    const uint64_t local = is_query ? id - total : id;
+    const uint32_t heads = is_query ? p.query_heads : p.kv_heads;
+    const uint32_t c8 = (uint32_t)(local % pieces), head = (uint32_t)(local / pieces % heads);
+    const uint32_t token = (uint32_t)(local / pieces / heads);
+    const uint64_t in = ((uint64_t)token * heads + head) * p.head_dim + c8 * 8u;
     const uint64_t row = p.first_row + token;
-    const uint16_t *key = (const uint16_t *)p.key, *value = (const uint16_t *)p.value;
-    uint16_t *kdst = (uint16_t *)p.key_history + row * p.key_token_stride + (uint64_t)head * p.head_dim + c8 * 8u;
-    uint16_t *vdst = (uint16_t *)p.value_history + row * p.value_token_stride + (uint64_t)head * p.head_dim + c8 * 8u;
+    const uint16_t *key = is_query ? (const uint16_t *)p.query : (const uint16_t *)p.key;
+    uint16_t *kdst = is_query ? (uint16_t *)p.query + in
+                              : (uint16_t *)p.key_history + row * p.key_token_stride +
+                                    (uint64_t)head * p.head_dim + c8 * 8u;
     KeyChunk k;
     k.t = 0u;
     k.c8 = c8;
     k.role = c8 < pairs ? kLower : c8 < 2u * pairs ? kUpper : kPlain;
-    const u32x4 v = load_b128(value + in);
+    u32x4 v = {0u, 0u, 0u, 0u};
+    if (!is_query) v = load_b128((const uint16_t *)p.value + in);
     if (k.role != kUpper) k.own = load_b128(key + in);
     if (k.role == kLower) {
         const uint64_t at = (uint64_t)token * p.rotary_dim + c8 * 8u;
@@ -482,7 +490,9 @@ yvex_rocm_history_append_bf16(const yvex_rocm_history_append_params p)
     }
     u32x4 lower, upper;
     bool ok = key_finish(k, lower, upper, p.rotary_mode != 0u) && finite_bits(v);
-    *reinterpret_cast<u32x4 *>(vdst) = v;
+    if (!is_query)
+        *reinterpret_cast<u32x4 *>((uint16_t *)p.value_history + row * p.value_token_stride +
+                                   (uint64_t)head * p.head_dim + c8 * 8u) = v;
     if (k.role != kUpper) *reinterpret_cast<u32x4 *>(kdst) = lower;
     if (k.role == kLower) *reinterpret_cast<u32x4 *>(kdst + p.rotary_dim / 2u) = upper;
     if (!ok) flag(p.status, YVEX_ROCM_DEVICE_NUMERIC);
@@ -521,17 +531,22 @@ yvex_rocm_history_append_f32(const yvex_rocm_history_append_params p)
     const uint32_t pieces = p.head_dim / 4u, pairs = p.rotary_dim / 8u;
     const uint64_t id = (uint64_t)blockIdx.x * 256u + threadIdx.x;
     const uint64_t total = (uint64_t)p.tokens * p.kv_heads * pieces;
-    if (id >= total) return;
-    const uint32_t c4 = (uint32_t)(id % pieces), head = (uint32_t)(id / pieces % p.kv_heads);
-    const uint32_t token = (uint32_t)(id / pieces / p.kv_heads);
-    const uint64_t in = ((uint64_t)token * p.kv_heads + head) * p.head_dim + c4 * 4u;
+    if (id >= total + (uint64_t)p.tokens * p.query_heads * pieces) return;
+    // pieces behind the key/value ones belong to the query tensor, rotated where it lies
+    const bool is_query = id >= total;
+    const uint64_t local = is_query ? id - total : id;
+    const uint32_t heads = is_query ? p.query_heads : p.kv_heads;
+    const uint32_t c4 = (uint32_t)(local % pieces), head = (uint32_t)(local / pieces % heads);
+    const uint32_t token = (uint32_t)(local / pieces / heads);
+    const uint64_t in = ((uint64_t)token * heads + head) * p.head_dim + c4 * 4u;
     const uint64_t row = p.first_row + token;
-    const float *key = (const float *)p.key, *value = (const float *)p.value;
-    float *kdst = (float *)p.key_history + row * p.key_token_stride + (uint64_t)head * p.head_dim + c4 * 4u;
-    float *vdst = (float *)p.value_history + row * p.value_token_stride + (uint64_t)head * p.head_dim + c4 * 4u;
+    const float *key = is_query ? (const float *)p.query : (const float *)p.key;
+    float *kdst = is_query ? (float *)p.query + in
+                           : (float *)p.key_history + row * p.key_token_stride +
+                                 (uint64_t)head * p.head_dim + c4 * 4u;
     const int role = c4 < pairs ? kLower : c4 < 2u * pairs ? kUpper : kPlain;
-    const u32x4 v = load_b128(value + in);
-    u32x4 own = {0u, 0u, 0u, 0u}, other = own, cs = own, sn = own;
+    u32x4 own = {0u, 0u, 0u, 0u}, other = own, cs = own, sn = own, v = own;
+    if (!is_query) v = load_b128((const float *)p.value + in);
     if (role != kUpper) own = load_b128(key + in);
     if (role == kLower) {
         const uint64_t at = (uint64_t)token * p.rotary_dim + c4 * 4u;
@@ -540,7 +555,9 @@ yvex_rocm_history_append_f32(const yvex_rocm_history_append_params p)
         sn = load_b128(p.sine + at);
     }
     bool ok = finite_floats(v);
-    *reinterpret_cast<u32x4 *>(vdst) = v;
+    if (!is_query)
+        *reinterpret_cast<u32x4 *>((float *)p.value_history + row * p.value_token_stride +
+                                   (uint64_t)head * p.head_dim + c4 * 4u) = v;
     if (role == kPlain) {
         ok &= finite_floats(own);
         if (p.rotary_mode != 0u) {

@@ -724,13 +724,17 @@ typedef struct yvex_rocm_kv_append_request {
  * products as they are, as in yvex_rotary_half_f32, and the results are bf16 values stored
  * as F32).  Over a reserved address range the rows must be committed first.  Rows, strides
  * and rotary halves must be multiples of 16 bytes; non-finite inputs, table entries or
- * results are YVEX_ERR_FORMAT.
+ * results are YVEX_ERR_FORMAT.  With query_heads and a query tensor the same launch also
+ * rotates the new tokens' queries where they lie, with the arithmetic and mode of the keys
+ * (the decoder's pass over the queries, src/runtime/decoder.c:1235-1238), so that attention
+ * is the next call; the query tensor must not overlap any other tensor of the request.
  */
 typedef struct yvex_rocm_history_append_requirement {
     unsigned long long tokens, first_row;
     unsigned long long key_value_heads, head_dimension, rotary_dimension;
     unsigned long long key_token_stride, value_token_stride;
     yvex_rocm_rotary_mode rotary_mode; /* F32_ROUNDED also rounds the key lanes behind the rotary ones */
+    unsigned long long query_heads;    /* 0 without a query tensor */
 } yvex_rocm_history_append_requirement;
 
 typedef struct yvex_rocm_history_append_request {
@@ -738,6 +742,7 @@ typedef struct yvex_rocm_history_append_request {
     const yvex_device_tensor *key, *value;   /* BF16 or F32 [tokens][kv_heads][d] */
     const yvex_device_tensor *cosine, *sine; /* F32 [tokens][rotary_dimension], or NULL without rotary */
     yvex_device_tensor *key_history, *value_history; /* the element type of key and value */
+    yvex_device_tensor *query; /* [tokens][query_heads][d] of that type, or NULL */
 } yvex_rocm_history_append_request;
 
 /*

@@ -466,3 +466,67 @@ def test_session_backend_on_the_device_copies_between_streams(backend):
         received.release()
     finally:
         session.close()
+
+
+@pytest.mark.parametrize("f32", [False, True], ids=["bf16", "f32"])
+@pytest.mark.parametrize("mode", [B.ROTARY_BF16_STAGED, B.ROTARY_F32_ROUNDED], ids=["staged", "decoder-order"])
+@pytest.mark.parametrize("tokens,hq,hkv,d,rotary", [
+    (1, 40, 8, 128, 64), (1, 16, 2, 256, 64), (37, 5, 1, 64, 64), (300, 6, 2, 128, 0), (9, 3, 3, 96, 32)])
+def test_history_append_rotates_the_queries_in_the_same_launch(backend, f32, mode, tokens, hq, hkv, d, rotary):
+    """With a query tensor the launch also does the decoder's rotary pass over the queries
+    (src/runtime/decoder.c:1235-1238) where they lie: the queries equal the restatement's
+    rotation for the element type and mode, the histories equal those of a call without."""
+    rng = np.random.default_rng(tokens * 31 + hq * 7 + d + rotary + int(f32) + 2 * mode)
+    if d % (8 if not f32 else 4) or (not f32 and rotary % 16):
+        pytest.skip("not a geometry of this element type")
+    first, width = 11, hkv * d
+    used = first + tokens
+    cosine, sine = tables(rng, tokens, rotary)
+    cs, sn = cosine[:, :rotary], sine[:, :rotary]
+    if f32:
+        dtype, elem = B.DTYPE_F32, 4
+        q, k_new, v_new = (rng.standard_normal((tokens, h, d)).astype(np.float32) for h in (hq, hkv, hkv))
+        before = rng.standard_normal((used, 2 * width)).astype(np.float32)
+        rotate = ORACLE.rotary_half_f32 if mode == B.ROTARY_BF16_STAGED else ORACLE.rotary_half_f32_rounded
+        if rotary:
+            want_q = rotate(q, cs, sn, rotary)
+        else:  # the decoder's order still rounds every lane once
+            want_q = ORACLE.bf16_decode(ORACLE.bf16_encode(q)) if mode == B.ROTARY_F32_ROUNDED else q
+    else:
+        dtype, elem = B.DTYPE_BF16, 2
+        q, k_new, v_new = (bf16_normal(rng, (tokens, h, d)) for h in (hq, hkv, hkv))
+        before = bf16_normal(rng, (used, 2 * width))
+        if not rotary:
+            want_q = q
+        elif mode == B.ROTARY_BF16_STAGED:
+            want_q = ORACLE.rotary_half_bf16(q, cs, sn, rotary)
+        else:
+            want_q = ORACLE.bf16_encode(ORACLE.rotary_half_f32_rounded(ORACLE.bf16_decode(q), cs, sn, rotary))
+    bits = np.uint32 if f32 else np.uint16
+    held = [backend.tensor("k-new", dtype, k_new.shape, k_new), backend.tensor("v-new", dtype, v_new.shape, v_new),
+            backend.tensor("q", dtype, q.shape, q), backend.tensor("with", dtype, before.shape, before),
+            backend.tensor("without", dtype, before.shape, before)]
+    tc = ts = None
+    if rotary:
+        tc, ts = backend.tensor("cos", B.DTYPE_F32, cs.shape, cs), backend.tensor("sin", B.DTYPE_F32, sn.shape, sn)
+        held += [tc, ts]
+    count = (used - 1) * 2 * width + width
+    common = dict(head_dimension=d, cosine=tc, sine=ts, rotary_dimension=rotary, key_token_stride=2 * width,
+                  value_token_stride=2 * width, rotary_mode=mode)
+    views = [(s.view(0, dtype, (count,)), s.view(elem * width, dtype, (count,))) for s in (held[3], held[4])]
+    facts = backend.history_append_execute(held[0], held[1], *views[0], first, hkv, query=held[2],
+                                           query_heads=hq, **common)
+    assert facts.kernel_launches == 1
+    backend.history_append_execute(held[0], held[1], *views[1], first, hkv, **common)
+    assert np.array_equal(held[2].read().view(bits), np.ascontiguousarray(want_q).view(bits))
+    assert np.array_equal(held[3].read().view(bits), held[4].read().view(bits))
+    assert not np.array_equal(held[3].read().view(bits), before.view(bits))
+    # the new rows are untouched, and a query that overlaps them or comes without a head count is refused
+    assert np.array_equal(held[0].read().view(bits), k_new.view(bits))
+    for bad in (dict(query=held[2], query_heads=0), dict(query=None, query_heads=hq),
+                dict(query=held[0], query_heads=hkv)):
+        with pytest.raises(YvexError) as e:
+            backend.history_append_execute(held[0], held[1], *views[0], first, hkv, **bad, **common)
+        assert e.value.code == B.YVEX_ERR_INVALID_ARG
+    for t in held:
+        t.release()

@@ -860,7 +860,7 @@ def test_kv_append_admission():
         assert e.value.code == B.YVEX_ERR_FORMAT
 
 
-def test_history_append_admission():
+def test_history_append_admission(fake_runtime):
     """Refusal order of the token-major history writer: arguments, geometry, what the kernel
     does not cover, then tensor views (uncommitted rows of a reserved range included)."""
     with Backend() as b:
@@ -926,6 +926,24 @@ def test_history_append_admission():
         assert e.value.code == B.YVEX_ERR_STATE and "not committed" in e.value.message
         reserved.commit(0, (first + tokens) * row_bytes)
         assert b.history_append_execute(key, value, rk, rv, first, hkv, **strides).kernel_launches == 1
+        # the optional query tensor: its pieces join the launch; it comes with its head count, has
+        # the element type and geometry of the new rows and overlaps nothing else
+        hq = 12
+        query = written(b, "q", B.DTYPE_BF16, (tokens, hq, d))
+        assert b.history_append_execute(*args, query=query, query_heads=hq, **strides).kernel_launches == 1
+        fake_runtime.fake_hip_last_grid_x.restype = C.c_uint
+        assert fake_runtime.fake_hip_last_grid_x() == (tokens * (hkv + hq) * (d // 8) + 255) // 256
+        for kwargs, code in [(dict(query=query), B.YVEX_ERR_INVALID_ARG),
+                             (dict(query_heads=hq), B.YVEX_ERR_INVALID_ARG),
+                             (dict(query=query, query_heads=hq + 1), B.YVEX_ERR_FORMAT),
+                             (dict(query=query, query_heads=65536), B.YVEX_ERR_UNSUPPORTED),
+                             (dict(query=key32, query_heads=hkv), B.YVEX_ERR_FORMAT),
+                             (dict(query=key, query_heads=hkv), B.YVEX_ERR_INVALID_ARG),
+                             (dict(query=b.tensor("q2", B.DTYPE_BF16, (tokens, hq, d)), query_heads=hq),
+                              B.YVEX_ERR_FORMAT)]:
+            with pytest.raises(YvexError) as e:
+                b.history_append_execute(*args, **kwargs, **strides)
+            assert e.value.code == code, kwargs
 
 
 def test_fused_gate_admission():
