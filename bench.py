@@ -16,8 +16,8 @@ By name only (not configurations of the metric): exact2 and exact1 (configuratio
 under the EXACT_F32 contract: fp32 matrix cores, and double-precision split decode),
 append_bf16 / append_q8_0 (the KV page writer), history_append (the token-major writer), paged3_p64 / paged4_p64
 (configurations 3 and 4 with pages of 64 tokens), prefill_d256 / prefill_d64 (causal prefill at head
-dimension 256, 24/4 heads, and 64, 16/4 heads), paged_d256 / paged_d64 (configuration 3 at those head
-dimensions), decoder_block / decoder_block_fused (one decode step of the reference's decoder attention
+dimension 256, 24/4 heads, and 64, 16/4 heads), paged_d256 / paged_d64 and decode_d256 / decode_d64 (configurations 3 and 1
+at those head dimensions), decoder_block / decoder_block_fused (one decode step of the reference's decoder attention
 block: call for call through the reference's slots, and through the two fused entry points), copy.
 
 Prints ONE JSON line.  `value` is the headline workload's throughput; every workload
@@ -213,8 +213,8 @@ def workload_paged(backend, rng, steps, warmup, q8=False, page=16, hq=32, hkv=8,
                 launches=int(facts.kernel_launches), kernels=kernels, **timed)
 
 
-def workload_decode1(backend, rng, steps, warmup):
-    hq, hkv, d, ctx = 32, 8, 128, 4096
+def workload_decode1(backend, rng, steps, warmup, hq=32, hkv=8, d=128, name="decode1"):
+    ctx = 4096
     q = backend.tensor("q", B.DTYPE_BF16, (1, hq, d), random_bf16(rng, hq * d))
     k = backend.tensor("k", B.DTYPE_BF16, (ctx, hkv, d), random_bf16(rng, ctx * hkv * d))
     v = backend.tensor("v", B.DTYPE_BF16, (ctx, hkv, d), random_bf16(rng, ctx * hkv * d))
@@ -227,14 +227,14 @@ def workload_decode1(backend, rng, steps, warmup):
     backend.workspace_attach(work)
     run = lambda: backend.attention_execute(req, q, k, v, out, lse=lse)  # noqa: E731
     facts = run()
-    # one launch: teams of eight waves per stretch of the history, merged through LDS and then
-    # between the teams by the one that arrives last
-    kernels = ["yvex_rocm_decode_rows_bf16_team"]
+    # one launch: teams of eight waves (four at head dimension 256) per stretch of the history,
+    # merged through LDS and then between the teams by the one that arrives last
+    kernels = ["yvex_rocm_decode_rows_bf16_team" + ("" if d == 128 else "_%d" % d)]
     timed = time_steps(backend, run, steps, warmup, kernels)
     backend.workspace_detach()
     algo = 2 * ctx * hkv * d * 2 + 2 * hq * d * 2 + hq * 4
-    return dict(name="decode1",
-                workload="GQA decode: batch 1, 32/8 heads, d=128, context 4096, contiguous bf16 KV",
+    return dict(name=name,
+                workload="GQA decode: batch 1, %d/%d heads, d=%d, context 4096, contiguous bf16 KV" % (hq, hkv, d),
                 bound="hbm", algorithmic_bytes=algo, tokens=ctx,
                 launches=int(facts.kernel_launches), kernels=kernels, **timed)
 
@@ -547,6 +547,8 @@ EXTRA_WORKLOADS = {
     # the reference's own Qwen attention geometry (24/4 heads, head dimension 256) and a narrow one
     "prefill_d256": lambda b, r, s, w: workload_prefill2(b, r, s, w, hq=24, hkv=4, d=256, name="prefill_d256"),
     "prefill_d64": lambda b, r, s, w: workload_prefill2(b, r, s, w, hq=16, hkv=4, d=64, name="prefill_d64"),
+    "decode_d256": lambda b, r, s, w: workload_decode1(b, r, s, w, hq=24, hkv=4, d=256, name="decode_d256"),
+    "decode_d64": lambda b, r, s, w: workload_decode1(b, r, s, w, hq=16, hkv=4, d=64, name="decode_d64"),
     "paged_d256": lambda b, r, s, w: workload_paged(b, r, s, w, hq=24, hkv=4, d=256, name="paged_d256"),
     "paged_d64": lambda b, r, s, w: workload_paged(b, r, s, w, hq=16, hkv=4, d=64, name="paged_d64"),
     "decoder_block": workload_decoder_block,
@@ -555,7 +557,7 @@ EXTRA_WORKLOADS = {
 SEEDS = {"decode1": 1, "prefill2": 2, "paged3": 3, "paged4": 4, "mla5": 5, "append_bf16": 6,
          "append_q8_0": 7, "exact2": 8, "exact1": 9, "history_append": 10, "paged3_p64": 3, "paged4_p64": 4,
          "prefill_d256": 11, "prefill_d64": 12, "paged_d256": 13, "paged_d64": 14, "decoder_block": 15,
-         "decoder_block_fused": 15}
+         "decoder_block_fused": 15, "decode_d256": 16, "decode_d64": 17}
 
 
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")

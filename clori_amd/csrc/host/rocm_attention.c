@@ -28,6 +28,7 @@ enum {
     ROCM_DECODE_MIN_TILES = 8, /* 8 and 16 measure alike on a 4096-token context; 4 and 32 are a third slower */
     ROCM_TEAM_WAVES = 8,       /* waves of a decode team (one workgroup) */
     ROCM_TEAM_TILES = 2,       /* tiles a wave of a team is given when the history is short enough (context 4096: 10.3 us; 1: 11.6, 4: 11.9, 8: 15.9) */
+    ROCM_TEAM_TILES_WIDE = 4,  /* the same at head dimension 256, teams of four waves (24/4 heads, context 4096: 16.0 us; 2: 18.3, 8: 19.7) */
     ROCM_TEAMS_MAX = 32,       /* teams per (session, kv head): two load trips of the last team's merge */
     ROCM_TEAM_GROUP_MAX = 8,   /* query heads per kv head a team's LDS holds */
     ROCM_PREFILL_ROWS = YVEX_ROCM_PREFILL_ROWS, /* query rows per prefill workgroup */
@@ -135,17 +136,35 @@ static int decode_workspace_bytes(unsigned long long slots, unsigned long long h
  * one is bound by launch latency and merges inside the decode kernel (arrival counters). */
 static int decode_merges_in_kernel(unsigned int waves) { return waves < ROCM_DECODE_WAVES; }
 
+/* Waves of a team: eight, two per SIMD; four at head dimension 256, whose tiles and
+ * accumulators take twice the registers. */
+static unsigned int decode_team_waves(unsigned long long head_dim)
+{
+    return head_dim > ROCM_MFMA_HEAD_DIM ? ROCM_TEAM_WAVES / 2u : ROCM_TEAM_WAVES;
+}
+
 /* Teams per (session, kv head) of the token-major decode, 0 when that form does not apply
  * (paged pools, wide groups).  A pure function of the request geometry. */
 static unsigned int decode_team_count(int paged, unsigned long long group, unsigned long long head_dim,
                                       unsigned long long max_context)
 {
     const unsigned long long tiles = (max_context + ROCM_PAGE_TOKENS - 1ull) / ROCM_PAGE_TOKENS;
-    unsigned long long teams = (tiles + ROCM_TEAM_WAVES * ROCM_TEAM_TILES - 1ull) /
-                               (ROCM_TEAM_WAVES * ROCM_TEAM_TILES);
-    if (paged || group > ROCM_TEAM_GROUP_MAX || head_dim != ROCM_MFMA_HEAD_DIM) return 0u;
+    const unsigned long long per_team = (unsigned long long)decode_team_waves(head_dim) *
+                                        (head_dim > ROCM_MFMA_HEAD_DIM ? ROCM_TEAM_TILES_WIDE : ROCM_TEAM_TILES);
+    unsigned long long teams = (tiles + per_team - 1ull) / per_team;
+    if (paged || group > ROCM_TEAM_GROUP_MAX) return 0u;
     if (teams > ROCM_TEAMS_MAX) teams = ROCM_TEAMS_MAX;
     return (unsigned int)(teams ? teams : 1ull);
+}
+
+/* A single query token over a token-major bf16 history takes the split decode kernels at
+ * head dimension 128, and the team form of them at 64 and 256 (groups of at most eight query
+ * heads); other single tokens run as a one-row tile of the prefill kernel. */
+static int decode_rows_geometry(const yvex_transformer_attention_requirement *r)
+{
+    return r->query_tokens == 1ull &&
+           (r->head_dimension == ROCM_MFMA_HEAD_DIM ||
+            r->query_heads / r->key_value_heads <= ROCM_TEAM_GROUP_MAX);
 }
 
 /* Balanced decode: two partial slots per wave, then (two-kernel form) the per-session offset
@@ -244,10 +263,13 @@ static int decode_run(yvex_backend *backend, const decode_job *job, const char *
     dp.fixed_context = (uint32_t)job->fixed_context;
     dp.waves = waves;
     dp.scale_log2 = job->scale * 1.4426950408889634f;
-    if (teams) /* teams of eight waves, merged through LDS and then between the teams */
-        rc = yvex_rocm_launch(backend, YVEX_ROCM_FN_DECODE_ROWS_BF16_TEAM, job->variant, teams,
-                              (unsigned int)job->kv_heads, (unsigned int)job->sessions,
-                              64u * ROCM_TEAM_WAVES, 0u, &dp, where, err);
+    if (teams) /* teams of waves, merged through LDS and then between the teams */
+        rc = yvex_rocm_launch(backend,
+                              job->head_dim == 64ull    ? YVEX_ROCM_FN_DECODE_ROWS_BF16_TEAM_64
+                              : job->head_dim == 256ull ? YVEX_ROCM_FN_DECODE_ROWS_BF16_TEAM_256
+                                                        : YVEX_ROCM_FN_DECODE_ROWS_BF16_TEAM,
+                              job->variant, teams, (unsigned int)job->kv_heads, (unsigned int)job->sessions,
+                              64u * decode_team_waves(job->head_dim), 0u, &dp, where, err);
     else
         rc = yvex_rocm_launch(backend, in_kernel ? job->merged_function : job->function, job->variant,
                               waves, 1u, 1u, 64u, 0u, &dp, where, err);
@@ -416,7 +438,7 @@ static int rocm_attention_workspace_required(const yvex_transformer_attention_re
     if (rc != YVEX_OK) return rc;
     if (!bytes) return refuse(err, YVEX_ERR_INVALID_ARG, where, "workspace byte output is required");
     if (r->numeric_contract == YVEX_TRANSFORMER_ATTENTION_NUMERIC_BF16_F32_ACCUMULATE &&
-        r->query_tokens == 1ull && r->head_dimension == ROCM_MFMA_HEAD_DIM) {
+        decode_rows_geometry(r)) {
         /* split-K decode partials; geometry must match decode_run */
         const unsigned int waves = decode_wave_count(1ull, r->key_value_heads, visible_tokens(r));
         const unsigned long long group = r->query_heads / r->key_value_heads;
@@ -649,9 +671,7 @@ static int attention_execute_common(yvex_backend *backend,
                 if (err) *err = cleanup;
             }
         }
-    } else if (r->query_tokens == 1ull && r->head_dimension == ROCM_MFMA_HEAD_DIM) {
-        /* the split decode kernels are built for head dimension 128; a single query token of
-         * another width runs as a one-row tile of the prefill kernel below */
+    } else if (decode_rows_geometry(r)) {
         decode_job job;
         memset(&job, 0, sizeof(job));
         job.function = YVEX_ROCM_FN_DECODE_ROWS_BF16;

@@ -87,6 +87,10 @@ static const rocm_kernel_binding rocm_kernel_bindings[] = {
      YVEX_ROCM_FN_DECODE_ROWS_BF16_MERGED},
     {"yvex_rocm_decode_rows_bf16_team", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_BF16,
      YVEX_ROCM_FN_DECODE_ROWS_BF16_TEAM},
+    {"yvex_rocm_decode_rows_bf16_team_64", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_BF16,
+     YVEX_ROCM_FN_DECODE_ROWS_BF16_TEAM_64},
+    {"yvex_rocm_decode_rows_bf16_team_256", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_BF16,
+     YVEX_ROCM_FN_DECODE_ROWS_BF16_TEAM_256},
     {"yvex_rocm_gather_rows", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_MLA_BF16, YVEX_ROCM_FN_GATHER_ROWS},
     {"yvex_rocm_kv_append_bf16", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_PAGED_BF16,
      YVEX_ROCM_FN_KV_APPEND_BF16},

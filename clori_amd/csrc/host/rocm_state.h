@@ -31,6 +31,8 @@ typedef enum {
     YVEX_ROCM_FN_DECODE_PAGED_Q8_0_MERGED,
     YVEX_ROCM_FN_DECODE_ROWS_BF16_MERGED,
     YVEX_ROCM_FN_DECODE_ROWS_BF16_TEAM,
+    YVEX_ROCM_FN_DECODE_ROWS_BF16_TEAM_64,
+    YVEX_ROCM_FN_DECODE_ROWS_BF16_TEAM_256,
     YVEX_ROCM_FN_PREFILL_BF16,
     YVEX_ROCM_FN_PREFILL_BF16_64,
     YVEX_ROCM_FN_PREFILL_BF16_256,

@@ -67,10 +67,16 @@ constexpr int kPageTokens = 16;
 __device__ inline void flag(int32_t *status, int code) { atomicCAS(status, 0, code); }
 
 typedef __attribute__((address_space(3))) short4v lds_short4;
-// LDS staging of a token-major V tile: row r (256 bytes) keeps its 16-byte chunk c at
-// position c ^ (r & 14), which spreads the 16 rows a transposed read touches over all banks
-// (each 32-byte column segment is hit by exactly two rows).
-__device__ inline uint32_t vt_offset(int row, int chunk) { return (uint32_t)(row * 256 + ((chunk ^ (row & 14)) << 4)); }
+// LDS staging of a token-major V tile: row r (256 bytes at head dimension 128) keeps its
+// 16-byte chunk c at position c ^ (r & 14), which spreads the 16 rows a transposed read
+// touches over all banks (each 32-byte column segment is hit by exactly two rows).  A row of
+// 64 lanes has eight chunks and swizzles over them (r & 6); one of 256 lanes swizzles within
+// each half.
+template <int kDim>
+__device__ inline uint32_t vt_offset(int row, int chunk)
+{
+    return (uint32_t)(row * (kDim * 2) + ((chunk ^ (row & (kDim >= 128 ? 14 : 6))) << 4));
+}
 
 template <int kDim>
 struct State {
@@ -106,7 +112,8 @@ template <int kDim>
 struct Bf16Tile {
     u32x4 k[kDim / 32];  // K[token = lane%16][32*j + 8*(lane/16) .. +7]
     u32x2 v[kDim / 16];  // paged: V[tokens 4*(lane/16)..+3][dim 16*b + lane%16]
-                 // token-major: raw row chunks, (v[2j], v[2j+1]) = V[token 4j + lane/16][8*(lane%16)..+7]
+                 // token-major: raw row chunks, (v[2j], v[2j+1]) = chunk e = 64 * j + lane of the tile,
+                 // V[token e / (kDim / 8)][8 * (e % (kDim / 8)) .. +7]
 };
 
 // kHeadDimension: 128 is the tuned build (paged and token-major); 64 and 256 are the same
@@ -135,17 +142,18 @@ struct Bf16Kv {
                                             const yvex_rocm_decode_params &p, uint32_t first,
                                             uint32_t rows_left, int lane)
     {
-        static_assert(kDim == 128, "token-major rows: 16 lanes x 8 dims cover the row");
+        constexpr int kChunks = kDim / 8;  // 16-byte chunks of a row
         const int n = lane & 15, g = lane >> 4;
         const uint16_t *k = (const uint16_t *)kbytes, *v = (const uint16_t *)vbytes;
         const uint32_t last = rows_left - 1u;
         const uint16_t *krow = k + (uint64_t)(first + min((uint32_t)n, last)) * p.k_token_stride;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) t.k[j] = load_b128(krow + j * 32 + g * 8);
+        for (int j = 0; j < kDim / 32; ++j) t.k[j] = load_b128(krow + j * 32 + g * 8);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const uint16_t *vrow = v + (uint64_t)(first + min((uint32_t)(4 * j + g), last)) * p.v_token_stride;
-            const u32x4 chunk = load_b128(vrow + n * 8);
+        for (int j = 0; j < kDim / 32; ++j) {
+            const int e = 64 * j + lane;
+            const uint16_t *vrow = v + (uint64_t)(first + min((uint32_t)(e / kChunks), last)) * p.v_token_stride;
+            const u32x4 chunk = load_b128(vrow + (e % kChunks) * 8);
             t.v[2 * j] = (u32x2){chunk.x, chunk.y};
             t.v[2 * j + 1] = (u32x2){chunk.z, chunk.w};
         }
@@ -156,17 +164,19 @@ struct Bf16Kv {
     // wave execute in order, so the area can be reused tile after tile without a barrier.
     __device__ static inline void transpose_rows(Tile &t, unsigned char *vt, int lane)
     {
+        constexpr int kChunks = kDim / 8;
         const int a = lane & 15, g = lane >> 4;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+        for (int j = 0; j < kDim / 32; ++j) {
+            const int e = 64 * j + lane;
             const u32x4 chunk = {t.v[2 * j].x, t.v[2 * j].y, t.v[2 * j + 1].x, t.v[2 * j + 1].y};
-            *reinterpret_cast<u32x4 *>(vt + vt_offset(4 * j + g, a)) = chunk;
+            *reinterpret_cast<u32x4 *>(vt + vt_offset<kDim>(e / kChunks, e % kChunks)) = chunk;
         }
         const int row = 4 * g + (a >> 2);
 #pragma unroll
-        for (int b = 0; b < 8; ++b) {
+        for (int b = 0; b < kDim / 16; ++b) {
             const short4v w = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                (lds_short4 *)(vt + vt_offset(row, 2 * b + ((a >> 1) & 1)) + 8 * (a & 1)));
+                (lds_short4 *)(vt + vt_offset<kDim>(row, 2 * b + ((a >> 1) & 1)) + 8 * (a & 1)));
             t.v[b] = __builtin_bit_cast(u32x2, w);
         }
     }
@@ -327,7 +337,6 @@ __device__ inline uint32_t wave_inclusive_scan(uint32_t v, int lane)
 template <class Kv, bool PAGED, int kDepth, bool MERGE>
 struct Decoder {
     static constexpr int kDim = Kv::kDim;
-    static_assert(kDim == 128 || (PAGED && !MERGE), "other head dimensions: the two-launch paged form");
     typedef typename Kv::Tile Tile;
     typedef ::State<kDim> State;
     const yvex_rocm_decode_params &p;
@@ -615,6 +624,8 @@ struct Decoder {
 
     __device__ inline void run() const
     {
+        static_assert(kDim == 128 || (PAGED && !MERGE),
+                      "other head dimensions: the two-launch paged form, or teams over token-major rows");
         const uint32_t wave = blockIdx.x, waves = gridDim.x;
         uint32_t session = 0u, offset = 0u, tiles = 0u, total = 0u;
         (void)locate(0xffffffffu, session, offset, tiles, total);
@@ -695,9 +706,11 @@ struct Decoder {
     // grid = (teams per segment, kv_heads, sessions), block = 64 * kTeam; group <= 8.
     // team_lds: kTeam areas of 4 KB, a wave's V transposition first and its accumulators
     // ([group][128] F32) once it has streamed its tiles, then [kTeam][8][2] (max, sum).
-    static constexpr int kTeam = 8;
-    static constexpr uint32_t kTeamArea = kPageTokens * kHeadDim * 2u / sizeof(float);  // floats
-    static constexpr uint32_t kTeamLdsBytes = kTeam * (kPageTokens * kHeadDim * 2u + 8u * 2u * sizeof(float));
+    // At head dimension 256 a wave's tiles and accumulators take twice the registers: teams
+    // of four waves, one per SIMD.
+    static constexpr int kTeam = kDim > 128 ? 4 : 8;
+    static constexpr uint32_t kTeamArea = kPageTokens * kDim * 2u / sizeof(float);  // floats
+    static constexpr uint32_t kTeamLdsBytes = kTeam * (kPageTokens * kDim * 2u + 8u * 2u * sizeof(float));
 
     __device__ inline void run_team(float *parts) const
     {
@@ -710,12 +723,12 @@ struct Decoder {
         const uint32_t first = min(tiles, (team * kTeam + wave) * per_wave);
         const uint32_t count = min(per_wave, tiles - first);
 
-        bf16x8 q[4];
+        bf16x8 q[kDim / 32];
         {
             const uint16_t *qrow = p.q + ((uint64_t)session * p.query_heads + kv_head * group +
-                                          min((uint32_t)n, group - 1u)) * kHeadDim;
+                                          min((uint32_t)n, group - 1u)) * kDim;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
+            for (int j = 0; j < kDim / 32; ++j) {
                 u32x4 raw = load_b128(qrow + j * 32 + g * 8);
                 if ((uint32_t)n >= group) raw = (u32x4){0u, 0u, 0u, 0u};
                 q[j] = as_bf16x8(raw);
@@ -723,7 +736,7 @@ struct Decoder {
         }
         State st;
 #pragma unroll
-        for (int b = 0; b < 8; ++b) st.o[b] = (floatx4){0.f, 0.f, 0.f, 0.f};
+        for (int b = 0; b < kDim / 16; ++b) st.o[b] = (floatx4){0.f, 0.f, 0.f, 0.f};
         st.m = -INFINITY;
         st.l = 0.f;
         for (uint32_t done = 0u; done < count; done += 128u)
@@ -735,9 +748,9 @@ struct Decoder {
         // the wave's part into LDS (a wave without tiles leaves max -inf, sum 0, zeros)
         float *acc = parts, *ml = parts + kTeam * kTeamArea;
         if ((uint32_t)n < group) {
-            float *row = acc + wave * kTeamArea + (uint32_t)n * kHeadDim + g * 4;
+            float *row = acc + wave * kTeamArea + (uint32_t)n * kDim + g * 4;
 #pragma unroll
-            for (int b = 0; b < 8; ++b) *reinterpret_cast<floatx4 *>(row + b * 16) = st.o[b];
+            for (int b = 0; b < kDim / 16; ++b) *reinterpret_cast<floatx4 *>(row + b * 16) = st.o[b];
             if (g == 0) {
                 ml[(wave * 8u + (uint32_t)n) * 2u] = st.m;
                 ml[(wave * 8u + (uint32_t)n) * 2u + 1u] = l;
@@ -745,14 +758,14 @@ struct Decoder {
         }
         __syncthreads();
 
-        // the team's part: thread t merges (head, dim) pairs t, t + 512, ... over the waves,
+        // the team's part: thread t merges (head, dim) pairs t, t + 64 * kTeam, ... over the waves,
         // in wave order
-        const uint32_t values = group * kHeadDim;
+        const uint32_t values = group * kDim;
         const uint64_t segment = (uint64_t)session * p.kv_heads + kv_head;
         const uint64_t slot0 = (segment * teams + team) * group;
         const bool whole = teams == 1u;
         for (uint32_t at = threadIdx.x; at < values; at += 64u * kTeam) {
-            const uint32_t hh = at / kHeadDim, d = at % kHeadDim;
+            const uint32_t hh = at / kDim, d = at % kDim;
             float top = -INFINITY;
 #pragma unroll
             for (int w = 0; w < kTeam; ++w) top = fmaxf(top, ml[(w * 8u + hh) * 2u]);
@@ -762,12 +775,12 @@ struct Decoder {
                 const float m = ml[(w * 8u + hh) * 2u];
                 const float weight = m == -INFINITY ? 0.f : fast_exp2(m - top);
                 sum += weight * ml[(w * 8u + hh) * 2u + 1u];
-                o += weight * acc[w * kTeamArea + hh * kHeadDim + d];
+                o += weight * acc[w * kTeamArea + hh * kDim + d];
             }
             if (whole) {
                 publish_value(session, kv_head * group + hh, d, o, sum, top);
             } else {
-                __hip_atomic_store(p.part_acc + (slot0 + hh) * kHeadDim + d, o, __ATOMIC_RELAXED,
+                __hip_atomic_store(p.part_acc + (slot0 + hh) * kDim + d, o, __ATOMIC_RELAXED,
                                    __HIP_MEMORY_SCOPE_AGENT);
                 if (d == 0u) store_b64_device(p.part_ml + (slot0 + hh) * 2u, top, sum);
             }
@@ -792,17 +805,29 @@ struct Decoder {
         // zero): one memory round trip per kTeamsPerTrip teams
         loads_ordered();
         constexpr uint32_t kTeamsPerTrip = 16u;
-        for (uint32_t at = threadIdx.x; at < values; at += 64u * kTeam) {
-            const uint32_t hh = at / kHeadDim, d = at % kHeadDim;
-            float top = -INFINITY, sum = 0.f, o = 0.f;
+        // a thread takes kLanes neighbouring lanes of a head at a time: one at head dimension
+        // 64 and 128, where a thread has one value or two in all; eight at 256, whose team of
+        // four waves would otherwise walk up to eight values per thread, two dependent trips each
+        constexpr uint32_t kLanes = kDim > 128 ? 8u : 1u;
+        for (uint32_t at = threadIdx.x * kLanes; at < values; at += 64u * kTeam * kLanes) {
+            const uint32_t hh = at / kDim, d = at % kDim;
+            float top = -INFINITY, sum = 0.f, o[kLanes];
+#pragma unroll
+            for (uint32_t e = 0u; e < kLanes; ++e) o[e] = 0.f;
             for (uint32_t t0 = 0u; t0 < teams; t0 += kTeamsPerTrip) {
-                float m[kTeamsPerTrip], part_l[kTeamsPerTrip], v[kTeamsPerTrip];
+                float m[kTeamsPerTrip], part_l[kTeamsPerTrip], v[kTeamsPerTrip][kLanes];
 #pragma unroll
                 for (uint32_t i = 0u; i < kTeamsPerTrip; ++i) {
                     const uint64_t slot = (segment * teams + min(t0 + i, teams - 1u)) * group + hh;
                     load_b64_device(p.part_ml + slot * 2u, m[i], part_l[i]);
-                    v[i] = __hip_atomic_load(p.part_acc + slot * kHeadDim + d, __ATOMIC_RELAXED,
-                                             __HIP_MEMORY_SCOPE_AGENT);
+                    if constexpr (kLanes == 1u) {
+                        v[i][0] = __hip_atomic_load(p.part_acc + slot * kDim + d, __ATOMIC_RELAXED,
+                                                    __HIP_MEMORY_SCOPE_AGENT);
+                    } else {
+#pragma unroll
+                        for (uint32_t e = 0u; e < kLanes; e += 2u)
+                            load_b64_device(p.part_acc + slot * kDim + d + e, v[i][e], v[i][e + 1u]);
+                    }
                 }
                 float trip = -INFINITY;
 #pragma unroll
@@ -813,16 +838,20 @@ struct Decoder {
                 const float m_new = fmaxf(top, trip);
                 const float keep = top == -INFINITY ? 0.f : fast_exp2(top - m_new);
                 sum *= keep;
-                o *= keep;
+#pragma unroll
+                for (uint32_t e = 0u; e < kLanes; ++e) o[e] *= keep;
 #pragma unroll
                 for (uint32_t i = 0u; i < kTeamsPerTrip; ++i) {
                     const float weight = m[i] == -INFINITY ? 0.f : fast_exp2(m[i] - m_new);
                     sum += weight * part_l[i];
-                    o += weight * v[i];
+#pragma unroll
+                    for (uint32_t e = 0u; e < kLanes; ++e) o[e] += weight * v[i][e];
                 }
                 top = m_new;
             }
-            publish_value(session, kv_head * group + hh, d, o, sum, top);
+#pragma unroll
+            for (uint32_t e = 0u; e < kLanes; ++e)
+                publish_value(session, kv_head * group + hh, d + e, o[e], sum, top);
         }
     }
 
@@ -830,7 +859,7 @@ struct Decoder {
     __device__ inline void publish_value(uint32_t session, uint32_t head, uint32_t d, float o, float sum,
                                          float top) const
     {
-        const uint64_t at = ((uint64_t)session * p.query_heads + head) * kHeadDim + d;
+        const uint64_t at = ((uint64_t)session * p.query_heads + head) * kDim + d;
         float value = o / sum;
         if (p.gate) value = bf16_to_f32(bf16_bits(value)) * sigmoid(bf16_to_f32(p.gate[at]));
         if (!isfinite(value)) flag(p.status, YVEX_ROCM_DEVICE_NUMERIC);
@@ -864,15 +893,22 @@ YVEX_DECODE_KERNEL(yvex_rocm_decode_paged_bf16_merged, Bf16Kv<128>, true, 3, tru
 YVEX_DECODE_KERNEL(yvex_rocm_decode_paged_q8_0_merged, Q8Kv, true, 3, true)
 YVEX_DECODE_KERNEL(yvex_rocm_decode_rows_bf16_merged, Bf16Kv<128>, false, 2, true)
 
-// teams of eight waves over a token-major history (see Decoder::run_team)
-extern "C" __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
-yvex_rocm_decode_rows_bf16_team(const yvex_rocm_decode_params p)
-{
-    typedef Decoder<Bf16Kv<128>, false, 2, true> Team;
-    __shared__ __attribute__((aligned(16))) unsigned char team_lds[Team::kTeamLdsBytes];
-    const uint32_t wave = threadIdx.x >> 6;
-    Team(p, team_lds + wave * (kPageTokens * kHeadDim * 2)).run_team(reinterpret_cast<float *>(team_lds));
-}
+// teams of waves over a token-major history (see Decoder::run_team): eight waves, two per
+// SIMD; four, one per SIMD, at head dimension 256
+#define YVEX_DECODE_TEAM_KERNEL(name, head_dim, THREADS, WAVES)                                      \
+    extern "C" __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(WAVES, WAVES))) \
+    name(const yvex_rocm_decode_params p)                                                      \
+    {                                                                                          \
+        typedef Decoder<Bf16Kv<head_dim>, false, 2, true> Team;                                \
+        static_assert(THREADS == 64 * Team::kTeam, "one workgroup is one team");               \
+        __shared__ __attribute__((aligned(16))) unsigned char team_lds[Team::kTeamLdsBytes];   \
+        const uint32_t wave = threadIdx.x >> 6;                                                \
+        Team(p, team_lds + wave * (kPageTokens * head_dim * 2)).run_team(reinterpret_cast<float *>(team_lds)); \
+    }
+
+YVEX_DECODE_TEAM_KERNEL(yvex_rocm_decode_rows_bf16_team, 128, 512, 2)
+YVEX_DECODE_TEAM_KERNEL(yvex_rocm_decode_rows_bf16_team_64, 64, 512, 2)
+YVEX_DECODE_TEAM_KERNEL(yvex_rocm_decode_rows_bf16_team_256, 256, 256, 1)
 
 // Merge of the split segments of the balanced decode when the decode kernel was launched
 // without arrival counters (large launches).  grid = (query_heads, sessions), block =

@@ -110,6 +110,43 @@ def test_rows_decode_interleaved_kv_history_rows(backend):
     assert_close_bf16(got, ref, "interleaved")
 
 
+@pytest.mark.parametrize("d", [64, 256])
+@pytest.mark.parametrize("hq,hkv,ctx", [(24, 4, 4096), (1, 1, 1), (8, 1, 17), (6, 2, 1000), (16, 2, 9000),
+                                        (4, 4, 40000), (32, 2, 700)])
+def test_rows_decode_other_head_dimensions(backend, d, hq, hkv, ctx):
+    """One query token over a token-major history at head dimension 64 and 256 (the reference's
+    own Qwen pattern is 24/4/256, tests/unit/cuda/quant_qtype.c:2413-2418): teams of waves as at
+    128 for groups of at most eight query heads (partials in the workspace once there is more
+    than one team), a one-row tile of the prefill kernel for wider groups.  Packed and
+    interleaved [K|V] rows give the same bits; the FULL mask sees the rows behind the query."""
+    rng = np.random.default_rng(d * 1000003 + hq * 1009 + ctx)
+    q = bf16_normal(rng, (1, hq, d))
+    k = bf16_normal(rng, (ctx + 2, hkv, d))
+    v = bf16_normal(rng, (ctx + 2, hkv, d))
+    label = "d=%d hq=%d hkv=%d ctx=%d" % (d, hq, hkv, ctx)
+    got, lse, facts = run_rows_decode(backend, q, k, v, query_start=ctx - 1)
+    rc, ref, _, ref_lse = ORACLE.gqa_bf16(q, k, v, query_start=ctx - 1, causal=True)
+    assert rc == 0
+    assert_close_bf16(got, ref, label)
+    assert_lse(lse, ref_lse, label)
+    assert facts.kernel_launches == 1
+    assert (facts.temporary_bytes > 0) == (hq // hkv <= 8), label   # teams leave partials, the tile none
+    again, lse_again, _ = run_rows_decode(backend, q, k, v, query_start=ctx - 1)
+    assert np.array_equal(got, again) and np.array_equal(lse, lse_again)
+    width, tk = hkv * d, ctx + 2
+    store = np.zeros((tk, 2 * width), dtype=np.uint16)
+    store[:, :width] = k.reshape(tk, width)
+    store[:, width:] = v.reshape(tk, width)
+    strided, lse_strided, _ = run_rows_decode(backend, q, k, v, query_start=ctx - 1, k_stride=2 * width,
+                                              v_stride=2 * width, kv_storage=store)
+    assert np.array_equal(got, strided) and np.array_equal(lse, lse_strided)
+    if ctx <= 9000:
+        full, lse_full, _ = run_rows_decode(backend, q, k, v, query_start=ctx - 1, causal=False)
+        rc, ref, _, ref_lse = ORACLE.gqa_bf16(q, k, v, query_start=ctx - 1, causal=False)
+        assert_close_bf16(full, ref, "full " + label)
+        assert_lse(lse_full, ref_lse, "full " + label)
+
+
 def make_paged_case(rng, contexts, hq, hkv, d=128, page_tokens=16, spare=5, q8=False):
     sessions = len(contexts)
     need = [(c + page_tokens - 1) // page_tokens for c in contexts]

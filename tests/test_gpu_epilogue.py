@@ -56,13 +56,14 @@ def test_prefill_with_fused_gate(backend, tq, tk, start, hq, hkv, causal):
         x.release()
 
 
+@pytest.mark.parametrize("d", [128, 64, 256])
 @pytest.mark.parametrize("ctx", [1, 17, 300, 4096])
-def test_row_decode_with_fused_gate(backend, ctx):
-    rng = np.random.default_rng(7100 + ctx)
-    q = bf16_normal(rng, (1, 32, 128))
-    k, v = bf16_normal(rng, (ctx, 8, 128)), bf16_normal(rng, (ctx, 8, 128))
-    gate = bf16_normal(rng, (1, 32, 128), scale=2.5)
-    req = backend.attention_requirement(1, ctx, 32, 8, 128, causal=True, query_start=ctx - 1,
+def test_row_decode_with_fused_gate(backend, ctx, d):
+    rng = np.random.default_rng(7100 + ctx + d)
+    q = bf16_normal(rng, (1, 32, d))
+    k, v = bf16_normal(rng, (ctx, 8, d)), bf16_normal(rng, (ctx, 8, d))
+    gate = bf16_normal(rng, (1, 32, d), scale=2.5)
+    req = backend.attention_requirement(1, ctx, 32, 8, d, causal=True, query_start=ctx - 1,
                                         dtype=B.DTYPE_BF16, contract=B.NUMERIC_BF16_F32_ACCUMULATE)
     t = [backend.tensor("q", B.DTYPE_BF16, q.shape, q), backend.tensor("k", B.DTYPE_BF16, k.shape, k),
          backend.tensor("v", B.DTYPE_BF16, v.shape, v)]

@@ -1358,3 +1358,28 @@ def test_causal_exact_prefill_gets_item_lists_with_equal_work_per_unit(fake_runt
         b.attention_execute(other, q3, k, v, out3)
         assert fake_runtime.fake_hip_last_grid_x() == 512
         assert launch()[0] == items
+
+
+def test_single_token_bf16_requests_take_the_team_kernels_at_every_head_dimension(fake_runtime):
+    """One query token over a token-major bf16 history: teams of waves at head dimension 64,
+    128 and 256 for groups of at most eight query heads (grid = teams x kv heads, the
+    workspace holds one partial per team), the one-row prefill tile for wider groups at 64
+    and 256 (no workspace)."""
+    fake_runtime.fake_hip_last_grid_x.restype = C.c_uint
+    with Backend() as b:
+        for d, hq, hkv, ctx, grid, partials in [(128, 32, 8, 4096, 16, True), (64, 16, 4, 4096, 16, True),
+                                                (256, 24, 4, 4096, 16, True), (256, 24, 4, 300, 2, True),
+                                                (256, 24, 4, 100000, 32, True), (64, 4, 4, 16, 1, True),
+                                                (256, 32, 2, 4096, 32, False), (64, 12, 1, 300, 12, False)]:
+            req = b.attention_requirement(1, ctx, hq, hkv, d, causal=True, query_start=ctx - 1,
+                                          dtype=B.DTYPE_BF16, contract=B.NUMERIC_BF16_F32_ACCUMULATE)
+            q, out = written(b, "q", B.DTYPE_BF16, (1, hq, d)), b.tensor("o", B.DTYPE_BF16, (1, hq, d))
+            k, v = written(b, "k", B.DTYPE_BF16, (ctx, hkv, d)), written(b, "v", B.DTYPE_BF16, (ctx, hkv, d))
+            need = b.attention_workspace_required(req)
+            facts = b.attention_execute(req, q, k, v, out)
+            label = (d, hq, hkv, ctx)
+            assert facts.kernel_launches == 1, label
+            assert fake_runtime.fake_hip_last_grid_x() == grid, label
+            assert (need > 0) == partials and facts.temporary_bytes == need, label
+            for t in (q, out, k, v):
+                t.release()
