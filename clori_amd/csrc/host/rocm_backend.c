@@ -541,6 +541,7 @@ static int rocm_close(yvex_backend *backend, yvex_error *err)
     rc = yvex_rocm_kernel_bundle_close(backend, err);
     if (rc != YVEX_OK) return rc; /* impl retained: checked close can be retried */
     if (state->device_status) (void)state->driver.hipFree(state->device_status);
+    if (state->status_mailbox) (void)state->driver.hipHostFree((void *)state->status_mailbox);
     if (state->decode_arrivals) (void)state->driver.hipFree(state->decode_arrivals);
     if (state->schedule_device) (void)state->driver.hipFree(state->schedule_device);
     probe_release(state);
@@ -688,6 +689,19 @@ static int rocm_open(yvex_backend **out, const char *device, unsigned long long 
                               state->driver.hipMemsetAsync(state->device_status, 0, 256u,
                                                            state->stream),
                               where, err);
+    if (rc == YVEX_OK && state->driver.pinned_memory) {
+        /* the status mailbox is an economy, not a requirement: without it the word is copied */
+        void *host = NULL, *device = NULL;
+        if (state->driver.hipHostMalloc(&host, 256u, hipHostMallocMapped) == hipSuccess && host) {
+            if (state->driver.hipHostGetDevicePointer(&device, host, 0u) == hipSuccess && device) {
+                memset(host, 0, 256u);
+                state->status_mailbox = (volatile uint64_t *)host;
+                state->status_mailbox_device = (uint64_t *)device;
+            } else {
+                (void)state->driver.hipHostFree(host);
+            }
+        }
+    }
     if (rc == YVEX_OK)
         rc = yvex_rocm_status(&state->driver,
                               state->driver.hipMalloc((void **)&state->decode_arrivals,
@@ -711,6 +725,7 @@ static int rocm_open(yvex_backend **out, const char *device, unsigned long long 
         yvex_error keep = err ? *err : (yvex_error){0};
         yvex_error scratch;
         if (state->device_status) (void)state->driver.hipFree(state->device_status);
+        if (state->status_mailbox) (void)state->driver.hipHostFree((void *)state->status_mailbox);
         if (state->decode_arrivals) (void)state->driver.hipFree(state->decode_arrivals);
         if (state->schedule_device) (void)state->driver.hipFree(state->schedule_device);
         if (state->timing_start) (void)state->driver.hipEventDestroy(state->timing_start);

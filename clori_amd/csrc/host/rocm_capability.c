@@ -7,10 +7,15 @@
  * YVEX_TEST_ROCM_BUNDLE_FAILURE (module | symbol | <function name>),
  * YVEX_TEST_ROCM_LAUNCH_FAILURE, YVEX_TEST_ROCM_SYNC_FAILURE (all | <variant name>) and
  * YVEX_TEST_ROCM_CLEANUP_FAILURE, mirroring the YVEX_TEST_CUDA_* switches. */
+#ifndef _POSIX_C_SOURCE
+#define _POSIX_C_SOURCE 200809L /* clock_gettime */
+#endif
 #include "rocm_state.h"
+#include "../kernel_params.h"
 
 #include <stdlib.h>
 #include <string.h>
+#include <time.h>
 
 typedef struct {
     const char *name;
@@ -91,6 +96,8 @@ static const rocm_kernel_binding rocm_kernel_bindings[] = {
      YVEX_ROCM_FN_DECODE_ROWS_BF16_TEAM_64},
     {"yvex_rocm_decode_rows_bf16_team_256", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_BF16,
      YVEX_ROCM_FN_DECODE_ROWS_BF16_TEAM_256},
+    {"yvex_rocm_status_forward", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_F32,
+     YVEX_ROCM_FN_STATUS_FORWARD},
     {"yvex_rocm_gather_rows", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_MLA_BF16, YVEX_ROCM_FN_GATHER_ROWS},
     {"yvex_rocm_kv_append_bf16", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_PAGED_BF16,
      YVEX_ROCM_FN_KV_APPEND_BF16},
@@ -476,26 +483,94 @@ int yvex_rocm_synchronize(yvex_backend *backend, yvex_backend_operation_variant 
     return rc;
 }
 
-/* Reads the device status word (the stream is synchronised by the copy's own wait),
- * clears it when set, and maps it like src/backend/cuda/transformer.c:648-660. */
+/* How long the host watches the mailbox before it leaves the wait to the runtime. */
+#define ROCM_MAILBOX_SPIN_NS 200000ll
+
+static long long monotonic_ns(void)
+{
+    struct timespec now;
+    clock_gettime(CLOCK_MONOTONIC, &now);
+    return (long long)now.tv_sec * 1000000000ll + (long long)now.tv_nsec;
+}
+
+/* The status word by way of the mailbox: a one-thread kernel behind the operation's kernels
+ * stores (sequence, status) into host memory and the host watches for the sequence number,
+ * about 8 us for an operation of one small kernel where a copy of the word and a wait for the
+ * stream take 22.  A device that does not answer within ROCM_MAILBOX_SPIN_NS is waited for
+ * through the runtime, which also reports a device that has failed.  Returns YVEX_ERR_UNSUPPORTED
+ * (and has done nothing) when this backend has no mailbox. */
+static int status_by_mailbox(yvex_backend *backend, const char *where, int32_t *host_status,
+                             yvex_error *err)
+{
+    yvex_rocm_backend_state *state = yvex_rocm_state(backend);
+    yvex_rocm_status_forward_params fp;
+    void *arguments[1];
+    uint64_t seen;
+    long long deadline;
+    unsigned int turn = 0u;
+    int rc;
+    if (!state->status_mailbox || !state->functions[YVEX_ROCM_FN_STATUS_FORWARD])
+        return YVEX_ERR_UNSUPPORTED;
+    fp.status = state->device_status;
+    fp.mailbox = state->status_mailbox_device;
+    fp.sequence = ++state->status_sequence;
+    arguments[0] = &fp;
+    rc = yvex_rocm_status(&state->driver,
+                          state->driver.hipModuleLaunchKernel(
+                              state->functions[YVEX_ROCM_FN_STATUS_FORWARD], 1u, 1u, 1u, 64u, 1u, 1u, 0u,
+                              state->stream, arguments, NULL),
+                          where, err);
+    if (rc != YVEX_OK) return rc;
+    deadline = monotonic_ns() + ROCM_MAILBOX_SPIN_NS;
+    for (;;) {
+        seen = __atomic_load_n(state->status_mailbox, __ATOMIC_ACQUIRE);
+        if ((uint32_t)(seen >> 32) == fp.sequence) break;
+        if ((++turn & 63u) == 0u && monotonic_ns() > deadline) {
+            rc = yvex_rocm_synchronize(backend, YVEX_BACKEND_VARIANT_TENSOR_READ, where, err);
+            if (rc != YVEX_OK) return rc;
+            seen = __atomic_load_n(state->status_mailbox, __ATOMIC_ACQUIRE);
+            if ((uint32_t)(seen >> 32) != fp.sequence) {
+                yvex_error_set(err, YVEX_ERR_BACKEND, where,
+                               "the stream ended without the operation's status reaching the host");
+                return YVEX_ERR_BACKEND;
+            }
+            break;
+        }
+    }
+    *host_status = (int32_t)(uint32_t)seen;
+    return YVEX_OK;
+}
+
+/* Reads the device status word once the stream's work has ended (through the mailbox, or
+ * with a copy whose wait synchronises the stream), clears it when set, and maps it like
+ * src/backend/cuda/transformer.c:648-660. */
 int yvex_rocm_status_check(yvex_backend *backend, const char *where,
                            yvex_backend_operation_facts *facts, yvex_error *err)
 {
     yvex_rocm_backend_state *state = yvex_rocm_state(backend);
     int32_t host_status = 0;
-    int rc;
+    int rc, cleared = 0;
     if (state->recording) {
         yvex_error_set(err, YVEX_ERR_STATE, where,
                        "cannot read the device status while a launch sequence is being recorded");
         return YVEX_ERR_STATE;
     }
-    rc = yvex_rocm_status(&state->driver,
-                          state->driver.hipMemcpyAsync(&host_status, state->device_status,
-                                                       sizeof(host_status), hipMemcpyDeviceToHost,
-                                                       state->stream),
-                          where, err);
-    if (rc == YVEX_OK)
-        rc = yvex_rocm_synchronize(backend, YVEX_BACKEND_VARIANT_TENSOR_READ, where, err);
+    rc = backend_dispatch_admit(backend, where, err);
+    if (rc != YVEX_OK) return rc;
+    rc = test_failure_matches("YVEX_TEST_ROCM_SYNC_FAILURE", YVEX_BACKEND_VARIANT_TENSOR_READ)
+             ? YVEX_ERR_UNSUPPORTED /* the injected failure belongs to the runtime's wait */
+             : status_by_mailbox(backend, where, &host_status, err);
+    if (rc == YVEX_OK) {
+        cleared = 1; /* the forwarding kernel cleared a word that was set */
+    } else if (rc == YVEX_ERR_UNSUPPORTED) {
+        rc = yvex_rocm_status(&state->driver,
+                              state->driver.hipMemcpyAsync(&host_status, state->device_status,
+                                                           sizeof(host_status), hipMemcpyDeviceToHost,
+                                                           state->stream),
+                              where, err);
+        if (rc == YVEX_OK)
+            rc = yvex_rocm_synchronize(backend, YVEX_BACKEND_VARIANT_TENSOR_READ, where, err);
+    }
     if (rc != YVEX_OK) return rc;
     state->status_dirty = 0;
     backend->stats.d2h_bytes += sizeof(host_status);
@@ -508,11 +583,13 @@ int yvex_rocm_status_check(yvex_backend *backend, const char *where,
         yvex_error_clear(err);
         return YVEX_OK;
     }
-    rc = yvex_rocm_status(&state->driver,
-                          state->driver.hipMemsetAsync(state->device_status, 0,
-                                                       sizeof(host_status), state->stream),
-                          where, err);
-    if (rc != YVEX_OK) return rc;
+    if (!cleared) {
+        rc = yvex_rocm_status(&state->driver,
+                              state->driver.hipMemsetAsync(state->device_status, 0,
+                                                           sizeof(host_status), state->stream),
+                              where, err);
+        if (rc != YVEX_OK) return rc;
+    }
     switch (host_status) {
     case 2:
         yvex_error_set(err, YVEX_ERR_BOUNDS, where,

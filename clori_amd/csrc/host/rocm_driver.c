@@ -52,6 +52,15 @@ int yvex_rocm_driver_load(yvex_rocm_driver *driver, yvex_error *err)
 #define X(name) driver->name = NULL;
     if (!driver->virtual_memory) { YVEX_ROCM_DRIVER_VIRTUAL_ENTRIES(X) }
 #undef X
+    driver->pinned_memory = 1;
+#define X(name)                                                                          \
+    driver->name = (__typeof__(driver->name))dlsym(driver->library, #name);              \
+    if (!driver->name) driver->pinned_memory = 0;
+    YVEX_ROCM_DRIVER_PINNED_ENTRIES(X)
+#undef X
+#define X(name) driver->name = NULL;
+    if (!driver->pinned_memory) { YVEX_ROCM_DRIVER_PINNED_ENTRIES(X) }
+#undef X
     driver->timed_launch =
         (yvex_rocm_timed_launch_fn)dlsym(driver->library, "hipExtModuleLaunchKernel");
     yvex_error_clear(err);

@@ -31,6 +31,10 @@
     X(hipMemGetAllocationGranularity) X(hipMemAddressReserve) X(hipMemAddressFree)       \
     X(hipMemCreate) X(hipMemRelease) X(hipMemMap) X(hipMemUnmap) X(hipMemSetAccess)
 
+/* Host memory the device can write: the mailbox through which an operation's status word
+ * reaches the host without a copy.  Bound all or none; without them the status is copied. */
+#define YVEX_ROCM_DRIVER_PINNED_ENTRIES(X) X(hipHostMalloc) X(hipHostFree) X(hipHostGetDevicePointer)
+
 /* hipExtModuleLaunchKernel (hip/hip_ext.h, a C++ header): a launch whose two events take the
  * kernel's own begin and end timestamps.  Work sizes are in threads, not workgroups. */
 typedef hipError_t (*yvex_rocm_timed_launch_fn)(hipFunction_t, uint32_t, uint32_t, uint32_t, uint32_t,
@@ -43,8 +47,10 @@ typedef struct yvex_rocm_driver {
 #define X(name) __typeof__(&name) name;
     YVEX_ROCM_DRIVER_ENTRIES(X)
     YVEX_ROCM_DRIVER_VIRTUAL_ENTRIES(X) /* optional: all NULL when any is missing */
+    YVEX_ROCM_DRIVER_PINNED_ENTRIES(X)  /* optional, likewise */
 #undef X
     int virtual_memory;                 /* the virtual memory entries are bound */
+    int pinned_memory;                  /* the pinned host memory entries are bound */
     yvex_rocm_timed_launch_fn timed_launch; /* optional: NULL when the runtime lacks it */
 } yvex_rocm_driver;
 

@@ -49,6 +49,7 @@ typedef enum {
     YVEX_ROCM_FN_BF16_ROUND_F32,
     YVEX_ROCM_FN_SIGMOID_PRODUCT_BF16_F32,
     YVEX_ROCM_FN_SPLIT_INTERLEAVED_TWO_F32,
+    YVEX_ROCM_FN_STATUS_FORWARD,
     YVEX_ROCM_FN_GATHER_ROWS,
     YVEX_ROCM_FN_COUNT
 } yvex_rocm_function_id;
@@ -99,6 +100,11 @@ typedef struct yvex_rocm_backend_state {
     yvex_backend_capability_reason variant_failures[YVEX_BACKEND_VARIANT_ROCM_END];
     yvex_backend_capability_reason backend_failure_reason;
     int32_t *device_status; /* one status word, zero between operations */
+    /* the status word's way to the host without a copy: a word of host memory the device can
+     * write, its device address, and the sequence number of the last forward asked for */
+    volatile uint64_t *status_mailbox;
+    uint64_t *status_mailbox_device;
+    uint32_t status_sequence;
     uint32_t *decode_arrivals; /* YVEX_ROCM_DECODE_SEGMENTS_MAX counters, zero between operations */
     int status_dirty;       /* deferred mode: launches since the last check */
     yvex_rocm_completion_mode completion_mode;

@@ -126,6 +126,15 @@ typedef struct {
     double rope_frequency[YVEX_ROCM_ROPE_PAIRS_MAX];
 } yvex_rocm_decode_merge_params;
 
+/* Completion: one workgroup of 64 threads behind an operation's kernels.  Takes the status
+ * word (and clears it when set) and leaves (sequence << 32 | status) in a word of host memory,
+ * which the host is watching. */
+typedef struct {
+    int32_t *status;
+    uint64_t *mailbox;
+    uint32_t sequence;
+} yvex_rocm_status_forward_params;
+
 /* The element-wise operators the reference's decoder runs around attention on F32 activations
  * (src/runtime/decoder.c:989-997,1030-1046,1112-1131,1266-1269): one thread per element (per
  * rotated pair for the rotation), blocks of YVEX_ROCM_ELEMENTWISE_BLOCK threads.

@@ -84,3 +84,17 @@ yvex_rocm_split_interleaved_two_f32(const yvex_rocm_elementwise_params p)
     p.values[index] = p.left[at];
     p.second[index] = p.left[at + p.head_dim];
 }
+
+// Completion of an operation without a copy: the status word as the operation's kernels left
+// it (cleared here when set) goes, with the sequence number the host is waiting for, into a
+// word of host memory in one 8-byte store.  It runs behind those kernels on their stream, so
+// the host that sees the number knows they have ended.
+extern "C" __global__ void __launch_bounds__(64)
+yvex_rocm_status_forward(const yvex_rocm_status_forward_params p)
+{
+    if (threadIdx.x != 0u) return;
+    const int32_t status = __hip_atomic_load(p.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (status != 0) __hip_atomic_store(p.status, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(p.mailbox, ((uint64_t)p.sequence << 32) | (uint32_t)status, __ATOMIC_RELEASE,
+                       __HIP_MEMORY_SCOPE_SYSTEM);
+}

@@ -1,8 +1,9 @@
 /* A stand-in HIP runtime for host-logic tests on machines without a GPU.
  *
  * It implements exactly the entry points the backend binds (rocm_driver.h) with host
- * memory and no computation: kernel launches are counted and otherwise do nothing, so
- * nothing numerical can be tested (or accidentally served) through it.  It is loaded
+ * memory and no computation: kernel launches are counted and otherwise do nothing (but for
+ * the one-thread kernel that hands the status word to the host), so nothing numerical can be
+ * tested (or accidentally served) through it.  It is loaded
  * only when a test sets YVEX_TEST_ROCM_DRIVER_LIBRARY; it exists so admission,
  * bookkeeping, failure transitions and cleanup of the C host can run on the CPU, the
  * way the reference swaps entries of its driver table in tests/unit/cuda/graph.c:265-289.
@@ -15,13 +16,15 @@
 #include <string.h>
 #include <sys/mman.h>
 
-static unsigned long long launches, allocations, frees, loads, unloads;
+static unsigned long long launches, allocations, frees, loads, unloads, forwards;
 static int capturing;                       /* a stream capture is open */
 static unsigned long long captured_launches;
 
 static unsigned int last_grid_x;
 static unsigned char last_params[512];
 unsigned long long fake_hip_launches(void) { return launches; }
+/* status words handed to the host through its mailbox */
+unsigned long long fake_hip_status_forwards(void) { return forwards; }
 unsigned int fake_hip_last_grid_x(void) { return last_grid_x; }
 /* the bytes kept of the last launch's parameter struct */
 const unsigned char *fake_hip_last_params(void) { return last_params; }
@@ -113,6 +116,23 @@ hipError_t hipFree(void *ptr)
     return hipSuccess;
 }
 
+/* host memory the device can write: the stand-in's device is the host */
+hipError_t hipHostMalloc(void **ptr, size_t size, unsigned int flags)
+{
+    (void)flags;
+    if (env_is("FAKE_HIP_HOST_MALLOC", "fail")) return hipErrorOutOfMemory;
+    return hipMalloc(ptr, size);
+}
+
+hipError_t hipHostFree(void *ptr) { return hipFree(ptr); }
+
+hipError_t hipHostGetDevicePointer(void **device, void *host, unsigned int flags)
+{
+    (void)flags;
+    *device = host;
+    return hipSuccess;
+}
+
 hipError_t hipMemcpyAsync(void *dst, const void *src, size_t size, hipMemcpyKind kind,
                           hipStream_t stream)
 {
@@ -160,9 +180,19 @@ hipError_t hipModuleLaunchKernel(hipFunction_t f, unsigned int gx, unsigned int 
                                  unsigned int shared, hipStream_t stream, void **params,
                                  void **extra)
 {
-    (void)f; (void)gy; (void)gz; (void)bx; (void)by; (void)bz;
+    (void)gy; (void)gz; (void)bx; (void)by; (void)bz;
     (void)shared; (void)stream; (void)extra;
     if (env_is("FAKE_HIP_LAUNCH", "fail")) return hipErrorLaunchFailure;
+    if (f && strcmp((const char *)f, "yvex_rocm_status_forward") == 0 && params && params[0]) {
+        /* the one kernel the stand-in carries out: (sequence, status) into the host's mailbox,
+         * the status word cleared.  Not counted as a launch of the operation. */
+        struct { int32_t *status; uint64_t *mailbox; uint32_t sequence; } *p = params[0];
+        const int32_t status = *p->status;
+        *p->status = 0;
+        *p->mailbox = ((uint64_t)p->sequence << 32) | (uint32_t)status;
+        ++forwards;
+        return hipSuccess;
+    }
     /* the last launch's grid width and the head of its one by-value parameter, for tests that
      * look at what the host handed to a kernel */
     last_grid_x = gx;

@@ -1383,3 +1383,38 @@ def test_single_token_bf16_requests_take_the_team_kernels_at_every_head_dimensio
             assert (need > 0) == partials and facts.temporary_bytes == need, label
             for t in (q, out, k, v):
                 t.release()
+
+
+def test_status_word_reaches_the_host_through_the_mailbox_or_by_copy(env, fake_runtime):
+    """An operation that completes at once hands its status word to the host through a word of
+    host memory the device can write (one forward per completion, and per yvex_backend_sync in
+    deferred mode); a runtime that gives no such memory leaves the copy of the word, with the
+    same facts either way."""
+    fake_runtime.fake_hip_status_forwards.restype = C.c_ulonglong
+    facts_seen = []
+    for pinned in (True, False):
+        env("FAKE_HIP_HOST_MALLOC", None if pinned else "fail")
+        with Backend() as b:
+            x = written(b, "x", B.DTYPE_F32, (128,))
+            before = fake_runtime.fake_hip_status_forwards()
+            launches = fake_runtime.fake_hip_launches()
+            facts = b.bf16_round(x, 128)
+            assert fake_runtime.fake_hip_status_forwards() - before == (1 if pinned else 0)
+            assert fake_runtime.fake_hip_launches() - launches == 1      # the operation's own kernel
+            facts_seen.append((facts.kernel_launches, facts.device_synchronizations, facts.download_count,
+                               facts.d2h_bytes))
+            b.set_completion_mode(B.COMPLETION_DEFERRED)
+            for _ in range(5):
+                b.bf16_round(x, 128)
+            assert fake_runtime.fake_hip_status_forwards() - before == (1 if pinned else 0)
+            b.sync()
+            assert fake_runtime.fake_hip_status_forwards() - before == (2 if pinned else 0)
+            b.set_completion_mode(B.COMPLETION_IMMEDIATE)
+            env("FAKE_HIP_SYNC", "fail")                                  # the runtime's wait fails
+            env("YVEX_TEST_ROCM_SYNC_FAILURE", None)
+            if not pinned:
+                with pytest.raises(YvexError) as e:
+                    b.bf16_round(x, 128)
+                assert e.value.code == B.YVEX_ERR_BACKEND
+            env("FAKE_HIP_SYNC", None)
+    assert facts_seen[0] == facts_seen[1] == (1, 1, 1, 4)
