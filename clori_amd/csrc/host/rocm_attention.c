@@ -291,7 +291,7 @@ static int decode_run(yvex_backend *backend, const decode_job *job, const char *
         backend->status != YVEX_BACKEND_STATUS_FAILED)
         (void)state->driver.hipMemsetAsync(state->decode_arrivals, 0,
                                            YVEX_ROCM_DECODE_SEGMENTS_MAX * sizeof(uint32_t),
-                                           state->stream);
+                                           yvex_rocm_stream(state));
     yvex_error_clear(&cleanup);
     cleanup_rc = yvex_rocm_temporary_release(backend, work, total, owned, &cleanup);
     backend_workspace_reset(backend);
@@ -645,7 +645,7 @@ static int attention_execute_common(yvex_backend *backend,
             if (rc != YVEX_OK && !state->recording && backend->status != YVEX_BACKEND_STATUS_FAILED)
                 (void)state->driver.hipMemsetAsync(state->decode_arrivals, 0,
                                                    YVEX_ROCM_DECODE_SEGMENTS_MAX * sizeof(uint32_t),
-                                                   state->stream);
+                                                   yvex_rocm_stream(state));
         } else {
             split_runs = 0ull;
             rc = yvex_rocm_launch(backend, YVEX_ROCM_FN_GQA_F32,

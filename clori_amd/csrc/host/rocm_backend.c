@@ -60,7 +60,7 @@ static int rocm_tensor_alloc(yvex_backend *backend, const yvex_backend_tensor_de
         return YVEX_ERR_NOMEM;
     }
     rc = yvex_rocm_status(&state->driver,
-                          state->driver.hipMemsetAsync(ptr, 0, (size_t)desc->bytes, state->stream),
+                          state->driver.hipMemsetAsync(ptr, 0, (size_t)desc->bytes, yvex_rocm_stream(state)),
                           where, err);
     if (rc == YVEX_OK)
         rc = yvex_rocm_synchronize(backend, YVEX_BACKEND_VARIANT_TENSOR_ZERO,
@@ -114,7 +114,7 @@ static int rocm_tensor_free(yvex_backend *backend, yvex_device_tensor *tensor, y
     }
     if (backend->workspace_device_tensor == tensor) yvex_backend_workspace_detach(backend);
     /* nothing may still read the allocation: drain the stream first */
-    rc = yvex_rocm_status(&state->driver, state->driver.hipStreamSynchronize(state->stream), where,
+    rc = yvex_rocm_status(&state->driver, state->driver.hipStreamSynchronize(yvex_rocm_stream(state)), where,
                           err);
     if (rc == YVEX_OK && getenv("YVEX_TEST_ROCM_CLEANUP_FAILURE"))
         rc = refuse(err, YVEX_ERR_BACKEND, where, "injected ROCm tensor cleanup failure");
@@ -147,7 +147,7 @@ static int rocm_copy(yvex_backend *backend, void *dst, const void *src, unsigned
     int rc = yvex_rocm_require_capability(backend, variant, where, err);
     if (rc != YVEX_OK) return rc;
     rc = yvex_rocm_status(&state->driver,
-                          state->driver.hipMemcpyAsync(dst, src, (size_t)bytes, kind, state->stream),
+                          state->driver.hipMemcpyAsync(dst, src, (size_t)bytes, kind, yvex_rocm_stream(state)),
                           where, err);
     if (rc == YVEX_OK) rc = yvex_rocm_synchronize(backend, variant, where, err);
     return rc;
@@ -196,7 +196,7 @@ static int rocm_tensor_zero(yvex_backend *backend, yvex_device_tensor *tensor, y
     if (rc != YVEX_OK) return rc;
     rc = yvex_rocm_status(&state->driver,
                           state->driver.hipMemsetAsync(tensor->data, 0, (size_t)tensor->bytes,
-                                                       state->stream),
+                                                       yvex_rocm_stream(state)),
                           where, err);
     if (rc == YVEX_OK) rc = yvex_rocm_synchronize(backend, YVEX_BACKEND_VARIANT_TENSOR_ZERO, where, err);
     if (rc != YVEX_OK) return rc;
@@ -223,6 +223,72 @@ static int rocm_tensor_copy(yvex_backend *backend, yvex_device_tensor *dst,
 
 /* src/backend/cuda/backend.c:1159-1191: the copy goes on the launch stream and is not waited
  * for; whatever is enqueued behind it sees the bytes. */
+/* ---- queued copies ----------------------------------------------------------------------
+ * The reference's session layer appends every new token to a layer's history with two
+ * asynchronous copies of one row each (src/runtime/stateful_attention.c:183-222): 4096 calls
+ * for a prompt of 2048 tokens, each a launch of its own if handed to the runtime one by one.
+ * Small copies wait in a queue instead and leave together, one launch per
+ * YVEX_ROCM_COPY_BATCH_MAX of them, as soon as anything else is asked of the stream
+ * (yvex_rocm_stream): the order the caller sees is the stream's order.  The copies of one
+ * launch run side by side, so one that touches what a queued one writes, or writes what a
+ * queued one reads, sends the queue off first. */
+enum { ROCM_COPY_QUEUE_BYTES_MAX = 256 * 1024, ROCM_COPY_PIECE_BYTES = 256 * 16 };
+
+void yvex_rocm_copy_queue_flush(yvex_rocm_backend_state *state)
+{
+    const uint32_t count = state->copy_queue.count;
+    void *arguments[1] = {&state->copy_queue.params};
+    unsigned int columns = (state->copy_queue.largest + ROCM_COPY_PIECE_BYTES - 1u) / ROCM_COPY_PIECE_BYTES;
+    uint32_t i;
+    if (!count) return;
+    state->copy_queue.count = 0u; /* first: the stream is taken below without another flush */
+    state->copy_queue.largest = 0u;
+    if (columns > 16u) columns = 16u;
+    if (state->functions[YVEX_ROCM_FN_COPY_BATCH] &&
+        state->driver.hipModuleLaunchKernel(state->functions[YVEX_ROCM_FN_COPY_BATCH], columns, count, 1u,
+                                            256u, 1u, 1u, 0u, state->stream_handle, arguments,
+                                            NULL) == hipSuccess)
+        return;
+    /* the launch was refused: the copies one by one; what still fails is reported by the next wait */
+    for (i = 0u; i < count; ++i)
+        if (state->driver.hipMemcpyAsync((void *)(uintptr_t)state->copy_queue.params.dst[i],
+                                         (const void *)(uintptr_t)state->copy_queue.params.src[i],
+                                         state->copy_queue.params.bytes[i], hipMemcpyDeviceToDevice,
+                                         state->stream_handle) != hipSuccess)
+            state->copy_queue.failed = 1;
+}
+
+static int ranges_meet(uint64_t a, uint64_t a_bytes, uint64_t b, uint64_t b_bytes)
+{
+    return a < b + b_bytes && b < a + a_bytes;
+}
+
+/* 1 when the copy was queued, 0 when it is for the runtime (large, not in 16-byte pieces, or
+ * no kernel to carry it). */
+static int copy_queue_take(yvex_rocm_backend_state *state, const void *dst, const void *src,
+                           unsigned long long bytes)
+{
+    yvex_rocm_copy_batch_params *q = &state->copy_queue.params;
+    const uint64_t to = (uint64_t)(uintptr_t)dst, from = (uint64_t)(uintptr_t)src;
+    uint32_t i;
+    if (!state->functions[YVEX_ROCM_FN_COPY_BATCH] || !bytes || bytes > ROCM_COPY_QUEUE_BYTES_MAX ||
+        ((to | from | bytes) & 15ull))
+        return 0;
+    for (i = 0u; i < state->copy_queue.count; ++i)
+        if (ranges_meet(to, bytes, q->dst[i], q->bytes[i]) || ranges_meet(to, bytes, q->src[i], q->bytes[i]) ||
+            ranges_meet(from, bytes, q->dst[i], q->bytes[i])) {
+            yvex_rocm_copy_queue_flush(state);
+            break;
+        }
+    if (state->copy_queue.count == YVEX_ROCM_COPY_BATCH_MAX) yvex_rocm_copy_queue_flush(state);
+    i = state->copy_queue.count++;
+    q->dst[i] = to;
+    q->src[i] = from;
+    q->bytes[i] = (uint32_t)bytes;
+    if ((uint32_t)bytes > state->copy_queue.largest) state->copy_queue.largest = (uint32_t)bytes;
+    return 1;
+}
+
 static int rocm_tensor_copy_async(yvex_backend *backend, yvex_device_tensor *dst,
                                   const yvex_device_tensor *src, yvex_error *err)
 {
@@ -236,10 +302,11 @@ static int rocm_tensor_copy_async(yvex_backend *backend, yvex_device_tensor *dst
         return refuse(err, YVEX_ERR_STATE, where, kUnbacked);
     rc = yvex_rocm_require_capability(backend, YVEX_BACKEND_VARIANT_TENSOR_COPY, where, err);
     if (rc != YVEX_OK) return rc;
-    rc = yvex_rocm_status(&state->driver,
-                          state->driver.hipMemcpyAsync(dst->data, src->data, (size_t)src->bytes,
-                                                       hipMemcpyDeviceToDevice, state->stream),
-                          where, err);
+    if (!copy_queue_take(state, dst->data, src->data, src->bytes))
+        rc = yvex_rocm_status(&state->driver,
+                              state->driver.hipMemcpyAsync(dst->data, src->data, (size_t)src->bytes,
+                                                           hipMemcpyDeviceToDevice, yvex_rocm_stream(state)),
+                              where, err);
     if (rc != YVEX_OK) return rc;
     dst->is_written = src->is_written;
     yvex_error_clear(err);
@@ -259,32 +326,32 @@ static int rocm_tensor_copy_shared_async(yvex_backend *backend, yvex_device_tens
     yvex_rocm_backend_state *source_state = src && src->owner ? yvex_rocm_state(src->owner) : NULL;
     hipEvent_t ready = NULL, consumed = NULL;
     int rc = YVEX_OK, cleanup;
-    if (!state || !source_state || !dst || !state->stream || !source_state->stream)
+    if (!state || !source_state || !dst || !state->stream_handle || !source_state->stream_handle)
         return refuse(err, YVEX_ERR_UNSUPPORTED, where, "ROCm cross-stream event ordering is unavailable");
     if (!yvex_rocm_tensor_backed(dst) || !yvex_rocm_tensor_backed(src))
         return refuse(err, YVEX_ERR_STATE, where, kUnbacked);
-    if (source_state->stream != state->stream) {
+    if (source_state->stream_handle != state->stream_handle) {
         rc = yvex_rocm_status(&state->driver, state->driver.hipEventCreate(&ready), where, err);
         if (rc == YVEX_OK)
             rc = yvex_rocm_status(&state->driver, state->driver.hipEventCreate(&consumed), where, err);
         if (rc == YVEX_OK)
             rc = yvex_rocm_status(&state->driver,
-                                  state->driver.hipEventRecord(ready, source_state->stream), where, err);
+                                  state->driver.hipEventRecord(ready, yvex_rocm_stream(source_state)), where, err);
         if (rc == YVEX_OK)
             rc = yvex_rocm_status(&state->driver,
-                                  state->driver.hipStreamWaitEvent(state->stream, ready, 0u), where, err);
+                                  state->driver.hipStreamWaitEvent(yvex_rocm_stream(state), ready, 0u), where, err);
     }
     if (rc == YVEX_OK)
         rc = yvex_rocm_status(&state->driver,
                               state->driver.hipMemcpyAsync(dst->data, src->data, (size_t)src->bytes,
-                                                           hipMemcpyDeviceToDevice, state->stream),
+                                                           hipMemcpyDeviceToDevice, yvex_rocm_stream(state)),
                               where, err);
     if (rc == YVEX_OK && consumed) {
-        rc = yvex_rocm_status(&state->driver, state->driver.hipEventRecord(consumed, state->stream),
+        rc = yvex_rocm_status(&state->driver, state->driver.hipEventRecord(consumed, yvex_rocm_stream(state)),
                               where, err);
         if (rc == YVEX_OK)
             rc = yvex_rocm_status(&state->driver,
-                                  state->driver.hipStreamWaitEvent(source_state->stream, consumed, 0u),
+                                  state->driver.hipStreamWaitEvent(yvex_rocm_stream(source_state), consumed, 0u),
                                   where, err);
     }
     if (consumed) {
@@ -354,7 +421,7 @@ static int bandwidth_sample(yvex_backend *backend, yvex_device_tensor *source,
                                   state->driver.hipMemcpyAsync(copy->data, source->data,
                                                                (size_t)source->bytes,
                                                                hipMemcpyDeviceToDevice,
-                                                               state->stream),
+                                                               yvex_rocm_stream(state)),
                                   where, err);
         else
             rc = yvex_rocm_launch(backend, YVEX_ROCM_FN_STREAM_READ,
@@ -455,7 +522,7 @@ static int rocm_device_info(const yvex_backend *backend, yvex_backend_device_inf
     yvex_rocm_backend_state *state = yvex_rocm_state(backend);
     size_t free_bytes = 0u, total_bytes = 0u;
     *out = backend->device_info;
-    if (state && state->stream &&
+    if (state && state->stream_handle &&
         state->driver.hipMemGetInfo(&free_bytes, &total_bytes) == hipSuccess) {
         out->free_memory_bytes = free_bytes;
         out->total_memory_bytes = total_bytes;
@@ -507,7 +574,7 @@ int yvex_rocm_temporary_release(yvex_backend *backend, void *address, unsigned l
     yvex_rocm_backend_state *state = yvex_rocm_state(backend);
     int rc;
     if (!owned || !address) return YVEX_OK;
-    rc = yvex_rocm_status(&state->driver, state->driver.hipStreamSynchronize(state->stream),
+    rc = yvex_rocm_status(&state->driver, state->driver.hipStreamSynchronize(yvex_rocm_stream(state)),
                           "rocm.temporary.release", err);
     if (rc == YVEX_OK)
         rc = yvex_rocm_status(&state->driver, state->driver.hipFree(address),
@@ -533,11 +600,11 @@ static int rocm_close(yvex_backend *backend, yvex_error *err)
     }
     if (state->recording) { /* an abandoned recording: end it and drop what it held */
         hipGraph_t dropped = NULL;
-        (void)state->driver.hipStreamEndCapture(state->stream, &dropped);
+        (void)state->driver.hipStreamEndCapture(yvex_rocm_stream(state), &dropped);
         if (dropped) (void)state->driver.hipGraphDestroy(dropped);
         state->recording = 0;
     }
-    if (state->stream) (void)state->driver.hipStreamSynchronize(state->stream);
+    if (state->stream_handle) (void)state->driver.hipStreamSynchronize(yvex_rocm_stream(state));
     rc = yvex_rocm_kernel_bundle_close(backend, err);
     if (rc != YVEX_OK) return rc; /* impl retained: checked close can be retried */
     if (state->device_status) (void)state->driver.hipFree(state->device_status);
@@ -547,7 +614,7 @@ static int rocm_close(yvex_backend *backend, yvex_error *err)
     probe_release(state);
     if (state->timing_start) (void)state->driver.hipEventDestroy(state->timing_start);
     if (state->timing_stop) (void)state->driver.hipEventDestroy(state->timing_stop);
-    if (state->stream) (void)state->driver.hipStreamDestroy(state->stream);
+    if (state->stream_handle) (void)state->driver.hipStreamDestroy(state->stream_handle);
     yvex_rocm_driver_unload(&state->driver);
     free(state);
     backend->impl = NULL;
@@ -672,7 +739,7 @@ static int rocm_open(yvex_backend **out, const char *device, unsigned long long 
         rc = yvex_rocm_status(&state->driver, state->driver.hipSetDevice(state->device_index),
                               where, err);
     if (rc == YVEX_OK)
-        rc = yvex_rocm_status(&state->driver, state->driver.hipStreamCreate(&state->stream), where,
+        rc = yvex_rocm_status(&state->driver, state->driver.hipStreamCreate(&state->stream_handle), where,
                               err);
     if (rc == YVEX_OK)
         rc = yvex_rocm_status(&state->driver, state->driver.hipEventCreate(&state->timing_start),
@@ -687,7 +754,7 @@ static int rocm_open(yvex_backend **out, const char *device, unsigned long long 
     if (rc == YVEX_OK)
         rc = yvex_rocm_status(&state->driver,
                               state->driver.hipMemsetAsync(state->device_status, 0, 256u,
-                                                           state->stream),
+                                                           yvex_rocm_stream(state)),
                               where, err);
     if (rc == YVEX_OK && state->driver.pinned_memory) {
         /* the status mailbox is an economy, not a requirement: without it the word is copied */
@@ -711,7 +778,7 @@ static int rocm_open(yvex_backend **out, const char *device, unsigned long long 
         rc = yvex_rocm_status(&state->driver,
                               state->driver.hipMemsetAsync(state->decode_arrivals, 0,
                                                            YVEX_ROCM_DECODE_SEGMENTS_MAX * sizeof(uint32_t),
-                                                           state->stream),
+                                                           yvex_rocm_stream(state)),
                               where, err);
     if (rc == YVEX_OK)
         rc = yvex_rocm_status(&state->driver,
@@ -719,7 +786,7 @@ static int rocm_open(yvex_backend **out, const char *device, unsigned long long 
                                                       sizeof(state->schedule.rows)),
                               where, err);
     if (rc == YVEX_OK)
-        rc = yvex_rocm_status(&state->driver, state->driver.hipStreamSynchronize(state->stream),
+        rc = yvex_rocm_status(&state->driver, state->driver.hipStreamSynchronize(yvex_rocm_stream(state)),
                               where, err);
     if (rc != YVEX_OK) {
         yvex_error keep = err ? *err : (yvex_error){0};
@@ -730,7 +797,7 @@ static int rocm_open(yvex_backend **out, const char *device, unsigned long long 
         if (state->schedule_device) (void)state->driver.hipFree(state->schedule_device);
         if (state->timing_start) (void)state->driver.hipEventDestroy(state->timing_start);
         if (state->timing_stop) (void)state->driver.hipEventDestroy(state->timing_stop);
-        if (state->stream) (void)state->driver.hipStreamDestroy(state->stream);
+        if (state->stream_handle) (void)state->driver.hipStreamDestroy(state->stream_handle);
         (void)scratch;
         free(state);
         free(backend);
@@ -921,7 +988,7 @@ int yvex_backend_rocm_timing_begin(yvex_backend *backend, yvex_error *err)
         return refuse(err, YVEX_ERR_STATE, "rocm.timing",
                       "not available while a launch sequence is being recorded");
     rc = yvex_rocm_status(&state->driver,
-                          state->driver.hipEventRecord(state->timing_start, state->stream),
+                          state->driver.hipEventRecord(state->timing_start, yvex_rocm_stream(state)),
                           "rocm.timing.begin", err);
     if (rc == YVEX_OK) state->timing_active = 1;
     return rc;
@@ -936,7 +1003,7 @@ int yvex_backend_rocm_timing_end(yvex_backend *backend, double *milliseconds, yv
         return refuse(err, YVEX_ERR_STATE, "rocm.timing.end",
                       "timing was not started, or a launch sequence is being recorded");
     rc = yvex_rocm_status(&state->driver,
-                          state->driver.hipEventRecord(state->timing_stop, state->stream),
+                          state->driver.hipEventRecord(state->timing_stop, yvex_rocm_stream(state)),
                           "rocm.timing.end", err);
     if (rc == YVEX_OK)
         rc = yvex_rocm_status(&state->driver, state->driver.hipEventSynchronize(state->timing_stop),
@@ -975,7 +1042,7 @@ int yvex_backend_rocm_graph_begin(yvex_backend *backend, yvex_error *err)
         if (rc != YVEX_OK) return rc;
     }
     rc = yvex_rocm_status(&state->driver,
-                          state->driver.hipStreamBeginCapture(state->stream,
+                          state->driver.hipStreamBeginCapture(yvex_rocm_stream(state),
                                                               hipStreamCaptureModeThreadLocal),
                           where, err);
     if (rc != YVEX_OK) return rc;
@@ -995,7 +1062,7 @@ int yvex_backend_rocm_graph_end(yvex_backend *backend, yvex_rocm_graph **out, yv
     if (out) *out = NULL;
     if (!state || !out) return refuse(err, YVEX_ERR_INVALID_ARG, where, "backend and out are required");
     if (!state->recording) return refuse(err, YVEX_ERR_STATE, where, "no launch sequence is being recorded");
-    rc = yvex_rocm_status(&state->driver, state->driver.hipStreamEndCapture(state->stream, &captured),
+    rc = yvex_rocm_status(&state->driver, state->driver.hipStreamEndCapture(yvex_rocm_stream(state), &captured),
                           where, err);
     state->recording = 0;
     if (rc != YVEX_OK) {
@@ -1047,7 +1114,7 @@ int yvex_backend_rocm_graph_launch(yvex_backend *backend, yvex_rocm_graph *graph
         return refuse(err, YVEX_ERR_STATE, where,
                       "the workspace attached when the sequence was recorded is no longer attached");
     if (facts) memset(facts, 0, sizeof(*facts));
-    rc = yvex_rocm_status(&state->driver, state->driver.hipGraphLaunch(graph->executable, state->stream),
+    rc = yvex_rocm_status(&state->driver, state->driver.hipGraphLaunch(graph->executable, yvex_rocm_stream(state)),
                           where, err);
     if (rc != YVEX_OK) {
         state->backend_failure_reason = YVEX_BACKEND_CAPABILITY_REASON_LAUNCH_FAILED;
@@ -1074,7 +1141,7 @@ int yvex_backend_rocm_graph_release(yvex_backend *backend, yvex_rocm_graph **gra
     if (state->recording)
         return refuse(err, YVEX_ERR_STATE, where, "a launch sequence is being recorded");
     /* a replay may still be running */
-    rc = yvex_rocm_status(&state->driver, state->driver.hipStreamSynchronize(state->stream), where, err);
+    rc = yvex_rocm_status(&state->driver, state->driver.hipStreamSynchronize(yvex_rocm_stream(state)), where, err);
     if (rc != YVEX_OK) return rc;
     {
         yvex_rocm_graph **link = &state->graphs;
@@ -1101,7 +1168,7 @@ int yvex_backend_rocm_report_get(const yvex_backend *backend, yvex_backend_rocm_
         return refuse(err, YVEX_ERR_INVALID_ARG, "rocm.report", "ROCm backend and out are required");
     memset(out, 0, sizeof(*out));
     out->driver_loaded = state->driver.library != NULL;
-    out->device_ready = state->stream != NULL;
+    out->device_ready = state->stream_handle != NULL;
     out->bundle_built = yvex_rocm_bundle_image_count() != 0u;
     out->bundle_admitted = state->kernel_bundle_state == YVEX_ROCM_KERNEL_BUNDLE_ADMITTED;
     out->image_count = yvex_rocm_bundle_image_count();

@@ -98,6 +98,7 @@ static const rocm_kernel_binding rocm_kernel_bindings[] = {
      YVEX_ROCM_FN_DECODE_ROWS_BF16_TEAM_256},
     {"yvex_rocm_status_forward", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_F32,
      YVEX_ROCM_FN_STATUS_FORWARD},
+    {"yvex_rocm_copy_batch", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_F32, YVEX_ROCM_FN_COPY_BATCH},
     {"yvex_rocm_gather_rows", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_MLA_BF16, YVEX_ROCM_FN_GATHER_ROWS},
     {"yvex_rocm_kv_append_bf16", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_PAGED_BF16,
      YVEX_ROCM_FN_KV_APPEND_BF16},
@@ -162,7 +163,7 @@ int yvex_rocm_kernel_bundle_admit(yvex_backend *backend, yvex_error *err)
     unsigned int loaded = 0u, index;
     size_t b;
     int rc = YVEX_OK;
-    if (!backend || !state || !state->stream) {
+    if (!backend || !state || !state->stream_handle) {
         yvex_error_set(err, YVEX_ERR_STATE, "rocm.kernels.admit",
                        "ROCm context is required for kernel admission");
         return YVEX_ERR_STATE;
@@ -327,9 +328,9 @@ int yvex_rocm_query_capability(const yvex_backend *backend, yvex_backend_operati
                        "backend, ROCm state, and out are required");
         return YVEX_ERR_INVALID_ARG;
     }
-    out->context_available = state->stream != NULL;
+    out->context_available = state->stream_handle != NULL;
     out->kernel_bundle_available = state->kernel_bundle_state == YVEX_ROCM_KERNEL_BUNDLE_ADMITTED;
-    if (!state->stream)
+    if (!state->stream_handle)
         return publish(out, YVEX_BACKEND_CAPABILITY_UNSUPPORTED,
                        YVEX_BACKEND_CAPABILITY_REASON_CONTEXT_UNAVAILABLE, 0, err);
     if (backend->status == YVEX_BACKEND_STATUS_FAILED &&
@@ -429,7 +430,7 @@ int yvex_rocm_launch(yvex_backend *backend, yvex_rocm_function_id function,
         rc = yvex_rocm_status(&state->driver,
                               state->driver.timed_launch(state->functions[function], grid_x * block,
                                                          grid_y, grid_z, block, 1u, 1u, lds_bytes,
-                                                         state->stream, arguments, NULL,
+                                                         yvex_rocm_stream(state), arguments, NULL,
                                                          state->probe_events[2u * state->probe_count],
                                                          state->probe_events[2u * state->probe_count + 1u],
                                                          0u),
@@ -438,21 +439,31 @@ int yvex_rocm_launch(yvex_backend *backend, yvex_rocm_function_id function,
     } else {
         if (probe)
             probe = state->driver.hipEventRecord(state->probe_events[2u * state->probe_count],
-                                                 state->stream) == hipSuccess;
+                                                 yvex_rocm_stream(state)) == hipSuccess;
         rc = yvex_rocm_status(&state->driver,
                               state->driver.hipModuleLaunchKernel(state->functions[function], grid_x,
                                                                   grid_y, grid_z, block, 1u, 1u,
-                                                                  lds_bytes, state->stream, arguments,
+                                                                  lds_bytes, yvex_rocm_stream(state), arguments,
                                                                   NULL),
                               where, err);
         if (probe && rc == YVEX_OK &&
             state->driver.hipEventRecord(state->probe_events[2u * state->probe_count + 1u],
-                                         state->stream) == hipSuccess)
+                                         yvex_rocm_stream(state)) == hipSuccess)
             state->probe_count++;
     }
     if (rc != YVEX_OK) capability_fail(backend, variant, YVEX_BACKEND_CAPABILITY_REASON_LAUNCH_FAILED);
     else if (state->recording) state->recorded_launches++;
     return rc;
+}
+
+/* A queued copy that neither the batch launch nor the runtime took: the stream's contents are
+ * not what the caller asked for, which fails the backend like a wait that failed. */
+static int refuse_copy_queue(yvex_backend *backend, const char *where, yvex_error *err)
+{
+    capability_fail(backend, YVEX_BACKEND_VARIANT_TENSOR_COPY,
+                    YVEX_BACKEND_CAPABILITY_REASON_SYNCHRONIZATION_FAILED);
+    yvex_error_set(err, YVEX_ERR_BACKEND, where, "a queued device-to-device copy could not be issued");
+    return YVEX_ERR_BACKEND;
 }
 
 /* src/backend/cuda/capability.c:793-830 */
@@ -476,8 +487,9 @@ int yvex_rocm_synchronize(yvex_backend *backend, yvex_backend_operation_variant 
         yvex_error_set(err, YVEX_ERR_BACKEND, where, "injected ROCm synchronization failure");
         return YVEX_ERR_BACKEND;
     }
-    rc = yvex_rocm_status(&state->driver, state->driver.hipStreamSynchronize(state->stream), where,
+    rc = yvex_rocm_status(&state->driver, state->driver.hipStreamSynchronize(yvex_rocm_stream(state)), where,
                           err);
+    if (rc == YVEX_OK && state->copy_queue.failed) return refuse_copy_queue(backend, where, err);
     if (rc != YVEX_OK)
         capability_fail(backend, variant, YVEX_BACKEND_CAPABILITY_REASON_SYNCHRONIZATION_FAILED);
     return rc;
@@ -518,7 +530,7 @@ static int status_by_mailbox(yvex_backend *backend, const char *where, int32_t *
     rc = yvex_rocm_status(&state->driver,
                           state->driver.hipModuleLaunchKernel(
                               state->functions[YVEX_ROCM_FN_STATUS_FORWARD], 1u, 1u, 1u, 64u, 1u, 1u, 0u,
-                              state->stream, arguments, NULL),
+                              yvex_rocm_stream(state), arguments, NULL),
                           where, err);
     if (rc != YVEX_OK) return rc;
     deadline = monotonic_ns() + ROCM_MAILBOX_SPIN_NS;
@@ -566,11 +578,13 @@ int yvex_rocm_status_check(yvex_backend *backend, const char *where,
         rc = yvex_rocm_status(&state->driver,
                               state->driver.hipMemcpyAsync(&host_status, state->device_status,
                                                            sizeof(host_status), hipMemcpyDeviceToHost,
-                                                           state->stream),
+                                                           yvex_rocm_stream(state)),
                               where, err);
         if (rc == YVEX_OK)
             rc = yvex_rocm_synchronize(backend, YVEX_BACKEND_VARIANT_TENSOR_READ, where, err);
     }
+    if (rc == YVEX_OK && state->copy_queue.failed)
+        rc = refuse_copy_queue(backend, where, err);
     if (rc != YVEX_OK) return rc;
     state->status_dirty = 0;
     backend->stats.d2h_bytes += sizeof(host_status);
@@ -586,7 +600,7 @@ int yvex_rocm_status_check(yvex_backend *backend, const char *where,
     if (!cleared) {
         rc = yvex_rocm_status(&state->driver,
                               state->driver.hipMemsetAsync(state->device_status, 0,
-                                                           sizeof(host_status), state->stream),
+                                                           sizeof(host_status), yvex_rocm_stream(state)),
                               where, err);
         if (rc != YVEX_OK) return rc;
     }

@@ -196,11 +196,11 @@ unsigned int yvex_rocm_schedule_lists(yvex_backend *backend, const yvex_rocm_sch
         if (state->schedule.seen != 1u || state->recording) return 0u;
         state->schedule.seen = 2u;
         if (!lists_build(state, key, (unsigned int)q_tiles, units) ||
-            state->driver.hipStreamSynchronize(state->stream) != hipSuccess ||
+            state->driver.hipStreamSynchronize(yvex_rocm_stream(state)) != hipSuccess ||
             state->driver.hipMemcpyAsync(state->schedule_device, state->schedule.rows,
                                          (size_t)lists * YVEX_ROCM_LIST_STRIDE * sizeof(uint16_t),
-                                         hipMemcpyHostToDevice, state->stream) != hipSuccess ||
-            state->driver.hipStreamSynchronize(state->stream) != hipSuccess)
+                                         hipMemcpyHostToDevice, yvex_rocm_stream(state)) != hipSuccess ||
+            state->driver.hipStreamSynchronize(yvex_rocm_stream(state)) != hipSuccess)
             return 0u;
         backend->stats.h2d_bytes += (unsigned long long)lists * YVEX_ROCM_LIST_STRIDE * sizeof(uint16_t);
         state->schedule.lists = lists;

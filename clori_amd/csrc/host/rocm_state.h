@@ -4,6 +4,7 @@
 
 #include "private.h"
 #include "rocm_driver.h"
+#include "../kernel_params.h"
 
 #define YVEX_ROCM_MODULE_MAX 8u
 
@@ -50,6 +51,7 @@ typedef enum {
     YVEX_ROCM_FN_SIGMOID_PRODUCT_BF16_F32,
     YVEX_ROCM_FN_SPLIT_INTERLEAVED_TWO_F32,
     YVEX_ROCM_FN_STATUS_FORWARD,
+    YVEX_ROCM_FN_COPY_BATCH,
     YVEX_ROCM_FN_GATHER_ROWS,
     YVEX_ROCM_FN_COUNT
 } yvex_rocm_function_id;
@@ -82,7 +84,14 @@ typedef struct yvex_rocm_backend_state {
     yvex_rocm_driver driver;
     int device_index;
     int compute_units;
-    hipStream_t stream;
+    hipStream_t stream_handle; /* work goes through yvex_rocm_stream(), which orders it behind queued copies */
+    /* small asynchronous device-to-device copies wait here to leave as one launch: the
+     * kernel's parameter block, how many entries it holds and the largest of them */
+    struct {
+        yvex_rocm_copy_batch_params params;
+        uint32_t count, largest;
+        int failed; /* a queued copy could not be issued: reported by the next wait */
+    } copy_queue;
     hipEvent_t timing_start, timing_stop;
     int timing_active;
     /* per-kernel probe: event pairs around launches of one function */
@@ -160,6 +169,18 @@ static inline yvex_rocm_backend_state *yvex_rocm_state(const yvex_backend *backe
     return backend && backend->kind == YVEX_BACKEND_KIND_ROCM
                ? (yvex_rocm_backend_state *)backend->impl
                : NULL;
+}
+
+/* Launches what the copy queue holds (rocm_backend.c). */
+void yvex_rocm_copy_queue_flush(yvex_rocm_backend_state *state);
+
+/* The backend's stream, for work that is ordered behind everything asked for so far: copies
+ * that are still queued are launched first.  Every submission and every wait takes the stream
+ * from here. */
+static inline hipStream_t yvex_rocm_stream(yvex_rocm_backend_state *state)
+{
+    if (state->copy_queue.count) yvex_rocm_copy_queue_flush(state);
+    return state->stream_handle;
 }
 
 /* rocm_capability.c */

@@ -303,7 +303,7 @@ int yvex_rocm_tensor_commit(yvex_backend *backend, yvex_device_tensor *tensor,
         if (rc == YVEX_OK)
             rc = yvex_rocm_status(&state->driver,
                                   state->driver.hipMemsetAsync(address, 0, range->granularity,
-                                                               state->stream),
+                                                               yvex_rocm_stream(state)),
                                   "rocm.tensor.commit.zero", err);
     }
     if (rc == YVEX_OK)
@@ -315,7 +315,7 @@ int yvex_rocm_tensor_commit(yvex_backend *backend, yvex_device_tensor *tensor,
         yvex_error_clear(&primary);
         if (err) primary = *err;
         /* the clears of this call may still be in flight */
-        (void)state->driver.hipStreamSynchronize(state->stream);
+        (void)state->driver.hipStreamSynchronize(yvex_rocm_stream(state));
         while (added && undone == YVEX_OK) {
             yvex_error_clear(&cleanup);
             undone = granule_release(backend, range, fresh[--added], &cleanup);
@@ -362,7 +362,7 @@ int yvex_rocm_tensor_decommit(yvex_backend *backend, yvex_device_tensor *tensor,
                       "a recorded launch sequence may still name this tensor: release the "
                       "sequence first");
     /* nothing may still read the pages: drain the stream first */
-    rc = yvex_rocm_status(&state->driver, state->driver.hipStreamSynchronize(state->stream), where,
+    rc = yvex_rocm_status(&state->driver, state->driver.hipStreamSynchronize(yvex_rocm_stream(state)), where,
                           err);
     for (granule = 0u; rc == YVEX_OK && granule < range->granule_count; ++granule)
         if (range->state[granule]) {

@@ -126,6 +126,17 @@ typedef struct {
     double rope_frequency[YVEX_ROCM_ROPE_PAIRS_MAX];
 } yvex_rocm_decode_merge_params;
 
+/* A batch of small device-to-device copies in one launch: the reference's session layer
+ * appends every new token to a layer's history with two asynchronous copies
+ * (src/runtime/stateful_attention.c:183-222), 4096 of them for a prompt of 2048 tokens.
+ * grid = (pieces, count): workgroup (x, y) copies 16-byte pieces x * 256 + thread,
+ * + gridDim.x * 256, ... of copy y; addresses and sizes are multiples of 16 bytes. */
+#define YVEX_ROCM_COPY_BATCH_MAX 128
+typedef struct {
+    uint64_t dst[YVEX_ROCM_COPY_BATCH_MAX], src[YVEX_ROCM_COPY_BATCH_MAX];
+    uint32_t bytes[YVEX_ROCM_COPY_BATCH_MAX];
+} yvex_rocm_copy_batch_params;
+
 /* Completion: one workgroup of 64 threads behind an operation's kernels.  Takes the status
  * word (and clears it when set) and leaves (sequence << 32 | status) in a word of host memory,
  * which the host is watching. */

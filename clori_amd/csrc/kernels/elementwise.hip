@@ -98,3 +98,14 @@ yvex_rocm_status_forward(const yvex_rocm_status_forward_params p)
     __hip_atomic_store(p.mailbox, ((uint64_t)p.sequence << 32) | (uint32_t)status, __ATOMIC_RELEASE,
                        __HIP_MEMORY_SCOPE_SYSTEM);
 }
+
+// Small device-to-device copies queued by the host, one workgroup column per copy.
+extern "C" __global__ void __launch_bounds__(256)
+yvex_rocm_copy_batch(const yvex_rocm_copy_batch_params p)
+{
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    const uint32_t copy = blockIdx.y, pieces = p.bytes[copy] / 16u;
+    const u32x4 *src = reinterpret_cast<const u32x4 *>(p.src[copy]);
+    u32x4 *dst = reinterpret_cast<u32x4 *>(p.dst[copy]);
+    for (uint32_t i = blockIdx.x * 256u + threadIdx.x; i < pieces; i += gridDim.x * 256u) dst[i] = src[i];
+}

@@ -2,8 +2,8 @@
  *
  * It implements exactly the entry points the backend binds (rocm_driver.h) with host
  * memory and no computation: kernel launches are counted and otherwise do nothing (but for
- * the one-thread kernel that hands the status word to the host), so nothing numerical can be
- * tested (or accidentally served) through it.  It is loaded
+ * the one-thread kernel that hands the status word to the host and the batch of queued
+ * copies), so nothing numerical can be tested (or accidentally served) through it.  It is loaded
  * only when a test sets YVEX_TEST_ROCM_DRIVER_LIBRARY; it exists so admission,
  * bookkeeping, failure transitions and cleanup of the C host can run on the CPU, the
  * way the reference swaps entries of its driver table in tests/unit/cuda/graph.c:265-289.
@@ -16,13 +16,16 @@
 #include <string.h>
 #include <sys/mman.h>
 
-static unsigned long long launches, allocations, frees, loads, unloads, forwards;
+static unsigned long long launches, allocations, frees, loads, unloads, forwards, copy_batches, async_copies;
 static int capturing;                       /* a stream capture is open */
 static unsigned long long captured_launches;
 
 static unsigned int last_grid_x;
 static unsigned char last_params[512];
 unsigned long long fake_hip_launches(void) { return launches; }
+/* launches that carried a batch of queued copies, and copies handed to the runtime one by one */
+unsigned long long fake_hip_copy_batches(void) { return copy_batches; }
+unsigned long long fake_hip_device_copies(void) { return async_copies; }
 /* status words handed to the host through its mailbox */
 unsigned long long fake_hip_status_forwards(void) { return forwards; }
 unsigned int fake_hip_last_grid_x(void) { return last_grid_x; }
@@ -136,8 +139,8 @@ hipError_t hipHostGetDevicePointer(void **device, void *host, unsigned int flags
 hipError_t hipMemcpyAsync(void *dst, const void *src, size_t size, hipMemcpyKind kind,
                           hipStream_t stream)
 {
-    (void)kind;
     (void)stream;
+    if (kind == hipMemcpyDeviceToDevice) ++async_copies;
     memcpy(dst, src, size);
     return hipSuccess;
 }
@@ -180,8 +183,18 @@ hipError_t hipModuleLaunchKernel(hipFunction_t f, unsigned int gx, unsigned int 
                                  unsigned int shared, hipStream_t stream, void **params,
                                  void **extra)
 {
-    (void)gy; (void)gz; (void)bx; (void)by; (void)bz;
+    (void)gz; (void)bx; (void)by; (void)bz;
     (void)shared; (void)stream; (void)extra;
+    if (f && strcmp((const char *)f, "yvex_rocm_copy_batch") == 0 && params && params[0]) {
+        /* the batch of small copies is carried out too: gy copies, as the host queued them */
+        struct { uint64_t dst[128], src[128]; uint32_t bytes[128]; } *p = params[0];
+        unsigned int i;
+        if (env_is("FAKE_HIP_COPY_BATCH", "fail")) return hipErrorLaunchFailure;
+        for (i = 0u; i < gy && i < 128u; ++i)
+            memcpy((void *)(uintptr_t)p->dst[i], (const void *)(uintptr_t)p->src[i], p->bytes[i]);
+        ++copy_batches;
+        return hipSuccess;
+    }
     if (env_is("FAKE_HIP_LAUNCH", "fail")) return hipErrorLaunchFailure;
     if (f && strcmp((const char *)f, "yvex_rocm_status_forward") == 0 && params && params[0]) {
         /* the one kernel the stand-in carries out: (sequence, status) into the host's mailbox,

@@ -373,15 +373,18 @@ def test_history_append_in_the_decoder_order_of_rotary(backend, f32, d, rotary):
         t.release()
 
 
-def test_session_layer_copy_loop_equals_the_history_writer(backend):
+@pytest.mark.parametrize("tokens", [5, 700])
+def test_session_layer_copy_loop_equals_the_history_writer(backend, tokens):
     """The unchanged caller (src/runtime/stateful_attention.c:183-222): per token, one
     asynchronous copy of the key row and one of the value row into the [K | V] history row,
     F32 as the session layer keeps it, nothing waited for; then attention over the views.  The
     history must equal, byte for byte, what the one-launch writer leaves (no rotary: the
     session layer's rows arrive rotated), and the attention enqueued right behind the copies,
-    with no synchronisation in between, must equal the attention over the writer's history."""
-    rng = np.random.default_rng(314)
-    hq, hkv, d, have, tokens = 8, 2, 64, 37, 5
+    with no synchronisation in between, must equal the attention over the writer's history.
+    The copies are small: they wait in the backend's queue and leave in batches, the last of
+    them when the attention asks for the stream."""
+    rng = np.random.default_rng(314 + tokens)
+    hq, hkv, d, have = 8, 2, 64, 37   # 700 tokens: 1400 small copies, eleven launches of the copy queue
     width = hkv * d
     rows = have + tokens
     before = rng.standard_normal((rows, 2 * width)).astype(np.float32)

@@ -1418,3 +1418,72 @@ def test_status_word_reaches_the_host_through_the_mailbox_or_by_copy(env, fake_r
                 assert e.value.code == B.YVEX_ERR_BACKEND
             env("FAKE_HIP_SYNC", None)
     assert facts_seen[0] == facts_seen[1] == (1, 1, 1, 4)
+
+
+def test_small_async_copies_leave_in_batches_in_stream_order(env, fake_runtime):
+    """The session layer's per-token copies (src/runtime/stateful_attention.c:183-222) wait in a
+    queue and leave as one launch per 128 of them when anything else is asked of the stream; a
+    copy that meets what a queued one reads or writes sends the queue off first; large and odd
+    sizes go to the runtime behind the queue; a refused batch is issued copy by copy."""
+    for name in ("fake_hip_copy_batches", "fake_hip_device_copies", "fake_hip_launches"):
+        getattr(fake_runtime, name).restype = C.c_ulonglong
+    batches, singles = fake_runtime.fake_hip_copy_batches, fake_runtime.fake_hip_device_copies
+    with Backend() as b:
+        tokens, width = 300, 64
+        keys, values = f32(b, "keys", (tokens, width)), f32(b, "values", (tokens, width))
+        rng = np.random.default_rng(5)
+        k, v = rng.standard_normal((tokens, width), dtype=np.float32), rng.standard_normal((tokens, width), dtype=np.float32)
+        keys.write(k)
+        values.write(v)
+        history = f32(b, "history", (tokens + 2, 2 * width))
+        history.zero()
+        b0, s0, l0 = batches(), singles(), fake_runtime.fake_hip_launches()
+        for token in range(tokens):
+            row = (1 + token) * 2 * width * 4
+            history.view(row, B.DTYPE_F32, (width,)).copy_from_async(keys.view(token * width * 4, B.DTYPE_F32, (width,)))
+            history.view(row + width * 4, B.DTYPE_F32, (width,)).copy_from_async(
+                values.view(token * width * 4, B.DTYPE_F32, (width,)))
+        assert batches() - b0 == (2 * tokens) // 128                    # full queues left, the rest waits
+        got = history.read().reshape(tokens + 2, 2 * width)              # the read is behind every copy
+        assert batches() - b0 == (2 * tokens + 127) // 128 and singles() == s0
+        assert fake_runtime.fake_hip_launches() == l0                    # not launches of an operation
+        assert np.all(got[0] == 0) and np.all(got[-1] == 0)
+        assert np.array_equal(got[1:-1, :width], k) and np.array_equal(got[1:-1, width:], v)
+        # a chain through one buffer: each copy reads what the one before wrote
+        a, mid, c = f32(b, "a", (64,)), f32(b, "mid", (64,)), f32(b, "c", (64,))
+        a.write(np.arange(64, dtype=np.float32))
+        mid.zero()
+        c.zero()
+        b1 = batches()
+        mid.copy_from_async(a)
+        c.copy_from_async(mid)                                            # reads a queued destination
+        mid.copy_from_async(values.view(0, B.DTYPE_F32, (64,)))           # writes a queued source
+        assert batches() - b1 == 2
+        assert np.array_equal(c.read(), np.arange(64, dtype=np.float32)) and np.array_equal(mid.read(), v[0])
+        assert batches() - b1 == 3
+        a.copy_from_async(mid)
+        # an odd size and a large one are the runtime's, behind what is queued
+        odd_from, odd_to = f32(b, "odd-from", (3,)), f32(b, "odd-to", (3,))
+        odd_from.write(np.array([1, 2, 3], np.float32))
+        big_from, big_to = f32(b, "big-from", (1 << 17,)), f32(b, "big-to", (1 << 17,))
+        big_from.zero()
+        s1, b2 = singles(), batches()
+        mid.copy_from_async(c)
+        odd_to.copy_from_async(odd_from)
+        assert singles() - s1 == 1 and batches() - b2 == 1
+        big_to.copy_from_async(big_from)
+        assert singles() - s1 == 2 and batches() - b2 == 1
+        assert np.array_equal(odd_to.read(), [1, 2, 3])
+        # the batch launch refused: the same copies, one by one
+        env("FAKE_HIP_COPY_BATCH", "fail")
+        s2 = singles()
+        mid.copy_from_async(a)
+        c.copy_from_async(keys.view(0, B.DTYPE_F32, (64,)))
+        assert np.array_equal(mid.read(), v[0]) and np.array_equal(c.read(), k[0])
+        assert singles() - s2 == 2
+        env("FAKE_HIP_COPY_BATCH", None)
+        # a tensor that queued copies name is not freed under them
+        b3 = batches()
+        mid.copy_from_async(c)
+        mid.release()
+        assert batches() - b3 == 1
