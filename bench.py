@@ -311,9 +311,10 @@ def workload_decoder_block(backend, rng, steps, warmup):
     """One decode step of the reference's decoder attention block, call for call through the
     reference's own operator slots (src/runtime/decoder.c:1225-1270,
     src/runtime/stateful_attention.c:183-222): split the query/gate projection, rotate and round
-    Q and K, two asynchronous copies into the [K | V] history, attention under EXACT_F32 over
-    the strided views, round, sigmoid gate.  Ten launches and copies per step on F32
-    activations; what an unchanged caller pays on this backend.  Run by name."""
+    Q and K, two asynchronous copies into the [K | V] history, the write of the token position
+    and the two reads of the new rows the session layer makes, attention under EXACT_F32 over
+    the strided views, round, sigmoid gate.  Thirteen calls per step on F32 activations; what an
+    unchanged caller pays on this backend.  Run by name."""
     hq, hkv, d, ctx, rotary = 32, 8, 128, 4096, 64
     width = hkv * d
     f32 = lambda name, shape, scale=1.0: backend.tensor(  # noqa: E731
@@ -336,6 +337,11 @@ def workload_decoder_block(backend, rng, steps, warmup):
     work = backend.tensor("workspace", B.DTYPE_I8, (backend.attention_workspace_required(req),))
     backend.workspace_attach(work)
 
+    positions = backend.tensor("positions", B.DTYPE_I64, (ctx,))
+    positions.zero()
+    position_slot = positions.view((ctx - 1) * 8, B.DTYPE_I64, (1,))
+    here = np.array([ctx - 1], dtype=np.int64)
+
     def run():
         backend.split_interleaved_two_f32(qg, q, gate, 1, hq, d)
         backend.rotary_half_f32(q, cosine, sine, 1, hq, d, rotary)
@@ -344,6 +350,9 @@ def workload_decoder_block(backend, rng, steps, warmup):
         backend.bf16_round(k_new, width)
         k_slot.copy_from_async(k_row)
         v_slot.copy_from_async(v_row)
+        position_slot.write(here)              # stateful_attention.c:222-243: the token positions
+        k_new.read()                           # :245-272: the new rows back to the host's delta
+        v_new.read()
         facts = backend.attention_execute(req, q, k_view, v_view, mixer)
         backend.bf16_round(mixer, hq * d)
         backend.sigmoid_product_bf16(mixer, gate, gated, hq * d)
@@ -355,11 +364,12 @@ def workload_decoder_block(backend, rng, steps, warmup):
     backend.workspace_detach()
     return dict(name="decoder_block",
                 workload="one decode step of the reference's decoder attention block, call for call "
-                         "(split, rotary and rounding of Q and K, two copies into the [K|V] history, "
-                         "EXACT_F32 attention over 4096 cached tokens, rounding, sigmoid gate): 32/8 "
-                         "heads, d=128, f32 activations",
+                         "(split, rotary and rounding of Q and K, two copies into the [K|V] history, one "
+                         "small write and two small reads of the session layer, EXACT_F32 attention "
+                         "over 4096 cached tokens, rounding, sigmoid gate): 32/8 heads, d=128, f32 "
+                         "activations",
                 bound="hbm", algorithmic_bytes=2 * ctx * hkv * d * 4 + 2 * hq * d * 4, tokens=ctx,
-                dtype="f64", launches=10, kernels=kernels, **timed)
+                dtype="f64", launches=13, kernels=kernels, **timed)
 
 
 def workload_decoder_block_fused(backend, rng, steps, warmup):

@@ -160,8 +160,12 @@ static int rocm_tensor_write(yvex_backend *backend, yvex_device_tensor *tensor, 
     int rc = yvex_backend_tensor_rw_validate(where, backend, tensor, len, err);
     if (rc != YVEX_OK) return rc;
     if (!yvex_rocm_tensor_backed(tensor)) return refuse(err, YVEX_ERR_STATE, where, kUnbacked);
-    rc = rocm_copy(backend, tensor->data, src, len, hipMemcpyHostToDevice,
-                   YVEX_BACKEND_VARIANT_TENSOR_WRITE, where, err);
+    rc = yvex_rocm_require_capability(backend, YVEX_BACKEND_VARIANT_TENSOR_WRITE, where, err);
+    if (rc != YVEX_OK) return rc;
+    rc = yvex_rocm_small_write(backend, tensor->data, src, len, where, err);
+    if (rc == YVEX_ERR_UNSUPPORTED)
+        rc = rocm_copy(backend, tensor->data, src, len, hipMemcpyHostToDevice,
+                       YVEX_BACKEND_VARIANT_TENSOR_WRITE, where, err);
     if (rc != YVEX_OK) return rc;
     backend->stats.h2d_bytes += len;
     tensor->is_written = 1;
@@ -176,8 +180,12 @@ static int rocm_tensor_read(yvex_backend *backend, const yvex_device_tensor *ten
     int rc = yvex_backend_tensor_rw_validate(where, backend, tensor, len, err);
     if (rc != YVEX_OK) return rc;
     if (!yvex_rocm_tensor_backed(tensor)) return refuse(err, YVEX_ERR_STATE, where, kUnbacked);
-    rc = rocm_copy(backend, dst, tensor->data, len, hipMemcpyDeviceToHost,
-                   YVEX_BACKEND_VARIANT_TENSOR_READ, where, err);
+    rc = yvex_rocm_require_capability(backend, YVEX_BACKEND_VARIANT_TENSOR_READ, where, err);
+    if (rc != YVEX_OK) return rc;
+    rc = yvex_rocm_small_read(backend, dst, tensor->data, len, where, err);
+    if (rc == YVEX_ERR_UNSUPPORTED)
+        rc = rocm_copy(backend, dst, tensor->data, len, hipMemcpyDeviceToHost,
+                       YVEX_BACKEND_VARIANT_TENSOR_READ, where, err);
     if (rc != YVEX_OK) return rc;
     backend->stats.d2h_bytes += len;
     yvex_error_clear(err);
@@ -759,11 +767,14 @@ static int rocm_open(yvex_backend **out, const char *device, unsigned long long 
     if (rc == YVEX_OK && state->driver.pinned_memory) {
         /* the status mailbox is an economy, not a requirement: without it the word is copied */
         void *host = NULL, *device = NULL;
-        if (state->driver.hipHostMalloc(&host, 256u, hipHostMallocMapped) == hipSuccess && host) {
+        if (state->driver.hipHostMalloc(&host, 256u + YVEX_ROCM_SMALL_READ_MAX, hipHostMallocMapped) ==
+                hipSuccess && host) {
             if (state->driver.hipHostGetDevicePointer(&device, host, 0u) == hipSuccess && device) {
-                memset(host, 0, 256u);
+                memset(host, 0, 256u + YVEX_ROCM_SMALL_READ_MAX);
                 state->status_mailbox = (volatile uint64_t *)host;
                 state->status_mailbox_device = (uint64_t *)device;
+                state->read_staging = (unsigned char *)host + 256u;
+                state->read_staging_device = (unsigned char *)device + 256u;
             } else {
                 (void)state->driver.hipHostFree(host);
             }

@@ -99,6 +99,8 @@ static const rocm_kernel_binding rocm_kernel_bindings[] = {
     {"yvex_rocm_status_forward", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_F32,
      YVEX_ROCM_FN_STATUS_FORWARD},
     {"yvex_rocm_copy_batch", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_F32, YVEX_ROCM_FN_COPY_BATCH},
+    {"yvex_rocm_small_write", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_F32, YVEX_ROCM_FN_SMALL_WRITE},
+    {"yvex_rocm_small_read", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_F32, YVEX_ROCM_FN_SMALL_READ},
     {"yvex_rocm_gather_rows", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_MLA_BF16, YVEX_ROCM_FN_GATHER_ROWS},
     {"yvex_rocm_kv_append_bf16", YVEX_BACKEND_VARIANT_ROCM_ATTENTION_PAGED_BF16,
      YVEX_ROCM_FN_KV_APPEND_BF16},
@@ -505,51 +507,116 @@ static long long monotonic_ns(void)
     return (long long)now.tv_sec * 1000000000ll + (long long)now.tv_nsec;
 }
 
+/* Watches the mailbox for `sequence`.  A device that does not answer within
+ * ROCM_MAILBOX_SPIN_NS is waited for through the runtime, which also reports a device that
+ * has failed. */
+static int mailbox_wait(yvex_backend *backend, uint32_t sequence, const char *where, uint64_t *seen,
+                        yvex_error *err)
+{
+    yvex_rocm_backend_state *state = yvex_rocm_state(backend);
+    const long long deadline = monotonic_ns() + ROCM_MAILBOX_SPIN_NS;
+    unsigned int turn = 0u;
+    int rc;
+    for (;;) {
+        *seen = __atomic_load_n(state->status_mailbox, __ATOMIC_ACQUIRE);
+        if ((uint32_t)(*seen >> 32) == sequence) return YVEX_OK;
+        if ((++turn & 63u) == 0u && monotonic_ns() > deadline) break;
+    }
+    rc = yvex_rocm_synchronize(backend, YVEX_BACKEND_VARIANT_TENSOR_READ, where, err);
+    if (rc != YVEX_OK) return rc;
+    *seen = __atomic_load_n(state->status_mailbox, __ATOMIC_ACQUIRE);
+    if ((uint32_t)(*seen >> 32) == sequence) return YVEX_OK;
+    yvex_error_set(err, YVEX_ERR_BACKEND, where,
+                   "the stream ended without the operation's answer reaching the host");
+    return YVEX_ERR_BACKEND;
+}
+
+static int mailbox_launch(yvex_rocm_backend_state *state, yvex_rocm_function_id function,
+                          unsigned int block, void *params, const char *where, yvex_error *err)
+{
+    void *arguments[1] = {params};
+    return yvex_rocm_status(&state->driver,
+                            state->driver.hipModuleLaunchKernel(state->functions[function], 1u, 1u, 1u,
+                                                                block, 1u, 1u, 0u, yvex_rocm_stream(state),
+                                                                arguments, NULL),
+                            where, err);
+}
+
 /* The status word by way of the mailbox: a one-thread kernel behind the operation's kernels
  * stores (sequence, status) into host memory and the host watches for the sequence number,
  * about 8 us for an operation of one small kernel where a copy of the word and a wait for the
- * stream take 22.  A device that does not answer within ROCM_MAILBOX_SPIN_NS is waited for
- * through the runtime, which also reports a device that has failed.  Returns YVEX_ERR_UNSUPPORTED
- * (and has done nothing) when this backend has no mailbox. */
+ * stream take 22.  Returns YVEX_ERR_UNSUPPORTED (and has done nothing) when this backend has
+ * no mailbox. */
 static int status_by_mailbox(yvex_backend *backend, const char *where, int32_t *host_status,
                              yvex_error *err)
 {
     yvex_rocm_backend_state *state = yvex_rocm_state(backend);
     yvex_rocm_status_forward_params fp;
-    void *arguments[1];
-    uint64_t seen;
-    long long deadline;
-    unsigned int turn = 0u;
+    uint64_t seen = 0ull;
     int rc;
     if (!state->status_mailbox || !state->functions[YVEX_ROCM_FN_STATUS_FORWARD])
         return YVEX_ERR_UNSUPPORTED;
     fp.status = state->device_status;
     fp.mailbox = state->status_mailbox_device;
     fp.sequence = ++state->status_sequence;
-    arguments[0] = &fp;
-    rc = yvex_rocm_status(&state->driver,
-                          state->driver.hipModuleLaunchKernel(
-                              state->functions[YVEX_ROCM_FN_STATUS_FORWARD], 1u, 1u, 1u, 64u, 1u, 1u, 0u,
-                              yvex_rocm_stream(state), arguments, NULL),
-                          where, err);
+    rc = mailbox_launch(state, YVEX_ROCM_FN_STATUS_FORWARD, 64u, &fp, where, err);
+    if (rc == YVEX_OK) rc = mailbox_wait(backend, fp.sequence, where, &seen, err);
     if (rc != YVEX_OK) return rc;
-    deadline = monotonic_ns() + ROCM_MAILBOX_SPIN_NS;
-    for (;;) {
-        seen = __atomic_load_n(state->status_mailbox, __ATOMIC_ACQUIRE);
-        if ((uint32_t)(seen >> 32) == fp.sequence) break;
-        if ((++turn & 63u) == 0u && monotonic_ns() > deadline) {
-            rc = yvex_rocm_synchronize(backend, YVEX_BACKEND_VARIANT_TENSOR_READ, where, err);
-            if (rc != YVEX_OK) return rc;
-            seen = __atomic_load_n(state->status_mailbox, __ATOMIC_ACQUIRE);
-            if ((uint32_t)(seen >> 32) != fp.sequence) {
-                yvex_error_set(err, YVEX_ERR_BACKEND, where,
-                               "the stream ended without the operation's status reaching the host");
-                return YVEX_ERR_BACKEND;
-            }
-            break;
-        }
-    }
     *host_status = (int32_t)(uint32_t)seen;
+    return YVEX_OK;
+}
+
+/* Transfers of a few bytes cost the runtime's copy path 13 us (to the device) and 21 us (from
+ * it) each, and the session layer makes three per layer and step
+ * (src/runtime/stateful_attention.c:222-272).  A write of up to YVEX_ROCM_SMALL_WRITE_MAX
+ * bytes travels in the arguments of a kernel instead (3 us, nothing waited for: the host's
+ * buffer is free when the launch returns and later work is behind it on the stream); a read of
+ * up to YVEX_ROCM_SMALL_READ_MAX bytes is copied by a kernel into host memory the device can
+ * write while the host watches the mailbox (8 us).  Not while a launch sequence is recorded,
+ * and not under an injected synchronisation failure, which belongs to the runtime's wait. */
+static int small_transfer_admitted(const yvex_rocm_backend_state *state, yvex_rocm_function_id function,
+                                   yvex_backend_operation_variant variant)
+{
+    return state && !state->recording && state->functions[function] &&
+           !test_failure_matches("YVEX_TEST_ROCM_SYNC_FAILURE", variant);
+}
+
+int yvex_rocm_small_write(yvex_backend *backend, void *dst, const void *src, unsigned long long bytes,
+                          const char *where, yvex_error *err)
+{
+    yvex_rocm_backend_state *state = yvex_rocm_state(backend);
+    yvex_rocm_small_write_params wp;
+    if (!bytes || bytes > YVEX_ROCM_SMALL_WRITE_MAX ||
+        !small_transfer_admitted(state, YVEX_ROCM_FN_SMALL_WRITE, YVEX_BACKEND_VARIANT_TENSOR_WRITE))
+        return YVEX_ERR_UNSUPPORTED;
+    wp.dst = dst;
+    wp.bytes = (uint32_t)bytes;
+    wp.reserved = 0u;
+    memcpy(wp.data, src, (size_t)bytes);
+    return mailbox_launch(state, YVEX_ROCM_FN_SMALL_WRITE, 256u, &wp, where, err);
+}
+
+int yvex_rocm_small_read(yvex_backend *backend, void *dst, const void *src, unsigned long long bytes,
+                         const char *where, yvex_error *err)
+{
+    yvex_rocm_backend_state *state = yvex_rocm_state(backend);
+    yvex_rocm_small_read_params rp;
+    uint64_t seen = 0ull;
+    int rc;
+    if (!bytes || bytes > YVEX_ROCM_SMALL_READ_MAX ||
+        !small_transfer_admitted(state, YVEX_ROCM_FN_SMALL_READ, YVEX_BACKEND_VARIANT_TENSOR_READ) ||
+        !state->status_mailbox || !state->read_staging)
+        return YVEX_ERR_UNSUPPORTED;
+    rp.src = src;
+    rp.staging = state->read_staging_device;
+    rp.mailbox = state->status_mailbox_device;
+    rp.bytes = (uint32_t)bytes;
+    rp.sequence = ++state->status_sequence;
+    rc = mailbox_launch(state, YVEX_ROCM_FN_SMALL_READ, 256u, &rp, where, err);
+    if (rc == YVEX_OK) rc = mailbox_wait(backend, rp.sequence, where, &seen, err);
+    if (rc == YVEX_OK && state->copy_queue.failed) rc = refuse_copy_queue(backend, where, err);
+    if (rc != YVEX_OK) return rc;
+    memcpy(dst, state->read_staging, (size_t)bytes);
     return YVEX_OK;
 }
 

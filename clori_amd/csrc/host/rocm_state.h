@@ -52,6 +52,8 @@ typedef enum {
     YVEX_ROCM_FN_SPLIT_INTERLEAVED_TWO_F32,
     YVEX_ROCM_FN_STATUS_FORWARD,
     YVEX_ROCM_FN_COPY_BATCH,
+    YVEX_ROCM_FN_SMALL_WRITE,
+    YVEX_ROCM_FN_SMALL_READ,
     YVEX_ROCM_FN_GATHER_ROWS,
     YVEX_ROCM_FN_COUNT
 } yvex_rocm_function_id;
@@ -114,6 +116,8 @@ typedef struct yvex_rocm_backend_state {
     volatile uint64_t *status_mailbox;
     uint64_t *status_mailbox_device;
     uint32_t status_sequence;
+    /* behind the mailbox in the same allocation: where small tensor reads arrive */
+    unsigned char *read_staging, *read_staging_device;
     uint32_t *decode_arrivals; /* YVEX_ROCM_DECODE_SEGMENTS_MAX counters, zero between operations */
     int status_dirty;       /* deferred mode: launches since the last check */
     yvex_rocm_completion_mode completion_mode;
@@ -184,6 +188,12 @@ static inline hipStream_t yvex_rocm_stream(yvex_rocm_backend_state *state)
 }
 
 /* rocm_capability.c */
+/* Small transfers by kernel (see kernel_params.h): YVEX_ERR_UNSUPPORTED, with nothing done,
+ * when the transfer is not one of them or the backend lacks what they need. */
+int yvex_rocm_small_write(yvex_backend *backend, void *dst, const void *src, unsigned long long bytes,
+                          const char *where, yvex_error *err);
+int yvex_rocm_small_read(yvex_backend *backend, void *dst, const void *src, unsigned long long bytes,
+                         const char *where, yvex_error *err);
 int yvex_rocm_kernel_bundle_admit(yvex_backend *backend, yvex_error *err);
 int yvex_rocm_kernel_bundle_close(yvex_backend *backend, yvex_error *err);
 int yvex_rocm_query_capability(const yvex_backend *backend, yvex_backend_operation_variant variant,

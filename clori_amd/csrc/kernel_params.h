@@ -137,6 +137,26 @@ typedef struct {
     uint32_t bytes[YVEX_ROCM_COPY_BATCH_MAX];
 } yvex_rocm_copy_batch_params;
 
+/* Small transfers between the host and a tensor without the runtime's copy path.
+ * write: up to YVEX_ROCM_SMALL_WRITE_MAX bytes travel in the kernel's arguments and one
+ * workgroup of 256 threads stores them at dst; the host does not wait.
+ * read: one workgroup copies `bytes` from src into host memory the device can write
+ * (staging) and then leaves sequence << 32 in the mailbox the host is watching. */
+#define YVEX_ROCM_SMALL_WRITE_MAX 2048
+#define YVEX_ROCM_SMALL_READ_MAX 16384
+typedef struct {
+    void *dst;
+    uint32_t bytes, reserved;
+    unsigned char data[YVEX_ROCM_SMALL_WRITE_MAX];
+} yvex_rocm_small_write_params;
+
+typedef struct {
+    const void *src;
+    void *staging;
+    uint64_t *mailbox;
+    uint32_t bytes, sequence;
+} yvex_rocm_small_read_params;
+
 /* Completion: one workgroup of 64 threads behind an operation's kernels.  Takes the status
  * word (and clears it when set) and leaves (sequence << 32 | status) in a word of host memory,
  * which the host is watching. */

@@ -109,3 +109,40 @@ yvex_rocm_copy_batch(const yvex_rocm_copy_batch_params p)
     u32x4 *dst = reinterpret_cast<u32x4 *>(p.dst[copy]);
     for (uint32_t i = blockIdx.x * 256u + threadIdx.x; i < pieces; i += gridDim.x * 256u) dst[i] = src[i];
 }
+
+// A tensor write of a few bytes (the session layer writes a layer's token positions, eight
+// bytes per token, at every step: src/runtime/stateful_attention.c:222-243): the bytes arrive
+// in the kernel's arguments, so the host's buffer is free when the launch returns and nothing
+// waits.
+extern "C" __global__ void __launch_bounds__(256)
+yvex_rocm_small_write(const yvex_rocm_small_write_params p)
+{
+    unsigned char *dst = static_cast<unsigned char *>(p.dst);
+    if (((reinterpret_cast<uintptr_t>(p.dst) | p.bytes) & 3u) == 0u) {
+        const uint32_t *words = reinterpret_cast<const uint32_t *>(p.data);
+        for (uint32_t i = threadIdx.x; i < p.bytes / 4u; i += 256u) reinterpret_cast<uint32_t *>(dst)[i] = words[i];
+    } else {
+        for (uint32_t i = threadIdx.x; i < p.bytes; i += 256u) dst[i] = p.data[i];
+    }
+}
+
+// A tensor read of a few KB (the session layer reads the new key and value rows back at every
+// step, src/runtime/stateful_attention.c:245-272): the bytes go into host memory the device
+// can write, then the sequence number the host is watching for.
+extern "C" __global__ void __launch_bounds__(256)
+yvex_rocm_small_read(const yvex_rocm_small_read_params p)
+{
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    const unsigned char *src = static_cast<const unsigned char *>(p.src);
+    unsigned char *staging = static_cast<unsigned char *>(p.staging);
+    if (((reinterpret_cast<uintptr_t>(p.src) | p.bytes) & 15u) == 0u) {
+        for (uint32_t i = threadIdx.x; i < p.bytes / 16u; i += 256u)
+            reinterpret_cast<u32x4 *>(staging)[i] = reinterpret_cast<const u32x4 *>(src)[i];
+    } else {
+        for (uint32_t i = threadIdx.x; i < p.bytes; i += 256u) staging[i] = src[i];
+    }
+    __threadfence_system();  // this thread's bytes are in host memory before the number is
+    __syncthreads();
+    if (threadIdx.x == 0u)
+        __hip_atomic_store(p.mailbox, (uint64_t)p.sequence << 32, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+}

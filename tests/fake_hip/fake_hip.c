@@ -16,7 +16,7 @@
 #include <string.h>
 #include <sys/mman.h>
 
-static unsigned long long launches, allocations, frees, loads, unloads, forwards, copy_batches, async_copies;
+static unsigned long long launches, allocations, frees, loads, unloads, forwards, copy_batches, async_copies, small_transfers;
 static int capturing;                       /* a stream capture is open */
 static unsigned long long captured_launches;
 
@@ -26,6 +26,8 @@ unsigned long long fake_hip_launches(void) { return launches; }
 /* launches that carried a batch of queued copies, and copies handed to the runtime one by one */
 unsigned long long fake_hip_copy_batches(void) { return copy_batches; }
 unsigned long long fake_hip_device_copies(void) { return async_copies; }
+/* tensor reads and writes of a few bytes carried by a kernel */
+unsigned long long fake_hip_small_transfers(void) { return small_transfers; }
 /* status words handed to the host through its mailbox */
 unsigned long long fake_hip_status_forwards(void) { return forwards; }
 unsigned int fake_hip_last_grid_x(void) { return last_grid_x; }
@@ -185,6 +187,21 @@ hipError_t hipModuleLaunchKernel(hipFunction_t f, unsigned int gx, unsigned int 
 {
     (void)gz; (void)bx; (void)by; (void)bz;
     (void)shared; (void)stream; (void)extra;
+    if (f && strcmp((const char *)f, "yvex_rocm_small_write") == 0 && params && params[0]) {
+        /* small transfers by kernel are carried out as well */
+        struct { void *dst; uint32_t bytes, reserved; unsigned char data[2048]; } *p = params[0];
+        memcpy(p->dst, p->data, p->bytes);
+        ++small_transfers;
+        return hipSuccess;
+    }
+    if (f && strcmp((const char *)f, "yvex_rocm_small_read") == 0 && params && params[0]) {
+        struct { const void *src; void *staging; uint64_t *mailbox; uint32_t bytes, sequence; } *p = params[0];
+        memcpy(p->staging, p->src, p->bytes);
+        /* a device that does not answer: the host's watch runs out and it asks the runtime */
+        if (!env_is("FAKE_HIP_SYNC", "fail")) *p->mailbox = (uint64_t)p->sequence << 32;
+        ++small_transfers;
+        return hipSuccess;
+    }
     if (f && strcmp((const char *)f, "yvex_rocm_copy_batch") == 0 && params && params[0]) {
         /* the batch of small copies is carried out too: gy copies, as the host queued them */
         struct { uint64_t dst[128], src[128]; uint32_t bytes[128]; } *p = params[0];
@@ -202,7 +219,7 @@ hipError_t hipModuleLaunchKernel(hipFunction_t f, unsigned int gx, unsigned int 
         struct { int32_t *status; uint64_t *mailbox; uint32_t sequence; } *p = params[0];
         const int32_t status = *p->status;
         *p->status = 0;
-        *p->mailbox = ((uint64_t)p->sequence << 32) | (uint32_t)status;
+        if (!env_is("FAKE_HIP_SYNC", "fail")) *p->mailbox = ((uint64_t)p->sequence << 32) | (uint32_t)status;
         ++forwards;
         return hipSuccess;
     }

@@ -184,3 +184,32 @@ def test_the_decoder_s_attention_block_call_for_call(backend):
     # the attention rows agree to F32 tolerance before the rounding, so a rounded row may sit one
     # bf16 step off where the unrounded value lies next to a tie; the gate adds the same
     assert step.max() <= 1 and np.count_nonzero(step) <= got.size // 50, (step.max(), np.count_nonzero(step))
+
+
+@pytest.mark.parametrize("offset", [0, 1, 2, 3, 16])
+def test_small_tensor_transfers_by_kernel_equal_the_runtime_copies(backend, offset):
+    """Writes of up to 2048 bytes travel in a kernel's arguments and reads of up to 16384 bytes
+    come back through host memory the device writes (the session layer's three small transfers
+    per layer and step, src/runtime/stateful_attention.c:222-272); longer ones take the runtime's
+    copies.  Every size either side of the limits, at every byte alignment, reads back what was
+    written, and a write that is not waited for is seen by the copy and the read behind it."""
+    rng = np.random.default_rng(900 + offset)
+    store = backend.tensor("bytes", B.DTYPE_I8, (1 << 17,))
+    store.zero()
+    for size in (1, 3, 4, 8, 15, 16, 17, 255, 2047, 2048, 2049, 4096, 16383, 16384, 16385, 65536):
+        data = rng.integers(-128, 128, size, dtype=np.int8)
+        view = store.view(offset, B.DTYPE_I8, (size,))
+        view.write(data)
+        assert np.array_equal(view.read(), data), size
+        guard = store.view(offset + size, B.DTYPE_I8, (16,)).read()
+        assert not guard.any(), size                                   # nothing behind the view was touched
+        view.write(np.zeros(size, np.int8))
+    # a small write, an asynchronous copy of it, a small read of the copy: stream order, no wait
+    a, b2 = backend.tensor("a", B.DTYPE_F32, (64,)), backend.tensor("b", B.DTYPE_F32, (64,))
+    for turn in range(20):
+        values = rng.standard_normal(64).astype(np.float32)
+        a.write(values)
+        b2.copy_from_async(a)
+        assert np.array_equal(b2.read(), values), turn
+    for t in (store, a, b2):
+        t.release()

@@ -1487,3 +1487,51 @@ def test_small_async_copies_leave_in_batches_in_stream_order(env, fake_runtime):
         mid.copy_from_async(c)
         mid.release()
         assert batches() - b3 == 1
+
+
+def test_small_transfers_take_the_kernel_path_and_fall_back(env, fake_runtime):
+    """Tensor writes of up to 2048 bytes and reads of up to 16384 go by kernel (no copy of the
+    runtime, and for the write no wait); longer ones, and every one when the runtime gives no
+    host memory the device can write or a failure of the wait is injected, take the runtime's
+    copy and its wait."""
+    fake_runtime.fake_hip_small_transfers.restype = C.c_ulonglong
+    small = fake_runtime.fake_hip_small_transfers
+    with Backend() as b:
+        t = b.tensor("t", B.DTYPE_I8, (1 << 16,))
+        t.zero()
+        for size, by_kernel_write, by_kernel_read in [(1, 1, 1), (7, 1, 1), (2048, 1, 1), (2049, 0, 1),
+                                                       (16384, 0, 1), (16385, 0, 0)]:
+            data = (np.arange(size) % 251).astype(np.int8)
+            view = t.view(3, B.DTYPE_I8, (size,))
+            before = small()
+            view.write(data)
+            assert small() - before == by_kernel_write, size
+            before = small()
+            assert np.array_equal(view.read(), data)
+            assert small() - before == by_kernel_read, size
+        stats = b.memory_stats()
+        assert stats.h2d_bytes == sum((1, 7, 2048, 2049, 16384, 16385))
+        assert stats.d2h_bytes == stats.h2d_bytes
+        env("YVEX_TEST_ROCM_SYNC_FAILURE", "tensor-read")
+        before = small()
+        with pytest.raises(YvexError) as e:
+            t.view(0, B.DTYPE_I8, (8,)).read()
+        assert e.value.code == B.YVEX_ERR_BACKEND and small() == before   # the injected failure is the wait's
+        env("YVEX_TEST_ROCM_SYNC_FAILURE", None)
+    env("FAKE_HIP_HOST_MALLOC", "fail")
+    with Backend() as b:
+        t = b.tensor("t", B.DTYPE_I8, (64,))
+        before = small()
+        t.write(np.arange(64, dtype=np.int8))
+        assert small() - before == 1                                      # the write needs no host memory
+        assert np.array_equal(t.read(), np.arange(64, dtype=np.int8))
+        assert small() - before == 1                                      # the read does
+    env("FAKE_HIP_HOST_MALLOC", None)
+    with Backend() as b:                                                  # a device that does not answer
+        t = b.tensor("t", B.DTYPE_I8, (64,))
+        t.write(np.arange(64, dtype=np.int8))
+        env("FAKE_HIP_SYNC", "fail")
+        with pytest.raises(YvexError) as e:
+            t.read()
+        assert e.value.code == B.YVEX_ERR_BACKEND
+        env("FAKE_HIP_SYNC", None)
