@@ -882,7 +882,10 @@ int yvex_backend_open_shared_rocm(yvex_backend **out, yvex_backend *context_owne
         return refuse(err, YVEX_ERR_INVALID_ARG, where, "one owning ROCm backend is required");
     rc = yvex_backend_shared_owner_acquire(context_owner, err);
     if (rc != YVEX_OK) return rc;
-    rc = rocm_open(out, NULL, memory_limit_bytes, context_owner, err);
+    /* from here on the primary waits for its small writes (yvex_rocm_small_write); the ones it
+     * made while it was alone are waited for now, before another stream can read them */
+    rc = yvex_rocm_synchronize(context_owner, YVEX_BACKEND_VARIANT_TENSOR_WRITE, where, err);
+    if (rc == YVEX_OK) rc = rocm_open(out, NULL, memory_limit_bytes, context_owner, err);
     if (rc != YVEX_OK) {
         /* nothing was published: give the lease back */
         atomic_fetch_sub_explicit(&context_owner->lifecycle, 1ull, memory_order_acq_rel);

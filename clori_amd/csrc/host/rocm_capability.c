@@ -581,11 +581,32 @@ static int small_transfer_admitted(const yvex_rocm_backend_state *state, yvex_ro
            !test_failure_matches("YVEX_TEST_ROCM_SYNC_FAILURE", variant);
 }
 
+/* Returns when everything asked of the stream so far has ended: an empty small read posts the
+ * number the host watches for; without a mailbox, the runtime's wait. */
+static int stream_reached(yvex_backend *backend, const char *where, yvex_error *err)
+{
+    yvex_rocm_backend_state *state = yvex_rocm_state(backend);
+    yvex_rocm_small_read_params rp;
+    uint64_t seen = 0ull;
+    int rc;
+    if (!state->status_mailbox || !state->functions[YVEX_ROCM_FN_SMALL_READ])
+        return yvex_rocm_synchronize(backend, YVEX_BACKEND_VARIANT_TENSOR_WRITE, where, err);
+    rp.src = NULL;
+    rp.staging = state->read_staging_device;
+    rp.mailbox = state->status_mailbox_device;
+    rp.bytes = 0u;
+    rp.sequence = ++state->status_sequence;
+    rc = mailbox_launch(state, YVEX_ROCM_FN_SMALL_READ, 256u, &rp, where, err);
+    if (rc == YVEX_OK) rc = mailbox_wait(backend, rp.sequence, where, &seen, err);
+    return rc;
+}
+
 int yvex_rocm_small_write(yvex_backend *backend, void *dst, const void *src, unsigned long long bytes,
                           const char *where, yvex_error *err)
 {
     yvex_rocm_backend_state *state = yvex_rocm_state(backend);
     yvex_rocm_small_write_params wp;
+    int rc;
     if (!bytes || bytes > YVEX_ROCM_SMALL_WRITE_MAX ||
         !small_transfer_admitted(state, YVEX_ROCM_FN_SMALL_WRITE, YVEX_BACKEND_VARIANT_TENSOR_WRITE))
         return YVEX_ERR_UNSUPPORTED;
@@ -593,7 +614,16 @@ int yvex_rocm_small_write(yvex_backend *backend, void *dst, const void *src, uns
     wp.bytes = (uint32_t)bytes;
     wp.reserved = 0u;
     memcpy(wp.data, src, (size_t)bytes);
-    return mailbox_launch(state, YVEX_ROCM_FN_SMALL_WRITE, 256u, &wp, where, err);
+    rc = mailbox_launch(state, YVEX_ROCM_FN_SMALL_WRITE, 256u, &wp, where, err);
+    /* Alone on its device, everything that can read the tensor is behind the write on this
+     * stream.  With session backends about (each has a stream of its own, and a written
+     * tensor may be read from any of them with no event in between) the write is waited for,
+     * as the runtime's copy was; opening a session backend waits for the primary's stream. */
+    if (rc == YVEX_OK &&
+        (backend->resource_owner != backend ||
+         (atomic_load_explicit(&backend->lifecycle, memory_order_acquire) & YVEX_BACKEND_LIFECYCLE_CHILD_MASK)))
+        rc = stream_reached(backend, where, err);
+    return rc;
 }
 
 int yvex_rocm_small_read(yvex_backend *backend, void *dst, const void *src, unsigned long long bytes,

@@ -1527,6 +1527,24 @@ def test_small_transfers_take_the_kernel_path_and_fall_back(env, fake_runtime):
         assert np.array_equal(t.read(), np.arange(64, dtype=np.int8))
         assert small() - before == 1                                      # the read does
     env("FAKE_HIP_HOST_MALLOC", None)
+    # with a session backend on the device a written tensor may be read from another stream with
+    # no event in between: the small write is waited for (a second, empty transfer) on both
+    primary = Backend()
+    t = primary.tensor("t", B.DTYPE_I8, (64,))
+    before = small()
+    t.write(np.arange(64, dtype=np.int8))
+    assert small() - before == 1
+    session = Backend(shared_with=primary)
+    u = session.tensor("u", B.DTYPE_I8, (64,))
+    for tensor in (t, u):
+        before = small()
+        tensor.write(np.arange(64, dtype=np.int8))
+        assert small() - before == 2
+    session.close()
+    before = small()
+    t.write(np.arange(64, dtype=np.int8))
+    assert small() - before == 1                                          # alone again
+    primary.close()
     with Backend() as b:                                                  # a device that does not answer
         t = b.tensor("t", B.DTYPE_I8, (64,))
         t.write(np.arange(64, dtype=np.int8))
