@@ -17,7 +17,7 @@ under the EXACT_F32 contract: fp32 matrix cores, and double-precision split deco
 append_bf16 / append_q8_0 (the KV page writer), history_append (the token-major writer), paged3_p64 / paged4_p64
 (configurations 3 and 4 with pages of 64 tokens), prefill_d256 / prefill_d64 (causal prefill at head
 dimension 256, 24/4 heads, and 64, 16/4 heads), paged_d256 / paged_d64 and decode_d256 / decode_d64 (configurations 3 and 1
-at those head dimensions), decoder_block / decoder_block_fused (one decode step of the reference's decoder attention
+at those head dimensions), exact2_d256 / exact1_d256 (the EXACT_F32 forms at 24/4 heads, head dimension 256), decoder_block / decoder_block_fused (one decode step of the reference's decoder attention
 block: call for call through the reference's slots, and through the two fused entry points), copy.
 
 Prints ONE JSON line.  `value` is the headline workload's throughput; every workload
@@ -263,10 +263,10 @@ def workload_prefill2(backend, rng, steps, warmup, hq=40, hkv=8, d=128, name="pr
                 launches=int(facts.kernel_launches), kernels=kernels, **timed)
 
 
-def workload_exact2(backend, rng, steps, warmup):
+def workload_exact2(backend, rng, steps, warmup, hq=40, hkv=8, d=128, name="exact2"):
     """Configuration 2 under the EXACT_F32 contract (F32 tensors, F32 products): the request
     the reference's engine makes.  Not one of the metric's configurations: run by name."""
-    t, hq, hkv, d = 2048, 40, 8, 128
+    t = 2048
     q = backend.tensor("q", B.DTYPE_F32, (t, hq, d), rng.standard_normal((t, hq, d), dtype=np.float32))
     k = backend.tensor("k", B.DTYPE_F32, (t, hkv, d), rng.standard_normal((t, hkv, d), dtype=np.float32))
     v = backend.tensor("v", B.DTYPE_F32, (t, hkv, d), rng.standard_normal((t, hkv, d), dtype=np.float32))
@@ -274,20 +274,20 @@ def workload_exact2(backend, rng, steps, warmup):
     req = backend.attention_requirement(t, t, hq, hkv, d, causal=True)
     run = lambda: backend.attention_execute(req, q, k, v, out)  # noqa: E731
     facts = run()
-    kernels = ["yvex_rocm_gqa_f32_tile_128"]
+    kernels = ["yvex_rocm_gqa_f32_tile_%d" % d]
     timed = time_steps(backend, run, steps, warmup, kernels)
-    return dict(name="exact2",
-                workload="causal GQA prefill, EXACT_F32 contract: batch 1, seq 2048, 40/8 heads, "
-                         "d=128, f32 in and out",
+    return dict(name=name,
+                workload="causal GQA prefill, EXACT_F32 contract: batch 1, seq 2048, %d/%d heads, "
+                         "d=%d, f32 in and out" % (hq, hkv, d),
                 bound="mfma", flops=4 * d * hq * t * (t + 1) // 2, peak_tflops=MFMA_F32_PEAK_TFLOPS,
                 algorithmic_bytes=(2 * t * hq * d + 2 * t * hkv * d) * 4, dtype="f32",
                 launches=int(facts.kernel_launches), kernels=kernels, **timed)
 
 
-def workload_exact1(backend, rng, steps, warmup):
+def workload_exact1(backend, rng, steps, warmup, hq=32, hkv=8, d=128, name="exact1"):
     """Configuration 1 under the EXACT_F32 contract: the decode step the reference's session
     layer makes (one query token over the cached F32 history).  Run by name."""
-    hq, hkv, d, ctx = 32, 8, 128, 4096
+    ctx = 4096
     q = backend.tensor("q", B.DTYPE_F32, (1, hq, d), rng.standard_normal((1, hq, d), dtype=np.float32))
     k = backend.tensor("k", B.DTYPE_F32, (ctx, hkv, d), rng.standard_normal((ctx, hkv, d), dtype=np.float32))
     v = backend.tensor("v", B.DTYPE_F32, (ctx, hkv, d), rng.standard_normal((ctx, hkv, d), dtype=np.float32))
@@ -297,12 +297,12 @@ def workload_exact1(backend, rng, steps, warmup):
     backend.workspace_attach(work)
     run = lambda: backend.attention_execute(req, q, k, v, out)  # noqa: E731
     facts = run()
-    kernels = ["yvex_rocm_gqa_f32_split"]
+    kernels = ["yvex_rocm_gqa_f32_split" + ("_wide" if d > 128 else "")]
     timed = time_steps(backend, run, steps, warmup, kernels)
     backend.workspace_detach()
-    return dict(name="exact1",
-                workload="GQA decode, EXACT_F32 contract: batch 1, 32/8 heads, d=128, context 4096, "
-                         "contiguous f32 KV",
+    return dict(name=name,
+                workload="GQA decode, EXACT_F32 contract: batch 1, %d/%d heads, d=%d, context 4096, "
+                         "contiguous f32 KV" % (hq, hkv, d),
                 bound="hbm", algorithmic_bytes=2 * ctx * hkv * d * 4 + 2 * hq * d * 4, tokens=ctx,
                 dtype="f64", launches=int(facts.kernel_launches), kernels=kernels, **timed)
 
@@ -557,6 +557,8 @@ EXTRA_WORKLOADS = {
     # the reference's own Qwen attention geometry (24/4 heads, head dimension 256) and a narrow one
     "prefill_d256": lambda b, r, s, w: workload_prefill2(b, r, s, w, hq=24, hkv=4, d=256, name="prefill_d256"),
     "prefill_d64": lambda b, r, s, w: workload_prefill2(b, r, s, w, hq=16, hkv=4, d=64, name="prefill_d64"),
+    "exact2_d256": lambda b, r, s, w: workload_exact2(b, r, s, w, hq=24, hkv=4, d=256, name="exact2_d256"),
+    "exact1_d256": lambda b, r, s, w: workload_exact1(b, r, s, w, hq=24, hkv=4, d=256, name="exact1_d256"),
     "decode_d256": lambda b, r, s, w: workload_decode1(b, r, s, w, hq=24, hkv=4, d=256, name="decode_d256"),
     "decode_d64": lambda b, r, s, w: workload_decode1(b, r, s, w, hq=16, hkv=4, d=64, name="decode_d64"),
     "paged_d256": lambda b, r, s, w: workload_paged(b, r, s, w, hq=24, hkv=4, d=256, name="paged_d256"),
@@ -567,7 +569,8 @@ EXTRA_WORKLOADS = {
 SEEDS = {"decode1": 1, "prefill2": 2, "paged3": 3, "paged4": 4, "mla5": 5, "append_bf16": 6,
          "append_q8_0": 7, "exact2": 8, "exact1": 9, "history_append": 10, "paged3_p64": 3, "paged4_p64": 4,
          "prefill_d256": 11, "prefill_d64": 12, "paged_d256": 13, "paged_d64": 14, "decoder_block": 15,
-         "decoder_block_fused": 15, "decode_d256": 16, "decode_d64": 17}
+         "decoder_block_fused": 15, "decode_d256": 16, "decode_d64": 17,
+         "exact2_d256": 18, "exact1_d256": 19}
 
 
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")

@@ -591,7 +591,8 @@ static int attention_execute_common(yvex_backend *backend,
             if (groups > 0x7fffffffull)
                 return refuse(err, YVEX_ERR_BOUNDS, "rocm.transformer.gqa",
                               "attention geometry exceeds the launch range");
-            /* two workgroups per unit at head dimension 64 and 128 (registers and LDS), one at 256 */
+            /* two workgroups per unit at head dimension 64 and 128 (registers and LDS), one (of eight
+             * waves) at 256 */
             const unsigned int per_unit = r->head_dimension == 256ull ? 1u : 2u;
             unsigned int workgroups = 0u;
             if (causal) {
@@ -615,7 +616,9 @@ static int attention_execute_common(yvex_backend *backend,
                     params.pair_units = (uint32_t)state->compute_units;
             }
             rc = yvex_rocm_launch(backend, tile_function, YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_F32,
-                                  workgroups ? workgroups : (unsigned int)groups, 1u, 1u, 256u, 0u,
+                                  workgroups ? workgroups : (unsigned int)groups, 1u, 1u,
+                                  /* at 256 pairs of waves split the head dimension: eight waves */
+                                  r->head_dimension == 256ull ? 512u : 256u, 0u,
                                   &params, "rocm.transformer.gqa", err);
             tiled = 1;
         } else if ((split_runs = exact_split_runs(r, &split_keys)) != 0ull &&
