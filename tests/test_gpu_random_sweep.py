@@ -1,6 +1,6 @@
-"""GPU parity: a seeded random sweep over the four kernel families (prefill with and without
+"""GPU parity: a seeded random sweep over the kernel families (prefill with and without
 the fused gate, paged decode bf16 / Q8_0, MLA decode with sinks, window and compressed rows,
-page writer with rotary) at shapes the fixed cases do not list: odd head groups, ragged
+page writer with rotary, single-token decode over token-major rows, EXACT_F32 requests) at shapes the fixed cases do not list: odd head groups, ragged
 contexts around tile and page edges, empty sessions, unaligned spans.  Same bar as the fixed
 cases; the page writer is byte-exact."""
 import numpy as np
@@ -234,15 +234,83 @@ def append_case(c):
     assert np.array_equal(got_v.reshape(want_v.shape), want_v), label
 
 
-FAMILIES = {"prefill": prefill_case, "paged": paged_case, "mla": mla_case, "append": append_case}
+def rows_case(c):
+    """One query token over a token-major bf16 history: head dimension 64, 128 or 256, groups of
+    1 to 16, packed or interleaved [K | V] rows, with and without the gate."""
+    b, rng = c.backend, c.rng
+    hkv = int(rng.choice([1, 2, 4, 8]))
+    hq = hkv * int(rng.choice([1, 2, 3, 4, 8, 16]))
+    d = int(rng.choice([128, 64, 256]))
+    ctx = int(rng.integers(1, int(rng.choice([40, 700, 9000]))))
+    causal = bool(rng.integers(0, 2))
+    tk = ctx if causal else ctx + int(rng.integers(0, 50))
+    width = hkv * d
+    q, k, v = c.bf16((1, hq, d)), c.bf16((tk, hkv, d)), c.bf16((tk, hkv, d))
+    gate = c.bf16(q.shape, 2.0) if rng.integers(0, 2) else None
+    interleaved = bool(rng.integers(0, 2))
+    req = b.attention_requirement(1, tk, hq, hkv, d, causal=causal, query_start=ctx - 1, dtype=B.DTYPE_BF16,
+                                  contract=CONTRACT, k_stride=2 * width if interleaved else 0,
+                                  v_stride=2 * width if interleaved else 0)
+    if interleaved:
+        rows = np.zeros((tk, 2 * width), np.uint16)
+        rows[:, :width], rows[:, width:] = k.reshape(tk, width), v.reshape(tk, width)
+        store = c.tensor("kv", B.DTYPE_BF16, rows.shape, rows)
+        count = (tk - 1) * 2 * width + width
+        tk_, tv_ = store.view(0, B.DTYPE_BF16, (count,)), store.view(2 * width, B.DTYPE_BF16, (count,))
+    else:
+        tk_, tv_ = c.tensor("k", B.DTYPE_BF16, k.shape, k), c.tensor("v", B.DTYPE_BF16, v.shape, v)
+    out, lse = c.tensor("o", B.DTYPE_BF16, q.shape), c.tensor("l", B.DTYPE_F32, (1, hq))
+    b.attention_execute(req, c.tensor("q", B.DTYPE_BF16, q.shape, q), tk_, tv_, out, lse=lse,
+                        gate=c.tensor("g", B.DTYPE_BF16, gate.shape, gate) if gate is not None else None)
+    rc, ref, _, ref_lse = ORACLE.gqa_bf16(q, k, v, query_start=ctx - 1, causal=causal)
+    assert rc == 0
+    label = ("rows", ctx, tk, hq, hkv, d, causal, interleaved, gate is not None)
+    close(out.read(), gated(ref, gate) if gate is not None else ref, label)
+    assert np.abs(lse.read() - ref_lse).max() <= LSE_ABS, label
+
+
+def exact_case(c):
+    """EXACT_F32 requests of every shape: the matrix-core tiles (head dimension 64, 128, 256 with
+    at least 32 query tokens), the runs of keys (long histories) and the row kernel (the rest),
+    at the reference's tolerance for its float device kernel against the CPU operator
+    (tests/unit/cuda/quant_qtype.c:2293-2333: 2e-5 on N(0,1)-scale rows)."""
+    b, rng = c.backend, c.rng
+    hkv = int(rng.choice([1, 2, 4]))
+    hq = hkv * int(rng.choice([1, 2, 5, 6]))
+    d = int(rng.choice([128, 64, 256, 256, 96, 8]))
+    tq = int(rng.choice([1, 1, rng.integers(2, 32), rng.integers(32, 300)]))
+    start = int(rng.choice([0, rng.integers(0, 40), rng.integers(500, 3000)])) if tq < 32 else int(rng.integers(0, 300))
+    causal = bool(rng.integers(0, 4))
+    tk = start + tq if causal else start + tq + int(rng.integers(0, 100))
+    q = rng.standard_normal((tq, hq, d)).astype(np.float32)
+    k = rng.standard_normal((tk, hkv, d)).astype(np.float32)
+    v = rng.standard_normal((tk, hkv, d)).astype(np.float32)
+    req = b.attention_requirement(tq, tk, hq, hkv, d, causal=causal, query_start=start)
+    work = c.tensor("w", B.DTYPE_I8, (max(b.attention_workspace_required(req), 16),))
+    b.workspace_attach(work)
+    try:
+        out, lse = c.tensor("o", B.DTYPE_F32, q.shape), c.tensor("l", B.DTYPE_F32, (tq, hq))
+        b.attention_execute(req, c.tensor("q", B.DTYPE_F32, q.shape, q), c.tensor("k", B.DTYPE_F32, k.shape, k),
+                            c.tensor("v", B.DTYPE_F32, v.shape, v), out, lse=lse)
+        got, got_lse = out.read(), lse.read()
+    finally:
+        b.workspace_detach()
+    rc, ref, ref_lse = ORACLE.gqa(q, k, v, query_start=start, causal=causal)
+    assert rc == 0
+    label = ("exact", tq, tk, start, hq, hkv, d, causal)
+    assert np.abs(got - ref).max() < 2e-5 and np.abs(got_lse - ref_lse).max() < 2e-5, label
+
+
+FAMILIES = {"prefill": prefill_case, "paged": paged_case, "mla": mla_case, "append": append_case,
+            "rows": rows_case, "exact": exact_case}
 
 
 @pytest.mark.parametrize("seed", [11, 12])
 def test_random_sweep(backend, seed):
     rng = np.random.default_rng(seed)
     counts = dict.fromkeys(FAMILIES, 0)
-    for _ in range(80):
-        kind = str(rng.choice(["prefill", "paged", "mla", "append"]))
+    for _ in range(120):
+        kind = str(rng.choice(sorted(FAMILIES)))
         case = Case(backend, rng)
         FAMILIES[kind](case)
         case.release()
