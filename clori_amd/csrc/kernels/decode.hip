@@ -92,8 +92,7 @@ template <int kDim>
 __device__ inline void softmax_step(State<kDim> &st, const float (&x)[4], float (&p)[4])
 {
     float mloc = fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3]));
-    mloc = fmaxf(mloc, xor_lanes(mloc, 16));
-    mloc = fmaxf(mloc, xor_lanes(mloc, 32));
+    mloc = max_xor32(max_xor16(mloc));
     const float m_new = fmaxf(st.m, mloc);
     if (__builtin_amdgcn_ballot_w64(m_new > st.m) != 0ull) {
         const float alpha = fast_exp2(st.m - m_new);
@@ -668,8 +667,7 @@ struct Decoder {
                 stream(st, q, session, kv_head, ctx, first + done, min(128u, count - done));
 
             float l = st.l;
-            l += xor_lanes(l, 16);
-            l += xor_lanes(l, 32);
+            l = sum_xor32(sum_xor16(l));
             if (first == 0u && stop == seg_end) {
                 publish(st, l, session, kv_head);  // the whole segment was ours
             } else {
@@ -747,8 +745,7 @@ struct Decoder {
         for (uint32_t done = 0u; done < count; done += 128u)
             stream(st, q, session, kv_head, ctx, first + done, min(128u, count - done));
         float l = st.l;
-        l += xor_lanes(l, 16);
-        l += xor_lanes(l, 32);
+        l = sum_xor32(sum_xor16(l));
 
         // the wave's part into LDS (a wave without tiles leaves max -inf, sum 0, zeros)
         float *acc = parts, *ml = parts + kTeam * kTeamArea;

@@ -208,7 +208,7 @@ struct GqaTile {
                     s[i] = visible ? s[i] * p.scale : -INFINITY;
                     peak = fmaxf(peak, s[i]);
                 }
-                peak = fmaxf(peak, xor_lanes(peak, 32));
+                peak = max_xor32(peak);
                 const float top_new = fmaxf(top, peak);
                 // key 0 is visible to every query, so top_new is finite from the first tile on
                 const float keep = fast_exp2((top - top_new) * YVEX_LOG2E);
@@ -237,7 +237,7 @@ struct GqaTile {
 
         // (no early exit above this point: every wave of the workgroup keeps the barriers)
         if (q0 + (uint64_t)column >= p.query_tokens) return;
-        sum += xor_lanes(sum, 32);
+        sum = sum_xor32(sum);
         if (!(sum > 0.f) || !isfinite(sum) || !isfinite(top)) {
             flag_status(p.status, YVEX_ROCM_DEVICE_NUMERIC);
             return;
@@ -435,7 +435,7 @@ struct GqaTilePair {
                     s[i] = visible ? s[i] * p.scale : -INFINITY;
                     peak = fmaxf(peak, s[i]);
                 }
-                peak = fmaxf(peak, xor_lanes(peak, 32));
+                peak = max_xor32(peak);
                 const float top_new = fmaxf(top, peak);
                 const float keep = fast_exp2((top - top_new) * YVEX_LOG2E);
                 sum *= keep;
@@ -460,7 +460,7 @@ struct GqaTilePair {
         }
 
         if (q0 + (uint64_t)column >= p.query_tokens) return;
-        sum += xor_lanes(sum, 32);
+        sum = sum_xor32(sum);
         if (!(sum > 0.f) || !isfinite(sum) || !isfinite(top)) {
             flag_status(p.status, YVEX_ROCM_DEVICE_NUMERIC);
             return;

@@ -56,6 +56,42 @@ __device__ inline float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 
 __device__ inline float xor_lanes(float v, int mask) { return __shfl_xor(v, mask, 64); }
 
+// A value combined with the one the lane 16 (32) away holds, on the vector ALU:
+// v_permlane16_swap / v_permlane32_swap of two copies leave the even rows (the lower half) in
+// one register and the odd rows (the upper half) in the other, in every lane, so a commutative
+// combination of the two is the answer in both partners.  __shfl_xor takes a trip through the
+// LDS permute network instead, which sits in the dependent chain of every softmax step.
+// (The two results go through scalars: a bit cast applied directly to a vector element reads
+// element 0 whatever the index with this compiler.)
+__device__ inline float max_xor16(float v)
+{
+    const uint32_t bits = __builtin_bit_cast(uint32_t, v);
+    const u32x2 r = __builtin_amdgcn_permlane16_swap(bits, bits, false, false);
+    const uint32_t even = r.x, odd = r.y;
+    return fmaxf(__builtin_bit_cast(float, even), __builtin_bit_cast(float, odd));
+}
+__device__ inline float max_xor32(float v)
+{
+    const uint32_t bits = __builtin_bit_cast(uint32_t, v);
+    const u32x2 r = __builtin_amdgcn_permlane32_swap(bits, bits, false, false);
+    const uint32_t lower = r.x, upper = r.y;
+    return fmaxf(__builtin_bit_cast(float, lower), __builtin_bit_cast(float, upper));
+}
+__device__ inline float sum_xor16(float v)
+{
+    const uint32_t bits = __builtin_bit_cast(uint32_t, v);
+    const u32x2 r = __builtin_amdgcn_permlane16_swap(bits, bits, false, false);
+    const uint32_t even = r.x, odd = r.y;
+    return __builtin_bit_cast(float, even) + __builtin_bit_cast(float, odd);
+}
+__device__ inline float sum_xor32(float v)
+{
+    const uint32_t bits = __builtin_bit_cast(uint32_t, v);
+    const u32x2 r = __builtin_amdgcn_permlane32_swap(bits, bits, false, false);
+    const uint32_t lower = r.x, upper = r.y;
+    return __builtin_bit_cast(float, lower) + __builtin_bit_cast(float, upper);
+}
+
 // Round-to-nearest-even narrowing with the quiet-NaN policy of the reference codec
 // (src/gguf/quant_scalar.c:131-143).
 __device__ inline uint16_t bf16_bits(float v)

@@ -307,10 +307,10 @@ __device__ __forceinline__ void mla_decode(const yvex_rocm_mla_params &p, unsign
         for (int i = 0; i < 16; ++i) mloc = fmaxf(mloc, s[i]);
         mloc *= p.scale_log2;
         if (decltype(first)::value) {
-            m_run = fmaxf(mloc, xor_lanes(mloc, 32));
+            m_run = max_xor32(mloc);
             neg_m = m_run == -INFINITY ? 0.f : -m_run;
         } else if (__builtin_amdgcn_ballot_w64(mloc > m_run + kLazyLog2) != 0ull) {
-            const float m_new = fmaxf(m_run, fmaxf(mloc, xor_lanes(mloc, 32)));
+            const float m_new = fmaxf(m_run, max_xor32(mloc));
             const float alpha = m_new == -INFINITY ? 1.0f : fast_exp2(m_run - m_new);
             l_run *= alpha;
             // one block at a time through the VALU; the accumulators live in AGPRs
@@ -444,7 +444,7 @@ __device__ __forceinline__ void mla_decode(const yvex_rocm_mla_params &p, unsign
     __builtin_amdgcn_s_waitcnt(0x0f70);
 
     float l = l_run;
-    l += xor_lanes(l, 32);
+    l = sum_xor32(l);
     const uint64_t slot = ((uint64_t)batch * p.slot_stride + p.first_slot + chunk) * p.heads + head;
     // The accumulators are lane = head, registers = dims; through LDS they become one
     // contiguous 1 KB bf16 row per head, written by one 16-byte store per lane.
