@@ -15,12 +15,15 @@
  * also 64 and 256 (the same formulas with fewer or more chunks):
  *   BF16  K  uint16 [d/8][16][8]        elem(t,c) at ((c/8)*16 + t)*8 + c%8
  *         V  uint16 [d][16]             elem(t,c) at c*16 + t
- *   Q8_0  K  codes int8 [4 g][16 t][4 j][8]   code(t, c=32j+8g+e) at ((g*16+t)*4+j)*8+e
- *            then f16 scale [16 t][4 j]
- *         V  codes int8 [4 tg][16 m][8 b][4 i]  code(t=4tg+i, c=16b+m) at ((tg*16+m)*8+b)*4+i
- *            then f16 scale [16 t][4 j]       (j = c/32)
+ *   Q8_0  K  codes int8: lane L = 16 g + t of a wave consumes the 32 bytes (j, e) of
+ *            code(t, c = 32j + 8g + e), byte r = 8j + e of them; it lies at
+ *            (r / 16) * 1024 + 16 L + r % 16 (YVEX_ROCM_Q8_CODE_OFFSET of 32 L + r): the halves of
+ *            all lanes side by side, one KB each.  Then f16 scale [16 t][4 j]
+ *         V  codes int8: lane L = 16 tg + m consumes the bytes (b, i) of code(t = 4tg + i,
+ *            c = 16b + m), byte r = 4b + i, placed the same way; then f16 scale [16 t][4 j]  (j = c/32)
  */
 #include "private.h"
+#include "../kernel_params.h"
 
 #include <string.h>
 
@@ -53,13 +56,15 @@ static size_t bf16_index(int is_value, unsigned int t, unsigned int c)
 
 static size_t q8_code_index(int is_value, unsigned int t, unsigned int c)
 {
+    unsigned int lane_byte; /* 32 * lane + byte of the lane's 32 */
     if (is_value) {
         unsigned int tg = t / 4u, i = t % 4u, b = c / 16u, m = c % 16u;
-        return (((size_t)tg * 16u + m) * 8u + b) * 4u + i;
+        lane_byte = ((tg * 16u + m) * 8u + b) * 4u + i;
     } else {
         unsigned int j = c / 32u, g = (c % 32u) / 8u, e = c % 8u;
-        return (((size_t)g * PAGE_TOKENS + t) * 4u + j) * 8u + e;
+        lane_byte = ((g * PAGE_TOKENS + t) * 4u + j) * 8u + e;
     }
+    return (size_t)YVEX_ROCM_Q8_CODE_OFFSET(lane_byte);
 }
 
 static int layout_move(yvex_rocm_kv_storage storage, int is_value, int pack,

@@ -126,6 +126,13 @@ typedef struct {
     double rope_frequency[YVEX_ROCM_ROPE_PAIRS_MAX];
 } yvex_rocm_decode_merge_params;
 
+/* Q8_0 pages: where byte r (0..31) of the 32 code bytes that lane L (0..63) of a wave consumes
+ * lies in the 2048 code bytes of a 16-token block, written for the offset o = 32 L + r.  The two
+ * 16-byte halves of a lane's bytes are 1 KB apart, so that each of a wave's two 16-byte loads
+ * reads one contiguous KB (lanes side by side): 230 us against 264 us for config 4's 1.5 GB
+ * when the lanes' loads were 32 bytes apart. */
+#define YVEX_ROCM_Q8_CODE_OFFSET(o) ((((o) & 16u) << 6) + (((o) >> 5) << 4) + ((o) & 15u))
+
 /* A batch of small device-to-device copies in one launch: the reference's session layer
  * appends every new token to a layer's history with two asynchronous copies
  * (src/runtime/stateful_attention.c:183-222), 4096 of them for a prompt of 2048 tokens.

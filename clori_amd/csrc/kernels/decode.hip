@@ -226,7 +226,7 @@ struct Bf16Kv {
 
 // ---- Q8_0 KV ----------------------------------------------------------------------
 struct Q8Tile {
-    u32x4 kc[2];  // 32 K codes: token lane%16, lanes 32j + 8*(lane/16) + e at byte 8j + e
+    u32x4 kc[2];  // 32 K codes: token lane%16, dims 32j + 8*(lane/16) + e at byte 8j + e
     u32x4 ks[2];  // 16 f16 K scales: tokens 4*(lane/16)+i, block j at half index 4i + j
     u32x4 vc[2];  // 32 V codes: dim 16b + lane%16, tokens 4*(lane/16)+i at byte 4b + i
     u32x4 vs[2];  // 16 f16 V scales, same indexing as ks
@@ -253,12 +253,13 @@ struct Q8Kv {
                                              const unsigned char *vblock, int lane)
     {
         const int g = lane >> 4;
-        t.kc[0] = stream_b128(kblock + lane * 32);
-        t.kc[1] = stream_b128(kblock + lane * 32 + 16);
+        // the two halves of a lane's 32 code bytes are 1 KB apart: each load is one contiguous KB
+        t.kc[0] = stream_b128(kblock + lane * 16);
+        t.kc[1] = stream_b128(kblock + lane * 16 + 1024);
         t.ks[0] = stream_b128(kblock + kCodeBytes + g * 32);
         t.ks[1] = stream_b128(kblock + kCodeBytes + g * 32 + 16);
-        t.vc[0] = stream_b128(vblock + lane * 32);
-        t.vc[1] = stream_b128(vblock + lane * 32 + 16);
+        t.vc[0] = stream_b128(vblock + lane * 16);
+        t.vc[1] = stream_b128(vblock + lane * 16 + 1024);
         t.vs[0] = stream_b128(vblock + kCodeBytes + g * 32);
         t.vs[1] = stream_b128(vblock + kCodeBytes + g * 32 + 16);
     }
@@ -290,28 +291,47 @@ struct Q8Kv {
                 x[i] += half_f32(t.ks[h >> 3][(h >> 1) & 3], h & 1) * s[i];
             }
         }
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-            x[i] = (uint32_t)(g * 4 + i) < valid ? x[i] * scale_log2 : -INFINITY;
-        softmax_step(st, x, p);
-        const bool tail = valid < (uint32_t)kPageTokens;  // wave-uniform
-        // fold the V scale of each 32-lane block into the probabilities; masked tokens
-        // get an exact zero whatever their (possibly garbage) scale bits are
+        // only a context's last tile has tokens to mask: the full tile takes a path of its own
+        // (wave-uniform), without the 20 selects per tile of the masked one
+        const bool tail = valid < (uint32_t)kPageTokens;
         short4v pv[4];
+        if (!tail) {
 #pragma unroll
-        for (int jb = 0; jb < 4; ++jb) {
-            float w[4];
+            for (int i = 0; i < 4; ++i) x[i] *= scale_log2;
+            softmax_step(st, x, p);
+            // fold the V scale of each 32-lane block into the probabilities
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int h = 4 * i + jb;
-                const float vs = half_f32(t.vs[h >> 3][(h >> 1) & 3], h & 1);
-                w[i] = p[i] * vs;
-                if (tail && (uint32_t)(g * 4 + i) >= valid) w[i] = 0.f;
+            for (int jb = 0; jb < 4; ++jb) {
+                float w[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int h = 4 * i + jb;
+                    w[i] = p[i] * half_f32(t.vs[h >> 3][(h >> 1) & 3], h & 1);
+                }
+                u32x2 pb;
+                pb.x = pack_bf16x2(w[0], w[1]);
+                pb.y = pack_bf16x2(w[2], w[3]);
+                pv[jb] = as_short4(pb);
             }
-            u32x2 pb;
-            pb.x = pack_bf16x2(w[0], w[1]);
-            pb.y = pack_bf16x2(w[2], w[3]);
-            pv[jb] = as_short4(pb);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                x[i] = (uint32_t)(g * 4 + i) < valid ? x[i] * scale_log2 : -INFINITY;
+            softmax_step(st, x, p);
+            // masked tokens get an exact zero whatever their (possibly garbage) scale bits are
+#pragma unroll
+            for (int jb = 0; jb < 4; ++jb) {
+                float w[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int h = 4 * i + jb;
+                    w[i] = (uint32_t)(g * 4 + i) < valid ? p[i] * half_f32(t.vs[h >> 3][(h >> 1) & 3], h & 1) : 0.f;
+                }
+                u32x2 pb;
+                pb.x = pack_bf16x2(w[0], w[1]);
+                pb.y = pack_bf16x2(w[2], w[3]);
+                pv[jb] = as_short4(pb);
+            }
         }
 #pragma unroll
         for (int b = 0; b < 8; ++b) {

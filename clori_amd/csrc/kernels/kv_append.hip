@@ -370,7 +370,7 @@ yvex_rocm_kv_append_q8_0(const yvex_rocm_kv_append_params p)
         if (partial) {
 #pragma unroll
             for (int i = 0; i < 8; ++i)
-                old[i] = *reinterpret_cast<const uint32_t *>(vdst + (lane + 64u * i) * 4u);
+                old[i] = *reinterpret_cast<const uint32_t *>(vdst + YVEX_ROCM_Q8_CODE_OFFSET((lane + 64u * i) * 4u));
         }
         // rotated key rows into LDS
 #pragma unroll
@@ -416,14 +416,16 @@ yvex_rocm_kv_append_q8_0(const yvex_rocm_kv_append_params p)
             }
             representable &= quantise(x, scale_bits, codes);
             *reinterpret_cast<uint16_t *>(kdst + kCodeBytes + (t * 4u + j) * 2u) = scale_bits;
-            // key codes: 8-byte groups at ((g * 16 + t) * 4 + j) * 8, dims 32j + 8g + e
+            // key codes: 8-byte groups, bytes 8j .. 8j+7 of the 32 that lane 16g + t of a reading
+            // wave consumes (dims 32j + 8g + e)
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
                 const u32x2 w = {codes[2 * g], codes[2 * g + 1]};
-                *reinterpret_cast<u32x2 *>(kdst + ((g * 16u + t) * 4u + j) * 8u) = w;
+                *reinterpret_cast<u32x2 *>(kdst + YVEX_ROCM_Q8_CODE_OFFSET(((g * 16u + t) * 4u + j) * 8u)) = w;
             }
         }
-        // value codes: 4-byte groups (4 tokens of one dim) at ((tg*16 + m)*8 + b)*4, c = 16b + m
+        // value codes: 4-byte groups (4 tokens of one dim), bytes 4b .. 4b+3 of the 32 that lane
+        // 16 tg + m of a reading wave consumes, c = 16b + m
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             const uint32_t id = lane + 64u * i;  // 512 groups = tg (4) x m (16) x b (8)
@@ -437,7 +439,7 @@ yvex_rocm_kv_append_q8_0(const yvex_rocm_kv_append_params p)
                 const uint32_t byte = fresh ? (uint32_t)v_codes[tt][c] : (old[i] >> (8 * q)) & 0xffu;
                 w |= byte << (8 * q);
             }
-            *reinterpret_cast<uint32_t *>(vdst + id * 4u) = w;
+            *reinterpret_cast<uint32_t *>(vdst + YVEX_ROCM_Q8_CODE_OFFSET(id * 4u)) = w;
         }
         // a block whose scale f16 cannot hold is refused like a non-finite value, as the
         // reference encoder refuses it (src/gguf/quant_block.c:172-174)

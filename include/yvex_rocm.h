@@ -564,9 +564,11 @@ typedef enum {
  * blocks one behind the other, tokens 16 s .. 16 s + 15 of the page in block s:
  *   BF16  K block: uint16 [d/8][16 tokens][8]           (4096 B)
  *         V block: uint16 [d][16 tokens]                (4096 B)
- *   Q8_0  K block: int8 [4 lane groups][16 tokens][4 blocks][8] + f16 scale [16 tokens][4 blocks]
- *         V block: int8 [4 token groups][16 dims][8 dim blocks][4 tokens] + f16 scale [16 tokens][4 blocks]
- *                                                        (2176 B each)
+ *   Q8_0  K block: 2048 int8 codes + f16 scale [16 tokens][4 blocks]; V block likewise (2176 B each).
+ *         The codes are ordered for the reading wave: lane L takes 32 of them ([4 blocks][8] of one
+ *         token for K, [8 dim blocks][4 tokens] of one dim for V), 16 at byte 16 L and 16 at byte
+ *         1024 + 16 L of the block.  Build and read pages with yvex_rocm_kv_pack_pages /
+ *         yvex_rocm_kv_unpack_pages, or write them with kv_append_execute.
  * Pool = [pool_pages][key_value_heads][page_tokens / 16][block].  yvex_rocm_kv_pack_* build these from
  * token-major rows.  page_table is I32 [sessions][page_table_stride]; context_tokens is
  * I32 [sessions] (both device tensors).  Output is BF16 [sessions][query_heads][d], lse is

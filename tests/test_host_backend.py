@@ -1217,9 +1217,11 @@ def test_page_layouts_follow_the_documented_index_formulas():
         canon = blocks.reshape(pages, 16, hkv, 4, 34)
         t, c = np.meshgrid(np.arange(16), np.arange(d), indexing="ij")
         if is_value:
-            index = (((t // 4) * 16 + c % 16) * 8 + c // 16) * 4 + t % 4
+            lane_byte = (((t // 4) * 16 + c % 16) * 8 + c // 16) * 4 + t % 4
         else:
-            index = ((((c % 32) // 8) * 16 + t) * 4 + c // 32) * 8 + c % 8
+            lane_byte = ((((c % 32) // 8) * 16 + t) * 4 + c // 32) * 8 + c % 8
+        # byte r of the 32 a lane consumes lies at (r // 16) * 1024 + 16 * lane + r % 16
+        index = ((lane_byte & 16) << 6) + ((lane_byte >> 5) << 4) + (lane_byte & 15)
         for page in range(pages):
             for head in range(hkv):
                 codes = canon[page, :, head, :, 2:].reshape(16, d)
