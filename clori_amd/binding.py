@@ -1,4 +1,5 @@
-"""ctypes declarations for libyvex_rocm.so (the C ABI of include/yvex_rocm.h).
+"""ctypes declarations for libyvex_rocm.so (the C ABI of include/yvex_rocm.h and
+include/yvex_rocm_operations.h).
 
 The library is the product; this module only declares its types and prototypes.
 There is no fallback: a missing library raises at import.
@@ -290,7 +291,7 @@ class TimingDistribution(C.Structure):
     _fields_ = [("available", C.c_int), ("values", ull * BENCHMARK_STATISTIC_COUNT)]
 
 
-#: every symbol include/yvex_rocm.h declares
+#: every symbol include/yvex_rocm.h and include/yvex_rocm_operations.h declare
 EXPORTED_SYMBOLS = [
     "yvex_status_name", "yvex_error_clear", "yvex_error_set",
     "yvex_backend_open", "yvex_backend_open_rocm_impl", "yvex_backend_rocm_context_available",

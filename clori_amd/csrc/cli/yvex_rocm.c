@@ -14,6 +14,7 @@
 #include <string.h>
 
 #include "yvex_rocm.h"
+#include "yvex_rocm_operations.h"
 
 static int usage(FILE *fp, int code)
 {

@@ -17,10 +17,12 @@
 #include "src/backend/private.h"
 #include <yvex/internal/core.h>
 #include "yvex_rocm.h"
+#include "yvex_rocm_operations.h"
 int yvex_backend_shared_owner_acquire(yvex_backend *owner, yvex_error *err);
 #else
 
 #include "yvex_rocm.h"
+#include "yvex_rocm_operations.h"
 
 /* The slots of the reference vtable (src/backend/private.h:16-81) that lie on the
  * attention path, under the reference's names.  Everything else (embed, matmul, MoE,

@@ -27,8 +27,12 @@ enum {
     ROCM_DECODE_WAVES = 2048,
     ROCM_DECODE_MIN_TILES = 8, /* 8 and 16 measure alike on a 4096-token context; 4 and 32 are a third slower */
     ROCM_TEAM_WAVES = 8,       /* waves of a decode team (one workgroup) */
-    ROCM_TEAM_TILES = 2,       /* tiles a wave of a team is given when the history is short enough (context 4096: 10.3 us; 1: 11.6, 4: 11.9, 8: 15.9) */
-    ROCM_TEAM_TILES_WIDE = 4,  /* the same at head dimension 256, teams of four waves (24/4 heads, context 4096: 16.0 us; 2: 18.3, 8: 19.7) */
+    /* tiles a wave of a team is given when the history is short enough (context 4096: 10.3 us;
+     * 1: 11.6, 4: 11.9, 8: 15.9) */
+    ROCM_TEAM_TILES = 2,
+    /* the same at head dimension 256, teams of four waves (24/4 heads, context 4096: 16.0 us;
+     * 2: 18.3, 8: 19.7) */
+    ROCM_TEAM_TILES_WIDE = 4,
     ROCM_TEAMS_MAX = 32,       /* teams per (session, kv head): two load trips of the last team's merge */
     ROCM_TEAM_GROUP_MAX = 8,   /* query heads per kv head a team's LDS holds */
     ROCM_PREFILL_ROWS = YVEX_ROCM_PREFILL_ROWS, /* query rows per prefill workgroup */
@@ -508,6 +512,197 @@ static int exact_tile_function(const yvex_transformer_attention_requirement *r,
     return 1;
 }
 
+/* What attention_execute_common has worked out of a request before it picks a kernel. */
+typedef struct attention_geometry {
+    unsigned long long q_stride, k_stride, v_stride; /* elements between tokens */
+    unsigned long long rows;                         /* query tokens x query heads */
+    int causal;
+} attention_geometry;
+
+/* The EXACT_F32 contract: the tile kernel on the fp32 matrix cores for prefill-shaped requests,
+ * runs of keys for single rows over long histories, the row kernel for the rest. */
+static int attention_execute_exact(yvex_backend *backend, const yvex_transformer_attention_request *request,
+                                   yvex_device_tensor *lse, const attention_geometry *g,
+                                   yvex_backend_operation_facts *facts, yvex_error *err)
+{
+    yvex_rocm_backend_state *state = yvex_rocm_state(backend);
+    const yvex_transformer_attention_requirement *r = &request->requirement;
+    int rc;
+    yvex_rocm_gqa_f32_params params;
+    yvex_rocm_function_id tile_function = YVEX_ROCM_FN_GQA_F32;
+    unsigned long long split_runs = 0ull, split_keys = 0ull, split_bytes = 0ull;
+    void *split_work = NULL;
+    int tiled = 0, split_owned = 0;
+    memset(&params, 0, sizeof(params));
+    params.q = (const float *)request->query->data;
+    params.k = (const float *)request->key->data;
+    params.v = (const float *)request->value->data;
+    params.out = (float *)request->output->data;
+    params.lse = lse ? (float *)lse->data : NULL;
+    params.status = state->device_status;
+    params.query_tokens = r->query_tokens;
+    params.kv_tokens = r->key_value_tokens;
+    params.query_start = r->query_start;
+    params.query_heads = r->query_heads;
+    params.kv_heads = r->key_value_heads;
+    params.head_dim = r->head_dimension;
+    params.q_stride = g->q_stride;
+    params.k_stride = g->k_stride;
+    params.v_stride = g->v_stride;
+    params.scale = 1.0f / sqrtf((float)r->head_dimension);
+    params.causal = g->causal;
+    backend_workspace_reset(backend);
+    if (exact_tile_function(r, g->q_stride, g->k_stride, g->v_stride, request, &tile_function)) {
+        /* 128 query tokens of one head per workgroup, on the fp32 matrix cores */
+        const unsigned long long groups =
+            r->query_heads * ((r->query_tokens + ROCM_EXACT_TILE_QUERIES - 1ull) / ROCM_EXACT_TILE_QUERIES);
+        if (groups > 0x7fffffffull)
+            return refuse(err, YVEX_ERR_BOUNDS, "rocm.transformer.gqa",
+                          "attention geometry exceeds the launch range");
+        /* two workgroups per unit at head dimension 64 and 128 (registers and LDS), one (of eight
+         * waves) at 256 */
+        const unsigned int per_unit = r->head_dimension == 256ull ? 1u : 2u;
+        unsigned int workgroups = 0u;
+        if (g->causal) {
+            /* a geometry that repeats gets item lists with equal work per unit; until then,
+             * and when no lists can be made, the pairs of workgroups of a unit at least sum
+             * to the same */
+            yvex_rocm_schedule_key key;
+            memset(&key, 0, sizeof(key));
+            key.query_tokens = r->query_tokens;
+            key.kv_tokens = r->key_value_tokens;
+            key.query_start = r->query_start;
+            key.query_heads = (uint32_t)r->query_heads;
+            key.item_rows = (uint32_t)ROCM_EXACT_TILE_QUERIES;
+            key.step_keys = 32u;
+            key.per_unit = per_unit;
+            key.kind = (uint32_t)tile_function;
+            if (r->query_heads <= 0xffffull)
+                workgroups = yvex_rocm_schedule_lists(backend, &key, &params.lists);
+            if (!workgroups && per_unit == 2u && state->compute_units > 0 &&
+                groups >= 2ull * (unsigned long long)state->compute_units)
+                params.pair_units = (uint32_t)state->compute_units;
+        }
+        rc = yvex_rocm_launch(backend, tile_function, YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_F32,
+                              workgroups ? workgroups : (unsigned int)groups, 1u, 1u,
+                              /* at 256 pairs of waves split the head dimension: eight waves */
+                              r->head_dimension == 256ull ? 512u : 256u, 0u,
+                              &params, "rocm.transformer.gqa", err);
+        tiled = 1;
+    } else if ((split_runs = exact_split_runs(r, &split_keys)) != 0ull &&
+               !(((uintptr_t)request->query->data | (uintptr_t)request->key->data |
+                  (uintptr_t)request->value->data) & 15u)) {
+        /* runs of keys, one wave per (token, head, run), eight runs per workgroup */
+        unsigned long long acc_bytes = 0ull;
+        if (!exact_split_workspace(r, split_runs, &acc_bytes, &split_bytes))
+            return refuse(err, YVEX_ERR_BOUNDS, "rocm.transformer.gqa",
+                          "attention workspace geometry overflowed");
+        rc = yvex_rocm_temporary_acquire(backend, split_bytes, &split_work, &split_owned,
+                                         "rocm.transformer.gqa", err);
+        if (rc != YVEX_OK) return rc;
+        params.part_acc = (double *)split_work;
+        params.part_ml = (double *)((unsigned char *)split_work + acc_bytes);
+        params.splits = (uint32_t)split_runs;
+        params.keys_per_split = (uint32_t)split_keys;
+        params.arrivals = state->decode_arrivals;
+        rc = yvex_rocm_launch(backend,
+                              r->head_dimension > 128ull ? YVEX_ROCM_FN_GQA_F32_SPLIT_WIDE
+                                                         : YVEX_ROCM_FN_GQA_F32_SPLIT,
+                              YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_F32, (unsigned int)g->rows,
+                              (unsigned int)((split_runs + ROCM_EXACT_SPLIT_TEAM - 1ull) /
+                                             ROCM_EXACT_SPLIT_TEAM),
+                              1u, 64u * ROCM_EXACT_SPLIT_TEAM, 0u, &params, "rocm.transformer.gqa", err);
+        /* a launch that did not run to a clean end may leave arrival counts behind */
+        if (rc != YVEX_OK && !state->recording && backend->status != YVEX_BACKEND_STATUS_FAILED)
+            (void)state->driver.hipMemsetAsync(state->decode_arrivals, 0,
+                                               YVEX_ROCM_DECODE_SEGMENTS_MAX * sizeof(uint32_t),
+                                               yvex_rocm_stream(state));
+    } else {
+        split_runs = 0ull;
+        rc = yvex_rocm_launch(backend, YVEX_ROCM_FN_GQA_F32,
+                              YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_F32, (unsigned int)g->rows, 1u,
+                              1u, 64u, 0u, &params, "rocm.transformer.gqa", err);
+    }
+    if (rc == YVEX_OK) {
+        facts->kernel_launches = 1ull;
+        facts->accelerated_matrix_launches = tiled ? 1ull : 0ull;
+        facts->temporary_bytes = split_bytes;
+        facts->compulsory_memory_facts_available = 1;
+        rc = yvex_rocm_complete(backend, YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_F32,
+                                "rocm.transformer.gqa", facts, err);
+    }
+    if (split_work) {
+        yvex_error cleanup;
+        int cleanup_rc;
+        yvex_error_clear(&cleanup);
+        cleanup_rc = yvex_rocm_temporary_release(backend, split_work, split_bytes, split_owned, &cleanup);
+        backend_workspace_reset(backend);
+        if (rc == YVEX_OK && cleanup_rc != YVEX_OK) {
+            rc = cleanup_rc;
+            if (err) *err = cleanup;
+        }
+    }
+    return rc;
+}
+
+/* The BF16 contract over more than one query row (or a geometry the decode teams do not take):
+ * the MFMA prefill kernel, 128 query rows of one head per workgroup. */
+static int attention_execute_prefill(yvex_backend *backend, const yvex_transformer_attention_request *request,
+                                     yvex_device_tensor *lse, const yvex_device_tensor *gate,
+                                     const attention_geometry *g, yvex_backend_operation_facts *facts,
+                                     yvex_error *err)
+{
+    static const char where[] = "rocm.transformer.attention";
+    yvex_rocm_backend_state *state = yvex_rocm_state(backend);
+    const yvex_transformer_attention_requirement *r = &request->requirement;
+    int rc;
+    yvex_rocm_prefill_params params;
+    const unsigned long long q_tiles = (r->query_tokens + ROCM_PREFILL_ROWS - 1ull) /
+                                       ROCM_PREFILL_ROWS;
+    memset(&params, 0, sizeof(params));
+    params.q = (const uint16_t *)request->query->data;
+    params.k = (const uint16_t *)request->key->data;
+    params.v = (const uint16_t *)request->value->data;
+    params.out = (uint16_t *)request->output->data;
+    params.lse = lse ? (float *)lse->data : NULL;
+    params.gate = gate ? (const uint16_t *)gate->data : NULL;
+    params.status = state->device_status;
+    params.q_stride = g->q_stride;
+    params.k_stride = g->k_stride;
+    params.v_stride = g->v_stride;
+    params.query_tokens = (uint32_t)r->query_tokens;
+    params.kv_tokens = (uint32_t)r->key_value_tokens;
+    params.query_start = (uint32_t)r->query_start;
+    params.query_heads = (uint32_t)r->query_heads;
+    params.kv_heads = (uint32_t)r->key_value_heads;
+    params.head_dim = (uint32_t)r->head_dimension;
+    params.causal = (uint32_t)g->causal;
+    params.scale_log2 = (1.0f / sqrtf((float)r->head_dimension)) * 1.4426950408889634f;
+    backend_workspace_reset(backend);
+    /* the kernel addresses K and V through 32-bit buffer offsets */
+    if (r->query_heads > 65535ull || q_tiles > 65535ull ||
+        r->query_heads * q_tiles > 0x7fffffffull ||
+        r->key_value_tokens * g->k_stride * 2ull >= 0xffffffffull ||
+        r->key_value_tokens * g->v_stride * 2ull >= 0xffffffffull)
+        return refuse(err, YVEX_ERR_BOUNDS, where,
+                      "prefill geometry exceeds admitted launch range");
+    rc = yvex_rocm_launch(backend,
+                          r->head_dimension == 64ull    ? YVEX_ROCM_FN_PREFILL_BF16_64
+                          : r->head_dimension == 256ull ? YVEX_ROCM_FN_PREFILL_BF16_256
+                                                        : YVEX_ROCM_FN_PREFILL_BF16,
+                          YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_BF16,
+                          (unsigned int)(r->query_heads * q_tiles), 1u, 1u, 256u, 0u,
+                          &params, "rocm.transformer.gqa.prefill", err);
+    if (rc == YVEX_OK) {
+        facts->kernel_launches = 1ull;
+        facts->accelerated_matrix_launches = 1ull;
+        facts->compulsory_memory_facts_available = 1;
+        rc = yvex_rocm_complete(backend, YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_BF16,
+                                "rocm.transformer.gqa.prefill", facts, err);
+    }
+    return rc;
+}
+
 static int attention_execute_common(yvex_backend *backend,
                                     const yvex_transformer_attention_request *request,
                                     yvex_device_tensor *lse, const yvex_device_tensor *gate,
@@ -518,6 +713,7 @@ static int attention_execute_common(yvex_backend *backend,
     const yvex_transformer_attention_requirement *r;
     unsigned long long q_width, kv_width, q_stride, k_stride, v_stride;
     unsigned long long q_elements, k_elements, v_elements, o_elements, rows;
+    attention_geometry geometry;
     int exact, rc, causal;
     if (!request || !request->query || !request->key || !request->value || !request->output ||
         !facts)
@@ -559,121 +755,13 @@ static int attention_execute_common(yvex_backend *backend,
                   gate->data == request->output->data)))
         return view_refusal(backend, err, "rocm.transformer.gqa",
                       "bounded Q/K/V views matching the declared token strides are required");
+    geometry.q_stride = q_stride;
+    geometry.k_stride = k_stride;
+    geometry.v_stride = v_stride;
+    geometry.rows = rows;
+    geometry.causal = causal;
     if (exact) {
-        yvex_rocm_gqa_f32_params params;
-        yvex_rocm_function_id tile_function = YVEX_ROCM_FN_GQA_F32;
-        unsigned long long split_runs = 0ull, split_keys = 0ull, split_bytes = 0ull;
-        void *split_work = NULL;
-        int tiled = 0, split_owned = 0;
-        memset(&params, 0, sizeof(params));
-        params.q = (const float *)request->query->data;
-        params.k = (const float *)request->key->data;
-        params.v = (const float *)request->value->data;
-        params.out = (float *)request->output->data;
-        params.lse = lse ? (float *)lse->data : NULL;
-        params.status = state->device_status;
-        params.query_tokens = r->query_tokens;
-        params.kv_tokens = r->key_value_tokens;
-        params.query_start = r->query_start;
-        params.query_heads = r->query_heads;
-        params.kv_heads = r->key_value_heads;
-        params.head_dim = r->head_dimension;
-        params.q_stride = q_stride;
-        params.k_stride = k_stride;
-        params.v_stride = v_stride;
-        params.scale = 1.0f / sqrtf((float)r->head_dimension);
-        params.causal = causal;
-        backend_workspace_reset(backend);
-        if (exact_tile_function(r, q_stride, k_stride, v_stride, request, &tile_function)) {
-            /* 128 query tokens of one head per workgroup, on the fp32 matrix cores */
-            const unsigned long long groups =
-                r->query_heads * ((r->query_tokens + ROCM_EXACT_TILE_QUERIES - 1ull) / ROCM_EXACT_TILE_QUERIES);
-            if (groups > 0x7fffffffull)
-                return refuse(err, YVEX_ERR_BOUNDS, "rocm.transformer.gqa",
-                              "attention geometry exceeds the launch range");
-            /* two workgroups per unit at head dimension 64 and 128 (registers and LDS), one (of eight
-             * waves) at 256 */
-            const unsigned int per_unit = r->head_dimension == 256ull ? 1u : 2u;
-            unsigned int workgroups = 0u;
-            if (causal) {
-                /* a geometry that repeats gets item lists with equal work per unit; until then,
-                 * and when no lists can be made, the pairs of workgroups of a unit at least sum
-                 * to the same */
-                yvex_rocm_schedule_key key;
-                memset(&key, 0, sizeof(key));
-                key.query_tokens = r->query_tokens;
-                key.kv_tokens = r->key_value_tokens;
-                key.query_start = r->query_start;
-                key.query_heads = (uint32_t)r->query_heads;
-                key.item_rows = (uint32_t)ROCM_EXACT_TILE_QUERIES;
-                key.step_keys = 32u;
-                key.per_unit = per_unit;
-                key.kind = (uint32_t)tile_function;
-                if (r->query_heads <= 0xffffull)
-                    workgroups = yvex_rocm_schedule_lists(backend, &key, &params.lists);
-                if (!workgroups && per_unit == 2u && state->compute_units > 0 &&
-                    groups >= 2ull * (unsigned long long)state->compute_units)
-                    params.pair_units = (uint32_t)state->compute_units;
-            }
-            rc = yvex_rocm_launch(backend, tile_function, YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_F32,
-                                  workgroups ? workgroups : (unsigned int)groups, 1u, 1u,
-                                  /* at 256 pairs of waves split the head dimension: eight waves */
-                                  r->head_dimension == 256ull ? 512u : 256u, 0u,
-                                  &params, "rocm.transformer.gqa", err);
-            tiled = 1;
-        } else if ((split_runs = exact_split_runs(r, &split_keys)) != 0ull &&
-                   !(((uintptr_t)request->query->data | (uintptr_t)request->key->data |
-                      (uintptr_t)request->value->data) & 15u)) {
-            /* runs of keys, one wave per (token, head, run), eight runs per workgroup */
-            unsigned long long acc_bytes = 0ull;
-            if (!exact_split_workspace(r, split_runs, &acc_bytes, &split_bytes))
-                return refuse(err, YVEX_ERR_BOUNDS, "rocm.transformer.gqa",
-                              "attention workspace geometry overflowed");
-            rc = yvex_rocm_temporary_acquire(backend, split_bytes, &split_work, &split_owned,
-                                             "rocm.transformer.gqa", err);
-            if (rc != YVEX_OK) return rc;
-            params.part_acc = (double *)split_work;
-            params.part_ml = (double *)((unsigned char *)split_work + acc_bytes);
-            params.splits = (uint32_t)split_runs;
-            params.keys_per_split = (uint32_t)split_keys;
-            params.arrivals = state->decode_arrivals;
-            rc = yvex_rocm_launch(backend,
-                                  r->head_dimension > 128ull ? YVEX_ROCM_FN_GQA_F32_SPLIT_WIDE
-                                                             : YVEX_ROCM_FN_GQA_F32_SPLIT,
-                                  YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_F32, (unsigned int)rows,
-                                  (unsigned int)((split_runs + ROCM_EXACT_SPLIT_TEAM - 1ull) /
-                                                 ROCM_EXACT_SPLIT_TEAM),
-                                  1u, 64u * ROCM_EXACT_SPLIT_TEAM, 0u, &params, "rocm.transformer.gqa", err);
-            /* a launch that did not run to a clean end may leave arrival counts behind */
-            if (rc != YVEX_OK && !state->recording && backend->status != YVEX_BACKEND_STATUS_FAILED)
-                (void)state->driver.hipMemsetAsync(state->decode_arrivals, 0,
-                                                   YVEX_ROCM_DECODE_SEGMENTS_MAX * sizeof(uint32_t),
-                                                   yvex_rocm_stream(state));
-        } else {
-            split_runs = 0ull;
-            rc = yvex_rocm_launch(backend, YVEX_ROCM_FN_GQA_F32,
-                                  YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_F32, (unsigned int)rows, 1u,
-                                  1u, 64u, 0u, &params, "rocm.transformer.gqa", err);
-        }
-        if (rc == YVEX_OK) {
-            facts->kernel_launches = 1ull;
-            facts->accelerated_matrix_launches = tiled ? 1ull : 0ull;
-            facts->temporary_bytes = split_bytes;
-            facts->compulsory_memory_facts_available = 1;
-            rc = yvex_rocm_complete(backend, YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_F32,
-                                    "rocm.transformer.gqa", facts, err);
-        }
-        if (split_work) {
-            yvex_error cleanup;
-            int cleanup_rc;
-            yvex_error_clear(&cleanup);
-            cleanup_rc = yvex_rocm_temporary_release(backend, split_work, split_bytes, split_owned, &cleanup);
-            backend_workspace_reset(backend);
-            if (rc == YVEX_OK && cleanup_rc != YVEX_OK) {
-                rc = cleanup_rc;
-                if (err) *err = cleanup;
-            }
-        }
+        rc = attention_execute_exact(backend, request, lse, &geometry, facts, err);
     } else if (decode_rows_geometry(r)) {
         decode_job job;
         memset(&job, 0, sizeof(job));
@@ -696,50 +784,7 @@ static int attention_execute_common(yvex_backend *backend,
         job.scale = 1.0f / sqrtf((float)r->head_dimension);
         rc = decode_run(backend, &job, "rocm.transformer.gqa.decode", facts, err);
     } else {
-        yvex_rocm_prefill_params params;
-        const unsigned long long q_tiles = (r->query_tokens + ROCM_PREFILL_ROWS - 1ull) /
-                                           ROCM_PREFILL_ROWS;
-        memset(&params, 0, sizeof(params));
-        params.q = (const uint16_t *)request->query->data;
-        params.k = (const uint16_t *)request->key->data;
-        params.v = (const uint16_t *)request->value->data;
-        params.out = (uint16_t *)request->output->data;
-        params.lse = lse ? (float *)lse->data : NULL;
-        params.gate = gate ? (const uint16_t *)gate->data : NULL;
-        params.status = state->device_status;
-        params.q_stride = q_stride;
-        params.k_stride = k_stride;
-        params.v_stride = v_stride;
-        params.query_tokens = (uint32_t)r->query_tokens;
-        params.kv_tokens = (uint32_t)r->key_value_tokens;
-        params.query_start = (uint32_t)r->query_start;
-        params.query_heads = (uint32_t)r->query_heads;
-        params.kv_heads = (uint32_t)r->key_value_heads;
-        params.head_dim = (uint32_t)r->head_dimension;
-        params.causal = (uint32_t)causal;
-        params.scale_log2 = (1.0f / sqrtf((float)r->head_dimension)) * 1.4426950408889634f;
-        backend_workspace_reset(backend);
-        /* the kernel addresses K and V through 32-bit buffer offsets */
-        if (r->query_heads > 65535ull || q_tiles > 65535ull ||
-            r->query_heads * q_tiles > 0x7fffffffull ||
-            r->key_value_tokens * k_stride * 2ull >= 0xffffffffull ||
-            r->key_value_tokens * v_stride * 2ull >= 0xffffffffull)
-            return refuse(err, YVEX_ERR_BOUNDS, where,
-                          "prefill geometry exceeds admitted launch range");
-        rc = yvex_rocm_launch(backend,
-                              r->head_dimension == 64ull    ? YVEX_ROCM_FN_PREFILL_BF16_64
-                              : r->head_dimension == 256ull ? YVEX_ROCM_FN_PREFILL_BF16_256
-                                                            : YVEX_ROCM_FN_PREFILL_BF16,
-                              YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_BF16,
-                              (unsigned int)(r->query_heads * q_tiles), 1u, 1u, 256u, 0u,
-                              &params, "rocm.transformer.gqa.prefill", err);
-        if (rc == YVEX_OK) {
-            facts->kernel_launches = 1ull;
-            facts->accelerated_matrix_launches = 1ull;
-            facts->compulsory_memory_facts_available = 1;
-            rc = yvex_rocm_complete(backend, YVEX_BACKEND_VARIANT_ROCM_ATTENTION_GQA_BF16,
-                                    "rocm.transformer.gqa.prefill", facts, err);
-        }
+        rc = attention_execute_prefill(backend, request, lse, gate, &geometry, facts, err);
     }
     if (rc != YVEX_OK) return rc;
     request->output->is_written = 1;

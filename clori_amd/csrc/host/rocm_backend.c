@@ -766,15 +766,15 @@ static int rocm_open(yvex_backend **out, const char *device, unsigned long long 
                               where, err);
     if (rc == YVEX_OK && state->driver.pinned_memory) {
         /* the status mailbox is an economy, not a requirement: without it the word is copied */
-        void *host = NULL, *device = NULL;
+        void *host = NULL, *mapped = NULL;
         if (state->driver.hipHostMalloc(&host, 256u + YVEX_ROCM_SMALL_READ_MAX, hipHostMallocMapped) ==
                 hipSuccess && host) {
-            if (state->driver.hipHostGetDevicePointer(&device, host, 0u) == hipSuccess && device) {
+            if (state->driver.hipHostGetDevicePointer(&mapped, host, 0u) == hipSuccess && mapped) {
                 memset(host, 0, 256u + YVEX_ROCM_SMALL_READ_MAX);
                 state->status_mailbox = (volatile uint64_t *)host;
-                state->status_mailbox_device = (uint64_t *)device;
+                state->status_mailbox_device = (uint64_t *)mapped;
                 state->read_staging = (unsigned char *)host + 256u;
-                state->read_staging_device = (unsigned char *)device + 256u;
+                state->read_staging_device = (unsigned char *)mapped + 256u;
             } else {
                 (void)state->driver.hipHostFree(host);
             }

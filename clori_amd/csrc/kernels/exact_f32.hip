@@ -501,7 +501,8 @@ yvex_rocm_stream_read(const yvex_rocm_stream_params p)
         const u32x4 *base = words + b * 512u + lane;
         u32x4 v[8];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) v[j] = __builtin_nontemporal_load(base + j * 64);  // read once, as the page blocks are
+        // read once, as the page blocks are
+        for (int j = 0; j < 8; ++j) v[j] = __builtin_nontemporal_load(base + j * 64);
 #pragma unroll
         for (int j = 0; j < 8; ++j) acc ^= v[j];
     }

@@ -24,8 +24,14 @@ __device__ inline u32x2 load_b64(const void *p) { return *reinterpret_cast<const
 // batch of sessions): with the non-temporal hint random 4 KB blocks arrive at 6.2 TB/s on this
 // part where plain loads reach 5.7.  Data that the caches can keep between launches (a history
 // of a few MB, the latent pool of one MLA step) is slower that way.
-__device__ inline u32x4 stream_b128(const void *p) { return __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(p)); }
-__device__ inline u32x2 stream_b64(const void *p) { return __builtin_nontemporal_load(reinterpret_cast<const u32x2 *>(p)); }
+__device__ inline u32x4 stream_b128(const void *p)
+{
+    return __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(p));
+}
+__device__ inline u32x2 stream_b64(const void *p)
+{
+    return __builtin_nontemporal_load(reinterpret_cast<const u32x2 *>(p));
+}
 
 __device__ inline bf16x8 as_bf16x8(u32x4 v) { return __builtin_bit_cast(bf16x8, v); }
 __device__ inline short4v as_short4(u32x2 v) { return __builtin_bit_cast(short4v, v); }

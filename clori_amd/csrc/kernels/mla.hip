@@ -291,8 +291,8 @@ __device__ __forceinline__ void mla_decode(const yvex_rocm_mla_params &p, unsign
             __builtin_amdgcn_sched_barrier(0);
         }
     };
-    // masks the tail (and the keys in front of a sliding window), then raises the running maximum if this tile needs it (both token
-    // halves of a head must agree on the reference maximum)
+    // masks the tail (and the keys in front of a sliding window), then raises the running maximum if this
+    // tile needs it (both token halves of a head must agree on the reference maximum)
     // `first`: the chunk's first tile, nothing accumulated yet: the maximum is taken as it is
     // and there is nothing to rescale (the general path would multiply 256 zeros)
     auto settle = [&](uint32_t key0, floatx16 &s, uint32_t (&pending)[8], auto first) {
@@ -464,7 +464,8 @@ __device__ __forceinline__ void mla_decode(const yvex_rocm_mla_params &p, unsign
     // only this wave reads what it wrote: no workgroup barrier needed
     __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
     {
-        const uint64_t slot0 = ((uint64_t)batch * p.slot_stride + p.first_slot + chunk) * p.heads + wave * kHeadsPerWave;
+        const uint64_t slot0 =
+            ((uint64_t)batch * p.slot_stride + p.first_slot + chunk) * p.heads + wave * kHeadsPerWave;
         uint16_t *dst = p.part_acc + slot0 * kValueDim + lane * 8;
         // every workgroup starts its 32 rows at another one: the rows of all workgroups are
         // 1 KB apart at the same offsets of 128 KB regions, and written in step they would all

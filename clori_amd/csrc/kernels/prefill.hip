@@ -351,7 +351,8 @@ struct Prefill {
             for (int i = 0; i < kSlots; ++i) {
                 // ---- the MFMA of this slot ----
                 if (i < kHalfSlots) {
-                    const floatx16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+                    const floatx16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f,
+                                           0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
                     s_next[i & 1] = mfma_32x32x16(as_bf16x8(frag[i % kDepth]), q[i >> 1],
                                                   i < 2 ? zero : s_next[i & 1]);
                 } else {

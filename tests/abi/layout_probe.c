@@ -8,6 +8,7 @@
 #include <yvex/internal/transformer.h>
 #else
 #include "yvex_rocm.h"
+#include "yvex_rocm_operations.h"
 #endif
 
 #define SIZE(type) printf("sizeof %s %zu\n", #type, sizeof(type))

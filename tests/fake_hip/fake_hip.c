@@ -16,7 +16,8 @@
 #include <string.h>
 #include <sys/mman.h>
 
-static unsigned long long launches, allocations, frees, loads, unloads, forwards, copy_batches, async_copies, small_transfers;
+static unsigned long long launches, allocations, frees, loads, unloads, forwards, copy_batches, async_copies,
+    small_transfers;
 static int capturing;                       /* a stream capture is open */
 static unsigned long long captured_launches;
 

@@ -68,7 +68,8 @@ def test_library_exports_every_declared_symbol():
     library = lib()
     for name in B.EXPORTED_SYMBOLS:
         assert hasattr(library, name), name
-    header = open(os.path.join(ROOT, "include", "yvex_rocm.h")).read()
+    header = "".join(open(os.path.join(ROOT, "include", name)).read()
+                     for name in ("yvex_rocm.h", "yvex_rocm_operations.h"))
     for name in B.EXPORTED_SYMBOLS:
         assert name + "(" in header, "declared in binding but not in the header: " + name
 
