@@ -84,3 +84,18 @@ def test_host_objects_are_built_with_the_required_warnings():
     flags = makefile[makefile.index("CFLAGS :="):makefile.index("HIPFLAGS :=")]
     for warning in REQUIRED_C_WARNINGS:
         assert warning in flags, warning
+
+
+def test_exported_symbols_follow_the_reference_namespace():
+    # config/c_policy.json:108-113: public symbols carry the yvex_ prefix and none of the
+    # fragments that mark test, fixture, rendering or family code
+    import subprocess
+    library = os.path.join(ROOT, "clori_amd", "libyvex_rocm.so")
+    listing = subprocess.run(["nm", "-D", "--defined-only", library], check=True,
+                             capture_output=True, text=True).stdout
+    names = [line.split()[-1] for line in listing.splitlines() if line.strip()]
+    assert len(names) > 40
+    for name in names:
+        assert name.startswith("yvex_"), name
+        for fragment in ("_fixture_", "_reference_", "_test_", "_render_", "_deepseek_"):
+            assert fragment not in name, name
