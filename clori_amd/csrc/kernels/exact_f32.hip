@@ -247,6 +247,46 @@ __device__ __forceinline__ void split_unit(const yvex_rocm_gqa_f32_params &p, ui
     if ((p.query_heads & 7u) == 0u) head = (head & 7u) * (p.query_heads >> 3) + (head >> 3);
 }
 
+// The partials of a unit's teams (maximum, sum and one value per thread), merged in team order:
+// what the last team of a unit to arrive does.  Eight teams per trip of independent loads.
+__device__ __forceinline__ void merge_team_partials(const yvex_rocm_gqa_f32_params &p, uint64_t unit,
+                                                    uint32_t teams, uint32_t t, uint64_t d, double &top,
+                                                    double &total, double &o)
+{
+    top = -INFINITY;
+    total = 0.0;
+    o = 0.0;
+    // eight teams per trip of independent loads (teams past the end alias the last one
+    // with weight zero)
+    for (uint32_t t0 = 0u; t0 < teams; t0 += 8u) {
+        double mt[8], lt[8], vt[8];
+#pragma unroll
+        for (uint32_t i = 0u; i < 8u; ++i) {
+            const uint64_t from = unit * teams + min(t0 + i, teams - 1u);
+            mt[i] = load_f64_device(p.part_ml + from * 2u);
+            lt[i] = load_f64_device(p.part_ml + from * 2u + 1u);
+            vt[i] = t < d ? load_f64_device(p.part_acc + from * d + t) : 0.0;
+        }
+        double trip = -INFINITY;
+#pragma unroll
+        for (uint32_t i = 0u; i < 8u; ++i) {
+            if (t0 + i >= teams) mt[i] = -INFINITY;
+            trip = fmax(trip, mt[i]);
+        }
+        const double top_new = fmax(top, trip);
+        const double keep = top == -INFINITY ? 0.0 : exp(top - top_new);
+        total *= keep;
+        o *= keep;
+#pragma unroll
+        for (uint32_t i = 0u; i < 8u; ++i) {
+            const double weight = mt[i] == -INFINITY ? 0.0 : exp(mt[i] - top_new);
+            total += weight * lt[i];
+            o += weight * vt[i];
+        }
+        top = top_new;
+    }
+}
+
 template <int kPieces>
 __device__ __forceinline__ void gqa_f32_split(const yvex_rocm_gqa_f32_params &p, double *team_lds)
 {
@@ -416,38 +456,7 @@ __device__ __forceinline__ void gqa_f32_split(const yvex_rocm_gqa_f32_params &p,
         __syncthreads();
         if (*last == 0u) return;
         loads_ordered();
-        top = -INFINITY;
-        total = 0.0;
-        o = 0.0;
-        // eight teams per trip of independent loads (teams past the end alias the last one
-        // with weight zero)
-        for (uint32_t t0 = 0u; t0 < teams; t0 += 8u) {
-            double mt[8], lt[8], vt[8];
-#pragma unroll
-            for (uint32_t i = 0u; i < 8u; ++i) {
-                const uint64_t from = unit * teams + min(t0 + i, teams - 1u);
-                mt[i] = load_f64_device(p.part_ml + from * 2u);
-                lt[i] = load_f64_device(p.part_ml + from * 2u + 1u);
-                vt[i] = t < d ? load_f64_device(p.part_acc + from * d + t) : 0.0;
-            }
-            double trip = -INFINITY;
-#pragma unroll
-            for (uint32_t i = 0u; i < 8u; ++i) {
-                if (t0 + i >= teams) mt[i] = -INFINITY;
-                trip = fmax(trip, mt[i]);
-            }
-            const double top_new = fmax(top, trip);
-            const double keep = top == -INFINITY ? 0.0 : exp(top - top_new);
-            total *= keep;
-            o *= keep;
-#pragma unroll
-            for (uint32_t i = 0u; i < 8u; ++i) {
-                const double weight = mt[i] == -INFINITY ? 0.0 : exp(mt[i] - top_new);
-                total += weight * lt[i];
-                o += weight * vt[i];
-            }
-            top = top_new;
-        }
+        merge_team_partials(p, unit, teams, t, d, top, total, o);
     }
     if (!(total > 0.0) || !isfinite(total) || !isfinite(top)) {
         if (t == 0u) flag(p.status, YVEX_ROCM_DEVICE_NUMERIC);
